@@ -1,0 +1,89 @@
+"""ctypes loader for ``librecis_hip.so`` (the C-ABI HIP library).
+
+The product path never falls back to a CPU implementation: if the library is
+missing it is built once (hipcc cross-compiles without a GPU); if that fails,
+or a call returns an error, a ``RuntimeError`` is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "librecis_hip.so")
+HEADER_PATH = os.path.join(_HERE, "..", "include", "recis_hip.h")
+
+_lib = None
+
+F32, BF16, F16 = 0, 1, 2
+SUM, MEAN, TILE, MAX = 0, 1, 2, 3
+FLAG_REV_UNIQUE = 1
+
+DEVERR_INDEX_RANGE = 1
+DEVERR_OFFSETS = 2
+DEVERR_TABLE_FULL = 4
+
+_DTYPES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+MODES = {"sum": SUM, "mean": MEAN, "tile": TILE, "max": MAX}
+
+
+class RecisHipError(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded library (built first if no binary is present)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            from . import build as _build
+
+            _build.build(verbose=False)
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.recis_hip_last_error.restype = ctypes.c_char_p
+        abi = _lib.recis_hip_abi_version()
+        if abi != 1:
+            raise RecisHipError("librecis_hip.so ABI %d, expected 1: rebuild with "
+                                "python -m recis_amd.build" % abi)
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise RecisHipError("librecis_hip: %s (code %d)" %
+                            (lib().recis_hip_last_error().decode(), rc))
+
+
+def dtype_code(dt):
+    try:
+        return _DTYPES[dt]
+    except KeyError:
+        raise TypeError("unsupported row dtype %s (float32, bfloat16, float16)" % dt)
+
+
+def ptr(t):
+    """Device pointer of a tensor as a ctypes void pointer (None -> NULL)."""
+    if t is None:
+        return ctypes.c_void_p(0)
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def i64(x):
+    return ctypes.c_int64(int(x))
+
+
+def stream_ptr(device=None):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RecisHipError("expected a GPU tensor, got one on %s" % t.device)
+
+
+def poll_device_errors():
+    """Synchronises the device and returns (and clears) the soft-error bits."""
+    bits = ctypes.c_int(0)
+    check(lib().recis_hip_poll_device_errors(ctypes.byref(bits)))
+    return bits.value

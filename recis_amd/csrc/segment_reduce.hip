@@ -1,0 +1,650 @@
+// Ragged gather + segment reduce (pooling) forward and backward for gfx950.
+//
+// Design (differs from the reference's one-atomic-per-element kernels,
+// csrc/ops/embedding_segment_reduce_kernel.cu:23-120):
+//   * a power-of-two "team" of lanes owns one segment; the team is split into
+//     row groups of LPR lanes, each lane moving one 16-byte vector of a row, so
+//     a 64-lane wave streams TEAM/LPR rows per step with fully coalesced
+//     16-byte accesses
+//   * partial sums stay in registers (fp32) and the row groups are combined
+//     with wave shuffles; each output row is written exactly once, with no
+//     atomics and no pre-zeroed output
+//   * segment offsets of the segments a workgroup owns are staged in LDS once
+//   * the backward pass walks segments the same way: the pooled gradient row is
+//     read once per segment and fanned out to its occurrences, by plain stores
+//     when the caller guarantees distinct rows, by fp32 atomics otherwise
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "common.cuh"
+
+namespace recis_hip {
+namespace {
+
+__device__ __forceinline__ float load_weight(const void* w, int wdt, int64_t i) {
+  if (wdt == RECIS_F32) return static_cast<const float*>(w)[i];
+  if (wdt == RECIS_BF16) return to_float(static_cast<const bf16_t*>(w)[i]);
+  return to_float(static_cast<const f16_t*>(w)[i]);
+}
+
+struct SegArgs {
+  const void* weight;
+  const void* rev;
+  const void* offs;
+  int64_t B, U, S;
+  int D;
+  int wdt, rev64, off64;
+  int lpr_log2, team_log2;
+  int mean;
+  int* err;
+};
+
+// Stage offsets[s0 .. s0 + teams_per_block] into LDS and return this team's
+// [start, end). Returns false for teams beyond the last segment.
+__device__ __forceinline__ bool team_segment(const SegArgs& a, int64_t* s_off,
+                                             int64_t& s, int64_t& start,
+                                             int64_t& end) {
+  const int tid = threadIdx.x;
+  const int teams_per_block = kBlock >> a.team_log2;
+  const int64_t s0 = static_cast<int64_t>(blockIdx.x) * teams_per_block;
+  for (int i = tid; i <= teams_per_block; i += kBlock) {
+    int64_t si = s0 + i;
+    if (si <= a.S) s_off[i] = load_index(a.offs, a.off64, si);
+  }
+  __syncthreads();
+  const int team = tid >> a.team_log2;
+  s = s0 + team;
+  if (s >= a.S) return false;
+  start = s_off[team];
+  end = s_off[team + 1];
+  if (start < 0 || end > a.B || end < start) {
+    raise_device_error(a.err, RECIS_DEVERR_OFFSETS);
+    start = end = 0;
+  }
+  return true;
+}
+
+// ------------------------------------------------------------------ forward
+template <typename TIn, typename TOut, int VEC>
+__global__ void __launch_bounds__(kBlock)
+seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
+  __shared__ int64_t s_off[kBlock + 1];
+  int64_t s, start, end;
+  if (!team_segment(a, s_off, s, start, end)) return;
+
+  const int lane_t = threadIdx.x & ((1 << a.team_log2) - 1);
+  const int rg = lane_t >> a.lpr_log2;
+  const int cl = lane_t & ((1 << a.lpr_log2) - 1);
+  const int64_t step = int64_t(1) << (a.team_log2 - a.lpr_log2);
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+  const float scale = (a.mean && end > start) ? 1.0f / static_cast<float>(end - start) : 1.0f;
+
+  auto fetch = [&](int64_t r, int c0, float (&v)[VEC], float& w) {
+    int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+    w = a.weight ? load_weight(a.weight, a.wdt, r) : 1.0f;
+    if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+      raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+      w = 0.f;
+      return;
+    }
+    load_pack<TIn, VEC>(emb + idx * D + c0, v);
+  };
+
+  for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+
+    int64_t r = start + rg;
+    for (; r + 3 * step < end; r += 4 * step) {
+      float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
+      float w0, w1, w2, w3;
+      fetch(r, c0, v0, w0);
+      fetch(r + step, c0, v1, w1);
+      fetch(r + 2 * step, c0, v2, w2);
+      fetch(r + 3 * step, c0, v3, w3);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        acc[j] = fmaf(v0[j], w0, acc[j]);
+        acc[j] = fmaf(v1[j], w1, acc[j]);
+        acc[j] = fmaf(v2[j], w2, acc[j]);
+        acc[j] = fmaf(v3[j], w3, acc[j]);
+      }
+    }
+    for (; r < end; r += step) {
+      float v0[VEC];
+      float w0;
+      fetch(r, c0, v0, w0);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v0[j], w0, acc[j]);
+    }
+    // combine the row groups of the team (partners share cl, hence c0)
+    for (int off = 1 << a.lpr_log2; off < (1 << a.team_log2); off <<= 1) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+    }
+    if (rg == 0) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] *= scale;
+      store_pack<TOut, VEC>(out + s * D + c0, acc);
+    }
+  }
+}
+
+// MAX combiner: element-wise maximum and the occurrence that produced it.
+template <typename TIn, typename TOut, int VEC>
+__global__ void __launch_bounds__(kBlock)
+seg_max_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out,
+                   int32_t* __restrict__ argmax, SegArgs a) {
+  __shared__ int64_t s_off[kBlock + 1];
+  int64_t s, start, end;
+  if (!team_segment(a, s_off, s, start, end)) return;
+
+  const int lane_t = threadIdx.x & ((1 << a.team_log2) - 1);
+  const int rg = lane_t >> a.lpr_log2;
+  const int cl = lane_t & ((1 << a.lpr_log2) - 1);
+  const int64_t step = int64_t(1) << (a.team_log2 - a.lpr_log2);
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+
+  for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
+    float best[VEC];
+    int32_t arg[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      best[j] = -INFINITY;
+      arg[j] = -1;
+    }
+    for (int64_t r = start + rg; r < end; r += step) {
+      int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+      if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+        raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        continue;
+      }
+      float v[VEC];
+      load_pack<TIn, VEC>(emb + idx * D + c0, v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        // strict > keeps the earliest occurrence within this row group;
+        // a NaN is taken once and then sticks (like torch's amax)
+        if (arg[j] < 0 || v[j] > best[j] || (v[j] != v[j] && best[j] == best[j])) {
+          best[j] = v[j];
+          arg[j] = static_cast<int32_t>(r);
+        }
+      }
+    }
+    for (int off = 1 << a.lpr_log2; off < (1 << a.team_log2); off <<= 1) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        float ob = __shfl_xor(best[j], off, kWave);
+        int32_t oa = __shfl_xor(arg[j], off, kWave);
+        bool mine_nan = best[j] != best[j];
+        bool other_nan = ob != ob;
+        bool take;
+        if (oa < 0) {
+          take = false;
+        } else if (arg[j] < 0) {
+          take = true;
+        } else if (mine_nan || other_nan) {
+          take = other_nan && (!mine_nan || oa < arg[j]);
+        } else {
+          take = (ob > best[j]) || (ob == best[j] && oa < arg[j]);
+        }
+        if (take) {
+          best[j] = ob;
+          arg[j] = oa;
+        }
+      }
+    }
+    if (rg == 0) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j)
+        if (arg[j] < 0) best[j] = 0.f;
+      store_pack<TOut, VEC>(out + s * D + c0, best);
+      if (argmax) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) argmax[s * D + c0 + j] = arg[j];
+      }
+    }
+  }
+}
+
+// TILE combiner forward: one row group per occurrence, out[i] = w_i * emb[rev_i];
+// occurrences outside [offsets[0], offsets[S]) produce zero rows.
+template <typename TIn, typename TOut, int VEC>
+__global__ void __launch_bounds__(kBlock)
+seg_tile_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * rows_per_block + (threadIdx.x >> a.lpr_log2);
+  if (r >= a.B) return;
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+  const int64_t lo = load_index(a.offs, a.off64, 0);
+  const int64_t hi = load_index(a.offs, a.off64, a.S);
+  bool live = r >= lo && r < hi;
+  int64_t idx = 0;
+  float w = 0.f;
+  if (live) {
+    idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+    w = a.weight ? load_weight(a.weight, a.wdt, r) : 1.0f;
+    if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+      raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      live = false;
+    }
+  }
+  for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
+    float v[VEC];
+    if (live) {
+      load_pack<TIn, VEC>(emb + idx * D + c0, v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] *= w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+    }
+    store_pack<TOut, VEC>(out + r * D + c0, v);
+  }
+}
+
+// ----------------------------------------------------------------- backward
+template <typename TOut, int VEC>
+__global__ void __launch_bounds__(kBlock)
+fill_zero_rows_kernel(TOut* __restrict__ p, int64_t n_packs) {
+  int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  float z[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) z[j] = 0.f;
+  for (; i < n_packs; i += stride) store_pack<TOut, VEC>(p + i * VEC, z);
+}
+
+// SUM / MEAN backward, segment-major. ATOMIC=false writes each touched row once.
+template <typename TG, typename TOut, int VEC, bool ATOMIC>
+__global__ void __launch_bounds__(kBlock)
+seg_pool_bwd_kernel(const TG* __restrict__ grad_out, TOut* __restrict__ grad_unique, SegArgs a) {
+  __shared__ int64_t s_off[kBlock + 1];
+  int64_t s, start, end;
+  if (!team_segment(a, s_off, s, start, end)) return;
+
+  const int lane_t = threadIdx.x & ((1 << a.team_log2) - 1);
+  const int rg = lane_t >> a.lpr_log2;
+  const int cl = lane_t & ((1 << a.lpr_log2) - 1);
+  const int64_t step = int64_t(1) << (a.team_log2 - a.lpr_log2);
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+  const float scale = (a.mean && end > start) ? 1.0f / static_cast<float>(end - start) : 1.0f;
+
+  for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
+    float g[VEC];
+    load_pack<TG, VEC>(grad_out + s * D + c0, g);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) g[j] *= scale;
+    for (int64_t r = start + rg; r < end; r += step) {
+      int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+      float w = a.weight ? load_weight(a.weight, a.wdt, r) : 1.0f;
+      if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+        raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        continue;
+      }
+      float v[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = g[j] * w;
+      if constexpr (ATOMIC) {
+        float* dst = reinterpret_cast<float*>(grad_unique) + idx * D + c0;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) unsafeAtomicAdd(dst + j, v[j]);
+      } else {
+        store_pack<TOut, VEC>(grad_unique + idx * D + c0, v);
+      }
+    }
+  }
+}
+
+// Rows of occurrences that no segment covers (before offsets[0], after
+// offsets[S]) when the caller promised a bijection occurrence <-> row and no
+// zero fill was done.
+template <typename TOut, int VEC>
+__global__ void __launch_bounds__(kBlock)
+seg_bwd_zero_uncovered_kernel(TOut* __restrict__ grad_unique, SegArgs a) {
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int64_t lo = load_index(a.offs, a.off64, 0);
+  const int64_t hi = load_index(a.offs, a.off64, a.S);
+  const int64_t head = lo < 0 ? 0 : (lo > a.B ? a.B : lo);
+  const int64_t tail_begin = hi < head ? head : (hi > a.B ? a.B : hi);
+  const int64_t n_uncovered = head + (a.B - tail_begin);
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int col_stride = VEC << a.lpr_log2;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * rows_per_block;
+  float z[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) z[j] = 0.f;
+  for (int64_t k = static_cast<int64_t>(blockIdx.x) * rows_per_block + (threadIdx.x >> a.lpr_log2);
+       k < n_uncovered; k += stride) {
+    int64_t r = k < head ? k : tail_begin + (k - head);
+    int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+    if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) continue;
+    for (int c0 = cl * VEC; c0 < a.D; c0 += col_stride)
+      store_pack<TOut, VEC>(grad_unique + idx * a.D + c0, z);
+  }
+}
+
+// TILE backward: one row group per occurrence.
+template <typename TG, typename TOut, int VEC, bool ATOMIC>
+__global__ void __launch_bounds__(kBlock)
+seg_tile_bwd_kernel(const TG* __restrict__ grad_out, TOut* __restrict__ grad_unique, SegArgs a) {
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * rows_per_block + (threadIdx.x >> a.lpr_log2);
+  if (r >= a.B) return;
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+  const int64_t lo = load_index(a.offs, a.off64, 0);
+  const int64_t hi = load_index(a.offs, a.off64, a.S);
+  const bool live = r >= lo && r < hi;
+  int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+  if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+    raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+    return;
+  }
+  if (ATOMIC && !live) return;
+  const float w = live ? (a.weight ? load_weight(a.weight, a.wdt, r) : 1.0f) : 0.f;
+  for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
+    float v[VEC];
+    if (live) {
+      load_pack<TG, VEC>(grad_out + r * D + c0, v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] *= w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+    }
+    if constexpr (ATOMIC) {
+      float* dst = reinterpret_cast<float*>(grad_unique) + idx * D + c0;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) unsafeAtomicAdd(dst + j, v[j]);
+    } else {
+      store_pack<TOut, VEC>(grad_unique + idx * D + c0, v);
+    }
+  }
+}
+
+// MAX backward: route each pooled-gradient element to the winning occurrence.
+// grad_unique is zero-filled by the caller. One thread per (segment, column).
+template <typename TG, typename TOut, bool ATOMIC>
+__global__ void __launch_bounds__(kBlock)
+seg_max_bwd_kernel(const TG* __restrict__ grad_out, const int32_t* __restrict__ argmax,
+                   TOut* __restrict__ grad_unique, SegArgs a) {
+  const int64_t total = a.S * a.D;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < total; e += stride) {
+    const int32_t r = argmax[e];
+    if (r < 0) continue;
+    if (static_cast<int64_t>(r) >= a.B) {
+      raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      continue;
+    }
+    const int d = static_cast<int>(e % a.D);
+    int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+    if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+      raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      continue;
+    }
+    const float g = to_float(grad_out[e]);
+    if constexpr (ATOMIC) {
+      unsafeAtomicAdd(reinterpret_cast<float*>(grad_unique) + idx * a.D + d, g);
+    } else {
+      grad_unique[idx * a.D + d] = from_float<TOut>(g);
+    }
+  }
+}
+
+// ------------------------------------------------------------ host dispatch
+// Team size: enough row groups to cover about half the average segment, so that
+// each group still has a few rows to pipeline.
+int pick_team_log2(int64_t B, int64_t S, int lpr_log2) {
+  int64_t avg = S > 0 ? B / S : 1;
+  int rows_log2 = 0;
+  while ((int64_t(2) << rows_log2) <= avg / 2 && rows_log2 + lpr_log2 < 6) ++rows_log2;
+  return lpr_log2 + rows_log2;
+}
+
+template <typename F>
+int dispatch_vec(int vec, F&& f) {
+  switch (vec) {
+    case 8: return f(std::integral_constant<int, 8>{});
+    case 4: return f(std::integral_constant<int, 4>{});
+    case 2: return f(std::integral_constant<int, 2>{});
+    case 1: return f(std::integral_constant<int, 1>{});
+    default: return fail(RECIS_ERR_ARG, "unsupported vector width %d", vec);
+  }
+}
+
+// Calls f(TIn tag, TOut tag) for the supported (in, out) storage pairs:
+// same type, or any type widened to fp32.
+template <typename F>
+int dispatch_types(int in_dt, int out_dt, F&& f) {
+  if (in_dt == RECIS_F32 && out_dt == RECIS_F32) return f(float{}, float{});
+  if (in_dt == RECIS_BF16 && out_dt == RECIS_BF16) return f(bf16_t{}, bf16_t{});
+  if (in_dt == RECIS_BF16 && out_dt == RECIS_F32) return f(bf16_t{}, float{});
+  if (in_dt == RECIS_F16 && out_dt == RECIS_F16) return f(f16_t{}, f16_t{});
+  if (in_dt == RECIS_F16 && out_dt == RECIS_F32) return f(f16_t{}, float{});
+  if (in_dt == RECIS_F32 && out_dt == RECIS_BF16) return f(float{}, bf16_t{});
+  if (in_dt == RECIS_F32 && out_dt == RECIS_F16) return f(float{}, f16_t{});
+  return fail(RECIS_ERR_ARG, "unsupported dtype pair (in=%d, out=%d)", in_dt, out_dt);
+}
+
+int check_common(const void* offsets, int64_t B, int64_t U, int64_t S, int64_t D,
+                 int mode, int wdt, const void* weight) {
+  RECIS_REQUIRE(B >= 0 && U >= 0 && S >= 0, "negative size (B=%lld U=%lld S=%lld)",
+                (long long)B, (long long)U, (long long)S);
+  RECIS_REQUIRE(D >= 1 && D <= (1 << 20), "embedding dim %lld out of range", (long long)D);
+  RECIS_REQUIRE(offsets != nullptr, "offsets must not be NULL");
+  RECIS_REQUIRE(mode >= RECIS_SUM && mode <= RECIS_MAX, "invalid mode %d", mode);
+  RECIS_REQUIRE(weight == nullptr || dtype_size(wdt) > 0, "invalid weight dtype %d", wdt);
+  RECIS_REQUIRE(B < (int64_t(1) << 31) || mode != RECIS_MAX,
+                "MAX combiner supports fewer than 2^31 occurrences");
+  return RECIS_OK;
+}
+
+}  // namespace
+}  // namespace recis_hip
+
+using namespace recis_hip;
+
+extern "C" int recis_segment_reduce_forward(
+    const void* unique_emb, int emb_dtype, const void* weight, int weight_dtype,
+    const void* reverse_indices, int rev_is64, const void* offsets, int off_is64,
+    void* out, int out_dtype, int32_t* argmax_out, int64_t B, int64_t U, int64_t S,
+    int64_t D, int mode, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = check_common(offsets, B, U, S, D, mode, weight_dtype, weight)) return rc;
+  RECIS_REQUIRE(reverse_indices != nullptr || U == B,
+                "reverse_indices == NULL (identity) needs U == B (U=%lld, B=%lld)",
+                (long long)U, (long long)B);
+  const int64_t out_rows = (mode == RECIS_TILE) ? B : S;
+  if (out_rows == 0) return RECIS_OK;
+  RECIS_REQUIRE(out != nullptr, "out must not be NULL");
+  RECIS_REQUIRE(unique_emb != nullptr || U == 0, "unique_emb must not be NULL");
+  const int in_sz = dtype_size(emb_dtype), out_sz = dtype_size(out_dtype);
+  RECIS_REQUIRE(in_sz && out_sz, "invalid dtype (emb=%d out=%d)", emb_dtype, out_dtype);
+
+  int* err = device_error_word(current_device());
+  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+
+  // vector width in elements, limited by both row widths and pointer alignment
+  const int vb_in = pick_vec_bytes(D * in_sz, reinterpret_cast<uintptr_t>(unique_emb));
+  const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(out));
+  int vec = std::min(vb_in / in_sz, vb_out / out_sz);
+  if (vec < 1) vec = 1;
+  if (mode == RECIS_MAX && argmax_out) vec = std::min(vec, 4);
+  RowGeom geom;
+  geom.vec = vec;
+  geom.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
+
+  SegArgs a;
+  a.weight = weight;
+  a.rev = reverse_indices;
+  a.offs = offsets;
+  a.B = B;
+  a.U = U;
+  a.S = S;
+  a.D = static_cast<int>(D);
+  a.wdt = weight_dtype;
+  a.rev64 = rev_is64;
+  a.off64 = off_is64;
+  a.lpr_log2 = geom.lpr_log2;
+  a.team_log2 = pick_team_log2(B, S, geom.lpr_log2);
+  a.mean = (mode == RECIS_MEAN);
+  a.err = err;
+
+  return dispatch_types(emb_dtype, out_dtype, [&](auto tin, auto tout) {
+    using TIn = decltype(tin);
+    using TOut = decltype(tout);
+    return dispatch_vec(vec, [&](auto vtag) {
+      constexpr int VEC = decltype(vtag)::value;
+      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 16) {
+        return fail(RECIS_ERR_ARG, "internal: vector too wide");
+      } else {
+        if (mode == RECIS_TILE) {
+          const int rows_per_block = kBlock >> a.lpr_log2;
+          const int64_t grid = (B + rows_per_block - 1) / rows_per_block;
+          seg_tile_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+              static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), a);
+        } else {
+          const int teams_per_block = kBlock >> a.team_log2;
+          const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
+          if (mode == RECIS_MAX) {
+            seg_max_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), argmax_out, a);
+          } else {
+            seg_pool_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), a);
+          }
+        }
+        RECIS_LAUNCH_CHECK();
+        return RECIS_OK;
+      }
+    });
+  });
+}
+
+extern "C" int recis_segment_reduce_backward(
+    const void* grad_out, int grad_dtype, const void* weight, int weight_dtype,
+    const void* reverse_indices, int rev_is64, const void* offsets, int off_is64,
+    const int32_t* argmax, void* grad_unique, int out_dtype, int64_t B, int64_t U,
+    int64_t S, int64_t D, int mode, int flags, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = check_common(offsets, B, U, S, D, mode, weight_dtype, weight)) return rc;
+  RECIS_REQUIRE(reverse_indices != nullptr || U == B,
+                "reverse_indices == NULL (identity) needs U == B (U=%lld, B=%lld)",
+                (long long)U, (long long)B);
+  if (U == 0) return RECIS_OK;
+  RECIS_REQUIRE(grad_unique != nullptr, "grad_unique must not be NULL");
+  const int64_t in_rows = (mode == RECIS_TILE) ? B : S;
+  RECIS_REQUIRE(grad_out != nullptr || in_rows == 0, "grad_out must not be NULL");
+  RECIS_REQUIRE(mode != RECIS_MAX || argmax != nullptr || S == 0,
+                "MAX backward needs the argmax written by the forward");
+  const int in_sz = dtype_size(grad_dtype), out_sz = dtype_size(out_dtype);
+  RECIS_REQUIRE(in_sz && out_sz, "invalid dtype (grad=%d out=%d)", grad_dtype, out_dtype);
+  const bool unique = (flags & RECIS_FLAG_REV_UNIQUE) || reverse_indices == nullptr;
+  RECIS_REQUIRE(unique || out_dtype == RECIS_F32,
+                "accumulating duplicates needs an fp32 grad_unique (got dtype %d); "
+                "pass RECIS_FLAG_REV_UNIQUE if reverse_indices has no duplicates",
+                out_dtype);
+
+  int* err = device_error_word(current_device());
+  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+
+  const int vb_in = pick_vec_bytes(D * in_sz, reinterpret_cast<uintptr_t>(grad_out));
+  const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(grad_unique));
+  int vec = std::min(vb_in / in_sz, vb_out / out_sz);
+  if (vec < 1) vec = 1;
+  const int lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
+
+  SegArgs a;
+  a.weight = weight;
+  a.rev = reverse_indices;
+  a.offs = offsets;
+  a.B = B;
+  a.U = U;
+  a.S = S;
+  a.D = static_cast<int>(D);
+  a.wdt = weight_dtype;
+  a.rev64 = rev_is64;
+  a.off64 = off_is64;
+  a.lpr_log2 = lpr_log2;
+  a.team_log2 = pick_team_log2(B, S, lpr_log2);
+  a.mean = (mode == RECIS_MEAN);
+  a.err = err;
+
+  // Rows no occurrence maps to must read zero. With a promised bijection
+  // (unique and U == B) every row is reached through its occurrence, so only
+  // occurrences outside the offsets range need clearing; otherwise clear all.
+  const bool bijection = unique && U == B && mode != RECIS_MAX;
+
+  return dispatch_types(grad_dtype, out_dtype, [&](auto tin, auto tout) {
+    using TG = decltype(tin);
+    using TOut = decltype(tout);
+    return dispatch_vec(vec, [&](auto vtag) {
+      constexpr int VEC = decltype(vtag)::value;
+      if constexpr (VEC * sizeof(TG) > 16 || VEC * sizeof(TOut) > 16) {
+        return fail(RECIS_ERR_ARG, "internal: vector too wide");
+      } else {
+        if (!bijection) {
+          const int64_t n_packs = U * D / VEC;  // D % VEC == 0 by construction
+          int64_t grid = std::min<int64_t>((n_packs + kBlock - 1) / kBlock, 256 * 32);
+          if (grid < 1) grid = 1;
+          fill_zero_rows_kernel<TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+              static_cast<TOut*>(grad_unique), n_packs);
+          RECIS_LAUNCH_CHECK();
+        } else if (mode != RECIS_TILE) {
+          seg_bwd_zero_uncovered_kernel<TOut, VEC><<<dim3(64), dim3(kBlock), 0, stream>>>(
+              static_cast<TOut*>(grad_unique), a);
+          RECIS_LAUNCH_CHECK();
+        }
+        if (mode == RECIS_MAX) {
+          const int64_t total = S * D;
+          if (total > 0) {
+            int64_t grid = std::min<int64_t>((total + kBlock - 1) / kBlock, 256 * 64);
+            if (unique)
+              seg_max_bwd_kernel<TG, TOut, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                  static_cast<const TG*>(grad_out), argmax, static_cast<TOut*>(grad_unique), a);
+            else
+              seg_max_bwd_kernel<TG, TOut, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                  static_cast<const TG*>(grad_out), argmax, static_cast<TOut*>(grad_unique), a);
+            RECIS_LAUNCH_CHECK();
+          }
+        } else if (mode == RECIS_TILE) {
+          if (B > 0) {
+            const int rows_per_block = kBlock >> a.lpr_log2;
+            const int64_t grid = (B + rows_per_block - 1) / rows_per_block;
+            if (unique)
+              seg_tile_bwd_kernel<TG, TOut, VEC, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                  static_cast<const TG*>(grad_out), static_cast<TOut*>(grad_unique), a);
+            else
+              seg_tile_bwd_kernel<TG, TOut, VEC, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                  static_cast<const TG*>(grad_out), static_cast<TOut*>(grad_unique), a);
+            RECIS_LAUNCH_CHECK();
+          }
+        } else if (S > 0) {
+          const int teams_per_block = kBlock >> a.team_log2;
+          const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
+          if (unique)
+            seg_pool_bwd_kernel<TG, TOut, VEC, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                static_cast<const TG*>(grad_out), static_cast<TOut*>(grad_unique), a);
+          else
+            seg_pool_bwd_kernel<TG, TOut, VEC, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                static_cast<const TG*>(grad_out), static_cast<TOut*>(grad_unique), a);
+          RECIS_LAUNCH_CHECK();
+        }
+        return RECIS_OK;
+      }
+    });
+  });
+}

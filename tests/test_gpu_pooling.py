@@ -1,0 +1,227 @@
+"""Parity of the HIP pooling kernels (through the C ABI) with the CPU oracle.
+
+fp32 tolerance: rtol 1e-5 and atol 1e-6 per unit of summed magnitude, i.e.
+|gpu - exact| <= 1e-5 * |exact| + 1e-6 * max(1, sum_i |w_i * x_i|), where
+`exact` is the oracle's double-precision sum: any two fp32 summation orders of a
+200-term segment differ by more than a flat 1e-6. bf16 storage: rtol 1e-2.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import ragged_offsets
+from recis_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+
+
+def _dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def _assert_pool_close(got, emb, w, rev, off, mode, rtol=RTOL, atol=ATOL):
+    exact, mag = oracle.segment_reduce_forward_f64(emb, w, rev, off, mode == "mean")
+    err = np.abs(got.astype(np.float64) - exact)
+    bound = rtol * np.abs(exact) + atol * np.maximum(1.0, mag)
+    bad = err > bound
+    assert not bad.any(), "max excess %g at %s" % ((err - bound).max(), np.argwhere(bad)[:3])
+
+
+def _case(rng, S, U, D, lo, hi, empty_frac=0.1, dup=True):
+    off = ragged_offsets(rng, S, lo, hi, empty_frac)
+    B = int(off[-1])
+    rev = rng.integers(0, U, size=B) if dup else rng.permutation(max(U, B))[:B]
+    emb = rng.standard_normal((U, D)).astype(np.float32)
+    w = rng.standard_normal(B).astype(np.float32)
+    return off, B, rev, emb, w
+
+
+@pytest.mark.parametrize("D", [1, 3, 4, 6, 16, 32, 48, 64, 128, 260, 512])
+@pytest.mark.parametrize("mode", ["sum", "mean"])
+def test_forward_fp32_dims(rng, D, mode):
+    off, B, rev, emb, w = _case(rng, 301, 97, D, 0, 40)
+    for use_w in (True, False):
+        got = ops.segment_reduce_forward(_dev(emb), _dev(w) if use_w else None, _dev(rev),
+                                         _dev(off), mode).cpu().numpy()
+        _assert_pool_close(got, emb, w if use_w else None, rev, off, mode)
+
+
+@pytest.mark.parametrize("lo,hi", [(1, 1), (0, 3), (1, 20), (150, 200)])
+@pytest.mark.parametrize("off_dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("rev_dtype", [np.int32, np.int64])
+def test_forward_lengths_and_index_types(rng, lo, hi, off_dtype, rev_dtype):
+    off, B, rev, emb, w = _case(rng, 513, 200, 64, lo, hi, empty_frac=0.0)
+    got = ops.segment_reduce_forward(_dev(emb), _dev(w), _dev(rev.astype(rev_dtype)),
+                                     _dev(off.astype(off_dtype)), "sum").cpu().numpy()
+    _assert_pool_close(got, emb, w, rev, off, "sum")
+
+
+def test_forward_identity_rev(rng):
+    off = ragged_offsets(rng, 1000, 1, 60)
+    B = int(off[-1])
+    emb = rng.standard_normal((B, 64)).astype(np.float32)
+    got = ops.segment_reduce_forward(_dev(emb), None, None, _dev(off.astype(np.int32)),
+                                     "mean").cpu().numpy()
+    _assert_pool_close(got, emb, None, np.arange(B), off, "mean")
+
+
+def test_forward_empty_inputs():
+    emb = torch.zeros((0, 16), device="cuda")
+    out = ops.segment_reduce_forward(emb, None, torch.zeros(0, dtype=torch.int64, device="cuda"),
+                                     torch.zeros(1, dtype=torch.int64, device="cuda"), "sum")
+    assert out.shape == (0, 16)
+    emb = torch.randn((5, 16), device="cuda")
+    off = torch.zeros(8, dtype=torch.int64, device="cuda")  # 7 empty segments
+    out = ops.segment_reduce_forward(emb, None, torch.zeros(0, dtype=torch.int64, device="cuda"),
+                                     off, "mean")
+    assert out.shape == (7, 16) and float(out.abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean", "tile"])
+@pytest.mark.parametrize("D", [4, 16, 64, 100])
+def test_tile_and_backward_fp32(rng, mode, D):
+    off, B, rev, emb, w = _case(rng, 211, 150, D, 0, 30)
+    B2 = B + 5
+    rev = np.concatenate([rev, rng.integers(0, 150, size=5)])  # occurrences after the last offset
+    w = np.concatenate([w, np.ones(5, np.float32)])
+    if mode == "tile":
+        got = ops.segment_reduce_forward(_dev(emb), _dev(w), _dev(rev), _dev(off), mode).cpu().numpy()
+        exp = oracle.segment_reduce_forward(emb, w, rev, off, mode)
+        np.testing.assert_allclose(got, exp, rtol=RTOL, atol=ATOL)
+    rows = B2 if mode == "tile" else 211
+    g = rng.standard_normal((rows, D)).astype(np.float32)
+    got = ops.segment_reduce_backward(_dev(g), _dev(w), _dev(rev), _dev(off), 150, mode).cpu().numpy()
+    exp = oracle.segment_reduce_backward(g, w, rev, off, 150, mode)
+    # each gradient row sums up to ~B/U * 30 terms of magnitude ~|g||w|
+    np.testing.assert_allclose(got, exp, rtol=1e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean", "tile"])
+def test_backward_unique_rev_plain_stores(rng, mode):
+    S, D = 333, 64
+    off = ragged_offsets(rng, S, 0, 25)
+    off[1:] += 4  # leading occurrences no segment covers
+    B = int(off[-1]) + 7
+    for U in (B, B + 50):
+        rev = rng.permutation(U)[:B]
+        w = rng.standard_normal(B).astype(np.float32)
+        g = rng.standard_normal((B if mode == "tile" else S, D)).astype(np.float32)
+        pre = torch.full((U, D), 7.0, device="cuda")  # stale memory must not leak through
+        del pre
+        got = ops.segment_reduce_backward(_dev(g), _dev(w), _dev(rev), _dev(off), U, mode,
+                                          rev_unique=True).cpu().numpy()
+        exp = oracle.segment_reduce_backward(g, w, rev, off, U, mode)
+        np.testing.assert_allclose(got, exp, rtol=1e-6, atol=1e-6)
+    # identity rev (rows materialised per occurrence)
+    g = rng.standard_normal((B if mode == "tile" else S, D)).astype(np.float32)
+    got = ops.segment_reduce_backward(_dev(g), _dev(w), None, _dev(off), B, mode).cpu().numpy()
+    exp = oracle.segment_reduce_backward(g, w, np.arange(B), off, B, mode)
+    np.testing.assert_allclose(got, exp, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("D", [2, 16, 64, 72])
+def test_max_forward_backward(rng, D):
+    S, U = 257, 120
+    off = ragged_offsets(rng, S, 0, 33, empty_frac=0.15)
+    B = int(off[-1])
+    rev = rng.integers(0, U, size=B)
+    emb = np.round(rng.standard_normal((U, D)) * 3).astype(np.float32)  # ties on purpose
+    out, arg = ops.segment_reduce_forward(_dev(emb), None, _dev(rev), _dev(off), "max",
+                                          return_argmax=True)
+    eo, ea = oracle.segment_max_forward(emb, rev, off)
+    np.testing.assert_array_equal(out.cpu().numpy(), eo)
+    np.testing.assert_array_equal(arg.cpu().numpy(), ea)
+    g = rng.standard_normal((S, D)).astype(np.float32)
+    got = ops.segment_reduce_backward(_dev(g), None, _dev(rev), _dev(off), U, "max", argmax=arg)
+    exp = oracle.segment_max_backward(g, ea, rev, U)
+    np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [8, 128, 136])
+def test_half_storage_fp32_accumulate(rng, dtype, D):
+    off, B, rev, emb, w = _case(rng, 199, 300, D, 0, 50)
+    emb_t = torch.from_numpy(emb).to(dtype)
+    emb_q = emb_t.float().numpy()  # what the rows really hold
+    for out_dtype in (torch.float32, dtype):
+        got = ops.segment_reduce_forward(emb_t.cuda(), _dev(w), _dev(rev), _dev(off), "mean",
+                                         out_dtype=out_dtype)
+        assert got.dtype == out_dtype
+        if out_dtype == torch.float32:  # fp32 accumulation: as tight as the fp32 path
+            _assert_pool_close(got.cpu().numpy(), emb_q, w, rev, off, "mean")
+        else:
+            _assert_pool_close(got.float().cpu().numpy(), emb_q, w, rev, off, "mean",
+                               rtol=1e-2, atol=1e-2)
+    g = rng.standard_normal((199, D)).astype(np.float32)
+    g_t = torch.from_numpy(g).to(dtype)
+    got = ops.segment_reduce_backward(g_t.cuda(), _dev(w), _dev(rev), _dev(off), 300, "sum",
+                                      out_dtype=torch.float32).cpu().numpy()
+    exp = oracle.segment_reduce_backward(g_t.float().numpy(), w, rev, off, 300, "sum")
+    np.testing.assert_allclose(got, exp, rtol=1e-5, atol=2e-5)
+
+
+def test_out_of_range_index_is_reported_not_faulting(rng):
+    from recis_amd import _lib
+
+    _lib.poll_device_errors()
+    emb = torch.randn((10, 16), device="cuda")
+    rev = torch.tensor([0, 3, 99, 2], device="cuda")  # 99 >= U
+    off = torch.tensor([0, 2, 4], device="cuda")
+    out = ops.segment_reduce_forward(emb, None, rev, off, "sum")
+    assert _lib.poll_device_errors() & _lib.DEVERR_INDEX_RANGE
+    torch.testing.assert_close(out[0], emb[0] + emb[3])
+    torch.testing.assert_close(out[1], emb[2])
+    assert _lib.poll_device_errors() == 0
+
+
+def test_argument_errors():
+    emb = torch.randn((10, 16), device="cuda")
+    off = torch.tensor([0, 2], device="cuda")
+    rev = torch.tensor([0, 1], device="cuda")
+    with pytest.raises(ValueError):
+        ops.segment_reduce_forward(emb, None, rev, off, "median")
+    with pytest.raises(TypeError):
+        ops.segment_reduce_forward(emb.double(), None, rev, off, "sum")
+    with pytest.raises(TypeError):
+        ops.segment_reduce_forward(emb, None, rev.float(), off, "sum")
+    with pytest.raises(RuntimeError):  # CPU tensors are refused, there is no CPU path
+        ops.segment_reduce_forward(emb.cpu(), None, rev.cpu(), off.cpu(), "sum")
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean"])
+def test_config2_shape_properties(mode):
+    """BASELINE config 2 at full size: linearity and a sum-of-sums checksum.
+
+    32 x 16384 segments, Poisson(30) lengths clipped to [1, 200], D = 64 fp32,
+    rows materialised per occurrence, int32 offsets."""
+    import workloads
+
+    c = workloads.config2(device="cuda")
+    emb, off, S = c["values"], c["offsets"], c["num_segments"]
+    out = ops.segment_reduce_forward(emb, None, None, off, mode)
+    assert out.shape == (S, 64)
+    # linearity: pool(2a + b) == 2 pool(a) + pool(b)
+    b = torch.roll(emb, 1, 0)
+    lin = ops.segment_reduce_forward(2 * emb + b, None, None, off, mode)
+    ref = 2 * out + ops.segment_reduce_forward(b, None, None, off, mode)
+    torch.testing.assert_close(lin, ref, rtol=1e-4, atol=1e-4)
+    if mode == "sum":  # checksum of checksums, in double
+        total = out.double().sum(0)
+        torch.testing.assert_close(total, emb.double().sum(0), rtol=1e-6, atol=1e-3)
+    # a slice of it against the oracle
+    k = 4096
+    nb = int(off[k])
+    got = out[:k].cpu().numpy()
+    _assert_pool_close(got, emb[:nb].cpu().numpy(), None, np.arange(nb), off[:k + 1].cpu().numpy(), mode)
+    # backward is the transpose: <pool(x), g> == <x, pool^T(g)>
+    g = torch.randn_like(out)
+    gx = ops.segment_reduce_backward(g, None, None, off, emb.shape[0], mode)
+    lhs = (out.double() * g.double()).sum()
+    rhs = (emb.double() * gx.double()).sum()
+    torch.testing.assert_close(lhs, rhs, rtol=1e-6, atol=1e-2)

@@ -1,0 +1,52 @@
+"""Seeded synthetic inputs for the BASELINE configurations.
+
+Used by ``bench.py`` and the tests; every generator is deterministic in its
+seed (numpy ``PCG64``) and returns torch tensors on the requested device.
+"""
+import numpy as np
+import torch
+
+
+def _rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def bounded_zipf(rng, n, alpha, num_keys):
+    """n ranks in [0, num_keys) with P(rank r) proportional to (r+1)^-alpha.
+
+    Inverse-CDF sampling on the exact cumulative table (numpy's ``zipf`` is
+    unbounded and only defined for alpha > 1)."""
+    p = np.arange(1, num_keys + 1, dtype=np.float64) ** (-alpha)
+    cdf = np.cumsum(p)
+    cdf /= cdf[-1]
+    return np.minimum(np.searchsorted(cdf, rng.random(n), side="left"), num_keys - 1).astype(np.int64)
+
+
+def splitmix64(x):
+    """Bijective 64-bit mix (numpy uint64 arrays), used to turn ranks into random keys."""
+    x = (x.astype(np.uint64) + np.uint64(0x9E3779B97F4A7C15))
+    x = (x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    x = (x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return x ^ (x >> np.uint64(31))
+
+
+def config2(device="cuda", seed=1, features=32, batch=16384, dim=64, mean_len=30, max_len=200):
+    """Standalone ragged segment_reduce on pre-materialised rows (BASELINE config 2)."""
+    rng = _rng(seed)
+    S = features * batch
+    lens = np.clip(rng.poisson(mean_len, size=S), 1, max_len).astype(np.int64)
+    off = np.zeros(S + 1, np.int64)
+    np.cumsum(lens, out=off[1:])
+    N = int(off[-1])
+    g = torch.Generator(device=device).manual_seed(seed)
+    values = torch.randn((N, dim), dtype=torch.float32, device=device, generator=g)
+    grad = torch.randn((S, dim), dtype=torch.float32, device=device, generator=g)
+    return {
+        "values": values,
+        "grad": grad,
+        "offsets": torch.from_numpy(off.astype(np.int32)).to(device),
+        "reverse_indices": None,
+        "num_segments": S,
+        "num_ids": N,
+        "dim": dim,
+    }
