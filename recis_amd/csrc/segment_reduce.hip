@@ -137,6 +137,21 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
 }
 
 // MAX combiner: element-wise maximum and the occurrence that produced it.
+// Value and occurrence travel as one 64-bit key: the high word is the float
+// mapped to an order-preserving unsigned integer (any NaN maps to the top, so it
+// propagates), the low word is 0xFFFFFFFF - occurrence, so that among equal
+// values the earliest occurrence is the largest key. Key 0 = "no row yet".
+__device__ __forceinline__ uint64_t max_key(float v, int64_t r) {
+  uint32_t b = (v == 0.f) ? 0u : __float_as_uint(v);  // -0 and +0 tie
+  uint32_t m = (v != v) ? 0xFFFFFFFFu : ((b & 0x80000000u) ? ~b : (b | 0x80000000u));
+  return (static_cast<uint64_t>(m) << 32) | (0xFFFFFFFFu - static_cast<uint32_t>(r));
+}
+__device__ __forceinline__ float max_key_value(uint64_t k) {
+  uint32_t m = static_cast<uint32_t>(k >> 32);
+  if (m == 0xFFFFFFFFu) return __uint_as_float(0x7FC00000u);
+  return __uint_as_float((m & 0x80000000u) ? (m & 0x7FFFFFFFu) : ~m);
+}
+
 template <typename TIn, typename TOut, int VEC>
 __global__ void __launch_bounds__(kBlock)
 seg_max_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out,
@@ -153,13 +168,9 @@ seg_max_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out,
   const int D = a.D;
 
   for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
-    float best[VEC];
-    int32_t arg[VEC];
+    uint64_t key[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      best[j] = -INFINITY;
-      arg[j] = -1;
-    }
+    for (int j = 0; j < VEC; ++j) key[j] = 0;
     for (int64_t r = start + rg; r < end; r += step) {
       int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
       if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
@@ -170,45 +181,29 @@ seg_max_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out,
       load_pack<TIn, VEC>(emb + idx * D + c0, v);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        // strict > keeps the earliest occurrence within this row group;
-        // a NaN is taken once and then sticks (like torch's amax)
-        if (arg[j] < 0 || v[j] > best[j] || (v[j] != v[j] && best[j] == best[j])) {
-          best[j] = v[j];
-          arg[j] = static_cast<int32_t>(r);
-        }
+        uint64_t k = max_key(v[j], r);
+        key[j] = k > key[j] ? k : key[j];
       }
     }
     for (int off = 1 << a.lpr_log2; off < (1 << a.team_log2); off <<= 1) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        float ob = __shfl_xor(best[j], off, kWave);
-        int32_t oa = __shfl_xor(arg[j], off, kWave);
-        bool mine_nan = best[j] != best[j];
-        bool other_nan = ob != ob;
-        bool take;
-        if (oa < 0) {
-          take = false;
-        } else if (arg[j] < 0) {
-          take = true;
-        } else if (mine_nan || other_nan) {
-          take = other_nan && (!mine_nan || oa < arg[j]);
-        } else {
-          take = (ob > best[j]) || (ob == best[j] && oa < arg[j]);
-        }
-        if (take) {
-          best[j] = ob;
-          arg[j] = oa;
-        }
+        uint32_t lo = __shfl_xor(static_cast<uint32_t>(key[j]), off, kWave);
+        uint32_t hi = __shfl_xor(static_cast<uint32_t>(key[j] >> 32), off, kWave);
+        uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
+        key[j] = other > key[j] ? other : key[j];
       }
     }
     if (rg == 0) {
+      float best[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        if (arg[j] < 0) best[j] = 0.f;
+      for (int j = 0; j < VEC; ++j) best[j] = key[j] ? max_key_value(key[j]) : 0.f;
       store_pack<TOut, VEC>(out + s * D + c0, best);
       if (argmax) {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) argmax[s * D + c0 + j] = arg[j];
+        for (int j = 0; j < VEC; ++j)
+          argmax[s * D + c0 + j] =
+              key[j] ? static_cast<int32_t>(0xFFFFFFFFu - static_cast<uint32_t>(key[j])) : -1;
       }
     }
   }

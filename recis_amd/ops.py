@@ -25,6 +25,15 @@ def _contig(t):
     return t if t is None or t.is_contiguous() else t.contiguous()
 
 
+def _rev_ptr(rev, other):
+    """NULL means "identity" to the library; an empty (but given) index tensor has
+    a NULL data pointer too, so hand over another valid pointer: with zero
+    occurrences it is never dereferenced."""
+    if rev is None:
+        return ptr(None)
+    return ptr(rev) if rev.numel() else ptr(other)
+
+
 # --------------------------------------------------------------------- pooling
 def segment_reduce_forward(unique_emb, weight, reverse_indices, offsets, mode, *,
                            out_dtype=None, return_argmax=False):
@@ -50,7 +59,7 @@ def segment_reduce_forward(unique_emb, weight, reverse_indices, offsets, mode, *
     check(lib().recis_segment_reduce_forward(
         ptr(unique_emb), dtype_code(unique_emb.dtype),
         ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
-        ptr(reverse_indices),
+        _rev_ptr(reverse_indices, offsets),
         _index_kind(reverse_indices, "reverse_indices") if reverse_indices is not None else 1,
         ptr(offsets), _index_kind(offsets, "offsets"),
         ptr(out), dtype_code(out_dtype), ptr(argmax),
@@ -85,7 +94,7 @@ def segment_reduce_backward(grad_output, weight, reverse_indices, offsets, uniqu
     check(lib().recis_segment_reduce_backward(
         ptr(grad_output), dtype_code(grad_output.dtype),
         ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
-        ptr(reverse_indices),
+        _rev_ptr(reverse_indices, offsets),
         _index_kind(reverse_indices, "reverse_indices") if reverse_indices is not None else 1,
         ptr(offsets), _index_kind(offsets, "offsets"), ptr(argmax),
         ptr(out), dtype_code(work_dtype), i64(B), i64(U), i64(S), i64(D), _lib.MODES[mode],
