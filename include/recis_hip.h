@@ -109,6 +109,238 @@ int recis_segment_reduce_backward(const void* grad_out, int grad_dtype,
                                   int out_dtype, int64_t B, int64_t U, int64_t S,
                                   int64_t D, int mode, int flags, void* stream);
 
+/*
+ * Sparse-mode pooling (short segments addressed by segment id).
+ * Replaces: segment_sum_cuda / segment_mean_cuda, csrc/ops/segment_ops_kernel.cu:192-291
+ *           (ops csrc/ops/segment_ops.cc:6-52).
+ *   segment_sum:  out[seg[i]] += data[indices[i]] * w[i]; out [num_segments, D] fp32,
+ *                 zeroed by the call. use_weight == 0 broadcasts weight[0]
+ *                 (weight == NULL means 1).
+ *   segment_mean_weight: weight_sum[s] = sum of w_i with seg_i == s;
+ *                 weight_norm[i] = w_i / weight_sum[seg_i]; an out-of-range
+ *                 segment id keeps the raw weight.
+ */
+int recis_segment_sum(const void* data, int dtype, int64_t data_rows, const void* weight,
+                      int weight_dtype, int use_weight, const void* indices,
+                      const void* segment_ids, int idx_is64, float* out, int64_t n,
+                      int64_t num_segments, int64_t D, void* stream);
+int recis_segment_mean_weight(const float* weight, int use_weight, const void* segment_ids,
+                              int idx_is64, float* weight_sum, float* weight_norm, int64_t n,
+                              int64_t num_segments, void* stream);
+
+/*
+ * out[j] = s with offsets[s] <= j < offsets[s+1], for j in [0, total); out has the
+ * integer type of offsets. `total` = offsets[S] is supplied by the caller.
+ * Replaces: gen_segment_indices_by_offset, csrc/ops/embedding_segment_reduce_kernel.cu:395-423.
+ */
+int recis_gen_segment_indices(const void* offsets, int off_is64, int64_t S, void* out,
+                              int64_t total, void* stream);
+
+/*
+ * Unpooled gather padded / truncated to seq[f] rows per sample, several features
+ * per call; weights play no part.
+ * Replaces: ragged_tile / ragged_tile_back, csrc/ops/ragged_tile_kernel.cu:214-280.
+ *   batch, seq     host arrays [n_features]
+ *   value          [n_values] row of `table` per occurrence (int32/int64)
+ *   offset         [sum(batch) + 1] merged sample boundaries into value
+ *   table          [table_rows, D];  out [sum(batch*seq), D]   (dtype)
+ *   backward: dy [sum(batch*seq), D] (dtype) -> d_table [table_rows, D] fp32,
+ *   zeroed and accumulated (fp32 atomics) by the call.
+ */
+int recis_ragged_tile(const int64_t* batch, const int64_t* seq, int64_t n_features,
+                      const void* value, int value_is64, int64_t n_values, const void* offset,
+                      int off_is64, const void* table, int64_t table_rows, int dtype, void* out,
+                      int64_t D, void* stream);
+int recis_ragged_tile_back(const int64_t* batch, const int64_t* seq, int64_t n_features,
+                           const void* value, int value_is64, int64_t n_values,
+                           const void* offset, int off_is64, const void* dy, int dtype,
+                           float* d_table, int64_t table_rows, int64_t D, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * IDMap: 64-bit key -> row index, with the row-index allocator
+ * ------------------------------------------------------------------------- */
+
+/*
+ * Opaque device-resident map. Replaces GpuIdMap (csrc/embedding/gpu_id_map.h:9-33,
+ * gpu_id_map.cu:9-121) together with its cuco::dynamic_map and its IdAllocator
+ * (csrc/embedding/id_allocator.cc:8-64). Keys -1 and -2 are reserved, as in the
+ * reference (gpu_id_map.h:11-16). An object belongs to the device that was
+ * current at creation and must be used from one stream at a time.
+ */
+typedef struct recis_idmap recis_idmap;
+
+/* reserve_keys: number of keys the table should hold without a rebuild. */
+int recis_idmap_create(int64_t reserve_keys, recis_idmap** out);
+int recis_idmap_destroy(recis_idmap* m);
+
+/*
+ * Find-or-insert (GpuIdMap::Lookup, gpu_id_map.cu:19-45). index_out[i] = row of
+ * ids[i]; keys not present are inserted and take row indices in input order by
+ * the rule of IdAllocator::GenIds (csrc/ops/hashtable_ops.cc:15-27): with n
+ * missing keys, the k-th takes free_list[free - n + k] if that position is >= 0,
+ * else the fresh index cur - (free - n + k + 1). A key repeated inside one call
+ * gets one row. No host synchronisation unless the table must be rebuilt.
+ */
+int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* index_out,
+                       void* stream);
+/* GpuIdMap::LookupReadOnly (gpu_id_map.cu:47-62): -1 for a missing key. */
+int recis_idmap_lookup_readonly(recis_idmap* m, const int64_t* ids, int64_t n,
+                                int64_t* index_out, void* stream);
+/* GpuIdMap::DeleteIds (gpu_id_map.cu:84-96): erases ids, appends `index` (all n
+ * entries, in order) to the free list (IdAllocator::FreeIds). */
+int recis_idmap_erase(recis_idmap* m, const int64_t* ids, const int64_t* index, int64_t n,
+                      void* stream);
+/* Synchronises `stream`. live = keys present, id_num = allocator high-water mark
+ * (IdMap::GetIdNum, id_map.h:29), free_size = free-list length. Any may be NULL. */
+int recis_idmap_stats(recis_idmap* m, int64_t* live, int64_t* id_num, int64_t* free_size,
+                      int64_t* capacity, void* stream);
+/* GpuIdMap::SnapShot (gpu_id_map.cu:64-77): all live (key, row) pairs, unordered.
+ * Synchronises; *count = number of live pairs (only min(count, max_out) written). */
+int recis_idmap_snapshot(recis_idmap* m, int64_t* ids_out, int64_t* index_out, int64_t max_out,
+                         int64_t* count, void* stream);
+/* GpuIdMap::Clear (gpu_id_map.cu:98-103). */
+int recis_idmap_clear(recis_idmap* m, void* stream);
+/* IdMap::Reserve (not implemented for the reference GPU map, gpu_id_map.cu:105-108). */
+int recis_idmap_reserve(recis_idmap* m, int64_t n_keys, void* stream);
+
+/*
+ * Stand-alone allocator ops over a caller-held free list kept in blocks
+ * (device array of block pointers).
+ * Replace: generate_ids_cuda_op, free_ids_cuda_op, mask_key_index_cuda_op,
+ * scatter_ids_with_mask_cuda_op, csrc/ops/hashtable_ops_kernel.cu:32-173.
+ */
+int recis_generate_ids(int64_t n, const int64_t* const* free_blocks_dev, int64_t free_count,
+                       int64_t cur_count, int64_t free_block_size, int64_t* out, void* stream);
+int recis_free_ids(const int64_t* ids, int64_t n, int64_t* const* free_blocks_dev,
+                   int64_t free_count, int64_t free_block_size, void* stream);
+int recis_mask_key_index(const int64_t* keys, const uint8_t* mask, const int64_t* cumsum,
+                         int64_t n, int64_t out_size, int64_t* out_keys, int64_t* out_index,
+                         void* stream);
+int recis_scatter_ids_with_mask(int64_t* out_ids, int64_t out_size, const int64_t* in_ids,
+                                const int64_t* mask_index, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * EmbeddingBlocks: rows stored as a list of equally sized blocks
+ * ------------------------------------------------------------------------- */
+
+/*
+ * blocks_dev is a DEVICE array of n_blocks pointers to [block_size, row_bytes]
+ * arrays; row `idx` lives in block idx / block_size at row idx % block_size.
+ * Rows are moved as bytes, so any element type works. Block bases must be
+ * aligned to the largest power of two (<= 16) that divides row_bytes.
+ *
+ * Replace the device branches of csrc/ops/block_ops.cc:
+ *   recis_gather             gather_cuda              (block_ops.cc:262-268)
+ *   recis_block_gather       block_gather_cuda        (block_ops.cc:270-282, also
+ *                            block_gather_by_range when ids is offset by `beg`)
+ *   recis_block_insert       block_insert_cuda / block_insert_with_mask_cuda
+ *                            (block_ops.cc:353-360, 385-397); broadcast = emb has
+ *                            one row; mask may be NULL
+ *   recis_block_filter       block_filter_cuda        (block_ops.cc:284-293):
+ *                            mask_out[i] = slot[ids[i]] < threshold (int32/int64 slot)
+ * readonly != 0: an index equal to default_key yields a zero row.
+ */
+int recis_gather(const void* ids, int ids_is64, const void* emb, int64_t rows, void* out,
+                 int64_t n, int64_t row_bytes, void* stream);
+int recis_block_gather(const int64_t* ids, void* const* blocks_dev, int64_t n_blocks,
+                       int64_t block_size, int64_t default_key, int readonly, void* out,
+                       int64_t n, int64_t row_bytes, void* stream);
+int recis_block_insert(const int64_t* ids, const void* emb, int broadcast, const uint8_t* mask,
+                       void* const* blocks_dev, int64_t n_blocks, int64_t block_size, int64_t n,
+                       int64_t row_bytes, void* stream);
+int recis_block_filter(const int64_t* ids, void* const* blocks_dev, int64_t n_blocks,
+                       int64_t block_size, int64_t threshold, int slot_is64, uint8_t* mask_out,
+                       int64_t n, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * Fused sparse optimizer row updates
+ * ------------------------------------------------------------------------- */
+
+/*
+ * Replaces: block_apply_adamw, csrc/ops/block_apply_adamw_op.cc:114-132.
+ * beta1_t / beta2_t: device scalars holding the running powers (float, or double
+ * when beta_is_f64), advanced in place; alpha = -lr / (1 - b1_t) * sqrtf(1 - b2_t).
+ * Per element of row index[i] (weight_decay is the multiplicative factor):
+ *   w *= weight_decay; m = m*beta1 + g*(1-beta1); v = v*beta2 + (1-beta2)*g*g;
+ *   w += alpha * (m / (sqrtf(v) + eps))
+ * computed as the reference CPU functor does (double products, float sqrt, one
+ * rounding per assignment). index must not contain duplicates.
+ */
+int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dtype,
+                            void* const* emb_blocks_dev, void* const* exp_avg_blocks_dev,
+                            void* const* exp_avg_sq_blocks_dev, int64_t n_blocks,
+                            int64_t block_size, int row_dtype, void* beta1_t, void* beta2_t,
+                            int beta_is_f64, double lr, double beta1, double beta2,
+                            double weight_decay, double eps, int64_t n, int64_t D, void* stream);
+
+/*
+ * Sparse Adagrad row update; no reference counterpart (RecIS ships only the Adam
+ * family); follows the conventions of block_apply_adamw:
+ *   s += g*g;  w -= lr * g / (sqrtf(s) + eps)      (float arithmetic)
+ */
+int recis_block_apply_adagrad(const int64_t* index, const void* grad, int grad_dtype,
+                              void* const* emb_blocks_dev, void* const* accum_blocks_dev,
+                              int64_t n_blocks, int64_t block_size, int row_dtype, double lr,
+                              double eps, int64_t n, int64_t D, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * Key tagging, offset merging, dedup
+ * ------------------------------------------------------------------------- */
+
+/*
+ * Lists of tensors are passed as HOST arrays of device pointers and sizes.
+ * recis_ids_encode   ids_encode_cuda, csrc/ops/ids_encode_kernel.cu:22-59:
+ *                    out = concat_t ((ids_t & (2^52-1)) | (table_ids[t] << 52))
+ * recis_merge_offsets  merge_offsets, csrc/ops/embedding_segment_reduce_kernel.cu:357-391:
+ *                    tensor t contributes its first size_t - 1 entries (all of them
+ *                    for the last tensor) plus sum_{u<t} max_values[u]
+ */
+int recis_ids_encode(const int64_t* const* ids_ptrs, const int64_t* sizes,
+                     const int64_t* table_ids, int64_t n_tensors, int64_t* out, void* stream);
+int recis_merge_offsets(const void* const* offsets_ptrs, const int64_t* sizes,
+                        const int64_t* max_values, int64_t n_tensors, int is64, void* out,
+                        void* stream);
+
+/*
+ * Dedup: unique ids (in order of first occurrence), inverse (int32 or int64) with
+ * unique_out[inverse[i]] == ids[i], and the number of unique ids written to the
+ * device word count_out_dev. unique_out must have room for n entries.
+ * Replaces the unique half of ids_partition_cuda (csrc/ops/ids_partition_kernel.cu:86-131)
+ * and the torch.unique of recis/nn/modules/hashtable.py:278; the reference orders
+ * the unique ids by sort key instead (sorted variants are built on top of this by
+ * the host layer).
+ */
+int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inverse_out,
+                 int inverse_is64, int64_t* count_out_dev, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * Feature-engine scalar ops (lists as HOST arrays of device pointers)
+ * ------------------------------------------------------------------------- */
+
+/*
+ * recis_fused_hash        fused_hash_cuda, csrc/ops/fused_hash_kernel.cu:421-458:
+ *                         out_t[i] = hash(values_t[off_t[i] .. off_t[i+1])), kind 0 =
+ *                         FarmHash Hash64, 1 = MurmurHash64A seed 0
+ * recis_fused_uint64_mod  fused_uint64_mod_cuda, csrc/ops/fused_uint64_mod_kernel.cu:12-39
+ *                         (and uint64_mod_cuda with one tensor): (int64)((uint64)x % mod_t)
+ * recis_fused_bucketized  fused_bucketized_cuda, csrc/ops/fused_bucketized_kernel.cu:19-60
+ *                         (and bucketize_cuda_op): number of boundaries <= v, NaN -> len
+ * recis_fused_multi_hash  fused_multi_hash_cuda, csrc/ops/multi_hash_kernel.cu:11-74:
+ *                         one job per (tensor, hash): (((x*mul) % p + p) % p) % bucket
+ */
+int recis_fused_hash(const int8_t* const* values_ptrs, const int64_t* values_sizes,
+                     const void* const* offsets_ptrs, int off_is64, const int64_t* n_strings,
+                     int64_t* const* out_ptrs, int64_t n_tensors, int kind, void* stream);
+int recis_fused_uint64_mod(const int64_t* const* in_ptrs, const int64_t* sizes,
+                           const int64_t* mods, int64_t* const* out_ptrs, int64_t n_tensors,
+                           void* stream);
+int recis_fused_bucketized(const float* const* in_ptrs, const int64_t* sizes,
+                           const float* const* boundaries_ptrs, const int64_t* boundary_lens,
+                           int64_t* const* out_ptrs, int64_t n_tensors, void* stream);
+int recis_fused_multi_hash(const int64_t* const* in_ptrs, const int64_t* sizes,
+                           const int64_t* muls, const int64_t* primes, const int64_t* buckets,
+                           int64_t* const* out_ptrs, int64_t n_jobs, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

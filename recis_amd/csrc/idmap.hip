@@ -1,0 +1,702 @@
+// IDMap for gfx950: 64-bit key -> row index, with the row-index allocator folded in.
+//
+// Stands in for GpuIdMap + cuco::dynamic_map + IdAllocator
+// (csrc/embedding/gpu_id_map.cu:19-121, csrc/embedding/id_allocator.cc:17-64,
+// csrc/ops/hashtable_ops_kernel.cu:32-173). Design:
+//   * ONE flat open-addressing table of 16-byte slots {key, row}, power-of-two
+//     capacity, linear probing, load factor <= 1/2; claims are a 64-bit
+//     atomicCAS on the key word (empty = -1, tombstone = -2, as in the reference)
+//   * allocator state (high-water mark, free count) and the free list live in
+//     device memory, so a find-or-insert needs no host round trip: four
+//     back-to-back launches (probe+claim, scan, assign, resolve) replace the
+//     reference's find / cumsum / .item() / GenIds+sync / compact / scatter /
+//     insert+sync-per-submap sequence
+//   * row indices are assigned exactly as IdAllocator::GenIds does: missing keys
+//     are ranked in input order; rank i of n takes free_list[free - n + i] when
+//     that index is >= 0, else the fresh index cur - (free - n + i + 1)
+//   * erase leaves tombstones, later inserts reuse them; the table is rebuilt
+//     (sized up) only when live + tombstones would pass the load limit
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "common.cuh"
+
+namespace recis_hip {
+namespace {
+
+struct Slot {
+  int64_t key;
+  int64_t val;
+};
+
+constexpr int64_t kEmpty = -1;
+constexpr int64_t kTomb = -2;
+constexpr int64_t kValUnset = -1;
+
+enum { ST_CUR = 0, ST_FREE, ST_LIVE, ST_OCC, ST_NNEW, ST_OLD_CUR, ST_OLD_FREE, ST_TMP, ST_DUPS, ST_WORDS };
+
+__device__ __forceinline__ uint64_t mix_key(int64_t key) {
+  uint64_t x = static_cast<uint64_t>(key);
+  x ^= x >> 33;
+  x *= 0xff51afd7ed558ccdULL;
+  x ^= x >> 33;
+  x *= 0xc4ceb9fe1a85ec53ULL;
+  x ^= x >> 33;
+  return x;
+}
+
+__device__ __forceinline__ int64_t ld_relaxed(const int64_t* p) {
+  return __atomic_load_n(p, __ATOMIC_RELAXED);
+}
+__device__ __forceinline__ void st_relaxed(int64_t* p, int64_t v) {
+  __atomic_store_n(p, v, __ATOMIC_RELAXED);
+}
+
+__global__ void __launch_bounds__(kBlock) fill_slots_kernel(Slot* t, int64_t n) {
+  int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  for (; i < n; i += stride) {
+    t[i].key = kEmpty;
+    t[i].val = kValUnset;
+  }
+}
+
+__global__ void zero_words_kernel(int64_t* p, int n) {
+  if (threadIdx.x < n) p[threadIdx.x] = 0;
+}
+
+// Block-wide sum of a 0/1 flag; returns the total in every thread and the
+// exclusive rank of this thread among the set flags.
+__device__ __forceinline__ void block_rank(bool flag, int& rank, int& total) {
+  __shared__ int wave_counts[kBlock / kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const uint64_t ballot = __ballot(flag);
+  const int prior = __popcll(ballot & ((uint64_t(1) << lane) - 1));
+  if (lane == 0) wave_counts[wave] = __popcll(ballot);
+  __syncthreads();
+  int base = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < kBlock / kWave; ++w) {
+    if (w < wave) base += wave_counts[w];
+    tot += wave_counts[w];
+  }
+  __syncthreads();
+  rank = base + prior;
+  total = tot;
+}
+
+// Pass 1 of find-or-insert. slotpos[i]: -1 = resolved (out[i] written),
+// >= 0 = this thread claimed that slot (a new key), <= -2 = the key is being
+// inserted by another thread of this call, slot = -(slotpos + 2).
+__global__ void __launch_bounds__(kBlock)
+find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __restrict__ ids,
+                     int64_t n, int64_t* __restrict__ out, int64_t* __restrict__ slotpos,
+                     int32_t* __restrict__ block_counts, int64_t* __restrict__ state, int* err) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  bool is_new = false;
+  bool took_empty = false;
+  if (i < n) {
+    const int64_t key = ids[i];
+    int64_t sp = -1;
+    if (key == kEmpty || key == kTomb) {
+      raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+      out[i] = -1;
+    } else {
+      const uint64_t h = mix_key(key) & mask;
+      uint64_t p = h;
+      int64_t first_tomb = -1;
+      uint64_t probes = 0;
+      for (;;) {
+        const int64_t k = ld_relaxed(&table[p].key);
+        if (k == key) {
+          const int64_t v = ld_relaxed(&table[p].val);
+          if (v >= 0) {
+            out[i] = v;
+          } else {
+            sp = -(static_cast<int64_t>(p) + 2);
+            atomicOr(reinterpret_cast<unsigned long long*>(&state[ST_DUPS]), 1ull);
+          }
+          break;
+        }
+        if (k == kEmpty) {
+          const bool use_tomb = first_tomb >= 0;
+          const int64_t target = use_tomb ? first_tomb : static_cast<int64_t>(p);
+          const int64_t expect = use_tomb ? kTomb : kEmpty;
+          const int64_t old = static_cast<int64_t>(atomicCAS(
+              reinterpret_cast<unsigned long long*>(&table[target].key),
+              static_cast<unsigned long long>(expect), static_cast<unsigned long long>(key)));
+          if (old == expect) {
+            st_relaxed(&table[target].val, -(i + 2));  // pending, owner = occurrence i
+            sp = target;
+            is_new = true;
+            took_empty = !use_tomb;
+            break;
+          }
+          // somebody else took that slot: start over, keys never vanish meanwhile
+          p = h;
+          first_tomb = -1;
+          probes = 0;
+          continue;
+        }
+        if (k == kTomb && first_tomb < 0) first_tomb = static_cast<int64_t>(p);
+        p = (p + 1) & mask;
+        if (++probes > mask) {
+          raise_device_error(err, RECIS_DEVERR_TABLE_FULL);
+          out[i] = -1;
+          break;
+        }
+      }
+    }
+    slotpos[i] = sp;
+  }
+  int rank, total;
+  block_rank(is_new, rank, total);
+  int rank_e, total_e;
+  block_rank(took_empty, rank_e, total_e);
+  if (threadIdx.x == 0) {
+    block_counts[blockIdx.x] = total;
+    if (total_e)
+      atomicAdd(reinterpret_cast<unsigned long long*>(&state[ST_OCC]),
+                static_cast<unsigned long long>(total_e));
+  }
+}
+
+// Pass 2: exclusive scan of the per-block counts (single workgroup) and the
+// allocator bookkeeping of IdAllocator::GenIds (id_allocator.cc:17-26).
+__global__ void __launch_bounds__(1024)
+scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t* __restrict__ state) {
+  __shared__ int64_t partial[1024];
+  const int t = threadIdx.x;
+  const int64_t per = (nb + 1023) / 1024;
+  const int64_t lo = std::min<int64_t>(t * per, nb), hi = std::min<int64_t>(lo + per, nb);
+  int64_t sum = 0;
+  for (int64_t b = lo; b < hi; ++b) sum += block_counts[b];
+  partial[t] = sum;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over the 1024 partials
+  for (int off = 1; off < 1024; off <<= 1) {
+    int64_t add = t >= off ? partial[t - off] : 0;
+    __syncthreads();
+    partial[t] += add;
+    __syncthreads();
+  }
+  int64_t run = t ? partial[t - 1] : 0;
+  for (int64_t b = lo; b < hi; ++b) {
+    int32_t c = block_counts[b];
+    block_counts[b] = static_cast<int32_t>(run);  // per-call counts fit 31 bits
+    run += c;
+  }
+  if (t == 1023) {
+    const int64_t total = partial[1023];
+    const int64_t cur = state[ST_CUR], fr = state[ST_FREE];
+    state[ST_OLD_CUR] = cur;
+    state[ST_OLD_FREE] = fr;
+    state[ST_NNEW] = total;
+    const int64_t fresh = fr >= total ? 0 : total - fr;
+    state[ST_CUR] = cur + fresh;
+    state[ST_FREE] = fr >= total ? fr - total : 0;
+    state[ST_LIVE] += total;
+  }
+}
+
+// Pass 3: give every claimed slot its row index (IdGeneratorFunctor,
+// hashtable_ops.cc:15-27) in input order.
+__global__ void __launch_bounds__(kBlock)
+assign_rows_kernel(Slot* __restrict__ table, const int64_t* __restrict__ slotpos, int64_t n,
+                   const int32_t* __restrict__ block_prefix, const int64_t* __restrict__ state,
+                   const int64_t* __restrict__ free_list, int64_t* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  const int64_t sp = i < n ? slotpos[i] : -1;
+  const bool is_new = sp >= 0;
+  int rank, total;
+  block_rank(is_new, rank, total);
+  if (!is_new) return;
+  const int64_t n_new = state[ST_NNEW];
+  const int64_t free_index = state[ST_OLD_FREE] - n_new + block_prefix[blockIdx.x] + rank;
+  const int64_t row = free_index >= 0 ? free_list[free_index] : state[ST_OLD_CUR] - (free_index + 1);
+  st_relaxed(&table[sp].val, row);
+  out[i] = row;
+}
+
+// Pass 4: occurrences whose key was claimed by another occurrence of the same call.
+__global__ void __launch_bounds__(kBlock)
+resolve_dups_kernel(const Slot* __restrict__ table, const int64_t* __restrict__ slotpos, int64_t n,
+                    const int64_t* __restrict__ state, int64_t* __restrict__ out) {
+  if (state[ST_DUPS] == 0) return;
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const int64_t sp = slotpos[i];
+  if (sp <= -2) out[i] = table[-(sp + 2)].val;
+}
+
+__global__ void __launch_bounds__(kBlock)
+find_kernel(const Slot* __restrict__ table, uint64_t mask, const int64_t* __restrict__ ids,
+            int64_t n, int64_t* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const int64_t key = ids[i];
+  int64_t res = -1;
+  if (key != kEmpty && key != kTomb) {
+    uint64_t p = mix_key(key) & mask;
+    for (uint64_t probes = 0; probes <= mask; ++probes) {
+      const int64_t k = table[p].key;
+      if (k == key) {
+        res = table[p].val;
+        break;
+      }
+      if (k == kEmpty) break;
+      p = (p + 1) & mask;
+    }
+  }
+  out[i] = res;
+}
+
+// DeleteIds (gpu_id_map.cu:84-96): tombstone the keys, append `index` to the
+// free list in the order given (IdFreeFunctor, hashtable_ops.cc:39-58).
+__global__ void __launch_bounds__(kBlock)
+erase_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __restrict__ ids,
+             const int64_t* __restrict__ index, int64_t n, int64_t* __restrict__ free_list,
+             int64_t* __restrict__ state) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  bool found = false;
+  if (i < n) {
+    const int64_t key = ids[i];
+    if (key != kEmpty && key != kTomb) {
+      uint64_t p = mix_key(key) & mask;
+      for (uint64_t probes = 0; probes <= mask; ++probes) {
+        const int64_t k = ld_relaxed(&table[p].key);
+        if (k == key) {
+          // a key listed twice is erased once: only the CAS winner counts it
+          const int64_t old = static_cast<int64_t>(atomicCAS(
+              reinterpret_cast<unsigned long long*>(&table[p].key),
+              static_cast<unsigned long long>(key), static_cast<unsigned long long>(kTomb)));
+          if (old == key) {
+            st_relaxed(&table[p].val, kValUnset);
+            found = true;
+          }
+          break;
+        }
+        if (k == kEmpty) break;
+        p = (p + 1) & mask;
+      }
+    }
+    free_list[state[ST_FREE] + i] = index[i];
+  }
+  int rank, total;
+  block_rank(found, rank, total);
+  if (threadIdx.x == 0 && total)
+    atomicAdd(reinterpret_cast<unsigned long long*>(&state[ST_TMP]),
+              static_cast<unsigned long long>(total));
+}
+
+__global__ void erase_commit_kernel(int64_t* state, int64_t n) {
+  state[ST_FREE] += n;
+  state[ST_LIVE] -= state[ST_TMP];
+  state[ST_TMP] = 0;
+}
+
+__global__ void reset_dups_kernel(int64_t* state) { state[ST_DUPS] = 0; }
+
+// retrieve_all: every live (key, row) pair, in no particular order.
+__global__ void __launch_bounds__(kBlock)
+snapshot_kernel(const Slot* __restrict__ table, int64_t capacity, int64_t* __restrict__ ids_out,
+                int64_t* __restrict__ index_out, int64_t max_out, int64_t* __restrict__ state) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  bool live = false;
+  int64_t k = 0, v = 0;
+  if (i < capacity) {
+    k = table[i].key;
+    v = table[i].val;
+    live = k != kEmpty && k != kTomb && v >= 0;
+  }
+  int rank, total;
+  block_rank(live, rank, total);
+  __shared__ int64_t base;
+  if (threadIdx.x == 0)
+    base = total ? static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&state[ST_TMP]),
+                                                  static_cast<unsigned long long>(total)))
+                 : 0;
+  __syncthreads();
+  if (live) {
+    const int64_t pos = base + rank;
+    if (pos < max_out) {
+      ids_out[pos] = k;
+      index_out[pos] = v;
+    }
+  }
+}
+
+// Re-insert all live entries of an old table into a new, empty one.
+__global__ void __launch_bounds__(kBlock)
+rehash_kernel(const Slot* __restrict__ old_table, int64_t old_capacity, Slot* __restrict__ table,
+              uint64_t mask) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (i >= old_capacity) return;
+  const int64_t key = old_table[i].key;
+  const int64_t val = old_table[i].val;
+  if (key == kEmpty || key == kTomb || val < 0) return;
+  uint64_t p = mix_key(key) & mask;
+  for (uint64_t probes = 0; probes <= mask; ++probes) {
+    const int64_t old = static_cast<int64_t>(atomicCAS(
+        reinterpret_cast<unsigned long long*>(&table[p].key),
+        static_cast<unsigned long long>(kEmpty), static_cast<unsigned long long>(key)));
+    if (old == kEmpty) {
+      table[p].val = val;
+      return;
+    }
+    p = (p + 1) & mask;
+  }
+}
+
+// ---- standalone allocator ops (csrc/ops/hashtable_ops_kernel.cu:32-173)
+__global__ void __launch_bounds__(kBlock)
+generate_ids_kernel(int64_t n, const int64_t* const* __restrict__ free_blocks, int64_t free_count,
+                    int64_t cur_count, int64_t free_block_size, int64_t* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const int64_t free_index = free_count - n + i;
+  out[i] = free_index >= 0 ? free_blocks[free_index / free_block_size][free_index % free_block_size]
+                           : cur_count - (free_index + 1);
+}
+
+__global__ void __launch_bounds__(kBlock)
+free_ids_kernel(const int64_t* __restrict__ ids, int64_t n, int64_t* const* __restrict__ free_blocks,
+                int64_t free_count, int64_t free_block_size) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const int64_t free_index = free_count + i;
+  free_blocks[free_index / free_block_size][free_index % free_block_size] = ids[i];
+}
+
+__global__ void __launch_bounds__(kBlock)
+mask_key_index_kernel(const int64_t* __restrict__ keys, const uint8_t* __restrict__ mask,
+                      const int64_t* __restrict__ cumsum, int64_t n, int64_t out_size,
+                      int64_t* __restrict__ out_keys, int64_t* __restrict__ out_index, int* err) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (i >= n || !mask[i]) return;
+  const int64_t pos = cumsum[i] - 1;
+  if (static_cast<uint64_t>(pos) >= static_cast<uint64_t>(out_size)) {
+    raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+    return;
+  }
+  out_keys[pos] = keys[i];
+  out_index[pos] = i;
+}
+
+__global__ void __launch_bounds__(kBlock)
+scatter_ids_kernel(int64_t* __restrict__ out_ids, int64_t out_size, const int64_t* __restrict__ in_ids,
+                   const int64_t* __restrict__ mask_index, int64_t n, int* err) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const int64_t pos = mask_index[i];
+  if (static_cast<uint64_t>(pos) >= static_cast<uint64_t>(out_size)) {
+    raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+    return;
+  }
+  out_ids[pos] = in_ids[i];
+}
+
+inline int64_t blocks_for(int64_t n) { return (n + kBlock - 1) / kBlock; }
+
+int64_t capacity_for(int64_t keys) {
+  int64_t cap = 1024;
+  while (cap < keys * 2) cap <<= 1;
+  return cap;
+}
+
+}  // namespace
+}  // namespace recis_hip
+
+using namespace recis_hip;
+
+struct recis_idmap {
+  int device = 0;
+  int64_t capacity = 0;
+  Slot* table = nullptr;
+  int64_t* state = nullptr;     // device, ST_WORDS int64
+  int64_t* free_list = nullptr; // device
+  int64_t free_cap = 0;
+  // host-side upper bounds, refreshed by sync_stats()
+  int64_t occ_ub = 0;   // non-empty slots (live + tombstones)
+  int64_t free_ub = 0;  // entries in the free list
+  int* err = nullptr;
+};
+
+namespace {
+
+int alloc_table(recis_idmap* m, int64_t capacity, hipStream_t stream, Slot** out) {
+  Slot* t = nullptr;
+  RECIS_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&t), sizeof(Slot) * static_cast<size_t>(capacity)));
+  int64_t grid = std::min<int64_t>(blocks_for(capacity), 256 * 64);
+  fill_slots_kernel<<<dim3(grid), dim3(kBlock), 0, stream>>>(t, capacity);
+  RECIS_LAUNCH_CHECK();
+  *out = t;
+  (void)m;
+  return RECIS_OK;
+}
+
+int sync_stats(recis_idmap* m, hipStream_t stream, int64_t* words) {
+  RECIS_CHECK_HIP(hipMemcpyAsync(words, m->state, sizeof(int64_t) * ST_WORDS, hipMemcpyDeviceToHost, stream));
+  RECIS_CHECK_HIP(hipStreamSynchronize(stream));
+  m->occ_ub = words[ST_OCC];
+  m->free_ub = words[ST_FREE];
+  return RECIS_OK;
+}
+
+int rebuild(recis_idmap* m, int64_t new_capacity, hipStream_t stream) {
+  Slot* nt = nullptr;
+  if (int rc = alloc_table(m, new_capacity, stream, &nt)) return rc;
+  rehash_kernel<<<dim3(blocks_for(m->capacity)), dim3(kBlock), 0, stream>>>(
+      m->table, m->capacity, nt, static_cast<uint64_t>(new_capacity - 1));
+  RECIS_LAUNCH_CHECK();
+  int64_t words[ST_WORDS];
+  if (int rc = sync_stats(m, stream, words)) return rc;
+  // tombstones are gone: occupied == live
+  RECIS_CHECK_HIP(hipMemcpyAsync(m->state + ST_OCC, &words[ST_LIVE], sizeof(int64_t),
+                                 hipMemcpyHostToDevice, stream));
+  RECIS_CHECK_HIP(hipStreamSynchronize(stream));
+  RECIS_CHECK_HIP(hipFree(m->table));
+  m->table = nt;
+  m->capacity = new_capacity;
+  m->occ_ub = words[ST_LIVE];
+  return RECIS_OK;
+}
+
+// Make room for up to `incoming` more claimed slots.
+int ensure_table_room(recis_idmap* m, int64_t incoming, hipStream_t stream) {
+  if ((m->occ_ub + incoming) * 2 <= m->capacity) return RECIS_OK;
+  int64_t words[ST_WORDS];
+  if (int rc = sync_stats(m, stream, words)) return rc;
+  if ((m->occ_ub + incoming) * 2 <= m->capacity) return RECIS_OK;
+  const int64_t live = words[ST_LIVE];
+  return rebuild(m, capacity_for(live + incoming + (live + incoming) / 2), stream);
+}
+
+int ensure_free_room(recis_idmap* m, int64_t incoming, hipStream_t stream) {
+  if (m->free_ub + incoming <= m->free_cap) return RECIS_OK;
+  int64_t words[ST_WORDS];
+  if (int rc = sync_stats(m, stream, words)) return rc;
+  if (m->free_ub + incoming <= m->free_cap) return RECIS_OK;
+  int64_t cap = std::max<int64_t>(m->free_cap * 2, 10240);
+  while (cap < m->free_ub + incoming) cap *= 2;
+  int64_t* nf = nullptr;
+  RECIS_CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&nf), sizeof(int64_t) * static_cast<size_t>(cap)));
+  if (m->free_ub > 0)
+    RECIS_CHECK_HIP(hipMemcpyAsync(nf, m->free_list, sizeof(int64_t) * static_cast<size_t>(m->free_ub),
+                                   hipMemcpyDeviceToDevice, stream));
+  RECIS_CHECK_HIP(hipStreamSynchronize(stream));
+  if (m->free_list) RECIS_CHECK_HIP(hipFree(m->free_list));
+  m->free_list = nf;
+  m->free_cap = cap;
+  return RECIS_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int recis_idmap_create(int64_t reserve_keys, recis_idmap** out) {
+  RECIS_REQUIRE(out != nullptr, "out must not be NULL");
+  RECIS_REQUIRE(reserve_keys >= 0, "reserve_keys must be >= 0");
+  recis_idmap* m = new recis_idmap();
+  m->device = current_device();
+  m->err = device_error_word(m->device);
+  if (!m->err) {
+    delete m;
+    return fail(RECIS_ERR_HIP, "could not allocate the device error word");
+  }
+  // The reference starts at 640000 slots (gpu_id_map.h:12); we start at the
+  // next power of two unless the caller reserves more.
+  m->capacity = capacity_for(std::max<int64_t>(reserve_keys, 320000));
+  int rc = alloc_table(m, m->capacity, nullptr, &m->table);
+  if (rc == RECIS_OK && hipMalloc(reinterpret_cast<void**>(&m->state), sizeof(int64_t) * ST_WORDS) != hipSuccess)
+    rc = fail(RECIS_ERR_HIP, "hipMalloc of the allocator state failed");
+  if (rc == RECIS_OK) {
+    zero_words_kernel<<<1, 64>>>(m->state, ST_WORDS);
+    if (hipStreamSynchronize(nullptr) != hipSuccess) rc = fail(RECIS_ERR_HIP, "id-map initialisation failed");
+  }
+  if (rc == RECIS_OK) rc = ensure_free_room(m, 10240, nullptr);
+  if (rc != RECIS_OK) {
+    if (m->table) (void)hipFree(m->table);
+    if (m->state) (void)hipFree(m->state);
+    delete m;
+    return rc;
+  }
+  *out = m;
+  return RECIS_OK;
+}
+
+int recis_idmap_destroy(recis_idmap* m) {
+  if (!m) return RECIS_OK;
+  (void)hipDeviceSynchronize();
+  if (m->table) (void)hipFree(m->table);
+  if (m->state) (void)hipFree(m->state);
+  if (m->free_list) (void)hipFree(m->free_list);
+  delete m;
+  return RECIS_OK;
+}
+
+int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* index_out,
+                       void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr, "id map is NULL");
+  RECIS_REQUIRE(n >= 0 && n < (int64_t(1) << 31), "n out of range: %lld", (long long)n);
+  if (n == 0) return RECIS_OK;
+  RECIS_REQUIRE(ids != nullptr && index_out != nullptr, "ids/index_out must not be NULL");
+  if (int rc = ensure_table_room(m, n, stream)) return rc;
+  const int64_t nb = blocks_for(n);
+  void* ws = nullptr;
+  const size_t ws_bytes = sizeof(int64_t) * static_cast<size_t>(n) + sizeof(int32_t) * static_cast<size_t>(nb);
+  if (int rc = get_workspace(stream, ws_bytes, &ws)) return rc;
+  int64_t* slotpos = static_cast<int64_t*>(ws);
+  int32_t* block_counts = reinterpret_cast<int32_t*>(slotpos + n);
+  const uint64_t mask = static_cast<uint64_t>(m->capacity - 1);
+
+  reset_dups_kernel<<<1, 1, 0, stream>>>(m->state);
+  find_or_claim_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, mask, ids, n, index_out, slotpos,
+                                                             block_counts, m->state, m->err);
+  RECIS_LAUNCH_CHECK();
+  scan_commit_kernel<<<1, 1024, 0, stream>>>(block_counts, nb, m->state);
+  RECIS_LAUNCH_CHECK();
+  assign_rows_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, block_counts, m->state,
+                                                           m->free_list, index_out);
+  RECIS_LAUNCH_CHECK();
+  resolve_dups_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, m->state, index_out);
+  RECIS_LAUNCH_CHECK();
+  m->occ_ub += n;
+  return RECIS_OK;
+}
+
+int recis_idmap_lookup_readonly(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* index_out,
+                                void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr, "id map is NULL");
+  RECIS_REQUIRE(n >= 0, "n out of range: %lld", (long long)n);
+  if (n == 0) return RECIS_OK;
+  RECIS_REQUIRE(ids != nullptr && index_out != nullptr, "ids/index_out must not be NULL");
+  find_kernel<<<dim3(blocks_for(n)), dim3(kBlock), 0, stream>>>(
+      m->table, static_cast<uint64_t>(m->capacity - 1), ids, n, index_out);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+int recis_idmap_erase(recis_idmap* m, const int64_t* ids, const int64_t* index, int64_t n,
+                      void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr, "id map is NULL");
+  RECIS_REQUIRE(n >= 0, "n out of range: %lld", (long long)n);
+  if (n == 0) return RECIS_OK;
+  RECIS_REQUIRE(ids != nullptr && index != nullptr, "ids/index must not be NULL");
+  if (int rc = ensure_free_room(m, n, stream)) return rc;
+  erase_kernel<<<dim3(blocks_for(n)), dim3(kBlock), 0, stream>>>(
+      m->table, static_cast<uint64_t>(m->capacity - 1), ids, index, n, m->free_list, m->state);
+  RECIS_LAUNCH_CHECK();
+  erase_commit_kernel<<<1, 1, 0, stream>>>(m->state, n);
+  RECIS_LAUNCH_CHECK();
+  m->free_ub += n;
+  return RECIS_OK;
+}
+
+int recis_idmap_stats(recis_idmap* m, int64_t* live, int64_t* id_num, int64_t* free_size,
+                      int64_t* capacity, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr, "id map is NULL");
+  int64_t words[ST_WORDS];
+  if (int rc = sync_stats(m, stream, words)) return rc;
+  if (live) *live = words[ST_LIVE];
+  if (id_num) *id_num = words[ST_CUR];
+  if (free_size) *free_size = words[ST_FREE];
+  if (capacity) *capacity = m->capacity;
+  return RECIS_OK;
+}
+
+int recis_idmap_snapshot(recis_idmap* m, int64_t* ids_out, int64_t* index_out, int64_t max_out,
+                         int64_t* count, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr && count != nullptr, "id map / count is NULL");
+  RECIS_REQUIRE(max_out >= 0 && (max_out == 0 || (ids_out && index_out)), "bad output buffers");
+  snapshot_kernel<<<dim3(blocks_for(m->capacity)), dim3(kBlock), 0, stream>>>(
+      m->table, m->capacity, ids_out, index_out, max_out, m->state);
+  RECIS_LAUNCH_CHECK();
+  int64_t words[ST_WORDS];
+  if (int rc = sync_stats(m, stream, words)) return rc;
+  *count = words[ST_TMP];
+  zero_words_kernel<<<1, 64, 0, stream>>>(m->state + ST_TMP, 1);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+int recis_idmap_clear(recis_idmap* m, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr, "id map is NULL");
+  int64_t grid = std::min<int64_t>(blocks_for(m->capacity), 256 * 64);
+  fill_slots_kernel<<<dim3(grid), dim3(kBlock), 0, stream>>>(m->table, m->capacity);
+  RECIS_LAUNCH_CHECK();
+  zero_words_kernel<<<1, 64, 0, stream>>>(m->state, ST_WORDS);
+  RECIS_LAUNCH_CHECK();
+  m->occ_ub = 0;
+  m->free_ub = 0;
+  return RECIS_OK;
+}
+
+int recis_idmap_reserve(recis_idmap* m, int64_t n_keys, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr, "id map is NULL");
+  const int64_t want = capacity_for(n_keys);
+  if (want <= m->capacity) return RECIS_OK;
+  return rebuild(m, want, stream);
+}
+
+int recis_generate_ids(int64_t n, const int64_t* const* free_blocks_dev, int64_t free_count,
+                       int64_t cur_count, int64_t free_block_size, int64_t* out, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n >= 0 && free_block_size > 0, "bad sizes");
+  if (n == 0) return RECIS_OK;
+  RECIS_REQUIRE(out != nullptr && (free_blocks_dev != nullptr || free_count == 0), "NULL argument");
+  generate_ids_kernel<<<dim3(blocks_for(n)), dim3(kBlock), 0, stream>>>(n, free_blocks_dev, free_count,
+                                                                       cur_count, free_block_size, out);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+int recis_free_ids(const int64_t* ids, int64_t n, int64_t* const* free_blocks_dev, int64_t free_count,
+                   int64_t free_block_size, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n >= 0 && free_block_size > 0, "bad sizes");
+  if (n == 0) return RECIS_OK;
+  RECIS_REQUIRE(ids != nullptr && free_blocks_dev != nullptr, "NULL argument");
+  free_ids_kernel<<<dim3(blocks_for(n)), dim3(kBlock), 0, stream>>>(ids, n, free_blocks_dev, free_count,
+                                                                   free_block_size);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+int recis_mask_key_index(const int64_t* keys, const uint8_t* mask, const int64_t* cumsum, int64_t n,
+                         int64_t out_size, int64_t* out_keys, int64_t* out_index, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n >= 0 && out_size >= 0, "bad sizes");
+  if (n == 0 || out_size == 0) return RECIS_OK;
+  RECIS_REQUIRE(keys && mask && cumsum && out_keys && out_index, "NULL argument");
+  int* err = device_error_word(current_device());
+  mask_key_index_kernel<<<dim3(blocks_for(n)), dim3(kBlock), 0, stream>>>(keys, mask, cumsum, n, out_size,
+                                                                         out_keys, out_index, err);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+int recis_scatter_ids_with_mask(int64_t* out_ids, int64_t out_size, const int64_t* in_ids,
+                                const int64_t* mask_index, int64_t n, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n >= 0 && out_size >= 0, "bad sizes");
+  if (n == 0 || out_size == 0) return RECIS_OK;
+  RECIS_REQUIRE(out_ids && in_ids && mask_index, "NULL argument");
+  int* err = device_error_word(current_device());
+  scatter_ids_kernel<<<dim3(blocks_for(n)), dim3(kBlock), 0, stream>>>(out_ids, out_size, in_ids,
+                                                                      mask_index, n, err);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+}  // extern "C"

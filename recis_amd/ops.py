@@ -100,3 +100,550 @@ def segment_reduce_backward(grad_output, weight, reverse_indices, offsets, uniqu
         ptr(out), dtype_code(work_dtype), i64(B), i64(U), i64(S), i64(D), _lib.MODES[mode],
         _lib.FLAG_REV_UNIQUE if unique else 0, stream_ptr(grad_output.device)))
     return out if work_dtype == out_dtype else out.to(out_dtype)
+
+
+# ------------------------------------------------------------- small helpers
+def _host_ptrs(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def _host_i64(values):
+    return (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+
+
+_PTR_TABLE_CACHE = {}
+
+
+def block_ptr_table(blocks):
+    """Device int64 tensor holding the base pointer of every block.
+
+    Cached on the tuple of pointers, so a slot that does not grow pays the
+    host-to-device copy once, not per launch."""
+    key = (blocks[0].device.index,) + tuple(b.data_ptr() for b in blocks)
+    tab = _PTR_TABLE_CACHE.get(key)
+    if tab is None:
+        if len(_PTR_TABLE_CACHE) > 256:
+            _PTR_TABLE_CACHE.clear()
+        tab = torch.tensor(key[1:], dtype=torch.int64).to(blocks[0].device)
+        _PTR_TABLE_CACHE[key] = tab
+    return tab
+
+
+def _check_blocks(blocks, block_size):
+    if len(blocks) == 0:
+        raise ValueError("empty block list")
+    b0 = blocks[0]
+    for b in blocks:
+        require_cuda(b)
+        if b.dtype != b0.dtype or b.shape[1:] != b0.shape[1:] or not b.is_contiguous():
+            raise ValueError("blocks must be contiguous and share dtype and row shape")
+        if b.shape[0] < block_size:
+            raise ValueError("block with %d rows is smaller than block_size %d" % (b.shape[0], block_size))
+    return b0
+
+
+def _row_bytes(block):
+    n = block.element_size()
+    for d in block.shape[1:]:
+        n *= d
+    return n
+
+
+def _ids64(ids):
+    require_cuda(ids)
+    if ids.dtype != torch.int64:
+        raise TypeError("ids must be int64, got %s" % ids.dtype)
+    return _contig(ids).view(-1)
+
+
+# ---------------------------------------------------------------- row blocks
+def gather(ids, emb):
+    """``torch.ops.recis.gather`` (block_ops.h:6): ``emb[ids]`` for a flat table."""
+    require_cuda(ids, emb)
+    ids, emb = _contig(ids).view(-1), _contig(emb)
+    out = torch.empty((ids.numel(),) + tuple(emb.shape[1:]), dtype=emb.dtype, device=emb.device)
+    check(lib().recis_gather(ptr(ids), _index_kind(ids, "ids"), ptr(emb), i64(emb.shape[0]), ptr(out),
+                             i64(ids.numel()), i64(_row_bytes(emb)), stream_ptr(emb.device)))
+    return out
+
+
+def block_gather(ids, emb_blocks, block_size, default_key=-1, readonly=False):
+    """``torch.ops.recis.block_gather`` (block_ops.h:8-12)."""
+    b0 = _check_blocks(emb_blocks, block_size)
+    ids = _ids64(ids)
+    out = torch.empty((ids.numel(),) + tuple(b0.shape[1:]), dtype=b0.dtype, device=b0.device)
+    tab = block_ptr_table(emb_blocks)
+    check(lib().recis_block_gather(ptr(ids), ptr(tab), i64(len(emb_blocks)), i64(block_size),
+                                   i64(default_key), int(bool(readonly)), ptr(out), i64(ids.numel()),
+                                   i64(_row_bytes(b0)), stream_ptr(b0.device)))
+    return out
+
+
+def block_gather_by_range(ids, emb_blocks, block_size, beg, end):
+    """``block_gather_by_range`` (block_ops.cc:305-314): rows of ``ids[beg:end]``."""
+    return block_gather(_ids64(ids)[beg:end], emb_blocks, block_size, -1, False)
+
+
+def block_insert(ids, embedding, emb_blocks, block_size):
+    """``torch.ops.recis.block_insert`` (block_ops.h:28-30); one embedding row is broadcast."""
+    b0 = _check_blocks(emb_blocks, block_size)
+    ids = _ids64(ids)
+    require_cuda(embedding)
+    embedding = _contig(embedding)
+    if embedding.dtype != b0.dtype:
+        raise TypeError("embedding dtype %s does not match the blocks (%s)" % (embedding.dtype, b0.dtype))
+    if not (embedding.shape[0] == ids.numel() or embedding.shape[0] == 1):
+        raise ValueError("ids batch_size must = embedding batch size or embedding batch size = 1")
+    broadcast = int(embedding.shape[0] == 1 and ids.numel() != 1)
+    tab = block_ptr_table(emb_blocks)
+    check(lib().recis_block_insert(ptr(ids), ptr(embedding), broadcast, ptr(None), ptr(tab),
+                                   i64(len(emb_blocks)), i64(block_size), i64(ids.numel()),
+                                   i64(_row_bytes(b0)), stream_ptr(b0.device)))
+
+
+def block_insert_with_mask(ids, embedding, mask, emb_blocks, block_size):
+    """``torch.ops.recis.block_insert_with_mask`` (block_ops.h:32-36)."""
+    b0 = _check_blocks(emb_blocks, block_size)
+    ids = _ids64(ids)
+    require_cuda(embedding, mask)
+    embedding = _contig(embedding)
+    if embedding.dtype != b0.dtype:
+        raise TypeError("embedding dtype %s does not match the blocks (%s)" % (embedding.dtype, b0.dtype))
+    if mask.dtype != torch.bool:
+        raise TypeError("mask must be bool")
+    mask = _contig(mask)
+    tab = block_ptr_table(emb_blocks)
+    check(lib().recis_block_insert(ptr(ids), ptr(embedding), 0, ptr(mask), ptr(tab),
+                                   i64(len(emb_blocks)), i64(block_size), i64(ids.numel()),
+                                   i64(_row_bytes(b0)), stream_ptr(b0.device)))
+
+
+def block_filter(ids, emb_blocks, block_size, threshold):
+    """``torch.ops.recis.block_filter`` (block_ops.h:20-22): ``slot[ids] < threshold``."""
+    b0 = _check_blocks(emb_blocks, block_size)
+    if b0.dtype not in (torch.int32, torch.int64) or _row_bytes(b0) != b0.element_size():
+        raise TypeError("block_filter needs an int32/int64 slot of width 1")
+    ids = _ids64(ids)
+    out = torch.empty(ids.numel(), dtype=torch.bool, device=b0.device)
+    tab = block_ptr_table(emb_blocks)
+    check(lib().recis_block_filter(ptr(ids), ptr(tab), i64(len(emb_blocks)), i64(block_size),
+                                   i64(threshold), int(b0.dtype == torch.int64), ptr(out),
+                                   i64(ids.numel()), stream_ptr(b0.device)))
+    return out
+
+
+# ----------------------------------------------------------------- optimizers
+def block_apply_adamw(index, grad, emb_blocks, beta1_t, beta2_t, step, exp_avg, exp_avg_sq, lr,
+                      beta1, beta2, weight_decay, eps, block_size):
+    """``torch.ops.recis.block_apply_adamw`` (block_apply_adamw_op.h:6-12).
+
+    In place on the three block lists and on ``beta1_t`` / ``beta2_t`` (GPU scalars,
+    float32 or float64). ``weight_decay`` is the multiplicative factor applied to the
+    row. ``step`` is accepted and left untouched, as in the reference
+    (block_apply_adamw_op.cc:121 discards the result of ``step.add(1)``)."""
+    b0 = _check_blocks(emb_blocks, block_size)
+    _check_blocks(exp_avg, block_size)
+    _check_blocks(exp_avg_sq, block_size)
+    if len(exp_avg) != len(emb_blocks) or len(exp_avg_sq) != len(emb_blocks):
+        raise ValueError("state slots must have as many blocks as the embedding slot")
+    index = _ids64(index)
+    require_cuda(grad, beta1_t, beta2_t)
+    grad = _contig(grad)
+    if beta1_t.dtype != beta2_t.dtype or beta1_t.dtype not in (torch.float32, torch.float64):
+        raise TypeError("beta1_t / beta2_t must both be float32 or float64")
+    D = _row_bytes(b0) // b0.element_size()
+    if grad.numel() != index.numel() * D:
+        raise ValueError("grad has %d elements, expected %d x %d" % (grad.numel(), index.numel(), D))
+    check(lib().recis_block_apply_adamw(
+        ptr(index), ptr(grad), dtype_code(grad.dtype), ptr(block_ptr_table(emb_blocks)),
+        ptr(block_ptr_table(exp_avg)), ptr(block_ptr_table(exp_avg_sq)), i64(len(emb_blocks)),
+        i64(block_size), dtype_code(b0.dtype), ptr(beta1_t), ptr(beta2_t),
+        int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1),
+        ctypes.c_double(beta2), ctypes.c_double(weight_decay), ctypes.c_double(eps),
+        i64(index.numel()), i64(D), stream_ptr(b0.device)))
+
+
+def block_apply_adagrad(index, grad, emb_blocks, accum_blocks, lr, eps, block_size):
+    """Sparse Adagrad row update (an addition; same conventions as block_apply_adamw)."""
+    b0 = _check_blocks(emb_blocks, block_size)
+    _check_blocks(accum_blocks, block_size)
+    if len(accum_blocks) != len(emb_blocks):
+        raise ValueError("state slot must have as many blocks as the embedding slot")
+    index = _ids64(index)
+    require_cuda(grad)
+    grad = _contig(grad)
+    D = _row_bytes(b0) // b0.element_size()
+    if grad.numel() != index.numel() * D:
+        raise ValueError("grad has %d elements, expected %d x %d" % (grad.numel(), index.numel(), D))
+    check(lib().recis_block_apply_adagrad(
+        ptr(index), ptr(grad), dtype_code(grad.dtype), ptr(block_ptr_table(emb_blocks)),
+        ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)), i64(block_size), dtype_code(b0.dtype),
+        ctypes.c_double(lr), ctypes.c_double(eps), i64(index.numel()), i64(D), stream_ptr(b0.device)))
+
+
+# ------------------------------------------------------------- allocator ops
+def generate_ids(gen_num, free_blocks, free_count, cur_count, free_block_size):
+    """``torch.ops.recis.generate_ids`` (hashtable_ops.h:17-21)."""
+    dev = free_blocks[0].device
+    out = torch.empty(gen_num, dtype=torch.int64, device=dev)
+    check(lib().recis_generate_ids(i64(gen_num), ptr(block_ptr_table(free_blocks)), i64(free_count),
+                                   i64(cur_count), i64(free_block_size), ptr(out), stream_ptr(dev)))
+    return out
+
+
+def free_ids(ids, free_blocks, free_count, free_block_size):
+    """``torch.ops.recis.free_ids`` (hashtable_ops.h:23-25); in place on ``free_blocks``."""
+    ids = _ids64(ids)
+    check(lib().recis_free_ids(ptr(ids), i64(ids.numel()), ptr(block_ptr_table(free_blocks)),
+                               i64(free_count), i64(free_block_size), stream_ptr(ids.device)))
+
+
+def mask_key_index(in_keys, mask, in_out_index, out_size):
+    """``torch.ops.recis.mask_key_index`` (hashtable_ops.h:27-30)."""
+    in_keys, in_out_index = _ids64(in_keys), _ids64(in_out_index)
+    require_cuda(mask)
+    if mask.dtype != torch.bool:
+        raise TypeError("mask must be bool")
+    mask = _contig(mask)
+    out_keys = torch.empty(out_size, dtype=torch.int64, device=in_keys.device)
+    out_index = torch.empty_like(out_keys)
+    check(lib().recis_mask_key_index(ptr(in_keys), ptr(mask), ptr(in_out_index), i64(in_keys.numel()),
+                                     i64(out_size), ptr(out_keys), ptr(out_index),
+                                     stream_ptr(in_keys.device)))
+    return out_keys, out_index
+
+
+def scatter_ids_with_mask(out_ids, in_ids, mask_index):
+    """``torch.ops.recis.scatter_ids_with_mask`` (hashtable_ops.h:32-34); in place, returns ``out_ids``."""
+    require_cuda(out_ids, in_ids, mask_index)
+    if not out_ids.is_contiguous():
+        raise ValueError("out_ids must be contiguous")
+    in_ids, mask_index = _ids64(in_ids), _ids64(mask_index)
+    check(lib().recis_scatter_ids_with_mask(ptr(out_ids), i64(out_ids.numel()), ptr(in_ids),
+                                            ptr(mask_index), i64(in_ids.numel()),
+                                            stream_ptr(out_ids.device)))
+    return out_ids
+
+
+# ------------------------------------------------------------ tagging / dedup
+def ids_encode(ids_list, table_ids):
+    """``torch.ops.recis.ids_encode`` (ids_encode.h:15): tag and concatenate."""
+    ids_list = [_ids64(t) for t in ids_list]
+    tids = table_ids.tolist() if torch.is_tensor(table_ids) else list(table_ids)
+    total = sum(t.numel() for t in ids_list)
+    dev = ids_list[0].device
+    out = torch.empty(total, dtype=torch.int64, device=dev)
+    check(lib().recis_ids_encode(_host_ptrs(ids_list), _host_i64([t.numel() for t in ids_list]),
+                                 _host_i64(tids), i64(len(ids_list)), ptr(out), stream_ptr(dev)))
+    return out
+
+
+def merge_offsets(offsets_list, max_value):
+    """``torch.ops.recis.merge_offsets`` (embedding_segment_reduce.h:19-20).
+
+    ``max_value`` (host tensor or list): number of values each tensor's offsets run over."""
+    offsets_list = [_contig(o) for o in offsets_list]
+    require_cuda(*offsets_list)
+    dt = offsets_list[0].dtype
+    if any(o.dtype != dt for o in offsets_list):
+        raise TypeError("offsets must share one integer dtype")
+    is64 = _index_kind(offsets_list[0], "offsets")
+    mv = max_value.tolist() if torch.is_tensor(max_value) else list(max_value)
+    n = len(offsets_list)
+    total = sum(o.numel() for o in offsets_list) - (n - 1)
+    dev = offsets_list[0].device
+    out = torch.empty(total, dtype=dt, device=dev)
+    check(lib().recis_merge_offsets(_host_ptrs(offsets_list), _host_i64([o.numel() for o in offsets_list]),
+                                    _host_i64(mv), i64(n), is64, ptr(out), stream_ptr(dev)))
+    return out
+
+
+def ids_unique(ids, inverse_dtype=torch.int32):
+    """Dedup: ``(unique, inverse, count)`` with the unique ids in order of first
+    occurrence. ``unique`` has room for ``len(ids)`` entries, of which the first
+    ``count`` (a one-element GPU tensor) are valid: no host synchronisation."""
+    ids = _ids64(ids)
+    n = ids.numel()
+    uniq = torch.empty(n, dtype=torch.int64, device=ids.device)
+    inv = torch.empty(n, dtype=inverse_dtype, device=ids.device)
+    count = torch.empty(1, dtype=torch.int64, device=ids.device)
+    check(lib().recis_unique(ptr(ids), i64(n), ptr(uniq), ptr(inv), int(inverse_dtype == torch.int64),
+                             ptr(count), stream_ptr(ids.device)))
+    return uniq, inv, count
+
+
+_SLICE_SIZE = 65536
+
+
+def ids_partition(ids, num_parts):
+    """``torch.ops.recis.ids_partition`` (ids_partition.h:14), device ordering
+    (ids_partition_kernel.cu:36-55): unique ids ascending by ``rotr64(id, 16)`` as
+    unsigned, per-shard counts, int32 inverse. The dedup is the hash kernel; the
+    ordering of the (much smaller) unique set uses torch.sort."""
+    if ids.dim() != 1:
+        raise ValueError("ids must be 1-dim")
+    uniq, inv, count = ids_unique(ids)
+    u = uniq[: int(count.item())]
+    rot = torch.bitwise_or(torch.bitwise_left_shift(u, 48),
+                           torch.bitwise_and(torch.bitwise_right_shift(u, 16), (1 << 48) - 1))
+    order = torch.argsort(torch.bitwise_xor(rot, -(1 << 63)))  # signed sort of the flipped key = unsigned sort
+    rank = torch.empty_like(order)
+    rank[order] = torch.arange(order.numel(), device=ids.device)
+    sorted_u = u[order]
+    m, r = divmod(_SLICE_SIZE, num_parts)
+    slot = torch.bitwise_and(sorted_u, _SLICE_SIZE - 1)
+    part = torch.maximum(torch.div(slot, m + 1, rounding_mode="floor"),
+                         torch.div(slot - r, m, rounding_mode="trunc"))
+    counts = torch.bincount(part, minlength=num_parts).to(torch.int64)
+    return sorted_u, counts, rank[inv.long()].to(torch.int32)
+
+
+# --------------------------------------------------------- sparse-mode pooling
+def segment_sum(data, weight, indices, segment_ids, num_segments):
+    """``torch.ops.recis.segment_sum`` (segment_ops.h:5-8)."""
+    require_cuda(data, weight, indices, segment_ids)
+    data, indices, segment_ids = _contig(data), _contig(indices), _contig(segment_ids)
+    if indices.dtype != segment_ids.dtype:
+        raise TypeError("indices and segment_ids must share a dtype")
+    num_segments = int(num_segments)
+    D = data.shape[1]
+    out = torch.empty((num_segments, D), dtype=torch.float32, device=data.device)
+    use_w = weight is not None
+    weight = _contig(weight)
+    check(lib().recis_segment_sum(ptr(data), dtype_code(data.dtype), i64(data.shape[0]), ptr(weight),
+                                  dtype_code(weight.dtype) if use_w else 0, int(use_w), ptr(indices),
+                                  ptr(segment_ids), _index_kind(indices, "indices"), ptr(out),
+                                  i64(indices.numel()), i64(num_segments), i64(D), stream_ptr(data.device)))
+    return out if data.dtype == torch.float32 else out.to(data.dtype)
+
+
+def segment_mean(data, weight, segment_ids, num_segments):
+    """``torch.ops.recis.segment_mean`` (segment_ops.h:10-13): the normalised weights."""
+    require_cuda(data, weight, segment_ids)
+    segment_ids = _contig(segment_ids)
+    num_segments = int(num_segments)
+    n = segment_ids.numel()
+    use_w = weight is not None
+    w = _contig(weight).float() if use_w else torch.ones(1, dtype=torch.float32, device=data.device)
+    wsum = torch.empty(num_segments, dtype=torch.float32, device=data.device)
+    wnorm = torch.empty(n, dtype=torch.float32, device=data.device)
+    check(lib().recis_segment_mean_weight(ptr(w), int(use_w), ptr(segment_ids),
+                                          _index_kind(segment_ids, "segment_ids"), ptr(wsum), ptr(wnorm),
+                                          i64(n), i64(num_segments), stream_ptr(data.device)))
+    return wnorm if data.dtype == torch.float32 else wnorm.to(data.dtype)
+
+
+def gen_segment_indices_by_offset(offsets):
+    """``torch.ops.recis.gen_segment_indices_by_offset`` (embedding_segment_reduce.h:22)."""
+    require_cuda(offsets)
+    offsets = _contig(offsets)
+    S = offsets.numel() - 1
+    total = int(offsets[-1].item())  # the reference reads it back too (.item() at :405)
+    out = torch.empty(total, dtype=offsets.dtype, device=offsets.device)
+    check(lib().recis_gen_segment_indices(ptr(offsets), _index_kind(offsets, "offsets"), i64(S), ptr(out),
+                                          i64(total), stream_ptr(offsets.device)))
+    return out
+
+
+# ------------------------------------------------------------ padded gather
+def ragged_tile(batch, seq, value, offset, table):
+    """``torch.ops.recis.ragged_tile`` (ragged_tile.h:9-13). Returns ``[out, batch_seq]``;
+    ``batch_seq`` is the [3 * (n + 1)] bookkeeping tensor the reference's backward expects
+    (cumulative batch, cumulative batch*seq, seq per feature)."""
+    require_cuda(value, offset, table)
+    value, offset, table = _contig(value), _contig(offset), _contig(table)
+    batch, seq = [int(b) for b in batch], [int(s) for s in seq]
+    D = table.shape[1]
+    rows = sum(b * s for b, s in zip(batch, seq))
+    out = torch.empty((rows, D), dtype=table.dtype, device=table.device)
+    check(lib().recis_ragged_tile(_host_i64(batch), _host_i64(seq), i64(len(batch)), ptr(value),
+                                  _index_kind(value, "value"), i64(value.numel()), ptr(offset),
+                                  _index_kind(offset, "offset"), ptr(table), i64(table.shape[0]),
+                                  dtype_code(table.dtype), ptr(out), i64(D), stream_ptr(table.device)))
+    cum = [0, 0, 0]
+    ba = bs = 0
+    for b, s in zip(batch, seq):
+        ba += b
+        bs += b * s
+        cum += [ba, bs, s]
+    return [out, torch.tensor(cum, dtype=torch.int64)]
+
+
+def ragged_tile_back(batch_seq, batch_info, value, offset, dy):
+    """``torch.ops.recis.ragged_tile_back`` (ragged_tile.h:15-18).
+    ``batch_info`` = [table_rows, n_features, batch_max, seq_min]."""
+    require_cuda(value, offset, dy)
+    value, offset, dy = _contig(value), _contig(offset), _contig(dy)
+    cum = batch_seq.tolist()
+    n = int(batch_info[1])
+    batch = [cum[3 * (f + 1)] - cum[3 * f] for f in range(n)]
+    seq = [cum[3 * (f + 1) + 2] for f in range(n)]
+    table_rows = int(batch_info[0])
+    D = dy.shape[1]
+    out = torch.empty((table_rows, D), dtype=torch.float32, device=dy.device)
+    check(lib().recis_ragged_tile_back(_host_i64(batch), _host_i64(seq), i64(n), ptr(value),
+                                       _index_kind(value, "value"), i64(value.numel()), ptr(offset),
+                                       _index_kind(offset, "offset"), ptr(dy), dtype_code(dy.dtype),
+                                       ptr(out), i64(table_rows), i64(D), stream_ptr(dy.device)))
+    return out if dy.dtype == torch.float32 else out.to(dy.dtype)
+
+
+# ------------------------------------------------------------- feature ops
+def fused_uint64_mod(inputs, mods):
+    """``torch.ops.recis.fused_uint64_mod`` (fused_uint64_mod.h)."""
+    inputs = [_ids64(t) for t in inputs]
+    mods = mods.tolist() if torch.is_tensor(mods) else list(mods)
+    outs = [torch.empty_like(t) for t in inputs]
+    if inputs:
+        check(lib().recis_fused_uint64_mod(_host_ptrs(inputs), _host_i64([t.numel() for t in inputs]),
+                                           _host_i64(mods), _host_ptrs(outs), i64(len(inputs)),
+                                           stream_ptr(inputs[0].device)))
+    return outs
+
+
+def uint64_mod(inputs, num):
+    """``torch.ops.recis.uint64_mod`` (uint64_mod.h)."""
+    shape = inputs.shape
+    return fused_uint64_mod([inputs], [int(num)])[0].view(shape)
+
+
+def fused_bucketized(inputs, boundaries):
+    """``torch.ops.recis.fused_bucketized`` (fused_bucketized.h); the outputs are views of one buffer."""
+    require_cuda(*inputs)
+    require_cuda(*boundaries)
+    inputs = [_contig(t).view(-1) for t in inputs]
+    boundaries = [_contig(b) for b in boundaries]
+    for t in list(inputs) + list(boundaries):
+        if t.dtype != torch.float32:
+            raise TypeError("fused_bucketized takes float32 values and boundaries")
+    if not inputs:
+        return []
+    sizes = [t.numel() for t in inputs]
+    buf = torch.empty(sum(sizes), dtype=torch.int64, device=inputs[0].device)
+    outs = list(torch.split(buf, sizes))
+    check(lib().recis_fused_bucketized(_host_ptrs(inputs), _host_i64(sizes), _host_ptrs(boundaries),
+                                       _host_i64([b.numel() for b in boundaries]), _host_ptrs(outs),
+                                       i64(len(inputs)), stream_ptr(inputs[0].device)))
+    return outs
+
+
+def bucketize_op(values, boundaries):
+    """``torch.ops.recis.bucketize_op`` (bucketize_op.h)."""
+    if values.dtype != torch.float32:
+        values, boundaries = values.float(), boundaries.float()
+    return fused_bucketized([values], [boundaries.float()])[0].view(values.shape)
+
+
+def fused_multi_hash(inputs, muls, primes, bucket_num):
+    """``torch.ops.recis.fused_multi_hash`` (multi_hash.h): one output per (tensor, hash)."""
+    inputs = [_ids64(t) for t in inputs]
+    jobs_in, jobs_out, sizes, m, p, b = [], [], [], [], [], []
+    for t, tm, tp, tb in zip(inputs, muls, primes, bucket_num):
+        tm = tm.tolist() if torch.is_tensor(tm) else list(tm)
+        tp = tp.tolist() if torch.is_tensor(tp) else list(tp)
+        tb = tb.tolist() if torch.is_tensor(tb) else list(tb)
+        for j in range(len(tm)):
+            jobs_in.append(t)
+            jobs_out.append(torch.empty_like(t))
+            sizes.append(t.numel())
+            m.append(tm[j])
+            p.append(tp[j])
+            b.append(tb[j])
+    if jobs_in:
+        check(lib().recis_fused_multi_hash(_host_ptrs(jobs_in), _host_i64(sizes), _host_i64(m), _host_i64(p),
+                                           _host_i64(b), _host_ptrs(jobs_out), i64(len(jobs_in)),
+                                           stream_ptr(inputs[0].device)))
+    return jobs_out
+
+
+def fused_hash(inputs, input_offsets, hash_type):
+    """``torch.ops.recis.fused_hash`` (fused_hash.h): "farm" | "murmur" over int8 byte strings."""
+    if hash_type not in ("farm", "murmur"):
+        raise RuntimeError("Unsupported hash type: %s" % hash_type)
+    require_cuda(*inputs)
+    require_cuda(*input_offsets)
+    inputs = [_contig(t) for t in inputs]
+    offs = [_contig(o) for o in input_offsets]
+    for t in inputs:
+        if t.dtype not in (torch.int8, torch.uint8):
+            raise TypeError("hash input must be int8 bytes")
+    if not inputs:
+        return []
+    is64 = _index_kind(offs[0], "offsets")
+    if any(_index_kind(o, "offsets") != is64 for o in offs):
+        raise TypeError("offsets must share one integer dtype")
+    outs = [torch.empty(o.numel() - 1, dtype=torch.int64, device=o.device) for o in offs]
+    check(lib().recis_fused_hash(_host_ptrs(inputs), _host_i64([t.numel() for t in inputs]), _host_ptrs(offs),
+                                 is64, _host_i64([o.numel() - 1 for o in offs]), _host_ptrs(outs),
+                                 i64(len(inputs)), 0 if hash_type == "farm" else 1,
+                                 stream_ptr(inputs[0].device)))
+    return outs
+
+
+# ------------------------------------------------------------------- id map
+class IdMap:
+    """GPU key -> row map with the row-index allocator (``recis_idmap_*``)."""
+
+    def __init__(self, device=None, reserve=0):
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        if self.device.type != "cuda":
+            raise _lib.RecisHipError("IdMap lives on the GPU; got device %s" % self.device)
+        self._h = ctypes.c_void_p()
+        with torch.cuda.device(self.device):
+            check(lib().recis_idmap_create(i64(reserve), ctypes.byref(self._h)))
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h is not None and h.value:
+            try:
+                lib().recis_idmap_destroy(h)
+            except Exception:
+                pass
+            self._h = None
+
+    def lookup(self, ids):
+        ids = _ids64(ids)
+        out = torch.empty(ids.numel(), dtype=torch.int64, device=ids.device)
+        check(lib().recis_idmap_lookup(self._h, ptr(ids), i64(ids.numel()), ptr(out), stream_ptr(ids.device)))
+        return out
+
+    def lookup_readonly(self, ids):
+        ids = _ids64(ids)
+        out = torch.empty(ids.numel(), dtype=torch.int64, device=ids.device)
+        check(lib().recis_idmap_lookup_readonly(self._h, ptr(ids), i64(ids.numel()), ptr(out),
+                                                stream_ptr(ids.device)))
+        return out
+
+    def erase(self, ids, index):
+        ids, index = _ids64(ids), _ids64(index)
+        if ids.numel() != index.numel():
+            raise ValueError("ids and index differ in length")
+        check(lib().recis_idmap_erase(self._h, ptr(ids), ptr(index), i64(ids.numel()), stream_ptr(ids.device)))
+
+    def stats(self):
+        """(live keys, allocator high-water mark, free-list length, slot capacity); synchronises."""
+        vals = [ctypes.c_int64(0) for _ in range(4)]
+        check(lib().recis_idmap_stats(self._h, *[ctypes.byref(v) for v in vals], stream_ptr(self.device)))
+        return tuple(v.value for v in vals)
+
+    def size(self):
+        return self.stats()[0]
+
+    def id_num(self):
+        return self.stats()[1]
+
+    def snapshot(self):
+        n = self.size()
+        ids = torch.empty(n, dtype=torch.int64, device=self.device)
+        index = torch.empty(n, dtype=torch.int64, device=self.device)
+        count = ctypes.c_int64(0)
+        check(lib().recis_idmap_snapshot(self._h, ptr(ids), ptr(index), i64(n), ctypes.byref(count),
+                                         stream_ptr(self.device)))
+        assert count.value == n, (count.value, n)
+        return ids, index
+
+    def clear(self):
+        check(lib().recis_idmap_clear(self._h, stream_ptr(self.device)))
+
+    def reserve(self, n_keys):
+        check(lib().recis_idmap_reserve(self._h, i64(n_keys), stream_ptr(self.device)))

@@ -1,0 +1,191 @@
+"""Parity of the HIP tagging / dedup / feature ops / padded gather (through the
+C ABI) with the CPU oracle and the golden vectors: everything here is integer or
+byte work and is compared bit for bit (ragged_tile copies rows: exact too; its
+backward sums in fp32: rtol 1e-5)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import ragged_offsets
+from recis_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def test_hash_kats_and_golden():
+    a = torch.tensor([0, 1, 2, 1, 2, 3], dtype=torch.int8).cuda()
+    b = torch.tensor([0, 5, 5, 5, 6, 7], dtype=torch.int8).cuda()
+    off = [torch.tensor([0, 3, 6], dtype=torch.int32).cuda()] * 2
+    farm = ops.fused_hash([a, b], off, "farm")
+    mur = ops.fused_hash([a, b], off, "murmur")
+    assert farm[0].tolist() == [-7736835464683084646, -5546720800891377920]
+    assert farm[1].tolist() == [-4442022684725028445, -909183002746659612]
+    assert mur[0].tolist() == [-4003751876240412087, -1042754718167355375]
+    assert mur[1].tolist() == [-5541886947548579749, 4434088491466393040]
+    with open(os.path.join(GOLDEN, "hash_vectors.json")) as f:
+        vec = json.load(f)["vectors"]
+    data = np.frombuffer(b"".join(bytes.fromhex(v["hex"]) for v in vec), dtype=np.uint8)
+    offs = np.concatenate([[0], np.cumsum([len(v["hex"]) // 2 for v in vec])])
+    got = ops.fused_hash([_dev(data.view(np.int8))], [_dev(offs)], "farm")[0]
+    assert got.tolist() == [v["farm"] for v in vec]
+    got = ops.fused_hash([_dev(data.view(np.int8))], [_dev(offs)], "murmur")[0]
+    assert got.tolist() == [v["murmur"] for v in vec]
+    with pytest.raises(RuntimeError):
+        ops.fused_hash([a], off[:1], "sha1")
+
+
+def test_hash_random_strings_vs_oracle(rng):
+    vals, offs = [], []
+    for t in range(5):
+        lens = rng.integers(0, 200, size=int(rng.integers(1, 3000)))
+        vals.append(rng.integers(-128, 128, size=int(lens.sum()), dtype=np.int8))
+        offs.append(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
+    for kind in ("farm", "murmur"):
+        got = ops.fused_hash([_dev(v) for v in vals], [_dev(o) for o in offs], kind)
+        for g, v, o in zip(got, vals, offs):
+            np.testing.assert_array_equal(g.cpu().numpy(), oracle.hash_strings(v, o, kind))
+
+
+def test_uint64_mod(rng):
+    xs = [rng.integers(-2**63, 2**63 - 1, size=n, dtype=np.int64) for n in (1000, 1, 65536)]
+    mods = [1000000, 7, 2**40 + 3]
+    got = ops.fused_uint64_mod([_dev(x) for x in xs], mods)
+    for g, x, m in zip(got, xs, mods):
+        np.testing.assert_array_equal(g.cpu().numpy(), oracle.uint64_mod(x, m))
+    assert ops.uint64_mod(torch.tensor([1001, 1002, 1003], device="cuda"), 1000).tolist() == [1, 2, 3]
+
+
+def test_bucketize(rng):
+    bs = [np.sort(rng.standard_normal(n)).astype(np.float32) for n in (64, 5, 9000)]
+    vs = [(rng.standard_normal(n) * 2).astype(np.float32) for n in (65536, 10, 3000)]
+    vs[0][:64] = bs[0]
+    vs[1][:5] = [np.nan, np.inf, -np.inf, bs[1][0], bs[1][-1]]
+    got = ops.fused_bucketized([_dev(v) for v in vs], [_dev(b) for b in bs])
+    for g, v, b in zip(got, vs, bs):
+        np.testing.assert_array_equal(g.cpu().numpy(), oracle.bucketize(v, b))
+    # the fused outputs are views of one buffer (fused_bucketized.cc:47-52)
+    assert got[0].untyped_storage().data_ptr() == got[1].untyped_storage().data_ptr()
+    v = torch.randn(100, device="cuda") * 3
+    b = torch.tensor([1.0, 2, 3, 4, 5], device="cuda")
+    assert torch.equal(ops.bucketize_op(v, b), torch.bucketize(v, b, right=True))
+
+
+def test_multi_hash(rng):
+    x1 = rng.integers(-2**63, 2**63 - 1, size=5000, dtype=np.int64)
+    x2 = np.array([1001, 1002, 1003], np.int64)
+    muls, primes, buckets = [1, 3, 5, 7], [28979, 46997, 66973, 82997], [1000] * 4
+    got = ops.fused_multi_hash([_dev(x1), _dev(x2)], [muls, muls], [primes, primes], [buckets, buckets])
+    exp = oracle.multi_hash(x1, muls, primes, buckets) + oracle.multi_hash(x2, muls, primes, buckets)
+    assert len(got) == 8
+    for g, e in zip(got, exp):
+        np.testing.assert_array_equal(g.cpu().numpy(), e)
+    assert [g.tolist() for g in got[4:]] == [[1, 2, 3], [3, 6, 9], [5, 10, 15], [7, 14, 21]]
+
+
+def test_ids_encode_and_merge_offsets(rng):
+    ids = [rng.integers(-2**62, 2**62, size=n, dtype=np.int64) for n in (1000, 10000, 7, 100000)]
+    tids = [0, 1, 2, 4094]
+    got = ops.ids_encode([_dev(i) for i in ids], torch.tensor(tids))
+    np.testing.assert_array_equal(got.cpu().numpy(), oracle.ids_encode(ids, tids))
+    # tests/ops/emb_segment_reduce_test.py:50-55
+    r = ops.merge_offsets([torch.tensor([0, 2, 5]).cuda(), torch.tensor([0, 3, 6]).cuda()], torch.tensor([5, 8]))
+    assert r.tolist() == [0, 2, 5, 8, 11]
+    offs = [ragged_offsets(rng, n, 0, 5) for n in (65536, 10, 300)]
+    mv = [int(o[-1]) for o in offs]
+    for dt in (np.int32, np.int64):
+        r = ops.merge_offsets([_dev(o.astype(dt)) for o in offs], mv)
+        np.testing.assert_array_equal(r.cpu().numpy(), oracle.merge_offsets(offs, mv))
+    # more tensors than one launch carries
+    many = [np.array([0, 1, 3]) for _ in range(130)]
+    r = ops.merge_offsets([_dev(o) for o in many], [3] * 130)
+    np.testing.assert_array_equal(r.cpu().numpy(), oracle.merge_offsets(many, [3] * 130))
+
+
+@pytest.mark.parametrize("n,hi", [(0, 10), (1, 10), (1000, 50), (200000, 3000), (1000000, 10**7)])
+def test_unique_first_occurrence_order(rng, n, hi):
+    ids = rng.integers(-hi, hi, size=n)
+    if n > 5:
+        ids[3] = -1  # the empty-marker value is a legal id here
+    uniq, inv, count = ops.ids_unique(_dev(ids))
+    c = int(count.item())
+    u = uniq[:c].cpu().numpy()
+    # first-occurrence order == np.unique's first indices, sorted
+    _, first = np.unique(ids, return_index=True)
+    np.testing.assert_array_equal(u, ids[np.sort(first)])
+    np.testing.assert_array_equal(u[inv.cpu().numpy()], ids)
+    uniq64, inv64, _ = ops.ids_unique(_dev(ids), inverse_dtype=torch.int64)
+    assert torch.equal(inv64, inv.long())
+
+
+@pytest.mark.parametrize("n,world", [(10, 1), (1000, 128), (100000, 256), (5000, 3)])
+def test_ids_partition_matches_oracle(rng, n, world):
+    ids = rng.integers(-n * 50, n * 50, size=n)
+    u, c, inv = ops.ids_partition(_dev(ids), world)
+    eu, ec, einv = oracle.ids_partition(ids, world)
+    np.testing.assert_array_equal(u.cpu().numpy(), eu)
+    np.testing.assert_array_equal(c.cpu().numpy(), ec)
+    np.testing.assert_array_equal(inv.cpu().numpy(), einv)
+    assert inv.dtype == torch.int32
+
+
+def test_sparse_mode_ops(rng):
+    # tests/nn/segment_ops_test.py:62-113
+    data = torch.tensor([[1.0, 1.0], [2.0, 2.0], [3.0, 3.0]]).cuda()
+    weight = torch.tensor([2.0, 3.0, 0.5, 1.0]).cuda()
+    indices = torch.tensor([2, 0, 1, 0]).cuda()
+    seg = torch.tensor([0, 1, 1, 2]).cuda()
+    wn = ops.segment_mean(data, weight, seg, 4)
+    out = ops.segment_sum(data, wn, indices, seg, 4)
+    exp = torch.tensor([[3.0, 3.0], [4.0 / 3.5, 4.0 / 3.5], [1.0, 1.0], [0.0, 0]])
+    torch.testing.assert_close(out.cpu(), exp, atol=1e-7, rtol=0)
+    n, rows, S, D = 3000, 256, 512, 128
+    d = rng.random((rows, D)).astype(np.float32)
+    w = rng.random(n).astype(np.float32)
+    idx = rng.integers(0, rows, size=n)
+    sg = rng.integers(0, S, size=n)
+    got = ops.segment_sum(_dev(d), _dev(w), _dev(idx), _dev(sg), S).cpu().numpy()
+    np.testing.assert_allclose(got, oracle.segment_sum(d, w, idx, sg, S), rtol=1e-5, atol=1e-5)
+    got = ops.segment_mean(_dev(d), _dev(w), _dev(sg), S).cpu().numpy()
+    np.testing.assert_allclose(got, oracle.segment_mean_weight(w, sg, S), rtol=1e-5, atol=1e-6)
+    got = ops.segment_mean(_dev(d), None, _dev(sg), S).cpu().numpy()
+    np.testing.assert_allclose(got, oracle.segment_mean_weight(None, sg, S), rtol=1e-5, atol=1e-6)
+    # tests/ops/emb_segment_reduce_test.py:94-98
+    assert ops.gen_segment_indices_by_offset(torch.tensor([0, 2, 5]).cuda()).tolist() == [0, 0, 1, 1, 1]
+    off = ragged_offsets(rng, 5000, 0, 7, empty_frac=0.3)
+    for dt in (np.int32, np.int64):
+        got = ops.gen_segment_indices_by_offset(_dev(off.astype(dt)))
+        np.testing.assert_array_equal(got.cpu().numpy(), oracle.gen_segment_indices(off))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ragged_tile_forward_backward(rng, dtype):
+    batch, seq = [50, 31, 7], [12, 3, 40]
+    U, D = 300, 128
+    lens = np.concatenate([rng.integers(0, 20, size=b) for b in batch])
+    off = np.concatenate([[0], np.cumsum(lens)])
+    value = rng.integers(0, U, size=int(off[-1]))
+    table = rng.standard_normal((U, D)).astype(np.float32)
+    table_t = _dev(table, dtype)
+    out, batch_seq = ops.ragged_tile(batch, seq, _dev(value), _dev(off.astype(np.int32)), table_t)
+    exp = oracle.ragged_tile(batch, seq, value, off, table_t.float().cpu().numpy())
+    np.testing.assert_array_equal(out.float().cpu().numpy(), exp)
+    dy = rng.standard_normal(exp.shape).astype(np.float32)
+    dy_t = _dev(dy, dtype)
+    back = ops.ragged_tile_back(batch_seq, [U, len(batch), max(batch), min(seq)], _dev(value),
+                                _dev(off.astype(np.int32)), dy_t)
+    exp_b = oracle.ragged_tile_back(batch, seq, value, off, dy_t.float().cpu().numpy(), U)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=5e-2)
+    np.testing.assert_allclose(back.float().cpu().numpy(), exp_b, **tol)
+    assert _lib.poll_device_errors() == 0

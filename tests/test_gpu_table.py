@@ -1,0 +1,270 @@
+"""Parity of the HIP id map, row-block ops and optimizer row updates (through the
+C ABI) with the CPU oracle. Integer / index results are compared bit for bit; the
+Adam row update is compared bit for bit too, since the kernel does the same
+double-precision arithmetic as the reference's CPU functor; Adagrad within
+rtol 1e-6."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from recis_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+# --------------------------------------------------------------------- id map
+def test_row_placement_kat_gpu():
+    m = ops.IdMap()
+    rows = m.lookup(torch.arange(2048, device="cuda"))
+    np.testing.assert_array_equal(rows.cpu().numpy(), 2047 - np.arange(2048))
+    assert m.stats()[:3] == (2048, 2048, 0)
+
+
+def test_idmap_matches_oracle_sequence(rng):
+    """Same seeded sequence of lookups / read-only lookups / deletes on both sides."""
+    g, c = ops.IdMap(), oracle.IdMap()
+    live = {}
+    for step in range(30):
+        n = int(rng.integers(0, 5000))
+        ids = np.unique(rng.integers(-1000, 20000, size=n))
+        ids = ids[(ids != -1) & (ids != -2)]  # reserved by the GPU map, as in the reference
+        got = g.lookup(_dev(ids)).cpu().numpy()
+        exp = c.lookup(ids)
+        np.testing.assert_array_equal(got, exp)
+        live.update(zip(ids.tolist(), exp.tolist()))
+        probe = rng.integers(-1500, 25000, size=3000)
+        np.testing.assert_array_equal(g.lookup_readonly(_dev(probe)).cpu().numpy(), c.lookup_readonly(probe))
+        if step % 4 == 3:
+            keys = np.array(sorted(live))
+            victims = keys[rng.random(len(keys)) < 0.25]
+            rows = np.array([live[k] for k in victims.tolist()], np.int64)
+            g.erase(_dev(victims), _dev(rows))
+            c.delete(victims, rows)
+            for k in victims.tolist():
+                del live[k]
+        lv, idn, fr, _ = g.stats()
+        assert (lv, idn, fr) == (c.size(), c.id_num(), c.free_size())
+    ids_g, idx_g = g.snapshot()
+    assert dict(zip(ids_g.cpu().tolist(), idx_g.cpu().tolist())) == live
+    assert _lib.poll_device_errors() == 0
+
+
+def test_idmap_grows_past_initial_capacity(rng):
+    g, c = ops.IdMap(), oracle.IdMap()
+    cap0 = g.stats()[3]
+    total = 0
+    while total <= cap0 // 2 + 100000:
+        ids = np.arange(total, total + 300000, dtype=np.int64) * 2654435761 % (1 << 40)
+        np.testing.assert_array_equal(g.lookup(_dev(ids)).cpu().numpy(), c.lookup(ids))
+        total += 300000
+    assert g.stats()[3] > cap0
+    probe = np.arange(0, total, 997, dtype=np.int64) * 2654435761 % (1 << 40)
+    np.testing.assert_array_equal(g.lookup_readonly(_dev(probe)).cpu().numpy(), c.lookup_readonly(probe))
+
+
+def test_idmap_duplicate_key_in_one_call_gets_one_row():
+    g = ops.IdMap()
+    ids = torch.tensor([7, 7, 9, 7, 9, 11], device="cuda")
+    rows = g.lookup(ids).cpu().numpy()
+    assert rows[0] == rows[1] == rows[3] and rows[2] == rows[4]
+    assert len({rows[0], rows[2], rows[5]}) == 3
+    assert g.stats()[0] == 3
+    again = g.lookup(ids).cpu().numpy()
+    np.testing.assert_array_equal(rows, again)
+
+
+def test_idmap_tombstone_reuse_and_clear(rng):
+    g, c = ops.IdMap(), oracle.IdMap()
+    for rnd in range(6):
+        ids = np.arange(rnd * 1000, rnd * 1000 + 50000, dtype=np.int64)
+        r = g.lookup(_dev(ids)).cpu().numpy()
+        np.testing.assert_array_equal(r, c.lookup(ids))
+        g.erase(_dev(ids[::2]), _dev(r[::2]))
+        c.delete(ids[::2], r[::2])
+    assert g.stats()[:3] == (c.size(), c.id_num(), c.free_size())
+    g.clear()
+    assert g.stats()[:3] == (0, 0, 0)
+    np.testing.assert_array_equal(g.lookup(torch.arange(5, device="cuda")).cpu().numpy(), [4, 3, 2, 1, 0])
+
+
+def test_reserved_keys_are_reported():
+    g = ops.IdMap()
+    _lib.poll_device_errors()
+    rows = g.lookup(torch.tensor([5, -1, 6], device="cuda")).cpu().numpy()
+    assert rows[1] == -1 and _lib.poll_device_errors() & _lib.DEVERR_INDEX_RANGE
+    assert g.stats()[0] == 2
+
+
+def test_allocator_ops_kats():
+    # tests/ops/hashtable_ops_test.py:16-54
+    fb = [torch.arange(100000, dtype=torch.int64, device="cuda")]
+    r = ops.generate_ids(10000, fb, 0, 101, 100000)
+    assert torch.equal(r, torch.arange(101, 10101, device="cuda").flip(0))
+    r = ops.generate_ids(10000, fb, 2000, 101, 100000)
+    assert torch.equal(r, torch.cat([torch.arange(101, 8101, device="cuda").flip(0), fb[0][:2000]]))
+    free = torch.arange(101, 10101, device="cuda")
+    ops.free_ids(free, fb, 2000, 100000)
+    ans = torch.arange(100000, device="cuda")
+    ans[2000:12000] = free
+    assert torch.equal(fb[0], ans)
+    # blocks of 10240 like the reference allocator
+    blocks = [torch.zeros(10240, dtype=torch.int64, device="cuda") for _ in range(3)]
+    ops.free_ids(torch.arange(25000, device="cuda"), blocks, 100, 10240)
+    flat = torch.cat(blocks)
+    assert torch.equal(flat[100:25100], torch.arange(25000, device="cuda"))
+    r = ops.generate_ids(20000, blocks, 25100, 7, 10240)
+    assert torch.equal(r, flat[5100:25100])
+
+
+def test_mask_key_index_and_scatter(rng):
+    n = 10000
+    mask = torch.from_numpy(rng.random(n) < 0.2).cuda()
+    ids = torch.arange(101, 101 + n, device="cuda")
+    index = ids.flip(0).clone()
+    cs = torch.cumsum(mask, 0)
+    gen = int(cs[-1])
+    new_ids, range_index = ops.mask_key_index(ids, mask, cs, gen)
+    assert torch.equal(new_ids, ids[mask])
+    assert torch.equal(range_index, torch.arange(n, device="cuda")[mask])
+    new_index = torch.arange(5000, 5000 + gen, device="cuda")
+    exp = index.clone()
+    exp[range_index] = new_index
+    assert torch.equal(ops.scatter_ids_with_mask(index, new_index, range_index), exp)
+
+
+# ------------------------------------------------------------------ row blocks
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 16), (torch.float32, 5), (torch.bfloat16, 128),
+                                     (torch.int64, 1), (torch.int8, 3), (torch.float16, 24)])
+def test_block_gather_insert(rng, dtype, D):
+    bs, nb = 37, 5
+    if dtype.is_floating_point:
+        blocks = [torch.randn(bs, D, device="cuda").to(dtype) for _ in range(nb)]
+    else:
+        blocks = [torch.randint(-100, 100, (bs, D), device="cuda").to(dtype) for _ in range(nb)]
+    flat = torch.cat(blocks)
+    ids = torch.from_numpy(rng.integers(0, bs * nb, size=500)).cuda()
+    assert torch.equal(ops.block_gather(ids, blocks, bs, -1, False), flat[ids])
+    assert torch.equal(ops.gather(ids, flat), flat[ids])
+    assert torch.equal(ops.gather(ids.int(), flat), flat[ids])
+    ro = ids.clone()
+    ro[::3] = -1
+    exp = flat[ro.clamp(min=0)]
+    exp[ro == -1] = 0
+    assert torch.equal(ops.block_gather(ro, blocks, bs, -1, True), exp)
+    assert torch.equal(ops.block_gather_by_range(ids, blocks, bs, 100, 300), flat[ids[100:300]])
+    uids = torch.from_numpy(rng.permutation(bs * nb)[:60]).cuda()
+    emb = flat[torch.from_numpy(rng.integers(0, bs * nb, size=60)).cuda()].clone()
+    ops.block_insert(uids, emb, blocks, bs)
+    flat[uids] = emb
+    assert torch.equal(torch.cat(blocks), flat)
+    ops.block_insert(uids, emb[:1], blocks, bs)
+    flat[uids] = emb[0]
+    assert torch.equal(torch.cat(blocks), flat)
+    mask = torch.from_numpy(rng.random(60) < 0.5).cuda()
+    emb2 = flat[torch.from_numpy(rng.integers(0, bs * nb, size=60)).cuda()].clone()
+    ops.block_insert_with_mask(uids, emb2, mask, blocks, bs)
+    flat[uids[mask]] = emb2[mask]
+    assert torch.equal(torch.cat(blocks), flat)
+
+
+def test_block_gather_single_big_block_and_errors(rng):
+    big = [torch.randn(5000, 32, device="cuda")]
+    ids = torch.from_numpy(rng.integers(0, 5000, size=777)).cuda()
+    assert torch.equal(ops.block_gather(ids, big, 5000), big[0][ids])
+    _lib.poll_device_errors()
+    bad = torch.tensor([1, 5000, 2], device="cuda")
+    out = ops.block_gather(bad, big, 5000)
+    assert _lib.poll_device_errors() & _lib.DEVERR_INDEX_RANGE
+    assert torch.equal(out[0], big[0][1]) and float(out[1].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dt", [torch.int64, torch.int32])
+def test_block_filter(rng, dt):
+    bs, nb = 100, 4
+    blocks = [torch.randint(0, 200, (bs, 1), device="cuda").to(dt) for _ in range(nb)]
+    flat = torch.cat(blocks)[:, 0]
+    ids = torch.from_numpy(rng.integers(0, bs * nb, size=333)).cuda()
+    assert torch.equal(ops.block_filter(ids, blocks, bs, 77), flat[ids] < 77)
+
+
+# ------------------------------------------------------------------ optimizers
+def _np_blocks(w, bs):
+    nb = (w.shape[0] + bs - 1) // bs
+    pad = np.zeros((nb * bs - w.shape[0], w.shape[1]), w.dtype)
+    w = np.concatenate([w, pad])
+    return [np.ascontiguousarray(w[i * bs:(i + 1) * bs]) for i in range(nb)]
+
+
+@pytest.mark.parametrize("beta_dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("D,bs", [(16, 64), (32, 10240), (7, 5)])
+def test_adamw_bit_exact_vs_oracle(rng, beta_dtype, D, bs):
+    U, steps = 300, 12
+    lr, b1, b2, eps, decay = 1e-3, 0.9, 0.999, 1e-8, 1 - 1e-3 * 1e-2
+    rows0 = (0.01 * rng.standard_normal((U, D))).astype(np.float32)
+    c_emb, c_m, c_v = _np_blocks(rows0, bs), _np_blocks(np.zeros_like(rows0), bs), _np_blocks(np.zeros_like(rows0), bs)
+    g_emb = [_dev(b) for b in c_emb]
+    g_m = [_dev(b) for b in c_m]
+    g_v = [_dev(b) for b in c_v]
+    cb1, cb2 = np.ones(1, beta_dtype), np.ones(1, beta_dtype)
+    gb1, gb2 = _dev(cb1), _dev(cb2)
+    step_t = torch.zeros(1, dtype=torch.int64, device="cuda")
+    for _ in range(steps):
+        idx = np.sort(rng.permutation(U)[:rng.integers(1, U)])
+        g = rng.standard_normal((len(idx), D)).astype(np.float32)
+        oracle.block_apply_adamw(idx, g, c_emb, cb1, cb2, c_m, c_v, lr, b1, b2, decay, eps, bs)
+        ops.block_apply_adamw(_dev(idx), _dev(g), g_emb, gb1, gb2, step_t, g_m, g_v, lr, b1, b2, decay, eps, bs)
+    for gl, cl in ((g_emb, c_emb), (g_m, c_m), (g_v, c_v)):
+        np.testing.assert_array_equal(torch.cat(gl).cpu().numpy(), np.concatenate(cl))
+    np.testing.assert_array_equal(gb1.cpu().numpy(), cb1)
+    np.testing.assert_array_equal(gb2.cpu().numpy(), cb2)
+    assert int(step_t) == 0  # never advances, as in the reference
+
+
+def test_adamw_empty_index_still_advances_betas():
+    emb = [torch.zeros(4, 8, device="cuda")]
+    m, v = [torch.zeros(4, 8, device="cuda")], [torch.zeros(4, 8, device="cuda")]
+    b1t = torch.ones(1, device="cuda")
+    b2t = torch.ones(1, device="cuda")
+    ops.block_apply_adamw(torch.zeros(0, dtype=torch.int64, device="cuda"), torch.zeros(0, 8, device="cuda"),
+                          emb, b1t, b2t, torch.zeros(1, dtype=torch.int64, device="cuda"), m, v,
+                          1e-3, 0.9, 0.999, 1.0, 1e-8, 4)
+    assert abs(float(b1t) - 0.9) < 1e-7 and abs(float(b2t) - 0.999) < 1e-7
+
+
+@pytest.mark.parametrize("D,bs", [(16, 128), (128, 33)])
+def test_adagrad_vs_oracle(rng, D, bs):
+    U, steps, lr, eps = 200, 15, 0.01, 1e-8
+    rows0 = (0.01 * rng.standard_normal((U, D))).astype(np.float32)
+    c_emb, c_acc = _np_blocks(rows0, bs), _np_blocks(np.zeros_like(rows0), bs)
+    g_emb, g_acc = [_dev(b) for b in c_emb], [_dev(b) for b in c_acc]
+    for _ in range(steps):
+        idx = np.sort(rng.permutation(U)[:rng.integers(1, U)])
+        g = rng.standard_normal((len(idx), D)).astype(np.float32)
+        oracle.block_apply_adagrad(idx, g, c_emb, c_acc, lr, eps, bs)
+        ops.block_apply_adagrad(_dev(idx), _dev(g), g_emb, g_acc, lr, eps, bs)
+    np.testing.assert_allclose(torch.cat(g_emb).cpu().numpy(), np.concatenate(c_emb), rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(torch.cat(g_acc).cpu().numpy(), np.concatenate(c_acc), rtol=1e-6, atol=1e-8)
+
+
+def test_bf16_rows_fp32_grads_track_fp32_path(rng):
+    """bf16 row storage: compared with the fp32 oracle within rtol 1e-2 (there is no
+    bf16 CPU path in the reference)."""
+    U, D, bs, lr, eps = 128, 64, 128, 0.05, 1e-8
+    rows0 = rng.standard_normal((U, D)).astype(np.float32)
+    c_emb, c_acc = _np_blocks(rows0, bs), _np_blocks(np.zeros_like(rows0), bs)
+    g_emb = [_dev(b, torch.bfloat16) for b in c_emb]
+    g_acc = [_dev(b, torch.bfloat16) for b in c_acc]
+    idx = np.arange(U)
+    for _ in range(3):
+        g = rng.standard_normal((U, D)).astype(np.float32)
+        oracle.block_apply_adagrad(idx, g, c_emb, c_acc, lr, eps, bs)
+        ops.block_apply_adagrad(_dev(idx), _dev(g), g_emb, g_acc, lr, eps, bs)
+    np.testing.assert_allclose(torch.cat(g_emb).float().cpu().numpy(), np.concatenate(c_emb), rtol=2e-2, atol=2e-2)
