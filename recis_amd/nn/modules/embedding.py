@@ -1,0 +1,152 @@
+"""``EmbeddingOption`` and ``DynamicEmbedding``: the mirror of
+``recis.nn.modules.embedding`` (embedding.py:161-624) for one GPU that owns the whole
+table (world size 1: the id / row / gradient all-to-alls of the reference are the
+identity and are left out)."""
+import json
+import math
+import os
+from dataclasses import dataclass, field
+from typing import List, Optional, Union
+
+import torch
+
+from ... import ops
+from ...ragged.tensor import RaggedTensor
+from ..functional.embedding_ops import ragged_embedding_segment_reduce
+from ..hashtable_hook import AdmitHook, FilterHook
+from ..initializers import ConstantInitializer, Initializer
+from .hashtable import (GradIDMeanFunction, HashTable, HashTableLookupHelpFunction, gen_slice)
+
+
+@dataclass
+class EmbeddingOption:
+    embedding_dim: int = 16
+    block_size: int = 10240
+    dtype: torch.dtype = torch.float32
+    device: torch.device = torch.device("cuda")
+    trainable: bool = True
+    pg: object = None
+    max_partition_num: int = 65536
+    shared_name: str = "embedding"
+    children: List[str] = field(default_factory=list)
+    coalesced: Optional[bool] = False
+    initializer: Optional[Initializer] = None
+    use_weight: Optional[bool] = True
+    combiner: Optional[str] = "sum"
+    combiner_kwargs: Optional[dict] = None
+    grad_reduce_by: Optional[str] = "worker"
+    filter_hook: Optional[FilterHook] = None
+    admit_hook: Optional[AdmitHook] = None
+    fp16_enabled: bool = False
+    reserve_rows: int = 0  # addition: pre-size the map and the row storage
+
+    def __post_init__(self):
+        if not self.children:
+            self.children = [self.shared_name]
+        if self.initializer is None:
+            self.initializer = ConstantInitializer(init_val=0)
+        if self.fp16_enabled:
+            assert self.dtype in (torch.int8,), "only int8 emb can set fp16_enabled"
+        assert self.combiner in ["sum", "mean", "tile", "max"], \
+            "Hashtable combiner only support [sum/mean/tile/max], but got %s" % self.combiner
+        if self.combiner == "tile":
+            if self.combiner_kwargs is None:
+                raise RuntimeError("combiner_kwargs must be set when combiner is tile.")
+            if "tile_len" not in self.combiner_kwargs:
+                raise RuntimeError("tile_len must be in combiner_kwargs when combiner is tile.")
+
+    def coalesced_info(self):
+        return json.dumps({
+            "dim": self.embedding_dim, "dtype": str(self.dtype), "device": str(torch.device(self.device).type),
+            "initializer": str(self.initializer), "grad_reduce_by": self.grad_reduce_by,
+            "filter_hook": str(self.filter_hook),
+        })
+
+    def runtime_info(self):
+        return json.dumps({
+            "combiner": self.combiner, "use_weight": self.use_weight, "trainable": self.trainable,
+            "admit_hook": str(self.admit_hook), "fp16_enabled": self.fp16_enabled,
+        })
+
+
+def lookup_unique_rows(hashtable: HashTable, unique_ids, admit_hook=None, trainable=True):
+    """Rows of ids that are already unique: the lookup autograd function, the
+    last-seen-step stamp, no second dedup."""
+    from .hashtable_hook_impl import HashtableHookFactory
+
+    impl = hashtable._hashtable_impl
+    float_table = hashtable._dtype not in (torch.int8, torch.int32, torch.int64)
+    if hashtable.training and trainable and float_table:
+        admit_impl = HashtableHookFactory().create_admit_hook(hashtable, admit_hook) if admit_hook else None
+        emb_idx, emb = HashTableLookupHelpFunction.apply(unique_ids, impl, hashtable._backward_holder, admit_impl)
+        hashtable._filter_hook_impl(emb_idx)
+        return emb
+    readonly = (not hashtable.training) or admit_hook is not None or not float_table
+    _, emb = impl.embedding_lookup(unique_ids.detach(), readonly)
+    if hashtable.training and not readonly:
+        hashtable._filter_hook_impl(_)
+    return emb
+
+
+class DynamicEmbedding(torch.nn.Module):
+    def __init__(self, emb_opt: EmbeddingOption, pg=None):
+        super().__init__()
+        self._emb_opt = emb_opt
+        self._world_size = int(os.environ.get("WORLD_SIZE", 1))
+        self._rank = int(os.environ.get("RANK", 0))
+        if self._world_size != 1:
+            raise NotImplementedError("this build runs one GPU that owns the whole table (WORLD_SIZE=1)")
+        self._hashtable = HashTable(
+            embedding_shape=[emb_opt.embedding_dim], block_size=emb_opt.block_size, dtype=emb_opt.dtype,
+            device=emb_opt.device, initializer=emb_opt.initializer, children=emb_opt.children,
+            name=emb_opt.shared_name, coalesced=emb_opt.coalesced,
+            slice=gen_slice(shard_index=self._rank, shard_num=self._world_size),
+            grad_reduce_by=emb_opt.grad_reduce_by, filter_hook=emb_opt.filter_hook,
+            reserve_rows=emb_opt.reserve_rows)
+
+    def deal_with_tensor(self, input_tensor: Union[torch.Tensor, RaggedTensor]):
+        if isinstance(input_tensor, RaggedTensor):
+            val = input_tensor.values()
+            weight = input_tensor.weight()
+            offsets = input_tensor.offsets()[-1]
+            shape = input_tensor.real_shape(0, -1)
+            if not math.prod(shape) == (offsets.numel() - 1):
+                raise RuntimeError("RaggedTensor must pad before lookup, got: %s" % input_tensor)
+        elif isinstance(input_tensor, torch.Tensor):
+            if input_tensor.is_sparse:
+                raise TypeError("RaggedDynamicEmbedding doesn't support sparse ids")
+            val = input_tensor.reshape(-1)
+            bs, fea_dim = input_tensor.shape[0], input_tensor.shape[1]
+            offsets = torch.arange(bs + 1, device=val.device) * fea_dim
+            weight = None
+            shape = tuple(input_tensor.shape[:-1])
+        else:
+            raise TypeError("DynamicEmbedding only support RaggedTensor or dense tensor, got %s" % type(input_tensor))
+        return val, offsets, weight, shape
+
+    def forward(self, input_ids, input_weights=None):
+        opt = self._emb_opt
+        val, offsets, weight, shape = self.deal_with_tensor(input_ids)
+        dev = self._hashtable._hashtable_impl.device
+        val, offsets = val.to(dev), offsets.to(dev)
+        if input_weights is not None:
+            weight = input_weights
+        if weight is not None:
+            weight = weight.to(dev) if opt.use_weight else None
+        uniq, inverse, count = ops.ids_unique(val, inverse_dtype=torch.int32)
+        uniq = uniq[: int(count.item())]
+        emb = lookup_unique_rows(self._hashtable, uniq, opt.admit_hook, opt.trainable)
+        if opt.grad_reduce_by == "id" and self.training and opt.trainable:
+            # mean over the duplicates of each id: pool the expanded rows instead
+            emb = GradIDMeanFunction.apply(emb, inverse.long())
+            inverse = torch.arange(val.numel(), device=dev, dtype=torch.int32)
+        if weight is not None and weight.dtype != emb.dtype:
+            weight = weight.to(emb.dtype)
+        out = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner, opt.combiner_kwargs)
+        if opt.combiner == "tile":
+            return out.view(tuple(shape) + (opt.combiner_kwargs["tile_len"] * opt.embedding_dim,))
+        return out.view(tuple(shape) + (opt.embedding_dim,))
+
+    @property
+    def hashtable(self):
+        return self._hashtable

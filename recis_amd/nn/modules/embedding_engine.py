@@ -1,0 +1,139 @@
+"""``EmbeddingEngine``: looks up many features in one go (mirror of
+``recis.nn.modules.embedding_engine``, embedding_engine.py:17-832).
+
+Features whose options agree on dim / dtype / device / initializer / gradient
+reduction / filter hook are coalesced into ONE physical table, each feature's ids
+tagged with a 12-bit table index (embedding_engine.py:607-625, ids_encode). Within a
+table, features that also agree on combiner / use_weight / trainable / admit hook
+form one runtime group and are processed together:
+
+    ids_encode + merge_offsets  ->  dedup (hash)  ->  find-or-insert + row gather
+    ->  segment reduce over all the group's segments  ->  split per feature
+
+which is the reference's group_exchange_ids / group_exchange_embs / group_reduce
+pipeline with the all-to-alls removed (one GPU owns the whole table).
+"""
+import hashlib
+from collections import OrderedDict
+from typing import Dict, Union
+
+import torch
+
+from ... import ops
+from ...ragged.tensor import RaggedTensor
+from ..functional.embedding_ops import ragged_embedding_segment_reduce
+from .embedding import EmbeddingOption, lookup_unique_rows
+from .hashtable import HashTable, gen_slice
+
+
+def _key(text):
+    return hashlib.sha256(text.encode()).hexdigest()[:16]
+
+
+class _TableGroup:
+    def __init__(self, key, first_opt):
+        self.key = key
+        self.opt = first_opt
+        self.children = []          # shared names in order of first appearance
+        self.features = OrderedDict()  # feature name -> option
+
+
+class EmbeddingEngine(torch.nn.Module):
+    def __init__(self, emb_options: Dict[str, EmbeddingOption]):
+        super().__init__()
+        self._emb_options = OrderedDict(emb_options)
+        self._groups = OrderedDict()
+        for name, opt in self._emb_options.items():
+            gkey = _key(opt.coalesced_info())
+            grp = self._groups.get(gkey)
+            if grp is None:
+                grp = self._groups[gkey] = _TableGroup(gkey, opt)
+            if opt.shared_name not in grp.children:
+                grp.children.append(opt.shared_name)
+            grp.features[name] = opt
+        self._tables = torch.nn.ModuleDict()
+        for gkey, grp in self._groups.items():
+            opt = grp.opt
+            coalesced = len(grp.children) > 1
+            table_name = grp.children[0] if not coalesced else "CoalescedHashtable_" + gkey
+            reserve = sum(o.reserve_rows for o in grp.features.values())
+            self._tables[gkey] = HashTable(
+                embedding_shape=[opt.embedding_dim], block_size=opt.block_size, dtype=opt.dtype,
+                device=opt.device, coalesced=coalesced, children=list(grp.children), slice=gen_slice(0, 1),
+                initializer=opt.initializer, name=table_name, grad_reduce_by=opt.grad_reduce_by,
+                filter_hook=opt.filter_hook, reserve_rows=reserve)
+
+    def hashtables(self):
+        return {t._name: t for t in self._tables.values()}
+
+    @staticmethod
+    def _format(name, opt, data):
+        """(values int64 [N], weight | None, offsets int32 [S+1], output shape prefix)."""
+        if isinstance(data, RaggedTensor):
+            values = data.values()
+            offsets = data.offsets()[-1]
+            weight = data.weight() if opt.use_weight else None
+            shape = tuple(data.real_shape(0, -1))
+            prod = 1
+            for d in shape:
+                prod *= d
+            if prod != offsets.numel() - 1:
+                raise RuntimeError("RaggedTensor must pad before lookup, got: %s (%s)" % (data, name))
+        elif isinstance(data, torch.Tensor):
+            if data.dim() == 1:
+                data = data.view(-1, 1)
+            values = data.reshape(-1)
+            width = data.shape[-1]
+            rows = values.numel() // width
+            offsets = torch.arange(rows + 1, device=data.device, dtype=torch.int32) * width
+            weight = None
+            shape = tuple(data.shape[:-1])
+        else:
+            raise TypeError("feature %s: expected RaggedTensor or Tensor, got %s" % (name, type(data)))
+        if values.dtype != torch.int64:
+            values = values.long()
+        return values, weight, offsets.to(torch.int32), shape
+
+    def forward(self, inputs: Dict[str, Union[torch.Tensor, RaggedTensor]]):
+        outputs = {}
+        for gkey, grp in self._groups.items():
+            table = self._tables[gkey]
+            dev = table._hashtable_impl.device
+            info = table._hashtable_impl.children_info()
+            runtime = OrderedDict()
+            for name, opt in grp.features.items():
+                if name in inputs:
+                    runtime.setdefault(opt.runtime_info(), []).append(name)
+            for names in runtime.values():
+                opt0 = grp.features[names[0]]
+                vals, weights, offs, shapes, tags = [], [], [], [], []
+                for name in names:
+                    v, w, o, shape = self._format(name, grp.features[name], inputs[name])
+                    vals.append(v.to(dev))
+                    offs.append(o.to(dev))
+                    if w is None and opt0.use_weight and any(
+                            isinstance(inputs[n], RaggedTensor) and inputs[n].weight() is not None for n in names):
+                        w = torch.ones(v.numel(), device=dev)
+                    weights.append(None if w is None else w.to(dev))
+                    shapes.append(shape)
+                    tags.append(info.child_index(grp.features[name].shared_name))
+                if info.is_coalesce():
+                    ids = ops.ids_encode(vals, tags)
+                else:
+                    ids = vals[0] if len(vals) == 1 else torch.cat(vals)
+                offsets = offs[0] if len(offs) == 1 else ops.merge_offsets(offs, [v.numel() for v in vals])
+                weight = None
+                if all(w is not None for w in weights):
+                    weight = weights[0] if len(weights) == 1 else torch.cat(weights)
+                uniq, inverse, count = ops.ids_unique(ids, inverse_dtype=torch.int32)
+                uniq = uniq[: int(count.item())]
+                emb = lookup_unique_rows(table, uniq, opt0.admit_hook, opt0.trainable)
+                if weight is not None and weight.dtype != emb.dtype:
+                    weight = weight.to(emb.dtype)
+                pooled = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt0.combiner,
+                                                         opt0.combiner_kwargs)
+                seg_counts = [o.numel() - 1 for o in offs]
+                width = pooled.shape[1]
+                for name, part, shape in zip(names, torch.split(pooled, seg_counts), shapes):
+                    outputs[name] = part.reshape(tuple(shape) + (width,))
+        return outputs

@@ -1,0 +1,716 @@
+"""Dynamic hash table: host-side mirror of ``recis.nn.modules.hashtable`` and of the
+native classes behind it (``HashtableImpl``, ``SlotGroup``, ``Slot``,
+``ChildrenInfo``: csrc/embedding/hashtable.cc:46-313, slot_group.cc:26-201,
+children_info.h:12-37, registered at csrc/bind.cc:47-109).
+
+The table lives in GPU memory: the key -> row map is the HIP ``IdMap`` and every
+slot (the embedding rows, optimizer state, the last-seen step) is EmbeddingBlocks
+storage read and written by the HIP row kernels. There is no CPU-resident mode.
+
+Storage layout. The reference grows every slot one ``[block_size, D]`` tensor at a
+time. Here a slot is a short list of large chunks, each a whole number of blocks;
+``Slot.values()`` still hands out one aliasing ``[block_size, D]`` view per block,
+while the kernels address the chunks directly (a chunk is simply a bigger block,
+so the row arithmetic ``row // size, row % size`` is the same). Rows are
+initialised by the slot's generator when their chunk is allocated.
+"""
+import json
+import os
+from typing import List, Optional, Tuple
+
+import torch
+
+from ... import ops
+from ..._lib import RecisHipError
+from ..hashtable_hook import AdmitHook, FilterHook
+from ..initializers import ConstantInitializer
+
+_CHUNK_BYTES = 8 << 20
+
+
+class Slice:
+    def __init__(self, slice_begin, slice_end, slice_size):
+        self.slice_begin, self.slice_end, self.slice_size = slice_begin, slice_end, slice_size
+
+
+_default_slice = Slice(0, 65536, 65536)
+
+
+def gen_slice(shard_index=0, shard_num=1, slice_size=65536):
+    """Key-space range of one shard (recis/nn/modules/hashtable.py:48-92): ``slice_size``
+    slots split into ``shard_num`` contiguous ranges, the first ``slice_size % shard_num``
+    one longer."""
+    base, extra = divmod(slice_size, shard_num)
+    begin = shard_index * base + min(shard_index, extra)
+    return Slice(begin, begin + base + (1 if shard_index < extra else 0), slice_size)
+
+
+class HashtableRegister:
+    """Process-wide registry that rejects two tables with one name and different
+    configuration (recis/nn/modules/hashtable.py:674-731)."""
+
+    _instance = None
+
+    def __new__(cls):
+        if cls._instance is None:
+            cls._instance = super().__new__(cls)
+            cls._instance._tables = {}
+        return cls._instance
+
+    def register(self, name, info):
+        if name in self._tables:
+            raise ValueError("duplicate hashtable name: %s" % name)
+        self._tables[name] = info
+
+    def clear(self):
+        self._tables.clear()
+
+
+class ChildrenInfo:
+    """12-bit table tag / 52-bit id packing for coalesced tables (children_info.h:12-37)."""
+
+    def __init__(self, coalesce, children):
+        self._coalesce = bool(coalesce)
+        self._children = list(children)
+        if len(self._children) > self.max_children_num():
+            raise RuntimeError("too many children: %d" % len(self._children))
+        if not self._coalesce and len(self._children) != 1:
+            raise RuntimeError("a table that is not coalesced has exactly one child")
+
+    def index_bits_num(self):
+        return 12
+
+    def id_bits_num(self):
+        return 52
+
+    def index_mask(self):
+        return -(1 << 52)
+
+    def id_mask(self):
+        return (1 << 52) - 1
+
+    def max_children_num(self):
+        return 4095
+
+    def encode_id(self, id_, index):
+        v = (id_ & self.id_mask()) | ((index << 52) & 0xFFFFFFFFFFFFFFFF)
+        return v - (1 << 64) if v >= (1 << 63) else v
+
+    def children(self):
+        return list(self._children)
+
+    def child_index(self, name):
+        return self._children.index(name)
+
+    def has_child(self, name):
+        return name in self._children
+
+    def child_at(self, index):
+        return self._children[index]
+
+    def is_coalesce(self):
+        return self._coalesce
+
+
+class Slot:
+    """One named column of the table (slot_group.h:17-58)."""
+
+    def __init__(self, name, block_size, dtype, partial_shape, generator, device, chunk_rows):
+        self._name = name
+        self._block_size = block_size
+        self._dtype = dtype
+        self._row_shape = list(partial_shape[1:])
+        self._generator = generator
+        self._device = device
+        self._chunk_rows = chunk_rows
+        self._chunks = []
+        self._visible_blocks = 0
+        generator.set_device(device)
+
+    # -- reference surface
+    def block_size(self):
+        return self._block_size
+
+    def name(self):
+        return self._name
+
+    def flat_size(self):
+        n = 1
+        for d in self._row_shape:
+            n *= d
+        return n
+
+    def dtype(self):
+        return self._dtype
+
+    def values(self):
+        """One ``[block_size, D]`` view per block; the views alias live storage."""
+        per = self._chunk_rows // self._block_size
+        out = []
+        for b in range(self._visible_blocks):
+            c, k = divmod(b, per)
+            out.append(self._chunks[c][k * self._block_size:(k + 1) * self._block_size])
+        return out
+
+    def value(self):
+        rows = self._visible_blocks * self._block_size
+        if rows == 0:
+            return torch.empty([0] + self._row_shape, dtype=self._dtype, device=self._device)
+        full, rest = divmod(rows, self._chunk_rows)
+        parts = self._chunks[:full] + ([self._chunks[full][:rest]] if rest else [])
+        return torch.cat(parts, 0)
+
+    def index_select(self, index, beg=0, end=None):
+        end = index.numel() if end is None else end
+        return ops.block_gather_by_range(index, self._chunks, self._chunk_rows, beg, end)
+
+    def index_insert(self, index, value, accept_indicator=None):
+        if value.dim() == 0:
+            value = value.view(1)
+        if value.dim() == 1 and self._row_shape == [1]:
+            value = value.view(-1, 1)
+        value = value.to(device=self._device, dtype=self._dtype)
+        if accept_indicator is None:
+            ops.block_insert(index, value, self._chunks, self._chunk_rows)
+        else:
+            ops.block_insert_with_mask(index, value, accept_indicator, self._chunks, self._chunk_rows)
+
+    def gen_val(self, rows):
+        return self._generator.generate([rows] + self._row_shape)
+
+    # -- storage management
+    def kernel_blocks(self):
+        """(chunk list, rows per chunk): what the row kernels take as (blocks, block_size)."""
+        return self._chunks, self._chunk_rows
+
+    def _ensure_chunks(self, n_chunks):
+        while len(self._chunks) < n_chunks:
+            self._chunks.append(self._generator.generate([self._chunk_rows] + self._row_shape))
+
+    def _clear(self):
+        self._chunks = []
+        self._visible_blocks = 0
+
+
+class SlotGroup:
+    """All slots of one table; they grow together (slot_group.h:60-90)."""
+
+    def __init__(self, block_size, device, chunk_rows):
+        self._block_size = block_size
+        self._device = device
+        self._chunk_rows = chunk_rows
+        self._slots = []
+        self._name_to_index = {}
+        self._emb_slot_index = -1
+        self._n_chunks = 0
+        self._block_num = 0
+
+    @staticmethod
+    def emb_slot_name():
+        return "embedding"
+
+    def append_slot(self, name, dtype, partial_shape, generator=None, init_val=0.0):
+        if name in self._name_to_index:
+            raise RuntimeError("slot %r already exists" % name)
+        if generator is None:
+            generator = ConstantInitializer(init_val)
+            generator.set_shape([self._block_size] + list(partial_shape[1:]))
+            generator.set_dtype(dtype)
+            generator = generator.build().impl()
+        slot = Slot(name, self._block_size, dtype, partial_shape, generator, self._device, self._chunk_rows)
+        slot._ensure_chunks(self._n_chunks)  # a late slot catches up with the table
+        slot._visible_blocks = self._block_num
+        self._slots.append(slot)
+        self._name_to_index[name] = len(self._slots) - 1
+        return slot
+
+    def append_emb_slot(self, dtype, partial_shape, generator):
+        self.append_slot(self.emb_slot_name(), dtype, partial_shape, generator)
+        self._emb_slot_index = len(self._slots) - 1
+
+    def append_step_filter_slot(self, name, init_step):
+        return self.append_slot(name, torch.int64, [self._block_size, 1], init_val=int(init_step))
+
+    def slot_by_name(self, name):
+        return self._slots[self._name_to_index[name]]
+
+    def slot_by_index(self, index):
+        return self._slots[index]
+
+    slot_index = slot_by_index  # the reference binds this name to GetSlotByIndex (bind.cc:70)
+
+    def get_slot_index(self, name):
+        return self._name_to_index[name]
+
+    def slots(self):
+        return list(self._slots)
+
+    def emb_slot(self):
+        return self._slots[self._emb_slot_index]
+
+    def block_size(self):
+        return self._block_size
+
+    def block_num(self):
+        return self._block_num
+
+    def capacity_rows(self):
+        return self._n_chunks * self._chunk_rows
+
+    def ensure_rows(self, rows):
+        need = (rows + self._chunk_rows - 1) // self._chunk_rows
+        if need > self._n_chunks:
+            self._n_chunks = need
+            for s in self._slots:
+                s._ensure_chunks(need)
+
+    def set_block_num(self, block_num):
+        if block_num > self._block_num:
+            self.ensure_rows(block_num * self._block_size)
+            self._block_num = block_num
+            for s in self._slots:
+                s._visible_blocks = block_num
+
+    def clear(self):
+        for s in self._slots:
+            s._clear()
+        self._n_chunks = 0
+        self._block_num = 0
+
+
+class HashtableImpl:
+    """Counterpart of ``torch.classes.recis.HashtableImpl`` (bind.cc:92-109)."""
+
+    hashtable_tag = -1
+
+    def __init__(self, block_size, embedding_shape, dtype, device, coalesce, children, generator,
+                 slice_begin=0, slice_end=65536, slice_size=65536, reserve_rows=0):
+        device = torch.device(device)
+        if device.type != "cuda":
+            raise RecisHipError("tables live in GPU memory in this build; got device %s" % device)
+        if device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        self._device = device
+        self._dtype = dtype
+        self._embedding_shape = list(embedding_shape)
+        row_bytes = torch.empty((), dtype=dtype).element_size()
+        for d in embedding_shape:
+            row_bytes *= d
+        if reserve_rows > 0:
+            chunk_rows = -(-int(reserve_rows + 1) // block_size) * block_size
+        else:
+            chunk_rows = max(1, _CHUNK_BYTES // max(1, row_bytes * block_size)) * block_size
+        self._slot_group = SlotGroup(block_size, device, chunk_rows)
+        self._slot_group.append_emb_slot(dtype, [block_size] + self._embedding_shape, generator)
+        self._children_info = ChildrenInfo(coalesce, children)
+        self._slice = Slice(slice_begin, slice_end, slice_size)
+        self._idmap = ops.IdMap(device, reserve=reserve_rows)
+        self._rows_ub = 0  # upper bound of the allocator's high-water mark
+        self._grad_index, self._grad, self._grad_unique = [], [], []
+
+    # ------------------------------------------------------------- storage
+    def _make_room(self, incoming):
+        """After a find-or-insert of ``incoming`` keys: rows up to the allocator's
+        high-water mark (+1 spare) must exist before any row kernel runs. The exact
+        mark is read back only when the running upper bound passes the capacity."""
+        sg = self._slot_group
+        self._rows_ub += incoming
+        if self._rows_ub + 1 > sg.capacity_rows():
+            self._rows_ub = self._idmap.id_num()  # synchronises
+            if self._rows_ub + 1 > sg.capacity_rows():
+                sg.ensure_rows(self._rows_ub + 1 + max(2 * incoming, sg.block_size()))
+        if sg.capacity_rows() == 0:
+            sg.ensure_rows(1)
+
+    def _sync_block_num(self):
+        """block_num = (id_num + block_size) / block_size (hashtable.cc:255-261)."""
+        sg = self._slot_group
+        id_num = self._idmap.id_num()
+        self._rows_ub = id_num
+        sg.set_block_num((id_num + sg.block_size()) // sg.block_size())
+
+    # ------------------------------------------------------------- lookups
+    def embedding_lookup(self, ids, readonly=False):
+        ids = ids.to(self._device)
+        if ids.dtype != torch.int64:
+            ids = ids.long()
+        if readonly:
+            index = self._idmap.lookup_readonly(ids)
+            self._make_room(0)
+        else:
+            index = self._idmap.lookup(ids)
+            self._make_room(ids.numel())
+        chunks, chunk_rows = self._slot_group.emb_slot().kernel_blocks()
+        emb = ops.block_gather(index, chunks, chunk_rows, -1, bool(readonly))
+        return index, emb
+
+    def insert_lookup_index(self, ids):
+        ids = ids.to(self._device)
+        index = self._idmap.lookup(ids)
+        self._make_room(ids.numel())
+        return index
+
+    def insert(self, ids, embedding):
+        slot = self._slot_group.emb_slot()
+        if embedding.dtype != slot.dtype():
+            raise RuntimeError("embeding type must be [%s] but get %s" % (slot.dtype(), embedding.dtype))
+        if ids.shape[0] != embedding.shape[0]:
+            raise RuntimeError("size of ids and embedding dismatch, ids: %d embedding: %d"
+                               % (ids.shape[0], embedding.shape[0]))
+        index = self.insert_lookup_index(ids)
+        slot.index_insert(index, embedding.to(self._device))
+
+    def lookup_index_readonly(self, ids):
+        return self._idmap.lookup_readonly(ids.to(self._device))
+
+    # -------------------------------------------------------------- grads
+    def accept_grad(self, grad_index, grad, unique=False):
+        """``unique=True``: the caller knows ``grad_index`` has no duplicates (it is the
+        row index of unique ids), which spares ``grad()`` a dedup pass."""
+        if grad_index.dtype != torch.int64:
+            raise RuntimeError("grad_index must be int64")
+        if grad.dtype != self._dtype and not (grad.dtype == torch.float32 and self._dtype in
+                                              (torch.bfloat16, torch.float16)):
+            raise RuntimeError("grad dtype %s does not match the table (%s)" % (grad.dtype, self._dtype))
+        self._grad_index.append(grad_index)
+        self._grad.append(grad)
+        self._grad_unique.append(bool(unique))
+
+    def has_grad(self):
+        return len(self._grad) > 0
+
+    def grad_pairs(self, accumulate_steps=1):
+        """(row index, gradient rows) merged over the accepted gradients: what
+        ``grad()`` wraps as a sparse tensor (hashtable.cc:90-134), without the host
+        round trips. With duplicates the gradients are summed per row."""
+        index = self._grad_index[0] if len(self._grad_index) == 1 else torch.cat(self._grad_index, 0)
+        g = self._grad[0] if len(self._grad) == 1 else torch.cat(self._grad, 0)
+        if not (len(self._grad_unique) == 1 and self._grad_unique[0]):
+            uniq, inverse = torch.unique(index, sorted=False, return_inverse=True)
+            if uniq.numel() != index.numel():
+                summed = torch.zeros((uniq.numel(),) + tuple(g.shape[1:]), dtype=g.dtype, device=g.device)
+                summed.index_add_(0, inverse, g)
+                index, g = uniq, summed
+        if accumulate_steps != 1:
+            g = g / accumulate_steps
+        return index, g
+
+    def grad(self, accumulate_steps=1):
+        """Sparse COO gradient exactly as the reference builds it (hashtable.cc:90-134),
+        including its layout when rows repeat: positions 0..U-1 as indices and an
+        N-row value buffer whose first U rows hold the sums."""
+        index = torch.cat(self._grad_index, 0)
+        g = torch.cat(self._grad, 0)
+        uniq, inverse = torch.unique(index, sorted=False, return_inverse=True)
+        emb_shape = list(g.shape[1:])
+        if index.numel() == uniq.numel():
+            final_indices = index.view(1, -1)
+            final_grad = g
+            rows = int(index.max().item()) + 1 if index.numel() else 0
+        else:
+            final_indices = inverse.view(1, -1)
+            final_grad = torch.zeros([inverse.numel()] + emb_shape, dtype=g.dtype, device=g.device)
+            final_grad.index_add_(0, inverse.view(-1), g)
+            rows = int(uniq.max().item()) + 1 if uniq.numel() else 0
+        final_grad = final_grad / accumulate_steps
+        return torch.sparse_coo_tensor(final_indices, final_grad, [rows] + emb_shape,
+                                       check_invariants=False).detach_()
+
+    def clear_grad(self):
+        self._grad_index, self._grad, self._grad_unique = [], [], []
+
+    # ------------------------------------------------------------ bookkeeping
+    def clear(self):
+        self.clear_grad()
+        self._idmap.clear()
+        self._slot_group.clear()
+        self._rows_ub = 0
+
+    def clear_id(self):
+        self._idmap.clear()
+        self._rows_ub = 0
+
+    def ids(self):
+        return self._idmap.snapshot()[0]
+
+    def ids_map(self):
+        return self._idmap.snapshot()
+
+    def ids_num(self):
+        return self._idmap.id_num()
+
+    def slot_group(self):
+        self._sync_block_num()
+        return self._slot_group
+
+    def children_info(self):
+        return self._children_info
+
+    def slice_info(self):
+        return self._slice
+
+    def append_filter_slot(self, name, dtype, slot_dim, generator):
+        self._slot_group.append_slot(name, dtype, [0, slot_dim], generator)
+
+    def append_step_filter_slot(self, name, init_step):
+        if torch.is_tensor(init_step):
+            init_step = int(init_step.item())
+        self._slot_group.append_step_filter_slot(name, init_step)
+
+    def update_slot(self, slot_name, index, value):
+        slot = self._slot_group.slot_by_name(slot_name)
+        if value.dtype != slot.dtype():
+            raise RuntimeError("embedding type must be [%s] but get %s" % (slot.dtype(), value.dtype))
+        slot.index_insert(index.to(self._device), value)
+
+    def get_slot(self, name):
+        self._sync_block_num()
+        return self._slot_group.slot_by_name(name)
+
+    def delete(self, ids, index, preserve_slot=""):
+        """Erase keys, free their rows, re-initialise every slot but ``preserve_slot``
+        at those rows (hashtable.cc:263-278)."""
+        if ids.numel() == 0:
+            return
+        ids, index = ids.to(self._device), index.to(self._device)
+        self._idmap.erase(ids, index)
+        sg = self._slot_group
+        for i, slot in enumerate(sg.slots()):
+            if preserve_slot and sg.get_slot_index(preserve_slot) == i:
+                continue
+            slot.index_insert(index, slot.gen_val(ids.numel()))
+
+    def id_map(self):
+        return self._idmap
+
+    @property
+    def device(self):
+        return self._device
+
+    @property
+    def dtype(self):
+        return self._dtype
+
+
+def make_hashtable(block_size, embedding_shape, dtype, device, coalesce, children, generator,
+                   slice_begin=0, slice_end=65536, slice_size=65536, reserve_rows=0):
+    """``torch.ops.recis.make_hashtable`` (hashtable.h:36-41, bind.cc:145)."""
+    return HashtableImpl(block_size, embedding_shape, dtype, device, coalesce, children, generator,
+                         slice_begin, slice_end, slice_size, reserve_rows)
+
+
+def is_hashtable(obj):
+    return hasattr(obj, "hashtable_tag")
+
+
+def filter_out_sparse_param(model):
+    """name -> HashtableImpl for every table under ``model`` (what the sparse
+    optimizers take), mirroring ``recis.nn.modules.hashtable.filter_out_sparse_param``."""
+    out = {}
+    for module in model.modules():
+        if isinstance(module, HashTable):
+            out[module._name] = module._hashtable_impl
+    return out
+
+
+def split_sparse_dense_state_dict(state_dict):
+    sparse = {k: v for k, v in state_dict.items() if is_hashtable(v)}
+    dense = {k: v for k, v in state_dict.items() if not is_hashtable(v)}
+    return sparse, dense
+
+
+# ----------------------------------------------------------------- autograd
+class HashTableLookupHelpFunction(torch.autograd.Function):
+    """Lookup of unique ids; backward hands (row index, gradient) to the table
+    (recis/nn/modules/hashtable.py:425-481)."""
+
+    @staticmethod
+    def forward(ctx, ids, hashtable, backward_holder, admit_hook_impl):
+        from .hashtable_hook_impl import ReadOnlyHookImpl
+
+        assert admit_hook_impl is None or isinstance(admit_hook_impl, ReadOnlyHookImpl), \
+            "admit hook only support ReadOnlyHook yet, but got: %s" % admit_hook_impl
+        index, embedding = hashtable.embedding_lookup(ids.detach(), admit_hook_impl is not None)
+        ctx.save_for_backward(index)
+        ctx.hashtable = hashtable
+        ctx.mark_non_differentiable(index)
+        return index, embedding
+
+    @staticmethod
+    def backward(ctx, grad_output_index, grad_output_emb):
+        (index,) = ctx.saved_tensors
+        ctx.hashtable.accept_grad(index, grad_output_emb.contiguous(), unique=True)
+        return None, None, None, None
+
+
+class GradIDMeanFunction(torch.autograd.Function):
+    """Expand unique rows to request order; backward = mean over the duplicates of
+    each id (recis/nn/modules/hashtable.py:484-537)."""
+
+    @staticmethod
+    def forward(ctx, embedding, index):
+        ctx.save_for_backward(index)
+        ctx.unique_size = embedding.shape[0]
+        return ops.gather(index, embedding)
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        (index,) = ctx.saved_tensors
+        summed = _scatter_sum(grad_outputs, index, ctx.unique_size)
+        counts = torch.bincount(index.long(), minlength=ctx.unique_size).clamp_(min=1)
+        return (summed / counts.view(-1, 1).to(summed.dtype)).to(grad_outputs.dtype), None
+
+
+class GradWorkerMeanFunction(torch.autograd.Function):
+    """Expand unique rows to request order; backward = sum over duplicates divided
+    by the number of workers (recis/nn/modules/hashtable.py:540-586)."""
+
+    @staticmethod
+    def forward(ctx, embedding, index, slice_num):
+        ctx.save_for_backward(index)
+        ctx.unique_size = embedding.shape[0]
+        ctx.slice_num = slice_num
+        return ops.gather(index, embedding)
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        (index,) = ctx.saved_tensors
+        if ctx.slice_num != 1:
+            grad_outputs = grad_outputs / ctx.slice_num
+        return _scatter_sum(grad_outputs, index, ctx.unique_size).to(grad_outputs.dtype), None, None
+
+
+def _scatter_sum(grad_rows, index, unique_size):
+    """sum of ``grad_rows[i]`` into row ``index[i]`` of a ``[unique_size, D]`` result."""
+    n = index.numel()
+    flat = grad_rows.reshape(n, -1).contiguous()
+    span = torch.tensor([0, n], dtype=torch.int64, device=index.device)
+    out = ops.segment_reduce_backward(flat, None, index, span, unique_size, "tile", out_dtype=torch.float32)
+    return out.view((unique_size,) + tuple(grad_rows.shape[1:]))
+
+
+# ------------------------------------------------------------------- module
+class HashTable(torch.nn.Module):
+    """Dynamic embedding table (recis/nn/modules/hashtable.py:98-423).
+
+    ``dedup`` chooses how ``forward`` removes duplicate ids: ``"hash"`` (default) is the
+    HIP hash dedup, whose unique ids come in order of first occurrence; ``"sorted"`` is
+    ``torch.unique`` as in the reference, which also makes the row a new key receives
+    identical to the reference's (new keys are ranked in ascending key order).
+    ``reserve_rows`` pre-sizes the map and the row storage."""
+
+    def __init__(self, embedding_shape: List, block_size: int = 5, dtype: torch.dtype = torch.float32,
+                 device: torch.device = torch.device("cuda"), coalesced: bool = False,
+                 children: Optional[List[str]] = None, slice: Slice = _default_slice, initializer=None,
+                 name: str = "hashtable", grad_reduce_by: str = "worker",
+                 filter_hook: Optional[FilterHook] = None, dedup: str = "hash", reserve_rows: int = 0):
+        super().__init__()
+        from .hashtable_hook_impl import HashtableHookFactory
+
+        self._initializer = ConstantInitializer(init_val=0) if initializer is None else initializer
+        if children is None:
+            children = [name]
+        self._device = torch.device(device)
+        assert grad_reduce_by in ["id", "worker"]
+        assert dedup in ["hash", "sorted"]
+        self._grad_reduce_by = grad_reduce_by
+        self._dedup = dedup
+        self._initializer.set_shape([block_size] + list(embedding_shape))
+        self._initializer.set_dtype(dtype)
+        self._initializer.build()
+        self._dtype = dtype
+        self._name = name
+        for child in children:
+            info = json.dumps(dict(shape=list(embedding_shape), dtype=str(dtype),
+                                   initializer=str(self._initializer)))
+            HashtableRegister().register(child, info)
+        self._hashtable_impl = make_hashtable(block_size, list(embedding_shape), dtype, self._device, coalesced,
+                                              children, self._initializer.impl(), slice.slice_begin,
+                                              slice.slice_end, slice.slice_size, reserve_rows)
+        self._backward_holder = torch.tensor([0.0], requires_grad=True)
+        self._worker_num = int(os.environ.get("WORLD_SIZE", 1))
+
+        def state_dict_hook(module, state_dict, prefix, local_metadata):
+            state_dict[module._name] = module._hashtable_impl
+
+        self._register_state_dict_hook(state_dict_hook)
+        if filter_hook is not None:
+            self._filter_hook_impl = HashtableHookFactory().create_filter_hook(self, filter_hook)
+        else:
+            self._filter_hook_impl = torch.nn.Identity()
+
+    def _unique(self, ids):
+        if self._dedup == "sorted":
+            return ids.unique(return_inverse=True)
+        uniq, inverse, count = ops.ids_unique(ids, inverse_dtype=torch.int64)
+        return uniq[: int(count.item())], inverse
+
+    def forward(self, ids: torch.Tensor, admit_hook: AdmitHook = None) -> torch.Tensor:
+        from .hashtable_hook_impl import HashtableHookFactory
+
+        admit_hook_impl = HashtableHookFactory().create_admit_hook(self, admit_hook) if admit_hook else None
+        shape = tuple(ids.shape)
+        ids = ids.to(self._device).reshape(-1)
+        uids, index = self._unique(ids)
+        if self.training and self._dtype not in (torch.int8, torch.int32, torch.int64):
+            emb_idx, embedding = HashTableLookupHelpFunction.apply(uids, self._hashtable_impl,
+                                                                   self._backward_holder, admit_hook_impl)
+            if self._grad_reduce_by == "id":
+                embedding = GradIDMeanFunction.apply(embedding, index)
+            else:
+                embedding = GradWorkerMeanFunction.apply(embedding, index, self._worker_num)
+            self._filter_hook_impl(emb_idx)
+        else:
+            _, embedding = self._hashtable_impl.embedding_lookup(uids.detach(), True)
+            embedding = ops.gather(index, embedding)
+        return embedding.view(shape + tuple(embedding.shape[1:])) if len(shape) != 1 else embedding
+
+    def initializer(self):
+        return self._initializer
+
+    @property
+    def device(self):
+        return self._device
+
+    @property
+    def coalesce(self):
+        return self._hashtable_impl.children_info().is_coalesce()
+
+    @property
+    def children_hashtable(self):
+        return self._hashtable_impl.children_info().children()
+
+    def accept_grad(self, grad_index, grad) -> None:
+        self._hashtable_impl.accept_grad(grad_index, grad)
+
+    def grad(self, acc_step=1) -> torch.Tensor:
+        return self._hashtable_impl.grad(acc_step)
+
+    def clear_grad(self) -> None:
+        self._hashtable_impl.clear_grad()
+
+    def insert(self, ids, embeddings) -> None:
+        self._hashtable_impl.insert(ids, embeddings)
+
+    def clear(self) -> None:
+        self._hashtable_impl.clear()
+
+    def ids(self) -> torch.Tensor:
+        return self._hashtable_impl.ids()
+
+    def ids_map(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        return self._hashtable_impl.ids_map()
+
+    def embeddings(self) -> torch.Tensor:
+        return self._hashtable_impl.slot_group().slot_by_name("embedding").value()
+
+    def slot_group(self):
+        return self._hashtable_impl.slot_group()
+
+    def children_info(self):
+        return self._hashtable_impl.children_info()
+
+    def __str__(self) -> str:
+        return "HashTable_%s" % self._name
+
+    __repr__ = __str__

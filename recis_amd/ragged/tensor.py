@@ -1,0 +1,92 @@
+"""``RaggedTensor``: values + one offsets tensor per ragged dimension (+ optional
+per-value weight), the container of ``recis.ragged.tensor`` (tensor.py:41-541)
+reduced to what the embedding path reads."""
+from typing import List, Optional, Union
+
+import torch
+
+
+class RaggedTensor:
+    def __init__(self, values: torch.Tensor, offsets: Union[torch.Tensor, List[torch.Tensor]],
+                 weight: Optional[torch.Tensor] = None, dense_shape=None):
+        if isinstance(offsets, torch.Tensor):
+            offsets = [offsets]
+        if not offsets:
+            raise ValueError("RaggedTensor needs at least one offsets tensor")
+        self._values = values
+        self._offsets = list(offsets)
+        self._weight = weight
+        if dense_shape is None:
+            # rows = outermost offsets, one trailing ragged dimension per offsets tensor
+            dense_shape = tuple([self._offsets[0].numel() - 1] + [-1] * len(self._offsets))
+        self._dense_shape = tuple(dense_shape)
+
+    def values(self):
+        return self._values
+
+    def offsets(self):
+        return self._offsets
+
+    def weight(self):
+        return self._weight
+
+    def set_values(self, values):
+        self._values = values
+
+    def set_weight(self, weight):
+        self._weight = weight
+
+    def set_offsets(self, offsets):
+        self._offsets = [offsets] if isinstance(offsets, torch.Tensor) else list(offsets)
+
+    @property
+    def dense_shape(self):
+        return self._dense_shape
+
+    def real_shape(self, start=0, end=None):
+        shape = list(self._dense_shape)
+        shape[0] = self._offsets[0].numel() - 1
+        return tuple(shape[start:end])
+
+    @property
+    def device(self):
+        return self._values.device
+
+    @property
+    def dtype(self):
+        return self._values.dtype
+
+    def to(self, *args, **kwargs):
+        return RaggedTensor(self._values.to(*args, **kwargs), [o.to(*args, **kwargs) for o in self._offsets],
+                            None if self._weight is None else self._weight.to(*args, **kwargs),
+                            self._dense_shape)
+
+    def cuda(self):
+        return self.to("cuda")
+
+    def cpu(self):
+        return self.to("cpu")
+
+    def clone(self):
+        return RaggedTensor(self._values.clone(), [o.clone() for o in self._offsets],
+                            None if self._weight is None else self._weight.clone(), self._dense_shape)
+
+    def to_dense(self, default_value=0):
+        """Pads the innermost ragged dimension (one level) to its longest row."""
+        if len(self._offsets) != 1:
+            raise NotImplementedError("to_dense handles one ragged dimension")
+        off = self._offsets[0].long()
+        lens = off[1:] - off[:-1]
+        rows = lens.numel()
+        width = int(lens.max().item()) if rows else 0
+        out = torch.full((rows, width), default_value, dtype=self._values.dtype, device=self._values.device)
+        if self._values.numel():
+            row = torch.repeat_interleave(torch.arange(rows, device=off.device), lens)
+            col = torch.arange(self._values.numel(), device=off.device) - off[:-1][row]
+            out[row, col] = self._values
+        return out
+
+    def __repr__(self):
+        return "RaggedTensor(values=%s, offsets=%s, weight=%s)" % (
+            tuple(self._values.shape), [tuple(o.shape) for o in self._offsets],
+            None if self._weight is None else tuple(self._weight.shape))

@@ -1,0 +1,350 @@
+"""End-to-end parity of the GPU table + pooling + optimizer with the restated
+reference CPU path (oracle.cpu_path) on BASELINE config 1, and behaviour tests of
+the host-side modules that read like the reference's own module tests.
+
+Bars: key -> row assignment bit-exact when new keys are presented in the reference's
+order (``dedup="sorted"``), and a bijection-equivalent assignment with the hash dedup;
+fp32 rows / optimizer state / pooled outputs within rtol 1e-5, atol 1e-6.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import workloads
+from oracle import cpu_path
+from recis_amd import ops
+from recis_amd.hooks import HashTableFilterHook
+from recis_amd.nn import DynamicEmbedding, EmbeddingEngine, EmbeddingOption, HashTable
+from recis_amd.nn.functional.embedding_ops import ragged_embedding_segment_reduce
+from recis_amd.nn.hashtable_hook import AdmitHook, FilterHook
+from recis_amd.nn.initializers import ConstantInitializer, Initializer, NormalInitializer, _Generator
+from recis_amd.nn.modules.hashtable import HashtableRegister, filter_out_sparse_param
+from recis_amd.nn.modules.hashtable_hook_impl import HashtableHookFactory
+from recis_amd.optim import SparseAdagrad, SparseAdam, SparseAdamW, SparseAdamWTF
+from recis_amd.ragged.tensor import RaggedTensor
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _fresh_registries():
+    HashtableRegister().clear()
+    HashtableHookFactory().clear_filters()
+    yield
+
+
+class SeededBlockInitializer(Initializer):
+    """Hands out the same per-block rows as the CPU side (workloads.seeded_block), so
+    that both tables start from identical storage whatever the chunking."""
+
+    def __init__(self, seed, std=0.01):
+        super().__init__()
+        self._seed, self._std = seed, std
+
+    def _build_impl(self):
+        bs, dim = self._shape[0], self._shape[1]
+        state = {"next_block": 0}
+
+        def fill(t, gen):
+            rows = t.shape[0]
+            assert rows % bs == 0
+            parts = []
+            for _ in range(rows // bs):
+                parts.append(workloads.seeded_block(self._seed, state["next_block"], bs, dim, self._std))
+                state["next_block"] += 1
+            t.copy_(torch.from_numpy(np.concatenate(parts)))
+
+        return _Generator(self._shape, self._dtype, fill, "SeededBlockInitializer(seed=%d)" % self._seed)
+
+    def __str__(self):
+        return "SeededBlockInitializer(seed=%d)" % self._seed
+
+
+def _close(a, b, msg=""):
+    np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6, err_msg=msg)
+
+
+@pytest.mark.parametrize("steps", [100])
+def test_config1_hundred_steps_bit_exact_rows(steps):
+    """BASELINE config 1: Zipf(1.05) ids over 1e6 keys, batch 4096, lengths 1..20, dim 16 fp32,
+    rows N(0, 0.01), sum pooling, backward, sparse Adagrad (lr 0.01, eps 1e-8), 100 steps, seed 0."""
+    bs, dim = 1024, 16
+    cpu = cpu_path.CpuTable(dim, bs, lambda b: workloads.seeded_block(0, b, bs, dim), "adagrad", 0.01, 1e-8)
+    table = HashTable([dim], block_size=bs, device="cuda", initializer=SeededBlockInitializer(0),
+                      name="c1", dedup="sorted")
+    table.train()
+    opt = SparseAdagrad(filter_out_sparse_param(table), lr=0.01, eps=1e-8)
+    for step in range(steps):
+        ids, off, grad = workloads.config1_step(step)
+        pooled_c, uniq_c, index_c = cpu_path.train_step(cpu, ids, off, None, grad)
+        ids_t, off_t = torch.from_numpy(ids).cuda(), torch.from_numpy(off).cuda()
+        rows = table(ids_t)                                                    # [N, dim], request order
+        pooled = ragged_embedding_segment_reduce(rows, None, None, off_t, "sum")
+        pooled.backward(torch.from_numpy(grad).cuda())
+        opt.step()
+        opt.zero_grad()
+        if step % 10 == 0 or step == steps - 1:
+            _close(pooled.detach().cpu().numpy(), pooled_c, "pooled output, step %d" % step)
+            got_index = table._hashtable_impl.lookup_index_readonly(torch.from_numpy(uniq_c).cuda())
+            np.testing.assert_array_equal(got_index.cpu().numpy(), index_c)     # bit-exact row assignment
+    ids_g, idx_g = table.ids_map()
+    ids_c, idx_c = cpu.idmap.snapshot()
+    assert dict(zip(ids_g.cpu().tolist(), idx_g.cpu().tolist())) == dict(zip(ids_c.tolist(), idx_c.tolist()))
+    sg = table.slot_group()
+    assert sg.block_num() == len(cpu.emb)
+    _close(sg.slot_by_name("embedding").value().cpu().numpy(), np.concatenate(cpu.emb), "embedding rows")
+    _close(sg.slot_by_name("sparse_adagrad_accum").value().cpu().numpy(), np.concatenate(cpu.s0), "adagrad state")
+
+
+def test_config1_engine_path_matches_up_to_row_order():
+    """Same workload through EmbeddingEngine (hash dedup, fused group pipeline): the row a key
+    gets may differ, everything addressed by key must not."""
+    bs, dim, steps = 1024, 16, 30
+    cpu = cpu_path.CpuTable(dim, bs, lambda b: np.zeros((bs, dim), np.float32), "adam", 1e-3, 1e-8,
+                            decay=1.0, beta_dtype=np.float64)
+    eng = EmbeddingEngine({"f": EmbeddingOption(embedding_dim=dim, block_size=bs, shared_name="c1e",
+                                                combiner="sum", use_weight=False)})
+    eng.train()
+    opt = SparseAdam({n: t._hashtable_impl for n, t in eng.hashtables().items()}, lr=1e-3)
+    for step in range(steps):
+        ids, off, grad = workloads.config1_step(step, batch=512)
+        pooled_c, uniq_c, _ = cpu_path.train_step(cpu, ids, off, None, grad)
+        rt = RaggedTensor(torch.from_numpy(ids).cuda(), torch.from_numpy(off.astype(np.int32)).cuda())
+        out = eng({"f": rt})["f"]
+        out.backward(torch.from_numpy(grad).cuda())
+        opt.step()
+        opt.zero_grad()
+        _close(out.detach().cpu().numpy(), pooled_c, "pooled, step %d" % step)
+    table = eng.hashtables()["c1e"]
+    ids_c, _ = cpu.idmap.snapshot()
+    ids_c = np.sort(ids_c)
+    assert np.array_equal(np.sort(table.ids().cpu().numpy()), ids_c)
+    impl = table._hashtable_impl
+    rows_g = impl.lookup_index_readonly(torch.from_numpy(ids_c).cuda())
+    assert len(set(rows_g.cpu().tolist())) == len(ids_c)                       # bijection key <-> row
+    for slot, blocks in (("embedding", cpu.emb), ("sparse_adam_exp_avg", cpu.s0), ("sparse_adam_exp_avg_sq", cpu.s1)):
+        got = impl.get_slot(slot).index_select(rows_g).cpu().numpy()
+        exp = oracle.block_gather(cpu.idmap.lookup_readonly(ids_c), blocks, bs)
+        # the head Zipf keys receive several hundred gradient rows per step, summed in fp32 in a
+        # different order on each side: atol scales with that sum (1e-6 per unit, magnitude ~10)
+        np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-5, err_msg=slot)
+
+
+# ------------------------------------------------- module behaviour (reference-style tests)
+def test_lookup_insert_ids_eval():
+    # tests/hashtable/ht_lookup_test.py:16-112
+    ht = HashTable([8], block_size=16, device="cuda", name="ht_lookup",
+                   initializer=ConstantInitializer(0.0))
+    ids = torch.arange(100, device="cuda")
+    emb = ht(ids)
+    assert emb.shape == (100, 8) and float(emb.abs().sum()) == 0
+    vals = torch.randn(100, 8, device="cuda")
+    ht.insert(ids, vals)
+    torch.testing.assert_close(ht(ids), vals)
+    torch.testing.assert_close(ht(torch.tensor([5, 5, 7], device="cuda")), vals[[5, 5, 7]])
+    assert torch.equal(torch.sort(ht.ids())[0], ids)
+    ht.eval()
+    out = ht(torch.arange(90, 110, device="cuda"))
+    torch.testing.assert_close(out[:10], vals[90:])
+    assert float(out[10:].abs().sum()) == 0
+    assert ht.ids().numel() == 100                     # eval() admits nothing
+    ht.train()
+    out = ht(torch.arange(100, 105, device="cuda"), AdmitHook("ReadOnly"))
+    assert float(out.abs().sum()) == 0 and ht.ids().numel() == 100
+    ht(torch.arange(100, 105, device="cuda"))
+    assert ht.ids().numel() == 105
+    # missing keys take rows from the initializer
+    ht2 = HashTable([4], block_size=8, device="cuda", name="ht_init", initializer=ConstantInitializer(2.5))
+    assert torch.all(ht2(torch.tensor([3, 9], device="cuda")) == 2.5)
+    with pytest.raises(ValueError):
+        HashTable([4], device="cuda", name="ht_init")  # duplicate table name
+
+
+def test_slot_metadata_and_block_growth():
+    # tests/hashtable/ht_slot_test.py; block_num = (id_num + bs) / bs (hashtable.cc:255-261)
+    ht = HashTable([4], block_size=10, device="cuda", name="ht_slot", initializer=ConstantInitializer(1.0))
+    ht(torch.arange(25, device="cuda"))
+    sg = ht.slot_group()
+    slot = sg.slot_by_name("embedding")
+    assert slot.name() == "embedding" and slot.block_size() == 10 and slot.flat_size() == 4
+    assert len(slot.values()) == 3 and slot.value().shape == (30, 4)
+    assert float(slot.value().sum()) == 30 * 4
+    ht(torch.arange(25, 30, device="cuda"))
+    assert len(ht.slot_group().slot_by_name("embedding").values()) == 4   # 30 ids -> (30+10)/10
+    # values() alias live storage
+    ht.slot_group().slot_by_name("embedding").values()[0][0].fill_(9.0)
+    assert float(ht.embeddings()[0].sum()) == 36.0
+
+
+def test_grad_accumulation_kat():
+    # tests/hashtable/ht_grad_ga_test.py:9-33
+    ht = HashTable([4], device="cuda", name="ht_ga")
+    ht.accept_grad(torch.tensor([1, 2, 3], device="cuda"), torch.ones(3, 4, device="cuda"))
+    ht.accept_grad(torch.tensor([1, 1, 1], device="cuda"), torch.ones(3, 4, device="cuda") * 2)
+    ht.accept_grad(torch.tensor([2, 2, 2], device="cuda"), torch.ones(3, 4, device="cuda") * 3)
+    ga = ht.grad(3).coalesce()
+    assert ga.indices().cpu().tolist() == [[0, 1, 2]]
+    exp = torch.tensor([[7.0] * 4, [10.0] * 4, [1.0] * 4]) / 3.0
+    torch.testing.assert_close(ga.values().cpu(), exp)
+    # the merged pairs the optimizers consume: per-row sums / accumulation steps
+    index, g = ht._hashtable_impl.grad_pairs(3)
+    got = dict(zip(index.cpu().tolist(), g.cpu()[:, 0].tolist()))
+    assert got == pytest.approx({1: 7 / 3, 2: 10 / 3, 3: 1 / 3})
+
+
+@pytest.mark.parametrize("cls,ref_wd", [(SparseAdamW, "adamw"), (SparseAdamWTF, "tf"), (SparseAdam, "none")])
+def test_sparse_adam_family_tracks_torch_adamw(cls, ref_wd):
+    # tests/optim/sparse_adamw_test.py:84-175: zero-init rows, every row updated each step
+    U, D, steps, lr, wd = 512, 16, 20, 1e-2, 1e-2
+    ht = HashTable([D], block_size=128, device="cuda", name="adam_" + ref_wd)
+    ht.train()
+    opt = cls(filter_out_sparse_param(ht), lr=lr, weight_decay=wd)
+    torch_wd = {"adamw": wd, "tf": wd / lr, "none": 0.0}[ref_wd]
+    p = torch.nn.Parameter(torch.zeros(U, D, device="cuda"))
+    topt = torch.optim.AdamW([p], lr=lr, weight_decay=torch_wd)
+    ids = torch.arange(U, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(3)
+    for _ in range(steps):
+        target = torch.randn(U, D, device="cuda", generator=g)
+        loss = ((ht(ids) - target) ** 2).sum()
+        loss.backward()
+        opt.step()
+        opt.zero_grad()
+        topt.zero_grad()
+        ((p - target) ** 2).sum().backward()
+        topt.step()
+    torch.testing.assert_close(ht(ids).detach(), p.detach(), rtol=1e-5, atol=1e-4)
+    # row placement (sparse_adamw_test.py:177-208): first new key takes the largest fresh row
+    rows = ht._hashtable_impl.lookup_index_readonly(ids)
+    assert torch.equal(rows, torch.arange(U - 1, -1, -1, device="cuda"))
+    names = [s.name() for s in ht.slot_group().slots()]
+    prefix = {"adamw": "sparse_adamw_", "tf": "sparse_adamw_tf_", "none": "sparse_adam_"}[ref_wd]
+    assert names == ["embedding", prefix + "exp_avg", prefix + "exp_avg_sq"]
+    assert set(opt.state_dict()) == {prefix + "step", prefix + "beta1", prefix + "beta2"}
+
+
+def test_grad_reduce_by_id_and_worker():
+    for mode in ("worker", "id"):
+        ht = HashTable([2], device="cuda", name="gr_" + mode, grad_reduce_by=mode)
+        ht.train()
+        ids = torch.tensor([4, 4, 4, 9], device="cuda")
+        out = ht(ids)
+        out.backward(torch.tensor([[1.0, 1], [2, 2], [6, 6], [5, 5]], device="cuda"))
+        index, g = ht._hashtable_impl.grad_pairs(1)
+        rows = ht._hashtable_impl.lookup_index_readonly(torch.tensor([4, 9], device="cuda"))
+        got = {int(i): g[k, 0].item() for k, i in enumerate(index.cpu())}
+        exp4 = 9.0 if mode == "worker" else 3.0
+        assert got[int(rows[0])] == pytest.approx(exp4) and got[int(rows[1])] == pytest.approx(5.0)
+
+
+def test_global_step_filter_eviction_matches_cpu_path():
+    """Last-seen-step stamping + eviction (hashtable_hook_impl.py:487-551, filter_hook.py:82-117)
+    against the same policy on the CPU path; freed rows are recycled by later inserts."""
+    dim, bs, filter_step, interval = 4, 64, 3, 4
+    cpu = cpu_path.CpuTable(dim, bs, lambda b: np.zeros((bs, dim), np.float32), "adagrad", 0.1, 1e-8,
+                            step_filter=True)
+    ht = HashTable([dim], block_size=bs, device="cuda", name="evict", dedup="sorted",
+                   filter_hook=FilterHook("GlobalStepFilter", {"filter_step": filter_step}))
+    ht.train()
+    opt = SparseAdagrad(filter_out_sparse_param(ht), lr=0.1)
+    hook = HashTableFilterHook(filter_interval=interval)
+    rng = np.random.default_rng(5)
+    last = 0
+    for step in range(1, 25):
+        ids = rng.integers(step * 20, step * 20 + 150, size=200)
+        off = np.arange(0, 201, 4)
+        grad = rng.standard_normal((50, dim)).astype(np.float32)
+        cpu_path.train_step(cpu, ids, off, None, grad)          # advances cpu.global_step
+        rows = ht(torch.from_numpy(ids).cuda())
+        pooled = ragged_embedding_segment_reduce(rows, None, None, torch.from_numpy(off).cuda(), "sum")
+        pooled.backward(torch.from_numpy(grad).cuda())
+        opt.step()
+        opt.zero_grad()
+        hook.after_step(None, step)
+        if last == 0:
+            last = step
+        if step - last >= interval:
+            ev_ids, ev_rows = cpu.evict_older_than(filter_step)
+            # the reference re-initialises every slot but the stamp at the freed rows
+            if len(ev_rows):
+                oracle.block_insert(ev_rows, np.zeros((1, dim), np.float32), cpu.emb, bs)
+                oracle.block_insert(ev_rows, np.zeros((1, dim), np.float32), cpu.s0, bs)
+            last = step
+        assert np.array_equal(np.sort(ht.ids().cpu().numpy()), np.sort(cpu.idmap.snapshot()[0]))
+    live = np.sort(cpu.idmap.snapshot()[0])
+    rows_g = ht._hashtable_impl.lookup_index_readonly(torch.from_numpy(live).cuda()).cpu().numpy()
+    assert len(set(rows_g.tolist())) == len(live)
+    got = ht._hashtable_impl.get_slot("embedding").index_select(torch.from_numpy(rows_g).cuda()).cpu().numpy()
+    _close(got, cpu.rows_of(live)[1])
+    stamps = ht._hashtable_impl.get_slot("step_filter").index_select(torch.from_numpy(rows_g).cuda())
+    exp_stamps = oracle.block_gather(cpu.idmap.lookup_readonly(live), cpu.stamp, bs)
+    np.testing.assert_array_equal(stamps.cpu().numpy(), exp_stamps)
+    assert ht._hashtable_impl.id_map().stats()[1] < 24 * 150    # rows were reused, not only appended
+
+
+def test_engine_coalesces_and_pools():
+    """Two features sharing one configuration land in one physical table (12-bit tags keep equal
+    raw ids apart); a third with another dim gets its own; outputs match a direct computation."""
+    opts = {
+        "user": EmbeddingOption(embedding_dim=8, shared_name="user", combiner="sum", block_size=64,
+                                initializer=NormalInitializer(0, 0.1)),
+        "item": EmbeddingOption(embedding_dim=8, shared_name="item", combiner="sum", block_size=64,
+                                initializer=NormalInitializer(0, 0.1)),
+        "cate": EmbeddingOption(embedding_dim=4, shared_name="cate", combiner="mean", block_size=64,
+                                initializer=NormalInitializer(0, 0.1), use_weight=False),
+    }
+    eng = EmbeddingEngine(opts)
+    assert len(eng.hashtables()) == 2
+    eng.train()
+    user = RaggedTensor(torch.tensor([1, 2, 3, 1], device="cuda"), torch.tensor([0, 3, 4], device="cuda"),
+                        weight=torch.tensor([1.0, 2.0, 3.0, 4.0], device="cuda"))
+    item = torch.tensor([[1, 2], [3, 3]], device="cuda")
+    cate = RaggedTensor(torch.tensor([7, 8, 9], device="cuda"), torch.tensor([0, 0, 3], device="cuda"))
+    out = eng({"user": user, "item": item, "cate": cate})
+    assert out["user"].shape == (2, 8) and out["item"].shape == (2, 8) and out["cate"].shape == (2, 4)
+    big = [t for n, t in eng.hashtables().items() if t.coalesce][0]
+    info = big.children_info()
+    assert info.children() == ["user", "item"]
+
+    def row(child, raw):
+        key = torch.tensor([info.encode_id(raw, info.child_index(child))], device="cuda")
+        idx = big._hashtable_impl.lookup_index_readonly(key)
+        assert int(idx) >= 0
+        return big._hashtable_impl.get_slot("embedding").index_select(idx)[0]
+
+    torch.testing.assert_close(out["user"][0], row("user", 1) + 2 * row("user", 2) + 3 * row("user", 3))
+    torch.testing.assert_close(out["user"][1], 4 * row("user", 1))
+    torch.testing.assert_close(out["item"][1], 2 * row("item", 3))
+    assert not torch.equal(row("user", 1), row("item", 1))
+    assert float(out["cate"][0].abs().sum()) == 0
+    # gradients flow to the table
+    (out["user"].sum() + out["item"].sum() + out["cate"].sum()).backward()
+    assert all(t._hashtable_impl.has_grad() for t in eng.hashtables().values())
+
+
+def test_dynamic_embedding_tile_and_max():
+    opt = EmbeddingOption(embedding_dim=4, shared_name="tile_t", combiner="tile",
+                          combiner_kwargs={"tile_len": 3}, block_size=32, use_weight=False,
+                          initializer=NormalInitializer(0, 1.0))
+    emb = DynamicEmbedding(opt)
+    emb.train()
+    rt = RaggedTensor(torch.tensor([5, 6, 7, 8, 9, 5], device="cuda"), torch.tensor([0, 4, 4, 6], device="cuda"))
+    out = emb(rt)
+    assert out.shape == (3, 12)
+    rows = emb.hashtable(torch.tensor([5, 6, 7, 9], device="cuda")).detach()
+    torch.testing.assert_close(out[0].detach(), torch.cat([rows[0], rows[1], rows[2]]))   # truncated at 3
+    assert float(out[1].abs().sum()) == 0
+    torch.testing.assert_close(out[2].detach(), torch.cat([rows[3], rows[0], torch.zeros(4, device="cuda")]))
+    out.sum().backward()
+    index, g = emb.hashtable._hashtable_impl.grad_pairs(1)
+    r5 = int(emb.hashtable._hashtable_impl.lookup_index_readonly(torch.tensor([5], device="cuda")))
+    assert g[index.cpu().tolist().index(r5)].tolist() == [2.0] * 4              # id 5 kept twice
+    opt2 = EmbeddingOption(embedding_dim=4, shared_name="max_t", combiner="max", block_size=32,
+                           use_weight=False, initializer=NormalInitializer(0, 1.0))
+    emb2 = DynamicEmbedding(opt2)
+    emb2.train()
+    out2 = emb2(rt)
+    rows2 = emb2.hashtable(torch.tensor([5, 6, 7, 8, 9], device="cuda")).detach()
+    torch.testing.assert_close(out2[0].detach(), rows2[:4].max(0)[0])
+    torch.testing.assert_close(out2[2].detach(), rows2[[4, 0]].max(0)[0])

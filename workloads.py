@@ -50,3 +50,26 @@ def config2(device="cuda", seed=1, features=32, batch=16384, dim=64, mean_len=30
         "num_ids": N,
         "dim": dim,
     }
+
+
+def config1_step(step, seed=0, batch=4096, num_keys=1_000_000, alpha=1.05, max_len=20, dim=16, _cache={}):
+    """One batch of BASELINE config 1 as numpy arrays: (ids int64 [N], offsets int64 [batch+1],
+    upstream gradient float32 [batch, dim]). Deterministic in (seed, step)."""
+    key = (num_keys, alpha)
+    if key not in _cache:
+        p = np.arange(1, num_keys + 1, dtype=np.float64) ** (-alpha)
+        cdf = np.cumsum(p)
+        _cache[key] = cdf / cdf[-1]
+    rng = _rng([seed, step])
+    lens = rng.integers(1, max_len + 1, size=batch)
+    off = np.zeros(batch + 1, np.int64)
+    np.cumsum(lens, out=off[1:])
+    n = int(off[-1])
+    ids = np.minimum(np.searchsorted(_cache[key], rng.random(n), side="left"), num_keys - 1).astype(np.int64)
+    grad = rng.standard_normal((batch, dim)).astype(np.float32)
+    return ids, off, grad
+
+
+def seeded_block(seed, block_index, block_size, dim, std=0.01):
+    """Initial rows of one storage block, identical on the CPU and the GPU side."""
+    return (std * _rng([seed, 7919, block_index]).standard_normal((block_size, dim))).astype(np.float32)
