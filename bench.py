@@ -1,0 +1,303 @@
+"""Benchmark of the sparse-embedding hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W [--workload c4|c2] [--no-cpu-baseline]
+
+Prints ONE JSON line. A "step" is one pass of the hot path over one batch of synthetic
+input that is already resident in HBM. The default workload is BASELINE config 4
+(click-through-style merged table): feature ops (bucketize + mod) -> key tagging ->
+dedup -> find-or-insert -> row gather -> sum pooling -> backward scatter -> fused sparse
+Adam; `value` = id occurrences per second. Config 2 (standalone segment reduce, fwd + bwd
+for sum / mean / max) is measured in the same run and reported under "workloads".
+
+"roofline" describes the kernel that takes the largest share of the step: algorithmic
+bytes per launch / mean launch time (HIP events on the launch stream) against the 8 TB/s
+HBM peak. "cpu_baseline" is the restated reference CPU path (oracle.cpu_path) timed on
+this host on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import workloads  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _event_ms(fn, iters):
+    """Mean time of fn() over `iters` launches, HIP events on the current stream."""
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+# --------------------------------------------------------------------- config 2
+class Config2:
+    """Standalone ragged segment_reduce on pre-materialised rows: 32 x 16384 segments,
+    Poisson(30) lengths in [1, 200], D = 64 fp32, int32 offsets; forward + backward gradient
+    scatter for the sum, mean and max combiners."""
+
+    name = "c2_segment_reduce_32x16384_poisson30_d64_fp32"
+
+    def __init__(self):
+        from recis_amd import ops
+        self.ops = ops
+        c = workloads.config2()
+        self.emb, self.off, self.grad = c["values"], c["offsets"], c["grad"]
+        self.S, self.N, self.D = c["num_segments"], c["num_ids"], c["dim"]
+        self.ids_per_step = 3 * self.N
+        # algorithmic bytes of one pass: N rows of 256 B + 8 B index each, S rows of 256 B + offset
+        self.pass_bytes = self.N * (self.D * 4 + 8) + self.S * (self.D * 4 + 4)
+        self.rev = torch.arange(self.N, device="cuda")
+
+    def step(self):
+        o = self.ops
+        for mode in ("sum", "mean"):
+            o.segment_reduce_forward(self.emb, None, self.rev, self.off, mode)
+            o.segment_reduce_backward(self.grad, None, self.rev, self.off, self.N, mode, rev_unique=True)
+        _, arg = o.segment_reduce_forward(self.emb, None, self.rev, self.off, "max", return_argmax=True)
+        o.segment_reduce_backward(self.grad, None, self.rev, self.off, self.N, "max", argmax=arg, rev_unique=True)
+
+    def kernels(self):
+        o = self.ops
+        return {
+            "seg_pool_fwd_kernel(sum)": (lambda: o.segment_reduce_forward(self.emb, None, self.rev, self.off, "sum"),
+                                         self.pass_bytes),
+            "seg_pool_bwd_kernel(sum)": (lambda: o.segment_reduce_backward(self.grad, None, self.rev, self.off,
+                                                                          self.N, "sum", rev_unique=True),
+                                         self.pass_bytes),
+        }
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        k = 4096  # segments in the sample
+        off = self.off[: k + 1].cpu().numpy().astype(np.int64)
+        n = int(off[-1])
+        emb = self.emb[:n].cpu().numpy()
+        g = self.grad[:k].cpu().numpy()
+        rev = np.arange(n)
+        t0, reps = time.perf_counter(), 0
+        while time.perf_counter() - t0 < budget_s:
+            for mode in ("sum", "mean"):
+                oracle.segment_reduce_forward(emb, None, rev, off, mode)
+                oracle.segment_reduce_backward(g, None, rev, off, n, mode)
+            _, arg = oracle.segment_max_forward(emb, rev, off)
+            oracle.segment_max_backward(g, arg, rev, n)
+            reps += 1
+        dt = time.perf_counter() - t0
+        return 3 * n * reps / dt, "first %d segments (%d ids) of config 2, fwd+bwd x (sum, mean, max)" % (k, n)
+
+
+# --------------------------------------------------------------------- config 4
+class Config4:
+    """Click-through-style merged table: 26 id fields + 13 bucketized dense fields, batch 65536,
+    dim 16 fp32, one coalesced table, fused dedup + lookup + sum pool + backward + sparse Adam
+    (lr 1e-3, betas 0.9 / 0.999)."""
+
+    name = "c4_ctr_merged_table_39x65536_d16_fp32_adam"
+
+    def __init__(self, batch=65536):
+        from recis_amd import ops
+        from recis_amd.nn.initializers import NormalInitializer
+        from recis_amd.nn.modules.hashtable import HashtableImpl
+        from recis_amd.optim.sparse_impl import SparseAdamImpl
+        self.ops = ops
+        c = workloads.config4(batch=batch)
+        self.c = c
+        self.D = 16
+        self.n_feat = len(c["sparse"]) + len(c["dense"])
+        self.N = c["num_ids"]
+        self.ids_per_step = self.N
+        init = NormalInitializer(0.0, 0.01)
+        init.set_shape([10240, self.D])
+        init.set_dtype(torch.float32)
+        self.table = HashtableImpl(10240, [self.D], torch.float32, torch.device("cuda"), True,
+                                   ["f%d" % i for i in range(self.n_feat)], init.build().impl(),
+                                   reserve_rows=int(self.N * 1.05))
+        self.opt = SparseAdamImpl.make({"ctr": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0)
+        self.tags = list(range(self.n_feat))
+        self.offsets = torch.arange(self.N + 1, dtype=torch.int32, device="cuda")
+        g = torch.Generator(device="cuda").manual_seed(4)
+        self.grad_out = torch.randn((self.N, self.D), device="cuda", generator=g)
+        self.mods = [c["mod"]] * len(c["dense"])
+        self.U = None
+
+    # the stages, also timed one by one for the breakdown
+    def feature_ops(self):
+        o = self.ops
+        buckets = o.fused_bucketized(self.c["dense"], self.c["boundaries"])
+        extra = o.fused_uint64_mod(buckets, self.mods)
+        return o.ids_encode(self.c["sparse"] + extra, self.tags)
+
+    def dedup(self, ids):
+        uniq, inv, count = self.ops.ids_unique(ids)
+        self.U = int(count.item())
+        return uniq[: self.U], inv
+
+    def lookup(self, uniq):
+        return self.table.embedding_lookup(uniq, False)
+
+    def pool_fwd(self, rows, inv):
+        return self.ops.segment_reduce_forward(rows, None, inv, self.offsets, "sum")
+
+    def pool_bwd(self, inv):
+        return self.ops.segment_reduce_backward(self.grad_out, None, inv, self.offsets, self.U, "sum")
+
+    def update(self, index, g):
+        self.table.accept_grad(index, g, unique=True)
+        self.opt.step()
+        self.opt.zero_grad()
+
+    def step(self):
+        ids = self.feature_ops()
+        uniq, inv = self.dedup(ids)
+        index, rows = self.lookup(uniq)
+        pooled = self.pool_fwd(rows, inv)
+        g = self.pool_bwd(inv)
+        self.update(index, g)
+        return pooled
+
+    def algorithmic_bytes(self):
+        N, U, S, D = self.N, self.U, self.N, self.D
+        feat = 13 * self.c["batch"] * (4 + 8) + 13 * self.c["batch"] * (8 + 8) + N * 16
+        return {
+            "feature_ops": feat,
+            "dedup": N * (8 + 4) + U * 8,
+            "lookup": U * (16 + 8) + U * D * 4 * 2,
+            "pool_fwd": U * D * 4 + N * 4 + (S + 1) * 4 + S * D * 4,
+            "pool_bwd": S * D * 4 + N * 4 + (S + 1) * 4 + U * D * 4,
+            "adam": U * 8 + U * D * 4 * (1 + 6),
+        }
+
+    def stage_times(self, iters):
+        ids = self.feature_ops()
+        uniq, inv = self.dedup(ids)
+        index, rows = self.lookup(uniq)
+        g = self.pool_bwd(inv)
+        return {
+            "feature_ops": _event_ms(self.feature_ops, iters),
+            "dedup": _event_ms(lambda: self.dedup(ids), iters),
+            "lookup": _event_ms(lambda: self.lookup(uniq), iters),
+            "pool_fwd": _event_ms(lambda: self.pool_fwd(rows, inv), iters),
+            "pool_bwd": _event_ms(lambda: self.pool_bwd(inv), iters),
+            "adam": _event_ms(lambda: self.update(index, g), iters),
+        }
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        from oracle import cpu_path
+        b = 8192
+        sparse = [t[:b].cpu().numpy() for t in self.c["sparse"]]
+        dense = [t[:b].cpu().numpy() for t in self.c["dense"]]
+        bnd = self.c["boundaries"][0].cpu().numpy()
+        n = b * self.n_feat
+        off = np.arange(n + 1, dtype=np.int64)
+        grad = self.grad_out[:n].cpu().numpy()
+        table = cpu_path.CpuTable(self.D, 10240, lambda blk: np.zeros((10240, self.D), np.float32), "adam", 1e-3, 1e-8)
+        t0, reps = time.perf_counter(), 0
+        while time.perf_counter() - t0 < budget_s:
+            extra = [oracle.uint64_mod(oracle.bucketize(d, bnd), self.c["mod"]) for d in dense]
+            ids = oracle.ids_encode(sparse + extra, self.tags)
+            cpu_path.train_step(table, ids, off, None, grad)
+            reps += 1
+        dt = time.perf_counter() - t0
+        return n * reps / dt, "first %d samples (%d ids/step) of config 4, full step" % (b, n)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU that owns the whole table; --gpus %d is not supported "
+              "(the sharded exchange is described in DESIGN.md, not built)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    os.environ.setdefault("OMP_NUM_THREADS", "1")
+
+    classes = {"c4": Config4, "c2": Config2}
+    main_wl = classes[args.workload]()
+    for _ in range(args.warmup):
+        main_wl.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        main_wl.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    value = main_wl.ids_per_step / (dt / args.steps)
+
+    out = {
+        "metric": "embedding ids/sec (lookup+pool+bwd+sparse opt) at 1 GPU",
+        "value": value, "unit": "ids/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": main_wl.name, "ids_per_step": main_wl.ids_per_step},
+    }
+
+    extras = {}
+    if args.workload == "c4":
+        stages = main_wl.stage_times(max(5, args.steps))
+        ab = main_wl.algorithmic_bytes()
+        total_bytes = sum(ab.values())
+        dom = max(stages, key=stages.get)
+        out["config"]["unique_ids_per_step"] = main_wl.U
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": ab[dom] / stages[dom] / 1e6,
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": ab[dom] / stages[dom] / 1e6 / HBM_PEAK_GBS, "traffic": None}
+        out["step_roofline"] = {"algorithmic_bytes": total_bytes, "achieved": total_bytes / ms_per_step / 1e6,
+                                "frac": total_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, "unit": "GB/s"}
+        out["stages_ms"] = {k: round(v, 4) for k, v in stages.items()}
+        out["stages_gbs"] = {k: round(ab[k] / stages[k] / 1e6, 1) for k in stages}
+        if not args.no_extra:
+            c2 = Config2()
+            extras[c2.name] = {}
+            for kname, (fn, nbytes) in c2.kernels().items():
+                ms = _event_ms(fn, 10)
+                extras[c2.name][kname] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                                          "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            ms = _event_ms(c2.step, 5)
+            extras[c2.name]["ids_per_s"] = c2.ids_per_step / ms * 1e3
+            del c2
+    else:
+        kern = main_wl.kernels()
+        res = {k: _event_ms(fn, 10) for k, (fn, _) in kern.items()}
+        dom = max(res, key=res.get)
+        nbytes = kern[dom][1]
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": nbytes / res[dom] / 1e6, "peak": HBM_PEAK_GBS,
+                           "unit": "GB/s", "frac": nbytes / res[dom] / 1e6 / HBM_PEAK_GBS, "traffic": None}
+        out["stages_ms"] = {k: round(v, 4) for k, v in res.items()}
+    if extras:
+        out["workloads"] = extras
+
+    if not args.no_cpu_baseline:
+        v, sample = main_wl.cpu_baseline(12.0)
+        out["cpu_baseline"] = {"value": v, "unit": "ids/s", "cores": 1, "kind": "port", "sample": sample}
+    from recis_amd import _lib
+    out["device_errors"] = _lib.poll_device_errors()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -73,3 +73,21 @@ def config1_step(step, seed=0, batch=4096, num_keys=1_000_000, alpha=1.05, max_l
 def seeded_block(seed, block_index, block_size, dim, std=0.01):
     """Initial rows of one storage block, identical on the CPU and the GPU side."""
     return (std * _rng([seed, 7919, block_index]).standard_normal((block_size, dim))).astype(np.float32)
+
+
+def config4(device="cuda", seed=4, batch=65536, n_sparse=26, n_dense=13, n_boundaries=64, mod=1_000_000):
+    """Click-through-style merged table (BASELINE config 4): 26 int64 id fields with log-uniform
+    cardinalities in 10..1e7, 13 lognormal(0, 2) dense fields bucketized against 64 sorted
+    boundaries and taken mod 1e6; one id per field per sample."""
+    rng = _rng(seed)
+    cards = np.floor(10 ** rng.uniform(1, 7, size=n_sparse)).astype(np.int64)
+    sparse = [torch.from_numpy(rng.integers(0, c, size=batch, dtype=np.int64)).to(device) for c in cards]
+    dense = [torch.from_numpy(rng.lognormal(0.0, 2.0, size=batch).astype(np.float32)).to(device)
+             for _ in range(n_dense)]
+    # boundaries: 64 quantile-like points of lognormal(0, 2)
+    q = (np.arange(1, n_boundaries + 1) - 0.5) / n_boundaries
+    from scipy.special import erfinv
+    z = np.sqrt(2.0) * erfinv(2 * q - 1)
+    bnd = torch.from_numpy(np.exp(2.0 * z).astype(np.float32)).to(device)
+    return {"sparse": sparse, "dense": dense, "boundaries": [bnd] * n_dense, "mod": mod,
+            "cardinalities": cards, "batch": batch, "num_ids": batch * (n_sparse + n_dense)}
