@@ -144,9 +144,9 @@ class Config4:
         return o.ids_encode(self.c["sparse"] + extra, self.tags)
 
     def dedup(self, ids):
-        uniq, inv, count = self.ops.ids_unique(ids)
-        self.U = int(count.item())
-        return uniq[: self.U], inv
+        self.plan = self.ops.ids_unique_plan(ids)
+        self.U = self.plan.U
+        return self.plan.unique, self.plan.inverse
 
     def lookup(self, uniq):
         return self.table.embedding_lookup(uniq, False)
@@ -155,7 +155,7 @@ class Config4:
         return self.ops.segment_reduce_forward(rows, None, inv, self.offsets, "sum")
 
     def pool_bwd(self, inv):
-        return self.ops.segment_reduce_backward(self.grad_out, None, inv, self.offsets, self.U, "sum")
+        return self.ops.segment_reduce_backward_plan(self.grad_out, None, self.offsets, self.plan, "sum")
 
     def update(self, index, g):
         self.table.accept_grad(index, g, unique=True)
@@ -218,12 +218,199 @@ class Config4:
         return n * reps / dt, "first %d samples (%d ids/step) of config 4, full step" % (b, n)
 
 
+
+# --------------------------------------------------------------------- config 3
+class Config3:
+    """IDMap + EmbeddingBlocks at scale: 2e8 resident rows, dim 32 fp32 + two Adam state slots
+    (~77 GB), 2e6 lookups per step, Zipf(1.1), 10 % never-seen keys (admission inserts); rows are
+    expanded to one output row per lookup, the per-lookup gradients are reduced per key, fused
+    sparse Adam, last-seen-step stamp; eviction sweep (keys not seen for 50 steps) timed apart."""
+
+    name = "c3_idmap_blocks_2e8rows_d32_fp32_adam_2e6ids_zipf1.1_10pct_new"
+
+    def __init__(self, resident=200_000_000, ids_per_step=2_000_000, n_batches=8):
+        from recis_amd import ops
+        from recis_amd.nn.initializers import NormalInitializer
+        from recis_amd.nn.modules.hashtable import HashtableImpl
+        from recis_amd.optim.sparse_impl import SparseAdamImpl
+        self.ops = ops
+        self.D, self.N, self.resident = 32, ids_per_step, resident
+        self.ids_per_step = ids_per_step
+        init = NormalInitializer(0.0, 0.01)
+        init.set_shape([10240, self.D])
+        init.set_dtype(torch.float32)
+        reserve = int(resident * 1.12) + 40 * ids_per_step // 10
+        self.table = HashtableImpl(10240, [self.D], torch.float32, torch.device("cuda"), False, ["c3"],
+                                   init.build().impl(), reserve_rows=reserve)
+        self.table.append_step_filter_slot("step_filter", 0)
+        self.opt = SparseAdamImpl.make({"c3": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0)
+        chunk = 25_000_000
+        for lo in range(0, resident, chunk):
+            ranks = torch.arange(lo, min(lo + chunk, resident), device="cuda")
+            self.table.insert_lookup_index(workloads.splitmix64_torch(ranks))
+        self.batches = workloads.config3_batches(n_batches, resident, ids_per_step)
+        g = torch.Generator(device="cuda").manual_seed(3)
+        self.grad_out = torch.randn((ids_per_step, self.D), device="cuda", generator=g)
+        self.span = torch.tensor([0, ids_per_step], dtype=torch.int64, device="cuda")
+        self.step_no = 0
+        self.step_t = torch.zeros(1, dtype=torch.int64, device="cuda")
+        self.U = None
+        torch.cuda.synchronize()
+
+    def step(self):
+        o = self.ops
+        ids = self.batches[self.step_no % len(self.batches)]
+        self.step_no += 1
+        plan = o.ids_unique_plan(ids)
+        self.U = plan.U
+        index, rows = self.table.embedding_lookup(plan.unique, False)
+        self.table.update_slot("step_filter", index, self.step_t)
+        out = o.gather(plan.inverse, rows)                          # one row per lookup
+        g = o.segment_reduce_backward_plan(self.grad_out, None, self.span, plan, "tile")
+        self.table.accept_grad(index, g, unique=True)
+        self.opt.step()
+        self.opt.zero_grad()
+        self.step_t += 1
+        return out
+
+    def algorithmic_bytes(self):
+        N, U, D = self.N, self.U, self.D
+        return N * (8 + 4) + U * 8 + U * (16 + 8) + int(0.1 * N) * 16 + U * D * 4 + N * (4 + D * 4) \
+            + N * (4 + D * 4) + U * D * 4 * 7 + U * 8
+
+    def evict_sweep_ms(self, filter_step=50):
+        """One reference-style sweep: snapshot of all (key, row) pairs, stamp test, erase + free +
+        re-initialise. The threshold is set so that nothing is old enough: the sweep cost without
+        shrinking the table under the benchmark."""
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ids, index = self.table.ids_map()
+        chunks, chunk_rows = self.table.get_slot("step_filter").kernel_blocks()
+        mask = self.ops.block_filter(index, chunks, chunk_rows, -1)
+        self.table.delete(torch.masked_select(ids, mask), torch.masked_select(index, mask), "step_filter")
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3
+
+    def cpu_baseline(self, budget_s):
+        from oracle import cpu_path
+        import oracle
+        resident, n = 2_000_000, 200_000
+        table = cpu_path.CpuTable(self.D, 10240, lambda blk: np.zeros((10240, self.D), np.float32), "adam", 1e-3, 1e-8)
+        keys = workloads.splitmix64(np.arange(resident, dtype=np.uint64)).astype(np.int64)
+        table.lookup(np.unique(keys))
+        rng = np.random.default_rng(3)
+        grad = rng.standard_normal((n, self.D)).astype(np.float32)
+        span = np.array([0, n])
+        t0, reps = time.perf_counter(), 0
+        while time.perf_counter() - t0 < budget_s:
+            ranks = workloads.bounded_zipf(rng, n, 1.1, resident)
+            ranks[: n // 10] = resident + reps * (n // 10) + np.arange(n // 10)
+            ids = workloads.splitmix64(ranks.astype(np.uint64)).astype(np.int64)
+            uniq, inv = np.unique(ids, return_inverse=True)
+            index, rows = table.lookup(uniq)
+            oracle.gather(inv, rows)
+            g = oracle.segment_reduce_backward(grad, None, inv, span, len(uniq), "tile")
+            table.apply(index, g)
+            reps += 1
+        dt = time.perf_counter() - t0
+        return n * reps / dt, "table scaled to %d resident rows, %d lookups/step (1/100 and 1/10 of config 3)" % (resident, n)
+
+
+# --------------------------------------------------------------------- config 5
+class Config5:
+    """Long behaviour sequences: batch 2048 x 4 sequence fields, lognormal lengths (mean 200, max
+    1000), Zipf(1.2) ids over 5e7 keys, dim 128, bf16 row storage with fp32 accumulation; mean
+    pooling plus the unpooled gather padded to each field's longest sequence; backward of both
+    into the unique rows, sparse Adagrad."""
+
+    name = "c5_sequences_2048x4_lognormal200_d128_bf16_mean+padded_adagrad"
+
+    def __init__(self):
+        from recis_amd import ops
+        from recis_amd.nn.initializers import NormalInitializer
+        from recis_amd.nn.modules.hashtable import HashtableImpl
+        from recis_amd.optim.sparse_impl import SparseAdagradImpl
+        self.ops = ops
+        c = workloads.config5()
+        self.c = c
+        self.D, self.N = 128, c["num_ids"]
+        self.ids_per_step = self.N
+        self.fields = c["fields"]
+        self.batch = [c["batch"]] * len(self.fields)
+        self.seq = [f["pad_len"] for f in self.fields]
+        init = NormalInitializer(0.0, 0.01)
+        init.set_shape([10240, self.D])
+        init.set_dtype(torch.bfloat16)
+        self.table = HashtableImpl(10240, [self.D], torch.bfloat16, torch.device("cuda"), True,
+                                   ["s%d" % i for i in range(len(self.fields))], init.build().impl(),
+                                   reserve_rows=int(self.N * 1.1))
+        self.opt = SparseAdagradImpl.make({"c5": self.table}, 0.01, 1e-8)
+        self.S = sum(self.batch)
+        self.pad_rows = sum(b * s for b, s in zip(self.batch, self.seq))
+        g = torch.Generator(device="cuda").manual_seed(5)
+        self.g_pool = torch.randn((self.S, self.D), device="cuda", generator=g)
+        self.g_tile = torch.randn((self.pad_rows, self.D), device="cuda", generator=g).to(torch.bfloat16)
+        self.offsets = ops.merge_offsets([f["offsets"] for f in self.fields], [f["num_ids"] for f in self.fields])
+        self.U = None
+
+    def step(self):
+        o = self.ops
+        ids = o.ids_encode([f["values"] for f in self.fields], list(range(len(self.fields))))
+        plan = o.ids_unique_plan(ids)
+        self.U = plan.U
+        inv = plan.inverse
+        index, rows = self.table.embedding_lookup(plan.unique, False)
+        pooled = o.segment_reduce_forward(rows, None, inv, self.offsets, "mean", out_dtype=torch.float32)
+        padded, batch_seq = o.ragged_tile(self.batch, self.seq, inv, self.offsets, rows)
+        g = o.segment_reduce_backward_plan(self.g_pool, None, self.offsets, plan, "mean")
+        o.csr_gather_reduce(self.g_tile, plan, plan.src_for_tile(self.batch, self.seq, self.offsets), out=g,
+                            accumulate=True)
+        self.table.accept_grad(index, g, unique=True)
+        self.opt.step()
+        self.opt.zero_grad()
+        return pooled, padded
+
+    def algorithmic_bytes(self):
+        N, U, S, D = self.N, self.U, self.S, self.D
+        return 12 * N + U * (24 + 4 * D * 2) + S * (D * 4 + D * 4) + 2 * self.pad_rows * D * 2 + 8 * N
+
+    def cpu_baseline(self, budget_s):
+        import oracle
+        from oracle import cpu_path
+        b = 128
+        vals, offs = [], []
+        for f in self.fields:
+            off = f["offsets"][: b + 1].cpu().numpy().astype(np.int64)
+            vals.append(f["values"][: int(off[-1])].cpu().numpy())
+            offs.append(off)
+        n = sum(len(v) for v in vals)
+        offsets = oracle.merge_offsets(offs, [len(v) for v in vals])
+        ids = oracle.ids_encode(vals, list(range(len(vals))))
+        S = len(offsets) - 1
+        g_pool = self.g_pool[:S].cpu().numpy()
+        rows_pad = sum(b * s for s in self.seq)
+        g_tile = np.ones((rows_pad, self.D), np.float32)
+        table = cpu_path.CpuTable(self.D, 10240, lambda blk: np.zeros((10240, self.D), np.float32), "adagrad", 0.01, 1e-8)
+        t0, reps = time.perf_counter(), 0
+        while time.perf_counter() - t0 < budget_s:
+            uniq, inv = np.unique(ids, return_inverse=True)
+            index, rows = table.lookup(uniq)
+            oracle.segment_reduce_forward(rows, None, inv, offsets, "mean")
+            oracle.ragged_tile([b] * len(vals), self.seq, inv, offsets, rows)
+            g = oracle.segment_reduce_backward(g_pool, None, inv, offsets, len(uniq), "mean")
+            g += oracle.ragged_tile_back([b] * len(vals), self.seq, inv, offsets, g_tile, len(uniq))
+            table.apply(index, g)
+            reps += 1
+        dt = time.perf_counter() - t0
+        return n * reps / dt, "first %d of 2048 sequences per field (%d ids/step) of config 5, fp32 rows" % (b, n)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     args = ap.parse_args()
@@ -235,7 +422,7 @@ def main():
     torch.cuda.set_device(0)
     os.environ.setdefault("OMP_NUM_THREADS", "1")
 
-    classes = {"c4": Config4, "c2": Config2}
+    classes = {"c4": Config4, "c2": Config2, "c3": Config3, "c5": Config5}
     main_wl = classes[args.workload]()
     for _ in range(args.warmup):
         main_wl.step()
@@ -256,6 +443,31 @@ def main():
         "config": {"workload": main_wl.name, "ids_per_step": main_wl.ids_per_step},
     }
 
+    def timed_steps(wl, steps, warmup):
+        for _ in range(warmup):
+            wl.step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            wl.step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / steps * 1e3
+
+    def c2_summary(wl):
+        res = {}
+        for kname, (fn, nbytes) in wl.kernels().items():
+            ms = _event_ms(fn, 10)
+            res[kname] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                          "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        return res
+
+    def step_summary(wl, ms):
+        nbytes = wl.algorithmic_bytes()
+        nbytes = sum(nbytes.values()) if isinstance(nbytes, dict) else nbytes
+        return {"ms_per_step": round(ms, 4), "ids_per_s": wl.ids_per_step / ms * 1e3,
+                "unique_ids_per_step": wl.U, "algorithmic_bytes": nbytes,
+                "gbs": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
     extras = {}
     if args.workload == "c4":
         stages = main_wl.stage_times(max(5, args.steps))
@@ -270,24 +482,39 @@ def main():
                                 "frac": total_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, "unit": "GB/s"}
         out["stages_ms"] = {k: round(v, 4) for k, v in stages.items()}
         out["stages_gbs"] = {k: round(ab[k] / stages[k] / 1e6, 1) for k in stages}
-        if not args.no_extra:
-            c2 = Config2()
-            extras[c2.name] = {}
-            for kname, (fn, nbytes) in c2.kernels().items():
-                ms = _event_ms(fn, 10)
-                extras[c2.name][kname] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
-                                          "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
-            ms = _event_ms(c2.step, 5)
-            extras[c2.name]["ids_per_s"] = c2.ids_per_step / ms * 1e3
-            del c2
+    elif args.workload == "c2":
+        res = c2_summary(main_wl)
+        dom = max(res, key=lambda k: res[k]["ms"])
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": res[dom]["gbs"], "peak": HBM_PEAK_GBS,
+                           "unit": "GB/s", "frac": res[dom]["frac"], "traffic": None}
+        out["stages_ms"] = {k: v["ms"] for k, v in res.items()}
     else:
-        kern = main_wl.kernels()
-        res = {k: _event_ms(fn, 10) for k, (fn, _) in kern.items()}
-        dom = max(res, key=res.get)
-        nbytes = kern[dom][1]
-        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": nbytes / res[dom] / 1e6, "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": nbytes / res[dom] / 1e6 / HBM_PEAK_GBS, "traffic": None}
-        out["stages_ms"] = {k: round(v, 4) for k, v in res.items()}
+        s = step_summary(main_wl, ms_per_step)
+        out["config"]["unique_ids_per_step"] = main_wl.U
+        out["roofline"] = {"bound": "hbm", "kernel": "whole step", "achieved": s["gbs"], "peak": HBM_PEAK_GBS,
+                           "unit": "GB/s", "frac": s["frac"], "traffic": None}
+        if args.workload == "c3":
+            out["evict_sweep_ms"] = round(main_wl.evict_sweep_ms(), 3)
+    if not args.no_extra:
+        main_name = main_wl.name
+        if args.workload != "c4":
+            del main_wl
+            torch.cuda.empty_cache()
+        for key, cls in classes.items():
+            if key == args.workload:
+                continue
+            wl = cls()
+            if key == "c2":
+                extras[wl.name] = c2_summary(wl)
+                extras[wl.name]["ids_per_s"] = wl.ids_per_step / _event_ms(wl.step, 5) * 1e3
+            else:
+                extras[wl.name] = step_summary(wl, timed_steps(wl, 8, 3))
+                if key == "c3":
+                    extras[wl.name]["evict_sweep_ms"] = round(wl.evict_sweep_ms(), 3)
+            del wl
+            torch.cuda.empty_cache()
+        if args.workload != "c4":
+            main_wl = classes[args.workload]() if not args.no_cpu_baseline else None
     if extras:
         out["workloads"] = extras
 

@@ -313,6 +313,56 @@ int recis_merge_offsets(const void* const* offsets_ptrs, const int64_t* sizes,
 int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inverse_out,
                  int inverse_is64, int64_t* count_out_dev, void* stream);
 
+/*
+ * Batch plan: dedup plus the transposed index. On top of what recis_unique returns
+ * (unique ids in order of first occurrence, int32 inverse, count), the occurrences are
+ * grouped by unique id:
+ *   row_start_out [n + 1]  list of unique id u = list[row_start[u] .. row_start[u+1]);
+ *                          entries U .. n hold n
+ *   list_out      [n]      occurrence indices grouped by unique id
+ *   pos_out       [n]      position of occurrence i in list_out (may be NULL)
+ *   hot_items_out [2*hot_cap] (row, chunk) work items for ids with more than 256
+ *                          occurrences; hot_cap >= n/256 + n/8192 + 2, or 0 to skip
+ *   counts_out_dev [2]     device words: number of unique ids, number of hot items
+ * With it, a gradient scatter over duplicated ids (the atomic loops of
+ * csrc/ops/embedding_segment_reduce_kernel.cu:79-120, segment_ops_kernel.cu:133-165,
+ * ragged_tile_kernel.cu:46-60 and the unique + index_add_ of
+ * recis/nn/modules/hashtable.py:555-586) becomes a gather-reduce per unique row.
+ * No counterpart in the reference.
+ */
+int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
+                      int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
+                      int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev,
+                      void* stream);
+
+/*
+ * Per list entry, the input row it reads and its coefficient, for the backward of
+ *   pooled segments: src = segment of the occurrence, coef = weight (/ length for MEAN)
+ *                    (coef_out may be NULL when there are no weights and mean == 0)
+ *   padded gather:   src = padded output row of the occurrence, -1 beyond seq[f]
+ * pos = pos_out of recis_unique_plan. Entries of occurrences outside the offsets range
+ * get src = -1 (skipped).
+ */
+int recis_csr_fill_pool(const void* offsets, int off_is64, int64_t S, int64_t n, const void* weight,
+                        int weight_dtype, const int32_t* pos, int mean, int32_t* src_out,
+                        float* coef_out, void* stream);
+int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_features,
+                        const void* offsets, int off_is64, int64_t n, const int32_t* pos,
+                        int32_t* src_out, void* stream);
+
+/*
+ * out[u, :] (+)= sum over k in [row_start[u], row_start[u+1]) of coef[k] * rows[src[k], :]
+ * for u < U. Rows with at most 256 entries are reduced by a small group of lanes and
+ * written once; hot rows are reduced by whole workgroups per 8192-entry chunk and
+ * combined with a few fp32 atomics (out must then be fp32, D <= 1024). accumulate != 0
+ * adds to what out holds. src < 0 skips the entry; coef may be NULL (= 1).
+ */
+int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                            const void* coef, int coef_dtype, const int32_t* row_start,
+                            const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev,
+                            void* out, int out_dtype, int64_t U, int64_t D, int accumulate,
+                            void* stream);
+
 /* ------------------------------------------------------------------------- *
  * Feature-engine scalar ops (lists as HOST arrays of device pointers)
  * ------------------------------------------------------------------------- */

@@ -96,7 +96,10 @@ set_insert_kernel(int64_t* __restrict__ keys, int32_t* __restrict__ minpos, uint
   } else {
     p = mix_id(key) & mask;
     for (;;) {
-      int64_t k = __atomic_load_n(&keys[p], __ATOMIC_RELAXED);
+      // plain (L1-cacheable) load on purpose: thousands of duplicates of a hot id would
+      // otherwise queue up at one L2 channel. A stale "empty" is harmless, the CAS below
+      // then returns the real occupant; a slot never changes once it holds a key.
+      int64_t k = keys[p];
       if (k == kSetEmpty) {
         k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&keys[p]),
                                            static_cast<unsigned long long>(kSetEmpty),
@@ -107,7 +110,10 @@ set_insert_kernel(int64_t* __restrict__ keys, int32_t* __restrict__ minpos, uint
       p = (p + 1) & mask;  // capacity >= 2n: an empty slot always exists
     }
   }
-  atomicMin(&minpos[p], static_cast<int32_t>(i));
+  // duplicates of a hot id arrive by the thousand: only those that can still lower the
+  // minimum pay for the atomic (the stored value only ever decreases)
+  if (minpos[p] > static_cast<int32_t>(i))  // plain load: a stale (larger) value only costs an atomic
+    atomicMin(&minpos[p], static_cast<int32_t>(i));
   slotpos[i] = static_cast<int32_t>(p);
 }
 

@@ -47,10 +47,10 @@ __device__ __forceinline__ uint64_t mix_key(int64_t key) {
 }
 
 __device__ __forceinline__ int64_t ld_relaxed(const int64_t* p) {
-  return __atomic_load_n(p, __ATOMIC_RELAXED);
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void st_relaxed(int64_t* p, int64_t v) {
-  __atomic_store_n(p, v, __ATOMIC_RELAXED);
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __global__ void __launch_bounds__(kBlock) fill_slots_kernel(Slot* t, int64_t n) {

@@ -19,8 +19,9 @@ class EmbeddingSegmentReduceRagged(torch.autograd.Function):
     rows are kept per segment (zero padded), returned as ``[S, tile_len * D]``."""
 
     @staticmethod
-    def forward(ctx, unique_emb, weight, reverse_indices, offsets, combiner, combiner_kwargs):
+    def forward(ctx, unique_emb, weight, reverse_indices, offsets, combiner, combiner_kwargs, plan=None):
         ctx.combiner = combiner
+        ctx.plan = plan
         ctx.unique_size = unique_emb.shape[0]
         ctx.emb_dtype = unique_emb.dtype
         if combiner == "tile":
@@ -46,24 +47,33 @@ class EmbeddingSegmentReduceRagged(torch.autograd.Function):
             rev, offsets = ctx.saved_tensors
             batch_seq, info = ctx.tile
             D = grad.shape[1] // info[3]
-            g = ops.ragged_tile_back(batch_seq, info, rev, offsets, grad.view(-1, D))
-            return g.to(ctx.emb_dtype), None, None, None, None, None
+            if ctx.plan is not None:
+                src = ctx.plan.src_for_tile([info[2]], [info[3]], offsets)
+                g = ops.csr_gather_reduce(grad.view(-1, D), ctx.plan, src)
+            else:
+                g = ops.ragged_tile_back(batch_seq, info, rev, offsets, grad.view(-1, D))
+            return g.to(ctx.emb_dtype), None, None, None, None, None, None
         if ctx.combiner == "max":
             rev, offsets, argmax = ctx.saved_tensors
             g = ops.segment_reduce_backward(grad, None, rev, offsets, ctx.unique_size, "max", argmax=argmax,
                                             out_dtype=ctx.emb_dtype)
-            return g, None, None, None, None, None
+            return g, None, None, None, None, None, None
         rev, offsets, weight = ctx.saved_tensors
-        g = ops.segment_reduce_backward(grad, weight, rev, offsets, ctx.unique_size, ctx.combiner,
-                                        out_dtype=ctx.emb_dtype)
-        return g, None, None, None, None, None
+        if ctx.plan is not None:
+            g = ops.segment_reduce_backward_plan(grad, weight, offsets, ctx.plan, ctx.combiner).to(ctx.emb_dtype)
+        else:
+            g = ops.segment_reduce_backward(grad, weight, rev, offsets, ctx.unique_size, ctx.combiner,
+                                            out_dtype=ctx.emb_dtype)
+        return g, None, None, None, None, None, None
 
 
 def ragged_embedding_segment_reduce(unique_emb: torch.Tensor, weight: Optional[torch.Tensor],
                                     reverse_indices: torch.Tensor, offsets: torch.Tensor, combiner: str,
-                                    combiner_kwargs: Optional[dict] = None):
+                                    combiner_kwargs: Optional[dict] = None, plan=None):
     """``recis.nn.functional.embedding_ops.ragged_embedding_segment_reduce``
-    (embedding_ops.py:332-420), plus the ``"max"`` combiner."""
+    (embedding_ops.py:332-420), plus the ``"max"`` combiner. ``plan`` (the ``BatchPlan`` whose
+    ``inverse`` is ``reverse_indices``) switches the backward from atomics to the gather-reduce
+    over the plan's occurrence lists."""
     if combiner_kwargs is None:
         combiner_kwargs = {}
     assert combiner in ["sum", "mean", "tile", "max"], "combiner %s is not supported" % combiner
@@ -75,4 +85,4 @@ def ragged_embedding_segment_reduce(unique_emb: torch.Tensor, weight: Optional[t
         weight = ops.segment_mean(unique_emb, weight, seg, offsets.numel() - 1)
         combiner = "sum"
     return EmbeddingSegmentReduceRagged.apply(unique_emb, weight, reverse_indices, offsets, combiner,
-                                              combiner_kwargs)
+                                              combiner_kwargs, plan)

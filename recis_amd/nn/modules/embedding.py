@@ -133,16 +133,17 @@ class DynamicEmbedding(torch.nn.Module):
             weight = input_weights
         if weight is not None:
             weight = weight.to(dev) if opt.use_weight else None
-        uniq, inverse, count = ops.ids_unique(val, inverse_dtype=torch.int32)
-        uniq = uniq[: int(count.item())]
+        plan = ops.ids_unique_plan(val)
+        uniq, inverse = plan.unique, plan.inverse
         emb = lookup_unique_rows(self._hashtable, uniq, opt.admit_hook, opt.trainable)
         if opt.grad_reduce_by == "id" and self.training and opt.trainable:
             # mean over the duplicates of each id: pool the expanded rows instead
-            emb = GradIDMeanFunction.apply(emb, inverse.long())
-            inverse = torch.arange(val.numel(), device=dev, dtype=torch.int32)
+            emb = GradIDMeanFunction.apply(emb, inverse, plan)
+            inverse, plan = None, None
         if weight is not None and weight.dtype != emb.dtype:
             weight = weight.to(emb.dtype)
-        out = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner, opt.combiner_kwargs)
+        out = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner, opt.combiner_kwargs,
+                                              plan=plan)
         if opt.combiner == "tile":
             return out.view(tuple(shape) + (opt.combiner_kwargs["tile_len"] * opt.embedding_dim,))
         return out.view(tuple(shape) + (opt.embedding_dim,))

@@ -125,13 +125,13 @@ class EmbeddingEngine(torch.nn.Module):
                 weight = None
                 if all(w is not None for w in weights):
                     weight = weights[0] if len(weights) == 1 else torch.cat(weights)
-                uniq, inverse, count = ops.ids_unique(ids, inverse_dtype=torch.int32)
-                uniq = uniq[: int(count.item())]
-                emb = lookup_unique_rows(table, uniq, opt0.admit_hook, opt0.trainable)
+                plan = ops.ids_unique_plan(ids)
+                inverse = plan.inverse
+                emb = lookup_unique_rows(table, plan.unique, opt0.admit_hook, opt0.trainable)
                 if weight is not None and weight.dtype != emb.dtype:
                     weight = weight.to(emb.dtype)
                 pooled = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt0.combiner,
-                                                         opt0.combiner_kwargs)
+                                                         opt0.combiner_kwargs, plan=plan)
                 seg_counts = [o.numel() - 1 for o in offs]
                 width = pooled.shape[1]
                 for name, part, shape in zip(names, torch.split(pooled, seg_counts), shapes):

@@ -548,17 +548,18 @@ class GradIDMeanFunction(torch.autograd.Function):
     each id (recis/nn/modules/hashtable.py:484-537)."""
 
     @staticmethod
-    def forward(ctx, embedding, index):
+    def forward(ctx, embedding, index, plan=None):
         ctx.save_for_backward(index)
         ctx.unique_size = embedding.shape[0]
+        ctx.plan = plan
         return ops.gather(index, embedding)
 
     @staticmethod
     def backward(ctx, grad_outputs):
         (index,) = ctx.saved_tensors
-        summed = _scatter_sum(grad_outputs, index, ctx.unique_size)
+        summed = _scatter_sum(grad_outputs, index, ctx.unique_size, ctx.plan)
         counts = torch.bincount(index.long(), minlength=ctx.unique_size).clamp_(min=1)
-        return (summed / counts.view(-1, 1).to(summed.dtype)).to(grad_outputs.dtype), None
+        return (summed / counts.view(-1, 1).to(summed.dtype)).to(grad_outputs.dtype), None, None
 
 
 class GradWorkerMeanFunction(torch.autograd.Function):
@@ -566,10 +567,11 @@ class GradWorkerMeanFunction(torch.autograd.Function):
     by the number of workers (recis/nn/modules/hashtable.py:540-586)."""
 
     @staticmethod
-    def forward(ctx, embedding, index, slice_num):
+    def forward(ctx, embedding, index, slice_num, plan=None):
         ctx.save_for_backward(index)
         ctx.unique_size = embedding.shape[0]
         ctx.slice_num = slice_num
+        ctx.plan = plan
         return ops.gather(index, embedding)
 
     @staticmethod
@@ -577,15 +579,19 @@ class GradWorkerMeanFunction(torch.autograd.Function):
         (index,) = ctx.saved_tensors
         if ctx.slice_num != 1:
             grad_outputs = grad_outputs / ctx.slice_num
-        return _scatter_sum(grad_outputs, index, ctx.unique_size).to(grad_outputs.dtype), None, None
+        return _scatter_sum(grad_outputs, index, ctx.unique_size, ctx.plan).to(grad_outputs.dtype), None, None, None
 
 
-def _scatter_sum(grad_rows, index, unique_size):
-    """sum of ``grad_rows[i]`` into row ``index[i]`` of a ``[unique_size, D]`` result."""
+def _scatter_sum(grad_rows, index, unique_size, plan=None):
+    """sum of ``grad_rows[i]`` into row ``index[i]`` of a ``[unique_size, D]`` result: a
+    gather-reduce over the batch plan's occurrence lists when there is one, fp32 atomics else."""
     n = index.numel()
     flat = grad_rows.reshape(n, -1).contiguous()
-    span = torch.tensor([0, n], dtype=torch.int64, device=index.device)
-    out = ops.segment_reduce_backward(flat, None, index, span, unique_size, "tile", out_dtype=torch.float32)
+    if plan is not None:
+        out = ops.csr_gather_reduce(flat, plan, plan.occ)
+    else:
+        span = torch.tensor([0, n], dtype=torch.int64, device=index.device)
+        out = ops.segment_reduce_backward(flat, None, index, span, unique_size, "tile", out_dtype=torch.float32)
     return out.view((unique_size,) + tuple(grad_rows.shape[1:]))
 
 
@@ -640,10 +646,12 @@ class HashTable(torch.nn.Module):
             self._filter_hook_impl = torch.nn.Identity()
 
     def _unique(self, ids):
+        """(unique ids, inverse, batch plan | None)."""
         if self._dedup == "sorted":
-            return ids.unique(return_inverse=True)
-        uniq, inverse, count = ops.ids_unique(ids, inverse_dtype=torch.int64)
-        return uniq[: int(count.item())], inverse
+            uniq, inverse = ids.unique(return_inverse=True)
+            return uniq, inverse, None
+        plan = ops.ids_unique_plan(ids)
+        return plan.unique, plan.inverse, plan
 
     def forward(self, ids: torch.Tensor, admit_hook: AdmitHook = None) -> torch.Tensor:
         from .hashtable_hook_impl import HashtableHookFactory
@@ -651,14 +659,14 @@ class HashTable(torch.nn.Module):
         admit_hook_impl = HashtableHookFactory().create_admit_hook(self, admit_hook) if admit_hook else None
         shape = tuple(ids.shape)
         ids = ids.to(self._device).reshape(-1)
-        uids, index = self._unique(ids)
+        uids, index, plan = self._unique(ids)
         if self.training and self._dtype not in (torch.int8, torch.int32, torch.int64):
             emb_idx, embedding = HashTableLookupHelpFunction.apply(uids, self._hashtable_impl,
                                                                    self._backward_holder, admit_hook_impl)
             if self._grad_reduce_by == "id":
-                embedding = GradIDMeanFunction.apply(embedding, index)
+                embedding = GradIDMeanFunction.apply(embedding, index, plan)
             else:
-                embedding = GradWorkerMeanFunction.apply(embedding, index, self._worker_num)
+                embedding = GradWorkerMeanFunction.apply(embedding, index, self._worker_num, plan)
             self._filter_hook_impl(emb_idx)
         else:
             _, embedding = self._hashtable_impl.embedding_lookup(uids.detach(), True)

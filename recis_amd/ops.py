@@ -647,3 +647,108 @@ class IdMap:
 
     def reserve(self, n_keys):
         check(lib().recis_idmap_reserve(self._h, i64(n_keys), stream_ptr(self.device)))
+
+
+# ------------------------------------------------------------------ batch plan
+_HOT_LEN, _HOT_CHUNK = 256, 8192
+
+
+class BatchPlan:
+    """Dedup of one batch of ids plus the occurrence lists per unique id.
+
+    ``unique`` [U], ``inverse`` int32 [N] (``unique[inverse] == ids``), ``row_start`` int32
+    [N + 1] and ``occ`` int32 [N]: the occurrences of unique id ``u`` are
+    ``occ[row_start[u]:row_start[u + 1]]``; ``pos`` [N] is the position of each occurrence
+    in ``occ``. ``U`` is the host copy of the unique count (reading it synchronises once).
+    """
+
+    __slots__ = ("n", "U", "unique", "inverse", "row_start", "occ", "pos", "hot_items", "hot_cap", "counts",
+                 "_pool_fill")
+
+    def src_coef_for_pool(self, offsets, weight, mean):
+        """(src, coef) per list entry for the backward of pooled segments, cached per
+        (offsets, weight, mean) so that forward-time and backward-time callers share it."""
+        S = offsets.numel() - 1
+        if S == self.n and weight is None:
+            return self.occ, None  # one id per segment: the segment of an occurrence is itself
+        key = (offsets.data_ptr(), 0 if weight is None else weight.data_ptr(), bool(mean))
+        if self._pool_fill is not None and self._pool_fill[0] == key:
+            return self._pool_fill[1], self._pool_fill[2]
+        src = torch.empty(self.n, dtype=torch.int32, device=offsets.device)
+        need_coef = weight is not None or mean
+        coef = torch.empty(self.n, dtype=torch.float32, device=offsets.device) if need_coef else None
+        weight = _contig(weight)
+        check(lib().recis_csr_fill_pool(ptr(offsets), _index_kind(offsets, "offsets"), i64(S), i64(self.n),
+                                        ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
+                                        ptr(self.pos), int(bool(mean)), ptr(src), ptr(coef),
+                                        stream_ptr(offsets.device)))
+        self._pool_fill = (key, src, coef)
+        return src, coef
+
+    def src_for_tile(self, batch, seq, offsets):
+        """src per list entry for the backward of the padded gather (``ragged_tile``)."""
+        src = torch.empty(self.n, dtype=torch.int32, device=offsets.device)
+        if self.n:
+            check(lib().recis_csr_fill_tile(_host_i64(batch), _host_i64(seq), i64(len(batch)), ptr(offsets),
+                                            _index_kind(offsets, "offsets"), i64(self.n), ptr(self.pos), ptr(src),
+                                            stream_ptr(offsets.device)))
+        return src
+
+
+def ids_unique_plan(ids):
+    """Dedup + transposed index of a batch of ids (``recis_unique_plan``)."""
+    ids = _ids64(ids)
+    n = ids.numel()
+    dev = ids.device
+    p = BatchPlan()
+    p.n = n
+    uniq = torch.empty(n, dtype=torch.int64, device=dev)
+    p.inverse = torch.empty(n, dtype=torch.int32, device=dev)
+    p.row_start = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    p.occ = torch.empty(n, dtype=torch.int32, device=dev)
+    p.pos = torch.empty(n, dtype=torch.int32, device=dev)
+    p.hot_cap = n // _HOT_LEN + n // _HOT_CHUNK + 2
+    p.hot_items = torch.empty(2 * p.hot_cap, dtype=torch.int32, device=dev)
+    p.counts = torch.empty(2, dtype=torch.int64, device=dev)
+    p._pool_fill = None
+    check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(uniq), ptr(p.inverse), ptr(p.row_start), ptr(p.occ),
+                                  ptr(p.pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts), stream_ptr(dev)))
+    p.U = int(p.counts[0].item())
+    p.unique = uniq[: p.U]
+    return p
+
+
+def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False):
+    """``out[u] (+)= sum_k coef[k] * rows[src[k]]`` over the list of every unique id of
+    ``plan``; returns the fp32 ``[U, D]`` result."""
+    require_cuda(rows, src, coef)
+    rows = _contig(rows)
+    D = rows.shape[1]
+    if out is None:
+        out = torch.empty((plan.U, D), dtype=torch.float32, device=rows.device)
+        accumulate = False
+    check(lib().recis_csr_gather_reduce(ptr(rows), dtype_code(rows.dtype), i64(rows.shape[0]), ptr(src), ptr(coef),
+                                        dtype_code(coef.dtype) if coef is not None else 0, ptr(plan.row_start),
+                                        ptr(plan.hot_items), i64(plan.hot_cap), ptr(plan.counts), ptr(out),
+                                        dtype_code(out.dtype), i64(plan.U), i64(D), int(bool(accumulate)),
+                                        stream_ptr(rows.device)))
+    return out
+
+
+def segment_reduce_backward_plan(grad_output, weight, offsets, plan, mode, out=None, accumulate=False):
+    """Backward of the pooling for duplicated ids without atomics on row data: the same
+    result as ``segment_reduce_backward(grad, weight, plan.inverse, offsets, plan.U, mode)``
+    (sum | mean | tile), computed as a gather-reduce over ``plan``'s occurrence lists."""
+    if mode not in ("sum", "mean", "tile"):
+        raise ValueError("Invalid mode for the planned backward: %s" % mode)
+    grad_output, weight, offsets = _contig(grad_output), _contig(weight), _contig(offsets)
+    if mode == "tile":
+        src = plan.occ
+        coef = None if weight is None else gather(plan.occ, weight.view(-1, 1)).view(-1)
+        lo, hi = offsets[0], offsets[-1]
+        if offsets.numel() and (int(lo) != 0 or int(hi) != plan.n):  # rare: occurrences no segment covers
+            cov = ((plan.occ >= lo) & (plan.occ < hi)).float()
+            coef = cov if coef is None else coef.float() * cov
+    else:
+        src, coef = plan.src_coef_for_pool(offsets, weight, mode == "mean")
+    return csr_gather_reduce(grad_output, plan, src, coef, out=out, accumulate=accumulate)

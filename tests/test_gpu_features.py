@@ -189,3 +189,69 @@ def test_ragged_tile_forward_backward(rng, dtype):
     tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=5e-2)
     np.testing.assert_allclose(back.float().cpu().numpy(), exp_b, **tol)
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("n,hi", [(0, 10), (1, 10), (1000, 50), (300000, 40), (200000, 3000), (1000000, 10**7)])
+def test_unique_plan_lists(rng, n, hi):
+    """The plan's dedup equals ids_unique; its lists are a permutation of the occurrences grouped
+    by unique id (hot ids with tens of thousands of repeats included)."""
+    ids = rng.integers(-hi, hi, size=n)
+    if n > 5:
+        ids[3] = -1
+    p = ops.ids_unique_plan(_dev(ids))
+    _, first = np.unique(ids, return_index=True)
+    np.testing.assert_array_equal(p.unique.cpu().numpy(), ids[np.sort(first)])
+    inv = p.inverse.cpu().numpy()
+    np.testing.assert_array_equal(p.unique.cpu().numpy()[inv] if n else inv, ids)
+    rs, occ, pos = p.row_start.cpu().numpy(), p.occ.cpu().numpy(), p.pos.cpu().numpy()
+    assert rs[0] == 0 and np.all(rs[p.U:] == n) and np.all(np.diff(rs[: p.U + 1]) >= 1 if p.U else True)
+    np.testing.assert_array_equal(np.sort(occ), np.arange(n))
+    np.testing.assert_array_equal(occ[pos], np.arange(n))
+    row_of_entry = np.repeat(np.arange(p.U), np.diff(rs[: p.U + 1]))
+    np.testing.assert_array_equal(inv[occ], row_of_entry)
+    counts = p.counts.cpu().numpy()
+    lens = np.diff(rs[: p.U + 1])
+    assert counts[0] == p.U and counts[1] == int(np.sum(np.ceil(lens[lens > 256] / 8192)))
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean", "tile"])
+@pytest.mark.parametrize("D,dtype", [(16, torch.float32), (128, torch.bfloat16), (40, torch.float32)])
+def test_planned_backward_matches_oracle(rng, mode, D, dtype):
+    """Gradient scatter over heavily duplicated ids (Zipf-like head + a cold tail) through the plan:
+    same numbers as the oracle's sequential scatter, hot rows (> 256 occurrences) included."""
+    S = 3000
+    off = ragged_offsets(rng, S, 0, 40, empty_frac=0.1)
+    N = int(off[-1])
+    ids = np.where(rng.random(N) < 0.5, rng.integers(0, 6, size=N), rng.integers(100, 50000, size=N))
+    w = rng.random(N).astype(np.float32)
+    p = ops.ids_unique_plan(_dev(ids))
+    inv = p.inverse.cpu().numpy().astype(np.int64)
+    g = rng.standard_normal((N if mode == "tile" else S, D)).astype(np.float32)
+    g_t = _dev(g, dtype)
+    g_q = g_t.float().cpu().numpy()
+    for use_w in (True, False):
+        got = ops.segment_reduce_backward_plan(g_t, _dev(w) if use_w else None, _dev(off), p, mode).cpu().numpy()
+        exp = oracle.segment_reduce_backward(g_q, w if use_w else None, inv, off, p.U, mode)
+        # hot rows sum up to ~N/12 terms of size ~1: atol scales with that (1e-6 per unit)
+        np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-6 * max(1.0, N / 12.0))
+    acc = torch.ones((p.U, D), device="cuda")
+    ops.segment_reduce_backward_plan(g_t, None, _dev(off), p, mode, out=acc, accumulate=True)
+    exp = 1.0 + oracle.segment_reduce_backward(g_q, None, inv, off, p.U, mode)
+    np.testing.assert_allclose(acc.cpu().numpy(), exp, rtol=1e-5, atol=1e-6 * max(1.0, N / 12.0))
+    assert _lib.poll_device_errors() == 0
+
+
+def test_planned_tile_backward_matches_oracle(rng):
+    batch, seq = [50, 31, 7], [12, 3, 40]
+    D = 32
+    lens = np.concatenate([rng.integers(0, 20, size=b) for b in batch])
+    off = np.concatenate([[0], np.cumsum(lens)])
+    ids = rng.integers(0, 40, size=int(off[-1]))
+    p = ops.ids_unique_plan(_dev(ids))
+    inv = p.inverse.cpu().numpy().astype(np.int64)
+    rows = sum(b * s for b, s in zip(batch, seq))
+    dy = rng.standard_normal((rows, D)).astype(np.float32)
+    src = p.src_for_tile(batch, seq, _dev(off.astype(np.int32)))
+    got = ops.csr_gather_reduce(_dev(dy), p, src).cpu().numpy()
+    exp = oracle.ragged_tile_back(batch, seq, inv, off, dy, p.U)
+    np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-4)

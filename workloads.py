@@ -91,3 +91,77 @@ def config4(device="cuda", seed=4, batch=65536, n_sparse=26, n_dense=13, n_bound
     bnd = torch.from_numpy(np.exp(2.0 * z).astype(np.float32)).to(device)
     return {"sparse": sparse, "dense": dense, "boundaries": [bnd] * n_dense, "mod": mod,
             "cardinalities": cards, "batch": batch, "num_ids": batch * (n_sparse + n_dense)}
+
+
+# ---------------------------------------------------------------- GPU-side helpers (config 3 / 5)
+_M64 = (1 << 64) - 1
+
+
+def _lsr(x, k):
+    """Logical right shift of int64 tensors (torch shifts int64 arithmetically)."""
+    return torch.bitwise_and(torch.bitwise_right_shift(x, k), (1 << (64 - k)) - 1)
+
+
+def _i64(v):
+    v &= _M64
+    return v - (1 << 64) if v >= (1 << 63) else v
+
+
+def splitmix64_torch(x):
+    """The same bijective mix as ``splitmix64`` on int64 tensors (wrapping arithmetic)."""
+    x = x + _i64(0x9E3779B97F4A7C15)
+    x = torch.bitwise_xor(x, _lsr(x, 30)) * _i64(0xBF58476D1CE4E5B9)
+    x = torch.bitwise_xor(x, _lsr(x, 27)) * _i64(0x94D049BB133111EB)
+    return torch.bitwise_xor(x, _lsr(x, 31))
+
+
+def zipf_cdf_torch(num_keys, alpha, device="cuda"):
+    """Cumulative table of the bounded Zipf(alpha) law over ranks 1..num_keys (float64)."""
+    cdf = torch.arange(1, num_keys + 1, dtype=torch.float64, device=device).pow_(-alpha).cumsum_(0)
+    return cdf.div_(cdf[-1].clone())
+
+
+def zipf_ranks_torch(cdf, n, generator):
+    u = torch.rand(n, dtype=torch.float64, device=cdf.device, generator=generator)
+    return torch.searchsorted(cdf, u).clamp_(max=cdf.numel() - 1)
+
+
+def config3_batches(n_batches, resident, ids_per_step=2_000_000, alpha=1.1, new_frac=0.1, seed=3,
+                    device="cuda"):
+    """BASELINE config 3 lookups: per step `ids_per_step` keys, Zipf(alpha) over the `resident`
+    pre-populated keys (key of rank r = splitmix64(r)), a fraction `new_frac` of the positions
+    replaced by keys never seen before (ranks beyond the resident set, distinct per step)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    cdf = zipf_cdf_torch(resident, alpha, device)
+    n_new = int(ids_per_step * new_frac)
+    out = []
+    for b in range(n_batches):
+        ranks = zipf_ranks_torch(cdf, ids_per_step, g)
+        pos = torch.randperm(ids_per_step, device=device, generator=g)[:n_new]
+        ranks[pos] = resident + b * n_new + torch.arange(n_new, device=device)
+        out.append(splitmix64_torch(ranks))
+    del cdf
+    return out
+
+
+def config5(device="cuda", seed=5, batch=2048, n_fields=4, num_keys=50_000_000, alpha=1.2, mean_len=200,
+            max_len=1000):
+    """Long behaviour sequences (BASELINE config 5): per field `batch` sequences with lognormal
+    lengths (sigma 1, mean `mean_len`, clipped to [1, max_len]) of Zipf(alpha) ids over `num_keys`
+    keys. Returns per-field values / int32 offsets and the per-field padded length (= longest
+    sequence of that field)."""
+    rng = _rng(seed)
+    g = torch.Generator(device=device).manual_seed(seed)
+    cdf = zipf_cdf_torch(num_keys, alpha, device)
+    mu = np.log(mean_len) - 0.5
+    fields = []
+    for f in range(n_fields):
+        lens = np.clip(np.round(rng.lognormal(mu, 1.0, size=batch)), 1, max_len).astype(np.int64)
+        off = np.zeros(batch + 1, np.int64)
+        np.cumsum(lens, out=off[1:])
+        ranks = zipf_ranks_torch(cdf, int(off[-1]), g)
+        fields.append({"values": _lsr(splitmix64_torch(ranks + f * num_keys), 12),  # 52 id bits
+                       "offsets": torch.from_numpy(off.astype(np.int32)).to(device),
+                       "pad_len": int(lens.max()), "num_ids": int(off[-1])})
+    del cdf
+    return {"fields": fields, "batch": batch, "num_ids": sum(f["num_ids"] for f in fields)}
