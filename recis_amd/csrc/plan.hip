@@ -47,40 +47,49 @@ __device__ __forceinline__ uint64_t mix_id(int64_t key) {
   return x;
 }
 
+// One 16-byte slot of the global scratch set: everything a unique id needs sits in one
+// cache line, so the probe, the first-occurrence atomicMin and the count atomicAdd of an id
+// touch HBM once. `cnt` is reused for the unique index once the count has been consumed.
+struct alignas(16) PSlot {
+  int64_t key;
+  int32_t minpos;
+  int32_t cnt;
+};
+
 __global__ void __launch_bounds__(kBlock)
-plan_init_kernel(int64_t* keys, int32_t* minpos, int32_t* cnt, int64_t slots, int64_t* counts) {
+plan_init_kernel(PSlot* tab, int64_t slots, int64_t* counts) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < slots; i += stride) {
-    keys[i] = kSetEmpty;
-    minpos[i] = kNoPos;
-    cnt[i] = 0;
-  }
+  PSlot empty;
+  empty.key = kSetEmpty;
+  empty.minpos = kNoPos;
+  empty.cnt = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < slots; i += stride) tab[i] = empty;
   if (blockIdx.x == 0 && threadIdx.x < 2) counts[threadIdx.x] = 0;
 }
 
-// Global scratch set: slot `mask + 1` is reserved for the id that equals the empty marker.
-__device__ __forceinline__ uint32_t global_slot(int64_t* keys, uint64_t mask, int64_t key) {
-  if (key == kSetEmpty) return static_cast<uint32_t>(mask + 1);
-  uint64_t p = mix_id(key) & mask;
+// Global scratch set of `cap` probed slots (any size: the start slot is the high half of
+// hash * cap); slot `cap` is reserved for the id that equals the empty marker.
+__device__ __forceinline__ uint32_t global_slot(PSlot* tab, uint64_t cap, int64_t key) {
+  if (key == kSetEmpty) return static_cast<uint32_t>(cap);
+  uint64_t p = __umul64hi(mix_id(key), cap);
   for (;;) {
     // plain (L1-cacheable) load: a stale "empty" is corrected by the CAS, a slot never
     // changes once it holds a key
-    int64_t k = keys[p];
+    int64_t k = tab[p].key;
     if (k == kSetEmpty) {
-      k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&keys[p]),
+      k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&tab[p].key),
                                          static_cast<unsigned long long>(kSetEmpty),
                                          static_cast<unsigned long long>(key)));
       if (k == kSetEmpty) break;
     }
     if (k == key) break;
-    p = (p + 1) & mask;  // capacity >= 2n: an empty slot always exists
+    if (++p == cap) p = 0;  // cap >= 2n: an empty slot always exists
   }
   return static_cast<uint32_t>(p);
 }
 
 __global__ void __launch_bounds__(kPlanBlock)
-plan_insert_kernel(int64_t* __restrict__ keys, int32_t* __restrict__ minpos, int32_t* __restrict__ cnt,
-                   uint64_t mask, const int64_t* __restrict__ ids, int64_t n,
+plan_insert_kernel(PSlot* __restrict__ tab, uint64_t cap, const int64_t* __restrict__ ids, int64_t n,
                    int32_t* __restrict__ slotpos, int32_t* __restrict__ rank) {
   __shared__ int64_t l_key[kLdsSlots + 1];
   __shared__ int32_t l_min[kLdsSlots + 1];
@@ -121,9 +130,9 @@ plan_insert_kernel(int64_t* __restrict__ keys, int32_t* __restrict__ minpos, int
   }
   __syncthreads();
   if (live && l_min[e] == tid) {  // the block's first occurrence speaks for all of them
-    const uint32_t p = global_slot(keys, mask, key);
-    atomicMin(&minpos[p], static_cast<int32_t>(i));
-    l_base[e] = atomicAdd(&cnt[p], l_cnt[e]);
+    const uint32_t p = global_slot(tab, cap, key);
+    atomicMin(&tab[p].minpos, static_cast<int32_t>(i));
+    l_base[e] = atomicAdd(&tab[p].cnt, l_cnt[e]);
     l_slot[e] = p;
   }
   __syncthreads();
@@ -153,10 +162,10 @@ __device__ __forceinline__ void block_rank256(bool flag, int& rank, int& total) 
 }
 
 __global__ void __launch_bounds__(kBlock)
-plan_first_count_kernel(const int32_t* __restrict__ minpos, const int32_t* __restrict__ slotpos, int64_t n,
+plan_first_count_kernel(const PSlot* __restrict__ tab, const int32_t* __restrict__ slotpos, int64_t n,
                         int32_t* __restrict__ block_counts) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const bool first = i < n && minpos[slotpos[i]] == static_cast<int32_t>(i);
+  const bool first = i < n && tab[slotpos[i]].minpos == static_cast<int32_t>(i);
   int rank, total;
   block_rank256(first, rank, total);
   if (threadIdx.x == 0) block_counts[blockIdx.x] = total;
@@ -189,20 +198,20 @@ scan_partials_kernel(int32_t* __restrict__ v, int64_t n, int64_t* __restrict__ t
 }
 
 __global__ void __launch_bounds__(kBlock)
-plan_emit_unique_kernel(const int64_t* __restrict__ ids, const int32_t* __restrict__ minpos,
-                        const int32_t* __restrict__ cnt, const int32_t* __restrict__ slotpos, int64_t n,
+plan_emit_unique_kernel(const int64_t* __restrict__ ids, PSlot* __restrict__ tab,
+                        const int32_t* __restrict__ slotpos, int64_t n,
                         const int32_t* __restrict__ block_prefix, int64_t* __restrict__ unique_out,
-                        int32_t* __restrict__ uid, int32_t* __restrict__ row_start) {
+                        int32_t* __restrict__ row_start) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   const int32_t sp = i < n ? slotpos[i] : 0;
-  const bool first = i < n && minpos[sp] == static_cast<int32_t>(i);
+  const bool first = i < n && tab[sp].minpos == static_cast<int32_t>(i);
   int rank, total;
   block_rank256(first, rank, total);
   if (!first) return;
   const int32_t u = block_prefix[blockIdx.x] + rank;
   unique_out[u] = ids[i];
-  uid[sp] = u;
-  row_start[u] = cnt[sp];  // counts for now; scanned in place afterwards
+  row_start[u] = tab[sp].cnt;  // counts for now; scanned in place afterwards
+  tab[sp].cnt = u;             // from here on the field holds the unique index
 }
 
 // Device-wide exclusive scan of row_start[0 .. U) (U read from device memory), three phases
@@ -245,11 +254,11 @@ tile_scan_kernel(int32_t* __restrict__ v, const int64_t* __restrict__ count, con
 
 __global__ void __launch_bounds__(kBlock)
 plan_emit_lists_kernel(const int32_t* __restrict__ slotpos, const int32_t* __restrict__ rank,
-                       const int32_t* __restrict__ uid, const int32_t* __restrict__ row_start, int64_t n,
+                       const PSlot* __restrict__ tab, const int32_t* __restrict__ row_start, int64_t n,
                        int32_t* __restrict__ inverse, int32_t* __restrict__ list, int32_t* __restrict__ pos_out) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   if (i >= n) return;
-  const int32_t u = uid[slotpos[i]];
+  const int32_t u = tab[slotpos[i]].cnt;
   const int32_t pos = row_start[u] + rank[i];
   inverse[i] = u;
   list[pos] = static_cast<int32_t>(i);
@@ -494,39 +503,35 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   RECIS_REQUIRE(hot_cap == 0 || (hot_items_out && hot_cap >= n / kHotLen + n / kHotChunk + 2),
                 "hot_items_out must hold at least n/%d + n/%d + 2 items", kHotLen, kHotChunk);
   RECIS_REQUIRE(n == 0 || (ids && unique_out && inverse_out && list_out), "NULL argument");
-  int64_t cap = 1024;
-  while (cap < 2 * n) cap <<= 1;
+  const int64_t cap = std::max<int64_t>(1024, 2 * n);
   const int64_t slots = cap + 1;
   const int64_t nb = std::max<int64_t>(1, (n + kBlock - 1) / kBlock);
   const int64_t n_tiles = (n + 1 + 1023) / 1024;
-  // workspace: keys[slots] | minpos | cnt | uid [slots each] | slotpos[n] | rank[n] | block_counts[nb] | tiles
-  const size_t bytes = sizeof(int64_t) * slots + sizeof(int32_t) * (3 * slots + 2 * n + nb + n_tiles) + 256;
+  // workspace: tab[slots] | slotpos[n] | rank[n] | block_counts[nb] | tile sums
+  const size_t bytes = sizeof(PSlot) * slots + sizeof(int32_t) * (2 * n + nb + n_tiles) + 256;
   void* ws = nullptr;
   if (int rc = get_workspace(stream, bytes, &ws)) return rc;
-  int64_t* keys = static_cast<int64_t*>(ws);
-  int32_t* minpos = reinterpret_cast<int32_t*>(keys + slots);
-  int32_t* cnt = minpos + slots;
-  int32_t* uid = cnt + slots;
-  int32_t* slotpos = uid + slots;
+  PSlot* tab = static_cast<PSlot*>(ws);
+  int32_t* slotpos = reinterpret_cast<int32_t*>(tab + slots);
   int32_t* rank = slotpos + n;
   int32_t* block_counts = rank + n;
   int32_t* tile_sums = block_counts + nb;
 
   plan_init_kernel<<<dim3(std::min<int64_t>((slots + kBlock - 1) / kBlock, 256 * 16)), dim3(kBlock), 0, stream>>>(
-      keys, minpos, cnt, slots, counts_out_dev);
+      tab, slots, counts_out_dev);
   RECIS_LAUNCH_CHECK();
   if (n > 0) {
     plan_insert_kernel<<<dim3((n + kPlanBlock - 1) / kPlanBlock), dim3(kPlanBlock), 0, stream>>>(
-        keys, minpos, cnt, static_cast<uint64_t>(cap - 1), ids, n, slotpos, rank);
+        tab, static_cast<uint64_t>(cap), ids, n, slotpos, rank);
     RECIS_LAUNCH_CHECK();
-    plan_first_count_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(minpos, slotpos, n, block_counts);
+    plan_first_count_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(tab, slotpos, n, block_counts);
     RECIS_LAUNCH_CHECK();
   }
   scan_partials_kernel<<<1, 1024, 0, stream>>>(block_counts, n > 0 ? nb : 0, counts_out_dev);
   RECIS_LAUNCH_CHECK();
   if (n > 0) {
-    plan_emit_unique_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(ids, minpos, cnt, slotpos, n, block_counts,
-                                                                   unique_out, uid, row_start_out);
+    plan_emit_unique_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(ids, tab, slotpos, n, block_counts, unique_out,
+                                                                   row_start_out);
     RECIS_LAUNCH_CHECK();
   }
   tile_sum_kernel<<<dim3(n_tiles), dim3(1024), 0, stream>>>(row_start_out, counts_out_dev, tile_sums);
@@ -537,7 +542,7 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
                                                             static_cast<int32_t>(n));
   RECIS_LAUNCH_CHECK();
   if (n > 0) {
-    plan_emit_lists_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(slotpos, rank, uid, row_start_out, n,
+    plan_emit_lists_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(slotpos, rank, tab, row_start_out, n,
                                                                   inverse_out, list_out, pos_out);
     RECIS_LAUNCH_CHECK();
     if (hot_cap > 0) {
