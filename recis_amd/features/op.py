@@ -1,0 +1,141 @@
+"""Feature-engine ops on the hot path: the mirror of ``recis.features.op`` for
+``SelectField``, ``Mod``, ``Bucketize``, ``Hash`` and ``IDMultiHash``
+(recis/features/op.py:129-686). ``SequenceTruncate`` and ``FeatureCross`` belong to
+the ops that feed this path and are not part of this build.
+
+Every op works on a ``RaggedTensor`` (its values) or a plain tensor; the engine
+batches same-typed ops of one step into a single fused HIP launch.
+"""
+import hashlib
+import json
+from typing import Dict, List, Union
+
+import torch
+from torch import nn
+
+from .. import ops
+from ..ragged.tensor import RaggedTensor
+
+
+def _values(x):
+    return x.values() if isinstance(x, RaggedTensor) else x
+
+
+def _with_values(x, values):
+    if isinstance(x, RaggedTensor):
+        return RaggedTensor(values, x.offsets(), x.weight(), x.dense_shape)
+    return values
+
+
+class _OP(nn.Module):
+    def get_hash(self) -> int:
+        text = json.dumps({"type": type(self).__name__, "config": self._get_config()}, sort_keys=True)
+        return int(hashlib.sha256(text.encode()).hexdigest()[:16], 16)
+
+    def _get_config(self) -> Dict:
+        raise NotImplementedError
+
+
+class SelectField(_OP):
+    def __init__(self, name: str, dtype=torch.long, dim=None, from_dict=True):
+        super().__init__()
+        self._name, self._dtype, self._dim, self._from_dict = name, dtype, dim, from_dict
+
+    def forward(self, data):
+        if self._from_dict:
+            assert isinstance(data, dict), "data must be a dict, fn:%s" % self._name
+            return data[self._name]
+        return data
+
+    def _get_config(self):
+        return {"name": self._name, "dtype": str(self._dtype), "dim": self._dim, "from_dict": self._from_dict}
+
+
+class Mod(_OP):
+    """``(int64)((uint64) x % mod)``."""
+
+    def __init__(self, mod_value):
+        super().__init__()
+        self.mod_value = int(mod_value)
+
+    def forward(self, x: Union[RaggedTensor, torch.Tensor]):
+        return _with_values(x, ops.uint64_mod(_values(x).cuda(), self.mod_value))
+
+    def _get_config(self):
+        return {"mod": self.mod_value}
+
+
+class Bucketize(_OP):
+    """Number of boundaries <= value (int64)."""
+
+    def __init__(self, boundary):
+        super().__init__()
+        b = torch.tensor(boundary, dtype=torch.float) if isinstance(boundary, list) else boundary.float()
+        self.register_buffer("boundary", b)
+
+    def forward(self, x):
+        return _with_values(x, ops.bucketize_op(_values(x).cuda().float(), self.boundary.cuda()))
+
+    def _get_config(self):
+        return {"boundary": self.boundary.tolist()}
+
+
+class Hash(_OP):
+    """64-bit hash ("farm" | "murmur") of the byte strings of a two-level ragged tensor: the
+    innermost offsets delimit the strings, the hashed values replace them (one per string)."""
+
+    def __init__(self, hash_type: str):
+        super().__init__()
+        assert hash_type in ("farm", "murmur"), "hash_type must be farm or murmur"
+        self.hash_type = hash_type
+
+    def forward(self, x: RaggedTensor):
+        assert isinstance(x, RaggedTensor), "Hash takes a RaggedTensor of bytes"
+        values = x.values().cuda()
+        out = ops.fused_hash([values], [x.offsets()[-1].cuda()], self.hash_type)[0]
+        rest = [o.cuda() for o in x.offsets()[:-1]]
+        if not rest:
+            rest = [torch.arange(out.numel() + 1, device=out.device)]
+        return RaggedTensor(out, rest, None)
+
+    def _get_config(self):
+        return {"hash_type": self.hash_type}
+
+
+def _largest_prime_le(n):
+    def is_prime(k):
+        if k < 2:
+            return False
+        d = 2
+        while d * d <= k:
+            if k % d == 0:
+                return False
+            d += 1
+        return True
+    while not is_prime(n):
+        n -= 1
+    return n
+
+
+class IDMultiHash(_OP):
+    """``multi_hash_j = (((x * mul_j) % p_j + p_j) % p_j) % bucket_j`` with mul = [1, 3, 5, 7] and
+    p_j the largest prime <= [29, 47, 67, 83][j] * bucket_j (recis/features/op.py:520-577)."""
+
+    _MULS = [1, 3, 5, 7]
+    _MODS = [29, 47, 67, 83]
+
+    def __init__(self, num_buckets: List[int], prefix: str = "multi_hash"):
+        super().__init__()
+        assert 1 <= len(num_buckets) <= 4, "IDMultiHash supports 1 to 4 hashes"
+        self.num_buckets = [int(b) for b in num_buckets]
+        self.prefix = prefix
+        n = len(self.num_buckets)
+        self.muls = self._MULS[:n]
+        self.primes = [_largest_prime_le(m * b) for m, b in zip(self._MODS[:n], self.num_buckets)]
+
+    def forward(self, x):
+        outs = ops.fused_multi_hash([_values(x).cuda()], [self.muls], [self.primes], [self.num_buckets])
+        return {"%s_%d" % (self.prefix, j): _with_values(x, o) for j, o in enumerate(outs)}
+
+    def _get_config(self):
+        return {"num_buckets": self.num_buckets, "prefix": self.prefix}

@@ -348,3 +348,41 @@ def test_dynamic_embedding_tile_and_max():
     rows2 = emb2.hashtable(torch.tensor([5, 6, 7, 8, 9], device="cuda")).detach()
     torch.testing.assert_close(out2[0].detach(), rows2[:4].max(0)[0])
     torch.testing.assert_close(out2[2].detach(), rows2[[4, 0]].max(0)[0])
+
+
+def test_feature_engine_ops_and_fusion():
+    """Restated from tests/feature_engine/op_test.py:17-36,95-131 and feature_engine_test.py: Mod,
+    Bucketize, IDMultiHash, Hash known answers, through the fused engine path."""
+    from recis_amd.features import Bucketize, Feature, FeatureEngine, Hash, IDMultiHash, Mod, SelectField
+
+    vals = torch.randn(10) * 5
+    feats = [
+        Feature("a").add_op(SelectField("a")).add_op(Mod(1000)),
+        Feature("b").add_op(SelectField("b")).add_op(Mod(7)),
+        Feature("c").add_op(SelectField("c")).add_op(Bucketize([1.0, 2, 3, 4, 5])),
+        Feature("d").add_op(SelectField("c")).add_op(Bucketize([0.0])),
+        Feature("a_dup").add_op(SelectField("a")).add_op(Mod(1000)),
+        Feature("h").add_op(SelectField("h")).add_op(Hash("farm")).add_op(Mod(1 << 62)),
+        Feature("m").add_op(SelectField("h")).add_op(Hash("murmur")),
+        Feature("mh").add_op(SelectField("a")).add_op(IDMultiHash([1000] * 4)),
+    ]
+    engine = FeatureEngine(feats)
+    data = {
+        "a": RaggedTensor(torch.tensor([1001, 1002, 1003]).cuda(), torch.tensor([0, 1, 2, 3]).cuda()),
+        "b": torch.tensor([-1, 15], device="cuda"),
+        "c": RaggedTensor(vals.cuda(), torch.arange(0, 11).cuda()),
+        "h": RaggedTensor(torch.tensor([0, 1, 2, 1, 2, 3], dtype=torch.int8).cuda(),
+                          [torch.tensor([0, 1, 2]).cuda(), torch.tensor([0, 3, 6]).cuda()]),
+    }
+    out = engine(data)
+    assert out["a"].values().tolist() == [1, 2, 3] and out["a_dup"].values().tolist() == [1, 2, 3]
+    assert out["b"].tolist() == [(2 ** 64 - 1) % 7, 1]
+    assert torch.equal(out["c"].values().cpu(), torch.bucketize(vals, torch.tensor([1.0, 2, 3, 4, 5]), right=True))
+    assert torch.equal(out["d"].values().cpu(), (vals >= 0).long())
+    farm = [-7736835464683084646, -5546720800891377920]
+    assert out["h"].values().tolist() == [(f + 2 ** 64) % (1 << 62) for f in farm]
+    assert out["m"].values().tolist() == [-4003751876240412087, -1042754718167355375]
+    assert out["m"].offsets()[-1].tolist() == [0, 1, 2]
+    exp = [[1, 2, 3], [3, 6, 9], [5, 10, 15], [7, 14, 21]]
+    for j in range(4):
+        assert out["multi_hash_%d" % j].values().tolist() == exp[j]
