@@ -32,6 +32,29 @@ import workloads  # noqa: E402
 HBM_PEAK_GBS = 8000.0
 
 
+def _kernel_profile(fn, iters):
+    """Per-kernel mean launch time in microseconds over `iters` calls of fn(), measured by the
+    library's own HIP events around each kernel launch (on the launch stream)."""
+    import ctypes
+
+    from recis_amd import _lib
+    lib = _lib.lib()
+    fn()
+    torch.cuda.synchronize()
+    buf = ctypes.create_string_buffer(1 << 16)
+    _lib.check(lib.recis_hip_profile_enable(1))
+    _lib.check(lib.recis_hip_profile_report(buf, ctypes.c_int64(len(buf))))  # drop warm-up records
+    for _ in range(iters):
+        fn()
+    _lib.check(lib.recis_hip_profile_report(buf, ctypes.c_int64(len(buf))))
+    _lib.check(lib.recis_hip_profile_enable(0))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, calls, total_ms = line.split()
+        out[name] = {"calls_per_step": int(calls) / iters, "us": float(total_ms) * 1e3 / int(calls)}
+    return out
+
+
 def _event_ms(fn, iters):
     """Mean time of fn() over `iters` launches, HIP events on the current stream."""
     fn()
@@ -181,6 +204,23 @@ class Config4:
             "pool_fwd": U * D * 4 + N * 4 + (S + 1) * 4 + S * D * 4,
             "pool_bwd": S * D * 4 + N * 4 + (S + 1) * 4 + U * D * 4,
             "adam": U * 8 + U * D * 4 * (1 + 6),
+        }
+
+    def kernel_bytes(self):
+        """Algorithmic (compulsory) HBM bytes of one launch of each heavy kernel of the step."""
+        N, U, S, D = self.N, self.U, self.N, self.D
+        return {
+            "plan_insert_kernel": 8 * N + 8 * N + 32 * U,           # ids in; slot + rank out; one 16-B set slot RMW
+            "plan_first_count_kernel": 4 * N + 16 * U,
+            "plan_emit_unique_kernel": 8 * N + 4 * N + 16 * U + 12 * U,
+            "plan_emit_lists_kernel": 8 * N + 16 * U + 12 * N,
+            "plan_init_kernel": 32 * N,                              # 2N set slots of 16 B
+            "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,          # ids, one table slot, index + slot pos
+            "block_gather_kernel": 8 * U + 2 * U * D * 4,
+            "seg_pool_fwd_kernel": U * D * 4 + 4 * N + 4 * (S + 1) + S * D * 4,
+            "csr_cold_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,
+            "csr_hot_kernel": 0,
+            "adamw_rows_kernel": U * (8 + D * 4 * 7),
         }
 
     def stage_times(self, iters):
@@ -473,11 +513,16 @@ def main():
         stages = main_wl.stage_times(max(5, args.steps))
         ab = main_wl.algorithmic_bytes()
         total_bytes = sum(ab.values())
-        dom = max(stages, key=stages.get)
+        kern = _kernel_profile(main_wl.step, max(5, args.steps))
+        kb = main_wl.kernel_bytes()
+        dom = max(kern, key=lambda k: kern[k]["us"] * kern[k]["calls_per_step"])
         out["config"]["unique_ids_per_step"] = main_wl.U
-        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": ab[dom] / stages[dom] / 1e6,
-                           "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": ab[dom] / stages[dom] / 1e6 / HBM_PEAK_GBS, "traffic": None}
+        ach = kb.get(dom, 0) / kern[dom]["us"] / 1e3
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": ach / HBM_PEAK_GBS, "traffic": None, "launch_us": round(kern[dom]["us"], 2),
+                           "algorithmic_bytes_per_launch": kb.get(dom, 0)}
+        out["kernels_us"] = {k: round(v["us"], 2) for k, v in sorted(kern.items(), key=lambda kv: -kv[1]["us"])}
+        out["kernels_gbs"] = {k: round(kb[k] / kern[k]["us"] / 1e3, 1) for k in kern if kb.get(k)}
         out["step_roofline"] = {"algorithmic_bytes": total_bytes, "achieved": total_bytes / ms_per_step / 1e6,
                                 "frac": total_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, "unit": "GB/s"}
         out["stages_ms"] = {k: round(v, 4) for k, v in stages.items()}

@@ -53,6 +53,15 @@ extern "C" {
 const char* recis_hip_last_error(void);
 int recis_hip_abi_version(void);
 
+/*
+ * Optional per-kernel timing for benchmarks (off by default). When on, the heavy kernels
+ * of every entry point are bracketed by HIP events on their launch stream;
+ * recis_hip_profile_report synchronises the device, writes one line
+ * "kernel_name calls total_ms" per kernel into buf and resets the record.
+ */
+int recis_hip_profile_enable(int on);
+int recis_hip_profile_report(char* buf, int64_t cap);
+
 /* Synchronises the current device, returns the soft-error bits raised by
  * kernels since the last poll in *bits and clears them. */
 int recis_hip_poll_device_errors(int* bits);

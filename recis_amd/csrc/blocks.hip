@@ -195,6 +195,7 @@ int recis_gather(const void* ids, int ids_is64, const void* emb, int64_t rows, v
   const int64_t grid = (n + rows_per_block - 1) / rows_per_block;
   return dispatch_vb(vb, [&](auto tag) {
     constexpr int VB = decltype(tag)::value;
+    RECIS_TIME_KERNEL("gather_kernel", stream)
     gather_kernel<VB><<<dim3(grid), dim3(kBlock), 0, stream>>>(
         ids, ids_is64, static_cast<const char*>(emb), rows, static_cast<char*>(out), n,
         static_cast<int>(row_bytes), lpr_log2, err);
@@ -216,6 +217,7 @@ int recis_block_gather(const int64_t* ids, void* const* blocks_dev, int64_t n_bl
   const int64_t grid = (n + rows_per_block - 1) / rows_per_block;
   return dispatch_vb(vb, [&](auto tag) {
     constexpr int VB = decltype(tag)::value;
+    RECIS_TIME_KERNEL("block_gather_kernel", stream)
     block_gather_kernel<VB><<<dim3(grid), dim3(kBlock), 0, stream>>>(a, default_key, readonly,
                                                                     static_cast<char*>(out));
     RECIS_LAUNCH_CHECK();

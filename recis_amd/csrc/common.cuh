@@ -198,6 +198,35 @@ inline int dtype_size(int dtype) {
   }
 }
 
+// Optional per-kernel timing (off by default): when enabled through
+// recis_hip_profile_enable(1), a KernelTimer brackets a launch with two HIP
+// events on the launch stream; recis_hip_profile_report() sums them per kernel name.
+extern bool g_profile_on;
+struct KernelTimer {
+  KernelTimer(const char* name, hipStream_t stream) : active_(g_profile_on) {
+    if (active_) begin(name, stream);
+  }
+  ~KernelTimer() {
+    if (active_) end();
+  }
+  // makes `for (KernelTimer t(...); t.once();) launch;` run the launch exactly once
+  bool once() {
+    const bool first = !done_;
+    done_ = true;
+    return first;
+  }
+
+ private:
+  void begin(const char* name, hipStream_t stream);
+  void end();
+  bool active_;
+  bool done_ = false;
+  int slot_ = -1;
+  hipStream_t stream_ = nullptr;
+};
+// usage: RECIS_TIME_KERNEL("name", stream) kernel<<<grid, block, 0, stream>>>(...);
+#define RECIS_TIME_KERNEL(name, stream) for (::recis_hip::KernelTimer _recis_kt(name, stream); _recis_kt.once();)
+
 // Per-(device, stream) scratch that grows on demand and is reused by later
 // calls on that stream. Never shrinks; released at process exit.
 int get_workspace(hipStream_t stream, size_t bytes, void** out);

@@ -555,6 +555,7 @@ int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* i
   const uint64_t mask = static_cast<uint64_t>(m->capacity - 1);
 
   reset_dups_kernel<<<1, 1, 0, stream>>>(m->state);
+  RECIS_TIME_KERNEL("find_or_claim_kernel", stream)
   find_or_claim_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, mask, ids, n, index_out, slotpos,
                                                              block_counts, m->state, m->err);
   RECIS_LAUNCH_CHECK();

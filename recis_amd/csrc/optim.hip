@@ -227,6 +227,7 @@ int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dty
       if constexpr (VEC * sizeof(T) > 16 || VEC * sizeof(TG) > 16) {
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
+        RECIS_TIME_KERNEL("adamw_rows_kernel", stream)
         adamw_rows_kernel<T, TG, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
             a, static_cast<const TG*>(grad), reinterpret_cast<T* const*>(emb_blocks_dev),
             reinterpret_cast<T* const*>(exp_avg_blocks_dev), reinterpret_cast<T* const*>(exp_avg_sq_blocks_dev),
@@ -258,6 +259,7 @@ int recis_block_apply_adagrad(const int64_t* index, const void* grad, int grad_d
       if constexpr (VEC * sizeof(T) > 16 || VEC * sizeof(TG) > 16) {
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
+        RECIS_TIME_KERNEL("adagrad_rows_kernel", stream)
         adagrad_rows_kernel<T, TG, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
             a, static_cast<const TG*>(grad), reinterpret_cast<T* const*>(emb_blocks_dev),
             reinterpret_cast<T* const*>(accum_blocks_dev), static_cast<float>(lr), static_cast<float>(eps));

@@ -517,19 +517,24 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   int32_t* block_counts = rank + n;
   int32_t* tile_sums = block_counts + nb;
 
+  RECIS_TIME_KERNEL("plan_init_kernel", stream)
+
   plan_init_kernel<<<dim3(std::min<int64_t>((slots + kBlock - 1) / kBlock, 256 * 16)), dim3(kBlock), 0, stream>>>(
       tab, slots, counts_out_dev);
   RECIS_LAUNCH_CHECK();
   if (n > 0) {
+    RECIS_TIME_KERNEL("plan_insert_kernel", stream)
     plan_insert_kernel<<<dim3((n + kPlanBlock - 1) / kPlanBlock), dim3(kPlanBlock), 0, stream>>>(
         tab, static_cast<uint64_t>(cap), ids, n, slotpos, rank);
     RECIS_LAUNCH_CHECK();
+    RECIS_TIME_KERNEL("plan_first_count_kernel", stream)
     plan_first_count_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(tab, slotpos, n, block_counts);
     RECIS_LAUNCH_CHECK();
   }
   scan_partials_kernel<<<1, 1024, 0, stream>>>(block_counts, n > 0 ? nb : 0, counts_out_dev);
   RECIS_LAUNCH_CHECK();
   if (n > 0) {
+    RECIS_TIME_KERNEL("plan_emit_unique_kernel", stream)
     plan_emit_unique_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(ids, tab, slotpos, n, block_counts, unique_out,
                                                                    row_start_out);
     RECIS_LAUNCH_CHECK();
@@ -542,6 +547,7 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
                                                             static_cast<int32_t>(n));
   RECIS_LAUNCH_CHECK();
   if (n > 0) {
+    RECIS_TIME_KERNEL("plan_emit_lists_kernel", stream)
     plan_emit_lists_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(slotpos, rank, tab, row_start_out, n,
                                                                   inverse_out, list_out, pos_out);
     RECIS_LAUNCH_CHECK();
@@ -634,6 +640,7 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
       if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 16) {
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
+        RECIS_TIME_KERNEL("csr_cold_kernel", stream)
         csr_cold_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
             static_cast<const TIn*>(rows), static_cast<TOut*>(out), a);
         RECIS_LAUNCH_CHECK();
@@ -641,6 +648,7 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
           if (hot_cap > 0) {
             const int64_t hot_grid = std::min<int64_t>(hot_cap, 2048);
             const size_t lds = sizeof(float) * (kPlanBlock / kWave) * static_cast<size_t>(D);
+            RECIS_TIME_KERNEL("csr_hot_kernel", stream)
             csr_hot_kernel<TIn, VEC><<<dim3(hot_grid), dim3(kPlanBlock), lds, stream>>>(
                 static_cast<const TIn*>(rows), static_cast<float*>(out), a, hot_items, counts_dev, hot_cap);
             RECIS_LAUNCH_CHECK();

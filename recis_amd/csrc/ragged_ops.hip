@@ -217,6 +217,7 @@ int recis_ragged_tile(const int64_t* batch, const int64_t* seq, int64_t n_featur
       int rc = dispatch_t_vec(dtype, vec, [&](auto t, auto vtag) {
         using T = decltype(t);
         constexpr int VEC = decltype(vtag)::value;
+        RECIS_TIME_KERNEL("tile_fwd_kernel", stream)
         tile_fwd_kernel<T, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
             value, value_is64, off_f, off_is64, static_cast<const T*>(table), table_rows,
             static_cast<T*>(out) + rbase * D, batch[f], seq[f], n_values, static_cast<int>(D), lpr_log2, err);

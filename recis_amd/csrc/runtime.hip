@@ -5,7 +5,9 @@
 
 #include <map>
 #include <mutex>
+#include <string>
 #include <utility>
+#include <vector>
 
 #include "common.cuh"
 
@@ -76,9 +78,69 @@ int get_workspace(hipStream_t stream, size_t bytes, void** out) {
   return RECIS_OK;
 }
 
+bool g_profile_on = false;
+
+struct TimedLaunch {
+  const char* name;
+  hipEvent_t start, stop;
+};
+static std::vector<TimedLaunch> g_timed;
+
+void KernelTimer::begin(const char* name, hipStream_t stream) {
+  std::lock_guard<std::mutex> l(g_mu);
+  TimedLaunch t;
+  t.name = name;
+  if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) {
+    active_ = false;
+    return;
+  }
+  (void)hipEventRecord(t.start, stream);
+  g_timed.push_back(t);
+  slot_ = static_cast<int>(g_timed.size()) - 1;
+  stream_ = stream;
+}
+
+void KernelTimer::end() {
+  std::lock_guard<std::mutex> l(g_mu);
+  if (slot_ >= 0 && slot_ < static_cast<int>(g_timed.size())) (void)hipEventRecord(g_timed[slot_].stop, stream_);
+}
+
 }  // namespace recis_hip
 
 extern "C" {
+
+int recis_hip_profile_enable(int on) {
+  std::lock_guard<std::mutex> l(recis_hip::g_mu);
+  recis_hip::g_profile_on = on != 0;
+  return RECIS_OK;
+}
+
+int recis_hip_profile_report(char* buf, int64_t cap) {
+  using namespace recis_hip;
+  RECIS_REQUIRE(buf != nullptr && cap > 0, "buf must hold the report");
+  RECIS_CHECK_HIP(hipDeviceSynchronize());
+  std::lock_guard<std::mutex> l(g_mu);
+  std::map<std::string, std::pair<int64_t, double>> agg;
+  for (auto& t : g_timed) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, t.start, t.stop) == hipSuccess) {
+      auto& a = agg[t.name];
+      a.first += 1;
+      a.second += ms;
+    }
+    (void)hipEventDestroy(t.start);
+    (void)hipEventDestroy(t.stop);
+  }
+  g_timed.clear();
+  std::string out;
+  char line[256];
+  for (auto& kv : agg) {
+    snprintf(line, sizeof(line), "%s %lld %.6f\n", kv.first.c_str(), (long long)kv.second.first, kv.second.second);
+    out += line;
+  }
+  snprintf(buf, static_cast<size_t>(cap), "%s", out.c_str());
+  return RECIS_OK;
+}
 
 const char* recis_hip_last_error(void) { return recis_hip::g_err; }
 

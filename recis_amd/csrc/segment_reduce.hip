@@ -515,9 +515,11 @@ extern "C" int recis_segment_reduce_forward(
           const int teams_per_block = kBlock >> a.team_log2;
           const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
           if (mode == RECIS_MAX) {
+            RECIS_TIME_KERNEL("seg_max_fwd_kernel", stream)
             seg_max_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
                 static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), argmax_out, a);
           } else {
+            RECIS_TIME_KERNEL("seg_pool_fwd_kernel", stream)
             seg_pool_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
                 static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), a);
           }
@@ -631,9 +633,11 @@ extern "C" int recis_segment_reduce_backward(
           const int teams_per_block = kBlock >> a.team_log2;
           const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
           if (unique)
+            RECIS_TIME_KERNEL("seg_pool_bwd_kernel", stream)
             seg_pool_bwd_kernel<TG, TOut, VEC, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(
                 static_cast<const TG*>(grad_out), static_cast<TOut*>(grad_unique), a);
           else
+            RECIS_TIME_KERNEL("seg_pool_bwd_kernel", stream)
             seg_pool_bwd_kernel<TG, TOut, VEC, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(
                 static_cast<const TG*>(grad_out), static_cast<TOut*>(grad_unique), a);
           RECIS_LAUNCH_CHECK();
