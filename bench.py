@@ -453,6 +453,9 @@ def main():
     ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch a plain elementwise kernel that reads 1 GiB and writes 1 GiB "
+                         "(scale for hardware-counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU that owns the whole table; --gpus %d is not supported "
@@ -507,6 +510,14 @@ def main():
         return {"ms_per_step": round(ms, 4), "ids_per_s": wl.ids_per_step / ms * 1e3,
                 "unique_ids_per_step": wl.U, "algorithmic_bytes": nbytes,
                 "gbs": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    if args.calib_copy:
+        src = torch.zeros(1 << 28, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     extras = {}
     if args.workload == "c4":
