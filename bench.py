@@ -445,6 +445,18 @@ class Config5:
         return n * reps / dt, "first %d of 2048 sequences per field (%d ids/step) of config 5, fp32 rows" % (b, n)
 
 
+# HBM bytes per launch in the config-4 step, from hardware-counter runs of this file
+# (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE, with --calib-copy): each counter is
+# scaled by what it reads for the calibration kernel that moves 1 GiB each way
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
+MEASURED_TRAFFIC_C4 = {
+    "plan_insert_kernel": 380658672, "adamw_rows_kernel": 400841547, "seg_pool_fwd_kernel": 277264266,
+    "plan_emit_unique_kernel": 272778425, "plan_emit_lists_kernel": 234571357, "csr_cold_kernel": 200464118,
+    "find_or_claim_kernel": 188212736, "plan_first_count_kernel": 157875229, "csr_hot_kernel": 139709319,
+    "block_gather_kernel": 119564740, "plan_init_kernel": 81795174,
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -530,7 +542,8 @@ def main():
         out["config"]["unique_ids_per_step"] = main_wl.U
         ach = kb.get(dom, 0) / kern[dom]["us"] / 1e3
         out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": ach / HBM_PEAK_GBS, "traffic": None, "launch_us": round(kern[dom]["us"], 2),
+                           "frac": ach / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_C4.get(dom),
+                           "launch_us": round(kern[dom]["us"], 2),
                            "algorithmic_bytes_per_launch": kb.get(dom, 0)}
         out["kernels_us"] = {k: round(v["us"], 2) for k, v in sorted(kern.items(), key=lambda kv: -kv[1]["us"])}
         out["kernels_gbs"] = {k: round(kb[k] / kern[k]["us"] / 1e3, 1) for k in kern if kb.get(k)}
