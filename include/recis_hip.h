@@ -49,6 +49,7 @@ extern "C" {
 #define RECIS_DEVERR_INDEX_RANGE 1  /* an index fell outside [0, rows)        */
 #define RECIS_DEVERR_OFFSETS 2      /* offsets not monotone / outside [0, B]  */
 #define RECIS_DEVERR_TABLE_FULL 4   /* id-map probe sequence found no slot    */
+#define RECIS_DEVERR_PLAN_OVERFLOW 8 /* batch plan: too many distinct ids fell into one hash bucket */
 
 const char* recis_hip_last_error(void);
 int recis_hip_abi_version(void);
@@ -323,9 +324,9 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
                  int inverse_is64, int64_t* count_out_dev, void* stream);
 
 /*
- * Batch plan: dedup plus the transposed index. On top of what recis_unique returns
- * (unique ids in order of first occurrence, int32 inverse, count), the occurrences are
- * grouped by unique id:
+ * Batch plan: dedup plus the transposed index. Unique ids (no duplicates, every id of the
+ * batch present), an int32 inverse with unique_out[inverse[i]] == ids[i], the count, and the
+ * occurrences grouped by unique id:
  *   row_start_out [n + 1]  list of unique id u = list[row_start[u] .. row_start[u+1]);
  *                          entries U .. n hold n
  *   list_out      [n]      occurrence indices grouped by unique id
@@ -333,7 +334,11 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
  *   hot_items_out [2*hot_cap] (row, chunk) work items for ids with more than 256
  *                          occurrences; hot_cap >= n/256 + n/8192 + 2, or 0 to skip
  *   counts_out_dev [2]     device words: number of unique ids, number of hot items
- * With it, a gradient scatter over duplicated ids (the atomic loops of
+ * The unique ids are ordered by (hash bucket, first occurrence): the order, the inverse and
+ * row_start depend on the input only; the order of the entries inside one id's list and of
+ * the hot items is not specified. No global atomics are used: ids are partitioned by hash
+ * and deduplicated in LDS.
+ * With the plan, a gradient scatter over duplicated ids (the atomic loops of
  * csrc/ops/embedding_segment_reduce_kernel.cu:79-120, segment_ops_kernel.cu:133-165,
  * ragged_tile_kernel.cu:46-60 and the unique + index_add_ of
  * recis/nn/modules/hashtable.py:555-586) becomes a gather-reduce per unique row.

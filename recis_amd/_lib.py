@@ -22,6 +22,7 @@ FLAG_REV_UNIQUE = 1
 DEVERR_INDEX_RANGE = 1
 DEVERR_OFFSETS = 2
 DEVERR_TABLE_FULL = 4
+DEVERR_PLAN_OVERFLOW = 8
 
 _DTYPES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 MODES = {"sum": SUM, "mean": MEAN, "tile": TILE, "max": MAX}

@@ -3,23 +3,27 @@
 //
 // The reference scatters gradients back to unique rows with one global atomic per
 // element (csrc/ops/embedding_segment_reduce_kernel.cu:79-120, segment_ops_kernel.cu:133-165)
-// and dedups with a radix sort (csrc/ops/ids_partition_kernel.cu:86-131). On MI355X fp32
-// atomics run at a few percent of HBM speed and ids of low-cardinality features repeat
-// tens of thousands of times per batch, so this build never scatters rows: the plan below
-// groups the occurrences by unique id once per batch, after which the gradient of a
-// unique row is a gather-reduce over its own list, written once.
+// and dedups with a radix sort (csrc/ops/ids_partition_kernel.cu:86-131). On MI355X
+// device-scope atomics run at some 3e10 per second whatever they touch (a few percent of
+// HBM speed) and ids of low-cardinality features repeat tens of thousands of times per
+// batch, so this build never scatters rows and never builds the plan with global atomics:
+// ids are partitioned by hash into buckets small enough to be deduplicated in LDS.
 //
-//   insert   one workgroup dedups its 1024 ids in an LDS hash first (LDS atomics), so an id
-//            repeated k times in the block costs ONE probe of the global scratch set, one
-//            atomicMin (first occurrence) and one atomicAdd (occurrence count, whose return
-//            value hands every occurrence its rank inside the id's list)
-//   unique   first occurrences are ranked in input order by a scan: unique ids come out in
-//            order of first occurrence (deterministic)
-//   lists    exclusive scan of the per-unique counts -> row_start; occurrence i goes to
-//            list[row_start[u] + rank_i]
-//   hot      unique ids with more than kHotLen occurrences are listed as (row, chunk) work
-//            items for a workgroup-per-chunk reduction; everything else is one small team
-//            of lanes per row
+//   tile     a workgroup dedups tiles of 1024 ids in an LDS hash: an id repeated k times in
+//            a tile becomes ONE record {id, first position, k}; records per bucket are
+//            counted in an LDS histogram (one row per workgroup)
+//   colscan  exclusive scan of every histogram column -> where each workgroup's records of
+//            each bucket go; bucket sizes
+//   scatter  records move to their bucket (bucket = top bits of the mixed id)
+//   bucket   one workgroup per bucket: LDS hash over the bucket's records gives every unique
+//            id its first position and its count; unique ids are ranked by first position
+//            inside the bucket, counts are scanned into list offsets
+//   scan     bucket totals -> first unique index and first list entry of every bucket
+//   emit     per occurrence: unique index (inverse), list position; per unique id: id,
+//            row_start, hot work items
+//
+// Unique ids come out ordered by (bucket, first occurrence): a function of the input only.
+// The order of the occurrences inside one id's list is not specified.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -30,8 +34,13 @@
 namespace recis_hip {
 namespace {
 
-constexpr int kPlanBlock = 1024;
-constexpr int kLdsSlots = 2048;  // LDS hash entries per workgroup (load <= 1/2)
+constexpr int kPlanBlock = 1024;  // ids per tile == threads of the tile / scatter / hot kernels
+constexpr int kLdsSlots = 2048;   // LDS hash entries of a tile (load <= 1/2)
+constexpr int kBucketBlock = 256;
+constexpr int kBucketSlots = 1024;  // LDS hash entries of a bucket round
+constexpr int kMaxBuckets = 8192;
+constexpr int kMinBuckets = 32;
+constexpr int kMaxRows = 512;  // histogram rows (= workgroups of the tile and scatter kernels)
 constexpr int64_t kSetEmpty = -1;
 constexpr int32_t kNoPos = 0x7fffffff;
 constexpr int kHotLen = 256;      // rows with more occurrences than this are "hot"
@@ -47,103 +56,34 @@ __device__ __forceinline__ uint64_t mix_id(int64_t key) {
   return x;
 }
 
-// One 16-byte slot of the global scratch set: everything a unique id needs sits in one
-// cache line, so the probe, the first-occurrence atomicMin and the count atomicAdd of an id
-// touch HBM once. `cnt` is reused for the unique index once the count has been consumed.
-struct alignas(16) PSlot {
+// One deduplicated run of a tile: `word` = (count - 1) << 10 | index of the record in its tile.
+struct alignas(16) Rec {
   int64_t key;
-  int32_t minpos;
+  int32_t pos;  // first position of the id in its tile (absolute)
+  uint32_t word;
+};
+
+// A unique id of a bucket, in bucket-local terms.
+struct alignas(16) URec {
+  int64_t key;
+  int32_t list_off;  // first list entry, relative to the bucket's first
   int32_t cnt;
 };
 
-__global__ void __launch_bounds__(kBlock)
-plan_init_kernel(PSlot* tab, int64_t slots, int64_t* counts) {
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
-  PSlot empty;
-  empty.key = kSetEmpty;
-  empty.minpos = kNoPos;
-  empty.cnt = 0;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < slots; i += stride) tab[i] = empty;
-  if (blockIdx.x == 0 && threadIdx.x < 2) counts[threadIdx.x] = 0;
+struct PlanGeom {
+  int64_t n;
+  int tiles;         // ceil(n / 1024)
+  int tiles_per_wg;  // tiles a workgroup of the tile / scatter kernels walks
+  int rows;          // workgroups of those kernels == histogram rows
+  int nb_log2;       // buckets = 1 << nb_log2
+};
+
+__device__ __forceinline__ int bucket_of(int64_t key, int nb_log2) {
+  return static_cast<int>(mix_id(key) >> (64 - nb_log2));
 }
 
-// Global scratch set of `cap` probed slots (any size: the start slot is the high half of
-// hash * cap); slot `cap` is reserved for the id that equals the empty marker.
-__device__ __forceinline__ uint32_t global_slot(PSlot* tab, uint64_t cap, int64_t key) {
-  if (key == kSetEmpty) return static_cast<uint32_t>(cap);
-  uint64_t p = __umul64hi(mix_id(key), cap);
-  for (;;) {
-    // plain (L1-cacheable) load: a stale "empty" is corrected by the CAS, a slot never
-    // changes once it holds a key
-    int64_t k = tab[p].key;
-    if (k == kSetEmpty) {
-      k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&tab[p].key),
-                                         static_cast<unsigned long long>(kSetEmpty),
-                                         static_cast<unsigned long long>(key)));
-      if (k == kSetEmpty) break;
-    }
-    if (k == key) break;
-    if (++p == cap) p = 0;  // cap >= 2n: an empty slot always exists
-  }
-  return static_cast<uint32_t>(p);
-}
-
-__global__ void __launch_bounds__(kPlanBlock)
-plan_insert_kernel(PSlot* __restrict__ tab, uint64_t cap, const int64_t* __restrict__ ids, int64_t n,
-                   int32_t* __restrict__ slotpos, int32_t* __restrict__ rank) {
-  __shared__ int64_t l_key[kLdsSlots + 1];
-  __shared__ int32_t l_min[kLdsSlots + 1];
-  __shared__ int32_t l_cnt[kLdsSlots + 1];
-  __shared__ uint32_t l_slot[kLdsSlots + 1];
-  __shared__ int32_t l_base[kLdsSlots + 1];
-  const int tid = threadIdx.x;
-  for (int e = tid; e <= kLdsSlots; e += kPlanBlock) {
-    l_key[e] = kSetEmpty;
-    l_min[e] = kNoPos;
-    l_cnt[e] = 0;
-  }
-  __syncthreads();
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kPlanBlock + tid;
-  const bool live = i < n;
-  int64_t key = 0;
-  int e = 0, local_rank = 0;
-  if (live) {
-    key = ids[i];
-    if (key == kSetEmpty) {
-      e = kLdsSlots;
-    } else {
-      e = static_cast<int>(mix_id(key) >> 40) & (kLdsSlots - 1);
-      for (;;) {
-        int64_t k = l_key[e];
-        if (k == kSetEmpty) {
-          k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&l_key[e]),
-                                             static_cast<unsigned long long>(kSetEmpty),
-                                             static_cast<unsigned long long>(key)));
-          if (k == kSetEmpty) break;
-        }
-        if (k == key) break;
-        e = (e + 1) & (kLdsSlots - 1);  // at most 1024 distinct ids in 2048 entries
-      }
-    }
-    local_rank = atomicAdd(&l_cnt[e], 1);
-    atomicMin(&l_min[e], tid);
-  }
-  __syncthreads();
-  if (live && l_min[e] == tid) {  // the block's first occurrence speaks for all of them
-    const uint32_t p = global_slot(tab, cap, key);
-    atomicMin(&tab[p].minpos, static_cast<int32_t>(i));
-    l_base[e] = atomicAdd(&tab[p].cnt, l_cnt[e]);
-    l_slot[e] = p;
-  }
-  __syncthreads();
-  if (live) {
-    slotpos[i] = static_cast<int32_t>(l_slot[e]);
-    rank[i] = l_base[e] + local_rank;
-  }
-}
-
-__device__ __forceinline__ void block_rank256(bool flag, int& rank, int& total) {
-  __shared__ int wave_counts[kBlock / kWave];
+// Rank of the set flags among the 1024 threads of a workgroup (by thread index) and their total.
+__device__ __forceinline__ void block_rank1024(bool flag, int& rank, int& total, int* wave_counts /*[16]*/) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const uint64_t ballot = __ballot(flag);
@@ -152,135 +92,428 @@ __device__ __forceinline__ void block_rank256(bool flag, int& rank, int& total) 
   __syncthreads();
   int base = 0, tot = 0;
 #pragma unroll
-  for (int w = 0; w < kBlock / kWave; ++w) {
-    if (w < wave) base += wave_counts[w];
-    tot += wave_counts[w];
+  for (int w = 0; w < kPlanBlock / kWave; ++w) {
+    const int c = wave_counts[w];
+    if (w < wave) base += c;
+    tot += c;
   }
   __syncthreads();
   rank = base + prior;
   total = tot;
 }
 
-__global__ void __launch_bounds__(kBlock)
-plan_first_count_kernel(const PSlot* __restrict__ tab, const int32_t* __restrict__ slotpos, int64_t n,
-                        int32_t* __restrict__ block_counts) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const bool first = i < n && tab[slotpos[i]].minpos == static_cast<int32_t>(i);
-  int rank, total;
-  block_rank256(first, rank, total);
-  if (threadIdx.x == 0) block_counts[blockIdx.x] = total;
-}
-
-// Single-workgroup exclusive scan of up to millions of int32 partials (in place), total out.
-__global__ void __launch_bounds__(1024)
-scan_partials_kernel(int32_t* __restrict__ v, int64_t n, int64_t* __restrict__ total_out) {
-  __shared__ int64_t partial[1024];
-  const int t = threadIdx.x;
-  const int64_t per = (n + 1023) / 1024;
-  const int64_t lo = std::min<int64_t>(t * per, n), hi = std::min<int64_t>(lo + per, n);
-  int64_t sum = 0;
-  for (int64_t b = lo; b < hi; ++b) sum += v[b];
-  partial[t] = sum;
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    int64_t add = t >= off ? partial[t - off] : 0;
+// tile: LDS dedup of tiles of 1024 ids -> records, per-occurrence (record, rank in run), histogram row
+__global__ void __launch_bounds__(kPlanBlock)
+plan_tile_kernel(const int64_t* __restrict__ ids, PlanGeom g, Rec* __restrict__ tile_rec,
+                 int32_t* __restrict__ tile_nrec, uint32_t* __restrict__ occ_rec, uint16_t* __restrict__ hist,
+                 int64_t* __restrict__ counts) {
+  __shared__ int64_t l_key[kLdsSlots + 1];
+  __shared__ int32_t l_min[kLdsSlots + 1];
+  __shared__ int32_t l_cnt[kLdsSlots + 1];
+  __shared__ uint32_t l_hist[kMaxBuckets / 2];  // two 16-bit counters per word
+  __shared__ int wave_counts[kPlanBlock / kWave];
+  const int tid = threadIdx.x;
+  const int nb = 1 << g.nb_log2;
+  if (blockIdx.x == 0 && tid < 2) counts[tid] = 0;
+  for (int w = tid; w < nb / 2; w += kPlanBlock) l_hist[w] = 0;
+  const int t_lo = blockIdx.x * g.tiles_per_wg;
+  const int t_hi = min(g.tiles, t_lo + g.tiles_per_wg);
+  int64_t key_next = 0;
+  if (static_cast<int64_t>(t_lo) * kPlanBlock + tid < g.n) key_next = ids[static_cast<int64_t>(t_lo) * kPlanBlock + tid];
+  for (int t = t_lo; t < t_hi; ++t) {
+    for (int e = tid; e <= kLdsSlots; e += kPlanBlock) {
+      l_key[e] = kSetEmpty;
+      l_min[e] = kNoPos;
+      l_cnt[e] = 0;
+    }
     __syncthreads();
-    partial[t] += add;
+    const int64_t i = static_cast<int64_t>(t) * kPlanBlock + tid;
+    const bool live = i < g.n;
+    const int64_t key = key_next;
+    if (t + 1 < t_hi && i + kPlanBlock < g.n) key_next = ids[i + kPlanBlock];  // in flight while this tile is worked
+    int e = 0, local_rank = 0;
+    if (live) {
+      if (key == kSetEmpty) {
+        e = kLdsSlots;  // reserved entry for the id that equals the empty marker
+      } else {
+        e = static_cast<int>(mix_id(key) >> 20) & (kLdsSlots - 1);
+        for (;;) {
+          int64_t k = l_key[e];
+          if (k == kSetEmpty) {
+            k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&l_key[e]),
+                                               static_cast<unsigned long long>(kSetEmpty),
+                                               static_cast<unsigned long long>(key)));
+            if (k == kSetEmpty) break;
+          }
+          if (k == key) break;
+          e = (e + 1) & (kLdsSlots - 1);  // at most 1024 distinct ids in 2048 entries
+        }
+      }
+      local_rank = atomicAdd(&l_cnt[e], 1);
+      atomicMin(&l_min[e], tid);
+    }
+    __syncthreads();
+    const bool first = live && l_min[e] == tid;
+    int j, total;
+    block_rank1024(first, j, total, wave_counts);
+    if (first) {
+      Rec r;
+      r.key = key;
+      r.pos = static_cast<int32_t>(i);
+      r.word = (static_cast<uint32_t>(l_cnt[e] - 1) << 10) | static_cast<uint32_t>(j);
+      tile_rec[static_cast<int64_t>(t) * kPlanBlock + j] = r;
+      l_min[e] = j;  // every occurrence of the run reads its record index here
+      const int b = bucket_of(key, g.nb_log2);
+      atomicAdd(&l_hist[b >> 1], 1u << ((b & 1) * 16));
+    }
+    if (tid == 0) tile_nrec[t] = total;
+    __syncthreads();
+    if (live) occ_rec[i] = (static_cast<uint32_t>(local_rank) << 10) | static_cast<uint32_t>(l_min[e]);
     __syncthreads();
   }
-  int64_t run = t ? partial[t - 1] : 0;
-  for (int64_t b = lo; b < hi; ++b) {
-    int32_t c = v[b];
-    v[b] = static_cast<int32_t>(run);
+  uint32_t* row = reinterpret_cast<uint32_t*>(hist + static_cast<int64_t>(blockIdx.x) * nb);
+  for (int w = tid; w < nb / 2; w += kPlanBlock) row[w] = l_hist[w];
+}
+
+// colscan: for every bucket, exclusive scan of its histogram column over the rows.
+// Workgroup = 32 buckets x 32 groups of rows.
+__global__ void __launch_bounds__(1024)
+plan_colscan_kernel(const uint16_t* __restrict__ hist, PlanGeom g, int32_t* __restrict__ off,
+                    int32_t* __restrict__ bucket_total) {
+  __shared__ int32_t part[32][33];
+  const int nb = 1 << g.nb_log2;
+  const int bl = threadIdx.x & 31, rg = threadIdx.x >> 5;
+  const int b = blockIdx.x * 32 + bl;
+  const int per = (g.rows + 31) / 32;
+  const int r_lo = min(g.rows, rg * per), r_hi = min(g.rows, r_lo + per);
+  int32_t sum = 0;
+  for (int r = r_lo; r < r_hi; ++r) sum += hist[static_cast<int64_t>(r) * nb + b];
+  part[rg][bl] = sum;
+  __syncthreads();
+  int32_t run = 0;
+  for (int q = 0; q < rg; ++q) run += part[q][bl];
+  for (int r = r_lo; r < r_hi; ++r) {
+    const int64_t at = static_cast<int64_t>(r) * nb + b;
+    const int32_t c = hist[at];
+    off[at] = run;
     run += c;
   }
-  if (t == 1023 && total_out) total_out[0] = partial[1023];
+  if (rg == 31) bucket_total[b] = run;
 }
 
-__global__ void __launch_bounds__(kBlock)
-plan_emit_unique_kernel(const int64_t* __restrict__ ids, PSlot* __restrict__ tab,
-                        const int32_t* __restrict__ slotpos, int64_t n,
-                        const int32_t* __restrict__ block_prefix, int64_t* __restrict__ unique_out,
-                        int32_t* __restrict__ row_start) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const int32_t sp = i < n ? slotpos[i] : 0;
-  const bool first = i < n && tab[sp].minpos == static_cast<int32_t>(i);
-  int rank, total;
-  block_rank256(first, rank, total);
-  if (!first) return;
-  const int32_t u = block_prefix[blockIdx.x] + rank;
-  unique_out[u] = ids[i];
-  row_start[u] = tab[sp].cnt;  // counts for now; scanned in place afterwards
-  tab[sp].cnt = u;             // from here on the field holds the unique index
-}
-
-// Device-wide exclusive scan of row_start[0 .. U) (U read from device memory), three phases
-// over tiles of 1024; entries U .. n are set to the grand total.
+// Exclusive scan of one or two int32 arrays of nb <= 8192 entries by one workgroup;
+// out arrays have nb + 1 entries (the last one is the total); total of the first to total_out.
 __global__ void __launch_bounds__(1024)
-tile_sum_kernel(const int32_t* __restrict__ v, const int64_t* __restrict__ count, int32_t* __restrict__ tile_sums) {
-  __shared__ int wave_sums[16];
-  const int64_t U = count[0];
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * 1024 + threadIdx.x;
-  int x = i < U ? v[i] : 0;
-  for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, kWave);
-  if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = x;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int s = 0;
-    for (int w = 0; w < 16; ++w) s += wave_sums[w];
-    tile_sums[blockIdx.x] = s;
+plan_scan_kernel(const int32_t* __restrict__ in0, int32_t* __restrict__ out0, const int32_t* __restrict__ in1,
+                 int32_t* __restrict__ out1, int nb, int64_t* __restrict__ total_out) {
+  __shared__ int32_t partial[1024];
+  const int t = threadIdx.x;
+  const int per = (nb + 1023) / 1024;
+  const int lo = min(nb, t * per), hi = min(nb, lo + per);
+  for (int pass = 0; pass < 2; ++pass) {
+    const int32_t* in = pass ? in1 : in0;
+    int32_t* out = pass ? out1 : out0;
+    if (in == nullptr) break;
+    int32_t sum = 0;
+    for (int b = lo; b < hi; ++b) sum += in[b];
+    partial[t] = sum;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+      const int32_t add = t >= o ? partial[t - o] : 0;
+      __syncthreads();
+      partial[t] += add;
+      __syncthreads();
+    }
+    int32_t run = t ? partial[t - 1] : 0;
+    for (int b = lo; b < hi; ++b) {
+      const int32_t c = in[b];
+      out[b] = run;
+      run += c;
+    }
+    if (t == 1023) {
+      out[nb] = partial[1023];
+      if (pass == 0 && total_out) total_out[0] = partial[1023];
+    }
+    __syncthreads();
   }
 }
 
-__global__ void __launch_bounds__(1024)
-tile_scan_kernel(int32_t* __restrict__ v, const int64_t* __restrict__ count, const int32_t* __restrict__ tile_prefix,
-                 int64_t n_plus_1, int32_t total) {
-  __shared__ int wave_sums[16];
-  const int64_t U = count[0];
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * 1024 + threadIdx.x;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int x = i < U ? v[i] : 0;
-  int incl = x;
-  for (int off = 1; off < 64; off <<= 1) {
-    int y = __shfl_up(incl, off, kWave);
-    if (lane >= off) incl += y;
-  }
-  if (lane == 63) wave_sums[wave] = incl;
+// scatter: records of a workgroup's tiles go to their buckets
+__global__ void __launch_bounds__(kPlanBlock)
+plan_scatter_kernel(const Rec* __restrict__ tile_rec, const int32_t* __restrict__ tile_nrec, PlanGeom g,
+                    const int32_t* __restrict__ off, const int32_t* __restrict__ bucket_start,
+                    Rec* __restrict__ bucket_rec) {
+  __shared__ int32_t cursor[kMaxBuckets];
+  const int nb = 1 << g.nb_log2;
+  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nb;
+  for (int b = threadIdx.x; b < nb; b += kPlanBlock) cursor[b] = bucket_start[b] + off_row[b];
   __syncthreads();
-  int base = tile_prefix[blockIdx.x];
-  for (int w = 0; w < wave; ++w) base += wave_sums[w];
-  if (i < n_plus_1) v[i] = i < U ? base + incl - x : total;
+  const int t_lo = blockIdx.x * g.tiles_per_wg;
+  const int t_hi = min(g.tiles, t_lo + g.tiles_per_wg);
+  for (int t0 = t_lo; t0 < t_hi; t0 += 4) {  // four tiles' loads in flight
+    Rec r[4];
+    bool have[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int t = t0 + x;
+      have[x] = t < t_hi && static_cast<int>(threadIdx.x) < tile_nrec[t];
+      if (have[x]) r[x] = tile_rec[static_cast<int64_t>(t) * kPlanBlock + threadIdx.x];
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      if (have[x]) bucket_rec[atomicAdd(&cursor[bucket_of(r[x].key, g.nb_log2)], 1)] = r[x];
+    }
+  }
 }
 
+// bucket: dedup of the records of one bucket in LDS. A bucket with more records than one
+// LDS table takes (kBucketSlots / 2) is worked in rounds: round r admits the ids whose hash
+// falls in its share, so every id is handled in exactly one round. The first kBucketRegs
+// records of a thread stay in registers between the two passes over the records; further
+// ones (rare: hot buckets) go through `result` in global memory.
+constexpr int kBucketRegs = 4;
+
+__device__ __forceinline__ bool in_round(int64_t key, uint32_t rounds, uint32_t round) {
+  return rounds == 1 || static_cast<uint32_t>((mix_id(key) >> 8) & 0xffffff) % rounds == round;
+}
+
+__global__ void __launch_bounds__(kBucketBlock)
+plan_bucket_kernel(const Rec* __restrict__ bucket_rec, const int32_t* __restrict__ bucket_start, PlanGeom g,
+                   int2* __restrict__ result, URec* __restrict__ bucket_uniq, int32_t* __restrict__ ucnt,
+                   int32_t* __restrict__ ocnt, int* __restrict__ err) {
+  constexpr int kPad = 16;  // d_min is read 16 entries at a time
+  __shared__ int64_t l_key[kBucketSlots + 1];
+  __shared__ int32_t l_min[kBucketSlots + 1];
+  __shared__ int32_t l_cnt[kBucketSlots + 1];
+  __shared__ uint16_t l_rank[kBucketSlots + 2];
+  __shared__ uint16_t d_ent[kBucketSlots + 2];
+  __shared__ __attribute__((aligned(16))) int32_t d_min[kBucketSlots + 1 + kPad];
+  __shared__ int32_t s_cnt[kBucketSlots + 1];
+  __shared__ int wave_counts[kBucketBlock / kWave];
+  __shared__ int s_n_ent, s_total;
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x;
+  const int32_t r_lo = bucket_start[b], r_hi = bucket_start[b + 1];
+  const int nrec = r_hi - r_lo;
+  const uint32_t rounds = static_cast<uint32_t>(max(1, (nrec + kBucketSlots / 2 - 1) / (kBucketSlots / 2)));
+  Rec reg[kBucketRegs];
+#pragma unroll
+  for (int x = 0; x < kBucketRegs; ++x) {
+    const int32_t q = r_lo + tid + x * kBucketBlock;
+    if (q < r_hi) reg[x] = bucket_rec[q];
+  }
+  int32_t u_done = 0, occ_done = 0;
+
+  // inserts one record; returns the entry (or -1) and the offset of the record's run in the id's list
+  auto insert = [&](const Rec& r, int& e, int& base) {
+    if (r.key == kSetEmpty) {
+      e = kBucketSlots;
+    } else {
+      e = static_cast<int>(mix_id(r.key) >> 32) & (kBucketSlots - 1);
+      int probes = 0;
+      for (;;) {
+        int64_t k = l_key[e];
+        if (k == kSetEmpty) {
+          k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&l_key[e]),
+                                             static_cast<unsigned long long>(kSetEmpty),
+                                             static_cast<unsigned long long>(r.key)));
+          if (k == kSetEmpty) break;
+        }
+        if (k == r.key) break;
+        e = (e + 1) & (kBucketSlots - 1);
+        if (++probes >= kBucketSlots) {  // table full: more distinct ids than a round can take
+          e = -1;
+          base = 0;
+          raise_device_error(err, RECIS_DEVERR_PLAN_OVERFLOW);
+          return;
+        }
+      }
+    }
+    base = atomicAdd(&l_cnt[e], static_cast<int>(r.word >> 10) + 1);
+    atomicMin(&l_min[e], r.pos);
+    if (base == 0) d_ent[atomicAdd(&s_n_ent, 1)] = static_cast<uint16_t>(e);  // first run of the id: list the entry
+  };
+  auto origin_of = [](const Rec& r) { return (static_cast<int64_t>(r.pos) >> 10 << 10) | (r.word & 1023u); };
+
+  for (uint32_t round = 0; round < rounds; ++round) {
+    for (int e = tid; e <= kBucketSlots; e += kBucketBlock) {
+      l_key[e] = kSetEmpty;
+      l_min[e] = kNoPos;
+      l_cnt[e] = 0;
+      l_rank[e] = 0;
+    }
+    if (tid == 0) s_n_ent = 0;
+    __syncthreads();
+    // A: insert the round's records
+    int e_reg[kBucketRegs], base_reg[kBucketRegs];
+#pragma unroll
+    for (int x = 0; x < kBucketRegs; ++x) {
+      e_reg[x] = -2;  // not of this round
+      base_reg[x] = 0;
+      const int32_t q = r_lo + tid + x * kBucketBlock;
+      if (q < r_hi && in_round(reg[x].key, rounds, round)) insert(reg[x], e_reg[x], base_reg[x]);
+    }
+    for (int32_t q = r_lo + tid + kBucketRegs * kBucketBlock; q < r_hi; q += kBucketBlock) {
+      const Rec r = bucket_rec[q];
+      if (!in_round(r.key, rounds, round)) continue;
+      int e, base;
+      insert(r, e, base);
+      result[origin_of(r)] = make_int2(e, base);
+    }
+    __syncthreads();
+    const int n_ent = s_n_ent;
+    for (int k = tid; k < n_ent + kPad; k += kBucketBlock) d_min[k] = k < n_ent ? l_min[d_ent[k]] : kNoPos;
+    __syncthreads();
+    // rank by first position (positions are distinct), counts in rank order
+    for (int k = tid; k < n_ent; k += kBucketBlock) {
+      const int32_t m = d_min[k];
+      int rnk = 0;
+      for (int q = 0; q < n_ent; q += kPad) {
+        const int4 a0 = *reinterpret_cast<const int4*>(&d_min[q]);
+        const int4 a1 = *reinterpret_cast<const int4*>(&d_min[q + 4]);
+        const int4 a2 = *reinterpret_cast<const int4*>(&d_min[q + 8]);
+        const int4 a3 = *reinterpret_cast<const int4*>(&d_min[q + 12]);
+        rnk += (a0.x < m) + (a0.y < m) + (a0.z < m) + (a0.w < m) + (a1.x < m) + (a1.y < m) + (a1.z < m) + (a1.w < m) +
+               (a2.x < m) + (a2.y < m) + (a2.z < m) + (a2.w < m) + (a3.x < m) + (a3.y < m) + (a3.z < m) + (a3.w < m);
+      }
+      const int e = d_ent[k];
+      l_rank[e] = static_cast<uint16_t>(rnk);
+      s_cnt[rnk] = l_cnt[e];
+    }
+    __syncthreads();
+    // exclusive scan of s_cnt[0 .. n_ent) in place (n_ent <= 1025): 5 consecutive entries per thread
+    {
+      constexpr int kPer = (kBucketSlots + 1 + kBucketBlock - 1) / kBucketBlock;
+      int32_t v[kPer];
+      int32_t sum = 0;
+#pragma unroll
+      for (int x = 0; x < kPer; ++x) {
+        const int k = tid * kPer + x;
+        v[x] = k < n_ent ? s_cnt[k] : 0;
+        sum += v[x];
+      }
+      const int lane = tid & (kWave - 1), wave = tid / kWave;
+      int32_t incl = sum;
+      for (int o = 1; o < kWave; o <<= 1) {
+        const int32_t y = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += y;
+      }
+      if (lane == kWave - 1) wave_counts[wave] = incl;
+      __syncthreads();
+      int32_t run = incl - sum;
+      int32_t tot = 0;
+#pragma unroll
+      for (int w = 0; w < kBucketBlock / kWave; ++w) {
+        if (w < wave) run += wave_counts[w];
+        tot += wave_counts[w];
+      }
+      if (tid == 0) s_total = tot;
+#pragma unroll
+      for (int x = 0; x < kPer; ++x) {
+        const int k = tid * kPer + x;
+        if (k < n_ent) s_cnt[k] = run;
+        run += v[x];
+      }
+    }
+    __syncthreads();
+    for (int k = tid; k < n_ent; k += kBucketBlock) {
+      const int e = d_ent[k];
+      const int rnk = l_rank[e];
+      URec u;
+      u.key = e == kBucketSlots ? kSetEmpty : l_key[e];
+      u.list_off = occ_done + s_cnt[rnk];
+      u.cnt = l_cnt[e];
+      bucket_uniq[r_lo + u_done + rnk] = u;
+    }
+    // B: every record learns its unique id (bucket-local) and the list offset of its run
+#pragma unroll
+    for (int x = 0; x < kBucketRegs; ++x) {
+      if (e_reg[x] == -2) continue;
+      int2 out = make_int2(0, 0);  // overflow (flagged): keep the indices in range
+      if (e_reg[x] >= 0) {
+        const int rnk = l_rank[e_reg[x]];
+        out = make_int2(u_done + rnk, occ_done + s_cnt[rnk] + base_reg[x]);
+      }
+      result[origin_of(reg[x])] = out;
+    }
+    for (int32_t q = r_lo + tid + kBucketRegs * kBucketBlock; q < r_hi; q += kBucketBlock) {
+      const Rec r = bucket_rec[q];
+      if (!in_round(r.key, rounds, round)) continue;
+      const int64_t origin = origin_of(r);
+      const int2 eb = result[origin];
+      int2 out = make_int2(0, 0);
+      if (eb.x >= 0) {
+        const int rnk = l_rank[eb.x];
+        out = make_int2(u_done + rnk, occ_done + s_cnt[rnk] + eb.y);
+      }
+      result[origin] = out;
+    }
+    __syncthreads();
+    u_done += n_ent;
+    occ_done += s_total;
+    __syncthreads();
+  }
+  if (tid == 0) {
+    ucnt[b] = u_done;
+    ocnt[b] = occ_done;
+  }
+}
+
+__global__ void plan_empty_kernel(int64_t* __restrict__ counts, int32_t* __restrict__ row_start) {
+  if (threadIdx.x < 2) counts[threadIdx.x] = 0;
+  if (threadIdx.x == 0) row_start[0] = 0;
+}
+
+// emit, per occurrence: inverse, list entry, position in the list
 __global__ void __launch_bounds__(kBlock)
-plan_emit_lists_kernel(const int32_t* __restrict__ slotpos, const int32_t* __restrict__ rank,
-                       const PSlot* __restrict__ tab, const int32_t* __restrict__ row_start, int64_t n,
-                       int32_t* __restrict__ inverse, int32_t* __restrict__ list, int32_t* __restrict__ pos_out) {
+plan_emit_occ_kernel(const int64_t* __restrict__ ids, const uint32_t* __restrict__ occ_rec,
+                     const int2* __restrict__ result, const int32_t* __restrict__ ubase,
+                     const int32_t* __restrict__ lbase, PlanGeom g, int32_t* __restrict__ inverse,
+                     int32_t* __restrict__ list, int32_t* __restrict__ pos_out) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  if (i >= n) return;
-  const int32_t u = tab[slotpos[i]].cnt;
-  const int32_t pos = row_start[u] + rank[i];
-  inverse[i] = u;
-  list[pos] = static_cast<int32_t>(i);
+  if (i >= g.n) return;
+  const uint32_t w = occ_rec[i];
+  const int2 r = result[(i >> 10 << 10) | (w & 1023u)];
+  const int b = bucket_of(ids[i], g.nb_log2);
+  const int32_t pos = lbase[b] + r.y + static_cast<int32_t>(w >> 10);
+  inverse[i] = ubase[b] + r.x;
+  if (static_cast<uint32_t>(pos) < static_cast<uint64_t>(g.n)) list[pos] = static_cast<int32_t>(i);  // else: overflow flagged
   if (pos_out) pos_out[i] = pos;
 }
 
-// (row, chunk) work items for rows with more than kHotLen occurrences.
+// emit, per unique id (workgroups 0 .. buckets-1: one bucket each): id, row_start, hot work
+// items; the remaining workgroups set row_start[U .. n] = n.
 __global__ void __launch_bounds__(kBlock)
-plan_hot_items_kernel(const int32_t* __restrict__ row_start, int64_t* __restrict__ counts,
-                      int32_t* __restrict__ hot_items, int64_t hot_cap) {
-  const int64_t U = counts[0];
-  const int64_t u = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  if (u >= U) return;
-  const int32_t len = row_start[u + 1] - row_start[u];
-  if (len <= kHotLen) return;
-  const int n_items = (len + kHotChunk - 1) / kHotChunk;
-  const int64_t base = static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&counts[1]),
-                                                      static_cast<unsigned long long>(n_items)));
-  for (int k = 0; k < n_items; ++k) {
-    if (base + k < hot_cap) {
-      hot_items[2 * (base + k)] = static_cast<int32_t>(u);
-      hot_items[2 * (base + k) + 1] = k;
+plan_emit_uniq_kernel(const URec* __restrict__ bucket_uniq, const int32_t* __restrict__ bucket_start,
+                      const int32_t* __restrict__ ubase, const int32_t* __restrict__ lbase, PlanGeom g,
+                      int64_t* __restrict__ unique_out, int32_t* __restrict__ row_start,
+                      int64_t* __restrict__ counts, int32_t* __restrict__ hot_items, int64_t hot_cap) {
+  const int nb = 1 << g.nb_log2;
+  if (static_cast<int>(blockIdx.x) >= nb) {
+    const int64_t U = ubase[nb];
+    const int64_t chunk = static_cast<int64_t>(kBlock) * 16;
+    const int64_t lo = U + (static_cast<int64_t>(blockIdx.x) - nb) * chunk;
+    const int64_t hi = min(lo + chunk, g.n + 1);
+    for (int64_t x = lo + threadIdx.x; x < hi; x += kBlock) row_start[x] = static_cast<int32_t>(g.n);
+    return;
+  }
+  const int b = blockIdx.x;
+  const int32_t u0 = ubase[b], cnt = ubase[b + 1] - u0, l0 = lbase[b];
+  const URec* src = bucket_uniq + bucket_start[b];
+  for (int k = threadIdx.x; k < cnt; k += kBlock) {
+    const URec u = src[k];
+    unique_out[u0 + k] = u.key;
+    row_start[u0 + k] = l0 + u.list_off;
+    if (hot_cap > 0 && u.cnt > kHotLen) {
+      const int n_items = (u.cnt + kHotChunk - 1) / kHotChunk;
+      const int64_t base = static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&counts[1]),
+                                                          static_cast<unsigned long long>(n_items)));
+      for (int c = 0; c < n_items; ++c) {
+        if (base + c < hot_cap) {
+          hot_items[2 * (base + c)] = u0 + k;
+          hot_items[2 * (base + c) + 1] = c;
+        }
+      }
     }
   }
 }
@@ -503,59 +736,95 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   RECIS_REQUIRE(hot_cap == 0 || (hot_items_out && hot_cap >= n / kHotLen + n / kHotChunk + 2),
                 "hot_items_out must hold at least n/%d + n/%d + 2 items", kHotLen, kHotChunk);
   RECIS_REQUIRE(n == 0 || (ids && unique_out && inverse_out && list_out), "NULL argument");
-  const int64_t cap = std::max<int64_t>(1024, 2 * n);
-  const int64_t slots = cap + 1;
-  const int64_t nb = std::max<int64_t>(1, (n + kBlock - 1) / kBlock);
-  const int64_t n_tiles = (n + 1 + 1023) / 1024;
-  // workspace: tab[slots] | slotpos[n] | rank[n] | block_counts[nb] | tile sums
-  const size_t bytes = sizeof(PSlot) * slots + sizeof(int32_t) * (2 * n + nb + n_tiles) + 256;
+  int* err = device_error_word(current_device());
+  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  if (n == 0) {
+    plan_empty_kernel<<<1, 64, 0, stream>>>(counts_out_dev, row_start_out);
+    RECIS_LAUNCH_CHECK();
+    return RECIS_OK;
+  }
+  PlanGeom g;
+  g.n = n;
+  g.tiles = static_cast<int>((n + kPlanBlock - 1) / kPlanBlock);
+  g.tiles_per_wg = std::min(63, (g.tiles + kMaxRows - 1) / kMaxRows);  // 16-bit histogram counters
+  g.rows = (g.tiles + g.tiles_per_wg - 1) / g.tiles_per_wg;
+  // about 512 ids per bucket: a few hundred distinct ids for the LDS table of a bucket
+  int nb_log2 = 5;
+  while ((int64_t(1) << (nb_log2 + 1)) <= kMaxBuckets && (int64_t(1) << (nb_log2 + 1)) * 512 <= n) ++nb_log2;
+  g.nb_log2 = nb_log2;
+  const int64_t nb = int64_t(1) << nb_log2;
+  const int64_t n_pad = static_cast<int64_t>(g.tiles) * kPlanBlock;
+  // workspace: tile_rec[n_pad] (later: the unique ids of every bucket) | bucket_rec[n_pad] | result[n_pad] |
+  //            occ_rec[n] | hist[rows*nb] u16 | off[rows*nb] | tile_nrec[tiles] | 6 arrays of nb + 1
+  size_t bytes = 0;
+  auto take = [&](size_t b) {
+    const size_t at = bytes;
+    bytes += (b + 255) & ~size_t(255);
+    return at;
+  };
+  const size_t o_tile = take(sizeof(Rec) * n_pad), o_brec = take(sizeof(Rec) * n_pad);
+  const size_t o_res = take(sizeof(int2) * n_pad), o_occ = take(sizeof(uint32_t) * n_pad);
+  const size_t o_hist = take(sizeof(uint16_t) * g.rows * nb), o_off = take(sizeof(int32_t) * g.rows * nb);
+  const size_t o_nrec = take(sizeof(int32_t) * g.tiles), o_small = take(sizeof(int32_t) * 6 * (nb + 1));
   void* ws = nullptr;
   if (int rc = get_workspace(stream, bytes, &ws)) return rc;
-  PSlot* tab = static_cast<PSlot*>(ws);
-  int32_t* slotpos = reinterpret_cast<int32_t*>(tab + slots);
-  int32_t* rank = slotpos + n;
-  int32_t* block_counts = rank + n;
-  int32_t* tile_sums = block_counts + nb;
+  char* base = static_cast<char*>(ws);
+  Rec* tile_rec = reinterpret_cast<Rec*>(base + o_tile);
+  Rec* bucket_rec = reinterpret_cast<Rec*>(base + o_brec);
+  int2* result = reinterpret_cast<int2*>(base + o_res);
+  uint32_t* occ_rec = reinterpret_cast<uint32_t*>(base + o_occ);
+  uint16_t* hist = reinterpret_cast<uint16_t*>(base + o_hist);
+  int32_t* off = reinterpret_cast<int32_t*>(base + o_off);
+  int32_t* tile_nrec = reinterpret_cast<int32_t*>(base + o_nrec);
+  int32_t* bucket_total = reinterpret_cast<int32_t*>(base + o_small);
+  int32_t* bucket_start = bucket_total + (nb + 1);
+  int32_t* ucnt = bucket_start + (nb + 1);
+  int32_t* ocnt = ucnt + (nb + 1);
+  int32_t* ubase = ocnt + (nb + 1);
+  int32_t* lbase = ubase + (nb + 1);
+  URec* bucket_uniq = reinterpret_cast<URec*>(tile_rec);  // the tile records are dead after the scatter
 
-  RECIS_TIME_KERNEL("plan_init_kernel", stream)
-
-  plan_init_kernel<<<dim3(std::min<int64_t>((slots + kBlock - 1) / kBlock, 256 * 16)), dim3(kBlock), 0, stream>>>(
-      tab, slots, counts_out_dev);
-  RECIS_LAUNCH_CHECK();
-  if (n > 0) {
-    RECIS_TIME_KERNEL("plan_insert_kernel", stream)
-    plan_insert_kernel<<<dim3((n + kPlanBlock - 1) / kPlanBlock), dim3(kPlanBlock), 0, stream>>>(
-        tab, static_cast<uint64_t>(cap), ids, n, slotpos, rank);
-    RECIS_LAUNCH_CHECK();
-    RECIS_TIME_KERNEL("plan_first_count_kernel", stream)
-    plan_first_count_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(tab, slotpos, n, block_counts);
+  {
+    RECIS_TIME_KERNEL("plan_tile_kernel", stream)
+    plan_tile_kernel<<<dim3(g.rows), dim3(kPlanBlock), 0, stream>>>(ids, g, tile_rec, tile_nrec, occ_rec, hist,
+                                                                   counts_out_dev);
     RECIS_LAUNCH_CHECK();
   }
-  scan_partials_kernel<<<1, 1024, 0, stream>>>(block_counts, n > 0 ? nb : 0, counts_out_dev);
-  RECIS_LAUNCH_CHECK();
-  if (n > 0) {
-    RECIS_TIME_KERNEL("plan_emit_unique_kernel", stream)
-    plan_emit_unique_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(ids, tab, slotpos, n, block_counts, unique_out,
-                                                                   row_start_out);
+  {
+    RECIS_TIME_KERNEL("plan_colscan_kernel", stream)
+    plan_colscan_kernel<<<dim3(nb / 32), dim3(1024), 0, stream>>>(hist, g, off, bucket_total);
     RECIS_LAUNCH_CHECK();
   }
-  tile_sum_kernel<<<dim3(n_tiles), dim3(1024), 0, stream>>>(row_start_out, counts_out_dev, tile_sums);
+  plan_scan_kernel<<<1, 1024, 0, stream>>>(bucket_total, bucket_start, nullptr, nullptr, static_cast<int>(nb),
+                                           nullptr);
   RECIS_LAUNCH_CHECK();
-  scan_partials_kernel<<<1, 1024, 0, stream>>>(tile_sums, n_tiles, nullptr);
-  RECIS_LAUNCH_CHECK();
-  tile_scan_kernel<<<dim3(n_tiles), dim3(1024), 0, stream>>>(row_start_out, counts_out_dev, tile_sums, n + 1,
-                                                            static_cast<int32_t>(n));
-  RECIS_LAUNCH_CHECK();
-  if (n > 0) {
-    RECIS_TIME_KERNEL("plan_emit_lists_kernel", stream)
-    plan_emit_lists_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(slotpos, rank, tab, row_start_out, n,
-                                                                  inverse_out, list_out, pos_out);
+  {
+    RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
+    plan_scatter_kernel<<<dim3(g.rows), dim3(kPlanBlock), 0, stream>>>(tile_rec, tile_nrec, g, off, bucket_start,
+                                                                      bucket_rec);
     RECIS_LAUNCH_CHECK();
-    if (hot_cap > 0) {
-      plan_hot_items_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(row_start_out, counts_out_dev, hot_items_out,
-                                                                   hot_cap);
-      RECIS_LAUNCH_CHECK();
-    }
+  }
+  {
+    RECIS_TIME_KERNEL("plan_bucket_kernel", stream)
+    plan_bucket_kernel<<<dim3(nb), dim3(kBucketBlock), 0, stream>>>(bucket_rec, bucket_start, g, result, bucket_uniq,
+                                                                   ucnt, ocnt, err);
+    RECIS_LAUNCH_CHECK();
+  }
+  plan_scan_kernel<<<1, 1024, 0, stream>>>(ucnt, ubase, ocnt, lbase, static_cast<int>(nb), counts_out_dev);
+  RECIS_LAUNCH_CHECK();
+  {
+    RECIS_TIME_KERNEL("plan_emit_occ_kernel", stream)
+    plan_emit_occ_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(
+        ids, occ_rec, result, ubase, lbase, g, inverse_out, list_out, pos_out);
+    RECIS_LAUNCH_CHECK();
+  }
+  {
+    const int64_t tail_blocks = (n + 1 + kBlock * 16 - 1) / (kBlock * 16);
+    RECIS_TIME_KERNEL("plan_emit_uniq_kernel", stream)
+    plan_emit_uniq_kernel<<<dim3(nb + tail_blocks), dim3(kBlock), 0, stream>>>(
+        bucket_uniq, bucket_start, ubase, lbase, g, unique_out, row_start_out, counts_out_dev, hot_items_out,
+        hot_cap);
+    RECIS_LAUNCH_CHECK();
   }
   return RECIS_OK;
 }

@@ -600,7 +600,7 @@ class HashTable(torch.nn.Module):
     """Dynamic embedding table (recis/nn/modules/hashtable.py:98-423).
 
     ``dedup`` chooses how ``forward`` removes duplicate ids: ``"hash"`` (default) is the
-    HIP hash dedup, whose unique ids come in order of first occurrence; ``"sorted"`` is
+    HIP hash dedup, whose unique ids come in a fixed, input-determined order (hash bucket, then first occurrence); ``"sorted"`` is
     ``torch.unique`` as in the reference, which also makes the row a new key receives
     identical to the reference's (new keys are ranked in ascending key order).
     ``reserve_rows`` pre-sizes the map and the row storage."""

@@ -197,7 +197,7 @@ def test_grad_accumulation_kat():
 def test_sparse_adam_family_tracks_torch_adamw(cls, ref_wd):
     # tests/optim/sparse_adamw_test.py:84-175: zero-init rows, every row updated each step
     U, D, steps, lr, wd = 512, 16, 20, 1e-2, 1e-2
-    ht = HashTable([D], block_size=128, device="cuda", name="adam_" + ref_wd)
+    ht = HashTable([D], block_size=128, device="cuda", name="adam_" + ref_wd, dedup="sorted")
     ht.train()
     opt = cls(filter_out_sparse_param(ht), lr=lr, weight_decay=wd)
     torch_wd = {"adamw": wd, "tf": wd / lr, "none": 0.0}[ref_wd]

@@ -191,18 +191,17 @@ def test_ragged_tile_forward_backward(rng, dtype):
     assert _lib.poll_device_errors() == 0
 
 
-@pytest.mark.parametrize("n,hi", [(0, 10), (1, 10), (1000, 50), (300000, 40), (200000, 3000), (1000000, 10**7)])
-def test_unique_plan_lists(rng, n, hi):
-    """The plan's dedup equals ids_unique; its lists are a permutation of the occurrences grouped
-    by unique id (hot ids with tens of thousands of repeats included)."""
-    ids = rng.integers(-hi, hi, size=n)
-    if n > 5:
-        ids[3] = -1
+def _check_plan(ids):
+    """Invariants of a batch plan: the unique ids are exactly the set of ids, the inverse maps
+    back, the lists partition the occurrences by unique id; the result is a function of the
+    input only (two calls agree bit for bit on everything but the order inside a list)."""
+    n = len(ids)
     p = ops.ids_unique_plan(_dev(ids))
-    _, first = np.unique(ids, return_index=True)
-    np.testing.assert_array_equal(p.unique.cpu().numpy(), ids[np.sort(first)])
+    uniq = p.unique.cpu().numpy()
+    np.testing.assert_array_equal(np.sort(uniq), np.unique(ids))
     inv = p.inverse.cpu().numpy()
-    np.testing.assert_array_equal(p.unique.cpu().numpy()[inv] if n else inv, ids)
+    assert p.U == len(uniq) and (n == 0 or (inv.min() >= 0 and inv.max() < p.U))
+    np.testing.assert_array_equal(uniq[inv] if n else inv, ids)
     rs, occ, pos = p.row_start.cpu().numpy(), p.occ.cpu().numpy(), p.pos.cpu().numpy()
     assert rs[0] == 0 and np.all(rs[p.U:] == n) and np.all(np.diff(rs[: p.U + 1]) >= 1 if p.U else True)
     np.testing.assert_array_equal(np.sort(occ), np.arange(n))
@@ -212,6 +211,40 @@ def test_unique_plan_lists(rng, n, hi):
     counts = p.counts.cpu().numpy()
     lens = np.diff(rs[: p.U + 1])
     assert counts[0] == p.U and counts[1] == int(np.sum(np.ceil(lens[lens > 256] / 8192)))
+    hot = p.hot_items.cpu().numpy()[: 2 * counts[1]].reshape(-1, 2)
+    exp_hot = sorted((int(u), c) for u in np.nonzero(lens > 256)[0] for c in range(-(-int(lens[u]) // 8192)))
+    assert sorted(map(tuple, hot.tolist())) == exp_hot
+    q = ops.ids_unique_plan(_dev(ids))
+    np.testing.assert_array_equal(q.unique.cpu().numpy(), uniq)
+    np.testing.assert_array_equal(q.inverse.cpu().numpy(), inv)
+    np.testing.assert_array_equal(q.row_start.cpu().numpy(), rs)
+    assert _lib.poll_device_errors() == 0
+    return p
+
+
+@pytest.mark.parametrize("n,hi", [(0, 10), (1, 10), (1000, 50), (1025, 10**6), (300000, 40), (200000, 3000),
+                                  (1000000, 10**7), (3000000, 10**12)])
+def test_unique_plan_lists(rng, n, hi):
+    """Random ids from hot (tens of thousands of repeats of each id) to nearly all distinct, the id
+    that equals the library's empty marker included."""
+    ids = rng.integers(-hi, hi, size=n)
+    if n > 5:
+        ids[3] = -1
+    _check_plan(ids)
+
+
+def test_unique_plan_skewed_buckets(rng):
+    """Shapes that stress the hash partition: one id everywhere; a few ids present in every tile
+    next to a distinct tail (buckets worked in several rounds); ids that differ in the low bits
+    only; a sorted run."""
+    n = 600000
+    _check_plan(np.full(n, 7, dtype=np.int64))
+    hot = rng.integers(0, 300, size=n)
+    tail = np.arange(n, dtype=np.int64) * 2**32 + 5
+    _check_plan(np.where(rng.random(n) < 0.5, hot, tail))
+    _check_plan(np.arange(n, dtype=np.int64))
+    _check_plan(np.sort(rng.integers(0, 5000, size=n)))
+    _check_plan(np.arange(n, dtype=np.int64)[::-1] << 40)
 
 
 @pytest.mark.parametrize("mode", ["sum", "mean", "tile"])
