@@ -25,7 +25,7 @@
 namespace recis_hip {
 namespace {
 
-struct Slot {
+struct alignas(16) Slot {
   int64_t key;
   int64_t val;
 };
@@ -44,6 +44,12 @@ __device__ __forceinline__ uint64_t mix_key(int64_t key) {
   x *= 0xc4ceb9fe1a85ec53ULL;
   x ^= x >> 33;
   return x;
+}
+
+// First slot probed for a key: the TOP bits of the mixed key. Batches come out of the batch
+// plan ordered by the top bits of the same mix, so their probes walk the table front to back.
+__device__ __forceinline__ uint64_t home_slot(int64_t key, uint64_t mask) {
+  return mix_key(key) >> __builtin_clzll(mask);  // mask = capacity - 1, capacity a power of two >= 2
 }
 
 __device__ __forceinline__ int64_t ld_relaxed(const int64_t* p) {
@@ -104,11 +110,27 @@ find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __r
       raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
       out[i] = -1;
     } else {
-      const uint64_t h = mix_key(key) & mask;
+      const uint64_t h = home_slot(key, mask);
       uint64_t p = h;
       int64_t first_tomb = -1;
       uint64_t probes = 0;
       for (;;) {
+        // Hint from one plain 16-byte load (L1-cacheable, may be stale). Two things it shows cannot
+        // change while this kernel runs: a key with an assigned row, and a slot held by another key.
+        const longlong2 hint = *reinterpret_cast<const longlong2*>(&table[p]);
+        if (hint.x == key && hint.y >= 0) {
+          out[i] = hint.y;
+          break;
+        }
+        if (hint.x != key && hint.x != kEmpty && hint.x != kTomb) {
+          p = (p + 1) & mask;
+          if (++probes > mask) {
+            raise_device_error(err, RECIS_DEVERR_TABLE_FULL);
+            out[i] = -1;
+            break;
+          }
+          continue;
+        }
         const int64_t k = ld_relaxed(&table[p].key);
         if (k == key) {
           const int64_t v = ld_relaxed(&table[p].val);
@@ -239,7 +261,7 @@ find_kernel(const Slot* __restrict__ table, uint64_t mask, const int64_t* __rest
   const int64_t key = ids[i];
   int64_t res = -1;
   if (key != kEmpty && key != kTomb) {
-    uint64_t p = mix_key(key) & mask;
+    uint64_t p = home_slot(key, mask);
     for (uint64_t probes = 0; probes <= mask; ++probes) {
       const int64_t k = table[p].key;
       if (k == key) {
@@ -264,7 +286,7 @@ erase_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __restrict_
   if (i < n) {
     const int64_t key = ids[i];
     if (key != kEmpty && key != kTomb) {
-      uint64_t p = mix_key(key) & mask;
+      uint64_t p = home_slot(key, mask);
       for (uint64_t probes = 0; probes <= mask; ++probes) {
         const int64_t k = ld_relaxed(&table[p].key);
         if (k == key) {
@@ -337,7 +359,7 @@ rehash_kernel(const Slot* __restrict__ old_table, int64_t old_capacity, Slot* __
   const int64_t key = old_table[i].key;
   const int64_t val = old_table[i].val;
   if (key == kEmpty || key == kTomb || val < 0) return;
-  uint64_t p = mix_key(key) & mask;
+  uint64_t p = home_slot(key, mask);
   for (uint64_t probes = 0; probes <= mask; ++probes) {
     const int64_t old = static_cast<int64_t>(atomicCAS(
         reinterpret_cast<unsigned long long*>(&table[p].key),
