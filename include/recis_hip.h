@@ -43,6 +43,11 @@ extern "C" {
 #define RECIS_MAX 3
 
 /* flags */
+/* batch plan: unique ids with more than HOT_LEN occurrences are reduced by whole workgroups,
+ * one (row, chunk of HOT_CHUNK occurrences) work item each */
+#define RECIS_PLAN_HOT_LEN 256
+#define RECIS_PLAN_HOT_CHUNK 2048
+
 #define RECIS_FLAG_REV_UNIQUE 1 /* caller guarantees reverse_indices has no duplicates */
 
 /* bits of the device-side soft-error word (recis_hip_poll_device_errors) */
@@ -332,7 +337,7 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
  *   list_out      [n]      occurrence indices grouped by unique id
  *   pos_out       [n]      position of occurrence i in list_out (may be NULL)
  *   hot_items_out [2*hot_cap] (row, chunk) work items for ids with more than 256
- *                          occurrences; hot_cap >= n/256 + n/8192 + 2, or 0 to skip
+ *                          occurrences; hot_cap >= n/HOT_LEN + n/HOT_CHUNK + 2, or 0 to skip
  *   counts_out_dev [2]     device words: number of unique ids, number of hot items
  * The unique ids are ordered by (hash bucket, first occurrence): the order, the inverse and
  * row_start depend on the input only; the order of the entries inside one id's list and of
@@ -367,7 +372,7 @@ int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_feat
 /*
  * out[u, :] (+)= sum over k in [row_start[u], row_start[u+1]) of coef[k] * rows[src[k], :]
  * for u < U. Rows with at most 256 entries are reduced by a small group of lanes and
- * written once; hot rows are reduced by whole workgroups per 8192-entry chunk and
+ * written once; hot rows are reduced by whole workgroups per RECIS_PLAN_HOT_CHUNK-entry chunk and
  * combined with a few fp32 atomics (out must then be fp32, D <= 1024). accumulate != 0
  * adds to what out holds. src < 0 skips the entry; coef may be NULL (= 1).
  */

@@ -43,8 +43,8 @@ constexpr int kMinBuckets = 32;
 constexpr int kMaxRows = 512;  // histogram rows (= workgroups of the tile and scatter kernels)
 constexpr int64_t kSetEmpty = -1;
 constexpr int32_t kNoPos = 0x7fffffff;
-constexpr int kHotLen = 256;      // rows with more occurrences than this are "hot"
-constexpr int kHotChunk = 8192;   // occurrences per hot work item
+constexpr int kHotLen = RECIS_PLAN_HOT_LEN;  // rows with more occurrences than this are "hot"
+constexpr int kHotChunk = RECIS_PLAN_HOT_CHUNK;  // occurrences per hot work item
 
 __device__ __forceinline__ uint64_t mix_id(int64_t key) {
   uint64_t x = static_cast<uint64_t>(key);
@@ -538,16 +538,22 @@ struct CsrArgs {
 };
 
 // One group of LPR lanes per unique row (cold rows); hot rows are cleared here and summed by
-// csr_hot_kernel.
+// csr_hot_kernel. A wave that holds a row with more than kCoopLen occurrences switches, as a
+// whole, to working its rows one after the other with all its lane groups striding over the
+// row's list (a row of 200 occurrences would otherwise be 50 dependent gathers of one group).
+constexpr int kCoopLen = 8;
+
 template <typename TIn, typename TOut, int VEC>
 __global__ void __launch_bounds__(kBlock)
 csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a) {
   const int rows_per_block = kBlock >> a.lpr_log2;
   const int64_t u = static_cast<int64_t>(blockIdx.x) * rows_per_block + (threadIdx.x >> a.lpr_log2);
-  if (u >= a.U) return;
+  const bool valid = u < a.U;
   const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
-  const int32_t start = a.row_start[u], end = a.row_start[u + 1];
+  const int32_t start = valid ? a.row_start[u] : 0;
+  int32_t end = valid ? a.row_start[u + 1] : 0;
   const bool hot = end - start > kHotLen;
+  if (hot) end = start;  // nothing to gather here
   const int D = a.D;
 
   auto fetch = [&](int32_t k, int c0, float (&v)[VEC], float& w) {
@@ -562,45 +568,77 @@ csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
     }
     load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
   };
-
-  for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
-    float acc[VEC];
+  // acc += sum over list entries k = first, first + step, ... < last (4 gathers in flight)
+  auto gather_sum = [&](int32_t first, int32_t last, int32_t step, int c0, float (&acc)[VEC]) {
+    int32_t k = first;
+    for (; k + 3 * step < last; k += 4 * step) {
+      float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
+      float w0, w1, w2, w3;
+      fetch(k, c0, v0, w0);
+      fetch(k + step, c0, v1, w1);
+      fetch(k + 2 * step, c0, v2, w2);
+      fetch(k + 3 * step, c0, v3, w3);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    if (!hot) {
-      int32_t k = start;
-      for (; k + 3 < end; k += 4) {
-        float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
-        float w0, w1, w2, w3;
-        fetch(k, c0, v0, w0);
-        fetch(k + 1, c0, v1, w1);
-        fetch(k + 2, c0, v2, w2);
-        fetch(k + 3, c0, v3, w3);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          acc[j] = fmaf(v0[j], w0, acc[j]);
-          acc[j] = fmaf(v1[j], w1, acc[j]);
-          acc[j] = fmaf(v2[j], w2, acc[j]);
-          acc[j] = fmaf(v3[j], w3, acc[j]);
-        }
-      }
-      for (; k < end; ++k) {
-        float v0[VEC];
-        float w0;
-        fetch(k, c0, v0, w0);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v0[j], w0, acc[j]);
+      for (int j = 0; j < VEC; ++j) {
+        acc[j] = fmaf(v0[j], w0, acc[j]);
+        acc[j] = fmaf(v1[j], w1, acc[j]);
+        acc[j] = fmaf(v2[j], w2, acc[j]);
+        acc[j] = fmaf(v3[j], w3, acc[j]);
       }
     }
-    TOut* dst = out + u * D + c0;
+    for (; k < last; k += step) {
+      float v0[VEC];
+      float w0;
+      fetch(k, c0, v0, w0);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v0[j], w0, acc[j]);
+    }
+  };
+  auto finish = [&](int64_t row, bool row_hot, int c0, float (&acc)[VEC]) {
+    TOut* dst = out + row * D + c0;
     if (a.accumulate) {
-      if (hot) continue;  // keep what is there; the hot kernel adds to it
+      if (row_hot) return;  // keep what is there; the hot kernel adds to it
       float old[VEC];
       load_pack<TOut, VEC>(dst, old);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] += old[j];
     }
     store_pack<TOut, VEC>(dst, acc);
+  };
+
+  // short rows: every lane group works its own row
+  const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;  // with one group per wave there is nobody to share with
+  if (valid && !is_long) {
+    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+      float acc[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+      gather_sum(start, end, 1, c0, acc);
+      finish(u, hot, c0, acc);
+    }
+  }
+  // long rows of this wave, one after the other: every lane group strides over the row's list
+  const int lane = threadIdx.x & (kWave - 1);
+  const int groups = kWave >> a.lpr_log2;
+  const int g = lane >> a.lpr_log2;
+  uint64_t todo = __ballot(is_long);
+  while (todo) {
+    const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;  // first lane of the owning group
+    todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);  // the group's lanes (fewer than 64 here)
+    const int r = owner >> a.lpr_log2;
+    const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
+    const int64_t row = u - g + r;  // rows of a wave are consecutive
+    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+      float acc[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+      gather_sum(r_start + g, r_end, groups, c0, acc);
+      for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+      }
+      if (g == r) finish(row, false, c0, acc);
+    }
   }
 }
 
@@ -628,12 +666,37 @@ csr_hot_kernel(const TIn* __restrict__ rows, float* __restrict__ out, CsrArgs a,
       float acc[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      for (int32_t k = start + g; k < end; k += groups) {
+      auto fetch = [&](int32_t k, float (&v)[VEC], float& w) {
         const int32_t s = a.src[k];
-        if (s < 0 || static_cast<int64_t>(s) >= a.n_rows) continue;
-        const float w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
-        float v[VEC];
+        w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
+        if (s < 0 || static_cast<int64_t>(s) >= a.n_rows) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+          w = 0.f;
+          return;
+        }
         load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
+      };
+      int32_t k = start + g;
+      for (; k + 3 * groups < end; k += 4 * groups) {  // four gathers in flight per lane
+        float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
+        float w0, w1, w2, w3;
+        fetch(k, v0, w0);
+        fetch(k + groups, v1, w1);
+        fetch(k + 2 * groups, v2, w2);
+        fetch(k + 3 * groups, v3, w3);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          acc[j] = fmaf(v0[j], w0, acc[j]);
+          acc[j] = fmaf(v1[j], w1, acc[j]);
+          acc[j] = fmaf(v2[j], w2, acc[j]);
+          acc[j] = fmaf(v3[j], w3, acc[j]);
+        }
+      }
+      for (; k < end; k += groups) {
+        float v[VEC];
+        float w;
+        fetch(k, v, w);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[j], w, acc[j]);
       }

@@ -650,7 +650,7 @@ class IdMap:
 
 
 # ------------------------------------------------------------------ batch plan
-_HOT_LEN, _HOT_CHUNK = 256, 8192
+_HOT_LEN, _HOT_CHUNK = 256, 2048  # RECIS_PLAN_HOT_LEN / RECIS_PLAN_HOT_CHUNK of the library
 
 
 class BatchPlan:

@@ -210,9 +210,9 @@ def _check_plan(ids):
     np.testing.assert_array_equal(inv[occ], row_of_entry)
     counts = p.counts.cpu().numpy()
     lens = np.diff(rs[: p.U + 1])
-    assert counts[0] == p.U and counts[1] == int(np.sum(np.ceil(lens[lens > 256] / 8192)))
+    assert counts[0] == p.U and counts[1] == int(np.sum(np.ceil(lens[lens > 256] / ops._HOT_CHUNK)))
     hot = p.hot_items.cpu().numpy()[: 2 * counts[1]].reshape(-1, 2)
-    exp_hot = sorted((int(u), c) for u in np.nonzero(lens > 256)[0] for c in range(-(-int(lens[u]) // 8192)))
+    exp_hot = sorted((int(u), c) for u in np.nonzero(lens > 256)[0] for c in range(-(-int(lens[u]) // ops._HOT_CHUNK)))
     assert sorted(map(tuple, hot.tolist())) == exp_hot
     q = ops.ids_unique_plan(_dev(ids))
     np.testing.assert_array_equal(q.unique.cpu().numpy(), uniq)
