@@ -266,9 +266,11 @@ plan_scatter_kernel(const Rec* __restrict__ tile_rec, const int32_t* __restrict_
   }
 }
 
-// bucket: dedup of the records of one bucket in LDS. A bucket with more records than one
-// LDS table takes (kBucketSlots / 2) is worked in rounds: round r admits the ids whose hash
-// falls in its share, so every id is handled in exactly one round. The first kBucketRegs
+// bucket: dedup of the records of one bucket in LDS. A bucket normally holds a few hundred
+// distinct ids (its records can be many more: a hot id brings one record per tile). When the
+// distinct ids do not fit the LDS table, the bucket is started over in twice as many rounds:
+// round r admits the ids whose hash falls in its share, so every id is handled in exactly one
+// round. The first kBucketRegs
 // records of a thread stay in registers between the two passes over the records; further
 // ones (rare: hot buckets) go through `result` in global memory.
 constexpr int kBucketRegs = 4;
@@ -290,12 +292,12 @@ plan_bucket_kernel(const Rec* __restrict__ bucket_rec, const int32_t* __restrict
   __shared__ __attribute__((aligned(16))) int32_t d_min[kBucketSlots + 1 + kPad];
   __shared__ int32_t s_cnt[kBucketSlots + 1];
   __shared__ int wave_counts[kBucketBlock / kWave];
-  __shared__ int s_n_ent, s_total;
+  __shared__ int s_n_ent, s_total, s_overflow;
   const int tid = threadIdx.x;
   const int b = blockIdx.x;
   const int32_t r_lo = bucket_start[b], r_hi = bucket_start[b + 1];
   const int nrec = r_hi - r_lo;
-  const uint32_t rounds = static_cast<uint32_t>(max(1, (nrec + kBucketSlots / 2 - 1) / (kBucketSlots / 2)));
+  uint32_t rounds = 1;
   Rec reg[kBucketRegs];
 #pragma unroll
   for (int x = 0; x < kBucketRegs; ++x) {
@@ -324,14 +326,18 @@ plan_bucket_kernel(const Rec* __restrict__ bucket_rec, const int32_t* __restrict
         if (++probes >= kBucketSlots) {  // table full: more distinct ids than a round can take
           e = -1;
           base = 0;
-          raise_device_error(err, RECIS_DEVERR_PLAN_OVERFLOW);
+          s_overflow = 1;
           return;
         }
       }
     }
     base = atomicAdd(&l_cnt[e], static_cast<int>(r.word >> 10) + 1);
     atomicMin(&l_min[e], r.pos);
-    if (base == 0) d_ent[atomicAdd(&s_n_ent, 1)] = static_cast<uint16_t>(e);  // first run of the id: list the entry
+    if (base == 0) {  // first run of the id: list the entry
+      const int k = atomicAdd(&s_n_ent, 1);
+      d_ent[k] = static_cast<uint16_t>(e);
+      if (k >= kBucketSlots * 7 / 8) s_overflow = 1;  // too loaded to go on probing
+    }
   };
   auto origin_of = [](const Rec& r) { return (static_cast<int64_t>(r.pos) >> 10 << 10) | (r.word & 1023u); };
 
@@ -342,7 +348,10 @@ plan_bucket_kernel(const Rec* __restrict__ bucket_rec, const int32_t* __restrict
       l_cnt[e] = 0;
       l_rank[e] = 0;
     }
-    if (tid == 0) s_n_ent = 0;
+    if (tid == 0) {
+      s_n_ent = 0;
+      s_overflow = 0;
+    }
     __syncthreads();
     // A: insert the round's records
     int e_reg[kBucketRegs], base_reg[kBucketRegs];
@@ -361,6 +370,18 @@ plan_bucket_kernel(const Rec* __restrict__ bucket_rec, const int32_t* __restrict
       result[origin_of(r)] = make_int2(e, base);
     }
     __syncthreads();
+    if (s_overflow) {  // start the bucket over with twice the rounds
+      __syncthreads();
+      if (rounds >= (1u << 16)) {
+        if (tid == 0) raise_device_error(err, RECIS_DEVERR_PLAN_OVERFLOW);
+        break;
+      }
+      rounds *= 2;
+      round = static_cast<uint32_t>(-1);  // ++ makes it 0
+      u_done = 0;
+      occ_done = 0;
+      continue;
+    }
     const int n_ent = s_n_ent;
     for (int k = tid; k < n_ent + kPad; k += kBucketBlock) d_min[k] = k < n_ent ? l_min[d_ent[k]] : kNoPos;
     __syncthreads();
@@ -811,7 +832,8 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   g.tiles = static_cast<int>((n + kPlanBlock - 1) / kPlanBlock);
   g.tiles_per_wg = std::min(63, (g.tiles + kMaxRows - 1) / kMaxRows);  // 16-bit histogram counters
   g.rows = (g.tiles + g.tiles_per_wg - 1) / g.tiles_per_wg;
-  // about 512 ids per bucket: a few hundred distinct ids for the LDS table of a bucket
+  // 512 to 1024 ids per bucket while the bucket count allows: a few hundred distinct ids for the
+  // LDS table of a bucket
   int nb_log2 = 5;
   while ((int64_t(1) << (nb_log2 + 1)) <= kMaxBuckets && (int64_t(1) << (nb_log2 + 1)) * 512 <= n) ++nb_log2;
   g.nb_log2 = nb_log2;
