@@ -339,6 +339,9 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
  *   hot_items_out [2*hot_cap] (row, chunk) work items for ids with more than 256
  *                          occurrences; hot_cap >= n/HOT_LEN + n/HOT_CHUNK + 2, or 0 to skip
  *   counts_out_dev [2]     device words: number of unique ids, number of hot items
+ *   unique_count_host      host word or NULL: when given, the call returns only once the number
+ *                          of unique ids is known and stores it there (the last kernels of the
+ *                          plan may still be running: the wait is for the count alone)
  * The unique ids are ordered by (hash bucket, first occurrence): the order, the inverse and
  * row_start depend on the input only; the order of the entries inside one id's list and of
  * the hot items is not specified. No global atomics are used: ids are partitioned by hash
@@ -352,7 +355,7 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
 int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
                       int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
                       int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev,
-                      void* stream);
+                      int64_t* unique_count_host, void* stream);
 
 /*
  * Per list entry, the input row it reads and its coefficient, for the backward of
@@ -375,11 +378,15 @@ int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_feat
  * written once; hot rows are reduced by whole workgroups per RECIS_PLAN_HOT_CHUNK-entry chunk and
  * combined with a few fp32 atomics (out must then be fp32, D <= 1024). accumulate != 0
  * adds to what out holds. src < 0 skips the entry; coef may be NULL (= 1).
+ * cover_offsets (device, [cover_S + 1], int32 or int64) or NULL: entries whose src lies outside
+ * [cover_offsets[0], cover_offsets[cover_S]) are skipped too (occurrences no segment covers,
+ * for the backward of the TILE mode where src is the occurrence itself).
  */
 int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
                             const void* coef, int coef_dtype, const int32_t* row_start,
                             const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev,
                             void* out, int out_dtype, int64_t U, int64_t D, int accumulate,
+                            const void* cover_offsets, int cover_is64, int64_t cover_S,
                             void* stream);
 
 /* ------------------------------------------------------------------------- *

@@ -231,4 +231,8 @@ struct KernelTimer {
 // calls on that stream. Never shrinks; released at process exit.
 int get_workspace(hipStream_t stream, size_t bytes, void** out);
 
+// Per-(device, stream) pinned host words and an event, for handing a device-side count to the
+// host while later kernels of the same call are still running.
+int get_count_staging(hipStream_t stream, int64_t** host, hipEvent_t* event);
+
 }  // namespace recis_hip

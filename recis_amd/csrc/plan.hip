@@ -556,7 +556,19 @@ struct CsrArgs {
   int lpr_log2;
   int accumulate;
   int* err;
+  const void* cover;  // offsets [cover_S + 1] or NULL: entries whose src lies outside
+  int cover64;        // [cover[0], cover[cover_S]) are skipped
+  int64_t cover_S;
 };
+
+__device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64_t& hi) {
+  lo = 0;
+  hi = a.n_rows;
+  if (a.cover) {
+    lo = max(lo, load_index(a.cover, a.cover64, 0));
+    hi = min(hi, load_index(a.cover, a.cover64, a.cover_S));
+  }
+}
 
 // One group of LPR lanes per unique row (cold rows); hot rows are cleared here and summed by
 // csr_hot_kernel. A wave that holds a row with more than kCoopLen occurrences switches, as a
@@ -576,12 +588,14 @@ csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
   const bool hot = end - start > kHotLen;
   if (hot) end = start;  // nothing to gather here
   const int D = a.D;
+  int64_t c_lo, c_hi;
+  cover_range(a, c_lo, c_hi);
 
   auto fetch = [&](int32_t k, int c0, float (&v)[VEC], float& w) {
     const int32_t s = a.src[k];
     w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
-    if (s < 0 || static_cast<int64_t>(s) >= a.n_rows) {
-      if (s >= 0) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+    if (s < c_lo || s >= c_hi) {
+      if (static_cast<int64_t>(s) >= a.n_rows) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) v[j] = 0.f;
       w = 0.f;
@@ -670,6 +684,8 @@ __global__ void __launch_bounds__(kPlanBlock)
 csr_hot_kernel(const TIn* __restrict__ rows, float* __restrict__ out, CsrArgs a,
                const int32_t* __restrict__ hot_items, const int64_t* __restrict__ counts, int64_t hot_cap) {
   extern __shared__ float s_part[];  // [waves][D]
+  int64_t c_lo, c_hi;
+  cover_range(a, c_lo, c_hi);
   int64_t n_items = counts[1];
   if (n_items > hot_cap) n_items = hot_cap;
   const int D = a.D;
@@ -690,7 +706,7 @@ csr_hot_kernel(const TIn* __restrict__ rows, float* __restrict__ out, CsrArgs a,
       auto fetch = [&](int32_t k, float (&v)[VEC], float& w) {
         const int32_t s = a.src[k];
         w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
-        if (s < 0 || static_cast<int64_t>(s) >= a.n_rows) {
+        if (s < c_lo || s >= c_hi) {
 #pragma unroll
           for (int j = 0; j < VEC; ++j) v[j] = 0.f;
           w = 0.f;
@@ -813,7 +829,7 @@ extern "C" {
 
 int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
                       int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
-                      int64_t hot_cap, int64_t* counts_out_dev, void* stream_) {
+                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* unique_count_host, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   RECIS_REQUIRE(n >= 0 && n < (int64_t(1) << 30), "n out of range: %lld", (long long)n);
   RECIS_REQUIRE(counts_out_dev && row_start_out, "counts_out_dev / row_start_out must not be NULL");
@@ -825,6 +841,7 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   if (n == 0) {
     plan_empty_kernel<<<1, 64, 0, stream>>>(counts_out_dev, row_start_out);
     RECIS_LAUNCH_CHECK();
+    if (unique_count_host) *unique_count_host = 0;
     return RECIS_OK;
   }
   PlanGeom g;
@@ -897,6 +914,15 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   }
   plan_scan_kernel<<<1, 1024, 0, stream>>>(ucnt, ubase, ocnt, lbase, static_cast<int>(nb), counts_out_dev);
   RECIS_LAUNCH_CHECK();
+  // The count is final here: send it to the host now and wait for it only after the emit kernels
+  // are queued, so that the GPU works while the host learns the size of the next launches.
+  int64_t* staged = nullptr;
+  hipEvent_t staged_event = nullptr;
+  if (unique_count_host) {
+    if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
+    RECIS_CHECK_HIP(hipMemcpyAsync(staged, counts_out_dev, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+    RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
+  }
   {
     RECIS_TIME_KERNEL("plan_emit_occ_kernel", stream)
     plan_emit_occ_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(
@@ -910,6 +936,10 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
         bucket_uniq, bucket_start, ubase, lbase, g, unique_out, row_start_out, counts_out_dev, hot_items_out,
         hot_cap);
     RECIS_LAUNCH_CHECK();
+  }
+  if (unique_count_host) {
+    RECIS_CHECK_HIP(hipEventSynchronize(staged_event));
+    *unique_count_host = *staged;
   }
   return RECIS_OK;
 }
@@ -956,7 +986,8 @@ int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_feat
 int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
                             int coef_dtype, const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
                             const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t D,
-                            int accumulate, void* stream_) {
+                            int accumulate, const void* cover_offsets, int cover_is64, int64_t cover_S,
+                            void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   RECIS_REQUIRE(U >= 0 && n_rows >= 0, "negative size");
   RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
@@ -979,6 +1010,9 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   a.coef_dt = coef_dtype;
   a.U = U;
   a.n_rows = n_rows;
+  a.cover = cover_offsets;
+  a.cover64 = cover_is64;
+  a.cover_S = cover_S;
   a.D = static_cast<int>(D);
   a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
   a.accumulate = accumulate;

@@ -78,6 +78,25 @@ int get_workspace(hipStream_t stream, size_t bytes, void** out) {
   return RECIS_OK;
 }
 
+struct CountStaging {
+  int64_t* host = nullptr;  // pinned
+  hipEvent_t event = nullptr;
+};
+static std::map<std::pair<int, hipStream_t>, CountStaging> g_staging;
+
+int get_count_staging(hipStream_t stream, int64_t** host, hipEvent_t* event) {
+  int dev = current_device();
+  std::lock_guard<std::mutex> l(g_mu);
+  CountStaging& c = g_staging[std::make_pair(dev, stream)];
+  if (c.host == nullptr) {
+    RECIS_CHECK_HIP(hipHostMalloc(reinterpret_cast<void**>(&c.host), 64, hipHostMallocDefault));
+    RECIS_CHECK_HIP(hipEventCreateWithFlags(&c.event, hipEventDisableTiming));
+  }
+  *host = c.host;
+  *event = c.event;
+  return RECIS_OK;
+}
+
 bool g_profile_on = false;
 
 struct TimedLaunch {

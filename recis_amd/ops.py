@@ -711,14 +711,16 @@ def ids_unique_plan(ids):
     p.hot_items = torch.empty(2 * p.hot_cap, dtype=torch.int32, device=dev)
     p.counts = torch.empty(2, dtype=torch.int64, device=dev)
     p._pool_fill = None
+    count = ctypes.c_int64(0)
     check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(uniq), ptr(p.inverse), ptr(p.row_start), ptr(p.occ),
-                                  ptr(p.pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts), stream_ptr(dev)))
-    p.U = int(p.counts[0].item())
+                                  ptr(p.pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts), ctypes.byref(count),
+                                  stream_ptr(dev)))
+    p.U = int(count.value)
     p.unique = uniq[: p.U]
     return p
 
 
-def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False):
+def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False, cover=None):
     """``out[u] (+)= sum_k coef[k] * rows[src[k]]`` over the list of every unique id of
     ``plan``; returns the fp32 ``[U, D]`` result."""
     require_cuda(rows, src, coef)
@@ -731,6 +733,8 @@ def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False):
                                         dtype_code(coef.dtype) if coef is not None else 0, ptr(plan.row_start),
                                         ptr(plan.hot_items), i64(plan.hot_cap), ptr(plan.counts), ptr(out),
                                         dtype_code(out.dtype), i64(plan.U), i64(D), int(bool(accumulate)),
+                                        ptr(cover), _index_kind(cover, "offsets") if cover is not None else 0,
+                                        i64(cover.numel() - 1 if cover is not None else 0),
                                         stream_ptr(rows.device)))
     return out
 
@@ -745,10 +749,8 @@ def segment_reduce_backward_plan(grad_output, weight, offsets, plan, mode, out=N
     if mode == "tile":
         src = plan.occ
         coef = None if weight is None else gather(plan.occ, weight.view(-1, 1)).view(-1)
-        lo, hi = offsets[0], offsets[-1]
-        if offsets.numel() and (int(lo) != 0 or int(hi) != plan.n):  # rare: occurrences no segment covers
-            cov = ((plan.occ >= lo) & (plan.occ < hi)).float()
-            coef = cov if coef is None else coef.float() * cov
-    else:
-        src, coef = plan.src_coef_for_pool(offsets, weight, mode == "mean")
+        # occurrences no segment covers are skipped by the kernel (no host read of the offsets)
+        return csr_gather_reduce(grad_output, plan, src, coef, out=out, accumulate=accumulate,
+                                 cover=offsets if offsets.numel() else None)
+    src, coef = plan.src_coef_for_pool(offsets, weight, mode == "mean")
     return csr_gather_reduce(grad_output, plan, src, coef, out=out, accumulate=accumulate)

@@ -275,6 +275,23 @@ def test_planned_backward_matches_oracle(rng, mode, D, dtype):
     assert _lib.poll_device_errors() == 0
 
 
+def test_planned_tile_backward_partial_cover(rng):
+    """TILE backward through the plan when the offsets cover only part of the occurrences: the rest
+    contributes nothing (checked on the device, no host read of the offsets)."""
+    N, D = 5000, 8
+    ids = rng.integers(0, 300, size=N)
+    p = ops.ids_unique_plan(_dev(ids))
+    inv = p.inverse.cpu().numpy().astype(np.int64)
+    g = rng.standard_normal((N, D)).astype(np.float32)
+    off = np.array([700, 900, 900, 4100], dtype=np.int32)
+    got = ops.segment_reduce_backward_plan(_dev(g), None, _dev(off), p, "tile").cpu().numpy()
+    exp = np.zeros((p.U, D), np.float64)
+    np.add.at(exp, inv[700:4100], g[700:4100])
+    np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-4)
+    np.testing.assert_allclose(got, oracle.segment_reduce_backward(g, None, inv, off, p.U, "tile"), rtol=1e-5, atol=1e-4)
+    assert _lib.poll_device_errors() == 0
+
+
 def test_planned_tile_backward_matches_oracle(rng):
     batch, seq = [50, 31, 7], [12, 3, 40]
     D = 32
