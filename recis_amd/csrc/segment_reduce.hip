@@ -67,7 +67,14 @@ __device__ __forceinline__ bool team_segment(const SegArgs& a, int64_t* s_off,
 }
 
 // ------------------------------------------------------------------ forward
-template <typename TIn, typename TOut, int VEC>
+// KIND selects what a row fetch has to do, so that the common cases keep few registers live
+// (the kernel is bound by the number of waves a CU can hold):
+//   kFwdGeneric   weights and/or 64-bit reverse indices, all checked at run time
+//   kFwdPlain     no reverse indices, no weights: rows of a segment are contiguous in emb
+//   kFwdRev32     int32 reverse indices, no weights
+enum { kFwdGeneric = 0, kFwdPlain = 1, kFwdRev32 = 2 };
+
+template <typename TIn, typename TOut, int VEC, int KIND>
 __global__ void __launch_bounds__(kBlock)
 seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
   __shared__ int64_t s_off[kBlock + 1];
@@ -77,14 +84,23 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
   const int lane_t = threadIdx.x & ((1 << a.team_log2) - 1);
   const int rg = lane_t >> a.lpr_log2;
   const int cl = lane_t & ((1 << a.lpr_log2) - 1);
-  const int64_t step = int64_t(1) << (a.team_log2 - a.lpr_log2);
+  const int step = 1 << (a.team_log2 - a.lpr_log2);
   const int col_stride = VEC << a.lpr_log2;
   const int D = a.D;
   const float scale = (a.mean && end > start) ? 1.0f / static_cast<float>(end - start) : 1.0f;
 
   auto fetch = [&](int64_t r, int c0, float (&v)[VEC], float& w) {
-    int64_t idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
-    w = a.weight ? load_weight(a.weight, a.wdt, r) : 1.0f;
+    int64_t idx;
+    if constexpr (KIND == kFwdPlain) {
+      idx = r;
+      w = 1.0f;
+    } else if constexpr (KIND == kFwdRev32) {
+      idx = static_cast<const int32_t*>(a.rev)[r];
+      w = 1.0f;
+    } else {
+      idx = a.rev ? load_index(a.rev, a.rev64, r) : r;
+      w = a.weight ? load_weight(a.weight, a.wdt, r) : 1.0f;
+    }
     if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
       raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
 #pragma unroll
@@ -93,6 +109,16 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
       return;
     }
     load_pack<TIn, VEC>(emb + idx * D + c0, v);
+  };
+  auto add = [&](float (&acc)[VEC], const float (&v)[VEC], float w) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      if constexpr (KIND == kFwdGeneric) {
+        acc[j] = fmaf(v[j], w, acc[j]);
+      } else {
+        acc[j] = fmaf(v[j], w, acc[j]);  // w is 1 or 0 here; same rounding as the generic path
+      }
+    }
   };
 
   for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
@@ -108,20 +134,16 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
       fetch(r + step, c0, v1, w1);
       fetch(r + 2 * step, c0, v2, w2);
       fetch(r + 3 * step, c0, v3, w3);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        acc[j] = fmaf(v0[j], w0, acc[j]);
-        acc[j] = fmaf(v1[j], w1, acc[j]);
-        acc[j] = fmaf(v2[j], w2, acc[j]);
-        acc[j] = fmaf(v3[j], w3, acc[j]);
-      }
+      add(acc, v0, w0);
+      add(acc, v1, w1);
+      add(acc, v2, w2);
+      add(acc, v3, w3);
     }
     for (; r < end; r += step) {
       float v0[VEC];
       float w0;
       fetch(r, c0, v0, w0);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v0[j], w0, acc[j]);
+      add(acc, v0, w0);
     }
     // combine the row groups of the team (partners share cl, hence c0)
     for (int off = 1 << a.lpr_log2; off < (1 << a.team_log2); off <<= 1) {
@@ -519,9 +541,15 @@ extern "C" int recis_segment_reduce_forward(
             seg_max_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
                 static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), argmax_out, a);
           } else {
+            const TIn* e = static_cast<const TIn*>(unique_emb);
+            TOut* o = static_cast<TOut*>(out);
             RECIS_TIME_KERNEL("seg_pool_fwd_kernel", stream)
-            seg_pool_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
-                static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), a);
+            if (a.weight == nullptr && a.rev == nullptr)
+              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+            else if (a.weight == nullptr && !a.rev64)
+              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+            else
+              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdGeneric><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
           }
         }
         RECIS_LAUNCH_CHECK();
