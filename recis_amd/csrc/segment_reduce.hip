@@ -158,6 +158,99 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
   }
 }
 
+// Unweighted pooling of segments of several rows, built to keep many bytes in flight per wave: the
+// kernel is bound by memory latency x resident waves, so
+//   * the two offsets of a segment are read directly (no LDS staging, no barrier)
+//   * the reverse indices of up to TEAM rows are read by ONE coalesced load (a lane each) and
+//     handed to the lanes that need them with shuffles, instead of one dependent load per row
+//   * every lane then has up to eight independent row loads in flight
+// Rows are summed per row group in increasing order, like the generic kernel. Requires U < 2^31.
+enum { kFastPlain = 0, kFastRev32 = 1, kFastRev64 = 2 };
+
+template <typename TIn, typename TOut, int VEC, int KIND>
+__global__ void __launch_bounds__(kBlock)
+seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
+  const int64_t s = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.team_log2) + (threadIdx.x >> a.team_log2);
+  if (s >= a.S) return;  // whole teams leave together
+  int64_t start = load_index(a.offs, a.off64, s);
+  int64_t end = load_index(a.offs, a.off64, s + 1);
+  if (start < 0 || end > a.B || end < start) {
+    raise_device_error(a.err, RECIS_DEVERR_OFFSETS);
+    start = end = 0;
+  }
+  const int team = 1 << a.team_log2;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int lane_t = lane & (team - 1);
+  const int team_lane0 = lane - lane_t;
+  const int rg = lane_t >> a.lpr_log2;
+  const int cl = lane_t & ((1 << a.lpr_log2) - 1);
+  const int step = team >> a.lpr_log2;
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+  const float scale = (a.mean && end > start) ? 1.0f / static_cast<float>(end - start) : 1.0f;
+
+  for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
+    const int c0 = cbase + cl * VEC;
+    const bool col_ok = c0 < D;
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    for (int64_t base = start; base < end; base += team) {
+      const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
+      int32_t mine = -1;  // row of occurrence base + lane_t
+      if (lane_t < n_here) {
+        int64_t idx;
+        if constexpr (KIND == kFastPlain) {
+          idx = base + lane_t;
+        } else if constexpr (KIND == kFastRev32) {
+          idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
+        } else {
+          idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
+        }
+        if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        } else {
+          mine = static_cast<int32_t>(idx);
+        }
+      }
+      for (int q0 = 0; q0 < n_here; q0 += 8 * step) {  // same trip count for the whole team (shuffles inside)
+        const int q = q0 + rg;
+        float v[8][VEC];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const int src = q + k * step;
+          int32_t id = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
+          if (src >= n_here || !col_ok) id = -1;
+          if (id >= 0) {
+            if constexpr (KIND == kFastPlain) {
+              load_pack_stream<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);  // read once
+            } else {
+              load_pack<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[k][j] = 0.f;
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) acc[j] += v[k][j];
+        }
+      }
+    }
+    for (int off = 1 << a.lpr_log2; off < team; off <<= 1) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+    }
+    if (rg == 0 && col_ok) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] *= scale;
+      store_pack<TOut, VEC>(out + s * D + c0, acc);
+    }
+  }
+}
+
 // MAX combiner: element-wise maximum and the occurrence that produced it.
 // Value and occurrence travel as one 64-bit key: the high word is the float
 // mapped to an order-preserving unsigned integer (any NaN maps to the top, so it
@@ -543,8 +636,16 @@ extern "C" int recis_segment_reduce_forward(
           } else {
             const TIn* e = static_cast<const TIn*>(unique_emb);
             TOut* o = static_cast<TOut*>(out);
+            // several rows per segment: the latency-oriented kernel; about one row: the lean one
+            const bool fast = a.weight == nullptr && U < (int64_t(1) << 31) && a.team_log2 > a.lpr_log2;
             RECIS_TIME_KERNEL("seg_pool_fwd_kernel", stream)
-            if (a.weight == nullptr && a.rev == nullptr)
+            if (fast && a.rev == nullptr)
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+            else if (fast && !a.rev64)
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+            else if (fast)
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev64><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+            else if (a.weight == nullptr && a.rev == nullptr)
               seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
             else if (a.weight == nullptr && !a.rev64)
               seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
