@@ -375,6 +375,82 @@ fill_zero_rows_kernel(TOut* __restrict__ p, int64_t n_packs) {
 }
 
 // SUM / MEAN backward, segment-major. ATOMIC=false writes each touched row once.
+// Unweighted backward onto distinct rows (no atomics): the pooled gradient row of a segment is
+// read once and stored to every row of the segment. As in the forward, the reverse indices of
+// up to TEAM rows come from one coalesced load and travel by shuffles, so the stores of a lane
+// follow each other without a dependent index load in between. Requires U < 2^31.
+template <typename TG, typename TOut, int VEC, int KIND>
+__global__ void __launch_bounds__(kBlock)
+seg_pool_bwd_fast_kernel(const TG* __restrict__ grad_out, TOut* __restrict__ grad_unique, SegArgs a) {
+  const int64_t s = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.team_log2) + (threadIdx.x >> a.team_log2);
+  if (s >= a.S) return;  // whole teams leave together
+  int64_t start = load_index(a.offs, a.off64, s);
+  int64_t end = load_index(a.offs, a.off64, s + 1);
+  if (start < 0 || end > a.B || end < start) {
+    raise_device_error(a.err, RECIS_DEVERR_OFFSETS);
+    start = end = 0;
+  }
+  const int team = 1 << a.team_log2;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int lane_t = lane & (team - 1);
+  const int team_lane0 = lane - lane_t;
+  const int rg = lane_t >> a.lpr_log2;
+  const int cl = lane_t & ((1 << a.lpr_log2) - 1);
+  const int step = team >> a.lpr_log2;
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+  const float scale = (a.mean && end > start) ? 1.0f / static_cast<float>(end - start) : 1.0f;
+
+  for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
+    const int c0 = cbase + cl * VEC;
+    const bool col_ok = c0 < D;
+    float g[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) g[j] = 0.f;
+    if (col_ok) load_pack<TG, VEC>(grad_out + s * D + c0, g);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) g[j] *= scale;
+    for (int64_t base = start; base < end; base += team) {
+      const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
+      int32_t mine = -1;  // row of occurrence base + lane_t
+      if (lane_t < n_here) {
+        int64_t idx;
+        if constexpr (KIND == kFastPlain) {
+          idx = base + lane_t;
+        } else if constexpr (KIND == kFastRev32) {
+          idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
+        } else {
+          idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
+        }
+        if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        } else {
+          mine = static_cast<int32_t>(idx);
+        }
+      }
+      for (int q0 = 0; q0 < n_here; q0 += 4 * step) {  // same trip count for the whole team
+        int32_t id[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int src = q0 + rg + k * step;
+          id[k] = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
+          if (src >= n_here || !col_ok) id[k] = -1;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (id[k] >= 0) {
+            if constexpr (KIND == kFastPlain) {
+              store_pack_stream<TOut, VEC>(grad_unique + static_cast<int64_t>(id[k]) * D + c0, g);
+            } else {
+              store_pack<TOut, VEC>(grad_unique + static_cast<int64_t>(id[k]) * D + c0, g);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
 template <typename TG, typename TOut, int VEC, bool ATOMIC>
 __global__ void __launch_bounds__(kBlock)
 seg_pool_bwd_kernel(const TG* __restrict__ grad_out, TOut* __restrict__ grad_unique, SegArgs a) {
@@ -761,7 +837,18 @@ extern "C" int recis_segment_reduce_backward(
         } else if (S > 0) {
           const int teams_per_block = kBlock >> a.team_log2;
           const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
-          if (unique)
+          const TG* gsrc = static_cast<const TG*>(grad_out);
+          TOut* gdst = static_cast<TOut*>(grad_unique);
+          const bool fast = unique && a.weight == nullptr && U < (int64_t(1) << 31) && a.team_log2 > a.lpr_log2;
+          if (fast) {
+            RECIS_TIME_KERNEL("seg_pool_bwd_kernel", stream)
+            if (a.rev == nullptr)
+              seg_pool_bwd_fast_kernel<TG, TOut, VEC, kFastPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(gsrc, gdst, a);
+            else if (!a.rev64)
+              seg_pool_bwd_fast_kernel<TG, TOut, VEC, kFastRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(gsrc, gdst, a);
+            else
+              seg_pool_bwd_fast_kernel<TG, TOut, VEC, kFastRev64><<<dim3(grid), dim3(kBlock), 0, stream>>>(gsrc, gdst, a);
+          } else if (unique)
             RECIS_TIME_KERNEL("seg_pool_bwd_kernel", stream)
             seg_pool_bwd_kernel<TG, TOut, VEC, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(
                 static_cast<const TG*>(grad_out), static_cast<TOut*>(grad_unique), a);
