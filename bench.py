@@ -103,7 +103,19 @@ class Config2:
             "seg_pool_bwd_kernel(sum)": (lambda: o.segment_reduce_backward(self.grad, None, self.rev, self.off,
                                                                           self.N, "sum", rev_unique=True),
                                          self.pass_bytes),
+            "seg_max_fwd_kernel": (lambda: o.segment_reduce_forward(self.emb, None, self.rev, self.off, "max",
+                                                                    return_argmax=True),
+                                   self.pass_bytes + self.S * self.D * 4),
+            "seg_max_bwd_kernel": (lambda: o.segment_reduce_backward(self.grad, None, self.rev, self.off, self.N,
+                                                                     "max", argmax=self._argmax(), rev_unique=True),
+                                   self.pass_bytes + self.S * self.D * 4),
         }
+
+    def _argmax(self):
+        if getattr(self, "_arg", None) is None:
+            _, self._arg = self.ops.segment_reduce_forward(self.emb, None, self.rev, self.off, "max",
+                                                           return_argmax=True)
+        return self._arg
 
     def cpu_baseline(self, budget_s):
         import oracle

@@ -324,6 +324,100 @@ seg_max_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out,
   }
 }
 
+// MAX forward with the memory behaviour of seg_pool_fwd_fast_kernel (indices by one coalesced
+// load + shuffles, four row loads in flight per lane). Requires U < 2^31.
+template <typename TIn, typename TOut, int VEC, int KIND>
+__global__ void __launch_bounds__(kBlock)
+seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int32_t* __restrict__ argmax,
+                        SegArgs a) {
+  const int64_t s = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.team_log2) + (threadIdx.x >> a.team_log2);
+  if (s >= a.S) return;  // whole teams leave together
+  int64_t start = load_index(a.offs, a.off64, s);
+  int64_t end = load_index(a.offs, a.off64, s + 1);
+  if (start < 0 || end > a.B || end < start) {
+    raise_device_error(a.err, RECIS_DEVERR_OFFSETS);
+    start = end = 0;
+  }
+  const int team = 1 << a.team_log2;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int lane_t = lane & (team - 1);
+  const int team_lane0 = lane - lane_t;
+  const int rg = lane_t >> a.lpr_log2;
+  const int cl = lane_t & ((1 << a.lpr_log2) - 1);
+  const int step = team >> a.lpr_log2;
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+
+  for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
+    const int c0 = cbase + cl * VEC;
+    const bool col_ok = c0 < D;
+    uint64_t key[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) key[j] = 0;
+    for (int64_t base = start; base < end; base += team) {
+      const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
+      int32_t mine = -1;  // row of occurrence base + lane_t
+      if (lane_t < n_here) {
+        int64_t idx;
+        if constexpr (KIND == kFastPlain) {
+          idx = base + lane_t;
+        } else if constexpr (KIND == kFastRev32) {
+          idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
+        } else {
+          idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
+        }
+        if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        } else {
+          mine = static_cast<int32_t>(idx);
+        }
+      }
+      for (int q0 = 0; q0 < n_here; q0 += 4 * step) {  // same trip count for the whole team
+        float v[4][VEC];
+        bool have[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int src = q0 + rg + k * step;
+          const int32_t id = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
+          have[k] = src < n_here && col_ok && id >= 0;
+          if (have[k]) load_pack<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (!have[k]) continue;
+          const int64_t r = base + q0 + rg + k * step;
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const uint64_t kk = max_key(v[k][j], r);
+            key[j] = kk > key[j] ? kk : key[j];
+          }
+        }
+      }
+    }
+    for (int off = 1 << a.lpr_log2; off < team; off <<= 1) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        uint32_t lo = __shfl_xor(static_cast<uint32_t>(key[j]), off, kWave);
+        uint32_t hi = __shfl_xor(static_cast<uint32_t>(key[j] >> 32), off, kWave);
+        uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
+        key[j] = other > key[j] ? other : key[j];
+      }
+    }
+    if (rg == 0 && col_ok) {
+      float best[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) best[j] = key[j] ? max_key_value(key[j]) : 0.f;
+      store_pack<TOut, VEC>(out + s * D + c0, best);
+      if (argmax) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+          argmax[s * D + c0 + j] =
+              key[j] ? static_cast<int32_t>(0xFFFFFFFFu - static_cast<uint32_t>(key[j])) : -1;
+      }
+    }
+  }
+}
+
 // TILE combiner forward: one row group per occurrence, out[i] = w_i * emb[rev_i];
 // occurrences outside [offsets[0], offsets[S]) produce zero rows.
 template <typename TIn, typename TOut, int VEC>
@@ -562,6 +656,87 @@ seg_tile_bwd_kernel(const TG* __restrict__ grad_out, TOut* __restrict__ grad_uni
 
 // MAX backward: route each pooled-gradient element to the winning occurrence.
 // grad_unique is zero-filled by the caller. One thread per (segment, column).
+// MAX backward onto distinct rows that are all reached (a bijection between occurrences and
+// rows): segment-major, every row of the segment is written in full -- the gradient where the
+// row won the column, zero elsewhere -- so no zero fill of the output and no scatter are needed.
+// Requires U < 2^31.
+template <typename TG, typename TOut, int VEC, int KIND>
+__global__ void __launch_bounds__(kBlock)
+seg_max_bwd_rows_kernel(const TG* __restrict__ grad_out, const int32_t* __restrict__ argmax,
+                        TOut* __restrict__ grad_unique, SegArgs a) {
+  const int64_t s = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.team_log2) + (threadIdx.x >> a.team_log2);
+  if (s >= a.S) return;  // whole teams leave together
+  int64_t start = load_index(a.offs, a.off64, s);
+  int64_t end = load_index(a.offs, a.off64, s + 1);
+  if (start < 0 || end > a.B || end < start) {
+    raise_device_error(a.err, RECIS_DEVERR_OFFSETS);
+    start = end = 0;
+  }
+  const int team = 1 << a.team_log2;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int lane_t = lane & (team - 1);
+  const int team_lane0 = lane - lane_t;
+  const int rg = lane_t >> a.lpr_log2;
+  const int cl = lane_t & ((1 << a.lpr_log2) - 1);
+  const int step = team >> a.lpr_log2;
+  const int col_stride = VEC << a.lpr_log2;
+  const int D = a.D;
+
+  for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
+    const int c0 = cbase + cl * VEC;
+    const bool col_ok = c0 < D;
+    float g[VEC];
+    int32_t win[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      g[j] = 0.f;
+      win[j] = -1;
+    }
+    if (col_ok) {
+      load_pack<TG, VEC>(grad_out + s * D + c0, g);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) win[j] = argmax[s * D + c0 + j];
+    }
+    for (int64_t base = start; base < end; base += team) {
+      const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
+      int32_t mine = -1;  // row of occurrence base + lane_t
+      if (lane_t < n_here) {
+        int64_t idx;
+        if constexpr (KIND == kFastPlain) {
+          idx = base + lane_t;
+        } else if constexpr (KIND == kFastRev32) {
+          idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
+        } else {
+          idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
+        }
+        if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        } else {
+          mine = static_cast<int32_t>(idx);
+        }
+      }
+      for (int q0 = 0; q0 < n_here; q0 += 4 * step) {  // same trip count for the whole team
+        int32_t id[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int src = q0 + rg + k * step;
+          id[k] = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
+          if (src >= n_here || !col_ok) id[k] = -1;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (id[k] < 0) continue;
+          const int32_t r = static_cast<int32_t>(base) + q0 + rg + k * step;
+          float v[VEC];
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[j] = win[j] == r ? g[j] : 0.f;
+          store_pack<TOut, VEC>(grad_unique + static_cast<int64_t>(id[k]) * D + c0, v);
+        }
+      }
+    }
+  }
+}
+
 template <typename TG, typename TOut, bool ATOMIC>
 __global__ void __launch_bounds__(kBlock)
 seg_max_bwd_kernel(const TG* __restrict__ grad_out, const int32_t* __restrict__ argmax,
@@ -706,9 +881,17 @@ extern "C" int recis_segment_reduce_forward(
           const int teams_per_block = kBlock >> a.team_log2;
           const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
           if (mode == RECIS_MAX) {
+            const TIn* e = static_cast<const TIn*>(unique_emb);
+            TOut* o = static_cast<TOut*>(out);
             RECIS_TIME_KERNEL("seg_max_fwd_kernel", stream)
-            seg_max_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
-                static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), argmax_out, a);
+            if (U >= (int64_t(1) << 31))
+              seg_max_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, argmax_out, a);
+            else if (a.rev == nullptr)
+              seg_max_fwd_fast_kernel<TIn, TOut, VEC, kFastPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, argmax_out, a);
+            else if (!a.rev64)
+              seg_max_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, argmax_out, a);
+            else
+              seg_max_fwd_fast_kernel<TIn, TOut, VEC, kFastRev64><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, argmax_out, a);
           } else {
             const TIn* e = static_cast<const TIn*>(unique_emb);
             TOut* o = static_cast<TOut*>(out);
@@ -788,7 +971,8 @@ extern "C" int recis_segment_reduce_backward(
   // Rows no occurrence maps to must read zero. With a promised bijection
   // (unique and U == B) every row is reached through its occurrence, so only
   // occurrences outside the offsets range need clearing; otherwise clear all.
-  const bool bijection = unique && U == B && mode != RECIS_MAX;
+  const bool max_rows = mode == RECIS_MAX && unique && U == B && U < (int64_t(1) << 31) && B < (int64_t(1) << 31);
+  const bool bijection = unique && U == B && (mode != RECIS_MAX || max_rows);
 
   return dispatch_types(grad_dtype, out_dtype, [&](auto tin, auto tout) {
     using TG = decltype(tin);
@@ -805,12 +989,27 @@ extern "C" int recis_segment_reduce_backward(
           fill_zero_rows_kernel<TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
               static_cast<TOut*>(grad_unique), n_packs);
           RECIS_LAUNCH_CHECK();
-        } else if (mode != RECIS_TILE) {
+        } else if (mode != RECIS_TILE) {  // bijection: only occurrences outside the offsets range need clearing
           seg_bwd_zero_uncovered_kernel<TOut, VEC><<<dim3(64), dim3(kBlock), 0, stream>>>(
               static_cast<TOut*>(grad_unique), a);
           RECIS_LAUNCH_CHECK();
         }
-        if (mode == RECIS_MAX) {
+        if (max_rows) {
+          if (S > 0) {
+            const int teams_per_block = kBlock >> a.team_log2;
+            const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
+            const TG* gsrc = static_cast<const TG*>(grad_out);
+            TOut* gdst = static_cast<TOut*>(grad_unique);
+            RECIS_TIME_KERNEL("seg_max_bwd_kernel", stream)
+            if (a.rev == nullptr)
+              seg_max_bwd_rows_kernel<TG, TOut, VEC, kFastPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(gsrc, argmax, gdst, a);
+            else if (!a.rev64)
+              seg_max_bwd_rows_kernel<TG, TOut, VEC, kFastRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(gsrc, argmax, gdst, a);
+            else
+              seg_max_bwd_rows_kernel<TG, TOut, VEC, kFastRev64><<<dim3(grid), dim3(kBlock), 0, stream>>>(gsrc, argmax, gdst, a);
+            RECIS_LAUNCH_CHECK();
+          }
+        } else if (mode == RECIS_MAX) {
           const int64_t total = S * D;
           if (total > 0) {
             int64_t grid = std::min<int64_t>((total + kBlock - 1) / kBlock, 256 * 64);
