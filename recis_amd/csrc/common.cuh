@@ -179,6 +179,14 @@ inline int pick_vec_bytes(int64_t row_bytes, uintptr_t align_or) {
   return vb;
 }
 
+// The same with a caller-chosen upper limit (fp32 rows written by kernels whose inputs are
+// 2-byte types go out as 32-byte packs, two 16-byte stores per lane).
+inline int pick_vec_bytes_max(int64_t row_bytes, uintptr_t align_or, int max_bytes) {
+  int vb = max_bytes;
+  while (vb > 1 && ((row_bytes % vb) != 0 || (align_or % vb) != 0)) vb >>= 1;
+  return vb;
+}
+
 inline RowGeom make_row_geom(int64_t D, int esize, int vec_bytes) {
   RowGeom g;
   g.vec = vec_bytes / esize;

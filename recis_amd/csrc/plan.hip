@@ -570,13 +570,66 @@ __device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64
   }
 }
 
+// A whole wave works the list entries [e_begin, e_end) (uniform arguments, every lane calls):
+// `src` and `coef` of 64 entries come from one coalesced load, a lane each, and reach the lanes
+// that gather the rows through shuffles; lane group g of `groups` takes entries g, g + groups,
+// ... with several row loads in flight. acc: this group's partial sum for columns
+// c0 .. c0 + VEC (the caller folds the groups).
+template <typename TIn, int VEC>
+__device__ __forceinline__ void wave_gather_range(const TIn* __restrict__ rows, const CsrArgs& a, int64_t c_lo,
+                                                  int64_t c_hi, int32_t e_begin, int32_t e_end, int c0, bool col_ok,
+                                                  int g, int groups, float (&acc)[VEC]) {
+  constexpr int kFly = VEC >= 8 ? 4 : 8;  // row loads in flight per lane
+  const int lane = threadIdx.x & (kWave - 1);
+  for (int32_t cb = e_begin; cb < e_end; cb += kWave) {
+    const int n_here = min(kWave, e_end - cb);
+    int32_t s_mine = -1;
+    float w_mine = 0.f;
+    if (lane < n_here) {
+      const int32_t sv = a.src[cb + lane];
+      if (sv >= c_lo && sv < c_hi) {
+        s_mine = sv;
+        w_mine = a.coef ? load_coef(a.coef, a.coef_dt, cb + lane) : 1.0f;
+      } else if (static_cast<int64_t>(sv) >= a.n_rows) {
+        raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      }
+    }
+    for (int q0 = 0; q0 < n_here; q0 += kFly * groups) {  // same trip count for the whole wave (shuffles inside)
+      float v[kFly][VEC];
+      float w[kFly];
+#pragma unroll
+      for (int k = 0; k < kFly; ++k) {
+        const int e = q0 + g + k * groups;
+        const int from = min(e, kWave - 1);
+        int32_t id = __shfl(s_mine, from, kWave);
+        w[k] = a.coef ? __shfl(w_mine, from, kWave) : 1.0f;
+        if (e >= n_here || !col_ok) id = -1;
+        if (id >= 0) {
+          load_pack<TIn, VEC>(rows + static_cast<int64_t>(id) * a.D + c0, v[k]);
+        } else {
+          w[k] = 0.f;
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[k][j] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kFly; ++k) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[k][j], w[k], acc[j]);
+      }
+    }
+  }
+}
+
 // One group of LPR lanes per unique row (cold rows); hot rows are cleared here and summed by
 // csr_hot_kernel. A wave that holds a row with more than kCoopLen occurrences switches, as a
 // whole, to working its rows one after the other with all its lane groups striding over the
 // row's list (a row of 200 occurrences would otherwise be 50 dependent gathers of one group).
 constexpr int kCoopLen = 8;
 
-template <typename TIn, typename TOut, int VEC>
+// SHUFFLE: long rows go through wave_gather_range (pays off when a wave has at most eight lane
+// groups, i.e. rows of 128 bytes and more); otherwise every group loads its own entries.
+template <typename TIn, typename TOut, int VEC, bool SHUFFLE>
 __global__ void __launch_bounds__(kBlock)
 csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a) {
   const int rows_per_block = kBlock >> a.lpr_log2;
@@ -663,23 +716,29 @@ csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
     const int r = owner >> a.lpr_log2;
     const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
     const int64_t row = u - g + r;  // rows of a wave are consecutive
-    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+      const int c0 = cbase + cl * VEC;
+      const bool col_ok = c0 < D;
       float acc[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      gather_sum(r_start + g, r_end, groups, c0, acc);
+      if constexpr (SHUFFLE) {
+        wave_gather_range<TIn, VEC>(rows, a, c_lo, c_hi, r_start, r_end, c0, col_ok, g, groups, acc);
+      } else {
+        if (col_ok) gather_sum(r_start + g, r_end, groups, c0, acc);
+      }
       for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
       }
-      if (g == r) finish(row, false, c0, acc);
+      if (g == r && col_ok) finish(row, false, c0, acc);
     }
   }
 }
 
 // One workgroup per (hot row, chunk): row groups stride over the chunk, partial sums are
 // combined through LDS and added to the (cleared) output row with a handful of atomics.
-template <typename TIn, int VEC>
+template <typename TIn, int VEC, bool SHUFFLE>
 __global__ void __launch_bounds__(kPlanBlock)
 csr_hot_kernel(const TIn* __restrict__ rows, float* __restrict__ out, CsrArgs a,
                const int32_t* __restrict__ hot_items, const int64_t* __restrict__ counts, int64_t hot_cap) {
@@ -689,8 +748,8 @@ csr_hot_kernel(const TIn* __restrict__ rows, float* __restrict__ out, CsrArgs a,
   int64_t n_items = counts[1];
   if (n_items > hot_cap) n_items = hot_cap;
   const int D = a.D;
-  const int groups = kPlanBlock >> a.lpr_log2;
-  const int g = threadIdx.x >> a.lpr_log2;
+  const int groups_w = kWave >> a.lpr_log2;                      // lane groups of a wave
+  const int gw = (threadIdx.x & (kWave - 1)) >> a.lpr_log2;      // this lane's group in its wave
   const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
   const int wave = threadIdx.x / kWave;
   constexpr int n_waves = kPlanBlock / kWave;
@@ -699,50 +758,59 @@ csr_hot_kernel(const TIn* __restrict__ rows, float* __restrict__ out, CsrArgs a,
     const int32_t chunk = hot_items[2 * item + 1];
     const int32_t start = a.row_start[u] + chunk * kHotChunk;
     const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
-    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+    // each wave takes a contiguous share of the chunk
+    const int32_t per_wave = (end - start + n_waves - 1) / n_waves;
+    const int32_t w_begin = min(end, start + wave * per_wave), w_end = min(end, w_begin + per_wave);
+    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+      const int c0 = cbase + cl * VEC;
+      const bool col_ok = c0 < D;
       float acc[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      auto fetch = [&](int32_t k, float (&v)[VEC], float& w) {
-        const int32_t s = a.src[k];
-        w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
-        if (s < c_lo || s >= c_hi) {
+      if constexpr (SHUFFLE) {
+        wave_gather_range<TIn, VEC>(rows, a, c_lo, c_hi, w_begin, w_end, c0, col_ok, gw, groups_w, acc);
+      } else if (col_ok) {
+        auto fetch = [&](int32_t k, float (&v)[VEC], float& w) {
+          const int32_t s = a.src[k];
+          w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
+          if (s < c_lo || s >= c_hi) {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) v[j] = 0.f;
-          w = 0.f;
-          return;
+            for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+            w = 0.f;
+            return;
+          }
+          load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
+        };
+        int32_t k = w_begin + gw;
+        for (; k + 3 * groups_w < w_end; k += 4 * groups_w) {  // four gathers in flight per lane
+          float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
+          float w0, w1, w2, w3;
+          fetch(k, v0, w0);
+          fetch(k + groups_w, v1, w1);
+          fetch(k + 2 * groups_w, v2, w2);
+          fetch(k + 3 * groups_w, v3, w3);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            acc[j] = fmaf(v0[j], w0, acc[j]);
+            acc[j] = fmaf(v1[j], w1, acc[j]);
+            acc[j] = fmaf(v2[j], w2, acc[j]);
+            acc[j] = fmaf(v3[j], w3, acc[j]);
+          }
         }
-        load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
-      };
-      int32_t k = start + g;
-      for (; k + 3 * groups < end; k += 4 * groups) {  // four gathers in flight per lane
-        float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
-        float w0, w1, w2, w3;
-        fetch(k, v0, w0);
-        fetch(k + groups, v1, w1);
-        fetch(k + 2 * groups, v2, w2);
-        fetch(k + 3 * groups, v3, w3);
+        for (; k < w_end; k += groups_w) {
+          float v[VEC];
+          float w;
+          fetch(k, v, w);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          acc[j] = fmaf(v0[j], w0, acc[j]);
-          acc[j] = fmaf(v1[j], w1, acc[j]);
-          acc[j] = fmaf(v2[j], w2, acc[j]);
-          acc[j] = fmaf(v3[j], w3, acc[j]);
+          for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[j], w, acc[j]);
         }
-      }
-      for (; k < end; k += groups) {
-        float v[VEC];
-        float w;
-        fetch(k, v, w);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[j], w, acc[j]);
       }
       // groups of one wave share columns when lpr < 64: fold them with shuffles
       for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
       }
-      if ((threadIdx.x & (kWave - 1)) < (1 << a.lpr_log2)) {
+      if (gw == 0 && col_ok) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) s_part[wave * D + c0 + j] = acc[j];
       }
@@ -1001,7 +1069,7 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
   RECIS_REQUIRE(coef == nullptr || dtype_size(coef_dtype), "invalid coef dtype");
   const int vb_in = pick_vec_bytes(D * in_sz, reinterpret_cast<uintptr_t>(rows));
-  const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(out));
+  const int vb_out = pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
   const int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
   CsrArgs a;
   a.row_start = row_start;
@@ -1025,20 +1093,30 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
     using TOut = decltype(tout);
     return dispatch_vec(vec, [&](auto vtag) {
       constexpr int VEC = decltype(vtag)::value;
-      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 16) {
+      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 32) {
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
-        RECIS_TIME_KERNEL("csr_cold_kernel", stream)
-        csr_cold_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
-            static_cast<const TIn*>(rows), static_cast<TOut*>(out), a);
-        RECIS_LAUNCH_CHECK();
+        const TIn* rin = static_cast<const TIn*>(rows);
+        const bool shuffle = a.lpr_log2 >= 3;  // at most eight lane groups per wave
+        {
+          RECIS_TIME_KERNEL("csr_cold_kernel", stream)
+          if (shuffle)
+            csr_cold_kernel<TIn, TOut, VEC, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(rin, static_cast<TOut*>(out), a);
+          else
+            csr_cold_kernel<TIn, TOut, VEC, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(rin, static_cast<TOut*>(out), a);
+          RECIS_LAUNCH_CHECK();
+        }
         if constexpr (std::is_same<TOut, float>::value) {
           if (hot_cap > 0) {
             const int64_t hot_grid = std::min<int64_t>(hot_cap, 2048);
             const size_t lds = sizeof(float) * (kPlanBlock / kWave) * static_cast<size_t>(D);
             RECIS_TIME_KERNEL("csr_hot_kernel", stream)
-            csr_hot_kernel<TIn, VEC><<<dim3(hot_grid), dim3(kPlanBlock), lds, stream>>>(
-                static_cast<const TIn*>(rows), static_cast<float*>(out), a, hot_items, counts_dev, hot_cap);
+            if (shuffle)
+              csr_hot_kernel<TIn, VEC, true><<<dim3(hot_grid), dim3(kPlanBlock), lds, stream>>>(
+                  rin, static_cast<float*>(out), a, hot_items, counts_dev, hot_cap);
+            else
+              csr_hot_kernel<TIn, VEC, false><<<dim3(hot_grid), dim3(kPlanBlock), lds, stream>>>(
+                  rin, static_cast<float*>(out), a, hot_items, counts_dev, hot_cap);
             RECIS_LAUNCH_CHECK();
           }
         }

@@ -213,11 +213,12 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
           mine = static_cast<int32_t>(idx);
         }
       }
-      for (int q0 = 0; q0 < n_here; q0 += 8 * step) {  // same trip count for the whole team (shuffles inside)
+      constexpr int kFly = VEC >= 8 ? 4 : 8;  // row loads in flight per lane
+      for (int q0 = 0; q0 < n_here; q0 += kFly * step) {  // same trip count for the whole team (shuffles inside)
         const int q = q0 + rg;
-        float v[8][VEC];
+        float v[kFly][VEC];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < kFly; ++k) {
           const int src = q + k * step;
           int32_t id = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
           if (src >= n_here || !col_ok) id = -1;
@@ -233,7 +234,7 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
           }
         }
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < kFly; ++k) {
 #pragma unroll
           for (int j = 0; j < VEC; ++j) acc[j] += v[k][j];
         }
@@ -840,7 +841,7 @@ extern "C" int recis_segment_reduce_forward(
 
   // vector width in elements, limited by both row widths and pointer alignment
   const int vb_in = pick_vec_bytes(D * in_sz, reinterpret_cast<uintptr_t>(unique_emb));
-  const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(out));
+  const int vb_out = pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
   int vec = std::min(vb_in / in_sz, vb_out / out_sz);
   if (vec < 1) vec = 1;
   if (mode == RECIS_MAX && argmax_out) vec = std::min(vec, 4);
@@ -869,7 +870,7 @@ extern "C" int recis_segment_reduce_forward(
     using TOut = decltype(tout);
     return dispatch_vec(vec, [&](auto vtag) {
       constexpr int VEC = decltype(vtag)::value;
-      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 16) {
+      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 32) {
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
         if (mode == RECIS_TILE) {
