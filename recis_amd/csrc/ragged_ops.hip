@@ -20,12 +20,14 @@ template <typename T, int VEC>
 __global__ void __launch_bounds__(kBlock)
 tile_fwd_kernel(const void* __restrict__ value, int val64, const void* __restrict__ offset, int off64,
                 const T* __restrict__ table, int64_t table_rows, T* __restrict__ out, int64_t batch,
-                int64_t seq, int64_t n_values, int D, int lpr_log2, int* err) {
+                int64_t seq, int64_t n_values, int D, int lpr_log2, int blocks_per_sample, int* err) {
+  // one sample per group of `blocks_per_sample` workgroups: no per-lane division, the sample's
+  // two offsets are uniform loads; most output rows are padding, written once and not read here
   const int rows_per_block = kBlock >> lpr_log2;
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * rows_per_block + (threadIdx.x >> lpr_log2);
-  if (row >= batch * seq) return;
+  const int64_t b = blockIdx.x / blocks_per_sample;
+  const int64_t t = static_cast<int64_t>(blockIdx.x % blocks_per_sample) * rows_per_block + (threadIdx.x >> lpr_log2);
+  if (t >= seq) return;
   const int cl = threadIdx.x & ((1 << lpr_log2) - 1);
-  const int64_t b = row / seq, t = row - b * seq;
   const int64_t start = load_index(offset, off64, b), end = load_index(offset, off64, b + 1);
   const T* src = nullptr;
   if (start < 0 || end < start || end > n_values) {
@@ -37,7 +39,7 @@ tile_fwd_kernel(const void* __restrict__ value, int val64, const void* __restric
     else
       raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
   }
-  T* dst = out + row * D;
+  T* dst = out + (b * seq + t) * D;
   for (int c0 = cl * VEC; c0 < D; c0 += VEC << lpr_log2) {
     Pack<T, VEC> v;
     if (src) {
@@ -46,7 +48,14 @@ tile_fwd_kernel(const void* __restrict__ value, int val64, const void* __restric
 #pragma unroll
       for (int j = 0; j < VEC; ++j) v.v[j] = from_float<T>(0.f);
     }
-    *reinterpret_cast<Pack<T, VEC>*>(dst + c0) = v;
+    if constexpr (sizeof(T) * VEC == 16) {
+      typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+      u4 raw;
+      __builtin_memcpy(&raw, &v, 16);
+      __builtin_nontemporal_store(raw, reinterpret_cast<u4*>(dst + c0));
+    } else {
+      *reinterpret_cast<Pack<T, VEC>*>(dst + c0) = v;
+    }
   }
 }
 
@@ -212,7 +221,9 @@ int recis_ragged_tile(const int64_t* batch, const int64_t* seq, int64_t n_featur
     const int64_t rows = batch[f] * seq[f];
     if (rows > 0) {
       RECIS_REQUIRE(out != nullptr, "out must not be NULL");
-      const int64_t grid = (rows + rows_per_block - 1) / rows_per_block;
+      const int64_t blocks_per_sample = (seq[f] + rows_per_block - 1) / rows_per_block;
+      const int64_t grid = batch[f] * blocks_per_sample;
+      RECIS_REQUIRE(grid < (int64_t(1) << 31) && blocks_per_sample < (int64_t(1) << 31), "padded output too large");
       const void* off_f = static_cast<const char*>(offset) + obase * osz;
       int rc = dispatch_t_vec(dtype, vec, [&](auto t, auto vtag) {
         using T = decltype(t);
@@ -220,7 +231,8 @@ int recis_ragged_tile(const int64_t* batch, const int64_t* seq, int64_t n_featur
         RECIS_TIME_KERNEL("tile_fwd_kernel", stream)
         tile_fwd_kernel<T, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
             value, value_is64, off_f, off_is64, static_cast<const T*>(table), table_rows,
-            static_cast<T*>(out) + rbase * D, batch[f], seq[f], n_values, static_cast<int>(D), lpr_log2, err);
+            static_cast<T*>(out) + rbase * D, batch[f], seq[f], n_values, static_cast<int>(D), lpr_log2,
+            static_cast<int>(blocks_per_sample), err);
         RECIS_LAUNCH_CHECK();
         return RECIS_OK;
       });
