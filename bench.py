@@ -222,11 +222,12 @@ class Config4:
         """Algorithmic (compulsory) HBM bytes of one launch of each heavy kernel of the step."""
         N, U, S, D = self.N, self.U, self.N, self.D
         return {
-            "plan_insert_kernel": 8 * N + 8 * N + 32 * U,           # ids in; slot + rank out; one 16-B set slot RMW
-            "plan_first_count_kernel": 4 * N + 16 * U,
-            "plan_emit_unique_kernel": 8 * N + 4 * N + 16 * U + 12 * U,
-            "plan_emit_lists_kernel": 8 * N + 16 * U + 12 * N,
-            "plan_init_kernel": 32 * N,                              # 2N set slots of 16 B
+            # plan: a record (16 B) per id and tile, at least one per unique id
+            "plan_tile_kernel": 8 * N + 4 * N + 16 * U,              # ids in; per-occurrence word + records out
+            "plan_scatter_kernel": 16 * U + 16 * U,
+            "plan_bucket_kernel": 16 * U + 8 * U + 16 * U,           # records in; per-record result + unique ids out
+            "plan_emit_occ_kernel": 8 * N + 4 * N + 8 * U + 12 * N,  # ids, word, result in; inverse, list, pos out
+            "plan_emit_uniq_kernel": 16 * U + 12 * U + 4 * (N + 1 - U),
             "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,          # ids, one table slot, index + slot pos
             "block_gather_kernel": 8 * U + 2 * U * D * 4,
             "seg_pool_fwd_kernel": U * D * 4 + 4 * N + 4 * (S + 1) + S * D * 4,
@@ -462,10 +463,10 @@ class Config5:
 # scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC_C4 = {
-    "plan_insert_kernel": 380658672, "adamw_rows_kernel": 400841547, "seg_pool_fwd_kernel": 277264266,
-    "plan_emit_unique_kernel": 272778425, "plan_emit_lists_kernel": 234571357, "csr_cold_kernel": 200464118,
-    "find_or_claim_kernel": 188212736, "plan_first_count_kernel": 157875229, "csr_hot_kernel": 139709319,
-    "block_gather_kernel": 119564740, "plan_init_kernel": 81795174,
+    "adamw_rows_kernel": 400841121, "seg_pool_fwd_kernel": 324971171, "csr_cold_kernel": 251810488,
+    "csr_hot_kernel": 143831573, "block_gather_kernel": 119564885, "plan_emit_occ_kernel": 115515050,
+    "find_or_claim_kernel": 114550648, "plan_bucket_kernel": 89176810, "plan_scatter_kernel": 77256686,
+    "plan_tile_kernel": 58195299, "plan_emit_uniq_kernel": 32875429,
 }
 
 
