@@ -332,15 +332,12 @@ class Config3:
             + N * (4 + D * 4) + U * D * 4 * 7 + U * 8
 
     def evict_sweep_ms(self, filter_step=50):
-        """One reference-style sweep: snapshot of all (key, row) pairs, stamp test, erase + free +
-        re-initialise. The threshold is set so that nothing is old enough: the sweep cost without
-        shrinking the table under the benchmark."""
+        """One eviction sweep over the 2e8-row table (keys not seen for `filter_step` steps): the
+        one-pass library sweep. The threshold is set so that nothing is old enough: the sweep cost
+        without shrinking the table under the benchmark."""
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        ids, index = self.table.ids_map()
-        chunks, chunk_rows = self.table.get_slot("step_filter").kernel_blocks()
-        mask = self.ops.block_filter(index, chunks, chunk_rows, -1)
-        self.table.delete(torch.masked_select(ids, mask), torch.masked_select(index, mask), "step_filter")
+        self.table.evict_older("step_filter", -1)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3
 

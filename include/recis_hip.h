@@ -213,6 +213,18 @@ int recis_idmap_stats(recis_idmap* m, int64_t* live, int64_t* id_num, int64_t* f
  * Synchronises; *count = number of live pairs (only min(count, max_out) written). */
 int recis_idmap_snapshot(recis_idmap* m, int64_t* ids_out, int64_t* index_out, int64_t max_out,
                          int64_t* count, void* stream);
+/* The eviction sweep of a step filter in one pass over the table. Replaces the sequence
+ * IdMap::SnapShot + block_filter + masked_select + DeleteIds of
+ * recis/nn/modules/hashtable_hook_impl.py:487-551 (do_filter / filter) and hashtable.cc:263-278:
+ * every live key whose row has stamp < threshold (stamp slot: int32 or int64, one value per row,
+ * blocks of block_rows rows, pointer table on the device) is erased and its row appended to the
+ * free list; the evicted (key, row) pairs are written to ids_out / index_out (unordered) for the
+ * caller to re-initialise the rows. At most max_out keys are evicted. Synchronises;
+ * *count = number of evicted keys. */
+int recis_idmap_evict_older(recis_idmap* m, const void* const* stamp_blocks_dev, int64_t n_blocks,
+                            int64_t block_rows, int stamp_is64, int64_t threshold,
+                            int64_t* ids_out, int64_t* index_out, int64_t max_out, int64_t* count,
+                            void* stream);
 /* GpuIdMap::Clear (gpu_id_map.cu:98-103). */
 int recis_idmap_clear(recis_idmap* m, void* stream);
 /* IdMap::Reserve (not implemented for the reference GPU map, gpu_id_map.cu:105-108). */

@@ -313,6 +313,59 @@ erase_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __restrict_
               static_cast<unsigned long long>(total));
 }
 
+// Eviction sweep in one pass over the table: every live slot reads the stamp of its row and,
+// when the stamp is older than the threshold, leaves the table (tombstone), hands its row to the
+// free list and reports (key, row) so that the caller can re-initialise the row. One atomic per
+// workgroup that evicts anything.
+__global__ void __launch_bounds__(kBlock)
+evict_older_kernel(Slot* __restrict__ table, int64_t capacity, const void* const* __restrict__ stamp_blocks,
+                   int64_t n_blocks, int64_t block_rows, int stamp64, int64_t threshold,
+                   int64_t* __restrict__ ids_out, int64_t* __restrict__ index_out, int64_t max_out,
+                   int64_t* __restrict__ free_list, int64_t* __restrict__ state, int* err) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  bool evict = false;
+  int64_t k = 0, v = 0;
+  if (i < capacity) {
+    const longlong2 kv = *reinterpret_cast<const longlong2*>(&table[i]);
+    k = kv.x;
+    v = kv.y;
+    if (k != kEmpty && k != kTomb && v >= 0) {
+      const int64_t b = v / block_rows, r = v - b * block_rows;
+      if (b < n_blocks) {
+        const int64_t stamp = stamp64 ? static_cast<const int64_t*>(stamp_blocks[b])[r]
+                                      : static_cast<int64_t>(static_cast<const int32_t*>(stamp_blocks[b])[r]);
+        evict = stamp < threshold;
+      } else {
+        raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+      }
+    }
+  }
+  int rank, total;
+  block_rank(evict, rank, total);
+  __shared__ int64_t base;
+  if (threadIdx.x == 0)
+    base = total ? static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&state[ST_TMP]),
+                                                  static_cast<unsigned long long>(total)))
+                 : 0;
+  __syncthreads();
+  if (evict) {
+    const int64_t pos = base + rank;
+    if (pos < max_out) {  // beyond the caller's buffers the key stays (counted, reported by the host)
+      ids_out[pos] = k;
+      index_out[pos] = v;
+      free_list[state[ST_FREE] + pos] = v;
+      table[i].key = kTomb;
+      table[i].val = kValUnset;
+    }
+  }
+}
+
+__global__ void evict_commit_kernel(int64_t* state, int64_t max_out) {
+  const int64_t n = state[ST_TMP] < max_out ? state[ST_TMP] : max_out;
+  state[ST_FREE] += n;
+  state[ST_LIVE] -= n;
+}
+
 __global__ void erase_commit_kernel(int64_t* state, int64_t n) {
   state[ST_FREE] += n;
   state[ST_LIVE] -= state[ST_TMP];
@@ -646,6 +699,33 @@ int recis_idmap_snapshot(recis_idmap* m, int64_t* ids_out, int64_t* index_out, i
   int64_t words[ST_WORDS];
   if (int rc = sync_stats(m, stream, words)) return rc;
   *count = words[ST_TMP];
+  zero_words_kernel<<<1, 64, 0, stream>>>(m->state + ST_TMP, 1);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+int recis_idmap_evict_older(recis_idmap* m, const void* const* stamp_blocks_dev, int64_t n_blocks,
+                            int64_t block_rows, int stamp_is64, int64_t threshold, int64_t* ids_out,
+                            int64_t* index_out, int64_t max_out, int64_t* count, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(m != nullptr && count != nullptr, "id map / count is NULL");
+  RECIS_REQUIRE(stamp_blocks_dev != nullptr && n_blocks >= 0 && block_rows > 0, "bad stamp blocks");
+  RECIS_REQUIRE(max_out >= 0 && (max_out == 0 || (ids_out && index_out)), "bad output buffers");
+  *count = 0;
+  if (max_out == 0) return RECIS_OK;
+  int* err = device_error_word(current_device());
+  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  if (int rc = ensure_free_room(m, max_out, stream)) return rc;
+  evict_older_kernel<<<dim3(blocks_for(m->capacity)), dim3(kBlock), 0, stream>>>(
+      m->table, m->capacity, stamp_blocks_dev, n_blocks, block_rows, stamp_is64, threshold, ids_out, index_out,
+      max_out, m->free_list, m->state, err);
+  RECIS_LAUNCH_CHECK();
+  evict_commit_kernel<<<1, 1, 0, stream>>>(m->state, max_out);
+  RECIS_LAUNCH_CHECK();
+  int64_t words[ST_WORDS];
+  if (int rc = sync_stats(m, stream, words)) return rc;
+  *count = std::min<int64_t>(words[ST_TMP], max_out);
+  m->free_ub += *count;
   zero_words_kernel<<<1, 64, 0, stream>>>(m->state + ST_TMP, 1);
   RECIS_LAUNCH_CHECK();
   return RECIS_OK;

@@ -480,6 +480,22 @@ class HashtableImpl:
                 continue
             slot.index_insert(index, slot.gen_val(ids.numel()))
 
+    def evict_older(self, stamp_slot, threshold):
+        """Eviction sweep of a step filter in one pass over the map: erase every key whose
+        row has ``stamp_slot < threshold``, free the rows and re-initialise every other slot
+        there. Same outcome as ``ids_map`` + ``block_filter`` + ``delete``
+        (hashtable_hook_impl.py:487-551, hashtable.cc:263-278) without materialising all
+        (key, row) pairs. Returns the evicted ``(ids, index)``."""
+        chunks, chunk_rows = self.get_slot(stamp_slot).kernel_blocks()
+        ids, index = self._idmap.evict_older(chunks, chunk_rows, threshold)
+        if ids.numel():
+            sg = self._slot_group
+            keep = sg.get_slot_index(stamp_slot)
+            for i, slot in enumerate(sg.slots()):
+                if i != keep:
+                    slot.index_insert(index, slot.gen_val(ids.numel()))
+        return ids, index
+
     def id_map(self):
         return self._idmap
 

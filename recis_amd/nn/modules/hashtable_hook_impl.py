@@ -100,6 +100,10 @@ class GlobalStepFilterHookImpl(BaseFilterHookImpl):
             self._global_step += step_size
         self._step_host += step_size
 
+    def do_filter(self) -> None:
+        # one pass over the id map instead of snapshot + filter + delete
+        self._ht.evict_older(self._name, self._step_host - self._filter_step)
+
     def filter(self, ids, index):
         slot = self._ht.get_slot(self._name)
         chunks, chunk_rows = slot.kernel_blocks()

@@ -642,6 +642,22 @@ class IdMap:
         assert count.value == n, (count.value, n)
         return ids, index
 
+    def evict_older(self, stamp_blocks, block_rows, threshold, max_out=None):
+        """One-pass eviction sweep: erase every key whose row has ``stamp < threshold`` and
+        free the row; returns the evicted ``(ids, index)`` (``recis_idmap_evict_older``)."""
+        b0 = _check_blocks(stamp_blocks, block_rows)
+        if b0.dtype not in (torch.int32, torch.int64) or _row_bytes(b0) != b0.element_size():
+            raise TypeError("the stamp slot must be int32/int64 of width 1")
+        n = self.size() if max_out is None else int(max_out)
+        ids = torch.empty(n, dtype=torch.int64, device=self.device)
+        index = torch.empty(n, dtype=torch.int64, device=self.device)
+        count = ctypes.c_int64(0)
+        tab = block_ptr_table(stamp_blocks)
+        check(lib().recis_idmap_evict_older(self._h, ptr(tab), i64(len(stamp_blocks)), i64(block_rows),
+                                            int(b0.dtype == torch.int64), i64(threshold), ptr(ids), ptr(index),
+                                            i64(n), ctypes.byref(count), stream_ptr(self.device)))
+        return ids[: count.value], index[: count.value]
+
     def clear(self):
         check(lib().recis_idmap_clear(self._h, stream_ptr(self.device)))
 

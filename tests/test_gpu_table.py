@@ -195,6 +195,46 @@ def test_block_filter(rng, dt):
     assert torch.equal(ops.block_filter(ids, blocks, bs, 77), flat[ids] < 77)
 
 
+@pytest.mark.parametrize("dt", [torch.int64, torch.int32])
+def test_evict_older_equals_snapshot_filter_erase(rng, dt):
+    """The one-pass eviction sweep against the reference's sequence (snapshot, block_filter,
+    masked_select, erase) on a twin map and against the oracle map: same evicted set, same
+    live set, same allocator counters; freed rows are handed out again."""
+    bs, nb = 1000, 8
+    keys = rng.integers(-10**15, 10**15, size=6000)
+    keys = np.unique(keys)
+    a, b, c = ops.IdMap(), ops.IdMap(), oracle.IdMap()
+    rows = a.lookup(_dev(keys)).cpu().numpy()
+    np.testing.assert_array_equal(b.lookup(_dev(keys)).cpu().numpy(), rows)
+    np.testing.assert_array_equal(c.lookup(keys), rows)
+    stamps = rng.integers(0, 100, size=bs * nb)
+    blocks = [torch.from_numpy(stamps[i * bs:(i + 1) * bs].reshape(bs, 1)).cuda().to(dt) for i in range(nb)]
+    thr = 40
+    ev_ids, ev_rows = a.evict_older(blocks, bs, thr)
+    ids_b, idx_b = b.snapshot()
+    mask = ops.block_filter(idx_b, blocks, bs, thr)
+    del_ids, del_rows = torch.masked_select(ids_b, mask), torch.masked_select(idx_b, mask)
+    b.erase(del_ids, del_rows)
+    exp_mask = stamps[rows] < thr
+    order = np.argsort(ev_ids.cpu().numpy())
+    np.testing.assert_array_equal(ev_ids.cpu().numpy()[order], np.sort(keys[exp_mask]))
+    np.testing.assert_array_equal(ev_rows.cpu().numpy()[order], rows[exp_mask][np.argsort(keys[exp_mask])])
+    c.delete(keys[exp_mask], rows[exp_mask])
+    assert a.stats()[:3] == b.stats()[:3] == (c.size(), c.id_num(), c.free_size())
+    for m in (a, b):
+        got = m.lookup_readonly(_dev(keys)).cpu().numpy()
+        np.testing.assert_array_equal(got, np.where(exp_mask, -1, rows))
+    # new keys take the freed rows (the free list holds exactly the evicted rows)
+    fresh = np.arange(10**16, 10**16 + int(exp_mask.sum()), dtype=np.int64)
+    assert sorted(a.lookup(_dev(fresh)).cpu().numpy().tolist()) == sorted(rows[exp_mask].tolist())
+    # nothing to evict: no change; a buffer smaller than the evictable set evicts just that many
+    assert a.evict_older(blocks, bs, -5)[0].numel() == 0
+    n_more = int((stamps[b.snapshot()[1].cpu().numpy()] < 90).sum())
+    part_ids, _ = b.evict_older(blocks, bs, 90, max_out=7)
+    assert part_ids.numel() == min(7, n_more) and b.stats()[0] == c.size() - part_ids.numel()
+    assert _lib.poll_device_errors() == 0
+
+
 # ------------------------------------------------------------------ optimizers
 def _np_blocks(w, bs):
     nb = (w.shape[0] + bs - 1) // bs
