@@ -184,10 +184,12 @@ class Config4:
         return self.plan.unique, self.plan.inverse
 
     def lookup(self, uniq):
-        return self.table.embedding_lookup(uniq, False)
+        return self.table.lookup_index(uniq, False)
 
-    def pool_fwd(self, rows, inv):
-        return self.ops.segment_reduce_forward(rows, None, inv, self.offsets, "sum")
+    def pool_fwd(self, index, inv):
+        # pooling reads the rows out of the table (no [U, D] copy), as EmbeddingEngine does
+        chunks, chunk_rows = self.table.emb_blocks()
+        return self.ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, None, inv, self.offsets, "sum")
 
     def pool_bwd(self, inv):
         return self.ops.segment_reduce_backward_plan(self.grad_out, None, self.offsets, self.plan, "sum")
@@ -200,8 +202,8 @@ class Config4:
     def step(self):
         ids = self.feature_ops()
         uniq, inv = self.dedup(ids)
-        index, rows = self.lookup(uniq)
-        pooled = self.pool_fwd(rows, inv)
+        index = self.lookup(uniq)
+        pooled = self.pool_fwd(index, inv)
         g = self.pool_bwd(inv)
         self.update(index, g)
         return pooled
@@ -212,8 +214,8 @@ class Config4:
         return {
             "feature_ops": feat,
             "dedup": N * (8 + 4) + U * 8,
-            "lookup": U * (16 + 8) + U * D * 4 * 2,
-            "pool_fwd": U * D * 4 + N * 4 + (S + 1) * 4 + S * D * 4,
+            "lookup": U * (16 + 8),
+            "pool_fwd": U * (8 + D * 4) + N * 4 + (S + 1) * 4 + S * D * 4,
             "pool_bwd": S * D * 4 + N * 4 + (S + 1) * 4 + U * D * 4,
             "adam": U * 8 + U * D * 4 * (1 + 6),
         }
@@ -229,8 +231,7 @@ class Config4:
             "plan_emit_occ_kernel": 8 * N + 4 * N + 8 * U + 12 * N,  # ids, word, result in; inverse, list, pos out
             "plan_emit_uniq_kernel": 16 * U + 12 * U + 4 * (N + 1 - U),
             "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,          # ids, one table slot, index + slot pos
-            "block_gather_kernel": 8 * U + 2 * U * D * 4,
-            "seg_pool_fwd_kernel": U * D * 4 + 4 * N + 4 * (S + 1) + S * D * 4,
+            "seg_pool_fwd_kernel": U * (8 + D * 4) + 4 * N + 4 * (S + 1) + S * D * 4,
             "csr_cold_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,
             "csr_hot_kernel": 0,
             "adamw_rows_kernel": U * (8 + D * 4 * 7),
@@ -239,13 +240,13 @@ class Config4:
     def stage_times(self, iters):
         ids = self.feature_ops()
         uniq, inv = self.dedup(ids)
-        index, rows = self.lookup(uniq)
+        index = self.lookup(uniq)
         g = self.pool_bwd(inv)
         return {
             "feature_ops": _event_ms(self.feature_ops, iters),
             "dedup": _event_ms(lambda: self.dedup(ids), iters),
             "lookup": _event_ms(lambda: self.lookup(uniq), iters),
-            "pool_fwd": _event_ms(lambda: self.pool_fwd(rows, inv), iters),
+            "pool_fwd": _event_ms(lambda: self.pool_fwd(index, inv), iters),
             "pool_bwd": _event_ms(lambda: self.pool_bwd(inv), iters),
             "adam": _event_ms(lambda: self.update(index, g), iters),
         }
@@ -318,7 +319,9 @@ class Config3:
         self.U = plan.U
         index, rows = self.table.embedding_lookup(plan.unique, False)
         self.table.update_slot("step_filter", index, self.step_t)
-        out = o.gather(plan.inverse, rows)                          # one row per lookup
+        # one row per lookup, expanded from the [U, D] copy: with a 25 GB table, pooling out of the
+        # table (segment_reduce_forward_blocks) gains nothing, the copy keeps the 2e6 reads local
+        out = o.gather(plan.inverse, rows)
         g = o.segment_reduce_backward_plan(self.grad_out, None, self.span, plan, "tile")
         self.table.accept_grad(index, g, unique=True)
         self.opt.step()

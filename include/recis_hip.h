@@ -105,6 +105,23 @@ int recis_segment_reduce_forward(const void* unique_emb, int emb_dtype,
                                  void* stream);
 
 /*
+ * The same forward with the unique rows read where the table keeps them instead of a dense
+ * [U, D] copy: row u is row row_index[u] (the id map's answer for unique id u; negative = key
+ * absent, reads as zeros) of the block list emb_blocks_dev (device array of n_blocks pointers,
+ * 16-byte aligned blocks of block_rows rows). Fuses block_gather
+ * (csrc/ops/block_ops.cc:281-290) into segment_reduce_forward
+ * (csrc/ops/embedding_segment_reduce_kernel.cu:199-273): the [U, D] intermediate of
+ * recis/nn/modules/embedding.py:592-624 (emb_reduce) is neither written nor read. SUM, MEAN and TILE.
+ */
+int recis_segment_reduce_forward_blocks(const void* const* emb_blocks_dev, int64_t n_blocks,
+                                        int64_t block_rows, const int64_t* row_index, int emb_dtype,
+                                        const void* weight, int weight_dtype,
+                                        const void* reverse_indices, int rev_is64,
+                                        const void* offsets, int off_is64, void* out, int out_dtype,
+                                        int64_t B, int64_t U, int64_t S, int64_t D, int mode,
+                                        void* stream);
+
+/*
  * Backward of the ragged-mode pooling: scatters the pooled gradient back to the
  * unique rows.
  * Replaces: segment_reduce_backward, csrc/ops/embedding_segment_reduce_kernel.cu:276-350

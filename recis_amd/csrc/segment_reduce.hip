@@ -39,7 +39,29 @@ struct SegArgs {
   int lpr_log2, team_log2;
   int mean;
   int* err;
+  // rows addressed through a table instead of a dense [U, D] array (BLK kernels): row u is row
+  // row_index[u] of the block list (blocks of block_rows rows); a negative row_index reads as zeros
+  const int64_t* row_index;
+  const void* const* blocks;
+  int64_t block_rows, n_blocks;
 };
+
+// Address of unique row idx (idx < U checked by the caller) in the block list, nullptr = zero row.
+template <typename TIn>
+__device__ __forceinline__ const TIn* block_row(const SegArgs& a, int64_t idx) {
+  const int64_t ri = a.row_index[idx];
+  if (ri < 0) return nullptr;  // key not in the table (read-only lookup)
+  int64_t b = 0, r = ri;
+  if (a.n_blocks > 1) {
+    b = ri / a.block_rows;
+    r = ri - b * a.block_rows;
+  }
+  if (b >= a.n_blocks || r >= a.block_rows) {
+    raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+    return nullptr;
+  }
+  return static_cast<const TIn*>(a.blocks[b]) + r * a.D;
+}
 
 // Stage offsets[s0 .. s0 + teams_per_block] into LDS and return this team's
 // [start, end). Returns false for teams beyond the last segment.
@@ -74,7 +96,7 @@ __device__ __forceinline__ bool team_segment(const SegArgs& a, int64_t* s_off,
 //   kFwdRev32     int32 reverse indices, no weights
 enum { kFwdGeneric = 0, kFwdPlain = 1, kFwdRev32 = 2 };
 
-template <typename TIn, typename TOut, int VEC, int KIND>
+template <typename TIn, typename TOut, int VEC, int KIND, bool BLK>
 __global__ void __launch_bounds__(kBlock)
 seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
   __shared__ int64_t s_off[kBlock + 1];
@@ -108,7 +130,17 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
       w = 0.f;
       return;
     }
-    load_pack<TIn, VEC>(emb + idx * D + c0, v);
+    if constexpr (BLK) {
+      const TIn* row = block_row<TIn>(a, idx);
+      if (row) {
+        load_pack<TIn, VEC>(row + c0, v);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+      }
+    } else {
+      load_pack<TIn, VEC>(emb + idx * D + c0, v);
+    }
   };
   auto add = [&](float (&acc)[VEC], const float (&v)[VEC], float w) {
 #pragma unroll
@@ -167,7 +199,7 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
 // Rows are summed per row group in increasing order, like the generic kernel. Requires U < 2^31.
 enum { kFastPlain = 0, kFastRev32 = 1, kFastRev64 = 2 };
 
-template <typename TIn, typename TOut, int VEC, int KIND>
+template <typename TIn, typename TOut, int VEC, int KIND, bool BLK>
 __global__ void __launch_bounds__(kBlock)
 seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
   const int64_t s = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.team_log2) + (threadIdx.x >> a.team_log2);
@@ -197,7 +229,8 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
     for (int64_t base = start; base < end; base += team) {
       const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
-      int32_t mine = -1;  // row of occurrence base + lane_t
+      int32_t mine = -1;       // row of occurrence base + lane_t in emb ...
+      uint64_t mine_addr = 0;  // ... or its address in the block list (BLK), 0 = zero row
       if (lane_t < n_here) {
         int64_t idx;
         if constexpr (KIND == kFastPlain) {
@@ -209,6 +242,8 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
         }
         if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
           raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        } else if constexpr (BLK) {
+          mine_addr = reinterpret_cast<uint64_t>(block_row<TIn>(a, idx));
         } else {
           mine = static_cast<int32_t>(idx);
         }
@@ -220,13 +255,22 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
 #pragma unroll
         for (int k = 0; k < kFly; ++k) {
           const int src = q + k * step;
-          int32_t id = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
-          if (src >= n_here || !col_ok) id = -1;
-          if (id >= 0) {
-            if constexpr (KIND == kFastPlain) {
-              load_pack_stream<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);  // read once
+          const int from = team_lane0 + min(src, team - 1);
+          const TIn* row = nullptr;
+          if constexpr (BLK) {
+            const uint32_t lo = __shfl(static_cast<uint32_t>(mine_addr), from, kWave);
+            const uint32_t hi = __shfl(static_cast<uint32_t>(mine_addr >> 32), from, kWave);
+            row = reinterpret_cast<const TIn*>((static_cast<uint64_t>(hi) << 32) | lo);
+          } else {
+            const int32_t id = __shfl(mine, from, kWave);
+            if (id >= 0) row = emb + static_cast<int64_t>(id) * D;
+          }
+          if (src >= n_here || !col_ok) row = nullptr;
+          if (row) {
+            if constexpr (KIND == kFastPlain && !BLK) {
+              load_pack_stream<TIn, VEC>(row + c0, v[k]);  // read once
             } else {
-              load_pack<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
+              load_pack<TIn, VEC>(row + c0, v[k]);
             }
           } else {
 #pragma unroll
@@ -421,7 +465,7 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
 
 // TILE combiner forward: one row group per occurrence, out[i] = w_i * emb[rev_i];
 // occurrences outside [offsets[0], offsets[S]) produce zero rows.
-template <typename TIn, typename TOut, int VEC>
+template <typename TIn, typename TOut, int VEC, bool BLK>
 __global__ void __launch_bounds__(kBlock)
 seg_tile_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
   const int rows_per_block = kBlock >> a.lpr_log2;
@@ -443,10 +487,19 @@ seg_tile_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
       live = false;
     }
   }
+  const TIn* row = nullptr;
+  if (live) {
+    if constexpr (BLK) {
+      row = block_row<TIn>(a, idx);
+    } else {
+      row = emb + idx * D;
+    }
+    live = row != nullptr;
+  }
   for (int c0 = cl * VEC; c0 < D; c0 += col_stride) {
     float v[VEC];
     if (live) {
-      load_pack<TIn, VEC>(emb + idx * D + c0, v);
+      load_pack<TIn, VEC>(row + c0, v);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) v[j] *= w;
     } else {
@@ -819,11 +872,17 @@ int check_common(const void* offsets, int64_t B, int64_t U, int64_t S, int64_t D
 
 using namespace recis_hip;
 
-extern "C" int recis_segment_reduce_forward(
-    const void* unique_emb, int emb_dtype, const void* weight, int weight_dtype,
-    const void* reverse_indices, int rev_is64, const void* offsets, int off_is64,
-    void* out, int out_dtype, int32_t* argmax_out, int64_t B, int64_t U, int64_t S,
-    int64_t D, int mode, void* stream_) {
+// Where the unique rows live when they are not a dense [U, D] array.
+struct BlockSource {
+  const int64_t* row_index;
+  const void* const* blocks;
+  int64_t block_rows, n_blocks;
+};
+
+static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_dtype, const void* weight,
+                        int weight_dtype, const void* reverse_indices, int rev_is64, const void* offsets,
+                        int off_is64, void* out, int out_dtype, int32_t* argmax_out, int64_t B, int64_t U,
+                        int64_t S, int64_t D, int mode, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (int rc = check_common(offsets, B, U, S, D, mode, weight_dtype, weight)) return rc;
   RECIS_REQUIRE(reverse_indices != nullptr || U == B,
@@ -832,7 +891,7 @@ extern "C" int recis_segment_reduce_forward(
   const int64_t out_rows = (mode == RECIS_TILE) ? B : S;
   if (out_rows == 0) return RECIS_OK;
   RECIS_REQUIRE(out != nullptr, "out must not be NULL");
-  RECIS_REQUIRE(unique_emb != nullptr || U == 0, "unique_emb must not be NULL");
+  RECIS_REQUIRE(unique_emb != nullptr || U == 0 || blk != nullptr, "unique_emb must not be NULL");
   const int in_sz = dtype_size(emb_dtype), out_sz = dtype_size(out_dtype);
   RECIS_REQUIRE(in_sz && out_sz, "invalid dtype (emb=%d out=%d)", emb_dtype, out_dtype);
 
@@ -840,7 +899,8 @@ extern "C" int recis_segment_reduce_forward(
   RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
 
   // vector width in elements, limited by both row widths and pointer alignment
-  const int vb_in = pick_vec_bytes(D * in_sz, reinterpret_cast<uintptr_t>(unique_emb));
+  // (blocks are 16-byte aligned by contract)
+  const int vb_in = pick_vec_bytes(D * in_sz, blk ? 16 : reinterpret_cast<uintptr_t>(unique_emb));
   const int vb_out = pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
   int vec = std::min(vb_in / in_sz, vb_out / out_sz);
   if (vec < 1) vec = 1;
@@ -864,6 +924,10 @@ extern "C" int recis_segment_reduce_forward(
   a.team_log2 = pick_team_log2(B, S, geom.lpr_log2);
   a.mean = (mode == RECIS_MEAN);
   a.err = err;
+  a.row_index = blk ? blk->row_index : nullptr;
+  a.blocks = blk ? blk->blocks : nullptr;
+  a.block_rows = blk ? blk->block_rows : 1;
+  a.n_blocks = blk ? blk->n_blocks : 0;
 
   return dispatch_types(emb_dtype, out_dtype, [&](auto tin, auto tout) {
     using TIn = decltype(tin);
@@ -876,8 +940,26 @@ extern "C" int recis_segment_reduce_forward(
         if (mode == RECIS_TILE) {
           const int rows_per_block = kBlock >> a.lpr_log2;
           const int64_t grid = (B + rows_per_block - 1) / rows_per_block;
-          seg_tile_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(
-              static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), a);
+          RECIS_TIME_KERNEL("seg_tile_fwd_kernel", stream)
+          if (blk)
+            seg_tile_fwd_kernel<TIn, TOut, VEC, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                nullptr, static_cast<TOut*>(out), a);
+          else
+            seg_tile_fwd_kernel<TIn, TOut, VEC, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(
+                static_cast<const TIn*>(unique_emb), static_cast<TOut*>(out), a);
+        } else if (blk) {
+          // rows in the table: the int32-index kernels (what a batch plan produces) and the generic one
+          const int teams_per_block = kBlock >> a.team_log2;
+          const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
+          TOut* o = static_cast<TOut*>(out);
+          const bool rev32 = a.weight == nullptr && a.rev != nullptr && !a.rev64;
+          RECIS_TIME_KERNEL("seg_pool_fwd_kernel", stream)
+          if (rev32 && U < (int64_t(1) << 31) && a.team_log2 > a.lpr_log2)
+            seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(nullptr, o, a);
+          else if (rev32)
+            seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdRev32, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(nullptr, o, a);
+          else
+            seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdGeneric, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(nullptr, o, a);
         } else {
           const int teams_per_block = kBlock >> a.team_log2;
           const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
@@ -900,17 +982,17 @@ extern "C" int recis_segment_reduce_forward(
             const bool fast = a.weight == nullptr && U < (int64_t(1) << 31) && a.team_log2 > a.lpr_log2;
             RECIS_TIME_KERNEL("seg_pool_fwd_kernel", stream)
             if (fast && a.rev == nullptr)
-              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastPlain, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
             else if (fast && !a.rev64)
-              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
             else if (fast)
-              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev64><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev64, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
             else if (a.weight == nullptr && a.rev == nullptr)
-              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdPlain, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
             else if (a.weight == nullptr && !a.rev64)
-              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdRev32><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdRev32, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
             else
-              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdGeneric><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
+              seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdGeneric, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
           }
         }
         RECIS_LAUNCH_CHECK();
@@ -918,6 +1000,28 @@ extern "C" int recis_segment_reduce_forward(
       }
     });
   });
+}
+
+extern "C" int recis_segment_reduce_forward(
+    const void* unique_emb, int emb_dtype, const void* weight, int weight_dtype,
+    const void* reverse_indices, int rev_is64, const void* offsets, int off_is64,
+    void* out, int out_dtype, int32_t* argmax_out, int64_t B, int64_t U, int64_t S,
+    int64_t D, int mode, void* stream_) {
+  return forward_impl(unique_emb, nullptr, emb_dtype, weight, weight_dtype, reverse_indices, rev_is64, offsets,
+                      off_is64, out, out_dtype, argmax_out, B, U, S, D, mode, stream_);
+}
+
+extern "C" int recis_segment_reduce_forward_blocks(
+    const void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows, const int64_t* row_index,
+    int emb_dtype, const void* weight, int weight_dtype, const void* reverse_indices, int rev_is64,
+    const void* offsets, int off_is64, void* out, int out_dtype, int64_t B, int64_t U, int64_t S,
+    int64_t D, int mode, void* stream_) {
+  RECIS_REQUIRE(mode != RECIS_MAX, "the MAX combiner takes dense rows (recis_segment_reduce_forward)");
+  RECIS_REQUIRE(n_blocks >= 0 && block_rows > 0, "bad block list");
+  RECIS_REQUIRE(U == 0 || (emb_blocks_dev != nullptr && row_index != nullptr), "NULL block list / row_index");
+  BlockSource blk{row_index, emb_blocks_dev, block_rows, n_blocks};
+  return forward_impl(nullptr, &blk, emb_dtype, weight, weight_dtype, reverse_indices, rev_is64, offsets, off_is64,
+                      out, out_dtype, nullptr, B, U, S, D, mode, stream_);
 }
 
 extern "C" int recis_segment_reduce_backward(

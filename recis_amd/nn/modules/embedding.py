@@ -88,6 +88,74 @@ def lookup_unique_rows(hashtable: HashTable, unique_ids, admit_hook=None, traina
     return emb
 
 
+class LookupPoolFunction(torch.autograd.Function):
+    """Lookup of a plan's unique ids and sum / mean pooling straight out of the table: the
+    ``[U, D]`` copy of the looked-up rows (lookup function + ``ragged_embedding_segment_reduce``,
+    recis/nn/modules/embedding.py:592-624) is never made. Backward reduces the pooled
+    gradients per unique row over the plan and hands (row index, gradient) to the table."""
+
+    @staticmethod
+    def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly):
+        index = impl.lookup_index(plan.unique, readonly)
+        chunks, chunk_rows = impl.emb_blocks()
+        out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets, combiner)
+        ctx.impl, ctx.plan, ctx.combiner, ctx.readonly = impl, plan, combiner, readonly
+        ctx.save_for_backward(index, weight, offsets)
+        ctx.mark_non_differentiable(index)
+        return index, out
+
+    @staticmethod
+    def backward(ctx, _grad_index, grad):
+        index, weight, offsets = ctx.saved_tensors
+        g = ops.segment_reduce_backward_plan(grad.contiguous(), weight, offsets, ctx.plan, ctx.combiner)
+        if ctx.readonly:  # keys the table does not hold take no gradient
+            keep = index >= 0
+            index, g = index[keep], g[keep]
+        ctx.impl.accept_grad(index, g, unique=True)
+        return None, None, None, None, None, None, None
+
+
+def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt):
+    """Rows of the plan's unique ids pooled per segment. Sum / mean over a float table go
+    through ``LookupPoolFunction`` (pooling reads the table directly); everything else looks the
+    rows up first and pools the copy."""
+    impl = hashtable._hashtable_impl
+    float_table = hashtable._dtype in (torch.float32, torch.bfloat16, torch.float16)
+    n_occ = plan.inverse.numel()
+    sparse_mean = opt.combiner == "mean" and not n_occ / offsets.numel() > 5
+    id_mean = opt.grad_reduce_by == "id" and hashtable.training and opt.trainable
+    if opt.combiner in ("sum", "mean") and float_table and not sparse_mean and not id_mean:
+        if weight is not None and weight.dtype != hashtable._dtype:
+            weight = weight.to(hashtable._dtype)
+        if hashtable.training and opt.trainable:
+            readonly = opt.admit_hook is not None
+            if readonly:
+                from .hashtable_hook_impl import HashtableHookFactory, ReadOnlyHookImpl
+                admit = HashtableHookFactory().create_admit_hook(hashtable, opt.admit_hook)
+                assert isinstance(admit, ReadOnlyHookImpl), "admit hook only support ReadOnlyHook yet, but got: %s" % admit
+            index, out = LookupPoolFunction.apply(hashtable._backward_holder, impl, plan, weight, offsets,
+                                                  opt.combiner, readonly)
+            hashtable._filter_hook_impl(index)
+            return out
+        readonly = (not hashtable.training) or opt.admit_hook is not None
+        index = impl.lookup_index(plan.unique.detach(), readonly)
+        if hashtable.training and not readonly:
+            hashtable._filter_hook_impl(index)
+        chunks, chunk_rows = impl.emb_blocks()
+        return ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets,
+                                                 opt.combiner)
+    emb = lookup_unique_rows(hashtable, plan.unique, opt.admit_hook, opt.trainable)
+    inverse = plan.inverse
+    if id_mean:
+        # mean over the duplicates of each id: pool the expanded rows instead
+        emb = GradIDMeanFunction.apply(emb, inverse, plan)
+        inverse, plan = None, None
+    if weight is not None and weight.dtype != emb.dtype:
+        weight = weight.to(emb.dtype)
+    return ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner, opt.combiner_kwargs,
+                                           plan=plan)
+
+
 class DynamicEmbedding(torch.nn.Module):
     def __init__(self, emb_opt: EmbeddingOption, pg=None):
         super().__init__()
@@ -134,16 +202,7 @@ class DynamicEmbedding(torch.nn.Module):
         if weight is not None:
             weight = weight.to(dev) if opt.use_weight else None
         plan = ops.ids_unique_plan(val)
-        uniq, inverse = plan.unique, plan.inverse
-        emb = lookup_unique_rows(self._hashtable, uniq, opt.admit_hook, opt.trainable)
-        if opt.grad_reduce_by == "id" and self.training and opt.trainable:
-            # mean over the duplicates of each id: pool the expanded rows instead
-            emb = GradIDMeanFunction.apply(emb, inverse, plan)
-            inverse, plan = None, None
-        if weight is not None and weight.dtype != emb.dtype:
-            weight = weight.to(emb.dtype)
-        out = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner, opt.combiner_kwargs,
-                                              plan=plan)
+        out = lookup_and_pool(self._hashtable, plan, weight, offsets, opt)
         if opt.combiner == "tile":
             return out.view(tuple(shape) + (opt.combiner_kwargs["tile_len"] * opt.embedding_dim,))
         return out.view(tuple(shape) + (opt.embedding_dim,))

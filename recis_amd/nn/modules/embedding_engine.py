@@ -21,8 +21,7 @@ import torch
 
 from ... import ops
 from ...ragged.tensor import RaggedTensor
-from ..functional.embedding_ops import ragged_embedding_segment_reduce
-from .embedding import EmbeddingOption, lookup_unique_rows
+from .embedding import EmbeddingOption, lookup_and_pool
 from .hashtable import HashTable, gen_slice
 
 
@@ -126,12 +125,7 @@ class EmbeddingEngine(torch.nn.Module):
                 if all(w is not None for w in weights):
                     weight = weights[0] if len(weights) == 1 else torch.cat(weights)
                 plan = ops.ids_unique_plan(ids)
-                inverse = plan.inverse
-                emb = lookup_unique_rows(table, plan.unique, opt0.admit_hook, opt0.trainable)
-                if weight is not None and weight.dtype != emb.dtype:
-                    weight = weight.to(emb.dtype)
-                pooled = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt0.combiner,
-                                                         opt0.combiner_kwargs, plan=plan)
+                pooled = lookup_and_pool(table, plan, weight, offsets, opt0)
                 seg_counts = [o.numel() - 1 for o in offs]
                 width = pooled.shape[1]
                 for name, part, shape in zip(names, torch.split(pooled, seg_counts), shapes):

@@ -363,6 +363,18 @@ class HashtableImpl:
     def lookup_index_readonly(self, ids):
         return self._idmap.lookup_readonly(ids.to(self._device))
 
+    def emb_blocks(self):
+        """(chunk list, rows per chunk) of the embedding slot, as the row kernels take them
+        (no read-back of the allocator state)."""
+        return self._slot_group.emb_slot().kernel_blocks()
+
+    def lookup_index(self, ids, readonly=False):
+        """Row index of ``ids`` (inserting missing keys unless ``readonly``) without
+        gathering the rows: for consumers that read the rows out of the table themselves."""
+        if readonly:
+            return self.lookup_index_readonly(ids)
+        return self.insert_lookup_index(ids)
+
     # -------------------------------------------------------------- grads
     def accept_grad(self, grad_index, grad, unique=False):
         """``unique=True``: the caller knows ``grad_index`` has no duplicates (it is the

@@ -69,6 +69,35 @@ def segment_reduce_forward(unique_emb, weight, reverse_indices, offsets, mode, *
     return out
 
 
+def segment_reduce_forward_blocks(emb_blocks, block_size, row_index, weight, reverse_indices, offsets, mode, *,
+                                  out_dtype=None):
+    """``segment_reduce_forward`` over rows that stay where the table keeps them: unique row
+    ``u`` is row ``row_index[u]`` of ``emb_blocks`` (a negative index reads as zeros). Same
+    result as ``segment_reduce_forward(block_gather(row_index, emb_blocks, block_size, -1, True),
+    weight, reverse_indices, offsets, mode)`` without the ``[U, D]`` intermediate
+    (``recis_segment_reduce_forward_blocks``). ``mode``: "sum" | "mean" | "tile"."""
+    if mode not in ("sum", "mean", "tile"):
+        raise ValueError("Invalid mode for pooling out of the table: %s" % mode)
+    b0 = _check_blocks(emb_blocks, block_size)
+    require_cuda(row_index, weight, reverse_indices, offsets)
+    row_index = _ids64(row_index)
+    weight, reverse_indices, offsets = _contig(weight), _contig(reverse_indices), _contig(offsets)
+    U, D = row_index.numel(), b0[0].numel()
+    S = offsets.numel() - 1
+    B = reverse_indices.numel() if reverse_indices is not None else U
+    out_dtype = out_dtype or b0.dtype
+    out = torch.empty((B if mode == "tile" else S, D), dtype=out_dtype, device=b0.device)
+    tab = block_ptr_table(emb_blocks)
+    check(lib().recis_segment_reduce_forward_blocks(
+        ptr(tab), i64(len(emb_blocks)), i64(block_size), ptr(row_index), dtype_code(b0.dtype),
+        ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
+        _rev_ptr(reverse_indices, offsets),
+        _index_kind(reverse_indices, "reverse_indices") if reverse_indices is not None else 1,
+        ptr(offsets), _index_kind(offsets, "offsets"), ptr(out), dtype_code(out_dtype),
+        i64(B), i64(U), i64(S), i64(D), _lib.MODES[mode], stream_ptr(b0.device)))
+    return out
+
+
 def segment_reduce_backward(grad_output, weight, reverse_indices, offsets, unique_size, mode, *,
                             rev_unique=False, argmax=None, out_dtype=None):
     """``torch.ops.recis.segment_reduce_backward`` (embedding_segment_reduce.h:14-17).

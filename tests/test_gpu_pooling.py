@@ -166,6 +166,43 @@ def test_half_storage_fp32_accumulate(rng, dtype, D):
     np.testing.assert_allclose(got, exp, rtol=1e-5, atol=2e-5)
 
 
+@pytest.mark.parametrize("mode", ["sum", "mean", "tile"])
+@pytest.mark.parametrize("D,dtype,lo,hi", [(16, torch.float32, 0, 3), (64, torch.float32, 5, 60),
+                                           (128, torch.bfloat16, 10, 90), (40, torch.float32, 0, 12)])
+def test_forward_out_of_table_blocks(rng, mode, D, dtype, lo, hi):
+    """Pooling straight out of the table blocks (row u = row row_index[u] of the block list, absent
+    keys read as zeros) against the oracle on the gathered rows, and bit-identical to
+    block_gather + segment_reduce_forward on the device (same kernels, same summation order);
+    one-row segments, multi-row segments, several blocks, weights, int32 / int64 indices."""
+    bs, nb, U, S = 700, 5, 1500, 900
+    blocks_np = [rng.standard_normal((bs, D)).astype(np.float32) for _ in range(nb)]
+    blocks = [_dev(b, dtype) for b in blocks_np]
+    table = torch.cat(blocks).float().cpu().numpy()
+    row_index = rng.permutation(bs * nb)[:U].astype(np.int64)
+    row_index[rng.integers(0, U, size=40)] = -1
+    rows = np.where(row_index[:, None] >= 0, table[np.maximum(row_index, 0)], 0).astype(np.float32)
+    off = ragged_offsets(rng, S, lo, hi, 0.1)
+    B = int(off[-1])
+    rev = rng.integers(0, U, size=B)
+    w = rng.random(B).astype(np.float32)
+    for use_w, rev_dt in ((False, np.int32), (True, np.int64), (False, np.int64)):
+        wt = _dev(w, dtype) if use_w else None
+        got = ops.segment_reduce_forward_blocks(blocks, bs, _dev(row_index), wt, _dev(rev.astype(rev_dt)),
+                                                _dev(off.astype(np.int32)), mode, out_dtype=torch.float32)
+        dense = ops.block_gather(_dev(row_index), blocks, bs, -1, True)
+        ref = ops.segment_reduce_forward(dense, wt, _dev(rev.astype(rev_dt)), _dev(off.astype(np.int32)), mode,
+                                         out_dtype=torch.float32)
+        assert torch.equal(got, ref)
+        wq = wt.float().cpu().numpy() if use_w else None
+        if mode == "tile":
+            exp = rows[rev] * (wq[:, None] if use_w else 1.0)
+            np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-6, atol=1e-6)
+        else:
+            _assert_pool_close(got.cpu().numpy(), rows, wq, rev, off, mode)
+    with pytest.raises(ValueError):
+        ops.segment_reduce_forward_blocks(blocks, bs, _dev(row_index), None, _dev(rev), _dev(off), "max")
+
+
 def test_out_of_range_index_is_reported_not_faulting(rng):
     from recis_amd import _lib
 
