@@ -73,7 +73,20 @@ def i64(x):
     return ctypes.c_int64(int(x))
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device=None):
+    """The current HIP stream of ``device`` as a void pointer (called once or more per op: the
+    raw getter is several times cheaper than building a ``torch.cuda.Stream`` object)."""
+    if _raw_stream is not None:
+        if device is None:
+            idx = torch.cuda.current_device()
+        else:
+            idx = device.index if isinstance(device, torch.device) else torch.device(device).index
+            if idx is None:
+                idx = torch.cuda.current_device()
+        return ctypes.c_void_p(_raw_stream(idx))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 

@@ -257,6 +257,9 @@ class SlotGroup:
     def capacity_rows(self):
         return self._n_chunks * self._chunk_rows
 
+    def chunk_rows(self):
+        return self._chunk_rows
+
     def ensure_rows(self, rows):
         need = (rows + self._chunk_rows - 1) // self._chunk_rows
         if need > self._n_chunks:
@@ -317,8 +320,14 @@ class HashtableImpl:
         self._rows_ub += incoming
         if self._rows_ub + 1 > sg.capacity_rows():
             self._rows_ub = self._idmap.id_num()  # synchronises
-            if self._rows_ub + 1 > sg.capacity_rows():
-                sg.ensure_rows(self._rows_ub + 1 + max(2 * incoming, sg.block_size()))
+            # Leave room for many calls of this size: the bound counts every looked-up key as
+            # new, so without headroom a table about as large as its batches would read the
+            # mark back (a pipeline bubble) every other step. Rows are cheap, bubbles are not --
+            # unless storage grows in chunks far larger than a batch (a pre-sized table).
+            roomy = sg.chunk_rows() <= 32 * max(incoming, 1)
+            want = self._rows_ub + 1 + max((16 if roomy else 2) * incoming, sg.block_size())
+            if want > sg.capacity_rows() and (roomy or self._rows_ub + 1 + incoming > sg.capacity_rows()):
+                sg.ensure_rows(want)
         if sg.capacity_rows() == 0:
             sg.ensure_rows(1)
 

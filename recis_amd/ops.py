@@ -179,9 +179,12 @@ def _row_bytes(block):
 
 
 def _ids64(ids):
-    require_cuda(ids)
+    if not ids.is_cuda:
+        require_cuda(ids)
     if ids.dtype != torch.int64:
         raise TypeError("ids must be int64, got %s" % ids.dtype)
+    if ids.dim() == 1 and ids.is_contiguous():
+        return ids
     return _contig(ids).view(-1)
 
 
