@@ -179,12 +179,14 @@ class Config4:
         return o.ids_encode(self.c["sparse"] + extra, self.tags)
 
     def dedup(self, ids):
-        self.plan = self.ops.ids_unique_plan(ids)
-        self.U = self.plan.U
-        return self.plan.unique, self.plan.inverse
+        self.plan = self.ops.ids_unique_plan(ids, wait=False)
+        return self.plan, self.plan.inverse
 
-    def lookup(self, uniq):
-        return self.table.lookup_index(uniq, False)
+    def lookup(self, plan):
+        # queued before the host has the unique count; the count arrives while plan and lookup run
+        index_buf = self.table.lookup_index_counted(plan)
+        self.U = plan.U
+        return self.table.settle_lookup(index_buf, self.U)
 
     def pool_fwd(self, index, inv):
         # pooling reads the rows out of the table (no [U, D] copy), as EmbeddingEngine does
@@ -315,9 +317,12 @@ class Config3:
         o = self.ops
         ids = self.batches[self.step_no % len(self.batches)]
         self.step_no += 1
-        plan = o.ids_unique_plan(ids)
+        plan = o.ids_unique_plan(ids, wait=False)
+        index_buf = self.table.lookup_index_counted(plan)   # queued before the host has the unique count
         self.U = plan.U
-        index, rows = self.table.embedding_lookup(plan.unique, False)
+        index = self.table.settle_lookup(index_buf, self.U)
+        chunks, chunk_rows = self.table.emb_blocks()
+        rows = o.block_gather(index, chunks, chunk_rows, -1, False)
         self.table.update_slot("step_filter", index, self.step_t)
         # one row per lookup, expanded from the [U, D] copy: with a 25 GB table, pooling out of the
         # table (segment_reduce_forward_blocks) gains nothing, the copy keeps the 2e6 reads local
@@ -409,10 +414,13 @@ class Config5:
     def step(self):
         o = self.ops
         ids = o.ids_encode([f["values"] for f in self.fields], list(range(len(self.fields))))
-        plan = o.ids_unique_plan(ids)
+        plan = o.ids_unique_plan(ids, wait=False)
+        index_buf = self.table.lookup_index_counted(plan)   # queued before the host has the unique count
         self.U = plan.U
         inv = plan.inverse
-        index, rows = self.table.embedding_lookup(plan.unique, False)
+        index = self.table.settle_lookup(index_buf, self.U)
+        chunks, chunk_rows = self.table.emb_blocks()
+        rows = o.block_gather(index, chunks, chunk_rows, -1, False)
         pooled = o.segment_reduce_forward(rows, None, inv, self.offsets, "mean", out_dtype=torch.float32)
         padded, batch_seq = o.ragged_tile(self.batch, self.seq, inv, self.offsets, rows)
         g = o.segment_reduce_backward_plan(self.g_pool, None, self.offsets, plan, "mean")

@@ -48,6 +48,8 @@ extern "C" {
 #define RECIS_PLAN_HOT_LEN 256
 #define RECIS_PLAN_HOT_CHUNK 2048
 
+#define RECIS_PLAN_STAGE_COUNT 1
+
 #define RECIS_FLAG_REV_UNIQUE 1 /* caller guarantees reverse_indices has no duplicates */
 
 /* bits of the device-side soft-error word (recis_hip_poll_device_errors) */
@@ -215,6 +217,21 @@ int recis_idmap_destroy(recis_idmap* m);
  */
 int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* index_out,
                        void* stream);
+/* recis_idmap_lookup for a batch whose size is still on the device (the unique ids of a batch
+ * plan whose count the host has not read yet): the first min(*n_dev, n_max) ids are looked up,
+ * index_out[i] for i beyond them is left untouched. Lets the host queue the lookup behind the
+ * plan and fetch the count while both run. No counterpart in the reference (its
+ * GpuIdMap::Lookup sizes everything on the host, gpu_id_map.cu:19-45). */
+int recis_idmap_lookup_counted(recis_idmap* m, const int64_t* ids, int64_t n_max,
+                               const int64_t* n_dev, int64_t* index_out, void* stream);
+/* Tells the map the true size of the last recis_idmap_lookup_counted once the host knows it,
+ * so that the bounds below stop counting all n_max ids of that call as possible new keys. */
+int recis_idmap_settle_count(recis_idmap* m, int64_t n_true);
+/* Upper bounds, without waiting for any stream, of the allocator's high-water mark
+ * (IdMap::GetIdNum, id_map.h:29) and of the occupied table slots: the values the last finished
+ * call published to pinned host memory plus every id of the calls queued since. Either
+ * pointer may be NULL. For callers that size row storage ahead of the device. */
+int recis_idmap_bounds(recis_idmap* m, int64_t* id_num_ub, int64_t* occupied_ub);
 /* GpuIdMap::LookupReadOnly (gpu_id_map.cu:47-62): -1 for a missing key. */
 int recis_idmap_lookup_readonly(recis_idmap* m, const int64_t* ids, int64_t n,
                                 int64_t* index_out, void* stream);
@@ -371,6 +388,9 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
  *   unique_count_host      host word or NULL: when given, the call returns only once the number
  *                          of unique ids is known and stores it there (the last kernels of the
  *                          plan may still be running: the wait is for the count alone)
+ *   flags                  RECIS_PLAN_STAGE_COUNT: send the count towards the host but do not
+ *                          wait; recis_unique_plan_count(stream) fetches it later (one staged
+ *                          count per stream: fetch it before the next plan on that stream)
  * The unique ids are ordered by (hash bucket, first occurrence): the order, the inverse and
  * row_start depend on the input only; the order of the entries inside one id's list and of
  * the hot items is not specified. No global atomics are used: ids are partitioned by hash
@@ -384,7 +404,9 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
 int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
                       int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
                       int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev,
-                      int64_t* unique_count_host, void* stream);
+                      int64_t* unique_count_host, int flags, void* stream);
+/* Waits for the count staged by the last recis_unique_plan(…, RECIS_PLAN_STAGE_COUNT, stream). */
+int recis_unique_plan_count(int64_t* unique_count_host, void* stream);
 
 /*
  * Per list entry, the input row it reads and its coefficient, for the backward of

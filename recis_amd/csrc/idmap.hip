@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <deque>
+#include <utility>
 
 #include "common.cuh"
 
@@ -50,6 +52,29 @@ __device__ __forceinline__ uint64_t mix_key(int64_t key) {
 // plan ordered by the top bits of the same mix, so their probes walk the table front to back.
 __device__ __forceinline__ uint64_t home_slot(int64_t key, uint64_t mask) {
   return mix_key(key) >> __builtin_clzll(mask);  // mask = capacity - 1, capacity a power of two >= 2
+}
+
+// Number of ids of a call whose count is still on the device: the first *n_dev of n_max.
+__device__ __forceinline__ int64_t counted(int64_t n_max, const int64_t* n_dev) {
+  if (n_dev == nullptr) return n_max;
+  const int64_t n = *n_dev;
+  return n < 0 ? 0 : (n < n_max ? n : n_max);
+}
+
+// Allocator words the host wants to know without waiting for the stream: written by the
+// last kernel of every call that changes them into pinned host memory, stamped with the
+// call's sequence number (written last, after a system-scope fence).
+enum { MR_SEQ = 0, MR_CUR, MR_FREE, MR_LIVE, MR_OCC, MR_WORDS };
+__device__ __forceinline__ void publish(const int64_t* state, volatile int64_t* mirror, int64_t seq) {
+  mirror[MR_CUR] = state[ST_CUR];
+  mirror[MR_FREE] = state[ST_FREE];
+  mirror[MR_LIVE] = state[ST_LIVE];
+  mirror[MR_OCC] = state[ST_OCC];
+  __threadfence_system();
+  mirror[MR_SEQ] = seq;
+}
+__global__ void publish_kernel(const int64_t* state, volatile int64_t* mirror, int64_t seq) {
+  publish(state, mirror, seq);
 }
 
 __device__ __forceinline__ int64_t ld_relaxed(const int64_t* p) {
@@ -98,8 +123,10 @@ __device__ __forceinline__ void block_rank(bool flag, int& rank, int& total) {
 // inserted by another thread of this call, slot = -(slotpos + 2).
 __global__ void __launch_bounds__(kBlock)
 find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __restrict__ ids,
-                     int64_t n, int64_t* __restrict__ out, int64_t* __restrict__ slotpos,
-                     int32_t* __restrict__ block_counts, int64_t* __restrict__ state, int* err) {
+                     int64_t n, const int64_t* __restrict__ n_dev, int64_t* __restrict__ out,
+                     int64_t* __restrict__ slotpos, int32_t* __restrict__ block_counts,
+                     int64_t* __restrict__ state, int* err) {
+  n = counted(n, n_dev);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   bool is_new = false;
   bool took_empty = false;
@@ -188,7 +215,8 @@ find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __r
 // Pass 2: exclusive scan of the per-block counts (single workgroup) and the
 // allocator bookkeeping of IdAllocator::GenIds (id_allocator.cc:17-26).
 __global__ void __launch_bounds__(1024)
-scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t* __restrict__ state) {
+scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t* __restrict__ state,
+                   volatile int64_t* mirror, int64_t seq) {
   __shared__ int64_t partial[1024];
   const int t = threadIdx.x;
   const int64_t per = (nb + 1023) / 1024;
@@ -220,6 +248,8 @@ scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t* __re
     state[ST_CUR] = cur + fresh;
     state[ST_FREE] = fr >= total ? fr - total : 0;
     state[ST_LIVE] += total;
+    __threadfence();
+    publish(state, mirror, seq);
   }
 }
 
@@ -227,8 +257,10 @@ scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t* __re
 // hashtable_ops.cc:15-27) in input order.
 __global__ void __launch_bounds__(kBlock)
 assign_rows_kernel(Slot* __restrict__ table, const int64_t* __restrict__ slotpos, int64_t n,
-                   const int32_t* __restrict__ block_prefix, const int64_t* __restrict__ state,
-                   const int64_t* __restrict__ free_list, int64_t* __restrict__ out) {
+                   const int64_t* __restrict__ n_dev, const int32_t* __restrict__ block_prefix,
+                   const int64_t* __restrict__ state, const int64_t* __restrict__ free_list,
+                   int64_t* __restrict__ out) {
+  n = counted(n, n_dev);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   const int64_t sp = i < n ? slotpos[i] : -1;
   const bool is_new = sp >= 0;
@@ -245,8 +277,10 @@ assign_rows_kernel(Slot* __restrict__ table, const int64_t* __restrict__ slotpos
 // Pass 4: occurrences whose key was claimed by another occurrence of the same call.
 __global__ void __launch_bounds__(kBlock)
 resolve_dups_kernel(const Slot* __restrict__ table, const int64_t* __restrict__ slotpos, int64_t n,
-                    const int64_t* __restrict__ state, int64_t* __restrict__ out) {
+                    const int64_t* __restrict__ n_dev, const int64_t* __restrict__ state,
+                    int64_t* __restrict__ out) {
   if (state[ST_DUPS] == 0) return;
+  n = counted(n, n_dev);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   if (i >= n) return;
   const int64_t sp = slotpos[i];
@@ -497,6 +531,10 @@ struct recis_idmap {
   int64_t occ_ub = 0;   // non-empty slots (live + tombstones)
   int64_t free_ub = 0;  // entries in the free list
   int* err = nullptr;
+  // pinned host mirror of the allocator words + the calls whose publication has not landed yet
+  volatile int64_t* mirror = nullptr;
+  int64_t seq_issued = 0;
+  std::deque<std::pair<int64_t, int64_t>> in_flight;  // (sequence number, ids of the call)
 };
 
 namespace {
@@ -512,12 +550,43 @@ int alloc_table(recis_idmap* m, int64_t capacity, hipStream_t stream, Slot** out
   return RECIS_OK;
 }
 
+void mirror_set(recis_idmap* m, const int64_t* words);
+
 int sync_stats(recis_idmap* m, hipStream_t stream, int64_t* words) {
   RECIS_CHECK_HIP(hipMemcpyAsync(words, m->state, sizeof(int64_t) * ST_WORDS, hipMemcpyDeviceToHost, stream));
   RECIS_CHECK_HIP(hipStreamSynchronize(stream));
   m->occ_ub = words[ST_OCC];
   m->free_ub = words[ST_FREE];
+  mirror_set(m, words);
   return RECIS_OK;
+}
+
+// Upper bounds of occupied slots and of the allocator's high-water mark from the mirror, without
+// waiting: what the last landed publication says plus every id of the calls issued after it.
+void mirror_bounds(recis_idmap* m, int64_t* occ_ub, int64_t* cur_ub) {
+  int64_t seq, occ, cur;
+  do {
+    seq = m->mirror[MR_SEQ];
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    occ = m->mirror[MR_OCC];
+    cur = m->mirror[MR_CUR];
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+  } while (seq != m->mirror[MR_SEQ]);
+  while (!m->in_flight.empty() && m->in_flight.front().first <= seq) m->in_flight.pop_front();
+  int64_t pending = 0;
+  for (const auto& c : m->in_flight) pending += c.second;
+  if (occ_ub) *occ_ub = occ + pending;
+  if (cur_ub) *cur_ub = cur + pending;
+}
+
+// After the stream has been drained and `words` read back: the mirror is exact.
+void mirror_set(recis_idmap* m, const int64_t* words) {
+  m->mirror[MR_CUR] = words[ST_CUR];
+  m->mirror[MR_FREE] = words[ST_FREE];
+  m->mirror[MR_LIVE] = words[ST_LIVE];
+  m->mirror[MR_OCC] = words[ST_OCC];
+  m->mirror[MR_SEQ] = m->seq_issued;
+  m->in_flight.clear();
 }
 
 int rebuild(recis_idmap* m, int64_t new_capacity, hipStream_t stream) {
@@ -536,11 +605,13 @@ int rebuild(recis_idmap* m, int64_t new_capacity, hipStream_t stream) {
   m->table = nt;
   m->capacity = new_capacity;
   m->occ_ub = words[ST_LIVE];
+  m->mirror[MR_OCC] = words[ST_LIVE];
   return RECIS_OK;
 }
 
 // Make room for up to `incoming` more claimed slots.
 int ensure_table_room(recis_idmap* m, int64_t incoming, hipStream_t stream) {
+  mirror_bounds(m, &m->occ_ub, nullptr);
   if ((m->occ_ub + incoming) * 2 <= m->capacity) return RECIS_OK;
   int64_t words[ST_WORDS];
   if (int rc = sync_stats(m, stream, words)) return rc;
@@ -592,8 +663,18 @@ int recis_idmap_create(int64_t reserve_keys, recis_idmap** out) {
     zero_words_kernel<<<1, 64>>>(m->state, ST_WORDS);
     if (hipStreamSynchronize(nullptr) != hipSuccess) rc = fail(RECIS_ERR_HIP, "id-map initialisation failed");
   }
+  if (rc == RECIS_OK) {
+    void* mp = nullptr;
+    if (hipHostMalloc(&mp, sizeof(int64_t) * MR_WORDS, hipHostMallocDefault) != hipSuccess) {
+      rc = fail(RECIS_ERR_HIP, "hipHostMalloc of the allocator mirror failed");
+    } else {
+      m->mirror = static_cast<volatile int64_t*>(mp);
+      for (int w = 0; w < MR_WORDS; ++w) m->mirror[w] = 0;
+    }
+  }
   if (rc == RECIS_OK) rc = ensure_free_room(m, 10240, nullptr);
   if (rc != RECIS_OK) {
+    if (m->mirror) (void)hipHostFree(const_cast<int64_t*>(m->mirror));
     if (m->table) (void)hipFree(m->table);
     if (m->state) (void)hipFree(m->state);
     delete m;
@@ -609,13 +690,13 @@ int recis_idmap_destroy(recis_idmap* m) {
   if (m->table) (void)hipFree(m->table);
   if (m->state) (void)hipFree(m->state);
   if (m->free_list) (void)hipFree(m->free_list);
+  if (m->mirror) (void)hipHostFree(const_cast<int64_t*>(m->mirror));
   delete m;
   return RECIS_OK;
 }
 
-int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* index_out,
-                       void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
+static int lookup_impl(recis_idmap* m, const int64_t* ids, int64_t n, const int64_t* n_dev, int64_t* index_out,
+                       hipStream_t stream) {
   RECIS_REQUIRE(m != nullptr, "id map is NULL");
   RECIS_REQUIRE(n >= 0 && n < (int64_t(1) << 31), "n out of range: %lld", (long long)n);
   if (n == 0) return RECIS_OK;
@@ -628,20 +709,45 @@ int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* i
   int64_t* slotpos = static_cast<int64_t*>(ws);
   int32_t* block_counts = reinterpret_cast<int32_t*>(slotpos + n);
   const uint64_t mask = static_cast<uint64_t>(m->capacity - 1);
+  const int64_t seq = ++m->seq_issued;
 
   reset_dups_kernel<<<1, 1, 0, stream>>>(m->state);
   RECIS_TIME_KERNEL("find_or_claim_kernel", stream)
-  find_or_claim_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, mask, ids, n, index_out, slotpos,
+  find_or_claim_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, mask, ids, n, n_dev, index_out, slotpos,
                                                              block_counts, m->state, m->err);
   RECIS_LAUNCH_CHECK();
-  scan_commit_kernel<<<1, 1024, 0, stream>>>(block_counts, nb, m->state);
+  scan_commit_kernel<<<1, 1024, 0, stream>>>(block_counts, nb, m->state, m->mirror, seq);
   RECIS_LAUNCH_CHECK();
-  assign_rows_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, block_counts, m->state,
+  assign_rows_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, n_dev, block_counts, m->state,
                                                            m->free_list, index_out);
   RECIS_LAUNCH_CHECK();
-  resolve_dups_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, m->state, index_out);
+  resolve_dups_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, n_dev, m->state, index_out);
   RECIS_LAUNCH_CHECK();
-  m->occ_ub += n;
+  m->in_flight.emplace_back(seq, n);
+  return RECIS_OK;
+}
+
+int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* index_out,
+                       void* stream_) {
+  return lookup_impl(m, ids, n, nullptr, index_out, static_cast<hipStream_t>(stream_));
+}
+
+int recis_idmap_lookup_counted(recis_idmap* m, const int64_t* ids, int64_t n_max, const int64_t* n_dev,
+                               int64_t* index_out, void* stream_) {
+  RECIS_REQUIRE(n_dev != nullptr, "n_dev must not be NULL");
+  return lookup_impl(m, ids, n_max, n_dev, index_out, static_cast<hipStream_t>(stream_));
+}
+
+int recis_idmap_settle_count(recis_idmap* m, int64_t n_true) {
+  RECIS_REQUIRE(m != nullptr && n_true >= 0, "bad arguments");
+  if (!m->in_flight.empty() && m->in_flight.back().first == m->seq_issued && m->in_flight.back().second > n_true)
+    m->in_flight.back().second = n_true;
+  return RECIS_OK;
+}
+
+int recis_idmap_bounds(recis_idmap* m, int64_t* id_num_ub, int64_t* occupied_ub) {
+  RECIS_REQUIRE(m != nullptr, "id map is NULL");
+  mirror_bounds(m, occupied_ub, id_num_ub);
   return RECIS_OK;
 }
 
@@ -739,7 +845,10 @@ int recis_idmap_clear(recis_idmap* m, void* stream_) {
   RECIS_LAUNCH_CHECK();
   zero_words_kernel<<<1, 64, 0, stream>>>(m->state, ST_WORDS);
   RECIS_LAUNCH_CHECK();
-  m->occ_ub = 0;
+  const int64_t seq = ++m->seq_issued;
+  publish_kernel<<<1, 1, 0, stream>>>(m->state, m->mirror, seq);
+  RECIS_LAUNCH_CHECK();
+  m->in_flight.emplace_back(seq, 0);
   m->free_ub = 0;
   return RECIS_OK;
 }

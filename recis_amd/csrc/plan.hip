@@ -897,7 +897,7 @@ extern "C" {
 
 int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
                       int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
-                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* unique_count_host, void* stream_) {
+                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* unique_count_host, int flags, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   RECIS_REQUIRE(n >= 0 && n < (int64_t(1) << 30), "n out of range: %lld", (long long)n);
   RECIS_REQUIRE(counts_out_dev && row_start_out, "counts_out_dev / row_start_out must not be NULL");
@@ -910,6 +910,13 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
     plan_empty_kernel<<<1, 64, 0, stream>>>(counts_out_dev, row_start_out);
     RECIS_LAUNCH_CHECK();
     if (unique_count_host) *unique_count_host = 0;
+    if (flags & RECIS_PLAN_STAGE_COUNT) {
+      int64_t* staged = nullptr;
+      hipEvent_t staged_event = nullptr;
+      if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
+      RECIS_CHECK_HIP(hipMemcpyAsync(staged, counts_out_dev, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+      RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
+    }
     return RECIS_OK;
   }
   PlanGeom g;
@@ -986,7 +993,7 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   // are queued, so that the GPU works while the host learns the size of the next launches.
   int64_t* staged = nullptr;
   hipEvent_t staged_event = nullptr;
-  if (unique_count_host) {
+  if (unique_count_host || (flags & RECIS_PLAN_STAGE_COUNT)) {
     if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
     RECIS_CHECK_HIP(hipMemcpyAsync(staged, counts_out_dev, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
     RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
@@ -1009,6 +1016,17 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
     RECIS_CHECK_HIP(hipEventSynchronize(staged_event));
     *unique_count_host = *staged;
   }
+  return RECIS_OK;
+}
+
+int recis_unique_plan_count(int64_t* unique_count_host, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(unique_count_host != nullptr, "unique_count_host must not be NULL");
+  int64_t* staged = nullptr;
+  hipEvent_t staged_event = nullptr;
+  if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
+  RECIS_CHECK_HIP(hipEventSynchronize(staged_event));
+  *unique_count_host = *staged;
   return RECIS_OK;
 }
 

@@ -96,7 +96,13 @@ class LookupPoolFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly):
-        index = impl.lookup_index(plan.unique, readonly)
+        if readonly:
+            index = impl.lookup_index(plan.unique, True)
+        else:
+            # queued behind the plan before the host has the unique count: the count arrives
+            # while the plan's last kernels and the lookup run
+            index_buf = impl.lookup_index_counted(plan)
+            index = impl.settle_lookup(index_buf, plan.U)
         chunks, chunk_rows = impl.emb_blocks()
         out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets, combiner)
         ctx.impl, ctx.plan, ctx.combiner, ctx.readonly = impl, plan, combiner, readonly
@@ -201,7 +207,7 @@ class DynamicEmbedding(torch.nn.Module):
             weight = input_weights
         if weight is not None:
             weight = weight.to(dev) if opt.use_weight else None
-        plan = ops.ids_unique_plan(val)
+        plan = ops.ids_unique_plan(val, wait=False)
         out = lookup_and_pool(self._hashtable, plan, weight, offsets, opt)
         if opt.combiner == "tile":
             return out.view(tuple(shape) + (opt.combiner_kwargs["tile_len"] * opt.embedding_dim,))

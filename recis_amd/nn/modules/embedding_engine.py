@@ -124,7 +124,7 @@ class EmbeddingEngine(torch.nn.Module):
                 weight = None
                 if all(w is not None for w in weights):
                     weight = weights[0] if len(weights) == 1 else torch.cat(weights)
-                plan = ops.ids_unique_plan(ids)
+                plan = ops.ids_unique_plan(ids, wait=False)
                 pooled = lookup_and_pool(table, plan, weight, offsets, opt0)
                 seg_counts = [o.numel() - 1 for o in offs]
                 width = pooled.shape[1]

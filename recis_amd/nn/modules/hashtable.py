@@ -314,19 +314,19 @@ class HashtableImpl:
     # ------------------------------------------------------------- storage
     def _make_room(self, incoming):
         """After a find-or-insert of ``incoming`` keys: rows up to the allocator's
-        high-water mark (+1 spare) must exist before any row kernel runs. The exact
-        mark is read back only when the running upper bound passes the capacity."""
+        high-water mark (+1 spare) must exist before any row kernel runs. The map keeps an
+        upper bound of the mark on the host (what the last finished call published plus every
+        id queued since); the exact mark is read back only when that bound passes the
+        capacity."""
         sg = self._slot_group
-        self._rows_ub += incoming
-        if self._rows_ub + 1 > sg.capacity_rows():
-            self._rows_ub = self._idmap.id_num()  # synchronises
-            # Leave room for many calls of this size: the bound counts every looked-up key as
-            # new, so without headroom a table about as large as its batches would read the
-            # mark back (a pipeline bubble) every other step. Rows are cheap, bubbles are not --
-            # unless storage grows in chunks far larger than a batch (a pre-sized table).
+        ub = self._idmap.id_num_bound()
+        if ub + 1 > sg.capacity_rows():
+            ub = self._idmap.id_num()  # synchronises
+            # Leave room for many calls of this size, unless storage grows in chunks far larger
+            # than a batch (a pre-sized table): rows are cheap, pipeline bubbles are not.
             roomy = sg.chunk_rows() <= 32 * max(incoming, 1)
-            want = self._rows_ub + 1 + max((16 if roomy else 2) * incoming, sg.block_size())
-            if want > sg.capacity_rows() and (roomy or self._rows_ub + 1 + incoming > sg.capacity_rows()):
+            want = ub + 1 + max((16 if roomy else 2) * incoming, sg.block_size())
+            if want > sg.capacity_rows() and (roomy or ub + 1 + incoming > sg.capacity_rows()):
                 sg.ensure_rows(want)
         if sg.capacity_rows() == 0:
             sg.ensure_rows(1)
@@ -376,6 +376,16 @@ class HashtableImpl:
         """(chunk list, rows per chunk) of the embedding slot, as the row kernels take them
         (no read-back of the allocator state)."""
         return self._slot_group.emb_slot().kernel_blocks()
+
+    def lookup_index_counted(self, plan):
+        """Queue the find-or-insert of a plan's unique ids before the host knows how many
+        there are; finish with ``settle_lookup`` once ``plan.U`` has been read."""
+        return self._idmap.lookup_counted(plan.unique_buf, plan.counts)
+
+    def settle_lookup(self, index_buf, n_true):
+        self._idmap.settle_count(n_true)
+        self._make_room(n_true)
+        return index_buf[:n_true]
 
     def lookup_index(self, ids, readonly=False):
         """Row index of ``ids`` (inserting missing keys unless ``readonly``) without

@@ -639,6 +639,25 @@ class IdMap:
         check(lib().recis_idmap_lookup(self._h, ptr(ids), i64(ids.numel()), ptr(out), stream_ptr(ids.device)))
         return out
 
+    def lookup_counted(self, ids_buf, n_dev):
+        """Find-or-insert of the first ``n_dev[0]`` (device word) ids of ``ids_buf``: queued
+        without the host knowing the count. Returns the full-length index buffer; entries
+        beyond the count are not written."""
+        ids_buf = _ids64(ids_buf)
+        out = torch.empty_like(ids_buf)
+        check(lib().recis_idmap_lookup_counted(self._h, ptr(ids_buf), i64(ids_buf.numel()), ptr(n_dev), ptr(out),
+                                               stream_ptr(self.device)))
+        return out
+
+    def settle_count(self, n_true):
+        check(lib().recis_idmap_settle_count(self._h, i64(n_true)))
+
+    def id_num_bound(self):
+        """Upper bound of ``id_num()`` without waiting for the device."""
+        v = ctypes.c_int64(0)
+        check(lib().recis_idmap_bounds(self._h, ctypes.byref(v), None))
+        return v.value
+
     def lookup_readonly(self, ids):
         ids = _ids64(ids)
         out = torch.empty(ids.numel(), dtype=torch.int64, device=ids.device)
@@ -701,17 +720,41 @@ class IdMap:
 _HOT_LEN, _HOT_CHUNK = 256, 2048  # RECIS_PLAN_HOT_LEN / RECIS_PLAN_HOT_CHUNK of the library
 
 
+_STAGED = {}  # stream -> the plan whose count is on its way to that stream's staging word
+
+
 class BatchPlan:
     """Dedup of one batch of ids plus the occurrence lists per unique id.
 
     ``unique`` [U], ``inverse`` int32 [N] (``unique[inverse] == ids``), ``row_start`` int32
     [N + 1] and ``occ`` int32 [N]: the occurrences of unique id ``u`` are
     ``occ[row_start[u]:row_start[u + 1]]``; ``pos`` [N] is the position of each occurrence
-    in ``occ``. ``U`` is the host copy of the unique count (reading it synchronises once).
+    in ``occ``. ``U`` is the host copy of the unique count. A plan made with ``wait=False``
+    fetches it on first use of ``U`` / ``unique`` (the count is on its way by then);
+    ``unique_buf`` [N] and ``counts`` (device) are there at once, for work that can be
+    queued before the host knows ``U`` (``IdMap.lookup_counted``).
     """
 
-    __slots__ = ("n", "U", "unique", "inverse", "row_start", "occ", "pos", "hot_items", "hot_cap", "counts",
-                 "_pool_fill")
+    __slots__ = ("n", "_U", "_unique", "unique_buf", "inverse", "row_start", "occ", "pos", "hot_items", "hot_cap",
+                 "counts", "_pool_fill", "_stream")
+
+    @property
+    def U(self):
+        if self._U is None:
+            if _STAGED.get(self._stream.value) is self:
+                count = ctypes.c_int64(0)
+                check(lib().recis_unique_plan_count(ctypes.byref(count), self._stream))
+                self._U = int(count.value)
+                _STAGED.pop(self._stream.value, None)
+            else:  # a later plan took the stream's staging word: read this plan's own device word
+                self._U = int(self.counts[0].item())
+        return self._U
+
+    @property
+    def unique(self):
+        if self._unique is None:
+            self._unique = self.unique_buf[: self.U]
+        return self._unique
 
     def src_coef_for_pool(self, offsets, weight, mean):
         """(src, coef) per list entry for the backward of pooled segments, cached per
@@ -743,14 +786,16 @@ class BatchPlan:
         return src
 
 
-def ids_unique_plan(ids):
-    """Dedup + transposed index of a batch of ids (``recis_unique_plan``)."""
+def ids_unique_plan(ids, wait=True):
+    """Dedup + transposed index of a batch of ids (``recis_unique_plan``). ``wait=False``
+    returns without the host copy of the unique count (see ``BatchPlan``); at most one such
+    plan per stream may have its count outstanding."""
     ids = _ids64(ids)
     n = ids.numel()
     dev = ids.device
     p = BatchPlan()
     p.n = n
-    uniq = torch.empty(n, dtype=torch.int64, device=dev)
+    p.unique_buf = torch.empty(n, dtype=torch.int64, device=dev)
     p.inverse = torch.empty(n, dtype=torch.int32, device=dev)
     p.row_start = torch.empty(n + 1, dtype=torch.int32, device=dev)
     p.occ = torch.empty(n, dtype=torch.int32, device=dev)
@@ -759,12 +804,15 @@ def ids_unique_plan(ids):
     p.hot_items = torch.empty(2 * p.hot_cap, dtype=torch.int32, device=dev)
     p.counts = torch.empty(2, dtype=torch.int64, device=dev)
     p._pool_fill = None
+    p._unique = None
+    p._stream = stream_ptr(dev)
     count = ctypes.c_int64(0)
-    check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(uniq), ptr(p.inverse), ptr(p.row_start), ptr(p.occ),
-                                  ptr(p.pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts), ctypes.byref(count),
-                                  stream_ptr(dev)))
-    p.U = int(count.value)
-    p.unique = uniq[: p.U]
+    check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(p.unique_buf), ptr(p.inverse), ptr(p.row_start), ptr(p.occ),
+                                  ptr(p.pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts),
+                                  ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
+    p._U = int(count.value) if wait else None
+    if not wait:
+        _STAGED[p._stream.value] = p
     return p
 
 
