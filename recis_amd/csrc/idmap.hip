@@ -215,8 +215,9 @@ find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __r
 // Pass 2: exclusive scan of the per-block counts (single workgroup) and the
 // allocator bookkeeping of IdAllocator::GenIds (id_allocator.cc:17-26).
 __global__ void __launch_bounds__(1024)
-scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t* __restrict__ state,
-                   volatile int64_t* mirror, int64_t seq) {
+scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t n, const int64_t* __restrict__ n_dev,
+                   int64_t* __restrict__ state, volatile int64_t* mirror, int64_t seq) {
+  nb = min(nb, (counted(n, n_dev) + kBlock - 1) / kBlock);  // later blocks hold nothing (and zero counts)
   __shared__ int64_t partial[1024];
   const int t = threadIdx.x;
   const int64_t per = (nb + 1023) / 1024;
@@ -716,7 +717,7 @@ static int lookup_impl(recis_idmap* m, const int64_t* ids, int64_t n, const int6
   find_or_claim_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, mask, ids, n, n_dev, index_out, slotpos,
                                                              block_counts, m->state, m->err);
   RECIS_LAUNCH_CHECK();
-  scan_commit_kernel<<<1, 1024, 0, stream>>>(block_counts, nb, m->state, m->mirror, seq);
+  scan_commit_kernel<<<1, 1024, 0, stream>>>(block_counts, nb, n, n_dev, m->state, m->mirror, seq);
   RECIS_LAUNCH_CHECK();
   assign_rows_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, n_dev, block_counts, m->state,
                                                            m->free_list, index_out);

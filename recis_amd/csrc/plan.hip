@@ -205,7 +205,8 @@ plan_colscan_kernel(const uint16_t* __restrict__ hist, PlanGeom g, int32_t* __re
 // out arrays have nb + 1 entries (the last one is the total); total of the first to total_out.
 __global__ void __launch_bounds__(1024)
 plan_scan_kernel(const int32_t* __restrict__ in0, int32_t* __restrict__ out0, const int32_t* __restrict__ in1,
-                 int32_t* __restrict__ out1, int nb, int64_t* __restrict__ total_out) {
+                 int32_t* __restrict__ out1, int nb, int64_t* __restrict__ total_out,
+                 volatile int64_t* total_host) {
   __shared__ int32_t partial[1024];
   const int t = threadIdx.x;
   const int per = (nb + 1023) / 1024;
@@ -233,6 +234,7 @@ plan_scan_kernel(const int32_t* __restrict__ in0, int32_t* __restrict__ out0, co
     if (t == 1023) {
       out[nb] = partial[1023];
       if (pass == 0 && total_out) total_out[0] = partial[1023];
+      if (pass == 0 && total_host) total_host[0] = partial[1023];  // pinned host word: no copy kernel needed
     }
     __syncthreads();
   }
@@ -973,7 +975,7 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
     RECIS_LAUNCH_CHECK();
   }
   plan_scan_kernel<<<1, 1024, 0, stream>>>(bucket_total, bucket_start, nullptr, nullptr, static_cast<int>(nb),
-                                           nullptr);
+                                           nullptr, nullptr);
   RECIS_LAUNCH_CHECK();
   {
     RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
@@ -987,17 +989,18 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
                                                                    ucnt, ocnt, err);
     RECIS_LAUNCH_CHECK();
   }
-  plan_scan_kernel<<<1, 1024, 0, stream>>>(ucnt, ubase, ocnt, lbase, static_cast<int>(nb), counts_out_dev);
-  RECIS_LAUNCH_CHECK();
-  // The count is final here: send it to the host now and wait for it only after the emit kernels
-  // are queued, so that the GPU works while the host learns the size of the next launches.
+  // The count is final after this scan: the kernel stores it into pinned host memory as well, and
+  // the host waits for it only after the emit kernels are queued, so that the GPU works while
+  // the host learns the size of the next launches.
   int64_t* staged = nullptr;
   hipEvent_t staged_event = nullptr;
-  if (unique_count_host || (flags & RECIS_PLAN_STAGE_COUNT)) {
+  const bool stage = unique_count_host || (flags & RECIS_PLAN_STAGE_COUNT);
+  if (stage) {
     if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
-    RECIS_CHECK_HIP(hipMemcpyAsync(staged, counts_out_dev, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
-    RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
   }
+  plan_scan_kernel<<<1, 1024, 0, stream>>>(ucnt, ubase, ocnt, lbase, static_cast<int>(nb), counts_out_dev, staged);
+  RECIS_LAUNCH_CHECK();
+  if (stage) RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
   {
     RECIS_TIME_KERNEL("plan_emit_occ_kernel", stream)
     plan_emit_occ_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(
