@@ -230,8 +230,8 @@ class Config4:
             "plan_tile_kernel": 8 * N + 4 * N + 16 * U,              # ids in; per-occurrence word + records out
             "plan_scatter_kernel": 16 * U + 16 * U,
             "plan_bucket_kernel": 16 * U + 8 * U + 16 * U,           # records in; per-record result + unique ids out
-            "plan_emit_occ_kernel": 8 * N + 4 * N + 8 * U + 12 * N,  # ids, word, result in; inverse, list, pos out
-            "plan_emit_uniq_kernel": 16 * U + 12 * U + 4 * (N + 1 - U),
+            # ids, word, result in; inverse, list, pos out; unique ids in, id + row_start out
+            "plan_emit_kernel": 8 * N + 4 * N + 8 * U + 12 * N + 16 * U + 12 * U + 4 * (N + 1 - U),
             "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,          # ids, one table slot, index + slot pos
             "seg_pool_fwd_kernel": U * (8 + D * 4) + 4 * N + 4 * (S + 1) + S * D * 4,
             "csr_cold_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,

@@ -19,8 +19,8 @@
 //            id its first position and its count; unique ids are ranked by first position
 //            inside the bucket, counts are scanned into list offsets
 //   scan     bucket totals -> first unique index and first list entry of every bucket
-//   emit     per occurrence: unique index (inverse), list position; per unique id: id,
-//            row_start, hot work items
+//   emit     one launch: per occurrence unique index (inverse) and list position; per unique
+//            id the id, row_start, hot work items
 //
 // Unique ids come out ordered by (bucket, first occurrence): a function of the input only.
 // The order of the occurrences inside one id's list is not specified.
@@ -488,12 +488,12 @@ __global__ void plan_empty_kernel(int64_t* __restrict__ counts, int32_t* __restr
 }
 
 // emit, per occurrence: inverse, list entry, position in the list
-__global__ void __launch_bounds__(kBlock)
-plan_emit_occ_kernel(const int64_t* __restrict__ ids, const uint32_t* __restrict__ occ_rec,
-                     const int2* __restrict__ result, const int32_t* __restrict__ ubase,
-                     const int32_t* __restrict__ lbase, PlanGeom g, int32_t* __restrict__ inverse,
-                     int32_t* __restrict__ list, int32_t* __restrict__ pos_out) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+__device__ __forceinline__ void
+emit_occ_block(int64_t vblock, const int64_t* __restrict__ ids, const uint32_t* __restrict__ occ_rec,
+               const int2* __restrict__ result, const int32_t* __restrict__ ubase,
+               const int32_t* __restrict__ lbase, const PlanGeom& g, int32_t* __restrict__ inverse,
+               int32_t* __restrict__ list, int32_t* __restrict__ pos_out) {
+  const int64_t i = vblock * kBlock + threadIdx.x;
   if (i >= g.n) return;
   const uint32_t w = occ_rec[i];
   const int2 r = result[(i >> 10 << 10) | (w & 1023u)];
@@ -506,21 +506,21 @@ plan_emit_occ_kernel(const int64_t* __restrict__ ids, const uint32_t* __restrict
 
 // emit, per unique id (workgroups 0 .. buckets-1: one bucket each): id, row_start, hot work
 // items; the remaining workgroups set row_start[U .. n] = n.
-__global__ void __launch_bounds__(kBlock)
-plan_emit_uniq_kernel(const URec* __restrict__ bucket_uniq, const int32_t* __restrict__ bucket_start,
-                      const int32_t* __restrict__ ubase, const int32_t* __restrict__ lbase, PlanGeom g,
-                      int64_t* __restrict__ unique_out, int32_t* __restrict__ row_start,
-                      int64_t* __restrict__ counts, int32_t* __restrict__ hot_items, int64_t hot_cap) {
+__device__ __forceinline__ void
+emit_uniq_block(int64_t vblock, const URec* __restrict__ bucket_uniq, const int32_t* __restrict__ bucket_start,
+                const int32_t* __restrict__ ubase, const int32_t* __restrict__ lbase, const PlanGeom& g,
+                int64_t* __restrict__ unique_out, int32_t* __restrict__ row_start,
+                int64_t* __restrict__ counts, int32_t* __restrict__ hot_items, int64_t hot_cap) {
   const int nb = 1 << g.nb_log2;
-  if (static_cast<int>(blockIdx.x) >= nb) {
+  if (vblock >= nb) {
     const int64_t U = ubase[nb];
     const int64_t chunk = static_cast<int64_t>(kBlock) * 16;
-    const int64_t lo = U + (static_cast<int64_t>(blockIdx.x) - nb) * chunk;
+    const int64_t lo = U + (vblock - nb) * chunk;
     const int64_t hi = min(lo + chunk, g.n + 1);
     for (int64_t x = lo + threadIdx.x; x < hi; x += kBlock) row_start[x] = static_cast<int32_t>(g.n);
     return;
   }
-  const int b = blockIdx.x;
+  const int b = static_cast<int>(vblock);
   const int32_t u0 = ubase[b], cnt = ubase[b + 1] - u0, l0 = lbase[b];
   const URec* src = bucket_uniq + bucket_start[b];
   for (int k = threadIdx.x; k < cnt; k += kBlock) {
@@ -539,6 +539,24 @@ plan_emit_uniq_kernel(const URec* __restrict__ bucket_uniq, const int32_t* __res
       }
     }
   }
+}
+
+// emit, one launch: the first `uniq_blocks` workgroups work per unique id (a bucket each, then
+// the row_start tail), the rest per occurrence.
+__global__ void __launch_bounds__(kBlock)
+plan_emit_kernel(int64_t uniq_blocks, const int64_t* __restrict__ ids, const uint32_t* __restrict__ occ_rec,
+                 const int2* __restrict__ result, const URec* __restrict__ bucket_uniq,
+                 const int32_t* __restrict__ bucket_start, const int32_t* __restrict__ ubase,
+                 const int32_t* __restrict__ lbase, PlanGeom g, int64_t* __restrict__ unique_out,
+                 int32_t* __restrict__ inverse, int32_t* __restrict__ row_start, int32_t* __restrict__ list,
+                 int32_t* __restrict__ pos_out, int64_t* __restrict__ counts, int32_t* __restrict__ hot_items,
+                 int64_t hot_cap) {
+  const int64_t vb = blockIdx.x;
+  if (vb < uniq_blocks)
+    emit_uniq_block(vb, bucket_uniq, bucket_start, ubase, lbase, g, unique_out, row_start, counts, hot_items,
+                    hot_cap);
+  else
+    emit_occ_block(vb - uniq_blocks, ids, occ_rec, result, ubase, lbase, g, inverse, list, pos_out);
 }
 
 // ---------------------------------------------------------------- consumers
@@ -1002,17 +1020,12 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   RECIS_LAUNCH_CHECK();
   if (stage) RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
   {
-    RECIS_TIME_KERNEL("plan_emit_occ_kernel", stream)
-    plan_emit_occ_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(
-        ids, occ_rec, result, ubase, lbase, g, inverse_out, list_out, pos_out);
-    RECIS_LAUNCH_CHECK();
-  }
-  {
     const int64_t tail_blocks = (n + 1 + kBlock * 16 - 1) / (kBlock * 16);
-    RECIS_TIME_KERNEL("plan_emit_uniq_kernel", stream)
-    plan_emit_uniq_kernel<<<dim3(nb + tail_blocks), dim3(kBlock), 0, stream>>>(
-        bucket_uniq, bucket_start, ubase, lbase, g, unique_out, row_start_out, counts_out_dev, hot_items_out,
-        hot_cap);
+    const int64_t uniq_blocks = nb + tail_blocks, occ_blocks = (n + kBlock - 1) / kBlock;
+    RECIS_TIME_KERNEL("plan_emit_kernel", stream)
+    plan_emit_kernel<<<dim3(uniq_blocks + occ_blocks), dim3(kBlock), 0, stream>>>(
+        uniq_blocks, ids, occ_rec, result, bucket_uniq, bucket_start, ubase, lbase, g, unique_out, inverse_out,
+        row_start_out, list_out, pos_out, counts_out_dev, hot_items_out, hot_cap);
     RECIS_LAUNCH_CHECK();
   }
   if (unique_count_host) {

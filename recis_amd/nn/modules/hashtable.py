@@ -308,7 +308,6 @@ class HashtableImpl:
         self._children_info = ChildrenInfo(coalesce, children)
         self._slice = Slice(slice_begin, slice_end, slice_size)
         self._idmap = ops.IdMap(device, reserve=reserve_rows)
-        self._rows_ub = 0  # upper bound of the allocator's high-water mark
         self._grad_index, self._grad, self._grad_unique = [], [], []
 
     # ------------------------------------------------------------- storage
@@ -335,7 +334,6 @@ class HashtableImpl:
         """block_num = (id_num + block_size) / block_size (hashtable.cc:255-261)."""
         sg = self._slot_group
         id_num = self._idmap.id_num()
-        self._rows_ub = id_num
         sg.set_block_num((id_num + sg.block_size()) // sg.block_size())
 
     # ------------------------------------------------------------- lookups
@@ -455,11 +453,9 @@ class HashtableImpl:
         self.clear_grad()
         self._idmap.clear()
         self._slot_group.clear()
-        self._rows_ub = 0
 
     def clear_id(self):
         self._idmap.clear()
-        self._rows_ub = 0
 
     def ids(self):
         return self._idmap.snapshot()[0]

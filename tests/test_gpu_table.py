@@ -195,6 +195,39 @@ def test_block_filter(rng, dt):
     assert torch.equal(ops.block_filter(ids, blocks, bs, 77), flat[ids] < 77)
 
 
+def test_counted_lookup_and_host_bounds(rng):
+    """Lookup of "the first n_dev[0] ids of a buffer" (size known to the device only) gives the
+    rows of a plain lookup of that prefix and leaves the rest of the output alone; the map's
+    host-side bounds never undercut the true allocator mark and settle to it."""
+    g, c = ops.IdMap(), oracle.IdMap()
+    for rnd in range(5):
+        buf = rng.integers(0, 4000, size=3000)
+        buf = buf[np.sort(np.unique(buf, return_index=True)[1])]  # unique ids, as a plan hands them over
+        n_true = int(rng.integers(0, len(buf) + 1))
+        n_dev = torch.tensor([n_true, 123], device="cuda")
+        out = g.lookup_counted(_dev(buf), n_dev)
+        assert g.id_num_bound() >= c.id_num()          # before anything is known: counts the whole buffer
+        got = out.cpu().numpy()
+        exp = c.lookup(buf[:n_true])
+        np.testing.assert_array_equal(got[:n_true], exp)
+        g.settle_count(n_true)
+        bound = g.id_num_bound()
+        torch.cuda.synchronize()
+        assert c.id_num() <= g.id_num_bound() <= bound
+        assert g.id_num_bound() == c.id_num() == g.id_num()
+        assert g.stats()[:3] == (c.size(), c.id_num(), c.free_size())
+        # erase a few, so that recycled rows take part in the next round
+        drop = buf[:n_true][::3]
+        rows = c.lookup_readonly(drop)
+        g.erase(_dev(drop), _dev(rows))
+        c.delete(drop, rows)
+    # a count beyond the buffer is clamped to the buffer
+    buf = np.arange(10**6, 10**6 + 50, dtype=np.int64)
+    out = g.lookup_counted(_dev(buf), torch.tensor([10**9], device="cuda"))
+    np.testing.assert_array_equal(out.cpu().numpy(), c.lookup(buf))
+    assert _lib.poll_device_errors() == 0
+
+
 @pytest.mark.parametrize("dt", [torch.int64, torch.int32])
 def test_evict_older_equals_snapshot_filter_erase(rng, dt):
     """The one-pass eviction sweep against the reference's sequence (snapshot, block_filter,
