@@ -234,8 +234,7 @@ class Config4:
             "plan_emit_kernel": 8 * N + 4 * N + 8 * U + 12 * N + 16 * U + 12 * U + 4 * (N + 1 - U),
             "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,          # ids, one table slot, index + slot pos
             "seg_pool_fwd_kernel": U * (8 + D * 4) + 4 * N + 4 * (S + 1) + S * D * 4,
-            "csr_cold_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,
-            "csr_hot_kernel": 0,
+            "csr_rows_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,
             "adamw_rows_kernel": U * (8 + D * 4 * 7),
         }
 

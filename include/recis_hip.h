@@ -425,10 +425,12 @@ int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_feat
 
 /*
  * out[u, :] (+)= sum over k in [row_start[u], row_start[u+1]) of coef[k] * rows[src[k], :]
- * for u < U. Rows with at most 256 entries are reduced by a small group of lanes and
- * written once; hot rows are reduced by whole workgroups per RECIS_PLAN_HOT_CHUNK-entry chunk and
- * combined with a few fp32 atomics (out must then be fp32, D <= 1024). accumulate != 0
- * adds to what out holds. src < 0 skips the entry; coef may be NULL (= 1).
+ * for u < U, every row written once, no atomics. Rows with at most RECIS_PLAN_HOT_LEN entries
+ * are reduced by lanes of one wave; hot rows through the plan's work items: workgroups store
+ * one partial row per RECIS_PLAN_HOT_CHUNK entries into library scratch, a second small
+ * launch adds them up in chunk order. Without work items (hot_cap == 0) every row goes the
+ * first way. accumulate != 0 adds to what out holds. src < 0 skips the entry; coef may be
+ * NULL (= 1). D <= 8192.
  * cover_offsets (device, [cover_S + 1], int32 or int64) or NULL: entries whose src lies outside
  * [cover_offsets[0], cover_offsets[cover_S]) are skipped too (occurrences no segment covers,
  * for the backward of the TILE mode where src is the occurrence itself).

@@ -27,6 +27,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <climits>
 #include <type_traits>
 
 #include "common.cuh"
@@ -579,6 +580,13 @@ struct CsrArgs {
   const void* cover;  // offsets [cover_S + 1] or NULL: entries whose src lies outside
   int cover64;        // [cover[0], cover[cover_S]) are skipped
   int64_t cover_S;
+  // hot rows (more than hot_len occurrences): (row, chunk) work items, partial sums per item
+  int32_t hot_len;           // INT_MAX when the caller brings no work items: every row is "cold"
+  const int32_t* hot_items;  // [2 * hot_cap]
+  const int64_t* counts;     // counts[1] = number of items
+  int64_t hot_cap;
+  float* hot_part;           // [hot_cap, D]
+  int64_t cold_blocks;       // the last cold_blocks workgroups work per row, the ones before per hot item
 };
 
 __device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64_t& hi) {
@@ -641,26 +649,26 @@ __device__ __forceinline__ void wave_gather_range(const TIn* __restrict__ rows, 
   }
 }
 
-// One group of LPR lanes per unique row (cold rows); hot rows are cleared here and summed by
-// csr_hot_kernel. A wave that holds a row with more than kCoopLen occurrences switches, as a
-// whole, to working its rows one after the other with all its lane groups striding over the
-// row's list (a row of 200 occurrences would otherwise be 50 dependent gathers of one group).
-constexpr int kCoopLen = 8;
+constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of a wave
 
-// SHUFFLE: long rows go through wave_gather_range (pays off when a wave has at most eight lane
+// One launch for all rows. The last cold_blocks workgroups: one group of LPR lanes per unique row
+// with at most hot_len occurrences ("cold"); a wave that holds a row with more than kCoopLen
+// occurrences works that row with all its lane groups striding over the list (a row of 200
+// occurrences would otherwise be 50 dependent gathers of one group). The first workgroups
+// walk the hot work items (row, chunk of kHotChunk occurrences): four waves share the chunk,
+// fold their sums through LDS and store ONE partial row per item; csr_hot_finish_kernel adds up
+// the partial rows of every hot row in chunk order. No atomics anywhere.
+// SHUFFLE: long lists go through wave_gather_range (pays off when a wave has at most eight lane
 // groups, i.e. rows of 128 bytes and more); otherwise every group loads its own entries.
 template <typename TIn, typename TOut, int VEC, bool SHUFFLE>
 __global__ void __launch_bounds__(kBlock)
-csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a) {
-  const int rows_per_block = kBlock >> a.lpr_log2;
-  const int64_t u = static_cast<int64_t>(blockIdx.x) * rows_per_block + (threadIdx.x >> a.lpr_log2);
-  const bool valid = u < a.U;
-  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
-  const int32_t start = valid ? a.row_start[u] : 0;
-  int32_t end = valid ? a.row_start[u + 1] : 0;
-  const bool hot = end - start > kHotLen;
-  if (hot) end = start;  // nothing to gather here
+csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a) {
+  extern __shared__ float s_part[];  // [waves][D], hot part only
   const int D = a.D;
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
+  const int g = lane >> a.lpr_log2;        // this lane's group in its wave
   int64_t c_lo, c_hi;
   cover_range(a, c_lo, c_hi);
 
@@ -702,10 +710,67 @@ csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
       for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v0[j], w0, acc[j]);
     }
   };
-  auto finish = [&](int64_t row, bool row_hot, int c0, float (&acc)[VEC]) {
+  // the wave's sum over the list entries [first, last) for columns c0.., the same in every group
+  auto wave_sum = [&](int32_t first, int32_t last, int c0, bool col_ok, float (&acc)[VEC]) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    if constexpr (SHUFFLE) {
+      wave_gather_range<TIn, VEC>(rows, a, c_lo, c_hi, first, last, c0, col_ok, g, groups, acc);
+    } else {
+      if (col_ok) gather_sum(first + g, last, groups, c0, acc);
+    }
+    for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+    }
+  };
+
+  const int64_t hot_blocks = static_cast<int64_t>(gridDim.x) - a.cold_blocks;
+  if (static_cast<int64_t>(blockIdx.x) < hot_blocks) {
+    // ---- hot work items (the first workgroups: the longest-running ones start first)
+    int64_t n_items = a.counts[1];
+    if (n_items > a.hot_cap) n_items = a.hot_cap;
+    const int wave = threadIdx.x / kWave;
+    constexpr int n_waves = kBlock / kWave;
+    for (int64_t item = blockIdx.x; item < n_items; item += hot_blocks) {
+      const int32_t u = a.hot_items[2 * item];
+      const int32_t chunk = a.hot_items[2 * item + 1];
+      const int32_t start = a.row_start[u] + chunk * kHotChunk;
+      const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
+      const int32_t per_wave = (end - start + n_waves - 1) / n_waves;  // a contiguous share per wave
+      const int32_t w_begin = min(end, start + wave * per_wave), w_end = min(end, w_begin + per_wave);
+      for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+        const int c0 = cbase + cl * VEC;
+        const bool col_ok = c0 < D;
+        float acc[VEC];
+        wave_sum(w_begin, w_end, c0, col_ok, acc);
+        if (g == 0 && col_ok) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) s_part[wave * D + c0 + j] = acc[j];
+        }
+      }
+      __syncthreads();
+      for (int d = threadIdx.x; d < D; d += kBlock) {
+        float sum = 0.f;
+        for (int w = 0; w < n_waves; ++w) sum += s_part[w * D + d];
+        a.hot_part[item * D + d] = sum;
+      }
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ---- cold rows
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
+  const bool valid = u < a.U;
+  const int32_t start = valid ? a.row_start[u] : 0;
+  int32_t end = valid ? a.row_start[u + 1] : 0;
+  const bool hot = end - start > a.hot_len;  // left to the work items and the finish kernel
+  if (hot) end = start;
+  auto finish = [&](int64_t row, int c0, float (&acc)[VEC]) {
     TOut* dst = out + row * D + c0;
     if (a.accumulate) {
-      if (row_hot) return;  // keep what is there; the hot kernel adds to it
       float old[VEC];
       load_pack<TOut, VEC>(dst, old);
 #pragma unroll
@@ -713,22 +778,18 @@ csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
     }
     store_pack<TOut, VEC>(dst, acc);
   };
-
   // short rows: every lane group works its own row
   const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;  // with one group per wave there is nobody to share with
-  if (valid && !is_long) {
+  if (valid && !is_long && !hot) {
     for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
       float acc[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
       gather_sum(start, end, 1, c0, acc);
-      finish(u, hot, c0, acc);
+      finish(u, c0, acc);
     }
   }
-  // long rows of this wave, one after the other: every lane group strides over the row's list
-  const int lane = threadIdx.x & (kWave - 1);
-  const int groups = kWave >> a.lpr_log2;
-  const int g = lane >> a.lpr_log2;
+  // long rows of this wave, one after the other
   uint64_t todo = __ballot(is_long);
   while (todo) {
     const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;  // first lane of the owning group
@@ -740,108 +801,48 @@ csr_cold_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
       const int c0 = cbase + cl * VEC;
       const bool col_ok = c0 < D;
       float acc[VEC];
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      if constexpr (SHUFFLE) {
-        wave_gather_range<TIn, VEC>(rows, a, c_lo, c_hi, r_start, r_end, c0, col_ok, g, groups, acc);
-      } else {
-        if (col_ok) gather_sum(r_start + g, r_end, groups, c0, acc);
-      }
-      for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
-      }
-      if (g == r && col_ok) finish(row, false, c0, acc);
+      wave_sum(r_start, r_end, c0, col_ok, acc);
+      if (g == r && col_ok) finish(row, c0, acc);
     }
   }
 }
 
-// One workgroup per (hot row, chunk): row groups stride over the chunk, partial sums are
-// combined through LDS and added to the (cleared) output row with a handful of atomics.
-template <typename TIn, int VEC, bool SHUFFLE>
-__global__ void __launch_bounds__(kPlanBlock)
-csr_hot_kernel(const TIn* __restrict__ rows, float* __restrict__ out, CsrArgs a,
-               const int32_t* __restrict__ hot_items, const int64_t* __restrict__ counts, int64_t hot_cap) {
-  extern __shared__ float s_part[];  // [waves][D]
-  int64_t c_lo, c_hi;
-  cover_range(a, c_lo, c_hi);
-  int64_t n_items = counts[1];
-  if (n_items > hot_cap) n_items = hot_cap;
+// out[u] (+)= sum of the partial rows of hot row u, in chunk order. One lane group per work item
+// with chunk 0 (the items of a row are consecutive).
+template <typename TOut, int VEC>
+__global__ void __launch_bounds__(kBlock)
+csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a) {
+  int64_t n_items = a.counts[1];
+  if (n_items > a.hot_cap) n_items = a.hot_cap;
   const int D = a.D;
-  const int groups_w = kWave >> a.lpr_log2;                      // lane groups of a wave
-  const int gw = (threadIdx.x & (kWave - 1)) >> a.lpr_log2;      // this lane's group in its wave
   const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
-  const int wave = threadIdx.x / kWave;
-  constexpr int n_waves = kPlanBlock / kWave;
-  for (int64_t item = blockIdx.x; item < n_items; item += gridDim.x) {
-    const int32_t u = hot_items[2 * item];
-    const int32_t chunk = hot_items[2 * item + 1];
-    const int32_t start = a.row_start[u] + chunk * kHotChunk;
-    const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
-    // each wave takes a contiguous share of the chunk
-    const int32_t per_wave = (end - start + n_waves - 1) / n_waves;
-    const int32_t w_begin = min(end, start + wave * per_wave), w_end = min(end, w_begin + per_wave);
-    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
-      const int c0 = cbase + cl * VEC;
-      const bool col_ok = c0 < D;
+  const int64_t groups_total = static_cast<int64_t>(gridDim.x) * (kBlock >> a.lpr_log2);
+  for (int64_t item = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.lpr_log2) + (threadIdx.x >> a.lpr_log2);
+       item < n_items; item += groups_total) {
+    if (a.hot_items[2 * item + 1] != 0) continue;
+    const int32_t u = a.hot_items[2 * item];
+    const int32_t len = a.row_start[u + 1] - a.row_start[u];
+    int64_t n_chunks = (len + kHotChunk - 1) / kHotChunk;
+    if (item + n_chunks > n_items) n_chunks = n_items - item;  // items cut off by hot_cap (cannot happen with the documented hot_cap)
+    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
       float acc[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      if constexpr (SHUFFLE) {
-        wave_gather_range<TIn, VEC>(rows, a, c_lo, c_hi, w_begin, w_end, c0, col_ok, gw, groups_w, acc);
-      } else if (col_ok) {
-        auto fetch = [&](int32_t k, float (&v)[VEC], float& w) {
-          const int32_t s = a.src[k];
-          w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
-          if (s < c_lo || s >= c_hi) {
+      for (int64_t k = 0; k < n_chunks; ++k) {
+        float v[VEC];
+        load_pack<float, VEC>(a.hot_part + (item + k) * D + c0, v);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) v[j] = 0.f;
-            w = 0.f;
-            return;
-          }
-          load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
-        };
-        int32_t k = w_begin + gw;
-        for (; k + 3 * groups_w < w_end; k += 4 * groups_w) {  // four gathers in flight per lane
-          float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
-          float w0, w1, w2, w3;
-          fetch(k, v0, w0);
-          fetch(k + groups_w, v1, w1);
-          fetch(k + 2 * groups_w, v2, w2);
-          fetch(k + 3 * groups_w, v3, w3);
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            acc[j] = fmaf(v0[j], w0, acc[j]);
-            acc[j] = fmaf(v1[j], w1, acc[j]);
-            acc[j] = fmaf(v2[j], w2, acc[j]);
-            acc[j] = fmaf(v3[j], w3, acc[j]);
-          }
-        }
-        for (; k < w_end; k += groups_w) {
-          float v[VEC];
-          float w;
-          fetch(k, v, w);
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[j], w, acc[j]);
-        }
+        for (int j = 0; j < VEC; ++j) acc[j] += v[j];
       }
-      // groups of one wave share columns when lpr < 64: fold them with shuffles
-      for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
+      TOut* dst = out + static_cast<int64_t>(u) * D + c0;
+      if (a.accumulate) {
+        float old[VEC];
+        load_pack<TOut, VEC>(dst, old);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+        for (int j = 0; j < VEC; ++j) acc[j] += old[j];
       }
-      if (gw == 0 && col_ok) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) s_part[wave * D + c0 + j] = acc[j];
-      }
+      store_pack<TOut, VEC>(dst, acc);
     }
-    __syncthreads();
-    for (int d = threadIdx.x; d < D; d += kPlanBlock) {
-      float s = 0.f;
-      for (int w = 0; w < n_waves; ++w) s += s_part[w * D + d];
-      unsafeAtomicAdd(out + static_cast<int64_t>(u) * D + d, s);
-    }
-    __syncthreads();
   }
 }
 
@@ -1097,8 +1098,6 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   RECIS_REQUIRE(src && row_start && out && counts_dev, "NULL argument");
   RECIS_REQUIRE(rows != nullptr || n_rows == 0, "rows must not be NULL");
   RECIS_REQUIRE(hot_cap == 0 || hot_items, "hot_items must not be NULL");
-  RECIS_REQUIRE(hot_cap == 0 || out_dtype == RECIS_F32, "hot rows are accumulated in fp32: out must be fp32");
-  RECIS_REQUIRE(hot_cap == 0 || D <= 1024, "hot-row reduction supports D <= 1024 (got %lld)", (long long)D);
   const int in_sz = dtype_size(rows_dtype), out_sz = dtype_size(out_dtype);
   RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
   RECIS_REQUIRE(coef == nullptr || dtype_size(coef_dtype), "invalid coef dtype");
@@ -1121,7 +1120,21 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   a.err = device_error_word(current_device());
   RECIS_REQUIRE(a.err != nullptr, "could not allocate the device error word");
   const int rows_per_block = kBlock >> a.lpr_log2;
-  const int64_t grid = (U + rows_per_block - 1) / rows_per_block;
+  a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
+  a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
+  a.hot_items = hot_items;
+  a.counts = counts_dev;
+  a.hot_cap = hot_cap;
+  a.hot_part = nullptr;
+  int64_t hot_blocks = 0;
+  if (hot_cap > 0) {
+    void* ws = nullptr;
+    if (int rc = get_workspace(stream, sizeof(float) * static_cast<size_t>(hot_cap) * static_cast<size_t>(D), &ws))
+      return rc;
+    a.hot_part = static_cast<float*>(ws);
+    hot_blocks = std::min<int64_t>(hot_cap, 4096);
+  }
+  const size_t lds = sizeof(float) * (kBlock / kWave) * static_cast<size_t>(D);
   auto with_types = [&](auto tin, auto tout) {
     using TIn = decltype(tin);
     using TOut = decltype(tout);
@@ -1131,28 +1144,20 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
         const TIn* rin = static_cast<const TIn*>(rows);
+        TOut* o = static_cast<TOut*>(out);
         const bool shuffle = a.lpr_log2 >= 3;  // at most eight lane groups per wave
         {
-          RECIS_TIME_KERNEL("csr_cold_kernel", stream)
+          RECIS_TIME_KERNEL("csr_rows_kernel", stream)
           if (shuffle)
-            csr_cold_kernel<TIn, TOut, VEC, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(rin, static_cast<TOut*>(out), a);
+            csr_rows_kernel<TIn, TOut, VEC, true><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
           else
-            csr_cold_kernel<TIn, TOut, VEC, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(rin, static_cast<TOut*>(out), a);
+            csr_rows_kernel<TIn, TOut, VEC, false><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
           RECIS_LAUNCH_CHECK();
         }
-        if constexpr (std::is_same<TOut, float>::value) {
-          if (hot_cap > 0) {
-            const int64_t hot_grid = std::min<int64_t>(hot_cap, 2048);
-            const size_t lds = sizeof(float) * (kPlanBlock / kWave) * static_cast<size_t>(D);
-            RECIS_TIME_KERNEL("csr_hot_kernel", stream)
-            if (shuffle)
-              csr_hot_kernel<TIn, VEC, true><<<dim3(hot_grid), dim3(kPlanBlock), lds, stream>>>(
-                  rin, static_cast<float*>(out), a, hot_items, counts_dev, hot_cap);
-            else
-              csr_hot_kernel<TIn, VEC, false><<<dim3(hot_grid), dim3(kPlanBlock), lds, stream>>>(
-                  rin, static_cast<float*>(out), a, hot_items, counts_dev, hot_cap);
-            RECIS_LAUNCH_CHECK();
-          }
+        if (hot_cap > 0) {
+          const int64_t fin = std::min<int64_t>((hot_cap + rows_per_block - 1) / rows_per_block, 1024);
+          csr_hot_finish_kernel<TOut, VEC><<<dim3(fin), dim3(kBlock), 0, stream>>>(o, a);
+          RECIS_LAUNCH_CHECK();
         }
         return RECIS_OK;
       }
