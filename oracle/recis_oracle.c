@@ -14,6 +14,9 @@
  * vector, a closed form / library routine, or a brute-force model in
  * tests/test_oracle_*.py, except those marked "parity unpinned" below:
  *   (none so far)
+ * and tests/test_oracle_ref_ops.py compares the table, allocator, row-block,
+ * optimizer, tagging, partition and feature functions bit for bit with the
+ * reference's own CPU operators where oracle/_ref/ref_ops has been built.
  * Additions with no reference counterpart (MAX combiner, Adagrad row update)
  * are pinned by torch / textbook closed forms instead.
  *

@@ -17,3 +17,40 @@ g++ -O2 -fPIC -shared -std=c++17 -fvisibility=hidden -w -I"$SRC" \
   "$HERE/ref_hash_driver.cc" "$SRC/farmhash.cc" "$SRC/hash_utils.cc" \
   -o "$HERE/_ref/libref_hash.so"
 echo "built $HERE/_ref/libref_hash.so"
+
+#   ref_ops        : the reference's CPU operators (csrc/ops/*.cc, csrc/embedding/{cpu_id_map,
+#                    id_allocator}.cc) compiled against the installed torch headers and driven by
+#                    ref_ops_driver.cc. Their CUDA counterparts (*_cuda / *_gpu, defined in .cu
+#                    files that need nvcc) stay unresolved: the binary binds lazily and every
+#                    tensor it sees is on the CPU, so they are never reached.
+TORCH="$(python3 -c 'import torch, os; print(os.path.dirname(torch.__file__))')"
+PYINC="$(python3 -c 'import sysconfig; print(sysconfig.get_paths()["include"])')"
+ABI="$(python3 -c 'import torch; print(int(torch._C._GLIBCXX_USE_CXX11_ABI))')"
+CSRC="$REF/csrc"
+OBJ="$HERE/_ref/obj"
+mkdir -p "$OBJ"
+CXXFLAGS="-std=c++17 -O2 -fPIC -fopenmp -w -D_GLIBCXX_USE_CXX11_ABI=$ABI -I$CSRC -I$CSRC/ops -I$TORCH/include -I$TORCH/include/torch/csrc/api/include -I$PYINC"
+SOURCES="ops/block_apply_adamw_op.cc ops/hashtable_ops.cc ops/block_ops.cc ops/ids_partition.cc ops/ids_encode.cc
+         ops/fused_uint64_mod.cc ops/fused_bucketized.cc ops/multi_hash.cc
+         embedding/id_allocator.cc embedding/cpu_id_map.cc embedding/parallel_util.cc"
+pids=()
+for s in $SOURCES; do
+  o="$OBJ/$(echo "$s" | tr '/' '_' | sed 's/\.cc$/.o/')"
+  ( g++ $CXXFLAGS -c "$CSRC/$s" -o "$o" ) &
+  pids+=($!)
+  if [ "${#pids[@]}" -ge 6 ]; then wait "${pids[0]}"; pids=("${pids[@]:1}"); fi
+done
+( g++ $CXXFLAGS -c "$HERE/ref_ops_driver.cc" -o "$OBJ/driver.o" ) &
+pids+=($!)
+for p in "${pids[@]}"; do wait "$p"; done
+PYLIB="$(python3 -c 'import sysconfig; print(sysconfig.get_config_var("LIBDIR"))')"
+# The reference objects go into a shared library, where undefined symbols are allowed; the driver
+# links against it with lazy binding, so a function that is never called is never looked up.
+g++ -shared -fopenmp -o "$HERE/_ref/libref_ops.so" $(ls "$OBJ"/*.o | grep -v driver.o) \
+  -Wl,-z,lazy -Wl,-rpath,"$TORCH/lib" \
+  -L"$TORCH/lib" -ltorch -ltorch_cpu -lc10 -ltorch_python -L"$PYLIB" -lpython3.10
+g++ -fopenmp -o "$HERE/_ref/ref_ops" "$OBJ/driver.o" \
+  -Wl,--allow-shlib-undefined -Wl,-z,lazy -Wl,-rpath,'$ORIGIN' -Wl,-rpath,"$TORCH/lib" \
+  -L"$HERE/_ref" -lref_ops -L"$TORCH/lib" -ltorch -ltorch_cpu -lc10 -L"$PYLIB" -lpython3.10
+rm -rf "$OBJ"
+echo "built $HERE/_ref/ref_ops"

@@ -1,0 +1,230 @@
+// Test infrastructure: runs the reference's OWN CPU implementations of the hot-path operators
+// (compiled from /root/reference/csrc where they lie, see ref_build.sh) on inputs read from a
+// file and writes their outputs to a file, so that the oracle (oracle/recis_oracle.c) can be
+// checked against the real code. Nothing here is reference code: this file only moves tensors
+// in and out and calls
+//   recis::functional::block_apply_adamw            (csrc/ops/block_apply_adamw_op.cc:114-130)
+//   recis::embedding::MakeCpuIdMap / CpuIdMap        (csrc/embedding/cpu_id_map.cc:73-190)
+//   recis::embedding::IdAllocator                    (csrc/embedding/id_allocator.cc:17-60)
+//   recis::functional::mask_key_index_op, scatter_ids_with_mask_op (csrc/ops/hashtable_ops.cc:150-214)
+//   recis::functional::block_gather / block_insert / block_insert_with_mask / block_filter / gather
+//                                                    (csrc/ops/block_ops.cc:270-397)
+//   recis::functional::ids_partition_cpu, ids_encode_cpu, fused_uint64_mod, fused_bucketized,
+//   fused_multi_hash                                 (csrc/ops/*.cc)
+// (segment_sum / segment_mean have no CPU implementation in the reference: segment_ops.cc only
+// forwards to the CUDA functions.)
+// The reference objects also refer to their CUDA counterparts (*_cuda, *_gpu); those symbols are
+// left unresolved at link time (lazy binding) and are never reached: every tensor here is on the CPU.
+//
+// File format (little endian): int64 count, then per tensor: int32 dtype code, int32 ndim,
+// int64 dims[ndim], raw bytes. dtype codes: 0 f32, 1 f64, 2 i64, 3 i32, 4 bool, 5 i8.
+#include <torch/extension.h>
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "embedding/id_allocator.h"
+#include "embedding/id_map.h"
+#include "ops/block_apply_adamw_op.h"
+#include "ops/block_ops.h"
+#include "ops/fused_bucketized.h"
+#include "ops/fused_uint64_mod.h"
+#include "ops/hashtable_ops.h"
+#include "ops/ids_encode.h"
+#include "ops/ids_partition.h"
+#include "ops/multi_hash.h"
+
+using torch::Tensor;
+
+static at::ScalarType code_to_type(int c) {
+  switch (c) {
+    case 0: return at::kFloat;
+    case 1: return at::kDouble;
+    case 2: return at::kLong;
+    case 3: return at::kInt;
+    case 4: return at::kBool;
+    case 5: return at::kChar;
+  }
+  TORCH_CHECK(false, "bad dtype code ", c);
+}
+static int type_to_code(at::ScalarType t) {
+  switch (t) {
+    case at::kFloat: return 0;
+    case at::kDouble: return 1;
+    case at::kLong: return 2;
+    case at::kInt: return 3;
+    case at::kBool: return 4;
+    case at::kChar: return 5;
+    default: TORCH_CHECK(false, "unsupported output dtype");
+  }
+}
+
+static std::vector<Tensor> read_tensors(const char* path) {
+  FILE* f = fopen(path, "rb");
+  TORCH_CHECK(f, "cannot open ", path);
+  int64_t n = 0;
+  TORCH_CHECK(fread(&n, 8, 1, f) == 1, "short file");
+  std::vector<Tensor> out;
+  for (int64_t i = 0; i < n; ++i) {
+    int32_t code = 0, ndim = 0;
+    TORCH_CHECK(fread(&code, 4, 1, f) == 1 && fread(&ndim, 4, 1, f) == 1, "short file");
+    std::vector<int64_t> dims(ndim);
+    if (ndim) TORCH_CHECK(fread(dims.data(), 8, ndim, f) == static_cast<size_t>(ndim), "short file");
+    Tensor t = torch::empty(dims, torch::TensorOptions().dtype(code_to_type(code)));
+    const size_t bytes = t.numel() * t.element_size();
+    if (bytes) TORCH_CHECK(fread(t.data_ptr(), 1, bytes, f) == bytes, "short file");
+    out.push_back(t);
+  }
+  fclose(f);
+  return out;
+}
+
+static void write_tensors(const char* path, const std::vector<Tensor>& ts) {
+  FILE* f = fopen(path, "wb");
+  TORCH_CHECK(f, "cannot open ", path);
+  int64_t n = ts.size();
+  fwrite(&n, 8, 1, f);
+  for (const Tensor& t0 : ts) {
+    Tensor t = t0.contiguous();
+    int32_t code = type_to_code(t.scalar_type()), ndim = t.dim();
+    fwrite(&code, 4, 1, f);
+    fwrite(&ndim, 4, 1, f);
+    for (int d = 0; d < ndim; ++d) {
+      int64_t v = t.size(d);
+      fwrite(&v, 8, 1, f);
+    }
+    const size_t bytes = t.numel() * t.element_size();
+    if (bytes) fwrite(t.data_ptr(), 1, bytes, f);
+  }
+  fclose(f);
+}
+
+// a [rows, ...] tensor as the list of [block_size, ...] blocks the reference ops take (views)
+static std::vector<Tensor> as_blocks(const Tensor& t, int64_t block_size) {
+  std::vector<Tensor> b;
+  for (int64_t r = 0; r + block_size <= t.size(0); r += block_size) b.push_back(t.narrow(0, r, block_size));
+  return b;
+}
+
+static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
+  namespace F = recis::functional;
+  if (op == "adamw") {
+    // index [T, n] i64, grad [T, n, D], emb / exp_avg / exp_avg_sq [R, D], beta1_t, beta2_t [1],
+    // scalars f64 [6] = lr, beta1, beta2, weight_decay, eps, block_size
+    Tensor index = in[0], grad = in[1], emb = in[2], m = in[3], v = in[4], b1t = in[5], b2t = in[6];
+    const double* s = in[7].data_ptr<double>();
+    const int64_t bs = static_cast<int64_t>(s[5]);
+    Tensor step = torch::zeros({1}, torch::kLong);
+    for (int64_t t = 0; t < index.size(0); ++t)
+      F::block_apply_adamw(index[t], grad[t], as_blocks(emb, bs), b1t, b2t, step, as_blocks(m, bs), as_blocks(v, bs),
+                           s[0], s[1], s[2], s[3], s[4], bs);
+    return {emb, m, v, b1t, b2t};
+  }
+  if (op == "idmap") {
+    // codes i64 [K] (0 lookup, 1 lookup read-only, 2 delete), lens i64 [K], ids i64 [sum lens]
+    auto map = recis::embedding::MakeCpuIdMap(torch::Device(torch::kCPU));
+    const int64_t* codes = in[0].data_ptr<int64_t>();
+    const int64_t* lens = in[1].data_ptr<int64_t>();
+    std::vector<Tensor> res;
+    int64_t at = 0;
+    for (int64_t k = 0; k < in[0].numel(); ++k) {
+      Tensor ids = in[2].narrow(0, at, lens[k]).clone();
+      at += lens[k];
+      if (codes[k] == 0) {
+        res.push_back(map->Lookup(ids));
+      } else if (codes[k] == 1) {
+        res.push_back(map->LookupReadOnly(ids));
+      } else {
+        Tensor idx = map->LookupReadOnly(ids);
+        map->DeleteIds(ids, idx);
+        res.push_back(idx);
+      }
+    }
+    auto snap = map->SnapShot();
+    Tensor out = res.empty() ? torch::empty({0}, torch::kLong) : torch::cat(res);
+    return {out, snap.first, snap.second, torch::tensor({map->GetIdNum()}, torch::kLong)};
+  }
+  if (op == "alloc") {
+    // codes i64 [K] (0 gen, 1 free), lens i64 [K], ids to free i64 [sum of free lens], params i64 [2] = init, block
+    const int64_t* codes = in[0].data_ptr<int64_t>();
+    const int64_t* lens = in[1].data_ptr<int64_t>();
+    const int64_t* prm = in[3].data_ptr<int64_t>();
+    auto alloc = c10::make_intrusive<recis::embedding::IdAllocator>(torch::Device(torch::kCPU), prm[0],
+                                                                    static_cast<size_t>(prm[1]));
+    std::vector<Tensor> res;
+    int64_t at = 0;
+    for (int64_t k = 0; k < in[0].numel(); ++k) {
+      if (codes[k] == 0) {
+        res.push_back(alloc->GenIds(static_cast<size_t>(lens[k])));
+      } else {
+        alloc->FreeIds(in[2].narrow(0, at, lens[k]).clone());
+        at += lens[k];
+      }
+    }
+    Tensor out = res.empty() ? torch::empty({0}, torch::kLong) : torch::cat(res);
+    return {out, torch::tensor({alloc->GetSize(), alloc->GetActiveSize()}, torch::kLong)};
+  }
+  if (op == "mask_key_index") {  // keys, mask (bool), cumsum, out_size [1]
+    auto r = F::mask_key_index_op(in[0], in[1], in[2], in[3].item<int64_t>());
+    return {std::get<0>(r), std::get<1>(r)};
+  }
+  if (op == "scatter_ids_with_mask") return {F::scatter_ids_with_mask_op(in[0], in[1], in[2])};
+  if (op == "block_gather") {  // ids, table [R, D], params i64 [3] = block_size, default_key, readonly
+    const int64_t* p = in[2].data_ptr<int64_t>();
+    return {F::block_gather(in[0], as_blocks(in[1], p[0]), p[0], p[1], p[2] != 0)};
+  }
+  if (op == "gather") return {F::gather(in[0], in[1])};
+  if (op == "block_insert") {  // ids, rows, table, block_size [1]
+    F::block_insert(in[0], in[1], as_blocks(in[2], in[3].item<int64_t>()), in[3].item<int64_t>());
+    return {in[2]};
+  }
+  if (op == "block_insert_with_mask") {  // ids, rows, mask, table, block_size [1]
+    F::block_insert_with_mask(in[0], in[1], in[2], as_blocks(in[3], in[4].item<int64_t>()), in[4].item<int64_t>());
+    return {in[3]};
+  }
+  if (op == "block_filter") {  // ids, slot [R, 1], params i64 [2] = block_size, threshold
+    const int64_t* p = in[2].data_ptr<int64_t>();
+    return {F::block_filter(in[0], as_blocks(in[1], p[0]), p[0], p[1])};
+  }
+  if (op == "ids_partition") {  // ids, num_parts [1]
+    auto r = F::ids_partition_cpu(in[0], in[1].item<int64_t>());
+    return {std::get<0>(r), std::get<1>(r), std::get<2>(r)};
+  }
+  if (op == "ids_encode") {  // table_ids, tensors...
+    std::vector<Tensor> l(in.begin() + 1, in.end());
+    return {F::ids_encode_cpu(l, in[0])};
+  }
+  if (op == "fused_uint64_mod") {  // mods, tensors...
+    std::vector<Tensor> l(in.begin() + 1, in.end());
+    return F::fused_uint64_mod(l, in[0]);
+  }
+  if (op == "fused_bucketized") {  // k values then k boundaries
+    const size_t k = in.size() / 2;
+    std::vector<Tensor> v(in.begin(), in.begin() + k), b(in.begin() + k, in.end());
+    return F::fused_bucketized(v, b);
+  }
+  if (op == "fused_multi_hash") {  // k inputs, k muls, k primes, k bucket counts
+    const size_t k = in.size() / 4;
+    std::vector<Tensor> a(in.begin(), in.begin() + k), m(in.begin() + k, in.begin() + 2 * k),
+        p(in.begin() + 2 * k, in.begin() + 3 * k), b(in.begin() + 3 * k, in.end());
+    return F::fused_multi_hash(a, m, p, b);
+  }
+  TORCH_CHECK(false, "unknown op ", op);
+}
+
+int main(int argc, char** argv) {
+  if (argc != 4) {
+    fprintf(stderr, "usage: %s <op> <in.bin> <out.bin>\n", argv[0]);
+    return 2;
+  }
+  try {
+    at::set_num_threads(1);  // the reference's id map assigns rows in thread order: one thread = input order
+    write_tensors(argv[3], run(argv[1], read_tensors(argv[2])));
+  } catch (const std::exception& e) {
+    fprintf(stderr, "ref_ops %s: %s\n", argv[1], e.what());
+    return 1;
+  }
+  return 0;
+}
