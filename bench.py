@@ -470,10 +470,10 @@ class Config5:
 # scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC_C4 = {
-    "adamw_rows_kernel": 400841121, "seg_pool_fwd_kernel": 324971171, "csr_cold_kernel": 251810488,
-    "csr_hot_kernel": 143831573, "block_gather_kernel": 119564885, "plan_emit_occ_kernel": 115515050,
-    "find_or_claim_kernel": 114550648, "plan_bucket_kernel": 89176810, "plan_scatter_kernel": 77256686,
-    "plan_tile_kernel": 58195299, "plan_emit_uniq_kernel": 32875429,
+    "adamw_rows_kernel": 400839616, "csr_rows_kernel": 395399229, "seg_pool_fwd_kernel": 381144772,
+    "plan_emit_kernel": 149236208, "find_or_claim_kernel": 114433209, "plan_bucket_kernel": 89179726,
+    "plan_scatter_kernel": 77185311, "plan_tile_kernel": 58194552, "ids_encode_kernel": 40936056,
+    "plan_colscan_kernel": 16425662,
 }
 
 

@@ -18,8 +18,8 @@ g++ -O2 -fPIC -shared -std=c++17 -fvisibility=hidden -w -I"$SRC" \
   -o "$HERE/_ref/libref_hash.so"
 echo "built $HERE/_ref/libref_hash.so"
 
-#   ref_ops        : the reference's CPU operators (csrc/ops/*.cc, csrc/embedding/{cpu_id_map,
-#                    id_allocator}.cc) compiled against the installed torch headers and driven by
+#   ref_ops        : the reference's CPU operators (csrc/ops/*.cc) and its CPU table and sparse
+#                    optimizers (csrc/embedding/*.cc) compiled against the installed torch headers and driven by
 #                    ref_ops_driver.cc. Their CUDA counterparts (*_cuda / *_gpu, defined in .cu
 #                    files that need nvcc) stay unresolved: the binary binds lazily and every
 #                    tensor it sees is on the CPU, so they are never reached.
@@ -32,7 +32,10 @@ mkdir -p "$OBJ"
 CXXFLAGS="-std=c++17 -O2 -fPIC -fopenmp -w -D_GLIBCXX_USE_CXX11_ABI=$ABI -I$CSRC -I$CSRC/ops -I$TORCH/include -I$TORCH/include/torch/csrc/api/include -I$PYINC"
 SOURCES="ops/block_apply_adamw_op.cc ops/hashtable_ops.cc ops/block_ops.cc ops/ids_partition.cc ops/ids_encode.cc
          ops/fused_uint64_mod.cc ops/fused_bucketized.cc ops/multi_hash.cc
-         embedding/id_allocator.cc embedding/cpu_id_map.cc embedding/parallel_util.cc"
+         embedding/id_allocator.cc embedding/cpu_id_map.cc embedding/parallel_util.cc
+         embedding/hashtable.cc embedding/slot_group.cc embedding/initializer.cc embedding/children_info.cc
+         embedding/slice_info.cc embedding/optim.cc embedding/adam.cc embedding/adamw.cc embedding/adamw_tf.cc
+         serialize/string_sep.cc serialize/register_preserved_key.cc utils/str_util.cc"
 pids=()
 for s in $SOURCES; do
   o="$OBJ/$(echo "$s" | tr '/' '_' | sed 's/\.cc$/.o/')"

@@ -6,6 +6,8 @@
 //   recis::functional::block_apply_adamw            (csrc/ops/block_apply_adamw_op.cc:114-130)
 //   recis::embedding::MakeCpuIdMap / CpuIdMap        (csrc/embedding/cpu_id_map.cc:73-190)
 //   recis::embedding::IdAllocator                    (csrc/embedding/id_allocator.cc:17-60)
+//   Hashtable (EmbeddingLookup, AcceptGrad, Delete, ids_map, slots) with SparseAdam / SparseAdamW /
+//   SparseAdamWTF::step                              (csrc/embedding/hashtable.cc:46-278, adam*.cc)
 //   recis::functional::mask_key_index_op, scatter_ids_with_mask_op (csrc/ops/hashtable_ops.cc:150-214)
 //   recis::functional::block_gather / block_insert / block_insert_with_mask / block_filter / gather
 //                                                    (csrc/ops/block_ops.cc:270-397)
@@ -25,7 +27,12 @@
 #include <string>
 #include <vector>
 
+#include "embedding/adam.h"
+#include "embedding/adamw.h"
+#include "embedding/adamw_tf.h"
+#include "embedding/hashtable.h"
 #include "embedding/id_allocator.h"
+#include "embedding/initializer.h"
 #include "embedding/id_map.h"
 #include "ops/block_apply_adamw_op.h"
 #include "ops/block_ops.h"
@@ -165,6 +172,75 @@ static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
     }
     Tensor out = res.empty() ? torch::empty({0}, torch::kLong) : torch::cat(res);
     return {out, torch::tensor({alloc->GetSize(), alloc->GetActiveSize()}, torch::kLong)};
+  }
+  if (op == "table_train") {
+    // A script on one CPU Hashtable (constant initialiser) with one sparse optimizer.
+    // params f64 [10] = block_size, D, optimizer (0 SparseAdam, 1 SparseAdamW, 2 SparseAdamWTF), lr,
+    //                   beta1, beta2, eps, weight_decay, initial row value, grad accumulation steps
+    // codes i64 [K]: 0 lookup + accept_grad, 1 optimizer step + zero_grad, 2 delete (ids must be
+    //                present), 3 read-only lookup;  lens i64 [K];  ids i64 [sum of lens of codes 0/2/3];
+    // grads f32 [sum of lens of code 0, D]
+    const double* p = in[0].data_ptr<double>();
+    const int64_t bs = static_cast<int64_t>(p[0]), D = static_cast<int64_t>(p[1]);
+    const int kind = static_cast<int>(p[2]);
+    auto gen = recis::embedding::MakeConstantGenerator({bs, D}, torch::kFloat, p[8]);
+    auto table = Hashtable::Make(bs, {D}, torch::kFloat, torch::Device(torch::kCPU), true, {"t"}, gen, 0, 65536, 65536);
+    // the optimizers are built from a plain map: the Dict overload (their static Make) needs the
+    // custom-class registration of csrc/bind.cc, which is not part of this build
+    std::unordered_map<std::string, HashTablePtr> tables{{"t", table}};
+    c10::intrusive_ptr<recis::optim::SparseOptimizer> opt;
+    std::string prefix;
+    if (kind == 0) {
+      recis::optim::SparseAdamOptions o;
+      o.lr(p[3]).betas(std::make_tuple(p[4], p[5])).eps(p[6]).weight_decay(p[7]);
+      opt = c10::make_intrusive<recis::optim::SparseAdam>(tables, o);
+      prefix = "sparse_adam_";
+    } else if (kind == 1) {
+      recis::optim::SparseAdamWOptions o;
+      o.lr(p[3]).betas(std::make_tuple(p[4], p[5])).eps(p[6]).weight_decay(p[7]);
+      opt = c10::make_intrusive<recis::optim::SparseAdamW>(tables, o);
+      prefix = "sparse_adamw_";
+    } else {
+      recis::optim::SparseAdamWTFOptions o;
+      o.lr(p[3]).betas(std::make_tuple(p[4], p[5])).eps(p[6]).weight_decay(p[7]);
+      opt = c10::make_intrusive<recis::optim::SparseAdamWTF>(tables, o);
+      prefix = "sparse_adamw_tf_";
+    }
+    opt->set_grad_accum_steps(static_cast<int64_t>(p[9]));
+    const int64_t* codes = in[1].data_ptr<int64_t>();
+    const int64_t* lens = in[2].data_ptr<int64_t>();
+    std::vector<Tensor> idx_out, emb_out;
+    int64_t at_id = 0, at_grad = 0;
+    for (int64_t k = 0; k < in[1].numel(); ++k) {
+      if (codes[k] == 1) {
+        opt->step();
+        opt->zero_grad();
+        continue;
+      }
+      Tensor ids = in[3].narrow(0, at_id, lens[k]).clone();
+      at_id += lens[k];
+      if (codes[k] == 0) {
+        auto r = table->EmbeddingLookup(ids, false);
+        idx_out.push_back(std::get<0>(r));
+        emb_out.push_back(std::get<1>(r));
+        table->AcceptGrad(std::get<0>(r), in[4].narrow(0, at_grad, lens[k]).clone());
+        at_grad += lens[k];
+      } else if (codes[k] == 3) {
+        auto r = table->EmbeddingLookup(ids, true);
+        idx_out.push_back(std::get<0>(r));
+        emb_out.push_back(std::get<1>(r));
+      } else {
+        auto r = table->EmbeddingLookup(ids, true);
+        table->Delete(ids, std::get<0>(r), "");
+      }
+    }
+    auto snap = table->ids_map();
+    return {idx_out.empty() ? torch::empty({0}, torch::kLong) : torch::cat(idx_out),
+            emb_out.empty() ? torch::empty({0, D}) : torch::cat(emb_out),
+            std::get<0>(snap), std::get<1>(snap),
+            table->SlotGroup()->EmbSlot()->Value(),
+            table->GetSlot(prefix + "exp_avg")->Value(),
+            table->GetSlot(prefix + "exp_avg_sq")->Value()};
   }
   if (op == "mask_key_index") {  // keys, mask (bool), cumsum, out_size [1]
     auto r = F::mask_key_index_op(in[0], in[1], in[2], in[3].item<int64_t>());

@@ -239,3 +239,74 @@ def test_feature_ops_match_cpu_ops():
         for o in oracle.multi_hash(x, mu, pr, bk):
             np.testing.assert_array_equal(o, ref[k])
             k += 1
+
+
+# ------------------------------------------------------------------ table + sparse optimizers, end to end
+@pytest.mark.parametrize("kind,beta_dtype,decay_of", [
+    (0, np.float64, lambda lr, wd: 1.0),            # SparseAdam ignores weight_decay (adam.cc:70-73)
+    (1, np.float32, lambda lr, wd: 1.0 - lr * wd),  # SparseAdamW (adamw.cc:64)
+    (2, np.float32, lambda lr, wd: 1.0 - wd),       # SparseAdamWTF (adamw_tf.cc:64)
+])
+def test_table_training_script_matches_hashtable_and_optimizers(kind, beta_dtype, decay_of):
+    # csrc/embedding/hashtable.cc:46-278 + adam*.cc::step on a CPU table: lookups that grow the table
+    # across block boundaries, accumulated gradients, deletes that recycle rows, read-only lookups
+    from oracle import cpu_path
+
+    rng = np.random.default_rng(20 + kind)
+    bs, D, init = 64, 8, 0.25
+    lr, b1, b2, eps, wd = 0.02, 0.9, 0.999, 1e-8, 0.05
+    codes, lens, ids, grads = [], [], [], []
+    live = []
+    for step in range(12):
+        batch = np.unique(rng.integers(0, 600, int(rng.integers(1, 200)))).astype(np.int64)
+        rng.shuffle(batch)
+        live = sorted(set(live) | set(batch.tolist()))
+        codes += [0, 1]
+        lens += [len(batch), 0]
+        ids.append(batch)
+        grads.append(rng.standard_normal((len(batch), D)).astype(np.float32))
+        if step % 3 == 1:
+            ro = rng.integers(0, 700, 50).astype(np.int64)
+            codes.append(3), lens.append(len(ro)), ids.append(ro)
+        if step % 4 == 2:
+            gone = rng.choice(np.asarray(live, np.int64), size=len(live) // 3, replace=False)
+            live = sorted(set(live) - set(gone.tolist()))
+            codes.append(2), lens.append(len(gone)), ids.append(gone)
+    r_idx, r_emb, r_ids, r_rows, r_w, r_m, r_v = ref_ops.run("table_train", [
+        np.asarray([bs, D, kind, lr, b1, b2, eps, wd, init, 1], np.float64), _i64(*codes), _i64(*lens),
+        np.concatenate(ids), np.concatenate(grads)])
+
+    t = cpu_path.CpuTable(D, bs, lambda b: np.full((bs, D), init, np.float32), "adam", lr, eps, b1, b2,
+                          decay_of(lr, wd), beta_dtype)
+    idx_out, emb_out = [], []
+    it_ids, it_grads = iter(ids), iter(grads)
+    pending = None
+    for c in codes:
+        if c == 0:
+            batch = next(it_ids)
+            index, rows = t.lookup(batch)
+            idx_out.append(index), emb_out.append(rows)
+            pending = (index, next(it_grads))
+        elif c == 1:
+            t.apply(*pending)
+        elif c == 3:
+            batch = next(it_ids)
+            index = t.idmap.lookup_readonly(batch)
+            t._grow()
+            idx_out.append(index), emb_out.append(oracle.block_gather(index, t.emb, bs, -1, True))
+        else:
+            batch = next(it_ids)
+            index = t.idmap.lookup_readonly(batch)
+            t.idmap.delete(batch, index)
+            # every slot of a freed row goes back to its initial value (slot_group.cc:153-160)
+            oracle.block_insert(index, np.full((len(batch), D), init, np.float32), t.emb, bs)
+            oracle.block_insert(index, np.zeros((len(batch), D), np.float32), t.s0, bs)
+            oracle.block_insert(index, np.zeros((len(batch), D), np.float32), t.s1, bs)
+    np.testing.assert_array_equal(np.concatenate(idx_out), r_idx)
+    np.testing.assert_array_equal(np.concatenate(emb_out), r_emb)
+    o_ids, o_rows = t.idmap.snapshot()
+    np.testing.assert_array_equal(o_rows[np.argsort(o_ids)], r_rows[np.argsort(r_ids)])
+    np.testing.assert_array_equal(np.sort(o_ids), np.sort(r_ids))
+    np.testing.assert_array_equal(np.concatenate(t.emb), r_w)
+    np.testing.assert_array_equal(np.concatenate(t.s0), r_m)
+    np.testing.assert_array_equal(np.concatenate(t.s1), r_v)
