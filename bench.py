@@ -477,12 +477,53 @@ MEASURED_TRAFFIC_C4 = {
 }
 
 
+def checkpoint_round_trip(rows=8 << 20, dim=16, parallel=8):
+    """Save and load of one table with Adam state (rows x (8 B key + 3 x dim x 4 B)) through the
+    checkpoint directory layout, to a scratch directory under TMPDIR. Not part of the step metric."""
+    import shutil
+    import tempfile
+
+    from recis_amd.nn import HashTable
+    from recis_amd.nn.modules.hashtable import HashtableRegister, filter_out_sparse_param
+    from recis_amd.optim import SparseAdam
+    from recis_amd.serialize import Loader, Saver
+
+    def make(name):
+        HashtableRegister().clear()
+        ht = HashTable([dim], block_size=10240, device="cuda", name=name, children=["ckpt_bench"])
+        SparseAdam(filter_out_sparse_param(ht), lr=1e-3)
+        return ht
+
+    ht = make("ckpt_bench_src")
+    ids = torch.randperm(4 * rows, device="cuda")[:rows]
+    ht._hashtable_impl.insert(ids, torch.randn(rows, dim, device="cuda"))
+    nbytes = rows * (8 + 3 * dim * 4)
+    path = tempfile.mkdtemp(prefix="recis_ckpt_")
+    try:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        Saver(0, 1, parallel, path, hashtables={"t": ht}).save()
+        t_save = time.perf_counter() - t0
+        dst = make("ckpt_bench_dst")
+        t0 = time.perf_counter()
+        Loader(path, hashtables={"t": dst}, parallel=parallel).load()
+        torch.cuda.synchronize()
+        t_load = time.perf_counter() - t0
+        ok = dst._hashtable_impl.ids_num() == rows
+    finally:
+        shutil.rmtree(path, ignore_errors=True)
+    return {"metric": "table checkpoint round trip", "rows": rows, "bytes": nbytes, "files": parallel,
+            "save_s": round(t_save, 3), "save_GBps": round(nbytes / t_save / 1e9, 2),
+            "load_s": round(t_load, 3), "load_GBps": round(nbytes / t_load / 1e9, 2), "loaded_all_rows": ok,
+            "directory": os.path.dirname(path)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "ckpt"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--calib-copy", action="store_true",
@@ -497,6 +538,9 @@ def main():
     torch.cuda.set_device(0)
     os.environ.setdefault("OMP_NUM_THREADS", "1")
 
+    if args.workload == "ckpt":
+        print(json.dumps(checkpoint_round_trip()))
+        return
     classes = {"c4": Config4, "c2": Config2, "c3": Config3, "c5": Config5}
     main_wl = classes[args.workload]()
     for _ in range(args.warmup):

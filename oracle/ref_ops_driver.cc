@@ -8,6 +8,10 @@
 //   recis::embedding::IdAllocator                    (csrc/embedding/id_allocator.cc:17-60)
 //   Hashtable (EmbeddingLookup, AcceptGrad, Delete, ids_map, slots) with SparseAdam / SparseAdamW /
 //   SparseAdamWTF::step                              (csrc/embedding/hashtable.cc:46-278, adam*.cc)
+//   recis::serialize::WriteBlock::MakeHTWriteBlock / MakeTensorWriteBlock + TableWriter (one data
+//   file) and LoadBundle (directory index + file headers)  (csrc/serialize/write_block.cc:27-77,
+//   table_writer.cc:48-88, load_bundle.cc:17-112). Saver/Loader themselves (save_bundle.cc,
+//   load_internal.cc, read_block.cc) include CUDA headers and are not part of this build.
 //   recis::functional::mask_key_index_op, scatter_ids_with_mask_op (csrc/ops/hashtable_ops.cc:150-214)
 //   recis::functional::block_gather / block_insert / block_insert_with_mask / block_filter / gather
 //                                                    (csrc/ops/block_ops.cc:270-397)
@@ -35,6 +39,10 @@
 #include "embedding/initializer.h"
 #include "embedding/id_map.h"
 #include "ops/block_apply_adamw_op.h"
+#include "serialize/load_bundle.h"
+#include "serialize/name.h"
+#include "serialize/table_writer.h"
+#include "serialize/write_block.h"
 #include "ops/block_ops.h"
 #include "ops/fused_bucketized.h"
 #include "ops/fused_uint64_mod.h"
@@ -241,6 +249,59 @@ static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
             table->SlotGroup()->EmbSlot()->Value(),
             table->GetSlot(prefix + "exp_avg")->Value(),
             table->GetSlot(prefix + "exp_avg_sq")->Value()};
+  }
+  if (op == "ckpt_write_file") {
+    // Writes ONE data file with the reference's TableWriter from a CPU Hashtable and a dense tensor.
+    // path i8 [len] = directory, params i64 [5] = block_size, coalesced (0/1), slice begin, end, size,
+    // ids i64 [n] (already tagged when coalesced: two children "a" and "b"), rows f32 [n, D], dense f32 [...]
+    std::string dir(reinterpret_cast<const char*>(in[0].data_ptr<int8_t>()), in[0].numel());
+    const int64_t* p = in[1].data_ptr<int64_t>();
+    const int64_t D = in[3].size(1);
+    auto gen = recis::embedding::MakeConstantGenerator({p[0], D}, torch::kFloat, 0.0);
+    std::vector<std::string> children = p[1] ? std::vector<std::string>{"a", "b"} : std::vector<std::string>{"a"};
+    auto table = Hashtable::Make(p[0], {D}, torch::kFloat, torch::Device(torch::kCPU), p[1] != 0, children, gen,
+                                 p[2], p[3], p[4]);
+    table->AppendStepFilterSlot("step_filter", 7);
+    table->Insert(in[2], in[3]);
+    namespace S = recis::serialize;
+    auto writer = S::TableWriter::Make(dir, "ref.safetensors", "ref.json");
+    auto blocks = S::WriteBlock::MakeHTWriteBlock(table);
+    blocks.push_back(S::WriteBlock::MakeTensorWriteBlock("dense_w", in[4]));
+    for (auto& b : blocks) writer->AppendWriteBlock(b);
+    writer->SequentialWrite();
+    return {torch::tensor({static_cast<int64_t>(blocks.size())}, torch::kLong)};
+  }
+  if (op == "ckpt_inspect") {
+    // Reads a checkpoint directory with the reference's LoadBundle. path i8 [len].
+    // Returns names (i8, one per line: "<tensor>\t<c10::ScalarType number>\t<slice>"), then per line
+    // shape row [4] (padded with -1) and the absolute byte range [2] of the block in its file.
+    std::string dir(reinterpret_cast<const char*>(in[0].data_ptr<int8_t>()), in[0].numel());
+    namespace S = recis::serialize;
+    auto bundle = S::LoadBundle::Make(dir);
+    auto names = bundle->ListTensor();
+    std::sort(names.begin(), names.end());
+    std::string text;
+    std::vector<int64_t> shapes, ranges, total_shapes;
+    for (const auto& name : names) {
+      auto slices = bundle->SliceInfos(name);
+      std::sort(slices.begin(), slices.end());
+      auto total = bundle->TensorShape(name);
+      for (const auto& sl : slices) {
+        auto bn = S::BlockNameEncode(name, sl);
+        auto info = bundle->GetBlockInfo(bn);
+        text += name + "\t" + std::to_string(static_cast<int>(info->Dtype())) + "\t" + sl + "\n";
+        auto shp = info->Shape();
+        for (int d = 0; d < 4; ++d) shapes.push_back(d < static_cast<int>(shp.size()) ? shp[d] : -1);
+        for (int d = 0; d < 4; ++d) total_shapes.push_back(d < static_cast<int>(total.size()) ? total[d] : -1);
+        ranges.push_back(info->OffsetBeg());
+        ranges.push_back(info->OffsetEnd());
+      }
+    }
+    Tensor t = torch::empty({static_cast<int64_t>(text.size())}, torch::kChar);
+    memcpy(t.data_ptr(), text.data(), text.size());
+    const int64_t rows = static_cast<int64_t>(ranges.size() / 2);
+    return {t, torch::tensor(shapes, torch::kLong).view({rows, 4}), torch::tensor(ranges, torch::kLong).view({rows, 2}),
+            torch::tensor(total_shapes, torch::kLong).view({rows, 4})};
   }
   if (op == "mask_key_index") {  // keys, mask (bool), cumsum, out_size [1]
     auto r = F::mask_key_index_op(in[0], in[1], in[2], in[3].item<int64_t>());

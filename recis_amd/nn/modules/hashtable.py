@@ -160,6 +160,9 @@ class Slot:
         parts = self._chunks[:full] + ([self._chunks[full][:rest]] if rest else [])
         return torch.cat(parts, 0)
 
+    def row_shape(self):
+        return list(self._row_shape)
+
     def index_select(self, index, beg=0, end=None):
         end = index.numel() if end is None else end
         return ops.block_gather_by_range(index, self._chunks, self._chunk_rows, beg, end)
@@ -355,6 +358,14 @@ class HashtableImpl:
         ids = ids.to(self._device)
         index = self._idmap.lookup(ids)
         self._make_room(ids.numel())
+        return index
+
+    def insert_lookup_index_with_indicator(self, ids, indicator):
+        """hashtable.cc:237-248: rows of the ids whose indicator is set (inserted when new), 0
+        for the others."""
+        ids, indicator = ids.to(self._device), indicator.to(self._device)
+        index = torch.zeros_like(ids)
+        index.masked_scatter_(indicator, self.insert_lookup_index(torch.masked_select(ids, indicator)))
         return index
 
     def insert(self, ids, embedding):
