@@ -470,6 +470,85 @@ int recis_fused_multi_hash(const int64_t* const* in_ptrs, const int64_t* sizes,
                            const int64_t* muls, const int64_t* primes, const int64_t* buckets,
                            int64_t* const* out_ptrs, int64_t n_jobs, void* stream);
 
+/* ------------------------------------------------------------------------- *
+ * Sequence truncation of lists of ragged tensors
+ * ------------------------------------------------------------------------- */
+
+/*
+ * fused_ragged_cutoff (2-D, inner_ptrs == NULL) and fused_ragged_cutoff_3D, the op functions of
+ * csrc/ops/fused_ragged_cutoff.cc:10-140 and :143-287 (kernels post_cutoff_lens_kernel,
+ * seg_scan_sum_kernel, seg_gen_offsets_kernel, fused_ragged_cutoff_kernel.cu:29-70,100-160,
+ * 260-371), for n_tensors ragged tensors at once. Lists are HOST arrays of device pointers.
+ *
+ * 2-D, tensor t with offsets outer_ptrs[t] [n_rows[t] + 1]: row r keeps min(len, keep[t])
+ * elements, the first ones, or the last ones when drop_left[t]; out_offsets_ptrs[t]
+ * [n_rows[t] + 1] receives the new offsets, drop_nums_ptrs[t] / pad_nums_ptrs[t] [n_rows[t]]
+ * (each may be NULL) len - keep where len >= keep (else 0) and keep - len where len < keep
+ * (else 0). pad_left is not used: a 2-D result is not padded.
+ * 3-D, outer offsets [n_rows[t] + 1] over inner rows, inner offsets inner_ptrs[t]
+ * [n_inner_rows[t] + 1] over values: every sequence comes out with exactly keep[t] inner rows.
+ * A longer one loses inner rows at the end (at the start when drop_left[t]); a shorter one gets
+ * empty rows at the end (at the start when pad_left[t]). out_outer_ptrs[t] [n_rows[t] + 1] =
+ * k * keep[t]; out_offsets_ptrs[t] [n_rows[t] * keep[t] + 1] = new inner offsets; drop / pad
+ * counts are per sequence.
+ * Both: src_ptrs[t] (int64 [output rows], caller's scratch, read by recis_ragged_cutoff_copy)
+ * receives the position of every output row's first element in the source values;
+ * totals_dev [n_tensors] the number of values each tensor keeps. Offsets are int32 or int64
+ * (off_is64), the same for inputs and outputs. A source range outside [0, n_values[t]) or an
+ * inner row outside [0, n_inner_rows[t]) gives an empty row and raises
+ * RECIS_DEVERR_INDEX_RANGE. Nothing here waits for the device.
+ */
+int recis_ragged_cutoff_rows(const void* const* outer_ptrs, const void* const* inner_ptrs,
+                             int off_is64, const int64_t* n_rows, const int64_t* n_inner_rows,
+                             const int64_t* n_values, const int64_t* keep,
+                             const uint8_t* drop_left, const uint8_t* pad_left, int64_t n_tensors,
+                             void* const* out_offsets_ptrs, void* const* out_outer_ptrs,
+                             void* const* drop_nums_ptrs, void* const* pad_nums_ptrs,
+                             int64_t* const* src_ptrs, int64_t* totals_dev, void* stream);
+
+/*
+ * The values of a cutoff (fused_ragged_cutoff_kernel / fused_ragged_cutoff_3D_kernel,
+ * fused_ragged_cutoff_kernel.cu:462-556,634-728): out_values_ptrs[t][e] for e < totals[t]
+ * (HOST array: what recis_ragged_cutoff_rows left in totals_dev, read back by the caller to
+ * size the outputs) = values_ptrs[t][src + (e - offset)] of the output row that holds e.
+ * elem_size 1, 2, 4 or 8 bytes. n_out_rows[t] = rows (2-D) or rows * keep (3-D).
+ */
+int recis_ragged_cutoff_copy(const void* const* values_ptrs, int elem_size,
+                             const void* const* out_offsets_ptrs, int off_is64,
+                             const int64_t* n_out_rows, const int64_t* const* src_ptrs,
+                             const int64_t* totals, void* const* out_values_ptrs,
+                             int64_t n_tensors, void* stream);
+
+/* element kinds of recis_dense_to_ragged_rows (the types the reference dispatches on) */
+#define RECIS_SEQ_F32 0
+#define RECIS_SEQ_F64 1
+#define RECIS_SEQ_I32 2
+#define RECIS_SEQ_I64 3
+
+/*
+ * ragged_to_dense_cuda (csrc/ops/ragged_to_dense_kernel.cu:34-152; CPU twin ragged_to_dense.cc:6-45):
+ * out [batch, widths[0], ..., widths[n_dims-1]] (batch = offsets_sizes[0] - 1) takes
+ * values[...] where every coordinate lies inside its row, default_value (elem_size raw bytes)
+ * elsewhere. offsets_ptrs / offsets_sizes / widths are HOST arrays (n_dims <= 5); the widths are
+ * the caller's (the reference takes the longest row of every level, which costs it a read-back
+ * per level; a row longer than its width is cut).
+ */
+int recis_ragged_to_dense(const void* values, int elem_size, int64_t n_values,
+                          const void* const* offsets_ptrs, const int64_t* offsets_sizes,
+                          int off_is64, const int64_t* widths, int n_dims,
+                          const void* default_value, void* out, void* stream);
+
+/*
+ * dense_to_ragged_cuda (csrc/ops/dense_to_ragged_kernel.cu:16-83), offsets part: the length of
+ * row r of data [rows, cols] is the position after its last element != *invalid_value;
+ * out_offsets (int32 [rows + 1]) receives the running sum, src (int64 [rows], caller's scratch)
+ * r * cols, total_dev [1] the number of values. The values follow from
+ * recis_ragged_cutoff_copy(data, ..., out_offsets, 0, rows, src, total, ...).
+ */
+int recis_dense_to_ragged_rows(const void* data, int dtype_kind, int64_t rows, int64_t cols,
+                               const void* invalid_value, int32_t* out_offsets, int64_t* src,
+                               int64_t* total_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

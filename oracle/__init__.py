@@ -402,3 +402,93 @@ def hash_strings(values, offsets, kind):
     lib().oracle_hash_strings(_p(values), _p(offsets), c_i64(n), {"farm": 0, "murmur": 1}[kind],
                               _p(out))
     return out
+
+
+# ------------------------------------------------------- sequence truncation
+
+
+def ragged_cutoff_2d(values, offsets, keep, drop_left):
+    """One 2-D ragged tensor cut to at most ``keep`` elements per row
+    (csrc/ops/fused_ragged_cutoff_kernel.cu:55-69 lengths, :706-727 which elements stay).
+    Returns (values, offsets, drop_nums, pad_nums)."""
+    values, offsets = np.asarray(values), np.asarray(offsets)
+    out_v, out_o, drops, pads = [], [0], [], []
+    for r in range(len(offsets) - 1):
+        beg, end = int(offsets[r]), int(offsets[r + 1])
+        n = end - beg
+        dropped = n >= keep
+        k = keep if dropped else n
+        drop = n - keep if dropped else 0
+        drops.append(drop)
+        pads.append(0 if dropped else keep - n)
+        first = beg + (drop if drop_left else 0)
+        out_v.append(values[first:first + k])
+        out_o.append(out_o[-1] + k)
+    vals = np.concatenate(out_v) if out_v else values[:0]
+    return vals, np.asarray(out_o, offsets.dtype), np.asarray(drops, offsets.dtype), np.asarray(pads, offsets.dtype)
+
+
+def ragged_cutoff_3d(values, outer, inner, keep, drop_left, pad_left):
+    """One 3-D ragged tensor with every sequence brought to exactly ``keep`` inner rows
+    (csrc/ops/fused_ragged_cutoff_kernel.cu:300-337 which inner row lands where, :513-550 the values).
+    Returns (values, outer_offsets, inner_offsets)."""
+    values, outer, inner = np.asarray(values), np.asarray(outer), np.asarray(inner)
+    out_v, out_inner = [], [0]
+    n_seq = len(outer) - 1
+    for s in range(n_seq):
+        beg, end = int(outer[s]), int(outer[s + 1])
+        n = end - beg
+        drop = n - keep if n >= keep else 0
+        pad = 0 if n >= keep else keep - n
+        for col in range(keep):
+            row, padded = col, False
+            if drop > 0:
+                if drop_left:
+                    row += drop
+            elif pad > 0:
+                if pad_left:
+                    padded = col < pad
+                    row -= pad
+                else:
+                    padded = keep <= pad + col
+            if padded:
+                out_inner.append(out_inner[-1])
+            else:
+                b, e = int(inner[beg + row]), int(inner[beg + row + 1])
+                out_v.append(values[b:e])
+                out_inner.append(out_inner[-1] + (e - b))
+    vals = np.concatenate(out_v) if out_v else values[:0]
+    return vals, (np.arange(n_seq + 1) * keep).astype(outer.dtype), np.asarray(out_inner, inner.dtype)
+
+
+def ragged_to_dense(values, offsets, default_value=0):
+    """Dense ``[batch, longest row of every level]`` of a ragged tensor with several levels of
+    offsets, ``default_value`` outside the rows (csrc/ops/ragged_to_dense.cc:6-45; the walk of
+    ragged_common.cuh:36-64)."""
+    values = np.asarray(values)
+    offsets = [np.asarray(o) for o in offsets]
+    widths = [int((o[1:] - o[:-1]).max()) if len(o) > 1 else 0 for o in offsets]
+    out = np.full([len(offsets[0]) - 1] + widths, default_value, values.dtype)
+    for coord in np.ndindex(*out.shape):
+        at = coord[0]
+        for d, o in enumerate(offsets):
+            beg, end = int(o[at]), int(o[at + 1])
+            if coord[d + 1] >= end - beg:
+                break
+            at = beg + coord[d + 1]
+        else:
+            out[coord] = values[at]
+    return out
+
+
+def dense_to_ragged(data, invalid_value):
+    """(values, int32 offsets): every row up to its last element that differs from
+    ``invalid_value`` (csrc/ops/dense_to_ragged.cc:6-53)."""
+    data = np.asarray(data)
+    vals, offs = [], [0]
+    for row in data:
+        keep = np.nonzero(row != invalid_value)[0]
+        n = int(keep[-1]) + 1 if len(keep) else 0
+        vals.append(row[:n])
+        offs.append(offs[-1] + n)
+    return (np.concatenate(vals) if vals else data.reshape(-1)[:0]), np.asarray(offs, np.int32)

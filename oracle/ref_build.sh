@@ -33,7 +33,7 @@ OBJ="$HERE/_ref/obj"
 mkdir -p "$OBJ"
 CXXFLAGS="-std=c++17 -O2 -fPIC -fopenmp -w -D_GLIBCXX_USE_CXX11_ABI=$ABI -I$CSRC -I$CSRC/ops -I$REF/third_party -I$TORCH/include -I$TORCH/include/torch/csrc/api/include -I$PYINC"
 SOURCES="ops/block_apply_adamw_op.cc ops/hashtable_ops.cc ops/block_ops.cc ops/ids_partition.cc ops/ids_encode.cc
-         ops/fused_uint64_mod.cc ops/fused_bucketized.cc ops/multi_hash.cc
+         ops/fused_uint64_mod.cc ops/fused_bucketized.cc ops/multi_hash.cc ops/dense_to_ragged.cc
          embedding/id_allocator.cc embedding/cpu_id_map.cc embedding/parallel_util.cc
          embedding/hashtable.cc embedding/slot_group.cc embedding/initializer.cc embedding/children_info.cc
          embedding/slice_info.cc embedding/optim.cc embedding/adam.cc embedding/adamw.cc embedding/adamw_tf.cc

@@ -16,7 +16,7 @@
 //   recis::functional::block_gather / block_insert / block_insert_with_mask / block_filter / gather
 //                                                    (csrc/ops/block_ops.cc:270-397)
 //   recis::functional::ids_partition_cpu, ids_encode_cpu, fused_uint64_mod, fused_bucketized,
-//   fused_multi_hash                                 (csrc/ops/*.cc)
+//   fused_multi_hash, dense_to_ragged                (csrc/ops/*.cc)
 // (segment_sum / segment_mean have no CPU implementation in the reference: segment_ops.cc only
 // forwards to the CUDA functions.)
 // The reference objects also refer to their CUDA counterparts (*_cuda, *_gpu); those symbols are
@@ -44,6 +44,7 @@
 #include "serialize/table_writer.h"
 #include "serialize/write_block.h"
 #include "ops/block_ops.h"
+#include "ops/dense_to_ragged.h"
 #include "ops/fused_bucketized.h"
 #include "ops/fused_uint64_mod.h"
 #include "ops/hashtable_ops.h"
@@ -302,6 +303,10 @@ static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
     const int64_t rows = static_cast<int64_t>(ranges.size() / 2);
     return {t, torch::tensor(shapes, torch::kLong).view({rows, 4}), torch::tensor(ranges, torch::kLong).view({rows, 2}),
             torch::tensor(total_shapes, torch::kLong).view({rows, 4})};
+  }
+  if (op == "dense_to_ragged") {  // data [rows, cols], invalid value [1] of the same dtype
+    auto r = F::dense_to_ragged(in[0], true, in[1]);
+    return {std::get<0>(r), std::get<1>(r)};
   }
   if (op == "mask_key_index") {  // keys, mask (bool), cumsum, out_size [1]
     auto r = F::mask_key_index_op(in[0], in[1], in[2], in[3].item<int64_t>());

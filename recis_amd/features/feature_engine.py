@@ -1,7 +1,7 @@
 """``FeatureEngine``: runs a list of features step by step, batching the same-typed ops
 of one step into ONE fused HIP launch (mirror of ``recis.features.feature_engine``,
 feature_engine.py:107-284, with the fused implementations of fused_op_impl.py:113-516
-for Mod, Bucketize, Hash and IDMultiHash). Features with identical op chains are computed
+for Mod, Bucketize, Hash, IDMultiHash and SequenceTruncate). Features with identical op chains are computed
 once and shared."""
 from collections import defaultdict
 from typing import Dict, List
@@ -11,7 +11,7 @@ from torch import nn
 from .. import ops
 from ..ragged.tensor import RaggedTensor
 from .feature import Feature
-from .op import Bucketize, Hash, IDMultiHash, Mod, _values, _with_values
+from .op import Bucketize, Hash, IDMultiHash, Mod, SequenceTruncate, _values, _with_values, sequence_truncate
 
 
 def _fused_mod(op_list, inputs):
@@ -52,7 +52,8 @@ def _fused_multi_hash(op_list, inputs):
     return results
 
 
-_FUSED = {Mod: _fused_mod, Bucketize: _fused_bucketize, Hash: _fused_hash, IDMultiHash: _fused_multi_hash}
+_FUSED = {Mod: _fused_mod, Bucketize: _fused_bucketize, Hash: _fused_hash, IDMultiHash: _fused_multi_hash,
+          SequenceTruncate: sequence_truncate}
 
 
 class FeatureEngine(nn.Module):

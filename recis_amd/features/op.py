@@ -1,7 +1,6 @@
 """Feature-engine ops on the hot path: the mirror of ``recis.features.op`` for
-``SelectField``, ``Mod``, ``Bucketize``, ``Hash`` and ``IDMultiHash``
-(recis/features/op.py:129-686). ``SequenceTruncate`` and ``FeatureCross`` belong to
-the ops that feed this path and are not part of this build.
+``SelectField``, ``Mod``, ``Bucketize``, ``Hash``, ``IDMultiHash`` and ``SequenceTruncate``
+(recis/features/op.py:129-686). ``FeatureCross`` is not part of this build.
 
 Every op works on a ``RaggedTensor`` (its values) or a plain tensor; the engine
 batches same-typed ops of one step into a single fused HIP launch.
@@ -139,3 +138,54 @@ class IDMultiHash(_OP):
 
     def _get_config(self):
         return {"num_buckets": self.num_buckets, "prefix": self.prefix}
+
+
+class SequenceTruncate(_OP):
+    """Cuts every sequence to ``seq_len`` (recis/features/op.py:408-517): a 2-D ragged tensor
+    keeps at most ``seq_len`` elements per row; a 3-D one comes out with exactly ``seq_len`` inner
+    rows per sequence (missing ones empty, added at the end). ``truncate_side`` "left" drops the
+    oldest entries (the start of the row)."""
+
+    def __init__(self, seq_len=64, check_length=True, truncate=True, truncate_side="left", n_dims=2,
+                 dtype=torch.long):
+        super().__init__()
+        assert n_dims in [2, 3]
+        self.n_dims, self.seq_len, self.check_length = n_dims, int(seq_len), check_length
+        self.truncate, self.truncate_side, self.dtype = truncate, truncate_side, dtype
+
+    def forward(self, x: RaggedTensor):
+        if self.check_length:
+            assert x.dense_shape[1] <= self.seq_len, "sequence length must be less than %d" % self.seq_len
+        if not self.truncate:
+            return None  # as the reference (op.py:489-507 has no other branch)
+        return sequence_truncate([self], [x])[0]
+
+    def _get_config(self):
+        return {"seq_len": self.seq_len, "check_length": self.check_length, "truncate": self.truncate,
+                "truncate_side": self.truncate_side, "n_dims": self.n_dims, "dtype": str(self.dtype)}
+
+
+def sequence_truncate(op_list, inputs):
+    """One fused launch per (value dtype, dimensionality) group (FusedCutoffOP, fused_op_impl.py:274-390)."""
+    from ..nn.functional import ragged_ops
+
+    results = [None] * len(inputs)
+    groups = {}
+    for i, (op, x) in enumerate(zip(op_list, inputs)):
+        groups.setdefault((x.values().dtype, op.n_dims), []).append(i)
+    for (_, n_dims), idx in groups.items():
+        keep = [op_list[i].seq_len for i in idx]
+        drop = [op_list[i].truncate_side == "left" for i in idx]
+        pad = [False] * len(idx)
+        vals = [inputs[i].values().cuda() for i in idx]
+        if n_dims == 2:
+            out = ragged_ops.fused_ragged_cutoff_2D(vals, [inputs[i].offsets()[-1].cuda() for i in idx], keep, drop, pad)
+            new_vals, new_offs = out[0], [[o] for o in out[1]]
+        else:
+            new_vals, new_offs = ragged_ops.fused_ragged_cutoff_3D(
+                vals, [[o.cuda() for o in inputs[i].offsets()] for i in idx], keep, drop, pad)
+        for k, i in enumerate(idx):
+            shape = list(inputs[i].dense_shape)
+            shape[1] = op_list[i].seq_len
+            results[i] = RaggedTensor(new_vals[k], new_offs[k], inputs[i].weight(), shape)
+    return results

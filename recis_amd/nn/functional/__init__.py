@@ -1,1 +1,1 @@
-from . import embedding_ops, fused_ops, hash_ops  # noqa: F401
+from . import embedding_ops, fused_ops, hash_ops, ragged_ops  # noqa: F401

@@ -850,3 +850,169 @@ def segment_reduce_backward_plan(grad_output, weight, offsets, plan, mode, out=N
                                  cover=offsets if offsets.numel() else None)
     src, coef = plan.src_coef_for_pool(offsets, weight, mode == "mean")
     return csr_gather_reduce(grad_output, plan, src, coef, out=out, accumulate=accumulate)
+
+
+# ------------------------------------------------------------ sequence truncation
+
+
+def _host_list(x, n, name):
+    """keep_lengths / drop_sides / pad_sides as a host list of n entries (a device tensor is read
+    back: pass host values where the step must not wait)."""
+    v = x.reshape(-1).tolist() if torch.is_tensor(x) else list(x)
+    if len(v) != n:
+        raise RuntimeError("%s.numel() = %d but is expected equals fea_num = %d" % (name, len(v), n))
+    return v
+
+
+def _host_u8(values):
+    return (ctypes.c_uint8 * len(values))(*[1 if v else 0 for v in values])
+
+
+def _ragged_cutoff(values, outer, inner, keep_lengths, drop_sides, pad_sides):
+    n = len(values)
+    if len(outer) != n or (inner is not None and len(inner) != n):
+        raise RuntimeError("offsets.numel() = %d but is expected equals fea_num = %d" % (len(outer), n))
+    require_cuda(*values)
+    require_cuda(*outer)
+    values = [_contig(v).reshape(-1) for v in values]
+    outer = [_contig(o) for o in outer]
+    if any(v.dtype != values[0].dtype for v in values):
+        raise RuntimeError("fused_ragged_cutoff: each value should be the same type")
+    is64 = _index_kind(outer[0], "offsets")
+    every = outer + ([_contig(o) for o in inner] if inner is not None else [])
+    if any(_index_kind(o, "offsets") != is64 for o in every):
+        raise RuntimeError("fused_ragged_cutoff: each offsets should be torch.int32 or torch.int64")
+    if inner is not None:
+        require_cuda(*inner)
+        inner = every[n:]
+    keep = _host_list(keep_lengths, n, "keep_lengths")
+    drop = _host_list(drop_sides, n, "drop_sides")
+    pad = _host_list(pad_sides, n, "pad_sides")
+    dev, odt = values[0].device, outer[0].dtype
+    rows = [o.numel() - 1 for o in outer]
+    out_rows = [r * k for r, k in zip(rows, keep)] if inner is not None else rows
+    # one allocation per kind of output, one view per tensor (as the reference slices its buffers)
+    off_buf = torch.empty(sum(out_rows) + n, dtype=odt, device=dev)
+    src_buf = torch.empty(max(sum(out_rows), 1), dtype=torch.int64, device=dev)
+    cnt_buf = torch.empty(2 * sum(rows), dtype=odt, device=dev)
+    totals = torch.empty(n, dtype=torch.int64, device=dev)
+    out_off, src, drop_nums, pad_nums, out_outer = [], [], [], [], []
+    a = b = 0
+    for t in range(n):
+        out_off.append(off_buf[a + t: a + t + out_rows[t] + 1])
+        src.append(src_buf[a: a + out_rows[t]] if out_rows[t] else src_buf[:0])
+        drop_nums.append(cnt_buf[b: b + rows[t]])
+        pad_nums.append(cnt_buf[sum(rows) + b: sum(rows) + b + rows[t]])
+        a += out_rows[t]
+        b += rows[t]
+    if inner is not None:
+        outer_buf = torch.empty(sum(rows) + n, dtype=odt, device=dev)
+        b = 0
+        for t in range(n):
+            out_outer.append(outer_buf[b + t: b + t + rows[t] + 1])
+            b += rows[t]
+    sp = stream_ptr(dev)
+
+    def ptrs_or_dummy(ts):   # an empty view has no address: any valid one will do, it is never used
+        return (ctypes.c_void_p * len(ts))(*[t.data_ptr() if t.numel() else src_buf.data_ptr() for t in ts])
+
+    check(lib().recis_ragged_cutoff_rows(
+        _host_ptrs(outer), _host_ptrs(inner) if inner is not None else None, is64, _host_i64(rows),
+        _host_i64([o.numel() - 1 for o in inner]) if inner is not None else None,
+        _host_i64([v.numel() for v in values]), _host_i64(keep), _host_u8(drop), _host_u8(pad), i64(n),
+        _host_ptrs(out_off), _host_ptrs(out_outer) if inner is not None else None, ptrs_or_dummy(drop_nums),
+        ptrs_or_dummy(pad_nums), ptrs_or_dummy(src), ptr(totals), sp))
+    total_host = totals.tolist()   # the one wait of this op: the outputs are sized by it
+    val_buf = torch.empty(sum(total_host), dtype=values[0].dtype, device=dev)
+    out_vals, a = [], 0
+    for t in range(n):
+        out_vals.append(val_buf[a: a + total_host[t]])
+        a += total_host[t]
+    check(lib().recis_ragged_cutoff_copy(
+        ptrs_or_dummy(values), values[0].element_size(), _host_ptrs(out_off), is64, _host_i64(out_rows),
+        ptrs_or_dummy(src), _host_i64(total_host), ptrs_or_dummy(out_vals), i64(n), sp))
+    return out_vals, out_off, drop_nums, pad_nums, out_outer
+
+
+def fused_ragged_cutoff(values, offsets, keep_lengths, drop_sides, pad_sides):
+    """``torch.ops.recis.fused_ragged_cutoff`` (fused_ragged_cutoff.cc:10-140): every row of every
+    2-D ragged tensor cut to at most keep_lengths[t] elements (the last ones when drop_sides[t]).
+    Returns (values, offsets, drop_nums, pad_nums, drop_sides, pad_sides)."""
+    if not values:
+        return [], [], [], [], drop_sides, pad_sides
+    vals, offs, drop_nums, pad_nums, _ = _ragged_cutoff(values, offsets, None, keep_lengths, drop_sides, pad_sides)
+    return vals, offs, drop_nums, pad_nums, drop_sides, pad_sides
+
+
+def fused_ragged_cutoff_3D(values, outer_offsets, inner_offsets, keep_lengths, drop_sides, pad_sides):
+    """``torch.ops.recis.fused_ragged_cutoff_3D`` (fused_ragged_cutoff.cc:143-287): every sequence
+    of every 3-D ragged tensor brought to exactly keep_lengths[t] inner rows, by dropping inner
+    rows or adding empty ones. Returns (values, outer_offsets, inner_offsets)."""
+    if not values:
+        return [], [], []
+    vals, inner, _, _, outer = _ragged_cutoff(values, outer_offsets, inner_offsets, keep_lengths, drop_sides,
+                                               pad_sides)
+    return vals, outer, inner
+
+
+# ------------------------------------------------------------ dense <-> ragged
+
+_SEQ_KIND = {torch.float32: 0, torch.float64: 1, torch.int32: 2, torch.int64: 3}
+
+
+def _scalar_bytes(value, dtype):
+    return torch.tensor([value], dtype=dtype).view(torch.uint8).numpy().tobytes()
+
+
+def ragged_to_dense(values, offsets, default_value=0, widths=None):
+    """``torch.ops.recis.ragged_to_dense`` (ragged_to_dense.cc:47-100): dense
+    ``[batch, max width of every ragged level]`` with ``default_value`` outside the rows.
+    ``widths`` (one per level) skips the read-back of the longest rows."""
+    require_cuda(values, *offsets)
+    if values.dim() != 1:
+        raise RuntimeError("values must dim == 1")
+    values = _contig(values)
+    offsets = [_contig(o) for o in offsets]
+    is64 = _index_kind(offsets[0], "offsets")
+    if any(_index_kind(o, "offsets") != is64 for o in offsets):
+        raise RuntimeError("ragged_to_dense: each offsets should be torch.int32 or torch.int64")
+    if widths is None:
+        widths = [int((o[1:] - o[:-1]).max()) if o.numel() > 1 else 0 for o in offsets]
+    shape = [offsets[0].numel() - 1] + [int(w) for w in widths]
+    out = torch.empty(shape, dtype=values.dtype, device=values.device)
+    fill = _scalar_bytes(default_value, values.dtype)
+    check(lib().recis_ragged_to_dense(ptr(values), values.element_size(), i64(values.numel()), _host_ptrs(offsets),
+                                      _host_i64([o.numel() for o in offsets]), is64, _host_i64(shape[1:]),
+                                      len(offsets), ctypes.c_char_p(fill), ptr(out), stream_ptr(values.device)))
+    return out
+
+
+def dense_to_ragged(data, check_invalid=True, invalid_value=0):
+    """``torch.ops.recis.dense_to_ragged`` (dense_to_ragged.cc:56-76): (values, int32 offsets) of a
+    2-D tensor; with ``check_invalid`` the trailing run of ``invalid_value`` of every row is dropped."""
+    if data.dim() != 2:
+        raise RuntimeError("Input must be a 2D tensor")
+    require_cuda(data)
+    rows, cols = data.shape
+    if not check_invalid:
+        return data.reshape(-1), torch.arange(0, rows * cols + 1, max(cols, 1), dtype=torch.int32,
+                                              device=data.device)[: rows + 1]
+    if data.dtype not in _SEQ_KIND:
+        raise TypeError("dense_to_ragged: float32, float64, int32 or int64 data, got %s" % data.dtype)
+    data = _contig(data)
+    if torch.is_tensor(invalid_value):
+        invalid_value = invalid_value.reshape(-1)[0].item()
+    offsets = torch.empty(rows + 1, dtype=torch.int32, device=data.device)
+    src = torch.empty(max(rows, 1), dtype=torch.int64, device=data.device)
+    total = torch.empty(1, dtype=torch.int64, device=data.device)
+    sp = stream_ptr(data.device)
+    check(lib().recis_dense_to_ragged_rows(ptr(data), _SEQ_KIND[data.dtype], i64(rows), i64(cols),
+                                           ctypes.c_char_p(_scalar_bytes(invalid_value, data.dtype)), ptr(offsets),
+                                           ptr(src), ptr(total), sp))
+    n = int(total.item())
+    values = torch.empty(n, dtype=data.dtype, device=data.device)
+    if n:
+        check(lib().recis_ragged_cutoff_copy(_host_ptrs([data]), data.element_size(), _host_ptrs([offsets]), 0,
+                                             _host_i64([rows]), _host_ptrs([src]), _host_i64([n]),
+                                             _host_ptrs([values]), i64(1), sp))
+    return values, offsets

@@ -71,20 +71,22 @@ class RaggedTensor:
         return RaggedTensor(self._values.clone(), [o.clone() for o in self._offsets],
                             None if self._weight is None else self._weight.clone(), self._dense_shape)
 
+    def dim(self):
+        return len(self._dense_shape)
+
     def to_dense(self, default_value=0):
-        """Pads the innermost ragged dimension (one level) to its longest row."""
-        if len(self._offsets) != 1:
-            raise NotImplementedError("to_dense handles one ragged dimension")
-        off = self._offsets[0].long()
-        lens = off[1:] - off[:-1]
-        rows = lens.numel()
-        width = int(lens.max().item()) if rows else 0
-        out = torch.full((rows, width), default_value, dtype=self._values.dtype, device=self._values.device)
-        if self._values.numel():
-            row = torch.repeat_interleave(torch.arange(rows, device=off.device), lens)
-            col = torch.arange(self._values.numel(), device=off.device) - off[:-1][row]
-            out[row, col] = self._values
-        return out
+        """Dense ``[rows, longest row of every ragged level]`` (tensor.py:229-248)."""
+        from .. import ops
+
+        return ops.ragged_to_dense(self._values, self._offsets, default_value)
+
+    @staticmethod
+    def from_dense(dense: torch.Tensor):
+        """Rows up to their last non-zero element (tensor.py:277-294)."""
+        from .. import ops
+
+        values, offsets = ops.dense_to_ragged(dense, True, 0)
+        return RaggedTensor(values, offsets, dense_shape=tuple(dense.shape))
 
     def __repr__(self):
         return "RaggedTensor(values=%s, offsets=%s, weight=%s)" % (

@@ -1,0 +1,203 @@
+"""Sequence ops on the GPU against the CPU oracle, bit for bit: truncation of lists of 2-D / 3-D
+ragged tensors, ragged_to_dense, dense_to_ragged (all through the C ABI)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from recis_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [(np.int64, torch.int64), (np.float32, torch.float32), (np.float64, torch.float64), (np.int32, torch.int32),
+          (np.int8, torch.int8), (np.float16, torch.float16)]
+
+
+def _ragged(rng, rows, max_len, off_dtype, empty_frac=0.2):
+    lens = rng.integers(0, max_len + 1, rows)
+    lens[rng.random(rows) < empty_frac] = 0
+    return np.concatenate([[0], np.cumsum(lens)]).astype(off_dtype)
+
+
+def _values(rng, n, np_dtype):
+    if np.issubdtype(np_dtype, np.integer):
+        info = np.iinfo(np_dtype)
+        return rng.integers(max(info.min, -(1 << 40)), min(info.max, 1 << 40), n).astype(np_dtype)
+    return rng.standard_normal(n).astype(np_dtype)
+
+
+@pytest.mark.parametrize("off_dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("np_dtype,t_dtype", DTYPES)
+def test_cutoff_2d_list_matches_oracle(rng, off_dtype, np_dtype, t_dtype):
+    n_tensors = 27   # more than one launch of the job table
+    rows = [int(r) for r in rng.integers(0, 5000, n_tensors)]
+    rows[3] = 0
+    offs = [_ragged(rng, r, 12, off_dtype) for r in rows]
+    vals = [_values(rng, int(o[-1]), np_dtype) for o in offs]
+    keep = [int(k) for k in rng.integers(0, 9, n_tensors)]
+    drop = [bool(b) for b in rng.integers(0, 2, n_tensors)]
+    pad = [bool(b) for b in rng.integers(0, 2, n_tensors)]
+    got = ops.fused_ragged_cutoff([torch.from_numpy(v).cuda() for v in vals], [torch.from_numpy(o).cuda() for o in offs],
+                                  torch.tensor(keep, dtype=torch.int32), torch.tensor(drop), torch.tensor(pad))
+    for t in range(n_tensors):
+        v, o, d, p = oracle.ragged_cutoff_2d(vals[t], offs[t], keep[t], drop[t])
+        assert got[0][t].dtype == t_dtype and got[1][t].dtype == torch.from_numpy(offs[t]).dtype
+        np.testing.assert_array_equal(got[0][t].cpu().numpy(), v)
+        np.testing.assert_array_equal(got[1][t].cpu().numpy(), o)
+        np.testing.assert_array_equal(got[2][t].cpu().numpy(), d)
+        np.testing.assert_array_equal(got[3][t].cpu().numpy(), p)
+    assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("off_dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("drop,pad", [(False, False), (True, False), (False, True), (True, True)])
+def test_cutoff_3d_list_matches_oracle(rng, off_dtype, drop, pad):
+    n_tensors = 6
+    outer = [_ragged(rng, int(r), 9, off_dtype) for r in rng.integers(0, 3000, n_tensors)]
+    inner = [_ragged(rng, int(o[-1]), 5, off_dtype) for o in outer]
+    vals = [_values(rng, int(i[-1]), np.int64) for i in inner]
+    keep = [int(k) for k in rng.integers(1, 8, n_tensors)]
+    got = ops.fused_ragged_cutoff_3D([torch.from_numpy(v).cuda() for v in vals],
+                                     [torch.from_numpy(o).cuda() for o in outer],
+                                     [torch.from_numpy(i).cuda() for i in inner], keep, [drop] * n_tensors,
+                                     [pad] * n_tensors)
+    for t in range(n_tensors):
+        v, o, i = oracle.ragged_cutoff_3d(vals[t], outer[t], inner[t], keep[t], drop, pad)
+        np.testing.assert_array_equal(got[0][t].cpu().numpy(), v)
+        np.testing.assert_array_equal(got[1][t].cpu().numpy(), o)
+        np.testing.assert_array_equal(got[2][t].cpu().numpy(), i)
+    assert _lib.poll_device_errors() == 0
+
+
+def test_cutoff_reference_examples():
+    # recis/nn/functional/ragged_ops.py:225-252
+    v, o, i = ops.fused_ragged_cutoff_3D([torch.arange(10, 20).cuda()],
+                                         [torch.tensor([0, 3, 4, 6], dtype=torch.int32).cuda()],
+                                         [torch.tensor([0, 1, 4, 4, 8, 8, 10], dtype=torch.int32).cuda()],
+                                         torch.tensor([2], dtype=torch.int32).cuda(), torch.tensor([True]).cuda(),
+                                         torch.tensor([True]).cuda())
+    assert v[0].tolist() == [11, 12, 13, 14, 15, 16, 17, 18, 19]
+    assert o[0].tolist() == [0, 2, 4, 6] and i[0].tolist() == [0, 3, 3, 3, 7, 7, 9]
+    # tests/feature_engine/op_test.py:81-93
+    out = ops.fused_ragged_cutoff([torch.randn(512).cuda()], [torch.tensor([0, 256, 512], dtype=torch.int32).cuda()],
+                                  [128], [True], [False])
+    assert out[1][0].tolist() == [0, 128, 256]
+
+
+def test_cutoff_sequence_workload_properties():
+    """The shape of the behaviour-sequence fields (2048 sequences, log-normal lengths, mean 200, cut
+    to 100 then to 50): truncation twice equals truncation once to the smaller length; kept
+    counts follow from the lengths alone."""
+    g = torch.Generator().manual_seed(5)
+    lens = torch.clamp(torch.exp(torch.randn(2048, generator=g) * 0.8 + 5.0).long(), 1, 1000)
+    off = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32).cuda()
+    vals = torch.arange(int(off[-1]), dtype=torch.int64).cuda()
+    for left in (False, True):
+        a = ops.fused_ragged_cutoff([vals] * 4, [off] * 4, [100] * 4, [left] * 4, [False] * 4)
+        b = ops.fused_ragged_cutoff(a[0], a[1], [50] * 4, [left] * 4, [False] * 4)
+        c = ops.fused_ragged_cutoff([vals] * 4, [off] * 4, [50] * 4, [left] * 4, [False] * 4)
+        for t in range(4):
+            assert torch.equal(b[0][t], c[0][t]) and torch.equal(b[1][t], c[1][t])
+            assert int(a[1][t][-1]) == int(torch.clamp(lens, max=100).sum())
+            first = vals[(off[1:].long() - 50).clamp(min=off[:-1].long())] if left else vals[off[:-1].long()]
+            assert torch.equal(c[0][t][c[1][t][:-1].long()], first)
+    assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("np_dtype,t_dtype", DTYPES)
+def test_ragged_to_dense_matches_oracle(rng, np_dtype, t_dtype):
+    for levels in (1, 2, 3):
+        offsets, n = [], 40
+        for _ in range(levels):
+            offsets.append(_ragged(rng, n, 5, np.int32 if levels != 2 else np.int64))
+            n = int(offsets[-1][-1])
+        values = _values(rng, n, np_dtype)
+        got = ops.ragged_to_dense(torch.from_numpy(values).cuda(), [torch.from_numpy(o).cuda() for o in offsets], 3)
+        np.testing.assert_array_equal(got.cpu().numpy(), oracle.ragged_to_dense(values, offsets, 3))
+    assert _lib.poll_device_errors() == 0
+
+
+def test_ragged_to_dense_reference_example_and_given_widths():
+    vals = torch.tensor([1, 2, 3, 4, 5, 6, 7, 8, 9, 9, 10, 11, 12]).cuda()
+    offs = [torch.tensor([0, 2, 2, 3, 6]).cuda(), torch.tensor([0, 2, 4, 6, 9, 11, 13]).cuda()]
+    got = ops.ragged_to_dense(vals, offs, 0)
+    assert got.tolist() == [[[1, 2, 0], [3, 4, 0], [0, 0, 0]], [[0, 0, 0], [0, 0, 0], [0, 0, 0]],
+                            [[5, 6, 0], [0, 0, 0], [0, 0, 0]], [[7, 8, 9], [9, 10, 0], [11, 12, 0]]]
+    wide = ops.ragged_to_dense(vals, offs, -1, widths=[4, 2])   # padded / cut to the caller's shape
+    assert wide.shape == (4, 4, 2) and wide[3].tolist() == [[7, 8], [9, 10], [11, 12], [-1, -1]]
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64, np.int32, np.int64])
+def test_dense_to_ragged_matches_oracle(rng, np_dtype):
+    for rows, cols in ((2, 5), (5000, 37), (3, 300), (0, 4), (7, 0)):
+        data = rng.integers(0, 3, (rows, cols)).astype(np_dtype)
+        if rows > 2:
+            data[2] = 0
+        for invalid in (0, 1):
+            v, o = ops.dense_to_ragged(torch.from_numpy(data).cuda(), True, invalid)
+            ev, eo = oracle.dense_to_ragged(data, invalid)
+            np.testing.assert_array_equal(v.cpu().numpy(), ev)
+            np.testing.assert_array_equal(o.cpu().numpy(), eo)
+            assert o.dtype == torch.int32
+    # tests/ops/dense_to_ragged_test.py:6-27,58-75
+    v, o = ops.dense_to_ragged(torch.tensor([[1.0, 0, 3, 0, 0], [6, 7, 8, 0, 0]]).cuda(), True, 0)
+    assert v.tolist() == [1, 0, 3, 6, 7, 8] and o.tolist() == [0, 3, 6]
+    d = torch.tensor([[1, 2, 3, 0, 0], [6, 7, 8, 0, 0]], dtype=torch.int32).cuda()
+    v, o = ops.dense_to_ragged(d, False, 0)
+    assert torch.equal(v, d.view(-1)) and o.tolist() == [0, 5, 10]
+    assert _lib.poll_device_errors() == 0
+
+
+# ------------------------------------------------------------------ feature-engine surface
+def test_sequence_truncate_op_and_engine_fusion():
+    from recis_amd.features import Feature, FeatureEngine, SelectField, SequenceTruncate
+    from recis_amd.ragged.tensor import RaggedTensor
+
+    # tests/feature_engine/op_test.py:66-93
+    data = RaggedTensor(torch.randn(512), [torch.tensor([0, 256, 512], dtype=torch.int32),
+                                           torch.arange(0, 513, dtype=torch.int32)],
+                        dense_shape=(2, 256, 1)).cuda()
+    with pytest.raises(AssertionError):
+        SequenceTruncate(seq_len=128, check_length=True)(data)
+    flat = RaggedTensor(torch.randn(512), [torch.tensor([0, 256, 512], dtype=torch.int32)]).cuda()
+    out = SequenceTruncate(seq_len=128, check_length=False, truncate=True, truncate_side="left")(flat)
+    assert out.offsets()[-1].tolist() == [0, 128, 256]
+    assert torch.equal(out.values(), torch.cat([flat.values()[128:256], flat.values()[384:512]]))
+    assert out.dense_shape[1] == 128
+
+    # tests/feature_engine/fused_op_test.py:81-150: several features through the engine (one fused
+    # launch per dtype and dimensionality) against each op on its own
+    feats, batch, single = [], {}, {}
+    for i in range(6):
+        dtype = torch.long if i % 2 == 0 else torch.float
+        op2 = SequenceTruncate(seq_len=2 + i % 3, check_length=False, truncate_side="left" if i < 3 else "right",
+                               n_dims=2, dtype=dtype)
+        op3 = SequenceTruncate(seq_len=1 + i % 3, check_length=False, truncate_side="left", n_dims=3, dtype=dtype)
+        x2 = RaggedTensor(torch.tensor([1, 2, 3, 4, 5, 6, 7, 8, 9, 10], dtype=dtype),
+                          torch.tensor([0, 4, 7, 10]).int()).cuda()
+        x3 = RaggedTensor(torch.tensor([1, 2, 3, 4, 5, 6, 7, 8], dtype=dtype),
+                          [torch.tensor([0, 2, 3]).int(), torch.tensor([0, 3, 5, 8]).int()]).cuda()
+        for tag, op, x in (("a", op2, x2), ("b", op3, x3)):
+            name = "%s%d" % (tag, i)
+            batch[name] = x
+            single[name] = op(x)
+            feats.append(Feature(name).add_op(SelectField(name)).add_op(
+                SequenceTruncate(**{k: v for k, v in op._get_config().items() if k != "dtype"}, dtype=dtype)))
+    outs = FeatureEngine(feats)(batch)
+    for name, exp in single.items():
+        got = outs[name]
+        assert torch.equal(got.values(), exp.values()), name
+        assert all(torch.equal(a, b) for a, b in zip(got.offsets(), exp.offsets())), name
+        assert got.dense_shape == exp.dense_shape
+    x3 = single["b2"]     # keep 3 inner rows of sequences with 2 and 1 rows: padded at the end
+    assert x3.offsets()[0].tolist() == [0, 3, 6] and x3.offsets()[1].tolist() == [0, 3, 5, 5, 8, 8, 8]
+
+
+def test_ragged_tensor_dense_round_trip():
+    from recis_amd.ragged.tensor import RaggedTensor
+
+    dense = torch.tensor([[1, 2, 0], [3, 4, 5], [6, 0, 0]]).cuda()
+    r = RaggedTensor.from_dense(dense)      # recis/ragged/tensor.py:277-294
+    assert r.values().tolist() == [1, 2, 3, 4, 5, 6] and r.offsets()[0].tolist() == [0, 2, 5, 6]
+    assert torch.equal(r.to_dense(), dense)
+    assert r.to_dense(default_value=-1).tolist() == [[1, 2, -1], [3, 4, 5], [6, -1, -1]]

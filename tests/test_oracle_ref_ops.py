@@ -310,3 +310,17 @@ def test_table_training_script_matches_hashtable_and_optimizers(kind, beta_dtype
     np.testing.assert_array_equal(np.concatenate(t.emb), r_w)
     np.testing.assert_array_equal(np.concatenate(t.s0), r_m)
     np.testing.assert_array_equal(np.concatenate(t.s1), r_v)
+
+
+def test_dense_to_ragged_matches_cpu_op():
+    # csrc/ops/dense_to_ragged.cc:6-53
+    rng = np.random.default_rng(30)
+    for dtype in (np.float32, np.int32, np.int64, np.float64):
+        data = rng.integers(0, 3, (200, 17)).astype(dtype)
+        data[5] = 0
+        for invalid in (0, 2):
+            rv, ro = ref_ops.run("dense_to_ragged", [data, np.asarray([invalid], dtype)])
+            v, o = oracle.dense_to_ragged(data, invalid)
+            np.testing.assert_array_equal(v, rv)
+            np.testing.assert_array_equal(o, ro)
+            assert ro.dtype == np.int32
