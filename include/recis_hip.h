@@ -549,6 +549,31 @@ int recis_dense_to_ragged_rows(const void* data, int dtype_kind, int64_t rows, i
                                const void* invalid_value, int32_t* out_offsets, int64_t* src,
                                int64_t* total_dev, void* stream);
 
+/*
+ * feature_cross_ragged_cuda (csrc/ops/feature_cross_ragged_kernel.cu:286-416; CPU twin
+ * feature_cross_ragged.cc:24-98): segment s of the result holds one entry for every pair
+ * (distinct id of x's row s, distinct id of y's row s): id = MurmurHash64A of the two 8-byte
+ * words with seed 0 (ragged_common.cuh:105-125), weight = product of the weights the two ids
+ * carry at their FIRST occurrence in their rows (NULL weights = 1). Entries are ordered by first
+ * occurrence, x outermost (the reference's order differs between its CPU and CUDA paths; its
+ * test compares rows as multisets). n_seg = min(rows of x, rows of y).
+ * recis_feature_cross_rows fills x_rank [nx] / y_rank [ny] (int32 scratch: rank of an element
+ * among the distinct ids of its row, -1 for a repeat), y_count [n_seg], out_offsets
+ * ([n_seg + 1], the type of the input offsets) and total_dev [1]; the caller reads the total
+ * back to size out_val / out_weight for recis_feature_cross_emit. Weights are float32, or
+ * float64 when weight_is_f64.
+ */
+int recis_feature_cross_rows(const int64_t* x_val, const void* x_off, int64_t nx,
+                             const int64_t* y_val, const void* y_off, int64_t ny, int off_is64,
+                             int64_t n_seg, int32_t* x_rank, int32_t* y_rank, int32_t* y_count,
+                             void* out_offsets, int64_t* total_dev, void* stream);
+int recis_feature_cross_emit(const int64_t* x_val, const void* x_off, const void* x_weight,
+                             int64_t nx, const int64_t* y_val, const void* y_off,
+                             const void* y_weight, int64_t ny, int off_is64, int weight_is_f64,
+                             int64_t n_seg, const int32_t* x_rank, const int32_t* y_rank,
+                             const int32_t* y_count, const void* out_offsets, int64_t total,
+                             int64_t* out_val, void* out_weight, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

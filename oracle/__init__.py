@@ -492,3 +492,49 @@ def dense_to_ragged(data, invalid_value):
         vals.append(row[:n])
         offs.append(offs[-1] + n)
     return (np.concatenate(vals) if vals else data.reshape(-1)[:0]), np.asarray(offs, np.int32)
+
+
+# ------------------------------------------------------------ feature cross
+
+
+def murmur_hash_64_words(words, seed=0):
+    """MurmurHash64A over 8-byte words (csrc/ops/ragged_common.cuh:105-125), as a Python int."""
+    mask = (1 << 64) - 1
+    m = 0xc6a4a7935bd1e995
+    h = (seed ^ (len(words) * 8 * m)) & mask
+    for k in words:
+        k = (int(k) & mask) * m & mask
+        k ^= k >> 47
+        k = k * m & mask
+        h = ((h ^ k) * m) & mask
+    h ^= h >> 47
+    h = h * m & mask
+    h ^= h >> 47
+    return h
+
+
+def feature_cross_ragged(x_val, x_off, x_w, y_val, y_off, y_w):
+    """Per segment: distinct ids of x crossed with distinct ids of y, each with the weight of its
+    first occurrence (csrc/ops/feature_cross_ragged.cc:7-20,60-92). Entries in first-occurrence
+    order, x outermost. Returns (ids int64, offsets, weights)."""
+    x_val, y_val, x_off, y_off = (np.asarray(a) for a in (x_val, y_val, x_off, y_off))
+    wdt = np.asarray(x_w if x_w is not None else y_w if y_w is not None else np.zeros(0, np.float32)).dtype
+    ids, ws, offs = [], [], [0]
+
+    def distinct(val, w, beg, end):
+        seen = {}
+        for i in range(beg, end):
+            if int(val[i]) not in seen:
+                seen[int(val[i])] = wdt.type(1) if w is None else w[i]
+        return seen
+
+    for s in range(min(len(x_off), len(y_off)) - 1):
+        ux = distinct(x_val, x_w, int(x_off[s]), int(x_off[s + 1]))
+        uy = distinct(y_val, y_w, int(y_off[s]), int(y_off[s + 1]))
+        for a, wa in ux.items():
+            for b, wb in uy.items():
+                h = murmur_hash_64_words([a, b])
+                ids.append(h - (1 << 64) if h >= 1 << 63 else h)
+                ws.append(wa * wb)
+        offs.append(len(ids))
+    return np.asarray(ids, np.int64), np.asarray(offs, x_off.dtype), np.asarray(ws, wdt)

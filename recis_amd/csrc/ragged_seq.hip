@@ -324,17 +324,115 @@ __global__ void __launch_bounds__(kBlock) dense_row_lengths_kernel(const T* data
 }
 
 // Sums of 2048-row blocks of lengths already stored in out_off (the input of the block scan).
-__global__ void __launch_bounds__(kBlock) length_block_sums_kernel(const int32_t* out_off, int64_t rows,
+__global__ void __launch_bounds__(kBlock) length_block_sums_kernel(const void* out_off, int is64, int64_t rows,
                                                                    int64_t* block_sums) {
   __shared__ int64_t lds[kBlock / kWave];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock;
   int64_t sum = 0;
   for (int i = 0; i < kItems; ++i) {
     const int64_t r = base + static_cast<int64_t>(i) * kBlock + threadIdx.x;
-    if (r < rows) sum += out_off[r];
+    if (r < rows) sum += load_index(out_off, is64, r);
   }
   const int64_t total = block_sum(sum, lds);
   if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+// ---------------------------------------------------------------- feature cross
+// feature_cross_ragged (csrc/ops/feature_cross_ragged.cc:24-98, feature_cross_ragged_kernel.cu:
+// 191-279): per segment, every distinct id of x paired with every distinct id of y; the pair's id is
+// MurmurHash64A of the two 8-byte words (seed 0, ragged_common.cuh:105-125), its weight the
+// product of the weights of the ids' first occurrences.
+
+// Pass 1: rank[i] = 1 when element i is the first occurrence of its id in its row, else 0
+// (a group of 2^g_log2 lanes per row; an element looks back over its row).
+__global__ void __launch_bounds__(kBlock) cross_first_kernel(const int64_t* val, const void* off, int is64,
+                                                             int64_t n_seg, int64_t n_val, int32_t* rank, int g_log2,
+                                                             int* err) {
+  const int g = 1 << g_log2;
+  const int sub = threadIdx.x & (g - 1);
+  const int64_t groups_per_grid = (static_cast<int64_t>(gridDim.x) * kBlock) >> g_log2;
+  for (int64_t s = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) >> g_log2; s < n_seg;
+       s += groups_per_grid) {
+    const int64_t beg = load_index(off, is64, s), end = load_index(off, is64, s + 1);
+    if (beg < 0 || end > n_val || end < beg) {
+      if (sub == 0) raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+      continue;
+    }
+    for (int64_t i = beg + sub; i < end; i += g) {
+      const int64_t v = val[i];
+      int32_t first = 1;
+      for (int64_t k = beg; k < i; ++k)
+        if (val[k] == v) {
+          first = 0;
+          break;
+        }
+      rank[i] = first;
+    }
+  }
+}
+
+// Pass 2: one thread per segment turns the flags into ranks (-1 for repeats), counts the distinct
+// ids of both sides and stores the segment's output length.
+__global__ void __launch_bounds__(kBlock) cross_rank_kernel(const void* x_off, const void* y_off, int is64,
+                                                            int64_t n_seg, int64_t nx, int64_t ny, int32_t* x_rank,
+                                                            int32_t* y_rank, int32_t* y_count, void* out_off) {
+  const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (s >= n_seg) return;
+  int64_t count[2];
+  for (int side = 0; side < 2; ++side) {
+    const void* off = side ? y_off : x_off;
+    int32_t* rank = side ? y_rank : x_rank;
+    const int64_t n = side ? ny : nx;
+    const int64_t beg = load_index(off, is64, s), end = load_index(off, is64, s + 1);
+    int32_t r = 0;
+    if (beg >= 0 && end <= n)
+      for (int64_t i = beg; i < end; ++i) rank[i] = rank[i] ? r++ : -1;
+    count[side] = r;
+  }
+  y_count[s] = static_cast<int32_t>(count[1]);
+  store_index(out_off, is64, s, count[0] * count[1]);
+}
+
+__device__ __forceinline__ uint64_t murmur_pair(uint64_t a, uint64_t b) {
+  const uint64_t m = 0xc6a4a7935bd1e995ULL;
+  uint64_t h = 0 ^ (16 * m);
+  a *= m; a ^= a >> 47; a *= m; h ^= a; h *= m;
+  b *= m; b ^= b >> 47; b *= m; h ^= b; h *= m;
+  h ^= h >> 47;
+  h *= m;
+  h ^= h >> 47;
+  return h;
+}
+
+// Pass 3: a lane group per segment walks the pairs of its rows; pairs of first occurrences land
+// at offset + rank_x * distinct_y + rank_y.
+template <typename W>
+__global__ void __launch_bounds__(kBlock) cross_emit_kernel(const int64_t* xv, const void* x_off, const W* xw,
+                                                            const int64_t* yv, const void* y_off, const W* yw,
+                                                            int is64, int64_t n_seg, int64_t nx, int64_t ny,
+                                                            const int32_t* x_rank, const int32_t* y_rank,
+                                                            const int32_t* y_count, const void* out_off,
+                                                            int64_t* out_val, W* out_w, int g_log2) {
+  const int g = 1 << g_log2;
+  const int sub = threadIdx.x & (g - 1);
+  const int64_t groups_per_grid = (static_cast<int64_t>(gridDim.x) * kBlock) >> g_log2;
+  for (int64_t s = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) >> g_log2; s < n_seg;
+       s += groups_per_grid) {
+    const int64_t xb = load_index(x_off, is64, s), xe = load_index(x_off, is64, s + 1);
+    const int64_t yb = load_index(y_off, is64, s), ye = load_index(y_off, is64, s + 1);
+    if (xb < 0 || xe > nx || xe < xb || yb < 0 || ye > ny || ye < yb) continue;
+    const int64_t ly = ye - yb, pairs = (xe - xb) * ly;
+    const int64_t base = load_index(out_off, is64, s);
+    const int64_t uy = y_count[s];
+    for (int64_t p = sub; p < pairs; p += g) {
+      const int64_t ix = xb + p / ly, iy = yb + p % ly;
+      const int32_t rx = x_rank[ix], ry = y_rank[iy];
+      if (rx < 0 || ry < 0) continue;
+      const int64_t at = base + rx * uy + ry;
+      out_val[at] = static_cast<int64_t>(murmur_pair(static_cast<uint64_t>(xv[ix]), static_cast<uint64_t>(yv[iy])));
+      out_w[at] = (xw ? xw[ix] : W(1)) * (yw ? yw[iy] : W(1));
+    }
+  }
 }
 
 }  // namespace
@@ -444,7 +542,7 @@ extern "C" int recis_dense_to_ragged_rows(const void* data, int dtype_kind, int6
       }
     }
     RECIS_LAUNCH_CHECK();
-    length_block_sums_kernel<<<dim3(static_cast<unsigned>(nb)), dim3(kBlock), 0, stream>>>(out_offsets, rows, sums);
+    length_block_sums_kernel<<<dim3(static_cast<unsigned>(nb)), dim3(kBlock), 0, stream>>>(out_offsets, 0, rows, sums);
     RECIS_LAUNCH_CHECK();
   }
   cutoff_scan_blocks_kernel<<<dim3(1), dim3(kBlock), 0, stream>>>(j, 0, sums, total_dev, 0);
@@ -579,5 +677,89 @@ extern "C" int recis_ragged_cutoff_copy(const void* const* values_ptrs, int elem
     }
     RECIS_LAUNCH_CHECK();
   }
+  return RECIS_OK;
+}
+
+static int group_log2(int64_t total, int64_t rows) {
+  int g = 0;
+  while (g < 6 && (int64_t(1) << g) * rows < total) ++g;
+  return g;
+}
+
+extern "C" int recis_feature_cross_rows(const int64_t* x_val, const void* x_off, int64_t nx, const int64_t* y_val,
+                                        const void* y_off, int64_t ny, int off_is64, int64_t n_seg,
+                                        int32_t* x_rank, int32_t* y_rank, int32_t* y_count, void* out_offsets,
+                                        int64_t* total_dev, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n_seg >= 0 && nx >= 0 && ny >= 0, "negative size");
+  RECIS_REQUIRE(out_offsets && total_dev, "NULL argument");
+  RECIS_REQUIRE(n_seg == 0 || (x_off && y_off && y_count), "NULL offsets pointer");
+  RECIS_REQUIRE((nx == 0 || (x_val && x_rank)) && (ny == 0 || (y_val && y_rank)), "NULL values pointer");
+  int* err = device_error_word(current_device());
+  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  CutJobs j;
+  j.out_off[0] = out_offsets;
+  j.out_rows[0] = n_seg;
+  j.sums_base[0] = 0;
+  const int64_t nb = (n_seg + kRowsPerBlock - 1) / kRowsPerBlock;
+  void* ws = nullptr;
+  int rc = get_workspace(stream, static_cast<size_t>(std::max<int64_t>(nb, 1)) * sizeof(int64_t), &ws);
+  if (rc != RECIS_OK) return rc;
+  int64_t* sums = static_cast<int64_t*>(ws);
+  if (n_seg > 0) {
+    for (int side = 0; side < 2; ++side) {
+      const int64_t n = side ? ny : nx;
+      if (n == 0) continue;
+      const int g = group_log2(n, n_seg);
+      const int64_t gx = std::min<int64_t>(((n_seg << g) + kBlock - 1) / kBlock, 1 << 20);
+      RECIS_TIME_KERNEL("cross_first_kernel", stream)
+      cross_first_kernel<<<dim3(static_cast<unsigned>(gx)), dim3(kBlock), 0, stream>>>(
+          side ? y_val : x_val, side ? y_off : x_off, off_is64, n_seg, n, side ? y_rank : x_rank, g, err);
+      RECIS_LAUNCH_CHECK();
+    }
+    const int64_t gr = (n_seg + kBlock - 1) / kBlock;
+    RECIS_REQUIRE(gr < (int64_t(1) << 31), "too many segments");
+    RECIS_TIME_KERNEL("cross_rank_kernel", stream)
+    cross_rank_kernel<<<dim3(static_cast<unsigned>(gr)), dim3(kBlock), 0, stream>>>(
+        x_off, y_off, off_is64, n_seg, nx, ny, x_rank, y_rank, y_count, out_offsets);
+    RECIS_LAUNCH_CHECK();
+    length_block_sums_kernel<<<dim3(static_cast<unsigned>(nb)), dim3(kBlock), 0, stream>>>(out_offsets, off_is64, n_seg,
+                                                                                          sums);
+    RECIS_LAUNCH_CHECK();
+  }
+  cutoff_scan_blocks_kernel<<<dim3(1), dim3(kBlock), 0, stream>>>(j, off_is64, sums, total_dev, 0);
+  RECIS_LAUNCH_CHECK();
+  if (nb > 0) {
+    cutoff_offsets_kernel<<<dim3(static_cast<unsigned>(nb), 1), dim3(kBlock), 0, stream>>>(j, off_is64, sums);
+    RECIS_LAUNCH_CHECK();
+  }
+  return RECIS_OK;
+}
+
+extern "C" int recis_feature_cross_emit(const int64_t* x_val, const void* x_off, const void* x_weight, int64_t nx,
+                                        const int64_t* y_val, const void* y_off, const void* y_weight, int64_t ny,
+                                        int off_is64, int weight_is_f64, int64_t n_seg, const int32_t* x_rank,
+                                        const int32_t* y_rank, const int32_t* y_count, const void* out_offsets,
+                                        int64_t total, int64_t* out_val, void* out_weight, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n_seg >= 0 && nx >= 0 && ny >= 0 && total >= 0, "negative size");
+  if (total == 0 || n_seg == 0) return RECIS_OK;
+  RECIS_REQUIRE(x_val && x_off && y_val && y_off && x_rank && y_rank && y_count && out_offsets && out_val && out_weight,
+                "NULL argument");
+  // pairs examined per segment on average decide the lanes per segment
+  const int g = group_log2(std::max<int64_t>(total, (nx / std::max<int64_t>(n_seg, 1)) * ny), n_seg);
+  const int64_t gx = std::min<int64_t>(((n_seg << g) + kBlock - 1) / kBlock, 1 << 20);
+  const dim3 grid(static_cast<unsigned>(gx));
+  RECIS_TIME_KERNEL("cross_emit_kernel", stream) {
+    if (weight_is_f64)
+      cross_emit_kernel<double><<<grid, dim3(kBlock), 0, stream>>>(
+          x_val, x_off, static_cast<const double*>(x_weight), y_val, y_off, static_cast<const double*>(y_weight),
+          off_is64, n_seg, nx, ny, x_rank, y_rank, y_count, out_offsets, out_val, static_cast<double*>(out_weight), g);
+    else
+      cross_emit_kernel<float><<<grid, dim3(kBlock), 0, stream>>>(
+          x_val, x_off, static_cast<const float*>(x_weight), y_val, y_off, static_cast<const float*>(y_weight),
+          off_is64, n_seg, nx, ny, x_rank, y_rank, y_count, out_offsets, out_val, static_cast<float*>(out_weight), g);
+  }
+  RECIS_LAUNCH_CHECK();
   return RECIS_OK;
 }

@@ -1,6 +1,6 @@
 """Feature-engine ops on the hot path: the mirror of ``recis.features.op`` for
 ``SelectField``, ``Mod``, ``Bucketize``, ``Hash``, ``IDMultiHash`` and ``SequenceTruncate``
-(recis/features/op.py:129-686). ``FeatureCross`` is not part of this build.
+and ``FeatureCross`` (recis/features/op.py:129-686).
 
 Every op works on a ``RaggedTensor`` (its values) or a plain tensor; the engine
 batches same-typed ops of one step into a single fused HIP launch.
@@ -138,6 +138,20 @@ class IDMultiHash(_OP):
 
     def _get_config(self):
         return {"num_buckets": self.num_buckets, "prefix": self.prefix}
+
+
+class FeatureCross(_OP):
+    """Cross of two id features, segment by segment (recis/features/op.py:357-405)."""
+
+    def forward(self, data: List[RaggedTensor]):
+        x, y = data
+        assert isinstance(x, RaggedTensor) and isinstance(y, RaggedTensor)
+        val, offsets, weight = ops.feature_cross_ragged(x.values(), x.offsets()[-1], x.weight(), y.values(),
+                                                        y.offsets()[-1], y.weight())
+        return RaggedTensor(val, offsets, weight, x.dense_shape)
+
+    def _get_config(self):
+        return {}
 
 
 class SequenceTruncate(_OP):

@@ -54,3 +54,8 @@ def fused_ragged_cutoff_3D(values: List[torch.Tensor], offsets: List[List[torch.
     vals, outer, inner = _fused_ragged_cutoff_3D(values, [o[0] for o in offsets], [o[1] for o in offsets],
                                                  keep_lengths, drop_sides, pad_sides)
     return vals, [[outer[i], inner[i]] for i in range(len(outer))]
+
+
+def feature_cross_ragged(x_value, x_offsets, y_value, y_offsets, x_weight=None, y_weight=None):
+    """ragged_ops.py:445-540: (values, offsets, weights) of the per-segment cross of x and y."""
+    return ops.feature_cross_ragged(x_value, x_offsets, x_weight, y_value, y_offsets, y_weight)

@@ -1016,3 +1016,42 @@ def dense_to_ragged(data, check_invalid=True, invalid_value=0):
                                              _host_i64([rows]), _host_ptrs([src]), _host_i64([n]),
                                              _host_ptrs([values]), i64(1), sp))
     return values, offsets
+
+
+def feature_cross_ragged(x_value, x_offsets, x_weight, y_value, y_offsets, y_weight):
+    """``torch.ops.recis.feature_cross_ragged`` (feature_cross_ragged.cc:24-98): per segment the
+    cross of the distinct ids of x and y. Returns (values, offsets, weights); an empty weight
+    tensor (or None) means all ones."""
+    require_cuda(x_value, x_offsets, y_value, y_offsets)
+    if x_value.dtype != torch.int64 or y_value.dtype != torch.int64:
+        raise RuntimeError("feature_cross_ragged: ids for x and y must be torch.int64")
+    is64 = _index_kind(x_offsets, "x_offsets")
+    if _index_kind(y_offsets, "y_offsets") != is64:
+        raise RuntimeError("feature_cross_ragged: each offset should be torch.int32 or torch.int64")
+    xv, yv, xo, yo = _contig(x_value), _contig(y_value), _contig(x_offsets), _contig(y_offsets)
+    dev = xv.device
+
+    def weight(w):
+        return None if w is None or w.numel() == 0 else _contig(w)
+
+    xw, yw = weight(x_weight), weight(y_weight)
+    wdt = (xw if xw is not None else yw if yw is not None else torch.empty(0)).dtype
+    if wdt not in (torch.float32, torch.float64) or any(w is not None and w.dtype != wdt for w in (xw, yw)):
+        raise TypeError("feature_cross_ragged: weights must share float32 or float64")
+    n_seg = min(xo.numel(), yo.numel()) - 1
+    nx, ny = xv.numel(), yv.numel()
+    x_rank = torch.empty(max(nx, 1), dtype=torch.int32, device=dev)
+    y_rank = torch.empty(max(ny, 1), dtype=torch.int32, device=dev)
+    y_count = torch.empty(max(n_seg, 1), dtype=torch.int32, device=dev)
+    out_off = torch.empty(n_seg + 1, dtype=xo.dtype, device=dev)
+    total = torch.empty(1, dtype=torch.int64, device=dev)
+    sp = stream_ptr(dev)
+    check(lib().recis_feature_cross_rows(ptr(xv), ptr(xo), i64(nx), ptr(yv), ptr(yo), i64(ny), is64, i64(n_seg),
+                                         ptr(x_rank), ptr(y_rank), ptr(y_count), ptr(out_off), ptr(total), sp))
+    n = int(total.item())
+    out_val = torch.empty(n, dtype=torch.int64, device=dev)
+    out_w = torch.empty(n, dtype=wdt, device=dev)
+    check(lib().recis_feature_cross_emit(ptr(xv), ptr(xo), ptr(xw), i64(nx), ptr(yv), ptr(yo), ptr(yw), i64(ny), is64,
+                                         int(wdt == torch.float64), i64(n_seg), ptr(x_rank), ptr(y_rank),
+                                         ptr(y_count), ptr(out_off), i64(n), ptr(out_val), ptr(out_w), sp))
+    return out_val, out_off, out_w

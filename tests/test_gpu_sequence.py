@@ -201,3 +201,34 @@ def test_ragged_tensor_dense_round_trip():
     assert r.values().tolist() == [1, 2, 3, 4, 5, 6] and r.offsets()[0].tolist() == [0, 2, 5, 6]
     assert torch.equal(r.to_dense(), dense)
     assert r.to_dense(default_value=-1).tolist() == [[1, 2, -1], [3, 4, 5], [6, -1, -1]]
+
+
+# ------------------------------------------------------------------ feature cross
+@pytest.mark.parametrize("off_dtype", [np.int32, np.int64])
+@pytest.mark.parametrize("w_dtype", [np.float32, np.float64, None])
+def test_feature_cross_matches_oracle(rng, off_dtype, w_dtype):
+    for rows, max_len, key_range in ((2000, 10, 6), (300, 70, 40), (5000, 1, 1000), (50, 0, 5)):
+        xo, yo = _ragged(rng, rows, max_len, off_dtype), _ragged(rng, rows + 3, max_len, off_dtype)
+        xv, yv = rng.integers(-key_range, key_range, int(xo[-1])), rng.integers(-key_range, key_range, int(yo[-1]))
+        xw = None if w_dtype is None else rng.random(int(xo[-1])).astype(w_dtype)
+        yw = None if w_dtype is None else rng.random(int(yo[-1])).astype(w_dtype)
+        dev = lambda a: None if a is None else torch.from_numpy(a).cuda()
+        v, o, w = ops.feature_cross_ragged(dev(xv), dev(xo), dev(xw), dev(yv), dev(yo), dev(yw))
+        ev, eo, ew = oracle.feature_cross_ragged(xv, xo, xw, yv, yo, yw)
+        np.testing.assert_array_equal(o.cpu().numpy(), eo)
+        np.testing.assert_array_equal(v.cpu().numpy(), ev)
+        np.testing.assert_array_equal(w.cpu().numpy(), ew)     # one product of two stored weights: exact
+        assert o.dtype == torch.from_numpy(xo).dtype
+    assert _lib.poll_device_errors() == 0
+
+
+def test_feature_cross_op_kat():
+    # tests/feature_engine/op_test.py:39-63
+    from recis_amd.features import FeatureCross
+    from recis_amd.ragged.tensor import RaggedTensor
+
+    x = RaggedTensor(torch.tensor([1001, 1002, 1003]), torch.tensor([0, 1, 2, 3]).int(), torch.ones(3)).cuda()
+    y = RaggedTensor(torch.tensor([1, 2, 3]), torch.tensor([0, 1, 2, 3]).int(), torch.ones(3)).cuda()
+    out = FeatureCross()([x, y])
+    assert out.values().tolist() == [-7808879811642834040, -4967483181219983279, 1752425377096056168]
+    assert out.offsets()[-1].tolist() == [0, 1, 2, 3] and out.weight().tolist() == [1.0, 1.0, 1.0]

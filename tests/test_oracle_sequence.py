@@ -111,3 +111,34 @@ def test_dense_to_ragged_kats():
     assert v.tolist() == [1, 2, 3, 6, 7, 8] and o.tolist() == [0, 3, 6]
     v, o = oracle.dense_to_ragged(np.zeros((3, 4), np.int32), 0)
     assert v.size == 0 and o.tolist() == [0, 0, 0, 0]
+
+
+def test_feature_cross_kat():
+    # tests/feature_engine/op_test.py:39-63
+    ids, offs, w = oracle.feature_cross_ragged(np.array([1001, 1002, 1003]), np.array([0, 1, 2, 3], np.int32),
+                                               np.ones(3, np.float32), np.array([1, 2, 3]),
+                                               np.array([0, 1, 2, 3], np.int32), np.ones(3, np.float32))
+    assert ids.tolist() == [-7808879811642834040, -4967483181219983279, 1752425377096056168]
+    assert offs.tolist() == [0, 1, 2, 3] and w.tolist() == [1, 1, 1]
+
+
+def test_murmur_words_is_murmur64a_over_the_bytes(rng):
+    """The word form used by the cross equals the reference's byte-string MurmurHash64A (the one
+    compiled from the reference into oracle/_ref and the one the string features use)."""
+    for _ in range(50):
+        words = rng.integers(-(1 << 63), (1 << 63) - 1, int(rng.integers(1, 5)))
+        raw = np.frombuffer(words.astype("<i8").tobytes(), np.uint8)
+        got = oracle.hash_strings(raw, np.array([0, raw.size]), "murmur")[0]
+        exp = oracle.murmur_hash_64_words(words.tolist())
+        assert int(got) == (exp - (1 << 64) if exp >= 1 << 63 else exp)
+
+
+def test_feature_cross_dedups_and_takes_first_weight():
+    ids, offs, w = oracle.feature_cross_ragged(np.array([5, 7, 5, 9]), np.array([0, 3, 4]),
+                                               np.array([2.0, 3.0, 100.0, 1.0]), np.array([1, 1, 4, 8]),
+                                               np.array([0, 2, 4]), np.array([0.5, 9.0, 1.0, 2.0]))
+    assert offs.tolist() == [0, 2, 4]                 # {5,7} x {1} and {9} x {4,8}
+    assert w.tolist() == [1.0, 1.5, 1.0, 2.0]
+    h = oracle.murmur_hash_64_words
+    signed = lambda v: v - (1 << 64) if v >= 1 << 63 else v
+    assert ids.tolist() == [signed(h([5, 1])), signed(h([7, 1])), signed(h([9, 4])), signed(h([9, 8]))]
