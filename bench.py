@@ -3,7 +3,7 @@
     python bench.py --gpus 1 --steps K --warmup W [--workload c4|c2] [--no-cpu-baseline]
 
 Prints ONE JSON line. A "step" is one pass of the hot path over one batch of synthetic
-input that is already resident in HBM. The default workload is BASELINE config 4
+input that is already resident in HBM. The default workload is benchmark config 4
 (click-through-style merged table): feature ops (bucketize + mod) -> key tagging ->
 dedup -> find-or-insert -> row gather -> sum pooling -> backward scatter -> fused sparse
 Adam; `value` = id occurrences per second. Config 2 (standalone segment reduce, fwd + bwd
@@ -532,7 +532,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU that owns the whole table; --gpus %d is not supported "
-              "(the sharded exchange is described in DESIGN.md, not built)" % args.gpus, file=sys.stderr)
+              "(every GPU box of this build has one GPU; a sharded table would exchange ids and rows per step)" % args.gpus, file=sys.stderr)
         sys.exit(2)
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)

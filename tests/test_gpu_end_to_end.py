@@ -1,5 +1,5 @@
 """End-to-end parity of the GPU table + pooling + optimizer with the restated
-reference CPU path (oracle.cpu_path) on BASELINE config 1, and behaviour tests of
+reference CPU path (oracle.cpu_path) on benchmark config 1, and behaviour tests of
 the host-side modules that read like the reference's own module tests.
 
 Bars: key -> row assignment bit-exact when new keys are presented in the reference's
@@ -67,7 +67,7 @@ def _close(a, b, msg=""):
 
 @pytest.mark.parametrize("steps", [100])
 def test_config1_hundred_steps_bit_exact_rows(steps):
-    """BASELINE config 1: Zipf(1.05) ids over 1e6 keys, batch 4096, lengths 1..20, dim 16 fp32,
+    """benchmark config 1: Zipf(1.05) ids over 1e6 keys, batch 4096, lengths 1..20, dim 16 fp32,
     rows N(0, 0.01), sum pooling, backward, sparse Adagrad (lr 0.01, eps 1e-8), 100 steps, seed 0."""
     bs, dim = 1024, 16
     cpu = cpu_path.CpuTable(dim, bs, lambda b: workloads.seeded_block(0, b, bs, dim), "adagrad", 0.01, 1e-8)

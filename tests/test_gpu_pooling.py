@@ -233,7 +233,7 @@ def test_argument_errors():
 
 @pytest.mark.parametrize("mode", ["sum", "mean"])
 def test_config2_shape_properties(mode):
-    """BASELINE config 2 at full size: linearity and a sum-of-sums checksum.
+    """benchmark config 2 at full size: linearity and a sum-of-sums checksum.
 
     32 x 16384 segments, Poisson(30) lengths clipped to [1, 200], D = 64 fp32,
     rows materialised per occurrence, int32 offsets."""

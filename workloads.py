@@ -1,4 +1,4 @@
-"""Seeded synthetic inputs for the BASELINE configurations.
+"""Seeded synthetic inputs for the benchmark configurations.
 
 Used by ``bench.py`` and the tests; every generator is deterministic in its
 seed (numpy ``PCG64``) and returns torch tensors on the requested device.
@@ -31,7 +31,7 @@ def splitmix64(x):
 
 
 def config2(device="cuda", seed=1, features=32, batch=16384, dim=64, mean_len=30, max_len=200):
-    """Standalone ragged segment_reduce on pre-materialised rows (BASELINE config 2)."""
+    """Standalone ragged segment_reduce on pre-materialised rows (benchmark config 2)."""
     rng = _rng(seed)
     S = features * batch
     lens = np.clip(rng.poisson(mean_len, size=S), 1, max_len).astype(np.int64)
@@ -53,7 +53,7 @@ def config2(device="cuda", seed=1, features=32, batch=16384, dim=64, mean_len=30
 
 
 def config1_step(step, seed=0, batch=4096, num_keys=1_000_000, alpha=1.05, max_len=20, dim=16, _cache={}):
-    """One batch of BASELINE config 1 as numpy arrays: (ids int64 [N], offsets int64 [batch+1],
+    """One batch of benchmark config 1 as numpy arrays: (ids int64 [N], offsets int64 [batch+1],
     upstream gradient float32 [batch, dim]). Deterministic in (seed, step)."""
     key = (num_keys, alpha)
     if key not in _cache:
@@ -76,7 +76,7 @@ def seeded_block(seed, block_index, block_size, dim, std=0.01):
 
 
 def config4(device="cuda", seed=4, batch=65536, n_sparse=26, n_dense=13, n_boundaries=64, mod=1_000_000):
-    """Click-through-style merged table (BASELINE config 4): 26 int64 id fields with log-uniform
+    """Click-through-style merged table (benchmark config 4): 26 int64 id fields with log-uniform
     cardinalities in 10..1e7, 13 lognormal(0, 2) dense fields bucketized against 64 sorted
     boundaries and taken mod 1e6; one id per field per sample."""
     rng = _rng(seed)
@@ -128,7 +128,7 @@ def zipf_ranks_torch(cdf, n, generator):
 
 def config3_batches(n_batches, resident, ids_per_step=2_000_000, alpha=1.1, new_frac=0.1, seed=3,
                     device="cuda"):
-    """BASELINE config 3 lookups: per step `ids_per_step` keys, Zipf(alpha) over the `resident`
+    """benchmark config 3 lookups: per step `ids_per_step` keys, Zipf(alpha) over the `resident`
     pre-populated keys (key of rank r = splitmix64(r)), a fraction `new_frac` of the positions
     replaced by keys never seen before (ranks beyond the resident set, distinct per step)."""
     g = torch.Generator(device=device).manual_seed(seed)
@@ -146,7 +146,7 @@ def config3_batches(n_batches, resident, ids_per_step=2_000_000, alpha=1.1, new_
 
 def config5(device="cuda", seed=5, batch=2048, n_fields=4, num_keys=50_000_000, alpha=1.2, mean_len=200,
             max_len=1000):
-    """Long behaviour sequences (BASELINE config 5): per field `batch` sequences with lognormal
+    """Long behaviour sequences (benchmark config 5): per field `batch` sequences with lognormal
     lengths (sigma 1, mean `mean_len`, clipped to [1, max_len]) of Zipf(alpha) ids over `num_keys`
     keys. Returns per-field values / int32 offsets and the per-field padded length (= longest
     sequence of that field)."""
