@@ -189,9 +189,11 @@ class Config4:
         return self.table.settle_lookup(index_buf, self.U)
 
     def pool_fwd(self, index, inv):
-        # pooling reads the rows out of the table (no [U, D] copy), as EmbeddingEngine does
+        # pooling reads the rows out of the table (no [U, D] copy); every field holds one id per
+        # sample, so, as EmbeddingEngine does for dense [B] id tensors, each unique row is read
+        # once and written to its occurrences
         chunks, chunk_rows = self.table.emb_blocks()
-        return self.ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, None, inv, self.offsets, "sum")
+        return self.ops.plan_expand_rows(self.plan, self.N, blocks=chunks, block_size=chunk_rows, row_index=index)
 
     def pool_bwd(self, inv):
         return self.ops.segment_reduce_backward_plan(self.grad_out, None, self.offsets, self.plan, "sum")
@@ -217,7 +219,7 @@ class Config4:
             "feature_ops": feat,
             "dedup": N * (8 + 4) + U * 8,
             "lookup": U * (16 + 8),
-            "pool_fwd": U * (8 + D * 4) + N * 4 + (S + 1) * 4 + S * D * 4,
+            "pool_fwd": U * (8 + D * 4) + N * 4 + (U + 1) * 4 + S * D * 4,
             "pool_bwd": S * D * 4 + N * 4 + (S + 1) * 4 + U * D * 4,
             "adam": U * 8 + U * D * 4 * (1 + 6),
         }
@@ -233,7 +235,7 @@ class Config4:
             # ids, word, result in; inverse, list, pos out; unique ids in, id + row_start out
             "plan_emit_kernel": 8 * N + 4 * N + 8 * U + 12 * N + 16 * U + 12 * U + 4 * (N + 1 - U),
             "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,          # ids, one table slot, index + slot pos
-            "seg_pool_fwd_kernel": U * (8 + D * 4) + 4 * N + 4 * (S + 1) + S * D * 4,
+            "csr_expand_kernel": U * (8 + D * 4) + 4 * N + 4 * (U + 1) + S * D * 4,
             "csr_rows_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,
             "adamw_rows_kernel": U * (8 + D * 4 * 7),
         }
@@ -321,11 +323,10 @@ class Config3:
         self.U = plan.U
         index = self.table.settle_lookup(index_buf, self.U)
         chunks, chunk_rows = self.table.emb_blocks()
-        rows = o.block_gather(index, chunks, chunk_rows, -1, False)
         self.table.update_slot("step_filter", index, self.step_t)
-        # one row per lookup, expanded from the [U, D] copy: with a 25 GB table, pooling out of the
-        # table (segment_reduce_forward_blocks) gains nothing, the copy keeps the 2e6 reads local
-        out = o.gather(plan.inverse, rows)
+        # one row per lookup: every unique row is read once out of the table and written to its
+        # occurrences (no [U, D] copy, no second pass over it)
+        out = o.plan_expand_rows(plan, self.N, blocks=chunks, block_size=chunk_rows, row_index=index)
         g = o.segment_reduce_backward_plan(self.grad_out, None, self.span, plan, "tile")
         self.table.accept_grad(index, g, unique=True)
         self.opt.step()
@@ -470,10 +471,10 @@ class Config5:
 # scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC_C4 = {
-    "adamw_rows_kernel": 400839616, "csr_rows_kernel": 395399229, "seg_pool_fwd_kernel": 381144772,
-    "plan_emit_kernel": 149236208, "find_or_claim_kernel": 114433209, "plan_bucket_kernel": 89179726,
-    "plan_scatter_kernel": 77185311, "plan_tile_kernel": 58194552, "ids_encode_kernel": 40936056,
-    "plan_colscan_kernel": 16425662,
+    "adamw_rows_kernel": 400839793, "csr_rows_kernel": 395465738, "csr_expand_kernel": 246127259,
+    "plan_emit_kernel": 149596294, "find_or_claim_kernel": 114443009, "plan_bucket_kernel": 89183328,
+    "plan_scatter_kernel": 77259166, "plan_tile_kernel": 58178389, "ids_encode_kernel": 40936481,
+    "plan_colscan_kernel": 16429764,
 }
 
 

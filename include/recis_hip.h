@@ -442,6 +442,24 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
                             const void* cover_offsets, int cover_is64, int64_t cover_S,
                             void* stream);
 
+/*
+ * The transpose of recis_csr_gather_reduce (no reference counterpart; it produces what
+ * segment_reduce_forward gives for one-id segments and for the TILE mode,
+ * embedding_segment_reduce_kernel.cu:23-75): out[dst[k], :] = weight[dst[k]] * row(u) for every
+ * list entry k in [row_start[u], row_start[u+1]) of every unique id u < U. Every unique row is
+ * read once and stored to all its occurrences (hot rows through the plan's work items, like the
+ * gather-reduce). Rows come from a dense [U, D] array (rows) or, when emb_blocks_dev != NULL,
+ * straight from a block list: row u is row row_index[u] (negative = zeros) of blocks of
+ * block_rows rows. weight ([n_out], per OUTPUT row) may be NULL. Output rows no list entry
+ * names are not written. dst outside [0, n_out) raises RECIS_DEVERR_INDEX_RANGE.
+ */
+int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks,
+                          int64_t block_rows, const int64_t* row_index, int rows_dtype,
+                          const void* weight, int weight_dtype, const int32_t* row_start,
+                          const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
+                          const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
+                          int64_t n_out, int64_t D, void* stream);
+
 /* ------------------------------------------------------------------------- *
  * Feature-engine scalar ops (lists as HOST arrays of device pointers)
  * ------------------------------------------------------------------------- */

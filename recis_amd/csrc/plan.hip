@@ -846,6 +846,145 @@ csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a) {
   }
 }
 
+// ------------------------------------------------------------------ expand (transpose of the gather-reduce)
+// out[dst[k], :] = w[dst[k]] * row(u) for every list entry k of every unique id u: the forward
+// of pooling when every segment holds exactly one id, and of the unpooled (tile) output. Each
+// unique row is read ONCE and stored to all its occurrences; stores do not wait for anything,
+// where the occurrence-major kernels chase index -> row index -> row for every output row.
+struct ExpArgs {
+  const int32_t* row_start;  // [U + 1]
+  const int32_t* dst;        // [n] output row per list entry
+  const void* weight;        // [n_out] per output row, or NULL
+  int wdt;
+  int64_t U, n_out;
+  int D;
+  int lpr_log2;
+  int* err;
+  const int64_t* row_index;  // rows in a block list: unique row u is row row_index[u] (negative = zeros)
+  const void* const* blocks;
+  int64_t block_rows, n_blocks;
+  int32_t hot_len;
+  const int32_t* hot_items;
+  const int64_t* counts;
+  int64_t hot_cap;
+  int64_t cold_blocks;
+};
+
+template <typename TIn, typename TOut, int VEC, bool BLK>
+__global__ void __launch_bounds__(kBlock)
+csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs a) {
+  const int D = a.D;
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
+  const int g = lane >> a.lpr_log2;        // this lane's group in its wave
+
+  auto load_row = [&](int64_t u, int c0, float (&v)[VEC]) {
+    const TIn* src = nullptr;
+    if constexpr (BLK) {
+      const int64_t ri = a.row_index[u];
+      if (ri >= 0) {
+        int64_t b = 0, r = ri;
+        if (a.n_blocks > 1) {
+          b = ri / a.block_rows;
+          r = ri - b * a.block_rows;
+        }
+        if (b >= a.n_blocks || r >= a.block_rows)
+          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        else
+          src = static_cast<const TIn*>(a.blocks[b]) + r * D;
+      }
+    } else {
+      src = rows + u * D;
+    }
+    if (src) {
+      load_pack<TIn, VEC>(src + c0, v);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+    }
+  };
+  auto store_to = [&](int64_t d, int c0, const float (&v)[VEC]) {
+    if (static_cast<uint64_t>(d) >= static_cast<uint64_t>(a.n_out)) {
+      raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      return;
+    }
+    float o[VEC];
+    const float w = a.weight ? load_coef(a.weight, a.wdt, d) : 1.0f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) o[j] = fmaf(v[j], w, 0.f);  // the pooled kernels' rounding
+    store_pack_stream<TOut, VEC>(out + d * D + c0, o);
+  };
+  // stores to the list entries first, first + step, ... < last; the destinations of four entries
+  // are fetched together so that their latencies overlap (more would cost resident waves)
+  auto store_list = [&](int32_t first, int32_t last, int32_t step, int c0, const float (&v)[VEC]) {
+    for (int32_t k = first; k < last; k += 4 * step) {
+      int32_t d[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = k + i * step < last ? a.dst[k + i * step] : -1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (k + i * step < last) store_to(d[i], c0, v);
+    }
+  };
+
+  const int64_t hot_blocks = static_cast<int64_t>(gridDim.x) - a.cold_blocks;
+  if (static_cast<int64_t>(blockIdx.x) < hot_blocks) {
+    // ---- hot work items: a workgroup per (row, chunk); all its lane groups hold the row
+    int64_t n_items = a.counts[1];
+    if (n_items > a.hot_cap) n_items = a.hot_cap;
+    const int groups_per_block = kBlock >> a.lpr_log2;
+    const int gb = threadIdx.x >> a.lpr_log2;
+    for (int64_t item = blockIdx.x; item < n_items; item += hot_blocks) {
+      const int32_t u = a.hot_items[2 * item];
+      const int32_t chunk = a.hot_items[2 * item + 1];
+      const int32_t start = a.row_start[u] + chunk * kHotChunk;
+      const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
+      for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+        float v[VEC];
+        load_row(u, c0, v);
+        store_list(start + gb, end, groups_per_block, c0, v);
+      }
+    }
+    return;
+  }
+
+  // ---- cold rows
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
+  const bool valid = u < a.U;
+  const int32_t start = valid ? a.row_start[u] : 0;
+  int32_t end = valid ? a.row_start[u + 1] : 0;
+  if (end - start > a.hot_len) end = start;  // written by the work items
+  const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;
+  if (valid && !is_long && end > start) {
+    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+      float v[VEC];
+      load_row(u, c0, v);
+      store_list(start, end, 1, c0, v);
+    }
+  }
+  // long rows of this wave, one after the other: the owner's row reaches every group by shuffles
+  uint64_t todo = __ballot(is_long);
+  while (todo) {
+    const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;
+    todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);
+    const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
+    const int64_t row = u - g + (owner >> a.lpr_log2);  // rows of a wave are consecutive
+    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+      const int c0 = cbase + cl * VEC;
+      const bool col_ok = c0 < D;
+      float mine[VEC], v[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) mine[j] = 0.f;
+      if (lane >> a.lpr_log2 == owner >> a.lpr_log2 && col_ok) load_row(row, c0, mine);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = __shfl(mine[j], owner + cl, kWave);
+      if (col_ok) store_list(r_start + g, r_end, groups, c0, v);
+    }
+  }
+}
+
 // src / coef of every list entry for pooled segments: occurrence i of segment s gets
 // src = s and coef = w_i (divided by the segment length for mean).
 __global__ void __launch_bounds__(kBlock)
@@ -1168,6 +1307,77 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F32) return with_types(f16_t{}, float{});
   if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_BF16) return with_types(bf16_t{}, bf16_t{});
   if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F16) return with_types(f16_t{}, f16_t{});
+  return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
+}
+
+int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows,
+                          const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
+                          const int32_t* row_start, const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
+                          const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t n_out, int64_t D,
+                          void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(U >= 0 && n_out >= 0, "negative size");
+  RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
+  if (U == 0 || n_out == 0) return RECIS_OK;
+  const bool blk = emb_blocks_dev != nullptr;
+  RECIS_REQUIRE(row_start && dst && out && counts_dev, "NULL argument");
+  RECIS_REQUIRE(blk ? (row_index != nullptr && n_blocks >= 1 && block_rows >= 1) : rows != nullptr,
+                "rows: a dense array or a block list with row_index");
+  RECIS_REQUIRE(hot_cap == 0 || hot_items, "hot_items must not be NULL");
+  const int in_sz = dtype_size(rows_dtype), out_sz = dtype_size(out_dtype);
+  RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
+  RECIS_REQUIRE(weight == nullptr || dtype_size(weight_dtype), "invalid weight dtype");
+  // block bases are allocator-aligned; a dense array brings its own alignment
+  const int vb_in = pick_vec_bytes(D * in_sz, blk ? 0 : reinterpret_cast<uintptr_t>(rows));
+  const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(out));
+  const int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
+  ExpArgs a;
+  a.row_start = row_start;
+  a.dst = dst;
+  a.weight = weight;
+  a.wdt = weight_dtype;
+  a.U = U;
+  a.n_out = n_out;
+  a.D = static_cast<int>(D);
+  a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
+  a.err = device_error_word(current_device());
+  RECIS_REQUIRE(a.err != nullptr, "could not allocate the device error word");
+  a.row_index = row_index;
+  a.blocks = emb_blocks_dev;
+  a.block_rows = block_rows;
+  a.n_blocks = n_blocks;
+  a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
+  a.hot_items = hot_items;
+  a.counts = counts_dev;
+  a.hot_cap = hot_cap;
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
+  const int64_t hot_blocks = hot_cap > 0 ? std::min<int64_t>(hot_cap, 4096) : 0;
+  const dim3 grid(static_cast<unsigned>(a.cold_blocks + hot_blocks));
+  auto with_types = [&](auto tin, auto tout) {
+    using TIn = decltype(tin);
+    using TOut = decltype(tout);
+    return dispatch_vec(vec, [&](auto vtag) {
+      constexpr int VEC = decltype(vtag)::value;
+      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 16) {
+        return fail(RECIS_ERR_ARG, "internal: vector too wide");
+      } else {
+        RECIS_TIME_KERNEL("csr_expand_kernel", stream)
+        if (blk)
+          csr_expand_kernel<TIn, TOut, VEC, true><<<grid, dim3(kBlock), 0, stream>>>(nullptr, static_cast<TOut*>(out), a);
+        else
+          csr_expand_kernel<TIn, TOut, VEC, false><<<grid, dim3(kBlock), 0, stream>>>(static_cast<const TIn*>(rows),
+                                                                                    static_cast<TOut*>(out), a);
+        RECIS_LAUNCH_CHECK();
+        return RECIS_OK;
+      }
+    });
+  };
+  if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F32) return with_types(float{}, float{});
+  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_BF16) return with_types(bf16_t{}, bf16_t{});
+  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F16) return with_types(f16_t{}, f16_t{});
+  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_F32) return with_types(bf16_t{}, float{});
+  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F32) return with_types(f16_t{}, float{});
   return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
 }
 

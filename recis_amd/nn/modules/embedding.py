@@ -95,7 +95,7 @@ class LookupPoolFunction(torch.autograd.Function):
     gradients per unique row over the plan and hands (row index, gradient) to the table."""
 
     @staticmethod
-    def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly):
+    def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly, unit_segments=False):
         if readonly:
             index = impl.lookup_index(plan.unique, True)
         else:
@@ -104,7 +104,14 @@ class LookupPoolFunction(torch.autograd.Function):
             index_buf = impl.lookup_index_counted(plan)
             index = impl.settle_lookup(index_buf, plan.U)
         chunks, chunk_rows = impl.emb_blocks()
-        out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets, combiner)
+        if unit_segments:
+            # one id per segment (sum == mean == the row itself): every unique row is read once and
+            # written to its occurrences, instead of one index chase per output row
+            out = ops.plan_expand_rows(plan, plan.inverse.numel(), blocks=chunks, block_size=chunk_rows,
+                                       row_index=index, weight=weight)
+        else:
+            out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets,
+                                                    combiner)
         ctx.impl, ctx.plan, ctx.combiner, ctx.readonly = impl, plan, combiner, readonly
         ctx.save_for_backward(index, weight, offsets)
         ctx.mark_non_differentiable(index)
@@ -118,13 +125,14 @@ class LookupPoolFunction(torch.autograd.Function):
             keep = index >= 0
             index, g = index[keep], g[keep]
         ctx.impl.accept_grad(index, g, unique=True)
-        return None, None, None, None, None, None, None
+        return None, None, None, None, None, None, None, None
 
 
-def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt):
+def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False):
     """Rows of the plan's unique ids pooled per segment. Sum / mean over a float table go
     through ``LookupPoolFunction`` (pooling reads the table directly); everything else looks the
-    rows up first and pools the copy."""
+    rows up first and pools the copy. ``unit_segments``: the caller built ``offsets`` as
+    0, 1, 2, ... (dense ``[B, 1]`` id tensors), so segment i holds exactly occurrence i."""
     impl = hashtable._hashtable_impl
     float_table = hashtable._dtype in (torch.float32, torch.bfloat16, torch.float16)
     n_occ = plan.inverse.numel()
@@ -140,7 +148,7 @@ def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt):
                 admit = HashtableHookFactory().create_admit_hook(hashtable, opt.admit_hook)
                 assert isinstance(admit, ReadOnlyHookImpl), "admit hook only support ReadOnlyHook yet, but got: %s" % admit
             index, out = LookupPoolFunction.apply(hashtable._backward_holder, impl, plan, weight, offsets,
-                                                  opt.combiner, readonly)
+                                                  opt.combiner, readonly, unit_segments)
             hashtable._filter_hook_impl(index)
             return out
         readonly = (not hashtable.training) or opt.admit_hook is not None
@@ -179,6 +187,7 @@ class DynamicEmbedding(torch.nn.Module):
             reserve_rows=emb_opt.reserve_rows)
 
     def deal_with_tensor(self, input_tensor: Union[torch.Tensor, RaggedTensor]):
+        self._unit_segments = False
         if isinstance(input_tensor, RaggedTensor):
             val = input_tensor.values()
             weight = input_tensor.weight()
@@ -194,6 +203,7 @@ class DynamicEmbedding(torch.nn.Module):
             offsets = torch.arange(bs + 1, device=val.device) * fea_dim
             weight = None
             shape = tuple(input_tensor.shape[:-1])
+            self._unit_segments = fea_dim == 1
         else:
             raise TypeError("DynamicEmbedding only support RaggedTensor or dense tensor, got %s" % type(input_tensor))
         return val, offsets, weight, shape
@@ -208,7 +218,7 @@ class DynamicEmbedding(torch.nn.Module):
         if weight is not None:
             weight = weight.to(dev) if opt.use_weight else None
         plan = ops.ids_unique_plan(val, wait=False)
-        out = lookup_and_pool(self._hashtable, plan, weight, offsets, opt)
+        out = lookup_and_pool(self._hashtable, plan, weight, offsets, opt, unit_segments=self._unit_segments)
         if opt.combiner == "tile":
             return out.view(tuple(shape) + (opt.combiner_kwargs["tile_len"] * opt.embedding_dim,))
         return out.view(tuple(shape) + (opt.embedding_dim,))

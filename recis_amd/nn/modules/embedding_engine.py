@@ -67,7 +67,9 @@ class EmbeddingEngine(torch.nn.Module):
 
     @staticmethod
     def _format(name, opt, data):
-        """(values int64 [N], weight | None, offsets int32 [S+1], output shape prefix)."""
+        """(values int64 [N], weight | None, offsets int32 [S+1], output shape prefix, whether the
+        offsets are 0, 1, 2, ... by construction)."""
+        unit = False
         if isinstance(data, RaggedTensor):
             values = data.values()
             offsets = data.offsets()[-1]
@@ -87,11 +89,12 @@ class EmbeddingEngine(torch.nn.Module):
             offsets = torch.arange(rows + 1, device=data.device, dtype=torch.int32) * width
             weight = None
             shape = tuple(data.shape[:-1])
+            unit = width == 1
         else:
             raise TypeError("feature %s: expected RaggedTensor or Tensor, got %s" % (name, type(data)))
         if values.dtype != torch.int64:
             values = values.long()
-        return values, weight, offsets.to(torch.int32), shape
+        return values, weight, offsets.to(torch.int32), shape, unit
 
     def forward(self, inputs: Dict[str, Union[torch.Tensor, RaggedTensor]]):
         outputs = {}
@@ -106,8 +109,10 @@ class EmbeddingEngine(torch.nn.Module):
             for names in runtime.values():
                 opt0 = grp.features[names[0]]
                 vals, weights, offs, shapes, tags = [], [], [], [], []
+                all_unit = True
                 for name in names:
-                    v, w, o, shape = self._format(name, grp.features[name], inputs[name])
+                    v, w, o, shape, unit = self._format(name, grp.features[name], inputs[name])
+                    all_unit = all_unit and unit
                     vals.append(v.to(dev))
                     offs.append(o.to(dev))
                     if w is None and opt0.use_weight and any(
@@ -125,7 +130,7 @@ class EmbeddingEngine(torch.nn.Module):
                 if all(w is not None for w in weights):
                     weight = weights[0] if len(weights) == 1 else torch.cat(weights)
                 plan = ops.ids_unique_plan(ids, wait=False)
-                pooled = lookup_and_pool(table, plan, weight, offsets, opt0)
+                pooled = lookup_and_pool(table, plan, weight, offsets, opt0, unit_segments=all_unit)
                 seg_counts = [o.numel() - 1 for o in offs]
                 width = pooled.shape[1]
                 for name, part, shape in zip(names, torch.split(pooled, seg_counts), shapes):

@@ -835,6 +835,28 @@ def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False, co
     return out
 
 
+def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_index=None, weight=None, out_dtype=None):
+    """``out[i] = weight[i] * row(unique id of occurrence i)`` for the ``n_out`` occurrences of
+    ``plan``: every unique row is read once and written to all its occurrences. Rows come from
+    ``rows`` ``[U, D]`` or from ``blocks`` (row u = row ``row_index[u]``, negative = zeros)."""
+    if blocks is not None:
+        require_cuda(row_index, weight)
+        table, dt, D, dev = block_ptr_table(blocks), blocks[0].dtype, blocks[0][0].numel(), blocks[0].device
+        n_blocks, rows_arg = len(blocks), None
+    else:
+        require_cuda(rows, weight)
+        rows = _contig(rows)
+        table, dt, D, dev, n_blocks, rows_arg = None, rows.dtype, rows.shape[1], rows.device, 0, rows
+    out = torch.empty((n_out, D), dtype=out_dtype or dt, device=dev)
+    weight = _contig(weight)
+    check(lib().recis_csr_expand_rows(ptr(rows_arg), ptr(table), i64(n_blocks), i64(block_size), ptr(row_index),
+                                      dtype_code(dt), ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
+                                      ptr(plan.row_start), ptr(plan.occ), ptr(plan.hot_items), i64(plan.hot_cap),
+                                      ptr(plan.counts), ptr(out), dtype_code(out.dtype), i64(plan.U), i64(n_out),
+                                      i64(D), stream_ptr(dev)))
+    return out
+
+
 def segment_reduce_backward_plan(grad_output, weight, offsets, plan, mode, out=None, accumulate=False):
     """Backward of the pooling for duplicated ids without atomics on row data: the same
     result as ``segment_reduce_backward(grad, weight, plan.inverse, offsets, plan.U, mode)``

@@ -262,3 +262,74 @@ def test_config2_shape_properties(mode):
     lhs = (out.double() * g.double()).sum()
     rhs = (emb.double() * gx.double()).sum()
     torch.testing.assert_close(lhs, rhs, rtol=1e-6, atol=1e-2)
+
+
+# ------------------------------------------------------------------ expand (one id per segment)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [1, 3, 16, 32, 128, 300])
+def test_expand_rows_equals_pooling_of_unit_segments(dtype, D):
+    """Reading each unique row once and writing it to its occurrences gives, bit for bit, what the
+    pooling kernels give for segments of one id (sum and mean), with and without weights, out of a
+    dense [U, D] array and straight out of table blocks, with hot ids that go through the plan's
+    work items."""
+    from recis_amd import _lib, ops
+
+    g = torch.Generator(device="cuda").manual_seed(D)
+    n = 50000
+    ids = torch.randint(0, 4000, (n,), device="cuda", generator=g)
+    ids[::3] = 7            # a hot id: ~16 700 occurrences
+    ids[1::50] = 9          # a medium one: the wave-cooperative path
+    plan = ops.ids_unique_plan(ids)
+    U = plan.U
+    rows = torch.randn(U, D, device="cuda", generator=g).to(dtype)
+    offsets = torch.arange(n + 1, device="cuda", dtype=torch.int32)
+    weight = torch.rand(n, device="cuda", generator=g).to(dtype)
+    for w in (None, weight):
+        exp = ops.segment_reduce_forward(rows, w, plan.inverse, offsets, "sum")
+        got = ops.plan_expand_rows(plan, n, rows=rows, weight=w)
+        assert got.dtype == exp.dtype and torch.equal(got, exp)
+    # out of a block list, with keys the table does not hold (row -1 reads as zeros)
+    bs, nb = 1024, -(-U // 1024) + 1
+    blocks = [torch.randn(bs, D, device="cuda", generator=g).to(dtype) for _ in range(nb)]
+    index = torch.randperm(bs * nb, device="cuda", generator=g)[:U]
+    index[::11] = -1
+    exp = ops.segment_reduce_forward_blocks(blocks, bs, index, None, plan.inverse, offsets, "mean")
+    got = ops.plan_expand_rows(plan, n, blocks=blocks, block_size=bs, row_index=index)
+    assert torch.equal(got, exp)
+    assert _lib.poll_device_errors() == 0
+
+
+def test_engine_takes_the_expand_path_for_dense_id_columns():
+    """Dense [B] id tensors through EmbeddingEngine (one id per sample: the click-through shape)
+    against the same ids as RaggedTensors with explicit offsets: same outputs, same gradients."""
+    from recis_amd.nn import EmbeddingEngine, EmbeddingOption
+    from recis_amd.nn.initializers import NormalInitializer
+    from recis_amd.nn.modules.hashtable import HashtableRegister
+    from recis_amd.ragged.tensor import RaggedTensor
+
+    def make():
+        HashtableRegister().clear()
+        torch.manual_seed(0)
+        return EmbeddingEngine({f: EmbeddingOption(embedding_dim=16, shared_name=f, combiner="sum", block_size=512,
+                                                   initializer=NormalInitializer(0, 0.1), use_weight=False)
+                                for f in ("a", "b")})
+
+    g = torch.Generator(device="cuda").manual_seed(1)
+    ids = {f: torch.randint(0, 300, (4096,), device="cuda", generator=g) for f in ("a", "b")}
+    up = torch.randn(4096, 16, device="cuda", generator=g)
+    results = []
+    for as_ragged in (False, True):
+        eng = make()
+        eng.train()
+        inputs = {f: RaggedTensor(v, torch.arange(4097, device="cuda", dtype=torch.int32)) if as_ragged else v
+                  for f, v in ids.items()}
+        out = eng(inputs)
+        (out["a"] * up).sum().backward()
+        impl = list(eng.hashtables().values())[0]._hashtable_impl
+        index, grad = impl.grad_pairs(1)
+        order = torch.argsort(index)
+        results.append((out["a"].detach().clone(), out["b"].detach().clone(), index[order], grad[order]))
+    for x, y in list(zip(*results))[:3]:
+        assert torch.equal(x, y)
+    # the order in which the occurrences of one id are summed is not fixed from run to run
+    torch.testing.assert_close(results[0][3], results[1][3], rtol=1e-5, atol=1e-5)
