@@ -1,0 +1,168 @@
+"""The benchmark workloads at their full sizes, checked through properties that do not need a
+CPU pass over the whole input: the dedup plan is a bijection onto the distinct ids, pooled rows
+are the table's rows, the per-row gradients sum to the incoming gradients and agree with a direct
+index_add, the optimizer step on a sample of rows equals the CPU oracle bit for bit, new keys get
+rows nobody holds. They run the stages of ``bench.py``'s workload classes, so they also check that
+the timed step computes what it is meant to."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from recis_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _rows_of(table, index):
+    chunks, chunk_rows = table.emb_blocks()
+    return ops.block_gather(index, chunks, chunk_rows, -1, True)
+
+
+def _slot_rows(table, name, index):
+    return table.get_slot(name).index_select(index)
+
+
+def test_config4_step_properties():
+    import bench
+
+    wl = bench.Config4()
+    for _ in range(2):          # second step: all keys known, rows and Adam state not trivial
+        wl.step()
+    ids = wl.feature_ops()
+    N, D = wl.N, wl.D
+    assert ids.numel() == N == 39 * 65536
+    # feature ops against their definitions on a full column
+    d0 = wl.c["dense"][0]
+    exp_bucket = torch.bucketize(d0, wl.c["boundaries"][0], right=True) % wl.c["mod"]
+    tag = 26
+    assert torch.equal(ids[26 * 65536: 27 * 65536], exp_bucket | (tag << 52))
+    assert torch.equal(ids[: 65536], wl.c["sparse"][0] & ((1 << 52) - 1))
+
+    plan, inv = wl.dedup(ids)
+    uniq = plan.unique
+    U = plan.U
+    assert torch.equal(uniq[inv.long()], ids)                      # inverse maps every id to itself
+    assert torch.unique(uniq).numel() == U == torch.unique(ids).numel()
+    rs = plan.row_start[: U + 1].long()
+    assert int(rs[0]) == 0 and int(rs[-1]) == N and bool((rs[1:] > rs[:-1]).all())
+    occ = plan.occ.long()
+    assert torch.equal(torch.sort(occ).values, torch.arange(N, device="cuda"))   # every occurrence listed once
+    owner = torch.repeat_interleave(torch.arange(U, device="cuda"), rs[1:] - rs[:-1])
+    assert torch.equal(inv.long()[occ], owner)                     # and under its own id
+
+    index = wl.lookup(plan)
+    assert torch.equal(index, wl.table.lookup_index_readonly(uniq[:U]))
+    assert torch.unique(index).numel() == U and int(index.min()) >= 0
+
+    pooled = wl.pool_fwd(index, inv)
+    assert torch.equal(pooled, _rows_of(wl.table, index)[inv.long()])   # one id per segment: its row
+
+    g = wl.pool_bwd(inv)
+    ref = torch.zeros(U, D, device="cuda", dtype=torch.float64).index_add_(0, inv.long(), wl.grad_out.double())
+    scale = torch.zeros(U, device="cuda", dtype=torch.float64).index_add_(
+        0, inv.long(), wl.grad_out.double().abs().sum(1)).clamp_(min=1.0)
+    assert float(((g.double() - ref).abs().sum(1) / scale).max()) < 1e-5
+    torch.testing.assert_close(g.double().sum(0), wl.grad_out.double().sum(0), rtol=1e-6, atol=1e-3)
+
+    # the Adam step on a sample of rows against the CPU oracle, bit for bit
+    pick = torch.randperm(U, device="cuda")[:4096]
+    rows = index[pick]
+    names = [s.name() for s in wl.table.slot_group().slots()]
+    before = [_slot_rows(wl.table, n, rows).cpu().numpy() for n in names[:3]]
+    state = wl.opt.state_dict()[1]
+    b1t = [v for k, v in state.items() if k.endswith("beta1")][0].cpu().numpy().copy().reshape(1)
+    b2t = [v for k, v in state.items() if k.endswith("beta2")][0].cpu().numpy().copy().reshape(1)
+    wl.update(index, g)
+    after = [_slot_rows(wl.table, n, rows).cpu().numpy() for n in names[:3]]
+    w, m, v = [b.copy() for b in before]
+    oracle.block_apply_adamw(np.arange(4096), g[pick].cpu().numpy(), [w], b1t, b2t, [m], [v], 1e-3, 0.9, 0.999, 1.0,
+                             1e-8, 4096)
+    for got, exp in zip(after, (w, m, v)):
+        np.testing.assert_array_equal(got, exp)
+    assert _lib.poll_device_errors() == 0
+
+
+def test_config3_lookups_at_scale():
+    """A tenth of the resident set of config 3 (2e7 rows, so that the test stays short) with the full
+    per-step lookup size: known keys keep their rows, never-seen keys get rows nobody holds, the
+    expansion gives every lookup its key's row, eviction removes exactly the keys not seen."""
+    import bench
+
+    wl = bench.Config3(resident=20_000_000, ids_per_step=2_000_000, n_batches=3)
+    t = wl.table
+    lv0, idn0, _, _ = t.id_map().stats()
+    assert lv0 == 20_000_000
+    ids = wl.batches[0]
+    known = t.lookup_index_readonly(ids)
+    n_new = int(torch.unique(ids[known < 0]).numel())
+    assert 0.05 * ids.numel() < n_new <= 0.1 * ids.numel() + 1
+    out = wl.step()                                            # consumes batch 0
+    lv1, idn1, _, _ = t.id_map().stats()
+    assert lv1 == lv0 + n_new and idn1 == idn0 + n_new
+    now = t.lookup_index_readonly(ids)
+    assert int(now.min()) >= 0
+    assert torch.equal(now[known >= 0], known[known >= 0])     # known keys keep their rows
+    fresh = torch.unique(now[known < 0])
+    assert fresh.numel() == n_new and int(fresh.min()) >= idn0  # new keys: rows above the old mark
+    # one output row per lookup = that key's row as it was read in the step (Adam moved it since):
+    # rows of equal keys are equal, rows of a sample agree with the table up to one Adam step
+    order = torch.argsort(ids, stable=True)
+    same = ids[order][1:] == ids[order][:-1]
+    assert torch.equal(out[order][1:][same], out[order][:-1][same])
+    drift = (out - _rows_of(t, now)).abs().max()
+    assert 0 < float(drift) < 0.02                             # lr 1e-3, a few steps at most
+    # eviction by last-seen step: everything not touched in step 0 is older than the threshold
+    wl.step_t.fill_(5)
+    wl.step()                                                  # batch 1 stamped with step 5
+    seen = torch.unique(wl.batches[1])
+    live_before = t.id_map().stats()[0]
+    gone_ids, gone_rows = t.evict_older("step_filter", 5)
+    lv2 = t.id_map().stats()[0]
+    assert lv2 == seen.numel() and gone_ids.numel() == live_before - lv2 == gone_rows.numel()
+    assert int(t.lookup_index_readonly(seen).min()) >= 0
+    assert int(t.lookup_index_readonly(gone_ids[:100000]).max()) == -1
+    assert _lib.poll_device_errors() == 0
+
+
+def test_config5_step_properties():
+    import bench
+
+    wl = bench.Config5()
+    wl.step()
+    o = ops
+    ids = o.ids_encode([f["values"] for f in wl.fields], list(range(len(wl.fields))))
+    plan = o.ids_unique_plan(ids)
+    inv, U = plan.inverse.long(), plan.U
+    assert torch.equal(plan.unique[inv], ids)
+    index = wl.table.lookup_index_readonly(plan.unique[:U])
+    assert int(index.min()) >= 0
+    rows = _rows_of(wl.table, index)                            # bf16 [U, 128]
+    off = wl.offsets.long()
+    assert int(off[-1]) == wl.N and off.numel() == wl.S + 1
+    pooled = o.segment_reduce_forward(rows, None, plan.inverse, wl.offsets, "mean", out_dtype=torch.float32)
+    lens = (off[1:] - off[:-1])
+    seg = torch.repeat_interleave(torch.arange(wl.S, device="cuda"), lens)
+    ref = torch.zeros(wl.S, wl.D, device="cuda", dtype=torch.float64).index_add_(0, seg, rows[inv].double())
+    ref /= lens.clamp(min=1).view(-1, 1)
+    torch.testing.assert_close(pooled.double(), ref, rtol=1e-5, atol=1e-6)
+    # the padded gather: position t of sample b of field f holds the row of its t-th id, zeros past its length
+    padded, _ = o.ragged_tile(wl.batch, wl.seq, plan.inverse, wl.offsets, rows)
+    assert padded.shape == (wl.pad_rows, wl.D) and padded.dtype == torch.bfloat16
+    base_row, base_seg = 0, 0
+    for b, L in zip(wl.batch, wl.seq):
+        view = padded[base_row: base_row + b * L].view(b, L, wl.D)
+        o_f = off[base_seg: base_seg + b + 1]
+        l_f = (o_f[1:] - o_f[:-1]).clamp(max=L)
+        pos = torch.arange(L, device="cuda").view(1, L)
+        mask = pos < l_f.view(-1, 1)
+        assert float(view[~mask].abs().sum()) == 0
+        src = (o_f[:-1].view(-1, 1) + pos)[mask]
+        assert torch.equal(view[mask], rows[inv[src]])
+        base_row += b * L
+        base_seg += b
+    # backward of both outputs: checksum against the incoming gradients
+    g = o.segment_reduce_backward_plan(wl.g_pool, None, wl.offsets, plan, "mean")
+    exp = (wl.g_pool.double() * (lens > 0).view(-1, 1)).sum(0)
+    torch.testing.assert_close(g.double().sum(0), exp, rtol=1e-5, atol=1e-2)
+    assert _lib.poll_device_errors() == 0
