@@ -636,6 +636,41 @@ class GradWorkerMeanFunction(torch.autograd.Function):
         return _scatter_sum(grad_outputs, index, ctx.unique_size, ctx.plan).to(grad_outputs.dtype), None, None, None
 
 
+class LookupExpandFunction(torch.autograd.Function):
+    """Lookup of a plan's unique ids and one output row per request in one pass over the table
+    (what HashTableLookupHelpFunction + GradWorkerMeanFunction give, hashtable.py:425-586, without
+    the ``[U, D]`` copy of the rows): every unique row is read once and written to its
+    occurrences. Backward: sum over the duplicates of each id, divided by the number of workers."""
+
+    @staticmethod
+    def forward(ctx, backward_holder, impl, plan, slice_num, readonly):
+        if readonly:
+            index = impl.lookup_index(plan.unique, True)
+        else:
+            index_buf = impl.lookup_index_counted(plan)   # queued before the host has the unique count
+            index = impl.settle_lookup(index_buf, plan.U)
+        chunks, chunk_rows = impl.emb_blocks()
+        out = ops.plan_expand_rows(plan, plan.inverse.numel(), blocks=chunks, block_size=chunk_rows, row_index=index)
+        ctx.impl, ctx.plan, ctx.slice_num, ctx.readonly = impl, plan, slice_num, readonly
+        ctx.save_for_backward(index)
+        ctx.mark_non_differentiable(index)
+        return index, out
+
+    @staticmethod
+    def backward(ctx, _grad_index, grad):
+        (index,) = ctx.saved_tensors
+        n = ctx.plan.inverse.numel()
+        flat = grad.reshape(n, -1).contiguous()
+        if ctx.slice_num != 1:
+            flat = flat / ctx.slice_num
+        g = ops.csr_gather_reduce(flat, ctx.plan, ctx.plan.occ).to(grad.dtype)
+        if ctx.readonly:  # keys the table does not hold take no gradient
+            keep = index >= 0
+            index, g = index[keep], g[keep]
+        ctx.impl.accept_grad(index, g, unique=True)
+        return None, None, None, None, None
+
+
 def _scatter_sum(grad_rows, index, unique_size, plan=None):
     """sum of ``grad_rows[i]`` into row ``index[i]`` of a ``[unique_size, D]`` result: a
     gather-reduce over the batch plan's occurrence lists when there is one, fp32 atomics else."""
@@ -713,6 +748,17 @@ class HashTable(torch.nn.Module):
         admit_hook_impl = HashtableHookFactory().create_admit_hook(self, admit_hook) if admit_hook else None
         shape = tuple(ids.shape)
         ids = ids.to(self._device).reshape(-1)
+        if self.training and self._dedup != "sorted" and self._grad_reduce_by != "id" and len(
+                self._hashtable_impl._embedding_shape) == 1 and self._dtype in (torch.float32, torch.bfloat16, torch.float16):
+            from .hashtable_hook_impl import ReadOnlyHookImpl
+
+            assert admit_hook_impl is None or isinstance(admit_hook_impl, ReadOnlyHookImpl), \
+                "admit hook only support ReadOnlyHook yet, but got: %s" % admit_hook_impl
+            plan = ops.ids_unique_plan(ids, wait=False)
+            emb_idx, embedding = LookupExpandFunction.apply(self._backward_holder, self._hashtable_impl, plan,
+                                                            self._worker_num, admit_hook_impl is not None)
+            self._filter_hook_impl(emb_idx)
+            return embedding.view(shape + tuple(embedding.shape[1:])) if len(shape) != 1 else embedding
         uids, index, plan = self._unique(ids)
         if self.training and self._dtype not in (torch.int8, torch.int32, torch.int64):
             emb_idx, embedding = HashTableLookupHelpFunction.apply(uids, self._hashtable_impl,
