@@ -13,7 +13,6 @@ import torch
 import oracle
 import workloads
 from oracle import cpu_path
-from recis_amd import ops
 from recis_amd.hooks import HashTableFilterHook
 from recis_amd.nn import DynamicEmbedding, EmbeddingEngine, EmbeddingOption, HashTable
 from recis_amd.nn.functional.embedding_ops import ragged_embedding_segment_reduce

@@ -4,7 +4,6 @@ back by the safetensors library, loaded into fresh tables, and saved again uncha
 import json
 import os
 
-import numpy as np
 import pytest
 import torch
 from safetensors import safe_open
