@@ -45,7 +45,7 @@ extern "C" {
 /* flags */
 /* batch plan: unique ids with more than HOT_LEN occurrences are reduced by whole workgroups,
  * one (row, chunk of HOT_CHUNK occurrences) work item each */
-#define RECIS_PLAN_HOT_LEN 256
+#define RECIS_PLAN_HOT_LEN 64
 #define RECIS_PLAN_HOT_CHUNK 2048
 
 #define RECIS_PLAN_STAGE_COUNT 1

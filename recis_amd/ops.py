@@ -717,7 +717,7 @@ class IdMap:
 
 
 # ------------------------------------------------------------------ batch plan
-_HOT_LEN, _HOT_CHUNK = 256, 2048  # RECIS_PLAN_HOT_LEN / RECIS_PLAN_HOT_CHUNK of the library
+_HOT_LEN, _HOT_CHUNK = 64, 2048  # RECIS_PLAN_HOT_LEN / RECIS_PLAN_HOT_CHUNK of the library
 
 
 _STAGED = {}  # stream -> the plan whose count is on its way to that stream's staging word

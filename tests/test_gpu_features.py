@@ -210,9 +210,9 @@ def _check_plan(ids):
     np.testing.assert_array_equal(inv[occ], row_of_entry)
     counts = p.counts.cpu().numpy()
     lens = np.diff(rs[: p.U + 1])
-    assert counts[0] == p.U and counts[1] == int(np.sum(np.ceil(lens[lens > 256] / ops._HOT_CHUNK)))
+    assert counts[0] == p.U and counts[1] == int(np.sum(np.ceil(lens[lens > ops._HOT_LEN] / ops._HOT_CHUNK)))
     hot = p.hot_items.cpu().numpy()[: 2 * counts[1]].reshape(-1, 2)
-    exp_hot = sorted((int(u), c) for u in np.nonzero(lens > 256)[0] for c in range(-(-int(lens[u]) // ops._HOT_CHUNK)))
+    exp_hot = sorted((int(u), c) for u in np.nonzero(lens > ops._HOT_LEN)[0] for c in range(-(-int(lens[u]) // ops._HOT_CHUNK)))
     assert sorted(map(tuple, hot.tolist())) == exp_hot
     q = ops.ids_unique_plan(_dev(ids))
     np.testing.assert_array_equal(q.unique.cpu().numpy(), uniq)
@@ -252,7 +252,7 @@ def test_unique_plan_skewed_buckets(rng):
 @pytest.mark.parametrize("D,dtype", [(16, torch.float32), (128, torch.bfloat16), (40, torch.float32)])
 def test_planned_backward_matches_oracle(rng, mode, D, dtype):
     """Gradient scatter over heavily duplicated ids (Zipf-like head + a cold tail) through the plan:
-    same numbers as the oracle's sequential scatter, hot rows (> 256 occurrences) included."""
+    same numbers as the oracle's sequential scatter, hot rows (many occurrences) included."""
     S = 3000
     off = ragged_offsets(rng, S, 0, 40, empty_frac=0.1)
     N = int(off[-1])
