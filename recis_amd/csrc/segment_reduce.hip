@@ -199,16 +199,29 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
 // Rows are summed per row group in increasing order, like the generic kernel. Requires U < 2^31.
 enum { kFastPlain = 0, kFastRev32 = 1, kFastRev64 = 2 };
 
-template <typename TIn, typename TOut, int VEC, int KIND, bool BLK>
+// WG: long segments (behaviour sequences of hundreds of rows): a whole workgroup per segment, each
+// of its waves sums a contiguous quarter of the rows and the quarters meet in LDS. With a wave per
+// segment the launch lasts as long as its longest segment takes one wave.
+template <typename TIn, typename TOut, int VEC, int KIND, bool BLK, bool WG = false>
 __global__ void __launch_bounds__(kBlock)
 seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs a) {
-  const int64_t s = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.team_log2) + (threadIdx.x >> a.team_log2);
+  extern __shared__ float s_wave_part[];  // WG only: [waves][D]
+  const int64_t s = WG ? static_cast<int64_t>(blockIdx.x)
+                       : static_cast<int64_t>(blockIdx.x) * (kBlock >> a.team_log2) + (threadIdx.x >> a.team_log2);
   if (s >= a.S) return;  // whole teams leave together
   int64_t start = load_index(a.offs, a.off64, s);
   int64_t end = load_index(a.offs, a.off64, s + 1);
   if (start < 0 || end > a.B || end < start) {
     raise_device_error(a.err, RECIS_DEVERR_OFFSETS);
     start = end = 0;
+  }
+  const int64_t seg_len = end - start;
+  const int wave = threadIdx.x / kWave;
+  if constexpr (WG) {  // this wave's share of the rows
+    constexpr int n_waves = kBlock / kWave;
+    const int64_t share = (seg_len + n_waves - 1) / n_waves;
+    start = min(end, start + wave * share);
+    end = min(end, start + share);
   }
   const int team = 1 << a.team_log2;
   const int lane = threadIdx.x & (kWave - 1);
@@ -219,7 +232,7 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
   const int step = team >> a.lpr_log2;
   const int col_stride = VEC << a.lpr_log2;
   const int D = a.D;
-  const float scale = (a.mean && end > start) ? 1.0f / static_cast<float>(end - start) : 1.0f;
+  const float scale = (a.mean && seg_len > 0) ? 1.0f / static_cast<float>(seg_len) : 1.0f;
 
   for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
     const int c0 = cbase + cl * VEC;
@@ -288,7 +301,24 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
     }
-    if (rg == 0 && col_ok) {
+    if constexpr (WG) {
+      constexpr int n_waves = kBlock / kWave;
+      if (rg == 0 && col_ok) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) s_wave_part[wave * D + c0 + j] = acc[j];
+      }
+      __syncthreads();
+      if (wave == 0 && rg == 0 && col_ok) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          float sum = s_wave_part[c0 + j];
+          for (int w = 1; w < n_waves; ++w) sum += s_wave_part[w * D + c0 + j];
+          acc[j] = sum * scale;
+        }
+        store_pack<TOut, VEC>(out + s * D + c0, acc);
+      }
+      __syncthreads();
+    } else if (rg == 0 && col_ok) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] *= scale;
       store_pack<TOut, VEC>(out + s * D + c0, acc);
@@ -980,8 +1010,17 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
             TOut* o = static_cast<TOut*>(out);
             // several rows per segment: the latency-oriented kernel; about one row: the lean one
             const bool fast = a.weight == nullptr && U < (int64_t(1) << 31) && a.team_log2 > a.lpr_log2;
+            // segments of hundreds of rows: a workgroup each (the team is a whole wave already)
+            const bool wg = fast && a.team_log2 == 6 && S > 0 && B / S >= 128 && D <= 4096;
+            const size_t wg_lds = sizeof(float) * (kBlock / kWave) * static_cast<size_t>(D);
             RECIS_TIME_KERNEL("seg_pool_fwd_kernel", stream)
-            if (fast && a.rev == nullptr)
+            if (wg && a.rev == nullptr)
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastPlain, false, true><<<dim3(S), dim3(kBlock), wg_lds, stream>>>(e, o, a);
+            else if (wg && !a.rev64)
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32, false, true><<<dim3(S), dim3(kBlock), wg_lds, stream>>>(e, o, a);
+            else if (wg)
+              seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev64, false, true><<<dim3(S), dim3(kBlock), wg_lds, stream>>>(e, o, a);
+            else if (fast && a.rev == nullptr)
               seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastPlain, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);
             else if (fast && !a.rev64)
               seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32, false><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, a);

@@ -333,3 +333,36 @@ def test_engine_takes_the_expand_path_for_dense_id_columns():
         assert torch.equal(x, y)
     # the order in which the occurrences of one id are summed is not fixed from run to run
     torch.testing.assert_close(results[0][3], results[1][3], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [3, 64, 128, 520])
+def test_long_segments_workgroup_path(dtype, D):
+    """Segments of hundreds of rows (a workgroup per segment) against a float64 sum, with and
+    without reverse indices, int32 and int64, empty and very short segments in between."""
+    from recis_amd import _lib, ops
+
+    g = torch.Generator(device="cuda").manual_seed(D)
+    lens = torch.randint(100, 900, (300,), generator=torch.Generator().manual_seed(D))
+    lens[::17] = 0
+    lens[5::29] = 3
+    off = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).cuda()
+    n, U = int(off[-1]), 5000
+    rows = torch.randn(U, D, device="cuda", generator=g).to(dtype)
+    rev = torch.randint(0, U, (n,), device="cuda", generator=g)
+    seg = torch.repeat_interleave(torch.arange(300, device="cuda"), lens.cuda())
+    for mode in ("sum", "mean"):
+        ref = torch.zeros(300, D, device="cuda", dtype=torch.float64).index_add_(0, seg, rows[rev].double())
+        mag = torch.zeros(300, device="cuda", dtype=torch.float64).index_add_(0, seg, rows[rev].double().abs().sum(1))
+        if mode == "mean":
+            ref /= lens.cuda().clamp(min=1).view(-1, 1)
+            mag /= lens.cuda().clamp(min=1)
+        for r in (rev, rev.int()):
+            for o in (off, off.int()):
+                got = ops.segment_reduce_forward(rows, None, r, o, mode, out_dtype=torch.float32)
+                err = (got.double() - ref).abs().sum(1)
+                assert bool((err <= 1e-5 * ref.abs().sum(1) + 1e-6 * mag.clamp(min=1.0)).all()), (mode, r.dtype, o.dtype)
+    plain = ops.segment_reduce_forward(rows[rev], None, None, off, "sum", out_dtype=torch.float32)
+    ref = torch.zeros(300, D, device="cuda", dtype=torch.float64).index_add_(0, seg, rows[rev].double())
+    torch.testing.assert_close(plain.double(), ref, rtol=1e-5, atol=1e-3)
+    assert _lib.poll_device_errors() == 0
