@@ -537,6 +537,9 @@ def main():
     ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "ckpt"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    ap.add_argument("--no-stages", action="store_true",
+                    help="skip the stage-by-stage timings, so that every kernel launch of the run belongs to a "
+                         "full step (the form a kernel trace is compared with kernels_us in)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch a plain elementwise kernel that reads 1 GiB and writes 1 GiB "
                          "(scale for hardware-counter runs)")
@@ -608,7 +611,7 @@ def main():
 
     extras = {}
     if args.workload == "c4":
-        stages = main_wl.stage_times(max(5, args.steps))
+        stages = None if args.no_stages else main_wl.stage_times(max(5, args.steps))
         ab = main_wl.algorithmic_bytes()
         total_bytes = sum(ab.values())
         kern = _kernel_profile(main_wl.step, max(5, args.steps))
@@ -624,10 +627,12 @@ def main():
         out["kernels_gbs"] = {k: round(kb[k] / kern[k]["us"] / 1e3, 1) for k in kern if kb.get(k)}
         out["step_roofline"] = {"algorithmic_bytes": total_bytes, "achieved": total_bytes / ms_per_step / 1e6,
                                 "frac": total_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, "unit": "GB/s"}
-        out["stages_ms"] = {k: round(v, 4) for k, v in stages.items()}
-        out["stages_gbs"] = {k: round(ab[k] / stages[k] / 1e6, 1) for k in stages}
-        host_ms = _event_ms(main_wl.step_from_host, max(5, args.steps))
-        out["inputs_from_pinned_host"] = {"ms_per_step": round(host_ms, 4), "ids_per_s": main_wl.N / host_ms * 1e3}
+        if stages is not None:
+            out["stages_ms"] = {k: round(v, 4) for k, v in stages.items()}
+            out["stages_gbs"] = {k: round(ab[k] / stages[k] / 1e6, 1) for k in stages}
+            host_ms = _event_ms(main_wl.step_from_host, max(5, args.steps))
+            out["inputs_from_pinned_host"] = {"ms_per_step": round(host_ms, 4),
+                                              "ids_per_s": main_wl.N / host_ms * 1e3}
     elif args.workload == "c2":
         res = c2_summary(main_wl)
         dom = max(res, key=lambda k: res[k]["ms"])
