@@ -12,7 +12,9 @@ for sum / mean / max) is measured in the same run and reported under "workloads"
 "roofline" describes the kernel that takes the largest share of the step: algorithmic
 bytes per launch / mean launch time (HIP events on the launch stream) against the 8 TB/s
 HBM peak. "cpu_baseline" is the restated reference CPU path (oracle.cpu_path) timed on
-this host on a bounded sample of the same workload.
+this host on a bounded sample of the same workload; "cpu_reference_<n>t" is the reference's own
+CPU code (oracle/_ref, when built) on the same sample with n threads, for the parts of the step
+the reference can run on a CPU.
 """
 import argparse
 import json
@@ -282,7 +284,23 @@ class Config4:
             cpu_path.train_step(table, ids, off, None, grad)
             reps += 1
         dt = time.perf_counter() - t0
+        self._cpu_sample_ids = ids
         return n * reps / dt, "first %d samples (%d ids/step) of config 4, full step" % (b, n)
+
+    def cpu_reference(self, budget_s, threads):
+        """The reference's own CPU operators (compiled from its sources into oracle/_ref) on the
+        ids of cpu_baseline's sample: ids_partition + Hashtable.EmbeddingLookup + AcceptGrad +
+        SparseAdam.step. The reference has no CPU pooling operator, so this is the step without
+        the pooling forward and backward. None when the reference build is absent."""
+        from oracle import ref_ops
+        if not ref_ops.available():
+            return None
+        ids = np.ascontiguousarray(self._cpu_sample_ids, dtype=np.int64)
+        params = np.array([10240, self.D, 1e-3, 0.9, 0.999, 1e-8, 0.0, budget_s, threads], np.float64)
+        secs, steps, uniq = ref_ops.run("table_step_time", [params, ids], threads=threads)[0]
+        return {"value": ids.size * steps / secs, "unit": "ids/s", "cores": threads, "kind": "reference",
+                "sample": "the same %d ids/step (%d distinct): ids_partition + EmbeddingLookup + AcceptGrad + "
+                          "SparseAdam.step of the reference; its pooling has no CPU operator" % (ids.size, int(uniq))}
 
 
 
@@ -672,6 +690,11 @@ def main():
     if not args.no_cpu_baseline:
         v, sample = main_wl.cpu_baseline(12.0)
         out["cpu_baseline"] = {"value": v, "unit": "ids/s", "cores": 1, "kind": "port", "sample": sample}
+        if hasattr(main_wl, "cpu_reference"):
+            for threads in (1, min(16, os.cpu_count() or 1)):
+                ref = main_wl.cpu_reference(5.0, threads)
+                if ref is not None:
+                    out["cpu_reference_%dt" % threads] = ref
     from recis_amd import _lib
     out["device_errors"] = _lib.poll_device_errors()
     print(json.dumps(out))

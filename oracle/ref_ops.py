@@ -41,13 +41,13 @@ def _read(path):
     return out
 
 
-def run(op, arrays):
+def run(op, arrays, threads=1, timeout=300):
     """Outputs (list of numpy arrays) of reference operator ``op`` on ``arrays``."""
     with tempfile.TemporaryDirectory() as d:
         fin, fout = os.path.join(d, "in.bin"), os.path.join(d, "out.bin")
         _write(fin, arrays)
-        env = dict(os.environ, OMP_NUM_THREADS="1")
-        r = subprocess.run([BINARY, op, fin, fout], capture_output=True, text=True, env=env, timeout=300)
+        env = dict(os.environ, OMP_NUM_THREADS=str(threads))
+        r = subprocess.run([BINARY, op, fin, fout], capture_output=True, text=True, env=env, timeout=timeout)
         if r.returncode != 0:
             raise RuntimeError("ref_ops %s failed (%d): %s" % (op, r.returncode, r.stderr[-2000:]))
         return _read(fout)

@@ -26,6 +26,7 @@
 // int64 dims[ndim], raw bytes. dtype codes: 0 f32, 1 f64, 2 i64, 3 i32, 4 bool, 5 i8.
 #include <torch/extension.h>
 
+#include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -250,6 +251,44 @@ static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
             table->SlotGroup()->EmbSlot()->Value(),
             table->GetSlot(prefix + "exp_avg")->Value(),
             table->GetSlot(prefix + "exp_avg_sq")->Value()};
+  }
+  if (op == "table_step_time") {
+    // Times the CPU-runnable parts of one training step of the reference on one Hashtable with
+    // SparseAdam: ids_partition_cpu (dedup) + EmbeddingLookup + AcceptGrad + step + zero_grad.
+    // (The pooling between lookup and gradient has no CPU operator in the reference.)
+    // params f64 [9] = block_size, D, lr, beta1, beta2, eps, weight_decay, time budget in seconds,
+    //                  threads;  ids i64 [n] = one step's ids (duplicates included)
+    // Returns f64 [3] = seconds, steps timed, unique ids per step. Gradients are a constant.
+    const double* p = in[0].data_ptr<double>();
+    const int64_t bs = static_cast<int64_t>(p[0]), D = static_cast<int64_t>(p[1]);
+    at::set_num_threads(static_cast<int>(p[8]));
+    auto gen = recis::embedding::MakeConstantGenerator({bs, D}, torch::kFloat, 0.01);
+    auto table = Hashtable::Make(bs, {D}, torch::kFloat, torch::Device(torch::kCPU), true, {"t"}, gen, 0, 65536, 65536);
+    std::unordered_map<std::string, HashTablePtr> tables{{"t", table}};
+    recis::optim::SparseAdamOptions o;
+    o.lr(p[2]).betas(std::make_tuple(p[3], p[4])).eps(p[5]).weight_decay(p[6]);
+    auto opt = c10::make_intrusive<recis::optim::SparseAdam>(tables, o);
+    int64_t uniq = 0, steps = 0;
+    Tensor grad;
+    auto one_step = [&]() {
+      auto part = F::ids_partition_cpu(in[1], 1);
+      Tensor u = std::get<0>(part);
+      uniq = u.numel();
+      if (!grad.defined() || grad.size(0) != uniq) grad = torch::full({uniq, D}, 1e-3f);
+      auto r = table->EmbeddingLookup(u, false);
+      table->AcceptGrad(std::get<0>(r), grad);
+      opt->step();
+      opt->zero_grad();
+    };
+    one_step();  // admission of the ids: not timed
+    const auto t0 = std::chrono::steady_clock::now();
+    double dt = 0;
+    do {
+      one_step();
+      ++steps;
+      dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    } while (dt < p[7]);
+    return {torch::tensor({dt, static_cast<double>(steps), static_cast<double>(uniq)}, torch::kDouble)};
   }
   if (op == "ckpt_write_file") {
     // Writes ONE data file with the reference's TableWriter from a CPU Hashtable and a dense tensor.
