@@ -592,6 +592,22 @@ int recis_feature_cross_emit(const int64_t* x_val, const void* x_off, const void
                              const int32_t* y_count, const void* out_offsets, int64_t total,
                              int64_t* out_val, void* out_weight, void* stream);
 
+/*
+ * calc_ragged_index, drop left / pad right (csrc/ops/calc_ragged_index.cc:15-84; the only side
+ * combination the reference implements, on the CPU): row r of topk [rows, cols] holds
+ * positions in ragged row src = indicator[r] (0 <= src < src_rows) of offset [src_rows + 1],
+ * counted from the first element kept by a left truncation of drop_num[src] elements. Kept:
+ * e = topk[r, c] + offset[src] + drop_num[src] with offset[src] <= e < offset[src + 1], in column
+ * order. out_index (the type of topk, room for rows * cols) receives the kept e of all rows back
+ * to back, out_offsets (the type of offset, [rows + 1]) their running count per row, total_dev
+ * [1] the count. Each of drop_num / offset / topk / indicator is int32 or int64 (its *_is64).
+ * An indicator outside [0, src_rows) keeps nothing and raises the index-range soft error.
+ */
+int recis_ragged_topk_index(const void* drop_num, int drop_is64, const void* offset, int off_is64,
+                            int64_t src_rows, const void* topk, int topk_is64,
+                            const void* indicator, int indicator_is64, int64_t rows, int64_t cols,
+                            void* out_index, void* out_offsets, int64_t* total_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

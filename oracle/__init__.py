@@ -538,3 +538,41 @@ def feature_cross_ragged(x_val, x_off, x_w, y_val, y_off, y_w):
                 ws.append(wa * wb)
         offs.append(len(ids))
     return np.asarray(ids, np.int64), np.asarray(offs, x_off.dtype), np.asarray(ws, wdt)
+
+
+def calc_ragged_index(drop_num, offset, topk_index, indicator):
+    """Drop left / pad right of csrc/ops/calc_ragged_index.cc:55-76: for row r of topk_index
+    [rows, cols] and src = indicator[r], the kept elements offset[src] + drop_num[src] +
+    topk_index[r, c] that fall inside [offset[src], offset[src + 1]), in column order, and the
+    running count per row. Returns (value_index of topk_index's dtype, offsets of offset's dtype)."""
+    drop_num, offset, topk_index, indicator = (np.asarray(a) for a in (drop_num, offset, topk_index, indicator))
+    out, offs = [], [0]
+    for r in range(topk_index.shape[0]):
+        src = int(indicator[r])
+        beg, end, drop = int(offset[src]), int(offset[src + 1]), int(drop_num[src])
+        for c in range(topk_index.shape[1]):
+            e = int(topk_index[r, c]) + beg + drop
+            if beg <= e < end:
+                out.append(e)
+        offs.append(len(out))
+    return np.asarray(out, topk_index.dtype), np.asarray(offs, offset.dtype)
+
+
+def ragged_to_sparse_indices(offsets):
+    """COO coordinates [levels + 1, n_values] of the values of a ragged tensor with the given
+    list of offsets, outermost level first (csrc/ops/ragged_to_sparse.cc:8-40): coordinate 0 is
+    the outermost row, coordinate k the position inside the row of level k - 1."""
+    offsets = [np.asarray(o).astype(np.int64) for o in offsets]
+    n = int(offsets[-1][-1]) if len(offsets[-1]) else 0
+    idx = np.zeros((len(offsets) + 1, n), np.int64)
+    for v in range(n):
+        child = v
+        for k in range(len(offsets) - 1, -1, -1):
+            o = offsets[k]
+            row = 0
+            while not (o[row] <= child < o[row + 1]):
+                row += 1
+            idx[k + 1, v] = child - o[row]
+            child = row
+        idx[0, v] = child
+    return idx

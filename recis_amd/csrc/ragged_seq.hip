@@ -435,6 +435,56 @@ __global__ void __launch_bounds__(kBlock) cross_emit_kernel(const int64_t* xv, c
   }
 }
 
+// ---------------------------------------------------------------- top-k index selection
+// calc_ragged_index, drop left / pad right (csrc/ops/calc_ragged_index.cc:15-84): row r of
+// topk [rows, cols] holds positions inside ragged row src = indicator[r], counted from the
+// first element that a left truncation by drop_num[src] kept; position p stands for element
+// offset[src] + drop_num[src] + p of the values and is kept when that lies inside the row.
+// A wave per row: pass 1 counts the kept positions, pass 2 (after the scan) writes them in
+// column order at out_off[r] + (kept positions before this column), by ballot and popcount.
+struct TopkArgs {
+  const void* drop_num;
+  const void* offset;
+  const void* topk;
+  const void* indicator;
+  int drop64, off64, topk64, ind64;
+  int64_t rows, cols, src_rows;
+};
+
+template <bool EMIT>
+__global__ void __launch_bounds__(kBlock) topk_index_kernel(TopkArgs a, void* out_off, void* out_index, int* err) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t r = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+  if (r >= a.rows) return;  // whole waves leave together
+  const int64_t src = load_index(a.indicator, a.ind64, r);
+  int64_t beg = 0, end = 0, drop = 0;
+  if (src < 0 || src >= a.src_rows) {
+    if (lane == 0) raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+  } else {
+    beg = load_index(a.offset, a.off64, src);
+    end = load_index(a.offset, a.off64, src + 1);
+    drop = load_index(a.drop_num, a.drop64, src);
+  }
+  int64_t at = EMIT ? load_index(out_off, a.off64, r) : 0;
+  for (int64_t c0 = 0; c0 < a.cols; c0 += kWave) {
+    const int64_t c = c0 + lane;
+    int64_t t = -1;
+    bool keep = false;
+    if (c < a.cols) {
+      t = load_index(a.topk, a.topk64, r * a.cols + c) + beg + drop;
+      keep = t >= beg && t < end;
+    }
+    const uint64_t mask = __ballot(keep);
+    if constexpr (EMIT) {
+      if (keep) store_index(out_index, a.topk64, at + __popcll(mask & ((uint64_t(1) << lane) - 1)), t);
+    }
+    at += __popcll(mask);
+  }
+  if constexpr (!EMIT) {
+    if (lane == 0) store_index(out_off, a.off64, r, at);
+  }
+}
+
 }  // namespace
 }  // namespace recis_hip
 
@@ -761,5 +811,54 @@ extern "C" int recis_feature_cross_emit(const int64_t* x_val, const void* x_off,
           off_is64, n_seg, nx, ny, x_rank, y_rank, y_count, out_offsets, out_val, static_cast<float*>(out_weight), g);
   }
   RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+extern "C" int recis_ragged_topk_index(const void* drop_num, int drop_is64, const void* offset, int off_is64,
+                                       int64_t src_rows, const void* topk, int topk_is64, const void* indicator,
+                                       int indicator_is64, int64_t rows, int64_t cols, void* out_index,
+                                       void* out_offsets, int64_t* total_dev, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(rows >= 0 && cols >= 0 && src_rows >= 0, "negative size");
+  RECIS_REQUIRE(out_offsets && total_dev, "NULL argument");
+  RECIS_REQUIRE(rows == 0 || (drop_num && offset && indicator), "NULL argument");
+  RECIS_REQUIRE(rows * cols == 0 || (topk && out_index), "NULL topk / out_index pointer");
+  TopkArgs a;
+  a.drop_num = drop_num; a.offset = offset; a.topk = topk; a.indicator = indicator;
+  a.drop64 = drop_is64; a.off64 = off_is64; a.topk64 = topk_is64; a.ind64 = indicator_is64;
+  a.rows = rows; a.cols = cols; a.src_rows = src_rows;
+  CutJobs j;
+  j.out_off[0] = out_offsets;
+  j.out_rows[0] = rows;
+  j.sums_base[0] = 0;
+  const int64_t nb = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  void* ws = nullptr;
+  int rc = get_workspace(stream, static_cast<size_t>(std::max<int64_t>(nb, 1)) * sizeof(int64_t), &ws);
+  if (rc != RECIS_OK) return rc;
+  int64_t* sums = static_cast<int64_t*>(ws);
+  const int64_t gw = (rows * kWave + kBlock - 1) / kBlock;
+  RECIS_REQUIRE(gw < (int64_t(1) << 31), "too many rows");
+  int* err = device_error_word(current_device());
+  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  if (nb > 0) {
+    RECIS_TIME_KERNEL("topk_index_kernel(count)", stream) {
+      topk_index_kernel<false><<<dim3(static_cast<unsigned>(gw)), dim3(kBlock), 0, stream>>>(a, out_offsets, nullptr, err);
+    }
+    RECIS_LAUNCH_CHECK();
+    length_block_sums_kernel<<<dim3(static_cast<unsigned>(nb)), dim3(kBlock), 0, stream>>>(out_offsets, off_is64, rows, sums);
+    RECIS_LAUNCH_CHECK();
+  }
+  cutoff_scan_blocks_kernel<<<dim3(1), dim3(kBlock), 0, stream>>>(j, off_is64, sums, total_dev, 0);
+  RECIS_LAUNCH_CHECK();
+  if (nb > 0) {
+    cutoff_offsets_kernel<<<dim3(static_cast<unsigned>(nb), 1), dim3(kBlock), 0, stream>>>(j, off_is64, sums);
+    RECIS_LAUNCH_CHECK();
+    if (cols > 0) {
+      RECIS_TIME_KERNEL("topk_index_kernel(emit)", stream) {
+        topk_index_kernel<true><<<dim3(static_cast<unsigned>(gw)), dim3(kBlock), 0, stream>>>(a, out_offsets, out_index, err);
+      }
+      RECIS_LAUNCH_CHECK();
+    }
+  }
   return RECIS_OK;
 }

@@ -59,3 +59,35 @@ def fused_ragged_cutoff_3D(values: List[torch.Tensor], offsets: List[List[torch.
 def feature_cross_ragged(x_value, x_offsets, y_value, y_offsets, x_weight=None, y_weight=None):
     """ragged_ops.py:445-540: (values, offsets, weights) of the per-segment cross of x and y."""
     return ops.feature_cross_ragged(x_value, x_offsets, x_weight, y_value, y_offsets, y_weight)
+
+
+def ragged_topk_index_cutoff(drop_num, pad_num, drop_side, pad_side, offset, topk_index, indicator):
+    """ragged_ops.py:719-787: indices into the values (and their offsets per row) of the elements
+    that ``topk_index`` picks out of rows truncated on the left by ``drop_num``."""
+    return ops.calc_ragged_index(drop_num, pad_num, drop_side, pad_side, offset, topk_index, indicator)
+
+
+def ragged_to_sparse(values: torch.Tensor, row_splits: List[torch.Tensor]):
+    """ragged_ops.py:52-100 / csrc/ops/ragged_to_sparse.cc:43-91: the ragged tensor as a coalesced
+    sparse COO tensor of shape [rows, longest row of level 0, ..., longest row of the last level];
+    coordinate k of a value is its position inside the row of level k - 1 that holds it. Works on
+    the device of the inputs (the reference has a CPU operator only)."""
+    if not row_splits:
+        raise RuntimeError("ragged_to_sparse: needs at least one level of offsets")
+    if any(o.dtype != row_splits[0].dtype or o.dtype not in (torch.int32, torch.int64) for o in row_splits):
+        raise RuntimeError("ragged_to_sparse: each offset_splits should be torch::kInt32 or torch::kInt64")
+    splits = [o.to(torch.int64) for o in row_splits]
+    n = int(splits[-1][-1].item()) if splits[-1].numel() else 0
+    shape = [splits[0].numel() - 1]
+    for o in splits:
+        shape.append(int((o[1:] - o[:-1]).max().item()) if o.numel() > 1 else 0)
+    coords = []
+    child = torch.arange(n, device=values.device, dtype=torch.int64)  # index among the rows of the level below
+    for o in reversed(splits):
+        parent = torch.searchsorted(o, child, right=True) - 1  # the row of this level that holds `child`
+        coords.append(child - o[parent])
+        child = parent
+    coords.append(child)
+    indices = torch.stack(coords[::-1]) if n else torch.empty((len(splits) + 1, 0), dtype=torch.int64,
+                                                              device=values.device)
+    return torch.sparse_coo_tensor(indices, values[:n], shape + list(values.shape[1:])).coalesce()

@@ -1077,3 +1077,36 @@ def feature_cross_ragged(x_value, x_offsets, x_weight, y_value, y_offsets, y_wei
                                          int(wdt == torch.float64), i64(n_seg), ptr(x_rank), ptr(y_rank),
                                          ptr(y_count), ptr(out_off), i64(n), ptr(out_val), ptr(out_w), sp))
     return out_val, out_off, out_w
+
+
+def calc_ragged_index(drop_num, pad_num, drop_side, pad_side, offset, topk_index, indicator):
+    """``torch.ops.recis.calc_ragged_index`` (calc_ragged_index.cc:93-131): indices into the
+    values of a ragged tensor selected by ``topk_index`` [rows, cols] (positions counted after a
+    left truncation by ``drop_num``), and their offsets per row. Only drop left / pad right is
+    implemented, as in the reference. Returns (value_index, offsets) on the device of the inputs."""
+    require_cuda(drop_num, offset, topk_index, indicator)
+    for t, what in ((drop_side, "drop_side"), (pad_side, "pad_side")):
+        if not torch.is_tensor(t) or t.dtype != torch.bool:
+            raise RuntimeError("drop_side and pad_side must be bool")
+    drop_left, pad_left = bool(drop_side.item()), bool(pad_side.item())
+    if not drop_left or pad_left:
+        raise RuntimeError("drop %s, pad %s is not supported yet" % ("left" if drop_left else "right",
+                                                                    "left" if pad_left else "right"))
+    if topk_index.dim() != 2:
+        raise RuntimeError("calc_ragged_index: topk_index must be [rows, cols]")
+    rows, cols = topk_index.shape
+    if indicator.numel() != rows:
+        raise RuntimeError("indicator==row_num;indicator.numel(): %d; row_num: %d" % (indicator.numel(), rows))
+    src_rows = offset.numel() - 1
+    if drop_num.numel() < src_rows:
+        raise RuntimeError("calc_ragged_index: drop_num is shorter than the rows of offset")
+    d, o, t, ind = _contig(drop_num), _contig(offset), _contig(topk_index), _contig(indicator)
+    kinds = [_index_kind(x, n) for x, n in ((d, "drop_num"), (o, "offset"), (t, "topk_index"), (ind, "indicator"))]
+    dev = t.device
+    out_index = torch.empty(max(rows * cols, 1), dtype=t.dtype, device=dev)
+    out_off = torch.empty(rows + 1, dtype=o.dtype, device=dev)
+    total = torch.empty(1, dtype=torch.int64, device=dev)
+    check(lib().recis_ragged_topk_index(ptr(d), kinds[0], ptr(o), kinds[1], i64(src_rows), ptr(t), kinds[2],
+                                        ptr(ind), kinds[3], i64(rows), i64(cols), ptr(out_index), ptr(out_off),
+                                        ptr(total), stream_ptr(dev)))
+    return out_index[: int(total.item())], out_off

@@ -80,6 +80,12 @@ class RaggedTensor:
 
         return ops.ragged_to_dense(self._values, self._offsets, default_value)
 
+    def to_sparse(self):
+        """Coalesced sparse COO tensor of the ragged values (tensor.py:296-309)."""
+        from ..nn.functional.ragged_ops import ragged_to_sparse
+
+        return ragged_to_sparse(self._values, self._offsets)
+
     @staticmethod
     def from_dense(dense: torch.Tensor):
         """Rows up to their last non-zero element (tensor.py:277-294)."""

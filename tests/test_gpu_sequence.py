@@ -232,3 +232,84 @@ def test_feature_cross_op_kat():
     out = FeatureCross()([x, y])
     assert out.values().tolist() == [-7808879811642834040, -4967483181219983279, 1752425377096056168]
     assert out.offsets()[-1].tolist() == [0, 1, 2, 3] and out.weight().tolist() == [1.0, 1.0, 1.0]
+
+
+# ------------------------------------------------------------------ top-k index selection
+def test_calc_ragged_index_reference_example():
+    # tests/ops/ragged_topk_index_cutoff_test.py:9-22
+    from recis_amd.nn.functional.ragged_ops import ragged_topk_index_cutoff
+    c = lambda t: t.cuda()
+    idx, off = ragged_topk_index_cutoff(c(torch.tensor([5, 0, 0])), c(torch.tensor([0, 0, 0])), torch.tensor(True),
+                                        torch.tensor(False), c(torch.tensor([0, 8, 10, 13], dtype=torch.int32)),
+                                        c(torch.tensor([[1, 2], [0, 2], [0, 1]])), c(torch.tensor([0, 1, 2])))
+    assert idx.tolist() == [6, 7, 8, 10, 11] and off.tolist() == [0, 2, 3, 5]
+    assert idx.dtype == torch.int64 and off.dtype == torch.int32
+    for drop_side, pad_side in ((True, True), (False, True), (False, False)):  # calc_ragged_index.cc:100-127
+        with pytest.raises(RuntimeError, match="not supported"):
+            ragged_topk_index_cutoff(c(torch.tensor([5, 0, 0])), None, torch.tensor(drop_side), torch.tensor(pad_side),
+                                     c(torch.tensor([0, 8, 10, 13])), c(torch.tensor([[1, 2]])), c(torch.tensor([0])))
+
+
+@pytest.mark.parametrize("off_dtype,topk_dtype,ind_dtype,drop_dtype",
+                         [(np.int32, np.int64, np.int64, np.int64), (np.int64, np.int32, np.int32, np.int32),
+                          (np.int32, np.int32, np.int64, np.int32), (np.int64, np.int64, np.int32, np.int64)])
+def test_calc_ragged_index_matches_oracle(rng, off_dtype, topk_dtype, ind_dtype, drop_dtype):
+    side = (torch.tensor(True), torch.tensor(False))
+    for src_rows, rows, cols, max_len in ((50, 70, 5, 9), (3000, 5000, 70, 100), (40, 0, 3, 5), (10, 30, 0, 5),
+                                          (200, 4100, 1, 3), (500, 300, 200, 150)):
+        offset = _ragged(rng, src_rows, max_len, off_dtype)
+        drop = rng.integers(0, max_len // 2 + 1, src_rows).astype(drop_dtype)
+        ind = rng.integers(0, src_rows, rows).astype(ind_dtype)
+        topk = rng.integers(-3, max_len + 3, (rows, cols)).astype(topk_dtype)
+        dev = lambda a: torch.from_numpy(a).cuda()
+        idx, off = ops.calc_ragged_index(dev(drop), None, *side, dev(offset), dev(topk), dev(ind))
+        e_idx, e_off = oracle.calc_ragged_index(drop, offset, topk, ind)
+        np.testing.assert_array_equal(off.cpu().numpy(), e_off)
+        np.testing.assert_array_equal(idx.cpu().numpy(), e_idx)
+        assert idx.cpu().numpy().dtype == topk_dtype and off.cpu().numpy().dtype == off_dtype
+    assert _lib.poll_device_errors() == 0
+
+
+def test_calc_ragged_index_on_a_sequence_batch(rng):
+    """Behaviour-sequence shape: 8192 sequences of up to 1000 elements cut to their last 200, top 50
+    picked per sequence. Every kept index lies inside its row's kept part, rows are in column order."""
+    rows, keep, k = 8192, 200, 50
+    lens = np.minimum(rng.lognormal(4.8, 0.9, rows).astype(np.int64) + 1, 1000)
+    offset = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    drop = np.maximum(lens - keep, 0)
+    topk = np.stack([rng.permutation(keep)[:k] for _ in range(rows)])
+    ind = np.arange(rows)
+    dev = lambda a: torch.from_numpy(a).cuda()
+    idx, off = ops.calc_ragged_index(dev(drop), None, torch.tensor(True), torch.tensor(False), dev(offset), dev(topk),
+                                     dev(ind))
+    e = topk + (offset[:-1].astype(np.int64) + drop)[:, None]
+    keep_mask = e < offset[1:, None]
+    np.testing.assert_array_equal(off.cpu().numpy(), np.concatenate([[0], np.cumsum(keep_mask.sum(1))]))
+    np.testing.assert_array_equal(idx.cpu().numpy(), e[keep_mask])
+    assert _lib.poll_device_errors() == 0
+
+
+def test_calc_ragged_index_flags_a_bad_indicator():
+    dev = lambda *v, dt=torch.int64: torch.tensor(v, dtype=dt).cuda()
+    idx, off = ops.calc_ragged_index(dev(0, 0), None, torch.tensor(True), torch.tensor(False), dev(0, 2, 4),
+                                     torch.tensor([[0, 1], [0, 1]]).cuda(), dev(1, 7))
+    assert idx.tolist() == [2, 3] and off.tolist() == [0, 2, 2]
+    assert _lib.poll_device_errors() != 0
+    assert _lib.poll_device_errors() == 0
+
+
+def test_ragged_to_sparse_on_device(rng):
+    from recis_amd.nn.functional.ragged_ops import ragged_to_sparse
+    from recis_amd.ragged.tensor import RaggedTensor
+    for levels in (1, 2):
+        offsets, n = [], 300
+        for _ in range(levels):
+            offsets.append(_ragged(rng, n, 4, np.int32))
+            n = int(offsets[-1][-1])
+        values = rng.integers(1, 1000, n)
+        sp = ragged_to_sparse(torch.from_numpy(values).cuda(), [torch.from_numpy(o).cuda() for o in offsets])
+        assert sp.is_cuda
+        np.testing.assert_array_equal(sp.indices().cpu().numpy(), oracle.ragged_to_sparse_indices(offsets))
+        np.testing.assert_array_equal(sp.to_dense().cpu().numpy(), oracle.ragged_to_dense(values, offsets, 0))
+        rt = RaggedTensor(torch.from_numpy(values).cuda(), [torch.from_numpy(o).cuda() for o in offsets])
+        assert torch.equal(rt.to_sparse().to_dense(), sp.to_dense())

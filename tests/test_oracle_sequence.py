@@ -142,3 +142,59 @@ def test_feature_cross_dedups_and_takes_first_weight():
     h = oracle.murmur_hash_64_words
     signed = lambda v: v - (1 << 64) if v >= 1 << 63 else v
     assert ids.tolist() == [signed(h([5, 1])), signed(h([7, 1])), signed(h([9, 4])), signed(h([9, 8]))]
+
+
+def test_calc_ragged_index_kat():
+    # tests/ops/ragged_topk_index_cutoff_test.py:9-22
+    idx, offs = oracle.calc_ragged_index(np.array([5, 0, 0]), np.array([0, 8, 10, 13], np.int32),
+                                         np.array([[1, 2], [0, 2], [0, 1]]), np.array([0, 1, 2]))
+    assert idx.tolist() == [6, 7, 8, 10, 11] and offs.tolist() == [0, 2, 3, 5]
+    assert idx.dtype == np.int64 and offs.dtype == np.int32
+
+
+def test_calc_ragged_index_against_masks(rng):
+    """Same selection written as whole-array masks: the kept entries of the [rows, cols] grid in
+    row-major order, counts per row as a cumulative sum."""
+    for _ in range(20):
+        src_rows, rows, cols = int(rng.integers(1, 9)), int(rng.integers(0, 12)), int(rng.integers(0, 7))
+        offset = np.concatenate([[0], np.cumsum(rng.integers(0, 9, src_rows))]).astype(np.int64)
+        drop = rng.integers(0, 5, src_rows)
+        ind = rng.integers(0, src_rows, rows)
+        topk = rng.integers(-2, 9, (rows, cols))
+        idx, offs = oracle.calc_ragged_index(drop, offset, topk, ind)
+        e = topk + (offset[ind] + drop[ind])[:, None]
+        keep = (e >= offset[ind][:, None]) & (e < offset[ind + 1][:, None])
+        assert idx.tolist() == e[keep].tolist()
+        assert offs.tolist() == np.concatenate([[0], np.cumsum(keep.sum(1))]).tolist()
+
+
+def test_ragged_to_sparse_indices_scatter_into_the_dense_form(rng):
+    """The coordinates place every value where ragged_to_dense (pinned by the reference's example)
+    puts it, and nowhere else."""
+    for levels in (1, 2, 3):
+        for _ in range(5):
+            offsets, n = [], int(rng.integers(1, 5))
+            for _ in range(levels):
+                o = np.concatenate([[0], np.cumsum(rng.integers(0, 4, n))]).astype(np.int32)
+                offsets.append(o)
+                n = int(o[-1])
+            values = rng.integers(1, 100, n).astype(np.int64)
+            dense = oracle.ragged_to_dense(values, offsets, 0)
+            idx = oracle.ragged_to_sparse_indices(offsets)
+            assert idx.shape == (levels + 1, n)
+            rebuilt = np.zeros_like(dense)
+            rebuilt[tuple(idx)] = values
+            assert np.array_equal(rebuilt, dense)
+
+
+def test_ragged_to_sparse_host_function_matches_the_coordinates(rng):
+    import torch
+    from recis_amd.nn.functional.ragged_ops import ragged_to_sparse
+    offsets = [np.array([0, 2, 5, 6], np.int32), np.array([0, 1, 3, 6, 8, 10, 11], np.int32)]
+    values = np.arange(1, 12, dtype=np.int64)
+    sp = ragged_to_sparse(torch.from_numpy(values), [torch.from_numpy(o) for o in offsets])
+    assert list(sp.shape) == [3, 3, 3]
+    assert np.array_equal(sp.indices().numpy(), oracle.ragged_to_sparse_indices(offsets))
+    assert np.array_equal(sp.to_dense().numpy(), oracle.ragged_to_dense(values, offsets, 0))
+    one = ragged_to_sparse(torch.from_numpy(values[:6]), [torch.from_numpy(offsets[0])])
+    assert one.indices().tolist() == [[0, 0, 1, 1, 1, 2], [0, 1, 0, 1, 2, 0]]
