@@ -91,3 +91,45 @@ def ragged_to_sparse(values: torch.Tensor, row_splits: List[torch.Tensor]):
     indices = torch.stack(coords[::-1]) if n else torch.empty((len(splits) + 1, 0), dtype=torch.int64,
                                                               device=values.device)
     return torch.sparse_coo_tensor(indices, values[:n], shape + list(values.shape[1:])).coalesce()
+
+
+class RaggedTile(torch.autograd.Function):
+    """ragged_ops.py:623-656: for several features at once, the first ``seq[f]`` rows
+    ``table[indices[...]]`` of every sample, zero padded; the backward adds the row gradients up."""
+
+    @staticmethod
+    def forward(ctx, batch: List[int], seq: List[int], indices: torch.Tensor, offset: torch.Tensor,
+                table: torch.Tensor):
+        out, batch_seq = ops.ragged_tile(batch, seq, indices, offset, table)
+        ctx.save_for_backward(indices, offset)
+        ctx.batch_seq = batch_seq
+        ctx.batch_info = (table.shape[0], len(batch), max(batch), min(seq))
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        indices, offset = ctx.saved_tensors
+        dx = ops.ragged_tile_back(ctx.batch_seq, ctx.batch_info, indices, offset, dy.contiguous())
+        return None, None, None, None, dx
+
+
+def check_para(batch: List[int], seq: List[int], indices: torch.Tensor, offset: torch.Tensor, table: torch.Tensor,
+               check_enable: bool):
+    """ragged_ops.py:694-714 (reads two values back when enabled)."""
+    if not check_enable:
+        return
+    assert len(batch) == len(seq)
+    assert indices.max().item() < table.shape[0]
+    assert offset[-1].item() <= len(indices)
+    assert indices.dtype in (torch.int, torch.long)
+    assert offset.dtype in (torch.int, torch.long)
+    assert table.dtype in (torch.float,)
+    assert indices.is_cuda and offset.is_cuda and table.is_cuda
+    assert table.is_contiguous()
+
+
+def ragged_tile(batch: List[int], seq: List[int], indices: torch.Tensor, offset: torch.Tensor, table: torch.Tensor,
+                check_enable: bool = False):
+    """ragged_ops.py:659-691."""
+    check_para(batch, seq, indices, offset, table, check_enable)
+    return RaggedTile.apply(batch, seq, indices, offset, table)
