@@ -13,7 +13,7 @@ import torch
 from torch import nn
 
 from .. import ops
-from ..ragged.tensor import RaggedTensor
+from ..ragged.tensor import RaggedPadInfo, RaggedTensor
 
 
 def _values(x):
@@ -24,6 +24,30 @@ def _with_values(x, values):
     if isinstance(x, RaggedTensor):
         return RaggedTensor(values, x.offsets(), x.weight(), x.dense_shape)
     return values
+
+
+class DataValueProcessor:
+    """The values an op works on, whatever container carries them, and the container rebuilt
+    around the op's result (op.py:22-84)."""
+
+    def __init__(self, data: Union[RaggedTensor, torch.Tensor]):
+        self._data = data
+
+    def get_input_value(self):
+        if isinstance(self._data, RaggedTensor):
+            return self._data.values()
+        if isinstance(self._data, torch.Tensor):
+            return self._data._values() if self._data.is_sparse else self._data
+        raise ValueError("Unsupported data type: %s" % type(self._data))
+
+    def get_output_value(self, result):
+        if isinstance(self._data, RaggedTensor):
+            return RaggedTensor(result, self._data.offsets(), self._data.weight(), self._data.dense_shape)
+        if isinstance(self._data, torch.Tensor):
+            if self._data.is_sparse:
+                return torch.sparse_coo_tensor(self._data._indices(), result, self._data.shape)
+            return result.reshape(self._data.shape)
+        raise ValueError("Unsupported data type: %s" % type(self._data))
 
 
 class _OP(nn.Module):
@@ -48,6 +72,20 @@ class SelectField(_OP):
 
     def _get_config(self):
         return {"name": self._name, "dtype": str(self._dtype), "dim": self._dim, "from_dict": self._from_dict}
+
+
+class SelectFields(_OP):
+    """Several fields at once, as a list (op.py:198-245)."""
+
+    def __init__(self, input_list: List[SelectField]):
+        super().__init__()
+        self.input_list = nn.ModuleList(input_list)
+
+    def forward(self, data):
+        return [op(data) for op in self.input_list]
+
+    def _get_config(self):
+        return {"input_hashes": [op.get_hash() for op in self.input_list]}
 
 
 class Mod(_OP):
@@ -195,11 +233,16 @@ def sequence_truncate(op_list, inputs):
         if n_dims == 2:
             out = ragged_ops.fused_ragged_cutoff_2D(vals, [inputs[i].offsets()[-1].cuda() for i in idx], keep, drop, pad)
             new_vals, new_offs = out[0], [[o] for o in out[1]]
+            pad_infos = [RaggedPadInfo(out[2][k], out[3][k], torch.tensor(drop[k]), torch.tensor(pad[k]))
+                         for k in range(len(idx))]
         else:
             new_vals, new_offs = ragged_ops.fused_ragged_cutoff_3D(
                 vals, [[o.cuda() for o in inputs[i].offsets()] for i in idx], keep, drop, pad)
+            pad_infos = None  # as in the reference, only the 2-D truncation records what it dropped
         for k, i in enumerate(idx):
             shape = list(inputs[i].dense_shape)
             shape[1] = op_list[i].seq_len
             results[i] = RaggedTensor(new_vals[k], new_offs[k], inputs[i].weight(), shape)
+            if pad_infos is not None:  # fused_op_impl.py:406-411
+                results[i].set_pad_info(pad_infos[k])
     return results

@@ -46,10 +46,18 @@ class HashtableHookFactory:
         self._filters.clear()
 
 
-class ReadOnlyHookImpl:
+class BaseAdmitHookImpl:
+    """Base of the admission hooks (hashtable_hook_impl.py:193-210)."""
+
+    def __init__(self, **kwargs) -> None:
+        pass
+
+
+class ReadOnlyHookImpl(BaseAdmitHookImpl):
     """Lookups under this hook return zero rows for unknown keys and admit nothing."""
 
     def __init__(self, ht: Any, **kwargs):
+        super().__init__(**kwargs)
         self._ht = ht._hashtable_impl
 
 

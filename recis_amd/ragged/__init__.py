@@ -1,1 +1,1 @@
-from .tensor import RaggedTensor  # noqa: F401
+from .tensor import RaggedPadInfo, RaggedTensor  # noqa: F401

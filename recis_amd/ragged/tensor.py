@@ -1,9 +1,21 @@
 """``RaggedTensor``: values + one offsets tensor per ragged dimension (+ optional
 per-value weight), the container of ``recis.ragged.tensor`` (tensor.py:41-541)
 reduced to what the embedding path reads."""
+from dataclasses import dataclass
 from typing import List, Optional, Union
 
 import torch
+
+
+@dataclass
+class RaggedPadInfo:
+    """What a truncation dropped and padded per row (tensor.py:8-38): the input of the top-k
+    index selection that follows a truncated sequence."""
+
+    drop_nums: List[torch.Tensor] = None
+    pad_nums: List[torch.Tensor] = None
+    drop_sides: torch.Tensor = None
+    pad_sides: torch.Tensor = None
 
 
 class RaggedTensor:
@@ -20,6 +32,13 @@ class RaggedTensor:
             # rows = outermost offsets, one trailing ragged dimension per offsets tensor
             dense_shape = tuple([self._offsets[0].numel() - 1] + [-1] * len(self._offsets))
         self._dense_shape = tuple(dense_shape)
+        self._pad_info = None
+
+    def pad_info(self):
+        return self._pad_info
+
+    def set_pad_info(self, pad_info: RaggedPadInfo):
+        self._pad_info = pad_info
 
     def values(self):
         return self._values

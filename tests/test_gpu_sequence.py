@@ -313,3 +313,40 @@ def test_ragged_to_sparse_on_device(rng):
         np.testing.assert_array_equal(sp.to_dense().cpu().numpy(), oracle.ragged_to_dense(values, offsets, 0))
         rt = RaggedTensor(torch.from_numpy(values).cuda(), [torch.from_numpy(o).cuda() for o in offsets])
         assert torch.equal(rt.to_sparse().to_dense(), sp.to_dense())
+
+
+def test_engine_cross_of_selected_fields_and_topk_after_truncation(rng):
+    """Two chains through the FeatureEngine: SelectFields -> FeatureCross, and a fused 2-D
+    SequenceTruncate whose recorded drop counts feed the top-k index selection
+    (fused_op_impl.py:406-411, ragged_ops.py:717-787)."""
+    from recis_amd.features import Feature, FeatureEngine, FeatureCross, SelectField, SelectFields, SequenceTruncate
+    from recis_amd.nn.functional.ragged_ops import ragged_topk_index_cutoff
+    from recis_amd.ragged import RaggedPadInfo, RaggedTensor
+
+    rows, keep = 300, 6
+    xo, yo, so = (_ragged(rng, rows, 12, np.int32) for _ in range(3))
+    xv, yv = rng.integers(0, 9, int(xo[-1])), rng.integers(0, 9, int(yo[-1]))
+    sv = rng.integers(0, 1 << 40, int(so[-1]))
+    dev = lambda a: torch.from_numpy(a).cuda()
+    data = {"x": RaggedTensor(dev(xv), dev(xo)), "y": RaggedTensor(dev(yv), dev(yo)), "s": RaggedTensor(dev(sv), dev(so))}
+    engine = FeatureEngine([
+        Feature("xy").add_op(SelectFields([SelectField("x"), SelectField("y")])).add_op(FeatureCross()),
+        Feature("s_cut").add_op(SelectField("s")).add_op(SequenceTruncate(seq_len=keep, check_length=False,
+                                                                          truncate=True, truncate_side="left")),
+    ])
+    out = engine(data)
+    ev, eo, _ = oracle.feature_cross_ragged(xv, xo, None, yv, yo, None)
+    np.testing.assert_array_equal(out["xy"].values().cpu().numpy(), ev)
+    np.testing.assert_array_equal(out["xy"].offsets()[-1].cpu().numpy(), eo)
+
+    cut = out["s_cut"]
+    info = cut.pad_info()
+    assert isinstance(info, RaggedPadInfo) and bool(info.drop_sides) and not bool(info.pad_sides)
+    lens = np.diff(so)
+    np.testing.assert_array_equal(info.drop_nums.cpu().numpy(), np.maximum(lens - keep, 0))
+    # positions 0..keep-1 of the truncated rows, as indices into the ORIGINAL values
+    topk = np.tile(np.arange(keep), (rows, 1))
+    idx, off = ragged_topk_index_cutoff(info.drop_nums, info.pad_nums, info.drop_sides, info.pad_sides, dev(so),
+                                        dev(topk), torch.arange(rows).cuda())
+    np.testing.assert_array_equal(off.cpu().numpy(), cut.offsets()[-1].cpu().numpy())
+    np.testing.assert_array_equal(sv[idx.cpu().numpy()], cut.values().cpu().numpy())
