@@ -207,7 +207,8 @@ class SequenceTruncate(_OP):
 
     def forward(self, x: RaggedTensor):
         if self.check_length:
-            assert x.dense_shape[1] <= self.seq_len, "sequence length must be less than %d" % self.seq_len
+            # x.shape resolves an unstated extent by reading the longest row back, as the reference does
+            assert x.shape[1] <= self.seq_len, "sequence length must be less than %d" % self.seq_len
         if not self.truncate:
             return None  # as the reference (op.py:489-507 has no other branch)
         return sequence_truncate([self], [x])[0]

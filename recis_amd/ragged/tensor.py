@@ -34,6 +34,7 @@ class RaggedTensor:
         self._dense_shape = tuple(dense_shape)
         self._pad_info = None
 
+    @property
     def pad_info(self):
         return self._pad_info
 
@@ -62,10 +63,58 @@ class RaggedTensor:
     def dense_shape(self):
         return self._dense_shape
 
-    def real_shape(self, start=0, end=None):
+    def set_dim_by_rank(self, dim, rank):
         shape = list(self._dense_shape)
-        shape[0] = self._offsets[0].numel() - 1
-        return tuple(shape[start:end])
+        shape[rank] = dim
+        self._dense_shape = tuple(shape)
+
+    def get_shape(self, dim):
+        """Extent of dimension ``dim``: the stated one, else the row count (dim 0) or the longest
+        row of that ragged level, which is read back from the device (tensor.py:205-227). The
+        reference resolves every unknown extent when the tensor is built; here that happens on
+        demand, so building a RaggedTensor never waits for the device."""
+        if self._dense_shape[dim] != -1:
+            return self._dense_shape[dim]
+        if dim < 0:
+            dim += len(self._dense_shape)
+        if dim == 0:
+            return self._offsets[0].numel() - 1
+        off = self._offsets[dim - 1]
+        if off.numel() < 2:
+            return 0
+        return int((off[1:] - off[:-1]).max().item())
+
+    def real_shape(self, start=0, end=None):
+        """Extents of dimensions [start, end) with unknown ones resolved (tensor.py:174-203)."""
+        n = len(self._dense_shape)
+        if end is None:
+            end = n
+        if end < 0:
+            end += n
+        return tuple(self.get_shape(i) for i in range(start, end))
+
+    @property
+    def max_length(self):
+        return self.get_shape(-1)
+
+    @property
+    def shape(self):
+        return self.real_shape()
+
+    def size(self):
+        return self.real_shape()
+
+    @staticmethod
+    def from_numpy(values, offsets):
+        import numpy as np
+
+        if isinstance(offsets, np.ndarray):
+            offsets = [offsets]
+        return RaggedTensor(torch.from_numpy(values), [torch.from_numpy(o) for o in offsets])
+
+    def pin_memory(self):
+        return RaggedTensor(self._values.pin_memory(), [o.pin_memory() for o in self._offsets],
+                            None if self._weight is None else self._weight.pin_memory(), self._dense_shape)
 
     @property
     def device(self):
@@ -90,6 +139,7 @@ class RaggedTensor:
         return RaggedTensor(self._values.clone(), [o.clone() for o in self._offsets],
                             None if self._weight is None else self._weight.clone(), self._dense_shape)
 
+    @property
     def dim(self):
         return len(self._dense_shape)
 
@@ -117,3 +167,8 @@ class RaggedTensor:
         return "RaggedTensor(values=%s, offsets=%s, weight=%s)" % (
             tuple(self._values.shape), [tuple(o.shape) for o in self._offsets],
             None if self._weight is None else tuple(self._weight.shape))
+
+    def __str__(self):
+        return ("RaggedTensor(\n  values=%s,\n  offsets=%s,\n  weight=%s,\n  dense_shape=%s,\n  dtype=%s,\n"
+                "  device=%s\n)" % (self._values, self._offsets, self._weight, self._dense_shape,
+                                    self._values.dtype, self._values.device))

@@ -340,7 +340,7 @@ def test_engine_cross_of_selected_fields_and_topk_after_truncation(rng):
     np.testing.assert_array_equal(out["xy"].offsets()[-1].cpu().numpy(), eo)
 
     cut = out["s_cut"]
-    info = cut.pad_info()
+    info = cut.pad_info
     assert isinstance(info, RaggedPadInfo) and bool(info.drop_sides) and not bool(info.pad_sides)
     lens = np.diff(so)
     np.testing.assert_array_equal(info.drop_nums.cpu().numpy(), np.maximum(lens - keep, 0))
@@ -350,3 +350,21 @@ def test_engine_cross_of_selected_fields_and_topk_after_truncation(rng):
                                         dev(topk), torch.arange(rows).cuda())
     np.testing.assert_array_equal(off.cpu().numpy(), cut.offsets()[-1].cpu().numpy())
     np.testing.assert_array_equal(sv[idx.cpu().numpy()], cut.values().cpu().numpy())
+
+
+def test_ragged_tensor_shape_accessors():
+    from recis_amd.ragged import RaggedTensor
+    rt = RaggedTensor(torch.arange(6), [torch.tensor([0, 2, 5, 6], dtype=torch.int32)]).cuda()
+    assert rt.dim == 2 and rt.dense_shape == (3, -1)
+    assert rt.shape == (3, 3) and rt.size() == (3, 3) and rt.max_length == 3 and rt.real_shape(0, -1) == (3,)
+    rt.set_dim_by_rank(8, 1)
+    assert rt.shape == (3, 8) and rt.get_shape(1) == 8
+    deep = RaggedTensor(torch.arange(11), [torch.tensor([0, 2, 5, 6]), torch.tensor([0, 1, 3, 6, 8, 10, 11])]).cuda()
+    assert deep.dim == 3 and deep.shape == (3, 3, 3) and deep.real_shape(0, -1) == (3, 3)
+    host = RaggedTensor.from_numpy(np.arange(6), np.array([0, 2, 5, 6], np.int32))
+    assert host.values().tolist() == list(range(6)) and host.pin_memory().values().is_pinned()
+    assert "dense_shape=(3, -1)" in str(host)
+    from recis_amd.features import SequenceTruncate
+    with pytest.raises(AssertionError, match="sequence length"):
+        SequenceTruncate(seq_len=2, check_length=True)(RaggedTensor(
+            torch.arange(6).cuda(), [torch.tensor([0, 2, 5, 6], dtype=torch.int32).cuda()]))
