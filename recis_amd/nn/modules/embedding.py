@@ -18,6 +18,41 @@ from ..initializers import ConstantInitializer, Initializer
 from .hashtable import (GradIDMeanFunction, HashTable, HashTableLookupHelpFunction, gen_slice)
 
 
+class _Done:
+    """Stands where the reference keeps the handle of an asynchronous all-to-all: with one GPU
+    there is nothing to wait for."""
+
+    def wait(self):
+        return None
+
+
+@dataclass
+class ExchangeIDsResults:
+    """embedding.py:121-140, for one GPU: ``ids`` are the distinct ids of the batch (what the
+    reference receives from its peers), ``parts`` / ``parts_reverse`` their count, ``plan`` the
+    batch plan the later stages reuse."""
+
+    ids: torch.Tensor
+    ids_await: object
+    parts: List[int]
+    parts_reverse: List[int]
+    reverse_index: torch.Tensor
+    offsets: torch.Tensor
+    plan: object = None
+
+
+@dataclass
+class ExchangeEmbResults:
+    """embedding.py:142-158."""
+
+    emb: torch.Tensor
+    reverse_index: torch.Tensor
+    emb_shape: List[int]
+    offsets: torch.Tensor
+    emb_await: Optional[object] = None
+    plan: object = None
+
+
 @dataclass
 class EmbeddingOption:
     embedding_dim: int = 16
@@ -222,6 +257,38 @@ class DynamicEmbedding(torch.nn.Module):
         if opt.combiner == "tile":
             return out.view(tuple(shape) + (opt.combiner_kwargs["tile_len"] * opt.embedding_dim,))
         return out.view(tuple(shape) + (opt.embedding_dim,))
+
+    # The staged form of forward (embedding.py:498-624), which EmbeddingEngine-style callers drive
+    # stage by stage. With one GPU the two all-to-alls are the identity: exchange_ids is the dedup,
+    # lookup_exchange_emb the table lookup of the distinct ids, emb_reduce the pooling. forward()
+    # above fuses the last two (pooling reads the table rows directly).
+    def exchange_ids(self, ids: torch.Tensor, offsets: torch.Tensor):
+        plan = ops.ids_unique_plan(ids, wait=True)
+        n = int(plan.U)
+        return ExchangeIDsResults(ids=plan.unique, ids_await=_Done(), parts=[n], parts_reverse=[n],
+                                  reverse_index=plan.inverse, offsets=offsets, plan=plan)
+
+    def lookup_exchange_emb(self, ids_exchange_result: ExchangeIDsResults, admit_hook=None):
+        ids_exchange_result.ids_await.wait()
+        emb = lookup_unique_rows(self._hashtable, ids_exchange_result.ids, admit_hook, self._emb_opt.trainable)
+        return ExchangeEmbResults(emb=emb, emb_await=_Done(), reverse_index=ids_exchange_result.reverse_index,
+                                  emb_shape=list(emb.shape), offsets=ids_exchange_result.offsets,
+                                  plan=ids_exchange_result.plan)
+
+    def wait_exchange_emb(self, emb_exchange_result: ExchangeEmbResults):
+        emb_exchange_result.emb_await.wait()
+        return emb_exchange_result.emb.view(emb_exchange_result.emb_shape)
+
+    def emb_reduce(self, emb_exchange_result: ExchangeEmbResults, weight, combiner, combiner_kwargs,
+                   fp16_enable=False):
+        emb = self.wait_exchange_emb(emb_exchange_result)
+        if emb.dtype in (torch.int8,):
+            emb = emb.to(torch.float16 if fp16_enable else torch.float32)
+        if weight is not None and weight.dtype != emb.dtype:
+            weight = weight.to(emb.dtype)
+        return ragged_embedding_segment_reduce(emb, weight, emb_exchange_result.reverse_index,
+                                               emb_exchange_result.offsets, combiner, combiner_kwargs,
+                                               plan=emb_exchange_result.plan)
 
     @property
     def hashtable(self):

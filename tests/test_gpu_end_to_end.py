@@ -349,6 +349,44 @@ def test_dynamic_embedding_tile_and_max():
     torch.testing.assert_close(out2[2].detach(), rows2[[4, 0]].max(0)[0])
 
 
+def test_dynamic_embedding_staged_calls_match_forward():
+    """exchange_ids -> lookup_exchange_emb -> emb_reduce (embedding.py:498-624), driven by hand as
+    the reference's engine does, gives what forward() gives, values and accumulated gradients."""
+    rng = np.random.default_rng(5)
+    lens = rng.integers(0, 12, 200)
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)])).cuda()
+    ids = torch.from_numpy(rng.integers(0, 150, int(off[-1]))).cuda()
+    w = torch.from_numpy(rng.random(int(off[-1])).astype(np.float32)).cuda()
+    for combiner in ("sum", "mean"):
+        embs = []
+        for name in ("fused", "staged"):
+            opt = EmbeddingOption(embedding_dim=8, shared_name="%s_%s" % (name, combiner), combiner=combiner,
+                                  block_size=64, initializer=ConstantInitializer(0.5))
+            e = DynamicEmbedding(opt)
+            e.train()
+            embs.append(e)
+        fused, staged = embs
+        out_f = fused(RaggedTensor(ids, off, w))
+        ex = staged.exchange_ids(ids, off)
+        assert ex.parts == ex.parts_reverse == [int(torch.unique(ids).numel())]
+        assert torch.equal(ex.ids[ex.reverse_index.long()], ids)
+        looked = staged.lookup_exchange_emb(ex, None)
+        assert looked.emb_shape == [ex.parts[0], 8] and staged.wait_exchange_emb(looked).shape == (ex.parts[0], 8)
+        out_s = staged.emb_reduce(looked, w, combiner, {})
+        torch.testing.assert_close(out_s, out_f, rtol=1e-5, atol=1e-6)
+        g = torch.from_numpy(rng.standard_normal(tuple(out_f.shape)).astype(np.float32)).cuda()
+        out_f.backward(g)
+        out_s.backward(g)
+        grads = []
+        for e in (fused, staged):
+            impl = e.hashtable._hashtable_impl
+            index, rows = impl.grad_pairs(1)
+            key_of_row = dict(zip(*[t.cpu().tolist() for t in impl.ids_map()][::-1]))
+            order = np.argsort([key_of_row[r] for r in index.cpu().tolist()])
+            grads.append(rows.cpu().numpy()[order])
+        np.testing.assert_allclose(grads[1], grads[0], rtol=1e-5, atol=1e-5)
+
+
 def test_feature_engine_ops_and_fusion():
     """Restated from tests/feature_engine/op_test.py:17-36,95-131 and feature_engine_test.py: Mod,
     Bucketize, IDMultiHash, Hash known answers, through the fused engine path."""
