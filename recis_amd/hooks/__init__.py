@@ -1,1 +1,2 @@
 from .filter_hook import HashTableFilterHook  # noqa: F401
+from .hook import Hook  # noqa: F401

@@ -4,9 +4,10 @@ every filter's step after each training step and runs the eviction every
 import torch
 
 from ..nn.modules.hashtable_hook_impl import HashtableHookFactory
+from .hook import Hook
 
 
-class HashTableFilterHook:
+class HashTableFilterHook(Hook):
     def __init__(self, filter_interval: int = 100):
         self.filter_interval = filter_interval
         self.ht_filters = HashtableHookFactory().get_filters()
