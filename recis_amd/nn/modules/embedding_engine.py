@@ -50,6 +50,9 @@ class EmbeddingEngine(torch.nn.Module):
             if opt.shared_name not in grp.children:
                 grp.children.append(opt.shared_name)
             grp.features[name] = opt
+        # per feature: the key of its runtime group (features of a table that are pooled together)
+        self._runtime_key = {name: opt.runtime_info() for name, opt in self._emb_options.items()}
+        self._offsets_cache = {}  # offsets of dense id tensors, which depend on their shape only
         self._tables = torch.nn.ModuleDict()
         for gkey, grp in self._groups.items():
             opt = grp.opt
@@ -65,11 +68,20 @@ class EmbeddingEngine(torch.nn.Module):
     def hashtables(self):
         return {t._name: t for t in self._tables.values()}
 
-    @staticmethod
-    def _format(name, opt, data):
+    def _dense_offsets(self, key, build):
+        """Offsets that follow from shapes alone (dense id tensors), built once per shape."""
+        hit = self._offsets_cache.get(key)
+        if hit is None:
+            if len(self._offsets_cache) >= 256:
+                self._offsets_cache.clear()
+            hit = self._offsets_cache[key] = build()
+        return hit
+
+    def _format(self, name, opt, data):
         """(values int64 [N], weight | None, offsets int32 [S+1], output shape prefix, whether the
-        offsets are 0, 1, 2, ... by construction)."""
+        offsets are 0, 1, 2, ... by construction, the (rows, width) of a dense id tensor | None)."""
         unit = False
+        dense = None
         if isinstance(data, RaggedTensor):
             values = data.values()
             offsets = data.offsets()[-1]
@@ -86,7 +98,9 @@ class EmbeddingEngine(torch.nn.Module):
             values = data.reshape(-1)
             width = data.shape[-1]
             rows = values.numel() // width
-            offsets = torch.arange(rows + 1, device=data.device, dtype=torch.int32) * width
+            dense = (rows, width)
+            offsets = self._dense_offsets((rows, width, data.device), lambda: torch.arange(
+                rows + 1, device=data.device, dtype=torch.int32) * width)
             weight = None
             shape = tuple(data.shape[:-1])
             unit = width == 1
@@ -94,7 +108,7 @@ class EmbeddingEngine(torch.nn.Module):
             raise TypeError("feature %s: expected RaggedTensor or Tensor, got %s" % (name, type(data)))
         if values.dtype != torch.int64:
             values = values.long()
-        return values, weight, offsets.to(torch.int32), shape, unit
+        return values, weight, offsets.to(torch.int32), shape, unit, dense
 
     def forward(self, inputs: Dict[str, Union[torch.Tensor, RaggedTensor]]):
         outputs = {}
@@ -105,18 +119,20 @@ class EmbeddingEngine(torch.nn.Module):
             runtime = OrderedDict()
             for name, opt in grp.features.items():
                 if name in inputs:
-                    runtime.setdefault(opt.runtime_info(), []).append(name)
+                    runtime.setdefault(self._runtime_key[name], []).append(name)
             for names in runtime.values():
                 opt0 = grp.features[names[0]]
-                vals, weights, offs, shapes, tags = [], [], [], [], []
+                vals, weights, offs, shapes, tags, dense = [], [], [], [], [], []
                 all_unit = True
+                any_weight = opt0.use_weight and any(
+                    isinstance(inputs[n], RaggedTensor) and inputs[n].weight() is not None for n in names)
                 for name in names:
-                    v, w, o, shape, unit = self._format(name, grp.features[name], inputs[name])
+                    v, w, o, shape, unit, d = self._format(name, grp.features[name], inputs[name])
                     all_unit = all_unit and unit
+                    dense.append(d)
                     vals.append(v.to(dev))
                     offs.append(o.to(dev))
-                    if w is None and opt0.use_weight and any(
-                            isinstance(inputs[n], RaggedTensor) and inputs[n].weight() is not None for n in names):
+                    if w is None and any_weight:
                         w = torch.ones(v.numel(), device=dev)
                     weights.append(None if w is None else w.to(dev))
                     shapes.append(shape)
@@ -125,7 +141,13 @@ class EmbeddingEngine(torch.nn.Module):
                     ids = ops.ids_encode(vals, tags)
                 else:
                     ids = vals[0] if len(vals) == 1 else torch.cat(vals)
-                offsets = offs[0] if len(offs) == 1 else ops.merge_offsets(offs, [v.numel() for v in vals])
+                if len(offs) == 1:
+                    offsets = offs[0]
+                elif all(d is not None for d in dense):  # dense id tensors only: a function of the shapes
+                    offsets = self._dense_offsets((tuple(dense), dev), lambda: ops.merge_offsets(
+                        offs, [v.numel() for v in vals]))
+                else:
+                    offsets = ops.merge_offsets(offs, [v.numel() for v in vals])
                 weight = None
                 if all(w is not None for w in weights):
                     weight = weights[0] if len(weights) == 1 else torch.cat(weights)
