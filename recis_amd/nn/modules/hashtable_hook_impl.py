@@ -97,7 +97,6 @@ class GlobalStepFilterHookImpl(BaseFilterHookImpl):
         self.register_buffer("_global_step", torch.tensor([0], dtype=torch.int64, device=ht.device))
         assert filter_step > 0, "GlobalStepFilterHookImpl: filter_step must > 0, but get %s" % filter_step
         self._filter_step = filter_step
-        self._step_host = 0  # host copy of the counter: no read-back on the hot path
         self._ht.append_step_filter_slot(self._name, 0)
 
     def update(self, index: torch.Tensor) -> None:
@@ -106,21 +105,24 @@ class GlobalStepFilterHookImpl(BaseFilterHookImpl):
     def update_step(self, step_size: int = 1) -> None:
         with torch.no_grad():
             self._global_step += step_size
-        self._step_host += step_size
+
+    def _threshold(self) -> int:
+        # the counter lives on the device (it is part of the checkpoint and may be loaded or reset
+        # behind this object's back); it is read back only here, when a sweep runs
+        return int(self._global_step.item()) - self._filter_step
 
     def do_filter(self) -> None:
         # one pass over the id map instead of snapshot + filter + delete
-        self._ht.evict_older(self._name, self._step_host - self._filter_step)
+        self._ht.evict_older(self._name, self._threshold())
 
     def filter(self, ids, index):
         slot = self._ht.get_slot(self._name)
         chunks, chunk_rows = slot.kernel_blocks()
-        mask = ops.block_filter(index, chunks, chunk_rows, self._step_host - self._filter_step)
+        mask = ops.block_filter(index, chunks, chunk_rows, self._threshold())
         return torch.masked_select(ids, mask), torch.masked_select(index, mask)
 
     def __str__(self) -> str:
-        return "GlobalStepFilterHookImpl(global_step=%d, filter_step=%d, slot_name=%r)" % (
-            self._step_host, self._filter_step, self._name)
+        return "GlobalStepFilterHookImpl(filter_step=%d, slot_name=%r)" % (self._filter_step, self._name)
 
 
 HashtableHookFactory().regist_admit("ReadOnly", ReadOnlyHookImpl)
