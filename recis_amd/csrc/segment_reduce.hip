@@ -38,6 +38,7 @@ struct SegArgs {
   int wdt, rev64, off64;
   int lpr_log2, team_log2;
   int mean;
+  int nt_out;  // output larger than the caches can hold: write it with non-temporal stores
   int* err;
   // rows addressed through a table instead of a dense [U, D] array (BLK kernels): row u is row
   // row_index[u] of the block list (blocks of block_rows rows); a negative row_index reads as zeros
@@ -400,7 +401,7 @@ seg_max_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out,
 }
 
 // MAX forward with the memory behaviour of seg_pool_fwd_fast_kernel (indices by one coalesced
-// load + shuffles, four row loads in flight per lane). Requires U < 2^31.
+// load + shuffles, four row loads in flight per lane). Requires U < 2^31 and B < 2^31.
 template <typename TIn, typename TOut, int VEC, int KIND>
 __global__ void __launch_bounds__(kBlock)
 seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int32_t* __restrict__ argmax,
@@ -426,9 +427,19 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
   for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
     const int c0 = cbase + cl * VEC;
     const bool col_ok = c0 < D;
-    uint64_t key[VEC];
+    // Inside a lane the occurrences come in ascending order, so a strict float comparison keeps
+    // the first of equal values (-0 == +0) and costs less than building a key per element. The
+    // running best starts as NaN so that the first row always wins; the first NaN of the data
+    // wins over every number and is kept from then on.
+    float best_v[VEC];
+    int32_t best_r[VEC];
+    bool nan_seen[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) key[j] = 0;
+    for (int j = 0; j < VEC; ++j) {
+      best_v[j] = __uint_as_float(0x7FC00000u);
+      best_r[j] = -1;
+      nan_seen[j] = false;
+    }
     for (int64_t base = start; base < end; base += team) {
       const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
       int32_t mine = -1;  // row of occurrence base + lane_t
@@ -460,15 +471,21 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           if (!have[k]) continue;
-          const int64_t r = base + q0 + rg + k * step;
+          const int32_t r = static_cast<int32_t>(base) + q0 + rg + k * step;
 #pragma unroll
           for (int j = 0; j < VEC; ++j) {
-            const uint64_t kk = max_key(v[k][j], r);
-            key[j] = kk > key[j] ? kk : key[j];
+            const float x = v[k][j];
+            const bool take = !(x <= best_v[j]) && !nan_seen[j];
+            nan_seen[j] = nan_seen[j] || (x != x);
+            best_v[j] = take ? x : best_v[j];
+            best_r[j] = take ? r : best_r[j];
           }
         }
       }
     }
+    uint64_t key[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) key[j] = best_r[j] >= 0 ? max_key(best_v[j], best_r[j]) : 0;
     for (int off = 1 << a.lpr_log2; off < team; off <<= 1) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
@@ -617,10 +634,11 @@ seg_pool_bwd_fast_kernel(const TG* __restrict__ grad_out, TOut* __restrict__ gra
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           if (id[k] >= 0) {
-            if constexpr (KIND == kFastPlain) {
-              store_pack_stream<TOut, VEC>(grad_unique + static_cast<int64_t>(id[k]) * D + c0, g);
+            TOut* dst = grad_unique + static_cast<int64_t>(id[k]) * D + c0;
+            if (KIND == kFastPlain || a.nt_out) {
+              store_pack_stream<TOut, VEC>(dst, g);
             } else {
-              store_pack<TOut, VEC>(grad_unique + static_cast<int64_t>(id[k]) * D + c0, g);
+              store_pack<TOut, VEC>(dst, g);  // a small gradient is read again by the next kernel
             }
           }
         }
@@ -814,7 +832,12 @@ seg_max_bwd_rows_kernel(const TG* __restrict__ grad_out, const int32_t* __restri
           float v[VEC];
 #pragma unroll
           for (int j = 0; j < VEC; ++j) v[j] = win[j] == r ? g[j] : 0.f;
-          store_pack<TOut, VEC>(grad_unique + static_cast<int64_t>(id[k]) * D + c0, v);
+          TOut* dst = grad_unique + static_cast<int64_t>(id[k]) * D + c0;
+          if (a.nt_out) {
+            store_pack_stream<TOut, VEC>(dst, v);
+          } else {
+            store_pack<TOut, VEC>(dst, v);
+          }
         }
       }
     }
@@ -953,6 +976,7 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
   a.lpr_log2 = geom.lpr_log2;
   a.team_log2 = pick_team_log2(B, S, geom.lpr_log2);
   a.mean = (mode == RECIS_MEAN);
+  a.nt_out = 0;
   a.err = err;
   a.row_index = blk ? blk->row_index : nullptr;
   a.blocks = blk ? blk->blocks : nullptr;
@@ -997,7 +1021,7 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
             const TIn* e = static_cast<const TIn*>(unique_emb);
             TOut* o = static_cast<TOut*>(out);
             RECIS_TIME_KERNEL("seg_max_fwd_kernel", stream)
-            if (U >= (int64_t(1) << 31))
+            if (U >= (int64_t(1) << 31) || B >= (int64_t(1) << 31))
               seg_max_fwd_kernel<TIn, TOut, VEC><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, argmax_out, a);
             else if (a.rev == nullptr)
               seg_max_fwd_fast_kernel<TIn, TOut, VEC, kFastPlain><<<dim3(grid), dim3(kBlock), 0, stream>>>(e, o, argmax_out, a);
@@ -1110,6 +1134,8 @@ extern "C" int recis_segment_reduce_backward(
   a.lpr_log2 = lpr_log2;
   a.team_log2 = pick_team_log2(B, S, lpr_log2);
   a.mean = (mode == RECIS_MEAN);
+  // 1 GiB is far past what L2 and the 256 MB memory-side cache keep for the next kernel
+  a.nt_out = U * D * out_sz >= (int64_t(1) << 30);
   a.err = err;
 
   // Rows no occurrence maps to must read zero. With a promised bijection

@@ -11,7 +11,7 @@ import torch
 
 import oracle
 from conftest import ragged_offsets
-from recis_amd import ops
+from recis_amd import _lib, ops
 
 pytestmark = pytest.mark.gpu
 
@@ -141,6 +141,28 @@ def test_max_forward_backward(rng, D):
     got = ops.segment_reduce_backward(_dev(g), None, _dev(rev), _dev(off), U, "max", argmax=arg)
     exp = oracle.segment_max_backward(g, ea, rev, U)
     np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("with_rev", [True, False])
+def test_max_special_values(rng, with_rev):
+    """NaN beats every number and the first NaN is kept, -inf alone still yields its occurrence,
+    -0 and +0 tie (first occurrence), +inf wins; segments long enough for several rounds per lane."""
+    S, D = 300, 16
+    off = ragged_offsets(rng, S, 0, 150, empty_frac=0.1)
+    B = int(off[-1])
+    U = B if not with_rev else 500
+    emb = np.round(rng.standard_normal((U, D)) * 2).astype(np.float32)
+    special = np.array([np.nan, np.inf, -np.inf, -0.0, 0.0], np.float32)
+    mask = rng.random((U, D)) < 0.15
+    emb[mask] = special[rng.integers(0, special.size, int(mask.sum()))]
+    emb[: U // 4] = -np.inf                                   # whole rows of -inf
+    rev = rng.integers(0, U, size=B) if with_rev else None
+    out, arg = ops.segment_reduce_forward(_dev(emb), None, None if rev is None else _dev(rev), _dev(off), "max",
+                                          return_argmax=True)
+    eo, ea = oracle.segment_max_forward(emb, np.arange(B) if rev is None else rev, off)
+    np.testing.assert_array_equal(arg.cpu().numpy(), ea)
+    np.testing.assert_array_equal(out.cpu().numpy(), eo)
+    assert _lib.poll_device_errors() == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
