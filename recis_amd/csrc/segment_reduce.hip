@@ -39,6 +39,7 @@ struct SegArgs {
   int lpr_log2, team_log2;
   int mean;
   int nt_out;  // output larger than the caches can hold: write it with non-temporal stores
+  int nt_in;   // likewise for the rows read
   int* err;
   // rows addressed through a table instead of a dense [U, D] array (BLK kernels): row u is row
   // row_index[u] of the block list (blocks of block_rows rows); a negative row_index reads as zeros
@@ -281,8 +282,8 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
           }
           if (src >= n_here || !col_ok) row = nullptr;
           if (row) {
-            if constexpr (KIND == kFastPlain && !BLK) {
-              load_pack_stream<TIn, VEC>(row + c0, v[k]);  // read once
+            if ((KIND == kFastPlain && !BLK) || a.nt_in) {
+              load_pack_stream<TIn, VEC>(row + c0, v[k]);  // read once, or too large to stay cached
             } else {
               load_pack<TIn, VEC>(row + c0, v[k]);
             }
@@ -466,7 +467,13 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
           const int src = q0 + rg + k * step;
           const int32_t id = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
           have[k] = src < n_here && col_ok && id >= 0;
-          if (have[k]) load_pack<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
+          if (have[k]) {
+            if (KIND == kFastPlain || a.nt_in) {
+              load_pack_stream<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
+            } else {
+              load_pack<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
+            }
+          }
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -977,6 +984,7 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
   a.team_log2 = pick_team_log2(B, S, geom.lpr_log2);
   a.mean = (mode == RECIS_MEAN);
   a.nt_out = 0;
+  a.nt_in = !blk && U * D * static_cast<int64_t>(dtype_size(emb_dtype)) >= (int64_t(1) << 30);
   a.err = err;
   a.row_index = blk ? blk->row_index : nullptr;
   a.blocks = blk ? blk->blocks : nullptr;
@@ -1136,6 +1144,7 @@ extern "C" int recis_segment_reduce_backward(
   a.mean = (mode == RECIS_MEAN);
   // 1 GiB is far past what L2 and the 256 MB memory-side cache keep for the next kernel
   a.nt_out = U * D * out_sz >= (int64_t(1) << 30);
+  a.nt_in = 0;
   a.err = err;
 
   // Rows no occurrence maps to must read zero. With a promised bijection
