@@ -147,13 +147,19 @@ class Config4:
 
     name = "c4_ctr_merged_table_39x65536_d16_fp32_adam"
 
-    def __init__(self, batch=65536):
+    def __init__(self, batch=65536, n_batches=8):
         from recis_amd import ops
         from recis_amd.nn.initializers import NormalInitializer
         from recis_amd.nn.modules.hashtable import HashtableImpl
         from recis_amd.optim.sparse_impl import SparseAdamImpl
         self.ops = ops
-        c = workloads.config4(batch=batch)
+        # the steps rotate over n_batches batches of the same fields, so that the table holds several
+        # batches' worth of rows and a step touches a scattered part of it (one batch replayed would
+        # keep the whole table in the caches)
+        self.batches = [workloads.config4(batch=batch)] + [
+            workloads.config4(batch=batch, data_seed=k) for k in range(1, n_batches)]
+        self._turn = 0
+        c = self.batches[0]
         self.c = c
         self.D = 16
         self.n_feat = len(c["sparse"]) + len(c["dense"])
@@ -164,7 +170,7 @@ class Config4:
         init.set_dtype(torch.float32)
         self.table = HashtableImpl(10240, [self.D], torch.float32, torch.device("cuda"), True,
                                    ["f%d" % i for i in range(self.n_feat)], init.build().impl(),
-                                   reserve_rows=int(self.N * 1.05))
+                                   reserve_rows=int(self.N * 1.05) * n_batches)
         self.opt = SparseAdamImpl.make({"ctr": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0)
         self.tags = list(range(self.n_feat))
         self.offsets = torch.arange(self.N + 1, dtype=torch.int32, device="cuda")
@@ -172,6 +178,9 @@ class Config4:
         self.grad_out = torch.randn((self.N, self.D), device="cuda", generator=g)
         self.mods = [c["mod"]] * len(c["dense"])
         self.U = None
+        for _ in self.batches:  # admission of every batch's keys happens here, not in the timed steps
+            self.step()
+        torch.cuda.synchronize()
 
     # the stages, also timed one by one for the breakdown
     def feature_ops(self):
@@ -205,7 +214,12 @@ class Config4:
         self.opt.step()
         self.opt.zero_grad()
 
+    def next_batch(self):
+        self.c = self.batches[self._turn % len(self.batches)]
+        self._turn += 1
+
     def step(self):
+        self.next_batch()
         ids = self.feature_ops()
         uniq, inv = self.dedup(ids)
         index = self.lookup(uniq)
@@ -218,9 +232,11 @@ class Config4:
         """The same step with the raw inputs starting in pinned host memory (26 id columns and 13
         float columns, 24 MB): what a caller that hands over host buffers would see."""
         if not hasattr(self, "_host"):
-            self._host = ([t.cpu().pin_memory() for t in self.c["sparse"]], [t.cpu().pin_memory() for t in self.c["dense"]])
-            self._dev = (self.c["sparse"], self.c["dense"])
-        for dst, src in zip(self._dev[0] + self._dev[1], self._host[0] + self._host[1]):
+            self._host = [([t.cpu().pin_memory() for t in b["sparse"]], [t.cpu().pin_memory() for t in b["dense"]])
+                          for b in self.batches]
+        k = self._turn % len(self.batches)
+        b, host = self.batches[k], self._host[k]
+        for dst, src in zip(b["sparse"] + b["dense"], host[0] + host[1]):
             dst.copy_(src, non_blocking=True)
         return self.step()
 
@@ -499,10 +515,10 @@ class Config5:
 # scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC_C4 = {
-    "adamw_rows_kernel": 400839793, "csr_rows_kernel": 395465738, "csr_expand_kernel": 246127259,
-    "plan_emit_kernel": 149596294, "find_or_claim_kernel": 114443009, "plan_bucket_kernel": 89183328,
-    "plan_scatter_kernel": 77259166, "plan_tile_kernel": 58178389, "ids_encode_kernel": 40936481,
-    "plan_colscan_kernel": 16429764,
+    "adamw_rows_kernel": 433714773, "csr_rows_kernel": 395422130, "csr_expand_kernel": 256908532,
+    "plan_emit_kernel": 149225867, "find_or_claim_kernel": 131811016, "plan_bucket_kernel": 89186262,
+    "plan_scatter_kernel": 77270206, "plan_tile_kernel": 58181470, "ids_encode_kernel": 40935979,
+    "plan_colscan_kernel": 16429891,
 }
 
 

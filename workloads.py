@@ -75,12 +75,16 @@ def seeded_block(seed, block_index, block_size, dim, std=0.01):
     return (std * _rng([seed, 7919, block_index]).standard_normal((block_size, dim))).astype(np.float32)
 
 
-def config4(device="cuda", seed=4, batch=65536, n_sparse=26, n_dense=13, n_boundaries=64, mod=1_000_000):
+def config4(device="cuda", seed=4, batch=65536, n_sparse=26, n_dense=13, n_boundaries=64, mod=1_000_000,
+            data_seed=None):
     """Click-through-style merged table (benchmark config 4): 26 int64 id fields with log-uniform
     cardinalities in 10..1e7, 13 lognormal(0, 2) dense fields bucketized against 64 sorted
-    boundaries and taken mod 1e6; one id per field per sample."""
+    boundaries and taken mod 1e6; one id per field per sample. ``data_seed`` draws another batch
+    of the same fields (same cardinalities and boundaries)."""
     rng = _rng(seed)
     cards = np.floor(10 ** rng.uniform(1, 7, size=n_sparse)).astype(np.int64)
+    if data_seed is not None:
+        rng = np.random.Generator(np.random.PCG64([seed, data_seed]))
     sparse = [torch.from_numpy(rng.integers(0, c, size=batch, dtype=np.int64)).to(device) for c in cards]
     dense = [torch.from_numpy(rng.lognormal(0.0, 2.0, size=batch).astype(np.float32)).to(device)
              for _ in range(n_dense)]
