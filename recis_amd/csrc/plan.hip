@@ -576,6 +576,7 @@ struct CsrArgs {
   int D;
   int lpr_log2;
   int accumulate;
+  int nt_in;  // the gathered rows are too many to stay cached: non-temporal loads
   int* err;
   const void* cover;  // offsets [cover_S + 1] or NULL: entries whose src lies outside
   int cover64;        // [cover[0], cover[cover_S]) are skipped
@@ -633,7 +634,11 @@ __device__ __forceinline__ void wave_gather_range(const TIn* __restrict__ rows, 
         w[k] = a.coef ? __shfl(w_mine, from, kWave) : 1.0f;
         if (e >= n_here || !col_ok) id = -1;
         if (id >= 0) {
-          load_pack<TIn, VEC>(rows + static_cast<int64_t>(id) * a.D + c0, v[k]);
+          if (a.nt_in) {
+            load_pack_stream<TIn, VEC>(rows + static_cast<int64_t>(id) * a.D + c0, v[k]);
+          } else {
+            load_pack<TIn, VEC>(rows + static_cast<int64_t>(id) * a.D + c0, v[k]);
+          }
         } else {
           w[k] = 0.f;
 #pragma unroll
@@ -682,7 +687,11 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
       w = 0.f;
       return;
     }
-    load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
+    if (a.nt_in) {
+      load_pack_stream<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
+    } else {
+      load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
+    }
   };
   // acc += sum over list entries k = first, first + step, ... < last (4 gathers in flight)
   auto gather_sum = [&](int32_t first, int32_t last, int32_t step, int c0, float (&acc)[VEC]) {
@@ -1256,6 +1265,7 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   a.D = static_cast<int>(D);
   a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
   a.accumulate = accumulate;
+  a.nt_in = n_rows * D * in_sz >= (int64_t(1) << 30);
   a.err = device_error_word(current_device());
   RECIS_REQUIRE(a.err != nullptr, "could not allocate the device error word");
   const int rows_per_block = kBlock >> a.lpr_log2;
