@@ -907,7 +907,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
       src = rows + u * D;
     }
     if (src) {
-      load_pack<TIn, VEC>(src + c0, v);
+      load_pack_stream<TIn, VEC>(src + c0, v);  // every row is read once here
     } else {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) v[j] = 0.f;
