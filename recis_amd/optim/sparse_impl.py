@@ -95,9 +95,11 @@ class _AdamFamilyImpl(_SparseOptimizerImpl):
     def state_dict(self):
         steps = {}
         for st in self._state.values():
-            steps[self.prefix + "step"] = st["step"]
-            steps[self.prefix + "beta1"] = st["beta1"]
+            # in the order the reference's map hands them out (its state-dict test lists the keys:
+            # tests/hashtable/ht_state_dict_test.py:44-49)
             steps[self.prefix + "beta2"] = st["beta2"]
+            steps[self.prefix + "beta1"] = st["beta1"]
+            steps[self.prefix + "step"] = st["step"]
         return {}, steps
 
 

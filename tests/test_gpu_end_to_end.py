@@ -387,6 +387,43 @@ def test_dynamic_embedding_staged_calls_match_forward():
         np.testing.assert_allclose(grads[1], grads[0], rtol=1e-5, atol=1e-5)
 
 
+def test_three_tables_state_dict_keys():
+    """tests/hashtable/ht_state_dict_test.py:27-49: three tables of 3 * 2^20 + 200 rows each, two
+    training steps, then the keys a checkpoint of the model would hold, in the reference's order."""
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self._emb_one = HashTable([16], name="16")
+            self._emb_two = HashTable([32], name="32")
+            self._emb_three = HashTable([64], name="64")
+
+        def forward(self, ids):
+            return torch.concat([self._emb_one(ids), self._emb_two(ids), self._emb_three(ids)], dim=1).sum()
+
+    model = Model()
+    sparse_state = filter_out_sparse_param(model)
+    optim = SparseAdamWTF(sparse_state)
+    ids_num = (1 << 20) * 3 + 200
+    ids = torch.arange(ids_num, device="cuda")
+    for _ in range(2):
+        model(ids).backward()
+        optim.step()
+        optim.zero_grad()
+    save_dict = dict(sparse_state)
+    assert list(save_dict.keys()) == ["16", "32", "64"]
+    save_dict.update(optim.state_dict())
+    assert list(save_dict.keys()) == ["16", "32", "64", "sparse_adamw_tf_beta2", "sparse_adamw_tf_beta1",
+                                      "sparse_adamw_tf_step"]
+    for t, dim in ((model._emb_one, 16), (model._emb_two, 32), (model._emb_three, 64)):
+        assert t.ids().numel() == ids_num
+        rows = t.embeddings()[:ids_num]
+        assert rows.shape == (ids_num, dim)
+        # every row took two identical steps from the zero initial value: all rows are equal and moved
+        assert bool((rows == rows[0]).all()) and float(rows[0].abs().min()) > 0
+    # block_apply_adamw_op.cc:121 calls step.add(1) and drops the result: the stored step stays 0
+    assert int(optim.state_dict()["sparse_adamw_tf_step"]) == 0
+
+
 def test_feature_engine_ops_and_fusion():
     """Restated from tests/feature_engine/op_test.py:17-36,95-131 and feature_engine_test.py: Mod,
     Bucketize, IDMultiHash, Hash known answers, through the fused engine path."""
