@@ -414,6 +414,17 @@ class Config3:
         return N * (8 + 4) + U * 8 + U * (16 + 8) + int(0.1 * N) * 16 + U * D * 4 + N * (4 + D * 4) \
             + N * (4 + D * 4) + U * D * 4 * 7 + U * 8
 
+    def kernel_bytes(self):
+        """Algorithmic HBM bytes of one launch of each heavy kernel of the step (one row per lookup,
+        so the segments are the occurrences)."""
+        N, U, D = self.N, self.U, self.D
+        return {
+            "csr_expand_kernel": U * (8 + D * 4) + 4 * N + 4 * (U + 1) + N * D * 4,
+            "csr_rows_kernel": N * D * 4 + 4 * N + 4 * U + U * D * 4,
+            "adamw_rows_kernel": U * (8 + D * 4 * 7),
+            "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,
+        }
+
     def evict_sweep_ms(self, filter_step=50):
         """One eviction sweep over the 2e8-row table (keys not seen for `filter_step` steps): the
         one-pass library sweep. The threshold is set so that nothing is old enough: the sweep cost
@@ -509,6 +520,19 @@ class Config5:
     def algorithmic_bytes(self):
         N, U, S, D = self.N, self.U, self.S, self.D
         return 12 * N + U * (24 + 4 * D * 2) + S * (D * 4 + D * 4) + 2 * self.pad_rows * D * 2 + 8 * N
+
+    def kernel_bytes(self):
+        """Algorithmic HBM bytes per launch: the padded gather runs once per field, the
+        gather-reduce once over the pooled gradients (fp32 rows, re-read out of the caches: priced
+        at one read per segment) and once over the padded gradients (bf16 rows)."""
+        N, U, S, D = self.N, self.U, self.S, self.D
+        n_fields = len(self.fields)
+        return {
+            "tile_fwd_kernel": (self.pad_rows * D * 2 + 4 * N + U * D * 2) // n_fields,  # distinct rows once
+            "csr_rows_kernel": (S * D * 4 + N * D * 2 + 2 * (8 * N + 4 * U) + 3 * U * D * 4) // 2,
+            "seg_pool_fwd_kernel": U * D * 2 + 4 * N + 4 * (S + 1) + S * D * 4,
+            "adagrad_rows_kernel": U * (8 + D * 4 + 4 * D * 2),
+        }
 
     def cpu_baseline(self, budget_s):
         import oracle
@@ -622,6 +646,11 @@ def main():
         return
     classes = {"c4": Config4, "c2": Config2, "c3": Config3, "c5": Config5}
     main_wl = classes[args.workload]()
+    # part of set-up, before the W warm-up steps: the first steps of a process pay for the device
+    # allocations of the step's outputs (config 5: 2 GB blocks, tens of ms)
+    for _ in range(10):
+        main_wl.step()
+    torch.cuda.synchronize()
     for _ in range(args.warmup):
         main_wl.step()
     torch.cuda.synchronize()
@@ -711,8 +740,16 @@ def main():
     else:
         s = step_summary(main_wl, ms_per_step)
         out["config"]["unique_ids_per_step"] = main_wl.U
-        out["roofline"] = {"bound": "hbm", "kernel": "whole step", "achieved": s["gbs"], "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": s["frac"], "traffic": None}
+        kern = _kernel_profile(main_wl.step, max(5, args.steps))
+        kb = main_wl.kernel_bytes()
+        dom = max((k for k in kern if k in kb), key=lambda k: kern[k]["us"] * kern[k]["calls_per_step"])
+        ach = kb[dom] / kern[dom]["us"] / 1e3
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": ach / HBM_PEAK_GBS, "traffic": None, "launch_us": round(kern[dom]["us"], 2),
+                           "launches_per_step": kern[dom]["calls_per_step"], "algorithmic_bytes_per_launch": kb[dom]}
+        out["kernels_us"] = {k: round(v["us"], 2) for k, v in sorted(kern.items(), key=lambda kv: -kv[1]["us"])}
+        out["step_roofline"] = {"algorithmic_bytes": s["algorithmic_bytes"], "achieved": s["gbs"], "frac": s["frac"],
+                                "unit": "GB/s"}
         if args.workload == "c3":
             out["evict_sweep_ms"] = round(main_wl.evict_sweep_ms(), 3)
     if not args.no_extra:
