@@ -125,7 +125,7 @@ __global__ void __launch_bounds__(kBlock)
 find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __restrict__ ids,
                      int64_t n, const int64_t* __restrict__ n_dev, int64_t* __restrict__ out,
                      int64_t* __restrict__ slotpos, int32_t* __restrict__ block_counts,
-                     int64_t* __restrict__ state, int* err) {
+                     int64_t* __restrict__ state, int64_t seq, int* err) {
   n = counted(n, n_dev);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   bool is_new = false;
@@ -165,7 +165,7 @@ find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __r
             out[i] = v;
           } else {
             sp = -(static_cast<int64_t>(p) + 2);
-            atomicOr(reinterpret_cast<unsigned long long*>(&state[ST_DUPS]), 1ull);
+            st_relaxed(&state[ST_DUPS], seq);  // "this call has duplicates": every writer stores the same word
           }
           break;
         }
@@ -278,9 +278,9 @@ assign_rows_kernel(Slot* __restrict__ table, const int64_t* __restrict__ slotpos
 // Pass 4: occurrences whose key was claimed by another occurrence of the same call.
 __global__ void __launch_bounds__(kBlock)
 resolve_dups_kernel(const Slot* __restrict__ table, const int64_t* __restrict__ slotpos, int64_t n,
-                    const int64_t* __restrict__ n_dev, const int64_t* __restrict__ state,
+                    const int64_t* __restrict__ n_dev, const int64_t* __restrict__ state, int64_t seq,
                     int64_t* __restrict__ out) {
-  if (state[ST_DUPS] == 0) return;
+  if (state[ST_DUPS] != seq) return;  // the calls of a map are numbered 1, 2, ...: no reset between them
   n = counted(n, n_dev);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
   if (i >= n) return;
@@ -406,8 +406,6 @@ __global__ void erase_commit_kernel(int64_t* state, int64_t n) {
   state[ST_LIVE] -= state[ST_TMP];
   state[ST_TMP] = 0;
 }
-
-__global__ void reset_dups_kernel(int64_t* state) { state[ST_DUPS] = 0; }
 
 // retrieve_all: every live (key, row) pair, in no particular order.
 __global__ void __launch_bounds__(kBlock)
@@ -712,17 +710,16 @@ static int lookup_impl(recis_idmap* m, const int64_t* ids, int64_t n, const int6
   const uint64_t mask = static_cast<uint64_t>(m->capacity - 1);
   const int64_t seq = ++m->seq_issued;
 
-  reset_dups_kernel<<<1, 1, 0, stream>>>(m->state);
   RECIS_TIME_KERNEL("find_or_claim_kernel", stream)
   find_or_claim_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, mask, ids, n, n_dev, index_out, slotpos,
-                                                             block_counts, m->state, m->err);
+                                                             block_counts, m->state, seq, m->err);
   RECIS_LAUNCH_CHECK();
   scan_commit_kernel<<<1, 1024, 0, stream>>>(block_counts, nb, n, n_dev, m->state, m->mirror, seq);
   RECIS_LAUNCH_CHECK();
   assign_rows_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, n_dev, block_counts, m->state,
                                                            m->free_list, index_out);
   RECIS_LAUNCH_CHECK();
-  resolve_dups_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, n_dev, m->state, index_out);
+  resolve_dups_kernel<<<dim3(nb), dim3(kBlock), 0, stream>>>(m->table, slotpos, n, n_dev, m->state, seq, index_out);
   RECIS_LAUNCH_CHECK();
   m->in_flight.emplace_back(seq, n);
   return RECIS_OK;
