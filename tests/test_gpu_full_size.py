@@ -166,3 +166,20 @@ def test_config5_step_properties():
     exp = (wl.g_pool.double() * (lens > 0).view(-1, 1)).sum(0)
     torch.testing.assert_close(g.double().sum(0), exp, rtol=1e-5, atol=1e-2)
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("n,key_range", [(40_000_000, 30_000_000), (70_000_000, 1000)])
+def test_batch_plan_at_tens_of_millions_of_ids(n, key_range):
+    """More tiles than one round of workgroups holds and buckets at their cap: the plan is still a
+    bijection onto the distinct ids with every occurrence listed once under its id."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+    ids = torch.randint(0, key_range, (n,), device="cuda", generator=g)
+    plan = ops.ids_unique_plan(ids)
+    U = plan.U
+    assert torch.equal(torch.sort(plan.unique).values, torch.unique(ids))
+    assert bool((plan.unique[plan.inverse.long()] == ids).all())
+    rs = plan.row_start[: U + 1].long()
+    assert int(rs[0]) == 0 and int(rs[-1]) == n and bool((rs[1:] > rs[:-1]).all())
+    owner = torch.repeat_interleave(torch.arange(U, device="cuda"), rs[1:] - rs[:-1])
+    assert bool((plan.inverse.long()[plan.occ.long()] == owner).all())
+    assert _lib.poll_device_errors() == 0
