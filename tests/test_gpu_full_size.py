@@ -183,3 +183,25 @@ def test_batch_plan_at_tens_of_millions_of_ids(n, key_range):
     owner = torch.repeat_interleave(torch.arange(U, device="cuda"), rs[1:] - rs[:-1])
     assert bool((plan.inverse.long()[plan.occ.long()] == owner).all())
     assert _lib.poll_device_errors() == 0
+
+
+def test_pooling_past_two_to_the_31_rows():
+    """Row counts that no 32-bit index holds (2^31 + 4096 bf16 rows, 17 GB) take the 64-bit
+    kernels: sums of 0/1 rows are exact, so the pooled rows are known in closed form."""
+    B, D, S = (1 << 31) + 4096, 4, 1 << 20
+    emb = torch.ones((B, D), dtype=torch.bfloat16, device="cuda")
+    emb[::3] = 0
+    off = torch.linspace(0, B, S + 1, device="cuda", dtype=torch.float64).long()
+    off[-1] = B
+    out = ops.segment_reduce_forward(emb, None, None, off, "sum", out_dtype=torch.float32)
+
+    def ones_before(x):        # rows whose index is not a multiple of 3, below x
+        return x - (x + 2) // 3
+
+    exp = (ones_before(off[1:]) - ones_before(off[:-1])).float()
+    assert torch.equal(out, exp[:, None].expand(S, D))
+    del emb, out
+    g = torch.ones((S, D), device="cuda")
+    back = ops.segment_reduce_backward(g, None, None, off, B, "sum", out_dtype=torch.bfloat16)
+    assert bool((back == 1).all())
+    assert _lib.poll_device_errors() == 0
