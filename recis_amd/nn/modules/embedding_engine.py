@@ -53,6 +53,7 @@ class EmbeddingEngine(torch.nn.Module):
         # per feature: the key of its runtime group (features of a table that are pooled together)
         self._runtime_key = {name: opt.runtime_info() for name, opt in self._emb_options.items()}
         self._offsets_cache = {}  # offsets of dense id tensors, which depend on their shape only
+        self._tags = {}
         self._tables = torch.nn.ModuleDict()
         for gkey, grp in self._groups.items():
             opt = grp.opt
@@ -116,29 +117,43 @@ class EmbeddingEngine(torch.nn.Module):
             table = self._tables[gkey]
             dev = table._hashtable_impl.device
             info = table._hashtable_impl.children_info()
+            tag_of = self._tags.get(gkey)
+            if tag_of is None:  # the 12-bit table index of every feature's shared name, fixed after construction
+                tag_of = self._tags[gkey] = {n: info.child_index(o.shared_name) for n, o in grp.features.items()}
             runtime = OrderedDict()
-            for name, opt in grp.features.items():
+            for name in grp.features:
                 if name in inputs:
                     runtime.setdefault(self._runtime_key[name], []).append(name)
             for names in runtime.values():
                 opt0 = grp.features[names[0]]
-                vals, weights, offs, shapes, tags, dense = [], [], [], [], [], []
+                vals, weights, offs, shapes, dense = [], [], [], [], []
                 all_unit = True
                 any_weight = opt0.use_weight and any(
                     isinstance(inputs[n], RaggedTensor) and inputs[n].weight() is not None for n in names)
                 for name in names:
-                    v, w, o, shape, unit, d = self._format(name, grp.features[name], inputs[name])
-                    all_unit = all_unit and unit
+                    data = inputs[name]
+                    if type(data) is torch.Tensor and data.dtype == torch.int64 and data.device == dev \
+                            and data.dim() == 2 and data.shape[1] == 1:
+                        # the common dense case, a [B, 1] id column: nothing to convert
+                        rows = data.shape[0]
+                        v, w, shape, d = data.view(-1), None, (rows,), (rows, 1)
+                        o = self._offsets_cache.get((rows, 1, dev))
+                        if o is None:
+                            o = self._dense_offsets((rows, 1, dev), lambda: torch.arange(
+                                rows + 1, device=dev, dtype=torch.int32))
+                    else:
+                        v, w, o, shape, unit, d = self._format(name, grp.features[name], data)
+                        all_unit = all_unit and unit
+                        v, o = v.to(dev), o.to(dev)
                     dense.append(d)
-                    vals.append(v.to(dev))
-                    offs.append(o.to(dev))
+                    vals.append(v)
+                    offs.append(o)
                     if w is None and any_weight:
                         w = torch.ones(v.numel(), device=dev)
                     weights.append(None if w is None else w.to(dev))
                     shapes.append(shape)
-                    tags.append(info.child_index(grp.features[name].shared_name))
                 if info.is_coalesce():
-                    ids = ops.ids_encode(vals, tags)
+                    ids = ops.ids_encode(vals, [tag_of[n] for n in names])
                 else:
                     ids = vals[0] if len(vals) == 1 else torch.cat(vals)
                 if len(offs) == 1:
@@ -156,5 +171,6 @@ class EmbeddingEngine(torch.nn.Module):
                 seg_counts = [o.numel() - 1 for o in offs]
                 width = pooled.shape[1]
                 for name, part, shape in zip(names, torch.split(pooled, seg_counts), shapes):
-                    outputs[name] = part.reshape(tuple(shape) + (width,))
+                    # [segments, width] already is the answer for a 1-D batch shape: no extra view node
+                    outputs[name] = part if len(shape) == 1 else part.reshape(tuple(shape) + (width,))
         return outputs
