@@ -97,7 +97,10 @@ class FeatureEngine(nn.Module):
                 if key in _FUSED and len(members) > 1:
                     outs = _FUSED[key](op_list, inputs)
                 else:
-                    outs = [op(x) for op, x in zip(op_list, inputs)]
+                    # Module.__call__ costs several microseconds of hook bookkeeping per op, which is
+                    # most of a SelectField; ops with no hooks registered are called directly
+                    outs = [op(x) if (op._forward_hooks or op._forward_pre_hooks) else op.forward(x)
+                            for op, x in zip(op_list, inputs)]
                 for n, o in zip(names, outs):
                     state[n] = o
         results = dict(data) if remain_no_use_data else {}

@@ -525,11 +525,14 @@ def fused_uint64_mod(inputs, mods):
     """``torch.ops.recis.fused_uint64_mod`` (fused_uint64_mod.h)."""
     inputs = [_ids64(t) for t in inputs]
     mods = mods.tolist() if torch.is_tensor(mods) else list(mods)
-    outs = [torch.empty_like(t) for t in inputs]
-    if inputs:
-        check(lib().recis_fused_uint64_mod(_host_ptrs(inputs), _host_i64([t.numel() for t in inputs]),
-                                           _host_i64(mods), _host_ptrs(outs), i64(len(inputs)),
-                                           stream_ptr(inputs[0].device)))
+    if not inputs:
+        return []
+    # one allocation for the whole list (a view per tensor), as fused_bucketized does
+    sizes = [t.numel() for t in inputs]
+    outs = [o.view(t.shape) for o, t in zip(torch.split(torch.empty(sum(sizes), dtype=torch.int64,
+                                                                    device=inputs[0].device), sizes), inputs)]
+    check(lib().recis_fused_uint64_mod(_host_ptrs(inputs), _host_i64(sizes), _host_i64(mods), _host_ptrs(outs),
+                                       i64(len(inputs)), stream_ptr(inputs[0].device)))
     return outs
 
 
