@@ -451,7 +451,9 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
  * gather-reduce). Rows come from a dense [U, D] array (rows) or, when emb_blocks_dev != NULL,
  * straight from a block list: row u is row row_index[u] (negative = zeros) of blocks of
  * block_rows rows. weight ([n_out], per OUTPUT row) may be NULL. Output rows no list entry
- * names are not written. dst outside [0, n_out) raises RECIS_DEVERR_INDEX_RANGE.
+ * names are not written. dst outside [0, n_out) raises RECIS_DEVERR_INDEX_RANGE. U may be an
+ * upper bound of the number of unique ids (a caller that has not read the plan's count back yet
+ * passes n): rows at and past counts_dev[0], the count the plan left on the device, are skipped.
  */
 int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks,
                           int64_t block_rows, const int64_t* row_index, int rows_dtype,

@@ -961,7 +961,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
   // ---- cold rows
   const int rows_per_block = kBlock >> a.lpr_log2;
   const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
-  const bool valid = u < a.U;
+  const bool valid = u < a.U && u < a.counts[0];  // U may be the caller's upper bound: the plan's own count decides
   const int32_t start = valid ? a.row_start[u] : 0;
   int32_t end = valid ? a.row_start[u + 1] : 0;
   if (end - start > a.hot_len) end = start;  // written by the work items

@@ -131,8 +131,13 @@ class LookupPoolFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly, unit_segments=False):
+        late_count = unit_segments and not readonly
         if readonly:
             index = impl.lookup_index(plan.unique, True)
+        elif late_count:
+            # the expansion below takes the unique count from device memory, so nothing in this
+            # forward waits for it: the host reads it in backward, long after it has arrived
+            index = impl.lookup_index_unsettled(plan)
         else:
             # queued behind the plan before the host has the unique count: the count arrives
             # while the plan's last kernels and the lookup run
@@ -147,7 +152,7 @@ class LookupPoolFunction(torch.autograd.Function):
         else:
             out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets,
                                                     combiner)
-        ctx.impl, ctx.plan, ctx.combiner, ctx.readonly = impl, plan, combiner, readonly
+        ctx.impl, ctx.plan, ctx.combiner, ctx.readonly, ctx.late_count = impl, plan, combiner, readonly, late_count
         ctx.save_for_backward(index, weight, offsets)
         ctx.mark_non_differentiable(index)
         return index, out
@@ -155,6 +160,9 @@ class LookupPoolFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, _grad_index, grad):
         index, weight, offsets = ctx.saved_tensors
+        if ctx.late_count:
+            ctx.impl.settle_count(ctx.plan.U)
+            index = index[: ctx.plan.U]
         g = ops.segment_reduce_backward_plan(grad.contiguous(), weight, offsets, ctx.plan, ctx.combiner)
         if ctx.readonly:  # keys the table does not hold take no gradient
             keep = index >= 0
@@ -184,7 +192,10 @@ def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segme
                 assert isinstance(admit, ReadOnlyHookImpl), "admit hook only support ReadOnlyHook yet, but got: %s" % admit
             index, out = LookupPoolFunction.apply(hashtable._backward_holder, impl, plan, weight, offsets,
                                                   opt.combiner, readonly, unit_segments)
-            hashtable._filter_hook_impl(index)
+            if not isinstance(hashtable._filter_hook_impl, torch.nn.Identity):
+                # a step filter stamps the looked-up rows: it needs the rows proper (the index may
+                # be the full-length buffer of the forward that does not wait for the count)
+                hashtable._filter_hook_impl(index[: plan.U] if not readonly else index)
             return out
         readonly = (not hashtable.training) or opt.admit_hook is not None
         index = impl.lookup_index(plan.unique.detach(), readonly)

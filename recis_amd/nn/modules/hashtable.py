@@ -391,6 +391,18 @@ class HashtableImpl:
         there are; finish with ``settle_lookup`` once ``plan.U`` has been read."""
         return self._idmap.lookup_counted(plan.unique_buf, plan.counts)
 
+    def lookup_index_unsettled(self, plan):
+        """``lookup_index_counted`` for consumers that take the unique count from device memory: the
+        rows every one of the plan's ids could need are made room for, nothing waits for the count.
+        Returns the full-length index buffer (its first ``plan.U`` entries are the rows); settle
+        with ``settle_count`` whenever the count has been read."""
+        index_buf = self._idmap.lookup_counted(plan.unique_buf, plan.counts)
+        self._make_room(plan.n)
+        return index_buf
+
+    def settle_count(self, n_true):
+        self._idmap.settle_count(n_true)
+
     def settle_lookup(self, index_buf, n_true):
         self._idmap.settle_count(n_true)
         self._make_room(n_true)

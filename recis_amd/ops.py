@@ -753,6 +753,11 @@ class BatchPlan:
                 self._U = int(self.counts[0].item())
         return self._U
 
+    def U_bound(self):
+        """The unique count if the host has it already, else the number of ids: for kernels that
+        take the count from device memory and only need a bound to size their grid."""
+        return self.n if self._U is None else self._U
+
     @property
     def unique(self):
         if self._unique is None:
@@ -855,8 +860,8 @@ def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_inde
     check(lib().recis_csr_expand_rows(ptr(rows_arg), ptr(table), i64(n_blocks), i64(block_size), ptr(row_index),
                                       dtype_code(dt), ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
                                       ptr(plan.row_start), ptr(plan.occ), ptr(plan.hot_items), i64(plan.hot_cap),
-                                      ptr(plan.counts), ptr(out), dtype_code(out.dtype), i64(plan.U), i64(n_out),
-                                      i64(D), stream_ptr(dev)))
+                                      ptr(plan.counts), ptr(out), dtype_code(out.dtype), i64(plan.U_bound()),
+                                      i64(n_out), i64(D), stream_ptr(dev)))
     return out
 
 
