@@ -131,18 +131,15 @@ class LookupPoolFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly, unit_segments=False):
-        late_count = unit_segments and not readonly
+        late_count = not readonly
         if readonly:
             index = impl.lookup_index(plan.unique, True)
-        elif late_count:
-            # the expansion below takes the unique count from device memory, so nothing in this
-            # forward waits for it: the host reads it in backward, long after it has arrived
-            index = impl.lookup_index_unsettled(plan)
         else:
-            # queued behind the plan before the host has the unique count: the count arrives
-            # while the plan's last kernels and the lookup run
-            index_buf = impl.lookup_index_counted(plan)
-            index = impl.settle_lookup(index_buf, plan.U)
+            # Nothing in this forward waits for the unique count: the lookup and the expansion take
+            # it from device memory, the pooling kernel only follows the plan's inverse (which names
+            # rows below the count), and the host reads it in backward, long after it has arrived.
+            # `index` is the full-length buffer; its first plan.U entries are the rows.
+            index = impl.lookup_index_unsettled(plan)
         chunks, chunk_rows = impl.emb_blocks()
         if unit_segments:
             # one id per segment (sum == mean == the row itself): every unique row is read once and
