@@ -168,7 +168,7 @@ class LookupPoolFunction(torch.autograd.Function):
         return None, None, None, None, None, None, None, None
 
 
-def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False):
+def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False, combiner_kwargs=None):
     """Rows of the plan's unique ids pooled per segment. Sum / mean over a float table go
     through ``LookupPoolFunction`` (pooling reads the table directly); everything else looks the
     rows up first and pools the copy. ``unit_segments``: the caller built ``offsets`` as
@@ -209,7 +209,8 @@ def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segme
         inverse, plan = None, None
     if weight is not None and weight.dtype != emb.dtype:
         weight = weight.to(emb.dtype)
-    return ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner, opt.combiner_kwargs,
+    return ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner,
+                                           combiner_kwargs if combiner_kwargs is not None else opt.combiner_kwargs,
                                            plan=plan)
 
 

@@ -113,6 +113,9 @@ class EmbeddingEngine(torch.nn.Module):
 
     def forward(self, inputs: Dict[str, Union[torch.Tensor, RaggedTensor]]):
         outputs = {}
+        # the same input objects under two combiners (a sequence pooled AND kept row by row) are
+        # tagged, merged and deduplicated once per call
+        plans = {}
         for gkey, grp in self._groups.items():
             table = self._tables[gkey]
             dev = table._hashtable_impl.device
@@ -152,23 +155,39 @@ class EmbeddingEngine(torch.nn.Module):
                         w = torch.ones(v.numel(), device=dev)
                     weights.append(None if w is None else w.to(dev))
                     shapes.append(shape)
-                if info.is_coalesce():
-                    ids = ops.ids_encode(vals, [tag_of[n] for n in names])
+                same = (gkey,) + tuple((id(inputs[n]), tag_of[n]) for n in names)
+                if same in plans:
+                    offsets, plan = plans[same]
                 else:
-                    ids = vals[0] if len(vals) == 1 else torch.cat(vals)
-                if len(offs) == 1:
-                    offsets = offs[0]
-                elif all(d is not None for d in dense):  # dense id tensors only: a function of the shapes
-                    offsets = self._dense_offsets((tuple(dense), dev), lambda: ops.merge_offsets(
-                        offs, [v.numel() for v in vals]))
-                else:
-                    offsets = ops.merge_offsets(offs, [v.numel() for v in vals])
+                    if info.is_coalesce():
+                        ids = ops.ids_encode(vals, [tag_of[n] for n in names])
+                    else:
+                        ids = vals[0] if len(vals) == 1 else torch.cat(vals)
+                    if len(offs) == 1:
+                        offsets = offs[0]
+                    elif all(d is not None for d in dense):  # dense id tensors only: a function of the shapes
+                        offsets = self._dense_offsets((tuple(dense), dev), lambda: ops.merge_offsets(
+                            offs, [v.numel() for v in vals]))
+                    else:
+                        offsets = ops.merge_offsets(offs, [v.numel() for v in vals])
+                    plan = ops.ids_unique_plan(ids, wait=False)
+                    plans[same] = (offsets, plan)
                 weight = None
                 if all(w is not None for w in weights):
                     weight = weights[0] if len(weights) == 1 else torch.cat(weights)
-                plan = ops.ids_unique_plan(ids, wait=False)
-                pooled = lookup_and_pool(table, plan, weight, offsets, opt0, unit_segments=all_unit)
                 seg_counts = [o.numel() - 1 for o in offs]
+                if opt0.combiner == "tile":
+                    # every feature keeps its own number of rows per sample: the list form of the
+                    # padded gather (embedding_engine.py:383-411, 453-455)
+                    tile_lens = [int(grp.features[n].combiner_kwargs["tile_len"]) for n in names]
+                    pooled = lookup_and_pool(table, plan, weight, offsets, opt0,
+                                             combiner_kwargs={"bs": seg_counts, "tile_len": tile_lens})
+                    width = pooled.shape[1]
+                    parts = torch.split(pooled, [b * t for b, t in zip(seg_counts, tile_lens)])
+                    for name, part, shape, t in zip(names, parts, shapes, tile_lens):
+                        outputs[name] = part.reshape(tuple(shape) + (t * width,))
+                    continue
+                pooled = lookup_and_pool(table, plan, weight, offsets, opt0, unit_segments=all_unit)
                 width = pooled.shape[1]
                 for name, part, shape in zip(names, torch.split(pooled, seg_counts), shapes):
                     # [segments, width] already is the answer for a 1-D batch shape: no extra view node

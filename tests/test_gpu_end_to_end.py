@@ -424,6 +424,62 @@ def test_three_tables_state_dict_keys():
     assert int(optim.state_dict()["sparse_adamw_tf_step"]) == 0
 
 
+def test_engine_sequence_pooled_and_tiled_from_one_plan():
+    """A sequence feature used twice, mean-pooled and kept row by row (two lengths), plus a second
+    sequence: the engine tags / merges / deduplicates the shared inputs once, and every output and
+    the accumulated row gradients equal what separate DynamicEmbedding-style calls give."""
+    rng = np.random.default_rng(11)
+    B = 64
+
+    def seq(max_len):
+        lens = rng.integers(0, max_len, B)
+        off = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)).cuda()
+        return RaggedTensor(torch.from_numpy(rng.integers(0, 40, int(off[-1]))).cuda(), off)
+
+    a, b = seq(30), seq(12)
+
+    def option(combiner, **kw):
+        return EmbeddingOption(embedding_dim=8, shared_name="seq_tab", combiner=combiner, use_weight=False,
+                               block_size=64, initializer=NormalInitializer(0, 1.0), **kw)
+
+    engine = EmbeddingEngine({
+        "a_mean": option("mean"), "b_mean": option("mean"),
+        "a_rows": option("tile", combiner_kwargs={"tile_len": 5}),
+        "b_rows": option("tile", combiner_kwargs={"tile_len": 9}),
+    })
+    engine.train()
+    out = engine({"a_mean": a, "b_mean": b, "a_rows": a, "b_rows": b})
+    table = next(iter(engine.hashtables().values()))
+    assert out["a_mean"].shape == (B, 8) and out["a_rows"].shape == (B, 5 * 8) and out["b_rows"].shape == (B, 9 * 8)
+
+    def rows_of(rt):
+        return table(rt.values()).detach()
+
+    for name, rt, t in (("a", a, 5), ("b", b, 9)):
+        rows, off = rows_of(rt), rt.offsets()[-1].cpu().numpy()
+        mean = torch.stack([rows[off[i]:off[i + 1]].mean(0) if off[i + 1] > off[i] else torch.zeros(8, device="cuda")
+                            for i in range(B)])
+        torch.testing.assert_close(out[name + "_mean"].detach(), mean, rtol=1e-5, atol=1e-6)
+        tiled = torch.zeros(B, t, 8, device="cuda")
+        for i in range(B):
+            k = min(t, off[i + 1] - off[i])
+            tiled[i, :k] = rows[off[i]:off[i] + k]
+        assert torch.equal(out[name + "_rows"].detach(), tiled.view(B, t * 8))
+    # gradients: every kept row of a_rows passes 1, every pooled occurrence 1 / len
+    (out["a_mean"].sum() + out["a_rows"].sum()).backward()
+    impl = table._hashtable_impl
+    index, g = impl.grad_pairs(1)
+    got = torch.zeros(impl.ids_num() + 1, 8, device="cuda").index_add_(0, index, g)
+    off = a.offsets()[-1].cpu().numpy()
+    exp = torch.zeros_like(got)
+    row_of = impl.lookup_index_readonly(a.values())
+    for i in range(B):
+        n = off[i + 1] - off[i]
+        for k in range(n):
+            exp[row_of[off[i] + k]] += 1.0 / n + (1.0 if k < 5 else 0.0)
+    torch.testing.assert_close(got, exp, rtol=1e-5, atol=1e-5)
+
+
 def test_feature_engine_ops_and_fusion():
     """Restated from tests/feature_engine/op_test.py:17-36,95-131 and feature_engine_test.py: Mod,
     Bucketize, IDMultiHash, Hash known answers, through the fused engine path."""
