@@ -136,6 +136,42 @@ class EmbeddingSegmentReduceRagged(torch.autograd.Function):
         return g, None, None, None, None, None, None
 
 
+class RaggedTileParts(torch.autograd.Function):
+    """The padded gather of several features at once with ONE output per feature
+    (``[bs[f], tile_len[f] * D]``, views of one buffer). Splitting a single output instead makes
+    autograd concatenate the features' gradients again before the backward sees them, a copy of
+    the whole padded gradient (2 GB for long behaviour sequences); here every feature's gradient
+    goes through its own gather-reduce pass over the plan's occurrence lists."""
+
+    @staticmethod
+    def forward(ctx, unique_emb, reverse_indices, offsets, plan, bs, tile_len):
+        bs, tile_len = [int(b) for b in bs], [int(t) for t in tile_len]
+        out, _ = ops.ragged_tile(bs, tile_len, reverse_indices, offsets, unique_emb)
+        D = unique_emb.shape[1]
+        ctx.plan, ctx.bs, ctx.tile_len, ctx.D = plan, bs, tile_len, D
+        ctx.unique_size, ctx.emb_dtype = unique_emb.shape[0], unique_emb.dtype
+        ctx.save_for_backward(offsets)
+        rows = [b * t for b, t in zip(bs, tile_len)]
+        return tuple(p.view(b, t * D) for p, b, t in zip(torch.split(out, rows), bs, tile_len))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        (offsets,) = ctx.saved_tensors
+        plan, D = ctx.plan, ctx.D
+        src = plan.src_for_tile(ctx.bs, ctx.tile_len, offsets)  # row of the whole padded output per list entry
+        g, lo = None, 0
+        for grad, b, t in zip(grads, ctx.bs, ctx.tile_len):
+            n = b * t
+            if grad is not None and n:
+                # this feature's rows only, counted from its own first row; the others are skipped
+                mine = torch.where((src >= lo) & (src < lo + n), src - lo, -1)
+                g = ops.csr_gather_reduce(grad.reshape(n, D), plan, mine, out=g, accumulate=g is not None)
+            lo += n
+        if g is None:
+            g = torch.zeros((ctx.unique_size, D), dtype=torch.float32, device=offsets.device)
+        return g.to(ctx.emb_dtype), None, None, None, None, None
+
+
 def ragged_embedding_segment_reduce(unique_emb: torch.Tensor, weight: Optional[torch.Tensor],
                                     reverse_indices: torch.Tensor, offsets: torch.Tensor, combiner: str,
                                     combiner_kwargs: Optional[dict] = None, plan=None):

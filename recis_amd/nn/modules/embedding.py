@@ -104,16 +104,17 @@ class EmbeddingOption:
         })
 
 
-def lookup_unique_rows(hashtable: HashTable, unique_ids, admit_hook=None, trainable=True):
+def lookup_unique_rows(hashtable: HashTable, unique_ids, admit_hook=None, trainable=True, grad_key=None):
     """Rows of ids that are already unique: the lookup autograd function, the
-    last-seen-step stamp, no second dedup."""
+    last-seen-step stamp, no second dedup. ``grad_key``: see ``HashtableImpl.accept_grad``."""
     from .hashtable_hook_impl import HashtableHookFactory
 
     impl = hashtable._hashtable_impl
     float_table = hashtable._dtype not in (torch.int8, torch.int32, torch.int64)
     if hashtable.training and trainable and float_table:
         admit_impl = HashtableHookFactory().create_admit_hook(hashtable, admit_hook) if admit_hook else None
-        emb_idx, emb = HashTableLookupHelpFunction.apply(unique_ids, impl, hashtable._backward_holder, admit_impl)
+        emb_idx, emb = HashTableLookupHelpFunction.apply(unique_ids, impl, hashtable._backward_holder, admit_impl,
+                                                         grad_key)
         hashtable._filter_hook_impl(emb_idx)
         return emb
     readonly = (not hashtable.training) or admit_hook is not None or not float_table
@@ -164,7 +165,7 @@ class LookupPoolFunction(torch.autograd.Function):
         if ctx.readonly:  # keys the table does not hold take no gradient
             keep = index >= 0
             index, g = index[keep], g[keep]
-        ctx.impl.accept_grad(index, g, unique=True)
+        ctx.impl.accept_grad(index, g, unique=True, key=None if ctx.readonly else ctx.plan.serial)
         return None, None, None, None, None, None, None, None
 
 

@@ -21,7 +21,8 @@ import torch
 
 from ... import ops
 from ...ragged.tensor import RaggedTensor
-from .embedding import EmbeddingOption, lookup_and_pool
+from ..functional.embedding_ops import RaggedTileParts
+from .embedding import EmbeddingOption, lookup_and_pool, lookup_unique_rows
 from .hashtable import HashTable, gen_slice
 
 
@@ -180,12 +181,18 @@ class EmbeddingEngine(torch.nn.Module):
                     # every feature keeps its own number of rows per sample: the list form of the
                     # padded gather (embedding_engine.py:383-411, 453-455)
                     tile_lens = [int(grp.features[n].combiner_kwargs["tile_len"]) for n in names]
-                    pooled = lookup_and_pool(table, plan, weight, offsets, opt0,
-                                             combiner_kwargs={"bs": seg_counts, "tile_len": tile_lens})
-                    width = pooled.shape[1]
-                    parts = torch.split(pooled, [b * t for b, t in zip(seg_counts, tile_lens)])
-                    for name, part, shape, t in zip(names, parts, shapes, tile_lens):
-                        outputs[name] = part.reshape(tuple(shape) + (t * width,))
+                    if opt0.grad_reduce_by == "id" and table.training and opt0.trainable:
+                        pooled = lookup_and_pool(table, plan, weight, offsets, opt0,
+                                                 combiner_kwargs={"bs": seg_counts, "tile_len": tile_lens})
+                        width = pooled.shape[1]
+                        parts = [p.view(b, t * width) for p, b, t in zip(
+                            torch.split(pooled, [b * t for b, t in zip(seg_counts, tile_lens)]), seg_counts, tile_lens)]
+                    else:
+                        emb = lookup_unique_rows(table, plan.unique, opt0.admit_hook, opt0.trainable,
+                                                 grad_key=plan.serial)
+                        parts = RaggedTileParts.apply(emb, plan.inverse, offsets, plan, seg_counts, tile_lens)
+                    for name, part, shape in zip(names, parts, shapes):
+                        outputs[name] = part if len(shape) == 1 else part.reshape(tuple(shape) + (part.shape[1],))
                     continue
                 pooled = lookup_and_pool(table, plan, weight, offsets, opt0, unit_segments=all_unit)
                 width = pooled.shape[1]

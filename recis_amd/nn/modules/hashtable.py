@@ -311,7 +311,7 @@ class HashtableImpl:
         self._children_info = ChildrenInfo(coalesce, children)
         self._slice = Slice(slice_begin, slice_end, slice_size)
         self._idmap = ops.IdMap(device, reserve=reserve_rows)
-        self._grad_index, self._grad, self._grad_unique = [], [], []
+        self._grad_index, self._grad, self._grad_unique, self._grad_keys = [], [], [], {}
 
     # ------------------------------------------------------------- storage
     def _make_room(self, incoming):
@@ -416,14 +416,23 @@ class HashtableImpl:
         return self.insert_lookup_index(ids)
 
     # -------------------------------------------------------------- grads
-    def accept_grad(self, grad_index, grad, unique=False):
+    def accept_grad(self, grad_index, grad, unique=False, key=None):
         """``unique=True``: the caller knows ``grad_index`` has no duplicates (it is the
-        row index of unique ids), which spares ``grad()`` a dedup pass."""
+        row index of unique ids), which spares ``grad()`` a dedup pass. ``key``: two calls of one
+        step with the same key hand over gradients for the SAME rows in the same order (the rows
+        of one batch plan's unique ids, looked up twice); the second is added onto the first
+        instead of being merged by row index later."""
         if grad_index.dtype != torch.int64:
             raise RuntimeError("grad_index must be int64")
         if grad.dtype != self._dtype and not (grad.dtype == torch.float32 and self._dtype in
                                               (torch.bfloat16, torch.float16)):
             raise RuntimeError("grad dtype %s does not match the table (%s)" % (grad.dtype, self._dtype))
+        if key is not None:
+            at = self._grad_keys.get(key)
+            if at is not None and self._grad[at].shape == grad.shape:
+                self._grad[at] = self._grad[at] + grad
+                return
+            self._grad_keys[key] = len(self._grad)
         self._grad_index.append(grad_index)
         self._grad.append(grad)
         self._grad_unique.append(bool(unique))
@@ -469,7 +478,7 @@ class HashtableImpl:
                                        check_invariants=False).detach_()
 
     def clear_grad(self):
-        self._grad_index, self._grad, self._grad_unique = [], [], []
+        self._grad_index, self._grad, self._grad_unique, self._grad_keys = [], [], [], {}
 
     # ------------------------------------------------------------ bookkeeping
     def clear(self):
@@ -591,8 +600,10 @@ class HashTableLookupHelpFunction(torch.autograd.Function):
     (recis/nn/modules/hashtable.py:425-481)."""
 
     @staticmethod
-    def forward(ctx, ids, hashtable, backward_holder, admit_hook_impl):
+    def forward(ctx, ids, hashtable, backward_holder, admit_hook_impl, grad_key=None):
         from .hashtable_hook_impl import ReadOnlyHookImpl
+
+        ctx.grad_key = grad_key if admit_hook_impl is None else None
 
         assert admit_hook_impl is None or isinstance(admit_hook_impl, ReadOnlyHookImpl), \
             "admit hook only support ReadOnlyHook yet, but got: %s" % admit_hook_impl
@@ -605,8 +616,8 @@ class HashTableLookupHelpFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output_index, grad_output_emb):
         (index,) = ctx.saved_tensors
-        ctx.hashtable.accept_grad(index, grad_output_emb.contiguous(), unique=True)
-        return None, None, None, None
+        ctx.hashtable.accept_grad(index, grad_output_emb.contiguous(), unique=True, key=ctx.grad_key)
+        return None, None, None, None, None
 
 
 class GradIDMeanFunction(torch.autograd.Function):

@@ -6,6 +6,7 @@ arguments the reference does not have are keyword-only and default to the
 reference behaviour. Tensors must live on the GPU: there is no CPU path here.
 """
 import ctypes
+import itertools
 
 import torch
 
@@ -739,7 +740,7 @@ class BatchPlan:
     """
 
     __slots__ = ("n", "_U", "_unique", "unique_buf", "inverse", "row_start", "occ", "pos", "hot_items", "hot_cap",
-                 "counts", "_pool_fill", "_stream")
+                 "counts", "_pool_fill", "_stream", "serial")
 
     @property
     def U(self):
@@ -794,6 +795,9 @@ class BatchPlan:
         return src
 
 
+_PLAN_SERIAL = itertools.count(1)
+
+
 def ids_unique_plan(ids, wait=True):
     """Dedup + transposed index of a batch of ids (``recis_unique_plan``). ``wait=False``
     returns without the host copy of the unique count (see ``BatchPlan``); at most one such
@@ -802,6 +806,7 @@ def ids_unique_plan(ids, wait=True):
     n = ids.numel()
     dev = ids.device
     p = BatchPlan()
+    p.serial = next(_PLAN_SERIAL)  # never reused, unlike id(p)
     p.n = n
     p.unique_buf = torch.empty(n, dtype=torch.int64, device=dev)
     p.inverse = torch.empty(n, dtype=torch.int32, device=dev)
