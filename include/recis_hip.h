@@ -443,6 +443,20 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
                             void* stream);
 
 /*
+ * recis_csr_gather_reduce over input rows that live in n_parts (1 to 8) separate arrays instead
+ * of one (no reference counterpart): src numbers the rows of part 0, then those of part 1, and so
+ * on (part f holds part_counts[f] rows of D elements of rows_dtype). No coefficients, fp32 output
+ * [U, D]. For callers that get the gradient of several outputs as several tensors (one padded
+ * gather per feature) and would otherwise concatenate them first. part_rows and part_counts are
+ * host arrays.
+ */
+int recis_csr_gather_reduce_parts(const void* const* part_rows, const int64_t* part_counts,
+                                  int n_parts, int rows_dtype, const int32_t* src,
+                                  const int32_t* row_start, const int32_t* hot_items,
+                                  int64_t hot_cap, const int64_t* counts_dev, void* out, int64_t U,
+                                  int64_t D, int accumulate, void* stream);
+
+/*
  * The transpose of recis_csr_gather_reduce (no reference counterpart; it produces what
  * segment_reduce_forward gives for one-id segments and for the TILE mode,
  * embedding_segment_reduce_kernel.cu:23-75): out[dst[k], :] = weight[dst[k]] * row(u) for every

@@ -567,6 +567,8 @@ __device__ __forceinline__ float load_coef(const void* w, int wdt, int64_t i) {
   return to_float(static_cast<const f16_t*>(w)[i]);
 }
 
+constexpr int kMaxParts = 8;  // input arrays of one gather-reduce launch (PARTS kernels)
+
 struct CsrArgs {
   const int32_t* row_start;  // [U + 1]
   const int32_t* src;        // [n] input row per list entry (negative = skip)
@@ -588,7 +590,34 @@ struct CsrArgs {
   int64_t hot_cap;
   float* hot_part;           // [hot_cap, D]
   int64_t cold_blocks;       // the last cold_blocks workgroups work per row, the ones before per hot item
+  // PARTS kernels: the input rows are n_parts arrays laid end to end in src's numbering; part f
+  // holds rows [part_lo[f], part_lo[f + 1])
+  int n_parts;
+  const void* part_rows[kMaxParts];
+  int64_t part_lo[kMaxParts + 1];
 };
+
+// Row s of the input: of the one array, or of the part that holds it.
+template <typename TIn, bool PARTS>
+__device__ __forceinline__ const TIn* src_row(const TIn* rows, const CsrArgs& a, int64_t s) {
+  if constexpr (!PARTS) {
+    return rows + s * a.D;
+  } else {
+    int f = 0;
+#pragma unroll
+    for (int k = 1; k < kMaxParts; ++k) f += (k < a.n_parts && s >= a.part_lo[k]) ? 1 : 0;
+    const TIn* base = static_cast<const TIn*>(a.part_rows[0]);
+    int64_t lo = 0;
+#pragma unroll
+    for (int k = 1; k < kMaxParts; ++k) {
+      if (k == f) {
+        base = static_cast<const TIn*>(a.part_rows[k]);
+        lo = a.part_lo[k];
+      }
+    }
+    return base + (s - lo) * a.D;
+  }
+}
 
 __device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64_t& hi) {
   lo = 0;
@@ -604,7 +633,7 @@ __device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64
 // that gather the rows through shuffles; lane group g of `groups` takes entries g, g + groups,
 // ... with several row loads in flight. acc: this group's partial sum for columns
 // c0 .. c0 + VEC (the caller folds the groups).
-template <typename TIn, int VEC>
+template <typename TIn, int VEC, bool PARTS>
 __device__ __forceinline__ void wave_gather_range(const TIn* __restrict__ rows, const CsrArgs& a, int64_t c_lo,
                                                   int64_t c_hi, int32_t e_begin, int32_t e_end, int c0, bool col_ok,
                                                   int g, int groups, float (&acc)[VEC]) {
@@ -634,10 +663,11 @@ __device__ __forceinline__ void wave_gather_range(const TIn* __restrict__ rows, 
         w[k] = a.coef ? __shfl(w_mine, from, kWave) : 1.0f;
         if (e >= n_here || !col_ok) id = -1;
         if (id >= 0) {
+          const TIn* row = src_row<TIn, PARTS>(rows, a, id);
           if (a.nt_in) {
-            load_pack_stream<TIn, VEC>(rows + static_cast<int64_t>(id) * a.D + c0, v[k]);
+            load_pack_stream<TIn, VEC>(row + c0, v[k]);
           } else {
-            load_pack<TIn, VEC>(rows + static_cast<int64_t>(id) * a.D + c0, v[k]);
+            load_pack<TIn, VEC>(row + c0, v[k]);
           }
         } else {
           w[k] = 0.f;
@@ -665,7 +695,7 @@ constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of
 // the partial rows of every hot row in chunk order. No atomics anywhere.
 // SHUFFLE: long lists go through wave_gather_range (pays off when a wave has at most eight lane
 // groups, i.e. rows of 128 bytes and more); otherwise every group loads its own entries.
-template <typename TIn, typename TOut, int VEC, bool SHUFFLE>
+template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false>
 __global__ void __launch_bounds__(kBlock)
 csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a) {
   extern __shared__ float s_part[];  // [waves][D], hot part only
@@ -687,10 +717,11 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
       w = 0.f;
       return;
     }
+    const TIn* row = src_row<TIn, PARTS>(rows, a, s);
     if (a.nt_in) {
-      load_pack_stream<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
+      load_pack_stream<TIn, VEC>(row + c0, v);
     } else {
-      load_pack<TIn, VEC>(rows + static_cast<int64_t>(s) * D + c0, v);
+      load_pack<TIn, VEC>(row + c0, v);
     }
   };
   // acc += sum over list entries k = first, first + step, ... < last (4 gathers in flight)
@@ -724,7 +755,7 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
     if constexpr (SHUFFLE) {
-      wave_gather_range<TIn, VEC>(rows, a, c_lo, c_hi, first, last, c0, col_ok, g, groups, acc);
+      wave_gather_range<TIn, VEC, PARTS>(rows, a, c_lo, c_hi, first, last, c0, col_ok, g, groups, acc);
     } else {
       if (col_ok) gather_sum(first + g, last, groups, c0, acc);
     }
@@ -1234,22 +1265,57 @@ int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_feat
   return RECIS_OK;
 }
 
+static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows, const int64_t* part_counts,
+                                  int n_parts, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
+                                  int coef_dtype, const int32_t* row_start, const int32_t* hot_items,
+                                  int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
+                                  int64_t D, int accumulate, const void* cover_offsets, int cover_is64,
+                                  int64_t cover_S, hipStream_t stream);
+
 int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
                             int coef_dtype, const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
                             const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t D,
                             int accumulate, const void* cover_offsets, int cover_is64, int64_t cover_S,
                             void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  return csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
+                                hot_items, hot_cap, counts_dev, out, out_dtype, U, D, accumulate, cover_offsets,
+                                cover_is64, cover_S, static_cast<hipStream_t>(stream_));
+}
+
+int recis_csr_gather_reduce_parts(const void* const* part_rows, const int64_t* part_counts, int n_parts,
+                                  int rows_dtype, const int32_t* src, const int32_t* row_start,
+                                  const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, void* out,
+                                  int64_t U, int64_t D, int accumulate, void* stream_) {
+  RECIS_REQUIRE(n_parts >= 1 && n_parts <= kMaxParts, "1 to %d parts (got %d)", kMaxParts, n_parts);
+  RECIS_REQUIRE(part_rows && part_counts, "NULL argument");
+  int64_t n_rows = 0;
+  for (int f = 0; f < n_parts; ++f) {
+    RECIS_REQUIRE(part_counts[f] >= 0 && (part_rows[f] != nullptr || part_counts[f] == 0), "bad part %d", f);
+    n_rows += part_counts[f];
+  }
+  return csr_gather_reduce_impl(nullptr, part_rows, part_counts, n_parts, rows_dtype, n_rows, src, nullptr, 0,
+                                row_start, hot_items, hot_cap, counts_dev, out, RECIS_F32, U, D, accumulate, nullptr,
+                                0, 0, static_cast<hipStream_t>(stream_));
+}
+
+static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows, const int64_t* part_counts,
+                                  int n_parts, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
+                                  int coef_dtype, const int32_t* row_start, const int32_t* hot_items,
+                                  int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
+                                  int64_t D, int accumulate, const void* cover_offsets, int cover_is64,
+                                  int64_t cover_S, hipStream_t stream) {
   RECIS_REQUIRE(U >= 0 && n_rows >= 0, "negative size");
   RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
   if (U == 0) return RECIS_OK;
   RECIS_REQUIRE(src && row_start && out && counts_dev, "NULL argument");
-  RECIS_REQUIRE(rows != nullptr || n_rows == 0, "rows must not be NULL");
+  RECIS_REQUIRE(n_parts > 0 || rows != nullptr || n_rows == 0, "rows must not be NULL");
   RECIS_REQUIRE(hot_cap == 0 || hot_items, "hot_items must not be NULL");
   const int in_sz = dtype_size(rows_dtype), out_sz = dtype_size(out_dtype);
   RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
   RECIS_REQUIRE(coef == nullptr || dtype_size(coef_dtype), "invalid coef dtype");
-  const int vb_in = pick_vec_bytes(D * in_sz, reinterpret_cast<uintptr_t>(rows));
+  uintptr_t align_of = reinterpret_cast<uintptr_t>(rows);
+  for (int f = 0; f < n_parts; ++f) align_of |= reinterpret_cast<uintptr_t>(part_rows[f]);  // the coarsest alignment
+  const int vb_in = pick_vec_bytes(D * in_sz, align_of);
   const int vb_out = pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
   const int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
   CsrArgs a;
@@ -1275,6 +1341,12 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   a.counts = counts_dev;
   a.hot_cap = hot_cap;
   a.hot_part = nullptr;
+  a.n_parts = n_parts;
+  a.part_lo[0] = 0;
+  for (int f = 0; f < kMaxParts; ++f) {
+    a.part_rows[f] = f < n_parts ? part_rows[f] : nullptr;
+    a.part_lo[f + 1] = a.part_lo[f] + (f < n_parts ? part_counts[f] : 0);
+  }
   int64_t hot_blocks = 0;
   if (hot_cap > 0) {
     void* ws = nullptr;
@@ -1297,7 +1369,14 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
         const bool shuffle = a.lpr_log2 >= 3;  // at most eight lane groups per wave
         {
           RECIS_TIME_KERNEL("csr_rows_kernel", stream)
-          if (shuffle)
+          if (n_parts > 0) {
+            if constexpr (sizeof(TOut) == 4) {  // parts go to fp32 rows only
+              if (shuffle)
+                csr_rows_kernel<TIn, TOut, VEC, true, true><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
+              else
+                csr_rows_kernel<TIn, TOut, VEC, false, true><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
+            }
+          } else if (shuffle)
             csr_rows_kernel<TIn, TOut, VEC, true><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
           else
             csr_rows_kernel<TIn, TOut, VEC, false><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);

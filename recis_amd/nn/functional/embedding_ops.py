@@ -159,6 +159,12 @@ class RaggedTileParts(torch.autograd.Function):
         (offsets,) = ctx.saved_tensors
         plan, D = ctx.plan, ctx.D
         src = plan.src_for_tile(ctx.bs, ctx.tile_len, offsets)  # row of the whole padded output per list entry
+        rows = [b * t for b, t in zip(ctx.bs, ctx.tile_len)]
+        if len(grads) <= 8 and all(g is not None for g in grads) and len({g.dtype for g in grads}) == 1 \
+                and grads[0].dtype in (torch.float32, torch.bfloat16, torch.float16):
+            # one pass: the kernel takes the features' gradients as separate arrays
+            g = ops.csr_gather_reduce_parts([grad.reshape(n, D) for grad, n in zip(grads, rows)], plan, src)
+            return g.to(ctx.emb_dtype), None, None, None, None, None
         g, lo = None, 0
         for grad, b, t in zip(grads, ctx.bs, ctx.tile_len):
             n = b * t

@@ -848,6 +848,24 @@ def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False, co
     return out
 
 
+def csr_gather_reduce_parts(parts, plan, src, out=None, accumulate=False):
+    """``csr_gather_reduce`` over rows that live in up to 8 separate ``[rows_f, D]`` arrays (one
+    dtype): ``src`` numbers the rows of ``parts[0]``, then those of ``parts[1]``, ..."""
+    require_cuda(src, *parts)
+    parts = [_contig(p) for p in parts]
+    D, dt, dev = parts[0].shape[1], parts[0].dtype, parts[0].device
+    if any(p.dtype != dt or p.shape[1] != D for p in parts):
+        raise TypeError("csr_gather_reduce_parts: the parts must share dtype and row width")
+    if out is None:
+        out = torch.empty((plan.U, D), dtype=torch.float32, device=dev)
+        accumulate = False
+    check(lib().recis_csr_gather_reduce_parts(_host_ptrs(parts), _host_i64([p.shape[0] for p in parts]),
+                                              len(parts), dtype_code(dt), ptr(src), ptr(plan.row_start),
+                                              ptr(plan.hot_items), i64(plan.hot_cap), ptr(plan.counts), ptr(out),
+                                              i64(plan.U), i64(D), int(bool(accumulate)), stream_ptr(dev)))
+    return out
+
+
 def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_index=None, weight=None, out_dtype=None):
     """``out[i] = weight[i] * row(unique id of occurrence i)`` for the ``n_out`` occurrences of
     ``plan``: every unique row is read once and written to all its occurrences. Rows come from

@@ -306,3 +306,24 @@ def test_planned_tile_backward_matches_oracle(rng):
     got = ops.csr_gather_reduce(_dev(dy), p, src).cpu().numpy()
     exp = oracle.ragged_tile_back(batch, seq, inv, off, dy, p.U)
     np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [16, 128])
+def test_gather_reduce_over_separate_arrays_equals_the_concatenation(rng, dtype, D):
+    """recis_csr_gather_reduce_parts: the rows in up to 8 arrays, numbered end to end, against the
+    plain gather-reduce over their concatenation: same kernel arithmetic, so bit for bit."""
+    n = 60000
+    ids = np.concatenate([rng.integers(0, 40, n // 2), rng.integers(0, 20000, n - n // 2)])  # hot and cold rows
+    plan = ops.ids_unique_plan(_dev(ids))
+    counts = [7000, 1, 0, 25000, 12999, 15000]
+    assert sum(counts) == n
+    parts = [torch.randn((c, D), device="cuda").to(dtype) for c in counts]
+    src = torch.from_numpy(rng.permutation(n).astype(np.int32)).cuda()
+    src[::17] = -1                                            # skipped entries
+    whole = ops.csr_gather_reduce(torch.cat(parts), plan, src)
+    split = ops.csr_gather_reduce_parts(parts, plan, src)
+    assert torch.equal(split, whole)
+    again = ops.csr_gather_reduce_parts(parts, plan, src, out=split.clone(), accumulate=True)
+    torch.testing.assert_close(again, 2 * whole, rtol=1e-6, atol=1e-6)
+    assert _lib.poll_device_errors() == 0
