@@ -480,6 +480,39 @@ def test_engine_sequence_pooled_and_tiled_from_one_plan():
     torch.testing.assert_close(got, exp, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("n_feat,skip", [(3, None), (3, 1), (9, None)])
+def test_padded_gather_with_one_output_per_feature(n_feat, skip):
+    """RaggedTileParts against the single-output list form of the tile combiner: same rows, same
+    gradient of the unique rows, with all gradients present (one gather-reduce launch over separate
+    arrays), with one output unused, and with more features than one launch takes (a pass each)."""
+    from recis_amd import ops
+    from recis_amd.nn.functional.embedding_ops import RaggedTileParts
+
+    rng = np.random.default_rng(n_feat)
+    U, D = 50, 16
+    bs = [int(rng.integers(3, 9)) for _ in range(n_feat)]
+    tile_len = [int(rng.integers(1, 7)) for _ in range(n_feat)]
+    lens = rng.integers(0, 9, sum(bs))
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)).cuda()
+    ids = torch.from_numpy(rng.integers(0, 1000, int(off[-1]))).cuda()
+    plan = ops.ids_unique_plan(ids)
+    emb = torch.randn(plan.U, D, device="cuda")
+    e1 = emb.clone().requires_grad_()
+    parts = RaggedTileParts.apply(e1, plan.inverse, off, plan, bs, tile_len)
+    e2 = emb.clone().requires_grad_()
+    whole = ragged_embedding_segment_reduce(e2, None, plan.inverse, off, "tile", {"bs": bs, "tile_len": tile_len},
+                                            plan=plan)
+    rows = [b * t for b, t in zip(bs, tile_len)]
+    for part, ref, b, t in zip(parts, torch.split(whole, rows), bs, tile_len):
+        assert part.shape == (b, t * D) and torch.equal(part.detach().reshape(-1, D), ref.detach())
+    ups = [torch.randn(p.shape, device="cuda") for p in parts]
+    used = [k for k in range(n_feat) if k != skip]
+    torch.autograd.backward([parts[k] for k in used], [ups[k] for k in used])
+    g_whole = torch.cat([(ups[k] if k != skip else torch.zeros_like(ups[k])).reshape(-1, D) for k in range(n_feat)])
+    whole.backward(g_whole)
+    torch.testing.assert_close(e1.grad, e2.grad, rtol=1e-5, atol=1e-5)
+
+
 def test_feature_engine_ops_and_fusion():
     """Restated from tests/feature_engine/op_test.py:17-36,95-131 and feature_engine_test.py: Mod,
     Bucketize, IDMultiHash, Hash known answers, through the fused engine path."""
