@@ -1015,8 +1015,14 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
           const int64_t grid = (S + teams_per_block - 1) / teams_per_block;
           TOut* o = static_cast<TOut*>(out);
           const bool rev32 = a.weight == nullptr && a.rev != nullptr && !a.rev64;
+          const bool fast_blk = rev32 && U < (int64_t(1) << 31) && a.team_log2 > a.lpr_log2;
+          // segments of hundreds of rows: a workgroup each, as for dense rows below
+          const bool wg_blk = fast_blk && a.team_log2 == 6 && S > 0 && B / S >= 128 && D <= 4096;
           RECIS_TIME_KERNEL("seg_pool_fwd_kernel", stream)
-          if (rev32 && U < (int64_t(1) << 31) && a.team_log2 > a.lpr_log2)
+          if (wg_blk)
+            seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32, true, true><<<dim3(S), dim3(kBlock),
+                sizeof(float) * (kBlock / kWave) * static_cast<size_t>(D), stream>>>(nullptr, o, a);
+          else if (fast_blk)
             seg_pool_fwd_fast_kernel<TIn, TOut, VEC, kFastRev32, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(nullptr, o, a);
           else if (rev32)
             seg_pool_fwd_kernel<TIn, TOut, VEC, kFwdRev32, true><<<dim3(grid), dim3(kBlock), 0, stream>>>(nullptr, o, a);

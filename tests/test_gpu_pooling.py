@@ -388,3 +388,27 @@ def test_long_segments_workgroup_path(dtype, D):
     ref = torch.zeros(300, D, device="cuda", dtype=torch.float64).index_add_(0, seg, rows[rev].double())
     torch.testing.assert_close(plain.double(), ref, rtol=1e-5, atol=1e-3)
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [8, 128])
+def test_long_segments_out_of_the_table_blocks(dtype, D):
+    """The workgroup-per-segment pooling reading rows straight out of table blocks (row u = row
+    row_index[u], some keys absent) equals pooling the gathered copy of the same rows."""
+    g = torch.Generator(device="cuda").manual_seed(D)
+    lens = torch.randint(100, 700, (200,), generator=torch.Generator().manual_seed(D))
+    lens[::13] = 0
+    off = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).int().cuda()
+    n, U, block_rows, n_blocks = int(off[-1]), 3000, 512, 9
+    blocks = [torch.randn(block_rows, D, device="cuda", generator=g).to(dtype) for _ in range(n_blocks)]
+    row_index = torch.randint(0, block_rows * n_blocks, (U,), device="cuda", generator=g)
+    row_index[::41] = -1                                     # keys the table does not hold read as zeros
+    rev = torch.randint(0, U, (n,), device="cuda", generator=g).int()
+    table = torch.cat(blocks)
+    rows = torch.where(row_index.view(-1, 1) >= 0, table[row_index.clamp(min=0)], torch.zeros((), dtype=dtype, device="cuda"))
+    for mode in ("sum", "mean"):
+        direct = ops.segment_reduce_forward_blocks(blocks, block_rows, row_index, None, rev, off, mode,
+                                                   out_dtype=torch.float32)
+        copied = ops.segment_reduce_forward(rows, None, rev, off, mode, out_dtype=torch.float32)
+        assert torch.equal(direct, copied)                   # the same rows summed in the same order
+    assert _lib.poll_device_errors() == 0
