@@ -356,13 +356,19 @@ class Config4:
 # --------------------------------------------------------------------- config 3
 class Config3:
     """IDMap + EmbeddingBlocks at scale: 2e8 resident rows, dim 32 fp32 + two Adam state slots
-    (~77 GB), 2e6 lookups per step, Zipf(1.1), 10 % never-seen keys (admission inserts); rows are
-    expanded to one output row per lookup, the per-lookup gradients are reduced per key, fused
-    sparse Adam, last-seen-step stamp; eviction sweep (keys not seen for 50 steps) timed apart."""
+    (~77 GB), 2e6 lookups per step, Zipf(1.1) over the resident keys with 10 % of the positions
+    replaced by keys never seen before (admission inserts, on EVERY step: batches are never
+    replayed); rows are expanded to one output row per lookup, the per-lookup gradients are
+    reduced per key, fused sparse Adam; every looked-up row is stamped with the step; every
+    `filter_interval` steps the sweep of the step filter evicts the keys not seen for `filter_step`
+    steps (threshold = step - filter_step: recis/nn/modules/hashtable_hook_impl.py:527-551,
+    recis/hooks/filter_hook.py:82-117), frees their rows and re-initialises them. The resident
+    keys were last seen before step 0 (stamp -1)."""
 
-    name = "c3_idmap_blocks_2e8rows_d32_fp32_adam_2e6ids_zipf1.1_10pct_new"
+    name = "c3_idmap_blocks_2e8rows_d32_fp32_adam_2e6ids_zipf1.1_10pct_new_evict50"
 
-    def __init__(self, resident=200_000_000, ids_per_step=2_000_000, n_batches=8):
+    def __init__(self, resident=200_000_000, ids_per_step=2_000_000, n_batches=48, filter_step=50,
+                 filter_interval=50):
         from recis_amd import ops
         from recis_amd.nn.initializers import NormalInitializer
         from recis_amd.nn.modules.hashtable import HashtableImpl
@@ -370,35 +376,51 @@ class Config3:
         self.ops = ops
         self.D, self.N, self.resident = 32, ids_per_step, resident
         self.ids_per_step = ids_per_step
+        self.filter_step, self.filter_interval = filter_step, filter_interval
         init = NormalInitializer(0.0, 0.01)
         init.set_shape([10240, self.D])
         init.set_dtype(torch.float32)
         reserve = int(resident * 1.12) + 40 * ids_per_step // 10
         self.table = HashtableImpl(10240, [self.D], torch.float32, torch.device("cuda"), False, ["c3"],
                                    init.build().impl(), reserve_rows=reserve)
-        self.table.append_step_filter_slot("step_filter", 0)
+        self.table.append_step_filter_slot("step_filter", -1)
         self.opt = SparseAdamImpl.make({"c3": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0)
         chunk = 25_000_000
         for lo in range(0, resident, chunk):
             ranks = torch.arange(lo, min(lo + chunk, resident), device="cuda")
             self.table.insert_lookup_index(workloads.splitmix64_torch(ranks))
-        self.batches = workloads.config3_batches(n_batches, resident, ids_per_step)
+        self.batches = []          # batch k = the lookups of step k; its new keys were never seen before
+        self._gen = workloads.Config3Lookups(resident, ids_per_step)
+        self.prepare(n_batches)
         g = torch.Generator(device="cuda").manual_seed(3)
         self.grad_out = torch.randn((ids_per_step, self.D), device="cuda", generator=g)
         self.span = torch.tensor([0, ids_per_step], dtype=torch.int64, device="cuda")
         self.step_no = 0
         self.step_t = torch.zeros(1, dtype=torch.int64, device="cuda")
         self.U = None
+        self.sweeps = []           # (step, keys evicted, ms) of every sweep so far
         torch.cuda.synchronize()
+
+    def prepare(self, steps):
+        """Draws the lookups of the next `steps` steps (input generation, outside any timed region)."""
+        done = getattr(self, "step_no", 0)
+        while len(self.batches) < done + steps:
+            self.batches.append(self._gen.batch(len(self.batches)))
+        for k in range(max(0, done - 2)):   # batches of finished steps are not needed again
+            self.batches[k] = None
 
     def step(self):
         o = self.ops
-        ids = self.batches[self.step_no % len(self.batches)]
+        if self.step_no >= len(self.batches):
+            self.prepare(16)
+        ids = self.batches[self.step_no]
+        if self.step_no and self.step_no % self.filter_interval == 0:
+            self.sweep(self.step_no - self.filter_step)
         self.step_no += 1
         plan = o.ids_unique_plan(ids, wait=False)
         index_buf = self.table.lookup_index_counted(plan)   # queued before the host has the unique count
         self.U = plan.U
-        index = self.table.settle_lookup(index_buf, self.U)
+        index = self.table.settle_lookup(index_buf, self.U, plan)
         chunks, chunk_rows = self.table.emb_blocks()
         self.table.update_slot("step_filter", index, self.step_t)
         # one row per lookup: every unique row is read once out of the table and written to its
@@ -410,6 +432,25 @@ class Config3:
         self.opt.zero_grad()
         self.step_t += 1
         return out
+
+    def sweep(self, threshold):
+        """The eviction sweep of the step filter (one pass over the id map + re-initialisation of
+        the freed rows); records (step, evicted keys, ms)."""
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        gone, _ = self.table.evict_older("step_filter", threshold)
+        torch.cuda.synchronize()
+        self.sweeps.append((self.step_no, int(gone.numel()), (time.perf_counter() - t0) * 1e3))
+        return self.sweeps[-1]
+
+    def run_to_next_sweep(self):
+        """Steps (untimed by the caller) up to the next multiple of `filter_interval`, then that
+        step with its sweep; returns the sweep's record."""
+        before = len(self.sweeps)
+        self.prepare(self.filter_interval + 1)
+        while len(self.sweeps) == before:
+            self.step()
+        return self.sweeps[-1]
 
     def algorithmic_bytes(self):
         N, U, D = self.N, self.U, self.D
@@ -426,16 +467,6 @@ class Config3:
             "adamw_rows_kernel": U * (8 + D * 4 * 7),
             "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,
         }
-
-    def evict_sweep_ms(self, filter_step=50):
-        """One eviction sweep over the 2e8-row table (keys not seen for `filter_step` steps): the
-        one-pass library sweep. The threshold is set so that nothing is old enough: the sweep cost
-        without shrinking the table under the benchmark."""
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        self.table.evict_older("step_filter", -1)
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3
 
     def cpu_baseline(self, budget_s):
         from oracle import cpu_path

@@ -213,7 +213,10 @@ int recis_idmap_destroy(recis_idmap* m);
  * the rule of IdAllocator::GenIds (csrc/ops/hashtable_ops.cc:15-27): with n
  * missing keys, the k-th takes free_list[free - n + k] if that position is >= 0,
  * else the fresh index cur - (free - n + k + 1). A key repeated inside one call
- * gets one row. No host synchronisation unless the table must be rebuilt.
+ * gets one row; which of its occurrences stands for it in the ranking of the missing keys is
+ * not specified, so with duplicate NEW keys in one call the rows of those keys may come out
+ * permuted from run to run (callers on the hot path dedup first and never see this).
+ * No host synchronisation unless the table must be rebuilt.
  */
 int recis_idmap_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* index_out,
                        void* stream);
@@ -227,6 +230,11 @@ int recis_idmap_lookup_counted(recis_idmap* m, const int64_t* ids, int64_t n_max
 /* Tells the map the true size of the last recis_idmap_lookup_counted once the host knows it,
  * so that the bounds below stop counting all n_max ids of that call as possible new keys. */
 int recis_idmap_settle_count(recis_idmap* m, int64_t n_true);
+/* The same for callers with several counted lookups outstanding on one map (two embedding modules
+ * that share a table): recis_idmap_last_call gives the number of the call just queued on the map,
+ * recis_idmap_settle_call settles that call, whichever calls followed it. */
+int recis_idmap_last_call(recis_idmap* m, int64_t* seq);
+int recis_idmap_settle_call(recis_idmap* m, int64_t seq, int64_t n_true);
 /* Upper bounds, without waiting for any stream, of the allocator's high-water mark
  * (IdMap::GetIdNum, id_map.h:29) and of the occupied table slots: the values the last finished
  * call published to pinned host memory plus every id of the calls queued since. Either
@@ -407,6 +415,11 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
                       int64_t* unique_count_host, int flags, void* stream);
 /* Waits for the count staged by the last recis_unique_plan(…, RECIS_PLAN_STAGE_COUNT, stream). */
 int recis_unique_plan_count(int64_t* unique_count_host, void* stream);
+/* The soft-error bits (RECIS_DEVERR_*) that were set on the device when the last count of `stream`
+ * was staged; read from host memory, never waits, clears nothing. Lets a caller that fetches the
+ * staged count every step notice, one step late at most, what recis_hip_poll_device_errors would
+ * report after a device-wide wait. */
+int recis_hip_staged_device_errors(int* bits, void* stream);
 
 /*
  * Per list entry, the input row it reads and its coefficient, for the backward of

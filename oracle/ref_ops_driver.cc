@@ -253,12 +253,16 @@ static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
             table->GetSlot(prefix + "exp_avg_sq")->Value()};
   }
   if (op == "table_step_time") {
-    // Times the CPU-runnable parts of one training step of the reference on one Hashtable with
-    // SparseAdam: ids_partition_cpu (dedup) + EmbeddingLookup + AcceptGrad + step + zero_grad.
-    // (The pooling between lookup and gradient has no CPU operator in the reference.)
+    // Times one training step of the reference on one CPU Hashtable with SparseAdam:
+    // ids_partition_cpu (dedup) + EmbeddingLookup + [pooling forward and backward] + AcceptGrad + step +
+    // zero_grad. The reference has no CPU pooling OPERATOR (segment_ops.cc only forwards to CUDA); with
+    // segment ids given (in[2]) the pooling runs as the reference's own "torch" backend does on CPU tensors
+    // (recis/nn/functional/embedding_ops.py:59-66: data[indices] then index_add_ by segment id; backward
+    // = the transpose, grad_out[segment_ids] index_add_-ed by unique row), on torch's CPU thread pool.
     // params f64 [9] = block_size, D, lr, beta1, beta2, eps, weight_decay, time budget in seconds,
-    //                  threads;  ids i64 [n] = one step's ids (duplicates included)
-    // Returns f64 [3] = seconds, steps timed, unique ids per step. Gradients are a constant.
+    //                  threads;  ids i64 [n] = one step's ids (duplicates included);
+    // optional segment_ids i64 [n] (sorted, last + 1 = number of segments).
+    // Returns f64 [3] = seconds, steps timed, unique ids per step.
     const double* p = in[0].data_ptr<double>();
     const int64_t bs = static_cast<int64_t>(p[0]), D = static_cast<int64_t>(p[1]);
     at::set_num_threads(static_cast<int>(p[8]));
@@ -268,14 +272,29 @@ static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
     recis::optim::SparseAdamOptions o;
     o.lr(p[2]).betas(std::make_tuple(p[3], p[4])).eps(p[5]).weight_decay(p[6]);
     auto opt = c10::make_intrusive<recis::optim::SparseAdam>(tables, o);
+    const bool pool = in.size() > 2;
+    Tensor seg, up;
+    int64_t S = 0;
+    if (pool) {
+      seg = in[2];
+      S = seg.numel() ? seg[seg.numel() - 1].item<int64_t>() + 1 : 0;
+      up = torch::full({S, D}, 1e-3f);
+    }
     int64_t uniq = 0, steps = 0;
     Tensor grad;
     auto one_step = [&]() {
       auto part = F::ids_partition_cpu(in[1], 1);
       Tensor u = std::get<0>(part);
       uniq = u.numel();
-      if (!grad.defined() || grad.size(0) != uniq) grad = torch::full({uniq, D}, 1e-3f);
       auto r = table->EmbeddingLookup(u, false);
+      if (pool) {
+        Tensor inverse = std::get<2>(part).to(torch::kLong);
+        Tensor pooled = torch::zeros({S, D}).index_add_(0, seg, std::get<1>(r).index_select(0, inverse));
+        grad = torch::zeros({uniq, D}).index_add_(0, inverse, up.index_select(0, seg));
+        (void)pooled;
+      } else if (!grad.defined() || grad.size(0) != uniq) {
+        grad = torch::full({uniq, D}, 1e-3f);
+      }
       table->AcceptGrad(std::get<0>(r), grad);
       opt->step();
       opt->zero_grad();
@@ -391,6 +410,33 @@ static std::vector<Tensor> run(const std::string& op, std::vector<Tensor> in) {
     std::vector<Tensor> a(in.begin(), in.begin() + k), m(in.begin() + k, in.begin() + 2 * k),
         p(in.begin() + 2 * k, in.begin() + 3 * k), b(in.begin() + 3 * k, in.end());
     return F::fused_multi_hash(a, m, p, b);
+  }
+  if (op == "generate") {
+    // params f64 [10] = kind, rows, dim, seed, p0, p1, p2, p3, fan mode (0 in, 1 out), generate rows (0 = own shape).
+    // kind: 0 constant(p0) 1 uniform(p0, p1) 2 normal(p0, p1) 3 xavier_uniform(gain p0) 4 xavier_normal(gain p0)
+    // 5 kaiming_uniform(a p0) 6 kaiming_normal(a p0) 7 trunc_normal(mean p0, std p1, a p2, b p3); the
+    // Kaiming generators with leaky_relu. Seeds torch's default generator, then calls the reference's
+    // generator (csrc/embedding/initializer.cc:26-366) once.
+    using namespace recis::embedding;
+    const double* q = in[0].data_ptr<double>();
+    const int kind = static_cast<int>(q[0]);
+    const std::vector<int64_t> shape = {static_cast<int64_t>(q[1]), static_cast<int64_t>(q[2])};
+    const std::string mode = q[8] != 0 ? "fan_out" : "fan_in";
+    torch::intrusive_ptr<Generator> g;
+    switch (kind) {
+      case 0: g = MakeConstantGenerator(shape, at::kFloat, q[4]); break;
+      case 1: g = MakeUniformGenerator(shape, at::kFloat, q[4], q[5], c10::nullopt); break;
+      case 2: g = MakeNormalGenerator(shape, at::kFloat, q[4], q[5], c10::nullopt); break;
+      case 3: g = MakeXavierUniFormGenerator(shape, at::kFloat, q[4], c10::nullopt); break;
+      case 4: g = MakeXavierNormalGenerator(shape, at::kFloat, q[4], c10::nullopt); break;
+      case 5: g = MakeKaimingUniformGenerator(shape, at::kFloat, q[4], mode, "leaky_relu", c10::nullopt); break;
+      case 6: g = MakeKaimingNormalGenerator(shape, at::kFloat, q[4], mode, "leaky_relu", c10::nullopt); break;
+      case 7: g = MakeTruncNormalGenerator(shape, at::kFloat, q[4], q[5], q[6], q[7], c10::nullopt); break;
+      default: TORCH_CHECK(false, "bad generator kind ", kind);
+    }
+    torch::manual_seed(static_cast<uint64_t>(q[3]));
+    if (q[9] != 0) return {g->Generate({static_cast<int64_t>(q[9]), shape[1]})};
+    return {g->Generate()};
   }
   TORCH_CHECK(false, "unknown op ", op);
 }

@@ -101,3 +101,22 @@ def poll_device_errors():
     bits = ctypes.c_int(0)
     check(lib().recis_hip_poll_device_errors(ctypes.byref(bits)))
     return bits.value
+
+
+DEVERR_TEXT = ((DEVERR_INDEX_RANGE, "an index outside the rows / blocks the caller passed"),
+               (DEVERR_OFFSETS, "offsets not monotone or out of range"),
+               (DEVERR_TABLE_FULL, "the id map found no free slot"),
+               (DEVERR_PLAN_OVERFLOW, "batch plan: too many distinct ids in one hash bucket"))
+
+
+def describe_device_errors(bits):
+    return "; ".join(t for b, t in DEVERR_TEXT if bits & b) + " (bits %d)" % bits
+
+
+def raise_device_errors(extra_bits=0):
+    """Waits for the device, clears the soft-error word and raises if any kernel since the last
+    poll skipped a faulty access (bad row index, full id map, ...). For host code that waits for
+    the device anyway: table statistics, checkpoint save / load."""
+    bits = poll_device_errors() | extra_bits
+    if bits:
+        raise RecisHipError("device-side errors in earlier kernels: " + describe_device_errors(bits))

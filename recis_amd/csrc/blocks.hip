@@ -169,7 +169,7 @@ int fill_args(BlockArgs& a, const int64_t* ids, void* const* blocks_dev, int64_t
   a.row_bytes = static_cast<int>(row_bytes);
   a.lpr_log2 = std::min(6, ilog2_ceil((row_bytes + vb - 1) / vb));
   a.err = device_error_word(current_device());
-  RECIS_REQUIRE(a.err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
   return RECIS_OK;
 }
 
@@ -190,7 +190,7 @@ int recis_gather(const void* ids, int ids_is64, const void* emb, int64_t rows, v
   const int vb = pick_vec_bytes(row_bytes, reinterpret_cast<uintptr_t>(emb) | reinterpret_cast<uintptr_t>(out));
   const int lpr_log2 = std::min(6, ilog2_ceil((row_bytes + vb - 1) / vb));
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   const int rows_per_block = kBlock >> lpr_log2;
   const int64_t grid = (n + rows_per_block - 1) / rows_per_block;
   return dispatch_vb(vb, [&](auto tag) {

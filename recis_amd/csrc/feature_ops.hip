@@ -272,7 +272,7 @@ int recis_fused_hash(const int8_t* const* values_ptrs, const int64_t* values_siz
   if (n_tensors == 0) return RECIS_OK;
   RECIS_REQUIRE(values_ptrs && values_sizes && offsets_ptrs && n_strings && out_ptrs, "NULL argument");
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   for (int64_t base = 0; base < n_tensors; base += kMaxJobs) {
     Jobs j;
     const int cnt = static_cast<int>(std::min<int64_t>(kMaxJobs, n_tensors - base));

@@ -13,7 +13,9 @@
 //     insert+sync-per-submap sequence
 //   * row indices are assigned exactly as IdAllocator::GenIds does: missing keys
 //     are ranked in input order; rank i of n takes free_list[free - n + i] when
-//     that index is >= 0, else the fresh index cur - (free - n + i + 1)
+//     that index is >= 0, else the fresh index cur - (free - n + i + 1). A missing
+//     key that occurs more than once in a call is ranked at whichever occurrence
+//     wins the claim, so only duplicate-free calls have a reproducible assignment
 //   * erase leaves tombstones, later inserts reuse them; the table is rebuilt
 //     (sized up) only when live + tombstones would pass the load limit
 #include <hip/hip_runtime.h>
@@ -650,7 +652,7 @@ int recis_idmap_create(int64_t reserve_keys, recis_idmap** out) {
   m->err = device_error_word(m->device);
   if (!m->err) {
     delete m;
-    return fail(RECIS_ERR_HIP, "could not allocate the device error word");
+    return fail(RECIS_ERR_HIP, "could not reach the device error word");
   }
   // The reference starts at 640000 slots (gpu_id_map.h:12); we start at the
   // next power of two unless the caller reserves more.
@@ -743,6 +745,23 @@ int recis_idmap_settle_count(recis_idmap* m, int64_t n_true) {
   return RECIS_OK;
 }
 
+int recis_idmap_last_call(recis_idmap* m, int64_t* seq) {
+  RECIS_REQUIRE(m != nullptr && seq != nullptr, "bad arguments");
+  *seq = m->seq_issued;
+  return RECIS_OK;
+}
+
+int recis_idmap_settle_call(recis_idmap* m, int64_t seq, int64_t n_true) {
+  RECIS_REQUIRE(m != nullptr && n_true >= 0, "bad arguments");
+  for (auto& c : m->in_flight) {
+    if (c.first == seq) {
+      if (c.second > n_true) c.second = n_true;
+      break;
+    }
+  }
+  return RECIS_OK;  // a call whose publication has landed is not in the list any more: nothing to settle
+}
+
 int recis_idmap_bounds(recis_idmap* m, int64_t* id_num_ub, int64_t* occupied_ub) {
   RECIS_REQUIRE(m != nullptr, "id map is NULL");
   mirror_bounds(m, occupied_ub, id_num_ub);
@@ -818,7 +837,7 @@ int recis_idmap_evict_older(recis_idmap* m, const void* const* stamp_blocks_dev,
   *count = 0;
   if (max_out == 0) return RECIS_OK;
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   if (int rc = ensure_free_room(m, max_out, stream)) return rc;
   evict_older_kernel<<<dim3(blocks_for(m->capacity)), dim3(kBlock), 0, stream>>>(
       m->table, m->capacity, stamp_blocks_dev, n_blocks, block_rows, stamp_is64, threshold, ids_out, index_out,

@@ -182,7 +182,7 @@ int fill_opt_args(OptArgs& a, const int64_t* index, const void* grad, int64_t n,
   a.D = static_cast<int>(D);
   a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
   a.err = device_error_word(current_device());
-  RECIS_REQUIRE(a.err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
   return RECIS_OK;
 }
 

@@ -207,7 +207,7 @@ plan_colscan_kernel(const uint16_t* __restrict__ hist, PlanGeom g, int32_t* __re
 __global__ void __launch_bounds__(1024)
 plan_scan_kernel(const int32_t* __restrict__ in0, int32_t* __restrict__ out0, const int32_t* __restrict__ in1,
                  int32_t* __restrict__ out1, int nb, int64_t* __restrict__ total_out,
-                 volatile int64_t* total_host) {
+                 volatile int64_t* total_host, const int* __restrict__ err) {
   __shared__ int32_t partial[1024];
   const int t = threadIdx.x;
   const int per = (nb + 1023) / 1024;
@@ -235,7 +235,10 @@ plan_scan_kernel(const int32_t* __restrict__ in0, int32_t* __restrict__ out0, co
     if (t == 1023) {
       out[nb] = partial[1023];
       if (pass == 0 && total_out) total_out[0] = partial[1023];
-      if (pass == 0 && total_host) total_host[0] = partial[1023];  // pinned host word: no copy kernel needed
+      if (pass == 0 && total_host) {  // pinned host words: no copy kernel needed
+        total_host[1] = err ? __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+        total_host[0] = partial[1023];
+      }
     }
     __syncthreads();
   }
@@ -483,9 +486,16 @@ plan_bucket_kernel(const Rec* __restrict__ bucket_rec, const int32_t* __restrict
   }
 }
 
-__global__ void plan_empty_kernel(int64_t* __restrict__ counts, int32_t* __restrict__ row_start) {
+__global__ void plan_empty_kernel(int64_t* __restrict__ counts, int32_t* __restrict__ row_start,
+                                  volatile int64_t* total_host, const int* __restrict__ err) {
   if (threadIdx.x < 2) counts[threadIdx.x] = 0;
-  if (threadIdx.x == 0) row_start[0] = 0;
+  if (threadIdx.x == 0) {
+    row_start[0] = 0;
+    if (total_host) {
+      total_host[1] = err ? __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+      total_host[0] = 0;
+    }
+  }
 }
 
 // emit, per occurrence: inverse, list entry, position in the list
@@ -1095,31 +1105,16 @@ using namespace recis_hip;
 
 extern "C" {
 
-int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
-                      int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
-                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* unique_count_host, int flags, void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  RECIS_REQUIRE(n >= 0 && n < (int64_t(1) << 30), "n out of range: %lld", (long long)n);
-  RECIS_REQUIRE(counts_out_dev && row_start_out, "counts_out_dev / row_start_out must not be NULL");
-  RECIS_REQUIRE(hot_cap == 0 || (hot_items_out && hot_cap >= n / kHotLen + n / kHotChunk + 2),
-                "hot_items_out must hold at least n/%d + n/%d + 2 items", kHotLen, kHotChunk);
-  RECIS_REQUIRE(n == 0 || (ids && unique_out && inverse_out && list_out), "NULL argument");
-  int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
-  if (n == 0) {
-    plan_empty_kernel<<<1, 64, 0, stream>>>(counts_out_dev, row_start_out);
-    RECIS_LAUNCH_CHECK();
-    if (unique_count_host) *unique_count_host = 0;
-    if (flags & RECIS_PLAN_STAGE_COUNT) {
-      int64_t* staged = nullptr;
-      hipEvent_t staged_event = nullptr;
-      if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
-      RECIS_CHECK_HIP(hipMemcpyAsync(staged, counts_out_dev, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
-      RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
-    }
-    return RECIS_OK;
-  }
+// Where the plan's scratch arrays lie in one buffer of `bytes` bytes, for n ids.
+struct PlanLayout {
   PlanGeom g;
+  int64_t nb;
+  size_t o_tile, o_brec, o_res, o_occ, o_hist, o_off, o_nrec, o_small, bytes;
+};
+
+static PlanLayout plan_layout(int64_t n) {
+  PlanLayout L;
+  PlanGeom& g = L.g;
   g.n = n;
   g.tiles = static_cast<int>((n + kPlanBlock - 1) / kPlanBlock);
   g.tiles_per_wg = std::min(63, (g.tiles + kMaxRows - 1) / kMaxRows);  // 16-bit histogram counters
@@ -1129,31 +1124,55 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
   int nb_log2 = 5;
   while ((int64_t(1) << (nb_log2 + 1)) <= kMaxBuckets && (int64_t(1) << (nb_log2 + 1)) * 512 <= n) ++nb_log2;
   g.nb_log2 = nb_log2;
-  const int64_t nb = int64_t(1) << nb_log2;
+  L.nb = int64_t(1) << nb_log2;
   const int64_t n_pad = static_cast<int64_t>(g.tiles) * kPlanBlock;
-  // workspace: tile_rec[n_pad] (later: the unique ids of every bucket) | bucket_rec[n_pad] | result[n_pad] |
-  //            occ_rec[n] | hist[rows*nb] u16 | off[rows*nb] | tile_nrec[tiles] | 6 arrays of nb + 1
+  // tile_rec[n_pad] (later: the unique ids of every bucket) | bucket_rec[n_pad] | result[n_pad] |
+  // occ_rec[n] | hist[rows*nb] u16 | off[rows*nb] | tile_nrec[tiles] | 6 arrays of nb + 1
   size_t bytes = 0;
   auto take = [&](size_t b) {
     const size_t at = bytes;
     bytes += (b + 255) & ~size_t(255);
     return at;
   };
-  const size_t o_tile = take(sizeof(Rec) * n_pad), o_brec = take(sizeof(Rec) * n_pad);
-  const size_t o_res = take(sizeof(int2) * n_pad), o_occ = take(sizeof(uint32_t) * n_pad);
-  const size_t o_hist = take(sizeof(uint16_t) * g.rows * nb), o_off = take(sizeof(int32_t) * g.rows * nb);
-  const size_t o_nrec = take(sizeof(int32_t) * g.tiles), o_small = take(sizeof(int32_t) * 6 * (nb + 1));
-  void* ws = nullptr;
-  if (int rc = get_workspace(stream, bytes, &ws)) return rc;
-  char* base = static_cast<char*>(ws);
-  Rec* tile_rec = reinterpret_cast<Rec*>(base + o_tile);
-  Rec* bucket_rec = reinterpret_cast<Rec*>(base + o_brec);
-  int2* result = reinterpret_cast<int2*>(base + o_res);
-  uint32_t* occ_rec = reinterpret_cast<uint32_t*>(base + o_occ);
-  uint16_t* hist = reinterpret_cast<uint16_t*>(base + o_hist);
-  int32_t* off = reinterpret_cast<int32_t*>(base + o_off);
-  int32_t* tile_nrec = reinterpret_cast<int32_t*>(base + o_nrec);
-  int32_t* bucket_total = reinterpret_cast<int32_t*>(base + o_small);
+  L.o_tile = take(sizeof(Rec) * n_pad);
+  L.o_brec = take(sizeof(Rec) * n_pad);
+  L.o_res = take(sizeof(int2) * n_pad);
+  L.o_occ = take(sizeof(uint32_t) * n_pad);
+  L.o_hist = take(sizeof(uint16_t) * g.rows * L.nb);
+  L.o_off = take(sizeof(int32_t) * g.rows * L.nb);
+  L.o_nrec = take(sizeof(int32_t) * g.tiles);
+  L.o_small = take(sizeof(int32_t) * 6 * (L.nb + 1));
+  L.bytes = bytes;
+  return L;
+}
+
+static int plan_check_args(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
+                           int32_t* row_start_out, int32_t* list_out, int32_t* hot_items_out, int64_t hot_cap,
+                           int64_t* counts_out_dev) {
+  RECIS_REQUIRE(n >= 0 && n < (int64_t(1) << 30), "n out of range: %lld", (long long)n);
+  RECIS_REQUIRE(counts_out_dev && row_start_out, "counts_out_dev / row_start_out must not be NULL");
+  RECIS_REQUIRE(hot_cap == 0 || (hot_items_out && hot_cap >= n / kHotLen + n / kHotChunk + 2),
+                "hot_items_out must hold at least n/%d + n/%d + 2 items", kHotLen, kHotChunk);
+  RECIS_REQUIRE(n == 0 || (ids && unique_out && inverse_out && list_out), "NULL argument");
+  return RECIS_OK;
+}
+
+// The plan's launches for n > 0 over the scratch buffer `base` (L.bytes bytes). `staged`: pinned host
+// word that receives the unique count as soon as it is final, or NULL.
+static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int64_t* unique_out,
+                       int32_t* inverse_out, int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
+                       int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev, int64_t* staged,
+                       hipEvent_t staged_event, int* err, hipStream_t stream) {
+  const PlanGeom& g = L.g;
+  const int64_t nb = L.nb, n = g.n;
+  Rec* tile_rec = reinterpret_cast<Rec*>(base + L.o_tile);
+  Rec* bucket_rec = reinterpret_cast<Rec*>(base + L.o_brec);
+  int2* result = reinterpret_cast<int2*>(base + L.o_res);
+  uint32_t* occ_rec = reinterpret_cast<uint32_t*>(base + L.o_occ);
+  uint16_t* hist = reinterpret_cast<uint16_t*>(base + L.o_hist);
+  int32_t* off = reinterpret_cast<int32_t*>(base + L.o_off);
+  int32_t* tile_nrec = reinterpret_cast<int32_t*>(base + L.o_nrec);
+  int32_t* bucket_total = reinterpret_cast<int32_t*>(base + L.o_small);
   int32_t* bucket_start = bucket_total + (nb + 1);
   int32_t* ucnt = bucket_start + (nb + 1);
   int32_t* ocnt = ucnt + (nb + 1);
@@ -1173,7 +1192,7 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
     RECIS_LAUNCH_CHECK();
   }
   plan_scan_kernel<<<1, 1024, 0, stream>>>(bucket_total, bucket_start, nullptr, nullptr, static_cast<int>(nb),
-                                           nullptr, nullptr);
+                                           nullptr, nullptr, nullptr);
   RECIS_LAUNCH_CHECK();
   {
     RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
@@ -1187,18 +1206,13 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
                                                                    ucnt, ocnt, err);
     RECIS_LAUNCH_CHECK();
   }
-  // The count is final after this scan: the kernel stores it into pinned host memory as well, and
-  // the host waits for it only after the emit kernels are queued, so that the GPU works while
-  // the host learns the size of the next launches.
-  int64_t* staged = nullptr;
-  hipEvent_t staged_event = nullptr;
-  const bool stage = unique_count_host || (flags & RECIS_PLAN_STAGE_COUNT);
-  if (stage) {
-    if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
-  }
-  plan_scan_kernel<<<1, 1024, 0, stream>>>(ucnt, ubase, ocnt, lbase, static_cast<int>(nb), counts_out_dev, staged);
+  // The count is final after this scan: the kernel stores it into pinned host memory as well (with
+  // the soft-error bits raised so far), and the host waits for it only after the emit kernels are
+  // queued, so that the GPU works while the host learns the size of the next launches.
+  plan_scan_kernel<<<1, 1024, 0, stream>>>(ucnt, ubase, ocnt, lbase, static_cast<int>(nb), counts_out_dev, staged,
+                                           err);
   RECIS_LAUNCH_CHECK();
-  if (stage) RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
+  if (staged) RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
   {
     const int64_t tail_blocks = (n + 1 + kBlock * 16 - 1) / (kBlock * 16);
     const int64_t uniq_blocks = nb + tail_blocks, occ_blocks = (n + kBlock - 1) / kBlock;
@@ -1208,9 +1222,40 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
         row_start_out, list_out, pos_out, counts_out_dev, hot_items_out, hot_cap);
     RECIS_LAUNCH_CHECK();
   }
+  return RECIS_OK;
+}
+
+int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
+                      int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
+                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* unique_count_host, int flags, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = plan_check_args(ids, n, unique_out, inverse_out, row_start_out, list_out, hot_items_out, hot_cap,
+                               counts_out_dev))
+    return rc;
+  int* err = device_error_word(current_device());
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
+  const bool stage = unique_count_host || (flags & RECIS_PLAN_STAGE_COUNT);
+  int64_t* staged = nullptr;
+  hipEvent_t staged_event = nullptr;
+  if (stage) {
+    if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
+  }
+  if (n == 0) {
+    plan_empty_kernel<<<1, 64, 0, stream>>>(counts_out_dev, row_start_out, staged, err);
+    RECIS_LAUNCH_CHECK();
+    if (stage) RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
+    if (unique_count_host) *unique_count_host = 0;
+    return RECIS_OK;
+  }
+  const PlanLayout L = plan_layout(n);
+  void* ws = nullptr;
+  if (int rc = get_workspace(stream, L.bytes, &ws)) return rc;
+  if (int rc = plan_launch(L, static_cast<char*>(ws), ids, unique_out, inverse_out, row_start_out, list_out, pos_out,
+                           hot_items_out, hot_cap, counts_out_dev, staged, staged_event, err, stream))
+    return rc;
   if (unique_count_host) {
     RECIS_CHECK_HIP(hipEventSynchronize(staged_event));
-    *unique_count_host = *staged;
+    *unique_count_host = staged[0];
   }
   return RECIS_OK;
 }
@@ -1222,7 +1267,17 @@ int recis_unique_plan_count(int64_t* unique_count_host, void* stream_) {
   hipEvent_t staged_event = nullptr;
   if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
   RECIS_CHECK_HIP(hipEventSynchronize(staged_event));
-  *unique_count_host = *staged;
+  *unique_count_host = staged[0];
+  return RECIS_OK;
+}
+
+int recis_hip_staged_device_errors(int* bits, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(bits != nullptr, "bits must not be NULL");
+  int64_t* staged = nullptr;
+  hipEvent_t staged_event = nullptr;
+  if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
+  *bits = static_cast<int>(staged[1]);
   return RECIS_OK;
 }
 
@@ -1333,7 +1388,7 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
   a.accumulate = accumulate;
   a.nt_in = n_rows * D * in_sz >= (int64_t(1) << 30);
   a.err = device_error_word(current_device());
-  RECIS_REQUIRE(a.err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
   const int rows_per_block = kBlock >> a.lpr_log2;
   a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
   a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
@@ -1430,7 +1485,7 @@ int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t
   a.D = static_cast<int>(D);
   a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
   a.err = device_error_word(current_device());
-  RECIS_REQUIRE(a.err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
   a.row_index = row_index;
   a.blocks = emb_blocks_dev;
   a.block_rows = block_rows;

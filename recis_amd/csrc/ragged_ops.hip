@@ -209,7 +209,7 @@ int recis_ragged_tile(const int64_t* batch, const int64_t* seq, int64_t n_featur
   const int esz = dtype_size(dtype);
   RECIS_REQUIRE(esz, "invalid dtype %d", dtype);
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   const int vb = pick_vec_bytes(D * esz, reinterpret_cast<uintptr_t>(table) | reinterpret_cast<uintptr_t>(out));
   const int vec = std::max(1, vb / esz);
   const int lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
@@ -264,7 +264,7 @@ int recis_ragged_tile_back(const int64_t* batch, const int64_t* seq, int64_t n_f
   if (n_features == 0) return RECIS_OK;
   RECIS_REQUIRE(batch && seq && offset, "NULL argument");
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   const int vb = pick_vec_bytes(D * esz, reinterpret_cast<uintptr_t>(dy));
   const int vec = std::max(1, vb / esz);
   const int lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
@@ -313,7 +313,7 @@ int recis_segment_sum(const void* data, int dtype, int64_t data_rows, const void
   RECIS_REQUIRE(data && indices && segment_ids, "NULL argument");
   RECIS_REQUIRE(weight == nullptr || dtype_size(weight_dtype), "invalid weight dtype");
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   const int vb = pick_vec_bytes(D * esz, reinterpret_cast<uintptr_t>(data));
   const int vec = std::max(1, vb / esz);
   const int lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));

@@ -539,7 +539,7 @@ extern "C" int recis_ragged_to_dense(const void* values, int elem_size, int64_t 
   if (a.batch * a.folded == 0) return RECIS_OK;
   RECIS_REQUIRE(out && (n_values == 0 || values), "NULL tensor pointer");
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   switch (elem_size) {
     case 1: return ragged_to_dense_launch<uint8_t>(values, out, a, off_is64, default_value, err, stream);
     case 2: return ragged_to_dense_launch<uint16_t>(values, out, a, off_is64, default_value, err, stream);
@@ -619,7 +619,7 @@ extern "C" int recis_ragged_cutoff_rows(const void* const* outer_ptrs, const voi
   const bool three_d = inner_ptrs != nullptr;
   RECIS_REQUIRE(!three_d || (n_inner_rows && out_outer_ptrs), "3-D cutoff needs inner row counts and outer outputs");
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   for (int64_t first = 0; first < n_tensors; first += kCutJobs) {
     CutJobs j;
     const int cnt = static_cast<int>(std::min<int64_t>(kCutJobs, n_tensors - first));
@@ -746,7 +746,7 @@ extern "C" int recis_feature_cross_rows(const int64_t* x_val, const void* x_off,
   RECIS_REQUIRE(n_seg == 0 || (x_off && y_off && y_count), "NULL offsets pointer");
   RECIS_REQUIRE((nx == 0 || (x_val && x_rank)) && (ny == 0 || (y_val && y_rank)), "NULL values pointer");
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   CutJobs j;
   j.out_off[0] = out_offsets;
   j.out_rows[0] = n_seg;
@@ -839,7 +839,7 @@ extern "C" int recis_ragged_topk_index(const void* drop_num, int drop_is64, cons
   const int64_t gw = (rows * kWave + kBlock - 1) / kBlock;
   RECIS_REQUIRE(gw < (int64_t(1) << 31), "too many rows");
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   if (nb > 0) {
     RECIS_TIME_KERNEL("topk_index_kernel(count)", stream) {
       topk_index_kernel<false><<<dim3(static_cast<unsigned>(gw)), dim3(kBlock), 0, stream>>>(a, out_offsets, nullptr, err);

@@ -37,17 +37,26 @@ int current_device() {
 }
 
 static std::mutex g_mu;
-static std::map<int, int*> g_err_words;
+
+// The soft-error word lives in the code object of this library (one copy per device that loads
+// it), so reaching it never allocates: entry points that must not allocate can use it too.
+static __device__ int g_error_word[4];
+constexpr int kMaxDevices = 64;
+static int* g_err_words[kMaxDevices];
 
 int* device_error_word(int device) {
+  if (device < 0 || device >= kMaxDevices) return nullptr;
   std::lock_guard<std::mutex> l(g_mu);
-  auto it = g_err_words.find(device);
-  if (it != g_err_words.end()) return it->second;
-  int* p = nullptr;
-  if (hipMalloc(reinterpret_cast<void**>(&p), sizeof(int)) != hipSuccess) return nullptr;
-  if (hipMemset(p, 0, sizeof(int)) != hipSuccess) return nullptr;
-  g_err_words[device] = p;
-  return p;
+  if (g_err_words[device]) return g_err_words[device];
+  int cur = -1;
+  if (hipGetDevice(&cur) != hipSuccess) return nullptr;
+  if (cur != device && hipSetDevice(device) != hipSuccess) return nullptr;
+  void* p = nullptr;
+  const hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(g_error_word));
+  if (cur != device) (void)hipSetDevice(cur);
+  if (rc != hipSuccess) return nullptr;
+  g_err_words[device] = static_cast<int*>(p);
+  return g_err_words[device];
 }
 
 struct Workspace {
@@ -90,6 +99,7 @@ int get_count_staging(hipStream_t stream, int64_t** host, hipEvent_t* event) {
   CountStaging& c = g_staging[std::make_pair(dev, stream)];
   if (c.host == nullptr) {
     RECIS_CHECK_HIP(hipHostMalloc(reinterpret_cast<void**>(&c.host), 64, hipHostMallocDefault));
+    for (int w = 0; w < 8; ++w) c.host[w] = 0;
     RECIS_CHECK_HIP(hipEventCreateWithFlags(&c.event, hipEventDisableTiming));
   }
   *host = c.host;
@@ -170,7 +180,7 @@ int recis_hip_poll_device_errors(int* bits) {
   RECIS_REQUIRE(bits != nullptr, "bits must not be NULL");
   int dev = current_device();
   int* w = device_error_word(dev);
-  RECIS_REQUIRE(w != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(w != nullptr, "could not reach the device error word");
   RECIS_CHECK_HIP(hipDeviceSynchronize());
   RECIS_CHECK_HIP(hipMemcpy(bits, w, sizeof(int), hipMemcpyDeviceToHost));
   if (*bits) RECIS_CHECK_HIP(hipMemset(w, 0, sizeof(int)));

@@ -956,7 +956,7 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
   RECIS_REQUIRE(in_sz && out_sz, "invalid dtype (emb=%d out=%d)", emb_dtype, out_dtype);
 
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
 
   // vector width in elements, limited by both row widths and pointer alignment
   // (blocks are 16-byte aligned by contract)
@@ -1126,7 +1126,7 @@ extern "C" int recis_segment_reduce_backward(
                 out_dtype);
 
   int* err = device_error_word(current_device());
-  RECIS_REQUIRE(err != nullptr, "could not allocate the device error word");
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
 
   const int vb_in = pick_vec_bytes(D * in_sz, reinterpret_cast<uintptr_t>(grad_out));
   const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(grad_unique));

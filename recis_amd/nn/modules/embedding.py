@@ -159,7 +159,7 @@ class LookupPoolFunction(torch.autograd.Function):
     def backward(ctx, _grad_index, grad):
         index, weight, offsets = ctx.saved_tensors
         if ctx.late_count:
-            ctx.impl.settle_count(ctx.plan.U)
+            ctx.impl.settle_count(ctx.plan.U, ctx.plan)
             index = index[: ctx.plan.U]
         g = ops.segment_reduce_backward_plan(grad.contiguous(), weight, offsets, ctx.plan, ctx.combiner)
         if ctx.readonly:  # keys the table does not hold take no gradient

@@ -188,7 +188,9 @@ class Slot:
 
     def _ensure_chunks(self, n_chunks):
         while len(self._chunks) < n_chunks:
-            self._chunks.append(self._generator.generate([self._chunk_rows] + self._row_shape))
+            # one tensor for several blocks; fan-dependent initialisers still see one [block_size, D] block
+            self._chunks.append(self._generator.generate([self._chunk_rows] + self._row_shape,
+                                                         fan_shape=[self._block_size] + self._row_shape))
 
     def _clear(self):
         self._chunks = []
@@ -389,7 +391,9 @@ class HashtableImpl:
     def lookup_index_counted(self, plan):
         """Queue the find-or-insert of a plan's unique ids before the host knows how many
         there are; finish with ``settle_lookup`` once ``plan.U`` has been read."""
-        return self._idmap.lookup_counted(plan.unique_buf, plan.counts)
+        index_buf = self._idmap.lookup_counted(plan.unique_buf, plan.counts)
+        plan.lookup_calls[id(self)] = self._idmap.last_call()
+        return index_buf
 
     def lookup_index_unsettled(self, plan):
         """``lookup_index_counted`` for consumers that take the unique count from device memory: the
@@ -397,14 +401,16 @@ class HashtableImpl:
         Returns the full-length index buffer (its first ``plan.U`` entries are the rows); settle
         with ``settle_count`` whenever the count has been read."""
         index_buf = self._idmap.lookup_counted(plan.unique_buf, plan.counts)
+        plan.lookup_calls[id(self)] = self._idmap.last_call()
         self._make_room(plan.n)
         return index_buf
 
-    def settle_count(self, n_true):
-        self._idmap.settle_count(n_true)
+    def settle_count(self, n_true, plan=None):
+        """The true size of the counted lookup queued for ``plan`` (default: of the last one)."""
+        self._idmap.settle_count(n_true, None if plan is None else plan.lookup_calls.get(id(self)))
 
-    def settle_lookup(self, index_buf, n_true):
-        self._idmap.settle_count(n_true)
+    def settle_lookup(self, index_buf, n_true, plan=None):
+        self.settle_count(n_true, plan)
         self._make_room(n_true)
         return index_buf[:n_true]
 
@@ -671,7 +677,7 @@ class LookupExpandFunction(torch.autograd.Function):
             index = impl.lookup_index(plan.unique, True)
         else:
             index_buf = impl.lookup_index_counted(plan)   # queued before the host has the unique count
-            index = impl.settle_lookup(index_buf, plan.U)
+            index = impl.settle_lookup(index_buf, plan.U, plan)
         chunks, chunk_rows = impl.emb_blocks()
         out = ops.plan_expand_rows(plan, plan.inverse.numel(), blocks=chunks, block_size=chunk_rows, row_index=index)
         ctx.impl, ctx.plan, ctx.slice_num, ctx.readonly = impl, plan, slice_num, readonly

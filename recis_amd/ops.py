@@ -653,8 +653,18 @@ class IdMap:
                                                stream_ptr(self.device)))
         return out
 
-    def settle_count(self, n_true):
-        check(lib().recis_idmap_settle_count(self._h, i64(n_true)))
+    def last_call(self):
+        """Number of the call just queued on this map (for ``settle_count(..., call=)``)."""
+        seq = ctypes.c_int64(0)
+        check(lib().recis_idmap_last_call(self._h, ctypes.byref(seq)))
+        return seq.value
+
+    def settle_count(self, n_true, call=None):
+        """Tell the map how many ids counted lookup number ``call`` (default: the last one) held."""
+        if call is None:
+            check(lib().recis_idmap_settle_count(self._h, i64(n_true)))
+        else:
+            check(lib().recis_idmap_settle_call(self._h, i64(call), i64(n_true)))
 
     def id_num_bound(self):
         """Upper bound of ``id_num()`` without waiting for the device."""
@@ -679,6 +689,7 @@ class IdMap:
         """(live keys, allocator high-water mark, free-list length, slot capacity); synchronises."""
         vals = [ctypes.c_int64(0) for _ in range(4)]
         check(lib().recis_idmap_stats(self._h, *[ctypes.byref(v) for v in vals], stream_ptr(self.device)))
+        _lib.raise_device_errors()   # the call above has waited for the stream already
         return tuple(v.value for v in vals)
 
     def size(self):
@@ -740,7 +751,7 @@ class BatchPlan:
     """
 
     __slots__ = ("n", "_U", "_unique", "unique_buf", "inverse", "row_start", "occ", "pos", "hot_items", "hot_cap",
-                 "counts", "_pool_fill", "_stream", "serial")
+                 "counts", "_pool_fill", "_stream", "serial", "lookup_calls")
 
     @property
     def U(self):
@@ -750,6 +761,7 @@ class BatchPlan:
                 check(lib().recis_unique_plan_count(ctypes.byref(count), self._stream))
                 self._U = int(count.value)
                 _STAGED.pop(self._stream.value, None)
+                _raise_staged_device_errors(self._stream)
             else:  # a later plan took the stream's staging word: read this plan's own device word
                 self._U = int(self.counts[0].item())
         return self._U
@@ -797,6 +809,15 @@ class BatchPlan:
 
 _PLAN_SERIAL = itertools.count(1)
 
+def _raise_staged_device_errors(stream):
+    """Soft errors of the device (bad row index, full id map, ...) as an exception: kernels skip the
+    faulty access and set a bit; the bits travel to host memory with every staged unique count, so
+    the training loop sees them at its next ``BatchPlan.U`` without any extra wait."""
+    bits = ctypes.c_int(0)
+    check(lib().recis_hip_staged_device_errors(ctypes.byref(bits), stream))
+    if bits.value:
+        _lib.raise_device_errors(bits.value)   # waits for the device and clears the word
+
 
 def ids_unique_plan(ids, wait=True):
     """Dedup + transposed index of a batch of ids (``recis_unique_plan``). ``wait=False``
@@ -817,15 +838,21 @@ def ids_unique_plan(ids, wait=True):
     p.hot_items = torch.empty(2 * p.hot_cap, dtype=torch.int32, device=dev)
     p.counts = torch.empty(2, dtype=torch.int64, device=dev)
     p._pool_fill = None
+    p.lookup_calls = {}   # table -> number of the counted lookup queued for this plan
     p._unique = None
     p._stream = stream_ptr(dev)
     count = ctypes.c_int64(0)
+    # every launch overwrites the stream's staging word: an earlier plan whose count is still
+    # outstanding there must read its own device word from now on
+    _STAGED.pop(p._stream.value, None)
     check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(p.unique_buf), ptr(p.inverse), ptr(p.row_start), ptr(p.occ),
                                   ptr(p.pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts),
                                   ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
     p._U = int(count.value) if wait else None
     if not wait:
         _STAGED[p._stream.value] = p
+    else:
+        _raise_staged_device_errors(p._stream)
     return p
 
 

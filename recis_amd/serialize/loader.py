@@ -7,6 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 import torch
 
 from . import format as fmt
+from .. import _lib
 
 
 def default_load_info(hashtables, tensors):
@@ -152,3 +153,5 @@ class Loader:
                     raise RuntimeError("shape not match")
                 with torch.no_grad():
                     target.copy_(b.read_tensor())
+        if torch.cuda.is_available():
+            _lib.raise_device_errors()   # rows the inserts had to skip would be missing silently

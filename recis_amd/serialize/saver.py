@@ -8,6 +8,7 @@ overlaps the file write of the piece before it."""
 import torch
 
 from . import format as fmt
+from .. import _lib
 
 
 class HTSlotWriteBlock(fmt.WriteBlock):
@@ -97,3 +98,5 @@ class Saver:
             bundle.add_block(b)
         bundle.save()
         bundle.merge_meta_info()
+        if torch.cuda.is_available():
+            _lib.raise_device_errors()   # a row index the gathers had to skip means a checkpoint with holes

@@ -13,6 +13,7 @@ import torch
 import oracle
 import workloads
 from oracle import cpu_path
+from recis_amd import _lib, ops
 from recis_amd.hooks import HashTableFilterHook
 from recis_amd.nn import DynamicEmbedding, EmbeddingEngine, EmbeddingOption, HashTable
 from recis_amd.nn.functional.embedding_ops import ragged_embedding_segment_reduce
@@ -549,3 +550,42 @@ def test_feature_engine_ops_and_fusion():
     exp = [[1, 2, 3], [3, 6, 9], [5, 10, 15], [7, 14, 21]]
     for j in range(4):
         assert out["multi_hash_%d" % j].values().tolist() == exp[j]
+
+
+def test_a_waiting_plan_between_forward_and_backward_does_not_steal_the_unique_count(rng):
+    """DynamicEmbedding's forward leaves its unique count on the way to the stream's staging word
+    and reads it in backward. Another plan on the same stream in between (here one that waits for
+    its own count, with a very different number of distinct ids, as HashTable._unique in eval mode
+    or exchange_ids make) reuses that word: backward must still see the count of ITS plan. Checked
+    by the gradient per key against the oracle's scatter."""
+    from recis_amd.nn.modules.hashtable import HashtableRegister
+
+    HashtableRegister().clear()
+    opt = EmbeddingOption(embedding_dim=8, shared_name="interleave", combiner="sum", block_size=256,
+                          use_weight=False, initializer=NormalInitializer(0, 0.1))
+    emb = DynamicEmbedding(opt)
+    emb.train()
+    S = 2000
+    lens = rng.integers(0, 6, size=S)
+    off = np.concatenate([[0], np.cumsum(lens)])
+    ids = rng.integers(0, 900, size=int(off[-1]))
+    rt = RaggedTensor(torch.from_numpy(ids).cuda(), torch.from_numpy(off.astype(np.int32)).cuda())
+    out = emb(rt)
+    other = ops.ids_unique_plan(torch.arange(17, device="cuda"), wait=True)     # U = 17 on the same stream
+    assert other.U == 17
+    third = ops.ids_unique_plan(torch.arange(50000, device="cuda"), wait=False)  # and one that does not wait
+    up = rng.standard_normal((S, 8)).astype(np.float32)
+    out.backward(torch.from_numpy(up).cuda())
+    assert third.U == 50000
+    impl = emb.hashtable._hashtable_impl
+    index, g = impl.grad_pairs(1)
+    uniq, inv = np.unique(ids, return_inverse=True)
+    assert index.numel() == len(uniq)
+    exp = oracle.segment_reduce_backward(up, None, inv, off, len(uniq), "sum")
+    rows = impl.lookup_index_readonly(torch.from_numpy(uniq).cuda())
+    order = torch.argsort(index)
+    assert torch.equal(index[order], torch.sort(rows).values)
+    by_row = dict(zip(rows.tolist(), range(len(uniq))))
+    perm = [by_row[r] for r in index[order].tolist()]
+    np.testing.assert_allclose(g[order].cpu().numpy(), exp[perm], rtol=1e-5, atol=1e-5)
+    assert _lib.poll_device_errors() == 0

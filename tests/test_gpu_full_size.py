@@ -83,16 +83,19 @@ def test_config4_step_properties():
     assert _lib.poll_device_errors() == 0
 
 
-def test_config3_lookups_at_scale():
-    """A tenth of the resident set of config 3 (2e7 rows, so that the test stays short) with the full
-    per-step lookup size: known keys keep their rows, never-seen keys get rows nobody holds, the
-    expansion gives every lookup its key's row, eviction removes exactly the keys not seen."""
+@pytest.mark.parametrize("resident", [20_000_000, 200_000_000])
+def test_config3_lookups_at_scale(resident):
+    """Config 3 with the full per-step lookup size, at a tenth of its resident set and at the full
+    2e8 rows (77 GB of rows and optimizer state, a 2^29-slot id map, 29 GB per slot in one
+    allocation, row addresses past 2^32 bytes): known keys keep their rows, never-seen keys get
+    rows nobody holds, the expansion gives every lookup its key's row, eviction removes exactly the
+    keys not seen."""
     import bench
 
-    wl = bench.Config3(resident=20_000_000, ids_per_step=2_000_000, n_batches=3)
+    wl = bench.Config3(resident=resident, ids_per_step=2_000_000, n_batches=3)
     t = wl.table
     lv0, idn0, _, _ = t.id_map().stats()
-    assert lv0 == 20_000_000
+    assert lv0 == resident
     ids = wl.batches[0]
     known = t.lookup_index_readonly(ids)
     n_new = int(torch.unique(ids[known < 0]).numel())
@@ -123,6 +126,8 @@ def test_config3_lookups_at_scale():
     assert int(t.lookup_index_readonly(seen).min()) >= 0
     assert int(t.lookup_index_readonly(gone_ids[:100000]).max()) == -1
     assert _lib.poll_device_errors() == 0
+    del wl, t
+    torch.cuda.empty_cache()
 
 
 def test_config5_step_properties():

@@ -130,22 +130,31 @@ def zipf_ranks_torch(cdf, n, generator):
     return torch.searchsorted(cdf, u).clamp_(max=cdf.numel() - 1)
 
 
+class Config3Lookups:
+    """benchmark config 3 lookups: step k draws `ids_per_step` keys, Zipf(alpha) over the `resident`
+    pre-populated keys (key of rank r = splitmix64(r)), with a fraction `new_frac` of the positions
+    replaced by keys never seen before: ranks resident + k * n_new + arange(n_new), beyond the
+    resident set and distinct for every step. Deterministic in (seed, k) whatever the order of the
+    calls."""
+
+    def __init__(self, resident, ids_per_step=2_000_000, alpha=1.1, new_frac=0.1, seed=3, device="cuda"):
+        self.resident, self.n, self.seed, self.device = resident, ids_per_step, seed, device
+        self.n_new = int(ids_per_step * new_frac)
+        self.cdf = zipf_cdf_torch(resident, alpha, device)
+
+    def batch(self, k):
+        g = torch.Generator(device=self.device).manual_seed(self.seed * 1_000_003 + k)
+        ranks = zipf_ranks_torch(self.cdf, self.n, g)
+        pos = torch.randperm(self.n, device=self.device, generator=g)[: self.n_new]
+        ranks[pos] = self.resident + k * self.n_new + torch.arange(self.n_new, device=self.device)
+        return splitmix64_torch(ranks)
+
+
 def config3_batches(n_batches, resident, ids_per_step=2_000_000, alpha=1.1, new_frac=0.1, seed=3,
                     device="cuda"):
-    """benchmark config 3 lookups: per step `ids_per_step` keys, Zipf(alpha) over the `resident`
-    pre-populated keys (key of rank r = splitmix64(r)), a fraction `new_frac` of the positions
-    replaced by keys never seen before (ranks beyond the resident set, distinct per step)."""
-    g = torch.Generator(device=device).manual_seed(seed)
-    cdf = zipf_cdf_torch(resident, alpha, device)
-    n_new = int(ids_per_step * new_frac)
-    out = []
-    for b in range(n_batches):
-        ranks = zipf_ranks_torch(cdf, ids_per_step, g)
-        pos = torch.randperm(ids_per_step, device=device, generator=g)[:n_new]
-        ranks[pos] = resident + b * n_new + torch.arange(n_new, device=device)
-        out.append(splitmix64_torch(ranks))
-    del cdf
-    return out
+    """The lookups of the first `n_batches` steps of benchmark config 3 (see Config3Lookups)."""
+    gen = Config3Lookups(resident, ids_per_step, alpha, new_frac, seed, device)
+    return [gen.batch(k) for k in range(n_batches)]
 
 
 def config5(device="cuda", seed=5, batch=2048, n_fields=4, num_keys=50_000_000, alpha=1.2, mean_len=200,
