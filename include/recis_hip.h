@@ -422,6 +422,26 @@ int recis_unique_plan_count(int64_t* unique_count_host, void* stream);
 int recis_hip_staged_device_errors(int* bits, void* stream);
 
 /*
+ * recis_unique_plan for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same outputs as
+ * recis_unique_plan for the same ids, bit for bit wherever that call specifies them (unique ids,
+ * inverse, row_start, counts; list / pos up to the order inside one id's list); the count stays on
+ * the device (counts_out_dev), nothing is staged for the host. The kernels' scratch is a fixed
+ * RECIS_PLAN_NOALLOC_SCRATCH_MIB MiB array inside the library's code object (every device the
+ * library runs on holds one until the process ends); the call makes no hipMalloc / hipFree /
+ * hipHostMalloc and creates no event or stream. n > RECIS_PLAN_NOALLOC_MAX_IDS returns
+ * RECIS_ERR_ARG. All calls on one device share the one array: two calls that overlap in time on a
+ * device (different streams or threads) race; calls queued on one stream do not. (With
+ * recis_hip_profile_enable(1) the profiler's own events are created as for every other call.)
+ */
+#define RECIS_PLAN_NOALLOC_SCRATCH_MIB 16
+#define RECIS_PLAN_NOALLOC_MAX_IDS 262144
+int recis_unique_plan_noalloc(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
+                              int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
+                              int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev,
+                              void* stream);
+
+/*
  * Per list entry, the input row it reads and its coefficient, for the backward of
  *   pooled segments: src = segment of the occurrence, coef = weight (/ length for MEAN)
  *                    (coef_out may be NULL when there are no weights and mean == 0)

@@ -28,6 +28,7 @@
 
 #include <algorithm>
 #include <climits>
+#include <mutex>
 #include <type_traits>
 
 #include "common.cuh"
@@ -1258,6 +1259,55 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
     *unique_count_host = staged[0];
   }
   return RECIS_OK;
+}
+
+// The scratch of recis_unique_plan_noalloc: part of the library's code object on every device that
+// loads it. Host code never uses this name as an address: the per-device address comes from
+// hipGetSymbolAddress (below) and travels to the kernels as an argument.
+constexpr size_t kStaticScratchBytes = size_t(RECIS_PLAN_NOALLOC_SCRATCH_MIB) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxScratchDevices = 64;
+static std::mutex g_scratch_mu;
+static char* g_scratch_ptr[kMaxScratchDevices];
+
+int recis_unique_plan_noalloc(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
+                              int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
+                              int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = plan_check_args(ids, n, unique_out, inverse_out, row_start_out, list_out, hot_items_out, hot_cap,
+                               counts_out_dev))
+    return rc;
+  const int dev = current_device();
+  RECIS_REQUIRE(dev >= 0 && dev < kMaxScratchDevices, "device %d out of range", dev);
+  char* base = nullptr;
+  {
+    std::lock_guard<std::mutex> l(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {  // first call on this device (it is the current one)
+      void* p = nullptr;
+      RECIS_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+      g_scratch_ptr[dev] = static_cast<char*>(p);
+    }
+    base = g_scratch_ptr[dev];
+  }
+  int* err = device_error_word(dev);
+  RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
+  if (n == 0) {
+    plan_empty_kernel<<<1, 64, 0, stream>>>(counts_out_dev, row_start_out, nullptr, err);
+    RECIS_LAUNCH_CHECK();
+    return RECIS_OK;
+  }
+  RECIS_REQUIRE(n <= RECIS_PLAN_NOALLOC_MAX_IDS, "recis_unique_plan_noalloc takes at most %lld ids per call (got %lld); "
+                "use recis_unique_plan for more", (long long)RECIS_PLAN_NOALLOC_MAX_IDS, (long long)n);
+  const PlanLayout L = plan_layout(n);
+  if (L.bytes > kStaticScratchBytes)
+    return fail(RECIS_ERR_CAPACITY,
+                "recis_unique_plan_noalloc: %lld ids need %zu bytes of scratch, the built-in buffer holds %zu "
+                "(at most %lld ids per call; use recis_unique_plan for more)",
+                (long long)n, L.bytes, kStaticScratchBytes, (long long)RECIS_PLAN_NOALLOC_MAX_IDS);
+  // every scratch array is fully written by the kernel that produces it before any kernel reads it:
+  // nothing of the previous call's contents is relied on, nothing needs clearing
+  return plan_launch(L, base, ids, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
+                     counts_out_dev, nullptr, nullptr, err, stream);
 }
 
 int recis_unique_plan_count(int64_t* unique_count_host, void* stream_) {
