@@ -192,14 +192,15 @@ class Config4:
         return o.ids_encode(self.c["sparse"] + extra, self.tags)
 
     def dedup(self, ids):
-        self.plan = self.ops.ids_unique_plan(ids, wait=False)
-        return self.plan, self.plan.inverse
+        """Dedup and find-or-insert in one pass: the plan carries the row of every unique id. Every
+        field holds one id per sample, so nothing per occurrence but the lists is asked for."""
+        self.plan = self.table.plan_lookup(ids, need_inverse=False, need_pos=False)
+        return self.plan, None
 
     def lookup(self, plan):
-        # queued before the host has the unique count; the count arrives while plan and lookup run
-        index_buf = self.table.lookup_index_counted(plan)
+        # the host reads the unique count here; the device has long gone on
         self.U = plan.U
-        return self.table.settle_lookup(index_buf, self.U)
+        return self.table.settle_lookup(plan.index_buf, self.U, plan)
 
     def pool_fwd(self, index, inv):
         # pooling reads the rows out of the table (no [U, D] copy); every field holds one id per
@@ -278,24 +279,26 @@ class Config4:
         feat = 13 * self.c["batch"] * (4 + 8) + 13 * self.c["batch"] * (8 + 8) + N * 16
         return {
             "feature_ops": feat,
-            "dedup": N * (8 + 4) + U * 8,
-            "lookup": U * (16 + 8),
+            "dedup+lookup": N * (8 + 4) + U * 8 + U * (16 + 8),
             "pool_fwd": U * (8 + D * 4) + N * 4 + (U + 1) * 4 + S * D * 4,
             "pool_bwd": S * D * 4 + N * 4 + (S + 1) * 4 + U * D * 4,
             "adam": U * 8 + U * D * 4 * (1 + 6),
         }
 
+    def survey_bytes(self):
+        """The step's compulsory bytes by the formula the survey of the reference prices config 4 with
+        (the [U, D] gradient between pooling backward and Adam counted as kept on chip)."""
+        N, U, S = self.N, self.U, self.N
+        return N * (8 + 4 + 4) + U * (16 + 8 + 384 + 8) + S * (64 + 64) + 13 * self.c["batch"] * (4 + 8 + 8 + 8)
+
     def kernel_bytes(self):
         """Algorithmic (compulsory) HBM bytes of one launch of each heavy kernel of the step."""
         N, U, S, D = self.N, self.U, self.N, self.D
         return {
-            # plan: a record (16 B) per id and tile, at least one per unique id
-            "plan_tile_kernel": 8 * N + 4 * N + 16 * U,              # ids in; per-occurrence word + records out
-            "plan_scatter_kernel": 16 * U + 16 * U,
-            "plan_bucket_kernel": 16 * U + 8 * U + 16 * U,           # records in; per-record result + unique ids out
-            # ids, word, result in; inverse, list, pos out; unique ids in, id + row_start out
-            "plan_emit_kernel": 8 * N + 4 * N + 8 * U + 12 * N + 16 * U + 12 * U + 4 * (N + 1 - U),
-            "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,          # ids, one table slot, index + slot pos
+            "plan_hist_kernel": 8 * N,                               # ids in
+            "plan_scatter_kernel": 8 * N + 12 * N,                   # ids in; (id, position) out, by bucket
+            # (id, position) in; list out; per unique id: the id, its list start, its row; one 16-byte slot of the map
+            "plan_bucket_kernel": 12 * N + 4 * N + U * (8 + 4 + 8) + 16 * U,
             "csr_expand_kernel": U * (8 + D * 4) + 4 * N + 4 * (U + 1) + S * D * 4,
             "csr_rows_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,
             "adamw_rows_kernel": U * (8 + D * 4 * 7),
@@ -306,10 +309,11 @@ class Config4:
         uniq, inv = self.dedup(ids)
         index = self.lookup(uniq)
         g = self.pool_bwd(inv)
+        def dedup_lookup():
+            self.lookup(self.dedup(ids)[0])
         return {
             "feature_ops": _event_ms(self.feature_ops, iters),
-            "dedup": _event_ms(lambda: self.dedup(ids), iters),
-            "lookup": _event_ms(lambda: self.lookup(uniq), iters),
+            "dedup+lookup": _event_ms(dedup_lookup, iters),
             "pool_fwd": _event_ms(lambda: self.pool_fwd(index, inv), iters),
             "pool_bwd": _event_ms(lambda: self.pool_bwd(inv), iters),
             "adam": _event_ms(lambda: self.update(index, g), iters),
@@ -337,19 +341,22 @@ class Config4:
         return n * reps / dt, "first %d samples (%d ids/step) of config 4, full step" % (b, n)
 
     def cpu_reference(self, budget_s, threads):
-        """The reference's own CPU operators (compiled from its sources into oracle/_ref) on the
-        ids of cpu_baseline's sample: ids_partition + Hashtable.EmbeddingLookup + AcceptGrad +
-        SparseAdam.step. The reference has no CPU pooling operator, so this is the step without
-        the pooling forward and backward. None when the reference build is absent."""
+        """The reference's own CPU code (compiled from its sources into oracle/_ref) on the ids of
+        cpu_baseline's sample, `threads` threads: ids_partition + Hashtable.EmbeddingLookup + sum
+        pooling forward and backward as the reference's "torch" backend runs them on CPU tensors
+        (index_select + index_add_: it has no CPU pooling operator) + AcceptGrad + SparseAdam.step.
+        None when the reference build is absent."""
         from oracle import ref_ops
         if not ref_ops.available():
             return None
         ids = np.ascontiguousarray(self._cpu_sample_ids, dtype=np.int64)
+        seg = np.arange(ids.size, dtype=np.int64)   # one id per sample and field
         params = np.array([10240, self.D, 1e-3, 0.9, 0.999, 1e-8, 0.0, budget_s, threads], np.float64)
-        secs, steps, uniq = ref_ops.run("table_step_time", [params, ids], threads=threads)[0]
+        secs, steps, uniq = ref_ops.run("table_step_time", [params, ids, seg], threads=threads)[0]
         return {"value": ids.size * steps / secs, "unit": "ids/s", "cores": threads, "kind": "reference",
-                "sample": "the same %d ids/step (%d distinct): ids_partition + EmbeddingLookup + AcceptGrad + "
-                          "SparseAdam.step of the reference; its pooling has no CPU operator" % (ids.size, int(uniq))}
+                "sample": "first %d samples (%d ids/step, %d distinct) of config 4: the reference's ids_partition + "
+                          "EmbeddingLookup + torch-backend sum pooling fwd/bwd + AcceptGrad + SparseAdam.step "
+                          "(feature ops left out)" % (ids.size // self.n_feat, ids.size, int(uniq))}
 
 
 
@@ -417,10 +424,9 @@ class Config3:
         if self.step_no and self.step_no % self.filter_interval == 0:
             self.sweep(self.step_no - self.filter_step)
         self.step_no += 1
-        plan = o.ids_unique_plan(ids, wait=False)
-        index_buf = self.table.lookup_index_counted(plan)   # queued before the host has the unique count
+        plan = self.table.plan_lookup(ids, need_inverse=False, need_pos=False)   # dedup + find-or-insert, one pass
         self.U = plan.U
-        index = self.table.settle_lookup(index_buf, self.U, plan)
+        index = self.table.settle_lookup(plan.index_buf, self.U, plan)
         chunks, chunk_rows = self.table.emb_blocks()
         self.table.update_slot("step_filter", index, self.step_t)
         # one row per lookup: every unique row is read once out of the table and written to its
@@ -452,6 +458,10 @@ class Config3:
             self.step()
         return self.sweeps[-1]
 
+    def survey_bytes(self):
+        N, U, D = self.N, self.U, self.D
+        return U * (16 + 8 + 768 + 8) + int(0.1 * N) * 16 + N * (8 + 4 + 128 + 128)
+
     def algorithmic_bytes(self):
         N, U, D = self.N, self.U, self.D
         return N * (8 + 4) + U * 8 + U * (16 + 8) + int(0.1 * N) * 16 + U * D * 4 + N * (4 + D * 4) \
@@ -465,7 +475,7 @@ class Config3:
             "csr_expand_kernel": U * (8 + D * 4) + 4 * N + 4 * (U + 1) + N * D * 4,
             "csr_rows_kernel": N * D * 4 + 4 * N + 4 * U + U * D * 4,
             "adamw_rows_kernel": U * (8 + D * 4 * 7),
-            "find_or_claim_kernel": 8 * U + 16 * U + 16 * U,
+            "plan_bucket_kernel": 12 * N + 4 * N + U * (8 + 4 + 8) + 16 * U,
         }
 
     def cpu_baseline(self, budget_s):
@@ -533,11 +543,10 @@ class Config5:
     def step(self):
         o = self.ops
         ids = o.ids_encode([f["values"] for f in self.fields], list(range(len(self.fields))))
-        plan = o.ids_unique_plan(ids, wait=False)
-        index_buf = self.table.lookup_index_counted(plan)   # queued before the host has the unique count
+        plan = self.table.plan_lookup(ids)   # dedup + find-or-insert, one pass
         self.U = plan.U
         inv = plan.inverse
-        index = self.table.settle_lookup(index_buf, self.U)
+        index = self.table.settle_lookup(plan.index_buf, self.U, plan)
         chunks, chunk_rows = self.table.emb_blocks()
         rows = o.block_gather(index, chunks, chunk_rows, -1, False)
         pooled = o.segment_reduce_forward(rows, None, inv, self.offsets, "mean", out_dtype=torch.float32)
@@ -549,6 +558,10 @@ class Config5:
         self.opt.step()
         self.opt.zero_grad()
         return pooled, padded
+
+    def survey_bytes(self):
+        N, U, S, D = self.N, self.U, self.S, self.D
+        return 12 * N + U * (24 + 1024) + S * (256 + 256) + self.pad_rows * 256
 
     def algorithmic_bytes(self):
         N, U, S, D = self.N, self.U, self.S, self.D
@@ -596,6 +609,96 @@ class Config5:
             reps += 1
         dt = time.perf_counter() - t0
         return n * reps / dt, "first %d of 2048 sequences per field (%d ids/step) of config 5, fp32 rows" % (b, n)
+
+
+# --------------------------------------------------------------------- the same steps through the modules
+class ModulePath4:
+    """Config 4 through the drop-in layer: FeatureEngine (bucketize + mod of the 13 dense columns) ->
+    EmbeddingEngine (39 features on one coalesced table) -> concatenation for a dense tower ->
+    backward -> SparseAdam.step, rotating over the same 8 batches as Config4."""
+
+    def __init__(self, n_batches=8):
+        from recis_amd.features import Bucketize, Feature, FeatureEngine, Mod, SelectField
+        from recis_amd.nn import EmbeddingEngine, EmbeddingOption
+        from recis_amd.nn.initializers import NormalInitializer
+        from recis_amd.nn.modules.hashtable import HashtableRegister, filter_out_sparse_param
+        from recis_amd.optim import SparseAdam
+        HashtableRegister().clear()
+        batches = [workloads.config4()] + [workloads.config4(data_seed=k) for k in range(1, n_batches)]
+        c = batches[0]
+        nd, ns = len(c["dense"]), len(c["sparse"])
+        self.fe = FeatureEngine([Feature("d%d" % i).add_op(SelectField("d%d" % i)).add_op(Bucketize(c["boundaries"][i]))
+                                 .add_op(Mod(c["mod"])) for i in range(nd)])
+        self.names = ["s%d" % i for i in range(ns)] + ["d%d" % i for i in range(nd)]
+        opts = {n: EmbeddingOption(embedding_dim=16, shared_name=n, combiner="sum", use_weight=False,
+                                   initializer=NormalInitializer(0, 0.01),
+                                   reserve_rows=int(c["num_ids"] * 1.05) * n_batches if k == 0 else 0)
+                for k, n in enumerate(self.names)}
+        self.eng = EmbeddingEngine(opts).cuda()
+        self.eng.train()
+        self.opt = SparseAdam(filter_out_sparse_param(self.eng), lr=1e-3)
+        self.data = []
+        for b in batches:
+            d = {"s%d" % i: t.view(-1, 1) for i, t in enumerate(b["sparse"])}
+            d.update({"d%d" % i: t for i, t in enumerate(b["dense"])})
+            self.data.append(d)
+        g = torch.Generator(device="cuda").manual_seed(4)
+        self.up = torch.randn((c["batch"], 16 * len(self.names)), device="cuda", generator=g)
+        self._turn = 0
+        for _ in range(n_batches + 2):
+            self.step()
+        torch.cuda.synchronize()
+
+    def step(self):
+        data = self.data[self._turn % len(self.data)]
+        self._turn += 1
+        x = dict(data)
+        x.update({k: v.view(-1, 1) for k, v in self.fe({k: data[k] for k in data if k[0] == "d"}).items()})
+        out = self.eng(x)
+        torch.cat([out[n] for n in self.names], dim=1).backward(self.up)
+        self.opt.step()
+        self.opt.zero_grad()
+
+
+class ModulePath5:
+    """Config 5 through the drop-in layer: each of the 4 sequence fields under two options of one
+    shared name (mean pooling, and the rows kept and padded to the field's longest sequence), bf16
+    table, backward of both, SparseAdagrad.step."""
+
+    def __init__(self):
+        from recis_amd.nn import EmbeddingEngine, EmbeddingOption
+        from recis_amd.nn.initializers import NormalInitializer
+        from recis_amd.nn.modules.hashtable import HashtableRegister, filter_out_sparse_param
+        from recis_amd.optim import SparseAdagrad
+        from recis_amd.ragged import RaggedTensor
+        HashtableRegister().clear()
+        c = workloads.config5()
+        opts, self.data = {}, {}
+        for i, f in enumerate(c["fields"]):
+            rt = RaggedTensor(f["values"], f["offsets"])
+            common = dict(embedding_dim=128, dtype=torch.bfloat16, shared_name="s%d" % i, use_weight=False,
+                          initializer=NormalInitializer(0, 0.01), reserve_rows=int(f["num_ids"] * 1.1))
+            opts["s%d_mean" % i] = EmbeddingOption(combiner="mean", **common)
+            opts["s%d_rows" % i] = EmbeddingOption(combiner="tile", combiner_kwargs={"tile_len": f["pad_len"]},
+                                                   **common)
+            self.data["s%d_mean" % i] = rt
+            self.data["s%d_rows" % i] = rt
+        self.eng = EmbeddingEngine(opts).cuda()
+        self.eng.train()
+        self.opt = SparseAdagrad(filter_out_sparse_param(self.eng), lr=0.01)
+        g = torch.Generator(device="cuda").manual_seed(5)
+        out = self.eng(self.data)
+        self.ups = {k: torch.randn(v.shape, device="cuda", generator=g).to(v.dtype) for k, v in out.items()}
+        del out
+        for _ in range(5):
+            self.step()
+        torch.cuda.synchronize()
+
+    def step(self):
+        out = self.eng(self.data)
+        torch.autograd.backward([out[k] for k in out], [self.ups[k] for k in out])
+        self.opt.step()
+        self.opt.zero_grad()
 
 
 # HBM bytes per launch in the config-4 step, from hardware-counter runs of this file
@@ -651,6 +754,66 @@ def checkpoint_round_trip(rows=8 << 20, dim=16, parallel=8):
             "directory": os.path.dirname(path)}
 
 
+def _timed_steps(wl, steps, warmup):
+    if hasattr(wl, "prepare"):
+        wl.prepare(steps + warmup)
+    for _ in range(warmup):
+        wl.step()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        wl.step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t) / steps * 1e3
+
+
+def _kernel_roofline(wl, iters):
+    """Per-kernel launch times of wl.step() (the library's HIP events on the launch stream) and the
+    roofline object of the kernel with the largest share: algorithmic bytes per launch / mean launch
+    time against the HBM peak."""
+    if hasattr(wl, "prepare"):
+        wl.prepare(iters + 2)
+    kern = _kernel_profile(wl.step, iters)
+    kb = wl.kernel_bytes()
+    dom = max((k for k in kern if k in kb), key=lambda k: kern[k]["us"] * kern[k]["calls_per_step"])
+    ach = kb[dom] / kern[dom]["us"] / 1e3
+    roof = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": ach / HBM_PEAK_GBS, "traffic": None, "launch_us": round(kern[dom]["us"], 2),
+            "launches_per_step": kern[dom]["calls_per_step"], "algorithmic_bytes_per_launch": kb[dom]}
+    kernels_us = {k: round(v["us"], 2) for k, v in sorted(kern.items(), key=lambda kv: -kv[1]["us"])}
+    kernels_gbs = {k: round(kb[k] / kern[k]["us"] / 1e3, 1) for k in kern if kb.get(k)}
+    return roof, kernels_us, kernels_gbs
+
+
+def _step_roofline(wl, ms):
+    """Whole-step fractions of the HBM peak, by this build's count of compulsory bytes and by the
+    survey's formula for the same config."""
+    nbytes = wl.algorithmic_bytes()
+    nbytes = sum(nbytes.values()) if isinstance(nbytes, dict) else nbytes
+    out = {"algorithmic_bytes": nbytes, "achieved": nbytes / ms / 1e6, "frac": nbytes / ms / 1e6 / HBM_PEAK_GBS,
+           "unit": "GB/s"}
+    if hasattr(wl, "survey_bytes"):
+        sb = wl.survey_bytes()
+        out["survey_bytes"] = sb
+        out["survey_frac"] = sb / ms / 1e6 / HBM_PEAK_GBS
+    return out
+
+
+def _c3_eviction(wl, step_ms):
+    """Runs config 3 on to its next sweep of the step filter (every 50 steps, threshold step - 50)
+    and reports it: the keys it evicted, its time, and the step time with the sweep spread over
+    the 50 steps it serves. New keys per step come from the id map's own counters."""
+    live0, idn0, _, _ = wl.table.id_map().stats()
+    step0 = wl.step_no
+    at, evicted, ms = wl.run_to_next_sweep()
+    live1, idn1, _, _ = wl.table.id_map().stats()
+    steps = wl.step_no - step0
+    return {"sweep_at_step": at, "evicted_per_sweep": evicted, "sweep_ms": round(ms, 3),
+            "sweep_interval_steps": wl.filter_interval, "live_keys_before": live0, "live_keys_after": live1,
+            "new_keys_per_step": round((live1 + evicted - live0) / max(steps, 1), 1),
+            "ms_per_step_with_sweep": round(step_ms + ms / wl.filter_interval, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -681,6 +844,8 @@ def main():
     main_wl = classes[args.workload]()
     # part of set-up, before the W warm-up steps: the first steps of a process pay for the device
     # allocations of the step's outputs (config 5: 2 GB blocks, tens of ms)
+    if hasattr(main_wl, "prepare"):
+        main_wl.prepare(10 + args.warmup + args.steps)
     for _ in range(10):
         main_wl.step()
     torch.cuda.synchronize()
@@ -703,30 +868,22 @@ def main():
         "config": {"workload": main_wl.name, "ids_per_step": main_wl.ids_per_step},
     }
 
-    def timed_steps(wl, steps, warmup):
-        for _ in range(warmup):
-            wl.step()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(steps):
-            wl.step()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t) / steps * 1e3
-
     def c2_summary(wl):
         res = {}
         for kname, (fn, nbytes) in wl.kernels().items():
             ms = _event_ms(fn, 10)
             res[kname] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
-                          "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                          "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_launch": nbytes}
         return res
 
-    def step_summary(wl, ms):
+    def step_summary(wl, ms, iters):
+        """One entry of "workloads": step time, ids/s, whole-step and dominant-kernel rooflines."""
+        roof, kernels_us, _ = _kernel_roofline(wl, iters)
         nbytes = wl.algorithmic_bytes()
         nbytes = sum(nbytes.values()) if isinstance(nbytes, dict) else nbytes
         return {"ms_per_step": round(ms, 4), "ids_per_s": wl.ids_per_step / ms * 1e3,
-                "unique_ids_per_step": wl.U, "algorithmic_bytes": nbytes,
-                "gbs": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                "unique_ids_per_step": wl.U, "step_roofline": _step_roofline(wl, ms), "roofline": roof,
+                "kernels_us": kernels_us}
 
     if args.calib_copy:
         src = torch.zeros(1 << 28, device="cuda")
@@ -737,24 +894,28 @@ def main():
         del src, dst
 
     extras = {}
-    if args.workload == "c4":
-        stages = None if args.no_stages else main_wl.stage_times(max(5, args.steps))
-        ab = main_wl.algorithmic_bytes()
-        total_bytes = sum(ab.values())
-        kern = _kernel_profile(main_wl.step, max(5, args.steps))
-        kb = main_wl.kernel_bytes()
-        dom = max(kern, key=lambda k: kern[k]["us"] * kern[k]["calls_per_step"])
+    if args.workload == "c2":
+        res = c2_summary(main_wl)
+        dom = max(res, key=lambda k: res[k]["ms"])
+        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": res[dom]["gbs"], "peak": HBM_PEAK_GBS,
+                           "unit": "GB/s", "frac": res[dom]["frac"], "traffic": None,
+                           "launch_us": round(res[dom]["ms"] * 1e3, 2),
+                           "algorithmic_bytes_per_launch": res[dom]["algorithmic_bytes_per_launch"]}
+        out["stages_ms"] = {k: v["ms"] for k, v in res.items()}
+    else:
+        stages = None
+        if args.workload == "c4" and not args.no_stages:
+            stages = main_wl.stage_times(max(5, args.steps))
+        roof, kernels_us, kernels_gbs = _kernel_roofline(main_wl, max(5, args.steps))
+        if args.workload == "c4":
+            roof["traffic"] = MEASURED_TRAFFIC_C4.get(roof["kernel"])
         out["config"]["unique_ids_per_step"] = main_wl.U
-        ach = kb.get(dom, 0) / kern[dom]["us"] / 1e3
-        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": ach / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_C4.get(dom),
-                           "launch_us": round(kern[dom]["us"], 2),
-                           "algorithmic_bytes_per_launch": kb.get(dom, 0)}
-        out["kernels_us"] = {k: round(v["us"], 2) for k, v in sorted(kern.items(), key=lambda kv: -kv[1]["us"])}
-        out["kernels_gbs"] = {k: round(kb[k] / kern[k]["us"] / 1e3, 1) for k in kern if kb.get(k)}
-        out["step_roofline"] = {"algorithmic_bytes": total_bytes, "achieved": total_bytes / ms_per_step / 1e6,
-                                "frac": total_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, "unit": "GB/s"}
+        out["roofline"] = roof
+        out["kernels_us"] = kernels_us
+        out["kernels_gbs"] = kernels_gbs
+        out["step_roofline"] = _step_roofline(main_wl, ms_per_step)
         if stages is not None:
+            ab = main_wl.algorithmic_bytes()
             out["stages_ms"] = {k: round(v, 4) for k, v in stages.items()}
             out["stages_gbs"] = {k: round(ab[k] / stages[k] / 1e6, 1) for k in stages}
             host_ms = _event_ms(main_wl.step_from_host, max(5, args.steps))
@@ -764,31 +925,12 @@ def main():
             torch.cuda.synchronize()
             out["inputs_from_pinned_host"]["overlapped_ms_per_step"] = round(over_ms, 4)
             out["inputs_from_pinned_host"]["overlapped_ids_per_s"] = main_wl.N / over_ms * 1e3
-    elif args.workload == "c2":
-        res = c2_summary(main_wl)
-        dom = max(res, key=lambda k: res[k]["ms"])
-        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": res[dom]["gbs"], "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": res[dom]["frac"], "traffic": None}
-        out["stages_ms"] = {k: v["ms"] for k, v in res.items()}
-    else:
-        s = step_summary(main_wl, ms_per_step)
-        out["config"]["unique_ids_per_step"] = main_wl.U
-        kern = _kernel_profile(main_wl.step, max(5, args.steps))
-        kb = main_wl.kernel_bytes()
-        dom = max((k for k in kern if k in kb), key=lambda k: kern[k]["us"] * kern[k]["calls_per_step"])
-        ach = kb[dom] / kern[dom]["us"] / 1e3
-        out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": ach / HBM_PEAK_GBS, "traffic": None, "launch_us": round(kern[dom]["us"], 2),
-                           "launches_per_step": kern[dom]["calls_per_step"], "algorithmic_bytes_per_launch": kb[dom]}
-        out["kernels_us"] = {k: round(v["us"], 2) for k, v in sorted(kern.items(), key=lambda kv: -kv[1]["us"])}
-        out["step_roofline"] = {"algorithmic_bytes": s["algorithmic_bytes"], "achieved": s["gbs"], "frac": s["frac"],
-                                "unit": "GB/s"}
         if args.workload == "c3":
-            out["evict_sweep_ms"] = round(main_wl.evict_sweep_ms(), 3)
+            out["eviction"] = _c3_eviction(main_wl, ms_per_step)
     if not args.no_extra:
-        main_name = main_wl.name
         if args.workload != "c4":
             del main_wl
+            main_wl = None
             torch.cuda.empty_cache()
         for key, cls in classes.items():
             if key == args.workload:
@@ -798,24 +940,38 @@ def main():
                 extras[wl.name] = c2_summary(wl)
                 extras[wl.name]["ids_per_s"] = wl.ids_per_step / _event_ms(wl.step, 5) * 1e3
             else:
-                extras[wl.name] = step_summary(wl, timed_steps(wl, 8, 3))
+                extras[wl.name] = step_summary(wl, _timed_steps(wl, 8, 5), 8)
                 if key == "c3":
-                    extras[wl.name]["evict_sweep_ms"] = round(wl.evict_sweep_ms(), 3)
+                    extras[wl.name]["eviction"] = _c3_eviction(wl, extras[wl.name]["ms_per_step"])
             del wl
             torch.cuda.empty_cache()
-        if args.workload != "c4":
-            main_wl = classes[args.workload]() if not args.no_cpu_baseline else None
+        # the same steps through the drop-in module layer (EmbeddingEngine + sparse optimizer)
+        for key, cls, name in (("c4", ModulePath4, Config4.name), ("c5", ModulePath5, Config5.name)):
+            mp = cls()
+            ms = _timed_steps(mp, 10, 3)
+            target = out if key == args.workload else extras.get(name)
+            if target is not None:
+                target["module_path_ms"] = round(ms, 4)
+            del mp
+            torch.cuda.empty_cache()
+        if main_wl is None and not args.no_cpu_baseline:
+            main_wl = classes[args.workload]()
     if extras:
         out["workloads"] = extras
 
     if not args.no_cpu_baseline:
-        v, sample = main_wl.cpu_baseline(12.0)
-        out["cpu_baseline"] = {"value": v, "unit": "ids/s", "cores": 1, "kind": "port", "sample": sample}
-        if hasattr(main_wl, "cpu_reference"):
-            for threads in (1, min(16, os.cpu_count() or 1)):
-                ref = main_wl.cpu_reference(5.0, threads)
-                if ref is not None:
-                    out["cpu_reference_%dt" % threads] = ref
+        cores = min(16, os.cpu_count() or 1)
+        v, sample = main_wl.cpu_baseline(10.0)
+        port = {"value": v, "unit": "ids/s", "cores": 1, "kind": "port", "sample": sample}
+        ref = main_wl.cpu_reference(8.0, cores) if hasattr(main_wl, "cpu_reference") else None
+        if ref is not None:   # the reference's own CPU code, all host cores of this box's share
+            out["cpu_baseline"] = ref
+            out["cpu_baseline_port_1core"] = port
+            ref1 = main_wl.cpu_reference(4.0, 1)
+            if ref1 is not None:
+                out["cpu_baseline_reference_1core"] = ref1
+        else:
+            out["cpu_baseline"] = port
     from recis_amd import _lib
     out["device_errors"] = _lib.poll_device_errors()
     print(json.dumps(out))

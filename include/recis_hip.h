@@ -386,33 +386,62 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
  * Batch plan: dedup plus the transposed index. Unique ids (no duplicates, every id of the
  * batch present), an int32 inverse with unique_out[inverse[i]] == ids[i], the count, and the
  * occurrences grouped by unique id:
- *   row_start_out [n + 1]  list of unique id u = list[row_start[u] .. row_start[u+1]);
- *                          entries U .. n hold n
+ *   inverse_out   [n]      may be NULL when the caller does not need it
+ *   row_start_out [n + 1]  list of unique id u = list[row_start[u] .. row_start[u+1]) for u < U;
+ *                          row_start[U] = n; entries past U are not written
  *   list_out      [n]      occurrence indices grouped by unique id
  *   pos_out       [n]      position of occurrence i in list_out (may be NULL)
- *   hot_items_out [2*hot_cap] (row, chunk) work items for ids with more than 256
+ *   hot_items_out [2*hot_cap] (row, chunk) work items for ids with more than RECIS_PLAN_HOT_LEN
  *                          occurrences; hot_cap >= n/HOT_LEN + n/HOT_CHUNK + 2, or 0 to skip
  *   counts_out_dev [2]     device words: number of unique ids, number of hot items
  *   unique_count_host      host word or NULL: when given, the call returns only once the number
- *                          of unique ids is known and stores it there (the last kernels of the
- *                          plan may still be running: the wait is for the count alone)
+ *                          of unique ids is known and stores it there
  *   flags                  RECIS_PLAN_STAGE_COUNT: send the count towards the host but do not
  *                          wait; recis_unique_plan_count(stream) fetches it later (one staged
  *                          count per stream: fetch it before the next plan on that stream)
- * The unique ids are ordered by (hash bucket, first occurrence): the order, the inverse and
- * row_start depend on the input only; the order of the entries inside one id's list and of
- * the hot items is not specified. No global atomics are used: ids are partitioned by hash
- * and deduplicated in LDS.
+ * The unique ids are ordered by hash bucket (the top bits of a 64-bit mix of the id) and, inside a
+ * bucket, by the place of the id in the bucket's hash table: the order, the inverse and row_start
+ * depend on the input only; the order of the entries inside one id's list and of the hot items
+ * is not specified. Ids are partitioned by hash (a histogram and a scatter pass over the ids),
+ * every bucket is deduplicated in LDS by one workgroup, and the workgroups learn where their
+ * unique ids start from a look-back over one word per bucket: the only global atomics are one
+ * ticket per bucket and one addition per hot id.
  * With the plan, a gradient scatter over duplicated ids (the atomic loops of
  * csrc/ops/embedding_segment_reduce_kernel.cu:79-120, segment_ops_kernel.cu:133-165,
  * ragged_tile_kernel.cu:46-60 and the unique + index_add_ of
  * recis/nn/modules/hashtable.py:555-586) becomes a gather-reduce per unique row.
- * No counterpart in the reference.
+ * No counterpart in the reference (its dedup is the radix sort of
+ * csrc/ops/ids_partition_kernel.cu:86-131).
  */
 int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
                       int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
                       int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev,
                       int64_t* unique_count_host, int flags, void* stream);
+/*
+ * recis_unique_plan and the find-or-insert of its unique ids in an id map in one pass:
+ * index_out [n] receives, for u < U, the row of unique id u, exactly as
+ * recis_idmap_lookup(m, unique_out, U, index_out) would assign it (missing keys take rows in the
+ * order of the unique ids). The workgroup that deduplicates a hash bucket probes the map for the
+ * bucket's distinct ids while they are still in LDS (the bucket is a contiguous range of the
+ * map's home slots), so the unique ids are not read back and the probe kernel, its scan and its
+ * row-assignment pass over all ids (csrc/embedding/gpu_id_map.cu:19-45) shrink to one small
+ * launch over the NEW keys. Replaces ids_partition + GpuIdMap::Lookup of
+ * recis/nn/modules/hashtable.py:262-293. Keys -1 and -2 raise RECIS_DEVERR_INDEX_RANGE and get
+ * row -1. The map's capacity is checked as for recis_idmap_lookup_counted with n ids.
+ */
+int recis_unique_plan_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int64_t* unique_out,
+                             int32_t* inverse_out, int32_t* row_start_out, int32_t* list_out,
+                             int32_t* pos_out, int32_t* hot_items_out, int64_t hot_cap,
+                             int64_t* counts_out_dev, int64_t* index_out, int64_t* unique_count_host,
+                             int flags, void* stream);
+/* inverse_out [n] and / or pos_out [n] of a plan that was made without them (either may be NULL),
+ * from its row_start, list and counts. No counterpart in the reference. */
+int recis_plan_inverse_from_lists(const int32_t* row_start, const int32_t* list, const int64_t* counts_dev,
+                                  int64_t n, int32_t* inverse_out, int32_t* pos_out, void* stream);
+/* How many times a workgroup of the plan polls the look-back word of an earlier bucket before it
+ * gives up, raises RECIS_DEVERR_PLAN_OVERFLOW and goes on with zero (default 2^24: seconds; a
+ * word is due within microseconds). For tests of that path. */
+int recis_plan_set_spin_limit(int64_t polls);
 /* Waits for the count staged by the last recis_unique_plan(…, RECIS_PLAN_STAGE_COUNT, stream). */
 int recis_unique_plan_count(int64_t* unique_count_host, void* stream);
 /* The soft-error bits (RECIS_DEVERR_*) that were set on the device when the last count of `stream`

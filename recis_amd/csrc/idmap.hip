@@ -25,36 +25,10 @@
 #include <utility>
 
 #include "common.cuh"
+#include "idmap_internal.cuh"
 
 namespace recis_hip {
 namespace {
-
-struct alignas(16) Slot {
-  int64_t key;
-  int64_t val;
-};
-
-constexpr int64_t kEmpty = -1;
-constexpr int64_t kTomb = -2;
-constexpr int64_t kValUnset = -1;
-
-enum { ST_CUR = 0, ST_FREE, ST_LIVE, ST_OCC, ST_NNEW, ST_OLD_CUR, ST_OLD_FREE, ST_TMP, ST_DUPS, ST_WORDS };
-
-__device__ __forceinline__ uint64_t mix_key(int64_t key) {
-  uint64_t x = static_cast<uint64_t>(key);
-  x ^= x >> 33;
-  x *= 0xff51afd7ed558ccdULL;
-  x ^= x >> 33;
-  x *= 0xc4ceb9fe1a85ec53ULL;
-  x ^= x >> 33;
-  return x;
-}
-
-// First slot probed for a key: the TOP bits of the mixed key. Batches come out of the batch
-// plan ordered by the top bits of the same mix, so their probes walk the table front to back.
-__device__ __forceinline__ uint64_t home_slot(int64_t key, uint64_t mask) {
-  return mix_key(key) >> __builtin_clzll(mask);  // mask = capacity - 1, capacity a power of two >= 2
-}
 
 // Number of ids of a call whose count is still on the device: the first *n_dev of n_max.
 __device__ __forceinline__ int64_t counted(int64_t n_max, const int64_t* n_dev) {
@@ -63,27 +37,8 @@ __device__ __forceinline__ int64_t counted(int64_t n_max, const int64_t* n_dev) 
   return n < 0 ? 0 : (n < n_max ? n : n_max);
 }
 
-// Allocator words the host wants to know without waiting for the stream: written by the
-// last kernel of every call that changes them into pinned host memory, stamped with the
-// call's sequence number (written last, after a system-scope fence).
-enum { MR_SEQ = 0, MR_CUR, MR_FREE, MR_LIVE, MR_OCC, MR_WORDS };
-__device__ __forceinline__ void publish(const int64_t* state, volatile int64_t* mirror, int64_t seq) {
-  mirror[MR_CUR] = state[ST_CUR];
-  mirror[MR_FREE] = state[ST_FREE];
-  mirror[MR_LIVE] = state[ST_LIVE];
-  mirror[MR_OCC] = state[ST_OCC];
-  __threadfence_system();
-  mirror[MR_SEQ] = seq;
-}
 __global__ void publish_kernel(const int64_t* state, volatile int64_t* mirror, int64_t seq) {
   publish(state, mirror, seq);
-}
-
-__device__ __forceinline__ int64_t ld_relaxed(const int64_t* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_relaxed(int64_t* p, int64_t v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __global__ void __launch_bounds__(kBlock) fill_slots_kernel(Slot* t, int64_t n) {
@@ -140,64 +95,25 @@ find_or_claim_kernel(Slot* __restrict__ table, uint64_t mask, const int64_t* __r
       out[i] = -1;
     } else {
       const uint64_t h = home_slot(key, mask);
-      uint64_t p = h;
-      int64_t first_tomb = -1;
-      uint64_t probes = 0;
-      for (;;) {
-        // Hint from one plain 16-byte load (L1-cacheable, may be stale). Two things it shows cannot
-        // change while this kernel runs: a key with an assigned row, and a slot held by another key.
-        const longlong2 hint = *reinterpret_cast<const longlong2*>(&table[p]);
-        if (hint.x == key && hint.y >= 0) {
-          out[i] = hint.y;
+      const longlong2 hint = *reinterpret_cast<const longlong2*>(&table[h]);
+      int64_t value = -1, slot = -1;
+      switch (probe_or_claim(table, mask, key, h, hint, -(i + 2) /* pending, owner = occurrence i */, &value, &slot,
+                             &took_empty)) {
+        case kProbeFound:
+          out[i] = value;
           break;
-        }
-        if (hint.x != key && hint.x != kEmpty && hint.x != kTomb) {
-          p = (p + 1) & mask;
-          if (++probes > mask) {
-            raise_device_error(err, RECIS_DEVERR_TABLE_FULL);
-            out[i] = -1;
-            break;
-          }
-          continue;
-        }
-        const int64_t k = ld_relaxed(&table[p].key);
-        if (k == key) {
-          const int64_t v = ld_relaxed(&table[p].val);
-          if (v >= 0) {
-            out[i] = v;
-          } else {
-            sp = -(static_cast<int64_t>(p) + 2);
-            st_relaxed(&state[ST_DUPS], seq);  // "this call has duplicates": every writer stores the same word
-          }
+        case kProbeClaimed:
+          sp = slot;
+          is_new = true;
           break;
-        }
-        if (k == kEmpty) {
-          const bool use_tomb = first_tomb >= 0;
-          const int64_t target = use_tomb ? first_tomb : static_cast<int64_t>(p);
-          const int64_t expect = use_tomb ? kTomb : kEmpty;
-          const int64_t old = static_cast<int64_t>(atomicCAS(
-              reinterpret_cast<unsigned long long*>(&table[target].key),
-              static_cast<unsigned long long>(expect), static_cast<unsigned long long>(key)));
-          if (old == expect) {
-            st_relaxed(&table[target].val, -(i + 2));  // pending, owner = occurrence i
-            sp = target;
-            is_new = true;
-            took_empty = !use_tomb;
-            break;
-          }
-          // somebody else took that slot: start over, keys never vanish meanwhile
-          p = h;
-          first_tomb = -1;
-          probes = 0;
-          continue;
-        }
-        if (k == kTomb && first_tomb < 0) first_tomb = static_cast<int64_t>(p);
-        p = (p + 1) & mask;
-        if (++probes > mask) {
+        case kProbePending:
+          sp = -(slot + 2);
+          st_relaxed(&state[ST_DUPS], seq);  // "this call has duplicates": every writer stores the same word
+          break;
+        case kProbeFull:
           raise_device_error(err, RECIS_DEVERR_TABLE_FULL);
           out[i] = -1;
           break;
-        }
       }
     }
     slotpos[i] = sp;
@@ -242,16 +158,7 @@ scan_commit_kernel(int32_t* __restrict__ block_counts, int64_t nb, int64_t n, co
     run += c;
   }
   if (t == 1023) {
-    const int64_t total = partial[1023];
-    const int64_t cur = state[ST_CUR], fr = state[ST_FREE];
-    state[ST_OLD_CUR] = cur;
-    state[ST_OLD_FREE] = fr;
-    state[ST_NNEW] = total;
-    const int64_t fresh = fr >= total ? 0 : total - fr;
-    state[ST_CUR] = cur + fresh;
-    state[ST_FREE] = fr >= total ? fr - total : 0;
-    state[ST_LIVE] += total;
-    __threadfence();
+    commit_new_keys(state, partial[1023]);
     publish(state, mirror, seq);
   }
 }
@@ -270,9 +177,8 @@ assign_rows_kernel(Slot* __restrict__ table, const int64_t* __restrict__ slotpos
   int rank, total;
   block_rank(is_new, rank, total);
   if (!is_new) return;
-  const int64_t n_new = state[ST_NNEW];
-  const int64_t free_index = state[ST_OLD_FREE] - n_new + block_prefix[blockIdx.x] + rank;
-  const int64_t row = free_index >= 0 ? free_list[free_index] : state[ST_OLD_CUR] - (free_index + 1);
+  const int64_t row = row_of_new_key(block_prefix[blockIdx.x] + rank, state[ST_NNEW], state[ST_OLD_CUR],
+                                     state[ST_OLD_FREE], free_list);
   st_relaxed(&table[sp].val, row);
   out[i] = row;
 }
@@ -521,23 +427,6 @@ int64_t capacity_for(int64_t keys) {
 
 using namespace recis_hip;
 
-struct recis_idmap {
-  int device = 0;
-  int64_t capacity = 0;
-  Slot* table = nullptr;
-  int64_t* state = nullptr;     // device, ST_WORDS int64
-  int64_t* free_list = nullptr; // device
-  int64_t free_cap = 0;
-  // host-side upper bounds, refreshed by sync_stats()
-  int64_t occ_ub = 0;   // non-empty slots (live + tombstones)
-  int64_t free_ub = 0;  // entries in the free list
-  int* err = nullptr;
-  // pinned host mirror of the allocator words + the calls whose publication has not landed yet
-  volatile int64_t* mirror = nullptr;
-  int64_t seq_issued = 0;
-  std::deque<std::pair<int64_t, int64_t>> in_flight;  // (sequence number, ids of the call)
-};
-
 namespace {
 
 int alloc_table(recis_idmap* m, int64_t capacity, hipStream_t stream, Slot** out) {
@@ -641,6 +530,15 @@ int ensure_free_room(recis_idmap* m, int64_t incoming, hipStream_t stream) {
 }
 
 }  // namespace
+
+namespace recis_hip {
+int idmap_begin_call(recis_idmap* m, int64_t incoming, hipStream_t stream, int64_t* seq) {
+  if (int rc = ensure_table_room(m, incoming, stream)) return rc;
+  *seq = ++m->seq_issued;
+  return RECIS_OK;
+}
+void idmap_end_call(recis_idmap* m, int64_t seq, int64_t incoming) { m->in_flight.emplace_back(seq, incoming); }
+}  // namespace recis_hip
 
 extern "C" {
 

@@ -32,162 +32,90 @@
 #include <type_traits>
 
 #include "common.cuh"
+#include "idmap_internal.cuh"
 
 namespace recis_hip {
 namespace {
 
-constexpr int kPlanBlock = 1024;  // ids per tile == threads of the tile / scatter / hot kernels
-constexpr int kLdsSlots = 2048;   // LDS hash entries of a tile (load <= 1/2)
-constexpr int kBucketBlock = 256;
-constexpr int kBucketSlots = 1024;  // LDS hash entries of a bucket round
-constexpr int kMaxBuckets = 8192;
+constexpr int kTile = 8192;        // ids per workgroup of the histogram / scatter kernels (more when n is huge)
+constexpr int kPartBlock = 512;    // threads of those kernels
+constexpr int kMaxRows = 1024;     // workgroups of those kernels == histogram rows
 constexpr int kMinBuckets = 32;
-constexpr int kMaxRows = 512;  // histogram rows (= workgroups of the tile and scatter kernels)
+constexpr int kMaxBuckets = 8192;   // the histogram of a workgroup lives in LDS
+constexpr int kBucketIds = 2560;    // ids per bucket aimed at: an LDS table of 4096 home slots holds them all
+constexpr int kTabHome = 4096;      // home slots of a bucket's LDS table
+constexpr int kTabAll = kTabHome + 256;  // linear probing runs on past the last home slot and never wraps;
+                                         // slot kTabAll - 1 is a guard that stays empty
+constexpr int kSpecial = kTabAll;   // entry of the id that equals the empty marker
+constexpr int kBucketBlock = 512;
+constexpr int kPer = 9;             // consecutive table entries owned by a thread (9 * 512 > kTabAll)
+constexpr int kRegs = 8;            // bucket records of a thread whose table entry stays in registers
 constexpr int64_t kSetEmpty = -1;
-constexpr int32_t kNoPos = 0x7fffffff;
 constexpr int kHotLen = RECIS_PLAN_HOT_LEN;  // rows with more occurrences than this are "hot"
 constexpr int kHotChunk = RECIS_PLAN_HOT_CHUNK;  // occurrences per hot work item
+static_assert(kPer * kBucketBlock > kTabAll, "every table entry needs an owner");
 
-__device__ __forceinline__ uint64_t mix_id(int64_t key) {
-  uint64_t x = static_cast<uint64_t>(key);
-  x ^= x >> 33;
-  x *= 0xff51afd7ed558ccdULL;
-  x ^= x >> 33;
-  x *= 0xc4ceb9fe1a85ec53ULL;
-  x ^= x >> 33;
-  return x;
-}
-
-// One deduplicated run of a tile: `word` = (count - 1) << 10 | index of the record in its tile.
-struct alignas(16) Rec {
-  int64_t key;
-  int32_t pos;  // first position of the id in its tile (absolute)
-  uint32_t word;
-};
-
-// A unique id of a bucket, in bucket-local terms.
-struct alignas(16) URec {
-  int64_t key;
-  int32_t list_off;  // first list entry, relative to the bucket's first
-  int32_t cnt;
-};
+__device__ __forceinline__ uint64_t mix_id(int64_t key) { return mix_key(key); }
 
 struct PlanGeom {
   int64_t n;
-  int tiles;         // ceil(n / 1024)
-  int tiles_per_wg;  // tiles a workgroup of the tile / scatter kernels walks
-  int rows;          // workgroups of those kernels == histogram rows
-  int nb_log2;       // buckets = 1 << nb_log2
+  int rows;     // workgroups of the histogram / scatter kernels == histogram rows
+  int tile;     // ids per row (a multiple of kPartBlock)
+  int nb_log2;  // buckets = 1 << nb_log2
 };
 
-__device__ __forceinline__ int bucket_of(int64_t key, int nb_log2) {
-  return static_cast<int>(mix_id(key) >> (64 - nb_log2));
+__device__ __forceinline__ int bucket_of_mix(uint64_t mixed, int nb_log2) {
+  return static_cast<int>(mixed >> (64 - nb_log2));
+}
+// Home entry of an id in its bucket's LDS table: the 12 bits below the bucket bits, so that the
+// entries of a bucket lie in the order of the mixed id, like the buckets themselves.
+__device__ __forceinline__ int home_of_mix(uint64_t mixed, int nb_log2) {
+  return static_cast<int>(mixed >> (64 - nb_log2 - 12)) & (kTabHome - 1);
 }
 
-// Rank of the set flags among the 1024 threads of a workgroup (by thread index) and their total.
-__device__ __forceinline__ void block_rank1024(bool flag, int& rank, int& total, int* wave_counts /*[16]*/) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  const uint64_t ballot = __ballot(flag);
-  const int prior = __popcll(ballot & ((uint64_t(1) << lane) - 1));
-  if (lane == 0) wave_counts[wave] = __popcll(ballot);
-  __syncthreads();
-  int base = 0, tot = 0;
-#pragma unroll
-  for (int w = 0; w < kPlanBlock / kWave; ++w) {
-    const int c = wave_counts[w];
-    if (w < wave) base += c;
-    tot += c;
-  }
-  __syncthreads();
-  rank = base + prior;
-  total = tot;
-}
-
-// tile: LDS dedup of tiles of 1024 ids -> records, per-occurrence (record, rank in run), histogram row
-__global__ void __launch_bounds__(kPlanBlock)
-plan_tile_kernel(const int64_t* __restrict__ ids, PlanGeom g, Rec* __restrict__ tile_rec,
-                 int32_t* __restrict__ tile_nrec, uint32_t* __restrict__ occ_rec, uint16_t* __restrict__ hist,
-                 int64_t* __restrict__ counts) {
-  __shared__ int64_t l_key[kLdsSlots + 1];
-  __shared__ int32_t l_min[kLdsSlots + 1];
-  __shared__ int32_t l_cnt[kLdsSlots + 1];
-  __shared__ uint32_t l_hist[kMaxBuckets / 2];  // two 16-bit counters per word
-  __shared__ int wave_counts[kPlanBlock / kWave];
+// hist: ids per (row, bucket)
+__global__ void __launch_bounds__(kPartBlock)
+plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, int32_t* __restrict__ hist,
+                 int64_t* __restrict__ counts, int32_t* __restrict__ sync) {
+  extern __shared__ int32_t l_hist[];
   const int tid = threadIdx.x;
   const int nb = 1 << g.nb_log2;
-  if (blockIdx.x == 0 && tid < 2) counts[tid] = 0;
-  for (int w = tid; w < nb / 2; w += kPlanBlock) l_hist[w] = 0;
-  const int t_lo = blockIdx.x * g.tiles_per_wg;
-  const int t_hi = min(g.tiles, t_lo + g.tiles_per_wg);
-  int64_t key_next = 0;
-  if (static_cast<int64_t>(t_lo) * kPlanBlock + tid < g.n) key_next = ids[static_cast<int64_t>(t_lo) * kPlanBlock + tid];
-  for (int t = t_lo; t < t_hi; ++t) {
-    for (int e = tid; e <= kLdsSlots; e += kPlanBlock) {
-      l_key[e] = kSetEmpty;
-      l_min[e] = kNoPos;
-      l_cnt[e] = 0;
-    }
-    __syncthreads();
-    const int64_t i = static_cast<int64_t>(t) * kPlanBlock + tid;
-    const bool live = i < g.n;
-    const int64_t key = key_next;
-    if (t + 1 < t_hi && i + kPlanBlock < g.n) key_next = ids[i + kPlanBlock];  // in flight while this tile is worked
-    int e = 0, local_rank = 0;
-    if (live) {
-      if (key == kSetEmpty) {
-        e = kLdsSlots;  // reserved entry for the id that equals the empty marker
-      } else {
-        e = static_cast<int>(mix_id(key) >> 20) & (kLdsSlots - 1);
-        for (;;) {
-          int64_t k = l_key[e];
-          if (k == kSetEmpty) {
-            k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&l_key[e]),
-                                               static_cast<unsigned long long>(kSetEmpty),
-                                               static_cast<unsigned long long>(key)));
-            if (k == kSetEmpty) break;
-          }
-          if (k == key) break;
-          e = (e + 1) & (kLdsSlots - 1);  // at most 1024 distinct ids in 2048 entries
-        }
-      }
-      local_rank = atomicAdd(&l_cnt[e], 1);
-      atomicMin(&l_min[e], tid);
-    }
-    __syncthreads();
-    const bool first = live && l_min[e] == tid;
-    int j, total;
-    block_rank1024(first, j, total, wave_counts);
-    if (first) {
-      Rec r;
-      r.key = key;
-      r.pos = static_cast<int32_t>(i);
-      r.word = (static_cast<uint32_t>(l_cnt[e] - 1) << 10) | static_cast<uint32_t>(j);
-      tile_rec[static_cast<int64_t>(t) * kPlanBlock + j] = r;
-      l_min[e] = j;  // every occurrence of the run reads its record index here
-      const int b = bucket_of(key, g.nb_log2);
-      atomicAdd(&l_hist[b >> 1], 1u << ((b & 1) * 16));
-    }
-    if (tid == 0) tile_nrec[t] = total;
-    __syncthreads();
-    if (live) occ_rec[i] = (static_cast<uint32_t>(local_rank) << 10) | static_cast<uint32_t>(l_min[e]);
-    __syncthreads();
+  if (blockIdx.x == 0) {
+    if (tid < 2) counts[tid] = 0;
+    if (tid < 4) sync[tid] = 0;  // [1] bucket tickets, [2] finished workgroups of the row assignment
   }
-  uint32_t* row = reinterpret_cast<uint32_t*>(hist + static_cast<int64_t>(blockIdx.x) * nb);
-  for (int w = tid; w < nb / 2; w += kPlanBlock) row[w] = l_hist[w];
+  for (int b = tid; b < nb; b += kPartBlock) l_hist[b] = 0;
+  __syncthreads();
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
+  for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {  // four loads in flight
+    int64_t k[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int64_t i = i0 + x * kPartBlock;
+      k[x] = i < hi ? ids[i] : 0;
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+      if (i0 + x * kPartBlock < hi) atomicAdd(&l_hist[bucket_of_mix(mix_id(k[x]), g.nb_log2)], 1);
+  }
+  __syncthreads();
+  int32_t* row = hist + static_cast<int64_t>(blockIdx.x) * nb;
+  for (int b = tid; b < nb; b += kPartBlock) row[b] = l_hist[b];
 }
 
-// colscan: for every bucket, exclusive scan of its histogram column over the rows.
-// Workgroup = 32 buckets x 32 groups of rows.
+// colscan: for every bucket, exclusive scan of its histogram column over the rows, in place, and
+// the bucket's total. Workgroup = kColBuckets buckets x (1024 / kColBuckets) groups of rows.
+constexpr int kColBuckets = 16;
+constexpr int kColGroups = 1024 / kColBuckets;
 __global__ void __launch_bounds__(1024)
-plan_colscan_kernel(const uint16_t* __restrict__ hist, PlanGeom g, int32_t* __restrict__ off,
-                    int32_t* __restrict__ bucket_total) {
-  __shared__ int32_t part[32][33];
+plan_colscan_kernel(int32_t* __restrict__ hist, PlanGeom g, int32_t* __restrict__ bucket_total) {
+  __shared__ int32_t part[kColGroups][kColBuckets + 1];
   const int nb = 1 << g.nb_log2;
-  const int bl = threadIdx.x & 31, rg = threadIdx.x >> 5;
-  const int b = blockIdx.x * 32 + bl;
-  const int per = (g.rows + 31) / 32;
-  const int r_lo = min(g.rows, rg * per), r_hi = min(g.rows, r_lo + per);
+  const int t = threadIdx.x;
+  const int bl = t % kColBuckets, rg = t / kColBuckets;
+  const int b = blockIdx.x * kColBuckets + bl;
+  const int per_rows = (g.rows + kColGroups - 1) / kColGroups;
+  const int r_lo = min(g.rows, rg * per_rows), r_hi = min(g.rows, r_lo + per_rows);
   int32_t sum = 0;
   for (int r = r_lo; r < r_hi; ++r) sum += hist[static_cast<int64_t>(r) * nb + b];
   part[rg][bl] = sum;
@@ -197,294 +125,717 @@ plan_colscan_kernel(const uint16_t* __restrict__ hist, PlanGeom g, int32_t* __re
   for (int r = r_lo; r < r_hi; ++r) {
     const int64_t at = static_cast<int64_t>(r) * nb + b;
     const int32_t c = hist[at];
-    off[at] = run;
+    hist[at] = run;
     run += c;
   }
-  if (rg == 31) bucket_total[b] = run;
+  if (rg == kColGroups - 1) bucket_total[b] = run;
 }
 
-// Exclusive scan of one or two int32 arrays of nb <= 8192 entries by one workgroup;
-// out arrays have nb + 1 entries (the last one is the total); total of the first to total_out.
-__global__ void __launch_bounds__(1024)
-plan_scan_kernel(const int32_t* __restrict__ in0, int32_t* __restrict__ out0, const int32_t* __restrict__ in1,
-                 int32_t* __restrict__ out1, int nb, int64_t* __restrict__ total_out,
-                 volatile int64_t* total_host, const int* __restrict__ err) {
-  __shared__ int32_t partial[1024];
-  const int t = threadIdx.x;
-  const int per = (nb + 1023) / 1024;
+// Exclusive scan of in[0 .. nb) into LDS (start[0 .. nb], start[nb] = the total) by the calling
+// workgroup of kPartBlock threads: a thread sums its own stretch, the waves scan those sums with
+// shuffles, one barrier joins the waves. `in` may be global or LDS memory (in == start is fine);
+// `partial` is scratch of kPartBlock / kWave words. Ends with a barrier.
+__device__ __forceinline__ void scan_counts(const int32_t* in, int nb, int32_t* start, int32_t* partial) {
+  const int t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
+  const int per = (nb + kPartBlock - 1) / kPartBlock;
   const int lo = min(nb, t * per), hi = min(nb, lo + per);
-  for (int pass = 0; pass < 2; ++pass) {
-    const int32_t* in = pass ? in1 : in0;
-    int32_t* out = pass ? out1 : out0;
-    if (in == nullptr) break;
-    int32_t sum = 0;
-    for (int b = lo; b < hi; ++b) sum += in[b];
-    partial[t] = sum;
-    __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) {
-      const int32_t add = t >= o ? partial[t - o] : 0;
-      __syncthreads();
-      partial[t] += add;
-      __syncthreads();
-    }
-    int32_t run = t ? partial[t - 1] : 0;
-    for (int b = lo; b < hi; ++b) {
-      const int32_t c = in[b];
-      out[b] = run;
-      run += c;
-    }
-    if (t == 1023) {
-      out[nb] = partial[1023];
-      if (pass == 0 && total_out) total_out[0] = partial[1023];
-      if (pass == 0 && total_host) {  // pinned host words: no copy kernel needed
-        total_host[1] = err ? __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
-        total_host[0] = partial[1023];
-      }
-    }
-    __syncthreads();
+  int32_t sum = 0;
+  for (int q = lo; q < hi; ++q) sum += in[q];
+  int32_t incl = sum;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int32_t y = __shfl_up(incl, o, kWave);
+    if (lane >= o) incl += y;
   }
-}
-
-// scatter: records of a workgroup's tiles go to their buckets
-__global__ void __launch_bounds__(kPlanBlock)
-plan_scatter_kernel(const Rec* __restrict__ tile_rec, const int32_t* __restrict__ tile_nrec, PlanGeom g,
-                    const int32_t* __restrict__ off, const int32_t* __restrict__ bucket_start,
-                    Rec* __restrict__ bucket_rec) {
-  __shared__ int32_t cursor[kMaxBuckets];
-  const int nb = 1 << g.nb_log2;
-  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nb;
-  for (int b = threadIdx.x; b < nb; b += kPlanBlock) cursor[b] = bucket_start[b] + off_row[b];
+  if (lane == kWave - 1) partial[wave] = incl;
   __syncthreads();
-  const int t_lo = blockIdx.x * g.tiles_per_wg;
-  const int t_hi = min(g.tiles, t_lo + g.tiles_per_wg);
-  for (int t0 = t_lo; t0 < t_hi; t0 += 4) {  // four tiles' loads in flight
-    Rec r[4];
-    bool have[4];
+  int32_t run = incl - sum, total = 0;
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int t = t0 + x;
-      have[x] = t < t_hi && static_cast<int>(threadIdx.x) < tile_nrec[t];
-      if (have[x]) r[x] = tile_rec[static_cast<int64_t>(t) * kPlanBlock + threadIdx.x];
-    }
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      if (have[x]) bucket_rec[atomicAdd(&cursor[bucket_of(r[x].key, g.nb_log2)], 1)] = r[x];
-    }
+  for (int w = 0; w < kPartBlock / kWave; ++w) {
+    const int32_t c = partial[w];
+    if (w < wave) run += c;
+    total += c;
   }
+  for (int q = lo; q < hi; ++q) {
+    const int32_t c = in[q];
+    start[q] = run;
+    run += c;
+  }
+  if (t == 0) start[nb] = total;
+  __syncthreads();
 }
 
-// bucket: dedup of the records of one bucket in LDS. A bucket normally holds a few hundred
-// distinct ids (its records can be many more: a hot id brings one record per tile). When the
-// distinct ids do not fit the LDS table, the bucket is started over in twice as many rounds:
-// round r admits the ids whose hash falls in its share, so every id is handled in exactly one
-// round. The first kBucketRegs
-// records of a thread stay in registers between the two passes over the records; further
-// ones (rare: hot buckets) go through `result` in global memory.
-constexpr int kBucketRegs = 4;
-
-__device__ __forceinline__ bool in_round(int64_t key, uint32_t rounds, uint32_t round) {
-  return rounds == 1 || static_cast<uint32_t>((mix_id(key) >> 8) & 0xffffff) % rounds == round;
-}
-
-__global__ void __launch_bounds__(kBucketBlock)
-plan_bucket_kernel(const Rec* __restrict__ bucket_rec, const int32_t* __restrict__ bucket_start, PlanGeom g,
-                   int2* __restrict__ result, URec* __restrict__ bucket_uniq, int32_t* __restrict__ ucnt,
-                   int32_t* __restrict__ ocnt, int* __restrict__ err) {
-  constexpr int kPad = 16;  // d_min is read 16 entries at a time
-  __shared__ int64_t l_key[kBucketSlots + 1];
-  __shared__ int32_t l_min[kBucketSlots + 1];
-  __shared__ int32_t l_cnt[kBucketSlots + 1];
-  __shared__ uint16_t l_rank[kBucketSlots + 2];
-  __shared__ uint16_t d_ent[kBucketSlots + 2];
-  __shared__ __attribute__((aligned(16))) int32_t d_min[kBucketSlots + 1 + kPad];
-  __shared__ int32_t s_cnt[kBucketSlots + 1];
-  __shared__ int wave_counts[kBucketBlock / kWave];
-  __shared__ int s_n_ent, s_total, s_overflow;
+// scatter: (id, position) of every occurrence goes to its bucket. Every workgroup scans the bucket
+// totals for itself (a thousand words), so no kernel stands between the column scan and this one;
+// the first workgroup also leaves bucket_start [nb + 1] for the bucket kernel and clears that
+// kernel's look-back words.
+__global__ void __launch_bounds__(kPartBlock)
+plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int32_t* __restrict__ off,
+                    const int32_t* __restrict__ bucket_total, int32_t* __restrict__ bucket_start,
+                    unsigned long long* __restrict__ agg, int64_t* __restrict__ bkt_id,
+                    int32_t* __restrict__ bkt_pos) {
+  extern __shared__ int32_t cursor[];  // [nb + 1], then kPartBlock words of scan scratch
   const int tid = threadIdx.x;
-  const int b = blockIdx.x;
-  const int32_t r_lo = bucket_start[b], r_hi = bucket_start[b + 1];
-  const int nrec = r_hi - r_lo;
-  uint32_t rounds = 1;
-  Rec reg[kBucketRegs];
-#pragma unroll
-  for (int x = 0; x < kBucketRegs; ++x) {
-    const int32_t q = r_lo + tid + x * kBucketBlock;
-    if (q < r_hi) reg[x] = bucket_rec[q];
+  const int nb = 1 << g.nb_log2;
+  scan_counts(bucket_total, nb, cursor, cursor + nb + 1);
+  if (blockIdx.x == 0) {
+    for (int b = tid; b <= nb; b += kPartBlock) bucket_start[b] = cursor[b];
+    for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
   }
-  int32_t u_done = 0, occ_done = 0;
-
-  // inserts one record; returns the entry (or -1) and the offset of the record's run in the id's list
-  auto insert = [&](const Rec& r, int& e, int& base) {
-    if (r.key == kSetEmpty) {
-      e = kBucketSlots;
-    } else {
-      e = static_cast<int>(mix_id(r.key) >> 32) & (kBucketSlots - 1);
-      int probes = 0;
-      for (;;) {
-        int64_t k = l_key[e];
-        if (k == kSetEmpty) {
-          k = static_cast<int64_t>(atomicCAS(reinterpret_cast<unsigned long long*>(&l_key[e]),
-                                             static_cast<unsigned long long>(kSetEmpty),
-                                             static_cast<unsigned long long>(r.key)));
-          if (k == kSetEmpty) break;
-        }
-        if (k == r.key) break;
-        e = (e + 1) & (kBucketSlots - 1);
-        if (++probes >= kBucketSlots) {  // table full: more distinct ids than a round can take
-          e = -1;
-          base = 0;
-          s_overflow = 1;
-          return;
-        }
+  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nb;
+  __syncthreads();
+  for (int b = tid; b < nb; b += kPartBlock) cursor[b] += off_row[b];
+  __syncthreads();
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
+  for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {
+    int64_t k[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int64_t i = i0 + x * kPartBlock;
+      k[x] = i < hi ? ids[i] : 0;
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int64_t i = i0 + x * kPartBlock;
+      if (i < hi) {
+        const int32_t p = atomicAdd(&cursor[bucket_of_mix(mix_id(k[x]), g.nb_log2)], 1);
+        bkt_id[p] = k[x];
+        bkt_pos[p] = static_cast<int32_t>(i);
       }
     }
-    base = atomicAdd(&l_cnt[e], static_cast<int>(r.word >> 10) + 1);
-    atomicMin(&l_min[e], r.pos);
-    if (base == 0) {  // first run of the id: list the entry
-      const int k = atomicAdd(&s_n_ent, 1);
-      d_ent[k] = static_cast<uint16_t>(e);
-      if (k >= kBucketSlots * 7 / 8) s_overflow = 1;  // too loaded to go on probing
+  }
+}
+
+// scatter in runs, for tiles of at most kTile ids and few enough buckets that a tile sends several
+// ids to each: a workgroup ranks its ids inside their buckets (LDS counters), orders them by bucket
+// in LDS and writes them out in that order, so that the ids a tile sends to one bucket leave
+// together as one run of consecutive words instead of one scattered 8-byte and one scattered
+// 4-byte store per id (scattered stores run at some 1e11 per second on this part whatever their
+// size).
+constexpr int kTilePer = kTile / kPartBlock;
+__global__ void __launch_bounds__(kPartBlock)
+plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int32_t* __restrict__ off,
+                         const int32_t* __restrict__ bucket_total, int32_t* __restrict__ bucket_start,
+                         unsigned long long* __restrict__ agg, int64_t* __restrict__ bkt_id,
+                         int32_t* __restrict__ bkt_pos) {
+  extern __shared__ int32_t lds[];
+  const int tid = threadIdx.x;
+  const int nb = 1 << g.nb_log2;
+  int32_t* gbase = lds;               // [nb + 1] where the tile's ids of a bucket go
+  int32_t* first = lds + nb + 1;      // [nb + 1] ids of the tile per bucket, then where they start in bucket order
+  int32_t* partial = first + nb + 1;  // [kPartBlock] scan scratch
+  uint16_t* sorted = reinterpret_cast<uint16_t*>(partial + kPartBlock);  // [kTile] the tile's ids in bucket order
+  uint16_t* sorted_bucket = sorted + kTile;                              // [kTile] and their buckets
+  for (int b = tid; b <= nb; b += kPartBlock) first[b] = 0;
+  scan_counts(bucket_total, nb, gbase, partial);
+  if (blockIdx.x == 0) {
+    for (int b = tid; b <= nb; b += kPartBlock) bucket_start[b] = gbase[b];
+    for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
+  }
+  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nb;
+  __syncthreads();
+  for (int b = tid; b < nb; b += kPartBlock) gbase[b] += off_row[b];
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile;
+  const int n_here = static_cast<int>(min(g.n, lo + g.tile) - lo);
+  int64_t k[kTilePer];
+  uint16_t rank[kTilePer], bucket[kTilePer];
+#pragma unroll
+  for (int x = 0; x < kTilePer; ++x) {  // all loads in flight
+    const int i = tid + x * kPartBlock;
+    k[x] = i < n_here ? ids[lo + i] : 0;
+  }
+#pragma unroll
+  for (int x = 0; x < kTilePer; ++x) {
+    rank[x] = 0;
+    bucket[x] = static_cast<uint16_t>(bucket_of_mix(mix_id(k[x]), g.nb_log2));
+    if (tid + x * kPartBlock < n_here) rank[x] = static_cast<uint16_t>(atomicAdd(&first[bucket[x]], 1));
+  }
+  __syncthreads();
+  scan_counts(first, nb, first, partial);  // counts -> starts in bucket order
+#pragma unroll
+  for (int x = 0; x < kTilePer; ++x) {
+    const int i = tid + x * kPartBlock;
+    if (i < n_here) {
+      const int j = first[bucket[x]] + rank[x];
+      sorted[j] = static_cast<uint16_t>(i);
+      sorted_bucket[j] = bucket[x];
+    }
+  }
+  __syncthreads();
+  for (int j0 = tid; j0 < n_here; j0 += 4 * kPartBlock) {
+    int64_t key[4];
+    int i[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int j = j0 + x * kPartBlock;
+      i[x] = j < n_here ? sorted[j] : 0;
+      key[x] = j < n_here ? ids[lo + i[x]] : 0;  // the tile was read a moment ago: a cache hit
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int j = j0 + x * kPartBlock;
+      if (j >= n_here) continue;
+      const int b = sorted_bucket[j];
+      const int32_t d = gbase[b] + (j - first[b]);
+      bkt_id[d] = key[x];
+      bkt_pos[d] = static_cast<int32_t>(lo + i[x]);
+    }
+  }
+}
+
+// A new key of the fused find-or-insert: where it sits in the id map, which unique id it is.
+struct alignas(16) NewRec {
+  int64_t slot;
+  int64_t u;
+};
+
+struct BucketArgs {
+  const int64_t* bkt_id;
+  const int32_t* bkt_pos;
+  const int32_t* bucket_start;  // [nb + 1]
+  PlanGeom g;
+  unsigned long long* agg;  // [nb] look-back words: distinct ids per bucket
+  int32_t* new_count;       // [nb] keys new to the id map per bucket
+  int32_t* sync;            // [1] = bucket tickets, [2] = workgroups of the row assignment that are done
+  int64_t* unique_out;
+  int32_t* inverse;    // may be NULL
+  int32_t* row_start;
+  int32_t* list;
+  int32_t* pos_out;    // may be NULL
+  int64_t* counts;
+  int32_t* hot_items;
+  int64_t hot_cap;
+  volatile int64_t* staged;  // pinned host words (unique count, soft-error bits) or NULL
+  int* err;
+  uint32_t spin_limit;
+  // fused find-or-insert in the id map
+  Slot* table;
+  uint64_t mask;
+  int64_t* index_out;
+  int64_t* state;
+  volatile int64_t* mirror;
+  int64_t seq;
+  NewRec* new_list;  // [n] the new keys of a bucket, at the bucket's own entries
+};
+
+__device__ __forceinline__ bool in_round(uint64_t mixed, uint32_t rounds, uint32_t round) {
+  return rounds == 1 || static_cast<uint32_t>((mixed >> 8) & 0xffffff) % rounds == round;
+}
+
+// Exclusive scan of a 64-bit value over the kBucketBlock threads of a workgroup (two counters
+// packed in one word); `total` is the sum over all threads. Ends with a barrier.
+__device__ __forceinline__ unsigned long long block_scan_u64(unsigned long long v, unsigned long long* s_wave,
+                                                             unsigned long long& total) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  unsigned long long incl = v;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const unsigned long long y = __shfl_up(incl, o, kWave);
+    if (lane >= o) incl += y;
+  }
+  __syncthreads();  // s_wave may still be read from the previous scan
+  if (lane == kWave - 1) s_wave[wave] = incl;
+  __syncthreads();
+  unsigned long long before = incl - v, tot = 0;
+#pragma unroll
+  for (int w = 0; w < kBucketBlock / kWave; ++w) {
+    const unsigned long long c = s_wave[w];
+    if (w < wave) before += c;
+    tot += c;
+  }
+  total = tot;
+  return before;
+}
+
+// atomicAdd(&arr[e], 1) for every lane with `active`, each lane getting back a value that no other
+// lane gets for the same entry. Ids of low-cardinality features repeat thousands of times in a
+// bucket, and atomics of one wave on one LDS word are served one after the other (some 3 ns each:
+// a bucket with a 6500-fold id spent 20 us there); so when many lanes of the wave name the entry
+// of the first (or of the last) active lane, one of them adds their number and hands out the places.
+__device__ __forceinline__ int32_t wave_add_one(int32_t* arr, int e, bool active) {
+  int32_t result = 0;
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const uint64_t todo = __ballot(active);
+    if (todo == 0) break;
+    const int leader = it == 0 ? __ffsll(static_cast<unsigned long long>(todo)) - 1 : 63 - __clzll(todo);
+    const int e_l = __shfl(e, leader, kWave);
+    const uint64_t same = __ballot(active && e == e_l);
+    const int n_same = __popcll(same);
+    if (n_same < 8) continue;
+    int32_t base = 0;
+    if (lane == leader) base = atomicAdd(&arr[e_l], n_same);
+    base = __shfl(base, leader, kWave);
+    if (active && e == e_l) {
+      result = base + __popcll(same & ((uint64_t(1) << lane) - 1));
+      active = false;
+    }
+  }
+  if (active) result = atomicAdd(&arr[e], 1);
+  return result;
+}
+
+constexpr unsigned long long kAggFlag = 1ull << 62, kPrefixFlag = 2ull << 62, kAggValue = (1ull << 62) - 1;
+
+// Sum of the distinct-id counts of all buckets before bucket b, by the whole workgroup: thread t
+// reads the look-back word of bucket hi - t (nearest first), so one round covers the 512 nearest
+// predecessors; rounds go on until a word carries an inclusive prefix. Every predecessor has
+// started (workgroups are dispatched in the order of their index) and publishes its word before it waits for anybody,
+// so each word arrives after a bounded time; a wait that outlasts spin_limit polls raises the
+// plan-overflow error bit and goes on with zero. A word carries its whole message (flag and value
+// in one 64-bit atomic), so relaxed device-scope atomics are enough: nothing else has to become
+// visible with it. (Release / acquire at device scope write back and invalidate the whole L2 of the
+// XCD on this part: tens of microseconds per workgroup.) Every thread calls; ends with a barrier.
+__device__ __forceinline__ int64_t look_back(unsigned long long* __restrict__ agg, int b, uint32_t spin_limit,
+                                             int* err, unsigned long long* s_look /* [kBucketBlock / kWave] */) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int64_t sum = 0;
+  for (int hi = b - 1;; hi -= kBucketBlock) {
+    const int j = hi - static_cast<int>(threadIdx.x);
+    unsigned long long w = kPrefixFlag;  // before the first bucket: an inclusive prefix of zero
+    if (j >= 0) {
+      uint32_t polls = 0;
+      for (;;) {
+        w = __hip_atomic_load(&agg[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((w >> 62) != 0) break;
+        if (++polls > spin_limit) {
+          raise_device_error(err, RECIS_DEVERR_PLAN_OVERFLOW);
+          w = kPrefixFlag;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+    }
+    const uint64_t is_prefix = __ballot((w >> 62) == 2);
+    const int first = is_prefix ? __ffsll(static_cast<unsigned long long>(is_prefix)) - 1 : kWave;
+    unsigned long long v = lane <= first ? (w & kAggValue) : 0;
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    __syncthreads();  // s_look may still be read
+    if (lane == 0) s_look[wave] = v | (is_prefix ? kPrefixFlag : 0ull);
+    __syncthreads();
+    bool done = false;
+#pragma unroll
+    for (int q = 0; q < kBucketBlock / kWave; ++q) {  // waves hold nearer buckets first
+      if (done) continue;
+      const unsigned long long x = s_look[q];
+      sum += static_cast<int64_t>(x & kAggValue);
+      done = (x >> 62) != 0;
+    }
+    if (done) break;
+  }
+  __syncthreads();
+  return sum;
+}
+
+// bucket: one workgroup per bucket, in the order of the workgroup index. The bucket's ids are
+// deduplicated in an LDS hash table with linear probing that never wraps. Insertion is the
+// phase-concurrent, history-independent kind: of two ids that want the same entry the one with the
+// smaller unsigned value stays and the other moves on, so the table ends up the same whatever the
+// order of the insertions, and the position of an id in the table is a function of the input
+// alone. That position orders the unique ids: one scan over the table gives every id its rank and
+// the start of its list. The number of distinct ids of all earlier buckets comes from a decoupled
+// look-back over one word per bucket. With PROBE, every distinct id is looked up in the id map
+// from here (find or claim); ids the map did not hold are listed per bucket, in the order of the
+// unique ids, for plan_assign_new_kernel to give them rows.
+// A bucket with more distinct ids than the table takes is worked in `rounds` hash-partitioned
+// rounds (first a dry run over all rounds to find a round count that fits).
+template <bool PROBE>
+__global__ void __launch_bounds__(kBucketBlock, 4)
+plan_bucket_kernel(BucketArgs a) {
+  __shared__ int64_t l_key[kTabAll + 1];
+  __shared__ int32_t l_cnt[kTabAll + 1];  // occurrences of the entry; after ranking: its next free list position
+  __shared__ int32_t l_u[kTabAll + 1];    // rank of the entry among the distinct ids of the round
+  __shared__ unsigned long long s_wave[kBucketBlock / kWave];
+  __shared__ int s_overflow;
+  const int tid = threadIdx.x;
+  const int nb_log2 = a.g.nb_log2;
+  // Buckets are taken in the order of the workgroup index. The look-back below waits for the
+  // workgroups of lower index; those have been dispatched before this one (the dispatcher walks
+  // the grid in order), so they run and publish without waiting for anything later. A ticket from
+  // a global counter would say the same, but a thousand atomics on one word are served one after
+  // the other (25 ns each on this part: the last workgroup would start 25 us late).
+  const int b = blockIdx.x;
+  const int32_t r_lo = a.bucket_start[b], r_hi = a.bucket_start[b + 1];
+  for (int e = tid; e <= kTabAll; e += kBucketBlock) {
+    l_key[e] = kSetEmpty;
+    l_cnt[e] = 0;
+  }
+  if (tid == 0) s_overflow = 0;
+  __syncthreads();
+  int e_reg[kRegs];  // table entry of the thread's first kRegs records (-2: none / not of this round)
+  int32_t pos_reg[kRegs];
+#pragma unroll
+  for (int x = 0; x < kRegs; ++x) {  // an empty bucket never enters the loops that set them
+    e_reg[x] = -2;
+    pos_reg[x] = 0;
+  }
+
+  // enters `key` into the table; false when the table cannot take it
+  auto insert = [&](int64_t key, uint64_t mixed) -> bool {
+    if (key == kSetEmpty) {
+      l_key[kSpecial] = 0;  // every writer stores the same word
+      return true;
+    }
+    unsigned long long v = static_cast<unsigned long long>(key);
+    int e = home_of_mix(mixed, nb_log2);
+    for (;;) {
+      const unsigned long long c = *reinterpret_cast<volatile unsigned long long*>(&l_key[e]);
+      if (c == v) return true;
+      if (c < v) {  // the id there keeps its place (the empty marker is the largest value)
+        if (++e >= kTabAll - 1) return false;  // the guard entry stays empty
+        continue;
+      }
+      if (atomicCAS(reinterpret_cast<unsigned long long*>(&l_key[e]), c, v) != c) continue;  // it changed: look again
+      if (c == static_cast<unsigned long long>(kSetEmpty)) return true;
+      v = c;  // the id that sat here moves on
+      if (++e >= kTabAll - 1) return false;
     }
   };
-  auto origin_of = [](const Rec& r) { return (static_cast<int64_t>(r.pos) >> 10 << 10) | (r.word & 1023u); };
+  auto find_from = [&](int64_t key, int e) -> int {  // e = the id's home entry
+    if (key == kSetEmpty) return kSpecial;
+    for (;;) {
+      const int64_t k = l_key[e];
+      if (k == key) return e;
+      if (k == kSetEmpty || ++e >= kTabAll - 1) return -1;
+    }
+  };
+  // the table of one round (cleared by the caller): every id of the round entered (pass 1), its
+  // occurrences counted (pass 2). The bucket's records are taken kRegs per thread at a time, all
+  // loads of a turn in flight together; for the first turn the table entry stays in e_reg.
+  auto build = [&](uint32_t rounds, uint32_t round) {
+    bool ok = true;
+    for (int32_t q0 = r_lo; q0 < r_hi; q0 += kRegs * kBucketBlock) {
+      int64_t k[kRegs];
+#pragma unroll
+      for (int x = 0; x < kRegs; ++x) {
+        const int32_t q = q0 + tid + x * kBucketBlock;
+        k[x] = q < r_hi ? a.bkt_id[q] : 0;
+        if (q0 == r_lo) pos_reg[x] = q < r_hi ? a.bkt_pos[q] : 0;
+      }
+#pragma unroll
+      for (int x = 0; x < kRegs; ++x) {
+        int mark = -2;  // not of this round
+        if (q0 + tid + x * kBucketBlock < r_hi) {
+          const uint64_t mixed = mix_id(k[x]);
+          if (in_round(mixed, rounds, round)) {
+            mark = -3 - home_of_mix(mixed, nb_log2);  // pass 2 starts its search there
+            ok = insert(k[x], mixed) && ok;
+          }
+        }
+        if (q0 == r_lo) e_reg[x] = mark;
+      }
+    }
+    if (!ok) s_overflow = 1;
+    __syncthreads();
+    if (s_overflow) return;
+    for (int32_t q0 = r_lo; q0 < r_hi; q0 += kRegs * kBucketBlock) {
+      const bool first_turn = q0 == r_lo;
+      int64_t k[kRegs];
+#pragma unroll
+      for (int x = 0; x < kRegs; ++x) {
+        const int32_t q = q0 + tid + x * kBucketBlock;
+        k[x] = q < r_hi ? a.bkt_id[q] : 0;  // the first turn reads what it has just read: a cache hit
+      }
+#pragma unroll
+      for (int x = 0; x < kRegs; ++x) {
+        int e = -2;
+        if (q0 + tid + x * kBucketBlock < r_hi) {
+          if (first_turn) {
+            if (e_reg[x] <= -3) e = find_from(k[x], -3 - e_reg[x]);
+          } else {
+            const uint64_t mixed = mix_id(k[x]);
+            if (in_round(mixed, rounds, round)) e = find_from(k[x], home_of_mix(mixed, nb_log2));
+          }
+        }
+        if (first_turn) e_reg[x] = e;
+        wave_add_one(l_cnt, e, e >= 0);
+      }
+    }
+    __syncthreads();
+  };
+  auto clear = [&]() {
+    __syncthreads();
+    for (int e = tid; e <= kTabAll; e += kBucketBlock) {
+      l_key[e] = kSetEmpty;
+      l_cnt[e] = 0;
+    }
+    if (tid == 0) s_overflow = 0;
+    __syncthreads();
+  };
+
+  uint32_t rounds = 1;
+  build(1, 0);
+  while (s_overflow) {  // dry runs: double the rounds until every round fits
+    if (rounds >= (1u << 16)) {
+      if (tid == 0) raise_device_error(a.err, RECIS_DEVERR_PLAN_OVERFLOW);
+      break;  // entries that found no room are dropped (flagged)
+    }
+    rounds *= 2;
+    bool fits = true;
+    for (uint32_t r = 0; r < rounds && fits; ++r) {
+      clear();
+      build(rounds, r);
+      fits = !s_overflow;
+    }
+    if (fits) {
+      clear();
+      build(rounds, 0);
+      break;
+    }
+  }
+
+  int64_t u_base = 0;  // distinct ids of all earlier buckets
+  // the rare case: learn the base first, publish the total after the last round
+  if (rounds > 1) u_base = look_back(a.agg, b, a.spin_limit, a.err, s_wave);
+  const int32_t l_base = r_lo;  // the bucket's occurrences are its list entries
+  int32_t u_done = 0, l_done = 0, new_done = 0;
+  const int s_lo = tid * kPer;
 
   for (uint32_t round = 0; round < rounds; ++round) {
-    for (int e = tid; e <= kBucketSlots; e += kBucketBlock) {
-      l_key[e] = kSetEmpty;
-      l_min[e] = kNoPos;
-      l_cnt[e] = 0;
-      l_rank[e] = 0;
+    if (round > 0) {
+      clear();
+      build(rounds, round);
     }
-    if (tid == 0) {
-      s_n_ent = 0;
-      s_overflow = 0;
-    }
-    __syncthreads();
-    // A: insert the round's records
-    int e_reg[kBucketRegs], base_reg[kBucketRegs];
+    // ---- rank the entries this thread owns: position in the table = order of the unique ids
+    int32_t cnt[kPer];
+    unsigned long long mine = 0;
 #pragma unroll
-    for (int x = 0; x < kBucketRegs; ++x) {
-      e_reg[x] = -2;  // not of this round
-      base_reg[x] = 0;
-      const int32_t q = r_lo + tid + x * kBucketBlock;
-      if (q < r_hi && in_round(reg[x].key, rounds, round)) insert(reg[x], e_reg[x], base_reg[x]);
+    for (int x = 0; x < kPer; ++x) {
+      const int e = s_lo + x;
+      const bool occ = e <= kTabAll && l_key[e] != kSetEmpty;
+      cnt[x] = occ ? l_cnt[e] : -1;  // -1: not occupied
+      if (occ) mine += (static_cast<unsigned long long>(cnt[x]) << 32) | 1ull;
     }
-    for (int32_t q = r_lo + tid + kBucketRegs * kBucketBlock; q < r_hi; q += kBucketBlock) {
-      const Rec r = bucket_rec[q];
-      if (!in_round(r.key, rounds, round)) continue;
-      int e, base;
-      insert(r, e, base);
-      result[origin_of(r)] = make_int2(e, base);
-    }
-    __syncthreads();
-    if (s_overflow) {  // start the bucket over with twice the rounds
-      __syncthreads();
-      if (rounds >= (1u << 16)) {
-        if (tid == 0) raise_device_error(err, RECIS_DEVERR_PLAN_OVERFLOW);
-        break;
-      }
-      rounds *= 2;
-      round = static_cast<uint32_t>(-1);  // ++ makes it 0
-      u_done = 0;
-      occ_done = 0;
-      continue;
-    }
-    const int n_ent = s_n_ent;
-    for (int k = tid; k < n_ent + kPad; k += kBucketBlock) d_min[k] = k < n_ent ? l_min[d_ent[k]] : kNoPos;
-    __syncthreads();
-    // rank by first position (positions are distinct), counts in rank order
-    for (int k = tid; k < n_ent; k += kBucketBlock) {
-      const int32_t m = d_min[k];
-      int rnk = 0;
-      for (int q = 0; q < n_ent; q += kPad) {
-        const int4 a0 = *reinterpret_cast<const int4*>(&d_min[q]);
-        const int4 a1 = *reinterpret_cast<const int4*>(&d_min[q + 4]);
-        const int4 a2 = *reinterpret_cast<const int4*>(&d_min[q + 8]);
-        const int4 a3 = *reinterpret_cast<const int4*>(&d_min[q + 12]);
-        rnk += (a0.x < m) + (a0.y < m) + (a0.z < m) + (a0.w < m) + (a1.x < m) + (a1.y < m) + (a1.z < m) + (a1.w < m) +
-               (a2.x < m) + (a2.y < m) + (a2.z < m) + (a2.w < m) + (a3.x < m) + (a3.y < m) + (a3.z < m) + (a3.w < m);
-      }
-      const int e = d_ent[k];
-      l_rank[e] = static_cast<uint16_t>(rnk);
-      s_cnt[rnk] = l_cnt[e];
-    }
-    __syncthreads();
-    // exclusive scan of s_cnt[0 .. n_ent) in place (n_ent <= 1025): 5 consecutive entries per thread
-    {
-      constexpr int kPer = (kBucketSlots + 1 + kBucketBlock - 1) / kBucketBlock;
-      int32_t v[kPer];
-      int32_t sum = 0;
+    unsigned long long total;
+    unsigned long long run = block_scan_u64(mine, s_wave, total);
+    const int32_t n_ent = static_cast<int32_t>(total & 0xffffffffull);
+    const int32_t n_occ = static_cast<int32_t>(total >> 32);
+    // the later buckets can go on as soon as they know how many unique ids this one has
+    if (rounds == 1 && tid == 0)
+      __hip_atomic_store(&a.agg[b], kAggFlag | static_cast<unsigned long long>(n_ent), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-      for (int x = 0; x < kPer; ++x) {
-        const int k = tid * kPer + x;
-        v[x] = k < n_ent ? s_cnt[k] : 0;
-        sum += v[x];
-      }
-      const int lane = tid & (kWave - 1), wave = tid / kWave;
-      int32_t incl = sum;
-      for (int o = 1; o < kWave; o <<= 1) {
-        const int32_t y = __shfl_up(incl, o, kWave);
-        if (lane >= o) incl += y;
-      }
-      if (lane == kWave - 1) wave_counts[wave] = incl;
-      __syncthreads();
-      int32_t run = incl - sum;
-      int32_t tot = 0;
+    for (int x = 0; x < kPer; ++x) {
+      if (cnt[x] < 0) continue;
+      l_u[s_lo + x] = static_cast<int32_t>(run & 0xffffffffull);
+      l_cnt[s_lo + x] = static_cast<int32_t>(run >> 32);  // only its owner has read the count
+      run += (static_cast<unsigned long long>(cnt[x]) << 32) | 1ull;
+    }
+
+    // ---- where this bucket's unique ids start
+    if (rounds == 1) {
+      u_base = look_back(a.agg, b, a.spin_limit, a.err, s_wave);
+      if (tid == 0)
+        __hip_atomic_store(&a.agg[b], kPrefixFlag | static_cast<unsigned long long>(u_base + n_ent), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---- per unique id: the id, the start of its list, hot work items, its row in the id map
+    int32_t my_new = 0, my_empty = 0;
 #pragma unroll
-      for (int w = 0; w < kBucketBlock / kWave; ++w) {
-        if (w < wave) run += wave_counts[w];
-        tot += wave_counts[w];
-      }
-      if (tid == 0) s_total = tot;
+    for (int x0 = 0; x0 < kPer; x0 += 3) {  // three probes of the id map in flight
+      int64_t key[3];
+      uint64_t home[3];
+      longlong2 hint[3];
 #pragma unroll
-      for (int x = 0; x < kPer; ++x) {
-        const int k = tid * kPer + x;
-        if (k < n_ent) s_cnt[k] = run;
-        run += v[x];
+      for (int y = 0; y < 3; ++y) {
+        const int x = x0 + y, e = s_lo + x;
+        key[y] = cnt[x] >= 0 ? (e == kSpecial ? kSetEmpty : l_key[e]) : kSetEmpty;
+        if constexpr (PROBE) {
+          home[y] = 0;
+          hint[y] = make_longlong2(0, 0);
+          if (cnt[x] >= 0 && key[y] != kEmpty && key[y] != kTomb) {
+            home[y] = home_slot(key[y], a.mask);
+            hint[y] = *reinterpret_cast<const longlong2*>(&a.table[home[y]]);
+          }
+        }
       }
-    }
-    __syncthreads();
-    for (int k = tid; k < n_ent; k += kBucketBlock) {
-      const int e = d_ent[k];
-      const int rnk = l_rank[e];
-      URec u;
-      u.key = e == kBucketSlots ? kSetEmpty : l_key[e];
-      u.list_off = occ_done + s_cnt[rnk];
-      u.cnt = l_cnt[e];
-      bucket_uniq[r_lo + u_done + rnk] = u;
-    }
-    // B: every record learns its unique id (bucket-local) and the list offset of its run
 #pragma unroll
-    for (int x = 0; x < kBucketRegs; ++x) {
-      if (e_reg[x] == -2) continue;
-      int2 out = make_int2(0, 0);  // overflow (flagged): keep the indices in range
-      if (e_reg[x] >= 0) {
-        const int rnk = l_rank[e_reg[x]];
-        out = make_int2(u_done + rnk, occ_done + s_cnt[rnk] + base_reg[x]);
+      for (int y = 0; y < 3; ++y) {
+        const int x = x0 + y, e = s_lo + x;
+        if (cnt[x] < 0) continue;
+        const int64_t u = u_base + u_done + l_u[e];
+        if (u < 0 || u >= a.g.n) {
+          raise_device_error(a.err, RECIS_DEVERR_PLAN_OVERFLOW);  // cannot happen; never store out of bounds
+          continue;
+        }
+        a.unique_out[u] = key[y];
+        a.row_start[u] = l_base + l_done + l_cnt[e];
+        if (a.hot_cap > 0 && cnt[x] > kHotLen) {
+          const int n_items = (cnt[x] + kHotChunk - 1) / kHotChunk;
+          const int64_t base = static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&a.counts[1]),
+                                                              static_cast<unsigned long long>(n_items)));
+          for (int c = 0; c < n_items; ++c) {
+            if (base + c < a.hot_cap) {
+              a.hot_items[2 * (base + c)] = static_cast<int32_t>(u);
+              a.hot_items[2 * (base + c) + 1] = c;
+            }
+          }
+        }
+        if constexpr (PROBE) {
+          int64_t row = -1;  // what index_out gets; a claimed slot travels as -(slot + 2) until rows are assigned
+          if (key[y] == kEmpty || key[y] == kTomb) {
+            raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);  // the map's reserved keys
+          } else {
+            int64_t value = -1, slot = -1;
+            bool took_empty = false;
+            switch (probe_or_claim(a.table, a.mask, key[y], home[y], hint[y], -2, &value, &slot, &took_empty)) {
+              case kProbeFound:
+                row = value;
+                break;
+              case kProbeClaimed:
+                row = -(slot + 2);
+                ++my_new;
+                my_empty += took_empty ? 1 : 0;
+                break;
+              default:  // no slot left, or the key is being inserted by a concurrent call (not allowed)
+                raise_device_error(a.err, RECIS_DEVERR_TABLE_FULL);
+                break;
+            }
+          }
+          a.index_out[u] = row;
+        }
       }
-      result[origin_of(reg[x])] = out;
     }
-    for (int32_t q = r_lo + tid + kBucketRegs * kBucketBlock; q < r_hi; q += kBucketBlock) {
-      const Rec r = bucket_rec[q];
-      if (!in_round(r.key, rounds, round)) continue;
-      const int64_t origin = origin_of(r);
-      const int2 eb = result[origin];
-      int2 out = make_int2(0, 0);
-      if (eb.x >= 0) {
-        const int rnk = l_rank[eb.x];
-        out = make_int2(u_done + rnk, occ_done + s_cnt[rnk] + eb.y);
+    // ---- new keys: listed per bucket in the order of the unique ids, for the row assignment
+    int32_t n_new = 0;
+    if constexpr (PROBE) {
+      unsigned long long new_total;
+      const unsigned long long new_before = block_scan_u64(
+          (static_cast<unsigned long long>(my_empty) << 32) | static_cast<unsigned long long>(my_new), s_wave,
+          new_total);
+      n_new = static_cast<int32_t>(new_total & 0xffffffffull);
+      if (tid == 0 && (new_total >> 32) != 0)
+        atomicAdd(reinterpret_cast<unsigned long long*>(&a.state[ST_OCC]), new_total >> 32);
+      if (my_new > 0) {
+        int32_t at = l_base + new_done + static_cast<int32_t>(new_before & 0xffffffffull);
+#pragma unroll
+        for (int x = 0; x < kPer; ++x) {
+          if (cnt[x] < 0) continue;
+          NewRec nr;
+          nr.u = u_base + u_done + l_u[s_lo + x];
+          if (nr.u < 0 || nr.u >= a.g.n) continue;  // flagged above
+          const int64_t row = a.index_out[nr.u];    // written by this thread above
+          if (row >= -1) continue;
+          nr.slot = -(row + 2);
+          if (at >= r_hi) continue;  // cannot happen: a bucket has no more new keys than records
+          a.new_list[at++] = nr;
+        }
       }
-      result[origin] = out;
     }
-    __syncthreads();
+    __syncthreads();  // the list starts have been read; ranks and starts of all entries are in place
+
+    // ---- per occurrence: its place in the list of its id, its unique index
+    auto place = [&](int e, int32_t pos) {  // every lane of the wave calls; e < 0: nothing to place
+      const int32_t at = wave_add_one(l_cnt, e, e >= 0);
+      if (e < 0) return;
+      const int32_t lp = l_base + l_done + at;
+      if (lp < r_lo || lp >= r_hi || static_cast<uint32_t>(pos) >= static_cast<uint64_t>(a.g.n)) {
+        raise_device_error(a.err, RECIS_DEVERR_PLAN_OVERFLOW);  // cannot happen; never store out of bounds
+        return;
+      }
+      a.list[lp] = pos;
+      if (a.pos_out) a.pos_out[pos] = lp;
+      if (a.inverse) a.inverse[pos] = static_cast<int32_t>(u_base + u_done + l_u[e]);
+    };
+#pragma unroll
+    for (int x = 0; x < kRegs; ++x) place(e_reg[x], pos_reg[x]);
+    for (int32_t q0 = r_lo + kRegs * kBucketBlock; q0 < r_hi; q0 += kRegs * kBucketBlock) {
+      int64_t k[kRegs];
+      int32_t pos[kRegs];
+#pragma unroll
+      for (int x = 0; x < kRegs; ++x) {
+        const int32_t q = q0 + tid + x * kBucketBlock;
+        k[x] = q < r_hi ? a.bkt_id[q] : 0;
+        pos[x] = q < r_hi ? a.bkt_pos[q] : 0;
+      }
+#pragma unroll
+      for (int x = 0; x < kRegs; ++x) {
+        int e = -1;
+        if (q0 + tid + x * kBucketBlock < r_hi) {
+          const uint64_t mixed = mix_id(k[x]);
+          if (in_round(mixed, rounds, round)) e = find_from(k[x], home_of_mix(mixed, nb_log2));
+        }
+        place(e, pos[x]);
+      }
+    }
     u_done += n_ent;
-    occ_done += s_total;
-    __syncthreads();
+    l_done += n_occ;
+    new_done += n_new;
   }
+
   if (tid == 0) {
-    ucnt[b] = u_done;
-    ocnt[b] = occ_done;
+    if (rounds > 1)
+      __hip_atomic_store(&a.agg[b], kPrefixFlag | static_cast<unsigned long long>(u_base + u_done), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    if constexpr (PROBE) a.new_count[b] = new_done;
+    if (b == (1 << nb_log2) - 1) {  // the last bucket knows the total
+      const int64_t U = u_base + u_done;
+      a.counts[0] = U;
+      a.row_start[U] = static_cast<int32_t>(a.g.n);
+      if (a.staged) {  // pinned host words: no copy kernel needed
+        a.staged[1] = __hip_atomic_load(a.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        a.staged[0] = U;
+      }
+    }
   }
+}
+
+// Rows of the keys the fused find-or-insert added to the id map, in the order of the unique ids
+// (IdAllocator::GenIds, csrc/embedding/id_allocator.cc:17-26): every workgroup scans the per-bucket
+// counts of new keys for itself, takes a share of the buckets and gives the k-th new key of bucket
+// b the rank (new keys of earlier buckets) + k. The workgroup that finishes last (all others have
+// read the allocator words by then) does the allocator's bookkeeping and publishes it to the host.
+__global__ void __launch_bounds__(kPartBlock)
+plan_assign_new_kernel(Slot* __restrict__ table, const NewRec* __restrict__ new_list,
+                       const int32_t* __restrict__ bucket_start, const int32_t* __restrict__ new_count, int nb,
+                       int64_t* __restrict__ state, volatile int64_t* mirror, int64_t seq,
+                       const int64_t* __restrict__ free_list, int64_t* __restrict__ index_out,
+                       int32_t* __restrict__ sync) {
+  extern __shared__ int32_t first_new[];  // [nb + 1], then kPartBlock words of scan scratch
+  scan_counts(new_count, nb, first_new, first_new + nb + 1);
+  const int64_t n_new = first_new[nb];
+  const int64_t old_cur = state[ST_CUR], old_free = state[ST_FREE];
+  for (int b = blockIdx.x; b < nb && n_new > 0; b += gridDim.x) {
+    const int32_t cnt = new_count[b];
+    const NewRec* mine = new_list + bucket_start[b];
+    for (int k = threadIdx.x; k < cnt; k += kPartBlock) {
+      const NewRec r = mine[k];
+      const int64_t row = row_of_new_key(first_new[b] + k, n_new, old_cur, old_free, free_list);
+      st_relaxed(&table[r.slot].val, row);
+      index_out[r.u] = row;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0 && atomicAdd(&sync[2], 1) == static_cast<int>(gridDim.x) - 1) {
+    commit_new_keys(state, n_new);
+    publish(state, mirror, seq);
+  }
+}
+
+// inverse / pos from the lists, for plans that were made without them: list entry k belongs to the
+// unique id u with row_start[u] <= k < row_start[u + 1] (binary search; the arrays are cache
+// resident right after the plan).
+__global__ void __launch_bounds__(kBlock)
+plan_inverse_from_lists_kernel(const int32_t* __restrict__ row_start, const int32_t* __restrict__ list,
+                               const int64_t* __restrict__ counts, int64_t n, int32_t* __restrict__ inverse,
+                               int32_t* __restrict__ pos_out) {
+  const int64_t k = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (k >= n) return;
+  int64_t lo = 0, hi = counts[0];  // row_start[lo] <= k < row_start[hi]
+  while (hi - lo > 1) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (row_start[mid] <= k)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  const int32_t i = list[k];
+  if (static_cast<uint32_t>(i) >= static_cast<uint64_t>(n)) return;
+  if (inverse) inverse[i] = static_cast<int32_t>(lo);
+  if (pos_out) pos_out[i] = static_cast<int32_t>(k);
 }
 
 __global__ void plan_empty_kernel(int64_t* __restrict__ counts, int32_t* __restrict__ row_start,
@@ -497,78 +848,6 @@ __global__ void plan_empty_kernel(int64_t* __restrict__ counts, int32_t* __restr
       total_host[0] = 0;
     }
   }
-}
-
-// emit, per occurrence: inverse, list entry, position in the list
-__device__ __forceinline__ void
-emit_occ_block(int64_t vblock, const int64_t* __restrict__ ids, const uint32_t* __restrict__ occ_rec,
-               const int2* __restrict__ result, const int32_t* __restrict__ ubase,
-               const int32_t* __restrict__ lbase, const PlanGeom& g, int32_t* __restrict__ inverse,
-               int32_t* __restrict__ list, int32_t* __restrict__ pos_out) {
-  const int64_t i = vblock * kBlock + threadIdx.x;
-  if (i >= g.n) return;
-  const uint32_t w = occ_rec[i];
-  const int2 r = result[(i >> 10 << 10) | (w & 1023u)];
-  const int b = bucket_of(ids[i], g.nb_log2);
-  const int32_t pos = lbase[b] + r.y + static_cast<int32_t>(w >> 10);
-  inverse[i] = ubase[b] + r.x;
-  if (static_cast<uint32_t>(pos) < static_cast<uint64_t>(g.n)) list[pos] = static_cast<int32_t>(i);  // else: overflow flagged
-  if (pos_out) pos_out[i] = pos;
-}
-
-// emit, per unique id (workgroups 0 .. buckets-1: one bucket each): id, row_start, hot work
-// items; the remaining workgroups set row_start[U .. n] = n.
-__device__ __forceinline__ void
-emit_uniq_block(int64_t vblock, const URec* __restrict__ bucket_uniq, const int32_t* __restrict__ bucket_start,
-                const int32_t* __restrict__ ubase, const int32_t* __restrict__ lbase, const PlanGeom& g,
-                int64_t* __restrict__ unique_out, int32_t* __restrict__ row_start,
-                int64_t* __restrict__ counts, int32_t* __restrict__ hot_items, int64_t hot_cap) {
-  const int nb = 1 << g.nb_log2;
-  if (vblock >= nb) {
-    const int64_t U = ubase[nb];
-    const int64_t chunk = static_cast<int64_t>(kBlock) * 16;
-    const int64_t lo = U + (vblock - nb) * chunk;
-    const int64_t hi = min(lo + chunk, g.n + 1);
-    for (int64_t x = lo + threadIdx.x; x < hi; x += kBlock) row_start[x] = static_cast<int32_t>(g.n);
-    return;
-  }
-  const int b = static_cast<int>(vblock);
-  const int32_t u0 = ubase[b], cnt = ubase[b + 1] - u0, l0 = lbase[b];
-  const URec* src = bucket_uniq + bucket_start[b];
-  for (int k = threadIdx.x; k < cnt; k += kBlock) {
-    const URec u = src[k];
-    unique_out[u0 + k] = u.key;
-    row_start[u0 + k] = l0 + u.list_off;
-    if (hot_cap > 0 && u.cnt > kHotLen) {
-      const int n_items = (u.cnt + kHotChunk - 1) / kHotChunk;
-      const int64_t base = static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&counts[1]),
-                                                          static_cast<unsigned long long>(n_items)));
-      for (int c = 0; c < n_items; ++c) {
-        if (base + c < hot_cap) {
-          hot_items[2 * (base + c)] = u0 + k;
-          hot_items[2 * (base + c) + 1] = c;
-        }
-      }
-    }
-  }
-}
-
-// emit, one launch: the first `uniq_blocks` workgroups work per unique id (a bucket each, then
-// the row_start tail), the rest per occurrence.
-__global__ void __launch_bounds__(kBlock)
-plan_emit_kernel(int64_t uniq_blocks, const int64_t* __restrict__ ids, const uint32_t* __restrict__ occ_rec,
-                 const int2* __restrict__ result, const URec* __restrict__ bucket_uniq,
-                 const int32_t* __restrict__ bucket_start, const int32_t* __restrict__ ubase,
-                 const int32_t* __restrict__ lbase, PlanGeom g, int64_t* __restrict__ unique_out,
-                 int32_t* __restrict__ inverse, int32_t* __restrict__ row_start, int32_t* __restrict__ list,
-                 int32_t* __restrict__ pos_out, int64_t* __restrict__ counts, int32_t* __restrict__ hot_items,
-                 int64_t hot_cap) {
-  const int64_t vb = blockIdx.x;
-  if (vb < uniq_blocks)
-    emit_uniq_block(vb, bucket_uniq, bucket_start, ubase, lbase, g, unique_out, row_start, counts, hot_items,
-                    hot_cap);
-  else
-    emit_occ_block(vb - uniq_blocks, ids, occ_rec, result, ubase, lbase, g, inverse, list, pos_out);
 }
 
 // ---------------------------------------------------------------- consumers
@@ -1110,129 +1389,152 @@ extern "C" {
 struct PlanLayout {
   PlanGeom g;
   int64_t nb;
-  size_t o_tile, o_brec, o_res, o_occ, o_hist, o_off, o_nrec, o_small, bytes;
+  size_t o_hist, o_total, o_start, o_agg, o_newc, o_sync, o_id, o_pos, o_new, bytes;
 };
 
-static PlanLayout plan_layout(int64_t n) {
+static PlanLayout plan_layout(int64_t n, bool with_lookup) {
   PlanLayout L;
   PlanGeom& g = L.g;
   g.n = n;
-  g.tiles = static_cast<int>((n + kPlanBlock - 1) / kPlanBlock);
-  g.tiles_per_wg = std::min(63, (g.tiles + kMaxRows - 1) / kMaxRows);  // 16-bit histogram counters
-  g.rows = (g.tiles + g.tiles_per_wg - 1) / g.tiles_per_wg;
-  // 512 to 1024 ids per bucket while the bucket count allows: a few hundred distinct ids for the
-  // LDS table of a bucket
+  g.rows = static_cast<int>(std::min<int64_t>((n + kTile - 1) / kTile, kMaxRows));
+  g.tile = static_cast<int>(((n + g.rows - 1) / g.rows + kPartBlock - 1) / kPartBlock * kPartBlock);
+  g.rows = static_cast<int>((n + g.tile - 1) / g.tile);
   int nb_log2 = 5;
-  while ((int64_t(1) << (nb_log2 + 1)) <= kMaxBuckets && (int64_t(1) << (nb_log2 + 1)) * 512 <= n) ++nb_log2;
+  while ((int64_t(1) << nb_log2) < kMaxBuckets && (int64_t(1) << nb_log2) * kBucketIds < n) ++nb_log2;
   g.nb_log2 = nb_log2;
   L.nb = int64_t(1) << nb_log2;
-  const int64_t n_pad = static_cast<int64_t>(g.tiles) * kPlanBlock;
-  // tile_rec[n_pad] (later: the unique ids of every bucket) | bucket_rec[n_pad] | result[n_pad] |
-  // occ_rec[n] | hist[rows*nb] u16 | off[rows*nb] | tile_nrec[tiles] | 6 arrays of nb + 1
+  // hist[rows * nb] (counts, then offsets, in place) | bucket_total[nb] | bucket_start[nb + 1] |
+  // agg[nb] look-back words | new_count[nb] | sync[4] | bkt_id[n] | bkt_pos[n] | new_list[n] (fused lookup only)
   size_t bytes = 0;
   auto take = [&](size_t b) {
     const size_t at = bytes;
     bytes += (b + 255) & ~size_t(255);
     return at;
   };
-  L.o_tile = take(sizeof(Rec) * n_pad);
-  L.o_brec = take(sizeof(Rec) * n_pad);
-  L.o_res = take(sizeof(int2) * n_pad);
-  L.o_occ = take(sizeof(uint32_t) * n_pad);
-  L.o_hist = take(sizeof(uint16_t) * g.rows * L.nb);
-  L.o_off = take(sizeof(int32_t) * g.rows * L.nb);
-  L.o_nrec = take(sizeof(int32_t) * g.tiles);
-  L.o_small = take(sizeof(int32_t) * 6 * (L.nb + 1));
+  L.o_hist = take(sizeof(int32_t) * g.rows * L.nb);
+  L.o_total = take(sizeof(int32_t) * L.nb);
+  L.o_start = take(sizeof(int32_t) * (L.nb + 1));
+  L.o_agg = take(sizeof(unsigned long long) * L.nb);
+  L.o_newc = take(sizeof(int32_t) * L.nb);
+  L.o_sync = take(sizeof(int32_t) * 4);
+  L.o_id = take(sizeof(int64_t) * n);
+  L.o_pos = take(sizeof(int32_t) * n);
+  L.o_new = with_lookup ? take(sizeof(NewRec) * n) : bytes;
   L.bytes = bytes;
   return L;
 }
 
-static int plan_check_args(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
-                           int32_t* row_start_out, int32_t* list_out, int32_t* hot_items_out, int64_t hot_cap,
-                           int64_t* counts_out_dev) {
+static int plan_check_args(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* row_start_out,
+                           int32_t* list_out, int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev) {
   RECIS_REQUIRE(n >= 0 && n < (int64_t(1) << 30), "n out of range: %lld", (long long)n);
   RECIS_REQUIRE(counts_out_dev && row_start_out, "counts_out_dev / row_start_out must not be NULL");
   RECIS_REQUIRE(hot_cap == 0 || (hot_items_out && hot_cap >= n / kHotLen + n / kHotChunk + 2),
                 "hot_items_out must hold at least n/%d + n/%d + 2 items", kHotLen, kHotChunk);
-  RECIS_REQUIRE(n == 0 || (ids && unique_out && inverse_out && list_out), "NULL argument");
+  RECIS_REQUIRE(n == 0 || (ids && unique_out && list_out), "NULL argument");
   return RECIS_OK;
 }
 
+// Polls of one look-back word before a workgroup gives up (a word is due within microseconds; the
+// limit only bounds a wait that can never end, e.g. after a failed launch of an earlier kernel).
+static uint32_t g_spin_limit = 1u << 22;
+
 // The plan's launches for n > 0 over the scratch buffer `base` (L.bytes bytes). `staged`: pinned host
-// word that receives the unique count as soon as it is final, or NULL.
+// words that receive the unique count (and the soft-error bits) as soon as they are final, or NULL.
+// With a map, every unique id is looked up (find or insert) from inside the bucket kernel and
+// index_out receives its row.
 static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int64_t* unique_out,
                        int32_t* inverse_out, int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
                        int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev, int64_t* staged,
-                       hipEvent_t staged_event, int* err, hipStream_t stream) {
+                       hipEvent_t staged_event, int* err, recis_idmap* map, int64_t map_seq, int64_t* index_out,
+                       hipStream_t stream) {
   const PlanGeom& g = L.g;
-  const int64_t nb = L.nb, n = g.n;
-  Rec* tile_rec = reinterpret_cast<Rec*>(base + L.o_tile);
-  Rec* bucket_rec = reinterpret_cast<Rec*>(base + L.o_brec);
-  int2* result = reinterpret_cast<int2*>(base + L.o_res);
-  uint32_t* occ_rec = reinterpret_cast<uint32_t*>(base + L.o_occ);
-  uint16_t* hist = reinterpret_cast<uint16_t*>(base + L.o_hist);
-  int32_t* off = reinterpret_cast<int32_t*>(base + L.o_off);
-  int32_t* tile_nrec = reinterpret_cast<int32_t*>(base + L.o_nrec);
-  int32_t* bucket_total = reinterpret_cast<int32_t*>(base + L.o_small);
-  int32_t* bucket_start = bucket_total + (nb + 1);
-  int32_t* ucnt = bucket_start + (nb + 1);
-  int32_t* ocnt = ucnt + (nb + 1);
-  int32_t* ubase = ocnt + (nb + 1);
-  int32_t* lbase = ubase + (nb + 1);
-  URec* bucket_uniq = reinterpret_cast<URec*>(tile_rec);  // the tile records are dead after the scatter
-
+  const int64_t nb = L.nb;
+  int32_t* hist = reinterpret_cast<int32_t*>(base + L.o_hist);
+  int32_t* bucket_total = reinterpret_cast<int32_t*>(base + L.o_total);
+  int32_t* bucket_start = reinterpret_cast<int32_t*>(base + L.o_start);
+  unsigned long long* agg = reinterpret_cast<unsigned long long*>(base + L.o_agg);
+  int32_t* sync = reinterpret_cast<int32_t*>(base + L.o_sync);
+  int64_t* bkt_id = reinterpret_cast<int64_t*>(base + L.o_id);
+  int32_t* bkt_pos = reinterpret_cast<int32_t*>(base + L.o_pos);
+  const size_t lds = sizeof(int32_t) * static_cast<size_t>(nb);
   {
-    RECIS_TIME_KERNEL("plan_tile_kernel", stream)
-    plan_tile_kernel<<<dim3(g.rows), dim3(kPlanBlock), 0, stream>>>(ids, g, tile_rec, tile_nrec, occ_rec, hist,
-                                                                   counts_out_dev);
+    RECIS_TIME_KERNEL("plan_hist_kernel", stream)
+    plan_hist_kernel<<<dim3(g.rows), dim3(kPartBlock), lds, stream>>>(ids, g, hist, counts_out_dev, sync);
     RECIS_LAUNCH_CHECK();
   }
   {
     RECIS_TIME_KERNEL("plan_colscan_kernel", stream)
-    plan_colscan_kernel<<<dim3(nb / 32), dim3(1024), 0, stream>>>(hist, g, off, bucket_total);
+    plan_colscan_kernel<<<dim3(nb / kColBuckets), dim3(1024), 0, stream>>>(hist, g, bucket_total);
     RECIS_LAUNCH_CHECK();
   }
-  plan_scan_kernel<<<1, 1024, 0, stream>>>(bucket_total, bucket_start, nullptr, nullptr, static_cast<int>(nb),
-                                           nullptr, nullptr, nullptr);
-  RECIS_LAUNCH_CHECK();
   {
     RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
-    plan_scatter_kernel<<<dim3(g.rows), dim3(kPlanBlock), 0, stream>>>(tile_rec, tile_nrec, g, off, bucket_start,
-                                                                      bucket_rec);
+    if (g.tile <= kTile && g.tile >= 4 * nb)  // a tile sends four ids or more to a bucket: worth ordering them
+      plan_scatter_runs_kernel<<<dim3(g.rows), dim3(kPartBlock),
+                                 sizeof(int32_t) * (2 * (nb + 1) + kPartBlock) + 2 * sizeof(uint16_t) * kTile, stream>>>(
+          ids, g, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
+    else
+      plan_scatter_kernel<<<dim3(g.rows), dim3(kPartBlock), lds + sizeof(int32_t) * (kPartBlock + 1), stream>>>(
+          ids, g, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
     RECIS_LAUNCH_CHECK();
   }
-  {
+  BucketArgs a;
+  a.bkt_id = bkt_id;
+  a.bkt_pos = bkt_pos;
+  a.bucket_start = bucket_start;
+  a.g = g;
+  a.agg = agg;
+  a.new_count = reinterpret_cast<int32_t*>(base + L.o_newc);
+  a.sync = sync;
+  a.unique_out = unique_out;
+  a.inverse = inverse_out;
+  a.row_start = row_start_out;
+  a.list = list_out;
+  a.pos_out = pos_out;
+  a.counts = counts_out_dev;
+  a.hot_items = hot_items_out;
+  a.hot_cap = hot_cap;
+  a.staged = staged;
+  a.err = err;
+  a.spin_limit = g_spin_limit;
+  a.table = nullptr;
+  a.mask = 0;
+  a.index_out = index_out;
+  a.state = nullptr;
+  a.mirror = nullptr;
+  a.seq = map_seq;
+  a.new_list = reinterpret_cast<NewRec*>(base + L.o_new);
+  if (map) {
+    a.table = map->table;
+    a.mask = static_cast<uint64_t>(map->capacity - 1);
+    a.state = map->state;
+    a.mirror = map->mirror;
+    {
+      RECIS_TIME_KERNEL("plan_bucket_kernel", stream)
+      plan_bucket_kernel<true><<<dim3(nb), dim3(kBucketBlock), 0, stream>>>(a);
+      RECIS_LAUNCH_CHECK();
+    }
+    plan_assign_new_kernel<<<dim3(std::max<int64_t>(nb / 4, 1)), dim3(kPartBlock),
+                             lds + sizeof(int32_t) * (kPartBlock + 1), stream>>>(
+        map->table, a.new_list, bucket_start, a.new_count, static_cast<int>(nb), map->state, map->mirror, map_seq,
+        map->free_list, index_out, sync);
+    RECIS_LAUNCH_CHECK();
+  } else {
     RECIS_TIME_KERNEL("plan_bucket_kernel", stream)
-    plan_bucket_kernel<<<dim3(nb), dim3(kBucketBlock), 0, stream>>>(bucket_rec, bucket_start, g, result, bucket_uniq,
-                                                                   ucnt, ocnt, err);
+    plan_bucket_kernel<false><<<dim3(nb), dim3(kBucketBlock), 0, stream>>>(a);
     RECIS_LAUNCH_CHECK();
   }
-  // The count is final after this scan: the kernel stores it into pinned host memory as well (with
-  // the soft-error bits raised so far), and the host waits for it only after the emit kernels are
-  // queued, so that the GPU works while the host learns the size of the next launches.
-  plan_scan_kernel<<<1, 1024, 0, stream>>>(ucnt, ubase, ocnt, lbase, static_cast<int>(nb), counts_out_dev, staged,
-                                           err);
-  RECIS_LAUNCH_CHECK();
   if (staged) RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
-  {
-    const int64_t tail_blocks = (n + 1 + kBlock * 16 - 1) / (kBlock * 16);
-    const int64_t uniq_blocks = nb + tail_blocks, occ_blocks = (n + kBlock - 1) / kBlock;
-    RECIS_TIME_KERNEL("plan_emit_kernel", stream)
-    plan_emit_kernel<<<dim3(uniq_blocks + occ_blocks), dim3(kBlock), 0, stream>>>(
-        uniq_blocks, ids, occ_rec, result, bucket_uniq, bucket_start, ubase, lbase, g, unique_out, inverse_out,
-        row_start_out, list_out, pos_out, counts_out_dev, hot_items_out, hot_cap);
-    RECIS_LAUNCH_CHECK();
-  }
   return RECIS_OK;
 }
 
-int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
+static int plan_entry(recis_idmap* map, const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
                       int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
-                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* unique_count_host, int flags, void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  if (int rc = plan_check_args(ids, n, unique_out, inverse_out, row_start_out, list_out, hot_items_out, hot_cap,
-                               counts_out_dev))
+                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* index_out, int64_t* unique_count_host,
+                      int flags, hipStream_t stream) {
+  if (int rc = plan_check_args(ids, n, unique_out, row_start_out, list_out, hot_items_out, hot_cap, counts_out_dev))
     return rc;
+  RECIS_REQUIRE(map == nullptr || n == 0 || index_out != nullptr, "index_out must not be NULL");
   int* err = device_error_word(current_device());
   RECIS_REQUIRE(err != nullptr, "could not reach the device error word");
   const bool stage = unique_count_host || (flags & RECIS_PLAN_STAGE_COUNT);
@@ -1248,16 +1550,56 @@ int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_
     if (unique_count_host) *unique_count_host = 0;
     return RECIS_OK;
   }
-  const PlanLayout L = plan_layout(n);
+  int64_t seq = 0;
+  if (map) {
+    if (int rc = idmap_begin_call(map, n, stream, &seq)) return rc;
+  }
+  const PlanLayout L = plan_layout(n, map != nullptr);
   void* ws = nullptr;
   if (int rc = get_workspace(stream, L.bytes, &ws)) return rc;
   if (int rc = plan_launch(L, static_cast<char*>(ws), ids, unique_out, inverse_out, row_start_out, list_out, pos_out,
-                           hot_items_out, hot_cap, counts_out_dev, staged, staged_event, err, stream))
+                           hot_items_out, hot_cap, counts_out_dev, staged, staged_event, err, map, seq, index_out,
+                           stream))
     return rc;
+  if (map) idmap_end_call(map, seq, n);
   if (unique_count_host) {
     RECIS_CHECK_HIP(hipEventSynchronize(staged_event));
     *unique_count_host = staged[0];
   }
+  return RECIS_OK;
+}
+
+int recis_unique_plan(const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
+                      int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
+                      int64_t hot_cap, int64_t* counts_out_dev, int64_t* unique_count_host, int flags, void* stream_) {
+  return plan_entry(nullptr, ids, n, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
+                    counts_out_dev, nullptr, unique_count_host, flags, static_cast<hipStream_t>(stream_));
+}
+
+int recis_unique_plan_lookup(recis_idmap* map, const int64_t* ids, int64_t n, int64_t* unique_out,
+                             int32_t* inverse_out, int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
+                             int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev, int64_t* index_out,
+                             int64_t* unique_count_host, int flags, void* stream_) {
+  RECIS_REQUIRE(map != nullptr, "id map is NULL");
+  return plan_entry(map, ids, n, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
+                    counts_out_dev, index_out, unique_count_host, flags, static_cast<hipStream_t>(stream_));
+}
+
+int recis_plan_inverse_from_lists(const int32_t* row_start, const int32_t* list, const int64_t* counts_dev, int64_t n,
+                                  int32_t* inverse_out, int32_t* pos_out, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n >= 0, "negative size");
+  if (n == 0 || (!inverse_out && !pos_out)) return RECIS_OK;
+  RECIS_REQUIRE(row_start && list && counts_dev, "NULL argument");
+  plan_inverse_from_lists_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(
+      row_start, list, counts_dev, n, inverse_out, pos_out);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
+int recis_plan_set_spin_limit(int64_t polls) {
+  RECIS_REQUIRE(polls >= 1 && polls <= (int64_t(1) << 31) - 1, "polls out of range");
+  g_spin_limit = static_cast<uint32_t>(polls);
   return RECIS_OK;
 }
 
@@ -1274,8 +1616,7 @@ int recis_unique_plan_noalloc(const int64_t* ids, int64_t n, int64_t* unique_out
                               int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
                               int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  if (int rc = plan_check_args(ids, n, unique_out, inverse_out, row_start_out, list_out, hot_items_out, hot_cap,
-                               counts_out_dev))
+  if (int rc = plan_check_args(ids, n, unique_out, row_start_out, list_out, hot_items_out, hot_cap, counts_out_dev))
     return rc;
   const int dev = current_device();
   RECIS_REQUIRE(dev >= 0 && dev < kMaxScratchDevices, "device %d out of range", dev);
@@ -1298,16 +1639,17 @@ int recis_unique_plan_noalloc(const int64_t* ids, int64_t n, int64_t* unique_out
   }
   RECIS_REQUIRE(n <= RECIS_PLAN_NOALLOC_MAX_IDS, "recis_unique_plan_noalloc takes at most %lld ids per call (got %lld); "
                 "use recis_unique_plan for more", (long long)RECIS_PLAN_NOALLOC_MAX_IDS, (long long)n);
-  const PlanLayout L = plan_layout(n);
+  const PlanLayout L = plan_layout(n, false);
   if (L.bytes > kStaticScratchBytes)
     return fail(RECIS_ERR_CAPACITY,
                 "recis_unique_plan_noalloc: %lld ids need %zu bytes of scratch, the built-in buffer holds %zu "
                 "(at most %lld ids per call; use recis_unique_plan for more)",
                 (long long)n, L.bytes, kStaticScratchBytes, (long long)RECIS_PLAN_NOALLOC_MAX_IDS);
-  // every scratch array is fully written by the kernel that produces it before any kernel reads it:
-  // nothing of the previous call's contents is relied on, nothing needs clearing
+  // What must start at zero (the two counters in `sync`, the look-back words) is cleared by the
+  // plan's own first two kernels; every other scratch array is fully written by the kernel that
+  // produces it before any kernel reads it: nothing of the previous call's contents is relied on.
   return plan_launch(L, base, ids, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
-                     counts_out_dev, nullptr, nullptr, err, stream);
+                     counts_out_dev, nullptr, nullptr, err, nullptr, 0, nullptr, stream);
 }
 
 int recis_unique_plan_count(int64_t* unique_count_host, void* stream_) {

@@ -139,13 +139,16 @@ class LookupPoolFunction(torch.autograd.Function):
             # Nothing in this forward waits for the unique count: the lookup and the expansion take
             # it from device memory, the pooling kernel only follows the plan's inverse (which names
             # rows below the count), and the host reads it in backward, long after it has arrived.
-            # `index` is the full-length buffer; its first plan.U entries are the rows.
-            index = impl.lookup_index_unsettled(plan)
+            # `index` is the full-length buffer; its first plan.U entries are the rows. A plan made by
+            # make_plan for this table brings them along (dedup and lookup were one pass).
+            index = impl.plan_index(plan)
+            if index is None:
+                index = impl.lookup_index_unsettled(plan)
         chunks, chunk_rows = impl.emb_blocks()
         if unit_segments:
             # one id per segment (sum == mean == the row itself): every unique row is read once and
             # written to its occurrences, instead of one index chase per output row
-            out = ops.plan_expand_rows(plan, plan.inverse.numel(), blocks=chunks, block_size=chunk_rows,
+            out = ops.plan_expand_rows(plan, plan.n, blocks=chunks, block_size=chunk_rows,
                                        row_index=index, weight=weight)
         else:
             out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets,
@@ -169,17 +172,35 @@ class LookupPoolFunction(torch.autograd.Function):
         return None, None, None, None, None, None, None, None
 
 
+def _pools_out_of_the_table(hashtable, opt, n_occ, n_offsets):
+    """Whether lookup_and_pool takes the path that pools straight out of the table rows."""
+    float_table = hashtable._dtype in (torch.float32, torch.bfloat16, torch.float16)
+    sparse_mean = opt.combiner == "mean" and not n_occ / n_offsets > 5
+    id_mean = opt.grad_reduce_by == "id" and hashtable.training and opt.trainable
+    return opt.combiner in ("sum", "mean") and float_table and not sparse_mean and not id_mean
+
+
+def make_plan(hashtable: HashTable, ids, offsets, opt, has_weight=False, unit_segments=False):
+    """The batch plan of ``ids`` for ``lookup_and_pool``. When what follows is the training lookup
+    that admits new keys and pools out of the table, dedup and find-or-insert run as one pass
+    (``HashtableImpl.plan_lookup``) and the plan carries the rows; ``unit_segments`` plans leave
+    out the per-occurrence arrays nobody reads (the expansion and its backward walk the lists)."""
+    if (hashtable.training and opt.trainable and opt.admit_hook is None
+            and _pools_out_of_the_table(hashtable, opt, ids.numel(), offsets.numel())):
+        lean = bool(unit_segments)
+        return hashtable._hashtable_impl.plan_lookup(ids, need_inverse=not lean,
+                                                     need_pos=not (lean and not has_weight))
+    return ops.ids_unique_plan(ids, wait=False)
+
+
 def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False, combiner_kwargs=None):
     """Rows of the plan's unique ids pooled per segment. Sum / mean over a float table go
     through ``LookupPoolFunction`` (pooling reads the table directly); everything else looks the
     rows up first and pools the copy. ``unit_segments``: the caller built ``offsets`` as
     0, 1, 2, ... (dense ``[B, 1]`` id tensors), so segment i holds exactly occurrence i."""
     impl = hashtable._hashtable_impl
-    float_table = hashtable._dtype in (torch.float32, torch.bfloat16, torch.float16)
-    n_occ = plan.inverse.numel()
-    sparse_mean = opt.combiner == "mean" and not n_occ / offsets.numel() > 5
     id_mean = opt.grad_reduce_by == "id" and hashtable.training and opt.trainable
-    if opt.combiner in ("sum", "mean") and float_table and not sparse_mean and not id_mean:
+    if _pools_out_of_the_table(hashtable, opt, plan.n, offsets.numel()):
         if weight is not None and weight.dtype != hashtable._dtype:
             weight = weight.to(hashtable._dtype)
         if hashtable.training and opt.trainable:
@@ -262,7 +283,7 @@ class DynamicEmbedding(torch.nn.Module):
             weight = input_weights
         if weight is not None:
             weight = weight.to(dev) if opt.use_weight else None
-        plan = ops.ids_unique_plan(val, wait=False)
+        plan = make_plan(self._hashtable, val, offsets, opt, weight is not None, self._unit_segments)
         out = lookup_and_pool(self._hashtable, plan, weight, offsets, opt, unit_segments=self._unit_segments)
         if opt.combiner == "tile":
             return out.view(tuple(shape) + (opt.combiner_kwargs["tile_len"] * opt.embedding_dim,))

@@ -22,7 +22,7 @@ import torch
 from ... import ops
 from ...ragged.tensor import RaggedTensor
 from ..functional.embedding_ops import RaggedTileParts
-from .embedding import EmbeddingOption, lookup_and_pool, lookup_unique_rows
+from .embedding import EmbeddingOption, lookup_and_pool, lookup_unique_rows, make_plan
 from .hashtable import HashTable, gen_slice
 
 
@@ -171,7 +171,11 @@ class EmbeddingEngine(torch.nn.Module):
                             offs, [v.numel() for v in vals]))
                     else:
                         offsets = ops.merge_offsets(offs, [v.numel() for v in vals])
-                    plan = ops.ids_unique_plan(ids, wait=False)
+                    if opt0.combiner == "tile":
+                        plan = ops.ids_unique_plan(ids, wait=False)
+                    else:  # lean (no per-occurrence arrays) only if no other option can come to share it
+                        alone = sum(1 for k in runtime.values() if any(inputs[n] is inputs[names[0]] for n in k)) == 1
+                        plan = make_plan(table, ids, offsets, opt0, any_weight, unit_segments=all_unit and alone)
                     plans[same] = (offsets, plan)
                 weight = None
                 if all(w is not None for w in weights):

@@ -395,6 +395,22 @@ class HashtableImpl:
         plan.lookup_calls[id(self)] = self._idmap.last_call()
         return index_buf
 
+    def plan_lookup(self, ids, wait=False, need_inverse=True, need_pos=True):
+        """Dedup of ``ids`` and find-or-insert of the distinct ids in this table in one pass
+        (``recis_unique_plan_lookup``): the batch plan with ``index_buf`` = the row of every unique
+        id. Replaces ``ids_partition`` / ``torch.unique`` + ``IdMap::Lookup`` of the training
+        lookup (recis/nn/modules/hashtable.py:262-293). Room is made for the rows every id of the
+        batch could need; settle with ``settle_count(plan.U, plan)`` once the count has been read."""
+        plan = ops.ids_unique_plan(ids, wait=wait, need_inverse=need_inverse, need_pos=need_pos, idmap=self._idmap)
+        plan.lookup_calls[id(self)] = self._idmap.last_call()
+        self._make_room(plan.n if wait is False else plan.U)
+        return plan
+
+    def plan_index(self, plan):
+        """The rows of ``plan``'s unique ids if the plan was made by ``plan_lookup`` of THIS table
+        (the full-length buffer: its first ``plan.U`` entries count), else None."""
+        return plan.index_buf if id(self) in plan.lookup_calls and plan.index_buf is not None else None
+
     def lookup_index_unsettled(self, plan):
         """``lookup_index_counted`` for consumers that take the unique count from device memory: the
         rows every one of the plan's ids could need are made room for, nothing waits for the count.
@@ -679,7 +695,7 @@ class LookupExpandFunction(torch.autograd.Function):
             index_buf = impl.lookup_index_counted(plan)   # queued before the host has the unique count
             index = impl.settle_lookup(index_buf, plan.U, plan)
         chunks, chunk_rows = impl.emb_blocks()
-        out = ops.plan_expand_rows(plan, plan.inverse.numel(), blocks=chunks, block_size=chunk_rows, row_index=index)
+        out = ops.plan_expand_rows(plan, plan.n, blocks=chunks, block_size=chunk_rows, row_index=index)
         ctx.impl, ctx.plan, ctx.slice_num, ctx.readonly = impl, plan, slice_num, readonly
         ctx.save_for_backward(index)
         ctx.mark_non_differentiable(index)
@@ -688,7 +704,7 @@ class LookupExpandFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, _grad_index, grad):
         (index,) = ctx.saved_tensors
-        n = ctx.plan.inverse.numel()
+        n = ctx.plan.n
         flat = grad.reshape(n, -1).contiguous()
         if ctx.slice_num != 1:
             flat = flat / ctx.slice_num

@@ -747,11 +747,14 @@ class BatchPlan:
     in ``occ``. ``U`` is the host copy of the unique count. A plan made with ``wait=False``
     fetches it on first use of ``U`` / ``unique`` (the count is on its way by then);
     ``unique_buf`` [N] and ``counts`` (device) are there at once, for work that can be
-    queued before the host knows ``U`` (``IdMap.lookup_counted``).
+    queued before the host knows ``U`` (``IdMap.lookup_counted``). ``inverse`` and ``pos`` are
+    filled by the plan when asked for (``need_inverse`` / ``need_pos``) and otherwise on first
+    use, from the lists. A plan made with an id map also carries ``index_buf`` [N]: the row of
+    every unique id (found or inserted), its first ``U`` entries valid.
     """
 
-    __slots__ = ("n", "_U", "_unique", "unique_buf", "inverse", "row_start", "occ", "pos", "hot_items", "hot_cap",
-                 "counts", "_pool_fill", "_stream", "serial", "lookup_calls")
+    __slots__ = ("n", "_U", "_unique", "unique_buf", "_inverse", "row_start", "occ", "_pos", "hot_items", "hot_cap",
+                 "counts", "_pool_fill", "_stream", "serial", "lookup_calls", "index_buf")
 
     @property
     def U(self):
@@ -776,6 +779,29 @@ class BatchPlan:
         if self._unique is None:
             self._unique = self.unique_buf[: self.U]
         return self._unique
+
+    def _fill_late(self):
+        inv = torch.empty(self.n, dtype=torch.int32, device=self.occ.device) if self._inverse is None else None
+        pos = torch.empty(self.n, dtype=torch.int32, device=self.occ.device) if self._pos is None else None
+        if self.n:
+            check(lib().recis_plan_inverse_from_lists(ptr(self.row_start), ptr(self.occ), ptr(self.counts), i64(self.n),
+                                                      ptr(inv), ptr(pos), self._stream))
+        if inv is not None:
+            self._inverse = inv
+        if pos is not None:
+            self._pos = pos
+
+    @property
+    def inverse(self):
+        if self._inverse is None:
+            self._fill_late()
+        return self._inverse
+
+    @property
+    def pos(self):
+        if self._pos is None:
+            self._fill_late()
+        return self._pos
 
     def src_coef_for_pool(self, offsets, weight, mean):
         """(src, coef) per list entry for the backward of pooled segments, cached per
@@ -819,10 +845,14 @@ def _raise_staged_device_errors(stream):
         _lib.raise_device_errors(bits.value)   # waits for the device and clears the word
 
 
-def ids_unique_plan(ids, wait=True):
+def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None):
     """Dedup + transposed index of a batch of ids (``recis_unique_plan``). ``wait=False``
     returns without the host copy of the unique count (see ``BatchPlan``); at most one such
-    plan per stream may have its count outstanding."""
+    plan per stream may have its count outstanding. ``need_inverse`` / ``need_pos`` = False leave
+    those two arrays to be derived from the lists if anybody asks (callers that only walk the
+    lists save two scattered writes per id). With ``idmap`` (an ``IdMap``) the unique ids are
+    found or inserted in that map in the same pass (``recis_unique_plan_lookup``) and
+    ``plan.index_buf`` holds their rows."""
     ids = _ids64(ids)
     n = ids.numel()
     dev = ids.device
@@ -830,24 +860,32 @@ def ids_unique_plan(ids, wait=True):
     p.serial = next(_PLAN_SERIAL)  # never reused, unlike id(p)
     p.n = n
     p.unique_buf = torch.empty(n, dtype=torch.int64, device=dev)
-    p.inverse = torch.empty(n, dtype=torch.int32, device=dev)
+    p._inverse = torch.empty(n, dtype=torch.int32, device=dev) if need_inverse else None
     p.row_start = torch.empty(n + 1, dtype=torch.int32, device=dev)
     p.occ = torch.empty(n, dtype=torch.int32, device=dev)
-    p.pos = torch.empty(n, dtype=torch.int32, device=dev)
+    p._pos = torch.empty(n, dtype=torch.int32, device=dev) if need_pos else None
     p.hot_cap = n // _HOT_LEN + n // _HOT_CHUNK + 2
     p.hot_items = torch.empty(2 * p.hot_cap, dtype=torch.int32, device=dev)
     p.counts = torch.empty(2, dtype=torch.int64, device=dev)
     p._pool_fill = None
     p.lookup_calls = {}   # table -> number of the counted lookup queued for this plan
     p._unique = None
+    p.index_buf = None
     p._stream = stream_ptr(dev)
     count = ctypes.c_int64(0)
     # every launch overwrites the stream's staging word: an earlier plan whose count is still
     # outstanding there must read its own device word from now on
     _STAGED.pop(p._stream.value, None)
-    check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(p.unique_buf), ptr(p.inverse), ptr(p.row_start), ptr(p.occ),
-                                  ptr(p.pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts),
-                                  ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
+    if idmap is None:
+        check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(p.unique_buf), ptr(p._inverse), ptr(p.row_start),
+                                      ptr(p.occ), ptr(p._pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts),
+                                      ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
+    else:
+        p.index_buf = torch.empty(n, dtype=torch.int64, device=dev)
+        check(lib().recis_unique_plan_lookup(idmap._h, ptr(ids), i64(n), ptr(p.unique_buf), ptr(p._inverse),
+                                             ptr(p.row_start), ptr(p.occ), ptr(p._pos), ptr(p.hot_items),
+                                             i64(p.hot_cap), ptr(p.counts), ptr(p.index_buf),
+                                             ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
     p._U = int(count.value) if wait else None
     if not wait:
         _STAGED[p._stream.value] = p

@@ -203,7 +203,7 @@ def _check_plan(ids):
     assert p.U == len(uniq) and (n == 0 or (inv.min() >= 0 and inv.max() < p.U))
     np.testing.assert_array_equal(uniq[inv] if n else inv, ids)
     rs, occ, pos = p.row_start.cpu().numpy(), p.occ.cpu().numpy(), p.pos.cpu().numpy()
-    assert rs[0] == 0 and np.all(rs[p.U:] == n) and np.all(np.diff(rs[: p.U + 1]) >= 1 if p.U else True)
+    assert rs[0] == 0 and rs[p.U] == n and np.all(np.diff(rs[: p.U + 1]) >= 1 if p.U else True)
     np.testing.assert_array_equal(np.sort(occ), np.arange(n))
     np.testing.assert_array_equal(occ[pos], np.arange(n))
     row_of_entry = np.repeat(np.arange(p.U), np.diff(rs[: p.U + 1]))
@@ -217,7 +217,14 @@ def _check_plan(ids):
     q = ops.ids_unique_plan(_dev(ids))
     np.testing.assert_array_equal(q.unique.cpu().numpy(), uniq)
     np.testing.assert_array_equal(q.inverse.cpu().numpy(), inv)
-    np.testing.assert_array_equal(q.row_start.cpu().numpy(), rs)
+    np.testing.assert_array_equal(q.row_start.cpu().numpy()[: p.U + 1], rs[: p.U + 1])
+    # a plan made without inverse / pos derives them from its lists on first use: the same arrays
+    lean = ops.ids_unique_plan(_dev(ids), need_inverse=False, need_pos=False)
+    assert lean._inverse is None and lean._pos is None
+    np.testing.assert_array_equal(lean.unique.cpu().numpy(), uniq)
+    np.testing.assert_array_equal(lean.inverse.cpu().numpy(), inv)
+    lean_occ = lean.occ.cpu().numpy()
+    np.testing.assert_array_equal(lean_occ[lean.pos.cpu().numpy()], np.arange(n))
     assert _lib.poll_device_errors() == 0
     return p
 

@@ -39,7 +39,8 @@ def test_config4_step_properties():
     assert torch.equal(ids[26 * 65536: 27 * 65536], exp_bucket | (tag << 52))
     assert torch.equal(ids[: 65536], wl.c["sparse"][0] & ((1 << 52) - 1))
 
-    plan, inv = wl.dedup(ids)
+    plan, _ = wl.dedup(ids)          # dedup + find-or-insert in one pass; inverse derived from the lists
+    inv = plan.inverse
     uniq = plan.unique
     U = plan.U
     assert torch.equal(uniq[inv.long()], ids)                      # inverse maps every id to itself

@@ -3,6 +3,8 @@ C ABI) with the CPU oracle. Integer / index results are compared bit for bit; th
 Adam row update is compared bit for bit too, since the kernel does the same
 double-precision arithmetic as the reference's CPU functor; Adagrad within
 rtol 1e-6."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -341,3 +343,80 @@ def test_bf16_rows_fp32_grads_track_fp32_path(rng):
         oracle.block_apply_adagrad(idx, g, c_emb, c_acc, lr, eps, bs)
         ops.block_apply_adagrad(_dev(idx), _dev(g), g_emb, g_acc, lr, eps, bs)
     np.testing.assert_allclose(torch.cat(g_emb).float().cpu().numpy(), np.concatenate(c_emb), rtol=2e-2, atol=2e-2)
+
+
+def test_plan_with_lookup_matches_the_oracle_map_and_the_separate_lookup(rng):
+    """recis_unique_plan_lookup (dedup and find-or-insert in one pass) over a script of batches with
+    duplicates, new and known keys, erasures in between (free-list reuse, tombstones) and a batch
+    that outgrows the initial slot table: the rows equal, bit for bit, what the oracle's map assigns
+    when it is given the plan's unique ids in the plan's order, and what a second GPU map assigns
+    through the plan followed by the stand-alone lookup; allocator state and snapshot agree."""
+    fused, split, cpu = ops.IdMap(), ops.IdMap(), oracle.IdMap()
+    live = {}
+    sizes = [0, 1, 700, 30000, 5000, 200000, 64, 1_500_000, 90000]
+    for step, n in enumerate(sizes):
+        hot = rng.integers(0, 50, size=n)
+        cold = rng.integers(-(1 << 62), 1 << 62, size=n)
+        seen = np.array(sorted(live))[: n // 3] if live else np.zeros(0, np.int64)
+        ids = np.where(rng.random(n) < 0.3, hot, cold)
+        if len(seen):
+            ids[: len(seen)] = seen                      # keys the maps already hold
+        ids_t = _dev(ids)
+        p = ops.ids_unique_plan(ids_t, idmap=fused, wait=(step % 2 == 0))
+        q = ops.ids_unique_plan(ids_t)
+        U = p.U
+        assert U == q.U == len(np.unique(ids))
+        uniq = p.unique.cpu().numpy()
+        np.testing.assert_array_equal(uniq, q.unique.cpu().numpy())
+        np.testing.assert_array_equal(p.inverse.cpu().numpy(), q.inverse.cpu().numpy())
+        got = p.index_buf[:U].cpu().numpy()
+        np.testing.assert_array_equal(got, split.lookup(q.unique).cpu().numpy())
+        np.testing.assert_array_equal(got, cpu.lookup(uniq))
+        live.update(zip(uniq.tolist(), got.tolist()))
+        assert fused.stats()[:3] == split.stats()[:3] == (cpu.size(), cpu.id_num(), cpu.free_size())
+        if step in (3, 5):
+            keys = np.array(sorted(live))
+            victims = keys[rng.random(len(keys)) < 0.4]
+            rows = np.array([live[k] for k in victims.tolist()], np.int64)
+            for m in (fused, split):
+                m.erase(_dev(victims), _dev(rows))
+            cpu.delete(victims, rows)
+            for k in victims.tolist():
+                del live[k]
+    ids_g, idx_g = fused.snapshot()
+    assert dict(zip(ids_g.cpu().tolist(), idx_g.cpu().tolist())) == live
+    assert _lib.poll_device_errors() == 0
+
+
+def test_plan_with_lookup_flags_the_reserved_keys():
+    m = ops.IdMap()
+    ids = torch.tensor([5, -1, 7, -2, 5, -1], device="cuda")
+    p = ops.ids_unique_plan(ids, idmap=m, wait=False)
+    assert int(p.counts[0]) == 4
+    rows = dict(zip(p.unique_buf[:4].tolist(), p.index_buf[:4].tolist()))
+    assert rows[-1] == -1 and rows[-2] == -1 and sorted((rows[5], rows[7])) == [0, 1]
+    # the soft error travels to the host with the staged count: reading the count raises it
+    with pytest.raises(_lib.RecisHipError, match="index outside"):
+        p.U
+    assert _lib.poll_device_errors() == 0          # raised once, cleared
+    assert m.stats()[:2] == (2, 2)
+
+
+def test_look_back_gives_up_instead_of_hanging():
+    """A workgroup of the plan that waits for the look-back word of an earlier bucket polls a bounded
+    number of times. With the bound forced to one poll (from the host) some waits give up: the
+    kernel still ends, the error bit says so, and the next plan with the default bound is right."""
+    lib = _lib.lib()
+    ids = torch.randint(0, 1 << 40, (400000,), device="cuda")
+    try:
+        _lib.check(lib.recis_plan_set_spin_limit(ctypes.c_int64(1)))
+        for _ in range(3):
+            ops.ids_unique_plan(ids, wait=False)   # the count is not read: a reader would raise the error bit
+        torch.cuda.synchronize()
+    finally:
+        _lib.check(lib.recis_plan_set_spin_limit(ctypes.c_int64(1 << 24)))
+    bits = _lib.poll_device_errors()
+    assert bits in (0, _lib.DEVERR_PLAN_OVERFLOW)
+    p = ops.ids_unique_plan(ids)
+    assert torch.equal(torch.sort(p.unique).values, torch.unique(ids))
+    assert _lib.poll_device_errors() == 0
