@@ -217,6 +217,13 @@ class Config4:
         self.opt.step()
         self.opt.zero_grad()
 
+    def bwd_update(self, index):
+        """Backward of the pooling and the Adam step in one launch: the gradient of every unique row is
+        summed over its occurrences and applied to the row by the lanes that summed it (the [U, D]
+        gradient is not written). Bit for bit what pool_bwd + update give
+        (tests/test_gpu_features.py::test_fused_gather_reduce_update_equals_the_two_calls)."""
+        self.opt.apply_planned(self.table, self.plan, self.grad_out, self.plan.occ, None, index)
+
     def next_batch(self):
         self.c = self.batches[self._turn % len(self.batches)]
         self._turn += 1
@@ -227,8 +234,7 @@ class Config4:
         uniq, inv = self.dedup(ids)
         index = self.lookup(uniq)
         pooled = self.pool_fwd(index, inv)
-        g = self.pool_bwd(inv)
-        self.update(index, g)
+        self.bwd_update(index)
         return pooled
 
     def step_from_host(self):
@@ -281,8 +287,7 @@ class Config4:
             "feature_ops": feat,
             "dedup+lookup": N * (8 + 4) + U * 8 + U * (16 + 8),
             "pool_fwd": U * (8 + D * 4) + N * 4 + (U + 1) * 4 + S * D * 4,
-            "pool_bwd": S * D * 4 + N * 4 + (S + 1) * 4 + U * D * 4,
-            "adam": U * 8 + U * D * 4 * (1 + 6),
+            "pool_bwd+adam": S * D * 4 + N * 4 + (U + 1) * 4 + U * 8 + U * D * 4 * 6,
         }
 
     def survey_bytes(self):
@@ -300,23 +305,21 @@ class Config4:
             # (id, position) in; list out; per unique id: the id, its list start, its row; one 16-byte slot of the map
             "plan_bucket_kernel": 12 * N + 4 * N + U * (8 + 4 + 8) + 16 * U,
             "csr_expand_kernel": U * (8 + D * 4) + 4 * N + 4 * (U + 1) + S * D * 4,
-            "csr_rows_kernel": S * D * 4 + 4 * N + 4 * U + U * D * 4,
-            "adamw_rows_kernel": U * (8 + D * 4 * 7),
+            # gradient rows in, list, list starts; per unique row: its index, parameter and two moments read and written
+            "csr_rows_adam_kernel": S * D * 4 + 4 * N + 4 * U + U * (8 + D * 4 * 6),
         }
 
     def stage_times(self, iters):
         ids = self.feature_ops()
         uniq, inv = self.dedup(ids)
         index = self.lookup(uniq)
-        g = self.pool_bwd(inv)
         def dedup_lookup():
             self.lookup(self.dedup(ids)[0])
         return {
             "feature_ops": _event_ms(self.feature_ops, iters),
             "dedup+lookup": _event_ms(dedup_lookup, iters),
             "pool_fwd": _event_ms(lambda: self.pool_fwd(index, inv), iters),
-            "pool_bwd": _event_ms(lambda: self.pool_bwd(inv), iters),
-            "adam": _event_ms(lambda: self.update(index, g), iters),
+            "pool_bwd+adam": _event_ms(lambda: self.bwd_update(index), iters),
         }
 
     def cpu_baseline(self, budget_s):
@@ -432,10 +435,8 @@ class Config3:
         # one row per lookup: every unique row is read once out of the table and written to its
         # occurrences (no [U, D] copy, no second pass over it)
         out = o.plan_expand_rows(plan, self.N, blocks=chunks, block_size=chunk_rows, row_index=index)
-        g = o.segment_reduce_backward_plan(self.grad_out, None, self.span, plan, "tile")
-        self.table.accept_grad(index, g, unique=True)
-        self.opt.step()
-        self.opt.zero_grad()
+        # the per-lookup gradients reduced per key and applied to the row in the same launch
+        self.opt.apply_planned(self.table, plan, self.grad_out, plan.occ, None, index, cover=self.span)
         self.step_t += 1
         return out
 
@@ -464,8 +465,10 @@ class Config3:
 
     def algorithmic_bytes(self):
         N, U, D = self.N, self.U, self.D
+        # dedup + lookup; rows read once and expanded per lookup; per-lookup gradients in; per unique row the
+        # parameter and two moments read and written (the [U, D] gradient stays on chip); the stamp
         return N * (8 + 4) + U * 8 + U * (16 + 8) + int(0.1 * N) * 16 + U * D * 4 + N * (4 + D * 4) \
-            + N * (4 + D * 4) + U * D * 4 * 7 + U * 8
+            + N * (4 + D * 4) + U * D * 4 * 6 + U * 8
 
     def kernel_bytes(self):
         """Algorithmic HBM bytes of one launch of each heavy kernel of the step (one row per lookup,
@@ -473,8 +476,7 @@ class Config3:
         N, U, D = self.N, self.U, self.D
         return {
             "csr_expand_kernel": U * (8 + D * 4) + 4 * N + 4 * (U + 1) + N * D * 4,
-            "csr_rows_kernel": N * D * 4 + 4 * N + 4 * U + U * D * 4,
-            "adamw_rows_kernel": U * (8 + D * 4 * 7),
+            "csr_rows_adam_kernel": N * D * 4 + 4 * N + 4 * U + U * (8 + D * 4 * 6),
             "plan_bucket_kernel": 12 * N + 4 * N + U * (8 + 4 + 8) + 16 * U,
         }
 

@@ -519,6 +519,37 @@ int recis_csr_gather_reduce_parts(const void* const* part_rows, const int64_t* p
                                   int64_t D, int accumulate, void* stream);
 
 /*
+ * recis_csr_gather_reduce whose result never reaches memory: the finished sum of row u IS the
+ * gradient of table row row_index[u] (a negative index skips the row), and the lane group that
+ * holds it applies the optimizer's row update at once. Same outcome, bit for bit, as
+ * recis_csr_gather_reduce into an fp32 [U, D] buffer followed by recis_block_apply_adamw /
+ * recis_block_apply_adagrad(row_index, buffer, ...): the fp32 gradient that the second call would
+ * read is the value the first holds in registers. Saves writing and re-reading the [U, D]
+ * gradient and one launch. Replaces the pair segment_reduce_backward
+ * (csrc/ops/embedding_segment_reduce_kernel.cu:276-350) + block_apply_adamw
+ * (csrc/ops/block_apply_adamw_op.cc:114-132) for callers that apply every gradient as it is
+ * produced (no gradient accumulation over several batches, one gradient per row per step). The
+ * arguments are those of the two calls; row_dtype is the type of the table's rows, beta1_t /
+ * beta2_t advance as in recis_block_apply_adamw (also when U == 0).
+ */
+int recis_csr_gather_reduce_adamw(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                  const void* coef, int coef_dtype, const int32_t* row_start,
+                                  const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev,
+                                  int64_t U, int64_t D, const void* cover_offsets, int cover_is64,
+                                  int64_t cover_S, const int64_t* row_index, void* const* emb_blocks_dev,
+                                  void* const* exp_avg_blocks_dev, void* const* exp_avg_sq_blocks_dev,
+                                  int64_t n_blocks, int64_t block_size, int row_dtype, void* beta1_t,
+                                  void* beta2_t, int beta_is_f64, double lr, double beta1, double beta2,
+                                  double weight_decay, double eps, void* stream);
+int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                    const void* coef, int coef_dtype, const int32_t* row_start,
+                                    const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev,
+                                    int64_t U, int64_t D, const void* cover_offsets, int cover_is64,
+                                    int64_t cover_S, const int64_t* row_index, void* const* emb_blocks_dev,
+                                    void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
+                                    int row_dtype, double lr, double eps, void* stream);
+
+/*
  * The transpose of recis_csr_gather_reduce (no reference counterpart; it produces what
  * segment_reduce_forward gives for one-id segments and for the TILE mode,
  * embedding_segment_reduce_kernel.cu:23-75): out[dst[k], :] = weight[dst[k]] * row(u) for every

@@ -15,6 +15,7 @@
 #include <type_traits>
 
 #include "common.cuh"
+#include "optim_rows.cuh"
 
 #pragma clang fp contract(off)
 
@@ -32,22 +33,8 @@ struct OptArgs {
 };
 
 __device__ __forceinline__ bool row_offset(const OptArgs& a, int64_t idx, int64_t& b, int64_t& off) {
-  if (idx < 0) return false;
-  if (a.n_blocks == 1) {
-    b = 0;
-    off = idx;
-    return idx < a.block_size;
-  }
-  if ((static_cast<uint64_t>(idx) | static_cast<uint64_t>(a.block_size)) >> 32) {
-    b = idx / a.block_size;
-    off = idx - b * a.block_size;
-  } else {
-    const uint32_t bs = static_cast<uint32_t>(a.block_size);
-    const uint32_t q = static_cast<uint32_t>(idx) / bs;
-    b = q;
-    off = static_cast<uint32_t>(idx) - q * bs;
-  }
-  return b < a.n_blocks;
+  const RowBlocks r{a.n_blocks, a.block_size, a.D};
+  return block_row(r, idx, b, off);
 }
 
 // cal_alpha (block_apply_adamw_op.cc:77-85): advances the running powers in
@@ -79,32 +66,15 @@ adamw_rows_kernel(OptArgs a, const TG* __restrict__ grad, T* const* __restrict__
     return;
   }
   const double alpha = alpha_ptr[0];
-  const double omb1 = 1 - beta1, omb2 = 1 - beta2;
+  const AdamCoef coef{alpha_ptr, beta1, beta2, decay, eps};
   T* w_row = emb_blocks[b] + off * a.D;
   T* m_row = m_blocks[b] + off * a.D;
   T* v_row = v_blocks[b] + off * a.D;
   const TG* g_row = grad + i * a.D;
   for (int c0 = cl * VEC; c0 < a.D; c0 += VEC << a.lpr_log2) {
-    Pack<T, VEC> w = *reinterpret_cast<const Pack<T, VEC>*>(w_row + c0);
-    Pack<T, VEC> m = *reinterpret_cast<const Pack<T, VEC>*>(m_row + c0);
-    Pack<T, VEC> v = *reinterpret_cast<const Pack<T, VEC>*>(v_row + c0);
-    Pack<TG, VEC> g = *reinterpret_cast<const Pack<TG, VEC>*>(g_row + c0);
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      // every line: double arithmetic, then one rounding to the storage type
-      float we = to_float(w.v[j]), me = to_float(m.v[j]), ve = to_float(v.v[j]);
-      const float ge = to_float(g.v[j]);
-      we = to_float(from_float<T>(static_cast<float>(we * decay)));
-      me = to_float(from_float<T>(static_cast<float>(me * beta1 + ge * omb1)));
-      ve = to_float(from_float<T>(static_cast<float>(ve * beta2 + omb2 * ge * ge)));
-      we = to_float(from_float<T>(static_cast<float>(we + alpha * (me / (sqrtf(ve) + eps)))));
-      w.v[j] = from_float<T>(we);
-      m.v[j] = from_float<T>(me);
-      v.v[j] = from_float<T>(ve);
-    }
-    *reinterpret_cast<Pack<T, VEC>*>(w_row + c0) = w;
-    *reinterpret_cast<Pack<T, VEC>*>(m_row + c0) = m;
-    *reinterpret_cast<Pack<T, VEC>*>(v_row + c0) = v;
+    float g[VEC];
+    load_pack<TG, VEC>(g_row + c0, g);
+    adam_update_pack<T, VEC>(w_row + c0, m_row + c0, v_row + c0, g, alpha, coef);
   }
 }
 
@@ -125,20 +95,9 @@ adagrad_rows_kernel(OptArgs a, const TG* __restrict__ grad, T* const* __restrict
   T* s_row = acc_blocks[b] + off * a.D;
   const TG* g_row = grad + i * a.D;
   for (int c0 = cl * VEC; c0 < a.D; c0 += VEC << a.lpr_log2) {
-    Pack<T, VEC> w = *reinterpret_cast<const Pack<T, VEC>*>(w_row + c0);
-    Pack<T, VEC> s = *reinterpret_cast<const Pack<T, VEC>*>(s_row + c0);
-    Pack<TG, VEC> g = *reinterpret_cast<const Pack<TG, VEC>*>(g_row + c0);
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      float we = to_float(w.v[j]), se = to_float(s.v[j]);
-      const float ge = to_float(g.v[j]);
-      se = to_float(from_float<T>(se + ge * ge));
-      we = we - lr * (ge / (sqrtf(se) + eps));
-      w.v[j] = from_float<T>(we);
-      s.v[j] = from_float<T>(se);
-    }
-    *reinterpret_cast<Pack<T, VEC>*>(w_row + c0) = w;
-    *reinterpret_cast<Pack<T, VEC>*>(s_row + c0) = s;
+    float g[VEC];
+    load_pack<TG, VEC>(g_row + c0, g);
+    adagrad_update_pack<T, VEC>(w_row + c0, s_row + c0, g, lr, eps);
   }
 }
 
@@ -187,6 +146,19 @@ int fill_opt_args(OptArgs& a, const int64_t* index, const void* grad, int64_t n,
 }
 
 }  // namespace
+
+int launch_cal_alpha(void* beta1_t, void* beta2_t, int beta_is_f64, double* alpha_out, double lr, double beta1,
+                     double beta2, hipStream_t stream) {
+  if (beta_is_f64)
+    cal_alpha_kernel<double><<<1, 1, 0, stream>>>(static_cast<double*>(beta1_t), static_cast<double*>(beta2_t),
+                                                   alpha_out, lr, beta1, beta2);
+  else
+    cal_alpha_kernel<float><<<1, 1, 0, stream>>>(static_cast<float*>(beta1_t), static_cast<float*>(beta2_t), alpha_out,
+                                                  lr, beta1, beta2);
+  RECIS_LAUNCH_CHECK();
+  return RECIS_OK;
+}
+
 }  // namespace recis_hip
 
 using namespace recis_hip;
@@ -205,13 +177,7 @@ int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dty
   void* ws = nullptr;
   if (int rc = get_workspace(stream, 256, &ws)) return rc;
   double* alpha = static_cast<double*>(ws);
-  if (beta_is_f64)
-    cal_alpha_kernel<double><<<1, 1, 0, stream>>>(static_cast<double*>(beta1_t),
-                                                   static_cast<double*>(beta2_t), alpha, lr, beta1, beta2);
-  else
-    cal_alpha_kernel<float><<<1, 1, 0, stream>>>(static_cast<float*>(beta1_t),
-                                                  static_cast<float*>(beta2_t), alpha, lr, beta1, beta2);
-  RECIS_LAUNCH_CHECK();
+  if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, alpha, lr, beta1, beta2, stream)) return rc;
   if (n == 0) return RECIS_OK;
   RECIS_REQUIRE(emb_blocks_dev && exp_avg_blocks_dev && exp_avg_sq_blocks_dev, "block tables must not be NULL");
   OptArgs a;

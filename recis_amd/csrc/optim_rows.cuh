@@ -1,0 +1,112 @@
+// The per-row arithmetic of the sparse optimizers, shared by the stand-alone row kernels
+// (optim.hip) and the gather-reduce kernels that apply the update as soon as a row's gradient is
+// summed (plan.hip).
+//
+// Adam family: what block_apply_adamw does per element (csrc/ops/block_apply_adamw_op.cc:32-58):
+// products and sums in double, sqrtf in float, every assignment rounded to the storage type, no
+// fused multiply-add. The kernels are bound by memory traffic, so the arithmetic is free, and
+// doing it this way reproduces the reference's CPU path bit for bit.
+// Adagrad has no reference counterpart; it is the textbook update in float.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "common.cuh"
+
+namespace recis_hip {
+
+// Where the rows of the table live and which of them a launch touches.
+struct RowBlocks {
+  int64_t n_blocks;
+  int64_t block_size;
+  int D;
+};
+
+// Block and row-in-block of table row idx; false when idx is negative or beyond the blocks.
+__device__ __forceinline__ bool block_row(const RowBlocks& r, int64_t idx, int64_t& b, int64_t& off) {
+  if (idx < 0) return false;
+  if (r.n_blocks == 1) {
+    b = 0;
+    off = idx;
+    return idx < r.block_size;
+  }
+  if ((static_cast<uint64_t>(idx) | static_cast<uint64_t>(r.block_size)) >> 32) {
+    b = idx / r.block_size;
+    off = idx - b * r.block_size;
+  } else {
+    const uint32_t bs = static_cast<uint32_t>(r.block_size);
+    const uint32_t q = static_cast<uint32_t>(idx) / bs;
+    b = q;
+    off = static_cast<uint32_t>(idx) - q * bs;
+  }
+  return b < r.n_blocks;
+}
+
+struct AdamCoef {
+  const double* alpha;  // device word left by cal_alpha: -lr / (1 - beta1^t) * sqrtf(1 - beta2^t)
+  double beta1, beta2, decay, eps;
+};
+
+// One pack of VEC elements of one row, in registers: g = gradient (fp32); w / m / v updated in place.
+template <typename T, int VEC>
+__device__ __forceinline__ void adam_compute_pack(Pack<T, VEC>& w, Pack<T, VEC>& m, Pack<T, VEC>& v,
+                                                  const float (&g)[VEC], double alpha, const AdamCoef& c) {
+#pragma clang fp contract(off)
+  const double omb1 = 1 - c.beta1, omb2 = 1 - c.beta2;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    // every line: double arithmetic, then one rounding to the storage type
+    float we = to_float(w.v[j]), me = to_float(m.v[j]), ve = to_float(v.v[j]);
+    const float ge = g[j];
+    we = to_float(from_float<T>(static_cast<float>(we * c.decay)));
+    me = to_float(from_float<T>(static_cast<float>(me * c.beta1 + ge * omb1)));
+    ve = to_float(from_float<T>(static_cast<float>(ve * c.beta2 + omb2 * ge * ge)));
+    we = to_float(from_float<T>(static_cast<float>(we + alpha * (me / (sqrtf(ve) + c.eps)))));
+    w.v[j] = from_float<T>(we);
+    m.v[j] = from_float<T>(me);
+    v.v[j] = from_float<T>(ve);
+  }
+}
+
+// The same on memory: read, update, write.
+template <typename T, int VEC>
+__device__ __forceinline__ void adam_update_pack(T* w_ptr, T* m_ptr, T* v_ptr, const float (&g)[VEC], double alpha,
+                                                 const AdamCoef& c) {
+  Pack<T, VEC> w = *reinterpret_cast<const Pack<T, VEC>*>(w_ptr);
+  Pack<T, VEC> m = *reinterpret_cast<const Pack<T, VEC>*>(m_ptr);
+  Pack<T, VEC> v = *reinterpret_cast<const Pack<T, VEC>*>(v_ptr);
+  adam_compute_pack<T, VEC>(w, m, v, g, alpha, c);
+  *reinterpret_cast<Pack<T, VEC>*>(w_ptr) = w;
+  *reinterpret_cast<Pack<T, VEC>*>(m_ptr) = m;
+  *reinterpret_cast<Pack<T, VEC>*>(v_ptr) = v;
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void adagrad_compute_pack(Pack<T, VEC>& w, Pack<T, VEC>& s, const float (&g)[VEC], float lr,
+                                                     float eps) {
+#pragma clang fp contract(off)
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    float we = to_float(w.v[j]), se = to_float(s.v[j]);
+    const float ge = g[j];
+    se = to_float(from_float<T>(se + ge * ge));
+    we = we - lr * (ge / (sqrtf(se) + eps));
+    w.v[j] = from_float<T>(we);
+    s.v[j] = from_float<T>(se);
+  }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void adagrad_update_pack(T* w_ptr, T* s_ptr, const float (&g)[VEC], float lr, float eps) {
+  Pack<T, VEC> w = *reinterpret_cast<const Pack<T, VEC>*>(w_ptr);
+  Pack<T, VEC> s = *reinterpret_cast<const Pack<T, VEC>*>(s_ptr);
+  adagrad_compute_pack<T, VEC>(w, s, g, lr, eps);
+  *reinterpret_cast<Pack<T, VEC>*>(w_ptr) = w;
+  *reinterpret_cast<Pack<T, VEC>*>(s_ptr) = s;
+}
+
+// cal_alpha (block_apply_adamw_op.cc:77-85) as a one-thread launch on `stream`: advances the
+// running powers in place, in their own precision, and leaves alpha (as double) in alpha_out.
+int launch_cal_alpha(void* beta1_t, void* beta2_t, int beta_is_f64, double* alpha_out, double lr, double beta1,
+                     double beta2, hipStream_t stream);
+
+}  // namespace recis_hip

@@ -33,6 +33,7 @@
 
 #include "common.cuh"
 #include "idmap_internal.cuh"
+#include "optim_rows.cuh"
 
 namespace recis_hip {
 namespace {
@@ -51,6 +52,10 @@ constexpr int kBucketBlock = 512;
 constexpr int kPer = 9;             // consecutive table entries owned by a thread (9 * 512 > kTabAll)
 constexpr int kRegs = 8;            // bucket records of a thread whose table entry stays in registers
 constexpr int64_t kSetEmpty = -1;
+constexpr int kHeavyMax = 64;       // ids that get a column of their own in the partition (see plan_heavy_kernel)
+constexpr int kHeavySamples = 2048; // ids sampled to find them
+constexpr int kHeavyTab = 4096;     // LDS table of the sampling kernel
+constexpr int kHeavySlots = 256;    // LDS table every partition workgroup looks ids up in
 constexpr int kHotLen = RECIS_PLAN_HOT_LEN;  // rows with more occurrences than this are "hot"
 constexpr int kHotChunk = RECIS_PLAN_HOT_CHUNK;  // occurrences per hot work item
 static_assert(kPer * kBucketBlock > kTabAll, "every table entry needs an owner");
@@ -73,18 +78,194 @@ __device__ __forceinline__ int home_of_mix(uint64_t mixed, int nb_log2) {
   return static_cast<int>(mixed >> (64 - nb_log2 - 12)) & (kTabHome - 1);
 }
 
-// hist: ids per (row, bucket)
-__global__ void __launch_bounds__(kPartBlock)
-plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, int32_t* __restrict__ hist,
-                 int64_t* __restrict__ counts, int32_t* __restrict__ sync) {
-  extern __shared__ int32_t l_hist[];
+// Heavy ids. An id that makes up a sizeable share of the batch (the head of a Zipf distribution, the
+// few values of a low-cardinality feature) would put all its occurrences into one bucket and leave
+// one workgroup with a hundred times the work of the others. Such ids are found beforehand by
+// sampling and get a column of their own in the partition: their occurrences go straight into
+// their list (no dedup needed: the column holds one id), and they become the first unique ids.
+//   heavy_ids [kHeavyMax], heavy_n [1]: the ids, ordered by (sample count descending, id ascending):
+//   a function of the input alone.
+// One workgroup: kHeavySamples ids at a fixed stride, counted in an LDS table; an id counts as heavy
+// when its estimated number of occurrences would fill more than a bucket and a half.
+__global__ void __launch_bounds__(1024)
+plan_heavy_kernel(const int64_t* __restrict__ ids, int64_t n, int64_t* __restrict__ heavy_ids,
+                  int32_t* __restrict__ heavy_n) {
+  __shared__ int64_t t_key[kHeavyTab];
+  __shared__ int32_t t_cnt[kHeavyTab];
+  __shared__ int64_t c_key[kHeavySamples / 8];
+  __shared__ int32_t c_cnt[kHeavySamples / 8];
+  __shared__ int32_t s_ncand, s_minus1;
   const int tid = threadIdx.x;
-  const int nb = 1 << g.nb_log2;
+  const int64_t stride = n / kHeavySamples;
+  if (stride < 4) {  // a batch this small is no burden for one workgroup per bucket
+    if (tid == 0) *heavy_n = 0;
+    return;
+  }
+  for (int e = tid; e < kHeavyTab; e += 1024) {
+    t_key[e] = kSetEmpty;
+    t_cnt[e] = 0;
+  }
+  if (tid == 0) {
+    s_ncand = 0;
+    s_minus1 = 0;
+  }
+  __syncthreads();
+  int64_t k[kHeavySamples / 1024];
+#pragma unroll
+  for (int x = 0; x < kHeavySamples / 1024; ++x) k[x] = ids[(static_cast<int64_t>(x) * 1024 + tid) * stride + stride / 2];
+#pragma unroll
+  for (int x = 0; x < kHeavySamples / 1024; ++x) {
+    if (k[x] == kSetEmpty) {  // the table's empty marker is a legal id: counted apart
+      atomicAdd(&s_minus1, 1);
+      continue;
+    }
+    int e = static_cast<int>(mix_id(k[x]) >> 40) & (kHeavyTab - 1);
+    for (;;) {  // half empty at worst: always ends
+      const int64_t c = *reinterpret_cast<volatile int64_t*>(&t_key[e]);
+      if (c == k[x]) break;
+      if (c == kSetEmpty) {
+        const unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&t_key[e]),
+                                                 static_cast<unsigned long long>(kSetEmpty),
+                                                 static_cast<unsigned long long>(k[x]));
+        if (old == static_cast<unsigned long long>(kSetEmpty) || old == static_cast<unsigned long long>(k[x])) break;
+        continue;  // somebody else's id landed there: look at it again
+      }
+      e = (e + 1) & (kHeavyTab - 1);
+    }
+    atomicAdd(&t_cnt[e], 1);
+  }
+  __syncthreads();
+  // estimated occurrences = count * stride; heavy from one and a half buckets' worth, and never on
+  // fewer than 8 samples (so at most kHeavySamples / 8 candidates)
+  const int64_t want = (3 * kBucketIds / 2 + stride - 1) / stride;
+  const int32_t thr = static_cast<int32_t>(want < 8 ? 8 : (want > kHeavySamples ? kHeavySamples + 1 : want));
+  for (int e = tid; e <= kHeavyTab; e += 1024) {
+    const int32_t c = e < kHeavyTab ? t_cnt[e] : s_minus1;
+    if (c >= thr) {
+      const int at = atomicAdd(&s_ncand, 1);
+      c_key[at] = e < kHeavyTab ? t_key[e] : kSetEmpty;
+      c_cnt[at] = c;
+    }
+  }
+  __syncthreads();
+  const int ncand = s_ncand;
+  for (int i = tid; i < ncand; i += 1024) {  // rank by (count descending, id ascending): the first kHeavyMax stay
+    int rank = 0;
+    const int32_t ci = c_cnt[i];
+    const uint64_t ki = static_cast<uint64_t>(c_key[i]);
+    for (int j = 0; j < ncand; ++j) {
+      const int32_t cj = c_cnt[j];
+      rank += (cj > ci || (cj == ci && static_cast<uint64_t>(c_key[j]) < ki)) ? 1 : 0;
+    }
+    if (rank < kHeavyMax) heavy_ids[rank] = c_key[i];
+  }
+  if (tid == 0) *heavy_n = ncand < kHeavyMax ? ncand : kHeavyMax;
+}
+
+// The heavy ids as an LDS table for the partition kernels: h_slot [kHeavySlots] holds the index of
+// a heavy id or -1, h_key its id (at most a quarter full: most ids end their search on the first
+// word they read). Every thread of the workgroup calls; ends with a barrier.
+__device__ __forceinline__ int load_heavy(const int64_t* __restrict__ heavy_ids, const int32_t* __restrict__ heavy_n,
+                                          int32_t* h_slot, int64_t* h_key) {
+  const int n_heavy = *heavy_n;
+  if (n_heavy == 0) return 0;  // uniform
+  for (int e = threadIdx.x; e < kHeavySlots; e += blockDim.x) h_slot[e] = -1;
+  __syncthreads();
+  if (static_cast<int>(threadIdx.x) < n_heavy) {
+    const int64_t key = heavy_ids[threadIdx.x];
+    int e = static_cast<int>(mix_id(key) >> 24) & (kHeavySlots - 1);
+    while (atomicCAS(&h_slot[e], -1, static_cast<int32_t>(threadIdx.x)) != -1) e = (e + 1) & (kHeavySlots - 1);
+    h_key[e] = key;
+  }
+  __syncthreads();
+  return n_heavy;
+}
+// Index of `key` among the heavy ids, or -1.
+__device__ __forceinline__ int heavy_index(int64_t key, uint64_t mixed, const int32_t* h_slot, const int64_t* h_key) {
+  int e = static_cast<int>(mixed >> 24) & (kHeavySlots - 1);
+  for (;;) {
+    const int32_t h = h_slot[e];
+    if (h < 0) return -1;
+    if (h_key[e] == key) return h;
+    e = (e + 1) & (kHeavySlots - 1);
+  }
+}
+// Column of an id in the partition: its own when it is heavy, else that of its bucket.
+__device__ __forceinline__ int column_of(int64_t key, int nb_log2, int n_heavy, const int32_t* h_slot,
+                                         const int64_t* h_key) {
+  const uint64_t mixed = mix_id(key);
+  if (n_heavy > 0) {
+    const int h = heavy_index(key, mixed, h_slot, h_key);
+    if (h >= 0) return h;
+  }
+  return kHeavyMax + bucket_of_mix(mixed, nb_log2);
+}
+
+// atomicAdd(&arr[e], 1) for every lane with `active`, each lane getting back a value that no other
+// lane gets for the same entry. Ids of low-cardinality features repeat thousands of times in a
+// bucket, and atomics of one wave on one LDS word are served one after the other (some 3 ns each:
+// a bucket with a 6500-fold id spent 20 us there); so when many lanes of the wave name the entry
+// of the first (or of the last) active lane, one of them adds their number and hands out the places.
+__device__ __forceinline__ int32_t wave_add_one(int32_t* arr, int e, bool active) {
+  int32_t result = 0;
+  if (__ballot(active) == 0) return result;  // uniform
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const uint64_t todo = __ballot(active);
+    if (todo == 0) break;
+    const int leader = it == 0 ? __ffsll(static_cast<unsigned long long>(todo)) - 1 : 63 - __clzll(todo);
+    const int e_l = __shfl(e, leader, kWave);
+    const uint64_t same = __ballot(active && e == e_l);
+    const int n_same = __popcll(same);
+    if (n_same < 8) continue;
+    int32_t base = 0;
+    if (lane == leader) base = atomicAdd(&arr[e_l], n_same);
+    base = __shfl(base, leader, kWave);
+    if (active && e == e_l) {
+      result = base + __popcll(same & ((uint64_t(1) << lane) - 1));
+      active = false;
+    }
+  }
+  if (active) result = atomicAdd(&arr[e], 1);
+  return result;
+}
+
+// arr[e] += 1 for every lane with `active`, lanes that name the same entry adding up among themselves first
+// when there are many of them (see wave_add_one, which also hands out the places).
+__device__ __forceinline__ void wave_count_one(int32_t* arr, int e, bool active) {
+  if (__ballot(active) == 0) return;  // uniform
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const uint64_t todo = __ballot(active);
+    if (todo == 0) return;
+    const int leader = it == 0 ? __ffsll(static_cast<unsigned long long>(todo)) - 1 : 63 - __clzll(todo);
+    const int e_l = __shfl(e, leader, kWave);
+    const uint64_t same = __ballot(active && e == e_l);
+    if (__popcll(same) < 8) continue;
+    if (lane == leader) atomicAdd(&arr[e_l], __popcll(same));
+    if (e == e_l) active = false;
+  }
+  if (active) atomicAdd(&arr[e], 1);
+}
+
+// hist: ids per (row, column); columns: the heavy ids, then the buckets
+__global__ void __launch_bounds__(kPartBlock)
+plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int64_t* __restrict__ heavy_ids,
+                 const int32_t* __restrict__ heavy_n, int32_t* __restrict__ hist, int64_t* __restrict__ counts,
+                 int32_t* __restrict__ sync) {
+  extern __shared__ int32_t l_hist[];  // [kHeavyMax + nb]
+  __shared__ int32_t h_slot[kHeavySlots];
+  __shared__ int64_t h_key[kHeavySlots];
+  const int tid = threadIdx.x;
+  const int nc = kHeavyMax + (1 << g.nb_log2);
   if (blockIdx.x == 0) {
     if (tid < 2) counts[tid] = 0;
-    if (tid < 4) sync[tid] = 0;  // [1] bucket tickets, [2] finished workgroups of the row assignment
+    if (tid < 4) sync[tid] = 0;  // [1] finished workgroups of the bucket kernel, [2] of the row assignment
   }
-  for (int b = tid; b < nb; b += kPartBlock) l_hist[b] = 0;
+  for (int b = tid; b < nc; b += kPartBlock) l_hist[b] = 0;
+  const int n_heavy = load_heavy(heavy_ids, heavy_n, h_slot, h_key);
   __syncthreads();
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
   for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {  // four loads in flight
@@ -95,12 +276,17 @@ plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, int32_t* __restric
       k[x] = i < hi ? ids[i] : 0;
     }
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
-      if (i0 + x * kPartBlock < hi) atomicAdd(&l_hist[bucket_of_mix(mix_id(k[x]), g.nb_log2)], 1);
+    for (int x = 0; x < 4; ++x) {
+      const bool valid = i0 + x * kPartBlock < hi;
+      const int c = column_of(k[x], g.nb_log2, n_heavy, h_slot, h_key);
+      const bool heavy = valid && c < kHeavyMax;
+      if (n_heavy > 0) wave_count_one(l_hist, c, heavy);  // a heavy id is many lanes on one word
+      if (valid && !heavy) atomicAdd(&l_hist[c], 1);
+    }
   }
   __syncthreads();
-  int32_t* row = hist + static_cast<int64_t>(blockIdx.x) * nb;
-  for (int b = tid; b < nb; b += kPartBlock) row[b] = l_hist[b];
+  int32_t* row = hist + static_cast<int64_t>(blockIdx.x) * nc;
+  for (int b = tid; b < nc; b += kPartBlock) row[b] = l_hist[b];
 }
 
 // colscan: for every bucket, exclusive scan of its histogram column over the rows, in place, and
@@ -110,7 +296,7 @@ constexpr int kColGroups = 1024 / kColBuckets;
 __global__ void __launch_bounds__(1024)
 plan_colscan_kernel(int32_t* __restrict__ hist, PlanGeom g, int32_t* __restrict__ bucket_total) {
   __shared__ int32_t part[kColGroups][kColBuckets + 1];
-  const int nb = 1 << g.nb_log2;
+  const int nb = kHeavyMax + (1 << g.nb_log2);  // columns (a multiple of kColBuckets)
   const int t = threadIdx.x;
   const int bl = t % kColBuckets, rg = t / kColBuckets;
   const int b = blockIdx.x * kColBuckets + bl;
@@ -165,26 +351,40 @@ __device__ __forceinline__ void scan_counts(const int32_t* in, int nb, int32_t* 
   __syncthreads();
 }
 
-// scatter: (id, position) of every occurrence goes to its bucket. Every workgroup scans the bucket
+// What the partition kernels need to put the occurrences of heavy ids straight into their lists.
+struct HeavyArgs {
+  const int64_t* ids;   // [kHeavyMax]
+  const int32_t* n;     // [1]
+  int32_t* list;        // the plan's list_out
+  int32_t* inverse;     // may be NULL
+  int32_t* pos_out;     // may be NULL
+};
+
+// scatter: (id, position) of every occurrence goes to its column: for a bucket into bkt_id / bkt_pos,
+// for a heavy id the position goes into the plan's list at once (list space and bucket space are
+// the same index space: a column's entries are its list entries). Every workgroup scans the column
 // totals for itself (a thousand words), so no kernel stands between the column scan and this one;
-// the first workgroup also leaves bucket_start [nb + 1] for the bucket kernel and clears that
+// the first workgroup also leaves bucket_start [columns + 1] for the bucket kernel and clears that
 // kernel's look-back words.
 __global__ void __launch_bounds__(kPartBlock)
-plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int32_t* __restrict__ off,
+plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs hv, const int32_t* __restrict__ off,
                     const int32_t* __restrict__ bucket_total, int32_t* __restrict__ bucket_start,
                     unsigned long long* __restrict__ agg, int64_t* __restrict__ bkt_id,
                     int32_t* __restrict__ bkt_pos) {
-  extern __shared__ int32_t cursor[];  // [nb + 1], then kPartBlock words of scan scratch
+  extern __shared__ int32_t cursor[];  // [nc + 1], then kPartBlock words of scan scratch
+  __shared__ int32_t h_slot[kHeavySlots];
+  __shared__ int64_t h_key[kHeavySlots];
   const int tid = threadIdx.x;
-  const int nb = 1 << g.nb_log2;
-  scan_counts(bucket_total, nb, cursor, cursor + nb + 1);
+  const int nb = 1 << g.nb_log2, nc = kHeavyMax + nb;
+  const int n_heavy = load_heavy(hv.ids, hv.n, h_slot, h_key);
+  scan_counts(bucket_total, nc, cursor, cursor + nc + 1);
   if (blockIdx.x == 0) {
-    for (int b = tid; b <= nb; b += kPartBlock) bucket_start[b] = cursor[b];
+    for (int b = tid; b <= nc; b += kPartBlock) bucket_start[b] = cursor[b];
     for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
   }
-  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nb;
+  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nc;
   __syncthreads();
-  for (int b = tid; b < nb; b += kPartBlock) cursor[b] += off_row[b];
+  for (int b = tid; b < nc; b += kPartBlock) cursor[b] += off_row[b];
   __syncthreads();
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
   for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {
@@ -197,8 +397,17 @@ plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int32_t* 
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
       const int64_t i = i0 + x * kPartBlock;
-      if (i < hi) {
-        const int32_t p = atomicAdd(&cursor[bucket_of_mix(mix_id(k[x]), g.nb_log2)], 1);
+      const int c = column_of(k[x], g.nb_log2, n_heavy, h_slot, h_key);
+      const bool heavy = i < hi && c < kHeavyMax;
+      int32_t p = 0;
+      if (n_heavy > 0) p = wave_add_one(cursor, c, heavy);
+      if (i < hi && !heavy) p = atomicAdd(&cursor[c], 1);
+      if (i >= hi) continue;
+      if (c < kHeavyMax) {
+        hv.list[p] = static_cast<int32_t>(i);
+        if (hv.inverse) hv.inverse[i] = c;
+        if (hv.pos_out) hv.pos_out[i] = p;
+      } else {
         bkt_id[p] = k[x];
         bkt_pos[p] = static_cast<int32_t>(i);
       }
@@ -214,27 +423,30 @@ plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int32_t* 
 // size).
 constexpr int kTilePer = kTile / kPartBlock;
 __global__ void __launch_bounds__(kPartBlock)
-plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int32_t* __restrict__ off,
-                         const int32_t* __restrict__ bucket_total, int32_t* __restrict__ bucket_start,
-                         unsigned long long* __restrict__ agg, int64_t* __restrict__ bkt_id,
-                         int32_t* __restrict__ bkt_pos) {
+plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs hv,
+                         const int32_t* __restrict__ off, const int32_t* __restrict__ bucket_total,
+                         int32_t* __restrict__ bucket_start, unsigned long long* __restrict__ agg,
+                         int64_t* __restrict__ bkt_id, int32_t* __restrict__ bkt_pos) {
   extern __shared__ int32_t lds[];
+  __shared__ int32_t h_slot[kHeavySlots];
+  __shared__ int64_t h_key[kHeavySlots];
   const int tid = threadIdx.x;
-  const int nb = 1 << g.nb_log2;
-  int32_t* gbase = lds;               // [nb + 1] where the tile's ids of a bucket go
-  int32_t* first = lds + nb + 1;      // [nb + 1] ids of the tile per bucket, then where they start in bucket order
-  int32_t* partial = first + nb + 1;  // [kPartBlock] scan scratch
-  uint16_t* sorted = reinterpret_cast<uint16_t*>(partial + kPartBlock);  // [kTile] the tile's ids in bucket order
-  uint16_t* sorted_bucket = sorted + kTile;                              // [kTile] and their buckets
-  for (int b = tid; b <= nb; b += kPartBlock) first[b] = 0;
-  scan_counts(bucket_total, nb, gbase, partial);
+  const int nb = 1 << g.nb_log2, nc = kHeavyMax + nb;
+  int32_t* gbase = lds;               // [nc + 1] where the tile's ids of a column go
+  int32_t* first = lds + nc + 1;      // [nc + 1] ids of the tile per column, then where they start in column order
+  int32_t* partial = first + nc + 1;  // [kPartBlock] scan scratch
+  uint16_t* sorted = reinterpret_cast<uint16_t*>(partial + kPartBlock);  // [kTile] the tile's ids in column order
+  uint16_t* sorted_bucket = sorted + kTile;                              // [kTile] and their columns
+  for (int b = tid; b <= nc; b += kPartBlock) first[b] = 0;
+  const int n_heavy = load_heavy(hv.ids, hv.n, h_slot, h_key);
+  scan_counts(bucket_total, nc, gbase, partial);
   if (blockIdx.x == 0) {
-    for (int b = tid; b <= nb; b += kPartBlock) bucket_start[b] = gbase[b];
+    for (int b = tid; b <= nc; b += kPartBlock) bucket_start[b] = gbase[b];
     for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
   }
-  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nb;
+  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nc;
   __syncthreads();
-  for (int b = tid; b < nb; b += kPartBlock) gbase[b] += off_row[b];
+  for (int b = tid; b < nc; b += kPartBlock) gbase[b] += off_row[b];
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile;
   const int n_here = static_cast<int>(min(g.n, lo + g.tile) - lo);
   int64_t k[kTilePer];
@@ -246,12 +458,15 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int3
   }
 #pragma unroll
   for (int x = 0; x < kTilePer; ++x) {
+    const bool valid = tid + x * kPartBlock < n_here;
+    bucket[x] = static_cast<uint16_t>(column_of(k[x], g.nb_log2, n_heavy, h_slot, h_key));
+    const bool heavy = valid && bucket[x] < kHeavyMax;
     rank[x] = 0;
-    bucket[x] = static_cast<uint16_t>(bucket_of_mix(mix_id(k[x]), g.nb_log2));
-    if (tid + x * kPartBlock < n_here) rank[x] = static_cast<uint16_t>(atomicAdd(&first[bucket[x]], 1));
+    if (n_heavy > 0) rank[x] = static_cast<uint16_t>(wave_add_one(first, bucket[x], heavy));
+    if (valid && !heavy) rank[x] = static_cast<uint16_t>(atomicAdd(&first[bucket[x]], 1));
   }
   __syncthreads();
-  scan_counts(first, nb, first, partial);  // counts -> starts in bucket order
+  scan_counts(first, nc, first, partial);  // counts -> starts in column order
 #pragma unroll
   for (int x = 0; x < kTilePer; ++x) {
     const int i = tid + x * kPartBlock;
@@ -277,8 +492,15 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int3
       if (j >= n_here) continue;
       const int b = sorted_bucket[j];
       const int32_t d = gbase[b] + (j - first[b]);
-      bkt_id[d] = key[x];
-      bkt_pos[d] = static_cast<int32_t>(lo + i[x]);
+      const int32_t at = static_cast<int32_t>(lo + i[x]);
+      if (b < kHeavyMax) {
+        hv.list[d] = at;
+        if (hv.inverse) hv.inverse[at] = b;
+        if (hv.pos_out) hv.pos_out[at] = d;
+      } else {
+        bkt_id[d] = key[x];
+        bkt_pos[d] = at;
+      }
     }
   }
 }
@@ -292,11 +514,13 @@ struct alignas(16) NewRec {
 struct BucketArgs {
   const int64_t* bkt_id;
   const int32_t* bkt_pos;
-  const int32_t* bucket_start;  // [nb + 1]
+  const int32_t* bucket_start;  // [kHeavyMax + nb + 1]: the columns of the heavy ids, then the buckets
+  const int64_t* heavy_ids;     // [kHeavyMax]
+  const int32_t* heavy_n;       // [1]
   PlanGeom g;
   unsigned long long* agg;  // [nb] look-back words: distinct ids per bucket
-  int32_t* new_count;       // [nb] keys new to the id map per bucket
-  int32_t* sync;            // [1] = bucket tickets, [2] = workgroups of the row assignment that are done
+  int32_t* new_count;       // [1 + nb] keys new to the id map: among the heavy ids, then per bucket
+  int32_t* sync;            // [1] = workgroups of the bucket kernel that are done, [2] = of the row assignment
   int64_t* unique_out;
   int32_t* inverse;    // may be NULL
   int32_t* row_start;
@@ -347,35 +571,6 @@ __device__ __forceinline__ unsigned long long block_scan_u64(unsigned long long 
   return before;
 }
 
-// atomicAdd(&arr[e], 1) for every lane with `active`, each lane getting back a value that no other
-// lane gets for the same entry. Ids of low-cardinality features repeat thousands of times in a
-// bucket, and atomics of one wave on one LDS word are served one after the other (some 3 ns each:
-// a bucket with a 6500-fold id spent 20 us there); so when many lanes of the wave name the entry
-// of the first (or of the last) active lane, one of them adds their number and hands out the places.
-__device__ __forceinline__ int32_t wave_add_one(int32_t* arr, int e, bool active) {
-  int32_t result = 0;
-  const int lane = threadIdx.x & (kWave - 1);
-#pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    const uint64_t todo = __ballot(active);
-    if (todo == 0) break;
-    const int leader = it == 0 ? __ffsll(static_cast<unsigned long long>(todo)) - 1 : 63 - __clzll(todo);
-    const int e_l = __shfl(e, leader, kWave);
-    const uint64_t same = __ballot(active && e == e_l);
-    const int n_same = __popcll(same);
-    if (n_same < 8) continue;
-    int32_t base = 0;
-    if (lane == leader) base = atomicAdd(&arr[e_l], n_same);
-    base = __shfl(base, leader, kWave);
-    if (active && e == e_l) {
-      result = base + __popcll(same & ((uint64_t(1) << lane) - 1));
-      active = false;
-    }
-  }
-  if (active) result = atomicAdd(&arr[e], 1);
-  return result;
-}
-
 constexpr unsigned long long kAggFlag = 1ull << 62, kPrefixFlag = 2ull << 62, kAggValue = (1ull << 62) - 1;
 
 // Sum of the distinct-id counts of all buckets before bucket b, by the whole workgroup: thread t
@@ -387,13 +582,15 @@ constexpr unsigned long long kAggFlag = 1ull << 62, kPrefixFlag = 2ull << 62, kA
 // in one 64-bit atomic), so relaxed device-scope atomics are enough: nothing else has to become
 // visible with it. (Release / acquire at device scope write back and invalidate the whole L2 of the
 // XCD on this part: tens of microseconds per workgroup.) Every thread calls; ends with a barrier.
-__device__ __forceinline__ int64_t look_back(unsigned long long* __restrict__ agg, int b, uint32_t spin_limit,
-                                             int* err, unsigned long long* s_look /* [kBucketBlock / kWave] */) {
+__device__ __forceinline__ int64_t look_back(unsigned long long* __restrict__ agg, int b, int n_heavy,
+                                             uint32_t spin_limit, int* err,
+                                             unsigned long long* s_look /* [kBucketBlock / kWave] */) {
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   int64_t sum = 0;
   for (int hi = b - 1;; hi -= kBucketBlock) {
     const int j = hi - static_cast<int>(threadIdx.x);
-    unsigned long long w = kPrefixFlag;  // before the first bucket: an inclusive prefix of zero
+    // before the first bucket: the heavy ids, which are the first unique ids
+    unsigned long long w = kPrefixFlag | static_cast<unsigned long long>(n_heavy);
     if (j >= 0) {
       uint32_t polls = 0;
       for (;;) {
@@ -401,7 +598,7 @@ __device__ __forceinline__ int64_t look_back(unsigned long long* __restrict__ ag
         if ((w >> 62) != 0) break;
         if (++polls > spin_limit) {
           raise_device_error(err, RECIS_DEVERR_PLAN_OVERFLOW);
-          w = kPrefixFlag;
+          w = kPrefixFlag;  // goes on with zero
           break;
         }
         __builtin_amdgcn_s_sleep(2);
@@ -429,6 +626,86 @@ __device__ __forceinline__ int64_t look_back(unsigned long long* __restrict__ ag
   return sum;
 }
 
+// One thread of a workgroup of the bucket kernel that is done calls this: the workgroup that
+// finishes last sends the count and the soft-error bits to the host (pinned words: no copy kernel
+// needed). Only then has every workgroup raised what it had to raise.
+__device__ __forceinline__ void finish_ticket(const BucketArgs& a) {
+  // this thread's earlier stores must have reached the L2 before its ticket does; a fence of
+  // workgroup scope waits for exactly that (one of device scope would write back the whole L2)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  if (atomicAdd(&a.sync[1], 1) == (1 << a.g.nb_log2)) {  // the buckets and the heavy ids' workgroup
+    a.staged[1] = __hip_atomic_load(a.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    a.staged[0] = __hip_atomic_load(&a.counts[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// The heavy ids' share of what the bucket kernel writes per unique id: heavy id h is unique id h, its
+// list is its column (filled by the scatter kernel). One workgroup, a thread per heavy id.
+template <bool PROBE>
+__device__ __forceinline__ void heavy_rows(const BucketArgs& a, int n_heavy, unsigned long long* s_wave) {
+  const int h = threadIdx.x;
+  int32_t my_new = 0, my_empty = 0;
+  int64_t row = -1;
+  if (h < n_heavy) {
+    const int64_t key = a.heavy_ids[h];
+    const int32_t start = a.bucket_start[h], n_here = a.bucket_start[h + 1] - start;
+    a.unique_out[h] = key;
+    a.row_start[h] = start;
+    if (a.hot_cap > 0 && n_here > kHotLen) {
+      const int n_items = (n_here + kHotChunk - 1) / kHotChunk;
+      const int64_t base = static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&a.counts[1]),
+                                                          static_cast<unsigned long long>(n_items)));
+      for (int c = 0; c < n_items; ++c) {
+        if (base + c < a.hot_cap) {
+          a.hot_items[2 * (base + c)] = h;
+          a.hot_items[2 * (base + c) + 1] = c;
+        }
+      }
+    }
+    if constexpr (PROBE) {
+      if (key == kEmpty || key == kTomb) {
+        raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);  // the map's reserved keys
+      } else {
+        const uint64_t home = home_slot(key, a.mask);
+        const longlong2 hint = *reinterpret_cast<const longlong2*>(&a.table[home]);
+        int64_t value = -1, slot = -1;
+        bool took_empty = false;
+        switch (probe_or_claim(a.table, a.mask, key, home, hint, -2, &value, &slot, &took_empty)) {
+          case kProbeFound:
+            row = value;
+            break;
+          case kProbeClaimed:
+            row = -(slot + 2);
+            my_new = 1;
+            my_empty = took_empty ? 1 : 0;
+            break;
+          default:
+            raise_device_error(a.err, RECIS_DEVERR_TABLE_FULL);
+            break;
+        }
+      }
+      a.index_out[h] = row;
+    }
+  }
+  if constexpr (PROBE) {  // new keys among them, in the order of the unique ids, at the first column's entries
+    unsigned long long new_total;
+    const unsigned long long new_before = block_scan_u64(
+        (static_cast<unsigned long long>(my_empty) << 32) | static_cast<unsigned long long>(my_new), s_wave, new_total);
+    if (threadIdx.x == 0) {
+      if ((new_total >> 32) != 0) atomicAdd(reinterpret_cast<unsigned long long*>(&a.state[ST_OCC]), new_total >> 32);
+      a.new_count[0] = static_cast<int32_t>(new_total & 0xffffffffull);
+    }
+    if (my_new) {
+      NewRec nr;
+      nr.u = h;
+      nr.slot = -(row + 2);
+      a.new_list[a.bucket_start[0] + static_cast<int32_t>(new_before & 0xffffffffull)] = nr;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0 && a.staged) finish_ticket(a);
+}
+
 // bucket: one workgroup per bucket, in the order of the workgroup index. The bucket's ids are
 // deduplicated in an LDS hash table with linear probing that never wraps. Insertion is the
 // phase-concurrent, history-independent kind: of two ids that want the same entry the one with the
@@ -447,8 +724,10 @@ plan_bucket_kernel(BucketArgs a) {
   __shared__ int64_t l_key[kTabAll + 1];
   __shared__ int32_t l_cnt[kTabAll + 1];  // occurrences of the entry; after ranking: its next free list position
   __shared__ int32_t l_u[kTabAll + 1];    // rank of the entry among the distinct ids of the round
+  __shared__ uint16_t l_ent[kTabAll + 1]; // the entry of every rank
   __shared__ unsigned long long s_wave[kBucketBlock / kWave];
   __shared__ int s_overflow;
+  __shared__ int s_claimed;  // entries of the table that the current build has taken
   const int tid = threadIdx.x;
   const int nb_log2 = a.g.nb_log2;
   // Buckets are taken in the order of the workgroup index. The look-back below waits for the
@@ -457,12 +736,20 @@ plan_bucket_kernel(BucketArgs a) {
   // a global counter would say the same, but a thousand atomics on one word are served one after
   // the other (25 ns each on this part: the last workgroup would start 25 us late).
   const int b = blockIdx.x;
-  const int32_t r_lo = a.bucket_start[b], r_hi = a.bucket_start[b + 1];
+  const int n_heavy = *a.heavy_n;
+  if (b == (1 << nb_log2)) {  // the workgroup after the last bucket's: the heavy ids
+    heavy_rows<PROBE>(a, n_heavy, s_wave);
+    return;
+  }
+  const int32_t r_lo = a.bucket_start[kHeavyMax + b], r_hi = a.bucket_start[kHeavyMax + b + 1];
   for (int e = tid; e <= kTabAll; e += kBucketBlock) {
     l_key[e] = kSetEmpty;
     l_cnt[e] = 0;
   }
-  if (tid == 0) s_overflow = 0;
+  if (tid == 0) {
+    s_overflow = 0;
+    s_claimed = 0;
+  }
   __syncthreads();
   int e_reg[kRegs];  // table entry of the thread's first kRegs records (-2: none / not of this round)
   int32_t pos_reg[kRegs];
@@ -472,10 +759,14 @@ plan_bucket_kernel(BucketArgs a) {
     pos_reg[x] = 0;
   }
 
-  // enters `key` into the table; false when the table cannot take it
+  // enters `key` into the table; false when the table cannot take it. Every distinct id takes
+  // exactly one empty entry, whoever ends up there: `claimed` counts the entries this thread took.
+  int claimed = 0;
   auto insert = [&](int64_t key, uint64_t mixed) -> bool {
     if (key == kSetEmpty) {
-      l_key[kSpecial] = 0;  // every writer stores the same word
+      if (atomicExch(reinterpret_cast<unsigned long long*>(&l_key[kSpecial]), 0ull) ==
+          static_cast<unsigned long long>(kSetEmpty))
+        ++claimed;
       return true;
     }
     unsigned long long v = static_cast<unsigned long long>(key);
@@ -488,7 +779,10 @@ plan_bucket_kernel(BucketArgs a) {
         continue;
       }
       if (atomicCAS(reinterpret_cast<unsigned long long*>(&l_key[e]), c, v) != c) continue;  // it changed: look again
-      if (c == static_cast<unsigned long long>(kSetEmpty)) return true;
+      if (c == static_cast<unsigned long long>(kSetEmpty)) {
+        ++claimed;
+        return true;
+      }
       v = c;  // the id that sat here moves on
       if (++e >= kTabAll - 1) return false;
     }
@@ -504,8 +798,11 @@ plan_bucket_kernel(BucketArgs a) {
   // the table of one round (cleared by the caller): every id of the round entered (pass 1), its
   // occurrences counted (pass 2). The bucket's records are taken kRegs per thread at a time, all
   // loads of a turn in flight together; for the first turn the table entry stays in e_reg.
-  auto build = [&](uint32_t rounds, uint32_t round) {
+  // `announce`: publish the number of distinct ids for the later buckets as soon as it is known
+  // (after the first pass; the ranking and the lists of this bucket are still to come)
+  auto build = [&](uint32_t rounds, uint32_t round, bool announce) {
     bool ok = true;
+    claimed = 0;
     for (int32_t q0 = r_lo; q0 < r_hi; q0 += kRegs * kBucketBlock) {
       int64_t k[kRegs];
 #pragma unroll
@@ -528,8 +825,16 @@ plan_bucket_kernel(BucketArgs a) {
       }
     }
     if (!ok) s_overflow = 1;
+    if (announce) {
+#pragma unroll
+      for (int o = kWave / 2; o > 0; o >>= 1) claimed += __shfl_xor(claimed, o, kWave);
+      if ((tid & (kWave - 1)) == 0 && claimed) atomicAdd(&s_claimed, claimed);
+    }
     __syncthreads();
     if (s_overflow) return;
+    if (announce && tid == 0)
+      __hip_atomic_store(&a.agg[b], kAggFlag | static_cast<unsigned long long>(s_claimed), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
     for (int32_t q0 = r_lo; q0 < r_hi; q0 += kRegs * kBucketBlock) {
       const bool first_turn = q0 == r_lo;
       int64_t k[kRegs];
@@ -566,7 +871,7 @@ plan_bucket_kernel(BucketArgs a) {
   };
 
   uint32_t rounds = 1;
-  build(1, 0);
+  build(1, 0, true);
   while (s_overflow) {  // dry runs: double the rounds until every round fits
     if (rounds >= (1u << 16)) {
       if (tid == 0) raise_device_error(a.err, RECIS_DEVERR_PLAN_OVERFLOW);
@@ -576,156 +881,95 @@ plan_bucket_kernel(BucketArgs a) {
     bool fits = true;
     for (uint32_t r = 0; r < rounds && fits; ++r) {
       clear();
-      build(rounds, r);
+      build(rounds, r, false);
       fits = !s_overflow;
     }
     if (fits) {
       clear();
-      build(rounds, 0);
+      build(rounds, 0, false);
       break;
     }
   }
 
   int64_t u_base = 0;  // distinct ids of all earlier buckets
   // the rare case: learn the base first, publish the total after the last round
-  if (rounds > 1) u_base = look_back(a.agg, b, a.spin_limit, a.err, s_wave);
+  if (rounds > 1) u_base = look_back(a.agg, b, n_heavy, a.spin_limit, a.err, s_wave);
   const int32_t l_base = r_lo;  // the bucket's occurrences are its list entries
   int32_t u_done = 0, l_done = 0, new_done = 0;
   const int s_lo = tid * kPer;
+  // The inverse holds unique indices, so with it the base must be known before the occurrences are
+  // placed. Without it the placing (bucket-local) comes first and the look-back after: by then the
+  // earlier buckets have published, and nobody waits.
+  const bool base_first = a.inverse != nullptr;
+  constexpr int kBatch = 2;  // unique ids of a thread whose id-map probes are in flight together
 
   for (uint32_t round = 0; round < rounds; ++round) {
     if (round > 0) {
       clear();
-      build(rounds, round);
+      build(rounds, round, false);
     }
     // ---- rank the entries this thread owns: position in the table = order of the unique ids
-    int32_t cnt[kPer];
-    unsigned long long mine = 0;
+    int32_t n_ent, n_occ;
+    {
+      int32_t cnt[kPer];
+      unsigned long long mine = 0;
 #pragma unroll
-    for (int x = 0; x < kPer; ++x) {
-      const int e = s_lo + x;
-      const bool occ = e <= kTabAll && l_key[e] != kSetEmpty;
-      cnt[x] = occ ? l_cnt[e] : -1;  // -1: not occupied
-      if (occ) mine += (static_cast<unsigned long long>(cnt[x]) << 32) | 1ull;
-    }
-    unsigned long long total;
-    unsigned long long run = block_scan_u64(mine, s_wave, total);
-    const int32_t n_ent = static_cast<int32_t>(total & 0xffffffffull);
-    const int32_t n_occ = static_cast<int32_t>(total >> 32);
-    // the later buckets can go on as soon as they know how many unique ids this one has
-    if (rounds == 1 && tid == 0)
-      __hip_atomic_store(&a.agg[b], kAggFlag | static_cast<unsigned long long>(n_ent), __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_AGENT);
+      for (int x = 0; x < kPer; ++x) {
+        const int e = s_lo + x;
+        const bool occ = e <= kTabAll && l_key[e] != kSetEmpty;
+        cnt[x] = occ ? l_cnt[e] : -1;  // -1: not occupied
+        if (occ) mine += (static_cast<unsigned long long>(cnt[x]) << 32) | 1ull;
+      }
+      unsigned long long total;
+      unsigned long long run = block_scan_u64(mine, s_wave, total);
+      n_ent = static_cast<int32_t>(total & 0xffffffffull);
+      n_occ = static_cast<int32_t>(total >> 32);
+      // (with one round the later buckets know n_ent already: build announced it)
 #pragma unroll
-    for (int x = 0; x < kPer; ++x) {
-      if (cnt[x] < 0) continue;
-      l_u[s_lo + x] = static_cast<int32_t>(run & 0xffffffffull);
-      l_cnt[s_lo + x] = static_cast<int32_t>(run >> 32);  // only its owner has read the count
-      run += (static_cast<unsigned long long>(cnt[x]) << 32) | 1ull;
+      for (int x = 0; x < kPer; ++x) {
+        if (cnt[x] < 0) continue;
+        const int32_t rank = static_cast<int32_t>(run & 0xffffffffull);
+        l_u[s_lo + x] = rank;
+        l_ent[rank] = static_cast<uint16_t>(s_lo + x);
+        l_cnt[s_lo + x] = static_cast<int32_t>(run >> 32);  // the start of its list; only its owner has read the count
+        run += (static_cast<unsigned long long>(cnt[x]) << 32) | 1ull;
+      }
     }
+    __syncthreads();
+
+    // ---- the unique ids are shared out by rank, a stretch of consecutive ranks per thread; the
+    // probes of the id map for the first kBatch of them start now and land while the lists are made
+    const int per = (n_ent + kBucketBlock - 1) / kBucketBlock;
+    const int rk_lo = min(n_ent, tid * per), rk_hi = min(n_ent, rk_lo + per);
+    longlong2 hint[kBatch];  // all that stays in registers meanwhile: the home slots as they were read
+    auto key_of_rank = [&](int r, int* e) -> int64_t {
+      *e = l_ent[r];
+      return *e == kSpecial ? kSetEmpty : l_key[*e];
+    };
+    auto fetch = [&](int r_first) {
+#pragma unroll
+      for (int y = 0; y < kBatch; ++y) {
+        hint[y] = make_longlong2(0, 0);
+        if constexpr (PROBE) {
+          if (r_first + y < rk_hi) {
+            int e;
+            const int64_t key = key_of_rank(r_first + y, &e);
+            if (key != kEmpty && key != kTomb)
+              hint[y] = *reinterpret_cast<const longlong2*>(&a.table[home_slot(key, a.mask)]);
+          }
+        }
+      }
+    };
+    fetch(rk_lo);
 
     // ---- where this bucket's unique ids start
-    if (rounds == 1) {
-      u_base = look_back(a.agg, b, a.spin_limit, a.err, s_wave);
+    auto learn_base = [&]() {
+      u_base = look_back(a.agg, b, n_heavy, a.spin_limit, a.err, s_wave);
       if (tid == 0)
         __hip_atomic_store(&a.agg[b], kPrefixFlag | static_cast<unsigned long long>(u_base + n_ent), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
-    }
-
-    // ---- per unique id: the id, the start of its list, hot work items, its row in the id map
-    int32_t my_new = 0, my_empty = 0;
-#pragma unroll
-    for (int x0 = 0; x0 < kPer; x0 += 3) {  // three probes of the id map in flight
-      int64_t key[3];
-      uint64_t home[3];
-      longlong2 hint[3];
-#pragma unroll
-      for (int y = 0; y < 3; ++y) {
-        const int x = x0 + y, e = s_lo + x;
-        key[y] = cnt[x] >= 0 ? (e == kSpecial ? kSetEmpty : l_key[e]) : kSetEmpty;
-        if constexpr (PROBE) {
-          home[y] = 0;
-          hint[y] = make_longlong2(0, 0);
-          if (cnt[x] >= 0 && key[y] != kEmpty && key[y] != kTomb) {
-            home[y] = home_slot(key[y], a.mask);
-            hint[y] = *reinterpret_cast<const longlong2*>(&a.table[home[y]]);
-          }
-        }
-      }
-#pragma unroll
-      for (int y = 0; y < 3; ++y) {
-        const int x = x0 + y, e = s_lo + x;
-        if (cnt[x] < 0) continue;
-        const int64_t u = u_base + u_done + l_u[e];
-        if (u < 0 || u >= a.g.n) {
-          raise_device_error(a.err, RECIS_DEVERR_PLAN_OVERFLOW);  // cannot happen; never store out of bounds
-          continue;
-        }
-        a.unique_out[u] = key[y];
-        a.row_start[u] = l_base + l_done + l_cnt[e];
-        if (a.hot_cap > 0 && cnt[x] > kHotLen) {
-          const int n_items = (cnt[x] + kHotChunk - 1) / kHotChunk;
-          const int64_t base = static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&a.counts[1]),
-                                                              static_cast<unsigned long long>(n_items)));
-          for (int c = 0; c < n_items; ++c) {
-            if (base + c < a.hot_cap) {
-              a.hot_items[2 * (base + c)] = static_cast<int32_t>(u);
-              a.hot_items[2 * (base + c) + 1] = c;
-            }
-          }
-        }
-        if constexpr (PROBE) {
-          int64_t row = -1;  // what index_out gets; a claimed slot travels as -(slot + 2) until rows are assigned
-          if (key[y] == kEmpty || key[y] == kTomb) {
-            raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);  // the map's reserved keys
-          } else {
-            int64_t value = -1, slot = -1;
-            bool took_empty = false;
-            switch (probe_or_claim(a.table, a.mask, key[y], home[y], hint[y], -2, &value, &slot, &took_empty)) {
-              case kProbeFound:
-                row = value;
-                break;
-              case kProbeClaimed:
-                row = -(slot + 2);
-                ++my_new;
-                my_empty += took_empty ? 1 : 0;
-                break;
-              default:  // no slot left, or the key is being inserted by a concurrent call (not allowed)
-                raise_device_error(a.err, RECIS_DEVERR_TABLE_FULL);
-                break;
-            }
-          }
-          a.index_out[u] = row;
-        }
-      }
-    }
-    // ---- new keys: listed per bucket in the order of the unique ids, for the row assignment
-    int32_t n_new = 0;
-    if constexpr (PROBE) {
-      unsigned long long new_total;
-      const unsigned long long new_before = block_scan_u64(
-          (static_cast<unsigned long long>(my_empty) << 32) | static_cast<unsigned long long>(my_new), s_wave,
-          new_total);
-      n_new = static_cast<int32_t>(new_total & 0xffffffffull);
-      if (tid == 0 && (new_total >> 32) != 0)
-        atomicAdd(reinterpret_cast<unsigned long long*>(&a.state[ST_OCC]), new_total >> 32);
-      if (my_new > 0) {
-        int32_t at = l_base + new_done + static_cast<int32_t>(new_before & 0xffffffffull);
-#pragma unroll
-        for (int x = 0; x < kPer; ++x) {
-          if (cnt[x] < 0) continue;
-          NewRec nr;
-          nr.u = u_base + u_done + l_u[s_lo + x];
-          if (nr.u < 0 || nr.u >= a.g.n) continue;  // flagged above
-          const int64_t row = a.index_out[nr.u];    // written by this thread above
-          if (row >= -1) continue;
-          nr.slot = -(row + 2);
-          if (at >= r_hi) continue;  // cannot happen: a bucket has no more new keys than records
-          a.new_list[at++] = nr;
-        }
-      }
-    }
-    __syncthreads();  // the list starts have been read; ranks and starts of all entries are in place
+    };
+    if (rounds == 1 && base_first) learn_base();
 
     // ---- per occurrence: its place in the list of its id, its unique index
     auto place = [&](int e, int32_t pos) {  // every lane of the wave calls; e < 0: nothing to place
@@ -761,25 +1005,105 @@ plan_bucket_kernel(BucketArgs a) {
         place(e, pos[x]);
       }
     }
+    __syncthreads();  // every entry's l_cnt now holds the END of its list
+    if (rounds == 1 && !base_first) learn_base();
+
+    // ---- per unique id: the id, the start of its list, hot work items, its row in the id map
+    int32_t my_new = 0, my_empty = 0;
+    for (int rb = rk_lo; rb < rk_hi; rb += kBatch) {
+      if (rb != rk_lo) fetch(rb);
+#pragma unroll
+      for (int y = 0; y < kBatch; ++y) {
+        const int r = rb + y;
+        if (r >= rk_hi) continue;
+        int e;
+        const int64_t key = key_of_rank(r, &e);
+        const int64_t u = u_base + u_done + r;
+        if (u < 0 || u >= a.g.n) {
+          raise_device_error(a.err, RECIS_DEVERR_PLAN_OVERFLOW);  // cannot happen; never store out of bounds
+          continue;
+        }
+        const int32_t start = r == 0 ? 0 : l_cnt[l_ent[r - 1]], n_here = l_cnt[e] - start;
+        a.unique_out[u] = key;
+        a.row_start[u] = l_base + l_done + start;
+        if (a.hot_cap > 0 && n_here > kHotLen) {
+          const int n_items = (n_here + kHotChunk - 1) / kHotChunk;
+          const int64_t base = static_cast<int64_t>(atomicAdd(reinterpret_cast<unsigned long long*>(&a.counts[1]),
+                                                              static_cast<unsigned long long>(n_items)));
+          for (int c = 0; c < n_items; ++c) {
+            if (base + c < a.hot_cap) {
+              a.hot_items[2 * (base + c)] = static_cast<int32_t>(u);
+              a.hot_items[2 * (base + c) + 1] = c;
+            }
+          }
+        }
+        if constexpr (PROBE) {
+          int64_t row = -1;  // what index_out gets; a claimed slot travels as -(slot + 2) until rows are assigned
+          if (key == kEmpty || key == kTomb) {
+            raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);  // the map's reserved keys
+          } else {
+            int64_t value = -1, slot = -1;
+            bool took_empty = false;
+            switch (probe_or_claim(a.table, a.mask, key, home_slot(key, a.mask), hint[y], -2, &value, &slot, &took_empty)) {
+              case kProbeFound:
+                row = value;
+                break;
+              case kProbeClaimed:
+                row = -(slot + 2);
+                ++my_new;
+                my_empty += took_empty ? 1 : 0;
+                break;
+              default:  // no slot left, or the key is being inserted by a concurrent call (not allowed)
+                raise_device_error(a.err, RECIS_DEVERR_TABLE_FULL);
+                break;
+            }
+          }
+          a.index_out[u] = row;
+        }
+      }
+    }
+    // ---- new keys: listed per bucket in the order of the unique ids, for the row assignment
+    int32_t n_new = 0;
+    if constexpr (PROBE) {
+      unsigned long long new_total;
+      const unsigned long long new_before = block_scan_u64(
+          (static_cast<unsigned long long>(my_empty) << 32) | static_cast<unsigned long long>(my_new), s_wave,
+          new_total);
+      n_new = static_cast<int32_t>(new_total & 0xffffffffull);
+      if (tid == 0 && (new_total >> 32) != 0)
+        atomicAdd(reinterpret_cast<unsigned long long*>(&a.state[ST_OCC]), new_total >> 32);
+      if (my_new > 0) {
+        int32_t at = l_base + new_done + static_cast<int32_t>(new_before & 0xffffffffull);
+        for (int r = rk_lo; r < rk_hi; ++r) {
+          NewRec nr;
+          nr.u = u_base + u_done + r;
+          if (nr.u < 0 || nr.u >= a.g.n) continue;  // flagged above
+          const int64_t row = a.index_out[nr.u];    // written by this thread above
+          if (row >= -1) continue;
+          nr.slot = -(row + 2);
+          if (at >= r_hi) continue;  // cannot happen: a bucket has no more new keys than records
+          a.new_list[at++] = nr;
+        }
+      }
+    }
     u_done += n_ent;
     l_done += n_occ;
     new_done += n_new;
   }
 
+  __syncthreads();
   if (tid == 0) {
     if (rounds > 1)
       __hip_atomic_store(&a.agg[b], kPrefixFlag | static_cast<unsigned long long>(u_base + u_done), __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
-    if constexpr (PROBE) a.new_count[b] = new_done;
+    if constexpr (PROBE) a.new_count[1 + b] = new_done;
     if (b == (1 << nb_log2) - 1) {  // the last bucket knows the total
       const int64_t U = u_base + u_done;
-      a.counts[0] = U;
+      __hip_atomic_store(&a.counts[0], U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       a.row_start[U] = static_cast<int32_t>(a.g.n);
-      if (a.staged) {  // pinned host words: no copy kernel needed
-        a.staged[1] = __hip_atomic_load(a.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        a.staged[0] = U;
-      }
     }
+    // (the barrier above this block orders the raises of this workgroup's threads before the ticket)
+    if (a.staged) finish_ticket(a);
   }
 }
 
@@ -794,13 +1118,14 @@ plan_assign_new_kernel(Slot* __restrict__ table, const NewRec* __restrict__ new_
                        int64_t* __restrict__ state, volatile int64_t* mirror, int64_t seq,
                        const int64_t* __restrict__ free_list, int64_t* __restrict__ index_out,
                        int32_t* __restrict__ sync) {
+  // nb here = 1 + buckets: the new keys among the heavy ids, then those of every bucket
   extern __shared__ int32_t first_new[];  // [nb + 1], then kPartBlock words of scan scratch
   scan_counts(new_count, nb, first_new, first_new + nb + 1);
   const int64_t n_new = first_new[nb];
   const int64_t old_cur = state[ST_CUR], old_free = state[ST_FREE];
   for (int b = blockIdx.x; b < nb && n_new > 0; b += gridDim.x) {
     const int32_t cnt = new_count[b];
-    const NewRec* mine = new_list + bucket_start[b];
+    const NewRec* mine = new_list + (b == 0 ? bucket_start[0] : bucket_start[kHeavyMax + b - 1]);
     for (int k = threadIdx.x; k < cnt; k += kPartBlock) {
       const NewRec r = mine[k];
       const int64_t row = row_of_new_key(first_new[b] + k, n_new, old_cur, old_free, free_list);
@@ -886,6 +1211,42 @@ struct CsrArgs {
   const void* part_rows[kMaxParts];
   int64_t part_lo[kMaxParts + 1];
 };
+
+// What a gather-reduce launch does with the finished sum of row u (template parameter EPI):
+//   kEpiStore    out[u] (+)= sum
+//   kEpiAdam     the sum is the gradient of table row row_index[u]: the Adam-family update of that
+//                row (parameter and both moments) is applied at once, the gradient never written
+//   kEpiAdagrad  the same with the Adagrad update
+enum { kEpiStore = 0, kEpiAdam = 1, kEpiAdagrad = 2 };
+struct FuseArgs {
+  const int64_t* row_index;  // [U]; a negative index skips the row
+  void* const* emb;          // block tables (device arrays of block pointers)
+  void* const* s0;           // exp_avg / the Adagrad accumulator
+  void* const* s1;           // exp_avg_sq
+  RowBlocks rb;
+  AdamCoef adam;
+  float lr, eps;             // Adagrad
+};
+
+// The epilogue of one pack of one finished row; T = the table's row type for the optimizer kinds.
+template <typename T, int VEC, int EPI>
+__device__ __forceinline__ void fused_row_update(const FuseArgs& f, int* err, int64_t u, int c0,
+                                                 const float (&acc)[VEC]) {
+  int64_t b, off;
+  const int64_t idx = f.row_index[u];
+  if (idx < 0) return;  // a key the table does not hold takes no gradient
+  if (!block_row(f.rb, idx, b, off)) {
+    raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+    return;
+  }
+  const int64_t at = off * f.rb.D + c0;
+  if constexpr (EPI == kEpiAdam) {
+    adam_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at,
+                             static_cast<T*>(f.s1[b]) + at, acc, f.adam.alpha[0], f.adam);
+  } else {
+    adagrad_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at, acc, f.lr, f.eps);
+  }
+}
 
 // Row s of the input: of the one array, or of the part that holds it.
 template <typename TIn, bool PARTS>
@@ -985,9 +1346,9 @@ constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of
 // the partial rows of every hot row in chunk order. No atomics anywhere.
 // SHUFFLE: long lists go through wave_gather_range (pays off when a wave has at most eight lane
 // groups, i.e. rows of 128 bytes and more); otherwise every group loads its own entries.
-template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false>
-__global__ void __launch_bounds__(kBlock)
-csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a) {
+template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false, int EPI = kEpiStore>
+__global__ void __launch_bounds__(kBlock, (!SHUFFLE && EPI != kEpiStore) ? 8 : 1)  // 64 registers where that costs no spills
+csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
   extern __shared__ float s_part[];  // [waves][D], hot part only
   const int D = a.D;
   const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
@@ -1099,18 +1460,25 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
   const bool hot = end - start > a.hot_len;  // left to the work items and the finish kernel
   if (hot) end = start;
   auto finish = [&](int64_t row, int c0, float (&acc)[VEC]) {
-    TOut* dst = out + row * D + c0;
-    if (a.accumulate) {
-      float old[VEC];
-      load_pack<TOut, VEC>(dst, old);
+    if constexpr (EPI != kEpiStore) {
+      fused_row_update<TOut, VEC, EPI>(f, a.err, row, c0, acc);
+    } else {
+      TOut* dst = out + row * D + c0;
+      if (a.accumulate) {
+        float old[VEC];
+        load_pack<TOut, VEC>(dst, old);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] += old[j];
+        for (int j = 0; j < VEC; ++j) acc[j] += old[j];
+      }
+      store_pack<TOut, VEC>(dst, acc);
     }
-    store_pack<TOut, VEC>(dst, acc);
   };
   // short rows: every lane group works its own row
   const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;  // with one group per wave there is nobody to share with
   if (valid && !is_long && !hot) {
+    // (Asking for the row's parameter and state packs before the gradient is gathered, to run their
+    // latency under that of the gathers, was measured and lost: 150 -> 205 us in config 4. The packs
+    // cost registers, hence resident waves, and the gathers then queue behind the table reads.)
     for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
       float acc[VEC];
 #pragma unroll
@@ -1139,9 +1507,9 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a)
 
 // out[u] (+)= sum of the partial rows of hot row u, in chunk order. One lane group per work item
 // with chunk 0 (the items of a row are consecutive).
-template <typename TOut, int VEC>
+template <typename TOut, int VEC, int EPI = kEpiStore>
 __global__ void __launch_bounds__(kBlock)
-csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a) {
+csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
   int64_t n_items = a.counts[1];
   if (n_items > a.hot_cap) n_items = a.hot_cap;
   const int D = a.D;
@@ -1164,14 +1532,18 @@ csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[j] += v[j];
       }
-      TOut* dst = out + static_cast<int64_t>(u) * D + c0;
-      if (a.accumulate) {
-        float old[VEC];
-        load_pack<TOut, VEC>(dst, old);
+      if constexpr (EPI != kEpiStore) {
+        fused_row_update<TOut, VEC, EPI>(f, a.err, u, c0, acc);
+      } else {
+        TOut* dst = out + static_cast<int64_t>(u) * D + c0;
+        if (a.accumulate) {
+          float old[VEC];
+          load_pack<TOut, VEC>(dst, old);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += old[j];
+          for (int j = 0; j < VEC; ++j) acc[j] += old[j];
+        }
+        store_pack<TOut, VEC>(dst, acc);
       }
-      store_pack<TOut, VEC>(dst, acc);
     }
   }
 }
@@ -1389,7 +1761,7 @@ extern "C" {
 struct PlanLayout {
   PlanGeom g;
   int64_t nb;
-  size_t o_hist, o_total, o_start, o_agg, o_newc, o_sync, o_id, o_pos, o_new, bytes;
+  size_t o_hist, o_total, o_start, o_agg, o_newc, o_sync, o_heavy, o_id, o_pos, o_new, bytes;
 };
 
 static PlanLayout plan_layout(int64_t n, bool with_lookup) {
@@ -1403,20 +1775,23 @@ static PlanLayout plan_layout(int64_t n, bool with_lookup) {
   while ((int64_t(1) << nb_log2) < kMaxBuckets && (int64_t(1) << nb_log2) * kBucketIds < n) ++nb_log2;
   g.nb_log2 = nb_log2;
   L.nb = int64_t(1) << nb_log2;
-  // hist[rows * nb] (counts, then offsets, in place) | bucket_total[nb] | bucket_start[nb + 1] |
-  // agg[nb] look-back words | new_count[nb] | sync[4] | bkt_id[n] | bkt_pos[n] | new_list[n] (fused lookup only)
+  // hist[rows * columns] (counts, then offsets, in place) | bucket_total[columns] | bucket_start[columns + 1] |
+  // agg[nb] look-back words | new_count[1 + nb] | sync[4] | heavy ids | bkt_id[n] | bkt_pos[n] |
+  // new_list[n] (fused lookup only)
   size_t bytes = 0;
   auto take = [&](size_t b) {
     const size_t at = bytes;
     bytes += (b + 255) & ~size_t(255);
     return at;
   };
-  L.o_hist = take(sizeof(int32_t) * g.rows * L.nb);
-  L.o_total = take(sizeof(int32_t) * L.nb);
-  L.o_start = take(sizeof(int32_t) * (L.nb + 1));
+  const int64_t nc = kHeavyMax + L.nb;  // columns of the partition: the heavy ids, then the buckets
+  L.o_hist = take(sizeof(int32_t) * g.rows * nc);
+  L.o_total = take(sizeof(int32_t) * nc);
+  L.o_start = take(sizeof(int32_t) * (nc + 1));
   L.o_agg = take(sizeof(unsigned long long) * L.nb);
-  L.o_newc = take(sizeof(int32_t) * L.nb);
+  L.o_newc = take(sizeof(int32_t) * (L.nb + 1));
   L.o_sync = take(sizeof(int32_t) * 4);
+  L.o_heavy = take(sizeof(int64_t) * kHeavyMax + sizeof(int32_t));  // heavy_ids[kHeavyMax], heavy_n
   L.o_id = take(sizeof(int64_t) * n);
   L.o_pos = take(sizeof(int32_t) * n);
   L.o_new = with_lookup ? take(sizeof(NewRec) * n) : bytes;
@@ -1456,32 +1831,49 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int6
   int32_t* sync = reinterpret_cast<int32_t*>(base + L.o_sync);
   int64_t* bkt_id = reinterpret_cast<int64_t*>(base + L.o_id);
   int32_t* bkt_pos = reinterpret_cast<int32_t*>(base + L.o_pos);
-  const size_t lds = sizeof(int32_t) * static_cast<size_t>(nb);
+  const int64_t nc = kHeavyMax + nb;
+  const size_t lds = sizeof(int32_t) * static_cast<size_t>(nc);
+  int64_t* heavy_ids = reinterpret_cast<int64_t*>(base + L.o_heavy);
+  int32_t* heavy_n = reinterpret_cast<int32_t*>(heavy_ids + kHeavyMax);
+  HeavyArgs hv;
+  hv.ids = heavy_ids;
+  hv.n = heavy_n;
+  hv.list = list_out;
+  hv.inverse = inverse_out;
+  hv.pos_out = pos_out;
+  {
+    RECIS_TIME_KERNEL("plan_heavy_kernel", stream)
+    plan_heavy_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, g.n, heavy_ids, heavy_n);
+    RECIS_LAUNCH_CHECK();
+  }
   {
     RECIS_TIME_KERNEL("plan_hist_kernel", stream)
-    plan_hist_kernel<<<dim3(g.rows), dim3(kPartBlock), lds, stream>>>(ids, g, hist, counts_out_dev, sync);
+    plan_hist_kernel<<<dim3(g.rows), dim3(kPartBlock), lds, stream>>>(ids, g, heavy_ids, heavy_n, hist, counts_out_dev,
+                                                                      sync);
     RECIS_LAUNCH_CHECK();
   }
   {
     RECIS_TIME_KERNEL("plan_colscan_kernel", stream)
-    plan_colscan_kernel<<<dim3(nb / kColBuckets), dim3(1024), 0, stream>>>(hist, g, bucket_total);
+    plan_colscan_kernel<<<dim3(nc / kColBuckets), dim3(1024), 0, stream>>>(hist, g, bucket_total);
     RECIS_LAUNCH_CHECK();
   }
   {
     RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
     if (g.tile <= kTile && g.tile >= 4 * nb)  // a tile sends four ids or more to a bucket: worth ordering them
       plan_scatter_runs_kernel<<<dim3(g.rows), dim3(kPartBlock),
-                                 sizeof(int32_t) * (2 * (nb + 1) + kPartBlock) + 2 * sizeof(uint16_t) * kTile, stream>>>(
-          ids, g, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
+                                 sizeof(int32_t) * (2 * (nc + 1) + kPartBlock) + 2 * sizeof(uint16_t) * kTile, stream>>>(
+          ids, g, hv, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
     else
       plan_scatter_kernel<<<dim3(g.rows), dim3(kPartBlock), lds + sizeof(int32_t) * (kPartBlock + 1), stream>>>(
-          ids, g, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
+          ids, g, hv, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
     RECIS_LAUNCH_CHECK();
   }
   BucketArgs a;
   a.bkt_id = bkt_id;
   a.bkt_pos = bkt_pos;
   a.bucket_start = bucket_start;
+  a.heavy_ids = heavy_ids;
+  a.heavy_n = heavy_n;
   a.g = g;
   a.agg = agg;
   a.new_count = reinterpret_cast<int32_t*>(base + L.o_newc);
@@ -1511,17 +1903,17 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int6
     a.mirror = map->mirror;
     {
       RECIS_TIME_KERNEL("plan_bucket_kernel", stream)
-      plan_bucket_kernel<true><<<dim3(nb), dim3(kBucketBlock), 0, stream>>>(a);
+      plan_bucket_kernel<true><<<dim3(nb + 1), dim3(kBucketBlock), 0, stream>>>(a);
       RECIS_LAUNCH_CHECK();
     }
     plan_assign_new_kernel<<<dim3(std::max<int64_t>(nb / 4, 1)), dim3(kPartBlock),
-                             lds + sizeof(int32_t) * (kPartBlock + 1), stream>>>(
-        map->table, a.new_list, bucket_start, a.new_count, static_cast<int>(nb), map->state, map->mirror, map_seq,
+                             sizeof(int32_t) * (nb + 2 + kPartBlock + 1), stream>>>(
+        map->table, a.new_list, bucket_start, a.new_count, static_cast<int>(nb + 1), map->state, map->mirror, map_seq,
         map->free_list, index_out, sync);
     RECIS_LAUNCH_CHECK();
   } else {
     RECIS_TIME_KERNEL("plan_bucket_kernel", stream)
-    plan_bucket_kernel<false><<<dim3(nb), dim3(kBucketBlock), 0, stream>>>(a);
+    plan_bucket_kernel<false><<<dim3(nb + 1), dim3(kBucketBlock), 0, stream>>>(a);
     RECIS_LAUNCH_CHECK();
   }
   if (staged) RECIS_CHECK_HIP(hipEventRecord(staged_event, stream));
@@ -1717,7 +2109,8 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
                                   int coef_dtype, const int32_t* row_start, const int32_t* hot_items,
                                   int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
                                   int64_t D, int accumulate, const void* cover_offsets, int cover_is64,
-                                  int64_t cover_S, hipStream_t stream);
+                                  int64_t cover_S, hipStream_t stream, int epi = kEpiStore,
+                                  const FuseArgs* fuse = nullptr, size_t extra_ws = 0, void** extra_out = nullptr);
 
 int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
                             int coef_dtype, const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
@@ -1750,11 +2143,14 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
                                   int coef_dtype, const int32_t* row_start, const int32_t* hot_items,
                                   int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
                                   int64_t D, int accumulate, const void* cover_offsets, int cover_is64,
-                                  int64_t cover_S, hipStream_t stream) {
+                                  int64_t cover_S, hipStream_t stream, int epi, const FuseArgs* fuse,
+                                  size_t extra_ws, void** extra_out) {
+  // epi != kEpiStore: `out` is NULL, out_dtype is the table's row type and *fuse says where the rows
+  // are. extra_ws bytes of the stream's workspace (after the partial rows of the hot items) are
+  // handed to the caller in *extra_out before anything is launched.
   RECIS_REQUIRE(U >= 0 && n_rows >= 0, "negative size");
   RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
-  if (U == 0) return RECIS_OK;
-  RECIS_REQUIRE(src && row_start && out && counts_dev, "NULL argument");
+  RECIS_REQUIRE(U == 0 || (src && row_start && (out || epi != kEpiStore) && counts_dev), "NULL argument");
   RECIS_REQUIRE(n_parts > 0 || rows != nullptr || n_rows == 0, "rows must not be NULL");
   RECIS_REQUIRE(hot_cap == 0 || hot_items, "hot_items must not be NULL");
   const int in_sz = dtype_size(rows_dtype), out_sz = dtype_size(out_dtype);
@@ -1763,7 +2159,9 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
   uintptr_t align_of = reinterpret_cast<uintptr_t>(rows);
   for (int f = 0; f < n_parts; ++f) align_of |= reinterpret_cast<uintptr_t>(part_rows[f]);  // the coarsest alignment
   const int vb_in = pick_vec_bytes(D * in_sz, align_of);
-  const int vb_out = pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
+  // table blocks are allocator-aligned and are read and written in 16-byte packs at most
+  const int vb_out = epi != kEpiStore ? pick_vec_bytes(D * out_sz, 16)
+                                      : pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
   const int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
   CsrArgs a;
   a.row_start = row_start;
@@ -1795,13 +2193,16 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
     a.part_lo[f + 1] = a.part_lo[f] + (f < n_parts ? part_counts[f] : 0);
   }
   int64_t hot_blocks = 0;
-  if (hot_cap > 0) {
+  if (hot_cap > 0 || extra_ws > 0) {
     void* ws = nullptr;
-    if (int rc = get_workspace(stream, sizeof(float) * static_cast<size_t>(hot_cap) * static_cast<size_t>(D), &ws))
-      return rc;
+    const size_t hot_bytes = (sizeof(float) * static_cast<size_t>(hot_cap) * static_cast<size_t>(D) + 255) & ~size_t(255);
+    if (int rc = get_workspace(stream, hot_bytes + extra_ws, &ws)) return rc;
     a.hot_part = static_cast<float*>(ws);
-    hot_blocks = std::min<int64_t>(hot_cap, 4096);
+    if (extra_out) *extra_out = static_cast<char*>(ws) + hot_bytes;
+    if (hot_cap > 0) hot_blocks = std::min<int64_t>(hot_cap, 4096);
   }
+  if (U == 0) return RECIS_OK;
+  const FuseArgs f = fuse ? *fuse : FuseArgs{};
   const size_t lds = sizeof(float) * (kBlock / kWave) * static_cast<size_t>(D);
   auto with_types = [&](auto tin, auto tout) {
     using TIn = decltype(tin);
@@ -1814,27 +2215,41 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
         const TIn* rin = static_cast<const TIn*>(rows);
         TOut* o = static_cast<TOut*>(out);
         const bool shuffle = a.lpr_log2 >= 3;  // at most eight lane groups per wave
-        {
-          RECIS_TIME_KERNEL("csr_rows_kernel", stream)
-          if (n_parts > 0) {
-            if constexpr (sizeof(TOut) == 4) {  // parts go to fp32 rows only
-              if (shuffle)
-                csr_rows_kernel<TIn, TOut, VEC, true, true><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
-              else
-                csr_rows_kernel<TIn, TOut, VEC, false, true><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
+        const dim3 grid(a.cold_blocks + hot_blocks), block(kBlock);
+        const int64_t fin = std::min<int64_t>((hot_cap + rows_per_block - 1) / rows_per_block, 1024);
+        auto launch = [&](auto epi_tag) {
+          constexpr int EPI = decltype(epi_tag)::value;
+          {
+            RECIS_TIME_KERNEL(EPI == kEpiStore ? "csr_rows_kernel" : EPI == kEpiAdam ? "csr_rows_adam_kernel"
+                                                                                      : "csr_rows_adagrad_kernel", stream)
+            if (n_parts > 0) {
+              if constexpr (sizeof(TOut) == 4 && EPI == kEpiStore) {  // parts go to fp32 rows only
+                if (shuffle)
+                  csr_rows_kernel<TIn, TOut, VEC, true, true><<<grid, block, lds, stream>>>(rin, o, a, f);
+                else
+                  csr_rows_kernel<TIn, TOut, VEC, false, true><<<grid, block, lds, stream>>>(rin, o, a, f);
+              }
+            } else if (shuffle) {
+              csr_rows_kernel<TIn, TOut, VEC, true, false, EPI><<<grid, block, lds, stream>>>(rin, o, a, f);
+            } else {
+              csr_rows_kernel<TIn, TOut, VEC, false, false, EPI><<<grid, block, lds, stream>>>(rin, o, a, f);
             }
-          } else if (shuffle)
-            csr_rows_kernel<TIn, TOut, VEC, true><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
-          else
-            csr_rows_kernel<TIn, TOut, VEC, false><<<dim3(a.cold_blocks + hot_blocks), dim3(kBlock), lds, stream>>>(rin, o, a);
-          RECIS_LAUNCH_CHECK();
+            RECIS_LAUNCH_CHECK();
+          }
+          if (hot_cap > 0) {
+            csr_hot_finish_kernel<TOut, VEC, EPI><<<dim3(fin), block, 0, stream>>>(o, a, f);
+            RECIS_LAUNCH_CHECK();
+          }
+          return RECIS_OK;
+        };
+        if (epi == kEpiAdam) {
+          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdam>{});
+        } else if (epi == kEpiAdagrad) {
+          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdagrad>{});
+        } else {
+          return launch(std::integral_constant<int, kEpiStore>{});
         }
-        if (hot_cap > 0) {
-          const int64_t fin = std::min<int64_t>((hot_cap + rows_per_block - 1) / rows_per_block, 1024);
-          csr_hot_finish_kernel<TOut, VEC><<<dim3(fin), dim3(kBlock), 0, stream>>>(o, a);
-          RECIS_LAUNCH_CHECK();
-        }
-        return RECIS_OK;
+        return fail(RECIS_ERR_ARG, "internal: vector too wide for a fused row update");
       }
     });
   };
@@ -1843,7 +2258,88 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
   if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F32) return with_types(f16_t{}, float{});
   if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_BF16) return with_types(bf16_t{}, bf16_t{});
   if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F16) return with_types(f16_t{}, f16_t{});
+  if (epi != kEpiStore) {  // fp32 gradients onto half-precision rows
+    if (rows_dtype == RECIS_F32 && out_dtype == RECIS_BF16) return with_types(float{}, bf16_t{});
+    if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F16) return with_types(float{}, f16_t{});
+  }
   return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
+}
+
+// Shared front of the two fused entry points: argument checks and the table description.
+static int fill_fuse_args(FuseArgs& f, const int64_t* row_index, void* const* emb, void* const* s0, void* const* s1,
+                          bool need_s1, int64_t n_blocks, int64_t block_size, int64_t D, int row_dtype) {
+  RECIS_REQUIRE(row_index && emb && s0 && (s1 || !need_s1), "row_index and the block tables must not be NULL");
+  RECIS_REQUIRE(n_blocks >= 1 && block_size >= 1, "bad block geometry (n_blocks=%lld block_size=%lld)",
+                (long long)n_blocks, (long long)block_size);
+  RECIS_REQUIRE(dtype_size(row_dtype), "invalid row dtype");
+  f = FuseArgs{};
+  f.row_index = row_index;
+  f.emb = emb;
+  f.s0 = s0;
+  f.s1 = s1;
+  f.rb.n_blocks = n_blocks;
+  f.rb.block_size = block_size;
+  f.rb.D = static_cast<int>(D);
+  return RECIS_OK;
+}
+
+int recis_csr_gather_reduce_adamw(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                  const void* coef, int coef_dtype, const int32_t* row_start,
+                                  const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
+                                  int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
+                                  const int64_t* row_index, void* const* emb_blocks_dev,
+                                  void* const* exp_avg_blocks_dev, void* const* exp_avg_sq_blocks_dev,
+                                  int64_t n_blocks, int64_t block_size, int row_dtype, void* beta1_t, void* beta2_t,
+                                  int beta_is_f64, double lr, double beta1, double beta2, double weight_decay,
+                                  double eps, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(beta1_t != nullptr && beta2_t != nullptr, "beta1_t / beta2_t must not be NULL");
+  FuseArgs f;
+  if (U > 0) {
+    if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, exp_avg_blocks_dev, exp_avg_sq_blocks_dev, true, n_blocks,
+                                block_size, D, row_dtype))
+      return rc;
+  } else {
+    f = FuseArgs{};
+  }
+  // the running powers advance even when no row is touched (cal_alpha runs first); alpha lives in
+  // the stream's workspace behind the partial rows of the hot items
+  void* alpha = nullptr;
+  // first pass: reserve the workspace and learn where alpha goes, launching nothing (U = 0)
+  if (int rc = csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
+                                      hot_items, hot_cap, counts_dev, nullptr, row_dtype, 0, D, 0, cover_offsets,
+                                      cover_is64, cover_S, stream, kEpiAdam, &f, 256, &alpha))
+    return rc;
+  if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, static_cast<double*>(alpha), lr, beta1, beta2, stream))
+    return rc;
+  if (U == 0) return RECIS_OK;
+  f.adam.alpha = static_cast<const double*>(alpha);
+  f.adam.beta1 = beta1;
+  f.adam.beta2 = beta2;
+  f.adam.decay = weight_decay;
+  f.adam.eps = eps;
+  return csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
+                                hot_items, hot_cap, counts_dev, nullptr, row_dtype, U, D, 0, cover_offsets, cover_is64,
+                                cover_S, stream, kEpiAdam, &f, 256, &alpha);
+}
+
+int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                    const void* coef, int coef_dtype, const int32_t* row_start,
+                                    const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
+                                    int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
+                                    const int64_t* row_index, void* const* emb_blocks_dev,
+                                    void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
+                                    int row_dtype, double lr, double eps, void* stream_) {
+  if (U == 0) return RECIS_OK;
+  FuseArgs f;
+  if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, accum_blocks_dev, nullptr, false, n_blocks, block_size, D,
+                              row_dtype))
+    return rc;
+  f.lr = static_cast<float>(lr);
+  f.eps = static_cast<float>(eps);
+  return csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
+                                hot_items, hot_cap, counts_dev, nullptr, row_dtype, U, D, 0, cover_offsets, cover_is64,
+                                cover_S, static_cast<hipStream_t>(stream_), kEpiAdagrad, &f);
 }
 
 int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows,

@@ -931,6 +931,57 @@ def csr_gather_reduce_parts(parts, plan, src, out=None, accumulate=False):
     return out
 
 
+def _fused_update_args(rows, plan, src, coef, cover, row_index, emb_blocks, block_size):
+    require_cuda(rows, src, coef, row_index)
+    rows = _contig(rows)
+    b0 = _check_blocks(emb_blocks, block_size)
+    D = rows.shape[1]
+    if _row_bytes(b0) // b0.element_size() != D:
+        raise ValueError("gradient rows have %d columns, the table's rows %d" % (D, _row_bytes(b0) // b0.element_size()))
+    row_index = _ids64(row_index)
+    if row_index.numel() < plan.U:
+        raise ValueError("row_index holds %d rows for %d unique ids" % (row_index.numel(), plan.U))
+    head = (ptr(rows), dtype_code(rows.dtype), i64(rows.shape[0]), ptr(src), ptr(coef),
+            dtype_code(coef.dtype) if coef is not None else 0, ptr(plan.row_start), ptr(plan.hot_items),
+            i64(plan.hot_cap), ptr(plan.counts), i64(plan.U), i64(D), ptr(cover),
+            _index_kind(cover, "offsets") if cover is not None else 0,
+            i64(cover.numel() - 1 if cover is not None else 0), ptr(row_index))
+    return head, b0, rows
+
+
+def csr_gather_reduce_adamw(rows, plan, src, coef, row_index, emb_blocks, beta1_t, beta2_t, exp_avg, exp_avg_sq, lr,
+                            beta1, beta2, weight_decay, eps, block_size, cover=None):
+    """``csr_gather_reduce`` + ``block_apply_adamw`` in one launch (``recis_csr_gather_reduce_adamw``): the
+    gradient of unique id ``u`` (the sum over its list of ``coef * rows[src]``) is applied to table row
+    ``row_index[u]`` by the lanes that summed it; the ``[U, D]`` gradient is never written. Bit for bit
+    what the two calls give."""
+    head, b0, rows = _fused_update_args(rows, plan, src, coef, cover, row_index, emb_blocks, block_size)
+    _check_blocks(exp_avg, block_size)
+    _check_blocks(exp_avg_sq, block_size)
+    if len(exp_avg) != len(emb_blocks) or len(exp_avg_sq) != len(emb_blocks):
+        raise ValueError("state slots must have as many blocks as the embedding slot")
+    require_cuda(beta1_t, beta2_t)
+    if beta1_t.dtype != beta2_t.dtype or beta1_t.dtype not in (torch.float32, torch.float64):
+        raise TypeError("beta1_t / beta2_t must both be float32 or float64")
+    check(lib().recis_csr_gather_reduce_adamw(
+        *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(exp_avg)), ptr(block_ptr_table(exp_avg_sq)),
+        i64(len(emb_blocks)), i64(block_size), dtype_code(b0.dtype), ptr(beta1_t), ptr(beta2_t),
+        int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1), ctypes.c_double(beta2),
+        ctypes.c_double(weight_decay), ctypes.c_double(eps), stream_ptr(rows.device)))
+
+
+def csr_gather_reduce_adagrad(rows, plan, src, coef, row_index, emb_blocks, accum_blocks, lr, eps, block_size,
+                              cover=None):
+    """``csr_gather_reduce`` + ``block_apply_adagrad`` in one launch (``recis_csr_gather_reduce_adagrad``)."""
+    head, b0, rows = _fused_update_args(rows, plan, src, coef, cover, row_index, emb_blocks, block_size)
+    _check_blocks(accum_blocks, block_size)
+    if len(accum_blocks) != len(emb_blocks):
+        raise ValueError("state slot must have as many blocks as the embedding slot")
+    check(lib().recis_csr_gather_reduce_adagrad(
+        *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)),
+        i64(block_size), dtype_code(b0.dtype), ctypes.c_double(lr), ctypes.c_double(eps), stream_ptr(rows.device)))
+
+
 def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_index=None, weight=None, out_dtype=None):
     """``out[i] = weight[i] * row(unique id of occurrence i)`` for the ``n_out`` occurrences of
     ``plan``: every unique row is read once and written to all its occurrences. Rows come from

@@ -92,6 +92,18 @@ class _AdamFamilyImpl(_SparseOptimizerImpl):
                               st["exp_avg"].kernel_blocks()[0], st["exp_avg_sq"].kernel_blocks()[0],
                               self._lr, self._beta1, self._beta2, self._decay(), self._eps, chunk_rows)
 
+    def apply_planned(self, ht, plan, grad_rows, src, coef, index, cover=None):
+        """One optimizer step for ``ht`` straight from the gradients of the lookups: the gradient of
+        unique id ``u`` of ``plan`` (sum over its occurrence list of ``coef * grad_rows[src]``) is applied
+        to row ``index[u]`` as it is summed (``ops.csr_gather_reduce_adamw``); the ``[U, D]`` gradient is
+        never written. Same result, bit for bit, as ``accept_grad(index, csr_gather_reduce(...))`` +
+        ``step()`` for a table that receives one gradient in the step and no gradient accumulation."""
+        st = self._state[id(ht)]
+        chunks, chunk_rows = ht._slot_group.emb_slot().kernel_blocks()
+        ops.csr_gather_reduce_adamw(grad_rows, plan, src, coef, index, chunks, st["beta1"], st["beta2"],
+                                    st["exp_avg"].kernel_blocks()[0], st["exp_avg_sq"].kernel_blocks()[0], self._lr,
+                                    self._beta1, self._beta2, self._decay(), self._eps, chunk_rows, cover=cover)
+
     def state_dict(self):
         steps = {}
         for st in self._state.values():
@@ -151,6 +163,13 @@ class SparseAdagradImpl(_SparseOptimizerImpl):
     def _update(self, ht, st, index, grad):
         chunks, chunk_rows = ht._slot_group.emb_slot().kernel_blocks()
         ops.block_apply_adagrad(index, grad, chunks, st["accum"].kernel_blocks()[0], self._lr, self._eps, chunk_rows)
+
+    def apply_planned(self, ht, plan, grad_rows, src, coef, index, cover=None):
+        """The Adagrad step of ``ht`` fused into the gather-reduce of its gradients (see the Adam family)."""
+        st = self._state[id(ht)]
+        chunks, chunk_rows = ht._slot_group.emb_slot().kernel_blocks()
+        ops.csr_gather_reduce_adagrad(grad_rows, plan, src, coef, index, chunks, st["accum"].kernel_blocks()[0],
+                                      self._lr, self._eps, chunk_rows, cover=cover)
 
     def state_dict(self):
         return {}, {}

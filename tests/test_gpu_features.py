@@ -255,6 +255,31 @@ def test_unique_plan_skewed_buckets(rng):
     _check_plan(np.arange(n, dtype=np.int64)[::-1] << 40)
 
 
+def test_unique_plan_heavy_ids(rng):
+    """Batches whose head ids make up a large share of all occurrences (Zipf(1.1) and Zipf(1.2) ranks
+    as in the table and sequence workloads; the empty-marker value and another id planted at 14 %
+    and 2 %): such ids get columns of their own in the partition and come out as the first unique
+    ids. Also through the fused find-or-insert: the rows are those a plain lookup gives."""
+    n = 2_000_000
+    for alpha in (1.1, 1.2):
+        ranks = np.minimum(rng.zipf(alpha, size=n), 10_000_000).astype(np.int64)
+        ids = ranks * 2654435761 % (1 << 40)
+        p = _check_plan(ids)
+        counts = np.diff(p.row_start[: p.U + 1].cpu().numpy())
+        assert counts[0] == counts.max() and counts[0] > n // 20   # the head id leads the unique ids
+    planted = ids.copy()
+    planted[::7] = -1
+    planted[1::50] = 77
+    _check_plan(planted)
+    m = ops.IdMap()
+    for _ in range(2):   # all keys new, then all keys known
+        p = ops.ids_unique_plan(_dev(ids), idmap=m)
+        assert torch.equal(p.index_buf[: p.U], m.lookup_readonly(p.unique))
+    assert m.size() == p.U == np.unique(ids).size
+    assert sorted(p.index_buf[: p.U].tolist()) == list(range(p.U))   # rows 0 .. U-1, each once
+    assert _lib.poll_device_errors() == 0
+
+
 @pytest.mark.parametrize("mode", ["sum", "mean", "tile"])
 @pytest.mark.parametrize("D,dtype", [(16, torch.float32), (128, torch.bfloat16), (40, torch.float32)])
 def test_planned_backward_matches_oracle(rng, mode, D, dtype):
@@ -333,4 +358,45 @@ def test_gather_reduce_over_separate_arrays_equals_the_concatenation(rng, dtype,
     assert torch.equal(split, whole)
     again = ops.csr_gather_reduce_parts(parts, plan, src, out=split.clone(), accumulate=True)
     torch.testing.assert_close(again, 2 * whole, rtol=1e-6, atol=1e-6)
+    assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("kind", ["adamw", "adagrad"])
+@pytest.mark.parametrize("D,row_dtype,grad_dtype", [(16, torch.float32, torch.float32), (128, torch.bfloat16, torch.bfloat16),
+                                                    (40, torch.float32, torch.float32), (32, torch.bfloat16, torch.float32)])
+def test_fused_gather_reduce_update_equals_the_two_calls(rng, kind, D, row_dtype, grad_dtype):
+    """recis_csr_gather_reduce_adamw / _adagrad against recis_csr_gather_reduce into an fp32 buffer followed
+    by recis_block_apply_adamw / _adagrad (which is bit-exact against the oracle, test_gpu_table.py): the
+    same rows, moments and beta powers bit for bit. Ids with tens of thousands of occurrences (hot work
+    items), rows the table does not hold (negative row index), pooled segments with weights."""
+    n, S, bs, nb = 120000, 30000, 4096, 5
+    ids = np.where(rng.random(n) < 0.3, rng.integers(0, 6, size=n), rng.integers(0, 15000, size=n))
+    plan = ops.ids_unique_plan(_dev(ids))
+    U = plan.U
+    off = ragged_offsets(rng, S, 0, 8)
+    off[-1] = n
+    off = np.minimum.accumulate(off[::-1])[::-1]
+    weight = _dev(rng.random(n).astype(np.float32))
+    src, coef = plan.src_coef_for_pool(_dev(off), weight, mean=True)
+    grad_rows = _dev(rng.standard_normal((S, D)).astype(np.float32)).to(grad_dtype)
+    row_index = torch.from_numpy(rng.permutation(bs * nb)[:U]).cuda()
+    row_index[::17] = -1
+    mk = lambda: [_dev(rng.random((bs, D)).astype(np.float32)).to(row_dtype) for _ in range(nb)]
+    emb, s0, s1 = mk(), mk(), mk()
+    emb2, s02, s12 = [b.clone() for b in emb], [b.clone() for b in s0], [b.clone() for b in s1]
+    b1, b2 = torch.tensor([0.9], device="cuda", dtype=torch.float64), torch.tensor([0.999], device="cuda", dtype=torch.float64)
+    b1f, b2f = b1.clone(), b2.clone()
+    keep = row_index >= 0
+    for _ in range(2):
+        g = ops.csr_gather_reduce(grad_rows, plan, src, coef)
+        if kind == "adamw":
+            ops.block_apply_adamw(row_index[keep], g[keep], emb, b1, b2, None, s0, s1, 1e-2, 0.9, 0.999, 0.99, 1e-8, bs)
+            ops.csr_gather_reduce_adamw(grad_rows, plan, src, coef, row_index, emb2, b1f, b2f, s02, s12, 1e-2, 0.9, 0.999,
+                                        0.99, 1e-8, bs)
+        else:
+            ops.block_apply_adagrad(row_index[keep], g[keep], emb, s0, 1e-2, 1e-8, bs)
+            ops.csr_gather_reduce_adagrad(grad_rows, plan, src, coef, row_index, emb2, s02, 1e-2, 1e-8, bs)
+    for a, b in zip(emb + s0 + (s1 if kind == "adamw" else []), emb2 + s02 + (s12 if kind == "adamw" else [])):
+        assert torch.equal(a, b)
+    assert torch.equal(b1, b1f) and torch.equal(b2, b2f)
     assert _lib.poll_device_errors() == 0
