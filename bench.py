@@ -708,10 +708,9 @@ class ModulePath5:
 # scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC_C4 = {
-    "adamw_rows_kernel": 433714773, "csr_rows_kernel": 395422130, "csr_expand_kernel": 256908532,
-    "plan_emit_kernel": 149225867, "find_or_claim_kernel": 131811016, "plan_bucket_kernel": 89186262,
-    "plan_scatter_kernel": 77270206, "plan_tile_kernel": 58181470, "ids_encode_kernel": 40935979,
-    "plan_colscan_kernel": 16429891,
+    "csr_rows_adam_kernel": 730625331, "csr_expand_kernel": 260825088, "plan_bucket_kernel": 193435648,
+    "plan_scatter_kernel": 105619149, "ids_encode_kernel": 40936858, "plan_hist_kernel": 21896499,
+    "uint64_mod_kernel": 13689037, "bucketize_kernel": 10261094, "plan_colscan_kernel": 4108493,
 }
 
 

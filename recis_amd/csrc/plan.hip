@@ -262,7 +262,7 @@ plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int64_t* __r
   const int nc = kHeavyMax + (1 << g.nb_log2);
   if (blockIdx.x == 0) {
     if (tid < 2) counts[tid] = 0;
-    if (tid < 4) sync[tid] = 0;  // [1] finished workgroups of the bucket kernel, [2] of the row assignment
+    if (tid < 4) sync[tid] = 0;  // [1] finished workgroups of the bucket kernel, [2] of the row assignment, [3] new keys
   }
   for (int b = tid; b < nc; b += kPartBlock) l_hist[b] = 0;
   const int n_heavy = load_heavy(heavy_ids, heavy_n, h_slot, h_key);
@@ -694,6 +694,7 @@ __device__ __forceinline__ void heavy_rows(const BucketArgs& a, int n_heavy, uns
     if (threadIdx.x == 0) {
       if ((new_total >> 32) != 0) atomicAdd(reinterpret_cast<unsigned long long*>(&a.state[ST_OCC]), new_total >> 32);
       a.new_count[0] = static_cast<int32_t>(new_total & 0xffffffffull);
+      if (new_total & 0xffffffffull) atomicAdd(&a.sync[3], static_cast<int32_t>(new_total & 0xffffffffull));
     }
     if (my_new) {
       NewRec nr;
@@ -1096,7 +1097,10 @@ plan_bucket_kernel(BucketArgs a) {
     if (rounds > 1)
       __hip_atomic_store(&a.agg[b], kPrefixFlag | static_cast<unsigned long long>(u_base + u_done), __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
-    if constexpr (PROBE) a.new_count[1 + b] = new_done;
+    if constexpr (PROBE) {
+      a.new_count[1 + b] = new_done;
+      if (new_done) atomicAdd(&a.sync[3], new_done);  // lets the row assignment leave at once when there are none
+    }
     if (b == (1 << nb_log2) - 1) {  // the last bucket knows the total
       const int64_t U = u_base + u_done;
       __hip_atomic_store(&a.counts[0], U, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1120,8 +1124,10 @@ plan_assign_new_kernel(Slot* __restrict__ table, const NewRec* __restrict__ new_
                        int32_t* __restrict__ sync) {
   // nb here = 1 + buckets: the new keys among the heavy ids, then those of every bucket
   extern __shared__ int32_t first_new[];  // [nb + 1], then kPartBlock words of scan scratch
-  scan_counts(new_count, nb, first_new, first_new + nb + 1);
-  const int64_t n_new = first_new[nb];
+  // a batch of known keys only (the steady state of a table that is not growing): nothing to scan
+  const bool any_new = __hip_atomic_load(&sync[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;  // uniform
+  if (any_new) scan_counts(new_count, nb, first_new, first_new + nb + 1);
+  const int64_t n_new = any_new ? first_new[nb] : 0;
   const int64_t old_cur = state[ST_CUR], old_free = state[ST_FREE];
   for (int b = blockIdx.x; b < nb && n_new > 0; b += gridDim.x) {
     const int32_t cnt = new_count[b];
@@ -1505,8 +1511,10 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   }
 }
 
-// out[u] (+)= sum of the partial rows of hot row u, in chunk order. One lane group per work item
-// with chunk 0 (the items of a row are consecutive).
+// out[u] (+)= sum of the partial rows of hot row u (or the optimizer's update of the row with that
+// sum). One wave per work item with chunk 0 (the items of a row are consecutive): its lane groups
+// share the row's partials out among themselves (an id that makes up a tenth of the batch has a
+// hundred of them) and fold their sums with shuffles, always in the same order.
 template <typename TOut, int VEC, int EPI = kEpiStore>
 __global__ void __launch_bounds__(kBlock)
 csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
@@ -1514,24 +1522,35 @@ csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
   if (n_items > a.hot_cap) n_items = a.hot_cap;
   const int D = a.D;
   const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
-  const int64_t groups_total = static_cast<int64_t>(gridDim.x) * (kBlock >> a.lpr_log2);
-  for (int64_t item = static_cast<int64_t>(blockIdx.x) * (kBlock >> a.lpr_log2) + (threadIdx.x >> a.lpr_log2);
-       item < n_items; item += groups_total) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int groups = kWave >> a.lpr_log2, g = lane >> a.lpr_log2;
+  const int64_t waves_total = static_cast<int64_t>(gridDim.x) * (kBlock / kWave);
+  for (int64_t item = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave; item < n_items;
+       item += waves_total) {  // uniform in the wave
     if (a.hot_items[2 * item + 1] != 0) continue;
     const int32_t u = a.hot_items[2 * item];
     const int32_t len = a.row_start[u + 1] - a.row_start[u];
     int64_t n_chunks = (len + kHotChunk - 1) / kHotChunk;
     if (item + n_chunks > n_items) n_chunks = n_items - item;  // items cut off by hot_cap (cannot happen with the documented hot_cap)
-    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+      const int c0 = cbase + cl * VEC;
+      const bool col_ok = c0 < D;
       float acc[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      for (int64_t k = 0; k < n_chunks; ++k) {
-        float v[VEC];
-        load_pack<float, VEC>(a.hot_part + (item + k) * D + c0, v);
+      if (col_ok) {
+        for (int64_t k = g; k < n_chunks; k += groups) {
+          float v[VEC];
+          load_pack<float, VEC>(a.hot_part + (item + k) * D + c0, v);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += v[j];
+          for (int j = 0; j < VEC; ++j) acc[j] += v[j];
+        }
       }
+      for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+      }
+      if (g != 0 || !col_ok) continue;
       if constexpr (EPI != kEpiStore) {
         fused_row_update<TOut, VEC, EPI>(f, a.err, u, c0, acc);
       } else {
@@ -2216,7 +2235,7 @@ static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows
         TOut* o = static_cast<TOut*>(out);
         const bool shuffle = a.lpr_log2 >= 3;  // at most eight lane groups per wave
         const dim3 grid(a.cold_blocks + hot_blocks), block(kBlock);
-        const int64_t fin = std::min<int64_t>((hot_cap + rows_per_block - 1) / rows_per_block, 1024);
+        const int64_t fin = std::min<int64_t>((hot_cap + kBlock / kWave - 1) / (kBlock / kWave), 2048);  // a wave per item
         auto launch = [&](auto epi_tag) {
           constexpr int EPI = decltype(epi_tag)::value;
           {
