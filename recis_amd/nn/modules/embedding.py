@@ -164,11 +164,12 @@ class LookupPoolFunction(torch.autograd.Function):
         if ctx.late_count:
             ctx.impl.settle_count(ctx.plan.U, ctx.plan)
             index = index[: ctx.plan.U]
-        g = ops.segment_reduce_backward_plan(grad.contiguous(), weight, offsets, ctx.plan, ctx.combiner)
-        if ctx.readonly:  # keys the table does not hold take no gradient
-            keep = index >= 0
-            index, g = index[keep], g[keep]
-        ctx.impl.accept_grad(index, g, unique=True, key=None if ctx.readonly else ctx.plan.serial)
+        # sum / mean: the gradient of a unique row is a gather-reduce over its occurrence list; it is handed
+        # over unsummed, so that the optimizer step can sum and update the row in one launch (keys the table
+        # does not hold carry a negative index and take no gradient)
+        src, coef = ctx.plan.src_coef_for_pool(offsets.contiguous(), weight, ctx.combiner == "mean")
+        ctx.impl.accept_planned_grad(index, ctx.plan, grad.contiguous(), src, coef,
+                                     key=None if ctx.readonly else ctx.plan.serial, may_miss=ctx.readonly)
         return None, None, None, None, None, None, None, None
 
 

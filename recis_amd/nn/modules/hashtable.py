@@ -314,6 +314,7 @@ class HashtableImpl:
         self._slice = Slice(slice_begin, slice_end, slice_size)
         self._idmap = ops.IdMap(device, reserve=reserve_rows)
         self._grad_index, self._grad, self._grad_unique, self._grad_keys = [], [], [], {}
+        self._planned = None   # a gradient handed over as a sum still to be taken (accept_planned_grad)
 
     # ------------------------------------------------------------- storage
     def _make_room(self, incoming):
@@ -446,6 +447,7 @@ class HashtableImpl:
         instead of being merged by row index later."""
         if grad_index.dtype != torch.int64:
             raise RuntimeError("grad_index must be int64")
+        self._sum_planned()   # a gradient waiting to be summed comes first, as it was handed over first
         if grad.dtype != self._dtype and not (grad.dtype == torch.float32 and self._dtype in
                                               (torch.bfloat16, torch.float16)):
             raise RuntimeError("grad dtype %s does not match the table (%s)" % (grad.dtype, self._dtype))
@@ -459,13 +461,49 @@ class HashtableImpl:
         self._grad.append(grad)
         self._grad_unique.append(bool(unique))
 
+    def accept_planned_grad(self, index, plan, rows, src, coef=None, cover=None, key=None, may_miss=False):
+        """A gradient handed over before it is summed: the gradient of ``plan``'s unique id ``u`` (table row
+        ``index[u]``; negative = the table does not hold the key, no gradient) is the sum over u's occurrence
+        list of ``coef * rows[src]`` (``ops.csr_gather_reduce``). If it stays the only gradient of the step, an
+        optimizer that can (``apply_planned``) takes the sum and applies the row update in one launch and the
+        ``[U, D]`` gradient is never written; anything else that asks for the gradient (``grad``, ``grad_pairs``,
+        a second gradient, accumulation over several steps) gets it summed first, as ``accept_grad`` would have.
+        ``may_miss``: ``index`` may hold negative entries (a read-only lookup)."""
+        if self._grad or self._planned is not None:
+            self._sum_planned()
+            g = ops.csr_gather_reduce(rows, plan, src, coef, cover=cover)
+            self._accept_summed(index, g, key, may_miss)
+            return
+        self._planned = (index, plan, rows, src, coef, cover, key, may_miss)
+
+    def _accept_summed(self, index, g, key, may_miss):
+        if may_miss:  # keys the table does not hold take no gradient
+            keep = index >= 0
+            index, g = index[keep], g[keep]
+        self.accept_grad(index, g, unique=True, key=key)
+
+    def _sum_planned(self):
+        if self._planned is not None:
+            index, plan, rows, src, coef, cover, key, may_miss = self._planned
+            self._planned = None
+            self._accept_summed(index, ops.csr_gather_reduce(rows, plan, src, coef, cover=cover), key, may_miss)
+
+    def take_planned_grad(self):
+        """The planned gradient if it is all this table received since the last ``clear_grad`` (and forgets
+        it), else None: ``(index, plan, rows, src, coef, cover)``."""
+        if self._planned is None or self._grad:
+            return None
+        planned, self._planned = self._planned, None
+        return planned[:6]
+
     def has_grad(self):
-        return len(self._grad) > 0
+        return len(self._grad) > 0 or self._planned is not None
 
     def grad_pairs(self, accumulate_steps=1):
         """(row index, gradient rows) merged over the accepted gradients: what
         ``grad()`` wraps as a sparse tensor (hashtable.cc:90-134), without the host
         round trips. With duplicates the gradients are summed per row."""
+        self._sum_planned()
         index = self._grad_index[0] if len(self._grad_index) == 1 else torch.cat(self._grad_index, 0)
         g = self._grad[0] if len(self._grad) == 1 else torch.cat(self._grad, 0)
         if not (len(self._grad_unique) == 1 and self._grad_unique[0]):
@@ -482,6 +520,7 @@ class HashtableImpl:
         """Sparse COO gradient exactly as the reference builds it (hashtable.cc:90-134),
         including its layout when rows repeat: positions 0..U-1 as indices and an
         N-row value buffer whose first U rows hold the sums."""
+        self._sum_planned()
         index = torch.cat(self._grad_index, 0)
         g = torch.cat(self._grad, 0)
         uniq, inverse = torch.unique(index, sorted=False, return_inverse=True)
@@ -501,6 +540,7 @@ class HashtableImpl:
 
     def clear_grad(self):
         self._grad_index, self._grad, self._grad_unique, self._grad_keys = [], [], [], {}
+        self._planned = None
 
     # ------------------------------------------------------------ bookkeeping
     def clear(self):
@@ -708,11 +748,9 @@ class LookupExpandFunction(torch.autograd.Function):
         flat = grad.reshape(n, -1).contiguous()
         if ctx.slice_num != 1:
             flat = flat / ctx.slice_num
-        g = ops.csr_gather_reduce(flat, ctx.plan, ctx.plan.occ).to(grad.dtype)
-        if ctx.readonly:  # keys the table does not hold take no gradient
-            keep = index >= 0
-            index, g = index[keep], g[keep]
-        ctx.impl.accept_grad(index, g, unique=True)
+        # the sum over the duplicates of each id is left to the optimizer step where it can be (one launch
+        # sums and updates the row); keys the table does not hold (negative index) take no gradient
+        ctx.impl.accept_planned_grad(index, ctx.plan, flat, ctx.plan.occ, may_miss=ctx.readonly)
         return None, None, None, None, None
 
 

@@ -48,6 +48,11 @@ class _SparseOptimizerImpl:
             for name, ht in self._params.items():
                 if not ht.has_grad():
                     continue
+                planned = ht.take_planned_grad() if self._grad_accum_steps == 1 and hasattr(self, "apply_planned") else None
+                if planned is not None:   # the gradient is still a sum to be taken: sum and update in one launch
+                    index, plan, rows, src, coef, cover = planned
+                    self.apply_planned(ht, plan, rows, src, coef, index, cover)
+                    continue
                 index, grad = ht.grad_pairs(self._grad_accum_steps)
                 self._update(ht, self._state[id(ht)], index, grad)
 

@@ -589,3 +589,48 @@ def test_a_waiting_plan_between_forward_and_backward_does_not_steal_the_unique_c
     perm = [by_row[r] for r in index[order].tolist()]
     np.testing.assert_allclose(g[order].cpu().numpy(), exp[perm], rtol=1e-5, atol=1e-5)
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("opt_cls", [SparseAdam, SparseAdagrad])
+def test_gradient_summed_in_the_optimizer_step_equals_summed_first(opt_cls):
+    """The module layer hands the table its gradient unsummed (accept_planned_grad) and the optimizer step
+    sums it and updates the rows in one launch. Two engines on the same data, one stepping that way, the other
+    made to sum first (grad_pairs() before step(), what any reader of the gradient triggers): rows and state
+    agree after every step to the last bit or two (each engine makes its own batch plan, and the order inside an
+    id's occurrence list, hence the order of its sum, is not fixed from plan to plan; on one plan the two ways
+    are equal bit for bit: test_fused_gather_reduce_update_equals_the_two_calls). A second gradient in the same
+    step is summed and merged as before."""
+    def make(tag):
+        HashtableRegister().clear()
+        init = NormalInitializer(0.0, 0.1, generator=torch.Generator(device="cuda").manual_seed(7))
+        eng = EmbeddingEngine({
+            "a": EmbeddingOption(embedding_dim=16, shared_name="t" + tag, combiner="sum", use_weight=False, initializer=init),
+            "b": EmbeddingOption(embedding_dim=16, shared_name="t" + tag, combiner="mean", use_weight=False, initializer=init),
+        }).cuda()
+        eng.train()
+        return eng, opt_cls(filter_out_sparse_param(eng), lr=1e-2)
+    (e1, o1), (e2, o2) = make("1"), make("2")
+    rng = np.random.default_rng(11)
+    for step in range(4):
+        dense = torch.from_numpy(rng.integers(0, 300, size=(512, 1))).cuda()           # one id per sample
+        lens = rng.integers(0, 9, size=512)
+        off = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)).cuda()
+        vals = torch.from_numpy(rng.integers(0, 300, size=int(lens.sum()))).cuda()
+        up = torch.randn(512, 16, device="cuda", generator=torch.Generator(device="cuda").manual_seed(step))
+        for eng, opt, sum_first in ((e1, o1, False), (e2, o2, True)):
+            feats = {"a": dense} if step % 2 == 0 else {"a": dense, "b": RaggedTensor(vals, off)}
+            out = eng(feats)
+            torch.autograd.backward([out[k] for k in out], [up for _ in out])
+            impls = [t._hashtable_impl for t in eng.hashtables().values()]
+            if step % 2 == 0:
+                assert all(i._planned is not None and not i._grad for i in impls)        # waiting unsummed
+            if sum_first:
+                for i in impls:
+                    i.grad_pairs(1)
+                    assert i._planned is None
+            opt.step()
+            opt.zero_grad()
+        for t1, t2 in zip(e1.hashtables().values(), e2.hashtables().values()):
+            for s1, s2 in zip(t1.slot_group().slots(), t2.slot_group().slots()):
+                torch.testing.assert_close(s1.value(), s2.value(), rtol=1e-5, atol=1e-7, msg=lambda m: "%s step %d slot %s" % (m, step, s1.name()))
+    assert _lib.poll_device_errors() == 0
