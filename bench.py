@@ -553,13 +553,14 @@ class Config5:
         rows = o.block_gather(index, chunks, chunk_rows, -1, False)
         pooled = o.segment_reduce_forward(rows, None, inv, self.offsets, "mean", out_dtype=torch.float32)
         padded, batch_seq = o.ragged_tile(self.batch, self.seq, inv, self.offsets, rows)
-        g = o.segment_reduce_backward_plan(self.g_pool, None, self.offsets, plan, "mean")
-        o.csr_gather_reduce(self.g_tile, plan, plan.src_for_tile(self.batch, self.seq, self.offsets), out=g,
-                            accumulate=True)
-        self.table.accept_grad(index, g, unique=True)
-        self.opt.step()
-        self.opt.zero_grad()
+        self.bwd_update(plan, index)
         return pooled, padded
+
+    def bwd_update(self, plan, index):
+        """Backward of both outputs into the unique rows and the Adagrad update of those rows, one
+        launch: the two gradients of an occurrence are summed where the row's gradient is summed."""
+        src_p, coef_p, src_t = plan.src_for_pool_and_tile(self.offsets, None, True, self.batch, self.seq)
+        self.opt.apply_planned2(self.table, plan, (self.g_pool, src_p, coef_p), (self.g_tile, src_t, None), index)
 
     def survey_bytes(self):
         N, U, S, D = self.N, self.U, self.S, self.D
@@ -571,15 +572,16 @@ class Config5:
 
     def kernel_bytes(self):
         """Algorithmic HBM bytes per launch: the padded gather runs once per field, the
-        gather-reduce once over the pooled gradients (fp32 rows, re-read out of the caches: priced
-        at one read per segment) and once over the padded gradients (bf16 rows)."""
+        gather-reduce with the Adagrad update once over both gradients."""
         N, U, S, D = self.N, self.U, self.S, self.D
         n_fields = len(self.fields)
         return {
             "tile_fwd_kernel": (self.pad_rows * D * 2 + 4 * N + U * D * 2) // n_fields,  # distinct rows once
-            "csr_rows_kernel": (S * D * 4 + N * D * 2 + 2 * (8 * N + 4 * U) + 3 * U * D * 4) // 2,
+            # pooled gradients (fp32 rows, re-read out of the caches: one read per segment), padded
+            # gradients (bf16 rows, one per occurrence inside its field's pad length), src + coef of
+            # both inputs, list starts, row index, parameter and accumulator rows read and written
+            "csr_rows_adagrad_kernel": S * D * 4 + N * D * 2 + (4 + 4 + 4) * N + (4 + 8) * U + 4 * U * D * 2,
             "seg_pool_fwd_kernel": U * D * 2 + 4 * N + 4 * (S + 1) + S * D * 4,
-            "adagrad_rows_kernel": U * (8 + D * 4 + 4 * D * 2),
         }
 
     def cpu_baseline(self, budget_s):

@@ -472,18 +472,21 @@ int recis_unique_plan_noalloc(const int64_t* ids, int64_t n, int64_t* unique_out
 
 /*
  * Per list entry, the input row it reads and its coefficient, for the backward of
- *   pooled segments: src = segment of the occurrence, coef = weight (/ length for MEAN)
- *                    (coef_out may be NULL when there are no weights and mean == 0)
- *   padded gather:   src = padded output row of the occurrence, -1 beyond seq[f]
- * pos = pos_out of recis_unique_plan. Entries of occurrences outside the offsets range
- * get src = -1 (skipped).
+ *   pooled segments: src_pool_out = segment of the occurrence, coef_out = weight (/ length for
+ *                    MEAN); coef_out may be NULL when there are no weights and mean == 0
+ *   padded gather:   src_tile_out = padded output row of the occurrence, -1 beyond seq[f]; the
+ *                    S segments are those of n_features features, batch[f] samples each, feature
+ *                    f padded to seq[f] rows per sample
+ * Either pair of outputs may be NULL (src_tile_out == NULL: batch / seq / n_features unused).
+ * list = list_out of recis_unique_plan (entry k lists occurrence list[k]); offsets [S + 1] are
+ * the segments' offsets. Entries of occurrences outside the offsets range get src = -1 (skipped).
+ * No reference counterpart: the reference's backward kernels search the offsets per element
+ * while they scatter (embedding_segment_reduce_kernel.cu:79-120).
  */
-int recis_csr_fill_pool(const void* offsets, int off_is64, int64_t S, int64_t n, const void* weight,
-                        int weight_dtype, const int32_t* pos, int mean, int32_t* src_out,
-                        float* coef_out, void* stream);
-int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_features,
-                        const void* offsets, int off_is64, int64_t n, const int32_t* pos,
-                        int32_t* src_out, void* stream);
+int recis_csr_fill_lists(const int32_t* list, int64_t n, const void* offsets, int off_is64, int64_t S,
+                         const void* weight, int weight_dtype, int mean, int32_t* src_pool_out,
+                         float* coef_out, const int64_t* batch, const int64_t* seq, int64_t n_features,
+                         int32_t* src_tile_out, void* stream);
 
 /*
  * out[u, :] (+)= sum over k in [row_start[u], row_start[u+1]) of coef[k] * rows[src[k], :]
@@ -548,6 +551,47 @@ int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_
                                     int64_t cover_S, const int64_t* row_index, void* const* emb_blocks_dev,
                                     void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
                                     int row_dtype, double lr, double eps, void* stream);
+
+/*
+ * Gather-reduce with TWO inputs over the same occurrence lists: list entry k of unique id u adds
+ * a.coef[k] * a.rows[a.src[k]] + b.coef[k] * b.rows[b.src[k]] (a negative src skips that term;
+ * coef NULL = 1). A lookup whose rows feed two outputs, a pooled one and an unpooled, padded one
+ * (the sequence features of the reference: csrc/ops/embedding_segment_reduce_kernel.cu:276-350
+ * and the ragged_tile backward, ragged_tile_kernel.cu), has two gradients per occurrence; the
+ * reference scatters each into the unique rows by itself, this sums both in the pass that owns the
+ * row. The first input must be fp32; the second fp32, or bf16 / f16 where noted.
+ *   recis_csr_gather_reduce2          out (fp32 [U, D]) (+)= sum; second input fp32 / bf16 / f16
+ *   recis_csr_gather_reduce2_adamw    the sum is the gradient of table row row_index[u]: the row
+ *   recis_csr_gather_reduce2_adagrad  update is applied at once, as by recis_csr_gather_reduce_adamw
+ *                                     / _adagrad; second input fp32 or of the table's row type
+ * The result equals recis_csr_gather_reduce(a) followed by recis_csr_gather_reduce(b, accumulate)
+ * up to fp32 rounding (here both inputs go through one chain of fused multiply-adds, there the
+ * first sum is rounded to the output before the second is added).
+ */
+typedef struct recis_csr_input {
+  const void* rows;   /* [n_rows, D] */
+  int rows_dtype;
+  int64_t n_rows;
+  const int32_t* src; /* [n] input row per list entry */
+  const void* coef;   /* [n] per list entry, or NULL */
+  int coef_dtype;
+} recis_csr_input;
+int recis_csr_gather_reduce2(const recis_csr_input* a, const recis_csr_input* b, const int32_t* row_start,
+                             const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev,
+                             void* out, int64_t U, int64_t D, int accumulate, void* stream);
+int recis_csr_gather_reduce2_adamw(const recis_csr_input* a, const recis_csr_input* b,
+                                   const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
+                                   const int64_t* counts_dev, int64_t U, int64_t D, const int64_t* row_index,
+                                   void* const* emb_blocks_dev, void* const* exp_avg_blocks_dev,
+                                   void* const* exp_avg_sq_blocks_dev, int64_t n_blocks, int64_t block_size,
+                                   int row_dtype, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
+                                   double beta1, double beta2, double weight_decay, double eps, void* stream);
+int recis_csr_gather_reduce2_adagrad(const recis_csr_input* a, const recis_csr_input* b,
+                                     const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
+                                     const int64_t* counts_dev, int64_t U, int64_t D, const int64_t* row_index,
+                                     void* const* emb_blocks_dev, void* const* accum_blocks_dev,
+                                     int64_t n_blocks, int64_t block_size, int row_dtype, double lr, double eps,
+                                     void* stream);
 
 /*
  * The transpose of recis_csr_gather_reduce (no reference counterpart; it produces what

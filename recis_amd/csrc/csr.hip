@@ -1,0 +1,462 @@
+// Consumers of the batch plan for gfx950: per-row work driven by the plan's occurrence lists.
+//
+//   gather-reduce  out[u] = sum over the list entries k of unique id u of coef[k] * rows[src[k]]
+//                  (the backward of pooling and of the padded gather), optionally ending in the
+//                  optimizer's update of table row row_index[u] instead of a store
+//   expand         out[dst[k]] = w[dst[k]] * row(u): the forward of the lookup, each table row
+//                  read once and written per occurrence
+//   fill_lists     the src / coef arrays of the gather-reduce for the two pooling shapes
+//
+// The reference scatters gradients back to unique rows with one global atomic per element
+// (csrc/ops/embedding_segment_reduce_kernel.cu:79-120, segment_ops_kernel.cu:133-165); here every
+// unique row is summed by the lanes that own it, rows with very many occurrences are cut into
+// work items whose partial sums a second small kernel folds, and nothing is atomic.
+#include "csr_rows.cuh"
+
+namespace recis_hip {
+namespace {
+
+// ------------------------------------------------------------------ expand (transpose of the gather-reduce)
+// out[dst[k], :] = w[dst[k]] * row(u) for every list entry k of every unique id u: the forward
+// of pooling when every segment holds exactly one id, and of the unpooled (tile) output. Each
+// unique row is read ONCE and stored to all its occurrences; stores do not wait for anything,
+// where the occurrence-major kernels chase index -> row index -> row for every output row.
+struct ExpArgs {
+  const int32_t* row_start;  // [U + 1]
+  const int32_t* dst;        // [n] output row per list entry
+  const void* weight;        // [n_out] per output row, or NULL
+  int wdt;
+  int64_t U, n_out;
+  int D;
+  int lpr_log2;
+  int* err;
+  const int64_t* row_index;  // rows in a block list: unique row u is row row_index[u] (negative = zeros)
+  const void* const* blocks;
+  int64_t block_rows, n_blocks;
+  int32_t hot_len;
+  const int32_t* hot_items;
+  const int64_t* counts;
+  int64_t hot_cap;
+  int64_t cold_blocks;
+};
+
+template <typename TIn, typename TOut, int VEC, bool BLK>
+__global__ void __launch_bounds__(kBlock)
+csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs a) {
+  const int D = a.D;
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
+  const int g = lane >> a.lpr_log2;        // this lane's group in its wave
+
+  auto load_row = [&](int64_t u, int c0, float (&v)[VEC]) {
+    const TIn* src = nullptr;
+    if constexpr (BLK) {
+      const int64_t ri = a.row_index[u];
+      if (ri >= 0) {
+        int64_t b = 0, r = ri;
+        if (a.n_blocks > 1) {
+          b = ri / a.block_rows;
+          r = ri - b * a.block_rows;
+        }
+        if (b >= a.n_blocks || r >= a.block_rows)
+          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+        else
+          src = static_cast<const TIn*>(a.blocks[b]) + r * D;
+      }
+    } else {
+      src = rows + u * D;
+    }
+    if (src) {
+      load_pack_stream<TIn, VEC>(src + c0, v);  // every row is read once here
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+    }
+  };
+  auto store_to = [&](int64_t d, int c0, const float (&v)[VEC]) {
+    if (static_cast<uint64_t>(d) >= static_cast<uint64_t>(a.n_out)) {
+      raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      return;
+    }
+    float o[VEC];
+    const float w = a.weight ? load_coef(a.weight, a.wdt, d) : 1.0f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) o[j] = fmaf(v[j], w, 0.f);  // the pooled kernels' rounding
+    store_pack_stream<TOut, VEC>(out + d * D + c0, o);
+  };
+  // stores to the list entries first, first + step, ... < last; the destinations of four entries
+  // are fetched together so that their latencies overlap (more would cost resident waves)
+  auto store_list = [&](int32_t first, int32_t last, int32_t step, int c0, const float (&v)[VEC]) {
+    for (int32_t k = first; k < last; k += 4 * step) {
+      int32_t d[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = k + i * step < last ? a.dst[k + i * step] : -1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (k + i * step < last) store_to(d[i], c0, v);
+    }
+  };
+
+  const int64_t hot_blocks = static_cast<int64_t>(gridDim.x) - a.cold_blocks;
+  if (static_cast<int64_t>(blockIdx.x) < hot_blocks) {
+    // ---- hot work items: a workgroup per (row, chunk); all its lane groups hold the row
+    int64_t n_items = a.counts[1];
+    if (n_items > a.hot_cap) n_items = a.hot_cap;
+    const int groups_per_block = kBlock >> a.lpr_log2;
+    const int gb = threadIdx.x >> a.lpr_log2;
+    for (int64_t item = blockIdx.x; item < n_items; item += hot_blocks) {
+      const int32_t u = a.hot_items[2 * item];
+      const int32_t chunk = a.hot_items[2 * item + 1];
+      const int32_t start = a.row_start[u] + chunk * kHotChunk;
+      const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
+      for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+        float v[VEC];
+        load_row(u, c0, v);
+        store_list(start + gb, end, groups_per_block, c0, v);
+      }
+    }
+    return;
+  }
+
+  // ---- cold rows
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
+  const bool valid = u < a.U && u < a.counts[0];  // U may be the caller's upper bound: the plan's own count decides
+  const int32_t start = valid ? a.row_start[u] : 0;
+  int32_t end = valid ? a.row_start[u + 1] : 0;
+  if (end - start > a.hot_len) end = start;  // written by the work items
+  const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;
+  if (valid && !is_long && end > start) {
+    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+      float v[VEC];
+      load_row(u, c0, v);
+      store_list(start, end, 1, c0, v);
+    }
+  }
+  // long rows of this wave, one after the other: the owner's row reaches every group by shuffles
+  uint64_t todo = __ballot(is_long);
+  while (todo) {
+    const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;
+    todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);
+    const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
+    const int64_t row = u - g + (owner >> a.lpr_log2);  // rows of a wave are consecutive
+    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+      const int c0 = cbase + cl * VEC;
+      const bool col_ok = c0 < D;
+      float mine[VEC], v[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) mine[j] = 0.f;
+      if (lane >> a.lpr_log2 == owner >> a.lpr_log2 && col_ok) load_row(row, c0, mine);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = __shfl(mine[j], owner + cl, kWave);
+      if (col_ok) store_list(r_start + g, r_end, groups, c0, v);
+    }
+  }
+}
+
+// src / coef of every list entry, for the backward of pooled segments and of the padded gather over
+// the same occurrences. Entry k lists occurrence i = list[k], which lies in segment s (the largest
+// s with offsets[s] <= i, found by bisection: the offsets of a batch stay in the caches) at place
+// t = i - offsets[s]:
+//   pooled segments  src = s, coef = w_i (divided by the segment length for mean)
+//   padded gather    segment s is sample b = s - seg_lo[f] of feature f, and place t of it is padded
+//                    row rbase[f] + b * seq[f] + t, or nothing (-1) when t >= seq[f]
+// Reads and writes go by list entry, so every array is streamed; one launch serves both shapes.
+constexpr int kFillFeatures = 32;  // features of the padded gather per launch
+struct FillArgs {
+  const int32_t* list;
+  int64_t n;
+  const void* offsets;
+  int off64;
+  int64_t S;
+  const void* weight;
+  int wdt;
+  int mean;
+  int32_t* src_pool;  // or NULL
+  float* coef;        // or NULL
+  int32_t* src_tile;  // or NULL
+  int n_features;
+  int first_group;    // this launch also marks the entries that no segment covers
+  int64_t seg_lo[kFillFeatures + 1];
+  int64_t seq[kFillFeatures];
+  int64_t rbase[kFillFeatures];
+};
+__global__ void __launch_bounds__(kBlock)
+fill_lists_kernel(FillArgs a) {
+  const int64_t k = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (k >= a.n) return;
+  const int64_t i = a.list[k];
+  const int64_t first = load_index(a.offsets, a.off64, 0), last = load_index(a.offsets, a.off64, a.S);
+  if (i < first || i >= last) {
+    if (a.first_group) {
+      if (a.src_pool) a.src_pool[k] = -1;
+      if (a.coef) a.coef[k] = 0.f;
+      if (a.src_tile) a.src_tile[k] = -1;
+    }
+    return;
+  }
+  int64_t lo = 0, hi = a.S;
+  while (hi - lo > 1) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (load_index(a.offsets, a.off64, mid) <= i)
+      lo = mid;
+    else
+      hi = mid;
+  }
+  const int64_t begin = load_index(a.offsets, a.off64, lo);
+  if (a.first_group) {
+    if (a.src_pool) a.src_pool[k] = static_cast<int32_t>(lo);
+    if (a.coef) {
+      float w = a.weight ? load_coef(a.weight, a.wdt, i) : 1.0f;
+      if (a.mean) w /= static_cast<float>(load_index(a.offsets, a.off64, lo + 1) - begin);
+      a.coef[k] = w;
+    }
+  }
+  if (a.src_tile && lo >= a.seg_lo[0] && lo < a.seg_lo[a.n_features]) {
+    int f = 0;
+#pragma unroll 4
+    for (int x = 1; x < kFillFeatures; ++x) f += (x < a.n_features && lo >= a.seg_lo[x]) ? 1 : 0;
+    const int64_t t = i - begin;
+    a.src_tile[k] = t < a.seq[f] ? static_cast<int32_t>(a.rbase[f] + (lo - a.seg_lo[f]) * a.seq[f] + t) : -1;
+  }
+}
+
+}  // namespace
+}  // namespace recis_hip
+
+using namespace recis_hip;
+
+extern "C" {
+
+int recis_csr_fill_lists(const int32_t* list, int64_t n, const void* offsets, int off_is64, int64_t S,
+                         const void* weight, int weight_dtype, int mean, int32_t* src_pool_out, float* coef_out,
+                         const int64_t* batch, const int64_t* seq, int64_t n_features, int32_t* src_tile_out,
+                         void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(n >= 0 && S >= 0 && n_features >= 0, "negative size");
+  if (n == 0) return RECIS_OK;
+  RECIS_REQUIRE(list && offsets, "NULL argument");
+  RECIS_REQUIRE(S >= 1, "occurrences without a segment");
+  RECIS_REQUIRE(src_pool_out || src_tile_out, "nothing to fill");
+  RECIS_REQUIRE(coef_out == nullptr || src_pool_out, "coef_out goes with src_pool_out");
+  RECIS_REQUIRE(!src_pool_out || coef_out || (!weight && !mean), "coef_out is needed for weights or mean");
+  RECIS_REQUIRE(weight == nullptr || dtype_size(weight_dtype), "invalid weight dtype");
+  RECIS_REQUIRE(!src_tile_out || (batch && seq && n_features >= 1), "the padded gather needs its features");
+  FillArgs a{};
+  a.list = list;
+  a.n = n;
+  a.offsets = offsets;
+  a.off64 = off_is64;
+  a.S = S;
+  a.weight = weight;
+  a.wdt = weight_dtype;
+  a.mean = mean;
+  a.src_pool = src_pool_out;
+  a.coef = coef_out;
+  a.src_tile = src_tile_out;
+  const dim3 grid(static_cast<unsigned>((n + kBlock - 1) / kBlock));
+  if (!src_tile_out) {
+    a.first_group = 1;
+    fill_lists_kernel<<<grid, dim3(kBlock), 0, stream>>>(a);
+    RECIS_LAUNCH_CHECK();
+    return RECIS_OK;
+  }
+  int64_t seg = 0, row = 0;
+  for (int64_t f = 0; f < n_features; ++f) {
+    RECIS_REQUIRE(batch[f] >= 0 && seq[f] >= 0, "negative batch/seq");
+    seg += batch[f];
+  }
+  RECIS_REQUIRE(seg == S, "the features hold %lld segments, the offsets %lld", (long long)seg, (long long)S);
+  seg = 0;
+  for (int64_t f0 = 0; f0 < n_features; f0 += kFillFeatures) {  // kFillFeatures features per launch
+    a.n_features = static_cast<int>(std::min<int64_t>(kFillFeatures, n_features - f0));
+    a.first_group = f0 == 0;
+    for (int x = 0; x < a.n_features; ++x) {
+      a.seg_lo[x] = seg;
+      a.seq[x] = seq[f0 + x];
+      a.rbase[x] = row;
+      seg += batch[f0 + x];
+      row += batch[f0 + x] * seq[f0 + x];
+    }
+    a.seg_lo[a.n_features] = seg;
+    fill_lists_kernel<<<grid, dim3(kBlock), 0, stream>>>(a);
+    RECIS_LAUNCH_CHECK();
+  }
+  return RECIS_OK;
+}
+
+static CsrRequest one_input_request(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                    const void* coef, int coef_dtype, const int32_t* row_start,
+                                    const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
+                                    int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
+                                    void* stream_) {
+  CsrRequest r;
+  r.in1 = CsrInput{rows, rows_dtype, n_rows, src, coef, coef_dtype};
+  r.row_start = row_start;
+  r.hot_items = hot_items;
+  r.hot_cap = hot_cap;
+  r.counts_dev = counts_dev;
+  r.U = U;
+  r.D = D;
+  r.cover = cover_offsets;
+  r.cover64 = cover_is64;
+  r.cover_S = cover_S;
+  r.stream = static_cast<hipStream_t>(stream_);
+  return r;
+}
+
+int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
+                            int coef_dtype, const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
+                            const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t D,
+                            int accumulate, const void* cover_offsets, int cover_is64, int64_t cover_S,
+                            void* stream_) {
+  CsrRequest r = one_input_request(rows, rows_dtype, n_rows, src, coef, coef_dtype, row_start, hot_items, hot_cap,
+                                   counts_dev, U, D, cover_offsets, cover_is64, cover_S, stream_);
+  r.out = out;
+  r.out_dtype = out_dtype;
+  r.accumulate = accumulate;
+  return csr_gather_reduce_run<false>(r);
+}
+
+int recis_csr_gather_reduce_parts(const void* const* part_rows, const int64_t* part_counts, int n_parts,
+                                  int rows_dtype, const int32_t* src, const int32_t* row_start,
+                                  const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, void* out,
+                                  int64_t U, int64_t D, int accumulate, void* stream_) {
+  RECIS_REQUIRE(n_parts >= 1 && n_parts <= kMaxParts, "1 to %d parts (got %d)", kMaxParts, n_parts);
+  RECIS_REQUIRE(part_rows && part_counts, "NULL argument");
+  int64_t n_rows = 0;
+  for (int f = 0; f < n_parts; ++f) {
+    RECIS_REQUIRE(part_counts[f] >= 0 && (part_rows[f] != nullptr || part_counts[f] == 0), "bad part %d", f);
+    n_rows += part_counts[f];
+  }
+  CsrRequest r = one_input_request(nullptr, rows_dtype, n_rows, src, nullptr, 0, row_start, hot_items, hot_cap,
+                                   counts_dev, U, D, nullptr, 0, 0, stream_);
+  r.part_rows = part_rows;
+  r.part_counts = part_counts;
+  r.n_parts = n_parts;
+  r.out = out;
+  r.out_dtype = RECIS_F32;
+  r.accumulate = accumulate;
+  return csr_gather_reduce_run<false>(r);
+}
+
+int recis_csr_gather_reduce_adamw(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                  const void* coef, int coef_dtype, const int32_t* row_start,
+                                  const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
+                                  int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
+                                  const int64_t* row_index, void* const* emb_blocks_dev,
+                                  void* const* exp_avg_blocks_dev, void* const* exp_avg_sq_blocks_dev,
+                                  int64_t n_blocks, int64_t block_size, int row_dtype, void* beta1_t, void* beta2_t,
+                                  int beta_is_f64, double lr, double beta1, double beta2, double weight_decay,
+                                  double eps, void* stream_) {
+  RECIS_REQUIRE(beta1_t != nullptr && beta2_t != nullptr, "beta1_t / beta2_t must not be NULL");
+  FuseArgs f{};
+  if (U > 0) {
+    if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, exp_avg_blocks_dev, exp_avg_sq_blocks_dev, true, n_blocks,
+                                block_size, D, row_dtype))
+      return rc;
+  }
+  CsrRequest r = one_input_request(rows, rows_dtype, n_rows, src, coef, coef_dtype, row_start, hot_items, hot_cap,
+                                   counts_dev, U, D, cover_offsets, cover_is64, cover_S, stream_);
+  r.out_dtype = row_dtype;
+  r.epi = kEpiAdam;
+  r.fuse = &f;
+  return run_with_alpha<false>(r, f, beta1_t, beta2_t, beta_is_f64, lr, beta1, beta2, weight_decay, eps);
+}
+
+int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                    const void* coef, int coef_dtype, const int32_t* row_start,
+                                    const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
+                                    int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
+                                    const int64_t* row_index, void* const* emb_blocks_dev,
+                                    void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
+                                    int row_dtype, double lr, double eps, void* stream_) {
+  if (U == 0) return RECIS_OK;
+  FuseArgs f;
+  if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, accum_blocks_dev, nullptr, false, n_blocks, block_size, D,
+                              row_dtype))
+    return rc;
+  f.lr = static_cast<float>(lr);
+  f.eps = static_cast<float>(eps);
+  CsrRequest r = one_input_request(rows, rows_dtype, n_rows, src, coef, coef_dtype, row_start, hot_items, hot_cap,
+                                   counts_dev, U, D, cover_offsets, cover_is64, cover_S, stream_);
+  r.out_dtype = row_dtype;
+  r.epi = kEpiAdagrad;
+  r.fuse = &f;
+  return csr_gather_reduce_run<false>(r);
+}
+
+
+int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows,
+                          const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
+                          const int32_t* row_start, const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
+                          const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t n_out, int64_t D,
+                          void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE(U >= 0 && n_out >= 0, "negative size");
+  RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
+  if (U == 0 || n_out == 0) return RECIS_OK;
+  const bool blk = emb_blocks_dev != nullptr;
+  RECIS_REQUIRE(row_start && dst && out && counts_dev, "NULL argument");
+  RECIS_REQUIRE(blk ? (row_index != nullptr && n_blocks >= 1 && block_rows >= 1) : rows != nullptr,
+                "rows: a dense array or a block list with row_index");
+  RECIS_REQUIRE(hot_cap == 0 || hot_items, "hot_items must not be NULL");
+  const int in_sz = dtype_size(rows_dtype), out_sz = dtype_size(out_dtype);
+  RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
+  RECIS_REQUIRE(weight == nullptr || dtype_size(weight_dtype), "invalid weight dtype");
+  // block bases are allocator-aligned; a dense array brings its own alignment
+  const int vb_in = pick_vec_bytes(D * in_sz, blk ? 0 : reinterpret_cast<uintptr_t>(rows));
+  const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(out));
+  const int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
+  ExpArgs a;
+  a.row_start = row_start;
+  a.dst = dst;
+  a.weight = weight;
+  a.wdt = weight_dtype;
+  a.U = U;
+  a.n_out = n_out;
+  a.D = static_cast<int>(D);
+  a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
+  a.err = device_error_word(current_device());
+  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
+  a.row_index = row_index;
+  a.blocks = emb_blocks_dev;
+  a.block_rows = block_rows;
+  a.n_blocks = n_blocks;
+  a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
+  a.hot_items = hot_items;
+  a.counts = counts_dev;
+  a.hot_cap = hot_cap;
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
+  const int64_t hot_blocks = hot_cap > 0 ? std::min<int64_t>(hot_cap, 4096) : 0;
+  const dim3 grid(static_cast<unsigned>(a.cold_blocks + hot_blocks));
+  auto with_types = [&](auto tin, auto tout) {
+    using TIn = decltype(tin);
+    using TOut = decltype(tout);
+    return dispatch_vec(vec, [&](auto vtag) {
+      constexpr int VEC = decltype(vtag)::value;
+      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 16) {
+        return fail(RECIS_ERR_ARG, "internal: vector too wide");
+      } else {
+        RECIS_TIME_KERNEL("csr_expand_kernel", stream)
+        if (blk)
+          csr_expand_kernel<TIn, TOut, VEC, true><<<grid, dim3(kBlock), 0, stream>>>(nullptr, static_cast<TOut*>(out), a);
+        else
+          csr_expand_kernel<TIn, TOut, VEC, false><<<grid, dim3(kBlock), 0, stream>>>(static_cast<const TIn*>(rows),
+                                                                                    static_cast<TOut*>(out), a);
+        RECIS_LAUNCH_CHECK();
+        return RECIS_OK;
+      }
+    });
+  };
+  if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F32) return with_types(float{}, float{});
+  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_BF16) return with_types(bf16_t{}, bf16_t{});
+  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F16) return with_types(f16_t{}, f16_t{});
+  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_F32) return with_types(bf16_t{}, float{});
+  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F32) return with_types(f16_t{}, float{});
+  return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
+}
+
+}  // extern "C"

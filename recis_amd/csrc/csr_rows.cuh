@@ -1,0 +1,719 @@
+// Gather-reduce over the occurrence lists of a batch plan (kernels and their launcher), shared by
+// the translation units that instantiate them: out[u] = sum over the list entries k of unique id u
+// of coef[k] * rows[src[k]], from one input or from two (the gradients of two outputs of one
+// lookup), ending in a store or in the optimizer's update of the table row.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <climits>
+#include <type_traits>
+
+#include "common.cuh"
+#include "optim_rows.cuh"
+
+namespace recis_hip {
+namespace {
+
+constexpr int kHotLen = RECIS_PLAN_HOT_LEN;      // rows with more occurrences than this are "hot"
+constexpr int kHotChunk = RECIS_PLAN_HOT_CHUNK;  // occurrences per hot work item
+
+__device__ __forceinline__ float load_coef(const void* w, int wdt, int64_t i) {
+  if (wdt == RECIS_F32) return static_cast<const float*>(w)[i];
+  if (wdt == RECIS_BF16) return to_float(static_cast<const bf16_t*>(w)[i]);
+  return to_float(static_cast<const f16_t*>(w)[i]);
+}
+
+constexpr int kMaxParts = 8;  // input arrays of one gather-reduce launch (PARTS kernels)
+
+struct CsrArgs {
+  const int32_t* row_start;  // [U + 1]
+  const int32_t* src;        // [n] input row per list entry (negative = skip)
+  const void* coef;          // [n] per list entry, or NULL
+  int coef_dt;
+  int64_t U, n_rows;
+  int D;
+  int lpr_log2;
+  int accumulate;
+  int nt_in;  // the gathered rows are too many to stay cached: non-temporal loads
+  // a second input over the same lists (kernels with TIn2 != void): entry k also adds
+  // coef2[k] * rows2[src2[k]]; the cover range does not apply to it
+  const void* rows2;
+  const int32_t* src2;
+  const void* coef2;
+  int coef2_dt;
+  int nt_in2;
+  int64_t n_rows2;
+  int* err;
+  const void* cover;  // offsets [cover_S + 1] or NULL: entries whose src lies outside
+  int cover64;        // [cover[0], cover[cover_S]) are skipped
+  int64_t cover_S;
+  // hot rows (more than hot_len occurrences): (row, chunk) work items, partial sums per item
+  int32_t hot_len;           // INT_MAX when the caller brings no work items: every row is "cold"
+  const int32_t* hot_items;  // [2 * hot_cap]
+  const int64_t* counts;     // counts[1] = number of items
+  int64_t hot_cap;
+  float* hot_part;           // [hot_cap, D]
+  int64_t cold_blocks;       // the last cold_blocks workgroups work per row, the ones before per hot item
+  // PARTS kernels: the input rows are n_parts arrays laid end to end in src's numbering; part f
+  // holds rows [part_lo[f], part_lo[f + 1])
+  int n_parts;
+  const void* part_rows[kMaxParts];
+  int64_t part_lo[kMaxParts + 1];
+};
+
+// What a gather-reduce launch does with the finished sum of row u (template parameter EPI):
+//   kEpiStore    out[u] (+)= sum
+//   kEpiAdam     the sum is the gradient of table row row_index[u]: the Adam-family update of that
+//                row (parameter and both moments) is applied at once, the gradient never written
+//   kEpiAdagrad  the same with the Adagrad update
+enum { kEpiStore = 0, kEpiAdam = 1, kEpiAdagrad = 2 };
+struct FuseArgs {
+  const int64_t* row_index;  // [U]; a negative index skips the row
+  void* const* emb;          // block tables (device arrays of block pointers)
+  void* const* s0;           // exp_avg / the Adagrad accumulator
+  void* const* s1;           // exp_avg_sq
+  RowBlocks rb;
+  AdamCoef adam;
+  float lr, eps;             // Adagrad
+};
+
+// The epilogue of one pack of one finished row; T = the table's row type for the optimizer kinds.
+// idx = row_index[u] of the finished row (callers load it early: it heads a chain of dependent accesses).
+template <typename T, int VEC, int EPI>
+__device__ __forceinline__ void fused_row_update(const FuseArgs& f, int* err, int64_t idx, int c0,
+                                                 const float (&acc)[VEC]) {
+  int64_t b, off;
+  if (idx < 0) return;  // a key the table does not hold takes no gradient
+  if (!block_row(f.rb, idx, b, off)) {
+    raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
+    return;
+  }
+  const int64_t at = off * f.rb.D + c0;
+  if constexpr (EPI == kEpiAdam) {
+    adam_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at,
+                             static_cast<T*>(f.s1[b]) + at, acc, f.adam.alpha[0], f.adam);
+  } else {
+    adagrad_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at, acc, f.lr, f.eps);
+  }
+}
+
+// One input as a kernel sees it: entries whose src lies outside [lo, hi) are skipped, those at or
+// past n_rows raise the index-range error.
+template <typename T>
+struct SrcView {
+  const T* rows;
+  const int32_t* src;
+  const void* coef;
+  int coef_dt;
+  int nt;
+  int64_t n_rows, lo, hi;
+};
+
+// Row s of the input: of the one array, or of the part that holds it.
+template <typename TIn, bool PARTS>
+__device__ __forceinline__ const TIn* src_row(const TIn* rows, const CsrArgs& a, int64_t s) {
+  if constexpr (!PARTS) {
+    return rows + s * a.D;
+  } else {
+    int f = 0;
+#pragma unroll
+    for (int k = 1; k < kMaxParts; ++k) f += (k < a.n_parts && s >= a.part_lo[k]) ? 1 : 0;
+    const TIn* base = static_cast<const TIn*>(a.part_rows[0]);
+    int64_t lo = 0;
+#pragma unroll
+    for (int k = 1; k < kMaxParts; ++k) {
+      if (k == f) {
+        base = static_cast<const TIn*>(a.part_rows[k]);
+        lo = a.part_lo[k];
+      }
+    }
+    return base + (s - lo) * a.D;
+  }
+}
+
+__device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64_t& hi) {
+  lo = 0;
+  hi = a.n_rows;
+  if (a.cover) {
+    lo = max(lo, load_index(a.cover, a.cover64, 0));
+    hi = min(hi, load_index(a.cover, a.cover64, a.cover_S));
+  }
+}
+
+// A whole wave works the list entries [e_begin, e_end) (uniform arguments, every lane calls):
+// `src` and `coef` of 64 entries come from one coalesced load, a lane each, and reach the lanes
+// that gather the rows through shuffles; lane group g of `groups` takes entries g, g + groups,
+// ... with several row loads in flight. acc: this group's partial sum for columns
+// c0 .. c0 + VEC (the caller folds the groups).
+template <typename TIn, int VEC, bool PARTS>
+__device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const CsrArgs& a, int32_t e_begin,
+                                                  int32_t e_end, int c0, bool col_ok, int g, int groups,
+                                                  float (&acc)[VEC]) {
+  constexpr int kFly = VEC >= 8 ? 4 : 8;  // row loads in flight per lane
+  const int lane = threadIdx.x & (kWave - 1);
+  for (int32_t cb = e_begin; cb < e_end; cb += kWave) {
+    const int n_here = min(kWave, e_end - cb);
+    int32_t s_mine = -1;
+    float w_mine = 0.f;
+    if (lane < n_here) {
+      const int32_t sv = s.src[cb + lane];
+      if (sv >= s.lo && sv < s.hi) {
+        s_mine = sv;
+        w_mine = s.coef ? load_coef(s.coef, s.coef_dt, cb + lane) : 1.0f;
+      } else if (static_cast<int64_t>(sv) >= s.n_rows) {
+        raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      }
+    }
+    for (int q0 = 0; q0 < n_here; q0 += kFly * groups) {  // same trip count for the whole wave (shuffles inside)
+      float v[kFly][VEC];
+      float w[kFly];
+#pragma unroll
+      for (int k = 0; k < kFly; ++k) {
+        const int e = q0 + g + k * groups;
+        const int from = min(e, kWave - 1);
+        int32_t id = __shfl(s_mine, from, kWave);
+        w[k] = s.coef ? __shfl(w_mine, from, kWave) : 1.0f;
+        if (e >= n_here || !col_ok) id = -1;
+        if (id >= 0) {
+          const TIn* row = src_row<TIn, PARTS>(s.rows, a, id);
+          if (s.nt) {
+            load_pack_stream<TIn, VEC>(row + c0, v[k]);
+          } else {
+            load_pack<TIn, VEC>(row + c0, v[k]);
+          }
+        } else {
+          w[k] = 0.f;
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[k][j] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kFly; ++k) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[k][j], w[k], acc[j]);
+      }
+    }
+  }
+}
+
+constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of a wave
+
+// One launch for all rows. The last cold_blocks workgroups: one group of LPR lanes per unique row
+// with at most hot_len occurrences ("cold"); a wave that holds a row with more than kCoopLen
+// occurrences works that row with all its lane groups striding over the list (a row of 200
+// occurrences would otherwise be 50 dependent gathers of one group). The first workgroups
+// walk the hot work items (row, chunk of kHotChunk occurrences): four waves share the chunk,
+// fold their sums through LDS and store ONE partial row per item; csr_hot_finish_kernel adds up
+// the partial rows of every hot row in chunk order. No atomics anywhere.
+// SHUFFLE: long lists go through wave_gather_range (pays off when a wave has at most eight lane
+// groups, i.e. rows of 128 bytes and more); otherwise every group loads its own entries.
+// TIn2 != void: every list entry adds a row of a second input as well (see CsrArgs).
+template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false, int EPI = kEpiStore,
+          typename TIn2 = void>
+__global__ void __launch_bounds__(kBlock, (!SHUFFLE && EPI != kEpiStore && (std::is_void<TIn2>::value || sizeof(TOut) == 4))
+                                              ? 8 : 1)  // 64 registers where that costs no spills
+csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
+  constexpr bool TWO = !std::is_void<TIn2>::value;
+  static_assert(!(TWO && PARTS), "a second input goes with one array as the first");
+  using TSecond = typename std::conditional<TWO, TIn2, TIn>::type;
+  extern __shared__ float s_part[];  // [waves][D], hot part only
+  const int D = a.D;
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
+  const int g = lane >> a.lpr_log2;        // this lane's group in its wave
+  SrcView<TIn> in1{rows, a.src, a.coef, a.coef_dt, a.nt_in, a.n_rows, 0, 0};
+  cover_range(a, in1.lo, in1.hi);
+  const SrcView<TSecond> in2{static_cast<const TSecond*>(a.rows2), a.src2, a.coef2, a.coef2_dt, a.nt_in2,
+                             a.n_rows2, 0, a.n_rows2};
+
+  auto fetch = [&](const auto& in, auto parts, int32_t k, int c0, float (&v)[VEC], float& w) {
+    using T = typename std::remove_cv<typename std::remove_pointer<decltype(in.rows)>::type>::type;
+    const int32_t s = in.src[k];
+    w = in.coef ? load_coef(in.coef, in.coef_dt, k) : 1.0f;
+    if (s < in.lo || s >= in.hi) {
+      if (static_cast<int64_t>(s) >= in.n_rows) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
+      w = 0.f;
+      return;
+    }
+    const T* row = src_row<T, decltype(parts)::value>(in.rows, a, s);
+    if (in.nt) {
+      load_pack_stream<T, VEC>(row + c0, v);
+    } else {
+      load_pack<T, VEC>(row + c0, v);
+    }
+  };
+  // acc += sum over list entries k = first, first + step, ... < last of one input (4 gathers in flight)
+  auto gather_one = [&](const auto& in, auto parts, int32_t first, int32_t last, int32_t step, int c0,
+                        float (&acc)[VEC]) {
+    int32_t k = first;
+    for (; k + 3 * step < last; k += 4 * step) {
+      float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
+      float w0, w1, w2, w3;
+      fetch(in, parts, k, c0, v0, w0);
+      fetch(in, parts, k + step, c0, v1, w1);
+      fetch(in, parts, k + 2 * step, c0, v2, w2);
+      fetch(in, parts, k + 3 * step, c0, v3, w3);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        acc[j] = fmaf(v0[j], w0, acc[j]);
+        acc[j] = fmaf(v1[j], w1, acc[j]);
+        acc[j] = fmaf(v2[j], w2, acc[j]);
+        acc[j] = fmaf(v3[j], w3, acc[j]);
+      }
+    }
+    for (; k < last; k += step) {
+      float v0[VEC];
+      float w0;
+      fetch(in, parts, k, c0, v0, w0);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v0[j], w0, acc[j]);
+    }
+  };
+  // the first input's entries, then the second's: one fixed order of summation
+  auto gather_sum = [&](int32_t first, int32_t last, int32_t step, int c0, float (&acc)[VEC]) {
+    gather_one(in1, std::integral_constant<bool, PARTS>{}, first, last, step, c0, acc);
+    if constexpr (TWO) gather_one(in2, std::false_type{}, first, last, step, c0, acc);
+  };
+  // the wave's sum over the list entries [first, last) for columns c0.., the same in every group
+  auto wave_sum = [&](int32_t first, int32_t last, int c0, bool col_ok, float (&acc)[VEC]) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    if constexpr (SHUFFLE) {
+      wave_gather_range<TIn, VEC, PARTS>(in1, a, first, last, c0, col_ok, g, groups, acc);
+      if constexpr (TWO) wave_gather_range<TSecond, VEC, false>(in2, a, first, last, c0, col_ok, g, groups, acc);
+    } else {
+      if (col_ok) gather_sum(first + g, last, groups, c0, acc);
+    }
+    for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+    }
+  };
+
+  const int64_t hot_blocks = static_cast<int64_t>(gridDim.x) - a.cold_blocks;
+  if (static_cast<int64_t>(blockIdx.x) < hot_blocks) {
+    // ---- hot work items (the first workgroups: the longest-running ones start first)
+    int64_t n_items = a.counts[1];
+    if (n_items > a.hot_cap) n_items = a.hot_cap;
+    const int wave = threadIdx.x / kWave;
+    constexpr int n_waves = kBlock / kWave;
+    for (int64_t item = blockIdx.x; item < n_items; item += hot_blocks) {
+      const int32_t u = a.hot_items[2 * item];
+      const int32_t chunk = a.hot_items[2 * item + 1];
+      const int32_t start = a.row_start[u] + chunk * kHotChunk;
+      const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
+      const int32_t per_wave = (end - start + n_waves - 1) / n_waves;  // a contiguous share per wave
+      const int32_t w_begin = min(end, start + wave * per_wave), w_end = min(end, w_begin + per_wave);
+      for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+        const int c0 = cbase + cl * VEC;
+        const bool col_ok = c0 < D;
+        float acc[VEC];
+        wave_sum(w_begin, w_end, c0, col_ok, acc);
+        if (g == 0 && col_ok) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) s_part[wave * D + c0 + j] = acc[j];
+        }
+      }
+      __syncthreads();
+      for (int d = threadIdx.x; d < D; d += kBlock) {
+        float sum = 0.f;
+        for (int w = 0; w < n_waves; ++w) sum += s_part[w * D + d];
+        a.hot_part[item * D + d] = sum;
+      }
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ---- cold rows
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
+  const bool valid = u < a.U;
+  const int32_t start = valid ? a.row_start[u] : 0;
+  int32_t end = valid ? a.row_start[u + 1] : 0;
+  const bool hot = end - start > a.hot_len;  // left to the work items and the finish kernel
+  if (hot) end = start;
+  int64_t idx_mine = -1;  // the table row of this group's unique id, asked for before the gathers
+  if constexpr (EPI != kEpiStore) {
+    if (valid && !hot) idx_mine = f.row_index[u];
+  }
+  // the finished sum of this lane group's own row u
+  auto finish = [&](int64_t row, int c0, float (&acc)[VEC]) {
+    if constexpr (EPI != kEpiStore) {
+      fused_row_update<TOut, VEC, EPI>(f, a.err, idx_mine, c0, acc);
+    } else {
+      TOut* dst = out + row * D + c0;
+      if (a.accumulate) {
+        float old[VEC];
+        load_pack<TOut, VEC>(dst, old);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += old[j];
+      }
+      store_pack<TOut, VEC>(dst, acc);
+    }
+  };
+  // short rows: every lane group works its own row
+  const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;  // with one group per wave there is nobody to share with
+  if (valid && !is_long && !hot) {
+    // (Asking for the row's parameter and state packs before the gradient is gathered, to run their
+    // latency under that of the gathers, was measured and lost: 150 -> 205 us in config 4. The packs
+    // cost registers, hence resident waves, and the gathers then queue behind the table reads.)
+    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+      float acc[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+      gather_sum(start, end, 1, c0, acc);
+      finish(u, c0, acc);
+    }
+  }
+  // long rows of this wave, one after the other, summed by all its lane groups; the owning group
+  // keeps the sum and every group finishes its row afterwards, all at once (a finish that updates
+  // the table row is a chain of dependent accesses: one per row in a row would leave the wave
+  // waiting on it with three quarters of its lanes idle). A wave with several groups has lanes for
+  // all of D (lpr_log2 < 6), so a long row is one pack per lane.
+  uint64_t todo = __ballot(is_long);
+  if (todo == 0) return;
+  const int c0 = cl * VEC;
+  const bool col_ok = c0 < D;
+  float keep[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) keep[j] = 0.f;
+  while (todo) {
+    const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;  // first lane of the owning group
+    todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);  // the group's lanes (fewer than 64 here)
+    const int r = owner >> a.lpr_log2;
+    const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
+    float acc[VEC];
+    wave_sum(r_start, r_end, c0, col_ok, acc);
+    if (g == r) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) keep[j] = acc[j];
+    }
+  }
+  if (is_long && col_ok) finish(u, c0, keep);
+}
+
+// out[u] (+)= sum of the partial rows of hot row u (or the optimizer's update of the row with that
+// sum). One wave per work item with chunk 0 (the items of a row are consecutive): its lane groups
+// share the row's partials out among themselves (an id that makes up a tenth of the batch has a
+// hundred of them) and fold their sums with shuffles, always in the same order.
+template <typename TOut, int VEC, int EPI = kEpiStore>
+__global__ void __launch_bounds__(kBlock)
+csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
+  int64_t n_items = a.counts[1];
+  if (n_items > a.hot_cap) n_items = a.hot_cap;
+  const int D = a.D;
+  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int groups = kWave >> a.lpr_log2, g = lane >> a.lpr_log2;
+  const int64_t waves_total = static_cast<int64_t>(gridDim.x) * (kBlock / kWave);
+  for (int64_t item = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave; item < n_items;
+       item += waves_total) {  // uniform in the wave
+    if (a.hot_items[2 * item + 1] != 0) continue;
+    const int32_t u = a.hot_items[2 * item];
+    const int32_t len = a.row_start[u + 1] - a.row_start[u];
+    int64_t n_chunks = (len + kHotChunk - 1) / kHotChunk;
+    if (item + n_chunks > n_items) n_chunks = n_items - item;  // items cut off by hot_cap (cannot happen with the documented hot_cap)
+    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+      const int c0 = cbase + cl * VEC;
+      const bool col_ok = c0 < D;
+      float acc[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+      if (col_ok) {
+        for (int64_t k = g; k < n_chunks; k += groups) {
+          float v[VEC];
+          load_pack<float, VEC>(a.hot_part + (item + k) * D + c0, v);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) acc[j] += v[j];
+        }
+      }
+      for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
+      }
+      if (g != 0 || !col_ok) continue;
+      if constexpr (EPI != kEpiStore) {
+        fused_row_update<TOut, VEC, EPI>(f, a.err, f.row_index[u], c0, acc);
+      } else {
+        TOut* dst = out + static_cast<int64_t>(u) * D + c0;
+        if (a.accumulate) {
+          float old[VEC];
+          load_pack<TOut, VEC>(dst, old);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) acc[j] += old[j];
+        }
+        store_pack<TOut, VEC>(dst, acc);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------ expand (transpose of the gather-reduce)
+// out[dst[k], :] = w[dst[k]] * row(u) for every list entry k of every unique id u: the forward
+// of pooling when every segment holds exactly one id, and of the unpooled (tile) output. Each
+// unique row is read ONCE and stored to all its occurrences; stores do not wait for anything,
+
+template <typename F>
+int dispatch_vec(int vec, F&& f) {
+  switch (vec) {
+    case 8: return f(std::integral_constant<int, 8>{});
+    case 4: return f(std::integral_constant<int, 4>{});
+    case 2: return f(std::integral_constant<int, 2>{});
+    case 1: return f(std::integral_constant<int, 1>{});
+    default: return fail(RECIS_ERR_ARG, "unsupported vector width %d", vec);
+  }
+}
+
+// ------------------------------------------------------------------ host side
+// One input of a gather-reduce as the caller describes it.
+struct CsrInput {
+  const void* rows;
+  int dtype;
+  int64_t n_rows;
+  const int32_t* src;
+  const void* coef;  // or NULL
+  int coef_dtype;
+};
+
+struct CsrRequest {
+  CsrInput in1;
+  const CsrInput* in2 = nullptr;                // the second input, with csr_gather_reduce_run<true>
+  const void* const* part_rows = nullptr;       // in1 as n_parts arrays laid end to end (in1.rows is NULL then)
+  const int64_t* part_counts = nullptr;
+  int n_parts = 0;
+  const int32_t* row_start = nullptr;
+  const int32_t* hot_items = nullptr;
+  int64_t hot_cap = 0;
+  const int64_t* counts_dev = nullptr;
+  void* out = nullptr;                          // NULL when epi != kEpiStore
+  int out_dtype = RECIS_F32;                    // the table's row type when epi != kEpiStore
+  int64_t U = 0, D = 0;
+  int accumulate = 0;
+  const void* cover = nullptr;
+  int cover64 = 0;
+  int64_t cover_S = 0;
+  hipStream_t stream = nullptr;
+  int epi = kEpiStore;
+  const FuseArgs* fuse = nullptr;               // where the table rows are, when epi != kEpiStore
+  size_t extra_ws = 0;                          // bytes of the stream's workspace (after the partial rows of the
+  void** extra_out = nullptr;                   // hot items) handed to the caller before anything is launched
+};
+
+// Checks, geometry, workspace and the launches of one gather-reduce. TWO picks the family of
+// kernels this translation unit instantiates: one input (any supported pair of input and output
+// types, PARTS included) or two inputs (the first fp32, the second fp32 or a half type).
+template <bool TWO>
+int csr_gather_reduce_run(const CsrRequest& r) {
+  const int64_t U = r.U, D = r.D, hot_cap = r.hot_cap;
+  const int epi = r.epi, n_parts = r.n_parts;
+  hipStream_t stream = r.stream;
+  RECIS_REQUIRE(U >= 0 && r.in1.n_rows >= 0, "negative size");
+  RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
+  RECIS_REQUIRE(U == 0 || (r.in1.src && r.row_start && (r.out || epi != kEpiStore) && r.counts_dev), "NULL argument");
+  RECIS_REQUIRE(n_parts > 0 || r.in1.rows != nullptr || r.in1.n_rows == 0, "rows must not be NULL");
+  RECIS_REQUIRE(hot_cap == 0 || r.hot_items, "hot_items must not be NULL");
+  const int in_sz = dtype_size(r.in1.dtype), out_sz = dtype_size(r.out_dtype);
+  RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
+  RECIS_REQUIRE(r.in1.coef == nullptr || dtype_size(r.in1.coef_dtype), "invalid coef dtype");
+  uintptr_t align_of = reinterpret_cast<uintptr_t>(r.in1.rows);
+  for (int f = 0; f < n_parts; ++f) align_of |= reinterpret_cast<uintptr_t>(r.part_rows[f]);  // the coarsest alignment
+  // with two inputs the first is fp32 and may go in 32-byte packs, so that a half-precision second
+  // input still gets its 16 bytes per lane
+  const int vb_in = TWO ? pick_vec_bytes_max(D * in_sz, align_of, 32) : pick_vec_bytes(D * in_sz, align_of);
+  // table blocks are allocator-aligned and are read and written in 16-byte packs at most
+  const int vb_out = epi != kEpiStore ? pick_vec_bytes(D * out_sz, 16)
+                                      : pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(r.out), 32);
+  int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
+  CsrArgs a{};
+  if constexpr (TWO) {
+    RECIS_REQUIRE(r.in2 != nullptr && n_parts == 0, "two inputs: the second must be given, the first one array");
+    const CsrInput& b = *r.in2;
+    const int in2_sz = dtype_size(b.dtype);
+    RECIS_REQUIRE(in2_sz, "invalid dtype of the second input");
+    RECIS_REQUIRE(b.n_rows >= 0 && (U == 0 || b.src), "second input: src must not be NULL");
+    RECIS_REQUIRE(b.rows != nullptr || b.n_rows == 0, "second input: rows must not be NULL");
+    RECIS_REQUIRE(b.coef == nullptr || dtype_size(b.coef_dtype), "invalid coef dtype of the second input");
+    vec = std::max(1, std::min(vec, pick_vec_bytes(D * in2_sz, reinterpret_cast<uintptr_t>(b.rows)) / in2_sz));
+    a.rows2 = b.rows;
+    a.src2 = b.src;
+    a.coef2 = b.coef;
+    a.coef2_dt = b.coef_dtype;
+    a.n_rows2 = b.n_rows;
+    a.nt_in2 = b.n_rows * D * in2_sz >= (int64_t(1) << 30);
+  }
+  a.row_start = r.row_start;
+  a.src = r.in1.src;
+  a.coef = r.in1.coef;
+  a.coef_dt = r.in1.coef_dtype;
+  a.U = U;
+  a.n_rows = r.in1.n_rows;
+  a.cover = r.cover;
+  a.cover64 = r.cover64;
+  a.cover_S = r.cover_S;
+  a.D = static_cast<int>(D);
+  a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
+  a.accumulate = r.accumulate;
+  a.nt_in = r.in1.n_rows * D * in_sz >= (int64_t(1) << 30);
+  a.err = device_error_word(current_device());
+  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
+  const int rows_per_block = kBlock >> a.lpr_log2;
+  a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
+  a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
+  a.hot_items = r.hot_items;
+  a.counts = r.counts_dev;
+  a.hot_cap = hot_cap;
+  a.hot_part = nullptr;
+  a.n_parts = n_parts;
+  a.part_lo[0] = 0;
+  for (int f = 0; f < kMaxParts; ++f) {
+    a.part_rows[f] = f < n_parts ? r.part_rows[f] : nullptr;
+    a.part_lo[f + 1] = a.part_lo[f] + (f < n_parts ? r.part_counts[f] : 0);
+  }
+  int64_t hot_blocks = 0;
+  if (hot_cap > 0 || r.extra_ws > 0) {
+    void* ws = nullptr;
+    const size_t hot_bytes = (sizeof(float) * static_cast<size_t>(hot_cap) * static_cast<size_t>(D) + 255) & ~size_t(255);
+    if (int rc = get_workspace(stream, hot_bytes + r.extra_ws, &ws)) return rc;
+    a.hot_part = static_cast<float*>(ws);
+    if (r.extra_out) *r.extra_out = static_cast<char*>(ws) + hot_bytes;
+    if (hot_cap > 0) hot_blocks = std::min<int64_t>(hot_cap, 4096);
+  }
+  if (U == 0) return RECIS_OK;
+  const FuseArgs f = r.fuse ? *r.fuse : FuseArgs{};
+  const size_t lds = sizeof(float) * (kBlock / kWave) * static_cast<size_t>(D);
+  auto with_types = [&](auto tin, auto tout, auto tin2) {
+    using TIn = decltype(tin);
+    using TOut = decltype(tout);
+    using TIn2 = typename std::conditional<TWO, decltype(tin2), void>::type;
+    constexpr size_t in2_bytes = TWO ? sizeof(decltype(tin2)) : 1;
+    return dispatch_vec(vec, [&](auto vtag) {
+      constexpr int VEC = decltype(vtag)::value;
+      if constexpr (VEC * sizeof(TIn) > (TWO ? 32 : 16) || VEC * in2_bytes > 16 || VEC * sizeof(TOut) > 32) {
+        return fail(RECIS_ERR_ARG, "internal: vector too wide");
+      } else {
+        const TIn* rin = static_cast<const TIn*>(r.in1.rows);
+        TOut* o = static_cast<TOut*>(r.out);
+        const bool shuffle = a.lpr_log2 >= 3;  // at most eight lane groups per wave
+        const dim3 grid(a.cold_blocks + hot_blocks), block(kBlock);
+        const int64_t fin = std::min<int64_t>((hot_cap + kBlock / kWave - 1) / (kBlock / kWave), 2048);  // a wave per item
+        auto launch = [&](auto epi_tag) {
+          constexpr int EPI = decltype(epi_tag)::value;
+          {
+            RECIS_TIME_KERNEL(EPI == kEpiStore ? "csr_rows_kernel" : EPI == kEpiAdam ? "csr_rows_adam_kernel"
+                                                                                      : "csr_rows_adagrad_kernel", stream)
+            if (n_parts > 0) {
+              if constexpr (sizeof(TOut) == 4 && EPI == kEpiStore && !TWO) {  // parts go to fp32 rows only
+                if (shuffle)
+                  csr_rows_kernel<TIn, TOut, VEC, true, true><<<grid, block, lds, stream>>>(rin, o, a, f);
+                else
+                  csr_rows_kernel<TIn, TOut, VEC, false, true><<<grid, block, lds, stream>>>(rin, o, a, f);
+              }
+            } else if (shuffle) {
+              csr_rows_kernel<TIn, TOut, VEC, true, false, EPI, TIn2><<<grid, block, lds, stream>>>(rin, o, a, f);
+            } else {
+              csr_rows_kernel<TIn, TOut, VEC, false, false, EPI, TIn2><<<grid, block, lds, stream>>>(rin, o, a, f);
+            }
+            RECIS_LAUNCH_CHECK();
+          }
+          if (hot_cap > 0) {
+            csr_hot_finish_kernel<TOut, VEC, EPI><<<dim3(fin), block, 0, stream>>>(o, a, f);
+            RECIS_LAUNCH_CHECK();
+          }
+          return RECIS_OK;
+        };
+        if (epi == kEpiAdam) {
+          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdam>{});
+        } else if (epi == kEpiAdagrad) {
+          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdagrad>{});
+        } else {
+          return launch(std::integral_constant<int, kEpiStore>{});
+        }
+        return fail(RECIS_ERR_ARG, "internal: vector too wide for a fused row update");
+      }
+    });
+  };
+  const int rows_dtype = r.in1.dtype, out_dtype = r.out_dtype;
+  if constexpr (!TWO) {
+    if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F32) return with_types(float{}, float{}, 0);
+    if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_F32) return with_types(bf16_t{}, float{}, 0);
+    if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F32) return with_types(f16_t{}, float{}, 0);
+    if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_BF16) return with_types(bf16_t{}, bf16_t{}, 0);
+    if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F16) return with_types(f16_t{}, f16_t{}, 0);
+    if (epi != kEpiStore) {  // fp32 gradients onto half-precision rows
+      if (rows_dtype == RECIS_F32 && out_dtype == RECIS_BF16) return with_types(float{}, bf16_t{}, 0);
+      if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F16) return with_types(float{}, f16_t{}, 0);
+    }
+    return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
+  } else {
+    // the first input fp32 (a pooled output's gradient); the second fp32 or of the output's type
+    // (the gradient of an output that has the table's row type)
+    const int d2 = r.in2->dtype;
+    RECIS_REQUIRE(rows_dtype == RECIS_F32, "two inputs: the first must be fp32 (got dtype %d)", rows_dtype);
+    if (out_dtype == RECIS_F32) {
+      if (d2 == RECIS_F32) return with_types(float{}, float{}, float{});
+      if (epi == kEpiStore) {
+        if (d2 == RECIS_BF16) return with_types(float{}, float{}, bf16_t{});
+        if (d2 == RECIS_F16) return with_types(float{}, float{}, f16_t{});
+      }
+    } else if (epi != kEpiStore) {
+      if (out_dtype == RECIS_BF16 && d2 == RECIS_F32) return with_types(float{}, bf16_t{}, float{});
+      if (out_dtype == RECIS_BF16 && d2 == RECIS_BF16) return with_types(float{}, bf16_t{}, bf16_t{});
+      if (out_dtype == RECIS_F16 && d2 == RECIS_F32) return with_types(float{}, f16_t{}, float{});
+      if (out_dtype == RECIS_F16 && d2 == RECIS_F16) return with_types(float{}, f16_t{}, f16_t{});
+    }
+    return fail(RECIS_ERR_ARG, "unsupported dtypes (second input=%d, out=%d)", d2, out_dtype);
+  }
+}
+
+// Shared front of the fused entry points: argument checks and the table description.
+inline int fill_fuse_args(FuseArgs& f, const int64_t* row_index, void* const* emb, void* const* s0, void* const* s1,
+                          bool need_s1, int64_t n_blocks, int64_t block_size, int64_t D, int row_dtype) {
+  RECIS_REQUIRE(row_index && emb && s0 && (s1 || !need_s1), "row_index and the block tables must not be NULL");
+  RECIS_REQUIRE(n_blocks >= 1 && block_size >= 1, "bad block geometry (n_blocks=%lld block_size=%lld)",
+                (long long)n_blocks, (long long)block_size);
+  RECIS_REQUIRE(dtype_size(row_dtype), "invalid row dtype");
+  f = FuseArgs{};
+  f.row_index = row_index;
+  f.emb = emb;
+  f.s0 = s0;
+  f.s1 = s1;
+  f.rb.n_blocks = n_blocks;
+  f.rb.block_size = block_size;
+  f.rb.D = static_cast<int>(D);
+  return RECIS_OK;
+}
+
+
+// The Adam-family variant of a request (r.epi == kEpiAdam, r.fuse == &f). The running powers of
+// the betas advance first, even when no row is touched (cal_alpha); alpha lives in the stream's
+// workspace behind the partial rows of the hot items, so a first pass with U = 0 reserves the
+// workspace and learns where alpha goes, launching nothing.
+template <bool TWO>
+int run_with_alpha(CsrRequest& r, FuseArgs& f, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
+                   double beta1, double beta2, double weight_decay, double eps) {
+  void* alpha = nullptr;
+  CsrRequest probe = r;
+  probe.U = 0;
+  probe.extra_ws = 256;
+  probe.extra_out = &alpha;
+  if (int rc = csr_gather_reduce_run<TWO>(probe)) return rc;
+  if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, static_cast<double*>(alpha), lr, beta1, beta2, r.stream))
+    return rc;
+  if (r.U == 0) return RECIS_OK;
+  f.adam.alpha = static_cast<const double*>(alpha);
+  f.adam.beta1 = beta1;
+  f.adam.beta2 = beta2;
+  f.adam.decay = weight_decay;
+  f.adam.eps = eps;
+  r.extra_ws = 256;
+  r.extra_out = &alpha;
+  return csr_gather_reduce_run<TWO>(r);
+}
+
+}  // namespace
+}  // namespace recis_hip

@@ -1181,594 +1181,6 @@ __global__ void plan_empty_kernel(int64_t* __restrict__ counts, int32_t* __restr
   }
 }
 
-// ---------------------------------------------------------------- consumers
-__device__ __forceinline__ float load_coef(const void* w, int wdt, int64_t i) {
-  if (wdt == RECIS_F32) return static_cast<const float*>(w)[i];
-  if (wdt == RECIS_BF16) return to_float(static_cast<const bf16_t*>(w)[i]);
-  return to_float(static_cast<const f16_t*>(w)[i]);
-}
-
-constexpr int kMaxParts = 8;  // input arrays of one gather-reduce launch (PARTS kernels)
-
-struct CsrArgs {
-  const int32_t* row_start;  // [U + 1]
-  const int32_t* src;        // [n] input row per list entry (negative = skip)
-  const void* coef;          // [n] per list entry, or NULL
-  int coef_dt;
-  int64_t U, n_rows;
-  int D;
-  int lpr_log2;
-  int accumulate;
-  int nt_in;  // the gathered rows are too many to stay cached: non-temporal loads
-  int* err;
-  const void* cover;  // offsets [cover_S + 1] or NULL: entries whose src lies outside
-  int cover64;        // [cover[0], cover[cover_S]) are skipped
-  int64_t cover_S;
-  // hot rows (more than hot_len occurrences): (row, chunk) work items, partial sums per item
-  int32_t hot_len;           // INT_MAX when the caller brings no work items: every row is "cold"
-  const int32_t* hot_items;  // [2 * hot_cap]
-  const int64_t* counts;     // counts[1] = number of items
-  int64_t hot_cap;
-  float* hot_part;           // [hot_cap, D]
-  int64_t cold_blocks;       // the last cold_blocks workgroups work per row, the ones before per hot item
-  // PARTS kernels: the input rows are n_parts arrays laid end to end in src's numbering; part f
-  // holds rows [part_lo[f], part_lo[f + 1])
-  int n_parts;
-  const void* part_rows[kMaxParts];
-  int64_t part_lo[kMaxParts + 1];
-};
-
-// What a gather-reduce launch does with the finished sum of row u (template parameter EPI):
-//   kEpiStore    out[u] (+)= sum
-//   kEpiAdam     the sum is the gradient of table row row_index[u]: the Adam-family update of that
-//                row (parameter and both moments) is applied at once, the gradient never written
-//   kEpiAdagrad  the same with the Adagrad update
-enum { kEpiStore = 0, kEpiAdam = 1, kEpiAdagrad = 2 };
-struct FuseArgs {
-  const int64_t* row_index;  // [U]; a negative index skips the row
-  void* const* emb;          // block tables (device arrays of block pointers)
-  void* const* s0;           // exp_avg / the Adagrad accumulator
-  void* const* s1;           // exp_avg_sq
-  RowBlocks rb;
-  AdamCoef adam;
-  float lr, eps;             // Adagrad
-};
-
-// The epilogue of one pack of one finished row; T = the table's row type for the optimizer kinds.
-template <typename T, int VEC, int EPI>
-__device__ __forceinline__ void fused_row_update(const FuseArgs& f, int* err, int64_t u, int c0,
-                                                 const float (&acc)[VEC]) {
-  int64_t b, off;
-  const int64_t idx = f.row_index[u];
-  if (idx < 0) return;  // a key the table does not hold takes no gradient
-  if (!block_row(f.rb, idx, b, off)) {
-    raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
-    return;
-  }
-  const int64_t at = off * f.rb.D + c0;
-  if constexpr (EPI == kEpiAdam) {
-    adam_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at,
-                             static_cast<T*>(f.s1[b]) + at, acc, f.adam.alpha[0], f.adam);
-  } else {
-    adagrad_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at, acc, f.lr, f.eps);
-  }
-}
-
-// Row s of the input: of the one array, or of the part that holds it.
-template <typename TIn, bool PARTS>
-__device__ __forceinline__ const TIn* src_row(const TIn* rows, const CsrArgs& a, int64_t s) {
-  if constexpr (!PARTS) {
-    return rows + s * a.D;
-  } else {
-    int f = 0;
-#pragma unroll
-    for (int k = 1; k < kMaxParts; ++k) f += (k < a.n_parts && s >= a.part_lo[k]) ? 1 : 0;
-    const TIn* base = static_cast<const TIn*>(a.part_rows[0]);
-    int64_t lo = 0;
-#pragma unroll
-    for (int k = 1; k < kMaxParts; ++k) {
-      if (k == f) {
-        base = static_cast<const TIn*>(a.part_rows[k]);
-        lo = a.part_lo[k];
-      }
-    }
-    return base + (s - lo) * a.D;
-  }
-}
-
-__device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64_t& hi) {
-  lo = 0;
-  hi = a.n_rows;
-  if (a.cover) {
-    lo = max(lo, load_index(a.cover, a.cover64, 0));
-    hi = min(hi, load_index(a.cover, a.cover64, a.cover_S));
-  }
-}
-
-// A whole wave works the list entries [e_begin, e_end) (uniform arguments, every lane calls):
-// `src` and `coef` of 64 entries come from one coalesced load, a lane each, and reach the lanes
-// that gather the rows through shuffles; lane group g of `groups` takes entries g, g + groups,
-// ... with several row loads in flight. acc: this group's partial sum for columns
-// c0 .. c0 + VEC (the caller folds the groups).
-template <typename TIn, int VEC, bool PARTS>
-__device__ __forceinline__ void wave_gather_range(const TIn* __restrict__ rows, const CsrArgs& a, int64_t c_lo,
-                                                  int64_t c_hi, int32_t e_begin, int32_t e_end, int c0, bool col_ok,
-                                                  int g, int groups, float (&acc)[VEC]) {
-  constexpr int kFly = VEC >= 8 ? 4 : 8;  // row loads in flight per lane
-  const int lane = threadIdx.x & (kWave - 1);
-  for (int32_t cb = e_begin; cb < e_end; cb += kWave) {
-    const int n_here = min(kWave, e_end - cb);
-    int32_t s_mine = -1;
-    float w_mine = 0.f;
-    if (lane < n_here) {
-      const int32_t sv = a.src[cb + lane];
-      if (sv >= c_lo && sv < c_hi) {
-        s_mine = sv;
-        w_mine = a.coef ? load_coef(a.coef, a.coef_dt, cb + lane) : 1.0f;
-      } else if (static_cast<int64_t>(sv) >= a.n_rows) {
-        raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-      }
-    }
-    for (int q0 = 0; q0 < n_here; q0 += kFly * groups) {  // same trip count for the whole wave (shuffles inside)
-      float v[kFly][VEC];
-      float w[kFly];
-#pragma unroll
-      for (int k = 0; k < kFly; ++k) {
-        const int e = q0 + g + k * groups;
-        const int from = min(e, kWave - 1);
-        int32_t id = __shfl(s_mine, from, kWave);
-        w[k] = a.coef ? __shfl(w_mine, from, kWave) : 1.0f;
-        if (e >= n_here || !col_ok) id = -1;
-        if (id >= 0) {
-          const TIn* row = src_row<TIn, PARTS>(rows, a, id);
-          if (a.nt_in) {
-            load_pack_stream<TIn, VEC>(row + c0, v[k]);
-          } else {
-            load_pack<TIn, VEC>(row + c0, v[k]);
-          }
-        } else {
-          w[k] = 0.f;
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) v[k][j] = 0.f;
-        }
-      }
-#pragma unroll
-      for (int k = 0; k < kFly; ++k) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[k][j], w[k], acc[j]);
-      }
-    }
-  }
-}
-
-constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of a wave
-
-// One launch for all rows. The last cold_blocks workgroups: one group of LPR lanes per unique row
-// with at most hot_len occurrences ("cold"); a wave that holds a row with more than kCoopLen
-// occurrences works that row with all its lane groups striding over the list (a row of 200
-// occurrences would otherwise be 50 dependent gathers of one group). The first workgroups
-// walk the hot work items (row, chunk of kHotChunk occurrences): four waves share the chunk,
-// fold their sums through LDS and store ONE partial row per item; csr_hot_finish_kernel adds up
-// the partial rows of every hot row in chunk order. No atomics anywhere.
-// SHUFFLE: long lists go through wave_gather_range (pays off when a wave has at most eight lane
-// groups, i.e. rows of 128 bytes and more); otherwise every group loads its own entries.
-template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false, int EPI = kEpiStore>
-__global__ void __launch_bounds__(kBlock, (!SHUFFLE && EPI != kEpiStore) ? 8 : 1)  // 64 registers where that costs no spills
-csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
-  extern __shared__ float s_part[];  // [waves][D], hot part only
-  const int D = a.D;
-  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
-  const int lane = threadIdx.x & (kWave - 1);
-  const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
-  const int g = lane >> a.lpr_log2;        // this lane's group in its wave
-  int64_t c_lo, c_hi;
-  cover_range(a, c_lo, c_hi);
-
-  auto fetch = [&](int32_t k, int c0, float (&v)[VEC], float& w) {
-    const int32_t s = a.src[k];
-    w = a.coef ? load_coef(a.coef, a.coef_dt, k) : 1.0f;
-    if (s < c_lo || s >= c_hi) {
-      if (static_cast<int64_t>(s) >= a.n_rows) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
-      w = 0.f;
-      return;
-    }
-    const TIn* row = src_row<TIn, PARTS>(rows, a, s);
-    if (a.nt_in) {
-      load_pack_stream<TIn, VEC>(row + c0, v);
-    } else {
-      load_pack<TIn, VEC>(row + c0, v);
-    }
-  };
-  // acc += sum over list entries k = first, first + step, ... < last (4 gathers in flight)
-  auto gather_sum = [&](int32_t first, int32_t last, int32_t step, int c0, float (&acc)[VEC]) {
-    int32_t k = first;
-    for (; k + 3 * step < last; k += 4 * step) {
-      float v0[VEC], v1[VEC], v2[VEC], v3[VEC];
-      float w0, w1, w2, w3;
-      fetch(k, c0, v0, w0);
-      fetch(k + step, c0, v1, w1);
-      fetch(k + 2 * step, c0, v2, w2);
-      fetch(k + 3 * step, c0, v3, w3);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        acc[j] = fmaf(v0[j], w0, acc[j]);
-        acc[j] = fmaf(v1[j], w1, acc[j]);
-        acc[j] = fmaf(v2[j], w2, acc[j]);
-        acc[j] = fmaf(v3[j], w3, acc[j]);
-      }
-    }
-    for (; k < last; k += step) {
-      float v0[VEC];
-      float w0;
-      fetch(k, c0, v0, w0);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v0[j], w0, acc[j]);
-    }
-  };
-  // the wave's sum over the list entries [first, last) for columns c0.., the same in every group
-  auto wave_sum = [&](int32_t first, int32_t last, int c0, bool col_ok, float (&acc)[VEC]) {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    if constexpr (SHUFFLE) {
-      wave_gather_range<TIn, VEC, PARTS>(rows, a, c_lo, c_hi, first, last, c0, col_ok, g, groups, acc);
-    } else {
-      if (col_ok) gather_sum(first + g, last, groups, c0, acc);
-    }
-    for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
-    }
-  };
-
-  const int64_t hot_blocks = static_cast<int64_t>(gridDim.x) - a.cold_blocks;
-  if (static_cast<int64_t>(blockIdx.x) < hot_blocks) {
-    // ---- hot work items (the first workgroups: the longest-running ones start first)
-    int64_t n_items = a.counts[1];
-    if (n_items > a.hot_cap) n_items = a.hot_cap;
-    const int wave = threadIdx.x / kWave;
-    constexpr int n_waves = kBlock / kWave;
-    for (int64_t item = blockIdx.x; item < n_items; item += hot_blocks) {
-      const int32_t u = a.hot_items[2 * item];
-      const int32_t chunk = a.hot_items[2 * item + 1];
-      const int32_t start = a.row_start[u] + chunk * kHotChunk;
-      const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
-      const int32_t per_wave = (end - start + n_waves - 1) / n_waves;  // a contiguous share per wave
-      const int32_t w_begin = min(end, start + wave * per_wave), w_end = min(end, w_begin + per_wave);
-      for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
-        const int c0 = cbase + cl * VEC;
-        const bool col_ok = c0 < D;
-        float acc[VEC];
-        wave_sum(w_begin, w_end, c0, col_ok, acc);
-        if (g == 0 && col_ok) {
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) s_part[wave * D + c0 + j] = acc[j];
-        }
-      }
-      __syncthreads();
-      for (int d = threadIdx.x; d < D; d += kBlock) {
-        float sum = 0.f;
-        for (int w = 0; w < n_waves; ++w) sum += s_part[w * D + d];
-        a.hot_part[item * D + d] = sum;
-      }
-      __syncthreads();
-    }
-    return;
-  }
-
-  // ---- cold rows
-  const int rows_per_block = kBlock >> a.lpr_log2;
-  const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
-  const bool valid = u < a.U;
-  const int32_t start = valid ? a.row_start[u] : 0;
-  int32_t end = valid ? a.row_start[u + 1] : 0;
-  const bool hot = end - start > a.hot_len;  // left to the work items and the finish kernel
-  if (hot) end = start;
-  auto finish = [&](int64_t row, int c0, float (&acc)[VEC]) {
-    if constexpr (EPI != kEpiStore) {
-      fused_row_update<TOut, VEC, EPI>(f, a.err, row, c0, acc);
-    } else {
-      TOut* dst = out + row * D + c0;
-      if (a.accumulate) {
-        float old[VEC];
-        load_pack<TOut, VEC>(dst, old);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += old[j];
-      }
-      store_pack<TOut, VEC>(dst, acc);
-    }
-  };
-  // short rows: every lane group works its own row
-  const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;  // with one group per wave there is nobody to share with
-  if (valid && !is_long && !hot) {
-    // (Asking for the row's parameter and state packs before the gradient is gathered, to run their
-    // latency under that of the gathers, was measured and lost: 150 -> 205 us in config 4. The packs
-    // cost registers, hence resident waves, and the gathers then queue behind the table reads.)
-    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
-      float acc[VEC];
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      gather_sum(start, end, 1, c0, acc);
-      finish(u, c0, acc);
-    }
-  }
-  // long rows of this wave, one after the other
-  uint64_t todo = __ballot(is_long);
-  while (todo) {
-    const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;  // first lane of the owning group
-    todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);  // the group's lanes (fewer than 64 here)
-    const int r = owner >> a.lpr_log2;
-    const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
-    const int64_t row = u - g + r;  // rows of a wave are consecutive
-    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
-      const int c0 = cbase + cl * VEC;
-      const bool col_ok = c0 < D;
-      float acc[VEC];
-      wave_sum(r_start, r_end, c0, col_ok, acc);
-      if (g == r && col_ok) finish(row, c0, acc);
-    }
-  }
-}
-
-// out[u] (+)= sum of the partial rows of hot row u (or the optimizer's update of the row with that
-// sum). One wave per work item with chunk 0 (the items of a row are consecutive): its lane groups
-// share the row's partials out among themselves (an id that makes up a tenth of the batch has a
-// hundred of them) and fold their sums with shuffles, always in the same order.
-template <typename TOut, int VEC, int EPI = kEpiStore>
-__global__ void __launch_bounds__(kBlock)
-csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
-  int64_t n_items = a.counts[1];
-  if (n_items > a.hot_cap) n_items = a.hot_cap;
-  const int D = a.D;
-  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
-  const int lane = threadIdx.x & (kWave - 1);
-  const int groups = kWave >> a.lpr_log2, g = lane >> a.lpr_log2;
-  const int64_t waves_total = static_cast<int64_t>(gridDim.x) * (kBlock / kWave);
-  for (int64_t item = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave; item < n_items;
-       item += waves_total) {  // uniform in the wave
-    if (a.hot_items[2 * item + 1] != 0) continue;
-    const int32_t u = a.hot_items[2 * item];
-    const int32_t len = a.row_start[u + 1] - a.row_start[u];
-    int64_t n_chunks = (len + kHotChunk - 1) / kHotChunk;
-    if (item + n_chunks > n_items) n_chunks = n_items - item;  // items cut off by hot_cap (cannot happen with the documented hot_cap)
-    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
-      const int c0 = cbase + cl * VEC;
-      const bool col_ok = c0 < D;
-      float acc[VEC];
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-      if (col_ok) {
-        for (int64_t k = g; k < n_chunks; k += groups) {
-          float v[VEC];
-          load_pack<float, VEC>(a.hot_part + (item + k) * D + c0, v);
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) acc[j] += v[j];
-        }
-      }
-      for (int off = 1 << a.lpr_log2; off < kWave; off <<= 1) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) acc[j] += __shfl_xor(acc[j], off, kWave);
-      }
-      if (g != 0 || !col_ok) continue;
-      if constexpr (EPI != kEpiStore) {
-        fused_row_update<TOut, VEC, EPI>(f, a.err, u, c0, acc);
-      } else {
-        TOut* dst = out + static_cast<int64_t>(u) * D + c0;
-        if (a.accumulate) {
-          float old[VEC];
-          load_pack<TOut, VEC>(dst, old);
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) acc[j] += old[j];
-        }
-        store_pack<TOut, VEC>(dst, acc);
-      }
-    }
-  }
-}
-
-// ------------------------------------------------------------------ expand (transpose of the gather-reduce)
-// out[dst[k], :] = w[dst[k]] * row(u) for every list entry k of every unique id u: the forward
-// of pooling when every segment holds exactly one id, and of the unpooled (tile) output. Each
-// unique row is read ONCE and stored to all its occurrences; stores do not wait for anything,
-// where the occurrence-major kernels chase index -> row index -> row for every output row.
-struct ExpArgs {
-  const int32_t* row_start;  // [U + 1]
-  const int32_t* dst;        // [n] output row per list entry
-  const void* weight;        // [n_out] per output row, or NULL
-  int wdt;
-  int64_t U, n_out;
-  int D;
-  int lpr_log2;
-  int* err;
-  const int64_t* row_index;  // rows in a block list: unique row u is row row_index[u] (negative = zeros)
-  const void* const* blocks;
-  int64_t block_rows, n_blocks;
-  int32_t hot_len;
-  const int32_t* hot_items;
-  const int64_t* counts;
-  int64_t hot_cap;
-  int64_t cold_blocks;
-};
-
-template <typename TIn, typename TOut, int VEC, bool BLK>
-__global__ void __launch_bounds__(kBlock)
-csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs a) {
-  const int D = a.D;
-  const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
-  const int lane = threadIdx.x & (kWave - 1);
-  const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
-  const int g = lane >> a.lpr_log2;        // this lane's group in its wave
-
-  auto load_row = [&](int64_t u, int c0, float (&v)[VEC]) {
-    const TIn* src = nullptr;
-    if constexpr (BLK) {
-      const int64_t ri = a.row_index[u];
-      if (ri >= 0) {
-        int64_t b = 0, r = ri;
-        if (a.n_blocks > 1) {
-          b = ri / a.block_rows;
-          r = ri - b * a.block_rows;
-        }
-        if (b >= a.n_blocks || r >= a.block_rows)
-          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-        else
-          src = static_cast<const TIn*>(a.blocks[b]) + r * D;
-      }
-    } else {
-      src = rows + u * D;
-    }
-    if (src) {
-      load_pack_stream<TIn, VEC>(src + c0, v);  // every row is read once here
-    } else {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = 0.f;
-    }
-  };
-  auto store_to = [&](int64_t d, int c0, const float (&v)[VEC]) {
-    if (static_cast<uint64_t>(d) >= static_cast<uint64_t>(a.n_out)) {
-      raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-      return;
-    }
-    float o[VEC];
-    const float w = a.weight ? load_coef(a.weight, a.wdt, d) : 1.0f;
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) o[j] = fmaf(v[j], w, 0.f);  // the pooled kernels' rounding
-    store_pack_stream<TOut, VEC>(out + d * D + c0, o);
-  };
-  // stores to the list entries first, first + step, ... < last; the destinations of four entries
-  // are fetched together so that their latencies overlap (more would cost resident waves)
-  auto store_list = [&](int32_t first, int32_t last, int32_t step, int c0, const float (&v)[VEC]) {
-    for (int32_t k = first; k < last; k += 4 * step) {
-      int32_t d[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) d[i] = k + i * step < last ? a.dst[k + i * step] : -1;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (k + i * step < last) store_to(d[i], c0, v);
-    }
-  };
-
-  const int64_t hot_blocks = static_cast<int64_t>(gridDim.x) - a.cold_blocks;
-  if (static_cast<int64_t>(blockIdx.x) < hot_blocks) {
-    // ---- hot work items: a workgroup per (row, chunk); all its lane groups hold the row
-    int64_t n_items = a.counts[1];
-    if (n_items > a.hot_cap) n_items = a.hot_cap;
-    const int groups_per_block = kBlock >> a.lpr_log2;
-    const int gb = threadIdx.x >> a.lpr_log2;
-    for (int64_t item = blockIdx.x; item < n_items; item += hot_blocks) {
-      const int32_t u = a.hot_items[2 * item];
-      const int32_t chunk = a.hot_items[2 * item + 1];
-      const int32_t start = a.row_start[u] + chunk * kHotChunk;
-      const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
-      for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
-        float v[VEC];
-        load_row(u, c0, v);
-        store_list(start + gb, end, groups_per_block, c0, v);
-      }
-    }
-    return;
-  }
-
-  // ---- cold rows
-  const int rows_per_block = kBlock >> a.lpr_log2;
-  const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
-  const bool valid = u < a.U && u < a.counts[0];  // U may be the caller's upper bound: the plan's own count decides
-  const int32_t start = valid ? a.row_start[u] : 0;
-  int32_t end = valid ? a.row_start[u + 1] : 0;
-  if (end - start > a.hot_len) end = start;  // written by the work items
-  const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;
-  if (valid && !is_long && end > start) {
-    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
-      float v[VEC];
-      load_row(u, c0, v);
-      store_list(start, end, 1, c0, v);
-    }
-  }
-  // long rows of this wave, one after the other: the owner's row reaches every group by shuffles
-  uint64_t todo = __ballot(is_long);
-  while (todo) {
-    const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;
-    todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);
-    const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
-    const int64_t row = u - g + (owner >> a.lpr_log2);  // rows of a wave are consecutive
-    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
-      const int c0 = cbase + cl * VEC;
-      const bool col_ok = c0 < D;
-      float mine[VEC], v[VEC];
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) mine[j] = 0.f;
-      if (lane >> a.lpr_log2 == owner >> a.lpr_log2 && col_ok) load_row(row, c0, mine);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = __shfl(mine[j], owner + cl, kWave);
-      if (col_ok) store_list(r_start + g, r_end, groups, c0, v);
-    }
-  }
-}
-
-// src / coef of every list entry for pooled segments: occurrence i of segment s gets
-// src = s and coef = w_i (divided by the segment length for mean).
-__global__ void __launch_bounds__(kBlock)
-fill_pool_kernel(const void* __restrict__ offsets, int off64, int64_t S, int64_t n, const void* __restrict__ weight,
-                 int wdt, const int32_t* __restrict__ pos, int mean, int32_t* __restrict__ src,
-                 float* __restrict__ coef) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  if (i >= n) return;
-  // segment of occurrence i: largest s with offsets[s] <= i
-  int64_t lo = 0, hi = S;
-  const int64_t first = load_index(offsets, off64, 0), last = load_index(offsets, off64, S);
-  const int32_t p = pos[i];
-  if (i < first || i >= last) {
-    src[p] = -1;
-    if (coef) coef[p] = 0.f;
-    return;
-  }
-  while (hi - lo > 1) {
-    const int64_t mid = (lo + hi) >> 1;
-    if (load_index(offsets, off64, mid) <= i)
-      lo = mid;
-    else
-      hi = mid;
-  }
-  src[p] = static_cast<int32_t>(lo);
-  if (coef) {
-    float w = weight ? load_coef(weight, wdt, i) : 1.0f;
-    if (mean) w /= static_cast<float>(load_index(offsets, off64, lo + 1) - load_index(offsets, off64, lo));
-    coef[p] = w;
-  }
-}
-
-// src of every list entry for the padded gather of one feature: occurrence t of sample b
-// maps to padded row rbase + b * seq + t, or to "skip" when t >= seq.
-__global__ void __launch_bounds__(kBlock)
-fill_tile_kernel(const void* __restrict__ offsets, int off64, int64_t batch, int64_t seq, int64_t rbase,
-                 const int32_t* __restrict__ pos, int32_t* __restrict__ src) {
-  const int64_t first = load_index(offsets, off64, 0), last = load_index(offsets, off64, batch);
-  const int64_t i = first + static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  if (i >= last) return;
-  int64_t lo = 0, hi = batch;
-  while (hi - lo > 1) {
-    const int64_t mid = (lo + hi) >> 1;
-    if (load_index(offsets, off64, mid) <= i)
-      lo = mid;
-    else
-      hi = mid;
-  }
-  const int64_t t = i - load_index(offsets, off64, lo);
-  src[pos[i]] = t < seq ? static_cast<int32_t>(rbase + lo * seq + t) : -1;
-}
-
-template <typename F>
-int dispatch_vec(int vec, F&& f) {
-  switch (vec) {
-    case 8: return f(std::integral_constant<int, 8>{});
-    case 4: return f(std::integral_constant<int, 4>{});
-    case 2: return f(std::integral_constant<int, 2>{});
-    case 1: return f(std::integral_constant<int, 1>{});
-    default: return fail(RECIS_ERR_ARG, "unsupported vector width %d", vec);
-  }
-}
-
 }  // namespace
 }  // namespace recis_hip
 
@@ -2082,354 +1494,6 @@ int recis_hip_staged_device_errors(int* bits, void* stream_) {
   if (int rc = get_count_staging(stream, &staged, &staged_event)) return rc;
   *bits = static_cast<int>(staged[1]);
   return RECIS_OK;
-}
-
-int recis_csr_fill_pool(const void* offsets, int off_is64, int64_t S, int64_t n, const void* weight,
-                        int weight_dtype, const int32_t* pos, int mean, int32_t* src_out, float* coef_out,
-                        void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  RECIS_REQUIRE(n >= 0 && S >= 0, "negative size");
-  if (n == 0) return RECIS_OK;
-  RECIS_REQUIRE(offsets && pos && src_out, "NULL argument");
-  RECIS_REQUIRE(S >= 1, "occurrences without a segment");
-  RECIS_REQUIRE(coef_out || (!weight && !mean), "coef_out is needed for weights or mean");
-  RECIS_REQUIRE(weight == nullptr || dtype_size(weight_dtype), "invalid weight dtype");
-  fill_pool_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(
-      offsets, off_is64, S, n, weight, weight_dtype, pos, mean, src_out, coef_out);
-  RECIS_LAUNCH_CHECK();
-  return RECIS_OK;
-}
-
-int recis_csr_fill_tile(const int64_t* batch, const int64_t* seq, int64_t n_features, const void* offsets,
-                        int off_is64, int64_t n, const int32_t* pos, int32_t* src_out, void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  RECIS_REQUIRE(n_features >= 0 && n >= 0, "negative size");
-  if (n_features == 0 || n == 0) return RECIS_OK;
-  RECIS_REQUIRE(batch && seq && offsets && pos && src_out, "NULL argument");
-  int64_t obase = 0, rbase = 0;
-  const int osz = off_is64 ? 8 : 4;
-  for (int64_t f = 0; f < n_features; ++f) {
-    RECIS_REQUIRE(batch[f] >= 0 && seq[f] >= 0, "negative batch/seq");
-    if (batch[f] > 0) {
-      // upper bound of this feature's occurrences is n; the kernel stops at its last offset
-      const void* off_f = static_cast<const char*>(offsets) + obase * osz;
-      fill_tile_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(off_f, off_is64, batch[f],
-                                                                                    seq[f], rbase, pos, src_out);
-      RECIS_LAUNCH_CHECK();
-    }
-    obase += batch[f];
-    rbase += batch[f] * seq[f];
-  }
-  return RECIS_OK;
-}
-
-static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows, const int64_t* part_counts,
-                                  int n_parts, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
-                                  int coef_dtype, const int32_t* row_start, const int32_t* hot_items,
-                                  int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
-                                  int64_t D, int accumulate, const void* cover_offsets, int cover_is64,
-                                  int64_t cover_S, hipStream_t stream, int epi = kEpiStore,
-                                  const FuseArgs* fuse = nullptr, size_t extra_ws = 0, void** extra_out = nullptr);
-
-int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
-                            int coef_dtype, const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
-                            const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t D,
-                            int accumulate, const void* cover_offsets, int cover_is64, int64_t cover_S,
-                            void* stream_) {
-  return csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
-                                hot_items, hot_cap, counts_dev, out, out_dtype, U, D, accumulate, cover_offsets,
-                                cover_is64, cover_S, static_cast<hipStream_t>(stream_));
-}
-
-int recis_csr_gather_reduce_parts(const void* const* part_rows, const int64_t* part_counts, int n_parts,
-                                  int rows_dtype, const int32_t* src, const int32_t* row_start,
-                                  const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, void* out,
-                                  int64_t U, int64_t D, int accumulate, void* stream_) {
-  RECIS_REQUIRE(n_parts >= 1 && n_parts <= kMaxParts, "1 to %d parts (got %d)", kMaxParts, n_parts);
-  RECIS_REQUIRE(part_rows && part_counts, "NULL argument");
-  int64_t n_rows = 0;
-  for (int f = 0; f < n_parts; ++f) {
-    RECIS_REQUIRE(part_counts[f] >= 0 && (part_rows[f] != nullptr || part_counts[f] == 0), "bad part %d", f);
-    n_rows += part_counts[f];
-  }
-  return csr_gather_reduce_impl(nullptr, part_rows, part_counts, n_parts, rows_dtype, n_rows, src, nullptr, 0,
-                                row_start, hot_items, hot_cap, counts_dev, out, RECIS_F32, U, D, accumulate, nullptr,
-                                0, 0, static_cast<hipStream_t>(stream_));
-}
-
-static int csr_gather_reduce_impl(const void* rows, const void* const* part_rows, const int64_t* part_counts,
-                                  int n_parts, int rows_dtype, int64_t n_rows, const int32_t* src, const void* coef,
-                                  int coef_dtype, const int32_t* row_start, const int32_t* hot_items,
-                                  int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
-                                  int64_t D, int accumulate, const void* cover_offsets, int cover_is64,
-                                  int64_t cover_S, hipStream_t stream, int epi, const FuseArgs* fuse,
-                                  size_t extra_ws, void** extra_out) {
-  // epi != kEpiStore: `out` is NULL, out_dtype is the table's row type and *fuse says where the rows
-  // are. extra_ws bytes of the stream's workspace (after the partial rows of the hot items) are
-  // handed to the caller in *extra_out before anything is launched.
-  RECIS_REQUIRE(U >= 0 && n_rows >= 0, "negative size");
-  RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
-  RECIS_REQUIRE(U == 0 || (src && row_start && (out || epi != kEpiStore) && counts_dev), "NULL argument");
-  RECIS_REQUIRE(n_parts > 0 || rows != nullptr || n_rows == 0, "rows must not be NULL");
-  RECIS_REQUIRE(hot_cap == 0 || hot_items, "hot_items must not be NULL");
-  const int in_sz = dtype_size(rows_dtype), out_sz = dtype_size(out_dtype);
-  RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
-  RECIS_REQUIRE(coef == nullptr || dtype_size(coef_dtype), "invalid coef dtype");
-  uintptr_t align_of = reinterpret_cast<uintptr_t>(rows);
-  for (int f = 0; f < n_parts; ++f) align_of |= reinterpret_cast<uintptr_t>(part_rows[f]);  // the coarsest alignment
-  const int vb_in = pick_vec_bytes(D * in_sz, align_of);
-  // table blocks are allocator-aligned and are read and written in 16-byte packs at most
-  const int vb_out = epi != kEpiStore ? pick_vec_bytes(D * out_sz, 16)
-                                      : pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
-  const int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
-  CsrArgs a;
-  a.row_start = row_start;
-  a.src = src;
-  a.coef = coef;
-  a.coef_dt = coef_dtype;
-  a.U = U;
-  a.n_rows = n_rows;
-  a.cover = cover_offsets;
-  a.cover64 = cover_is64;
-  a.cover_S = cover_S;
-  a.D = static_cast<int>(D);
-  a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
-  a.accumulate = accumulate;
-  a.nt_in = n_rows * D * in_sz >= (int64_t(1) << 30);
-  a.err = device_error_word(current_device());
-  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
-  const int rows_per_block = kBlock >> a.lpr_log2;
-  a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
-  a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
-  a.hot_items = hot_items;
-  a.counts = counts_dev;
-  a.hot_cap = hot_cap;
-  a.hot_part = nullptr;
-  a.n_parts = n_parts;
-  a.part_lo[0] = 0;
-  for (int f = 0; f < kMaxParts; ++f) {
-    a.part_rows[f] = f < n_parts ? part_rows[f] : nullptr;
-    a.part_lo[f + 1] = a.part_lo[f] + (f < n_parts ? part_counts[f] : 0);
-  }
-  int64_t hot_blocks = 0;
-  if (hot_cap > 0 || extra_ws > 0) {
-    void* ws = nullptr;
-    const size_t hot_bytes = (sizeof(float) * static_cast<size_t>(hot_cap) * static_cast<size_t>(D) + 255) & ~size_t(255);
-    if (int rc = get_workspace(stream, hot_bytes + extra_ws, &ws)) return rc;
-    a.hot_part = static_cast<float*>(ws);
-    if (extra_out) *extra_out = static_cast<char*>(ws) + hot_bytes;
-    if (hot_cap > 0) hot_blocks = std::min<int64_t>(hot_cap, 4096);
-  }
-  if (U == 0) return RECIS_OK;
-  const FuseArgs f = fuse ? *fuse : FuseArgs{};
-  const size_t lds = sizeof(float) * (kBlock / kWave) * static_cast<size_t>(D);
-  auto with_types = [&](auto tin, auto tout) {
-    using TIn = decltype(tin);
-    using TOut = decltype(tout);
-    return dispatch_vec(vec, [&](auto vtag) {
-      constexpr int VEC = decltype(vtag)::value;
-      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 32) {
-        return fail(RECIS_ERR_ARG, "internal: vector too wide");
-      } else {
-        const TIn* rin = static_cast<const TIn*>(rows);
-        TOut* o = static_cast<TOut*>(out);
-        const bool shuffle = a.lpr_log2 >= 3;  // at most eight lane groups per wave
-        const dim3 grid(a.cold_blocks + hot_blocks), block(kBlock);
-        const int64_t fin = std::min<int64_t>((hot_cap + kBlock / kWave - 1) / (kBlock / kWave), 2048);  // a wave per item
-        auto launch = [&](auto epi_tag) {
-          constexpr int EPI = decltype(epi_tag)::value;
-          {
-            RECIS_TIME_KERNEL(EPI == kEpiStore ? "csr_rows_kernel" : EPI == kEpiAdam ? "csr_rows_adam_kernel"
-                                                                                      : "csr_rows_adagrad_kernel", stream)
-            if (n_parts > 0) {
-              if constexpr (sizeof(TOut) == 4 && EPI == kEpiStore) {  // parts go to fp32 rows only
-                if (shuffle)
-                  csr_rows_kernel<TIn, TOut, VEC, true, true><<<grid, block, lds, stream>>>(rin, o, a, f);
-                else
-                  csr_rows_kernel<TIn, TOut, VEC, false, true><<<grid, block, lds, stream>>>(rin, o, a, f);
-              }
-            } else if (shuffle) {
-              csr_rows_kernel<TIn, TOut, VEC, true, false, EPI><<<grid, block, lds, stream>>>(rin, o, a, f);
-            } else {
-              csr_rows_kernel<TIn, TOut, VEC, false, false, EPI><<<grid, block, lds, stream>>>(rin, o, a, f);
-            }
-            RECIS_LAUNCH_CHECK();
-          }
-          if (hot_cap > 0) {
-            csr_hot_finish_kernel<TOut, VEC, EPI><<<dim3(fin), block, 0, stream>>>(o, a, f);
-            RECIS_LAUNCH_CHECK();
-          }
-          return RECIS_OK;
-        };
-        if (epi == kEpiAdam) {
-          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdam>{});
-        } else if (epi == kEpiAdagrad) {
-          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdagrad>{});
-        } else {
-          return launch(std::integral_constant<int, kEpiStore>{});
-        }
-        return fail(RECIS_ERR_ARG, "internal: vector too wide for a fused row update");
-      }
-    });
-  };
-  if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F32) return with_types(float{}, float{});
-  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_F32) return with_types(bf16_t{}, float{});
-  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F32) return with_types(f16_t{}, float{});
-  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_BF16) return with_types(bf16_t{}, bf16_t{});
-  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F16) return with_types(f16_t{}, f16_t{});
-  if (epi != kEpiStore) {  // fp32 gradients onto half-precision rows
-    if (rows_dtype == RECIS_F32 && out_dtype == RECIS_BF16) return with_types(float{}, bf16_t{});
-    if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F16) return with_types(float{}, f16_t{});
-  }
-  return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
-}
-
-// Shared front of the two fused entry points: argument checks and the table description.
-static int fill_fuse_args(FuseArgs& f, const int64_t* row_index, void* const* emb, void* const* s0, void* const* s1,
-                          bool need_s1, int64_t n_blocks, int64_t block_size, int64_t D, int row_dtype) {
-  RECIS_REQUIRE(row_index && emb && s0 && (s1 || !need_s1), "row_index and the block tables must not be NULL");
-  RECIS_REQUIRE(n_blocks >= 1 && block_size >= 1, "bad block geometry (n_blocks=%lld block_size=%lld)",
-                (long long)n_blocks, (long long)block_size);
-  RECIS_REQUIRE(dtype_size(row_dtype), "invalid row dtype");
-  f = FuseArgs{};
-  f.row_index = row_index;
-  f.emb = emb;
-  f.s0 = s0;
-  f.s1 = s1;
-  f.rb.n_blocks = n_blocks;
-  f.rb.block_size = block_size;
-  f.rb.D = static_cast<int>(D);
-  return RECIS_OK;
-}
-
-int recis_csr_gather_reduce_adamw(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
-                                  const void* coef, int coef_dtype, const int32_t* row_start,
-                                  const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
-                                  int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
-                                  const int64_t* row_index, void* const* emb_blocks_dev,
-                                  void* const* exp_avg_blocks_dev, void* const* exp_avg_sq_blocks_dev,
-                                  int64_t n_blocks, int64_t block_size, int row_dtype, void* beta1_t, void* beta2_t,
-                                  int beta_is_f64, double lr, double beta1, double beta2, double weight_decay,
-                                  double eps, void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  RECIS_REQUIRE(beta1_t != nullptr && beta2_t != nullptr, "beta1_t / beta2_t must not be NULL");
-  FuseArgs f;
-  if (U > 0) {
-    if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, exp_avg_blocks_dev, exp_avg_sq_blocks_dev, true, n_blocks,
-                                block_size, D, row_dtype))
-      return rc;
-  } else {
-    f = FuseArgs{};
-  }
-  // the running powers advance even when no row is touched (cal_alpha runs first); alpha lives in
-  // the stream's workspace behind the partial rows of the hot items
-  void* alpha = nullptr;
-  // first pass: reserve the workspace and learn where alpha goes, launching nothing (U = 0)
-  if (int rc = csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
-                                      hot_items, hot_cap, counts_dev, nullptr, row_dtype, 0, D, 0, cover_offsets,
-                                      cover_is64, cover_S, stream, kEpiAdam, &f, 256, &alpha))
-    return rc;
-  if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, static_cast<double*>(alpha), lr, beta1, beta2, stream))
-    return rc;
-  if (U == 0) return RECIS_OK;
-  f.adam.alpha = static_cast<const double*>(alpha);
-  f.adam.beta1 = beta1;
-  f.adam.beta2 = beta2;
-  f.adam.decay = weight_decay;
-  f.adam.eps = eps;
-  return csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
-                                hot_items, hot_cap, counts_dev, nullptr, row_dtype, U, D, 0, cover_offsets, cover_is64,
-                                cover_S, stream, kEpiAdam, &f, 256, &alpha);
-}
-
-int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
-                                    const void* coef, int coef_dtype, const int32_t* row_start,
-                                    const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
-                                    int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
-                                    const int64_t* row_index, void* const* emb_blocks_dev,
-                                    void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
-                                    int row_dtype, double lr, double eps, void* stream_) {
-  if (U == 0) return RECIS_OK;
-  FuseArgs f;
-  if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, accum_blocks_dev, nullptr, false, n_blocks, block_size, D,
-                              row_dtype))
-    return rc;
-  f.lr = static_cast<float>(lr);
-  f.eps = static_cast<float>(eps);
-  return csr_gather_reduce_impl(rows, nullptr, nullptr, 0, rows_dtype, n_rows, src, coef, coef_dtype, row_start,
-                                hot_items, hot_cap, counts_dev, nullptr, row_dtype, U, D, 0, cover_offsets, cover_is64,
-                                cover_S, static_cast<hipStream_t>(stream_), kEpiAdagrad, &f);
-}
-
-int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows,
-                          const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
-                          const int32_t* row_start, const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
-                          const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t n_out, int64_t D,
-                          void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  RECIS_REQUIRE(U >= 0 && n_out >= 0, "negative size");
-  RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
-  if (U == 0 || n_out == 0) return RECIS_OK;
-  const bool blk = emb_blocks_dev != nullptr;
-  RECIS_REQUIRE(row_start && dst && out && counts_dev, "NULL argument");
-  RECIS_REQUIRE(blk ? (row_index != nullptr && n_blocks >= 1 && block_rows >= 1) : rows != nullptr,
-                "rows: a dense array or a block list with row_index");
-  RECIS_REQUIRE(hot_cap == 0 || hot_items, "hot_items must not be NULL");
-  const int in_sz = dtype_size(rows_dtype), out_sz = dtype_size(out_dtype);
-  RECIS_REQUIRE(in_sz && out_sz, "invalid dtype");
-  RECIS_REQUIRE(weight == nullptr || dtype_size(weight_dtype), "invalid weight dtype");
-  // block bases are allocator-aligned; a dense array brings its own alignment
-  const int vb_in = pick_vec_bytes(D * in_sz, blk ? 0 : reinterpret_cast<uintptr_t>(rows));
-  const int vb_out = pick_vec_bytes(D * out_sz, reinterpret_cast<uintptr_t>(out));
-  const int vec = std::max(1, std::min(vb_in / in_sz, vb_out / out_sz));
-  ExpArgs a;
-  a.row_start = row_start;
-  a.dst = dst;
-  a.weight = weight;
-  a.wdt = weight_dtype;
-  a.U = U;
-  a.n_out = n_out;
-  a.D = static_cast<int>(D);
-  a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
-  a.err = device_error_word(current_device());
-  RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
-  a.row_index = row_index;
-  a.blocks = emb_blocks_dev;
-  a.block_rows = block_rows;
-  a.n_blocks = n_blocks;
-  a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
-  a.hot_items = hot_items;
-  a.counts = counts_dev;
-  a.hot_cap = hot_cap;
-  const int rows_per_block = kBlock >> a.lpr_log2;
-  a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
-  const int64_t hot_blocks = hot_cap > 0 ? std::min<int64_t>(hot_cap, 4096) : 0;
-  const dim3 grid(static_cast<unsigned>(a.cold_blocks + hot_blocks));
-  auto with_types = [&](auto tin, auto tout) {
-    using TIn = decltype(tin);
-    using TOut = decltype(tout);
-    return dispatch_vec(vec, [&](auto vtag) {
-      constexpr int VEC = decltype(vtag)::value;
-      if constexpr (VEC * sizeof(TIn) > 16 || VEC * sizeof(TOut) > 16) {
-        return fail(RECIS_ERR_ARG, "internal: vector too wide");
-      } else {
-        RECIS_TIME_KERNEL("csr_expand_kernel", stream)
-        if (blk)
-          csr_expand_kernel<TIn, TOut, VEC, true><<<grid, dim3(kBlock), 0, stream>>>(nullptr, static_cast<TOut*>(out), a);
-        else
-          csr_expand_kernel<TIn, TOut, VEC, false><<<grid, dim3(kBlock), 0, stream>>>(static_cast<const TIn*>(rows),
-                                                                                    static_cast<TOut*>(out), a);
-        RECIS_LAUNCH_CHECK();
-        return RECIS_OK;
-      }
-    });
-  };
-  if (rows_dtype == RECIS_F32 && out_dtype == RECIS_F32) return with_types(float{}, float{});
-  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_BF16) return with_types(bf16_t{}, bf16_t{});
-  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F16) return with_types(f16_t{}, f16_t{});
-  if (rows_dtype == RECIS_BF16 && out_dtype == RECIS_F32) return with_types(bf16_t{}, float{});
-  if (rows_dtype == RECIS_F16 && out_dtype == RECIS_F32) return with_types(f16_t{}, float{});
-  return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
 }
 
 }  // extern "C"

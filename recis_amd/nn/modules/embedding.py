@@ -189,9 +189,8 @@ def make_plan(hashtable: HashTable, ids, offsets, opt, has_weight=False, unit_se
     if (hashtable.training and opt.trainable and opt.admit_hook is None
             and _pools_out_of_the_table(hashtable, opt, ids.numel(), offsets.numel())):
         lean = bool(unit_segments)
-        return hashtable._hashtable_impl.plan_lookup(ids, need_inverse=not lean,
-                                                     need_pos=not (lean and not has_weight))
-    return ops.ids_unique_plan(ids, wait=False)
+        return hashtable._hashtable_impl.plan_lookup(ids, need_inverse=not lean)
+    return ops.ids_unique_plan(ids, wait=False, need_pos=False)
 
 
 def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False, combiner_kwargs=None):
@@ -295,7 +294,7 @@ class DynamicEmbedding(torch.nn.Module):
     # lookup_exchange_emb the table lookup of the distinct ids, emb_reduce the pooling. forward()
     # above fuses the last two (pooling reads the table rows directly).
     def exchange_ids(self, ids: torch.Tensor, offsets: torch.Tensor):
-        plan = ops.ids_unique_plan(ids, wait=True)
+        plan = ops.ids_unique_plan(ids, wait=True, need_pos=False)
         n = int(plan.U)
         return ExchangeIDsResults(ids=plan.unique, ids_await=_Done(), parts=[n], parts_reverse=[n],
                                   reverse_index=plan.inverse, offsets=offsets, plan=plan)

@@ -172,7 +172,7 @@ class EmbeddingEngine(torch.nn.Module):
                     else:
                         offsets = ops.merge_offsets(offs, [v.numel() for v in vals])
                     if opt0.combiner == "tile":
-                        plan = ops.ids_unique_plan(ids, wait=False)
+                        plan = ops.ids_unique_plan(ids, wait=False, need_pos=False)
                     else:  # lean (no per-occurrence arrays) only if no other option can come to share it
                         alone = sum(1 for k in runtime.values() if any(inputs[n] is inputs[names[0]] for n in k)) == 1
                         plan = make_plan(table, ids, offsets, opt0, any_weight, unit_segments=all_unit and alone)

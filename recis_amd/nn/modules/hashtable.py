@@ -396,7 +396,7 @@ class HashtableImpl:
         plan.lookup_calls[id(self)] = self._idmap.last_call()
         return index_buf
 
-    def plan_lookup(self, ids, wait=False, need_inverse=True, need_pos=True):
+    def plan_lookup(self, ids, wait=False, need_inverse=True, need_pos=False):
         """Dedup of ``ids`` and find-or-insert of the distinct ids in this table in one pass
         (``recis_unique_plan_lookup``): the batch plan with ``index_buf`` = the row of every unique
         id. Replaces ``ids_partition`` / ``torch.unique`` + ``IdMap::Lookup`` of the training
@@ -822,7 +822,7 @@ class HashTable(torch.nn.Module):
         if self._dedup == "sorted":
             uniq, inverse = ids.unique(return_inverse=True)
             return uniq, inverse, None
-        plan = ops.ids_unique_plan(ids)
+        plan = ops.ids_unique_plan(ids, need_pos=False)
         return plan.unique, plan.inverse, plan
 
     def forward(self, ids: torch.Tensor, admit_hook: AdmitHook = None) -> torch.Tensor:
@@ -837,7 +837,7 @@ class HashTable(torch.nn.Module):
 
             assert admit_hook_impl is None or isinstance(admit_hook_impl, ReadOnlyHookImpl), \
                 "admit hook only support ReadOnlyHook yet, but got: %s" % admit_hook_impl
-            plan = ops.ids_unique_plan(ids, wait=False)
+            plan = ops.ids_unique_plan(ids, wait=False, need_pos=False)
             emb_idx, embedding = LookupExpandFunction.apply(self._backward_holder, self._hashtable_impl, plan,
                                                             self._worker_num, admit_hook_impl is not None)
             self._filter_hook_impl(emb_idx)

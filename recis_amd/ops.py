@@ -803,6 +803,25 @@ class BatchPlan:
             self._fill_late()
         return self._pos
 
+    def _fill_lists(self, offsets, weight, mean, want_pool, batch, seq):
+        dev = offsets.device
+        S = offsets.numel() - 1
+        src = coef = tile = None
+        if want_pool:
+            src = torch.empty(self.n, dtype=torch.int32, device=dev)
+            if weight is not None or mean:
+                coef = torch.empty(self.n, dtype=torch.float32, device=dev)
+        if batch is not None:
+            tile = torch.empty(self.n, dtype=torch.int32, device=dev)
+        weight = _contig(weight)
+        if self.n:
+            check(lib().recis_csr_fill_lists(
+                ptr(self.occ), i64(self.n), ptr(offsets), _index_kind(offsets, "offsets"), i64(S), ptr(weight),
+                dtype_code(weight.dtype) if weight is not None else 0, int(bool(mean)), ptr(src), ptr(coef),
+                _host_i64(batch) if batch is not None else None, _host_i64(seq) if batch is not None else None,
+                i64(len(batch) if batch is not None else 0), ptr(tile), stream_ptr(dev)))
+        return src, coef, tile
+
     def src_coef_for_pool(self, offsets, weight, mean):
         """(src, coef) per list entry for the backward of pooled segments, cached per
         (offsets, weight, mean) so that forward-time and backward-time callers share it."""
@@ -812,25 +831,20 @@ class BatchPlan:
         key = (offsets.data_ptr(), 0 if weight is None else weight.data_ptr(), bool(mean))
         if self._pool_fill is not None and self._pool_fill[0] == key:
             return self._pool_fill[1], self._pool_fill[2]
-        src = torch.empty(self.n, dtype=torch.int32, device=offsets.device)
-        need_coef = weight is not None or mean
-        coef = torch.empty(self.n, dtype=torch.float32, device=offsets.device) if need_coef else None
-        weight = _contig(weight)
-        check(lib().recis_csr_fill_pool(ptr(offsets), _index_kind(offsets, "offsets"), i64(S), i64(self.n),
-                                        ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
-                                        ptr(self.pos), int(bool(mean)), ptr(src), ptr(coef),
-                                        stream_ptr(offsets.device)))
+        src, coef, _ = self._fill_lists(offsets, weight, mean, True, None, None)
         self._pool_fill = (key, src, coef)
         return src, coef
 
     def src_for_tile(self, batch, seq, offsets):
         """src per list entry for the backward of the padded gather (``ragged_tile``)."""
-        src = torch.empty(self.n, dtype=torch.int32, device=offsets.device)
-        if self.n:
-            check(lib().recis_csr_fill_tile(_host_i64(batch), _host_i64(seq), i64(len(batch)), ptr(offsets),
-                                            _index_kind(offsets, "offsets"), i64(self.n), ptr(self.pos), ptr(src),
-                                            stream_ptr(offsets.device)))
-        return src
+        return self._fill_lists(offsets, None, False, False, [int(b) for b in batch], [int(t) for t in seq])[2]
+
+    def src_for_pool_and_tile(self, offsets, weight, mean, batch, seq):
+        """``src_coef_for_pool`` and ``src_for_tile`` of the same segments in one launch:
+        ``(src_pool, coef_pool, src_tile)``."""
+        src, coef, tile = self._fill_lists(offsets, weight, mean, True, [int(b) for b in batch], [int(t) for t in seq])
+        self._pool_fill = ((offsets.data_ptr(), 0 if weight is None else weight.data_ptr(), bool(mean)), src, coef)
+        return src, coef, tile
 
 
 _PLAN_SERIAL = itertools.count(1)
@@ -980,6 +994,93 @@ def csr_gather_reduce_adagrad(rows, plan, src, coef, row_index, emb_blocks, accu
     check(lib().recis_csr_gather_reduce_adagrad(
         *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)),
         i64(block_size), dtype_code(b0.dtype), ctypes.c_double(lr), ctypes.c_double(eps), stream_ptr(rows.device)))
+
+
+class _CsrInput(ctypes.Structure):
+    """``recis_csr_input`` of the C header."""
+    _fields_ = [("rows", ctypes.c_void_p), ("rows_dtype", ctypes.c_int), ("n_rows", ctypes.c_int64),
+                ("src", ctypes.c_void_p), ("coef", ctypes.c_void_p), ("coef_dtype", ctypes.c_int)]
+
+
+def _csr_input(rows, src, coef):
+    """One input ``(rows, src, coef)`` of a two-input gather-reduce as the C struct, with the
+    tensors it points into (to be kept alive over the call)."""
+    require_cuda(rows, src, coef)
+    rows = _contig(rows)
+    if rows.dim() != 2:
+        raise ValueError("gradient rows must be [rows, D]")
+    c = _CsrInput(rows.data_ptr() if rows.numel() else None, dtype_code(rows.dtype), rows.shape[0],
+                  src.data_ptr() if src.numel() else None, coef.data_ptr() if coef is not None and coef.numel() else None,
+                  dtype_code(coef.dtype) if coef is not None else 0)
+    return c, (rows, src, coef)
+
+
+def _two_inputs(plan, first, second):
+    a, keep_a = _csr_input(*first)
+    b, keep_b = _csr_input(*second)
+    D = keep_a[0].shape[1]
+    if keep_b[0].shape[1] != D:
+        raise ValueError("the two inputs have rows of %d and %d columns" % (D, keep_b[0].shape[1]))
+    if keep_a[0].dtype != torch.float32:
+        raise TypeError("the first input of a two-input gather-reduce must be float32")
+    head = (ctypes.byref(a), ctypes.byref(b), ptr(plan.row_start), ptr(plan.hot_items), i64(plan.hot_cap),
+            ptr(plan.counts))
+    return head, D, keep_a[0].device, (a, b, keep_a, keep_b)
+
+
+def csr_gather_reduce2(plan, first, second, out=None, accumulate=False):
+    """``csr_gather_reduce`` with two inputs ``(rows, src, coef)`` over the lists of ``plan``
+    (``recis_csr_gather_reduce2``): ``out[u] (+)= sum_k coef1[k] * rows1[src1[k]] + coef2[k] *
+    rows2[src2[k]]``; the first input float32."""
+    head, D, dev, keep = _two_inputs(plan, first, second)
+    if out is None:
+        out = torch.empty((plan.U, D), dtype=torch.float32, device=dev)
+        accumulate = False
+    if out.dtype != torch.float32:
+        raise TypeError("csr_gather_reduce2 writes float32 rows")
+    check(lib().recis_csr_gather_reduce2(*head, ptr(out), i64(plan.U), i64(D), int(bool(accumulate)), stream_ptr(dev)))
+    return out
+
+
+def _two_inputs_table(plan, first, second, row_index, emb_blocks, block_size):
+    head, D, dev, keep = _two_inputs(plan, first, second)
+    require_cuda(row_index)
+    b0 = _check_blocks(emb_blocks, block_size)
+    if _row_bytes(b0) // b0.element_size() != D:
+        raise ValueError("gradient rows have %d columns, the table's rows %d" % (D, _row_bytes(b0) // b0.element_size()))
+    row_index = _ids64(row_index)
+    if row_index.numel() < plan.U:
+        raise ValueError("row_index holds %d rows for %d unique ids" % (row_index.numel(), plan.U))
+    return head + (i64(plan.U), i64(D), ptr(row_index)), b0, dev, (keep, row_index)
+
+
+def csr_gather_reduce2_adamw(plan, first, second, row_index, emb_blocks, beta1_t, beta2_t, exp_avg, exp_avg_sq, lr,
+                             beta1, beta2, weight_decay, eps, block_size):
+    """Two-input gather-reduce ending in the Adam-family row update (``recis_csr_gather_reduce2_adamw``)."""
+    head, b0, dev, keep = _two_inputs_table(plan, first, second, row_index, emb_blocks, block_size)
+    _check_blocks(exp_avg, block_size)
+    _check_blocks(exp_avg_sq, block_size)
+    if len(exp_avg) != len(emb_blocks) or len(exp_avg_sq) != len(emb_blocks):
+        raise ValueError("state slots must have as many blocks as the embedding slot")
+    require_cuda(beta1_t, beta2_t)
+    if beta1_t.dtype != beta2_t.dtype or beta1_t.dtype not in (torch.float32, torch.float64):
+        raise TypeError("beta1_t / beta2_t must both be float32 or float64")
+    check(lib().recis_csr_gather_reduce2_adamw(
+        *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(exp_avg)), ptr(block_ptr_table(exp_avg_sq)),
+        i64(len(emb_blocks)), i64(block_size), dtype_code(b0.dtype), ptr(beta1_t), ptr(beta2_t),
+        int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1), ctypes.c_double(beta2),
+        ctypes.c_double(weight_decay), ctypes.c_double(eps), stream_ptr(dev)))
+
+
+def csr_gather_reduce2_adagrad(plan, first, second, row_index, emb_blocks, accum_blocks, lr, eps, block_size):
+    """Two-input gather-reduce ending in the Adagrad row update (``recis_csr_gather_reduce2_adagrad``)."""
+    head, b0, dev, keep = _two_inputs_table(plan, first, second, row_index, emb_blocks, block_size)
+    _check_blocks(accum_blocks, block_size)
+    if len(accum_blocks) != len(emb_blocks):
+        raise ValueError("state slot must have as many blocks as the embedding slot")
+    check(lib().recis_csr_gather_reduce2_adagrad(
+        *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)),
+        i64(block_size), dtype_code(b0.dtype), ctypes.c_double(lr), ctypes.c_double(eps), stream_ptr(dev)))
 
 
 def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_index=None, weight=None, out_dtype=None):

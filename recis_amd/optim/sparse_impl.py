@@ -109,6 +109,16 @@ class _AdamFamilyImpl(_SparseOptimizerImpl):
                                     st["exp_avg"].kernel_blocks()[0], st["exp_avg_sq"].kernel_blocks()[0], self._lr,
                                     self._beta1, self._beta2, self._decay(), self._eps, chunk_rows, cover=cover)
 
+    def apply_planned2(self, ht, plan, first, second, index):
+        """``apply_planned`` for a table whose lookup fed two outputs: ``first`` and ``second`` are
+        ``(grad_rows, src, coef)`` of the two gradients (the first float32), summed per unique id in
+        one pass (``ops.csr_gather_reduce2_adamw``)."""
+        st = self._state[id(ht)]
+        chunks, chunk_rows = ht._slot_group.emb_slot().kernel_blocks()
+        ops.csr_gather_reduce2_adamw(plan, first, second, index, chunks, st["beta1"], st["beta2"],
+                                     st["exp_avg"].kernel_blocks()[0], st["exp_avg_sq"].kernel_blocks()[0], self._lr,
+                                     self._beta1, self._beta2, self._decay(), self._eps, chunk_rows)
+
     def state_dict(self):
         steps = {}
         for st in self._state.values():
@@ -175,6 +185,13 @@ class SparseAdagradImpl(_SparseOptimizerImpl):
         chunks, chunk_rows = ht._slot_group.emb_slot().kernel_blocks()
         ops.csr_gather_reduce_adagrad(grad_rows, plan, src, coef, index, chunks, st["accum"].kernel_blocks()[0],
                                       self._lr, self._eps, chunk_rows, cover=cover)
+
+    def apply_planned2(self, ht, plan, first, second, index):
+        """The Adagrad step of ``ht`` fused into the gather-reduce of two gradients (see the Adam family)."""
+        st = self._state[id(ht)]
+        chunks, chunk_rows = ht._slot_group.emb_slot().kernel_blocks()
+        ops.csr_gather_reduce2_adagrad(plan, first, second, index, chunks, st["accum"].kernel_blocks()[0],
+                                       self._lr, self._eps, chunk_rows)
 
     def state_dict(self):
         return {}, {}

@@ -400,3 +400,87 @@ def test_fused_gather_reduce_update_equals_the_two_calls(rng, kind, D, row_dtype
         assert torch.equal(a, b)
     assert torch.equal(b1, b1f) and torch.equal(b2, b2f)
     assert _lib.poll_device_errors() == 0
+
+
+def _two_gradient_case(rng, D, tile_dtype, n_hot=3):
+    """A lookup whose rows feed a mean-pooled output and a padded gather: ids (a few of them with
+    thousands of occurrences), the plan, and both gradients with their src / coef arrays."""
+    batch, seq = [300, 211, 64], [12, 5, 40]
+    lens = np.concatenate([rng.integers(0, 30, size=b) for b in batch])
+    off = np.concatenate([[0], np.cumsum(lens)])
+    n = int(off[-1])
+    ids = np.where(rng.random(n) < 0.4, rng.integers(0, n_hot, size=n), rng.integers(0, 3000, size=n))
+    plan = ops.ids_unique_plan(_dev(ids))
+    off_dev = _dev(off.astype(np.int32))
+    S = len(off) - 1
+    g_pool = rng.standard_normal((S, D)).astype(np.float32)
+    rows = sum(b * s for b, s in zip(batch, seq))
+    g_tile = _dev(rng.standard_normal((rows, D)).astype(np.float32)).to(tile_dtype)
+    src_p, coef_p = plan.src_coef_for_pool(off_dev, None, True)
+    src_t = plan.src_for_tile(batch, seq, off_dev)
+    return plan, batch, seq, off, (_dev(g_pool), src_p, coef_p), (g_tile, src_t, None)
+
+
+@pytest.mark.parametrize("D,tile_dtype", [(16, torch.float32), (128, torch.bfloat16), (40, torch.float16), (64, torch.float32)])
+def test_two_input_gather_reduce_matches_oracle(rng, D, tile_dtype):
+    """recis_csr_gather_reduce2 against the oracle's two backward passes added up (the backward of
+    mean pooling and of the padded gather into the same unique rows), and against the two
+    single-input calls it replaces."""
+    plan, batch, seq, off, first, second = _two_gradient_case(rng, D, tile_dtype)
+    inv = plan.inverse.cpu().numpy().astype(np.int64)
+    got = ops.csr_gather_reduce2(plan, first, second)
+    g_tile32 = second[0].float().cpu().numpy()
+    exp = (oracle.segment_reduce_backward(first[0].cpu().numpy(), None, inv, off, plan.U, "mean").astype(np.float64)
+           + oracle.ragged_tile_back(batch, seq, inv, off, g_tile32, plan.U))
+    # fp32 sums of up to thousands of terms in another order: atol scales with the summed magnitude
+    mag = np.zeros(plan.U)
+    np.add.at(mag, inv, 1.0)
+    tol = 1e-6 * np.maximum(1.0, mag)[:, None] * 8
+    assert np.all(np.abs(got.cpu().numpy() - exp) <= 1e-5 * np.abs(exp) + tol)
+    two = ops.csr_gather_reduce(first[0], plan, first[1], first[2])
+    two = ops.csr_gather_reduce(second[0], plan, second[1], None, out=two, accumulate=True)
+    assert np.all(np.abs(got.cpu().numpy() - two.cpu().numpy()) <= 1e-5 * np.abs(exp) + tol)
+    again = ops.csr_gather_reduce2(plan, first, second, out=got.clone(), accumulate=True)
+    torch.testing.assert_close(again, 2 * got, rtol=1e-6, atol=1e-6)
+    assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("kind", ["adamw", "adagrad"])
+@pytest.mark.parametrize("D,row_dtype,tile_dtype", [(16, torch.float32, torch.float32), (128, torch.bfloat16, torch.bfloat16),
+                                                    (128, torch.bfloat16, torch.float32), (24, torch.float16, torch.float16)])
+def test_two_input_fused_update_equals_gather_reduce_then_update(rng, kind, D, row_dtype, tile_dtype):
+    """recis_csr_gather_reduce2_adamw / _adagrad against recis_csr_gather_reduce2 into an fp32 buffer
+    followed by the row update (bit-exact against the oracle in test_gpu_table.py): the same rows
+    and state bit for bit, negative row indices skipped, two steps."""
+    plan, batch, seq, off, first, second = _two_gradient_case(rng, D, tile_dtype)
+    U, bs, nb = plan.U, 1024, 4
+    row_index = torch.from_numpy(rng.permutation(bs * nb)[:U]).cuda()
+    row_index[::13] = -1
+    mk = lambda: [_dev(rng.random((bs, D)).astype(np.float32)).to(row_dtype) for _ in range(nb)]
+    emb, s0, s1 = mk(), mk(), mk()
+    emb2, s02, s12 = [b.clone() for b in emb], [b.clone() for b in s0], [b.clone() for b in s1]
+    b1, b2 = torch.tensor(0.9, device="cuda"), torch.tensor(0.999, device="cuda")
+    b1f, b2f = b1.clone(), b2.clone()
+    keep = row_index >= 0
+    for _ in range(2):
+        g = ops.csr_gather_reduce2(plan, first, second)
+        if kind == "adamw":
+            ops.block_apply_adamw(row_index[keep], g[keep], emb, b1, b2, None, s0, s1, 1e-2, 0.9, 0.999, 0.99, 1e-8, bs)
+            ops.csr_gather_reduce2_adamw(plan, first, second, row_index, emb2, b1f, b2f, s02, s12, 1e-2, 0.9, 0.999,
+                                         0.99, 1e-8, bs)
+        else:
+            ops.block_apply_adagrad(row_index[keep], g[keep], emb, s0, 1e-2, 1e-8, bs)
+            ops.csr_gather_reduce2_adagrad(plan, first, second, row_index, emb2, s02, 1e-2, 1e-8, bs)
+    for a, b in zip(emb + s0 + (s1 if kind == "adamw" else []), emb2 + s02 + (s12 if kind == "adamw" else [])):
+        assert torch.equal(a, b)
+    assert torch.equal(b1, b1f) and torch.equal(b2, b2f)
+    assert _lib.poll_device_errors() == 0
+
+
+def test_two_input_gather_reduce_refuses_what_it_does_not_support(rng):
+    plan, batch, seq, off, first, second = _two_gradient_case(rng, 16, torch.float32)
+    half = (first[0].to(torch.bfloat16), first[1], first[2])
+    with pytest.raises(TypeError):
+        ops.csr_gather_reduce2(plan, half, second)                   # the first input must be float32
+    with pytest.raises(ValueError):
+        ops.csr_gather_reduce2(plan, first, (second[0][:, :8].contiguous(), second[1], None))

@@ -172,6 +172,32 @@ def test_config5_step_properties():
     g = o.segment_reduce_backward_plan(wl.g_pool, None, wl.offsets, plan, "mean")
     exp = (wl.g_pool.double() * (lens > 0).view(-1, 1)).sum(0)
     torch.testing.assert_close(g.double().sum(0), exp, rtol=1e-5, atol=1e-2)
+    # what the timed step runs: both gradients summed and the Adagrad update in one launch. On a sample of
+    # rows: the oracle's Adagrad (fp32 arithmetic on the bf16 rows widened) with the gradient that the
+    # two-input gather-reduce writes, which in turn is the sum of the two single-input passes.
+    src_t = plan.src_for_tile(wl.batch, wl.seq, wl.offsets)
+    g2 = o.csr_gather_reduce2(plan, (wl.g_pool,) + plan.src_coef_for_pool(wl.offsets, None, True), (wl.g_tile, src_t, None))
+    both = o.csr_gather_reduce(wl.g_tile, plan, src_t, out=g.clone(), accumulate=True)
+    scale = both.abs().amax(1, keepdim=True).clamp_(min=1.0)
+    assert float(((g2 - both).abs() / scale).max()) < 1e-4      # hot rows sum thousands of bf16 terms in another order
+    pick = torch.randperm(U, device="cuda")[:4096]
+    rows_at = index[pick]
+    names = [s.name() for s in wl.table.slot_group().slots()]
+    before = [_slot_rows(wl.table, n, rows_at).float().cpu().numpy() for n in names[:2]]
+    wl.bwd_update(plan, index)
+    after = [_slot_rows(wl.table, n, rows_at).float().cpu().numpy() for n in names[:2]]
+    # the accumulator first (the oracle's update of it, stored as bf16), then the oracle's row update
+    # reading the STORED accumulator, as a bf16 table does
+    bf16 = lambda a: torch.from_numpy(a).to(torch.bfloat16).float().numpy()
+    gp = g2[pick].cpu().numpy()
+    w, acc = [b.copy() for b in before]
+    oracle.block_apply_adagrad(np.arange(4096), gp, [w], [acc], 0.01, 1e-8, 4096)
+    acc_stored = bf16(acc)
+    np.testing.assert_allclose(after[1], acc_stored, rtol=2 ** -7, atol=1e-12)
+    w2, acc2 = before[0].copy(), (acc_stored - gp * gp).astype(np.float32)   # so that acc2 + g*g is the stored value
+    oracle.block_apply_adagrad(np.arange(4096), gp, [w2], [acc2], 0.01, 1e-8, 4096)
+    step = np.abs(w2 - before[0])
+    assert np.all(np.abs(after[0] - w2) <= 2 ** -7 * np.maximum(np.abs(w2), step) + 1e-9)
     assert _lib.poll_device_errors() == 0
 
 
