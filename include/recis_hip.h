@@ -559,11 +559,12 @@ int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_
  * (the sequence features of the reference: csrc/ops/embedding_segment_reduce_kernel.cu:276-350
  * and the ragged_tile backward, ragged_tile_kernel.cu), has two gradients per occurrence; the
  * reference scatters each into the unique rows by itself, this sums both in the pass that owns the
- * row. The first input must be fp32; the second fp32, or bf16 / f16 where noted.
- *   recis_csr_gather_reduce2          out (fp32 [U, D]) (+)= sum; second input fp32 / bf16 / f16
+ * row.
+ *   recis_csr_gather_reduce2          out (fp32 [U, D]) (+)= sum; each input fp32, bf16 or f16 (two
+ *                                     half-precision inputs must have one type)
  *   recis_csr_gather_reduce2_adamw    the sum is the gradient of table row row_index[u]: the row
  *   recis_csr_gather_reduce2_adagrad  update is applied at once, as by recis_csr_gather_reduce_adamw
- *                                     / _adagrad; second input fp32 or of the table's row type
+ *                                     / _adagrad; each input fp32 or of the table's row type
  * The result equals recis_csr_gather_reduce(a) followed by recis_csr_gather_reduce(b, accumulate)
  * up to fp32 rounding (here both inputs go through one chain of fused multiply-adds, there the
  * first sum is rounded to the output before the second is added).
@@ -575,6 +576,11 @@ typedef struct recis_csr_input {
   const int32_t* src; /* [n] input row per list entry */
   const void* coef;   /* [n] per list entry, or NULL */
   int coef_dtype;
+  /* the SECOND input may come as n_parts (<= 8) arrays laid end to end in src's numbering, as in
+   * recis_csr_gather_reduce_parts (rows and n_rows unused then); n_parts = 0: one array */
+  const void* const* part_rows; /* host array of device pointers */
+  const int64_t* part_counts;   /* host array: rows per part */
+  int n_parts;
 } recis_csr_input;
 int recis_csr_gather_reduce2(const recis_csr_input* a, const recis_csr_input* b, const int32_t* row_start,
                              const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev,

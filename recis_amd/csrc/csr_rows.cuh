@@ -55,11 +55,12 @@ struct CsrArgs {
   int64_t hot_cap;
   float* hot_part;           // [hot_cap, D]
   int64_t cold_blocks;       // the last cold_blocks workgroups work per row, the ones before per hot item
-  // PARTS kernels: the input rows are n_parts arrays laid end to end in src's numbering; part f
-  // holds rows [part_lo[f], part_lo[f + 1])
+  // PARTS kernels: the input rows as n_parts arrays laid end to end in src's numbering; part f
+  // holds rows from part_lo32[f] on (INT32_MAX for an unused part). Of the one input; in kernels
+  // with two inputs, of the SECOND.
   int n_parts;
   const void* part_rows[kMaxParts];
-  int64_t part_lo[kMaxParts + 1];
+  int32_t part_lo32[kMaxParts];
 };
 
 // What a gather-reduce launch does with the finished sum of row u (template parameter EPI):
@@ -110,25 +111,23 @@ struct SrcView {
   int64_t n_rows, lo, hi;
 };
 
-// Row s of the input: of the one array, or of the part that holds it.
+// Row s of the input: of the one array (PARTS == false), or of the part that holds it. No
+// branches: the callers keep several of these loads in flight.
 template <typename TIn, bool PARTS>
 __device__ __forceinline__ const TIn* src_row(const TIn* rows, const CsrArgs& a, int64_t s) {
   if constexpr (!PARTS) {
     return rows + s * a.D;
   } else {
-    int f = 0;
-#pragma unroll
-    for (int k = 1; k < kMaxParts; ++k) f += (k < a.n_parts && s >= a.part_lo[k]) ? 1 : 0;
     const TIn* base = static_cast<const TIn*>(a.part_rows[0]);
-    int64_t lo = 0;
+    int32_t lo = 0;
+    const int32_t s32 = static_cast<int32_t>(s);  // src entries are 32-bit, and so are the parts' first rows
 #pragma unroll
     for (int k = 1; k < kMaxParts; ++k) {
-      if (k == f) {
-        base = static_cast<const TIn*>(a.part_rows[k]);
-        lo = a.part_lo[k];
-      }
+      const bool past = s32 >= a.part_lo32[k];  // the first row of an unused part is past every row
+      base = past ? static_cast<const TIn*>(a.part_rows[k]) : base;
+      lo = past ? a.part_lo32[k] : lo;
     }
-    return base + (s - lo) * a.D;
+    return base + static_cast<int64_t>(s32 - lo) * a.D;
   }
 }
 
@@ -154,12 +153,16 @@ __device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const C
   const int lane = threadIdx.x & (kWave - 1);
   for (int32_t cb = e_begin; cb < e_end; cb += kWave) {
     const int n_here = min(kWave, e_end - cb);
+    // the row this lane's entry reads (none: -1 / NULL). With parts, where it lies is worked out once
+    // per entry, here, not by every lane that gathers it, and the address travels to those lanes.
     int32_t s_mine = -1;
+    const TIn* p_mine = nullptr;
     float w_mine = 0.f;
     if (lane < n_here) {
       const int32_t sv = s.src[cb + lane];
       if (sv >= s.lo && sv < s.hi) {
         s_mine = sv;
+        if constexpr (PARTS) p_mine = src_row<TIn, true>(s.rows, a, sv);
         w_mine = s.coef ? load_coef(s.coef, s.coef_dt, cb + lane) : 1.0f;
       } else if (static_cast<int64_t>(sv) >= s.n_rows) {
         raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
@@ -170,13 +173,22 @@ __device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const C
       float w[kFly];
 #pragma unroll
       for (int k = 0; k < kFly; ++k) {
-        const int e = q0 + g + k * groups;
+        const int first = q0 + k * groups;  // this round's entries: first + 0 .. first + groups - 1, one per group
+        const int e = first + g;
         const int from = min(e, kWave - 1);
-        int32_t id = __shfl(s_mine, from, kWave);
+        const TIn* row;
+        if constexpr (PARTS) {
+          const uintptr_t bits = reinterpret_cast<uintptr_t>(p_mine);
+          const uint32_t p_lo = __shfl(static_cast<uint32_t>(bits), from, kWave);
+          const uint32_t p_hi = __shfl(static_cast<uint32_t>(bits >> 32), from, kWave);
+          row = reinterpret_cast<const TIn*>((static_cast<uintptr_t>(p_hi) << 32) | p_lo);
+        } else {
+          const int32_t id = __shfl(s_mine, from, kWave);
+          row = id >= 0 ? s.rows + static_cast<int64_t>(id) * a.D : nullptr;
+        }
         w[k] = s.coef ? __shfl(w_mine, from, kWave) : 1.0f;
-        if (e >= n_here || !col_ok) id = -1;
-        if (id >= 0) {
-          const TIn* row = src_row<TIn, PARTS>(s.rows, a, id);
+        if (e >= n_here || !col_ok) row = nullptr;
+        if (row != nullptr) {
           if (s.nt) {
             load_pack_stream<TIn, VEC>(row + c0, v[k]);
           } else {
@@ -208,14 +220,14 @@ constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of
 // the partial rows of every hot row in chunk order. No atomics anywhere.
 // SHUFFLE: long lists go through wave_gather_range (pays off when a wave has at most eight lane
 // groups, i.e. rows of 128 bytes and more); otherwise every group loads its own entries.
-// TIn2 != void: every list entry adds a row of a second input as well (see CsrArgs).
+// TIn2 != void: every list entry adds a row of a second input as well (see CsrArgs); PARTS then
+// says that the second input comes in parts.
 template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false, int EPI = kEpiStore,
           typename TIn2 = void>
 __global__ void __launch_bounds__(kBlock, (!SHUFFLE && EPI != kEpiStore && (std::is_void<TIn2>::value || sizeof(TOut) == 4))
                                               ? 8 : 1)  // 64 registers where that costs no spills
 csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
   constexpr bool TWO = !std::is_void<TIn2>::value;
-  static_assert(!(TWO && PARTS), "a second input goes with one array as the first");
   using TSecond = typename std::conditional<TWO, TIn2, TIn>::type;
   extern __shared__ float s_part[];  // [waves][D], hot part only
   const int D = a.D;
@@ -275,16 +287,16 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   };
   // the first input's entries, then the second's: one fixed order of summation
   auto gather_sum = [&](int32_t first, int32_t last, int32_t step, int c0, float (&acc)[VEC]) {
-    gather_one(in1, std::integral_constant<bool, PARTS>{}, first, last, step, c0, acc);
-    if constexpr (TWO) gather_one(in2, std::false_type{}, first, last, step, c0, acc);
+    gather_one(in1, std::integral_constant<bool, PARTS && !TWO>{}, first, last, step, c0, acc);
+    if constexpr (TWO) gather_one(in2, std::integral_constant<bool, PARTS>{}, first, last, step, c0, acc);
   };
   // the wave's sum over the list entries [first, last) for columns c0.., the same in every group
   auto wave_sum = [&](int32_t first, int32_t last, int c0, bool col_ok, float (&acc)[VEC]) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
     if constexpr (SHUFFLE) {
-      wave_gather_range<TIn, VEC, PARTS>(in1, a, first, last, c0, col_ok, g, groups, acc);
-      if constexpr (TWO) wave_gather_range<TSecond, VEC, false>(in2, a, first, last, c0, col_ok, g, groups, acc);
+      wave_gather_range<TIn, VEC, PARTS && !TWO>(in1, a, first, last, c0, col_ok, g, groups, acc);
+      if constexpr (TWO) wave_gather_range<TSecond, VEC, PARTS>(in2, a, first, last, c0, col_ok, g, groups, acc);
     } else {
       if (col_ok) gather_sum(first + g, last, groups, c0, acc);
     }
@@ -478,6 +490,10 @@ struct CsrInput {
   const int32_t* src;
   const void* coef;  // or NULL
   int coef_dtype;
+  // the second of two inputs may come as n_parts arrays laid end to end (rows == NULL then)
+  const void* const* part_rows = nullptr;
+  const int64_t* part_counts = nullptr;
+  int n_parts = 0;
 };
 
 struct CsrRequest {
@@ -506,8 +522,10 @@ struct CsrRequest {
 
 // Checks, geometry, workspace and the launches of one gather-reduce. TWO picks the family of
 // kernels this translation unit instantiates: one input (any supported pair of input and output
-// types, PARTS included) or two inputs (the first fp32, the second fp32 or a half type).
-template <bool TWO>
+// types, PARTS included) or two inputs (each fp32 or the half type of the other / of the table).
+// ONLY_EPI >= 0: only the kernels with that ending are instantiated here (the others are refused),
+// so that the families can be compiled side by side.
+template <bool TWO, int ONLY_EPI = -1>
 int csr_gather_reduce_run(const CsrRequest& r) {
   const int64_t U = r.U, D = r.D, hot_cap = r.hot_cap;
   const int epi = r.epi, n_parts = r.n_parts;
@@ -522,9 +540,9 @@ int csr_gather_reduce_run(const CsrRequest& r) {
   RECIS_REQUIRE(r.in1.coef == nullptr || dtype_size(r.in1.coef_dtype), "invalid coef dtype");
   uintptr_t align_of = reinterpret_cast<uintptr_t>(r.in1.rows);
   for (int f = 0; f < n_parts; ++f) align_of |= reinterpret_cast<uintptr_t>(r.part_rows[f]);  // the coarsest alignment
-  // with two inputs the first is fp32 and may go in 32-byte packs, so that a half-precision second
-  // input still gets its 16 bytes per lane
-  const int vb_in = TWO ? pick_vec_bytes_max(D * in_sz, align_of, 32) : pick_vec_bytes(D * in_sz, align_of);
+  // with two inputs an fp32 one may go in 32-byte packs, so that a half-precision partner (or
+  // table row) still gets its 16 bytes per lane
+  const int vb_in = (TWO && in_sz == 4) ? pick_vec_bytes_max(D * in_sz, align_of, 32) : pick_vec_bytes(D * in_sz, align_of);
   // table blocks are allocator-aligned and are read and written in 16-byte packs at most
   const int vb_out = epi != kEpiStore ? pick_vec_bytes(D * out_sz, 16)
                                       : pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(r.out), 32);
@@ -535,16 +553,33 @@ int csr_gather_reduce_run(const CsrRequest& r) {
     const CsrInput& b = *r.in2;
     const int in2_sz = dtype_size(b.dtype);
     RECIS_REQUIRE(in2_sz, "invalid dtype of the second input");
-    RECIS_REQUIRE(b.n_rows >= 0 && (U == 0 || b.src), "second input: src must not be NULL");
-    RECIS_REQUIRE(b.rows != nullptr || b.n_rows == 0, "second input: rows must not be NULL");
+    RECIS_REQUIRE(b.n_parts >= 0 && b.n_parts <= kMaxParts, "second input: at most %d parts (got %d)", kMaxParts,
+                  b.n_parts);
+    int64_t n_rows2 = b.n_rows;
+    uintptr_t align2 = reinterpret_cast<uintptr_t>(b.rows);
+    if (b.n_parts > 0) {
+      RECIS_REQUIRE(b.part_rows && b.part_counts, "second input: NULL part tables");
+      n_rows2 = 0;
+      align2 = 0;
+      for (int f = 0; f < b.n_parts; ++f) {
+        RECIS_REQUIRE(b.part_counts[f] >= 0 && (b.part_rows[f] != nullptr || b.part_counts[f] == 0),
+                      "second input: bad part %d", f);
+        n_rows2 += b.part_counts[f];
+        align2 |= reinterpret_cast<uintptr_t>(b.part_rows[f]);
+      }
+    }
+    RECIS_REQUIRE(n_rows2 >= 0 && (U == 0 || b.src), "second input: src must not be NULL");
+    RECIS_REQUIRE(b.n_parts > 0 || b.rows != nullptr || n_rows2 == 0, "second input: rows must not be NULL");
     RECIS_REQUIRE(b.coef == nullptr || dtype_size(b.coef_dtype), "invalid coef dtype of the second input");
-    vec = std::max(1, std::min(vec, pick_vec_bytes(D * in2_sz, reinterpret_cast<uintptr_t>(b.rows)) / in2_sz));
+    const int vb2 = in2_sz == 4 ? pick_vec_bytes_max(D * in2_sz, align2, 32) : pick_vec_bytes(D * in2_sz, align2);
+    const int widest = 16 / std::min(std::min(in_sz, in2_sz), out_sz);  // 16 bytes of the narrowest type
+    vec = std::max(1, std::min(std::min(vec, widest), vb2 / in2_sz));
     a.rows2 = b.rows;
     a.src2 = b.src;
     a.coef2 = b.coef;
     a.coef2_dt = b.coef_dtype;
-    a.n_rows2 = b.n_rows;
-    a.nt_in2 = b.n_rows * D * in2_sz >= (int64_t(1) << 30);
+    a.n_rows2 = n_rows2;
+    a.nt_in2 = n_rows2 * D * in2_sz >= (int64_t(1) << 30);
   }
   a.row_start = r.row_start;
   a.src = r.in1.src;
@@ -568,12 +603,19 @@ int csr_gather_reduce_run(const CsrRequest& r) {
   a.counts = r.counts_dev;
   a.hot_cap = hot_cap;
   a.hot_part = nullptr;
-  a.n_parts = n_parts;
-  a.part_lo[0] = 0;
+  // the part table: of the one input, or of the second of two; the kernels find a row's part by
+  // comparing with the parts' first rows, so an unused part starts past every row
+  const void* const* parts_of = TWO ? r.in2->part_rows : r.part_rows;
+  const int64_t* counts_of = TWO ? r.in2->part_counts : r.part_counts;
+  a.n_parts = TWO ? r.in2->n_parts : n_parts;
+  int64_t part_first = 0;
   for (int f = 0; f < kMaxParts; ++f) {
-    a.part_rows[f] = f < n_parts ? r.part_rows[f] : nullptr;
-    a.part_lo[f + 1] = a.part_lo[f] + (f < n_parts ? r.part_counts[f] : 0);
+    a.part_rows[f] = f < a.n_parts ? parts_of[f] : nullptr;
+    a.part_lo32[f] = f < a.n_parts ? static_cast<int32_t>(part_first) : INT32_MAX;
+    if (f < a.n_parts) part_first += counts_of[f];
   }
+  RECIS_REQUIRE(part_first <= INT32_MAX, "the parts hold %lld rows, more than 32-bit src entries name",
+                (long long)part_first);
   int64_t hot_blocks = 0;
   if (hot_cap > 0 || r.extra_ws > 0) {
     void* ws = nullptr;
@@ -593,7 +635,7 @@ int csr_gather_reduce_run(const CsrRequest& r) {
     constexpr size_t in2_bytes = TWO ? sizeof(decltype(tin2)) : 1;
     return dispatch_vec(vec, [&](auto vtag) {
       constexpr int VEC = decltype(vtag)::value;
-      if constexpr (VEC * sizeof(TIn) > (TWO ? 32 : 16) || VEC * in2_bytes > 16 || VEC * sizeof(TOut) > 32) {
+      if constexpr (VEC * sizeof(TIn) > (TWO ? 32 : 16) || VEC * in2_bytes > 32 || VEC * sizeof(TOut) > 32) {
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
         const TIn* rin = static_cast<const TIn*>(r.in1.rows);
@@ -606,8 +648,13 @@ int csr_gather_reduce_run(const CsrRequest& r) {
           {
             RECIS_TIME_KERNEL(EPI == kEpiStore ? "csr_rows_kernel" : EPI == kEpiAdam ? "csr_rows_adam_kernel"
                                                                                       : "csr_rows_adagrad_kernel", stream)
-            if (n_parts > 0) {
-              if constexpr (sizeof(TOut) == 4 && EPI == kEpiStore && !TWO) {  // parts go to fp32 rows only
+            if (a.n_parts > 0) {
+              if constexpr (TWO) {  // the second input in parts
+                if (shuffle)
+                  csr_rows_kernel<TIn, TOut, VEC, true, true, EPI, TIn2><<<grid, block, lds, stream>>>(rin, o, a, f);
+                else
+                  csr_rows_kernel<TIn, TOut, VEC, false, true, EPI, TIn2><<<grid, block, lds, stream>>>(rin, o, a, f);
+              } else if constexpr (sizeof(TOut) == 4 && EPI == kEpiStore) {  // parts go to fp32 rows only
                 if (shuffle)
                   csr_rows_kernel<TIn, TOut, VEC, true, true><<<grid, block, lds, stream>>>(rin, o, a, f);
                 else
@@ -626,14 +673,17 @@ int csr_gather_reduce_run(const CsrRequest& r) {
           }
           return RECIS_OK;
         };
+        constexpr bool all = ONLY_EPI < 0;
         if (epi == kEpiAdam) {
-          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdam>{});
+          if constexpr ((all || ONLY_EPI == kEpiAdam) && VEC * sizeof(TOut) <= 16)
+            return launch(std::integral_constant<int, kEpiAdam>{});
         } else if (epi == kEpiAdagrad) {
-          if constexpr (VEC * sizeof(TOut) <= 16) return launch(std::integral_constant<int, kEpiAdagrad>{});
+          if constexpr ((all || ONLY_EPI == kEpiAdagrad) && VEC * sizeof(TOut) <= 16)
+            return launch(std::integral_constant<int, kEpiAdagrad>{});
         } else {
-          return launch(std::integral_constant<int, kEpiStore>{});
+          if constexpr (all || ONLY_EPI == kEpiStore) return launch(std::integral_constant<int, kEpiStore>{});
         }
-        return fail(RECIS_ERR_ARG, "internal: vector too wide for a fused row update");
+        return fail(RECIS_ERR_ARG, "internal: no kernel for this ending and vector width here");
       }
     });
   };
@@ -650,23 +700,39 @@ int csr_gather_reduce_run(const CsrRequest& r) {
     }
     return fail(RECIS_ERR_ARG, "unsupported dtype pair (rows=%d, out=%d)", rows_dtype, out_dtype);
   } else {
-    // the first input fp32 (a pooled output's gradient); the second fp32 or of the output's type
-    // (the gradient of an output that has the table's row type)
+    // each input fp32 or a half type; two half inputs of one type; with a fused row update a
+    // half input has the table's type
     const int d2 = r.in2->dtype;
-    RECIS_REQUIRE(rows_dtype == RECIS_F32, "two inputs: the first must be fp32 (got dtype %d)", rows_dtype);
+    auto second = [&](auto tin, auto tout) {
+      using TIn = decltype(tin);
+      using TOut = decltype(tout);
+      constexpr bool half_in = sizeof(TIn) == 2, half_out = sizeof(TOut) == 2;
+      if (d2 == RECIS_F32) return with_types(tin, tout, float{});
+      if constexpr (half_in) {
+        if (d2 == rows_dtype) return with_types(tin, tout, tin);
+      } else if constexpr (half_out) {
+        if (d2 == out_dtype) return with_types(tin, tout, tout);
+      } else {
+        if (epi == kEpiStore) {
+          if (d2 == RECIS_BF16) return with_types(tin, tout, bf16_t{});
+          if (d2 == RECIS_F16) return with_types(tin, tout, f16_t{});
+        }
+      }
+      return fail(RECIS_ERR_ARG, "unsupported dtypes (inputs=%d and %d, out=%d)", rows_dtype, d2, out_dtype);
+    };
     if (out_dtype == RECIS_F32) {
-      if (d2 == RECIS_F32) return with_types(float{}, float{}, float{});
+      if (rows_dtype == RECIS_F32) return second(float{}, float{});
       if (epi == kEpiStore) {
-        if (d2 == RECIS_BF16) return with_types(float{}, float{}, bf16_t{});
-        if (d2 == RECIS_F16) return with_types(float{}, float{}, f16_t{});
+        if (rows_dtype == RECIS_BF16) return second(bf16_t{}, float{});
+        if (rows_dtype == RECIS_F16) return second(f16_t{}, float{});
       }
     } else if (epi != kEpiStore) {
-      if (out_dtype == RECIS_BF16 && d2 == RECIS_F32) return with_types(float{}, bf16_t{}, float{});
-      if (out_dtype == RECIS_BF16 && d2 == RECIS_BF16) return with_types(float{}, bf16_t{}, bf16_t{});
-      if (out_dtype == RECIS_F16 && d2 == RECIS_F32) return with_types(float{}, f16_t{}, float{});
-      if (out_dtype == RECIS_F16 && d2 == RECIS_F16) return with_types(float{}, f16_t{}, f16_t{});
+      if (out_dtype == RECIS_BF16 && rows_dtype == RECIS_F32) return second(float{}, bf16_t{});
+      if (out_dtype == RECIS_BF16 && rows_dtype == RECIS_BF16) return second(bf16_t{}, bf16_t{});
+      if (out_dtype == RECIS_F16 && rows_dtype == RECIS_F32) return second(float{}, f16_t{});
+      if (out_dtype == RECIS_F16 && rows_dtype == RECIS_F16) return second(f16_t{}, f16_t{});
     }
-    return fail(RECIS_ERR_ARG, "unsupported dtypes (second input=%d, out=%d)", d2, out_dtype);
+    return fail(RECIS_ERR_ARG, "unsupported dtypes (inputs=%d and %d, out=%d)", rows_dtype, d2, out_dtype);
   }
 }
 
@@ -693,7 +759,7 @@ inline int fill_fuse_args(FuseArgs& f, const int64_t* row_index, void* const* em
 // the betas advance first, even when no row is touched (cal_alpha); alpha lives in the stream's
 // workspace behind the partial rows of the hot items, so a first pass with U = 0 reserves the
 // workspace and learns where alpha goes, launching nothing.
-template <bool TWO>
+template <bool TWO, int ONLY_EPI = -1>
 int run_with_alpha(CsrRequest& r, FuseArgs& f, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
                    double beta1, double beta2, double weight_decay, double eps) {
   void* alpha = nullptr;
@@ -701,7 +767,7 @@ int run_with_alpha(CsrRequest& r, FuseArgs& f, void* beta1_t, void* beta2_t, int
   probe.U = 0;
   probe.extra_ws = 256;
   probe.extra_out = &alpha;
-  if (int rc = csr_gather_reduce_run<TWO>(probe)) return rc;
+  if (int rc = csr_gather_reduce_run<TWO, ONLY_EPI>(probe)) return rc;
   if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, static_cast<double*>(alpha), lr, beta1, beta2, r.stream))
     return rc;
   if (r.U == 0) return RECIS_OK;
@@ -712,8 +778,30 @@ int run_with_alpha(CsrRequest& r, FuseArgs& f, void* beta1_t, void* beta2_t, int
   f.adam.eps = eps;
   r.extra_ws = 256;
   r.extra_out = &alpha;
-  return csr_gather_reduce_run<TWO>(r);
+  return csr_gather_reduce_run<TWO, ONLY_EPI>(r);
 }
+
+// The request of an entry point with two inputs; `second` must outlive the request.
+inline CsrRequest two_input_request(const recis_csr_input* a, const recis_csr_input* b, CsrInput& second,
+                             const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
+                             const int64_t* counts_dev, int64_t U, int64_t D, void* stream_) {
+  CsrRequest r;
+  r.in1 = CsrInput{a->rows, a->rows_dtype, a->n_rows, a->src, a->coef, a->coef_dtype};
+  second = CsrInput{b->rows, b->rows_dtype, b->n_rows, b->src, b->coef, b->coef_dtype};
+  second.part_rows = b->part_rows;
+  second.part_counts = b->part_counts;
+  second.n_parts = b->n_parts;
+  r.in2 = &second;
+  r.row_start = row_start;
+  r.hot_items = hot_items;
+  r.hot_cap = hot_cap;
+  r.counts_dev = counts_dev;
+  r.U = U;
+  r.D = D;
+  r.stream = static_cast<hipStream_t>(stream_);
+  return r;
+}
+
 
 }  // namespace
 }  // namespace recis_hip

@@ -173,6 +173,52 @@ class LookupPoolFunction(torch.autograd.Function):
         return None, None, None, None, None, None, None, None
 
 
+class LookupTileFunction(torch.autograd.Function):
+    """Lookup of a plan's unique ids and the padded gather of several features at once, ONE output
+    per feature (``[bs[f], tile_len[f] * D]``, views of one buffer: the list form of the tile
+    combiner, recis/nn/modules/embedding_engine.py:383-411). Backward hands the features' gradients
+    to the table unsummed, as separate arrays: no concatenation of the padded gradients, and the
+    optimizer step sums them (together with the gradient of a pooled output of the same lookup, if
+    there is one) where it updates the rows."""
+
+    @staticmethod
+    def forward(ctx, backward_holder, impl, plan, offsets, bs, tile_len, readonly):
+        bs, tile_len = [int(b) for b in bs], [int(t) for t in tile_len]
+        U = plan.U   # the padded gather reads a dense copy of the rows: this forward needs the count
+        if readonly:
+            index = impl.lookup_index(plan.unique, True)
+        else:
+            index = impl.plan_index(plan)   # a plan made for this table brings the rows along
+            if index is None:
+                index = impl.lookup_index_unsettled(plan)
+            index = impl.settle_lookup(index, U, plan)
+        chunks, chunk_rows = impl.emb_blocks()
+        rows = ops.block_gather(index, chunks, chunk_rows, -1, readonly)
+        out, _ = ops.ragged_tile(bs, tile_len, plan.inverse, offsets, rows)
+        D = rows.shape[1]
+        ctx.impl, ctx.plan, ctx.readonly, ctx.bs, ctx.tile_len, ctx.D = impl, plan, readonly, bs, tile_len, D
+        ctx.save_for_backward(index, offsets)
+        ctx.mark_non_differentiable(index)
+        n_rows = [b * t for b, t in zip(bs, tile_len)]
+        return (index,) + tuple(p.view(b, t * D) for p, b, t in zip(torch.split(out, n_rows), bs, tile_len))
+
+    @staticmethod
+    def backward(ctx, _grad_index, *grads):
+        index, offsets = ctx.saved_tensors
+        plan, D = ctx.plan, ctx.D
+        n_rows = [b * t for b, t in zip(ctx.bs, ctx.tile_len)]
+        like = next((g for g in grads if g is not None), None)
+        if like is not None:
+            src = plan.src_for_tile(ctx.bs, ctx.tile_len, offsets.contiguous())
+            parts = [(g if g is not None else like.new_zeros((n, D))).reshape(n, D) for g, n in zip(grads, n_rows)]
+            key = None if ctx.readonly else plan.serial
+            if len(parts) <= 8 and len({p.dtype for p in parts}) == 1:
+                ctx.impl.accept_planned_grad(index, plan, parts, src, key=key, may_miss=ctx.readonly)
+            else:
+                ctx.impl.accept_planned_grad(index, plan, torch.cat(parts), src, key=key, may_miss=ctx.readonly)
+        return (None,) * 7
+
+
 def _pools_out_of_the_table(hashtable, opt, n_occ, n_offsets):
     """Whether lookup_and_pool takes the path that pools straight out of the table rows."""
     float_table = hashtable._dtype in (torch.float32, torch.bfloat16, torch.float16)

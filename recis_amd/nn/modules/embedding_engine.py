@@ -22,7 +22,7 @@ import torch
 from ... import ops
 from ...ragged.tensor import RaggedTensor
 from ..functional.embedding_ops import RaggedTileParts
-from .embedding import EmbeddingOption, lookup_and_pool, lookup_unique_rows, make_plan
+from .embedding import EmbeddingOption, LookupTileFunction, lookup_and_pool, lookup_unique_rows, make_plan
 from .hashtable import HashTable, gen_slice
 
 
@@ -172,7 +172,11 @@ class EmbeddingEngine(torch.nn.Module):
                     else:
                         offsets = ops.merge_offsets(offs, [v.numel() for v in vals])
                     if opt0.combiner == "tile":
-                        plan = ops.ids_unique_plan(ids, wait=False, need_pos=False)
+                        if (table.training and opt0.trainable and opt0.admit_hook is None
+                                and table._dtype in (torch.float32, torch.bfloat16, torch.float16)):
+                            plan = table._hashtable_impl.plan_lookup(ids)   # dedup + find-or-insert, one pass
+                        else:
+                            plan = ops.ids_unique_plan(ids, wait=False, need_pos=False)
                     else:  # lean (no per-occurrence arrays) only if no other option can come to share it
                         alone = sum(1 for k in runtime.values() if any(inputs[n] is inputs[names[0]] for n in k)) == 1
                         plan = make_plan(table, ids, offsets, opt0, any_weight, unit_segments=all_unit and alone)
@@ -191,6 +195,13 @@ class EmbeddingEngine(torch.nn.Module):
                         width = pooled.shape[1]
                         parts = [p.view(b, t * width) for p, b, t in zip(
                             torch.split(pooled, [b * t for b, t in zip(seg_counts, tile_lens)]), seg_counts, tile_lens)]
+                    elif (table.training and opt0.trainable and opt0.admit_hook is None
+                          and table._dtype in (torch.float32, torch.bfloat16, torch.float16)):
+                        # lookup and padded gather as one function: the rows the plan brought along are used
+                        # (no second lookup of the same ids) and the gradients reach the table unsummed
+                        index, *parts = LookupTileFunction.apply(table._backward_holder, table._hashtable_impl,
+                                                                 plan, offsets, seg_counts, tile_lens, False)
+                        table._filter_hook_impl(index)
                     else:
                         emb = lookup_unique_rows(table, plan.unique, opt0.admit_hook, opt0.trainable,
                                                  grad_key=plan.serial)

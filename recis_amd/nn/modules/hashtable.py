@@ -314,7 +314,7 @@ class HashtableImpl:
         self._slice = Slice(slice_begin, slice_end, slice_size)
         self._idmap = ops.IdMap(device, reserve=reserve_rows)
         self._grad_index, self._grad, self._grad_unique, self._grad_keys = [], [], [], {}
-        self._planned = None   # a gradient handed over as a sum still to be taken (accept_planned_grad)
+        self._planned = []   # gradients handed over as sums still to be taken (accept_planned_grad): two at most
 
     # ------------------------------------------------------------- storage
     def _make_room(self, incoming):
@@ -464,17 +464,43 @@ class HashtableImpl:
     def accept_planned_grad(self, index, plan, rows, src, coef=None, cover=None, key=None, may_miss=False):
         """A gradient handed over before it is summed: the gradient of ``plan``'s unique id ``u`` (table row
         ``index[u]``; negative = the table does not hold the key, no gradient) is the sum over u's occurrence
-        list of ``coef * rows[src]`` (``ops.csr_gather_reduce``). If it stays the only gradient of the step, an
-        optimizer that can (``apply_planned``) takes the sum and applies the row update in one launch and the
-        ``[U, D]`` gradient is never written; anything else that asks for the gradient (``grad``, ``grad_pairs``,
-        a second gradient, accumulation over several steps) gets it summed first, as ``accept_grad`` would have.
-        ``may_miss``: ``index`` may hold negative entries (a read-only lookup)."""
-        if self._grad or self._planned is not None:
-            self._sum_planned()
-            g = ops.csr_gather_reduce(rows, plan, src, coef, cover=cover)
-            self._accept_summed(index, g, key, may_miss)
+        list of ``coef * rows[src]`` (``ops.csr_gather_reduce``; ``rows`` may be a list of arrays laid end to
+        end, ``ops.csr_gather_reduce_parts``). If it stays the only gradient of the step, or one of the two
+        gradients of one plan (a lookup whose rows fed a pooled and a padded output; same ``key``), an optimizer
+        that can (``apply_planned`` / ``apply_planned2``) takes the sum and applies the row update in one launch
+        and the ``[U, D]`` gradient is never written; anything else that asks for the gradient (``grad``,
+        ``grad_pairs``, a further gradient, accumulation over several steps) gets it summed first, as
+        ``accept_grad`` would have. ``may_miss``: ``index`` may hold negative entries (a read-only lookup)."""
+        entry = (index, plan, rows, src, coef, cover, key, may_miss)
+        if not self._grad and len(self._planned) == 1 and self._one_launch_sums(self._planned[0], entry):
+            self._planned.append(entry)
             return
-        self._planned = (index, plan, rows, src, coef, cover, key, may_miss)
+        if self._grad or self._planned:
+            self._sum_planned()
+            self._accept_summed(index, self._sum_of(entry), key, may_miss)
+            return
+        self._planned = [entry]
+
+    def _one_launch_sums(self, a, b):
+        """Whether two unsummed gradients are the two inputs of one ``ops.csr_gather_reduce2*`` launch: of one
+        plan and the same rows (one key), whole (no cover), each float32 or of the table's type, at most one
+        of them in parts."""
+        if a[1] is not b[1] or a[6] is None or a[6] != b[6] or a[7] != b[7] or a[5] is not None or b[5] is not None:
+            return False
+        if a[0].shape != b[0].shape:
+            return False
+        in_parts = [not torch.is_tensor(e[2]) for e in (a, b)]
+        if all(in_parts) or any(p and (e[4] is not None or not 1 <= len(e[2]) <= 8) for p, e in zip(in_parts, (a, b))):
+            return False
+        dtype_of = lambda e: e[2].dtype if torch.is_tensor(e[2]) else e[2][0].dtype
+        return all(dtype_of(e) in (torch.float32, self._dtype) for e in (a, b))
+
+    @staticmethod
+    def _sum_of(entry):
+        index, plan, rows, src, coef, cover, key, may_miss = entry
+        if torch.is_tensor(rows):
+            return ops.csr_gather_reduce(rows, plan, src, coef, cover=cover)
+        return ops.csr_gather_reduce_parts(rows, plan, src)
 
     def _accept_summed(self, index, g, key, may_miss):
         if may_miss:  # keys the table does not hold take no gradient
@@ -483,21 +509,25 @@ class HashtableImpl:
         self.accept_grad(index, g, unique=True, key=key)
 
     def _sum_planned(self):
-        if self._planned is not None:
-            index, plan, rows, src, coef, cover, key, may_miss = self._planned
-            self._planned = None
-            self._accept_summed(index, ops.csr_gather_reduce(rows, plan, src, coef, cover=cover), key, may_miss)
+        planned, self._planned = self._planned, []
+        for entry in planned:
+            self._accept_summed(entry[0], self._sum_of(entry), entry[6], entry[7])
 
     def take_planned_grad(self):
-        """The planned gradient if it is all this table received since the last ``clear_grad`` (and forgets
-        it), else None: ``(index, plan, rows, src, coef, cover)``."""
-        if self._planned is None or self._grad:
+        """The planned gradients if they are all this table received since the last ``clear_grad`` (and
+        forgets them), else None: a list of one or two ``(index, plan, rows, src, coef, cover)``; of two, the
+        first is one array (the other may be a list of arrays)."""
+        if not self._planned or self._grad:
             return None
-        planned, self._planned = self._planned, None
-        return planned[:6]
+        if len(self._planned) == 1 and not torch.is_tensor(self._planned[0][2]):
+            return None   # parts alone: no fused row update takes them
+        planned, self._planned = self._planned, []
+        if len(planned) == 2 and not torch.is_tensor(planned[0][2]):
+            planned.reverse()
+        return [e[:6] for e in planned]
 
     def has_grad(self):
-        return len(self._grad) > 0 or self._planned is not None
+        return len(self._grad) > 0 or len(self._planned) > 0
 
     def grad_pairs(self, accumulate_steps=1):
         """(row index, gradient rows) merged over the accepted gradients: what
@@ -540,7 +570,7 @@ class HashtableImpl:
 
     def clear_grad(self):
         self._grad_index, self._grad, self._grad_unique, self._grad_keys = [], [], [], {}
-        self._planned = None
+        self._planned = []
 
     # ------------------------------------------------------------ bookkeeping
     def clear(self):

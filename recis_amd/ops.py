@@ -999,30 +999,48 @@ def csr_gather_reduce_adagrad(rows, plan, src, coef, row_index, emb_blocks, accu
 class _CsrInput(ctypes.Structure):
     """``recis_csr_input`` of the C header."""
     _fields_ = [("rows", ctypes.c_void_p), ("rows_dtype", ctypes.c_int), ("n_rows", ctypes.c_int64),
-                ("src", ctypes.c_void_p), ("coef", ctypes.c_void_p), ("coef_dtype", ctypes.c_int)]
+                ("src", ctypes.c_void_p), ("coef", ctypes.c_void_p), ("coef_dtype", ctypes.c_int),
+                ("part_rows", ctypes.c_void_p), ("part_counts", ctypes.c_void_p), ("n_parts", ctypes.c_int)]
 
 
 def _csr_input(rows, src, coef):
-    """One input ``(rows, src, coef)`` of a two-input gather-reduce as the C struct, with the
-    tensors it points into (to be kept alive over the call)."""
-    require_cuda(rows, src, coef)
-    rows = _contig(rows)
-    if rows.dim() != 2:
-        raise ValueError("gradient rows must be [rows, D]")
-    c = _CsrInput(rows.data_ptr() if rows.numel() else None, dtype_code(rows.dtype), rows.shape[0],
-                  src.data_ptr() if src.numel() else None, coef.data_ptr() if coef is not None and coef.numel() else None,
-                  dtype_code(coef.dtype) if coef is not None else 0)
-    return c, (rows, src, coef)
+    """One input ``(rows, src, coef)`` of a two-input gather-reduce as the C struct, with what it
+    points into (to be kept alive over the call). ``rows``: a ``[rows, D]`` tensor, or a list of
+    up to 8 such tensors laid end to end in ``src``'s numbering (the second input only)."""
+    parts = None
+    if isinstance(rows, (list, tuple)):
+        parts = [_contig(p) for p in rows]
+        require_cuda(src, coef, *parts)
+        if any(p.dim() != 2 or p.dtype != parts[0].dtype or p.shape[1] != parts[0].shape[1] for p in parts):
+            raise TypeError("the parts of an input must be [rows, D] tensors of one dtype and row width")
+        rows = parts[0]
+        tables = (_host_ptrs(parts), _host_i64([p.shape[0] for p in parts]))
+    else:
+        require_cuda(rows, src, coef)
+        rows = _contig(rows)
+        if rows.dim() != 2:
+            raise ValueError("gradient rows must be [rows, D]")
+        tables = (None, None)
+    c = _CsrInput(rows.data_ptr() if parts is None and rows.numel() else None, dtype_code(rows.dtype),
+                  rows.shape[0] if parts is None else 0, src.data_ptr() if src.numel() else None,
+                  coef.data_ptr() if coef is not None and coef.numel() else None,
+                  dtype_code(coef.dtype) if coef is not None else 0,
+                  ctypes.cast(tables[0], ctypes.c_void_p) if parts is not None else None,
+                  ctypes.cast(tables[1], ctypes.c_void_p) if parts is not None else None,
+                  len(parts) if parts is not None else 0)
+    return c, (rows, src, coef, parts, tables)
 
 
 def _two_inputs(plan, first, second):
+    if isinstance(first[0], (list, tuple)):
+        if isinstance(second[0], (list, tuple)):
+            raise TypeError("only one input of a two-input gather-reduce may come in parts")
+        first, second = second, first   # the kernels take the parts as their second input
     a, keep_a = _csr_input(*first)
     b, keep_b = _csr_input(*second)
     D = keep_a[0].shape[1]
     if keep_b[0].shape[1] != D:
         raise ValueError("the two inputs have rows of %d and %d columns" % (D, keep_b[0].shape[1]))
-    if keep_a[0].dtype != torch.float32:
-        raise TypeError("the first input of a two-input gather-reduce must be float32")
     head = (ctypes.byref(a), ctypes.byref(b), ptr(plan.row_start), ptr(plan.hot_items), i64(plan.hot_cap),
             ptr(plan.counts))
     return head, D, keep_a[0].device, (a, b, keep_a, keep_b)
@@ -1031,7 +1049,8 @@ def _two_inputs(plan, first, second):
 def csr_gather_reduce2(plan, first, second, out=None, accumulate=False):
     """``csr_gather_reduce`` with two inputs ``(rows, src, coef)`` over the lists of ``plan``
     (``recis_csr_gather_reduce2``): ``out[u] (+)= sum_k coef1[k] * rows1[src1[k]] + coef2[k] *
-    rows2[src2[k]]``; the first input float32."""
+    rows2[src2[k]]``. Each input float32 or a half type (two half inputs of one type); one of them may
+    come as a list of arrays laid end to end in its ``src``'s numbering."""
     head, D, dev, keep = _two_inputs(plan, first, second)
     if out is None:
         out = torch.empty((plan.U, D), dtype=torch.float32, device=dev)

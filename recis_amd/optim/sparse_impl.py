@@ -50,8 +50,11 @@ class _SparseOptimizerImpl:
                     continue
                 planned = ht.take_planned_grad() if self._grad_accum_steps == 1 and hasattr(self, "apply_planned") else None
                 if planned is not None:   # the gradient is still a sum to be taken: sum and update in one launch
-                    index, plan, rows, src, coef, cover = planned
-                    self.apply_planned(ht, plan, rows, src, coef, index, cover)
+                    index, plan, rows, src, coef, cover = planned[0]
+                    if len(planned) == 1:
+                        self.apply_planned(ht, plan, rows, src, coef, index, cover)
+                    else:   # two gradients of one plan
+                        self.apply_planned2(ht, plan, (rows, src, coef), planned[1][2:5], index)
                     continue
                 index, grad = ht.grad_pairs(self._grad_accum_steps)
                 self._update(ht, self._state[id(ht)], index, grad)
@@ -111,7 +114,7 @@ class _AdamFamilyImpl(_SparseOptimizerImpl):
 
     def apply_planned2(self, ht, plan, first, second, index):
         """``apply_planned`` for a table whose lookup fed two outputs: ``first`` and ``second`` are
-        ``(grad_rows, src, coef)`` of the two gradients (the first float32), summed per unique id in
+        ``(grad_rows, src, coef)`` of the two gradients, summed per unique id in
         one pass (``ops.csr_gather_reduce2_adamw``)."""
         st = self._state[id(ht)]
         chunks, chunk_rows = ht._slot_group.emb_slot().kernel_blocks()

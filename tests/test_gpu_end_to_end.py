@@ -623,14 +623,65 @@ def test_gradient_summed_in_the_optimizer_step_equals_summed_first(opt_cls):
             torch.autograd.backward([out[k] for k in out], [up for _ in out])
             impls = [t._hashtable_impl for t in eng.hashtables().values()]
             if step % 2 == 0:
-                assert all(i._planned is not None and not i._grad for i in impls)        # waiting unsummed
+                assert all(len(i._planned) == 1 and not i._grad for i in impls)           # waiting unsummed
             if sum_first:
                 for i in impls:
                     i.grad_pairs(1)
-                    assert i._planned is None
+                    assert not i._planned
             opt.step()
             opt.zero_grad()
         for t1, t2 in zip(e1.hashtables().values(), e2.hashtables().values()):
             for s1, s2 in zip(t1.slot_group().slots(), t2.slot_group().slots()):
                 torch.testing.assert_close(s1.value(), s2.value(), rtol=1e-5, atol=1e-7, msg=lambda m: "%s step %d slot %s" % (m, step, s1.name()))
+    assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("opt_cls,dtype", [(SparseAdagrad, torch.float32), (SparseAdam, torch.float32),
+                                           (SparseAdagrad, torch.bfloat16)])
+def test_two_gradients_of_one_lookup_summed_in_the_optimizer_step(opt_cls, dtype):
+    """Sequence features used twice, mean-pooled and kept row by row: both backward passes hand their gradient
+    to the table unsummed (the padded one as one array per feature), and the optimizer step sums both and
+    updates the rows in one launch (apply_planned2). A second engine on the same data is made to sum first
+    (grad_pairs() before step()): rows and state agree after every step up to the order of the fp32 sums (each
+    engine makes its own plan; on one plan the two ways are pinned against each other bit for bit in
+    test_two_input_fused_update_equals_gather_reduce_then_update)."""
+    def make(tag):
+        HashtableRegister().clear()
+        init = NormalInitializer(0.0, 0.1, generator=torch.Generator(device="cuda").manual_seed(3))
+        opt = lambda combiner, **kw: EmbeddingOption(embedding_dim=32, shared_name="s" + tag, combiner=combiner, dtype=dtype,
+                                                     use_weight=False, initializer=init, **kw)
+        eng = EmbeddingEngine({"a_mean": opt("mean"), "b_mean": opt("mean"),
+                               "a_rows": opt("tile", combiner_kwargs={"tile_len": 6}),
+                               "b_rows": opt("tile", combiner_kwargs={"tile_len": 11})}).cuda()
+        eng.train()
+        return eng, opt_cls(filter_out_sparse_param(eng), lr=1e-2)
+    (e1, o1), (e2, o2) = make("1"), make("2")
+    rng = np.random.default_rng(5)
+    B = 256
+
+    def seq(max_len):
+        lens = rng.integers(0, max_len, B)
+        off = torch.from_numpy(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)).cuda()
+        return RaggedTensor(torch.from_numpy(rng.integers(0, 500, int(off[-1]))).cuda(), off)
+
+    for step in range(3):
+        a, b = seq(20), seq(9)
+        gen = torch.Generator(device="cuda").manual_seed(step)
+        ups = {"a_mean": torch.randn(B, 32, device="cuda", generator=gen), "b_mean": torch.randn(B, 32, device="cuda", generator=gen),
+               "a_rows": torch.randn(B, 6 * 32, device="cuda", generator=gen).to(dtype),
+               "b_rows": torch.randn(B, 11 * 32, device="cuda", generator=gen).to(dtype)}
+        for eng, opt, sum_first in ((e1, o1, False), (e2, o2, True)):
+            out = eng({"a_mean": a, "b_mean": b, "a_rows": a, "b_rows": b})
+            torch.autograd.backward([out[k] for k in ups], [ups[k].to(out[k].dtype) for k in ups])
+            impl = next(iter(eng.hashtables().values()))._hashtable_impl
+            assert len(impl._planned) == 2 and not impl._grad                       # both waiting unsummed
+            if sum_first:
+                impl.grad_pairs(1)
+                assert not impl._planned
+            opt.step()
+            opt.zero_grad()
+        t1, t2 = next(iter(e1.hashtables().values())), next(iter(e2.hashtables().values()))
+        for s1, s2 in zip(t1.slot_group().slots(), t2.slot_group().slots()):
+            tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=1e-6)
+            torch.testing.assert_close(s1.value().float(), s2.value().float(), msg=lambda m: "%s step %d slot %s" % (m, step, s1.name()), **tol)
     assert _lib.poll_device_errors() == 0

@@ -421,16 +421,19 @@ def _two_gradient_case(rng, D, tile_dtype, n_hot=3):
     return plan, batch, seq, off, (_dev(g_pool), src_p, coef_p), (g_tile, src_t, None)
 
 
-@pytest.mark.parametrize("D,tile_dtype", [(16, torch.float32), (128, torch.bfloat16), (40, torch.float16), (64, torch.float32)])
-def test_two_input_gather_reduce_matches_oracle(rng, D, tile_dtype):
+@pytest.mark.parametrize("D,tile_dtype,pool_dtype", [(16, torch.float32, torch.float32), (128, torch.bfloat16, torch.float32),
+                                                     (40, torch.float16, torch.float32), (64, torch.float32, torch.float32),
+                                                     (128, torch.bfloat16, torch.bfloat16), (32, torch.float32, torch.float16)])
+def test_two_input_gather_reduce_matches_oracle(rng, D, tile_dtype, pool_dtype):
     """recis_csr_gather_reduce2 against the oracle's two backward passes added up (the backward of
     mean pooling and of the padded gather into the same unique rows), and against the two
     single-input calls it replaces."""
     plan, batch, seq, off, first, second = _two_gradient_case(rng, D, tile_dtype)
+    first = (first[0].to(pool_dtype),) + first[1:]
     inv = plan.inverse.cpu().numpy().astype(np.int64)
     got = ops.csr_gather_reduce2(plan, first, second)
     g_tile32 = second[0].float().cpu().numpy()
-    exp = (oracle.segment_reduce_backward(first[0].cpu().numpy(), None, inv, off, plan.U, "mean").astype(np.float64)
+    exp = (oracle.segment_reduce_backward(first[0].float().cpu().numpy(), None, inv, off, plan.U, "mean").astype(np.float64)
            + oracle.ragged_tile_back(batch, seq, inv, off, g_tile32, plan.U))
     # fp32 sums of up to thousands of terms in another order: atol scales with the summed magnitude
     mag = np.zeros(plan.U)
@@ -446,13 +449,16 @@ def test_two_input_gather_reduce_matches_oracle(rng, D, tile_dtype):
 
 
 @pytest.mark.parametrize("kind", ["adamw", "adagrad"])
-@pytest.mark.parametrize("D,row_dtype,tile_dtype", [(16, torch.float32, torch.float32), (128, torch.bfloat16, torch.bfloat16),
-                                                    (128, torch.bfloat16, torch.float32), (24, torch.float16, torch.float16)])
-def test_two_input_fused_update_equals_gather_reduce_then_update(rng, kind, D, row_dtype, tile_dtype):
+@pytest.mark.parametrize("D,row_dtype,tile_dtype,pool_dtype", [
+    (16, torch.float32, torch.float32, torch.float32), (128, torch.bfloat16, torch.bfloat16, torch.float32),
+    (128, torch.bfloat16, torch.float32, torch.float32), (24, torch.float16, torch.float16, torch.float32),
+    (128, torch.bfloat16, torch.bfloat16, torch.bfloat16), (32, torch.float16, torch.float32, torch.float16)])
+def test_two_input_fused_update_equals_gather_reduce_then_update(rng, kind, D, row_dtype, tile_dtype, pool_dtype):
     """recis_csr_gather_reduce2_adamw / _adagrad against recis_csr_gather_reduce2 into an fp32 buffer
     followed by the row update (bit-exact against the oracle in test_gpu_table.py): the same rows
     and state bit for bit, negative row indices skipped, two steps."""
     plan, batch, seq, off, first, second = _two_gradient_case(rng, D, tile_dtype)
+    first = (first[0].to(pool_dtype),) + first[1:]
     U, bs, nb = plan.U, 1024, 4
     row_index = torch.from_numpy(rng.permutation(bs * nb)[:U]).cuda()
     row_index[::13] = -1
@@ -479,8 +485,33 @@ def test_two_input_fused_update_equals_gather_reduce_then_update(rng, kind, D, r
 
 def test_two_input_gather_reduce_refuses_what_it_does_not_support(rng):
     plan, batch, seq, off, first, second = _two_gradient_case(rng, 16, torch.float32)
-    half = (first[0].to(torch.bfloat16), first[1], first[2])
-    with pytest.raises(TypeError):
-        ops.csr_gather_reduce2(plan, half, second)                   # the first input must be float32
+    with pytest.raises(RuntimeError):                                # two half-precision inputs of different types
+        ops.csr_gather_reduce2(plan, (first[0].to(torch.bfloat16), first[1], first[2]),
+                               (second[0].to(torch.float16), second[1], None))
     with pytest.raises(ValueError):
         ops.csr_gather_reduce2(plan, first, (second[0][:, :8].contiguous(), second[1], None))
+
+
+def test_two_input_gather_reduce_second_input_in_parts(rng):
+    """The second input as separate arrays (one per feature of the padded gather) equals the same
+    rows concatenated, bit for bit; with the fused Adagrad update too."""
+    plan, batch, seq, off, first, second = _two_gradient_case(rng, 64, torch.bfloat16)
+    n_rows = [b * s for b, s in zip(batch, seq)]
+    parts = [p.clone() for p in torch.split(second[0], n_rows)]
+    whole = ops.csr_gather_reduce2(plan, first, second)
+    split = ops.csr_gather_reduce2(plan, first, (parts, second[1], None))
+    assert torch.equal(whole, split)
+    U, bs, nb = plan.U, 1024, 4
+    row_index = torch.from_numpy(rng.permutation(bs * nb)[:U]).cuda()
+    mk = lambda: [_dev(rng.random((bs, 64)).astype(np.float32)).to(torch.bfloat16) for _ in range(nb)]
+    emb, acc = mk(), mk()
+    emb2, acc2 = [b.clone() for b in emb], [b.clone() for b in acc]
+    ops.csr_gather_reduce2_adagrad(plan, first, second, row_index, emb, acc, 1e-2, 1e-8, bs)
+    ops.csr_gather_reduce2_adagrad(plan, first, (parts, second[1], None), row_index, emb2, acc2, 1e-2, 1e-8, bs)
+    for x, y in zip(emb + acc, emb2 + acc2):
+        assert torch.equal(x, y)
+    swapped = ops.csr_gather_reduce2(plan, (parts, second[1], None), first)     # the parts are made the second input
+    assert torch.equal(swapped, whole)
+    with pytest.raises(TypeError):
+        ops.csr_gather_reduce2(plan, ([first[0]], first[1], first[2]), (parts, second[1], None))   # not both in parts
+    assert _lib.poll_device_errors() == 0
