@@ -351,6 +351,73 @@ __device__ __forceinline__ void scan_counts(const int32_t* in, int nb, int32_t* 
   __syncthreads();
 }
 
+// Where every column's entries start in the partitioned arrays (start[0 .. nc), start[nc] = n), by
+// the calling workgroup of kPartBlock threads, from the column totals. The columns are NOT laid
+// out in the order of their index: the heavy ids' columns come first (as always), then the buckets
+// that hold more than one and a half times the average, then the others, each class in the order of
+// the index. The bucket kernel takes the buckets in the order of this layout, one workgroup each,
+// and the layout is the order of the unique ids; so the buckets that take longest (a bucket with
+// three times the entries keeps its workgroup almost twice as long) are dispatched first and the
+// short ones fill in behind them, instead of a long one starting last and the whole chip waiting
+// for it. Still a function of the input alone. rank_start (global, may be NULL): written with the
+// same starts indexed by the column's place in the layout ([nc + 1]), what the bucket kernel reads.
+// `partial` is scratch of kPartBlock words. Ends with a barrier.
+__device__ __forceinline__ void column_starts(const int32_t* __restrict__ total, int nc, int64_t n, int32_t* start,
+                                              int32_t* partial, int32_t* __restrict__ rank_start) {
+  unsigned long long* part64 =  // [2][waves], at the first 8-byte boundary of the scratch
+      reinterpret_cast<unsigned long long*>((reinterpret_cast<uintptr_t>(partial) + 7) & ~static_cast<uintptr_t>(7));
+  const int t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
+  constexpr int n_waves = kPartBlock / kWave;
+  const int per = (nc + kPartBlock - 1) / kPartBlock;
+  const int lo = min(nc, t * per), hi = min(nc, lo + per);
+  const int64_t fat_from = 3 * (n / (nc - kHeavyMax)) / 2 + 32;  // entries from which a bucket goes first
+  auto is_first = [&](int c, int32_t cnt) { return c < kHeavyMax || cnt > fat_from; };
+  // per class one word: entries << 14 | columns (n < 2^31 entries, fewer than 2^14 columns)
+  unsigned long long sum[2] = {0, 0};
+  for (int c = lo; c < hi; ++c) {
+    const int32_t cnt = total[c];
+    sum[is_first(c, cnt) ? 0 : 1] += (static_cast<unsigned long long>(cnt) << 14) | 1ull;
+  }
+  unsigned long long incl[2] = {sum[0], sum[1]};
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const unsigned long long y = __shfl_up(incl[k], o, kWave);
+      if (lane >= o) incl[k] += y;
+    }
+  }
+  if (lane == kWave - 1) {
+    part64[wave] = incl[0];
+    part64[n_waves + wave] = incl[1];
+  }
+  __syncthreads();
+  unsigned long long run[2] = {incl[0] - sum[0], incl[1] - sum[1]}, all_first = 0;
+#pragma unroll
+  for (int w = 0; w < n_waves; ++w) {
+    const unsigned long long c0 = part64[w], c1 = part64[n_waves + w];
+    if (w < wave) {
+      run[0] += c0;
+      run[1] += c1;
+    }
+    all_first += c0;
+  }
+  run[1] += all_first;  // the second class lies behind all of the first
+  for (int c = lo; c < hi; ++c) {
+    const int32_t cnt = total[c];
+    const int k = is_first(c, cnt) ? 0 : 1;
+    const int32_t at = static_cast<int32_t>(run[k] >> 14);
+    start[c] = at;
+    if (rank_start) rank_start[run[k] & 0x3fff] = at;
+    run[k] += (static_cast<unsigned long long>(cnt) << 14) | 1ull;
+  }
+  if (t == 0) {
+    start[nc] = static_cast<int32_t>(n);
+    if (rank_start) rank_start[nc] = static_cast<int32_t>(n);
+  }
+  __syncthreads();
+}
+
 // What the partition kernels need to put the occurrences of heavy ids straight into their lists.
 struct HeavyArgs {
   const int64_t* ids;   // [kHeavyMax]
@@ -377,9 +444,8 @@ plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs hv, c
   const int tid = threadIdx.x;
   const int nb = 1 << g.nb_log2, nc = kHeavyMax + nb;
   const int n_heavy = load_heavy(hv.ids, hv.n, h_slot, h_key);
-  scan_counts(bucket_total, nc, cursor, cursor + nc + 1);
+  column_starts(bucket_total, nc, g.n, cursor, cursor + nc + 1, blockIdx.x == 0 ? bucket_start : nullptr);
   if (blockIdx.x == 0) {
-    for (int b = tid; b <= nc; b += kPartBlock) bucket_start[b] = cursor[b];
     for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
   }
   const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nc;
@@ -439,9 +505,8 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs 
   uint16_t* sorted_bucket = sorted + kTile;                              // [kTile] and their columns
   for (int b = tid; b <= nc; b += kPartBlock) first[b] = 0;
   const int n_heavy = load_heavy(hv.ids, hv.n, h_slot, h_key);
-  scan_counts(bucket_total, nc, gbase, partial);
+  column_starts(bucket_total, nc, g.n, gbase, partial, blockIdx.x == 0 ? bucket_start : nullptr);
   if (blockIdx.x == 0) {
-    for (int b = tid; b <= nc; b += kPartBlock) bucket_start[b] = gbase[b];
     for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
   }
   const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nc;

@@ -201,6 +201,21 @@ seg_pool_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, SegArgs
 // Rows are summed per row group in increasing order, like the generic kernel. Requires U < 2^31.
 enum { kFastPlain = 0, kFastRev32 = 1, kFastRev64 = 2 };
 
+// A row of zeros, as long as any row these kernels take (D <= 8192 of at most 4 bytes). The fast
+// kernels keep several row loads in flight per lane; a lane with no row to read in some round reads
+// this one instead, so that the loads of a round stay one straight run of instructions (a branch
+// around each makes the compiler wait for every outstanding load before it issues the next).
+__device__ __align__(256) const unsigned char g_zero_row[8192 * 4] = {};
+
+template <typename T, int VEC, bool NT>
+__device__ __forceinline__ void load_row_pack(const T* p, float (&v)[VEC]) {
+  if constexpr (NT) {
+    load_pack_stream<T, VEC>(p, v);
+  } else {
+    load_pack<T, VEC>(p, v);
+  }
+}
+
 // WG: long segments (behaviour sequences of hundreds of rows): a whole workgroup per segment, each
 // of its waves sums a contiguous quarter of the rows and the quarters meet in LDS. With a wave per
 // segment the launch lasts as long as its longest segment takes one wave.
@@ -236,68 +251,71 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
   const int D = a.D;
   const float scale = (a.mean && seg_len > 0) ? 1.0f / static_cast<float>(seg_len) : 1.0f;
 
+  const TIn* zero_row = reinterpret_cast<const TIn*>(g_zero_row);
+  // rows read once, or too many to stay cached: streaming loads (picked here, outside the loops)
+  const bool nt = (KIND == kFastPlain && !BLK) || a.nt_in;
   for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
     const int c0 = cbase + cl * VEC;
     const bool col_ok = c0 < D;
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    for (int64_t base = start; base < end; base += team) {
-      const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
-      int32_t mine = -1;       // row of occurrence base + lane_t in emb ...
-      uint64_t mine_addr = 0;  // ... or its address in the block list (BLK), 0 = zero row
-      if (lane_t < n_here) {
-        int64_t idx;
-        if constexpr (KIND == kFastPlain) {
-          idx = base + lane_t;
-        } else if constexpr (KIND == kFastRev32) {
-          idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
-        } else {
-          idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
-        }
-        if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
-          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-        } else if constexpr (BLK) {
-          mine_addr = reinterpret_cast<uint64_t>(block_row<TIn>(a, idx));
-        } else {
-          mine = static_cast<int32_t>(idx);
-        }
-      }
-      constexpr int kFly = VEC >= 8 ? 4 : 8;  // row loads in flight per lane
-      for (int q0 = 0; q0 < n_here; q0 += kFly * step) {  // same trip count for the whole team (shuffles inside)
-        const int q = q0 + rg;
-        float v[kFly][VEC];
-#pragma unroll
-        for (int k = 0; k < kFly; ++k) {
-          const int src = q + k * step;
-          const int from = team_lane0 + min(src, team - 1);
-          const TIn* row = nullptr;
-          if constexpr (BLK) {
-            const uint32_t lo = __shfl(static_cast<uint32_t>(mine_addr), from, kWave);
-            const uint32_t hi = __shfl(static_cast<uint32_t>(mine_addr >> 32), from, kWave);
-            row = reinterpret_cast<const TIn*>((static_cast<uint64_t>(hi) << 32) | lo);
+    auto sum_rows = [&](auto nt_tag) {
+      constexpr bool NT = decltype(nt_tag)::value;
+      for (int64_t base = start; base < end; base += team) {
+        const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
+        int32_t mine = -1;       // row of occurrence base + lane_t in emb ...
+        uint64_t mine_addr = 0;  // ... or its address in the block list (BLK), 0 = zero row
+        if (lane_t < n_here) {
+          int64_t idx;
+          if constexpr (KIND == kFastPlain) {
+            idx = base + lane_t;
+          } else if constexpr (KIND == kFastRev32) {
+            idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
           } else {
-            const int32_t id = __shfl(mine, from, kWave);
-            if (id >= 0) row = emb + static_cast<int64_t>(id) * D;
+            idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
           }
-          if (src >= n_here || !col_ok) row = nullptr;
-          if (row) {
-            if ((KIND == kFastPlain && !BLK) || a.nt_in) {
-              load_pack_stream<TIn, VEC>(row + c0, v[k]);  // read once, or too large to stay cached
+          if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+            raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+          } else if constexpr (BLK) {
+            mine_addr = reinterpret_cast<uint64_t>(block_row<TIn>(a, idx));
+          } else {
+            mine = static_cast<int32_t>(idx);
+          }
+        }
+        constexpr int kFly = VEC >= 8 ? 4 : 8;  // row loads in flight per lane
+        for (int q0 = 0; q0 < n_here; q0 += kFly * step) {  // same trip count for the whole team (shuffles inside)
+          const int q = q0 + rg;
+          float v[kFly][VEC];
+#pragma unroll
+          for (int k = 0; k < kFly; ++k) {  // no branches in here: see g_zero_row
+            const int src = q + k * step;
+            const int from = (team_lane0 + src) & (kWave - 1);  // past the team: some other lane's row, not used
+            const bool want = src < n_here && col_ok;
+            const TIn* row;
+            if constexpr (BLK) {
+              const uint32_t lo = __shfl(static_cast<uint32_t>(mine_addr), from, kWave);
+              const uint32_t hi = __shfl(static_cast<uint32_t>(mine_addr >> 32), from, kWave);
+              const uint64_t addr = (static_cast<uint64_t>(hi) << 32) | lo;
+              row = (want && addr != 0) ? reinterpret_cast<const TIn*>(addr) + c0 : zero_row;
             } else {
-              load_pack<TIn, VEC>(row + c0, v[k]);
+              const int32_t id = __shfl(mine, from, kWave);
+              row = (want && id >= 0) ? emb + static_cast<int64_t>(id) * D + c0 : zero_row;
             }
-          } else {
+            load_row_pack<TIn, VEC, NT>(row, v[k]);
+          }
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) v[k][j] = 0.f;
+          for (int k = 0; k < kFly; ++k) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] += v[k][j];
           }
         }
-#pragma unroll
-        for (int k = 0; k < kFly; ++k) {
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) acc[j] += v[k][j];
-        }
       }
+    };
+    if (nt) {
+      sum_rows(std::true_type{});
+    } else {
+      sum_rows(std::false_type{});
     }
     for (int off = 1 << a.lpr_log2; off < team; off <<= 1) {
 #pragma unroll
@@ -424,6 +442,7 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
   const int step = team >> a.lpr_log2;
   const int col_stride = VEC << a.lpr_log2;
   const int D = a.D;
+  const TIn* zero_row = reinterpret_cast<const TIn*>(g_zero_row);
 
   for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
     const int c0 = cbase + cl * VEC;
@@ -431,64 +450,70 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
     // Inside a lane the occurrences come in ascending order, so a strict float comparison keeps
     // the first of equal values (-0 == +0) and costs less than building a key per element. The
     // running best starts as NaN so that the first row always wins; the first NaN of the data
-    // wins over every number and is kept from then on.
+    // wins over every number and is kept from then on. (Scanning without the NaN flags first and
+    // again with them only when a segment holds a NaN halves the arithmetic and was measured: no
+    // faster. The kernel waits on memory, not on the vector units.)
     float best_v[VEC];
     int32_t best_r[VEC];
-    bool nan_seen[VEC];
+    auto scan_rows = [&](auto nt_tag) {
+      constexpr bool NT = decltype(nt_tag)::value;
+      bool nan_seen[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      best_v[j] = __uint_as_float(0x7FC00000u);
-      best_r[j] = -1;
-      nan_seen[j] = false;
-    }
-    for (int64_t base = start; base < end; base += team) {
-      const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
-      int32_t mine = -1;  // row of occurrence base + lane_t
-      if (lane_t < n_here) {
-        int64_t idx;
-        if constexpr (KIND == kFastPlain) {
-          idx = base + lane_t;
-        } else if constexpr (KIND == kFastRev32) {
-          idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
-        } else {
-          idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
-        }
-        if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
-          raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-        } else {
-          mine = static_cast<int32_t>(idx);
-        }
+      for (int j = 0; j < VEC; ++j) {
+        best_v[j] = __uint_as_float(0x7FC00000u);
+        best_r[j] = -1;
+        nan_seen[j] = false;
       }
-      for (int q0 = 0; q0 < n_here; q0 += 4 * step) {  // same trip count for the whole team
-        float v[4][VEC];
-        bool have[4];
+      for (int64_t base = start; base < end; base += team) {
+        const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
+        int32_t mine = -1;  // row of occurrence base + lane_t
+        if (lane_t < n_here) {
+          int64_t idx;
+          if constexpr (KIND == kFastPlain) {
+            idx = base + lane_t;
+          } else if constexpr (KIND == kFastRev32) {
+            idx = static_cast<const int32_t*>(a.rev)[base + lane_t];
+          } else {
+            idx = static_cast<const int64_t*>(a.rev)[base + lane_t];
+          }
+          if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(a.U)) {
+            raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+          } else {
+            mine = static_cast<int32_t>(idx);
+          }
+        }
+        constexpr int kFly = 4;  // row loads in flight per lane (8 was measured: slower, fewer resident waves)
+        for (int q0 = 0; q0 < n_here; q0 += kFly * step) {  // same trip count for the whole team
+          float v[kFly][VEC];
+          bool have[kFly];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int src = q0 + rg + k * step;
-          const int32_t id = __shfl(mine, team_lane0 + min(src, team - 1), kWave);
-          have[k] = src < n_here && col_ok && id >= 0;
-          if (have[k]) {
-            if (KIND == kFastPlain || a.nt_in) {
-              load_pack_stream<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
-            } else {
-              load_pack<TIn, VEC>(emb + static_cast<int64_t>(id) * D + c0, v[k]);
+          for (int k = 0; k < kFly; ++k) {  // no branches in here: see g_zero_row
+            const int src = q0 + rg + k * step;
+            const int32_t id = __shfl(mine, (team_lane0 + src) & (kWave - 1), kWave);
+            have[k] = src < n_here && col_ok && id >= 0;
+            const TIn* row = have[k] ? emb + static_cast<int64_t>(id) * D + c0 : zero_row;
+            load_row_pack<TIn, VEC, NT>(row, v[k]);
+          }
+#pragma unroll
+          for (int k = 0; k < kFly; ++k) {
+            const int32_t r = static_cast<int32_t>(base) + q0 + rg + k * step;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              const float x = v[k][j];
+              // & and |, not && and ||: no branches (the values are all at hand)
+              const bool take = have[k] & !(x <= best_v[j]) & !nan_seen[j];
+              nan_seen[j] = nan_seen[j] | (have[k] & (x != x));
+              best_v[j] = take ? x : best_v[j];
+              best_r[j] = take ? r : best_r[j];
             }
           }
         }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          if (!have[k]) continue;
-          const int32_t r = static_cast<int32_t>(base) + q0 + rg + k * step;
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const float x = v[k][j];
-            const bool take = !(x <= best_v[j]) && !nan_seen[j];
-            nan_seen[j] = nan_seen[j] || (x != x);
-            best_v[j] = take ? x : best_v[j];
-            best_r[j] = take ? r : best_r[j];
-          }
-        }
       }
+    };
+    if (KIND == kFastPlain || a.nt_in) {
+      scan_rows(std::true_type{});
+    } else {
+      scan_rows(std::false_type{});
     }
     uint64_t key[VEC];
 #pragma unroll
