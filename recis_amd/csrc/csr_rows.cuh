@@ -77,13 +77,39 @@ struct FuseArgs {
   RowBlocks rb;
   AdamCoef adam;
   float lr, eps;             // Adagrad
+  // Adam without a cal_alpha launch in front (adam.alpha == NULL in the row kernel): every thread
+  // works alpha out from the running powers as they stand (nobody writes them while the row
+  // kernel runs) and leaves it in alpha_ws; the finish kernel, which runs afterwards, reads alpha
+  // from there (its adam.alpha) and its first thread advances the powers (advance_powers).
+  void* beta1_t;
+  void* beta2_t;
+  int beta_is_f64;
+  int advance_powers;
+  double adam_lr;
+  double* alpha_ws;
 };
 
+// alpha of this step from the running powers before the step; the advanced powers in b1 / b2 (as doubles).
+__device__ __forceinline__ double alpha_from_powers(const FuseArgs& f, double& b1, double& b2) {
+  if (f.beta_is_f64) {
+    return cal_alpha_step<double>(static_cast<const double*>(f.beta1_t)[0], static_cast<const double*>(f.beta2_t)[0],
+                                  f.adam_lr, f.adam.beta1, f.adam.beta2, b1, b2);
+  }
+  float n1, n2;
+  const double alpha = cal_alpha_step<float>(static_cast<const float*>(f.beta1_t)[0],
+                                             static_cast<const float*>(f.beta2_t)[0], f.adam_lr, f.adam.beta1,
+                                             f.adam.beta2, n1, n2);
+  b1 = n1;
+  b2 = n2;
+  return alpha;
+}
+
 // The epilogue of one pack of one finished row; T = the table's row type for the optimizer kinds.
-// idx = row_index[u] of the finished row (callers load it early: it heads a chain of dependent accesses).
+// idx = row_index[u] of the finished row (callers load it early: it heads a chain of dependent
+// accesses); alpha: of this step (Adam only).
 template <typename T, int VEC, int EPI>
 __device__ __forceinline__ void fused_row_update(const FuseArgs& f, int* err, int64_t idx, int c0,
-                                                 const float (&acc)[VEC]) {
+                                                 const float (&acc)[VEC], double alpha) {
   int64_t b, off;
   if (idx < 0) return;  // a key the table does not hold takes no gradient
   if (!block_row(f.rb, idx, b, off)) {
@@ -93,7 +119,7 @@ __device__ __forceinline__ void fused_row_update(const FuseArgs& f, int* err, in
   const int64_t at = off * f.rb.D + c0;
   if constexpr (EPI == kEpiAdam) {
     adam_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at,
-                             static_cast<T*>(f.s1[b]) + at, acc, f.adam.alpha[0], f.adam);
+                             static_cast<T*>(f.s1[b]) + at, acc, alpha, f.adam);
   } else {
     adagrad_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at, acc, f.lr, f.eps);
   }
@@ -235,6 +261,15 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   const int lane = threadIdx.x & (kWave - 1);
   const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
   const int g = lane >> a.lpr_log2;        // this lane's group in its wave
+  __shared__ double s_alpha;  // Adam: alpha of this step, worked out once per workgroup
+  if constexpr (EPI == kEpiAdam) {
+    if (threadIdx.x == 0) {
+      double b1, b2;
+      s_alpha = f.adam.alpha != nullptr ? f.adam.alpha[0] : alpha_from_powers(f, b1, b2);
+      if (f.adam.alpha == nullptr && blockIdx.x == 0) f.alpha_ws[0] = s_alpha;  // for the finish kernel
+    }
+    __syncthreads();
+  }
   SrcView<TIn> in1{rows, a.src, a.coef, a.coef_dt, a.nt_in, a.n_rows, 0, 0};
   cover_range(a, in1.lo, in1.hi);
   const SrcView<TSecond> in2{static_cast<const TSecond*>(a.rows2), a.src2, a.coef2, a.coef2_dt, a.nt_in2,
@@ -356,7 +391,7 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   // the finished sum of this lane group's own row u
   auto finish = [&](int64_t row, int c0, float (&acc)[VEC]) {
     if constexpr (EPI != kEpiStore) {
-      fused_row_update<TOut, VEC, EPI>(f, a.err, idx_mine, c0, acc);
+      fused_row_update<TOut, VEC, EPI>(f, a.err, idx_mine, c0, acc, EPI == kEpiAdam ? s_alpha : 0.0);
     } else {
       TOut* dst = out + row * D + c0;
       if (a.accumulate) {
@@ -416,6 +451,21 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
 template <typename TOut, int VEC, int EPI = kEpiStore>
 __global__ void __launch_bounds__(kBlock)
 csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
+  double alpha = 0;
+  if constexpr (EPI == kEpiAdam) {
+    alpha = f.adam.alpha[0];
+    if (f.advance_powers && blockIdx.x == 0 && threadIdx.x == 0) {  // nobody reads them in this kernel
+      double b1, b2;
+      alpha_from_powers(f, b1, b2);
+      if (f.beta_is_f64) {
+        static_cast<double*>(f.beta1_t)[0] = b1;
+        static_cast<double*>(f.beta2_t)[0] = b2;
+      } else {
+        static_cast<float*>(f.beta1_t)[0] = static_cast<float>(b1);
+        static_cast<float*>(f.beta2_t)[0] = static_cast<float>(b2);
+      }
+    }
+  }
   int64_t n_items = a.counts[1];
   if (n_items > a.hot_cap) n_items = a.hot_cap;
   const int D = a.D;
@@ -450,7 +500,7 @@ csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
       }
       if (g != 0 || !col_ok) continue;
       if constexpr (EPI != kEpiStore) {
-        fused_row_update<TOut, VEC, EPI>(f, a.err, f.row_index[u], c0, acc);
+        fused_row_update<TOut, VEC, EPI>(f, a.err, f.row_index[u], c0, acc, alpha);
       } else {
         TOut* dst = out + static_cast<int64_t>(u) * D + c0;
         if (a.accumulate) {
@@ -668,7 +718,12 @@ int csr_gather_reduce_run(const CsrRequest& r) {
             RECIS_LAUNCH_CHECK();
           }
           if (hot_cap > 0) {
-            csr_hot_finish_kernel<TOut, VEC, EPI><<<dim3(fin), block, 0, stream>>>(o, a, f);
+            FuseArgs f_fin = f;
+            if (EPI == kEpiAdam && f.adam.alpha == nullptr) {  // the row kernel worked alpha out itself
+              f_fin.adam.alpha = f.alpha_ws;
+              f_fin.advance_powers = 1;
+            }
+            csr_hot_finish_kernel<TOut, VEC, EPI><<<dim3(fin), block, 0, stream>>>(o, a, f_fin);
             RECIS_LAUNCH_CHECK();
           }
           return RECIS_OK;
@@ -755,10 +810,12 @@ inline int fill_fuse_args(FuseArgs& f, const int64_t* row_index, void* const* em
 }
 
 
-// The Adam-family variant of a request (r.epi == kEpiAdam, r.fuse == &f). The running powers of
-// the betas advance first, even when no row is touched (cal_alpha); alpha lives in the stream's
+// The Adam-family variant of a request (r.epi == kEpiAdam, r.fuse == &f). alpha lives in the stream's
 // workspace behind the partial rows of the hot items, so a first pass with U = 0 reserves the
-// workspace and learns where alpha goes, launching nothing.
+// workspace and learns where alpha goes, launching nothing. With hot work items (every batch plan
+// brings them) the kernels work alpha out and advance the running powers themselves (see
+// FuseArgs); otherwise, and when no row is touched (the powers advance all the same), cal_alpha
+// runs in front as in recis_block_apply_adamw.
 template <bool TWO, int ONLY_EPI = -1>
 int run_with_alpha(CsrRequest& r, FuseArgs& f, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
                    double beta1, double beta2, double weight_decay, double eps) {
@@ -768,14 +825,23 @@ int run_with_alpha(CsrRequest& r, FuseArgs& f, void* beta1_t, void* beta2_t, int
   probe.extra_ws = 256;
   probe.extra_out = &alpha;
   if (int rc = csr_gather_reduce_run<TWO, ONLY_EPI>(probe)) return rc;
-  if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, static_cast<double*>(alpha), lr, beta1, beta2, r.stream))
-    return rc;
-  if (r.U == 0) return RECIS_OK;
-  f.adam.alpha = static_cast<const double*>(alpha);
+  const bool in_kernel = r.U > 0 && r.hot_cap > 0;
+  if (!in_kernel) {
+    if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, static_cast<double*>(alpha), lr, beta1, beta2, r.stream))
+      return rc;
+    if (r.U == 0) return RECIS_OK;
+  }
+  f.adam.alpha = in_kernel ? nullptr : static_cast<const double*>(alpha);
   f.adam.beta1 = beta1;
   f.adam.beta2 = beta2;
   f.adam.decay = weight_decay;
   f.adam.eps = eps;
+  f.beta1_t = beta1_t;
+  f.beta2_t = beta2_t;
+  f.beta_is_f64 = beta_is_f64;
+  f.advance_powers = 0;
+  f.adam_lr = lr;
+  f.alpha_ws = static_cast<double*>(alpha);
   r.extra_ws = 256;
   r.extra_out = &alpha;
   return csr_gather_reduce_run<TWO, ONLY_EPI>(r);

@@ -42,12 +42,10 @@ __device__ __forceinline__ bool row_offset(const OptArgs& a, int64_t idx, int64_
 template <typename beta_t>
 __global__ void cal_alpha_kernel(beta_t* beta1_t, beta_t* beta2_t, double* alpha_out, double lr,
                                  double beta1, double beta2) {
-  beta1_t[0] = static_cast<beta_t>(beta1_t[0] * beta1);
-  beta2_t[0] = static_cast<beta_t>(beta2_t[0] * beta2);
-  const beta_t bc1 = 1 - beta1_t[0];
-  const beta_t bc2 = 1 - beta2_t[0];
-  const beta_t alpha = static_cast<beta_t>(-lr / bc1 * sqrtf(static_cast<float>(bc2)));
-  alpha_out[0] = static_cast<double>(alpha);
+  beta_t b1, b2;
+  alpha_out[0] = cal_alpha_step<beta_t>(beta1_t[0], beta2_t[0], lr, beta1, beta2, b1, b2);
+  beta1_t[0] = b1;
+  beta2_t[0] = b2;
 }
 
 template <typename T, typename TG, int VEC>

@@ -46,6 +46,20 @@ struct AdamCoef {
   double beta1, beta2, decay, eps;
 };
 
+// cal_alpha (block_apply_adamw_op.cc:77-85) on values: the running powers advance in their own
+// precision and alpha comes out of the advanced powers. One definition for the one-thread kernel
+// and for the kernels that work alpha out themselves, so both give the same bits.
+template <typename beta_t>
+__device__ __forceinline__ double cal_alpha_step(beta_t b1_old, beta_t b2_old, double lr, double beta1, double beta2,
+                                                 beta_t& b1_new, beta_t& b2_new) {
+  b1_new = static_cast<beta_t>(b1_old * beta1);
+  b2_new = static_cast<beta_t>(b2_old * beta2);
+  const beta_t bc1 = 1 - b1_new;
+  const beta_t bc2 = 1 - b2_new;
+  const beta_t alpha = static_cast<beta_t>(-lr / bc1 * sqrtf(static_cast<float>(bc2)));
+  return static_cast<double>(alpha);
+}
+
 // One pack of VEC elements of one row, in registers: g = gradient (fp32); w / m / v updated in place.
 template <typename T, int VEC>
 __device__ __forceinline__ void adam_compute_pack(Pack<T, VEC>& w, Pack<T, VEC>& m, Pack<T, VEC>& v,

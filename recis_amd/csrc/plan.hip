@@ -52,7 +52,7 @@ constexpr int kBucketBlock = 512;
 constexpr int kPer = 9;             // consecutive table entries owned by a thread (9 * 512 > kTabAll)
 constexpr int kRegs = 8;            // bucket records of a thread whose table entry stays in registers
 constexpr int64_t kSetEmpty = -1;
-constexpr int kHeavyMax = 64;       // ids that get a column of their own in the partition (see plan_heavy_kernel)
+constexpr int kHeavyMax = 64;       // ids that get a column of their own in the partition (see find_heavy)
 constexpr int kHeavySamples = 2048; // ids sampled to find them
 constexpr int kHeavyTab = 4096;     // LDS table of the sampling kernel
 constexpr int kHeavySlots = 256;    // LDS table every partition workgroup looks ids up in
@@ -83,48 +83,52 @@ __device__ __forceinline__ int home_of_mix(uint64_t mixed, int nb_log2) {
 // one workgroup with a hundred times the work of the others. Such ids are found beforehand by
 // sampling and get a column of their own in the partition: their occurrences go straight into
 // their list (no dedup needed: the column holds one id), and they become the first unique ids.
-//   heavy_ids [kHeavyMax], heavy_n [1]: the ids, ordered by (sample count descending, id ascending):
-//   a function of the input alone.
-// One workgroup: kHeavySamples ids at a fixed stride, counted in an LDS table; an id counts as heavy
-// when its estimated number of occurrences would fill more than a bucket and a half.
-__global__ void __launch_bounds__(1024)
-plan_heavy_kernel(const int64_t* __restrict__ ids, int64_t n, int64_t* __restrict__ heavy_ids,
-                  int32_t* __restrict__ heavy_n) {
-  __shared__ int64_t t_key[kHeavyTab];
-  __shared__ int32_t t_cnt[kHeavyTab];
-  __shared__ int64_t c_key[kHeavySamples / 8];
-  __shared__ int32_t c_cnt[kHeavySamples / 8];
-  __shared__ int32_t s_ncand, s_minus1;
+// kHeavySamples ids at a fixed stride are counted in an LDS table; an id counts as heavy when its
+// estimated number of occurrences would fill more than a bucket and a half. The heavy ids come out
+// ordered by (sample count descending, id ascending): a function of the input alone.
+// Every workgroup of the histogram kernel runs this for itself (the samples are the same 16 KB for
+// all of them, read out of the L2; a launch of one workgroup in front of the histogram cost more
+// than all of them doing it side by side); the first one leaves the result in global memory for
+// the kernels that follow.
+struct HeavyScratch {  // LDS of find_heavy
+  int64_t t_key[kHeavyTab];
+  int32_t t_cnt[kHeavyTab];
+  int64_t c_key[kHeavySamples / 8];
+  int32_t c_cnt[kHeavySamples / 8];
+  int32_t n_cand, minus1;
+};
+// out_ids [kHeavyMax] (LDS or global); returns their number (uniform). Every thread of a
+// workgroup of kPartBlock threads calls; ends with a barrier.
+__device__ __forceinline__ int find_heavy(const int64_t* __restrict__ ids, int64_t n, HeavyScratch& h,
+                                          int64_t* out_ids) {
   const int tid = threadIdx.x;
   const int64_t stride = n / kHeavySamples;
-  if (stride < 4) {  // a batch this small is no burden for one workgroup per bucket
-    if (tid == 0) *heavy_n = 0;
-    return;
-  }
-  for (int e = tid; e < kHeavyTab; e += 1024) {
-    t_key[e] = kSetEmpty;
-    t_cnt[e] = 0;
+  if (stride < 4) return 0;  // a batch this small is no burden for one workgroup per bucket (uniform)
+  for (int e = tid; e < kHeavyTab; e += kPartBlock) {
+    h.t_key[e] = kSetEmpty;
+    h.t_cnt[e] = 0;
   }
   if (tid == 0) {
-    s_ncand = 0;
-    s_minus1 = 0;
+    h.n_cand = 0;
+    h.minus1 = 0;
   }
   __syncthreads();
-  int64_t k[kHeavySamples / 1024];
+  constexpr int kMine = kHeavySamples / kPartBlock;
+  int64_t k[kMine];
 #pragma unroll
-  for (int x = 0; x < kHeavySamples / 1024; ++x) k[x] = ids[(static_cast<int64_t>(x) * 1024 + tid) * stride + stride / 2];
+  for (int x = 0; x < kMine; ++x) k[x] = ids[(static_cast<int64_t>(x) * kPartBlock + tid) * stride + stride / 2];
 #pragma unroll
-  for (int x = 0; x < kHeavySamples / 1024; ++x) {
+  for (int x = 0; x < kMine; ++x) {
     if (k[x] == kSetEmpty) {  // the table's empty marker is a legal id: counted apart
-      atomicAdd(&s_minus1, 1);
+      atomicAdd(&h.minus1, 1);
       continue;
     }
     int e = static_cast<int>(mix_id(k[x]) >> 40) & (kHeavyTab - 1);
     for (;;) {  // half empty at worst: always ends
-      const int64_t c = *reinterpret_cast<volatile int64_t*>(&t_key[e]);
+      const int64_t c = *reinterpret_cast<volatile int64_t*>(&h.t_key[e]);
       if (c == k[x]) break;
       if (c == kSetEmpty) {
-        const unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&t_key[e]),
+        const unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&h.t_key[e]),
                                                  static_cast<unsigned long long>(kSetEmpty),
                                                  static_cast<unsigned long long>(k[x]));
         if (old == static_cast<unsigned long long>(kSetEmpty) || old == static_cast<unsigned long long>(k[x])) break;
@@ -132,42 +136,41 @@ plan_heavy_kernel(const int64_t* __restrict__ ids, int64_t n, int64_t* __restric
       }
       e = (e + 1) & (kHeavyTab - 1);
     }
-    atomicAdd(&t_cnt[e], 1);
+    atomicAdd(&h.t_cnt[e], 1);
   }
   __syncthreads();
   // estimated occurrences = count * stride; heavy from one and a half buckets' worth, and never on
   // fewer than 8 samples (so at most kHeavySamples / 8 candidates)
   const int64_t want = (3 * kBucketIds / 2 + stride - 1) / stride;
   const int32_t thr = static_cast<int32_t>(want < 8 ? 8 : (want > kHeavySamples ? kHeavySamples + 1 : want));
-  for (int e = tid; e <= kHeavyTab; e += 1024) {
-    const int32_t c = e < kHeavyTab ? t_cnt[e] : s_minus1;
+  for (int e = tid; e <= kHeavyTab; e += kPartBlock) {
+    const int32_t c = e < kHeavyTab ? h.t_cnt[e] : h.minus1;
     if (c >= thr) {
-      const int at = atomicAdd(&s_ncand, 1);
-      c_key[at] = e < kHeavyTab ? t_key[e] : kSetEmpty;
-      c_cnt[at] = c;
+      const int at = atomicAdd(&h.n_cand, 1);
+      h.c_key[at] = e < kHeavyTab ? h.t_key[e] : kSetEmpty;
+      h.c_cnt[at] = c;
     }
   }
   __syncthreads();
-  const int ncand = s_ncand;
-  for (int i = tid; i < ncand; i += 1024) {  // rank by (count descending, id ascending): the first kHeavyMax stay
+  const int ncand = h.n_cand;
+  for (int i = tid; i < ncand; i += kPartBlock) {  // rank by (count descending, id ascending): the first kHeavyMax stay
     int rank = 0;
-    const int32_t ci = c_cnt[i];
-    const uint64_t ki = static_cast<uint64_t>(c_key[i]);
+    const int32_t ci = h.c_cnt[i];
+    const uint64_t ki = static_cast<uint64_t>(h.c_key[i]);
     for (int j = 0; j < ncand; ++j) {
-      const int32_t cj = c_cnt[j];
-      rank += (cj > ci || (cj == ci && static_cast<uint64_t>(c_key[j]) < ki)) ? 1 : 0;
+      const int32_t cj = h.c_cnt[j];
+      rank += (cj > ci || (cj == ci && static_cast<uint64_t>(h.c_key[j]) < ki)) ? 1 : 0;
     }
-    if (rank < kHeavyMax) heavy_ids[rank] = c_key[i];
+    if (rank < kHeavyMax) out_ids[rank] = h.c_key[i];
   }
-  if (tid == 0) *heavy_n = ncand < kHeavyMax ? ncand : kHeavyMax;
+  __syncthreads();
+  return ncand < kHeavyMax ? ncand : kHeavyMax;
 }
 
 // The heavy ids as an LDS table for the partition kernels: h_slot [kHeavySlots] holds the index of
 // a heavy id or -1, h_key its id (at most a quarter full: most ids end their search on the first
 // word they read). Every thread of the workgroup calls; ends with a barrier.
-__device__ __forceinline__ int load_heavy(const int64_t* __restrict__ heavy_ids, const int32_t* __restrict__ heavy_n,
-                                          int32_t* h_slot, int64_t* h_key) {
-  const int n_heavy = *heavy_n;
+__device__ __forceinline__ int heavy_table(const int64_t* heavy_ids, int n_heavy, int32_t* h_slot, int64_t* h_key) {
   if (n_heavy == 0) return 0;  // uniform
   for (int e = threadIdx.x; e < kHeavySlots; e += blockDim.x) h_slot[e] = -1;
   __syncthreads();
@@ -179,6 +182,10 @@ __device__ __forceinline__ int load_heavy(const int64_t* __restrict__ heavy_ids,
   }
   __syncthreads();
   return n_heavy;
+}
+__device__ __forceinline__ int load_heavy(const int64_t* __restrict__ heavy_ids, const int32_t* __restrict__ heavy_n,
+                                          int32_t* h_slot, int64_t* h_key) {
+  return heavy_table(heavy_ids, *heavy_n, h_slot, h_key);
 }
 // Index of `key` among the heavy ids, or -1.
 __device__ __forceinline__ int heavy_index(int64_t key, uint64_t mixed, const int32_t* h_slot, const int64_t* h_key) {
@@ -250,22 +257,31 @@ __device__ __forceinline__ void wave_count_one(int32_t* arr, int e, bool active)
   if (active) atomicAdd(&arr[e], 1);
 }
 
-// hist: ids per (row, column); columns: the heavy ids, then the buckets
+// hist: the heavy ids (found here, see find_heavy; left in heavy_ids / heavy_n by the first
+// workgroup), then ids per (row, column); columns: the heavy ids, then the buckets
 __global__ void __launch_bounds__(kPartBlock)
-plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, const int64_t* __restrict__ heavy_ids,
-                 const int32_t* __restrict__ heavy_n, int32_t* __restrict__ hist, int64_t* __restrict__ counts,
+plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, int64_t* __restrict__ heavy_ids,
+                 int32_t* __restrict__ heavy_n, int32_t* __restrict__ hist, int64_t* __restrict__ counts,
                  int32_t* __restrict__ sync) {
-  extern __shared__ int32_t l_hist[];  // [kHeavyMax + nb]
+  // the sampling's tables first, the histogram [kHeavyMax + nb] afterwards, in the same memory
+  extern __shared__ __align__(16) unsigned char l_raw[];
+  int32_t* l_hist = reinterpret_cast<int32_t*>(l_raw);
   __shared__ int32_t h_slot[kHeavySlots];
   __shared__ int64_t h_key[kHeavySlots];
+  __shared__ int64_t h_ids[kHeavyMax];
   const int tid = threadIdx.x;
   const int nc = kHeavyMax + (1 << g.nb_log2);
   if (blockIdx.x == 0) {
     if (tid < 2) counts[tid] = 0;
     if (tid < 4) sync[tid] = 0;  // [1] finished workgroups of the bucket kernel, [2] of the row assignment, [3] new keys
   }
+  const int n_found = find_heavy(ids, g.n, *reinterpret_cast<HeavyScratch*>(l_raw), h_ids);
+  if (blockIdx.x == 0) {
+    if (tid < n_found) heavy_ids[tid] = h_ids[tid];
+    if (tid == 0) *heavy_n = n_found;
+  }
   for (int b = tid; b < nc; b += kPartBlock) l_hist[b] = 0;
-  const int n_heavy = load_heavy(heavy_ids, heavy_n, h_slot, h_key);
+  const int n_heavy = heavy_table(h_ids, n_found, h_slot, h_key);
   __syncthreads();
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
   for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {  // four loads in flight
@@ -1338,14 +1354,9 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int6
   hv.inverse = inverse_out;
   hv.pos_out = pos_out;
   {
-    RECIS_TIME_KERNEL("plan_heavy_kernel", stream)
-    plan_heavy_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, g.n, heavy_ids, heavy_n);
-    RECIS_LAUNCH_CHECK();
-  }
-  {
     RECIS_TIME_KERNEL("plan_hist_kernel", stream)
-    plan_hist_kernel<<<dim3(g.rows), dim3(kPartBlock), lds, stream>>>(ids, g, heavy_ids, heavy_n, hist, counts_out_dev,
-                                                                      sync);
+    plan_hist_kernel<<<dim3(g.rows), dim3(kPartBlock), std::max(lds, sizeof(HeavyScratch)), stream>>>(
+        ids, g, heavy_ids, heavy_n, hist, counts_out_dev, sync);
     RECIS_LAUNCH_CHECK();
   }
   {

@@ -409,11 +409,12 @@ seg_max_fwd_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out,
 #pragma unroll
       for (int j = 0; j < VEC; ++j) best[j] = key[j] ? max_key_value(key[j]) : 0.f;
       store_pack<TOut, VEC>(out + s * D + c0, best);
-      if (argmax) {
+      if (argmax) {  // one store per lane, like the values (the host picks VEC so that it is aligned)
+        Pack<int32_t, VEC> am;
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
-          argmax[s * D + c0 + j] =
-              key[j] ? static_cast<int32_t>(0xFFFFFFFFu - static_cast<uint32_t>(key[j])) : -1;
+          am.v[j] = key[j] ? static_cast<int32_t>(0xFFFFFFFFu - static_cast<uint32_t>(key[j])) : -1;
+        *reinterpret_cast<Pack<int32_t, VEC>*>(argmax + s * D + c0) = am;
       }
     }
   }
@@ -532,11 +533,12 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
 #pragma unroll
       for (int j = 0; j < VEC; ++j) best[j] = key[j] ? max_key_value(key[j]) : 0.f;
       store_pack<TOut, VEC>(out + s * D + c0, best);
-      if (argmax) {
+      if (argmax) {  // one store per lane, like the values (the host picks VEC so that it is aligned)
+        Pack<int32_t, VEC> am;
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
-          argmax[s * D + c0 + j] =
-              key[j] ? static_cast<int32_t>(0xFFFFFFFFu - static_cast<uint32_t>(key[j])) : -1;
+          am.v[j] = key[j] ? static_cast<int32_t>(0xFFFFFFFFu - static_cast<uint32_t>(key[j])) : -1;
+        *reinterpret_cast<Pack<int32_t, VEC>*>(argmax + s * D + c0) = am;
       }
     }
   }
@@ -989,7 +991,8 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
   const int vb_out = pick_vec_bytes_max(D * out_sz, reinterpret_cast<uintptr_t>(out), 32);
   int vec = std::min(vb_in / in_sz, vb_out / out_sz);
   if (vec < 1) vec = 1;
-  if (mode == RECIS_MAX && argmax_out) vec = std::min(vec, 4);
+  if (mode == RECIS_MAX && argmax_out)  // the winners' occurrences leave as packs of VEC 32-bit words
+    vec = std::min(vec, pick_vec_bytes(D * 4, reinterpret_cast<uintptr_t>(argmax_out)) / 4);
   RowGeom geom;
   geom.vec = vec;
   geom.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
