@@ -186,15 +186,17 @@ class Config4:
 
     # the stages, also timed one by one for the breakdown
     def feature_ops(self):
+        """The 39 id columns of the batch: the sparse ones as they are, the dense ones bucketized and
+        reduced. They are tagged with their table (ids_encode) by the plan's own reads."""
         o = self.ops
         buckets = o.fused_bucketized(self.c["dense"], self.c["boundaries"])
         extra = o.fused_uint64_mod(buckets, self.mods)
-        return o.ids_encode(self.c["sparse"] + extra, self.tags)
+        return self.c["sparse"] + extra
 
     def dedup(self, ids):
-        """Dedup and find-or-insert in one pass: the plan carries the row of every unique id. Every
-        field holds one id per sample, so nothing per occurrence but the lists is asked for."""
-        self.plan = self.table.plan_lookup(ids, need_inverse=False, need_pos=False)
+        """Tagging, dedup and find-or-insert in one pass: the plan carries the row of every unique id.
+        Every field holds one id per sample, so nothing per occurrence but the lists is asked for."""
+        self.plan = self.table.plan_lookup(ids, need_inverse=False, need_pos=False, tags=self.tags)
         return self.plan, None
 
     def lookup(self, plan):
@@ -282,7 +284,7 @@ class Config4:
 
     def algorithmic_bytes(self):
         N, U, S, D = self.N, self.U, self.N, self.D
-        feat = 13 * self.c["batch"] * (4 + 8) + 13 * self.c["batch"] * (8 + 8) + N * 16
+        feat = 13 * self.c["batch"] * (4 + 8) + 13 * self.c["batch"] * (8 + 8)   # bucketize, mod (tagging: in the plan's reads)
         return {
             "feature_ops": feat,
             "dedup+lookup": N * (8 + 4) + U * 8 + U * (16 + 8),
@@ -544,8 +546,8 @@ class Config5:
 
     def step(self):
         o = self.ops
-        ids = o.ids_encode([f["values"] for f in self.fields], list(range(len(self.fields))))
-        plan = self.table.plan_lookup(ids)   # dedup + find-or-insert, one pass
+        # tagging (ids_encode), dedup and find-or-insert in one pass
+        plan = self.table.plan_lookup([f["values"] for f in self.fields], tags=list(range(len(self.fields))))
         self.U = plan.U
         inv = plan.inverse
         index = self.table.settle_lookup(plan.index_buf, self.U, plan)

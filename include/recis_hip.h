@@ -434,6 +434,23 @@ int recis_unique_plan_lookup(recis_idmap* m, const int64_t* ids, int64_t n, int6
                              int32_t* pos_out, int32_t* hot_items_out, int64_t hot_cap,
                              int64_t* counts_out_dev, int64_t* index_out, int64_t* unique_count_host,
                              int flags, void* stream);
+
+/*
+ * recis_unique_plan / recis_unique_plan_lookup (map != NULL) of a batch that is given as n_jobs
+ * (1..64) arrays laid end to end: array k holds sizes[k] ids, and with table_ids != NULL every id
+ * is tagged with its array's table on the way in, as recis_ids_encode does
+ * (csrc/ops/ids_encode_kernel.cu:16-20; table_ids == NULL: the plain concatenation). The kernels
+ * read the arrays directly, so the tagged batch that ids_encode would write and the plan read
+ * back never exists; unique_out holds tagged ids, positions (inverse, lists) count along the
+ * concatenation. ids_ptrs / sizes / table_ids are host arrays. Everything else as in
+ * recis_unique_plan_lookup (index_out unused without a map).
+ */
+int recis_unique_plan_jobs(recis_idmap* map, const int64_t* const* ids_ptrs, const int64_t* sizes,
+                           const int64_t* table_ids, int64_t n_jobs, int64_t* unique_out,
+                           int32_t* inverse_out, int32_t* row_start_out, int32_t* list_out,
+                           int32_t* pos_out, int32_t* hot_items_out, int64_t hot_cap,
+                           int64_t* counts_out_dev, int64_t* index_out, int64_t* unique_count_host,
+                           int flags, void* stream);
 /* inverse_out [n] and / or pos_out [n] of a plan that was made without them (either may be NULL),
  * from its row_start, list and counts. No counterpart in the reference. */
 int recis_plan_inverse_from_lists(const int32_t* row_start, const int32_t* list, const int64_t* counts_dev,

@@ -78,6 +78,103 @@ __device__ __forceinline__ int home_of_mix(uint64_t mixed, int nb_log2) {
   return static_cast<int>(mixed >> (64 - nb_log2 - 12)) & (kTabHome - 1);
 }
 
+// The batch as the partition kernels read it: one array of ids, or up to kPlanJobs arrays laid end
+// to end whose ids are tagged on the way in. The second form is ids_encode
+// (csrc/ops/ids_encode_kernel.cu:16-20: id & (2^52 - 1) | table << 52) or a plain concatenation
+// folded into the plan's own reads, so the encoded batch is never written and read back.
+constexpr int kPlanJobs = 64;
+struct IdJobs {
+  int n_jobs;  // 0: one array
+  int64_t mask;
+  const int64_t* in[kPlanJobs];
+  int64_t first[kPlanJobs + 1];  // place of the job's first id in the batch; first[n_jobs] = n
+  int64_t tag[kPlanJobs];        // in place (shifted)
+};
+struct JobTable {  // the same in LDS: lanes index it
+  const int64_t* in[kPlanJobs];
+  int64_t first[kPlanJobs + 1];
+  int64_t tag[kPlanJobs];
+};
+// Every thread of the workgroup calls; ends with a barrier. The kernels take IdJobs by value as
+// their SECOND argument, after one pointer: the table is read here straight out of the kernel
+// argument segment (ordinary memory), a lane per entry. Indexing the by-value argument with a
+// lane's own index instead makes the compiler copy the whole table into every lane's scratch
+// memory first, and a loop with uniform indices reads it one scalar load after the other (both
+// measured: 6 and 13 us per kernel).
+constexpr int kJobsArgOffset = 8;
+template <bool JOBS>
+__device__ __forceinline__ void load_jobs(const IdJobs& J, JobTable& t) {
+  if constexpr (JOBS) {
+    const IdJobs* in_memory = reinterpret_cast<const IdJobs*>(
+        reinterpret_cast<uintptr_t>(__builtin_amdgcn_kernarg_segment_ptr()) + kJobsArgOffset);
+    for (int k = threadIdx.x; k <= J.n_jobs; k += blockDim.x) {
+      t.first[k] = in_memory->first[k];
+      if (k < J.n_jobs) {
+        t.in[k] = in_memory->in[k];
+        t.tag[k] = in_memory->tag[k];
+      }
+    }
+    __syncthreads();
+  }
+}
+// The id at place i of the batch. A reader keeps the job of its last read in registers (where its
+// ids lie, its tag, where it ends): reads at ascending places, the usual case, cost one comparison
+// more than a plain load; any other place costs a short search of the table.
+template <bool JOBS>
+struct IdReader {
+  const int64_t* ids;  // one array: the batch; jobs: the current job's array moved so that place i is base[i]
+  const JobTable* t;
+  int n_jobs;
+  int64_t mask;
+  int j;
+  int64_t begin, end, tag;  // of the current job
+  __device__ __forceinline__ IdReader(const int64_t* ids_, const IdJobs& J, const JobTable& tab)
+      : ids(ids_), t(&tab), n_jobs(J.n_jobs), mask(J.mask), j(-1), begin(0), end(0), tag(0) {}
+  __device__ __forceinline__ void enter(int job) {
+    j = job;
+    begin = t->first[job];
+    ids = t->in[job] - begin;
+    end = t->first[job + 1];
+    tag = t->tag[job];
+  }
+  // Whether the places a .. b all lie in the current job: then raw() reads them with no test in
+  // between, so that a thread's loads stay in flight together.
+  __device__ __forceinline__ bool covers(int64_t a, int64_t b) const { return !JOBS || (a >= begin && b < end); }
+  __device__ __forceinline__ int64_t raw(int64_t i) const {
+    if constexpr (!JOBS) {
+      return ids[i];
+    } else {
+      return (ids[i] & mask) | tag;
+    }
+  }
+  __device__ __forceinline__ void seek(int64_t i) {  // enters the job that holds place i
+    int lo = 0, hi = n_jobs;                         // first[lo] <= i < first[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (t->first[mid] <= i)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    enter(lo);
+    while (i >= end) enter(j + 1);  // the search may land on an empty job before the right one
+  }
+  __device__ __forceinline__ int64_t at(int64_t i) {  // i at or after the last read's place (after a seek)
+    if constexpr (!JOBS) {
+      return ids[i];
+    } else {
+      while (i >= end) enter(j + 1);  // empty jobs are stepped over
+      return (ids[i] & mask) | tag;
+    }
+  }
+  __device__ __forceinline__ int64_t at_any(int64_t i) {
+    if constexpr (JOBS) {
+      if (i >= end || i < begin) seek(i);
+    }
+    return at(i);
+  }
+};
+
 // Heavy ids. An id that makes up a sizeable share of the batch (the head of a Zipf distribution, the
 // few values of a low-cardinality feature) would put all its occurrences into one bucket and leave
 // one workgroup with a hundred times the work of the others. Such ids are found beforehand by
@@ -99,8 +196,8 @@ struct HeavyScratch {  // LDS of find_heavy
 };
 // out_ids [kHeavyMax] (LDS or global); returns their number (uniform). Every thread of a
 // workgroup of kPartBlock threads calls; ends with a barrier.
-__device__ __forceinline__ int find_heavy(const int64_t* __restrict__ ids, int64_t n, HeavyScratch& h,
-                                          int64_t* out_ids) {
+template <bool JOBS>
+__device__ __forceinline__ int find_heavy(IdReader<JOBS> rd, int64_t n, HeavyScratch& h, int64_t* out_ids) {
   const int tid = threadIdx.x;
   const int64_t stride = n / kHeavySamples;
   if (stride < 4) return 0;  // a batch this small is no burden for one workgroup per bucket (uniform)
@@ -115,8 +212,22 @@ __device__ __forceinline__ int find_heavy(const int64_t* __restrict__ ids, int64
   __syncthreads();
   constexpr int kMine = kHeavySamples / kPartBlock;
   int64_t k[kMine];
+  if constexpr (JOBS) {  // where the samples lie first, then all loads in flight together
+    const int64_t* at[kMine];
+    int64_t tag[kMine];
 #pragma unroll
-  for (int x = 0; x < kMine; ++x) k[x] = ids[(static_cast<int64_t>(x) * kPartBlock + tid) * stride + stride / 2];
+    for (int x = 0; x < kMine; ++x) {
+      const int64_t i = (static_cast<int64_t>(x) * kPartBlock + tid) * stride + stride / 2;
+      rd.seek(i);
+      at[x] = rd.ids + i;
+      tag[x] = rd.tag;
+    }
+#pragma unroll
+    for (int x = 0; x < kMine; ++x) k[x] = (*at[x] & rd.mask) | tag[x];
+  } else {
+#pragma unroll
+    for (int x = 0; x < kMine; ++x) k[x] = rd.raw((static_cast<int64_t>(x) * kPartBlock + tid) * stride + stride / 2);
+  }
 #pragma unroll
   for (int x = 0; x < kMine; ++x) {
     if (k[x] == kSetEmpty) {  // the table's empty marker is a legal id: counted apart
@@ -259,10 +370,14 @@ __device__ __forceinline__ void wave_count_one(int32_t* arr, int e, bool active)
 
 // hist: the heavy ids (found here, see find_heavy; left in heavy_ids / heavy_n by the first
 // workgroup), then ids per (row, column); columns: the heavy ids, then the buckets
+template <bool JOBS>
 __global__ void __launch_bounds__(kPartBlock)
-plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, int64_t* __restrict__ heavy_ids,
+plan_hist_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, int64_t* __restrict__ heavy_ids,
                  int32_t* __restrict__ heavy_n, int32_t* __restrict__ hist, int64_t* __restrict__ counts,
                  int32_t* __restrict__ sync) {
+  __shared__ JobTable s_jobs;
+  load_jobs<JOBS>(jobs, s_jobs);
+  IdReader<JOBS> rd(ids, jobs, s_jobs);
   // the sampling's tables first, the histogram [kHeavyMax + nb] afterwards, in the same memory
   extern __shared__ __align__(16) unsigned char l_raw[];
   int32_t* l_hist = reinterpret_cast<int32_t*>(l_raw);
@@ -275,7 +390,7 @@ plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, int64_t* __restric
     if (tid < 2) counts[tid] = 0;
     if (tid < 4) sync[tid] = 0;  // [1] finished workgroups of the bucket kernel, [2] of the row assignment, [3] new keys
   }
-  const int n_found = find_heavy(ids, g.n, *reinterpret_cast<HeavyScratch*>(l_raw), h_ids);
+  const int n_found = find_heavy<JOBS>(rd, g.n, *reinterpret_cast<HeavyScratch*>(l_raw), h_ids);
   if (blockIdx.x == 0) {
     if (tid < n_found) heavy_ids[tid] = h_ids[tid];
     if (tid == 0) *heavy_n = n_found;
@@ -284,12 +399,21 @@ plan_hist_kernel(const int64_t* __restrict__ ids, PlanGeom g, int64_t* __restric
   const int n_heavy = heavy_table(h_ids, n_found, h_slot, h_key);
   __syncthreads();
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
+  if (JOBS && lo + tid < hi) rd.seek(lo + tid);
   for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {  // four loads in flight
     int64_t k[4];
+    if (rd.covers(i0, min(hi - 1, i0 + 3 * kPartBlock))) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int64_t i = i0 + x * kPartBlock;
-      k[x] = i < hi ? ids[i] : 0;
+      for (int x = 0; x < 4; ++x) {
+        const int64_t i = i0 + x * kPartBlock;
+        k[x] = i < hi ? rd.raw(i) : 0;
+      }
+    } else {  // the places straddle arrays
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int64_t i = i0 + x * kPartBlock;
+        k[x] = i < hi ? rd.at_any(i) : 0;
+      }
     }
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
@@ -449,14 +573,18 @@ struct HeavyArgs {
 // totals for itself (a thousand words), so no kernel stands between the column scan and this one;
 // the first workgroup also leaves bucket_start [columns + 1] for the bucket kernel and clears that
 // kernel's look-back words.
+template <bool JOBS>
 __global__ void __launch_bounds__(kPartBlock)
-plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs hv, const int32_t* __restrict__ off,
+plan_scatter_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, HeavyArgs hv, const int32_t* __restrict__ off,
                     const int32_t* __restrict__ bucket_total, int32_t* __restrict__ bucket_start,
                     unsigned long long* __restrict__ agg, int64_t* __restrict__ bkt_id,
                     int32_t* __restrict__ bkt_pos) {
   extern __shared__ int32_t cursor[];  // [nc + 1], then kPartBlock words of scan scratch
   __shared__ int32_t h_slot[kHeavySlots];
   __shared__ int64_t h_key[kHeavySlots];
+  __shared__ JobTable s_jobs;
+  load_jobs<JOBS>(jobs, s_jobs);
+  IdReader<JOBS> rd(ids, jobs, s_jobs);
   const int tid = threadIdx.x;
   const int nb = 1 << g.nb_log2, nc = kHeavyMax + nb;
   const int n_heavy = load_heavy(hv.ids, hv.n, h_slot, h_key);
@@ -469,12 +597,21 @@ plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs hv, c
   for (int b = tid; b < nc; b += kPartBlock) cursor[b] += off_row[b];
   __syncthreads();
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
+  if (JOBS && lo + tid < hi) rd.seek(lo + tid);
   for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {
     int64_t k[4];
+    if (rd.covers(i0, min(hi - 1, i0 + 3 * kPartBlock))) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int64_t i = i0 + x * kPartBlock;
-      k[x] = i < hi ? ids[i] : 0;
+      for (int x = 0; x < 4; ++x) {
+        const int64_t i = i0 + x * kPartBlock;
+        k[x] = i < hi ? rd.raw(i) : 0;
+      }
+    } else {  // the places straddle arrays
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int64_t i = i0 + x * kPartBlock;
+        k[x] = i < hi ? rd.at_any(i) : 0;
+      }
     }
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
@@ -504,14 +641,18 @@ plan_scatter_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs hv, c
 // 4-byte store per id (scattered stores run at some 1e11 per second on this part whatever their
 // size).
 constexpr int kTilePer = kTile / kPartBlock;
+template <bool JOBS>
 __global__ void __launch_bounds__(kPartBlock)
-plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs hv,
+plan_scatter_runs_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, HeavyArgs hv,
                          const int32_t* __restrict__ off, const int32_t* __restrict__ bucket_total,
                          int32_t* __restrict__ bucket_start, unsigned long long* __restrict__ agg,
                          int64_t* __restrict__ bkt_id, int32_t* __restrict__ bkt_pos) {
   extern __shared__ int32_t lds[];
   __shared__ int32_t h_slot[kHeavySlots];
   __shared__ int64_t h_key[kHeavySlots];
+  __shared__ JobTable s_jobs;
+  load_jobs<JOBS>(jobs, s_jobs);
+  IdReader<JOBS> rd(ids, jobs, s_jobs);
   const int tid = threadIdx.x;
   const int nb = 1 << g.nb_log2, nc = kHeavyMax + nb;
   int32_t* gbase = lds;               // [nc + 1] where the tile's ids of a column go
@@ -532,10 +673,20 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs 
   const int n_here = static_cast<int>(min(g.n, lo + g.tile) - lo);
   int64_t k[kTilePer];
   uint16_t rank[kTilePer], bucket[kTilePer];
+  if (JOBS && n_here > 0) rd.seek(lo);
+  const bool one_job = n_here > 0 && rd.covers(lo, lo + n_here - 1);  // the whole tile in one array (uniform)
+  if (one_job) {
 #pragma unroll
-  for (int x = 0; x < kTilePer; ++x) {  // all loads in flight
-    const int i = tid + x * kPartBlock;
-    k[x] = i < n_here ? ids[lo + i] : 0;
+    for (int x = 0; x < kTilePer; ++x) {  // all loads in flight
+      const int i = tid + x * kPartBlock;
+      k[x] = i < n_here ? rd.raw(lo + i) : 0;
+    }
+  } else {
+#pragma unroll
+    for (int x = 0; x < kTilePer; ++x) {
+      const int i = tid + x * kPartBlock;
+      k[x] = i < n_here ? rd.at_any(lo + i) : 0;
+    }
   }
 #pragma unroll
   for (int x = 0; x < kTilePer; ++x) {
@@ -565,7 +716,8 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, PlanGeom g, HeavyArgs 
     for (int x = 0; x < 4; ++x) {
       const int j = j0 + x * kPartBlock;
       i[x] = j < n_here ? sorted[j] : 0;
-      key[x] = j < n_here ? ids[lo + i[x]] : 0;  // the tile was read a moment ago: a cache hit
+      // the tile was read a moment ago: a cache hit
+      key[x] = j >= n_here ? 0 : (one_job ? rd.raw(lo + i[x]) : rd.at_any(lo + i[x]));
     }
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
@@ -1329,7 +1481,7 @@ static uint32_t g_spin_limit = 1u << 22;
 // words that receive the unique count (and the soft-error bits) as soon as they are final, or NULL.
 // With a map, every unique id is looked up (find or insert) from inside the bucket kernel and
 // index_out receives its row.
-static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int64_t* unique_out,
+static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, const IdJobs* jobs_in, int64_t* unique_out,
                        int32_t* inverse_out, int32_t* row_start_out, int32_t* list_out, int32_t* pos_out,
                        int32_t* hot_items_out, int64_t hot_cap, int64_t* counts_out_dev, int64_t* staged,
                        hipEvent_t staged_event, int* err, recis_idmap* map, int64_t map_seq, int64_t* index_out,
@@ -1353,10 +1505,21 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int6
   hv.list = list_out;
   hv.inverse = inverse_out;
   hv.pos_out = pos_out;
+  const bool by_jobs = jobs_in != nullptr;
+  IdJobs jobs;  // the kernels take it by value
+  if (by_jobs)
+    jobs = *jobs_in;
+  else
+    jobs.n_jobs = 0;
   {
+    const size_t hist_lds = std::max(lds, sizeof(HeavyScratch));
     RECIS_TIME_KERNEL("plan_hist_kernel", stream)
-    plan_hist_kernel<<<dim3(g.rows), dim3(kPartBlock), std::max(lds, sizeof(HeavyScratch)), stream>>>(
-        ids, g, heavy_ids, heavy_n, hist, counts_out_dev, sync);
+    if (by_jobs)
+      plan_hist_kernel<true><<<dim3(g.rows), dim3(kPartBlock), hist_lds, stream>>>(ids, jobs, g, heavy_ids, heavy_n, hist,
+                                                                                  counts_out_dev, sync);
+    else
+      plan_hist_kernel<false><<<dim3(g.rows), dim3(kPartBlock), hist_lds, stream>>>(ids, jobs, g, heavy_ids, heavy_n,
+                                                                                   hist, counts_out_dev, sync);
     RECIS_LAUNCH_CHECK();
   }
   {
@@ -1365,14 +1528,25 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int6
     RECIS_LAUNCH_CHECK();
   }
   {
+    const dim3 grid(g.rows), block(kPartBlock);
     RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
-    if (g.tile <= kTile && g.tile >= 4 * nb)  // a tile sends four ids or more to a bucket: worth ordering them
-      plan_scatter_runs_kernel<<<dim3(g.rows), dim3(kPartBlock),
-                                 sizeof(int32_t) * (2 * (nc + 1) + kPartBlock) + 2 * sizeof(uint16_t) * kTile, stream>>>(
-          ids, g, hv, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
-    else
-      plan_scatter_kernel<<<dim3(g.rows), dim3(kPartBlock), lds + sizeof(int32_t) * (kPartBlock + 1), stream>>>(
-          ids, g, hv, hist, bucket_total, bucket_start, agg, bkt_id, bkt_pos);
+    if (g.tile <= kTile && g.tile >= 4 * nb) {  // a tile sends four ids or more to a bucket: worth ordering them
+      const size_t runs_lds = sizeof(int32_t) * (2 * (nc + 1) + kPartBlock) + 2 * sizeof(uint16_t) * kTile;
+      if (by_jobs)
+        plan_scatter_runs_kernel<true><<<grid, block, runs_lds, stream>>>(ids, jobs, g, hv, hist, bucket_total,
+                                                                         bucket_start, agg, bkt_id, bkt_pos);
+      else
+        plan_scatter_runs_kernel<false><<<grid, block, runs_lds, stream>>>(ids, jobs, g, hv, hist, bucket_total,
+                                                                          bucket_start, agg, bkt_id, bkt_pos);
+    } else {
+      const size_t plain_lds = lds + sizeof(int32_t) * (kPartBlock + 1);
+      if (by_jobs)
+        plan_scatter_kernel<true><<<grid, block, plain_lds, stream>>>(ids, jobs, g, hv, hist, bucket_total, bucket_start,
+                                                                     agg, bkt_id, bkt_pos);
+      else
+        plan_scatter_kernel<false><<<grid, block, plain_lds, stream>>>(ids, jobs, g, hv, hist, bucket_total, bucket_start,
+                                                                      agg, bkt_id, bkt_pos);
+    }
     RECIS_LAUNCH_CHECK();
   }
   BucketArgs a;
@@ -1430,8 +1604,10 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, int6
 static int plan_entry(recis_idmap* map, const int64_t* ids, int64_t n, int64_t* unique_out, int32_t* inverse_out,
                       int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
                       int64_t hot_cap, int64_t* counts_out_dev, int64_t* index_out, int64_t* unique_count_host,
-                      int flags, hipStream_t stream) {
-  if (int rc = plan_check_args(ids, n, unique_out, row_start_out, list_out, hot_items_out, hot_cap, counts_out_dev))
+                      int flags, hipStream_t stream, const IdJobs* jobs = nullptr) {
+  // with jobs, `ids` is unused (the kernels read the jobs' arrays); any non-NULL value passes the checks
+  if (int rc = plan_check_args(jobs ? reinterpret_cast<const int64_t*>(jobs) : ids, n, unique_out, row_start_out,
+                               list_out, hot_items_out, hot_cap, counts_out_dev))
     return rc;
   RECIS_REQUIRE(map == nullptr || n == 0 || index_out != nullptr, "index_out must not be NULL");
   int* err = device_error_word(current_device());
@@ -1456,7 +1632,7 @@ static int plan_entry(recis_idmap* map, const int64_t* ids, int64_t n, int64_t* 
   const PlanLayout L = plan_layout(n, map != nullptr);
   void* ws = nullptr;
   if (int rc = get_workspace(stream, L.bytes, &ws)) return rc;
-  if (int rc = plan_launch(L, static_cast<char*>(ws), ids, unique_out, inverse_out, row_start_out, list_out, pos_out,
+  if (int rc = plan_launch(L, static_cast<char*>(ws), ids, jobs, unique_out, inverse_out, row_start_out, list_out, pos_out,
                            hot_items_out, hot_cap, counts_out_dev, staged, staged_event, err, map, seq, index_out,
                            stream))
     return rc;
@@ -1482,6 +1658,36 @@ int recis_unique_plan_lookup(recis_idmap* map, const int64_t* ids, int64_t n, in
   RECIS_REQUIRE(map != nullptr, "id map is NULL");
   return plan_entry(map, ids, n, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
                     counts_out_dev, index_out, unique_count_host, flags, static_cast<hipStream_t>(stream_));
+}
+
+int recis_unique_plan_jobs(recis_idmap* map, const int64_t* const* ids_ptrs, const int64_t* sizes,
+                           const int64_t* table_ids, int64_t n_jobs, int64_t* unique_out, int32_t* inverse_out,
+                           int32_t* row_start_out, int32_t* list_out, int32_t* pos_out, int32_t* hot_items_out,
+                           int64_t hot_cap, int64_t* counts_out_dev, int64_t* index_out, int64_t* unique_count_host,
+                           int flags, void* stream_) {
+  RECIS_REQUIRE(n_jobs >= 1 && n_jobs <= kPlanJobs, "1 to %d arrays of ids (got %lld)", kPlanJobs, (long long)n_jobs);
+  RECIS_REQUIRE(ids_ptrs && sizes, "NULL argument");
+  IdJobs jobs;
+  jobs.n_jobs = static_cast<int>(n_jobs);
+  jobs.mask = table_ids ? (int64_t(1) << 52) - 1 : ~int64_t(0);
+  int64_t n = 0;
+  for (int k = 0; k < kPlanJobs; ++k) {
+    jobs.in[k] = nullptr;
+    jobs.tag[k] = 0;
+    jobs.first[k] = n;
+    if (k >= n_jobs) continue;
+    RECIS_REQUIRE(sizes[k] >= 0 && (sizes[k] == 0 || ids_ptrs[k]), "bad array %d", k);
+    if (table_ids) {
+      RECIS_REQUIRE(table_ids[k] >= 0 && table_ids[k] < 4096, "table id %lld out of 12 bits", (long long)table_ids[k]);
+      jobs.tag[k] = static_cast<int64_t>(static_cast<uint64_t>(table_ids[k]) << 52);
+    }
+    jobs.in[k] = ids_ptrs[k];
+    n += sizes[k];
+  }
+  jobs.first[kPlanJobs] = n;
+  for (int k = static_cast<int>(n_jobs); k <= kPlanJobs; ++k) jobs.first[k] = n;
+  return plan_entry(map, nullptr, n, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
+                    counts_out_dev, index_out, unique_count_host, flags, static_cast<hipStream_t>(stream_), &jobs);
 }
 
 int recis_plan_inverse_from_lists(const int32_t* row_start, const int32_t* list, const int64_t* counts_dev, int64_t n,
@@ -1547,7 +1753,7 @@ int recis_unique_plan_noalloc(const int64_t* ids, int64_t n, int64_t* unique_out
   // What must start at zero (the two counters in `sync`, the look-back words) is cleared by the
   // plan's own first two kernels; every other scratch array is fully written by the kernel that
   // produces it before any kernel reads it: nothing of the previous call's contents is relied on.
-  return plan_launch(L, base, ids, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
+  return plan_launch(L, base, ids, nullptr, unique_out, inverse_out, row_start_out, list_out, pos_out, hot_items_out, hot_cap,
                      counts_out_dev, nullptr, nullptr, err, nullptr, 0, nullptr, stream);
 }
 

@@ -227,16 +227,18 @@ def _pools_out_of_the_table(hashtable, opt, n_occ, n_offsets):
     return opt.combiner in ("sum", "mean") and float_table and not sparse_mean and not id_mean
 
 
-def make_plan(hashtable: HashTable, ids, offsets, opt, has_weight=False, unit_segments=False):
+def make_plan(hashtable: HashTable, ids, offsets, opt, has_weight=False, unit_segments=False, tags=None):
     """The batch plan of ``ids`` for ``lookup_and_pool``. When what follows is the training lookup
     that admits new keys and pools out of the table, dedup and find-or-insert run as one pass
     (``HashtableImpl.plan_lookup``) and the plan carries the rows; ``unit_segments`` plans leave
-    out the per-occurrence arrays nobody reads (the expansion and its backward walk the lists)."""
+    out the per-occurrence arrays nobody reads (the expansion and its backward walk the lists).
+    ``ids`` may be a list of id tensors with their table ``tags`` (``ops.ids_unique_plan``)."""
+    n_occ = sum(t.numel() for t in ids) if isinstance(ids, (list, tuple)) else ids.numel()
     if (hashtable.training and opt.trainable and opt.admit_hook is None
-            and _pools_out_of_the_table(hashtable, opt, ids.numel(), offsets.numel())):
+            and _pools_out_of_the_table(hashtable, opt, n_occ, offsets.numel())):
         lean = bool(unit_segments)
-        return hashtable._hashtable_impl.plan_lookup(ids, need_inverse=not lean)
-    return ops.ids_unique_plan(ids, wait=False, need_pos=False)
+        return hashtable._hashtable_impl.plan_lookup(ids, need_inverse=not lean, tags=tags)
+    return ops.ids_unique_plan(ids, wait=False, need_pos=False, tags=tags)
 
 
 def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False, combiner_kwargs=None):

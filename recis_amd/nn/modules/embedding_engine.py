@@ -160,10 +160,10 @@ class EmbeddingEngine(torch.nn.Module):
                 if same in plans:
                     offsets, plan = plans[same]
                 else:
-                    if info.is_coalesce():
-                        ids = ops.ids_encode(vals, [tag_of[n] for n in names])
-                    else:
-                        ids = vals[0] if len(vals) == 1 else torch.cat(vals)
+                    # the id tensors go to the plan as they are: it tags (ids_encode) / concatenates them
+                    # in its own reads
+                    tags = [tag_of[n] for n in names] if info.is_coalesce() else None
+                    ids = vals if (tags is not None or len(vals) > 1) else vals[0]
                     if len(offs) == 1:
                         offsets = offs[0]
                     elif all(d is not None for d in dense):  # dense id tensors only: a function of the shapes
@@ -174,12 +174,13 @@ class EmbeddingEngine(torch.nn.Module):
                     if opt0.combiner == "tile":
                         if (table.training and opt0.trainable and opt0.admit_hook is None
                                 and table._dtype in (torch.float32, torch.bfloat16, torch.float16)):
-                            plan = table._hashtable_impl.plan_lookup(ids)   # dedup + find-or-insert, one pass
+                            plan = table._hashtable_impl.plan_lookup(ids, tags=tags)   # dedup + find-or-insert, one pass
                         else:
-                            plan = ops.ids_unique_plan(ids, wait=False, need_pos=False)
+                            plan = ops.ids_unique_plan(ids, wait=False, need_pos=False, tags=tags)
                     else:  # lean (no per-occurrence arrays) only if no other option can come to share it
                         alone = sum(1 for k in runtime.values() if any(inputs[n] is inputs[names[0]] for n in k)) == 1
-                        plan = make_plan(table, ids, offsets, opt0, any_weight, unit_segments=all_unit and alone)
+                        plan = make_plan(table, ids, offsets, opt0, any_weight, unit_segments=all_unit and alone,
+                                         tags=tags)
                     plans[same] = (offsets, plan)
                 weight = None
                 if all(w is not None for w in weights):

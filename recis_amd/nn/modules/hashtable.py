@@ -396,13 +396,14 @@ class HashtableImpl:
         plan.lookup_calls[id(self)] = self._idmap.last_call()
         return index_buf
 
-    def plan_lookup(self, ids, wait=False, need_inverse=True, need_pos=False):
+    def plan_lookup(self, ids, wait=False, need_inverse=True, need_pos=False, tags=None):
         """Dedup of ``ids`` and find-or-insert of the distinct ids in this table in one pass
         (``recis_unique_plan_lookup``): the batch plan with ``index_buf`` = the row of every unique
-        id. Replaces ``ids_partition`` / ``torch.unique`` + ``IdMap::Lookup`` of the training
+        id. ``ids`` may be a list of id tensors with their table ``tags`` (see ``ops.ids_unique_plan``). Replaces ``ids_partition`` / ``torch.unique`` + ``IdMap::Lookup`` of the training
         lookup (recis/nn/modules/hashtable.py:262-293). Room is made for the rows every id of the
         batch could need; settle with ``settle_count(plan.U, plan)`` once the count has been read."""
-        plan = ops.ids_unique_plan(ids, wait=wait, need_inverse=need_inverse, need_pos=need_pos, idmap=self._idmap)
+        plan = ops.ids_unique_plan(ids, wait=wait, need_inverse=need_inverse, need_pos=need_pos, idmap=self._idmap,
+                                   tags=tags)
         plan.lookup_calls[id(self)] = self._idmap.last_call()
         self._make_room(plan.n if wait is False else plan.U)
         return plan

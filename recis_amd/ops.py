@@ -859,17 +859,38 @@ def _raise_staged_device_errors(stream):
         _lib.raise_device_errors(bits.value)   # waits for the device and clears the word
 
 
-def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None):
-    """Dedup + transposed index of a batch of ids (``recis_unique_plan``). ``wait=False``
+_PLAN_JOBS = 64  # arrays one recis_unique_plan_jobs call takes
+
+
+def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None, tags=None):
+    """Dedup + transposed index of a batch of ids (``recis_unique_plan``). ``ids`` may be a list of
+    id tensors: the batch is their concatenation, tagged per tensor with ``tags`` as ``ids_encode``
+    does when given (``recis_unique_plan_jobs``: the kernels read the tensors directly, the tagged
+    batch is never written). ``wait=False``
     returns without the host copy of the unique count (see ``BatchPlan``); at most one such
     plan per stream may have its count outstanding. ``need_inverse`` / ``need_pos`` = False leave
     those two arrays to be derived from the lists if anybody asks (callers that only walk the
     lists save two scattered writes per id). With ``idmap`` (an ``IdMap``) the unique ids are
     found or inserted in that map in the same pass (``recis_unique_plan_lookup``) and
     ``plan.index_buf`` holds their rows."""
-    ids = _ids64(ids)
-    n = ids.numel()
-    dev = ids.device
+    jobs = None
+    if isinstance(ids, (list, tuple)):
+        jobs = [_ids64(t).reshape(-1) for t in ids]
+        if tags is not None and len(tags) != len(jobs):
+            raise ValueError("ids_unique_plan: %d tags for %d id tensors" % (len(tags), len(jobs)))
+        if len(jobs) > _PLAN_JOBS or len(jobs) == 0:  # too many for one call: make the batch first
+            ids = ids_encode(jobs, tags) if tags is not None else (torch.cat(jobs) if jobs else torch.empty(0, dtype=torch.int64))
+            jobs = None
+    elif tags is not None:
+        raise ValueError("ids_unique_plan: tags go with a list of id tensors")
+    if jobs is None:
+        ids = _ids64(ids)
+        n = ids.numel()
+        dev = ids.device
+    else:
+        require_cuda(*jobs)
+        n = sum(t.numel() for t in jobs)
+        dev = jobs[0].device
     p = BatchPlan()
     p.serial = next(_PLAN_SERIAL)  # never reused, unlike id(p)
     p.n = n
@@ -890,7 +911,16 @@ def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None
     # every launch overwrites the stream's staging word: an earlier plan whose count is still
     # outstanding there must read its own device word from now on
     _STAGED.pop(p._stream.value, None)
-    if idmap is None:
+    if jobs is not None:
+        if idmap is not None:
+            p.index_buf = torch.empty(n, dtype=torch.int64, device=dev)
+        check(lib().recis_unique_plan_jobs(idmap._h if idmap is not None else None, _host_ptrs(jobs),
+                                           _host_i64([t.numel() for t in jobs]),
+                                           _host_i64(tags) if tags is not None else None, i64(len(jobs)),
+                                           ptr(p.unique_buf), ptr(p._inverse), ptr(p.row_start), ptr(p.occ), ptr(p._pos),
+                                           ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts), ptr(p.index_buf),
+                                           ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
+    elif idmap is None:
         check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(p.unique_buf), ptr(p._inverse), ptr(p.row_start),
                                       ptr(p.occ), ptr(p._pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts),
                                       ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))

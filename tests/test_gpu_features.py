@@ -515,3 +515,37 @@ def test_two_input_gather_reduce_second_input_in_parts(rng):
     with pytest.raises(TypeError):
         ops.csr_gather_reduce2(plan, ([first[0]], first[1], first[2]), (parts, second[1], None))   # not both in parts
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("sizes,with_tags", [([70000, 0, 1, 123457, 8192, 300], True), ([5000] * 40, True),
+                                             ([1], True), ([100000, 250000], False), ([3] * 64, False)])
+def test_unique_plan_from_separate_arrays_equals_the_plan_of_the_encoded_batch(rng, sizes, with_tags):
+    """recis_unique_plan_jobs (the batch as separate arrays, tagged on the way in) against
+    recis_ids_encode + recis_unique_plan: the same unique ids in the same order, the same lists
+    (as sets per id: the order inside a list is unspecified), inverse and counts; with an id map,
+    the same rows. Empty arrays, arrays that end inside a tile, a heavy id, more arrays than a tile
+    has threads to spare."""
+    parts = [rng.integers(0, 5000, size=s) if k % 3 else rng.integers(0, 3, size=s) for k, s in enumerate(sizes)]
+    dev_parts = [_dev(p.astype(np.int64)) for p in parts]
+    tags = [(7 * k + 1) % 4096 for k in range(len(sizes))] if with_tags else None
+    batch = ops.ids_encode(dev_parts, tags) if with_tags else torch.cat(dev_parts)
+    ref = ops.ids_unique_plan(batch)
+    got = ops.ids_unique_plan(dev_parts, tags=tags)
+    assert got.U == ref.U and got.n == ref.n
+    U = ref.U
+    assert torch.equal(got.unique[:U], ref.unique[:U])
+    assert torch.equal(got.inverse, ref.inverse)
+    assert torch.equal(got.row_start[: U + 1], ref.row_start[: U + 1])
+    rs = ref.row_start[: U + 1].cpu().numpy()
+    a, b = got.occ.cpu().numpy(), ref.occ.cpu().numpy()
+    owner = np.repeat(np.arange(U), np.diff(rs))
+    assert np.array_equal(a[np.lexsort((a, owner))], b[np.lexsort((b, owner))])   # the same occurrences per id
+    assert torch.equal(got.counts, ref.counts)
+    # with an id map: rows of known keys are found, new keys get the rows the encoded batch would have got
+    from recis_amd.ops import IdMap
+    m1, m2 = IdMap(reserve=1 << 16), IdMap(reserve=1 << 16)
+    p1 = ops.ids_unique_plan(batch, idmap=m1)
+    p2 = ops.ids_unique_plan(dev_parts, tags=tags, idmap=m2)
+    assert torch.equal(p1.index_buf[:U], p2.index_buf[:U])
+    assert m1.stats()[:2] == m2.stats()[:2]
+    assert _lib.poll_device_errors() == 0

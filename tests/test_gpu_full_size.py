@@ -29,7 +29,8 @@ def test_config4_step_properties():
     wl = bench.Config4()
     for _ in range(2):          # second step: all keys known, rows and Adam state not trivial
         wl.step()
-    ids = wl.feature_ops()
+    cols = wl.feature_ops()                       # the 39 id columns; the plan tags them as it reads them
+    ids = ops.ids_encode(cols, wl.tags)           # what the plan sees
     N, D = wl.N, wl.D
     assert ids.numel() == N == 39 * 65536
     # feature ops against their definitions on a full column
@@ -39,7 +40,7 @@ def test_config4_step_properties():
     assert torch.equal(ids[26 * 65536: 27 * 65536], exp_bucket | (tag << 52))
     assert torch.equal(ids[: 65536], wl.c["sparse"][0] & ((1 << 52) - 1))
 
-    plan, _ = wl.dedup(ids)          # dedup + find-or-insert in one pass; inverse derived from the lists
+    plan, _ = wl.dedup(cols)         # tagging + dedup + find-or-insert in one pass; inverse derived from the lists
     inv = plan.inverse
     uniq = plan.unique
     U = plan.U
