@@ -11,10 +11,10 @@ for sum / mean / max) is measured in the same run and reported under "workloads"
 
 "roofline" describes the kernel that takes the largest share of the step: algorithmic
 bytes per launch / mean launch time (HIP events on the launch stream) against the 8 TB/s
-HBM peak. "cpu_baseline" is the restated reference CPU path (oracle.cpu_path) timed on
-this host on a bounded sample of the same workload; "cpu_reference_<n>t" is the reference's own
-CPU code (oracle/_ref, when built) on the same sample with n threads, for the parts of the step
-the reference can run on a CPU.
+HBM peak. "cpu_baseline" is the reference's own CPU code (oracle/_ref, when built) on all host
+cores of this box's share, on a bounded sample of the same workload; "cpu_baseline_reference_1core"
+the same on one thread, "cpu_baseline_port_1core" the restated CPU path (oracle.cpu_path) on one
+core. Without oracle/_ref, "cpu_baseline" is the port.
 """
 import argparse
 import json
@@ -712,9 +712,9 @@ class ModulePath5:
 # scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC_C4 = {
-    "csr_rows_adam_kernel": 730625331, "csr_expand_kernel": 260825088, "plan_bucket_kernel": 193435648,
-    "plan_scatter_kernel": 105619149, "ids_encode_kernel": 40936858, "plan_hist_kernel": 21896499,
-    "uint64_mod_kernel": 13689037, "bucketize_kernel": 10261094, "plan_colscan_kernel": 4108493,
+    "csr_rows_adam_kernel": 729275494, "csr_expand_kernel": 260871885, "plan_bucket_kernel": 192791142,
+    "plan_scatter_kernel": 107226112, "plan_hist_kernel": 23857869, "uint64_mod_kernel": 13688832,
+    "bucketize_kernel": 10261094, "plan_colscan_kernel": 4108493, "csr_hot_finish_kernel": 1176371,
 }
 
 

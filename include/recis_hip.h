@@ -399,10 +399,12 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
  *   flags                  RECIS_PLAN_STAGE_COUNT: send the count towards the host but do not
  *                          wait; recis_unique_plan_count(stream) fetches it later (one staged
  *                          count per stream: fetch it before the next plan on that stream)
- * The unique ids are ordered by hash bucket (the top bits of a 64-bit mix of the id) and, inside a
- * bucket, by the place of the id in the bucket's hash table: the order, the inverse and row_start
- * depend on the input only; the order of the entries inside one id's list and of the hot items
- * is not specified. Ids are partitioned by hash (a histogram and a scatter pass over the ids),
+ * The unique ids are ordered as follows: first the few ids that make up a sizeable share of the
+ * batch (found by sampling; at most 64), then the ids of the hash buckets (a bucket = the top bits
+ * of a 64-bit mix of the id) that hold more than one and a half times the average, then those of
+ * the other buckets, buckets in the order of their index and, inside a bucket, ids by their place
+ * in the bucket's hash table. The order, the inverse and row_start depend on the input only; the
+ * order of the entries inside one id's list and of the hot items is not specified. Ids are partitioned by hash (a histogram and a scatter pass over the ids),
  * every bucket is deduplicated in LDS by one workgroup, and the workgroups learn where their
  * unique ids start from a look-back over one word per bucket: the only global atomics are one
  * ticket per bucket and one addition per hot id.

@@ -9,21 +9,25 @@
 // batch, so this build never scatters rows and never builds the plan with global atomics:
 // ids are partitioned by hash into buckets small enough to be deduplicated in LDS.
 //
-//   tile     a workgroup dedups tiles of 1024 ids in an LDS hash: an id repeated k times in
-//            a tile becomes ONE record {id, first position, k}; records per bucket are
-//            counted in an LDS histogram (one row per workgroup)
-//   colscan  exclusive scan of every histogram column -> where each workgroup's records of
-//            each bucket go; bucket sizes
-//   scatter  records move to their bucket (bucket = top bits of the mixed id)
-//   bucket   one workgroup per bucket: LDS hash over the bucket's records gives every unique
-//            id its first position and its count; unique ids are ranked by first position
-//            inside the bucket, counts are scanned into list offsets
-//   scan     bucket totals -> first unique index and first list entry of every bucket
-//   emit     one launch: per occurrence unique index (inverse) and list position; per unique
-//            id the id, row_start, hot work items
+//   hist     ids per (tile, column) in an LDS histogram, a tile of ids per workgroup; a column is
+//            a hash bucket (top bits of the mixed id) or, for the few ids that make up a sizeable
+//            share of the batch, a column of their own (found by sampling, see find_heavy)
+//   colscan  exclusive scan of every histogram column -> where each tile's ids of each column
+//            go; column totals
+//   scatter  (id, position) of every occurrence moves to its column; the columns are laid out
+//            heavy ids first, then the fullest buckets, then the rest (see column_starts)
+//   bucket   one workgroup per bucket, in the order of the layout: the bucket's ids are
+//            deduplicated in an LDS hash table whose final state does not depend on the order of
+//            insertion; the place of an id in the table is its rank among the bucket's unique
+//            ids; occurrences are counted and placed into their id's list; the number of unique
+//            ids of the earlier buckets comes from a decoupled look-back; every unique id is
+//            written with its list start and, with an id map, found or inserted there
+//   assign   rows for the keys that were new to the id map, in the order of the unique ids
 //
-// Unique ids come out ordered by (bucket, first occurrence): a function of the input only.
-// The order of the occurrences inside one id's list is not specified.
+// The batch may be one array or several that are tagged and concatenated by the reads themselves
+// (IdJobs). Unique ids come out ordered by (place of their column in the layout, place in the
+// bucket's table): a function of the input only. The order of the occurrences inside one id's list
+// is not specified. The consumers of the plan (gather-reduce, expansion) live in csr*.hip.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -33,7 +37,6 @@
 
 #include "common.cuh"
 #include "idmap_internal.cuh"
-#include "optim_rows.cuh"
 
 namespace recis_hip {
 namespace {
