@@ -250,8 +250,13 @@ constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of
 // says that the second input comes in parts.
 template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false, int EPI = kEpiStore,
           typename TIn2 = void>
+// Register budgets of the variants that end in a row update, found by measurement: 64 registers (8
+// waves per SIMD) where that costs no spills; 72 (7 waves, a few spilled words) for the one-input
+// kernels that hand list entries round by shuffle (config 3: 187 us with no bound and 92 registers,
+// 178 at 80, 170 at 72, 228 at 64 with 92 bytes spilled); no bound for those with two inputs (a
+// bound of 80 registers spills 24-60 bytes and costs 20 us in config 5).
 __global__ void __launch_bounds__(kBlock, (!SHUFFLE && EPI != kEpiStore && (std::is_void<TIn2>::value || sizeof(TOut) == 4))
-                                              ? 8 : 1)  // 64 registers where that costs no spills
+                                              ? 8 : (SHUFFLE && EPI != kEpiStore && std::is_void<TIn2>::value) ? 7 : 1)
 csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
   constexpr bool TWO = !std::is_void<TIn2>::value;
   using TSecond = typename std::conditional<TWO, TIn2, TIn>::type;
