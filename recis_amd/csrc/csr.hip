@@ -40,6 +40,12 @@ struct ExpArgs {
   int64_t cold_blocks;
 };
 
+// A row of zeros as long as any row (D <= 8192 of at most 4 bytes): what a unique id reads whose
+// key the table does not hold, so that the row loads need no branch around them.
+__device__ __align__(256) const unsigned char g_expand_zero_row[8192 * 4] = {};
+
+constexpr int kExpandRows = 2;  // unique rows a lane group works at a time: their loads are in flight together (4: slower)
+
 template <typename TIn, typename TOut, int VEC, bool BLK>
 __global__ void __launch_bounds__(kBlock)
 csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs a) {
@@ -119,38 +125,82 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
     return;
   }
 
-  // ---- cold rows
-  const int rows_per_block = kBlock >> a.lpr_log2;
-  const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
-  const bool valid = u < a.U && u < a.counts[0];  // U may be the caller's upper bound: the plan's own count decides
-  const int32_t start = valid ? a.row_start[u] : 0;
-  int32_t end = valid ? a.row_start[u + 1] : 0;
-  if (end - start > a.hot_len) end = start;  // written by the work items
-  const bool is_long = a.lpr_log2 < 6 && end - start > kCoopLen;
-  if (valid && !is_long && end > start) {
-    for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
-      float v[VEC];
-      load_row(u, c0, v);
-      store_list(start, end, 1, c0, v);
+  // ---- cold rows: kExpandRows of them per lane group. The kernel is a chain of dependent accesses
+  // per row (list bounds -> row index -> row -> destinations -> stores) with 16 bytes per lane in
+  // flight; with every resident wave busy that is still too little to fill the memory system, so a
+  // group walks the chain for two rows at once.
+  const int groups_per_block = kBlock >> a.lpr_log2;
+  const int64_t first = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * (kExpandRows * groups_per_block) +
+                        (threadIdx.x >> a.lpr_log2);
+  const int64_t n_unique = min(a.U, a.counts[0]);  // U may be the caller's upper bound: the plan's own count decides
+  int64_t u[kExpandRows];
+  int32_t start[kExpandRows], end[kExpandRows];
+  bool is_long[kExpandRows], is_short[kExpandRows];
+#pragma unroll
+  for (int r = 0; r < kExpandRows; ++r) {
+    u[r] = first + r * groups_per_block;
+    const bool valid = u[r] < n_unique;
+    start[r] = valid ? a.row_start[u[r]] : 0;
+    end[r] = valid ? a.row_start[u[r] + 1] : 0;
+  }
+#pragma unroll
+  for (int r = 0; r < kExpandRows; ++r) {
+    if (end[r] - start[r] > a.hot_len) end[r] = start[r];  // written by the work items
+    is_long[r] = a.lpr_log2 < 6 && end[r] - start[r] > kCoopLen;
+    is_short[r] = !is_long[r] && end[r] > start[r];
+  }
+  // short rows: where the rows lie first (no branch around a load: a missing row reads zeros), then
+  // the rows, then the stores
+  const TIn* src[kExpandRows];
+  if constexpr (BLK) {
+    int64_t ri[kExpandRows];
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r) ri[r] = is_short[r] ? a.row_index[u[r]] : -1;
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r) {
+      int64_t b = 0, off = ri[r];
+      if (a.n_blocks > 1 && ri[r] >= 0) {
+        b = ri[r] / a.block_rows;
+        off = ri[r] - b * a.block_rows;
+      }
+      const bool bad = ri[r] >= 0 && (b >= a.n_blocks || off >= a.block_rows);
+      if (bad) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      src[r] = (ri[r] >= 0 && !bad) ? static_cast<const TIn*>(a.blocks[b]) + off * D
+                                    : reinterpret_cast<const TIn*>(g_expand_zero_row);
     }
+  } else {
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r)
+      src[r] = is_short[r] ? rows + u[r] * D : reinterpret_cast<const TIn*>(g_expand_zero_row);
+  }
+  for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
+    float v[kExpandRows][VEC];
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r) load_pack_stream<TIn, VEC>(src[r] + c0, v[r]);  // every row is read once here
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r)
+      if (is_short[r]) store_list(start[r], end[r], 1, c0, v[r]);
   }
   // long rows of this wave, one after the other: the owner's row reaches every group by shuffles
-  uint64_t todo = __ballot(is_long);
-  while (todo) {
-    const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;
-    todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);
-    const int32_t r_start = __shfl(start, owner, kWave), r_end = __shfl(end, owner, kWave);
-    const int64_t row = u - g + (owner >> a.lpr_log2);  // rows of a wave are consecutive
-    for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
-      const int c0 = cbase + cl * VEC;
-      const bool col_ok = c0 < D;
-      float mine[VEC], v[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) mine[j] = 0.f;
-      if (lane >> a.lpr_log2 == owner >> a.lpr_log2 && col_ok) load_row(row, c0, mine);
+  for (int r = 0; r < kExpandRows; ++r) {
+    uint64_t todo = __ballot(is_long[r]);
+    while (todo) {
+      const int owner = __ffsll(static_cast<unsigned long long>(todo)) - 1;
+      todo &= ~(((uint64_t(1) << (1 << a.lpr_log2)) - 1) << owner);
+      const int32_t r_start = __shfl(start[r], owner, kWave), r_end = __shfl(end[r], owner, kWave);
+      const int64_t row = u[r] - g + (owner >> a.lpr_log2);  // rows of a wave are consecutive
+      for (int cbase = 0; cbase < D; cbase += VEC << a.lpr_log2) {  // uniform: shuffles inside
+        const int c0 = cbase + cl * VEC;
+        const bool col_ok = c0 < D;
+        float mine[VEC], v[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = __shfl(mine[j], owner + cl, kWave);
-      if (col_ok) store_list(r_start + g, r_end, groups, c0, v);
+        for (int j = 0; j < VEC; ++j) mine[j] = 0.f;
+        if (lane >> a.lpr_log2 == owner >> a.lpr_log2 && col_ok) load_row(row, c0, mine);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = __shfl(mine[j], owner + cl, kWave);
+        if (col_ok) store_list(r_start + g, r_end, groups, c0, v);
+      }
     }
   }
 }
@@ -428,7 +478,7 @@ int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t
   a.hot_items = hot_items;
   a.counts = counts_dev;
   a.hot_cap = hot_cap;
-  const int rows_per_block = kBlock >> a.lpr_log2;
+  const int rows_per_block = kExpandRows * (kBlock >> a.lpr_log2);
   a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
   const int64_t hot_blocks = hot_cap > 0 ? std::min<int64_t>(hot_cap, 4096) : 0;
   const dim3 grid(static_cast<unsigned>(a.cold_blocks + hot_blocks));
