@@ -189,8 +189,7 @@ class Config4:
         """The 39 id columns of the batch: the sparse ones as they are, the dense ones bucketized and
         reduced. They are tagged with their table (ids_encode) by the plan's own reads."""
         o = self.ops
-        buckets = o.fused_bucketized(self.c["dense"], self.c["boundaries"])
-        extra = o.fused_uint64_mod(buckets, self.mods)
+        extra = o.fused_bucketized(self.c["dense"], self.c["boundaries"], mods=self.mods)   # Bucketize -> Mod, one pass
         return self.c["sparse"] + extra
 
     def dedup(self, ids):
@@ -284,7 +283,7 @@ class Config4:
 
     def algorithmic_bytes(self):
         N, U, S, D = self.N, self.U, self.N, self.D
-        feat = 13 * self.c["batch"] * (4 + 8) + 13 * self.c["batch"] * (8 + 8)   # bucketize, mod (tagging: in the plan's reads)
+        feat = 13 * self.c["batch"] * (4 + 8)   # bucketize + mod in one pass (tagging: in the plan's reads)
         return {
             "feature_ops": feat,
             "dedup+lookup": N * (8 + 4) + U * 8 + U * (16 + 8),

@@ -662,6 +662,13 @@ int recis_fused_uint64_mod(const int64_t* const* in_ptrs, const int64_t* sizes,
 int recis_fused_bucketized(const float* const* in_ptrs, const int64_t* sizes,
                            const float* const* boundaries_ptrs, const int64_t* boundary_lens,
                            int64_t* const* out_ptrs, int64_t n_tensors, void* stream);
+/* recis_fused_bucketized followed by recis_fused_uint64_mod(mods) on its outputs, in one pass (a
+ * Bucketize -> Mod chain of one feature; the bucket is reduced where it is found). mods: host
+ * array, one positive modulus per tensor. */
+int recis_fused_bucketized_mod(const float* const* in_ptrs, const int64_t* sizes,
+                               const float* const* boundaries_ptrs, const int64_t* boundary_lens,
+                               const int64_t* mods, int64_t* const* out_ptrs, int64_t n_tensors,
+                               void* stream);
 int recis_fused_multi_hash(const int64_t* const* in_ptrs, const int64_t* sizes,
                            const int64_t* muls, const int64_t* primes, const int64_t* buckets,
                            int64_t* const* out_ptrs, int64_t n_jobs, void* stream);

@@ -209,7 +209,8 @@ __global__ void __launch_bounds__(kBlock) uint64_mod_kernel(Jobs j) {
 
 constexpr int kLdsBoundaries = 8192;
 
-// upper bound: number of boundaries <= v, NaN -> len (fused_bucketized.cc:5-20)
+// upper bound: number of boundaries <= v, NaN -> len (fused_bucketized.cc:5-20); with a modulus
+// (p1 != 0) the bucket is reduced at once, as a following fused_uint64_mod would
 __global__ void __launch_bounds__(kBlock) bucketize_kernel(Jobs j) {
   __shared__ float s_b[kLdsBoundaries];
   const int t = blockIdx.y;
@@ -218,6 +219,7 @@ __global__ void __launch_bounds__(kBlock) bucketize_kernel(Jobs j) {
   const float* bnd = static_cast<const float*>(j.aux[t]);
   int64_t* out = static_cast<int64_t*>(j.out[t]);
   const int32_t blen = static_cast<int32_t>(j.p0[t]);
+  const uint32_t mod = static_cast<uint32_t>(j.p1[t]);  // buckets are below 2^31: a 32-bit remainder will do
   const bool in_lds = blen <= kLdsBoundaries;
   if (in_lds) {
     for (int k = threadIdx.x; k < blen; k += kBlock) s_b[k] = bnd[k];
@@ -238,7 +240,7 @@ __global__ void __launch_bounds__(kBlock) bucketize_kernel(Jobs j) {
         count = step;
       }
     }
-    out[i] = bucket;
+    out[i] = mod ? static_cast<int64_t>(static_cast<uint32_t>(bucket) % mod) : bucket;
   }
 }
 
@@ -330,6 +332,13 @@ int recis_fused_uint64_mod(const int64_t* const* in_ptrs, const int64_t* sizes, 
 int recis_fused_bucketized(const float* const* in_ptrs, const int64_t* sizes,
                            const float* const* boundaries_ptrs, const int64_t* boundary_lens,
                            int64_t* const* out_ptrs, int64_t n_tensors, void* stream_) {
+  return recis_fused_bucketized_mod(in_ptrs, sizes, boundaries_ptrs, boundary_lens, nullptr, out_ptrs, n_tensors,
+                                    stream_);
+}
+
+int recis_fused_bucketized_mod(const float* const* in_ptrs, const int64_t* sizes,
+                               const float* const* boundaries_ptrs, const int64_t* boundary_lens,
+                               const int64_t* mods, int64_t* const* out_ptrs, int64_t n_tensors, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   RECIS_REQUIRE(n_tensors >= 0, "n_tensors must be >= 0");
   if (n_tensors == 0) return RECIS_OK;
@@ -350,6 +359,11 @@ int recis_fused_bucketized(const float* const* in_ptrs, const int64_t* sizes,
       j.size[k] = sizes[t];
       j.p0[k] = boundary_lens[t];
       j.p1[k] = j.p2[k] = 0;
+      if (mods) {
+        // a bucket is at most the number of boundaries: a modulus past 32 bits changes nothing
+        RECIS_REQUIRE(mods[t] > 0, "mod must be positive (tensor %lld)", (long long)t);
+        j.p1[k] = mods[t] > boundary_lens[t] ? 0 : mods[t];
+      }
       max_size = std::max(max_size, sizes[t]);
     }
     if (max_size == 0) continue;

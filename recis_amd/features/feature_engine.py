@@ -24,6 +24,13 @@ def _fused_bucketize(op_list, inputs):
     return [_with_values(x, o) for x, o in zip(inputs, outs)]
 
 
+def _fused_bucketize_mod(op_list, inputs):
+    """Bucketize followed by Mod of the same feature: one pass (``op_list``: (Bucketize, Mod) pairs)."""
+    outs = ops.fused_bucketized([_values(x).cuda().float() for x in inputs], [b.boundary.cuda() for b, _ in op_list],
+                                mods=[m.mod_value for _, m in op_list])
+    return [_with_values(x, o) for x, o in zip(inputs, outs)]
+
+
 def _fused_hash(op_list, inputs):
     results = [None] * len(inputs)
     for kind in ("farm", "murmur"):
@@ -52,8 +59,9 @@ def _fused_multi_hash(op_list, inputs):
     return results
 
 
+_CHAIN = "bucketize+mod"   # a Bucketize whose feature goes on with a Mod: both in one launch
 _FUSED = {Mod: _fused_mod, Bucketize: _fused_bucketize, Hash: _fused_hash, IDMultiHash: _fused_multi_hash,
-          SequenceTruncate: sequence_truncate}
+          SequenceTruncate: sequence_truncate, _CHAIN: _fused_bucketize_mod}
 
 
 class FeatureEngine(nn.Module):
@@ -78,11 +86,18 @@ class FeatureEngine(nn.Module):
         self._steps = []
         feats = list(self._features.values())
         depth = max((len(f.ops) for f in feats), default=0)
+        done_early = set()  # (feature, k): op k of the feature was applied together with op k - 1
         for k in range(depth):
             groups = defaultdict(list)
             for f in feats:
-                if k < len(f.ops):
+                if k < len(f.ops) and (f.name, k) not in done_early:
                     op = f.ops[k]
+                    nxt = f.ops[k + 1] if k + 1 < len(f.ops) else None
+                    if type(op) is Bucketize and type(nxt) is Mod and 0 < nxt.mod_value and \
+                            not (nxt._forward_hooks or nxt._forward_pre_hooks or op._forward_hooks or op._forward_pre_hooks):
+                        groups[_CHAIN].append((f.name, (op, nxt)))
+                        done_early.add((f.name, k + 1))
+                        continue
                     groups[type(op) if type(op) in _FUSED else ("single", f.name)].append((f.name, op))
             self._steps.append(groups)
 
@@ -94,7 +109,7 @@ class FeatureEngine(nn.Module):
                 names = [n for n, _ in members]
                 op_list = [op for _, op in members]
                 inputs = [state[n] if step_idx > 0 else data for n in names]
-                if key in _FUSED and len(members) > 1:
+                if key in _FUSED and (len(members) > 1 or key == _CHAIN):
                     outs = _FUSED[key](op_list, inputs)
                 else:
                     # Module.__call__ costs several microseconds of hook bookkeeping per op, which is

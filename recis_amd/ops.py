@@ -543,8 +543,9 @@ def uint64_mod(inputs, num):
     return fused_uint64_mod([inputs], [int(num)])[0].view(shape)
 
 
-def fused_bucketized(inputs, boundaries):
-    """``torch.ops.recis.fused_bucketized`` (fused_bucketized.h); the outputs are views of one buffer."""
+def fused_bucketized(inputs, boundaries, mods=None):
+    """``torch.ops.recis.fused_bucketized`` (fused_bucketized.h); the outputs are views of one buffer.
+    ``mods`` (one positive modulus per tensor): ``fused_uint64_mod`` of the buckets in the same pass."""
     require_cuda(*inputs)
     require_cuda(*boundaries)
     inputs = [_contig(t).view(-1) for t in inputs]
@@ -557,9 +558,12 @@ def fused_bucketized(inputs, boundaries):
     sizes = [t.numel() for t in inputs]
     buf = torch.empty(sum(sizes), dtype=torch.int64, device=inputs[0].device)
     outs = list(torch.split(buf, sizes))
-    check(lib().recis_fused_bucketized(_host_ptrs(inputs), _host_i64(sizes), _host_ptrs(boundaries),
-                                       _host_i64([b.numel() for b in boundaries]), _host_ptrs(outs),
-                                       i64(len(inputs)), stream_ptr(inputs[0].device)))
+    if mods is not None and len(mods) != len(inputs):
+        raise ValueError("fused_bucketized: %d mods for %d tensors" % (len(mods), len(inputs)))
+    check(lib().recis_fused_bucketized_mod(_host_ptrs(inputs), _host_i64(sizes), _host_ptrs(boundaries),
+                                           _host_i64([b.numel() for b in boundaries]),
+                                           _host_i64(mods) if mods is not None else None, _host_ptrs(outs),
+                                           i64(len(inputs)), stream_ptr(inputs[0].device)))
     return outs
 
 

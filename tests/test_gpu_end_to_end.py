@@ -529,6 +529,9 @@ def test_feature_engine_ops_and_fusion():
         Feature("h").add_op(SelectField("h")).add_op(Hash("farm")).add_op(Mod(1 << 62)),
         Feature("m").add_op(SelectField("h")).add_op(Hash("murmur")),
         Feature("mh").add_op(SelectField("a")).add_op(IDMultiHash([1000] * 4)),
+        # Bucketize -> Mod of one feature: the engine runs the pair as one launch
+        Feature("cm").add_op(SelectField("c")).add_op(Bucketize([1.0, 2, 3, 4, 5])).add_op(Mod(4)),
+        Feature("cm2").add_op(SelectField("c")).add_op(Bucketize([-1.0, 0.0, 1.0])).add_op(Mod(2)).add_op(Mod(5)),
     ]
     engine = FeatureEngine(feats)
     data = {
@@ -543,6 +546,8 @@ def test_feature_engine_ops_and_fusion():
     assert out["b"].tolist() == [(2 ** 64 - 1) % 7, 1]
     assert torch.equal(out["c"].values().cpu(), torch.bucketize(vals, torch.tensor([1.0, 2, 3, 4, 5]), right=True))
     assert torch.equal(out["d"].values().cpu(), (vals >= 0).long())
+    assert torch.equal(out["cm"].values().cpu(), torch.bucketize(vals, torch.tensor([1.0, 2, 3, 4, 5]), right=True) % 4)
+    assert torch.equal(out["cm2"].values().cpu(), torch.bucketize(vals, torch.tensor([-1.0, 0.0, 1.0]), right=True) % 2 % 5)
     farm = [-7736835464683084646, -5546720800891377920]
     assert out["h"].values().tolist() == [(f + 2 ** 64) % (1 << 62) for f in farm]
     assert out["m"].values().tolist() == [-4003751876240412087, -1042754718167355375]

@@ -80,6 +80,13 @@ def test_bucketize(rng):
     v = torch.randn(100, device="cuda") * 3
     b = torch.tensor([1.0, 2, 3, 4, 5], device="cuda")
     assert torch.equal(ops.bucketize_op(v, b), torch.bucketize(v, b, right=True))
+    # bucketize followed by mod in one pass: the oracle's two functions one after the other
+    mods = [7, 100, 1]
+    both = ops.fused_bucketized([_dev(v) for v in vs], [_dev(b) for b in bs], mods=mods)
+    for g, v, b, m in zip(both, vs, bs, mods):
+        np.testing.assert_array_equal(g.cpu().numpy(), oracle.uint64_mod(oracle.bucketize(v, b), m))
+    with pytest.raises(_lib.RecisHipError):
+        ops.fused_bucketized([_dev(vs[0])], [_dev(bs[0])], mods=[0])
 
 
 def test_multi_hash(rng):
