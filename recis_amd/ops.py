@@ -546,13 +546,13 @@ def uint64_mod(inputs, num):
 def fused_bucketized(inputs, boundaries, mods=None):
     """``torch.ops.recis.fused_bucketized`` (fused_bucketized.h); the outputs are views of one buffer.
     ``mods`` (one positive modulus per tensor): ``fused_uint64_mod`` of the buckets in the same pass."""
-    require_cuda(*inputs)
-    require_cuda(*boundaries)
-    inputs = [_contig(t).view(-1) for t in inputs]
-    boundaries = [_contig(b) for b in boundaries]
     for t in list(inputs) + list(boundaries):
         if t.dtype != torch.float32:
             raise TypeError("fused_bucketized takes float32 values and boundaries")
+        if not t.is_cuda:
+            require_cuda(t)
+    inputs = [t if (t.dim() == 1 and t.is_contiguous()) else _contig(t).view(-1) for t in inputs]
+    boundaries = [b if b.is_contiguous() else _contig(b) for b in boundaries]
     if not inputs:
         return []
     sizes = [t.numel() for t in inputs]
@@ -879,7 +879,9 @@ def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None
     ``plan.index_buf`` holds their rows."""
     jobs = None
     if isinstance(ids, (list, tuple)):
-        jobs = [_ids64(t).reshape(-1) for t in ids]
+        # (the common case, flat contiguous int64 device tensors, goes through untouched: this runs per feature per step)
+        jobs = [t if (t.dim() == 1 and t.dtype == torch.int64 and t.is_cuda and t.is_contiguous()) else _ids64(t).reshape(-1)
+                for t in ids]
         if tags is not None and len(tags) != len(jobs):
             raise ValueError("ids_unique_plan: %d tags for %d id tensors" % (len(tags), len(jobs)))
         if len(jobs) > _PLAN_JOBS or len(jobs) == 0:  # too many for one call: make the batch first
@@ -892,8 +894,7 @@ def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None
         n = ids.numel()
         dev = ids.device
     else:
-        require_cuda(*jobs)
-        n = sum(t.numel() for t in jobs)
+        n = sum([t.numel() for t in jobs])
         dev = jobs[0].device
     p = BatchPlan()
     p.serial = next(_PLAN_SERIAL)  # never reused, unlike id(p)
