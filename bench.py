@@ -711,9 +711,9 @@ class ModulePath5:
 # scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC_C4 = {
-    "csr_rows_adam_kernel": 729275494, "csr_expand_kernel": 260871885, "plan_bucket_kernel": 192791142,
-    "plan_scatter_kernel": 107226112, "plan_hist_kernel": 23857869, "uint64_mod_kernel": 13688832,
-    "bucketize_kernel": 10261094, "plan_colscan_kernel": 4108493, "csr_hot_finish_kernel": 1176371,
+    "csr_rows_adam_kernel": 729268633, "csr_expand_kernel": 258992333, "plan_bucket_kernel": 192748441,
+    "plan_scatter_kernel": 100996199, "plan_hist_kernel": 23846604, "bucketize_kernel": 10266214,
+    "plan_colscan_kernel": 4109517, "csr_hot_finish_kernel": 1177395, "plan_assign_new_kernel": 59802,
 }
 
 
