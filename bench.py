@@ -706,15 +706,25 @@ class ModulePath5:
         self.opt.zero_grad()
 
 
-# HBM bytes per launch in the config-4 step, from hardware-counter runs of this file
-# (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE, with --calib-copy): each counter is
-# scaled by what it reads for the calibration kernel that moves 1 GiB each way
+# HBM bytes per launch by workload and kernel, from hardware-counter runs of this file
+# (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE, with --workload W --calib-copy): each
+# counter is scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
-MEASURED_TRAFFIC_C4 = {
-    "csr_rows_adam_kernel": 729268633, "csr_expand_kernel": 258992333, "plan_bucket_kernel": 192748441,
-    "plan_scatter_kernel": 100996199, "plan_hist_kernel": 23846604, "bucketize_kernel": 10266214,
-    "plan_colscan_kernel": 4109517, "csr_hot_finish_kernel": 1177395, "plan_assign_new_kernel": 59802,
+MEASURED_TRAFFIC = {
+    "c4": {"csr_rows_adam_kernel": 729268633, "csr_expand_kernel": 258992333, "plan_bucket_kernel": 192748441,
+           "plan_scatter_kernel": 100996199, "plan_hist_kernel": 23846604, "bucketize_kernel": 10266214,
+           "plan_colscan_kernel": 4109517, "csr_hot_finish_kernel": 1177395, "plan_assign_new_kernel": 59802},
+    "c3": {"csr_rows_adam_kernel": 750582579, "csr_expand_kernel": 350437787, "plan_bucket_kernel": 201073766,
+           "plan_scatter_kernel": 76368896, "plan_hist_kernel": 19057766},
+    "c5": {"tile_fwd_kernel": 549501543, "csr_rows_adagrad_kernel": 769008435, "seg_pool_fwd_kernel": 93373440,
+           "block_gather_kernel": 109106995, "plan_bucket_kernel": 95251968, "plan_scatter_kernel": 59015578},
+    "c2": {"seg_pool_fwd_kernel(sum)": 4319608218, "seg_pool_bwd_kernel(sum)": 4321975296,
+           "seg_max_fwd_kernel": 4453858099, "seg_max_bwd_kernel": 4453882573},
 }
+
+
+def _measured_traffic(wl):
+    return MEASURED_TRAFFIC.get(type(wl).__name__.lower().replace("config", "c"), {})
 
 
 def checkpoint_round_trip(rows=8 << 20, dim=16, parallel=8):
@@ -782,7 +792,7 @@ def _kernel_roofline(wl, iters):
     dom = max((k for k in kern if k in kb), key=lambda k: kern[k]["us"] * kern[k]["calls_per_step"])
     ach = kb[dom] / kern[dom]["us"] / 1e3
     roof = {"bound": "hbm", "kernel": dom, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": ach / HBM_PEAK_GBS, "traffic": None, "launch_us": round(kern[dom]["us"], 2),
+            "frac": ach / HBM_PEAK_GBS, "traffic": _measured_traffic(wl).get(dom), "launch_us": round(kern[dom]["us"], 2),
             "launches_per_step": kern[dom]["calls_per_step"], "algorithmic_bytes_per_launch": kb[dom]}
     kernels_us = {k: round(v["us"], 2) for k, v in sorted(kern.items(), key=lambda kv: -kv[1]["us"])}
     kernels_gbs = {k: round(kb[k] / kern[k]["us"] / 1e3, 1) for k in kern if kb.get(k)}
@@ -885,7 +895,8 @@ def main():
         for kname, (fn, nbytes) in wl.kernels().items():
             ms = _event_ms(fn, 10)
             res[kname] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
-                          "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_launch": nbytes}
+                          "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_launch": nbytes,
+                          "traffic": _measured_traffic(wl).get(kname)}
         return res
 
     def step_summary(wl, ms, iters):
@@ -910,7 +921,7 @@ def main():
         res = c2_summary(main_wl)
         dom = max(res, key=lambda k: res[k]["ms"])
         out["roofline"] = {"bound": "hbm", "kernel": dom, "achieved": res[dom]["gbs"], "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": res[dom]["frac"], "traffic": None,
+                           "unit": "GB/s", "frac": res[dom]["frac"], "traffic": res[dom]["traffic"],
                            "launch_us": round(res[dom]["ms"] * 1e3, 2),
                            "algorithmic_bytes_per_launch": res[dom]["algorithmic_bytes_per_launch"]}
         out["stages_ms"] = {k: v["ms"] for k, v in res.items()}
@@ -919,8 +930,6 @@ def main():
         if args.workload == "c4" and not args.no_stages:
             stages = main_wl.stage_times(max(5, args.steps))
         roof, kernels_us, kernels_gbs = _kernel_roofline(main_wl, max(5, args.steps))
-        if args.workload == "c4":
-            roof["traffic"] = MEASURED_TRAFFIC_C4.get(roof["kernel"])
         out["config"]["unique_ids_per_step"] = main_wl.U
         out["roofline"] = roof
         out["kernels_us"] = kernels_us
