@@ -33,6 +33,7 @@
 #include <algorithm>
 #include <climits>
 #include <mutex>
+#include <atomic>
 #include <type_traits>
 
 #include "common.cuh"
@@ -41,8 +42,9 @@
 namespace recis_hip {
 namespace {
 
-constexpr int kTile = 8192;        // ids per workgroup of the histogram / scatter kernels (more when n is huge)
-constexpr int kPartBlock = 512;    // threads of those kernels
+constexpr int kTile = 10240;       // most ids per workgroup of the histogram / scatter kernels (more when n is huge)
+constexpr int kTileMin = 2048;     // and fewest, when the batch is small
+constexpr int kPartBlock = 1024;   // threads of those kernels
 constexpr int kMaxRows = 1024;     // workgroups of those kernels == histogram rows
 constexpr int kMinBuckets = 32;
 constexpr int kMaxBuckets = 8192;   // the histogram of a workgroup lives in LDS
@@ -639,11 +641,20 @@ plan_scatter_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, He
 
 // scatter in runs, for tiles of at most kTile ids and few enough buckets that a tile sends several
 // ids to each: a workgroup ranks its ids inside their buckets (LDS counters), orders them by bucket
-// in LDS and writes them out in that order, so that the ids a tile sends to one bucket leave
-// together as one run of consecutive words instead of one scattered 8-byte and one scattered
-// 4-byte store per id (scattered stores run at some 1e11 per second on this part whatever their
-// size).
+// in LDS (id, place in the tile, column) and writes them out in that order, so that the ids a tile
+// sends to one bucket leave together as one run of consecutive words instead of one scattered
+// 8-byte and one scattered 4-byte store per id (scattered stores run at some 1e11 per second on
+// this part whatever their size). The tile in LDS is 12 bytes per id, so a compute unit holds one
+// workgroup (a second 1024-thread workgroup does not start beside the first on this part anyway);
+// the host sizes the tiles so that a batch of up to cus * kTile ids is one round of workgroups.
+// The tile's ids are requested first and arrive while the column starts are worked out; the
+// write-out phase reads LDS only, so nothing waits for earlier stores (loads and stores share one
+// counter on this part: with a load from global memory per id in that phase, every round of it
+// waited for the stores of the round before, 11 us of a 25 us workgroup).
 constexpr int kTilePer = kTile / kPartBlock;
+constexpr size_t scatter_runs_lds(int nc) {
+  return sizeof(int32_t) * (2 * (nc + 1) + kPartBlock) + 8 + (sizeof(int64_t) + 2 * sizeof(uint16_t)) * kTile;
+}
 template <bool JOBS>
 __global__ void __launch_bounds__(kPartBlock)
 plan_scatter_runs_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, HeavyArgs hv,
@@ -661,21 +672,13 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom 
   int32_t* gbase = lds;               // [nc + 1] where the tile's ids of a column go
   int32_t* first = lds + nc + 1;      // [nc + 1] ids of the tile per column, then where they start in column order
   int32_t* partial = first + nc + 1;  // [kPartBlock] scan scratch
-  uint16_t* sorted = reinterpret_cast<uint16_t*>(partial + kPartBlock);  // [kTile] the tile's ids in column order
-  uint16_t* sorted_bucket = sorted + kTile;                              // [kTile] and their columns
-  for (int b = tid; b <= nc; b += kPartBlock) first[b] = 0;
-  const int n_heavy = load_heavy(hv.ids, hv.n, h_slot, h_key);
-  column_starts(bucket_total, nc, g.n, gbase, partial, blockIdx.x == 0 ? bucket_start : nullptr);
-  if (blockIdx.x == 0) {
-    for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
-  }
-  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nc;
-  __syncthreads();
-  for (int b = tid; b < nc; b += kPartBlock) gbase[b] += off_row[b];
+  int64_t* s_key = reinterpret_cast<int64_t*>((reinterpret_cast<uintptr_t>(partial + kPartBlock) + 7) &
+                                              ~static_cast<uintptr_t>(7));  // [kTile] the tile's ids in column order
+  uint16_t* s_at = reinterpret_cast<uint16_t*>(s_key + kTile);              // [kTile] their places in the tile
+  uint16_t* s_col = s_at + kTile;                                           // [kTile] and their columns
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile;
   const int n_here = static_cast<int>(min(g.n, lo + g.tile) - lo);
   int64_t k[kTilePer];
-  uint16_t rank[kTilePer], bucket[kTilePer];
   if (JOBS && n_here > 0) rd.seek(lo);
   const bool one_job = n_here > 0 && rd.covers(lo, lo + n_here - 1);  // the whole tile in one array (uniform)
   if (one_job) {
@@ -691,14 +694,23 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom 
       k[x] = i < n_here ? rd.at_any(lo + i) : 0;
     }
   }
+  for (int b = tid; b <= nc; b += kPartBlock) first[b] = 0;
+  const int n_heavy = load_heavy(hv.ids, hv.n, h_slot, h_key);
+  column_starts(bucket_total, nc, g.n, gbase, partial, blockIdx.x == 0 ? bucket_start : nullptr);
+  if (blockIdx.x == 0) {
+    for (int b = tid; b < nb; b += kPartBlock) agg[b] = 0;
+  }
+  const int32_t* off_row = off + static_cast<int64_t>(blockIdx.x) * nc;
+  for (int b = tid; b < nc; b += kPartBlock) gbase[b] += off_row[b];  // column_starts ended with a barrier
+  uint16_t rank[kTilePer], col[kTilePer];
 #pragma unroll
   for (int x = 0; x < kTilePer; ++x) {
     const bool valid = tid + x * kPartBlock < n_here;
-    bucket[x] = static_cast<uint16_t>(column_of(k[x], g.nb_log2, n_heavy, h_slot, h_key));
-    const bool heavy = valid && bucket[x] < kHeavyMax;
+    col[x] = static_cast<uint16_t>(column_of(k[x], g.nb_log2, n_heavy, h_slot, h_key));
+    const bool heavy = valid && col[x] < kHeavyMax;
     rank[x] = 0;
-    if (n_heavy > 0) rank[x] = static_cast<uint16_t>(wave_add_one(first, bucket[x], heavy));
-    if (valid && !heavy) rank[x] = static_cast<uint16_t>(atomicAdd(&first[bucket[x]], 1));
+    if (n_heavy > 0) rank[x] = static_cast<uint16_t>(wave_add_one(first, col[x], heavy));
+    if (valid && !heavy) rank[x] = static_cast<uint16_t>(atomicAdd(&first[col[x]], 1));
   }
   __syncthreads();
   scan_counts(first, nc, first, partial);  // counts -> starts in column order
@@ -706,37 +718,24 @@ plan_scatter_runs_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom 
   for (int x = 0; x < kTilePer; ++x) {
     const int i = tid + x * kPartBlock;
     if (i < n_here) {
-      const int j = first[bucket[x]] + rank[x];
-      sorted[j] = static_cast<uint16_t>(i);
-      sorted_bucket[j] = bucket[x];
+      const int j = first[col[x]] + rank[x];
+      s_key[j] = k[x];
+      s_at[j] = static_cast<uint16_t>(i);
+      s_col[j] = col[x];
     }
   }
   __syncthreads();
-  for (int j0 = tid; j0 < n_here; j0 += 4 * kPartBlock) {
-    int64_t key[4];
-    int i[4];
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int j = j0 + x * kPartBlock;
-      i[x] = j < n_here ? sorted[j] : 0;
-      // the tile was read a moment ago: a cache hit
-      key[x] = j >= n_here ? 0 : (one_job ? rd.raw(lo + i[x]) : rd.at_any(lo + i[x]));
-    }
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int j = j0 + x * kPartBlock;
-      if (j >= n_here) continue;
-      const int b = sorted_bucket[j];
-      const int32_t d = gbase[b] + (j - first[b]);
-      const int32_t at = static_cast<int32_t>(lo + i[x]);
-      if (b < kHeavyMax) {
-        hv.list[d] = at;
-        if (hv.inverse) hv.inverse[at] = b;
-        if (hv.pos_out) hv.pos_out[at] = d;
-      } else {
-        bkt_id[d] = key[x];
-        bkt_pos[d] = at;
-      }
+  for (int j = tid; j < n_here; j += kPartBlock) {
+    const int b = s_col[j];
+    const int32_t d = gbase[b] + (j - first[b]);
+    const int32_t at = static_cast<int32_t>(lo) + s_at[j];
+    if (b < kHeavyMax) {
+      hv.list[d] = at;
+      if (hv.inverse) hv.inverse[at] = b;
+      if (hv.pos_out) hv.pos_out[at] = d;
+    } else {
+      bkt_id[d] = s_key[j];
+      bkt_pos[d] = at;
     }
   }
 }
@@ -1431,12 +1430,31 @@ struct PlanLayout {
   size_t o_hist, o_total, o_start, o_agg, o_newc, o_sync, o_heavy, o_id, o_pos, o_new, bytes;
 };
 
+static int compute_units() {  // of the current device; asked once per device
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int v = cached[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cached[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
 static PlanLayout plan_layout(int64_t n, bool with_lookup) {
   PlanLayout L;
   PlanGeom& g = L.g;
   g.n = n;
-  g.rows = static_cast<int>(std::min<int64_t>((n + kTile - 1) / kTile, kMaxRows));
-  g.tile = static_cast<int>(((n + g.rows - 1) / g.rows + kPartBlock - 1) / kPartBlock * kPartBlock);
+  // One workgroup per compute unit is what runs at a time (see plan_scatter_runs_kernel), so the
+  // rows are as many as the device has units while that keeps a tile between kTileMin and kTile
+  // ids: a batch of up to cus * kTile ids is one round of workgroups, none left over for a
+  // second round on a few units.
+  const int64_t cus = compute_units();
+  int64_t rows = (n + kTile - 1) / kTile;
+  if (rows <= cus) rows = std::max<int64_t>(1, std::min<int64_t>(cus, n / kTileMin));
+  rows = std::min<int64_t>(rows, kMaxRows);
+  g.tile = static_cast<int>(((n + rows - 1) / rows + kPartBlock - 1) / kPartBlock * kPartBlock);
   g.rows = static_cast<int>((n + g.tile - 1) / g.tile);
   int nb_log2 = 5;
   while ((int64_t(1) << nb_log2) < kMaxBuckets && (int64_t(1) << nb_log2) * kBucketIds < n) ++nb_log2;
@@ -1534,7 +1552,17 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, cons
     const dim3 grid(g.rows), block(kPartBlock);
     RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
     if (g.tile <= kTile && g.tile >= 4 * nb) {  // a tile sends four ids or more to a bucket: worth ordering them
-      const size_t runs_lds = sizeof(int32_t) * (2 * (nc + 1) + kPartBlock) + 2 * sizeof(uint16_t) * kTile;
+      const size_t runs_lds = scatter_runs_lds(nc);
+      static std::atomic<bool> lds_allowed{false};  // more than the 64 KB a kernel may take unasked
+      if (!lds_allowed.load(std::memory_order_acquire)) {
+        RECIS_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&plan_scatter_runs_kernel<true>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            static_cast<int>(scatter_runs_lds(kHeavyMax + kTile / 4))));
+        RECIS_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&plan_scatter_runs_kernel<false>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            static_cast<int>(scatter_runs_lds(kHeavyMax + kTile / 4))));
+        lds_allowed.store(true, std::memory_order_release);
+      }
       if (by_jobs)
         plan_scatter_runs_kernel<true><<<grid, block, runs_lds, stream>>>(ids, jobs, g, hv, hist, bucket_total,
                                                                          bucket_start, agg, bkt_id, bkt_pos);
