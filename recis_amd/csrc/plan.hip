@@ -45,6 +45,7 @@ namespace {
 constexpr int kTile = 10240;       // most ids per workgroup of the histogram / scatter kernels (more when n is huge)
 constexpr int kTileMin = 2048;     // and fewest, when the batch is small
 constexpr int kPartBlock = 1024;   // threads of those kernels
+constexpr int kTilePer = kTile / kPartBlock;  // ids of a tile of at most kTile per thread
 constexpr int kMaxRows = 1024;     // workgroups of those kernels == histogram rows
 constexpr int kMinBuckets = 32;
 constexpr int kMaxBuckets = 8192;   // the histogram of a workgroup lives in LDS
@@ -112,9 +113,11 @@ __device__ __forceinline__ void load_jobs(const IdJobs& J, JobTable& t) {
   if constexpr (JOBS) {
     const IdJobs* in_memory = reinterpret_cast<const IdJobs*>(
         reinterpret_cast<uintptr_t>(__builtin_amdgcn_kernarg_segment_ptr()) + kJobsArgOffset);
-    for (int k = threadIdx.x; k <= J.n_jobs; k += blockDim.x) {
+    // the whole table, used or not: the loads go out without waiting for n_jobs
+    const int k = threadIdx.x;
+    if (k <= kPlanJobs) {
       t.first[k] = in_memory->first[k];
-      if (k < J.n_jobs) {
+      if (k < kPlanJobs) {
         t.in[k] = in_memory->in[k];
         t.tag[k] = in_memory->tag[k];
       }
@@ -395,6 +398,28 @@ plan_hist_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, int64
     if (tid < 2) counts[tid] = 0;
     if (tid < 4) sync[tid] = 0;  // [1] finished workgroups of the bucket kernel, [2] of the row assignment, [3] new keys
   }
+  // the first kTile ids of the tile (all of it unless the batch is huge) are requested now and
+  // arrive while the heavy ids are looked for
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
+  const int64_t hi_regs = min(hi, lo + kTile);
+  int64_t k_first[kTilePer];
+  {
+    IdReader<JOBS> rt = rd;
+    if (JOBS && lo < hi_regs) rt.seek(lo);
+    if (lo < hi_regs && rt.covers(lo, hi_regs - 1)) {  // the whole stretch in one array (uniform)
+#pragma unroll
+      for (int x = 0; x < kTilePer; ++x) {
+        const int64_t i = lo + tid + x * kPartBlock;
+        k_first[x] = i < hi_regs ? rt.raw(i) : 0;
+      }
+    } else {
+#pragma unroll
+      for (int x = 0; x < kTilePer; ++x) {
+        const int64_t i = lo + tid + x * kPartBlock;
+        k_first[x] = i < hi_regs ? rt.at_any(i) : 0;
+      }
+    }
+  }
   const int n_found = find_heavy<JOBS>(rd, g.n, *reinterpret_cast<HeavyScratch*>(l_raw), h_ids);
   if (blockIdx.x == 0) {
     if (tid < n_found) heavy_ids[tid] = h_ids[tid];
@@ -403,9 +428,16 @@ plan_hist_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, int64
   for (int b = tid; b < nc; b += kPartBlock) l_hist[b] = 0;
   const int n_heavy = heavy_table(h_ids, n_found, h_slot, h_key);
   __syncthreads();
-  const int64_t lo = static_cast<int64_t>(blockIdx.x) * g.tile, hi = min(g.n, lo + g.tile);
-  if (JOBS && lo + tid < hi) rd.seek(lo + tid);
-  for (int64_t i0 = lo + tid; i0 < hi; i0 += 4 * kPartBlock) {  // four loads in flight
+  auto count = [&](int64_t key, bool valid) {
+    const int c = column_of(key, g.nb_log2, n_heavy, h_slot, h_key);
+    const bool heavy = valid && c < kHeavyMax;
+    if (n_heavy > 0) wave_count_one(l_hist, c, heavy);  // a heavy id is many lanes on one word
+    if (valid && !heavy) atomicAdd(&l_hist[c], 1);
+  };
+#pragma unroll
+  for (int x = 0; x < kTilePer; ++x) count(k_first[x], lo + tid + x * kPartBlock < hi_regs);
+  if (JOBS && hi_regs + tid < hi) rd.seek(hi_regs + tid);
+  for (int64_t i0 = hi_regs + tid; i0 < hi; i0 += 4 * kPartBlock) {  // four loads in flight
     int64_t k[4];
     if (rd.covers(i0, min(hi - 1, i0 + 3 * kPartBlock))) {
 #pragma unroll
@@ -421,13 +453,7 @@ plan_hist_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, int64
       }
     }
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const bool valid = i0 + x * kPartBlock < hi;
-      const int c = column_of(k[x], g.nb_log2, n_heavy, h_slot, h_key);
-      const bool heavy = valid && c < kHeavyMax;
-      if (n_heavy > 0) wave_count_one(l_hist, c, heavy);  // a heavy id is many lanes on one word
-      if (valid && !heavy) atomicAdd(&l_hist[c], 1);
-    }
+    for (int x = 0; x < 4; ++x) count(k[x], i0 + x * kPartBlock < hi);
   }
   __syncthreads();
   int32_t* row = hist + static_cast<int64_t>(blockIdx.x) * nc;
@@ -651,7 +677,6 @@ plan_scatter_kernel(const int64_t* __restrict__ ids, IdJobs jobs, PlanGeom g, He
 // write-out phase reads LDS only, so nothing waits for earlier stores (loads and stores share one
 // counter on this part: with a load from global memory per id in that phase, every round of it
 // waited for the stores of the round before, 11 us of a 25 us workgroup).
-constexpr int kTilePer = kTile / kPartBlock;
 constexpr size_t scatter_runs_lds(int nc) {
   return sizeof(int32_t) * (2 * (nc + 1) + kPartBlock) + 8 + (sizeof(int64_t) + 2 * sizeof(uint16_t)) * kTile;
 }
