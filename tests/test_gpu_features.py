@@ -237,11 +237,14 @@ def _check_plan(ids):
 
 
 @pytest.mark.parametrize("n,hi", [(0, 10), (1, 10), (1000, 50), (1025, 10**6), (300000, 40), (200000, 3000),
-                                  (1000000, 10**7), (3000000, 10**12), (8000000, 10**12)])
+                                  (1000000, 10**7), (3000000, 10**12), (8000000, 10**12),
+                                  (2047, 10**6), (2049, 10**6), (4097, 20), (256 * 10240 - 1, 300),
+                                  (256 * 10240, 10**12), (256 * 10240 + 1, 10**12)])
 def test_unique_plan_lists(rng, n, hi):
     """Random ids from hot (tens of thousands of repeats of each id) to nearly all distinct (the
     largest case has more distinct ids per hash bucket than one LDS table takes: several rounds),
-    the id that equals the library's empty marker included."""
+    the id that equals the library's empty marker included. The last cases sit on the edges of the
+    partition's geometry: the smallest tile, and one tile of the largest size per compute unit."""
     ids = rng.integers(-hi, hi, size=n)
     if n > 5:
         ids[3] = -1
