@@ -432,10 +432,12 @@ class Config3:
         self.U = plan.U
         index = self.table.settle_lookup(plan.index_buf, self.U, plan)
         chunks, chunk_rows = self.table.emb_blocks()
-        self.table.update_slot("step_filter", index, self.step_t)
         # one row per lookup: every unique row is read once out of the table and written to its
-        # occurrences (no [U, D] copy, no second pass over it)
-        out = o.plan_expand_rows(plan, self.N, blocks=chunks, block_size=chunk_rows, row_index=index)
+        # occurrences (no [U, D] copy, no second pass over it); the step filter's stamps of the
+        # rows go out in the same pass
+        stamps = self.table.slot_blocks("step_filter")[0]
+        out = o.plan_expand_rows(plan, self.N, blocks=chunks, block_size=chunk_rows, row_index=index,
+                                 stamp=(stamps, self.step_t))
         # the per-lookup gradients reduced per key and applied to the row in the same launch
         self.opt.apply_planned(self.table, plan, self.grad_out, plan.occ, None, index, cover=self.span)
         self.step_t += 1

@@ -637,6 +637,21 @@ int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t
                           const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
                           const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
                           int64_t n_out, int64_t D, void* stream);
+/*
+ * The same for a table with a step filter, rows from a block list only: every row that is read
+ * (row_index[u] >= 0) also gets stamp_value_dev[0] written at that row of an int64 slot of the
+ * same table (stamp_blocks_dev: its blocks, of block_rows rows like the embedding's), which is
+ * what the filter hook's update does after a training lookup
+ * (recis/nn/modules/hashtable_hook_impl.py:389-426: update_slot(name, index, global_step)): the
+ * stamps ride on the pass that reads the rows anyway instead of taking a launch of their own.
+ */
+int recis_csr_expand_rows_stamped(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks,
+                                  int64_t block_rows, const int64_t* row_index, int rows_dtype,
+                                  const void* weight, int weight_dtype, const int32_t* row_start,
+                                  const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
+                                  const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
+                                  int64_t n_out, int64_t D, void* const* stamp_blocks_dev,
+                                  const int64_t* stamp_value_dev, void* stream);
 
 /* ------------------------------------------------------------------------- *
  * Feature-engine scalar ops (lists as HOST arrays of device pointers)

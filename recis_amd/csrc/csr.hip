@@ -38,6 +38,10 @@ struct ExpArgs {
   const int64_t* counts;
   int64_t hot_cap;
   int64_t cold_blocks;
+  // rows in a block list only: every row that is read also gets *stamp_value written into an
+  // int64 slot of the same table (same blocks of block_rows rows), or NULL
+  void* const* stamp_blocks;
+  const int64_t* stamp_value;
 };
 
 // A row of zeros as long as any row (D <= 8192 of at most 4 bytes): what a unique id reads whose
@@ -55,7 +59,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
   const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
   const int g = lane >> a.lpr_log2;        // this lane's group in its wave
 
-  auto load_row = [&](int64_t u, int c0, float (&v)[VEC]) {
+  auto load_row = [&](int64_t u, int c0, float (&v)[VEC], bool stamp_here) {
     const TIn* src = nullptr;
     if constexpr (BLK) {
       const int64_t ri = a.row_index[u];
@@ -65,10 +69,12 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
           b = ri / a.block_rows;
           r = ri - b * a.block_rows;
         }
-        if (b >= a.n_blocks || r >= a.block_rows)
+        if (b >= a.n_blocks || r >= a.block_rows) {
           raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-        else
+        } else {
           src = static_cast<const TIn*>(a.blocks[b]) + r * D;
+          if (a.stamp_blocks && c0 == 0 && stamp_here) static_cast<int64_t*>(a.stamp_blocks[b])[r] = a.stamp_value[0];
+        }
       }
     } else {
       src = rows + u * D;
@@ -118,7 +124,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
       const int32_t end = min(a.row_start[u + 1], start + kHotChunk);
       for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
         float v[VEC];
-        load_row(u, c0, v);
+        load_row(u, c0, v, chunk == 0 && gb == 0);  // a hot row is stamped once: by its first work item
         store_list(start + gb, end, groups_per_block, c0, v);
       }
     }
@@ -167,6 +173,8 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
       if (bad) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
       src[r] = (ri[r] >= 0 && !bad) ? static_cast<const TIn*>(a.blocks[b]) + off * D
                                     : reinterpret_cast<const TIn*>(g_expand_zero_row);
+      if (a.stamp_blocks && cl == 0 && ri[r] >= 0 && !bad)
+        static_cast<int64_t*>(a.stamp_blocks[b])[off] = a.stamp_value[0];
     }
   } else {
 #pragma unroll
@@ -196,7 +204,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
         float mine[VEC], v[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; ++j) mine[j] = 0.f;
-        if (lane >> a.lpr_log2 == owner >> a.lpr_log2 && col_ok) load_row(row, c0, mine);
+        if (lane >> a.lpr_log2 == owner >> a.lpr_log2 && col_ok) load_row(row, c0, mine, true);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = __shfl(mine[j], owner + cl, kWave);
         if (col_ok) store_list(r_start + g, r_end, groups, c0, v);
@@ -474,7 +482,20 @@ int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t
                           const int32_t* row_start, const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
                           const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t n_out, int64_t D,
                           void* stream_) {
+  return recis_csr_expand_rows_stamped(rows, emb_blocks_dev, n_blocks, block_rows, row_index, rows_dtype, weight,
+                                       weight_dtype, row_start, dst, hot_items, hot_cap, counts_dev, out, out_dtype, U,
+                                       n_out, D, nullptr, nullptr, stream_);
+}
+
+int recis_csr_expand_rows_stamped(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows,
+                                  const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
+                                  const int32_t* row_start, const int32_t* dst, const int32_t* hot_items,
+                                  int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
+                                  int64_t n_out, int64_t D, void* const* stamp_blocks_dev,
+                                  const int64_t* stamp_value_dev, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  RECIS_REQUIRE((stamp_blocks_dev == nullptr) == (stamp_value_dev == nullptr), "stamp blocks and stamp value go together");
+  RECIS_REQUIRE(stamp_blocks_dev == nullptr || emb_blocks_dev != nullptr, "rows are stamped in a block list only");
   RECIS_REQUIRE(U >= 0 && n_out >= 0, "negative size");
   RECIS_REQUIRE(D >= 1 && D <= 8192, "embedding dim %lld out of range", (long long)D);
   if (U == 0 || n_out == 0) return RECIS_OK;
@@ -509,6 +530,8 @@ int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t
   a.hot_items = hot_items;
   a.counts = counts_dev;
   a.hot_cap = hot_cap;
+  a.stamp_blocks = stamp_blocks_dev;
+  a.stamp_value = stamp_value_dev;
   const int rows_per_block = kExpandRows * (kBlock >> a.lpr_log2);
   a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
   const int64_t hot_blocks = hot_cap > 0 ? std::min<int64_t>(hot_cap, 4096) : 0;

@@ -221,14 +221,16 @@ __global__ void __launch_bounds__(kBlock) bucketize_kernel(Jobs j) {
   const int32_t blen = static_cast<int32_t>(j.p0[t]);
   const uint32_t mod = static_cast<uint32_t>(j.p1[t]);  // buckets are below 2^31: a 32-bit remainder will do
   const bool in_lds = blen <= kLdsBoundaries;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+  const int64_t i_first = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  const float v_first = i_first < n ? in[i_first] : 0.f;  // on its way while the boundaries are staged
   if (in_lds) {
     for (int k = threadIdx.x; k < blen; k += kBlock) s_b[k] = bnd[k];
     __syncthreads();
   }
   const float* b = in_lds ? s_b : bnd;
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) {
-    const float v = in[i];
+  for (int64_t i = i_first; i < n; i += stride) {
+    const float v = i == i_first ? v_first : in[i];
     int32_t bucket = 0, count = blen;
     while (count > 0) {
       const int32_t step = count >> 1;

@@ -1578,7 +1578,10 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, cons
     RECIS_TIME_KERNEL("plan_scatter_kernel", stream)
     if (g.tile <= kTile && g.tile >= 4 * nb) {  // a tile sends four ids or more to a bucket: worth ordering them
       const size_t runs_lds = scatter_runs_lds(nc);
-      static std::atomic<bool> lds_allowed{false};  // more than the 64 KB a kernel may take unasked
+      static std::atomic<bool> lds_allowed_on[64];  // more than the 64 KB a kernel may take unasked; per device
+      int dev = 0;
+      RECIS_CHECK_HIP(hipGetDevice(&dev));
+      std::atomic<bool>& lds_allowed = lds_allowed_on[dev & 63];
       if (!lds_allowed.load(std::memory_order_acquire)) {
         RECIS_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&plan_scatter_runs_kernel<true>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -389,6 +389,10 @@ class HashtableImpl:
         (no read-back of the allocator state)."""
         return self._slot_group.emb_slot().kernel_blocks()
 
+    def slot_blocks(self, name):
+        """The same for the slot ``name``."""
+        return self._slot_group.slot_by_name(name).kernel_blocks()
+
     def lookup_index_counted(self, plan):
         """Queue the find-or-insert of a plan's unique ids before the host knows how many
         there are; finish with ``settle_lookup`` once ``plan.U`` has been read."""
@@ -759,14 +763,18 @@ class LookupExpandFunction(torch.autograd.Function):
     occurrences. Backward: sum over the duplicates of each id, divided by the number of workers."""
 
     @staticmethod
-    def forward(ctx, backward_holder, impl, plan, slice_num, readonly):
+    def forward(ctx, backward_holder, impl, plan, slice_num, readonly, stamp=None):
+        """``stamp`` = (name of the step filter's slot, its one-element step tensor): the rows read
+        are stamped in the same pass (what the filter hook's update would do in a launch of its own)."""
         if readonly:
             index = impl.lookup_index(plan.unique, True)
         else:
             index_buf = impl.lookup_index_counted(plan)   # queued before the host has the unique count
             index = impl.settle_lookup(index_buf, plan.U, plan)
         chunks, chunk_rows = impl.emb_blocks()
-        out = ops.plan_expand_rows(plan, plan.n, blocks=chunks, block_size=chunk_rows, row_index=index)
+        if stamp is not None:   # the slot's blocks as they are now, after the lookup may have grown the table
+            stamp = (impl.slot_blocks(stamp[0])[0], stamp[1])
+        out = ops.plan_expand_rows(plan, plan.n, blocks=chunks, block_size=chunk_rows, row_index=index, stamp=stamp)
         ctx.impl, ctx.plan, ctx.slice_num, ctx.readonly = impl, plan, slice_num, readonly
         ctx.save_for_backward(index)
         ctx.mark_non_differentiable(index)
@@ -782,7 +790,7 @@ class LookupExpandFunction(torch.autograd.Function):
         # the sum over the duplicates of each id is left to the optimizer step where it can be (one launch
         # sums and updates the row); keys the table does not hold (negative index) take no gradient
         ctx.impl.accept_planned_grad(index, ctx.plan, flat, ctx.plan.occ, may_miss=ctx.readonly)
-        return None, None, None, None, None
+        return None, None, None, None, None, None
 
 
 def _scatter_sum(grad_rows, index, unique_size, plan=None):
@@ -869,9 +877,12 @@ class HashTable(torch.nn.Module):
             assert admit_hook_impl is None or isinstance(admit_hook_impl, ReadOnlyHookImpl), \
                 "admit hook only support ReadOnlyHook yet, but got: %s" % admit_hook_impl
             plan = ops.ids_unique_plan(ids, wait=False, need_pos=False)
+            # a step filter's stamps ride on the pass that reads the rows
+            stamp = getattr(self._filter_hook_impl, "stamp_target", lambda: None)()
             emb_idx, embedding = LookupExpandFunction.apply(self._backward_holder, self._hashtable_impl, plan,
-                                                            self._worker_num, admit_hook_impl is not None)
-            self._filter_hook_impl(emb_idx)
+                                                            self._worker_num, admit_hook_impl is not None, stamp)
+            if stamp is None:
+                self._filter_hook_impl(emb_idx)
             return embedding.view(shape + tuple(embedding.shape[1:])) if len(shape) != 1 else embedding
         uids, index, plan = self._unique(ids)
         if self.training and self._dtype not in (torch.int8, torch.int32, torch.int64):

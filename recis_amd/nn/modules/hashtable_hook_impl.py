@@ -102,6 +102,11 @@ class GlobalStepFilterHookImpl(BaseFilterHookImpl):
     def update(self, index: torch.Tensor) -> None:
         self._ht.update_slot(self._name, index, self._global_step)
 
+    def stamp_target(self):
+        """(slot name, step tensor) for a lookup that can write the stamps itself, in the pass that
+        reads the rows (``ops.plan_expand_rows(stamp=...)``): the same stores as ``update``."""
+        return self._name, self._global_step
+
     def update_step(self, step_size: int = 1) -> None:
         with torch.no_grad():
             self._global_step += step_size

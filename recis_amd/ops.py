@@ -1137,10 +1137,13 @@ def csr_gather_reduce2_adagrad(plan, first, second, row_index, emb_blocks, accum
         i64(block_size), dtype_code(b0.dtype), ctypes.c_double(lr), ctypes.c_double(eps), stream_ptr(dev)))
 
 
-def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_index=None, weight=None, out_dtype=None):
+def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_index=None, weight=None, out_dtype=None,
+                     stamp=None):
     """``out[i] = weight[i] * row(unique id of occurrence i)`` for the ``n_out`` occurrences of
     ``plan``: every unique row is read once and written to all its occurrences. Rows come from
-    ``rows`` ``[U, D]`` or from ``blocks`` (row u = row ``row_index[u]``, negative = zeros)."""
+    ``rows`` ``[U, D]`` or from ``blocks`` (row u = row ``row_index[u]``, negative = zeros).
+    ``stamp`` = (blocks of an int64 slot of the same table, a one-element int64 device tensor):
+    every row that is read also gets that value written into the slot (the step filter's stamp)."""
     if blocks is not None:
         require_cuda(row_index, weight)
         table, dt, D, dev = block_ptr_table(blocks), blocks[0].dtype, blocks[0][0].numel(), blocks[0].device
@@ -1149,13 +1152,26 @@ def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_inde
         require_cuda(rows, weight)
         rows = _contig(rows)
         table, dt, D, dev, n_blocks, rows_arg = None, rows.dtype, rows.shape[1], rows.device, 0, rows
+    stamp_table = stamp_value = None
+    if stamp is not None:
+        stamp_blocks, stamp_value = stamp
+        if blocks is None:
+            raise ValueError("rows are stamped in a block list only")
+        if (len(stamp_blocks) != n_blocks or stamp_blocks[0].dtype != torch.int64
+                or stamp_blocks[0].numel() != blocks[0].shape[0]):
+            raise ValueError("the stamp slot must be an int64 slot with the blocks of the embedding's table")
+        if stamp_value.dtype != torch.int64 or stamp_value.numel() != 1:
+            raise TypeError("the stamp value must be a one-element int64 tensor")
+        require_cuda(stamp_value)
+        stamp_table = block_ptr_table(stamp_blocks)
     out = torch.empty((n_out, D), dtype=out_dtype or dt, device=dev)
     weight = _contig(weight)
-    check(lib().recis_csr_expand_rows(ptr(rows_arg), ptr(table), i64(n_blocks), i64(block_size), ptr(row_index),
-                                      dtype_code(dt), ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
-                                      ptr(plan.row_start), ptr(plan.occ), ptr(plan.hot_items), i64(plan.hot_cap),
-                                      ptr(plan.counts), ptr(out), dtype_code(out.dtype), i64(plan.U_bound()),
-                                      i64(n_out), i64(D), stream_ptr(dev)))
+    check(lib().recis_csr_expand_rows_stamped(ptr(rows_arg), ptr(table), i64(n_blocks), i64(block_size), ptr(row_index),
+                                              dtype_code(dt), ptr(weight),
+                                              dtype_code(weight.dtype) if weight is not None else 0,
+                                              ptr(plan.row_start), ptr(plan.occ), ptr(plan.hot_items), i64(plan.hot_cap),
+                                              ptr(plan.counts), ptr(out), dtype_code(out.dtype), i64(plan.U_bound()),
+                                              i64(n_out), i64(D), ptr(stamp_table), ptr(stamp_value), stream_ptr(dev)))
     return out
 
 

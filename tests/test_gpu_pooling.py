@@ -411,6 +411,19 @@ def test_expand_rows_equals_pooling_of_unit_segments(dtype, D):
     exp = ops.segment_reduce_forward_blocks(blocks, bs, index, None, plan.inverse, offsets, "mean")
     got = ops.plan_expand_rows(plan, n, blocks=blocks, block_size=bs, row_index=index)
     assert torch.equal(got, exp)
+    # with the step filter's stamps written in the same pass: the rows that are read, and only
+    # those, carry the new step; the output is the same
+    stamps = [torch.full((bs, 1), -5, dtype=torch.int64, device="cuda") for _ in range(nb)]
+    step = torch.tensor([41], dtype=torch.int64, device="cuda")
+    got = ops.plan_expand_rows(plan, n, blocks=blocks, block_size=bs, row_index=index, stamp=(stamps, step))
+    assert torch.equal(got, exp)
+    want = [torch.full((bs, 1), -5, dtype=torch.int64, device="cuda") for _ in range(nb)]
+    ops.block_insert(index[index >= 0], step.expand(int((index >= 0).sum()), 1).contiguous(), want, bs)
+    for a, b in zip(stamps, want):
+        assert torch.equal(a, b)
+    assert int(sum((b == 41).sum() for b in stamps)) == int((index >= 0).sum())
+    with pytest.raises(ValueError):
+        ops.plan_expand_rows(plan, n, rows=rows, stamp=(stamps, step))
     assert _lib.poll_device_errors() == 0
 
 
