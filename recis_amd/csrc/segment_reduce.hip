@@ -252,6 +252,7 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
   const float scale = (a.mean && seg_len > 0) ? 1.0f / static_cast<float>(seg_len) : 1.0f;
 
   const TIn* zero_row = reinterpret_cast<const TIn*>(g_zero_row);
+  const int64_t zero_at = BLK ? 0 : zero_row - emb;
   // rows read once, or too many to stay cached: streaming loads (picked here, outside the loops)
   const bool nt = (KIND == kFastPlain && !BLK) || a.nt_in;
   for (int cbase = 0; cbase < D; cbase += col_stride) {  // uniform: every lane takes part in the shuffles
@@ -299,8 +300,10 @@ seg_pool_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, Se
               const uint64_t addr = (static_cast<uint64_t>(hi) << 32) | lo;
               row = (want && addr != 0) ? reinterpret_cast<const TIn*>(addr) + c0 : zero_row;
             } else {
+              // (the row of zeros as an offset from emb: one global pointer for every load; a choice
+              // between two pointers makes the loads generic ones)
               const int32_t id = __shfl(mine, from, kWave);
-              row = (want && id >= 0) ? emb + static_cast<int64_t>(id) * D + c0 : zero_row;
+              row = emb + ((want && id >= 0) ? static_cast<int64_t>(id) * D + c0 : zero_at);
             }
             load_row_pack<TIn, VEC, NT>(row, v[k]);
           }
@@ -450,21 +453,24 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
     const bool col_ok = c0 < D;
     // Inside a lane the occurrences come in ascending order, so a strict float comparison keeps
     // the first of equal values (-0 == +0) and costs less than building a key per element. The
-    // running best starts as NaN so that the first row always wins; the first NaN of the data
-    // wins over every number and is kept from then on. (Scanning without the NaN flags first and
-    // again with them only when a segment holds a NaN halves the arithmetic and was measured: no
-    // faster. The kernel waits on memory, not on the vector units.)
+    // running best starts at -inf with no row; the first NaN of the data wins over every number
+    // and is kept from then on (nothing is taken once the best is a NaN). A lane whose values are
+    // all -inf never takes one: its first row is put in afterwards. No arrays of bool in here:
+    // those live in vector registers as bytes, and the selects and tests that go with them were
+    // two thirds of the loop's instructions (the vector units, not the memory, then set the pace:
+    // 3.4e8 vector instructions per launch of the 16 M row workload, 0.64 ms of SIMD time).
     float best_v[VEC];
     int32_t best_r[VEC];
     auto scan_rows = [&](auto nt_tag) {
       constexpr bool NT = decltype(nt_tag)::value;
-      bool nan_seen[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        best_v[j] = __uint_as_float(0x7FC00000u);
+        best_v[j] = -__builtin_huge_valf();
         best_r[j] = -1;
-        nan_seen[j] = false;
       }
+      // the row of zeros as an offset from emb, so that every load goes through the one global
+      // pointer (see the sum kernel)
+      const int64_t zero_at = zero_row - emb;
       for (int64_t base = start; base < end; base += team) {
         const int n_here = static_cast<int>(min(static_cast<int64_t>(team), end - base));
         int32_t mine = -1;  // row of occurrence base + lane_t
@@ -486,14 +492,14 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
         constexpr int kFly = 4;  // row loads in flight per lane (8 was measured: slower, fewer resident waves)
         for (int q0 = 0; q0 < n_here; q0 += kFly * step) {  // same trip count for the whole team
           float v[kFly][VEC];
-          bool have[kFly];
+          int32_t id[kFly];  // -1: nothing to read (a row of zeros is loaded and not looked at)
 #pragma unroll
           for (int k = 0; k < kFly; ++k) {  // no branches in here: see g_zero_row
             const int src = q0 + rg + k * step;
-            const int32_t id = __shfl(mine, (team_lane0 + src) & (kWave - 1), kWave);
-            have[k] = src < n_here && col_ok && id >= 0;
-            const TIn* row = have[k] ? emb + static_cast<int64_t>(id) * D + c0 : zero_row;
-            load_row_pack<TIn, VEC, NT>(row, v[k]);
+            const int32_t got = __shfl(mine, (team_lane0 + src) & (kWave - 1), kWave);
+            id[k] = (src < n_here && col_ok) ? got : -1;
+            const int64_t at = id[k] >= 0 ? static_cast<int64_t>(id[k]) * D + c0 : zero_at;
+            load_row_pack<TIn, VEC, NT>(emb + at, v[k]);
           }
 #pragma unroll
           for (int k = 0; k < kFly; ++k) {
@@ -501,9 +507,8 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
               const float x = v[k][j];
-              // & and |, not && and ||: no branches (the values are all at hand)
-              const bool take = have[k] & !(x <= best_v[j]) & !nan_seen[j];
-              nan_seen[j] = nan_seen[j] | (have[k] & (x != x));
+              // & not &&: no branches (the values are all at hand)
+              const bool take = (id[k] >= 0) & !(x <= best_v[j]) & (best_v[j] == best_v[j]);
               best_v[j] = take ? x : best_v[j];
               best_r[j] = take ? r : best_r[j];
             }
@@ -516,9 +521,14 @@ seg_max_fwd_fast_kernel(const TIn* __restrict__ emb, TOut* __restrict__ out, int
     } else {
       scan_rows(std::false_type{});
     }
+    // a lane that read rows and took none (all -inf): its first row holds the first -inf
+    const int64_t lane_first = start + rg;
     uint64_t key[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) key[j] = best_r[j] >= 0 ? max_key(best_v[j], best_r[j]) : 0;
+    for (int j = 0; j < VEC; ++j) {
+      if (best_r[j] < 0 && lane_first < end && col_ok) best_r[j] = static_cast<int32_t>(lane_first);
+      key[j] = best_r[j] >= 0 ? max_key(best_v[j], best_r[j]) : 0;
+    }
     for (int off = 1 << a.lpr_log2; off < team; off <<= 1) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
