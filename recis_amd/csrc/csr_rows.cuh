@@ -159,6 +159,12 @@ __device__ __forceinline__ void fused_row_update_at(const FuseArgs& f, const Row
   }
 }
 
+// A row of zeros as long as any row (D <= 8192 of at most 4 bytes): what a list entry reads that
+// has nothing to add (outside the cover, past the end of a round), so that the gathers need no
+// branch around a load. With a branch around each load the compiler waits for the loads in flight
+// before the next one goes out, and the gathers of a round run one after the other.
+__device__ __align__(256) const unsigned char g_csr_zero_row[8192 * 4] = {};
+
 // One input as a kernel sees it: entries whose src lies outside [lo, hi) are skipped, those at or
 // past n_rows raise the index-range error.
 template <typename T>
@@ -205,12 +211,15 @@ __device__ __forceinline__ void cover_range(const CsrArgs& a, int64_t& lo, int64
 // that gather the rows through shuffles; lane group g of `groups` takes entries g, g + groups,
 // ... with several row loads in flight. acc: this group's partial sum for columns
 // c0 .. c0 + VEC (the caller folds the groups).
-template <typename TIn, int VEC, bool PARTS>
-__device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const CsrArgs& a, int32_t e_begin,
-                                                  int32_t e_end, int c0, bool col_ok, int g, int groups,
-                                                  float (&acc)[VEC]) {
-  constexpr int kFly = VEC >= 8 ? 4 : 8;  // row loads in flight per lane
+template <typename TIn, int VEC, bool PARTS, bool NT>
+__device__ __forceinline__ void wave_gather_range_nt(const SrcView<TIn>& s, const CsrArgs& a, int32_t e_begin,
+                                                     int32_t e_end, int c0, bool col_ok, int g, int groups,
+                                                     float (&acc)[VEC]) {
+  constexpr int kFly = 4;  // row loads in flight per lane, all of them at once (no branches below)
   const int lane = threadIdx.x & (kWave - 1);
+  const TIn* zero_row = reinterpret_cast<const TIn*>(g_csr_zero_row);
+  const int64_t zero_at = PARTS ? 0 : zero_row - s.rows;  // the row of zeros as an offset from the input
+  bool beyond = false;
   for (int32_t cb = e_begin; cb < e_end; cb += kWave) {
     const int n_here = min(kWave, e_end - cb);
     // the row this lane's entry reads (none: -1 / NULL). With parts, where it lies is worked out once
@@ -224,40 +233,39 @@ __device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const C
         s_mine = sv;
         if constexpr (PARTS) p_mine = src_row<TIn, true>(s.rows, a, sv);
         w_mine = s.coef ? load_coef(s.coef, s.coef_dt, cb + lane) : 1.0f;
-      } else if (static_cast<int64_t>(sv) >= s.n_rows) {
-        raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+      } else {
+        beyond = beyond | (static_cast<int64_t>(sv) >= s.n_rows);
       }
     }
     for (int q0 = 0; q0 < n_here; q0 += kFly * groups) {  // same trip count for the whole wave (shuffles inside)
       float v[kFly][VEC];
       float w[kFly];
 #pragma unroll
-      for (int k = 0; k < kFly; ++k) {
+      for (int k = 0; k < kFly; ++k) {  // no branches in here: see g_csr_zero_row
         const int first = q0 + k * groups;  // this round's entries: first + 0 .. first + groups - 1, one per group
         const int e = first + g;
         const int from = min(e, kWave - 1);
+        const bool in_round = (e < n_here) & col_ok;
+        const float w_got = s.coef ? __shfl(w_mine, from, kWave) : 1.0f;  // every lane takes part in the shuffle
         const TIn* row;
         if constexpr (PARTS) {
           const uintptr_t bits = reinterpret_cast<uintptr_t>(p_mine);
           const uint32_t p_lo = __shfl(static_cast<uint32_t>(bits), from, kWave);
           const uint32_t p_hi = __shfl(static_cast<uint32_t>(bits >> 32), from, kWave);
-          row = reinterpret_cast<const TIn*>((static_cast<uintptr_t>(p_hi) << 32) | p_lo);
+          const uintptr_t got = (static_cast<uintptr_t>(p_hi) << 32) | p_lo;
+          const bool have = in_round & (got != 0);
+          row = have ? reinterpret_cast<const TIn*>(got) + c0 : zero_row;
+          w[k] = have ? w_got : 0.f;
         } else {
           const int32_t id = __shfl(s_mine, from, kWave);
-          row = id >= 0 ? s.rows + static_cast<int64_t>(id) * a.D : nullptr;
+          const bool have = in_round & (id >= 0);
+          row = s.rows + (have ? static_cast<int64_t>(id) * a.D + c0 : zero_at);
+          w[k] = have ? w_got : 0.f;
         }
-        w[k] = s.coef ? __shfl(w_mine, from, kWave) : 1.0f;
-        if (e >= n_here || !col_ok) row = nullptr;
-        if (row != nullptr) {
-          if (s.nt) {
-            load_pack_stream<TIn, VEC>(row + c0, v[k]);
-          } else {
-            load_pack<TIn, VEC>(row + c0, v[k]);
-          }
+        if constexpr (NT) {
+          load_pack_stream<TIn, VEC>(row, v[k]);
         } else {
-          w[k] = 0.f;
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) v[k][j] = 0.f;
+          load_pack<TIn, VEC>(row, v[k]);
         }
       }
 #pragma unroll
@@ -266,6 +274,17 @@ __device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const C
         for (int j = 0; j < VEC; ++j) acc[j] = fmaf(v[k][j], w[k], acc[j]);
       }
     }
+  }
+  if (beyond) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+}
+template <typename TIn, int VEC, bool PARTS>
+__device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const CsrArgs& a, int32_t e_begin,
+                                                  int32_t e_end, int c0, bool col_ok, int g, int groups,
+                                                  float (&acc)[VEC]) {
+  if (s.nt) {  // uniform; picked here, outside the loops
+    wave_gather_range_nt<TIn, VEC, PARTS, true>(s, a, e_begin, e_end, c0, col_ok, g, groups, acc);
+  } else {
+    wave_gather_range_nt<TIn, VEC, PARTS, false>(s, a, e_begin, e_end, c0, col_ok, g, groups, acc);
   }
 }
 
@@ -285,12 +304,13 @@ constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of
 template <typename TIn, typename TOut, int VEC, bool SHUFFLE, bool PARTS = false, int EPI = kEpiStore,
           typename TIn2 = void>
 // Register budgets of the variants that end in a row update, found by measurement: 64 registers (8
-// waves per SIMD) where that costs no spills; 72 (7 waves, a few spilled words) for the one-input
-// kernels that hand list entries round by shuffle (config 3: 187 us with no bound and 92 registers,
-// 178 at 80, 170 at 72, 228 at 64 with 92 bytes spilled); no bound for those with two inputs (a
-// bound of 80 registers spills 24-60 bytes and costs 20 us in config 5).
+// waves per SIMD) for the one-input kernels, also for those that hand list entries round by
+// shuffle (config 3: 187 us with no bound and 92 registers, 178 at 80, 170 at 72; with four
+// branch-free gathers in flight the kernel needs 65, and 64 with 44 bytes spilled reads 161 us
+// against 168 at 72); no bound for those with two inputs (a bound of 80 registers spills 24-60
+// bytes and costs 20 us in config 5).
 __global__ void __launch_bounds__(kBlock, (!SHUFFLE && EPI != kEpiStore && (std::is_void<TIn2>::value || sizeof(TOut) == 4))
-                                              ? 8 : (SHUFFLE && EPI != kEpiStore && std::is_void<TIn2>::value) ? 7 : 1)
+                                              ? 8 : (SHUFFLE && EPI != kEpiStore && std::is_void<TIn2>::value) ? 8 : 1)
 csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
   constexpr bool TWO = !std::is_void<TIn2>::value;
   using TSecond = typename std::conditional<TWO, TIn2, TIn>::type;
@@ -333,6 +353,9 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
     }
   };
   // acc += sum over list entries k = first, first + step, ... < last of one input (4 gathers in flight)
+  // (short lists, a lane group each: the entries are taken as they come, with a branch for the
+  // ones that add nothing; making these loads branch-free like those of wave_gather_range was
+  // measured and lost, 167 -> 199 us in config 3, where most lists hold one entry)
   auto gather_one = [&](const auto& in, auto parts, int32_t first, int32_t last, int32_t step, int c0,
                         float (&acc)[VEC]) {
     int32_t k = first;
