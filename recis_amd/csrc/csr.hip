@@ -138,16 +138,32 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
   const int groups_per_block = kBlock >> a.lpr_log2;
   const int64_t first = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * (kExpandRows * groups_per_block) +
                         (threadIdx.x >> a.lpr_log2);
-  const int64_t n_unique = min(a.U, a.counts[0]);  // U may be the caller's upper bound: the plan's own count decides
+  // Everything that depends on the row number alone is asked for at once: the plan's count, the
+  // list bounds, the table row (and, for a table in one block, the block's address): one round
+  // trip instead of three in a row. U may be the caller's upper bound (the plan's own count
+  // decides which rows exist): the arrays hold U entries, so a row below U is safe to read.
   int64_t u[kExpandRows];
   int32_t start[kExpandRows], end[kExpandRows];
+  int64_t ri_read[kExpandRows];
   bool is_long[kExpandRows], is_short[kExpandRows];
+  const void* base0 = nullptr;
+  void* stamp_base0 = nullptr;
+  if constexpr (BLK) {
+    base0 = a.blocks[0];
+    if (a.stamp_blocks) stamp_base0 = a.stamp_blocks[0];
+  }
 #pragma unroll
   for (int r = 0; r < kExpandRows; ++r) {
     u[r] = first + r * groups_per_block;
-    const bool valid = u[r] < n_unique;
-    start[r] = valid ? a.row_start[u[r]] : 0;
-    end[r] = valid ? a.row_start[u[r] + 1] : 0;
+    const int64_t at = u[r] < a.U ? u[r] : 0;
+    start[r] = a.row_start[at];
+    end[r] = a.row_start[at + 1];
+    ri_read[r] = BLK ? a.row_index[at] : 0;
+  }
+  const int64_t n_unique = min(a.U, a.counts[0]);
+#pragma unroll
+  for (int r = 0; r < kExpandRows; ++r) {
+    if (u[r] >= n_unique) start[r] = end[r] = 0;
   }
 #pragma unroll
   for (int r = 0; r < kExpandRows; ++r) {
@@ -159,23 +175,46 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
   // the rows, then the stores
   const TIn* src[kExpandRows];
   if constexpr (BLK) {
-    int64_t ri[kExpandRows];
+    // in stages, each stage's loads of all the rows in flight together and no branch around any of
+    // them: block pointers (of block 0 for a row that reads zeros; none for a table in one block),
+    // then the rows
+    int64_t ri[kExpandRows], off[kExpandRows], blk[kExpandRows];
+    int32_t ok[kExpandRows];
+    const int64_t stamp = a.stamp_blocks ? a.stamp_value[0] : 0;  // (uniform)
 #pragma unroll
-    for (int r = 0; r < kExpandRows; ++r) ri[r] = is_short[r] ? a.row_index[u[r]] : -1;
+    for (int r = 0; r < kExpandRows; ++r) ri[r] = is_short[r] ? ri_read[r] : -1;
+    bool bad_any = false;
 #pragma unroll
     for (int r = 0; r < kExpandRows; ++r) {
-      int64_t b = 0, off = ri[r];
-      if (a.n_blocks > 1 && ri[r] >= 0) {
-        b = ri[r] / a.block_rows;
-        off = ri[r] - b * a.block_rows;
+      int64_t b = 0;
+      off[r] = ri[r];
+      if (a.n_blocks > 1) {  // (uniform)
+        b = ri[r] >= 0 ? ri[r] / a.block_rows : 0;
+        off[r] = ri[r] - b * a.block_rows;
       }
-      const bool bad = ri[r] >= 0 && (b >= a.n_blocks || off >= a.block_rows);
-      if (bad) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
-      src[r] = (ri[r] >= 0 && !bad) ? static_cast<const TIn*>(a.blocks[b]) + off * D
-                                    : reinterpret_cast<const TIn*>(g_expand_zero_row);
-      if (a.stamp_blocks && cl == 0 && ri[r] >= 0 && !bad)
-        static_cast<int64_t*>(a.stamp_blocks[b])[off] = a.stamp_value[0];
+      const bool bad = (ri[r] >= 0) & ((b >= a.n_blocks) | (off[r] >= a.block_rows));
+      bad_any = bad_any | bad;
+      ok[r] = (ri[r] >= 0) & !bad;
+      blk[r] = ok[r] ? b : 0;
     }
+    const void* base[kExpandRows];
+    void* stamp_base[kExpandRows];
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r) {
+      if (a.n_blocks == 1) {  // (uniform) one block: its address came with the first round trip
+        base[r] = base0;
+        stamp_base[r] = stamp_base0;
+      } else {
+        base[r] = a.blocks[blk[r]];
+        stamp_base[r] = a.stamp_blocks ? a.stamp_blocks[blk[r]] : nullptr;  // (uniform choice)
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r) {
+      src[r] = ok[r] ? static_cast<const TIn*>(base[r]) + off[r] * D : reinterpret_cast<const TIn*>(g_expand_zero_row);
+      if (a.stamp_blocks && cl == 0 && ok[r]) static_cast<int64_t*>(stamp_base[r])[off[r]] = stamp;
+    }
+    if (bad_any) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
   } else {
 #pragma unroll
     for (int r = 0; r < kExpandRows; ++r)
