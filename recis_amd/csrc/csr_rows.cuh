@@ -455,7 +455,7 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   RowPlaces<TRow> places{nullptr, nullptr, nullptr};
   int64_t idx_mine = -1;
   if constexpr (EPI != kEpiStore) {
-    if (valid && !hot) idx_mine = f.row_index[u];
+    if (valid) idx_mine = f.row_index[u];  // (under the same test as the list bounds: the three loads go out together)
     if constexpr (kEarlyPlaces) places = row_places<TRow, EPI>(f, a.err, idx_mine);
   }
   // the finished sum of this lane group's own row u
