@@ -713,15 +713,15 @@ class ModulePath5:
 # counter is scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC = {
-    "c4": {"csr_rows_adam_kernel": 729235251, "csr_expand_kernel": 258970931, "plan_bucket_kernel": 192893132,
-           "plan_scatter_kernel": 60785152, "plan_hist_kernel": 23681024, "bucketize_kernel": 10266214,
-           "plan_colscan_kernel": 3310182, "csr_hot_finish_kernel": 1177395, "plan_assign_new_kernel": 60825},
-    "c3": {"csr_rows_adam_kernel": 750598963, "csr_expand_kernel": 350426009, "plan_bucket_kernel": 200780083,
-           "plan_scatter_kernel": 49644236, "plan_hist_kernel": 19164672},
-    "c5": {"tile_fwd_kernel": 549501747, "csr_rows_adagrad_kernel": 768845004, "seg_pool_fwd_kernel": 93374464,
-           "block_gather_kernel": 109106995, "plan_bucket_kernel": 95321600, "plan_scatter_kernel": 46208204},
-    "c2": {"seg_pool_fwd_kernel(sum)": 4319608217, "seg_pool_bwd_kernel(sum)": 4321929216,
-           "seg_max_fwd_kernel": 4453858099, "seg_max_bwd_kernel": 4453890048},
+    "c4": {"csr_rows_adam_kernel": 729493504, "csr_expand_kernel": 258966425, "plan_bucket_kernel": 192760832,
+           "plan_scatter_kernel": 60776960, "plan_hist_kernel": 23681024, "bucketize_kernel": 10267033,
+           "plan_colscan_kernel": 3317555, "csr_hot_finish_kernel": 1165516, "plan_assign_new_kernel": 60825},
+    "c3": {"csr_rows_adam_kernel": 787405721, "csr_expand_kernel": 369861734, "plan_bucket_kernel": 200892211,
+           "plan_scatter_kernel": 49639014, "plan_hist_kernel": 19164467},
+    "c5": {"tile_fwd_kernel": 549472153, "csr_rows_adagrad_kernel": 769460019, "seg_pool_fwd_kernel": 93479526,
+           "block_gather_kernel": 109106995, "plan_bucket_kernel": 95382425, "plan_scatter_kernel": 46241689},
+    "c2": {"seg_pool_fwd_kernel(sum)": 4319621529, "seg_pool_bwd_kernel(sum)": 4321926758,
+           "seg_max_fwd_kernel": 4453851545, "seg_max_bwd_kernel": 4453888307},
 }
 
 
