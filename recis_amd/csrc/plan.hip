@@ -244,7 +244,9 @@ __device__ __forceinline__ int find_heavy(IdReader<JOBS> rd, int64_t n, HeavyScr
     }
     int e = static_cast<int>(mix_id(k[x]) >> 40) & (kHeavyTab - 1);
     for (;;) {  // half empty at worst: always ends
-      const int64_t c = *reinterpret_cast<volatile int64_t*>(&h.t_key[e]);
+      // (an atomic load, not a volatile one: a volatile access loses the LDS address space and
+      // becomes a generic load, several times the latency of an LDS read)
+      const int64_t c = __hip_atomic_load(&h.t_key[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (c == k[x]) break;
       if (c == kSetEmpty) {
         const unsigned long long old = atomicCAS(reinterpret_cast<unsigned long long*>(&h.t_key[e]),
@@ -1033,7 +1035,8 @@ plan_bucket_kernel(BucketArgs a) {
     unsigned long long v = static_cast<unsigned long long>(key);
     int e = home_of_mix(mixed, nb_log2);
     for (;;) {
-      const unsigned long long c = *reinterpret_cast<volatile unsigned long long*>(&l_key[e]);
+      const unsigned long long c = static_cast<unsigned long long>(  // (atomic, not volatile: see find_heavy)
+          __hip_atomic_load(&l_key[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
       if (c == v) return true;
       if (c < v) {  // the id there keeps its place (the empty marker is the largest value)
         if (++e >= kTabAll - 1) return false;  // the guard entry stays empty
