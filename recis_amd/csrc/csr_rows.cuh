@@ -104,27 +104,6 @@ __device__ __forceinline__ double alpha_from_powers(const FuseArgs& f, double& b
   return alpha;
 }
 
-// The epilogue of one pack of one finished row; T = the table's row type for the optimizer kinds.
-// idx = row_index[u] of the finished row (callers load it early: it heads a chain of dependent
-// accesses); alpha: of this step (Adam only).
-template <typename T, int VEC, int EPI>
-__device__ __forceinline__ void fused_row_update(const FuseArgs& f, int* err, int64_t idx, int c0,
-                                                 const float (&acc)[VEC], double alpha) {
-  int64_t b, off;
-  if (idx < 0) return;  // a key the table does not hold takes no gradient
-  if (!block_row(f.rb, idx, b, off)) {
-    raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
-    return;
-  }
-  const int64_t at = off * f.rb.D + c0;
-  if constexpr (EPI == kEpiAdam) {
-    adam_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at,
-                             static_cast<T*>(f.s1[b]) + at, acc, alpha, f.adam);
-  } else {
-    adagrad_update_pack<T, VEC>(static_cast<T*>(f.emb[b]) + at, static_cast<T*>(f.s0[b]) + at, acc, f.lr, f.eps);
-  }
-}
-
 // Where table row idx lies in the parameter and state blocks, for a caller that asks as soon as
 // idx is known (see csr_rows_kernel).
 template <typename T>
@@ -153,11 +132,26 @@ __device__ __forceinline__ void fused_row_update_at(const FuseArgs& f, const Row
                                                     const float (&acc)[VEC], double alpha) {
   if (p.w == nullptr) return;
   if constexpr (EPI == kEpiAdam) {
-    adam_update_pack<T, VEC>(p.w + c0, p.s0 + c0, p.s1 + c0, acc, alpha, f.adam);
+    // streaming accesses to the table rows (see load_row_pack_of_table), whatever the table's size:
+    // choosing by size at run time means two copies of the update in the kernel, and those cost
+    // registers (measured: 126 -> 219 us); a table small enough to stay cached pays with reads
+    // from memory that the cache could have served
+    adam_update_pack<T, VEC, true>(p.w + c0, p.s0 + c0, p.s1 + c0, acc, alpha, f.adam);
   } else {
     adagrad_update_pack<T, VEC>(p.w + c0, p.s0 + c0, acc, f.lr, f.eps);
   }
 }
+
+// The epilogue of one pack of one finished row; T = the table's row type for the optimizer kinds.
+// idx = row_index[u] of the finished row (callers load it early: it heads a chain of dependent
+// accesses); alpha: of this step (Adam only).
+template <typename T, int VEC, int EPI>
+__device__ __forceinline__ void fused_row_update(const FuseArgs& f, int* err, int64_t idx, int c0,
+                                                 const float (&acc)[VEC], double alpha) {
+  // (a key the table does not hold, idx < 0, takes no gradient)
+  fused_row_update_at<T, VEC, EPI>(f, row_places<T, EPI>(f, err, idx), c0, acc, alpha);
+}
+
 
 // A row of zeros as long as any row (D <= 8192 of at most 4 bytes): what a list entry reads that
 // has nothing to add (outside the cover, past the end of a round), so that the gathers need no

@@ -81,17 +81,46 @@ __device__ __forceinline__ void adam_compute_pack(Pack<T, VEC>& w, Pack<T, VEC>&
   }
 }
 
+// One pack of a table row read or written. STREAM: with the streaming (non-temporal) hint, for
+// 16-byte packs: the rows of a table far larger than the caches are not touched again before they
+// are evicted anyway, and without the hint they push out what the step does read again (its
+// lists, the gradient rows): the fused update of a 340 MB-per-slot table ran 8 % faster with it,
+// and so did the kernels after it.
+template <typename T, int VEC, bool STREAM>
+__device__ __forceinline__ Pack<T, VEC> load_row_pack_of_table(const T* p) {
+  if constexpr (STREAM && sizeof(T) * VEC == 16) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const u4 raw = __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
+    Pack<T, VEC> pk;
+    __builtin_memcpy(&pk, &raw, 16);
+    return pk;
+  } else {
+    return *reinterpret_cast<const Pack<T, VEC>*>(p);
+  }
+}
+template <typename T, int VEC, bool STREAM>
+__device__ __forceinline__ void store_row_pack_of_table(T* p, const Pack<T, VEC>& pk) {
+  if constexpr (STREAM && sizeof(T) * VEC == 16) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    u4 raw;
+    __builtin_memcpy(&raw, &pk, 16);
+    __builtin_nontemporal_store(raw, reinterpret_cast<u4*>(p));
+  } else {
+    *reinterpret_cast<Pack<T, VEC>*>(p) = pk;
+  }
+}
+
 // The same on memory: read, update, write.
-template <typename T, int VEC>
+template <typename T, int VEC, bool STREAM = false>
 __device__ __forceinline__ void adam_update_pack(T* w_ptr, T* m_ptr, T* v_ptr, const float (&g)[VEC], double alpha,
                                                  const AdamCoef& c) {
-  Pack<T, VEC> w = *reinterpret_cast<const Pack<T, VEC>*>(w_ptr);
-  Pack<T, VEC> m = *reinterpret_cast<const Pack<T, VEC>*>(m_ptr);
-  Pack<T, VEC> v = *reinterpret_cast<const Pack<T, VEC>*>(v_ptr);
+  Pack<T, VEC> w = load_row_pack_of_table<T, VEC, STREAM>(w_ptr);
+  Pack<T, VEC> m = load_row_pack_of_table<T, VEC, STREAM>(m_ptr);
+  Pack<T, VEC> v = load_row_pack_of_table<T, VEC, STREAM>(v_ptr);
   adam_compute_pack<T, VEC>(w, m, v, g, alpha, c);
-  *reinterpret_cast<Pack<T, VEC>*>(w_ptr) = w;
-  *reinterpret_cast<Pack<T, VEC>*>(m_ptr) = m;
-  *reinterpret_cast<Pack<T, VEC>*>(v_ptr) = v;
+  store_row_pack_of_table<T, VEC, STREAM>(w_ptr, w);
+  store_row_pack_of_table<T, VEC, STREAM>(m_ptr, m);
+  store_row_pack_of_table<T, VEC, STREAM>(v_ptr, v);
 }
 
 template <typename T, int VEC>
@@ -109,13 +138,13 @@ __device__ __forceinline__ void adagrad_compute_pack(Pack<T, VEC>& w, Pack<T, VE
   }
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool STREAM = false>
 __device__ __forceinline__ void adagrad_update_pack(T* w_ptr, T* s_ptr, const float (&g)[VEC], float lr, float eps) {
-  Pack<T, VEC> w = *reinterpret_cast<const Pack<T, VEC>*>(w_ptr);
-  Pack<T, VEC> s = *reinterpret_cast<const Pack<T, VEC>*>(s_ptr);
+  Pack<T, VEC> w = load_row_pack_of_table<T, VEC, STREAM>(w_ptr);
+  Pack<T, VEC> s = load_row_pack_of_table<T, VEC, STREAM>(s_ptr);
   adagrad_compute_pack<T, VEC>(w, s, g, lr, eps);
-  *reinterpret_cast<Pack<T, VEC>*>(w_ptr) = w;
-  *reinterpret_cast<Pack<T, VEC>*>(s_ptr) = s;
+  store_row_pack_of_table<T, VEC, STREAM>(w_ptr, w);
+  store_row_pack_of_table<T, VEC, STREAM>(s_ptr, s);
 }
 
 // cal_alpha (block_apply_adamw_op.cc:77-85) as a one-thread launch on `stream`: advances the
