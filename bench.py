@@ -713,13 +713,13 @@ class ModulePath5:
 # counter is scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC = {
-    "c4": {"csr_rows_adam_kernel": 729493504, "csr_expand_kernel": 258966425, "plan_bucket_kernel": 192760832,
-           "plan_scatter_kernel": 60776960, "plan_hist_kernel": 23681024, "bucketize_kernel": 10267033,
-           "plan_colscan_kernel": 3317555, "csr_hot_finish_kernel": 1165516, "plan_assign_new_kernel": 60825},
-    "c3": {"csr_rows_adam_kernel": 787405721, "csr_expand_kernel": 369861734, "plan_bucket_kernel": 200892211,
-           "plan_scatter_kernel": 49639014, "plan_hist_kernel": 19164467},
-    "c5": {"tile_fwd_kernel": 549472153, "csr_rows_adagrad_kernel": 769460019, "seg_pool_fwd_kernel": 93479526,
-           "block_gather_kernel": 109106995, "plan_bucket_kernel": 95382425, "plan_scatter_kernel": 46241689},
+    "c4": {"csr_rows_adam_kernel": 733113958, "csr_expand_kernel": 258937651, "plan_bucket_kernel": 192621772,
+           "plan_scatter_kernel": 60780339, "plan_hist_kernel": 23678156, "bucketize_kernel": 10267033,
+           "plan_colscan_kernel": 3316121, "csr_hot_finish_kernel": 1168384, "plan_assign_new_kernel": 60825},
+    "c3": {"csr_rows_adam_kernel": 762296729, "csr_expand_kernel": 369877094, "plan_bucket_kernel": 201006899,
+           "plan_scatter_kernel": 49638809, "plan_hist_kernel": 19164467},
+    "c5": {"tile_fwd_kernel": 549494886, "csr_rows_adagrad_kernel": 769086668, "seg_pool_fwd_kernel": 93490380,
+           "block_gather_kernel": 109106995, "plan_bucket_kernel": 95353446, "plan_scatter_kernel": 46209536},
     "c2": {"seg_pool_fwd_kernel(sum)": 4319621529, "seg_pool_bwd_kernel(sum)": 4321926758,
            "seg_max_fwd_kernel": 4453851545, "seg_max_bwd_kernel": 4453888307},
 }
