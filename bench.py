@@ -150,9 +150,8 @@ class Config4:
     def __init__(self, batch=65536, n_batches=8):
         from recis_amd import ops
         from recis_amd.nn.initializers import NormalInitializer
-        from recis_amd.nn.modules.hashtable import HashtableImpl
-        from recis_amd.optim.sparse_impl import SparseAdamImpl
-        self.ops = ops
+        from recis_amd.nn.modules import hashtable as ht
+        self.ops, self.ht = ops, ht
         # the steps rotate over n_batches batches of the same fields, so that the table holds several
         # batches' worth of rows and a step touches a scattered part of it (one batch replayed would
         # keep the whole table in the caches)
@@ -168,10 +167,12 @@ class Config4:
         init = NormalInitializer(0.0, 0.01)
         init.set_shape([10240, self.D])
         init.set_dtype(torch.float32)
-        self.table = HashtableImpl(10240, [self.D], torch.float32, torch.device("cuda"), True,
-                                   ["f%d" % i for i in range(self.n_feat)], init.build().impl(),
-                                   reserve_rows=int(self.N * 1.05) * n_batches)
-        self.opt = SparseAdamImpl.make({"ctr": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0)
+        # the table and the optimizer are the objects of recis.so (torch.classes.recis.HashtableImpl / SparseAdam),
+        # the same ones the module layer drives
+        self.table = ht.make_hashtable(10240, [self.D], torch.float32, torch.device("cuda"), True,
+                                       ["f%d" % i for i in range(self.n_feat)], init.build().impl(),
+                                       reserve_rows=int(self.N * 1.05) * n_batches)
+        self.opt = torch.classes.recis.SparseAdam.make({"ctr": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0, False)
         self.tags = list(range(self.n_feat))
         self.offsets = torch.arange(self.N + 1, dtype=torch.int32, device="cuda")
         g = torch.Generator(device="cuda").manual_seed(4)
@@ -181,7 +182,7 @@ class Config4:
         for b in self.batches:  # admission of every batch's keys happens here, not in the timed steps
             self.c = b
             plan, _ = self.dedup(self.feature_ops())
-            self.lookup(plan)
+            self.settle(plan)
         torch.cuda.synchronize()
 
     # the stages, also timed one by one for the breakdown
@@ -195,26 +196,32 @@ class Config4:
     def dedup(self, ids):
         """Tagging, dedup and find-or-insert in one pass: the plan carries the row of every unique id.
         Every field holds one id per sample, so nothing per occurrence but the lists is asked for."""
-        self.plan = self.table.plan_lookup(ids, need_inverse=False, need_pos=False, tags=self.tags)
+        self.plan = self.ht.plan_lookup(self.table, ids, need_inverse=False, need_pos=False, tags=self.tags)
         return self.plan, None
 
     def lookup(self, plan):
-        # the host reads the unique count here; the device has long gone on
+        """The rows of the plan's unique ids: the full-length buffer the plan brought along (its first U entries
+        count). Nothing waits for U: what follows takes it from device memory; settle() reads it once the whole
+        step is queued."""
+        return plan.index_buf
+
+    def settle(self, plan):
+        """The host's copy of the unique count (it arrived in pinned memory while the device went on) tells the id
+        map how many ids the counted lookup held."""
         self.U = plan.U
-        return self.table.settle_lookup(plan.index_buf, self.U, plan)
+        self.table.settle_count(self.U, plan)
 
     def pool_fwd(self, index, inv):
         # pooling reads the rows out of the table (no [U, D] copy); every field holds one id per
         # sample, so, as EmbeddingEngine does for dense [B] id tensors, each unique row is read
         # once and written to its occurrences
-        chunks, chunk_rows = self.table.emb_blocks()
-        return self.ops.plan_expand_rows(self.plan, self.N, blocks=chunks, block_size=chunk_rows, row_index=index)
+        return self.table.expand_rows(self.plan, index, None, None, None)
 
     def pool_bwd(self, inv):
         return self.ops.segment_reduce_backward_plan(self.grad_out, None, self.offsets, self.plan, "sum")
 
     def update(self, index, g):
-        self.table.accept_grad(index, g, unique=True)
+        self.table.accept_grad_ex(index, g, True, 0)
         self.opt.step()
         self.opt.zero_grad()
 
@@ -223,7 +230,9 @@ class Config4:
         summed over its occurrences and applied to the row by the lanes that summed it (the [U, D]
         gradient is not written). Bit for bit what pool_bwd + update give
         (tests/test_gpu_features.py::test_fused_gather_reduce_update_equals_the_two_calls)."""
-        self.opt.apply_planned(self.table, self.plan, self.grad_out, self.plan.occ, None, index)
+        self.ht.accept_planned_grad(self.table, index, self.plan, self.grad_out, self.plan.occ)
+        self.opt.step()       # sums the gradient it was handed unsummed and updates the rows, one launch
+        self.opt.zero_grad()
 
     def next_batch(self):
         self.c = self.batches[self._turn % len(self.batches)]
@@ -236,6 +245,7 @@ class Config4:
         index = self.lookup(uniq)
         pooled = self.pool_fwd(index, inv)
         self.bwd_update(index)
+        self.settle(uniq)
         return pooled
 
     def step_from_host(self):
@@ -314,8 +324,9 @@ class Config4:
         ids = self.feature_ops()
         uniq, inv = self.dedup(ids)
         index = self.lookup(uniq)
+        self.settle(uniq)
         def dedup_lookup():
-            self.lookup(self.dedup(ids)[0])
+            self.settle(self.dedup(ids)[0])
         return {
             "feature_ops": _event_ms(self.feature_ops, iters),
             "dedup+lookup": _event_ms(dedup_lookup, iters),
@@ -382,9 +393,8 @@ class Config3:
                  filter_interval=50):
         from recis_amd import ops
         from recis_amd.nn.initializers import NormalInitializer
-        from recis_amd.nn.modules.hashtable import HashtableImpl
-        from recis_amd.optim.sparse_impl import SparseAdamImpl
-        self.ops = ops
+        from recis_amd.nn.modules import hashtable as ht
+        self.ops, self.ht = ops, ht
         self.D, self.N, self.resident = 32, ids_per_step, resident
         self.ids_per_step = ids_per_step
         self.filter_step, self.filter_interval = filter_step, filter_interval
@@ -392,10 +402,10 @@ class Config3:
         init.set_shape([10240, self.D])
         init.set_dtype(torch.float32)
         reserve = int(resident * 1.12) + 40 * ids_per_step // 10
-        self.table = HashtableImpl(10240, [self.D], torch.float32, torch.device("cuda"), False, ["c3"],
-                                   init.build().impl(), reserve_rows=reserve)
+        self.table = ht.make_hashtable(10240, [self.D], torch.float32, torch.device("cuda"), False, ["c3"],
+                                       init.build().impl(), reserve_rows=reserve)
         self.table.append_step_filter_slot("step_filter", -1)
-        self.opt = SparseAdamImpl.make({"c3": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0)
+        self.opt = torch.classes.recis.SparseAdam.make({"c3": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0, False)
         chunk = 25_000_000
         for lo in range(0, resident, chunk):
             ranks = torch.arange(lo, min(lo + chunk, resident), device="cuda")
@@ -428,19 +438,21 @@ class Config3:
         if self.step_no and self.step_no % self.filter_interval == 0:
             self.sweep(self.step_no - self.filter_step)
         self.step_no += 1
-        plan = self.table.plan_lookup(ids, need_inverse=False, need_pos=False)   # dedup + find-or-insert, one pass
-        self.U = plan.U
-        index = self.table.settle_lookup(plan.index_buf, self.U, plan)
-        chunks, chunk_rows = self.table.emb_blocks()
+        # dedup + find-or-insert, one pass; the plan brings the row of every unique id along
+        plan = self.ht.plan_lookup(self.table, ids, need_inverse=False, need_pos=False)
+        index = plan.index_buf
         # one row per lookup: every unique row is read once out of the table and written to its
         # occurrences (no [U, D] copy, no second pass over it); the step filter's stamps of the
         # rows go out in the same pass
-        stamps = self.table.slot_blocks("step_filter")[0]
-        out = o.plan_expand_rows(plan, self.N, blocks=chunks, block_size=chunk_rows, row_index=index,
-                                 stamp=(stamps, self.step_t))
+        out = self.table.expand_rows(plan, index, None, "step_filter", self.step_t)
         # the per-lookup gradients reduced per key and applied to the row in the same launch
-        self.opt.apply_planned(self.table, plan, self.grad_out, plan.occ, None, index, cover=self.span)
+        self.ht.accept_planned_grad(self.table, index, plan, self.grad_out, plan.occ, cover=self.span)
+        self.opt.step()
+        self.opt.zero_grad()
         self.step_t += 1
+        # the whole step is queued: the unique count has arrived in pinned memory meanwhile
+        self.U = plan.U
+        self.table.settle_count(self.U, plan)
         return out
 
     def sweep(self, threshold):
@@ -520,9 +532,8 @@ class Config5:
     def __init__(self):
         from recis_amd import ops
         from recis_amd.nn.initializers import NormalInitializer
-        from recis_amd.nn.modules.hashtable import HashtableImpl
-        from recis_amd.optim.sparse_impl import SparseAdagradImpl
-        self.ops = ops
+        from recis_amd.nn.modules import hashtable as ht
+        self.ops, self.ht = ops, ht
         c = workloads.config5()
         self.c = c
         self.D, self.N = 128, c["num_ids"]
@@ -533,10 +544,10 @@ class Config5:
         init = NormalInitializer(0.0, 0.01)
         init.set_shape([10240, self.D])
         init.set_dtype(torch.bfloat16)
-        self.table = HashtableImpl(10240, [self.D], torch.bfloat16, torch.device("cuda"), True,
-                                   ["s%d" % i for i in range(len(self.fields))], init.build().impl(),
-                                   reserve_rows=int(self.N * 1.1))
-        self.opt = SparseAdagradImpl.make({"c5": self.table}, 0.01, 1e-8)
+        self.table = ht.make_hashtable(10240, [self.D], torch.bfloat16, torch.device("cuda"), True,
+                                       ["s%d" % i for i in range(len(self.fields))], init.build().impl(),
+                                       reserve_rows=int(self.N * 1.1))
+        self.opt = torch.classes.recis.SparseAdagrad.make({"c5": self.table}, 0.01, 1e-8)
         self.S = sum(self.batch)
         self.pad_rows = sum(b * s for b, s in zip(self.batch, self.seq))
         g = torch.Generator(device="cuda").manual_seed(5)
@@ -548,7 +559,7 @@ class Config5:
     def step(self):
         o = self.ops
         # tagging (ids_encode), dedup and find-or-insert in one pass
-        plan = self.table.plan_lookup([f["values"] for f in self.fields], tags=list(range(len(self.fields))))
+        plan = self.ht.plan_lookup(self.table, [f["values"] for f in self.fields], tags=list(range(len(self.fields))))
         self.U = plan.U
         inv = plan.inverse
         index = self.table.settle_lookup(plan.index_buf, self.U, plan)
@@ -563,7 +574,10 @@ class Config5:
         """Backward of both outputs into the unique rows and the Adagrad update of those rows, one
         launch: the two gradients of an occurrence are summed where the row's gradient is summed."""
         src_p, coef_p, src_t = plan.src_for_pool_and_tile(self.offsets, None, True, self.batch, self.seq)
-        self.opt.apply_planned2(self.table, plan, (self.g_pool, src_p, coef_p), (self.g_tile, src_t, None), index)
+        self.ht.accept_planned_grad(self.table, index, plan, self.g_pool, src_p, coef_p, key=plan.serial)
+        self.ht.accept_planned_grad(self.table, index, plan, self.g_tile, src_t, None, key=plan.serial)
+        self.opt.step()       # both gradients of the plan summed and the rows updated in one launch
+        self.opt.zero_grad()
 
     def survey_bytes(self):
         N, U, S, D = self.N, self.U, self.S, self.D
@@ -621,10 +635,14 @@ class Config5:
 # --------------------------------------------------------------------- the same steps through the modules
 class ModulePath4:
     """Config 4 through the drop-in layer: FeatureEngine (bucketize + mod of the 13 dense columns) ->
-    EmbeddingEngine (39 features on one coalesced table) -> concatenation for a dense tower ->
-    backward -> SparseAdam.step, rotating over the same 8 batches as Config4."""
+    EmbeddingEngine (39 features on one coalesced table) -> backward from one gradient per feature output ->
+    SparseAdam.step, rotating over the same 8 batches as Config4. The work is Config4's: the engine returns
+    one [B, 16] output per feature (views of the one pooled buffer) and backward receives one gradient per
+    output, here 39 slices of one buffer, as Config4.grad_out is one buffer. (A dense tower that concatenates
+    the outputs along the feature axis adds a 168 MB copy each way; that copy is the model's, not the table's,
+    and is reported separately as module_path_with_concat_ms.)"""
 
-    def __init__(self, n_batches=8):
+    def __init__(self, n_batches=8, concat=False):
         from recis_amd.features import Bucketize, Feature, FeatureEngine, Mod, SelectField
         from recis_amd.nn import EmbeddingEngine, EmbeddingOption
         from recis_amd.nn.initializers import NormalInitializer
@@ -650,7 +668,11 @@ class ModulePath4:
             d.update({"d%d" % i: t for i, t in enumerate(b["dense"])})
             self.data.append(d)
         g = torch.Generator(device="cuda").manual_seed(4)
-        self.up = torch.randn((c["batch"], 16 * len(self.names)), device="cuda", generator=g)
+        self.concat = concat
+        if concat:
+            self.up = torch.randn((c["batch"], 16 * len(self.names)), device="cuda", generator=g)
+        else:
+            self.up = list(torch.randn((len(self.names) * c["batch"], 16), device="cuda", generator=g).split(c["batch"]))
         self._turn = 0
         for _ in range(n_batches + 2):
             self.step()
@@ -662,9 +684,60 @@ class ModulePath4:
         x = dict(data)
         x.update({k: v.view(-1, 1) for k, v in self.fe({k: data[k] for k in data if k[0] == "d"}).items()})
         out = self.eng(x)
-        torch.cat([out[n] for n in self.names], dim=1).backward(self.up)
+        if self.concat:
+            torch.cat([out[n] for n in self.names], dim=1).backward(self.up)
+        else:
+            torch.autograd.backward([out[n] for n in self.names], self.up)
         self.opt.step()
         self.opt.zero_grad()
+
+
+class TorchLibraryPath4:
+    """Config 4 through the reference's own boundary and its own call sequence, operator by operator
+    (torch.ops.recis.* / torch.classes.recis.* of recis.so, nothing else): fused_bucketized -> fused_uint64_mod ->
+    ids_encode -> ids_partition -> HashtableImpl.embedding_lookup -> segment_reduce_forward ->
+    segment_reduce_backward -> HashtableImpl.accept_grad -> SparseAdam.step
+    (recis/nn/modules/embedding_engine.py:627-675, csrc/embedding/hashtable.cc:153-165, adam.cc:98-135). Each
+    operator materialises its result as the reference's does (the sorted unique ids, the [U, D] rows, the [U, D]
+    gradient), so this is the unfused form of the step."""
+
+    def __init__(self, n_batches=8):
+        from recis_amd import torch_library
+        torch_library.load()
+        self.R = R = torch.ops.recis
+        self.batches = [workloads.config4()] + [workloads.config4(data_seed=k) for k in range(1, n_batches)]
+        c = self.batches[0]
+        self.n_feat = len(c["sparse"]) + len(c["dense"])
+        self.N, self.D = c["num_ids"], 16
+        gen = torch.classes.recis.Generator.make_normal_generator([10240, self.D], torch.float32, 0.0, 0.01, None)
+        self.table = R.make_hashtable(10240, [self.D], torch.float32, torch.device("cuda", 0), True,
+                                      ["f%d" % i for i in range(self.n_feat)], gen, 0, 65536, 65536)
+        self.table.reserve(int(self.N * 1.05) * n_batches)
+        self.opt = torch.classes.recis.SparseAdam.make({"ctr": self.table}, 1e-3, 0.9, 0.999, 1e-8, 0.0, False)
+        self.table_ids = torch.arange(self.n_feat, dtype=torch.int64)
+        self.mods = torch.full((len(c["dense"]),), c["mod"], dtype=torch.int64)
+        self.offsets = torch.arange(self.N + 1, dtype=torch.int32, device="cuda")
+        g = torch.Generator(device="cuda").manual_seed(4)
+        self.grad_out = torch.randn((self.N, self.D), device="cuda", generator=g)
+        self._turn = 0
+        for _ in range(n_batches + 2):
+            self.step()
+        torch.cuda.synchronize()
+
+    def step(self):
+        R = self.R
+        c = self.batches[self._turn % len(self.batches)]
+        self._turn += 1
+        extra = R.fused_uint64_mod(R.fused_bucketized(c["dense"], c["boundaries"]), self.mods)
+        ids = R.ids_encode(c["sparse"] + extra, self.table_ids)
+        uniq, _, inverse = R.ids_partition(ids, 1)
+        index, emb = self.table.embedding_lookup(uniq, False)
+        pooled = R.segment_reduce_forward(emb, None, inverse, self.offsets, "sum")
+        grad = R.segment_reduce_backward(self.grad_out, None, inverse, self.offsets, uniq.numel(), "sum")
+        self.table.accept_grad(index, grad)
+        self.opt.step()
+        self.opt.zero_grad()
+        return pooled
 
 
 class ModulePath5:
@@ -819,10 +892,10 @@ def _c3_eviction(wl, step_ms):
     """Runs config 3 on to its next sweep of the step filter (every 50 steps, threshold step - 50)
     and reports it: the keys it evicted, its time, and the step time with the sweep spread over
     the 50 steps it serves. New keys per step come from the id map's own counters."""
-    live0, idn0, _, _ = wl.table.id_map().stats()
+    live0, idn0, _, _ = wl.table.id_map_stats()
     step0 = wl.step_no
     at, evicted, ms = wl.run_to_next_sweep()
-    live1, idn1, _, _ = wl.table.id_map().stats()
+    live1, idn1, _, _ = wl.table.id_map_stats()
     steps = wl.step_no - step0
     out = {"sweep_at_step": at, "evicted_per_sweep": evicted, "sweep_ms": round(ms, 3),
            "sweep_interval_steps": wl.filter_interval, "live_keys_before": live0, "live_keys_after": live1,
@@ -833,7 +906,7 @@ def _c3_eviction(wl, step_ms):
     # not come back within the next.
     at2, evicted2, ms2 = wl.run_to_next_sweep()
     out["steady_sweep"] = {"sweep_at_step": at2, "evicted": evicted2, "sweep_ms": round(ms2, 3),
-                           "live_keys_after": wl.table.id_map().stats()[0],
+                           "live_keys_after": wl.table.id_map_stats()[0],
                            "ms_per_step_with_sweep": round(step_ms + ms2 / wl.filter_interval, 4)}
     return out
 
@@ -977,6 +1050,13 @@ def main():
                 target["module_path_ms"] = round(ms, 4)
             del mp
             torch.cuda.empty_cache()
+        if args.workload == "c4":
+            for key, make in (("module_path_with_concat_ms", lambda: ModulePath4(concat=True)),
+                              ("torch_library_path_ms", TorchLibraryPath4)):
+                wl = make()
+                out[key] = round(_timed_steps(wl, 10, 3), 4)
+                del wl
+                torch.cuda.empty_cache()
         if main_wl is None and not args.no_cpu_baseline:
             main_wl = classes[args.workload]()
     if extras:

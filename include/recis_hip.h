@@ -518,6 +518,10 @@ int recis_csr_fill_lists(const int32_t* list, int64_t n, const void* offsets, in
  * cover_offsets (device, [cover_S + 1], int32 or int64) or NULL: entries whose src lies outside
  * [cover_offsets[0], cover_offsets[cover_S]) are skipped too (occurrences no segment covers,
  * for the backward of the TILE mode where src is the occurrence itself).
+ * U may be an upper bound of the number of unique ids (a caller that has not read the plan's
+ * count back yet passes n): rows at and past counts_dev[0], the count the plan left on the device,
+ * are skipped (out must then hold U rows, of which the first counts_dev[0] are written). The same
+ * holds for every recis_csr_gather_reduce* entry point below.
  */
 int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
                             const void* coef, int coef_dtype, const int32_t* row_start,

@@ -32,6 +32,17 @@ class RecisHipError(RuntimeError):
     pass
 
 
+# A ScalarType that a method of a torch.classes.recis object returns crosses the binding as its
+# c10::ScalarType number (tests/test_torch_library.py checks the table against the library).
+SCALAR_TYPE_DTYPES = {0: torch.uint8, 1: torch.int8, 2: torch.int16, 3: torch.int32, 4: torch.int64,
+                      5: torch.float16, 6: torch.float32, 7: torch.float64, 11: torch.bool, 15: torch.bfloat16}
+
+
+def as_dtype(code):
+    """torch.dtype of a ScalarType number (a torch.dtype passes through)."""
+    return code if isinstance(code, torch.dtype) else SCALAR_TYPE_DTYPES[int(code)]
+
+
 def lib():
     """The loaded library (built first if no binary is present)."""
     global _lib

@@ -435,7 +435,9 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   // ---- cold rows
   const int rows_per_block = kBlock >> a.lpr_log2;
   const int64_t u = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * rows_per_block + (threadIdx.x >> a.lpr_log2);
-  const bool valid = u < a.U;
+  // a.U may be an upper bound (a caller that has not read the plan's count back passes the number of
+  // ids): rows at and past the count the plan left on the device have no list
+  const bool valid = u < a.U && u < a.counts[0];
   const int32_t start = valid ? a.row_start[u] : 0;
   int32_t end = valid ? a.row_start[u + 1] : 0;
   const bool hot = end - start > a.hot_len;  // left to the work items and the finish kernel

@@ -52,20 +52,18 @@ TORCH_LIBRARY(recis, m) {
       .def("child_at", &ChildrenInfo::ChildAt)
       .def("is_coalesce", &ChildrenInfo::IsCoalesce);
 
-  m.class_<Slot>("Slot")
-      .def("block_size", &Slot::BlockSize)
-      .def("name", &Slot::Name)
-      .def("flat_size", &Slot::FlatSize)
-      .def("value", &Slot::Value)
-      .def("values", &Slot::ValuesDeref);
-
-  m.class_<SlotGroup>("SlotGroup")
-      .def("slot_by_name", &SlotGroup::GetSlotByName)
-      .def("slot_by_index", &SlotGroup::GetSlotByIndex)
-      .def("slot_index", &SlotGroup::GetSlotByIndex)  // sic: the reference binds this name to GetSlotByIndex too
-      .def("slots", &SlotGroup::Slots);
-
+  // (classes are registered before the signatures that mention them)
   m.class_<Generator>("Generator")
+      // additions: a tensor of another shape (Slot::GenVal, slot_group.cc:112-116; fan-dependent
+      // initialisers take the fans from fan_shape when given), and the device the rows are drawn on
+      .def(
+          "gen",
+          [](const c10::intrusive_ptr<Generator>& self, c10::optional<std::vector<int64_t>> shape,
+             c10::optional<std::vector<int64_t>> fan_shape) {
+            return self->Generate(shape.value_or(std::vector<int64_t>{}), fan_shape.value_or(std::vector<int64_t>{}));
+          },
+          "", {torch::arg("shape") = c10::nullopt, torch::arg("fan_shape") = c10::nullopt})
+      .def("set_device", [](const c10::intrusive_ptr<Generator>& self, at::Device device) { self->set_device(device); })
       .def_static("generate", Generator::DoGenerator)
       .def_static("make_constant_generator", recis::embedding::MakeConstantGenerator)
       .def_static("make_uniform_generator", recis::embedding::MakeUniformGenerator)
@@ -74,7 +72,84 @@ TORCH_LIBRARY(recis, m) {
       .def_static("make_xavier_normal_generator", recis::embedding::MakeXavierNormalGenerator)
       .def_static("make_kaiming_uniform_generator", recis::embedding::MakeKaimingUniformGenerator)
       .def_static("make_kaiming_normal_generator", recis::embedding::MakeKaimingNormalGenerator)
-      .def_static("make_trunc_normal_generator", recis::embedding::MakeTruncNormalGenerator);
+      .def_static("make_trunc_normal_generator", recis::embedding::MakeTruncNormalGenerator)
+      .def_static("make_tensor_generator", recis::embedding::MakeTensorGenerator);  // an addition
+
+  using SlotSelf = c10::intrusive_ptr<Slot>;
+  m.class_<Slot>("Slot")
+      .def("block_size", &Slot::BlockSize)
+      .def("name", &Slot::Name)
+      .def("flat_size", &Slot::FlatSize)
+      .def("value", &Slot::Value)
+      .def("values", &Slot::ValuesDeref)
+      // additions: what the reference reaches from C++ (csrc/serialize, the optimizers) and this
+      // build's Python reaches through the binding
+      .def("dtype", &Slot::Dtype)
+      .def("row_shape", &Slot::RowShape)
+      .def(
+          "index_select",
+          [](const SlotSelf& self, const at::Tensor& index, int64_t beg, int64_t end) {
+            return self->IndexSelect(index, beg, end < 0 ? index.numel() : end);
+          },
+          "", {torch::arg("index"), torch::arg("beg") = 0, torch::arg("end") = -1})
+      .def(
+          "index_insert",
+          [](const SlotSelf& self, const at::Tensor& index, at::Tensor value, c10::optional<at::Tensor> accept) {
+            if (accept.has_value() && accept->defined()) {
+              self->IndexInsert(index, std::move(value), *accept);
+            } else {
+              self->IndexInsert(index, std::move(value));
+            }
+          },
+          "", {torch::arg("index"), torch::arg("value"), torch::arg("accept_indicator") = c10::nullopt})
+      .def("gen_val", &Slot::GenVal)
+      .def("kernel_blocks", [](const SlotSelf& self) { return std::make_tuple(self->Chunks(), self->ChunkRows()); });
+
+  using GroupSelf = c10::intrusive_ptr<SlotGroup>;
+  m.class_<SlotGroup>("SlotGroup")
+      .def("slot_by_name", &SlotGroup::GetSlotByName)
+      .def("slot_by_index", &SlotGroup::GetSlotByIndex)
+      .def("slot_index", &SlotGroup::GetSlotByIndex)  // sic: the reference binds this name to GetSlotByIndex too
+      .def("slots", &SlotGroup::Slots)
+      // additions
+      .def("emb_slot", &SlotGroup::EmbSlot)
+      .def("get_slot_index", &SlotGroup::GetSlotIndex)
+      .def("has_slot", &SlotGroup::HasSlot)
+      .def("block_size", &SlotGroup::BlockSize)
+      .def("block_num", &SlotGroup::BlockNum)
+      .def("capacity_rows", &SlotGroup::CapacityRows)
+      .def("chunk_rows", &SlotGroup::ChunkRows)
+      .def("append_slot",
+           [](const GroupSelf& self, const std::string& name, at::ScalarType dtype, std::vector<int64_t> partial_shape,
+              c10::optional<c10::intrusive_ptr<Generator>> generator, double init_val) {
+             if (generator.has_value() && generator->defined()) {
+               return self->AppendSlot(name, dtype, partial_shape, *generator);
+             }
+             return self->AppendSlot(name, dtype, partial_shape, init_val);
+           });
+
+  using recis::BatchPlan;
+  using PlanSelf = c10::intrusive_ptr<BatchPlan>;
+  m.class_<BatchPlan>("BatchPlan")  // an addition: see plan.h
+      .def_property("n", [](const PlanSelf& self) { return self->n(); })
+      .def_property("serial", [](const PlanSelf& self) { return self->serial(); })
+      .def_property("hot_cap", [](const PlanSelf& self) { return self->hot_cap(); })
+      .def_property("U", [](const PlanSelf& self) { return self->U(); })
+      .def_property("unique", [](const PlanSelf& self) { return self->unique(); })
+      .def_property("unique_buf", [](const PlanSelf& self) { return self->unique_buf(); })
+      .def_property("inverse", [](const PlanSelf& self) { return self->inverse(); })
+      .def_property("pos", [](const PlanSelf& self) { return self->pos(); })
+      .def_property("row_start", [](const PlanSelf& self) { return self->row_start(); })
+      .def_property("occ", [](const PlanSelf& self) { return self->occ(); })
+      .def_property("hot_items", [](const PlanSelf& self) { return self->hot_items(); })
+      .def_property("counts", [](const PlanSelf& self) { return self->counts(); })
+      .def_property("index_buf", [](const PlanSelf& self) { return self->index_buf(); })
+      .def("U_bound", [](const PlanSelf& self) { return self->U_bound(); })
+      .def("src_coef_for_pool", &BatchPlan::SrcCoefForPool, "",
+           {torch::arg("offsets"), torch::arg("weight"), torch::arg("mean")})
+      .def("src_for_tile", &BatchPlan::SrcForTile, "", {torch::arg("batch"), torch::arg("seq"), torch::arg("offsets")})
+      .def("src_for_pool_and_tile", &BatchPlan::SrcForPoolAndTile, "",
+           {torch::arg("offsets"), torch::arg("weight"), torch::arg("mean"), torch::arg("batch"), torch::arg("seq")});
 
   m.class_<Hashtable>("HashtableImpl")
       .def("accept_grad", &Hashtable::AcceptGrad)
@@ -93,7 +168,42 @@ TORCH_LIBRARY(recis, m) {
       .def("get_slot", &Hashtable::GetSlot)
       .def("delete", &Hashtable::Delete)
       .def("ids_map", &Hashtable::ids_map)
-      .def_readonly("hashtable_tag", &Hashtable::kNullIndex);
+      .def_readonly("hashtable_tag", &Hashtable::kNullIndex)
+      // additions (no counterpart in the reference's binding): what its C++ reaches directly
+      // (csrc/serialize: InsertLookupIndexWithIndicator, ids_num, SliceInfo) and the batch-plan path
+      .def("ids_num", &Hashtable::ids_num)
+      .def("slice_info", &Hashtable::SliceInfo)
+      .def("embedding_shape", &Hashtable::EmbeddingShape)
+      .def("device", [](const HashTablePtr& self) { return self->device(); })
+      .def("dtype", [](const HashTablePtr& self) { return self->dtype(); })
+      .def("has_grad", &Hashtable::has_grad)
+      .def("grad_pairs", &Hashtable::GradPairs)
+      .def("insert_lookup_index", &Hashtable::InsertLookupIndex)
+      .def("insert_lookup_index_with_indicator", &Hashtable::InsertLookupIndexWithIndicator)
+      .def("lookup_index_readonly", &Hashtable::LookupIndexReadOnly)
+      .def("lookup_index", &Hashtable::LookupIndex)
+      .def("reserve", &Hashtable::Reserve)
+      .def("emb_blocks",
+           [](const HashTablePtr& self) {
+             auto emb = self->RawSlotGroup()->EmbSlot();
+             return std::make_tuple(emb->Chunks(), emb->ChunkRows());
+           })
+      .def("slot_blocks",
+           [](const HashTablePtr& self, const std::string& name) {
+             return self->RawSlotGroup()->GetSlotByName(name)->Chunks();
+           })
+      .def("plan_lookup", &Hashtable::PlanLookup)
+      .def("plan_index", &Hashtable::PlanIndex)
+      .def("lookup_index_counted", &Hashtable::LookupIndexCounted)
+      .def("settle_count", &Hashtable::SettleCount)
+      .def("settle_lookup", &Hashtable::SettleLookup)
+      .def("expand_rows", &Hashtable::ExpandRows)
+      .def("accept_grad_ex", &Hashtable::AcceptGradEx)
+      .def("accept_planned_grad", &Hashtable::AcceptPlannedGrad)
+      .def("evict_older", &Hashtable::EvictOlder)
+      .def("id_map_stats", &Hashtable::IdMapStats)
+      .def("pending_grads", &Hashtable::PendingGrads)
+      .def("id_map_handle", [](const HashTablePtr& self) { return reinterpret_cast<int64_t>(self->id_map()); });
 
   def_optimizer<recis::optim::SparseAdamW>(m, "SparseAdamW");
   def_optimizer<recis::optim::SparseAdam>(m, "SparseAdam");
@@ -101,6 +211,9 @@ TORCH_LIBRARY(recis, m) {
   def_optimizer<recis::optim::SparseAdagrad>(m, "SparseAdagrad");  // an addition
 
   m.def("make_hashtable", Hashtable::Make);
+  m.def("unique_plan", recis::unique_plan);  // an addition: see plan.h
+  // an addition: the integer a ScalarType crosses the binding as (Slot.dtype(), HashtableImpl.dtype())
+  m.def("scalar_type_code", [](const at::Tensor& t) { return t.scalar_type(); });
 
   m.def("ragged_to_dense", recis::functional::ragged_to_dense);
   m.def("uint64_mod", recis::functional::uint64_mod);

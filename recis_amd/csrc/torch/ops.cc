@@ -431,7 +431,79 @@ std::tuple<Tensor, Tensor, Tensor> ids_partition(const Tensor& ids, int64_t num_
                       : at::div(slot, m + 1, "floor");
   Tensor counts = at::bincount(part, {}, num_parts).to(at::kLong);
   Tensor inverse = rank.index_select(0, inv.to(at::kLong)).to(at::kInt);
+  note_unique(sorted_u);
   return std::make_tuple(sorted_u, counts, inverse);
+}
+
+namespace {
+std::mutex g_unique_mu;
+struct NotedUnique {
+  Tensor t;
+  uint32_t version;
+};
+std::vector<NotedUnique> g_noted_unique;  // the last few, newest last
+}  // namespace
+
+void note_unique(const Tensor& t) {
+  std::lock_guard<std::mutex> lock(g_unique_mu);
+  if (g_noted_unique.size() >= 4) g_noted_unique.erase(g_noted_unique.begin());
+  g_noted_unique.push_back({t, t._version()});
+}
+
+bool known_unique(const Tensor& t) {
+  if (!t.defined() || t.numel() == 0) return t.defined();
+  std::lock_guard<std::mutex> lock(g_unique_mu);
+  for (const auto& e : g_noted_unique) {
+    if (e.t.data_ptr() == t.data_ptr() && e.t.numel() == t.numel() && e.t.scalar_type() == t.scalar_type() &&
+        t.is_contiguous() && e.version == t._version() && e.t._version() == e.version) {
+      return true;
+    }
+  }
+  return false;
+}
+
+// ------------------------------------------------------------------------------------ over a batch plan
+Tensor csr_gather_reduce(const Tensor& rows_in, const BatchPlanPtr& plan, const Tensor& src, const Tensor& coef,
+                         const Tensor& cover) {
+  require_gpu(rows_in, "rows");
+  require_gpu(src, "src");
+  TORCH_CHECK(rows_in.dim() == 2, "gradient rows must be [rows, D]");
+  c10::DeviceGuard guard(rows_in.device());
+  Tensor rows = rows_in.contiguous();
+  const int64_t D = rows.size(1), U = plan->U();
+  Tensor out = at::empty({U, D}, rows.options().dtype(at::kFloat));
+  check(recis_csr_gather_reduce(
+      rows.data_ptr(), dtype_code(rows.scalar_type()), rows.size(0), src.data_ptr<int32_t>(),
+      coef.defined() ? coef.data_ptr() : nullptr, coef.defined() ? dtype_code(coef.scalar_type()) : 0,
+      plan->row_start().data_ptr<int32_t>(), plan->hot_items().data_ptr<int32_t>(), plan->hot_cap(),
+      plan->counts().data_ptr<int64_t>(), out.data_ptr(), RECIS_F32, U, D, 0, cover.defined() ? cover.data_ptr() : nullptr,
+      cover.defined() ? index_kind(cover, "offsets") : 0, cover.defined() ? cover.numel() - 1 : 0,
+      stream_of(rows.device())));
+  return out;
+}
+
+Tensor csr_gather_reduce_parts(const TensorList& parts_in, const BatchPlanPtr& plan, const Tensor& src) {
+  TORCH_CHECK(!parts_in.empty() && parts_in.size() <= 8, "csr_gather_reduce_parts: 1 to 8 parts");
+  require_gpu(parts_in, "parts");
+  require_gpu(src, "src");
+  TensorList parts;
+  for (const auto& p : parts_in) {
+    TORCH_CHECK(p.dim() == 2 && p.scalar_type() == parts_in[0].scalar_type() && p.size(1) == parts_in[0].size(1),
+                "csr_gather_reduce_parts: the parts must be [rows, D] tensors of one dtype and row width");
+    parts.push_back(p.contiguous());
+  }
+  c10::DeviceGuard guard(parts[0].device());
+  const int64_t D = parts[0].size(1), U = plan->U();
+  Tensor out = at::empty({U, D}, parts[0].options().dtype(at::kFloat));
+  auto ptrs = host_ptrs<void>(parts);
+  std::vector<int64_t> counts;
+  for (const auto& p : parts) counts.push_back(p.size(0));
+  check(recis_csr_gather_reduce_parts(ptrs.data(), counts.data(), static_cast<int>(parts.size()),
+                                      dtype_code(parts[0].scalar_type()), src.data_ptr<int32_t>(),
+                                      plan->row_start().data_ptr<int32_t>(), plan->hot_items().data_ptr<int32_t>(),
+                                      plan->hot_cap(), plan->counts().data_ptr<int64_t>(), out.data_ptr(), U, D, 0,
+                                      stream_of(parts[0].device())));
+  return out;
 }
 
 // ------------------------------------------------------------------------------------ feature ops

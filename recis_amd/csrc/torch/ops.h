@@ -8,6 +8,8 @@
 #include <tuple>
 #include <vector>
 
+#include "plan.h"
+
 namespace recis {
 namespace functional {
 
@@ -78,6 +80,20 @@ std::tuple<Tensor, Tensor, Tensor> feature_cross_ragged(const Tensor& x_value, c
                                                         const Tensor& y_offsets, const Tensor& y_weight);
 std::tuple<Tensor, Tensor> calc_ragged_index(Tensor drop_num, Tensor pad_num, Tensor drop_side, Tensor pad_side,
                                              Tensor offset, Tensor topk_index, Tensor indicator);
+
+
+// ---- over a batch plan (additions: the reference scatters with atomics instead)
+// out[u] = sum over the occurrence list of unique id u of coef[k] * rows[src[k]]: fp32 [U, D]. coef
+// and cover may be undefined (see recis_csr_gather_reduce).
+Tensor csr_gather_reduce(const Tensor& rows, const BatchPlanPtr& plan, const Tensor& src, const Tensor& coef,
+                         const Tensor& cover);
+// the same over rows that live in up to 8 arrays laid end to end in src's numbering
+Tensor csr_gather_reduce_parts(const TensorList& parts, const BatchPlanPtr& plan, const Tensor& src);
+// ids_partition notes the unique ids it hands out; known_unique(t) says whether t is one of those
+// tensors, unchanged since (same memory, same length, same version counter). The noted tensors are
+// kept alive, so their addresses cannot be handed out to another tensor meanwhile.
+void note_unique(const Tensor& t);
+bool known_unique(const Tensor& t);
 
 }  // namespace functional
 }  // namespace recis

@@ -32,6 +32,12 @@ class SparseOptimizer : public torch::CustomClassHolder {
  protected:
   virtual void InitParamState(const std::string& name, const HashTablePtr& table) = 0;
   virtual void Update(const HashTablePtr& table, const at::Tensor& index, const at::Tensor& grad) = 0;
+  // One optimizer step for `table` straight from gradients that are still sums to be taken (one, or
+  // the two of one plan): the gradient of a unique id is summed over its occurrence list and applied
+  // to its row by the lanes that summed it (recis_csr_gather_reduce*_adamw / _adagrad); the [U, D]
+  // gradient is never written. Bit for bit what summing first and Update give.
+  virtual void UpdatePlanned(const HashTablePtr& table, const std::vector<PlannedGrad>& planned) = 0;
+  virtual const char* Label() const = 0;  // the name the profiler scope carries
   double lr_;
   int64_t grad_accum_steps_ = 1;
   std::vector<std::pair<std::string, HashTablePtr>> params_;  // in the order they were added
@@ -57,7 +63,10 @@ class SparseAdamFamily : public SparseOptimizer {
  protected:
   void InitParamState(const std::string& name, const HashTablePtr& table) override;
   void Update(const HashTablePtr& table, const at::Tensor& index, const at::Tensor& grad) override;
+  void UpdatePlanned(const HashTablePtr& table, const std::vector<PlannedGrad>& planned) override;
+  const char* Label() const override;
   static const char* Prefix();
+  double Decay() const;
 
  private:
   double beta1_, beta2_, eps_, weight_decay_;
@@ -78,6 +87,8 @@ class SparseAdagrad : public SparseOptimizer {
  protected:
   void InitParamState(const std::string& name, const HashTablePtr& table) override;
   void Update(const HashTablePtr& table, const at::Tensor& index, const at::Tensor& grad) override;
+  void UpdatePlanned(const HashTablePtr& table, const std::vector<PlannedGrad>& planned) override;
+  const char* Label() const override { return "FusedSparseAdagrad"; }
 
  private:
   double eps_;

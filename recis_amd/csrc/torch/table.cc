@@ -1,6 +1,9 @@
 #include "table.h"
 
+#include <ATen/record_function.h>
+
 #include <cmath>
+#include <set>
 
 #include "abi_util.h"
 #include "ops.h"
@@ -95,6 +98,16 @@ void Generator::Fill(at::Tensor& t, const std::vector<int64_t>& fan_shape) {
       }
       return;
     }
+    case Kind::kFromTensor: {
+      const int64_t have = source_.size(0);
+      for (int64_t done = 0, rows = t.size(0); done < rows;) {
+        const int64_t take = std::min(rows - done, have - cursor_);
+        t.narrow(0, done, take).copy_(source_.narrow(0, cursor_, take));
+        done += take;
+        cursor_ = (cursor_ + take) % have;
+      }
+      return;
+    }
     case Kind::kTruncNormal: {
       // inverse-CDF sampling between the absolute bounds p2_ (a) and p3_ (b); p0_ = mean, p1_ = std
       const float l = normal_cdf((p2_ - p0_) / p1_);
@@ -175,12 +188,23 @@ GeneratorPtr MakeTruncNormalGenerator(const std::vector<int64_t>& shape, at::Sca
                                         generator);
 }
 
+GeneratorPtr MakeTensorGenerator(const std::vector<int64_t>& shape, at::ScalarType dtype, at::Tensor source) {
+  TORCH_CHECK(source.dim() >= 1 && source.size(0) > 0, "the source tensor must hold at least one row");
+  auto g = c10::make_intrusive<Generator>(Generator::Kind::kFromTensor, shape, dtype);
+  g->SetSource(source.to(dtype));
+  return g;
+}
+
 // ------------------------------------------------------------------------------------ ChildrenInfo
 ChildrenInfo::ChildrenInfo(bool coalesce, const std::vector<std::string>& children)
     : coalesce_(coalesce), children_(children) {
-  TORCH_CHECK(static_cast<int64_t>(children_.size()) <= MaxChildrenNum(), "too many children: ", children_.size());
-  TORCH_CHECK(coalesce_ || children_.size() == 1, "a table that is not coalesced has exactly one child, got ",
-              children_.size());
+  // csrc/embedding/children_info.cc:38-48
+  TORCH_CHECK(!children_.empty(), "empty children");
+  TORCH_CHECK(static_cast<int64_t>(children_.size()) < MaxChildrenNum(), "children size[", children_.size(),
+              "] exceeds max children size[", MaxChildrenNum(), "]");
+  TORCH_CHECK(coalesce_ || children_.size() == 1, "non coalesce has more than one child");
+  std::set<std::string> names(children_.begin(), children_.end());
+  TORCH_CHECK(names.size() == children_.size(), "duplicate child[", children_, "]");
 }
 
 int64_t ChildrenInfo::EncodeId(int64_t id, int64_t index) const {
@@ -207,9 +231,22 @@ std::string ChildrenInfo::ChildAt(int64_t index) const {
   return children_[index];
 }
 
+// ------------------------------------------------------------------------------------ IdMapHolder
+IdMapHolder::~IdMapHolder() {
+  if (map != nullptr) recis_idmap_destroy(map);
+}
+
+int64_t IdMapHolder::IdNum() const {
+  c10::DeviceGuard guard(device);
+  int64_t id_num = 0;
+  check(recis_idmap_stats(map, nullptr, &id_num, nullptr, nullptr, stream_of(device)));
+  return id_num;
+}
+
 // ------------------------------------------------------------------------------------ Slot
 Slot::Slot(const std::string& name, int64_t block_size, at::ScalarType dtype,
-           const std::vector<int64_t>& partial_shape, GeneratorPtr generator, at::Device device, int64_t chunk_rows)
+           const std::vector<int64_t>& partial_shape, GeneratorPtr generator, at::Device device, int64_t chunk_rows,
+           std::shared_ptr<IdMapHolder> map)
     : name_(name),
       block_size_(block_size),
       dtype_(dtype),
@@ -217,23 +254,31 @@ Slot::Slot(const std::string& name, int64_t block_size, at::ScalarType dtype,
       generator_(std::move(generator)),
       device_(device),
       chunk_rows_(chunk_rows),
-      flat_size_(1) {
+      flat_size_(1),
+      map_(std::move(map)) {
   for (int64_t d : row_shape_) flat_size_ *= d;
   generator_->set_device(device);
 }
 
+int64_t Slot::VisibleBlocks() const {
+  if (chunks_.empty()) return 0;
+  const int64_t blocks = (map_->IdNum() + block_size_) / block_size_;
+  const int64_t have = static_cast<int64_t>(chunks_.size()) * (chunk_rows_ / block_size_);
+  return std::min(blocks, have);
+}
+
 std::vector<at::Tensor> Slot::ValuesDeref() {
-  const int64_t per = chunk_rows_ / block_size_;
+  const int64_t per = chunk_rows_ / block_size_, visible = VisibleBlocks();
   std::vector<at::Tensor> out;
-  out.reserve(visible_blocks_);
-  for (int64_t b = 0; b < visible_blocks_; ++b) {
+  out.reserve(visible);
+  for (int64_t b = 0; b < visible; ++b) {
     out.push_back(chunks_[b / per].narrow(0, (b % per) * block_size_, block_size_));
   }
   return out;
 }
 
 at::Tensor Slot::Value() {
-  const int64_t rows = visible_blocks_ * block_size_;
+  const int64_t rows = VisibleBlocks() * block_size_;
   std::vector<int64_t> shape{0};
   shape.insert(shape.end(), row_shape_.begin(), row_shape_.end());
   if (rows == 0) return at::empty(shape, at::TensorOptions().dtype(dtype_).device(device_));
@@ -268,6 +313,11 @@ at::Tensor Slot::GenVal(int64_t rows) {
   return generator_->Generate(shape);
 }
 
+void Slot::SetChunkRows(int64_t chunk_rows) {
+  TORCH_CHECK(chunks_.empty(), "slot ", name_, " already has storage");
+  chunk_rows_ = chunk_rows;
+}
+
 void Slot::EnsureChunks(int64_t n_chunks) {
   std::vector<int64_t> shape{chunk_rows_}, fan{block_size_};
   shape.insert(shape.end(), row_shape_.begin(), row_shape_.end());
@@ -276,22 +326,18 @@ void Slot::EnsureChunks(int64_t n_chunks) {
   while (static_cast<int64_t>(chunks_.size()) < n_chunks) chunks_.push_back(generator_->Generate(shape, fan));
 }
 
-void Slot::Clear() {
-  chunks_.clear();
-  visible_blocks_ = 0;
-}
+void Slot::Clear() { chunks_.clear(); }
 
 // ------------------------------------------------------------------------------------ SlotGroup
-SlotGroup::SlotGroup(int64_t block_size, at::Device device, int64_t chunk_rows)
-    : block_size_(block_size), device_(device), chunk_rows_(chunk_rows) {}
+SlotGroup::SlotGroup(int64_t block_size, at::Device device, int64_t chunk_rows, std::shared_ptr<IdMapHolder> map)
+    : block_size_(block_size), device_(device), chunk_rows_(chunk_rows), map_(std::move(map)) {}
 
 SlotPtr SlotGroup::AppendSlot(const std::string& name, at::ScalarType dtype,
                               const std::vector<int64_t>& partial_shape, GeneratorPtr generator) {
   TORCH_CHECK(name_to_index_.find(name) == name_to_index_.end(), "slot ", name, " already exists");
   auto slot = c10::make_intrusive<Slot>(name, block_size_, dtype, partial_shape, std::move(generator), device_,
-                                        chunk_rows_);
+                                        chunk_rows_, map_);
   slot->EnsureChunks(n_chunks_);  // a late slot catches up with the table
-  slot->SetVisibleBlocks(block_num_);
   name_to_index_[name] = static_cast<int64_t>(slots_.size());
   slots_.push_back(slot);
   return slot;
@@ -331,6 +377,17 @@ int64_t SlotGroup::GetSlotIndex(const std::string& name) {
   return it->second;
 }
 
+int64_t SlotGroup::BlockNum() const {
+  if (n_chunks_ == 0) return 0;
+  return std::min((map_->IdNum() + block_size_) / block_size_, CapacityRows() / block_size_);
+}
+
+void SlotGroup::SetChunkRows(int64_t chunk_rows) {
+  TORCH_CHECK(n_chunks_ == 0, "the table already has storage");
+  chunk_rows_ = chunk_rows;
+  for (auto& s : slots_) s->SetChunkRows(chunk_rows);
+}
+
 void SlotGroup::EnsureRows(int64_t rows) {
   const int64_t need = (rows + chunk_rows_ - 1) / chunk_rows_;
   if (need > n_chunks_) {
@@ -339,18 +396,9 @@ void SlotGroup::EnsureRows(int64_t rows) {
   }
 }
 
-void SlotGroup::SetBlockNum(int64_t block_num) {
-  if (block_num > block_num_) {
-    EnsureRows(block_num * block_size_);
-    block_num_ = block_num;
-    for (auto& s : slots_) s->SetVisibleBlocks(block_num);
-  }
-}
-
 void SlotGroup::Clear() {
   for (auto& s : slots_) s->Clear();
   n_chunks_ = 0;
-  block_num_ = 0;
 }
 
 }  // namespace embedding
@@ -359,30 +407,44 @@ void SlotGroup::Clear() {
 // ------------------------------------------------------------------------------------ Hashtable
 namespace {
 constexpr int64_t kChunkBytes = 8 << 20;
+using recis::BatchPlanPtr;
+using recis::hipabi::block_ptr_table;
+using recis::hipabi::dtype_code;
+using recis::hipabi::index_kind;
+
+int64_t row_bytes_of(at::ScalarType dtype, const std::vector<int64_t>& shape) {
+  int64_t b = static_cast<int64_t>(c10::elementSize(dtype));
+  for (int64_t d : shape) b *= d;
+  return b;
 }
+}  // namespace
 
 Hashtable::Hashtable(int64_t block_size, const std::vector<int64_t>& embedding_shape, at::ScalarType dtype,
                      at::Device device, bool coalesce, const std::vector<std::string>& children,
                      c10::intrusive_ptr<recis::embedding::Generator> generator, int64_t slice_begin,
                      int64_t slice_end, int64_t slice_size)
-    : device_(device), dtype_(dtype), slice_begin_(slice_begin), slice_end_(slice_end), slice_size_(slice_size) {
+    : device_(device),
+      dtype_(dtype),
+      embedding_shape_(embedding_shape),
+      slice_begin_(slice_begin),
+      slice_end_(slice_end),
+      slice_size_(slice_size) {
   TORCH_CHECK(device.is_cuda(), "tables live in GPU memory in this build; got device ", device);
   TORCH_CHECK(block_size > 0, "block_size must be positive");
   if (!device_.has_index()) device_ = at::Device(device.type(), c10::hip::current_device());
-  int64_t row_bytes = static_cast<int64_t>(c10::elementSize(dtype));
-  for (int64_t d : embedding_shape) row_bytes *= d;
+  children_info_ = c10::make_intrusive<recis::embedding::ChildrenInfo>(coalesce, children);
+  {
+    c10::DeviceGuard guard(device_);
+    recis_idmap* m = nullptr;
+    check(recis_idmap_create(0, &m));
+    map_ = std::make_shared<recis::embedding::IdMapHolder>(m, device_);
+  }
+  const int64_t row_bytes = row_bytes_of(dtype, embedding_shape);
   const int64_t chunk_rows = std::max<int64_t>(1, kChunkBytes / std::max<int64_t>(1, row_bytes * block_size)) * block_size;
-  slot_group_ = c10::make_intrusive<recis::embedding::SlotGroup>(block_size, device_, chunk_rows);
+  slot_group_ = c10::make_intrusive<recis::embedding::SlotGroup>(block_size, device_, chunk_rows, map_);
   std::vector<int64_t> partial_shape{block_size};
   partial_shape.insert(partial_shape.end(), embedding_shape.begin(), embedding_shape.end());
   slot_group_->AppendEmbSlot(dtype, partial_shape, std::move(generator));
-  children_info_ = c10::make_intrusive<recis::embedding::ChildrenInfo>(coalesce, children);
-  c10::DeviceGuard guard(device_);
-  check(recis_idmap_create(0, &id_map_));
-}
-
-Hashtable::~Hashtable() {
-  if (id_map_ != nullptr) recis_idmap_destroy(id_map_);
 }
 
 c10::intrusive_ptr<Hashtable> Hashtable::Make(int64_t block_size, const std::vector<int64_t>& embedding_shape,
@@ -392,6 +454,14 @@ c10::intrusive_ptr<Hashtable> Hashtable::Make(int64_t block_size, const std::vec
                                               int64_t slice_begin, int64_t slice_end, int64_t slice_size) {
   return c10::make_intrusive<Hashtable>(block_size, embedding_shape, dtype, device, coalesce, children,
                                         std::move(generator), slice_begin, slice_end, slice_size);
+}
+
+void Hashtable::Reserve(int64_t rows) {
+  if (rows <= 0) return;
+  c10::DeviceGuard guard(device_);
+  const int64_t bs = slot_group_->BlockSize();
+  slot_group_->SetChunkRows((rows + 1 + bs - 1) / bs * bs);
+  check(recis_idmap_reserve(map_->map, rows, stream_of(device_)));
 }
 
 at::Tensor Hashtable::OnDevice(const at::Tensor& ids) const {
@@ -406,9 +476,11 @@ at::Tensor Hashtable::OnDevice(const at::Tensor& ids) const {
 void Hashtable::MakeRoom(int64_t incoming) {
   auto& sg = *slot_group_;
   int64_t ub = 0;
-  check(recis_idmap_bounds(id_map_, &ub, nullptr));
+  check(recis_idmap_bounds(map_->map, &ub, nullptr));
   if (ub + 1 > sg.CapacityRows()) {
     ub = ids_num();  // synchronises
+    // Leave room for many calls of this size, unless storage grows in chunks far larger than a batch
+    // (a pre-sized table): rows are cheap, pipeline bubbles are not.
     const bool roomy = sg.ChunkRows() <= 32 * std::max<int64_t>(incoming, 1);
     const int64_t want = ub + 1 + std::max<int64_t>((roomy ? 16 : 2) * incoming, sg.BlockSize());
     if (want > sg.CapacityRows() && (roomy || ub + 1 + incoming > sg.CapacityRows())) sg.EnsureRows(want);
@@ -416,24 +488,23 @@ void Hashtable::MakeRoom(int64_t incoming) {
   if (sg.CapacityRows() == 0) sg.EnsureRows(1);
 }
 
-// block_num = (id_num + block_size) / block_size (csrc/embedding/hashtable.cc:255-261)
-void Hashtable::SyncBlockNum() {
-  auto& sg = *slot_group_;
-  sg.SetBlockNum((ids_num() + sg.BlockSize()) / sg.BlockSize());
-}
+int64_t Hashtable::ids_num() { return map_->IdNum(); }
 
-int64_t Hashtable::ids_num() {
+std::vector<int64_t> Hashtable::IdMapStats() {
   c10::DeviceGuard guard(device_);
-  int64_t id_num = 0;
-  check(recis_idmap_stats(id_map_, nullptr, &id_num, nullptr, nullptr, stream_of(device_)));
-  return id_num;
+  std::vector<int64_t> v(4, 0);
+  check(recis_idmap_stats(map_->map, &v[0], &v[1], &v[2], &v[3], stream_of(device_)));
+  int bits = 0;
+  check(recis_hip_poll_device_errors(&bits));  // the call above has waited for the stream already
+  TORCH_CHECK(bits == 0, "librecis_hip: device-side errors in earlier kernels (bits ", bits, ")");
+  return v;
 }
 
 at::Tensor Hashtable::InsertLookupIndex(const at::Tensor& ids) {
   c10::DeviceGuard guard(device_);
   at::Tensor i = OnDevice(ids);
   at::Tensor index = at::empty(i.sizes(), i.options());
-  check(recis_idmap_lookup(id_map_, i.data_ptr<int64_t>(), i.numel(), index.data_ptr<int64_t>(), stream_of(device_)));
+  check(recis_idmap_lookup(map_->map, i.data_ptr<int64_t>(), i.numel(), index.data_ptr<int64_t>(), stream_of(device_)));
   MakeRoom(i.numel());
   return index;
 }
@@ -442,9 +513,13 @@ at::Tensor Hashtable::LookupIndexReadOnly(const at::Tensor& ids) {
   c10::DeviceGuard guard(device_);
   at::Tensor i = OnDevice(ids);
   at::Tensor index = at::empty(i.sizes(), i.options());
-  check(recis_idmap_lookup_readonly(id_map_, i.data_ptr<int64_t>(), i.numel(), index.data_ptr<int64_t>(),
+  check(recis_idmap_lookup_readonly(map_->map, i.data_ptr<int64_t>(), i.numel(), index.data_ptr<int64_t>(),
                                     stream_of(device_)));
   return index;
+}
+
+at::Tensor Hashtable::LookupIndex(const at::Tensor& ids, bool readonly) {
+  return readonly ? LookupIndexReadOnly(ids) : InsertLookupIndex(ids);
 }
 
 std::tuple<at::Tensor, at::Tensor> Hashtable::EmbeddingLookup(const at::Tensor& ids, bool readonly) {
@@ -457,6 +532,8 @@ std::tuple<at::Tensor, at::Tensor> Hashtable::EmbeddingLookup(const at::Tensor& 
   }
   auto emb_slot = slot_group_->EmbSlot();
   at::Tensor emb = recis::functional::block_gather(index, emb_slot->Chunks(), emb_slot->ChunkRows(), kNullIndex, readonly);
+  last_lookup_index_ = index;
+  last_lookup_unique_ = recis::functional::known_unique(ids);
   return std::make_tuple(index, emb);
 }
 
@@ -503,17 +580,17 @@ void Hashtable::Clear() {
 
 void Hashtable::ClearId() {
   c10::DeviceGuard guard(device_);
-  check(recis_idmap_clear(id_map_, stream_of(device_)));
+  check(recis_idmap_clear(map_->map, stream_of(device_)));
 }
 
 std::tuple<at::Tensor, at::Tensor> Hashtable::ids_map() {
   c10::DeviceGuard guard(device_);
   int64_t live = 0, count = 0;
   void* stream = stream_of(device_);
-  check(recis_idmap_stats(id_map_, &live, nullptr, nullptr, nullptr, stream));
+  check(recis_idmap_stats(map_->map, &live, nullptr, nullptr, nullptr, stream));
   auto opt = at::TensorOptions().device(device_).dtype(at::kLong);
   at::Tensor ids = at::empty({live}, opt), index = at::empty({live}, opt);
-  check(recis_idmap_snapshot(id_map_, ids.data_ptr<int64_t>(), index.data_ptr<int64_t>(), live, &count, stream));
+  check(recis_idmap_snapshot(map_->map, ids.data_ptr<int64_t>(), index.data_ptr<int64_t>(), live, &count, stream));
   TORCH_CHECK(count == live, "id map changed during the snapshot: ", count, " keys, expected ", live);
   return std::make_tuple(ids, index);
 }
@@ -527,7 +604,7 @@ void Hashtable::Delete(const at::Tensor& ids, const at::Tensor& index, const std
   c10::DeviceGuard guard(device_);
   at::Tensor i = OnDevice(ids).view({-1}), x = OnDevice(index).view({-1});
   TORCH_CHECK(i.numel() == x.numel(), "ids and index differ in length");
-  check(recis_idmap_erase(id_map_, i.data_ptr<int64_t>(), x.data_ptr<int64_t>(), i.numel(), stream_of(device_)));
+  check(recis_idmap_erase(map_->map, i.data_ptr<int64_t>(), x.data_ptr<int64_t>(), i.numel(), stream_of(device_)));
   const int64_t keep = preserve_slot.empty() ? -1 : slot_group_->GetSlotIndex(preserve_slot);
   auto slots = slot_group_->Slots();
   for (int64_t s = 0; s < static_cast<int64_t>(slots.size()); ++s) {
@@ -535,19 +612,230 @@ void Hashtable::Delete(const at::Tensor& ids, const at::Tensor& index, const std
   }
 }
 
+std::tuple<at::Tensor, at::Tensor> Hashtable::EvictOlder(const std::string& stamp_slot, int64_t threshold) {
+  c10::DeviceGuard guard(device_);
+  auto stamps = slot_group_->GetSlotByName(stamp_slot);
+  TORCH_CHECK((stamps->Dtype() == at::kLong || stamps->Dtype() == at::kInt) && stamps->FlatSize() == 1,
+              "the stamp slot must be int32/int64 of width 1");
+  void* stream = stream_of(device_);
+  int64_t live = 0, count = 0;
+  check(recis_idmap_stats(map_->map, &live, nullptr, nullptr, nullptr, stream));
+  auto opt = at::TensorOptions().device(device_).dtype(at::kLong);
+  at::Tensor ids = at::empty({live}, opt), index = at::empty({live}, opt);
+  if (!stamps->Chunks().empty()) {
+    at::Tensor tab = block_ptr_table(stamps->Chunks());
+    check(recis_idmap_evict_older(map_->map, reinterpret_cast<const void* const*>(tab.data_ptr()),
+                                  static_cast<int64_t>(stamps->Chunks().size()), stamps->ChunkRows(),
+                                  stamps->Dtype() == at::kLong ? 1 : 0, threshold, ids.data_ptr<int64_t>(),
+                                  index.data_ptr<int64_t>(), live, &count, stream));
+  }
+  ids = ids.narrow(0, 0, count);
+  index = index.narrow(0, 0, count);
+  if (count) {
+    const int64_t keep = slot_group_->GetSlotIndex(stamp_slot);
+    auto slots = slot_group_->Slots();
+    for (int64_t s = 0; s < static_cast<int64_t>(slots.size()); ++s) {
+      if (s != keep) slots[s]->IndexInsert(index, slots[s]->GenVal(count));
+    }
+  }
+  return std::make_tuple(ids, index);
+}
+
+// ------------------------------------------------------------------------------------ batch plan
+BatchPlanPtr Hashtable::PlanLookup(const std::vector<at::Tensor>& ids, const c10::optional<std::vector<int64_t>>& tags,
+                                   bool wait, bool need_inverse, bool need_pos) {
+  c10::DeviceGuard guard(device_);
+  BatchPlanPtr plan = recis::BatchPlan::Make(ids, tags, map_->map, wait, need_inverse, need_pos);
+  int64_t call = 0;
+  check(recis_idmap_last_call(map_->map, &call));
+  plan->NoteLookup(this, call);
+  MakeRoom(wait ? plan->U() : plan->n());
+  return plan;
+}
+
+c10::optional<at::Tensor> Hashtable::PlanIndex(const BatchPlanPtr& plan) {
+  if (plan->LookupCall(this) != 0 && plan->IndexBufRaw().defined()) return plan->IndexBufRaw();
+  return c10::nullopt;
+}
+
+at::Tensor Hashtable::LookupIndexCounted(const BatchPlanPtr& plan, bool make_room) {
+  c10::DeviceGuard guard(device_);
+  at::Tensor out = at::empty_like(plan->unique_buf());
+  check(recis_idmap_lookup_counted(map_->map, plan->unique_buf().data_ptr<int64_t>(), plan->unique_buf().numel(),
+                                   plan->counts().data_ptr<int64_t>(), out.data_ptr<int64_t>(), stream_of(device_)));
+  int64_t call = 0;
+  check(recis_idmap_last_call(map_->map, &call));
+  plan->NoteLookup(this, call);
+  if (make_room) MakeRoom(plan->n());
+  return out;
+}
+
+void Hashtable::SettleCount(int64_t n_true, const c10::optional<BatchPlanPtr>& plan) {
+  const int64_t call = plan.has_value() && plan->defined() ? (*plan)->LookupCall(this) : 0;
+  if (call == 0) {
+    check(recis_idmap_settle_count(map_->map, n_true));
+  } else {
+    check(recis_idmap_settle_call(map_->map, call, n_true));
+  }
+}
+
+at::Tensor Hashtable::SettleLookup(const at::Tensor& index_buf, int64_t n_true, const BatchPlanPtr& plan) {
+  SettleCount(n_true, plan);
+  MakeRoom(n_true);
+  return index_buf.narrow(0, 0, n_true);
+}
+
+at::Tensor Hashtable::ExpandRows(const BatchPlanPtr& plan, const at::Tensor& row_index,
+                                 const c10::optional<at::Tensor>& weight, const c10::optional<std::string>& stamp_slot,
+                                 const c10::optional<at::Tensor>& stamp_value) {
+  c10::DeviceGuard guard(device_);
+  auto emb = slot_group_->EmbSlot();
+  const auto& chunks = emb->Chunks();
+  TORCH_CHECK(!chunks.empty(), "the table has no rows yet");
+  TORCH_CHECK(row_index.is_cuda() && row_index.scalar_type() == at::kLong && row_index.is_contiguous(),
+              "row_index must be a contiguous int64 GPU tensor");
+  const int64_t D = emb->FlatSize(), n = plan->n();
+  at::Tensor w;
+  if (weight.has_value() && weight->defined()) {
+    recis::hipabi::require_gpu(*weight, "weight");
+    w = weight->contiguous();
+  }
+  at::Tensor table = block_ptr_table(chunks), stamp_table;
+  const int64_t* stamp_ptr = nullptr;
+  if (stamp_slot.has_value()) {
+    auto stamps = slot_group_->GetSlotByName(*stamp_slot);
+    TORCH_CHECK(stamps->Dtype() == at::kLong && stamps->FlatSize() == 1 && stamps->Chunks().size() == chunks.size(),
+                "the stamp slot must be an int64 slot of width 1 of this table");
+    TORCH_CHECK(stamp_value.has_value() && stamp_value->is_cuda() && stamp_value->scalar_type() == at::kLong &&
+                    stamp_value->numel() == 1,
+                "the stamp value must be a one-element int64 GPU tensor");
+    stamp_table = block_ptr_table(stamps->Chunks());
+    stamp_ptr = stamp_value->data_ptr<int64_t>();
+  }
+  at::Tensor out = at::empty({n, D}, chunks[0].options());
+  const int code = dtype_code(dtype_);
+  check(recis_csr_expand_rows_stamped(
+      nullptr, reinterpret_cast<void* const*>(table.data_ptr()), static_cast<int64_t>(chunks.size()), emb->ChunkRows(),
+      row_index.data_ptr<int64_t>(), code, w.defined() ? w.data_ptr() : nullptr,
+      w.defined() ? dtype_code(w.scalar_type()) : 0, plan->row_start().data_ptr<int32_t>(),
+      plan->occ().data_ptr<int32_t>(), plan->hot_items().data_ptr<int32_t>(), plan->hot_cap(),
+      plan->counts().data_ptr<int64_t>(), out.data_ptr(), code, plan->U_bound(), n, D,
+      stamp_table.defined() ? reinterpret_cast<void* const*>(stamp_table.data_ptr()) : nullptr, stamp_ptr,
+      stream_of(device_)));
+  return out;
+}
+
+// ------------------------------------------------------------------------------------ gradients
 void Hashtable::AcceptGrad(const at::Tensor& grad_index, const at::Tensor& grad) {
+  // the index tensor the last embedding_lookup returned for ids that are known to be distinct has
+  // no duplicates either
+  const bool unique = last_lookup_unique_ && last_lookup_index_.defined() &&
+                      grad_index.data_ptr() == last_lookup_index_.data_ptr() &&
+                      grad_index.numel() == last_lookup_index_.numel() &&
+                      grad_index._version() == last_lookup_index_._version();
+  AcceptGradEx(grad_index, grad, unique, 0);
+}
+
+void Hashtable::AcceptGradEx(const at::Tensor& grad_index, const at::Tensor& grad, bool unique, int64_t key) {
   TORCH_CHECK(grad_index.scalar_type() == at::kLong, "grad_index must be int64");
+  SumPlanned();  // a gradient waiting to be summed comes first, as it was handed over first
   TORCH_CHECK(grad.scalar_type() == dtype_ ||
                   (grad.scalar_type() == at::kFloat && (dtype_ == at::kBFloat16 || dtype_ == at::kHalf)),
               "grad dtype ", grad.scalar_type(), " does not match the table (", dtype_, ")");
+  if (key != 0) {
+    for (const auto& k : grad_keys_) {
+      if (k.first == key && grad_[k.second].sizes() == grad.sizes()) {
+        grad_[k.second] = grad_[k.second] + grad;
+        return;
+      }
+    }
+    grad_keys_.emplace_back(key, grad_.size());
+  }
   grad_index_.push_back(grad_index);
   grad_.push_back(grad);
+  grad_unique_.push_back(unique);
+}
+
+void Hashtable::AcceptPlannedGrad(const at::Tensor& index, const BatchPlanPtr& plan, const std::vector<at::Tensor>& rows,
+                                  bool in_parts, const at::Tensor& src, const c10::optional<at::Tensor>& coef,
+                                  const c10::optional<at::Tensor>& cover, int64_t key, bool may_miss) {
+  TORCH_CHECK(!rows.empty() && (in_parts || rows.size() == 1), "accept_planned_grad: one array, or several in parts");
+  PlannedGrad g;
+  g.index = index;
+  g.plan = plan;
+  g.rows = rows;
+  g.in_parts = in_parts;
+  g.src = src;
+  if (coef.has_value() && coef->defined()) g.coef = *coef;
+  if (cover.has_value() && cover->defined()) g.cover = *cover;
+  g.key = key;
+  g.may_miss = may_miss;
+  if (grad_.empty() && planned_.size() == 1 && OneLaunchSums(planned_[0], g)) {
+    planned_.push_back(std::move(g));
+    return;
+  }
+  if (!grad_.empty() || !planned_.empty()) {
+    SumPlanned();
+    AcceptSummed(g, SumOf(g));
+    return;
+  }
+  planned_.push_back(std::move(g));
+}
+
+// Whether two unsummed gradients are the two inputs of one recis_csr_gather_reduce2* launch: of one
+// plan and the same rows (one key), whole (no cover), each float32 or of the table's type, at most
+// one of them in parts (which then has no coefficients and at most 8 parts).
+bool Hashtable::OneLaunchSums(const PlannedGrad& a, const PlannedGrad& b) const {
+  if (a.plan.get() != b.plan.get() || a.key == 0 || a.key != b.key || a.may_miss != b.may_miss ||
+      a.cover.defined() || b.cover.defined()) {
+    return false;
+  }
+  if (a.index.sizes() != b.index.sizes()) return false;
+  if (a.in_parts && b.in_parts) return false;
+  for (const PlannedGrad* g : {&a, &b}) {
+    if (g->in_parts && (g->coef.defined() || g->rows.size() > 8)) return false;
+    const auto t = g->rows[0].scalar_type();
+    if (t != at::kFloat && t != dtype_) return false;
+  }
+  return true;
+}
+
+at::Tensor Hashtable::SumOf(const PlannedGrad& g) const {
+  if (!g.in_parts) return recis::functional::csr_gather_reduce(g.rows[0], g.plan, g.src, g.coef, g.cover);
+  return recis::functional::csr_gather_reduce_parts(g.rows, g.plan, g.src);
+}
+
+void Hashtable::AcceptSummed(const PlannedGrad& g, at::Tensor summed) {
+  at::Tensor index = g.index.numel() > summed.size(0) ? g.index.narrow(0, 0, summed.size(0)) : g.index;
+  if (g.may_miss) {  // keys the table does not hold take no gradient
+    at::Tensor keep = index.ge(0);
+    index = index.masked_select(keep);
+    summed = summed.index({keep});
+  }
+  if (summed.scalar_type() != dtype_ && dtype_ == at::kFloat) summed = summed.to(dtype_);
+  AcceptGradEx(index, summed, true, g.key);
+}
+
+void Hashtable::SumPlanned() {
+  std::vector<PlannedGrad> planned;
+  planned.swap(planned_);
+  for (const auto& g : planned) AcceptSummed(g, SumOf(g));
+}
+
+std::vector<PlannedGrad> Hashtable::TakePlannedGrad() {
+  if (planned_.empty() || !grad_.empty()) return {};
+  if (planned_.size() == 1 && planned_[0].in_parts) return {};  // parts alone: no fused row update takes them
+  std::vector<PlannedGrad> planned;
+  planned.swap(planned_);
+  if (planned.size() == 2 && planned[0].in_parts) std::swap(planned[0], planned[1]);
+  return planned;
 }
 
 // The sparse COO gradient as the reference builds it (csrc/embedding/hashtable.cc:90-134),
 // including its layout when rows repeat: the inverse positions as indices and an N-row value buffer
 // whose first U rows hold the sums.
 at::Tensor Hashtable::grad(int64_t accumulate_steps) {
+  SumPlanned();
   at::Tensor index = at::cat(grad_index_, 0), g = at::cat(grad_, 0);
   auto uniq = at::_unique(index, /*sorted=*/false, /*return_inverse=*/true);
   const at::Tensor& values = std::get<0>(uniq);
@@ -571,16 +859,20 @@ at::Tensor Hashtable::grad(int64_t accumulate_steps) {
 }
 
 std::tuple<at::Tensor, at::Tensor> Hashtable::GradPairs(int64_t accumulate_steps) {
+  SumPlanned();
+  TORCH_CHECK(!grad_.empty(), "the table holds no gradient");
   at::Tensor index = grad_index_.size() == 1 ? grad_index_[0] : at::cat(grad_index_, 0);
   at::Tensor g = grad_.size() == 1 ? grad_[0] : at::cat(grad_, 0);
-  auto uniq = at::_unique(index, /*sorted=*/false, /*return_inverse=*/true);
-  if (std::get<0>(uniq).numel() != index.numel()) {
-    std::vector<int64_t> shape = g.sizes().vec();
-    shape[0] = std::get<0>(uniq).numel();
-    at::Tensor summed = at::zeros(shape, g.options());
-    summed.index_add_(0, std::get<1>(uniq).view({-1}), g);
-    index = std::get<0>(uniq);
-    g = summed;
+  if (!(grad_unique_.size() == 1 && grad_unique_[0])) {  // one gradient over distinct rows needs no merge
+    auto uniq = at::_unique(index, /*sorted=*/false, /*return_inverse=*/true);
+    if (std::get<0>(uniq).numel() != index.numel()) {
+      std::vector<int64_t> shape = g.sizes().vec();
+      shape[0] = std::get<0>(uniq).numel();
+      at::Tensor summed = at::zeros(shape, g.options());
+      summed.index_add_(0, std::get<1>(uniq).view({-1}), g);
+      index = std::get<0>(uniq);
+      g = summed;
+    }
   }
   if (accumulate_steps != 1) g = g / accumulate_steps;
   return std::make_tuple(index, g);
@@ -589,14 +881,11 @@ std::tuple<at::Tensor, at::Tensor> Hashtable::GradPairs(int64_t accumulate_steps
 void Hashtable::ClearGrad() {
   grad_index_.clear();
   grad_.clear();
-}
-
-c10::intrusive_ptr<recis::embedding::SlotGroup> Hashtable::SlotGroup() {
-  SyncBlockNum();
-  return slot_group_;
+  grad_unique_.clear();
+  grad_keys_.clear();
+  planned_.clear();
 }
 
 c10::intrusive_ptr<recis::embedding::Slot> Hashtable::GetSlot(const std::string& name) {
-  SyncBlockNum();
   return slot_group_->GetSlotByName(name);
 }

@@ -15,7 +15,8 @@ from ...ragged.tensor import RaggedTensor
 from ..functional.embedding_ops import ragged_embedding_segment_reduce
 from ..hashtable_hook import AdmitHook, FilterHook
 from ..initializers import ConstantInitializer, Initializer
-from .hashtable import (GradIDMeanFunction, HashTable, HashTableLookupHelpFunction, gen_slice)
+from .hashtable import (GradIDMeanFunction, HashTable, HashTableLookupHelpFunction, accept_planned_grad, gen_slice,
+                        plan_lookup)
 
 
 class _Done:
@@ -131,7 +132,11 @@ class LookupPoolFunction(torch.autograd.Function):
     gradients per unique row over the plan and hands (row index, gradient) to the table."""
 
     @staticmethod
-    def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly, unit_segments=False):
+    def forward(ctx, backward_holder, impl, plan, weight, offsets, combiner, readonly, unit_segments=False,
+                split=None):
+        """``split``: row counts to cut the pooled output into (one part per feature of a group that is pooled
+        in one go); the parts are returned as separate outputs, views of the one buffer, and backward takes
+        their gradients as they come: slices of one buffer are used in place, anything else is concatenated."""
         late_count = not readonly
         if readonly:
             index = impl.lookup_index(plan.unique, True)
@@ -143,34 +148,58 @@ class LookupPoolFunction(torch.autograd.Function):
             # make_plan for this table brings them along (dedup and lookup were one pass).
             index = impl.plan_index(plan)
             if index is None:
-                index = impl.lookup_index_unsettled(plan)
-        chunks, chunk_rows = impl.emb_blocks()
+                index = impl.lookup_index_counted(plan, True)
         if unit_segments:
             # one id per segment (sum == mean == the row itself): every unique row is read once and
             # written to its occurrences, instead of one index chase per output row
-            out = ops.plan_expand_rows(plan, plan.n, blocks=chunks, block_size=chunk_rows,
-                                       row_index=index, weight=weight)
+            out = impl.expand_rows(plan, index, weight, None, None)
         else:
+            chunks, chunk_rows = impl.emb_blocks()
             out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets,
                                                     combiner)
         ctx.impl, ctx.plan, ctx.combiner, ctx.readonly, ctx.late_count = impl, plan, combiner, readonly, late_count
+        ctx.split, ctx.out_shape = split, tuple(out.shape)
         ctx.save_for_backward(index, weight, offsets)
         ctx.mark_non_differentiable(index)
-        return index, out
+        if split is None:
+            return index, out
+        return (index,) + tuple(torch.split(out, split))
 
     @staticmethod
-    def backward(ctx, _grad_index, grad):
+    def backward(ctx, _grad_index, *grads):
         index, weight, offsets = ctx.saved_tensors
         if ctx.late_count:
             ctx.impl.settle_count(ctx.plan.U, ctx.plan)
             index = index[: ctx.plan.U]
+        grad = grads[0] if ctx.split is None else _joined(grads, ctx.split, ctx.out_shape)
         # sum / mean: the gradient of a unique row is a gather-reduce over its occurrence list; it is handed
         # over unsummed, so that the optimizer step can sum and update the row in one launch (keys the table
         # does not hold carry a negative index and take no gradient)
         src, coef = ctx.plan.src_coef_for_pool(offsets.contiguous(), weight, ctx.combiner == "mean")
-        ctx.impl.accept_planned_grad(index, ctx.plan, grad.contiguous(), src, coef,
-                                     key=None if ctx.readonly else ctx.plan.serial, may_miss=ctx.readonly)
-        return None, None, None, None, None, None, None, None
+        accept_planned_grad(ctx.impl, index, ctx.plan, grad.contiguous(), src, coef,
+                            key=None if ctx.readonly else ctx.plan.serial, may_miss=ctx.readonly)
+        return (None,) * 9
+
+
+def _joined(grads, split, shape):
+    """The gradients of the parts of one pooled output as one ``shape`` tensor: in place when they are
+    consecutive slices of one buffer (what a caller that keeps its gradients in one array hands over),
+    concatenated otherwise (a missing gradient counts as zeros)."""
+    like = next((g for g in grads if g is not None), None)
+    if like is None:
+        return torch.zeros(shape, device="cuda")
+    first = grads[0]
+    if first is not None and first.is_contiguous():
+        at = first.data_ptr()
+        for g, rows in zip(grads, split):
+            if g is None or g.dtype != first.dtype or not g.is_contiguous() or g.data_ptr() != at \
+                    or g.untyped_storage().data_ptr() != first.untyped_storage().data_ptr():
+                break
+            at += rows * shape[1] * g.element_size()
+        else:
+            whole = torch.as_strided(first, shape, (shape[1], 1), first.storage_offset())
+            return whole
+    return torch.cat([g if g is not None else like.new_zeros((rows, shape[1])) for g, rows in zip(grads, split)])
 
 
 class LookupTileFunction(torch.autograd.Function):
@@ -190,7 +219,7 @@ class LookupTileFunction(torch.autograd.Function):
         else:
             index = impl.plan_index(plan)   # a plan made for this table brings the rows along
             if index is None:
-                index = impl.lookup_index_unsettled(plan)
+                index = impl.lookup_index_counted(plan, True)
             index = impl.settle_lookup(index, U, plan)
         chunks, chunk_rows = impl.emb_blocks()
         rows = ops.block_gather(index, chunks, chunk_rows, -1, readonly)
@@ -213,9 +242,9 @@ class LookupTileFunction(torch.autograd.Function):
             parts = [(g if g is not None else like.new_zeros((n, D))).reshape(n, D) for g, n in zip(grads, n_rows)]
             key = None if ctx.readonly else plan.serial
             if len(parts) <= 8 and len({p.dtype for p in parts}) == 1:
-                ctx.impl.accept_planned_grad(index, plan, parts, src, key=key, may_miss=ctx.readonly)
+                accept_planned_grad(ctx.impl, index, plan, parts, src, key=key, may_miss=ctx.readonly)
             else:
-                ctx.impl.accept_planned_grad(index, plan, torch.cat(parts), src, key=key, may_miss=ctx.readonly)
+                accept_planned_grad(ctx.impl, index, plan, torch.cat(parts), src, key=key, may_miss=ctx.readonly)
         return (None,) * 7
 
 
@@ -237,15 +266,17 @@ def make_plan(hashtable: HashTable, ids, offsets, opt, has_weight=False, unit_se
     if (hashtable.training and opt.trainable and opt.admit_hook is None
             and _pools_out_of_the_table(hashtable, opt, n_occ, offsets.numel())):
         lean = bool(unit_segments)
-        return hashtable._hashtable_impl.plan_lookup(ids, need_inverse=not lean, tags=tags)
+        return plan_lookup(hashtable._hashtable_impl, ids, need_inverse=not lean, tags=tags)
     return ops.ids_unique_plan(ids, wait=False, need_pos=False, tags=tags)
 
 
-def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False, combiner_kwargs=None):
+def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segments=False, combiner_kwargs=None,
+                    split=None):
     """Rows of the plan's unique ids pooled per segment. Sum / mean over a float table go
     through ``LookupPoolFunction`` (pooling reads the table directly); everything else looks the
     rows up first and pools the copy. ``unit_segments``: the caller built ``offsets`` as
-    0, 1, 2, ... (dense ``[B, 1]`` id tensors), so segment i holds exactly occurrence i."""
+    0, 1, 2, ... (dense ``[B, 1]`` id tensors), so segment i holds exactly occurrence i.
+    ``split``: return the pooled rows cut into parts of these row counts (a tuple)."""
     impl = hashtable._hashtable_impl
     id_mean = opt.grad_reduce_by == "id" and hashtable.training and opt.trainable
     if _pools_out_of_the_table(hashtable, opt, plan.n, offsets.numel()):
@@ -257,20 +288,21 @@ def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segme
                 from .hashtable_hook_impl import HashtableHookFactory, ReadOnlyHookImpl
                 admit = HashtableHookFactory().create_admit_hook(hashtable, opt.admit_hook)
                 assert isinstance(admit, ReadOnlyHookImpl), "admit hook only support ReadOnlyHook yet, but got: %s" % admit
-            index, out = LookupPoolFunction.apply(hashtable._backward_holder, impl, plan, weight, offsets,
-                                                  opt.combiner, readonly, unit_segments)
+            index, *outs = LookupPoolFunction.apply(hashtable._backward_holder, impl, plan, weight, offsets,
+                                                    opt.combiner, readonly, unit_segments, split)
             if not isinstance(hashtable._filter_hook_impl, torch.nn.Identity):
                 # a step filter stamps the looked-up rows: it needs the rows proper (the index may
                 # be the full-length buffer of the forward that does not wait for the count)
                 hashtable._filter_hook_impl(index[: plan.U] if not readonly else index)
-            return out
+            return outs[0] if split is None else tuple(outs)
         readonly = (not hashtable.training) or opt.admit_hook is not None
         index = impl.lookup_index(plan.unique.detach(), readonly)
         if hashtable.training and not readonly:
             hashtable._filter_hook_impl(index)
         chunks, chunk_rows = impl.emb_blocks()
-        return ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets,
-                                                 opt.combiner)
+        out = ops.segment_reduce_forward_blocks(chunks, chunk_rows, index, weight, plan.inverse, offsets,
+                                                opt.combiner)
+        return out if split is None else torch.split(out, split)
     emb = lookup_unique_rows(hashtable, plan.unique, opt.admit_hook, opt.trainable)
     inverse = plan.inverse
     if id_mean:
@@ -279,9 +311,10 @@ def lookup_and_pool(hashtable: HashTable, plan, weight, offsets, opt, unit_segme
         inverse, plan = None, None
     if weight is not None and weight.dtype != emb.dtype:
         weight = weight.to(emb.dtype)
-    return ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner,
-                                           combiner_kwargs if combiner_kwargs is not None else opt.combiner_kwargs,
-                                           plan=plan)
+    out = ragged_embedding_segment_reduce(emb, weight, inverse, offsets, opt.combiner,
+                                          combiner_kwargs if combiner_kwargs is not None else opt.combiner_kwargs,
+                                          plan=plan)
+    return out if split is None else torch.split(out, split)
 
 
 class DynamicEmbedding(torch.nn.Module):
@@ -325,7 +358,7 @@ class DynamicEmbedding(torch.nn.Module):
     def forward(self, input_ids, input_weights=None):
         opt = self._emb_opt
         val, offsets, weight, shape = self.deal_with_tensor(input_ids)
-        dev = self._hashtable._hashtable_impl.device
+        dev = self._hashtable._impl_device
         val, offsets = val.to(dev), offsets.to(dev)
         if input_weights is not None:
             weight = input_weights

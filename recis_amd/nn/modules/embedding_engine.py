@@ -23,7 +23,7 @@ from ... import ops
 from ...ragged.tensor import RaggedTensor
 from ..functional.embedding_ops import RaggedTileParts
 from .embedding import EmbeddingOption, LookupTileFunction, lookup_and_pool, lookup_unique_rows, make_plan
-from .hashtable import HashTable, gen_slice
+from .hashtable import HashTable, gen_slice, plan_lookup
 
 
 def _key(text):
@@ -119,7 +119,7 @@ class EmbeddingEngine(torch.nn.Module):
         plans = {}
         for gkey, grp in self._groups.items():
             table = self._tables[gkey]
-            dev = table._hashtable_impl.device
+            dev = table._impl_device
             info = table._hashtable_impl.children_info()
             tag_of = self._tags.get(gkey)
             if tag_of is None:  # the 12-bit table index of every feature's shared name, fixed after construction
@@ -174,7 +174,7 @@ class EmbeddingEngine(torch.nn.Module):
                     if opt0.combiner == "tile":
                         if (table.training and opt0.trainable and opt0.admit_hook is None
                                 and table._dtype in (torch.float32, torch.bfloat16, torch.float16)):
-                            plan = table._hashtable_impl.plan_lookup(ids, tags=tags)   # dedup + find-or-insert, one pass
+                            plan = plan_lookup(table._hashtable_impl, ids, tags=tags)   # dedup + find-or-insert, one pass
                         else:
                             plan = ops.ids_unique_plan(ids, wait=False, need_pos=False, tags=tags)
                     else:  # lean (no per-occurrence arrays) only if no other option can come to share it
@@ -210,9 +210,8 @@ class EmbeddingEngine(torch.nn.Module):
                     for name, part, shape in zip(names, parts, shapes):
                         outputs[name] = part if len(shape) == 1 else part.reshape(tuple(shape) + (part.shape[1],))
                     continue
-                pooled = lookup_and_pool(table, plan, weight, offsets, opt0, unit_segments=all_unit)
-                width = pooled.shape[1]
-                for name, part, shape in zip(names, torch.split(pooled, seg_counts), shapes):
+                parts = lookup_and_pool(table, plan, weight, offsets, opt0, unit_segments=all_unit, split=seg_counts)
+                for name, part, shape in zip(names, parts, shapes):
                     # [segments, width] already is the answer for a 1-D batch shape: no extra view node
-                    outputs[name] = part if len(shape) == 1 else part.reshape(tuple(shape) + (width,))
+                    outputs[name] = part if len(shape) == 1 else part.reshape(tuple(shape) + (part.shape[1],))
         return outputs

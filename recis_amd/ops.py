@@ -739,208 +739,47 @@ class IdMap:
 _HOT_LEN, _HOT_CHUNK = 64, 2048  # RECIS_PLAN_HOT_LEN / RECIS_PLAN_HOT_CHUNK of the library
 
 
-_STAGED = {}  # stream -> the plan whose count is on its way to that stream's staging word
-
-
-class BatchPlan:
-    """Dedup of one batch of ids plus the occurrence lists per unique id.
-
-    ``unique`` [U], ``inverse`` int32 [N] (``unique[inverse] == ids``), ``row_start`` int32
-    [N + 1] and ``occ`` int32 [N]: the occurrences of unique id ``u`` are
-    ``occ[row_start[u]:row_start[u + 1]]``; ``pos`` [N] is the position of each occurrence
-    in ``occ``. ``U`` is the host copy of the unique count. A plan made with ``wait=False``
-    fetches it on first use of ``U`` / ``unique`` (the count is on its way by then);
-    ``unique_buf`` [N] and ``counts`` (device) are there at once, for work that can be
-    queued before the host knows ``U`` (``IdMap.lookup_counted``). ``inverse`` and ``pos`` are
-    filled by the plan when asked for (``need_inverse`` / ``need_pos``) and otherwise on first
-    use, from the lists. A plan made with an id map also carries ``index_buf`` [N]: the row of
-    every unique id (found or inserted), its first ``U`` entries valid.
-    """
-
-    __slots__ = ("n", "_U", "_unique", "unique_buf", "_inverse", "row_start", "occ", "_pos", "hot_items", "hot_cap",
-                 "counts", "_pool_fill", "_stream", "serial", "lookup_calls", "index_buf")
-
-    @property
-    def U(self):
-        if self._U is None:
-            if _STAGED.get(self._stream.value) is self:
-                count = ctypes.c_int64(0)
-                check(lib().recis_unique_plan_count(ctypes.byref(count), self._stream))
-                self._U = int(count.value)
-                _STAGED.pop(self._stream.value, None)
-                _raise_staged_device_errors(self._stream)
-            else:  # a later plan took the stream's staging word: read this plan's own device word
-                self._U = int(self.counts[0].item())
-        return self._U
-
-    def U_bound(self):
-        """The unique count if the host has it already, else the number of ids: for kernels that
-        take the count from device memory and only need a bound to size their grid."""
-        return self.n if self._U is None else self._U
-
-    @property
-    def unique(self):
-        if self._unique is None:
-            self._unique = self.unique_buf[: self.U]
-        return self._unique
-
-    def _fill_late(self):
-        inv = torch.empty(self.n, dtype=torch.int32, device=self.occ.device) if self._inverse is None else None
-        pos = torch.empty(self.n, dtype=torch.int32, device=self.occ.device) if self._pos is None else None
-        if self.n:
-            check(lib().recis_plan_inverse_from_lists(ptr(self.row_start), ptr(self.occ), ptr(self.counts), i64(self.n),
-                                                      ptr(inv), ptr(pos), self._stream))
-        if inv is not None:
-            self._inverse = inv
-        if pos is not None:
-            self._pos = pos
-
-    @property
-    def inverse(self):
-        if self._inverse is None:
-            self._fill_late()
-        return self._inverse
-
-    @property
-    def pos(self):
-        if self._pos is None:
-            self._fill_late()
-        return self._pos
-
-    def _fill_lists(self, offsets, weight, mean, want_pool, batch, seq):
-        dev = offsets.device
-        S = offsets.numel() - 1
-        src = coef = tile = None
-        if want_pool:
-            src = torch.empty(self.n, dtype=torch.int32, device=dev)
-            if weight is not None or mean:
-                coef = torch.empty(self.n, dtype=torch.float32, device=dev)
-        if batch is not None:
-            tile = torch.empty(self.n, dtype=torch.int32, device=dev)
-        weight = _contig(weight)
-        if self.n:
-            check(lib().recis_csr_fill_lists(
-                ptr(self.occ), i64(self.n), ptr(offsets), _index_kind(offsets, "offsets"), i64(S), ptr(weight),
-                dtype_code(weight.dtype) if weight is not None else 0, int(bool(mean)), ptr(src), ptr(coef),
-                _host_i64(batch) if batch is not None else None, _host_i64(seq) if batch is not None else None,
-                i64(len(batch) if batch is not None else 0), ptr(tile), stream_ptr(dev)))
-        return src, coef, tile
-
-    def src_coef_for_pool(self, offsets, weight, mean):
-        """(src, coef) per list entry for the backward of pooled segments, cached per
-        (offsets, weight, mean) so that forward-time and backward-time callers share it."""
-        S = offsets.numel() - 1
-        if S == self.n and weight is None:
-            return self.occ, None  # one id per segment: the segment of an occurrence is itself
-        key = (offsets.data_ptr(), 0 if weight is None else weight.data_ptr(), bool(mean))
-        if self._pool_fill is not None and self._pool_fill[0] == key:
-            return self._pool_fill[1], self._pool_fill[2]
-        src, coef, _ = self._fill_lists(offsets, weight, mean, True, None, None)
-        self._pool_fill = (key, src, coef)
-        return src, coef
-
-    def src_for_tile(self, batch, seq, offsets):
-        """src per list entry for the backward of the padded gather (``ragged_tile``)."""
-        return self._fill_lists(offsets, None, False, False, [int(b) for b in batch], [int(t) for t in seq])[2]
-
-    def src_for_pool_and_tile(self, offsets, weight, mean, batch, seq):
-        """``src_coef_for_pool`` and ``src_for_tile`` of the same segments in one launch:
-        ``(src_pool, coef_pool, src_tile)``."""
-        src, coef, tile = self._fill_lists(offsets, weight, mean, True, [int(b) for b in batch], [int(t) for t in seq])
-        self._pool_fill = ((offsets.data_ptr(), 0 if weight is None else weight.data_ptr(), bool(mean)), src, coef)
-        return src, coef, tile
-
-
-_PLAN_SERIAL = itertools.count(1)
-
-def _raise_staged_device_errors(stream):
-    """Soft errors of the device (bad row index, full id map, ...) as an exception: kernels skip the
-    faulty access and set a bit; the bits travel to host memory with every staged unique count, so
-    the training loop sees them at its next ``BatchPlan.U`` without any extra wait."""
-    bits = ctypes.c_int(0)
-    check(lib().recis_hip_staged_device_errors(ctypes.byref(bits), stream))
-    if bits.value:
-        _lib.raise_device_errors(bits.value)   # waits for the device and clears the word
-
-
-_PLAN_JOBS = 64  # arrays one recis_unique_plan_jobs call takes
+def _recis_ops():
+    from . import torch_library
+    torch_library.load()
+    return torch.ops.recis
 
 
 def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None, tags=None):
-    """Dedup + transposed index of a batch of ids (``recis_unique_plan``). ``ids`` may be a list of
-    id tensors: the batch is their concatenation, tagged per tensor with ``tags`` as ``ids_encode``
-    does when given (``recis_unique_plan_jobs``: the kernels read the tensors directly, the tagged
-    batch is never written). ``wait=False``
-    returns without the host copy of the unique count (see ``BatchPlan``); at most one such
-    plan per stream may have its count outstanding. ``need_inverse`` / ``need_pos`` = False leave
-    those two arrays to be derived from the lists if anybody asks (callers that only walk the
-    lists save two scattered writes per id). With ``idmap`` (an ``IdMap``) the unique ids are
-    found or inserted in that map in the same pass (``recis_unique_plan_lookup``) and
-    ``plan.index_buf`` holds their rows."""
-    jobs = None
+    """Dedup + transposed index of a batch of ids: a ``torch.classes.recis.BatchPlan``
+    (``recis_unique_plan``; recis_amd/csrc/torch/plan.h). Its attributes: ``unique`` [U], ``inverse``
+    int32 [N] (``unique[inverse] == ids``), ``row_start`` int32 [N + 1] and ``occ`` int32 [N] (the
+    occurrences of unique id ``u`` are ``occ[row_start[u]:row_start[u + 1]]``), ``pos`` [N] (the
+    position of each occurrence in ``occ``), ``hot_items`` / ``hot_cap`` / ``counts`` (device words),
+    ``n``, ``serial``, ``U`` (the host copy of the unique count; a plan made with ``wait=False`` fetches
+    it on first use) and ``U_bound()``; ``unique_buf`` [N] is there at once, for work that can be
+    queued before the host knows ``U``. ``inverse`` and ``pos`` are filled by the plan when asked for
+    (``need_inverse`` / ``need_pos``) and otherwise on first use, from the lists.
+
+    ``ids`` may be a list of id tensors: the batch is their concatenation, tagged per tensor with
+    ``tags`` as ``ids_encode`` does when given (the kernels read the tensors directly, the tagged
+    batch is never written). ``wait=False`` returns without the host copy of the unique count; at
+    most one such plan per stream may have its count outstanding. With ``idmap`` (an ``IdMap``) the
+    unique ids are found or inserted in that map in the same pass (``recis_unique_plan_lookup``) and
+    ``plan.index_buf`` holds their rows; a table does the same through ``HashtableImpl.plan_lookup``."""
     if isinstance(ids, (list, tuple)):
-        # (the common case, flat contiguous int64 device tensors, goes through untouched: this runs per feature per step)
-        jobs = [t if (t.dim() == 1 and t.dtype == torch.int64 and t.is_cuda and t.is_contiguous()) else _ids64(t).reshape(-1)
-                for t in ids]
+        jobs = list(ids)
         if tags is not None and len(tags) != len(jobs):
             raise ValueError("ids_unique_plan: %d tags for %d id tensors" % (len(tags), len(jobs)))
-        if len(jobs) > _PLAN_JOBS or len(jobs) == 0:  # too many for one call: make the batch first
-            ids = ids_encode(jobs, tags) if tags is not None else (torch.cat(jobs) if jobs else torch.empty(0, dtype=torch.int64))
-            jobs = None
-    elif tags is not None:
-        raise ValueError("ids_unique_plan: tags go with a list of id tensors")
-    if jobs is None:
-        ids = _ids64(ids)
-        n = ids.numel()
-        dev = ids.device
+        if not jobs:
+            jobs = [torch.empty(0, dtype=torch.int64, device="cuda")]
+            tags = None
     else:
-        n = sum([t.numel() for t in jobs])
-        dev = jobs[0].device
-    p = BatchPlan()
-    p.serial = next(_PLAN_SERIAL)  # never reused, unlike id(p)
-    p.n = n
-    p.unique_buf = torch.empty(n, dtype=torch.int64, device=dev)
-    p._inverse = torch.empty(n, dtype=torch.int32, device=dev) if need_inverse else None
-    p.row_start = torch.empty(n + 1, dtype=torch.int32, device=dev)
-    p.occ = torch.empty(n, dtype=torch.int32, device=dev)
-    p._pos = torch.empty(n, dtype=torch.int32, device=dev) if need_pos else None
-    p.hot_cap = n // _HOT_LEN + n // _HOT_CHUNK + 2
-    p.hot_items = torch.empty(2 * p.hot_cap, dtype=torch.int32, device=dev)
-    p.counts = torch.empty(2, dtype=torch.int64, device=dev)
-    p._pool_fill = None
-    p.lookup_calls = {}   # table -> number of the counted lookup queued for this plan
-    p._unique = None
-    p.index_buf = None
-    p._stream = stream_ptr(dev)
-    count = ctypes.c_int64(0)
-    # every launch overwrites the stream's staging word: an earlier plan whose count is still
-    # outstanding there must read its own device word from now on
-    _STAGED.pop(p._stream.value, None)
-    if jobs is not None:
-        if idmap is not None:
-            p.index_buf = torch.empty(n, dtype=torch.int64, device=dev)
-        check(lib().recis_unique_plan_jobs(idmap._h if idmap is not None else None, _host_ptrs(jobs),
-                                           _host_i64([t.numel() for t in jobs]),
-                                           _host_i64(tags) if tags is not None else None, i64(len(jobs)),
-                                           ptr(p.unique_buf), ptr(p._inverse), ptr(p.row_start), ptr(p.occ), ptr(p._pos),
-                                           ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts), ptr(p.index_buf),
-                                           ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
-    elif idmap is None:
-        check(lib().recis_unique_plan(ptr(ids), i64(n), ptr(p.unique_buf), ptr(p._inverse), ptr(p.row_start),
-                                      ptr(p.occ), ptr(p._pos), ptr(p.hot_items), i64(p.hot_cap), ptr(p.counts),
-                                      ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
-    else:
-        p.index_buf = torch.empty(n, dtype=torch.int64, device=dev)
-        check(lib().recis_unique_plan_lookup(idmap._h, ptr(ids), i64(n), ptr(p.unique_buf), ptr(p._inverse),
-                                             ptr(p.row_start), ptr(p.occ), ptr(p._pos), ptr(p.hot_items),
-                                             i64(p.hot_cap), ptr(p.counts), ptr(p.index_buf),
-                                             ctypes.byref(count) if wait else None, 0 if wait else 1, p._stream))
-    p._U = int(count.value) if wait else None
-    if not wait:
-        _STAGED[p._stream.value] = p
-    else:
-        _raise_staged_device_errors(p._stream)
-    return p
+        if tags is not None:
+            raise ValueError("ids_unique_plan: tags go with a list of id tensors")
+        jobs = [ids]
+    for t in jobs:
+        if t.dtype != torch.int64:
+            raise TypeError("ids must be int64, got %s" % t.dtype)
+        require_cuda(t)
+    handle = 0 if idmap is None else int(idmap._h.value or 0)
+    return _recis_ops().unique_plan(jobs, None if tags is None else [int(t) for t in tags], handle, bool(wait),
+                                    bool(need_inverse), bool(need_pos))
 
 
 def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False, cover=None):

@@ -1,10 +1,19 @@
 """Python face of the sparse optimizers (``recis.optim``): gradient-accumulation
 gating, learning-rate plumbing and state dicts (recis/optim/sparse_optim.py:13-181)
-over the implementations in ``sparse_impl``."""
+over ``torch.classes.recis.SparseAdam`` / ``SparseAdamW`` / ``SparseAdamWTF`` / ``SparseAdagrad``."""
 from torch.optim.optimizer import Optimizer
 
+import torch
+
 from ..nn.modules.hashtable import split_sparse_dense_state_dict
-from . import sparse_impl
+
+
+def _classes():
+    """``torch.classes.recis``: the optimizers are the native ones of recis.so
+    (recis_amd/csrc/torch/sparse_optim.cc), as the reference's are (csrc/bind.cc:112-143)."""
+    from .. import torch_library
+    torch_library.load()
+    return torch.classes.recis
 
 
 class SparseOptimizer(Optimizer):
@@ -60,14 +69,14 @@ class SparseOptimizer(Optimizer):
 class SparseAdam(SparseOptimizer):
     def __init__(self, param_dict, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-2, amsgrad=False):
         super().__init__(lr=lr)
-        self._imp = sparse_impl.SparseAdamImpl.make(self.filter_param_dict(param_dict), lr, beta1, beta2, eps,
+        self._imp = _classes().SparseAdam.make(self.filter_param_dict(param_dict), lr, beta1, beta2, eps,
                                                     weight_decay, amsgrad)
 
 
 class SparseAdamW(SparseOptimizer):
     def __init__(self, param_dict, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=1e-2, amsgrad=False):
         super().__init__(lr=lr)
-        self._imp = sparse_impl.SparseAdamWImpl.make(self.filter_param_dict(param_dict), lr, beta1, beta2, eps,
+        self._imp = _classes().SparseAdamW.make(self.filter_param_dict(param_dict), lr, beta1, beta2, eps,
                                                      weight_decay, amsgrad)
 
 
@@ -77,7 +86,7 @@ class SparseAdamWTF(SparseOptimizer):
         super().__init__(lr=lr)
         if use_nesterov:
             raise ValueError("use_nesterov is not support now")
-        self._imp = sparse_impl.SparseAdamWTFImpl.make(self.filter_param_dict(param_dict), lr, beta1, beta2, eps,
+        self._imp = _classes().SparseAdamWTF.make(self.filter_param_dict(param_dict), lr, beta1, beta2, eps,
                                                        weight_decay, use_nesterov)
 
 
@@ -86,4 +95,4 @@ class SparseAdagrad(SparseOptimizer):
 
     def __init__(self, param_dict, lr=1e-2, eps=1e-8):
         super().__init__(lr=lr)
-        self._imp = sparse_impl.SparseAdagradImpl.make(self.filter_param_dict(param_dict), lr, eps)
+        self._imp = _classes().SparseAdagrad.make(self.filter_param_dict(param_dict), lr, eps)

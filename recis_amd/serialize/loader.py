@@ -23,14 +23,15 @@ def default_load_info(hashtables, tensors):
     return info
 
 
-def _accept_mask(ids, s):
+def _accept_mask(ids, slice_info):
     """read_block.cc:52-65: a key belongs to this table when (uint64)key % slice_size is in
     [slice_begin, slice_end)."""
-    if s.slice_size & (s.slice_size - 1) == 0:
-        mod = ids & (s.slice_size - 1)
+    slice_begin, slice_end, slice_size = slice_info
+    if slice_size & (slice_size - 1) == 0:
+        mod = ids & (slice_size - 1)
     else:
-        mod = torch.from_numpy(ids.numpy().view("uint64") % s.slice_size).to(torch.int64)
-    return (mod >= s.slice_begin) & (mod < s.slice_end)
+        mod = torch.from_numpy(ids.numpy().view("uint64") % slice_size).to(torch.int64)
+    return (mod >= slice_begin) & (mod < slice_end)
 
 
 def _load_table_blocks(ht, child, id_block, slot_blocks, parallel=1):
@@ -42,7 +43,7 @@ def _load_table_blocks(ht, child, id_block, slot_blocks, parallel=1):
     if info.is_coalesce():
         tagged = (ids & info.id_mask()) | (info.child_index(child) << info.id_bits_num())
         ids = torch.where(accept, tagged, ids)
-    device = ht.device
+    device = ht.device()
     accept_dev = accept.to(device)
     index = ht.insert_lookup_index_with_indicator(ids.to(device), accept_dev)
     step = fmt.block_read_size()
@@ -51,7 +52,7 @@ def _load_table_blocks(ht, child, id_block, slot_blocks, parallel=1):
         want = [b.shape[0]] + slot.row_shape()
         if want != b.shape:
             raise RuntimeError("shape not match")
-        if slot.dtype() != b.dtype:
+        if _lib.as_dtype(slot.dtype()) != b.dtype:
             raise RuntimeError("dtype not match")
         pieces += [(slot, b, beg, min(beg + step, b.shape[0])) for beg in range(0, b.shape[0], step)]
     if not pieces:
@@ -115,8 +116,7 @@ class Loader:
             if shared_name not in name_to_ht:
                 continue
             ht = name_to_ht[shared_name]
-            s = ht.slice_info()
-            mine = (s.slice_begin, s.slice_end, s.slice_size)
+            mine = tuple(ht.slice_info())
             for load_shared_name, slot_names in entries.items():
                 groups = {}
                 for slot_name in slot_names:

@@ -16,7 +16,7 @@ class HTSlotWriteBlock(fmt.WriteBlock):
 
     def __init__(self, tensor_name, slice_info, index, slot):
         shape = [index.numel()] + slot.row_shape()
-        super().__init__(tensor_name, slice_info, False, slot.dtype(), shape)
+        super().__init__(tensor_name, slice_info, False, _lib.as_dtype(slot.dtype()), shape)
         self._index, self._slot = index, slot
 
     def chunks(self):
@@ -59,8 +59,7 @@ def make_ht_write_blocks(ht):
             raise RuntimeError("table holds keys tagged for a child it does not have")
     else:
         counts = [ids.numel()]
-    s = ht.slice_info()
-    slice_info = fmt.slice_to_string(s.slice_begin, s.slice_end, s.slice_size)
+    slice_info = fmt.slice_to_string(*ht.slice_info())
     ids_host = ids.cpu()
     blocks, beg = [], 0
     slots = ht.slot_group().slots()

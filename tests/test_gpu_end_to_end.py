@@ -18,7 +18,7 @@ from recis_amd.hooks import HashTableFilterHook
 from recis_amd.nn import DynamicEmbedding, EmbeddingEngine, EmbeddingOption, HashTable
 from recis_amd.nn.functional.embedding_ops import ragged_embedding_segment_reduce
 from recis_amd.nn.hashtable_hook import AdmitHook, FilterHook
-from recis_amd.nn.initializers import ConstantInitializer, Initializer, NormalInitializer, _Generator
+from recis_amd.nn.initializers import ConstantInitializer, NormalInitializer, TensorInitializer
 from recis_amd.nn.modules.hashtable import HashtableRegister, filter_out_sparse_param
 from recis_amd.nn.modules.hashtable_hook_impl import HashtableHookFactory
 from recis_amd.optim import SparseAdagrad, SparseAdam, SparseAdamW, SparseAdamWTF
@@ -34,31 +34,12 @@ def _fresh_registries():
     yield
 
 
-class SeededBlockInitializer(Initializer):
-    """Hands out the same per-block rows as the CPU side (workloads.seeded_block), so
-    that both tables start from identical storage whatever the chunking."""
-
-    def __init__(self, seed, std=0.01):
-        super().__init__()
-        self._seed, self._std = seed, std
-
-    def _build_impl(self):
-        bs, dim = self._shape[0], self._shape[1]
-        state = {"next_block": 0}
-
-        def fill(t, gen):
-            rows = t.shape[0]
-            assert rows % bs == 0
-            parts = []
-            for _ in range(rows // bs):
-                parts.append(workloads.seeded_block(self._seed, state["next_block"], bs, dim, self._std))
-                state["next_block"] += 1
-            t.copy_(torch.from_numpy(np.concatenate(parts)))
-
-        return _Generator(self._shape, self._dtype, fill, "SeededBlockInitializer(seed=%d)" % self._seed)
-
-    def __str__(self):
-        return "SeededBlockInitializer(seed=%d)" % self._seed
+def SeededBlockInitializer(seed, std=0.01, blocks=512, bs=1024, dim=16):
+    """Hands out the same per-block rows as the CPU side (workloads.seeded_block), so that both
+    tables start from identical storage whatever the chunking: the first ``blocks`` blocks as one
+    tensor, handed out in order by the tensor-backed generator."""
+    rows = np.concatenate([workloads.seeded_block(seed, b, bs, dim, std) for b in range(blocks)])
+    return TensorInitializer(torch.from_numpy(rows))
 
 
 def _close(a, b, msg=""):
@@ -280,7 +261,7 @@ def test_global_step_filter_eviction_matches_cpu_path():
     stamps = ht._hashtable_impl.get_slot("step_filter").index_select(torch.from_numpy(rows_g).cuda())
     exp_stamps = oracle.block_gather(cpu.idmap.lookup_readonly(live), cpu.stamp, bs)
     np.testing.assert_array_equal(stamps.cpu().numpy(), exp_stamps)
-    assert ht._hashtable_impl.id_map().stats()[1] < 24 * 150    # rows were reused, not only appended
+    assert ht._hashtable_impl.id_map_stats()[1] < 24 * 150    # rows were reused, not only appended
 
 
 def test_engine_coalesces_and_pools():
@@ -628,11 +609,11 @@ def test_gradient_summed_in_the_optimizer_step_equals_summed_first(opt_cls):
             torch.autograd.backward([out[k] for k in out], [up for _ in out])
             impls = [t._hashtable_impl for t in eng.hashtables().values()]
             if step % 2 == 0:
-                assert all(len(i._planned) == 1 and not i._grad for i in impls)           # waiting unsummed
+                assert all(i.pending_grads() == [1, 0] for i in impls)           # waiting unsummed
             if sum_first:
                 for i in impls:
                     i.grad_pairs(1)
-                    assert not i._planned
+                    assert i.pending_grads()[0] == 0
             opt.step()
             opt.zero_grad()
         for t1, t2 in zip(e1.hashtables().values(), e2.hashtables().values()):
@@ -679,10 +660,10 @@ def test_two_gradients_of_one_lookup_summed_in_the_optimizer_step(opt_cls, dtype
             out = eng({"a_mean": a, "b_mean": b, "a_rows": a, "b_rows": b})
             torch.autograd.backward([out[k] for k in ups], [ups[k].to(out[k].dtype) for k in ups])
             impl = next(iter(eng.hashtables().values()))._hashtable_impl
-            assert len(impl._planned) == 2 and not impl._grad                       # both waiting unsummed
+            assert impl.pending_grads() == [2, 0]                       # both waiting unsummed
             if sum_first:
                 impl.grad_pairs(1)
-                assert not impl._planned
+                assert impl.pending_grads()[0] == 0
             opt.step()
             opt.zero_grad()
         t1, t2 = next(iter(e1.hashtables().values())), next(iter(e2.hashtables().values()))

@@ -53,7 +53,7 @@ def test_config4_step_properties():
     owner = torch.repeat_interleave(torch.arange(U, device="cuda"), rs[1:] - rs[:-1])
     assert torch.equal(inv.long()[occ], owner)                     # and under its own id
 
-    index = wl.lookup(plan)
+    index = wl.lookup(plan)[:U]
     assert torch.equal(index, wl.table.lookup_index_readonly(uniq[:U]))
     assert torch.unique(index).numel() == U and int(index.min()) >= 0
 
@@ -97,14 +97,14 @@ def test_config3_lookups_at_scale(resident):
 
     wl = bench.Config3(resident=resident, ids_per_step=2_000_000, n_batches=3)
     t = wl.table
-    lv0, idn0, _, _ = t.id_map().stats()
+    lv0, idn0, _, _ = t.id_map_stats()
     assert lv0 == resident
     ids = wl.batches[0]
     known = t.lookup_index_readonly(ids)
     n_new = int(torch.unique(ids[known < 0]).numel())
     assert 0.05 * ids.numel() < n_new <= 0.1 * ids.numel() + 1
     out = wl.step()                                            # consumes batch 0
-    lv1, idn1, _, _ = t.id_map().stats()
+    lv1, idn1, _, _ = t.id_map_stats()
     assert lv1 == lv0 + n_new and idn1 == idn0 + n_new
     now = t.lookup_index_readonly(ids)
     assert int(now.min()) >= 0
@@ -122,9 +122,9 @@ def test_config3_lookups_at_scale(resident):
     wl.step_t.fill_(5)
     wl.step()                                                  # batch 1 stamped with step 5
     seen = torch.unique(wl.batches[1])
-    live_before = t.id_map().stats()[0]
+    live_before = t.id_map_stats()[0]
     gone_ids, gone_rows = t.evict_older("step_filter", 5)
-    lv2 = t.id_map().stats()[0]
+    lv2 = t.id_map_stats()[0]
     assert lv2 == seen.numel() and gone_ids.numel() == live_before - lv2 == gone_rows.numel()
     assert int(t.lookup_index_readonly(seen).min()) >= 0
     assert int(t.lookup_index_readonly(gone_ids[:100000]).max()) == -1

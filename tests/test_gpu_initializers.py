@@ -51,5 +51,5 @@ def test_rows_of_a_table_follow_the_initialiser(name, make, lo, hi, mean, var):
 def test_a_cpu_generator_is_refused_for_a_gpu_table():
     init = I.UniformInitializer(generator=torch.Generator(device="cpu"))
     init.set_shape([BS, D])
-    with pytest.raises(ValueError, match="lives on"):
+    with pytest.raises(RuntimeError, match="lives on"):
         HashtableImpl(BS, [D], torch.float32, torch.device("cuda"), False, ["t"], init.build().impl())

@@ -164,7 +164,7 @@ def test_slices_filter_on_load(tmp_path):
         Loader(path, hashtables={"t": h}).load()
         halves.append(h._hashtable_impl)
     s0 = halves[0].slice_info()
-    mine = ((ids % 65536) >= s0.slice_begin) & ((ids % 65536) < s0.slice_end)
+    mine = ((ids % 65536) >= s0[0]) & ((ids % 65536) < s0[1])
     assert halves[0].ids_num() + halves[1].ids_num() >= n  # every key lands in exactly one half
     assert sorted(halves[0].ids().cpu().tolist()) == sorted(ids[mine].cpu().tolist())
     assert sorted(halves[1].ids().cpu().tolist()) == sorted(ids[~mine].cpu().tolist())

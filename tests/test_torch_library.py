@@ -113,20 +113,22 @@ GEN_CASES = [
 
 
 @pytest.mark.parametrize("kind,args,py", GEN_CASES, ids=[c[0] for c in GEN_CASES])
-def test_generator_matches_python_mirror_bit_for_bit(kind, args, py):
-    """Same RNG state, same rows as recis_amd.nn.initializers, which tests/test_initializers.py pins
-    bit for bit against the reference's own generators (csrc/embedding/initializer.cc:26-366)."""
+def test_python_initializers_build_the_registered_generators(kind, args, py):
+    """recis_amd.nn.initializers builds torch.classes.recis.Generator objects with the arguments of the
+    registered factories (the rows they draw are pinned bit for bit against the reference's own generators,
+    csrc/embedding/initializer.cc:26-366, in tests/test_initializers.py)."""
     shape = [64, 16]
     py.set_shape(shape)
     py.set_dtype(torch.float32)
     py.build()
     torch.manual_seed(7)
-    want = py.impl().generate()
-    want2 = py.impl().generate([5, 16])
+    want = py.generate()
     g = _gen(kind, shape, torch.float32, *args)
     torch.manual_seed(7)
     got = torch.classes.recis.Generator.generate(g)
     assert got.shape == (64, 16) and torch.equal(got, want)
+    torch.manual_seed(7)
+    assert torch.equal(g.gen(), want) and g.gen([5, 16]).shape == (5, 16)
 
 
 def test_kaiming_normal_generator_moments():
@@ -155,3 +157,10 @@ def test_gpu_only_ops_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU"):
         g = _gen("constant", [4, 2], torch.float32, 0.0)
         torch.ops.recis.make_hashtable(4, [2], torch.float32, torch.device("cpu"), False, ["t"], g, 0, 65536, 65536)
+
+
+def test_scalar_type_numbers_of_the_binding():
+    """Methods that return a ScalarType (Slot.dtype(), HashtableImpl.dtype()) hand Python its number."""
+    from recis_amd import _lib
+    for code, dtype in _lib.SCALAR_TYPE_DTYPES.items():
+        assert torch.ops.recis.scalar_type_code(torch.empty(0, dtype=dtype)) == code
