@@ -198,6 +198,8 @@ TORCH_LIBRARY(recis, m) {
       .def("settle_count", &Hashtable::SettleCount)
       .def("settle_lookup", &Hashtable::SettleLookup)
       .def("expand_rows", &Hashtable::ExpandRows)
+      .def("dense_lookup_expand", &Hashtable::DenseLookupExpand)
+      .def("accept_split_grad", &Hashtable::AcceptSplitGrad)
       .def("accept_grad_ex", &Hashtable::AcceptGradEx)
       .def("accept_planned_grad", &Hashtable::AcceptPlannedGrad)
       .def("evict_older", &Hashtable::EvictOlder)
@@ -229,6 +231,7 @@ TORCH_LIBRARY(recis, m) {
   m.def("gather", recis::functional::gather);
   m.def("block_apply_adamw", recis::functional::block_apply_adamw);
   m.def("block_apply_adagrad", recis::functional::block_apply_adagrad);  // an addition
+  m.def("fused_bucketized_mod", recis::functional::fused_bucketized_mod);  // an addition
 
   m.def("generate_ids", recis::functional::generate_ids_op);
   m.def("free_ids", recis::functional::free_ids_op);

@@ -61,6 +61,8 @@ using namespace recis::hipabi;
 
 namespace {
 
+std::mutex g_unique_mu;  // guards the notes of ids_partition's outputs (note_unique / note_partition)
+
 int mode_code(const std::string& mode) {
   if (mode == "sum") return RECIS_SUM;
   if (mode == "mean") return RECIS_MEAN;
@@ -121,6 +123,20 @@ Tensor segment_reduce_backward(Tensor grad_output, c10::optional<Tensor> weight,
   offsets = offsets.contiguous();
   Tensor w = opt_contig(weight, "weight");
   const int64_t D = grad_output.size(1), S = offsets.numel() - 1, B = reverse_indices.numel();
+  {
+    // reverse_indices as ids_partition handed them out, untouched since: the occurrence lists of that
+    // dedup are still there, so the gradient of every unique id is a gather-reduce over its list (no
+    // atomics), computed in the plan's order and brought into the sorted order of the unique ids
+    BatchPlanPtr plan;
+    Tensor order;
+    if ((m == RECIS_SUM || m == RECIS_MEAN) && known_partition(reverse_indices, &plan, &order) &&
+        plan->U() == unique_size) {
+      auto sc = plan->SrcCoefForPool(offsets, w.defined() ? c10::optional<Tensor>(w) : c10::nullopt, m == RECIS_MEAN);
+      Tensor coef = std::get<1>(sc).has_value() ? *std::get<1>(sc) : Tensor();
+      Tensor out = csr_gather_reduce(grad_output, plan, std::get<0>(sc), coef, Tensor()).index_select(0, order);
+      return grad_output.scalar_type() == at::kFloat ? out : out.to(grad_output.scalar_type());
+    }
+  }
   // duplicates in reverse_indices are accumulated with fp32 atomics, whatever the gradient's type
   Tensor out = at::empty({unique_size, D}, grad_output.options().dtype(at::kFloat));
   check(recis_segment_reduce_backward(
@@ -410,14 +426,13 @@ std::tuple<Tensor, Tensor, Tensor> ids_partition(const Tensor& ids, int64_t num_
   TORCH_CHECK(num_parts >= 1, "num_parts must be positive");
   Tensor i = flat_i64(ids, "ids");
   c10::DeviceGuard guard(i.device());
-  const int64_t n = i.numel();
-  Tensor uniq = at::empty({n}, i.options());
-  Tensor inv = at::empty({n}, i.options().dtype(at::kInt));
-  Tensor count = at::empty({1}, i.options());
-  check(recis_unique(i.data_ptr<int64_t>(), n, uniq.data_ptr<int64_t>(), inv.data_ptr(), 0,
-                     count.data_ptr<int64_t>(), stream_of(i.device())));
-  const int64_t U = n ? count.item<int64_t>() : 0;
-  Tensor u = uniq.narrow(0, 0, U);
+  // the dedup is a batch plan: its occurrence lists are kept (see note_partition) so that the backward
+  // over this call's inverse can be a gather-reduce per unique id instead of an atomic scatter
+  BatchPlanPtr plan = BatchPlan::Make({i}, c10::nullopt, nullptr, /*wait=*/true, /*need_inverse=*/true,
+                                      /*need_pos=*/false);
+  const int64_t U = plan->U();
+  Tensor u = plan->unique();
+  Tensor inv = plan->inverse();
   Tensor rot = at::bitwise_or(at::bitwise_left_shift(u, 48),
                               at::bitwise_and(at::bitwise_right_shift(u, 16), (int64_t(1) << 48) - 1));
   // a signed sort of the key with its top bit flipped is the unsigned sort
@@ -429,14 +444,45 @@ std::tuple<Tensor, Tensor, Tensor> ids_partition(const Tensor& ids, int64_t num_
   Tensor slot = at::bitwise_and(sorted_u, slice - 1);
   Tensor part = m > 0 ? at::maximum(at::div(slot, m + 1, "floor"), at::div(slot - r, m, "trunc"))
                       : at::div(slot, m + 1, "floor");
-  Tensor counts = at::bincount(part, {}, num_parts).to(at::kLong);
+  Tensor counts = num_parts == 1 ? at::full({1}, U, u.options()) : at::bincount(part, {}, num_parts).to(at::kLong);
   Tensor inverse = rank.index_select(0, inv.to(at::kLong)).to(at::kInt);
   note_unique(sorted_u);
+  note_partition(inverse, plan, order);
   return std::make_tuple(sorted_u, counts, inverse);
 }
 
 namespace {
-std::mutex g_unique_mu;
+struct NotedPartition {
+  Tensor inverse;
+  uint32_t version;
+  BatchPlanPtr plan;
+  Tensor order;  // sorted position -> the plan's unique id
+};
+std::vector<NotedPartition> g_noted_partitions;  // the last few, newest last
+}  // namespace
+
+void note_partition(const Tensor& inverse, const BatchPlanPtr& plan, const Tensor& order) {
+  std::lock_guard<std::mutex> lock(g_unique_mu);
+  if (g_noted_partitions.size() >= 2) g_noted_partitions.erase(g_noted_partitions.begin());
+  g_noted_partitions.push_back({inverse, inverse._version(), plan, order});
+}
+
+bool known_partition(const Tensor& inverse, BatchPlanPtr* plan, Tensor* order) {
+  if (!inverse.defined() || inverse.numel() == 0) return false;
+  std::lock_guard<std::mutex> lock(g_unique_mu);
+  for (const auto& e : g_noted_partitions) {
+    if (e.inverse.data_ptr() == inverse.data_ptr() && e.inverse.numel() == inverse.numel() &&
+        e.inverse.scalar_type() == inverse.scalar_type() && inverse.is_contiguous() &&
+        e.version == inverse._version() && e.inverse._version() == e.version) {
+      *plan = e.plan;
+      *order = e.order;
+      return true;
+    }
+  }
+  return false;
+}
+
+namespace {
 struct NotedUnique {
   Tensor t;
   uint32_t version;
@@ -533,7 +579,21 @@ Tensor uint64_mod(Tensor inputs, at::Scalar num) {
   return fused_uint64_mod({inputs}, mod)[0];
 }
 
+namespace {
+TensorList bucketized_impl(const TensorList& inputs, const TensorList& boundaries, const std::vector<int64_t>* mods);
+}
+
 TensorList fused_bucketized(TensorList inputs, TensorList boundaries) {
+  return bucketized_impl(inputs, boundaries, nullptr);
+}
+
+TensorList fused_bucketized_mod(TensorList inputs, TensorList boundaries, std::vector<int64_t> mods) {
+  TORCH_CHECK(mods.size() == inputs.size(), "fused_bucketized_mod: ", mods.size(), " mods for ", inputs.size(), " tensors");
+  return bucketized_impl(inputs, boundaries, &mods);
+}
+
+namespace {
+TensorList bucketized_impl(const TensorList& inputs, const TensorList& boundaries, const std::vector<int64_t>* mods) {
   if (inputs.empty()) return {};
   TORCH_CHECK(inputs.size() == boundaries.size(), "fused_bucketized: one boundary tensor per input");
   require_gpu(inputs, "inputs");
@@ -556,10 +616,11 @@ TensorList fused_bucketized(TensorList inputs, TensorList boundaries) {
   auto ip = host_ptrs<float>(in);
   auto bp = host_ptrs<float>(bd);
   auto op = host_mut_ptrs<int64_t>(outs);
-  check(recis_fused_bucketized(ip.data(), sizes.data(), bp.data(), blens.data(), op.data(),
-                               static_cast<int64_t>(in.size()), stream_of(in[0].device())));
+  check(recis_fused_bucketized_mod(ip.data(), sizes.data(), bp.data(), blens.data(), mods ? mods->data() : nullptr,
+                                   op.data(), static_cast<int64_t>(in.size()), stream_of(in[0].device())));
   return outs;
 }
+}  // namespace
 
 Tensor bucketize_op(Tensor values, Tensor boundaries) {
   return fused_bucketized({values.to(at::kFloat)}, {boundaries.to(at::kFloat)})[0].view(values.sizes());

@@ -57,6 +57,9 @@ Tensor uint64_mod(Tensor inputs, at::Scalar num);
 Tensor bucketize_op(Tensor values, Tensor boundaries);
 TensorList fused_uint64_mod(TensorList inputs, Tensor mod_vec);
 TensorList fused_bucketized(TensorList inputs, TensorList boundaries);
+// fused_bucketized followed by fused_uint64_mod of the buckets (one positive modulus per tensor) in one
+// pass: an addition (the reference runs the two operators one after the other).
+TensorList fused_bucketized_mod(TensorList inputs, TensorList boundaries, std::vector<int64_t> mods);
 TensorList fused_hash(TensorList inputs, TensorList input_offsets, const std::string& hash_type);
 TensorList fused_multi_hash(TensorList inputs, TensorList muls, TensorList primes, TensorList bucket_num);
 // csrc/ops/ragged_tile.h:9-18
@@ -94,6 +97,10 @@ Tensor csr_gather_reduce_parts(const TensorList& parts, const BatchPlanPtr& plan
 // kept alive, so their addresses cannot be handed out to another tensor meanwhile.
 void note_unique(const Tensor& t);
 bool known_unique(const Tensor& t);
+// The same for the inverse ids_partition hands out: the plan of that dedup and the order its unique
+// ids were sorted into stay available to the backward over that inverse (the last two calls).
+void note_partition(const Tensor& inverse, const BatchPlanPtr& plan, const Tensor& order);
+bool known_partition(const Tensor& inverse, BatchPlanPtr* plan, Tensor* order);
 
 }  // namespace functional
 }  // namespace recis

@@ -725,6 +725,71 @@ at::Tensor Hashtable::ExpandRows(const BatchPlanPtr& plan, const at::Tensor& row
   return out;
 }
 
+c10::optional<std::tuple<BatchPlanPtr, at::Tensor, at::Tensor>> Hashtable::DenseLookupExpand(
+    const std::vector<at::Tensor>& cols, const c10::optional<std::vector<int64_t>>& tags,
+    const c10::optional<std::string>& stamp_slot, const c10::optional<at::Tensor>& stamp_value) {
+  if (cols.empty()) return c10::nullopt;
+  for (const auto& c : cols) {
+    const bool column = c.defined() && c.is_cuda() && c.scalar_type() == at::kLong && c.is_contiguous() &&
+                        (c.dim() == 1 || (c.dim() == 2 && c.size(1) == 1)) && c.device() == device_;
+    if (!column) return c10::nullopt;
+  }
+  BatchPlanPtr plan = PlanLookup(cols, tags, /*wait=*/false, /*need_inverse=*/false, /*need_pos=*/false);
+  at::Tensor index = plan->IndexBufRaw();
+  at::Tensor out = ExpandRows(plan, index, c10::nullopt, stamp_slot, stamp_value);
+  return std::make_tuple(plan, index, out);
+}
+
+void Hashtable::AcceptSplitGrad(const at::Tensor& index_in, const BatchPlanPtr& plan,
+                                const std::vector<c10::optional<at::Tensor>>& grads, const std::vector<int64_t>& split,
+                                const c10::optional<at::Tensor>& src, const c10::optional<at::Tensor>& coef, int64_t key,
+                                bool may_miss, bool settle) {
+  TORCH_CHECK(grads.size() == split.size() && !grads.empty(), "one gradient per part");
+  const int64_t D = slot_group_->EmbSlot()->FlatSize();
+  int64_t rows = 0;
+  for (int64_t r : split) rows += r;
+  // consecutive slices of one buffer? then the whole gradient is that buffer, in place
+  at::Tensor whole;
+  const c10::optional<at::Tensor>& g0 = grads[0];
+  if (g0.has_value() && g0->defined() && g0->is_contiguous() && g0->dim() == 2 && g0->size(1) == D) {
+    const char* at_byte = static_cast<const char*>(g0->data_ptr());
+    const void* storage = g0->storage().data();
+    bool adjacent = true;
+    for (size_t f = 0; f < grads.size() && adjacent; ++f) {
+      const c10::optional<at::Tensor>& g = grads[f];
+      adjacent = g.has_value() && g->defined() && g->scalar_type() == g0->scalar_type() && g->is_contiguous() &&
+                 g->dim() == 2 && g->size(0) == split[f] && g->size(1) == D && g->data_ptr() == at_byte &&
+                 g->storage().data() == storage;
+      at_byte += split[f] * D * g0->element_size();
+    }
+    if (adjacent) whole = at::as_strided(*g0, {rows, D}, {D, 1}, g0->storage_offset());
+  }
+  if (!whole.defined()) {
+    at::Tensor like;
+    for (const auto& g : grads) {
+      if (g.has_value() && g->defined()) {
+        like = *g;
+        break;
+      }
+    }
+    if (!like.defined()) return;  // no gradient reached any part
+    std::vector<at::Tensor> parts;
+    for (size_t f = 0; f < grads.size(); ++f) {
+      parts.push_back(grads[f].has_value() && grads[f]->defined() ? grads[f]->reshape({split[f], D})
+                                                                  : at::zeros({split[f], D}, like.options()));
+    }
+    whole = at::cat(parts, 0);
+  }
+  at::Tensor index = index_in;
+  if (settle) {
+    const int64_t U = plan->U();
+    SettleCount(U, plan);
+    if (index.numel() > U) index = index.narrow(0, 0, U);
+  }
+  AcceptPlannedGrad(index, plan, {whole}, false, src.has_value() && src->defined() ? *src : plan->occ(), coef,
+                    c10::nullopt, key, may_miss);
+}
+
 // ------------------------------------------------------------------------------------ gradients
 void Hashtable::AcceptGrad(const at::Tensor& grad_index, const at::Tensor& grad) {
   // the index tensor the last embedding_lookup returned for ids that are known to be distinct has

@@ -274,6 +274,22 @@ class Hashtable : public torch::CustomClassHolder {
   at::Tensor ExpandRows(const recis::BatchPlanPtr& plan, const at::Tensor& row_index,
                         const c10::optional<at::Tensor>& weight, const c10::optional<std::string>& stamp_slot,
                         const c10::optional<at::Tensor>& stamp_value);
+  // PlanLookup + ExpandRows for a group of dense id columns ([B] or [B, 1] int64 GPU tensors, one id
+  // per sample: every segment holds one id, so sum == mean == the row itself) in ONE call from
+  // Python: (plan, full-length row index, [N, D] rows, column after column). None when a column is
+  // something else (the caller then takes the general path).
+  c10::optional<std::tuple<recis::BatchPlanPtr, at::Tensor, at::Tensor>> DenseLookupExpand(
+      const std::vector<at::Tensor>& cols, const c10::optional<std::vector<int64_t>>& tags,
+      const c10::optional<std::string>& stamp_slot, const c10::optional<at::Tensor>& stamp_value);
+  // The backward of an output that was handed out in parts (`split` rows each): `grads` are the parts'
+  // gradients as autograd delivers them (None = zeros). Consecutive slices of one buffer are used in
+  // place, anything else is concatenated; then the count of `plan` is settled (`settle`) and the
+  // gradient accepted unsummed (AcceptPlannedGrad with src / coef; src undefined = the occurrence
+  // itself, one id per segment).
+  void AcceptSplitGrad(const at::Tensor& index, const recis::BatchPlanPtr& plan,
+                       const std::vector<c10::optional<at::Tensor>>& grads, const std::vector<int64_t>& split,
+                       const c10::optional<at::Tensor>& src, const c10::optional<at::Tensor>& coef, int64_t key,
+                       bool may_miss, bool settle);
   // accept_grad whose caller knows that grad_index has no duplicates (`unique`), and / or that two
   // calls with one `key` (!= 0) hand over gradients for the same rows in the same order (the second
   // is then added onto the first).

@@ -6,6 +6,7 @@ once and shared."""
 from collections import defaultdict
 from typing import Dict, List
 
+import torch
 from torch import nn
 
 from .. import ops
@@ -26,8 +27,15 @@ def _fused_bucketize(op_list, inputs):
 
 def _fused_bucketize_mod(op_list, inputs):
     """Bucketize followed by Mod of the same feature: one pass (``op_list``: (Bucketize, Mod) pairs)."""
-    outs = ops.fused_bucketized([_values(x).cuda().float() for x in inputs], [b.boundary.cuda() for b, _ in op_list],
-                                mods=[m.mod_value for _, m in op_list])
+    vals = [_values(x) for x in inputs]
+    if all(v.is_cuda and v.dtype == torch.float32 for v in vals):
+        # the common case needs no conversions: one call of the registered operator
+        outs = ops.recis_ops().fused_bucketized_mod(vals, [b.boundary_on(v.device) for (b, _), v in zip(op_list, vals)],
+                                                    [m.mod_value for _, m in op_list])
+        outs = [o.view(v.shape) for o, v in zip(outs, vals)]
+    else:
+        outs = ops.fused_bucketized([v.cuda().float() for v in vals], [b.boundary.cuda() for b, _ in op_list],
+                                    mods=[m.mod_value for _, m in op_list])
     return [_with_values(x, o) for x, o in zip(inputs, outs)]
 
 

@@ -109,9 +109,22 @@ class Bucketize(_OP):
         super().__init__()
         b = torch.tensor(boundary, dtype=torch.float) if isinstance(boundary, list) else boundary.float()
         self.register_buffer("boundary", b)
+        self._on_device = None
+
+    def boundary_on(self, device):
+        """The boundaries on ``device``: the buffer itself when it lives there, else a copy made once (and
+        again if the buffer is replaced or written to)."""
+        b = self.boundary
+        if b.device == device:
+            return b
+        hit = self._on_device
+        if hit is None or hit[0] is not b or hit[1] != b._version or hit[2].device != device:
+            hit = self._on_device = (b, b._version, b.to(device))
+        return hit[2]
 
     def forward(self, x):
-        return _with_values(x, ops.bucketize_op(_values(x).cuda().float(), self.boundary.cuda()))
+        v = _values(x).cuda().float()
+        return _with_values(x, ops.bucketize_op(v, self.boundary_on(v.device)))
 
     def _get_config(self):
         return {"boundary": self.boundary.tolist()}

@@ -202,6 +202,37 @@ def _joined(grads, split, shape):
     return torch.cat([g if g is not None else like.new_zeros((rows, shape[1])) for g, rows in zip(grads, split)])
 
 
+class DenseLookupFunction(torch.autograd.Function):
+    """Dedup, lookup and pooling of a group of dense id columns (``[B]`` / ``[B, 1]`` int64: one id per
+    sample, so sum == mean == the row itself) as ONE native call each way
+    (``HashtableImpl.dense_lookup_expand`` forward, ``accept_split_grad`` backward): what the per-feature
+    loop of ``EmbeddingEngine.forward`` + ``LookupPoolFunction`` do for such a group, without the Python
+    work per feature. One output per column, views of the one ``[N, D]`` buffer; nothing waits for the
+    unique count. ``forward`` returns None instead when a column is something else."""
+
+    @staticmethod
+    def forward(ctx, backward_holder, impl, cols, tags, stamp):
+        res = impl.dense_lookup_expand(cols, tags, None if stamp is None else stamp[0],
+                                       None if stamp is None else stamp[1])
+        if res is None:
+            ctx.mark_non_differentiable()
+            return None
+        plan, index, out = res
+        split = [c.shape[0] for c in cols]
+        ctx.impl, ctx.plan, ctx.split = impl, plan, split
+        ctx.save_for_backward(index)
+        ctx.mark_non_differentiable(index)
+        return (index,) + tuple(torch.split(out, split))
+
+    @staticmethod
+    def backward(ctx, _grad_index, *grads):
+        (index,) = ctx.saved_tensors
+        # the gradients of the columns, as they come (slices of one buffer are used in place); the sum per
+        # unique row is left to the optimizer step, which then updates the row in the same launch
+        ctx.impl.accept_split_grad(index, ctx.plan, list(grads), ctx.split, None, None, ctx.plan.serial, False, True)
+        return None, None, None, None, None
+
+
 class LookupTileFunction(torch.autograd.Function):
     """Lookup of a plan's unique ids and the padded gather of several features at once, ONE output
     per feature (``[bs[f], tile_len[f] * D]``, views of one buffer: the list form of the tile

@@ -22,7 +22,8 @@ import torch
 from ... import ops
 from ...ragged.tensor import RaggedTensor
 from ..functional.embedding_ops import RaggedTileParts
-from .embedding import EmbeddingOption, LookupTileFunction, lookup_and_pool, lookup_unique_rows, make_plan
+from .embedding import (DenseLookupFunction, EmbeddingOption, LookupTileFunction, lookup_and_pool, lookup_unique_rows,
+                        make_plan)
 from .hashtable import HashTable, gen_slice, plan_lookup
 
 
@@ -130,6 +131,19 @@ class EmbeddingEngine(torch.nn.Module):
                     runtime.setdefault(self._runtime_key[name], []).append(name)
             for names in runtime.values():
                 opt0 = grp.features[names[0]]
+                if (table.training and opt0.combiner in ("sum", "mean") and opt0.trainable and opt0.admit_hook is None
+                        and opt0.grad_reduce_by != "id" and table._dtype in (torch.float32, torch.bfloat16, torch.float16)
+                        and all(type(inputs[n]) is torch.Tensor for n in names)):
+                    # dense id columns only: tagging, dedup, lookup and the rows of every column in one native call
+                    stamp = getattr(table._filter_hook_impl, "stamp_target", lambda: None)()
+                    if stamp is not None or isinstance(table._filter_hook_impl, torch.nn.Identity):
+                        res = DenseLookupFunction.apply(table._backward_holder, table._hashtable_impl,
+                                                        [inputs[n] for n in names],
+                                                        [tag_of[n] for n in names] if info.is_coalesce() else None, stamp)
+                        if res is not None:
+                            for name, part in zip(names, res[1:]):
+                                outputs[name] = part
+                            continue
                 vals, weights, offs, shapes, dense = [], [], [], [], []
                 all_unit = True
                 any_weight = opt0.use_weight and any(

@@ -739,10 +739,20 @@ class IdMap:
 _HOT_LEN, _HOT_CHUNK = 64, 2048  # RECIS_PLAN_HOT_LEN / RECIS_PLAN_HOT_CHUNK of the library
 
 
-def _recis_ops():
-    from . import torch_library
-    torch_library.load()
-    return torch.ops.recis
+_RECIS_OPS = None
+
+
+def recis_ops():
+    """``torch.ops.recis`` of recis.so (loaded on first use)."""
+    global _RECIS_OPS
+    if _RECIS_OPS is None:
+        from . import torch_library
+        torch_library.load()
+        _RECIS_OPS = torch.ops.recis
+    return _RECIS_OPS
+
+
+_recis_ops = recis_ops
 
 
 def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None, tags=None):

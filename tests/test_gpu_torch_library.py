@@ -457,3 +457,80 @@ def test_initialiser_rows_on_device():
     ht = _make_table(32, 8, gen)
     _, emb = ht.embedding_lookup(torch.arange(100, device="cuda"), False)
     assert emb.is_cuda and float(emb.min()) >= -0.5 and float(emb.max()) <= 0.5 and float(emb.std()) > 0.2
+
+
+def test_config4_shaped_step_through_the_library_boundary():
+    """A config-4-shaped step (26 id columns + 13 bucketized float columns on one coalesced table, dim 16,
+    sum pooling of one id per sample, SparseAdam) three ways against the CPU restatement of the reference's
+    step: (a) the reference's own call sequence operator by operator (fused_bucketized -> fused_uint64_mod ->
+    ids_encode -> ids_partition -> embedding_lookup -> segment_reduce_forward -> segment_reduce_backward ->
+    accept_grad -> step), (b) the fused calls behind the same classes (dense_lookup_expand ->
+    accept_split_grad -> step: one plan, gradient summed where the rows are updated). Each side orders new
+    keys its own way (the CPU path by np.unique, ids_partition by shard, the plan by hash bucket), so rows start
+    from one constant and are compared by key; pooled outputs sample by sample; fp32 within rtol 1e-5 /
+    atol 1e-6."""
+    import workloads
+
+    batch, dim, bs, lr = 2048, 16, 1024, 1e-3
+    n_feat = 39
+    # every row starts at the same value: the three sides hand new keys their rows in different orders
+    cpu = cpu_path.CpuTable(dim, bs, lambda b: np.full((bs, dim), 0.05, np.float32), "adam", lr, 1e-8)
+
+    def table():
+        gen = C.Generator.make_constant_generator([bs, dim], torch.float32, 0.05)
+        ht = _make_table(bs, dim, gen, ["f%d" % i for i in range(n_feat)], True)
+        return ht, C.SparseAdam.make({"ctr": ht}, lr, 0.9, 0.999, 1e-8, 0.0, False)
+
+    (ht_a, opt_a), (ht_b, opt_b) = table(), table()
+    tags = list(range(n_feat))
+    offsets = torch.arange(batch * n_feat + 1, dtype=torch.int32, device="cuda")
+    rng = np.random.default_rng(44)
+    for step in range(4):
+        c = workloads.config4(batch=batch, data_seed=step)
+        grad = rng.standard_normal((batch * n_feat, dim)).astype(np.float32)
+        extra_c = [oracle.uint64_mod(oracle.bucketize(d.cpu().numpy(), c["boundaries"][0].cpu().numpy()), c["mod"])
+                   for d in c["dense"]]
+        ids_c = oracle.ids_encode([t.cpu().numpy() for t in c["sparse"]] + extra_c, tags)
+        pooled_c, uniq_c, index_c = cpu_path.train_step(cpu, ids_c, np.arange(ids_c.size + 1), None, grad)
+        # (a) the reference's sequence
+        extra = R.fused_uint64_mod(R.fused_bucketized(c["dense"], c["boundaries"]),
+                                   torch.full((len(c["dense"]),), c["mod"], dtype=torch.int64))
+        ids = R.ids_encode(c["sparse"] + extra, torch.tensor(tags))
+        np.testing.assert_array_equal(ids.cpu().numpy(), ids_c)
+        uniq, counts, inverse = R.ids_partition(ids, 1)
+        assert counts.tolist() == [uniq.numel()] and torch.equal(uniq[inverse.long()], ids)
+        index, emb = ht_a.embedding_lookup(uniq, False)
+        pooled = R.segment_reduce_forward(emb, None, inverse, offsets, "sum")
+        np.testing.assert_allclose(pooled.cpu().numpy(), pooled_c, rtol=1e-5, atol=1e-6)
+        g_unique = R.segment_reduce_backward(_dev(grad), None, inverse, offsets, uniq.numel(), "sum")
+        exp_g = oracle.segment_reduce_backward(grad, None, inverse.cpu().numpy().astype(np.int64),
+                                               np.arange(ids_c.size + 1), uniq.numel(), "sum")
+        np.testing.assert_allclose(g_unique.cpu().numpy(), exp_g, rtol=1e-5, atol=1e-5)
+        ht_a.accept_grad(index, g_unique)
+        assert ht_a.pending_grads() == [0, 1]
+        opt_a.step()
+        opt_a.zero_grad()
+        # (b) the fused calls: one plan, nothing waits for the unique count, the gradient stays unsummed
+        cols = c["sparse"] + R.fused_bucketized_mod(c["dense"], c["boundaries"], [c["mod"]] * len(c["dense"]))
+        plan, index_b, out = ht_b.dense_lookup_expand(cols, tags, None, None)
+        np.testing.assert_allclose(out.cpu().numpy(), pooled_c, rtol=1e-5, atol=1e-6)
+        g = _dev(grad)
+        ht_b.accept_split_grad(index_b, plan, list(g.split(batch)), [batch] * n_feat, None, None, plan.serial, False, True)
+        assert ht_b.pending_grads() == [1, 0]
+        opt_b.step()
+        opt_b.zero_grad()
+        assert ht_b.pending_grads() == [0, 0]
+    keys_c, rows_c = cpu.idmap.snapshot()
+    order = np.argsort(keys_c)
+    keys_c, rows_c = keys_c[order], rows_c[order]
+    want = [np.concatenate(blocks)[rows_c] for blocks in (cpu.emb, cpu.s0, cpu.s1)]
+    for ht in (ht_a, ht_b):
+        keys, rows = ht.ids_map()
+        keys, at = torch.sort(keys)
+        np.testing.assert_array_equal(keys.cpu().numpy(), keys_c)
+        rows = rows[at]
+        assert torch.unique(rows).numel() == rows.numel() and ht.ids_num() == cpu.idmap.id_num()
+        for name, exp in zip(("embedding", "sparse_adam_exp_avg", "sparse_adam_exp_avg_sq"), want):
+            got = ht.get_slot(name).index_select(rows).cpu().numpy()
+            np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-6, err_msg=name)
+    assert _lib.poll_device_errors() == 0
