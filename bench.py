@@ -667,6 +667,7 @@ class ModulePath4:
             d = {"s%d" % i: t.view(-1, 1) for i, t in enumerate(b["sparse"])}
             d.update({"d%d" % i: t for i, t in enumerate(b["dense"])})
             self.data.append(d)
+        self.dense_of = {id(d): {k: v for k, v in d.items() if k[0] == "d"} for d in self.data}
         g = torch.Generator(device="cuda").manual_seed(4)
         self.concat = concat
         if concat:
@@ -682,14 +683,29 @@ class ModulePath4:
         data = self.data[self._turn % len(self.data)]
         self._turn += 1
         x = dict(data)
-        x.update({k: v.view(-1, 1) for k, v in self.fe({k: data[k] for k in data if k[0] == "d"}).items()})
+        x.update(self.fe(self.dense_of[id(data)]))     # [B] id columns: the engine takes them as [B, 1]
         out = self.eng(x)
         if self.concat:
             torch.cat([out[n] for n in self.names], dim=1).backward(self.up)
         else:
-            torch.autograd.backward([out[n] for n in self.names], self.up)
+            _HandGradients.apply(self.up, *[out[n] for n in self.names]).backward()
         self.opt.step()
         self.opt.zero_grad()
+
+
+class _HandGradients(torch.autograd.Function):
+    """Stands where a model's backward would be: a scalar whose backward hands each input its preset gradient
+    (torch.autograd.backward with a list of 39 tensors and 39 gradients spends 0.1 ms of Python on checking
+    them one by one, which no model's backward does)."""
+
+    @staticmethod
+    def forward(ctx, grads, *outs):
+        ctx.grads = grads
+        return outs[0].new_zeros(())
+
+    @staticmethod
+    def backward(ctx, _):
+        return (None,) + tuple(ctx.grads)
 
 
 class TorchLibraryPath4:
@@ -1044,7 +1060,7 @@ def main():
         # the same steps through the drop-in module layer (EmbeddingEngine + sparse optimizer)
         for key, cls, name in (("c4", ModulePath4, Config4.name), ("c5", ModulePath5, Config5.name)):
             mp = cls()
-            ms = _timed_steps(mp, 10, 3)
+            ms = _timed_steps(mp, 20, 5)
             target = out if key == args.workload else extras.get(name)
             if target is not None:
                 target["module_path_ms"] = round(ms, 4)
@@ -1054,7 +1070,7 @@ def main():
             for key, make in (("module_path_with_concat_ms", lambda: ModulePath4(concat=True)),
                               ("torch_library_path_ms", TorchLibraryPath4)):
                 wl = make()
-                out[key] = round(_timed_steps(wl, 10, 3), 4)
+                out[key] = round(_timed_steps(wl, 20, 5), 4)
                 del wl
                 torch.cuda.empty_cache()
         if main_wl is None and not args.no_cpu_baseline:

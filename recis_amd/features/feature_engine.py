@@ -32,7 +32,7 @@ def _fused_bucketize_mod(op_list, inputs):
         # the common case needs no conversions: one call of the registered operator
         outs = ops.recis_ops().fused_bucketized_mod(vals, [b.boundary_on(v.device) for (b, _), v in zip(op_list, vals)],
                                                     [m.mod_value for _, m in op_list])
-        outs = [o.view(v.shape) for o, v in zip(outs, vals)]
+        outs = [o if v.dim() == 1 else o.view(v.shape) for o, v in zip(outs, vals)]
     else:
         outs = ops.fused_bucketized([v.cuda().float() for v in vals], [b.boundary.cuda() for b, _ in op_list],
                                     mods=[m.mod_value for _, m in op_list])
