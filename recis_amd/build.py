@@ -101,7 +101,10 @@ def build_torch_library(verbose=True):
         objs = list(ex.map(_compile_host, [(s, flags) for s in srcs]))
     cmd = ["g++", "-shared", "-fPIC", "-o", TORCH_LIB_PATH] + objs + [
         "-L", LIB_DIR, "-lrecis_hip", "-Wl,-rpath,$ORIGIN", "-L", torch_lib, "-Wl,-rpath," + torch_lib,
-        "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip", "-Wl,--no-undefined", "-Wl,--allow-shlib-undefined"]
+        "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+        # the event helpers of ATen's headers are inline and call the HIP runtime directly
+        "-L", os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib"), "-lamdhip64",
+        "-Wl,--no-undefined", "-Wl,--allow-shlib-undefined"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link of recis.so failed:\n" + r.stdout + r.stderr)

@@ -1,13 +1,13 @@
 // The registration block the reference has at csrc/bind.cc:46-211: namespace `recis`, the same
 // class and operator names, the reference's C++ signatures (torch infers the schemas from them).
 // Loaded with torch.classes.load_library(<package>/lib/recis.so), as recis/__init__.py:8-16 does.
-// Not registered: gauc_calc, adam_tf_apply, ragged_to_sparse and the Saver / Loader /
-// CheckpointReader / WriteBlock classes (metrics, the dense optimizer and a CPU-only op are outside
-// this build; checkpoints are written and read by the Python package recis_amd.serialize).
+// Not registered: gauc_calc and adam_tf_apply (a metric and the dense optimizer: outside the
+// sparse-embedding path this build covers).
 #include <torch/custom_class.h>
 #include <torch/library.h>
 
 #include "ops.h"
+#include "serialize.h"
 #include "sparse_optim.h"
 #include "table.h"
 
@@ -213,11 +213,57 @@ TORCH_LIBRARY(recis, m) {
   def_optimizer<recis::optim::SparseAdagrad>(m, "SparseAdagrad");  // an addition
 
   m.def("make_hashtable", Hashtable::Make);
+
+  // ---- checkpoints (csrc/bind.cc:147-170)
+  using namespace recis::serialize;
+  m.class_<WriteBlock>("WriteBlock")
+      .def("tensor_name", [](const WriteBlockPtr& self) { return self->TensorName(); })
+      .def("slice_info", [](const WriteBlockPtr& self) { return self->SliceInfo(); })
+      .def("is_dense", [](const WriteBlockPtr& self) { return self->IsDense(); })  // an addition
+      // additions: blocks made from tensors the caller holds (tools, tests)
+      .def_static("make_tensor", MakeTensorWriteBlock)
+      .def_static("make_array", MakeArrayWriteBlock);
+  m.class_<Saver>("Saver")
+      .def(torch::init<int64_t, int64_t, int64_t, const std::string>())
+      .def("make_write_blocks", &Saver::MakeWriteBlocks)
+      .def("save", &Saver::Save);
+  m.class_<Loader>("Loader")
+      .def(torch::init<const std::string, int64_t, c10::Dict<std::string, HashTablePtr>,
+                       c10::Dict<std::string, at::Tensor>>())
+      .def("default_load_info", &Loader::DefaultLoadInfo)
+      .def("load", &Loader::Load);
+  m.class_<CheckpointReader>("CheckpointReader")
+      .def(torch::init<std::string>())
+      .def("init", &CheckpointReader::Init)
+      .def("list_tensor_names", &CheckpointReader::ListTensors)
+      .def("read_tensor", &CheckpointReader::LoadTensor)
+      .def("tensor_shape", &CheckpointReader::TensorShape)
+      .def("tensor_dtype", &CheckpointReader::TensorType);
+  // additions: the directory writer by itself (the reference reaches it from C++ only) and two
+  // helpers for tools that read or write single data files
+  m.class_<SaveBundle>("SaveBundle")
+      .def(torch::init<std::string, int64_t, int64_t, int64_t, double>())
+      .def("add_block", &SaveBundle::AddBlock)
+      .def("save", &SaveBundle::Save)
+      .def("merge_meta_info", &SaveBundle::MergeMetaInfo);
+  m.def("write_data_file", [](const std::string& path, const std::string& json_path, std::vector<WriteBlockPtr> blocks) {
+    WriteDataFile(path, json_path, blocks);
+  });
+  // per block of the file, in file order: (name, dtype string, shape, first byte, end byte)
+  m.def("read_data_file_header", [](const std::string& path) {
+    std::vector<std::tuple<std::string, std::string, std::vector<int64_t>, int64_t, int64_t>> out;
+    for (const auto& kv : ReadDataFileHeader(path, nullptr)) {
+      out.emplace_back(kv.first, DtypeToString(kv.second.dtype), kv.second.shape, kv.second.offset_beg,
+                       kv.second.offset_end);
+    }
+    return out;
+  });
   m.def("unique_plan", recis::unique_plan);  // an addition: see plan.h
   // an addition: the integer a ScalarType crosses the binding as (Slot.dtype(), HashtableImpl.dtype())
   m.def("scalar_type_code", [](const at::Tensor& t) { return t.scalar_type(); });
 
   m.def("ragged_to_dense", recis::functional::ragged_to_dense);
+  m.def("ragged_to_sparse", recis::functional::ragged_to_sparse);
   m.def("uint64_mod", recis::functional::uint64_mod);
   m.def("bucketize_op", recis::functional::bucketize_op);
   m.def("fused_multi_hash", recis::functional::fused_multi_hash);

@@ -754,6 +754,42 @@ std::vector<char> scalar_bytes(const at::Scalar& value, at::ScalarType dtype) {
 }
 }  // namespace
 
+// The ragged tensor as a coalesced sparse COO tensor of shape [rows, longest row of level 0, ...,
+// longest row of the last level]; coordinate k of a value is its position inside the row of level
+// k - 1 that holds it (csrc/ops/ragged_to_sparse.cc:43-91; the reference has a CPU kernel only, this
+// one is library calls on the device of its inputs, whichever that is).
+Tensor ragged_to_sparse(Tensor values, TensorList offset_splits) {
+  TORCH_CHECK(!offset_splits.empty(), "ragged_to_sparse: needs at least one level of offsets");
+  for (const auto& o : offset_splits) {
+    TORCH_CHECK(o.scalar_type() == offset_splits[0].scalar_type() &&
+                    (o.scalar_type() == at::kInt || o.scalar_type() == at::kLong),
+                "ragged_to_sparse: each offset_splits should be torch::kInt32 or torch::kInt64");
+    TORCH_CHECK(o.device() == values.device(), "ragged_to_sparse: offset_splits and value should be all on cpu or cuda");
+  }
+  c10::DeviceGuard guard(values.device());
+  TensorList splits;
+  for (const auto& o : offset_splits) splits.push_back(o.to(at::kLong).contiguous());
+  const Tensor& last = splits.back();
+  const int64_t n = last.numel() ? last[last.numel() - 1].item<int64_t>() : 0;
+  std::vector<int64_t> shape{splits[0].numel() - 1};
+  for (const auto& o : splits) {
+    shape.push_back(o.numel() > 1 ? (o.slice(0, 1) - o.slice(0, 0, o.numel() - 1)).max().item<int64_t>() : 0);
+  }
+  auto i64 = values.options().dtype(at::kLong);
+  TensorList coords;
+  Tensor child = at::arange(n, i64);  // index among the rows of the level below
+  for (auto it = splits.rbegin(); it != splits.rend(); ++it) {
+    Tensor parent = at::searchsorted(*it, child, /*out_int32=*/false, /*right=*/true) - 1;  // the row that holds `child`
+    coords.push_back(child - it->index_select(0, parent));
+    child = parent;
+  }
+  coords.push_back(child);
+  std::reverse(coords.begin(), coords.end());
+  Tensor indices = n ? at::stack(coords) : at::empty({static_cast<int64_t>(splits.size()) + 1, 0}, i64);
+  for (int64_t d = 1; d < values.dim(); ++d) shape.push_back(values.size(d));
+  return at::sparse_coo_tensor(indices, values.slice(0, 0, n), shape).coalesce();
+}
+
 Tensor ragged_to_dense(Tensor values, const TensorList& offsets, at::Scalar default_value) {
   require_gpu(values, "values");
   require_gpu(offsets, "offsets");

@@ -69,6 +69,8 @@ Tensor ragged_tile_back(Tensor batch_seq, const std::vector<int64_t>& batch_info
                         Tensor dy);
 // csrc/ops/ragged_to_dense.h:5-7, dense_to_ragged.h:8-10
 Tensor ragged_to_dense(Tensor values, const TensorList& offsets, at::Scalar default_value);
+// csrc/ops/ragged_to_sparse.h: the ragged tensor as a coalesced sparse COO tensor
+Tensor ragged_to_sparse(Tensor values, TensorList offset_splits);
 std::tuple<Tensor, Tensor> dense_to_ragged(const Tensor& data, bool check_invalid, const Tensor& invalid_value);
 // csrc/ops/fused_ragged_cutoff.h:9-14,33-39
 std::tuple<TensorList, TensorList, TensorList, TensorList, Tensor, Tensor> fused_ragged_cutoff(

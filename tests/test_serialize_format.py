@@ -106,7 +106,7 @@ def test_two_shards_merge(tmp_path):
     path = str(tmp_path)
     b1, d1 = _make_blocks(rng, (32768, 65536, 65536))
     b0, d0 = _make_blocks(rng, (0, 32768, 65536))
-    _save(path, [b for b in b1 if not b.dense], 2, shard_index=1, shard_num=2)   # a non-zero shard saves no dense tensors
+    _save(path, [b for b in b1 if not b.is_dense()], 2, shard_index=1, shard_num=2)   # a non-zero shard saves no dense tensors
     _save(path, b0, 2, shard_index=0, shard_num=2)
     assert sorted(f for f in os.listdir(path) if f.endswith(".safetensors")) == [
         "model-%06d-of-000004.safetensors" % i for i in range(4)]
