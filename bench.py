@@ -438,22 +438,33 @@ class Config3:
         if self.step_no and self.step_no % self.filter_interval == 0:
             self.sweep(self.step_no - self.filter_step)
         self.step_no += 1
-        # dedup + find-or-insert, one pass; the plan brings the row of every unique id along
-        plan = self.ht.plan_lookup(self.table, ids, need_inverse=False, need_pos=False)
-        index = plan.index_buf
-        # one row per lookup: every unique row is read once out of the table and written to its
-        # occurrences (no [U, D] copy, no second pass over it); the step filter's stamps of the
-        # rows go out in the same pass
-        out = self.table.expand_rows(plan, index, None, "step_filter", self.step_t)
-        # the per-lookup gradients reduced per key and applied to the row in the same launch
-        self.ht.accept_planned_grad(self.table, index, plan, self.grad_out, plan.occ, cover=self.span)
+        plan = self.plan_of(ids)
+        out = self.expand(plan)
+        self.update(plan)
+        self.step_t += 1
+        self.settle(plan)
+        return out
+
+    # the stages of a step (tests look at the table between them)
+    def plan_of(self, ids):
+        """Dedup + find-or-insert, one pass; the plan brings the row of every unique id along (index_buf)."""
+        return self.ht.plan_lookup(self.table, ids, need_inverse=False, need_pos=False)
+
+    def expand(self, plan):
+        """One row per lookup: every unique row is read once out of the table and written to its occurrences (no
+        [U, D] copy, no second pass over it); the step filter's stamps of the rows go out in the same pass."""
+        return self.table.expand_rows(plan, plan.index_buf, None, "step_filter", self.step_t)
+
+    def update(self, plan):
+        """The per-lookup gradients reduced per key and applied to the row in the same launch."""
+        self.ht.accept_planned_grad(self.table, plan.index_buf, plan, self.grad_out, plan.occ, cover=self.span)
         self.opt.step()
         self.opt.zero_grad()
-        self.step_t += 1
-        # the whole step is queued: the unique count has arrived in pinned memory meanwhile
+
+    def settle(self, plan):
+        """The whole step is queued: the unique count has arrived in pinned memory meanwhile."""
         self.U = plan.U
         self.table.settle_count(self.U, plan)
-        return out
 
     def sweep(self, threshold):
         """The eviction sweep of the step filter (one pass over the id map + re-initialisation of

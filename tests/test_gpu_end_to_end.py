@@ -78,6 +78,42 @@ def test_config1_hundred_steps_bit_exact_rows(steps):
     _close(sg.slot_by_name("sparse_adagrad_accum").value().cpu().numpy(), np.concatenate(cpu.s0), "adagrad state")
 
 
+def test_config1_hundred_steps_hash_dedup_by_key():
+    """Benchmark config 1 again (batch 4096, 100 steps from seed 0, sum pooling, sparse Adagrad) with the
+    default dedup, the hash plan: lookup, expansion, the gradient handed over unsummed and the fused
+    gather-reduce + Adagrad. The plan orders new keys its own way, so every key that occurs in the 100 steps
+    is given its N(0, 0.01) row by key on both sides first (insert); everything is then compared by key with
+    the contract's flat tolerance: pooled outputs at every step, rows and Adagrad state at the end."""
+    bs, dim, steps = 1024, 16, 100
+    batches = [workloads.config1_step(step) for step in range(steps)]
+    keys = np.unique(np.concatenate([b[0] for b in batches]))
+    rows0 = (0.01 * np.random.default_rng(1).standard_normal((len(keys), dim))).astype(np.float32)
+    cpu = cpu_path.CpuTable(dim, bs, lambda b: np.zeros((bs, dim), np.float32), "adagrad", 0.01, 1e-8)
+    index_c, _ = cpu.lookup(keys)
+    oracle.block_insert(index_c, rows0, cpu.emb, bs)
+    table = HashTable([dim], block_size=bs, device="cuda", name="c1h")      # dedup="hash" is the default
+    table.insert(torch.from_numpy(keys).cuda(), torch.from_numpy(rows0).cuda())
+    table.train()
+    opt = SparseAdagrad(filter_out_sparse_param(table), lr=0.01, eps=1e-8)
+    for step, (ids, off, grad) in enumerate(batches):
+        pooled_c, _, _ = cpu_path.train_step(cpu, ids, off, None, grad)
+        rows = table(torch.from_numpy(ids).cuda())                              # [N, dim], request order
+        pooled = ragged_embedding_segment_reduce(rows, None, None, torch.from_numpy(off).cuda(), "sum")
+        pooled.backward(torch.from_numpy(grad).cuda())
+        assert table._hashtable_impl.pending_grads() == [1, 0]                 # handed over unsummed
+        opt.step()
+        opt.zero_grad()
+        _close(pooled.detach().cpu().numpy(), pooled_c, "pooled output, step %d" % step)
+    impl = table._hashtable_impl
+    rows_g = impl.lookup_index_readonly(torch.from_numpy(keys).cuda())
+    assert int(rows_g.min()) >= 0 and torch.unique(rows_g).numel() == len(keys) == impl.id_map_stats()[0]
+    rows_c = cpu.idmap.lookup_readonly(keys)
+    for slot, blocks in (("embedding", cpu.emb), ("sparse_adagrad_accum", cpu.s0)):
+        got = impl.get_slot(slot).index_select(rows_g).cpu().numpy()
+        _close(got, oracle.block_gather(rows_c, blocks, bs), slot)
+    assert _lib.poll_device_errors() == 0
+
+
 def test_config1_engine_path_matches_up_to_row_order():
     """Same workload through EmbeddingEngine (hash dedup, fused group pipeline): the row a key
     gets may differ, everything addressed by key must not."""

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import oracle
+import workloads
 from recis_amd import _lib, ops
 
 pytestmark = pytest.mark.gpu
@@ -103,7 +104,46 @@ def test_config3_lookups_at_scale(resident):
     known = t.lookup_index_readonly(ids)
     n_new = int(torch.unique(ids[known < 0]).numel())
     assert 0.05 * ids.numel() < n_new <= 0.1 * ids.numel() + 1
-    out = wl.step()                                            # consumes batch 0
+    # step 0 stage by stage (what wl.step() runs), with a look at the table between the stages
+    untouched_keys = workloads.splitmix64_torch(torch.arange(resident - 4096, resident, device="cuda"))
+    untouched_keys = untouched_keys[~torch.isin(untouched_keys, ids)]
+    wl.step_no += 1
+    plan = wl.plan_of(ids)
+    out = wl.expand(plan)
+    U = plan.U
+    index = plan.index_buf[:U]
+    # the gradient of every unique key, summed over its lookups on the plan the update will use, against a
+    # float64 index_add_ over the plan's inverse
+    g = ops.csr_gather_reduce(wl.grad_out, plan, plan.occ, cover=wl.span)
+    inv = plan.inverse.long()
+    assert torch.equal(plan.unique[inv], ids)
+    ref = torch.zeros(U, wl.D, device="cuda", dtype=torch.float64).index_add_(0, inv, wl.grad_out.double())
+    scale = torch.zeros(U, device="cuda", dtype=torch.float64).index_add_(
+        0, inv, wl.grad_out.double().abs().sum(1)).clamp_(min=1.0)
+    assert float(((g.double() - ref).abs().sum(1) / scale).max()) < 1e-5
+    del ref, scale, inv
+    # the fused gather-reduce + Adam on 4096 sampled keys (rows anywhere in the 29 GB slots) against the CPU
+    # oracle's Adam on those gradient rows, bit for bit
+    pick = torch.randperm(U, device="cuda")[:4096]
+    rows = index[pick]
+    names = ["embedding", "sparse_adam_exp_avg", "sparse_adam_exp_avg_sq"]
+    before = [_slot_rows(t, n, rows).cpu().numpy() for n in names]
+    state = wl.opt.state_dict()[1]
+    b1t = state["sparse_adam_beta1"].cpu().numpy().copy().reshape(1)
+    b2t = state["sparse_adam_beta2"].cpu().numpy().copy().reshape(1)
+    wl.update(plan)
+    wl.step_t += 1
+    wl.settle(plan)
+    after = [_slot_rows(t, n, rows).cpu().numpy() for n in names]
+    w, m, v = [b.copy() for b in before]
+    oracle.block_apply_adamw(np.arange(4096), g[pick].cpu().numpy(), [w], b1t, b2t, [m], [v], 1e-3, 0.9, 0.999, 1.0,
+                             1e-8, 4096)
+    for name, got, exp in zip(names, after, (w, m, v)):
+        np.testing.assert_array_equal(got, exp, err_msg=name)
+    # the stamps the expansion wrote: the step (0) at every looked-up row, the initial -1 elsewhere
+    assert bool((_slot_rows(t, "step_filter", index) == 0).all())
+    assert bool((_slot_rows(t, "step_filter", t.lookup_index_readonly(untouched_keys)) == -1).all())
+    del g
     lv1, idn1, _, _ = t.id_map_stats()
     assert lv1 == lv0 + n_new and idn1 == idn0 + n_new
     now = t.lookup_index_readonly(ids)
