@@ -458,9 +458,15 @@ int recis_unique_plan_jobs(recis_idmap* map, const int64_t* const* ids_ptrs, con
 int recis_plan_inverse_from_lists(const int32_t* row_start, const int32_t* list, const int64_t* counts_dev,
                                   int64_t n, int32_t* inverse_out, int32_t* pos_out, void* stream);
 /* How many times a workgroup of the plan polls the look-back word of an earlier bucket before it
- * gives up, raises RECIS_DEVERR_PLAN_OVERFLOW and goes on with zero (default 2^24: seconds; a
- * word is due within microseconds). For tests of that path. */
+ * gives up, raises RECIS_DEVERR_PLAN_OVERFLOW and goes on with zero (default
+ * RECIS_PLAN_SPIN_LIMIT_DEFAULT polls: about a second; a word is due within microseconds). A plan
+ * whose wait gave up has a wrong unique base from that bucket on; the error bit is the only sign
+ * of it, so callers that never fetch the staged count (which raises the bit) should poll
+ * recis_hip_staged_device_errors / recis_hip_poll_device_errors now and then. For tests of that
+ * path; the value applies to launches made after the call. */
+#define RECIS_PLAN_SPIN_LIMIT_DEFAULT (1u << 22)
 int recis_plan_set_spin_limit(int64_t polls);
+int recis_plan_get_spin_limit(int64_t* polls);
 /* Waits for the count staged by the last recis_unique_plan(…, RECIS_PLAN_STAGE_COUNT, stream). */
 int recis_unique_plan_count(int64_t* unique_count_host, void* stream);
 /* The soft-error bits (RECIS_DEVERR_*) that were set on the device when the last count of `stream`
@@ -478,7 +484,10 @@ int recis_hip_staged_device_errors(int* bits, void* stream);
  * RECIS_PLAN_NOALLOC_SCRATCH_MIB MiB array inside the library's code object (every device the
  * library runs on holds one until the process ends); the call makes no hipMalloc / hipFree /
  * hipHostMalloc and creates no event or stream. n > RECIS_PLAN_NOALLOC_MAX_IDS returns
- * RECIS_ERR_ARG. All calls on one device share the one array: two calls that overlap in time on a
+ * RECIS_ERR_ARG; on a device with so many compute units that the scratch layout of n ids (its
+ * histogram has one row per partition tile, and the tiles are sized by the compute-unit count)
+ * passes the array, the call returns RECIS_ERR_CAPACITY instead of launching (no gfx950 part does,
+ * up to the maximum). All calls on one device share the one array: two calls that overlap in time on a
  * device (different streams or threads) race; calls queued on one stream do not. (With
  * recis_hip_profile_enable(1) the profiler's own events are created as for every other call.)
  */

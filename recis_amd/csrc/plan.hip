@@ -1524,7 +1524,7 @@ static int plan_check_args(const int64_t* ids, int64_t n, int64_t* unique_out, i
 
 // Polls of one look-back word before a workgroup gives up (a word is due within microseconds; the
 // limit only bounds a wait that can never end, e.g. after a failed launch of an earlier kernel).
-static uint32_t g_spin_limit = 1u << 22;
+static std::atomic<uint32_t> g_spin_limit{RECIS_PLAN_SPIN_LIMIT_DEFAULT};
 
 // The plan's launches for n > 0 over the scratch buffer `base` (L.bytes bytes). `staged`: pinned host
 // words that receive the unique count (and the soft-error bits) as soon as they are final, or NULL.
@@ -1631,7 +1631,7 @@ static int plan_launch(const PlanLayout& L, char* base, const int64_t* ids, cons
   a.hot_cap = hot_cap;
   a.staged = staged;
   a.err = err;
-  a.spin_limit = g_spin_limit;
+  a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
   a.table = nullptr;
   a.mask = 0;
   a.index_out = index_out;
@@ -1766,7 +1766,13 @@ int recis_plan_inverse_from_lists(const int32_t* row_start, const int32_t* list,
 
 int recis_plan_set_spin_limit(int64_t polls) {
   RECIS_REQUIRE(polls >= 1 && polls <= (int64_t(1) << 31) - 1, "polls out of range");
-  g_spin_limit = static_cast<uint32_t>(polls);
+  g_spin_limit.store(static_cast<uint32_t>(polls), std::memory_order_relaxed);
+  return RECIS_OK;
+}
+
+int recis_plan_get_spin_limit(int64_t* polls) {
+  RECIS_REQUIRE(polls != nullptr, "polls must not be NULL");
+  *polls = g_spin_limit.load(std::memory_order_relaxed);
   return RECIS_OK;
 }
 

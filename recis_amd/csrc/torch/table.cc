@@ -429,10 +429,10 @@ Hashtable::Hashtable(int64_t block_size, const std::vector<int64_t>& embedding_s
       slice_begin_(slice_begin),
       slice_end_(slice_end),
       slice_size_(slice_size) {
-  TORCH_CHECK(device.is_cuda(), "tables live in GPU memory in this build; got device ", device);
+  children_info_ = c10::make_intrusive<recis::embedding::ChildrenInfo>(coalesce, children);  // validates the names
   TORCH_CHECK(block_size > 0, "block_size must be positive");
+  TORCH_CHECK(device.is_cuda(), "tables live in GPU memory in this build; got device ", device);
   if (!device_.has_index()) device_ = at::Device(device.type(), c10::hip::current_device());
-  children_info_ = c10::make_intrusive<recis::embedding::ChildrenInfo>(coalesce, children);
   {
     c10::DeviceGuard guard(device_);
     recis_idmap* m = nullptr;

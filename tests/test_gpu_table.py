@@ -408,13 +408,16 @@ def test_look_back_gives_up_instead_of_hanging():
     kernel still ends, the error bit says so, and the next plan with the default bound is right."""
     lib = _lib.lib()
     ids = torch.randint(0, 1 << 40, (400000,), device="cuda")
+    default = ctypes.c_int64(0)
+    _lib.check(lib.recis_plan_get_spin_limit(ctypes.byref(default)))
+    assert default.value == 1 << 22          # RECIS_PLAN_SPIN_LIMIT_DEFAULT
     try:
         _lib.check(lib.recis_plan_set_spin_limit(ctypes.c_int64(1)))
         for _ in range(3):
             ops.ids_unique_plan(ids, wait=False)   # the count is not read: a reader would raise the error bit
         torch.cuda.synchronize()
     finally:
-        _lib.check(lib.recis_plan_set_spin_limit(ctypes.c_int64(1 << 24)))
+        _lib.check(lib.recis_plan_set_spin_limit(default))
     bits = _lib.poll_device_errors()
     assert bits in (0, _lib.DEVERR_PLAN_OVERFLOW)
     p = ops.ids_unique_plan(ids)

@@ -534,3 +534,20 @@ def test_config4_shaped_step_through_the_library_boundary():
             got = ht.get_slot(name).index_select(rows).cpu().numpy()
             np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-6, err_msg=name)
     assert _lib.poll_device_errors() == 0
+
+
+def test_slot_handle_taken_before_an_insert_sees_the_new_blocks():
+    """Slot.values() aliases the live storage: a handle (the optimizer's state slots, a saver's) that was taken
+    before later lookups added blocks lists those blocks too (block_num = (id_num + block_size) / block_size,
+    csrc/embedding/hashtable.cc:255-261)."""
+    ht = _make_table(16, 4)
+    emb = ht.slot_group().slot_by_name("embedding")        # taken while the table is empty
+    assert len(emb.values()) == 0
+    ht.embedding_lookup(torch.arange(10, device="cuda"), False)
+    assert len(emb.values()) == 1 and emb.value().shape == (16, 4)
+    ht.embedding_lookup(torch.arange(100, 150, device="cuda"), False)   # 60 ids: (60 + 16) / 16 = 4 blocks
+    blocks = emb.values()
+    assert len(blocks) == 4 and all(b.shape == (16, 4) for b in blocks)
+    blocks[3].fill_(2.5)                                                 # a view, not a copy
+    assert float(ht.get_slot("embedding").value()[48:].min()) == 2.5
+    assert _lib.poll_device_errors() == 0

@@ -189,3 +189,23 @@ def test_every_name_the_reference_registers_is_registered():
         assert not lost, (cls, lost)
     # (read-only attributes need an instance: tests/test_gpu_torch_library.py reads HashtableImpl.hashtable_tag)
     assert golden["readonly_attributes"] == {"HashtableImpl": ["hashtable_tag"]}
+
+
+def test_children_are_validated_as_in_the_reference():
+    """csrc/embedding/children_info.cc:38-48: no children, too many, more than one without coalescing and
+    duplicate names are refused (before anything touches a device)."""
+    gen = torch.classes.recis.Generator.make_constant_generator([4, 2], torch.float32, 0.0)
+
+    def make(coalesce, children):
+        return torch.ops.recis.make_hashtable(4, [2], torch.float32, torch.device("cpu"), coalesce, children, gen, 0,
+                                              65536, 65536)
+    with pytest.raises(RuntimeError, match="empty children"):
+        make(True, [])
+    with pytest.raises(RuntimeError, match="exceeds max children size"):
+        make(True, ["c%d" % i for i in range(4095)])
+    with pytest.raises(RuntimeError, match="non coalesce has more than one child"):
+        make(False, ["a", "b"])
+    with pytest.raises(RuntimeError, match="duplicate child"):
+        make(True, ["a", "b", "a"])
+    with pytest.raises(RuntimeError, match="tables live in GPU memory"):   # valid names: the device is looked at next
+        make(True, ["c%d" % i for i in range(4094)])

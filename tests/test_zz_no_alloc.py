@@ -85,3 +85,28 @@ def test_noalloc_plan_rejects_what_does_not_fit():
     t = torch.zeros(n, dtype=torch.int64, device="cuda")
     with pytest.raises(_lib.RecisHipError, match="at most"):
         _run("noalloc", t)
+
+
+def test_noalloc_plan_allocates_nothing(rng):
+    """Free device memory as the runtime reports it (hipMemGetInfo) is the same before and after a call:
+    the outputs are the caller's, the scratch is the library's static array. (The first call on a device
+    looks the array's address up; the one measured is a later one.)"""
+    ids = torch.from_numpy(_ids(rng, 100_000, 0.3)).cuda()
+    n, dev = ids.numel(), ids.device
+    hot_cap = n // 64 + n // 2048 + 2
+    i32 = lambda k: torch.empty(k, dtype=torch.int32, device=dev)
+    outs = (torch.empty(n, dtype=torch.int64, device=dev), i32(n), i32(n + 1), i32(n), i32(n), i32(2 * hot_cap),
+            torch.empty(2, dtype=torch.int64, device=dev))
+    lib = _lib.lib()
+
+    def call():
+        check(lib.recis_unique_plan_noalloc(ptr(ids), i64(n), ptr(outs[0]), ptr(outs[1]), ptr(outs[2]), ptr(outs[3]),
+                                            ptr(outs[4]), ptr(outs[5]), i64(hot_cap), ptr(outs[6]), stream_ptr(dev)))
+        torch.cuda.synchronize()
+
+    call()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        call()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert int(outs[6][0]) == len(np.unique(ids.cpu().numpy()))
