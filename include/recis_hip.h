@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define RECIS_HIP_ABI_VERSION 1
+#define RECIS_HIP_ABI_VERSION 2
 
 /* status codes */
 #define RECIS_OK 0
@@ -116,7 +116,8 @@ int recis_segment_reduce_forward(const void* unique_emb, int emb_dtype,
  * recis/nn/modules/embedding.py:592-624 (emb_reduce) is neither written nor read. SUM, MEAN and TILE.
  */
 int recis_segment_reduce_forward_blocks(const void* const* emb_blocks_dev, int64_t n_blocks,
-                                        int64_t block_rows, const int64_t* row_index, int emb_dtype,
+                                        int64_t block_rows, int64_t row_pitch_bytes,
+                                        const int64_t* row_index, int emb_dtype,
                                         const void* weight, int weight_dtype,
                                         const void* reverse_indices, int rev_is64,
                                         const void* offsets, int off_is64, void* out, int out_dtype,
@@ -298,6 +299,16 @@ int recis_scatter_ids_with_mask(int64_t* out_ids, int64_t out_size, const int64_
  * Rows are moved as bytes, so any element type works. Block bases must be
  * aligned to the largest power of two (<= 16) that divides row_bytes.
  *
+ * row_pitch_bytes, here and in every entry point below that takes a block list: the
+ * distance from one row of a block to the next, 0 when rows lie back to back (the
+ * reference's layout, one array per slot). A table that keeps a parameter row and its
+ * optimizer state next to each other (w | m | v in one allocation, the pointer tables of
+ * the three slots offset by one row width each) passes the combined width, so that one
+ * key's rows share DRAM pages and cache lines. The pitch must be a multiple of the
+ * element size and of the alignment above (recis_block_gather / recis_block_insert, which
+ * move bytes, narrow their vector to what the pitch allows instead). Slots that share one
+ * call share one pitch.
+ *
  * Replace the device branches of csrc/ops/block_ops.cc:
  *   recis_gather             gather_cuda              (block_ops.cc:262-268)
  *   recis_block_gather       block_gather_cuda        (block_ops.cc:270-282, also
@@ -312,11 +323,11 @@ int recis_scatter_ids_with_mask(int64_t* out_ids, int64_t out_size, const int64_
 int recis_gather(const void* ids, int ids_is64, const void* emb, int64_t rows, void* out,
                  int64_t n, int64_t row_bytes, void* stream);
 int recis_block_gather(const int64_t* ids, void* const* blocks_dev, int64_t n_blocks,
-                       int64_t block_size, int64_t default_key, int readonly, void* out,
+                       int64_t block_size, int64_t row_pitch_bytes, int64_t default_key, int readonly, void* out,
                        int64_t n, int64_t row_bytes, void* stream);
 int recis_block_insert(const int64_t* ids, const void* emb, int broadcast, const uint8_t* mask,
-                       void* const* blocks_dev, int64_t n_blocks, int64_t block_size, int64_t n,
-                       int64_t row_bytes, void* stream);
+                       void* const* blocks_dev, int64_t n_blocks, int64_t block_size,
+                       int64_t row_pitch_bytes, int64_t n, int64_t row_bytes, void* stream);
 int recis_block_filter(const int64_t* ids, void* const* blocks_dev, int64_t n_blocks,
                        int64_t block_size, int64_t threshold, int slot_is64, uint8_t* mask_out,
                        int64_t n, void* stream);
@@ -338,8 +349,8 @@ int recis_block_filter(const int64_t* ids, void* const* blocks_dev, int64_t n_bl
 int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dtype,
                             void* const* emb_blocks_dev, void* const* exp_avg_blocks_dev,
                             void* const* exp_avg_sq_blocks_dev, int64_t n_blocks,
-                            int64_t block_size, int row_dtype, void* beta1_t, void* beta2_t,
-                            int beta_is_f64, double lr, double beta1, double beta2,
+                            int64_t block_size, int64_t row_pitch_bytes, int row_dtype,
+                            void* beta1_t, void* beta2_t, int beta_is_f64, double lr, double beta1, double beta2,
                             double weight_decay, double eps, int64_t n, int64_t D, void* stream);
 
 /*
@@ -349,8 +360,9 @@ int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dty
  */
 int recis_block_apply_adagrad(const int64_t* index, const void* grad, int grad_dtype,
                               void* const* emb_blocks_dev, void* const* accum_blocks_dev,
-                              int64_t n_blocks, int64_t block_size, int row_dtype, double lr,
-                              double eps, int64_t n, int64_t D, void* stream);
+                              int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes,
+                              int row_dtype, double lr, double eps, int64_t n, int64_t D,
+                              void* stream);
 
 /* ------------------------------------------------------------------------- *
  * Key tagging, offset merging, dedup
@@ -573,8 +585,8 @@ int recis_csr_gather_reduce_adamw(const void* rows, int rows_dtype, int64_t n_ro
                                   int64_t U, int64_t D, const void* cover_offsets, int cover_is64,
                                   int64_t cover_S, const int64_t* row_index, void* const* emb_blocks_dev,
                                   void* const* exp_avg_blocks_dev, void* const* exp_avg_sq_blocks_dev,
-                                  int64_t n_blocks, int64_t block_size, int row_dtype, void* beta1_t,
-                                  void* beta2_t, int beta_is_f64, double lr, double beta1, double beta2,
+                                  int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes,
+                                  int row_dtype, void* beta1_t, void* beta2_t, int beta_is_f64, double lr, double beta1, double beta2,
                                   double weight_decay, double eps, void* stream);
 int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
                                     const void* coef, int coef_dtype, const int32_t* row_start,
@@ -582,7 +594,8 @@ int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_
                                     int64_t U, int64_t D, const void* cover_offsets, int cover_is64,
                                     int64_t cover_S, const int64_t* row_index, void* const* emb_blocks_dev,
                                     void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
-                                    int row_dtype, double lr, double eps, void* stream);
+                                    int64_t row_pitch_bytes, int row_dtype, double lr, double eps,
+                                    void* stream);
 
 /*
  * Gather-reduce with TWO inputs over the same occurrence lists: list entry k of unique id u adds
@@ -622,14 +635,14 @@ int recis_csr_gather_reduce2_adamw(const recis_csr_input* a, const recis_csr_inp
                                    const int64_t* counts_dev, int64_t U, int64_t D, const int64_t* row_index,
                                    void* const* emb_blocks_dev, void* const* exp_avg_blocks_dev,
                                    void* const* exp_avg_sq_blocks_dev, int64_t n_blocks, int64_t block_size,
-                                   int row_dtype, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
+                                   int64_t row_pitch_bytes, int row_dtype, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
                                    double beta1, double beta2, double weight_decay, double eps, void* stream);
 int recis_csr_gather_reduce2_adagrad(const recis_csr_input* a, const recis_csr_input* b,
                                      const int32_t* row_start, const int32_t* hot_items, int64_t hot_cap,
                                      const int64_t* counts_dev, int64_t U, int64_t D, const int64_t* row_index,
                                      void* const* emb_blocks_dev, void* const* accum_blocks_dev,
-                                     int64_t n_blocks, int64_t block_size, int row_dtype, double lr, double eps,
-                                     void* stream);
+                                     int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes,
+                                     int row_dtype, double lr, double eps, void* stream);
 
 /*
  * The transpose of recis_csr_gather_reduce (no reference counterpart; it produces what
@@ -645,7 +658,7 @@ int recis_csr_gather_reduce2_adagrad(const recis_csr_input* a, const recis_csr_i
  * passes n): rows at and past counts_dev[0], the count the plan left on the device, are skipped.
  */
 int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks,
-                          int64_t block_rows, const int64_t* row_index, int rows_dtype,
+                          int64_t block_rows, int64_t row_pitch_bytes, const int64_t* row_index, int rows_dtype,
                           const void* weight, int weight_dtype, const int32_t* row_start,
                           const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
                           const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
@@ -659,7 +672,8 @@ int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t
  * stamps ride on the pass that reads the rows anyway instead of taking a launch of their own.
  */
 int recis_csr_expand_rows_stamped(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks,
-                                  int64_t block_rows, const int64_t* row_index, int rows_dtype,
+                                  int64_t block_rows, int64_t row_pitch_bytes,
+                                  const int64_t* row_index, int rows_dtype,
                                   const void* weight, int weight_dtype, const int32_t* row_start,
                                   const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
                                   const int64_t* counts_dev, void* out, int out_dtype, int64_t U,

@@ -54,8 +54,8 @@ def lib():
         _lib = ctypes.CDLL(LIB_PATH)
         _lib.recis_hip_last_error.restype = ctypes.c_char_p
         abi = _lib.recis_hip_abi_version()
-        if abi != 1:
-            raise RecisHipError("librecis_hip.so ABI %d, expected 1: rebuild with "
+        if abi != 2:
+            raise RecisHipError("librecis_hip.so ABI %d, expected 2: rebuild with "
                                 "python -m recis_amd.build" % abi)
     return _lib
 

@@ -31,6 +31,7 @@ struct BlockArgs {
   int64_t block_size;
   int64_t n;
   int row_bytes;
+  int64_t pitch_bytes;  // from one row of a block to the next (row_bytes when the rows are dense)
   int lpr_log2;
   int* err;
 };
@@ -53,7 +54,7 @@ __device__ __forceinline__ char* row_address(const BlockArgs& a, int64_t idx) {
     r = static_cast<uint32_t>(idx) - q * bs;
   }
   if (b >= a.n_blocks) return nullptr;
-  return a.blocks[b] + r * static_cast<int64_t>(a.row_bytes);
+  return a.blocks[b] + r * a.pitch_bytes;
 }
 
 template <int VB>
@@ -155,7 +156,7 @@ int dispatch_vb(int vb, F&& f) {
 }
 
 int fill_args(BlockArgs& a, const int64_t* ids, void* const* blocks_dev, int64_t n_blocks,
-              int64_t block_size, int64_t n, int64_t row_bytes, int vb) {
+              int64_t block_size, int64_t row_pitch_bytes, int64_t n, int64_t row_bytes, int vb) {
   RECIS_REQUIRE(n >= 0, "n must be >= 0");
   RECIS_REQUIRE(n_blocks >= 1 && block_size >= 1, "need at least one block (n_blocks=%lld block_size=%lld)",
                 (long long)n_blocks, (long long)block_size);
@@ -167,6 +168,10 @@ int fill_args(BlockArgs& a, const int64_t* ids, void* const* blocks_dev, int64_t
   a.block_size = block_size;
   a.n = n;
   a.row_bytes = static_cast<int>(row_bytes);
+  a.pitch_bytes = row_pitch_bytes > 0 ? row_pitch_bytes : row_bytes;
+  RECIS_REQUIRE(a.pitch_bytes >= row_bytes && a.pitch_bytes % vb == 0,
+                "row pitch %lld does not fit rows of %lld bytes moved %d bytes at a time", (long long)a.pitch_bytes,
+                (long long)row_bytes, vb);
   a.lpr_log2 = std::min(6, ilog2_ceil((row_bytes + vb - 1) / vb));
   a.err = device_error_word(current_device());
   RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
@@ -205,14 +210,14 @@ int recis_gather(const void* ids, int ids_is64, const void* emb, int64_t rows, v
 }
 
 int recis_block_gather(const int64_t* ids, void* const* blocks_dev, int64_t n_blocks,
-                       int64_t block_size, int64_t default_key, int readonly, void* out, int64_t n,
-                       int64_t row_bytes, void* stream_) {
+                       int64_t block_size, int64_t row_pitch_bytes, int64_t default_key, int readonly, void* out,
+                       int64_t n, int64_t row_bytes, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (n == 0) return RECIS_OK;
   RECIS_REQUIRE(out != nullptr, "out must not be NULL");
-  const int vb = pick_vec_bytes(row_bytes, reinterpret_cast<uintptr_t>(out));
+  const int vb = pick_vec_bytes(row_bytes, reinterpret_cast<uintptr_t>(out) | static_cast<uintptr_t>(row_pitch_bytes));
   BlockArgs a;
-  if (int rc = fill_args(a, ids, blocks_dev, n_blocks, block_size, n, row_bytes, vb)) return rc;
+  if (int rc = fill_args(a, ids, blocks_dev, n_blocks, block_size, row_pitch_bytes, n, row_bytes, vb)) return rc;
   const int rows_per_block = kBlock >> a.lpr_log2;
   const int64_t grid = (n + rows_per_block - 1) / rows_per_block;
   return dispatch_vb(vb, [&](auto tag) {
@@ -226,14 +231,14 @@ int recis_block_gather(const int64_t* ids, void* const* blocks_dev, int64_t n_bl
 }
 
 int recis_block_insert(const int64_t* ids, const void* emb, int broadcast, const uint8_t* mask,
-                       void* const* blocks_dev, int64_t n_blocks, int64_t block_size, int64_t n,
-                       int64_t row_bytes, void* stream_) {
+                       void* const* blocks_dev, int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes,
+                       int64_t n, int64_t row_bytes, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (n == 0) return RECIS_OK;
   RECIS_REQUIRE(emb != nullptr, "emb must not be NULL");
-  const int vb = pick_vec_bytes(row_bytes, reinterpret_cast<uintptr_t>(emb));
+  const int vb = pick_vec_bytes(row_bytes, reinterpret_cast<uintptr_t>(emb) | static_cast<uintptr_t>(row_pitch_bytes));
   BlockArgs a;
-  if (int rc = fill_args(a, ids, blocks_dev, n_blocks, block_size, n, row_bytes, vb)) return rc;
+  if (int rc = fill_args(a, ids, blocks_dev, n_blocks, block_size, row_pitch_bytes, n, row_bytes, vb)) return rc;
   const int rows_per_block = kBlock >> a.lpr_log2;
   const int64_t grid = (n + rows_per_block - 1) / rows_per_block;
   return dispatch_vb(vb, [&](auto tag) {
@@ -252,7 +257,7 @@ int recis_block_filter(const int64_t* ids, void* const* blocks_dev, int64_t n_bl
   if (n == 0) return RECIS_OK;
   RECIS_REQUIRE(mask_out != nullptr, "mask_out must not be NULL");
   BlockArgs a;
-  if (int rc = fill_args(a, ids, blocks_dev, n_blocks, block_size, n, slot_is64 ? 8 : 4, slot_is64 ? 8 : 4))
+  if (int rc = fill_args(a, ids, blocks_dev, n_blocks, block_size, 0, n, slot_is64 ? 8 : 4, slot_is64 ? 8 : 4))
     return rc;
   block_filter_kernel<<<dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, stream>>>(a, threshold, slot_is64,
                                                                                    mask_out);

@@ -33,6 +33,7 @@ struct ExpArgs {
   const int64_t* row_index;  // rows in a block list: unique row u is row row_index[u] (negative = zeros)
   const void* const* blocks;
   int64_t block_rows, n_blocks;
+  int64_t pitch;  // elements from one row of a block to the next
   int32_t hot_len;
   const int32_t* hot_items;
   const int64_t* counts;
@@ -50,7 +51,10 @@ __device__ __align__(256) const unsigned char g_expand_zero_row[8192 * 4] = {};
 
 constexpr int kExpandRows = 2;  // unique rows a lane group works at a time: their loads are in flight together (4: slower)
 
-template <typename TIn, typename TOut, int VEC, bool BLK>
+// STREAM: the rows are read with the streaming hint (a table larger than the caches keep, and any
+// dense array of rows: each row is read once here); without it for a small table, whose rows the
+// update at the end of the step and the next step's lookups find in the caches again.
+template <typename TIn, typename TOut, int VEC, bool BLK, bool STREAM = true>
 __global__ void __launch_bounds__(kBlock)
 csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs a) {
   const int D = a.D;
@@ -72,7 +76,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
         if (b >= a.n_blocks || r >= a.block_rows) {
           raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
         } else {
-          src = static_cast<const TIn*>(a.blocks[b]) + r * D;
+          src = static_cast<const TIn*>(a.blocks[b]) + r * a.pitch;
           if (a.stamp_blocks && c0 == 0 && stamp_here) static_cast<int64_t*>(a.stamp_blocks[b])[r] = a.stamp_value[0];
         }
       }
@@ -80,7 +84,10 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
       src = rows + u * D;
     }
     if (src) {
-      load_pack_stream<TIn, VEC>(src + c0, v);  // every row is read once here
+      if constexpr (STREAM)
+        load_pack_stream<TIn, VEC>(src + c0, v);  // every row is read once here
+      else
+        load_pack<TIn, VEC>(src + c0, v);
     } else {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) v[j] = 0.f;
@@ -211,7 +218,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
     }
 #pragma unroll
     for (int r = 0; r < kExpandRows; ++r) {
-      src[r] = ok[r] ? static_cast<const TIn*>(base[r]) + off[r] * D : reinterpret_cast<const TIn*>(g_expand_zero_row);
+      src[r] = ok[r] ? static_cast<const TIn*>(base[r]) + off[r] * a.pitch : reinterpret_cast<const TIn*>(g_expand_zero_row);
       if (a.stamp_blocks && cl == 0 && ok[r]) static_cast<int64_t*>(stamp_base[r])[off[r]] = stamp;
     }
     if (bad_any) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
@@ -223,7 +230,12 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
   for (int c0 = cl * VEC; c0 < D; c0 += VEC << a.lpr_log2) {
     float v[kExpandRows][VEC];
 #pragma unroll
-    for (int r = 0; r < kExpandRows; ++r) load_pack_stream<TIn, VEC>(src[r] + c0, v[r]);  // every row is read once here
+    for (int r = 0; r < kExpandRows; ++r) {
+      if constexpr (STREAM)
+        load_pack_stream<TIn, VEC>(src[r] + c0, v[r]);  // every row is read once here
+      else
+        load_pack<TIn, VEC>(src[r] + c0, v[r]);
+    }
 #pragma unroll
     for (int r = 0; r < kExpandRows; ++r)
       if (is_short[r]) store_list(start[r], end[r], 1, c0, v[r]);
@@ -475,14 +487,14 @@ int recis_csr_gather_reduce_adamw(const void* rows, int rows_dtype, int64_t n_ro
                                   int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
                                   const int64_t* row_index, void* const* emb_blocks_dev,
                                   void* const* exp_avg_blocks_dev, void* const* exp_avg_sq_blocks_dev,
-                                  int64_t n_blocks, int64_t block_size, int row_dtype, void* beta1_t, void* beta2_t,
-                                  int beta_is_f64, double lr, double beta1, double beta2, double weight_decay,
-                                  double eps, void* stream_) {
+                                  int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes, int row_dtype,
+                                  void* beta1_t, void* beta2_t, int beta_is_f64, double lr, double beta1, double beta2,
+                                  double weight_decay, double eps, void* stream_) {
   RECIS_REQUIRE(beta1_t != nullptr && beta2_t != nullptr, "beta1_t / beta2_t must not be NULL");
   FuseArgs f{};
   if (U > 0) {
     if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, exp_avg_blocks_dev, exp_avg_sq_blocks_dev, true, n_blocks,
-                                block_size, D, row_dtype))
+                                block_size, row_pitch_bytes, D, row_dtype))
       return rc;
   }
   CsrRequest r = one_input_request(rows, rows_dtype, n_rows, src, coef, coef_dtype, row_start, hot_items, hot_cap,
@@ -499,11 +511,11 @@ int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_
                                     int64_t D, const void* cover_offsets, int cover_is64, int64_t cover_S,
                                     const int64_t* row_index, void* const* emb_blocks_dev,
                                     void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
-                                    int row_dtype, double lr, double eps, void* stream_) {
+                                    int64_t row_pitch_bytes, int row_dtype, double lr, double eps, void* stream_) {
   if (U == 0) return RECIS_OK;
   FuseArgs f;
-  if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, accum_blocks_dev, nullptr, false, n_blocks, block_size, D,
-                              row_dtype))
+  if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, accum_blocks_dev, nullptr, false, n_blocks, block_size,
+                              row_pitch_bytes, D, row_dtype))
     return rc;
   f.lr = static_cast<float>(lr);
   f.eps = static_cast<float>(eps);
@@ -517,17 +529,17 @@ int recis_csr_gather_reduce_adagrad(const void* rows, int rows_dtype, int64_t n_
 
 
 int recis_csr_expand_rows(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows,
-                          const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
+                          int64_t row_pitch_bytes, const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
                           const int32_t* row_start, const int32_t* dst, const int32_t* hot_items, int64_t hot_cap,
                           const int64_t* counts_dev, void* out, int out_dtype, int64_t U, int64_t n_out, int64_t D,
                           void* stream_) {
-  return recis_csr_expand_rows_stamped(rows, emb_blocks_dev, n_blocks, block_rows, row_index, rows_dtype, weight,
+  return recis_csr_expand_rows_stamped(rows, emb_blocks_dev, n_blocks, block_rows, row_pitch_bytes, row_index, rows_dtype, weight,
                                        weight_dtype, row_start, dst, hot_items, hot_cap, counts_dev, out, out_dtype, U,
                                        n_out, D, nullptr, nullptr, stream_);
 }
 
 int recis_csr_expand_rows_stamped(const void* rows, void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows,
-                                  const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
+                                  int64_t row_pitch_bytes, const int64_t* row_index, int rows_dtype, const void* weight, int weight_dtype,
                                   const int32_t* row_start, const int32_t* dst, const int32_t* hot_items,
                                   int64_t hot_cap, const int64_t* counts_dev, void* out, int out_dtype, int64_t U,
                                   int64_t n_out, int64_t D, void* const* stamp_blocks_dev,
@@ -564,6 +576,9 @@ int recis_csr_expand_rows_stamped(const void* rows, void* const* emb_blocks_dev,
   a.row_index = row_index;
   a.blocks = emb_blocks_dev;
   a.block_rows = block_rows;
+  a.pitch = blk ? pitch_elements(row_pitch_bytes, D, in_sz, vb_in) : D;
+  RECIS_REQUIRE(a.pitch >= D, "row pitch of %lld bytes does not fit rows of %lld elements", (long long)row_pitch_bytes,
+                (long long)D);
   a.n_blocks = n_blocks;
   a.hot_len = hot_cap > 0 ? kHotLen : INT_MAX;
   a.hot_items = hot_items;
@@ -584,8 +599,11 @@ int recis_csr_expand_rows_stamped(const void* rows, void* const* emb_blocks_dev,
         return fail(RECIS_ERR_ARG, "internal: vector too wide");
       } else {
         RECIS_TIME_KERNEL("csr_expand_kernel", stream)
-        if (blk)
+        if (blk && stream_table_rows(RowBlocks{n_blocks, block_rows, a.D, a.pitch}, sizeof(TIn), 1))
           csr_expand_kernel<TIn, TOut, VEC, true><<<grid, dim3(kBlock), 0, stream>>>(nullptr, static_cast<TOut*>(out), a);
+        else if (blk)
+          csr_expand_kernel<TIn, TOut, VEC, true, false><<<grid, dim3(kBlock), 0, stream>>>(nullptr,
+                                                                                           static_cast<TOut*>(out), a);
         else
           csr_expand_kernel<TIn, TOut, VEC, false><<<grid, dim3(kBlock), 0, stream>>>(static_cast<const TIn*>(rows),
                                                                                     static_cast<TOut*>(out), a);

@@ -68,7 +68,12 @@ struct CsrArgs {
 //   kEpiAdam     the sum is the gradient of table row row_index[u]: the Adam-family update of that
 //                row (parameter and both moments) is applied at once, the gradient never written
 //   kEpiAdagrad  the same with the Adagrad update
-enum { kEpiStore = 0, kEpiAdam = 1, kEpiAdagrad = 2 };
+//   kEpiAdamCached  kEpiAdam without the streaming hint on the table rows: what the host launches
+//                for a kEpiAdam request on a table small enough to stay in the caches (see
+//                stream_table_rows); a kernel of its own, because one kernel holding both kinds of
+//                access costs registers (measured: 126 -> 219 us)
+enum { kEpiStore = 0, kEpiAdam = 1, kEpiAdagrad = 2, kEpiAdamCached = 3 };
+constexpr bool epi_is_adam(int epi) { return epi == kEpiAdam || epi == kEpiAdamCached; }
 struct FuseArgs {
   const int64_t* row_index;  // [U]; a negative index skips the row
   void* const* emb;          // block tables (device arrays of block pointers)
@@ -121,22 +126,19 @@ __device__ __forceinline__ RowPlaces<T> row_places(const FuseArgs& f, int* err, 
     raise_device_error(err, RECIS_DEVERR_INDEX_RANGE);
     return p;
   }
-  const int64_t at = off * f.rb.D;
+  const int64_t at = off * f.rb.pitch;
   p.w = static_cast<T*>(f.emb[b]) + at;
   p.s0 = static_cast<T*>(f.s0[b]) + at;
-  if constexpr (EPI == kEpiAdam) p.s1 = static_cast<T*>(f.s1[b]) + at;
+  if constexpr (epi_is_adam(EPI)) p.s1 = static_cast<T*>(f.s1[b]) + at;
   return p;
 }
 template <typename T, int VEC, int EPI>
 __device__ __forceinline__ void fused_row_update_at(const FuseArgs& f, const RowPlaces<T>& p, int c0,
                                                     const float (&acc)[VEC], double alpha) {
   if (p.w == nullptr) return;
-  if constexpr (EPI == kEpiAdam) {
-    // streaming accesses to the table rows (see load_row_pack_of_table), whatever the table's size:
-    // choosing by size at run time means two copies of the update in the kernel, and those cost
-    // registers (measured: 126 -> 219 us); a table small enough to stay cached pays with reads
-    // from memory that the cache could have served
-    adam_update_pack<T, VEC, true>(p.w + c0, p.s0 + c0, p.s1 + c0, acc, alpha, f.adam);
+  if constexpr (epi_is_adam(EPI)) {
+    // kEpiAdam: streaming accesses to the table rows (see load_row_pack_of_table)
+    adam_update_pack<T, VEC, EPI == kEpiAdam>(p.w + c0, p.s0 + c0, p.s1 + c0, acc, alpha, f.adam);
   } else {
     adagrad_update_pack<T, VEC>(p.w + c0, p.s0 + c0, acc, f.lr, f.eps);
   }
@@ -315,7 +317,7 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   const int groups = kWave >> a.lpr_log2;  // lane groups of a wave
   const int g = lane >> a.lpr_log2;        // this lane's group in its wave
   __shared__ double s_alpha;  // Adam: alpha of this step, worked out once per workgroup
-  if constexpr (EPI == kEpiAdam) {
+  if constexpr (epi_is_adam(EPI)) {
     if (threadIdx.x == 0) {
       double b1, b2;
       s_alpha = f.adam.alpha != nullptr ? f.adam.alpha[0] : alpha_from_powers(f, b1, b2);
@@ -458,9 +460,9 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
   auto finish = [&](int64_t row, int c0, float (&acc)[VEC]) {
     if constexpr (EPI != kEpiStore) {
       if constexpr (kEarlyPlaces)
-        fused_row_update_at<TRow, VEC, EPI>(f, places, c0, acc, EPI == kEpiAdam ? s_alpha : 0.0);
+        fused_row_update_at<TRow, VEC, EPI>(f, places, c0, acc, epi_is_adam(EPI) ? s_alpha : 0.0);
       else
-        fused_row_update<TOut, VEC, EPI>(f, a.err, idx_mine, c0, acc, EPI == kEpiAdam ? s_alpha : 0.0);
+        fused_row_update<TOut, VEC, EPI>(f, a.err, idx_mine, c0, acc, epi_is_adam(EPI) ? s_alpha : 0.0);
     } else {
       TOut* dst = out + row * D + c0;
       if (a.accumulate) {
@@ -521,7 +523,7 @@ template <typename TOut, int VEC, int EPI = kEpiStore>
 __global__ void __launch_bounds__(kBlock)
 csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
   double alpha = 0;
-  if constexpr (EPI == kEpiAdam) {
+  if constexpr (epi_is_adam(EPI)) {
     alpha = f.adam.alpha[0];
     if (f.advance_powers && blockIdx.x == 0 && threadIdx.x == 0) {  // nobody reads them in this kernel
       double b1, b2;
@@ -765,7 +767,7 @@ int csr_gather_reduce_run(const CsrRequest& r) {
         auto launch = [&](auto epi_tag) {
           constexpr int EPI = decltype(epi_tag)::value;
           {
-            RECIS_TIME_KERNEL(EPI == kEpiStore ? "csr_rows_kernel" : EPI == kEpiAdam ? "csr_rows_adam_kernel"
+            RECIS_TIME_KERNEL(EPI == kEpiStore ? "csr_rows_kernel" : epi_is_adam(EPI) ? "csr_rows_adam_kernel"
                                                                                       : "csr_rows_adagrad_kernel", stream)
             if (a.n_parts > 0) {
               if constexpr (TWO) {  // the second input in parts
@@ -788,7 +790,7 @@ int csr_gather_reduce_run(const CsrRequest& r) {
           }
           if (hot_cap > 0) {
             FuseArgs f_fin = f;
-            if (EPI == kEpiAdam && f.adam.alpha == nullptr) {  // the row kernel worked alpha out itself
+            if (epi_is_adam(EPI) && f.adam.alpha == nullptr) {  // the row kernel worked alpha out itself
               f_fin.adam.alpha = f.alpha_ws;
               f_fin.advance_powers = 1;
             }
@@ -799,8 +801,10 @@ int csr_gather_reduce_run(const CsrRequest& r) {
         };
         constexpr bool all = ONLY_EPI < 0;
         if (epi == kEpiAdam) {
-          if constexpr ((all || ONLY_EPI == kEpiAdam) && VEC * sizeof(TOut) <= 16)
-            return launch(std::integral_constant<int, kEpiAdam>{});
+          if constexpr ((all || ONLY_EPI == kEpiAdam) && VEC * sizeof(TOut) <= 16) {
+            if (stream_table_rows(f.rb, sizeof(TOut), 3)) return launch(std::integral_constant<int, kEpiAdam>{});
+            return launch(std::integral_constant<int, kEpiAdamCached>{});
+          }
         } else if (epi == kEpiAdagrad) {
           if constexpr ((all || ONLY_EPI == kEpiAdagrad) && VEC * sizeof(TOut) <= 16)
             return launch(std::integral_constant<int, kEpiAdagrad>{});
@@ -862,7 +866,8 @@ int csr_gather_reduce_run(const CsrRequest& r) {
 
 // Shared front of the fused entry points: argument checks and the table description.
 inline int fill_fuse_args(FuseArgs& f, const int64_t* row_index, void* const* emb, void* const* s0, void* const* s1,
-                          bool need_s1, int64_t n_blocks, int64_t block_size, int64_t D, int row_dtype) {
+                          bool need_s1, int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes, int64_t D,
+                          int row_dtype) {
   RECIS_REQUIRE(row_index && emb && s0 && (s1 || !need_s1), "row_index and the block tables must not be NULL");
   RECIS_REQUIRE(n_blocks >= 1 && block_size >= 1, "bad block geometry (n_blocks=%lld block_size=%lld)",
                 (long long)n_blocks, (long long)block_size);
@@ -875,6 +880,10 @@ inline int fill_fuse_args(FuseArgs& f, const int64_t* row_index, void* const* em
   f.rb.n_blocks = n_blocks;
   f.rb.block_size = block_size;
   f.rb.D = static_cast<int>(D);
+  // block bases and the pitch are required to be aligned like the row width allows
+  f.rb.pitch = pitch_elements(row_pitch_bytes, D, dtype_size(row_dtype), pick_vec_bytes(D * dtype_size(row_dtype), 16));
+  RECIS_REQUIRE(f.rb.pitch >= D, "row pitch of %lld bytes does not fit rows of %lld elements", (long long)row_pitch_bytes,
+                (long long)D);
   return RECIS_OK;
 }
 

@@ -15,13 +15,13 @@ int recis_csr_gather_reduce2_adagrad(const recis_csr_input* a, const recis_csr_i
                                      const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
                                      int64_t D, const int64_t* row_index, void* const* emb_blocks_dev,
                                      void* const* accum_blocks_dev, int64_t n_blocks, int64_t block_size,
-                                     int row_dtype, double lr, double eps, void* stream_) {
+                                     int64_t row_pitch_bytes, int row_dtype, double lr, double eps, void* stream_) {
   RECIS_REQUIRE(a && b, "both inputs must be given");
   RECIS_REQUIRE(a->n_parts == 0, "only the second input may come in parts");
   if (U == 0) return RECIS_OK;
   FuseArgs f;
-  if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, accum_blocks_dev, nullptr, false, n_blocks, block_size, D,
-                              row_dtype))
+  if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, accum_blocks_dev, nullptr, false, n_blocks, block_size,
+                              row_pitch_bytes, D, row_dtype))
     return rc;
   f.lr = static_cast<float>(lr);
   f.eps = static_cast<float>(eps);

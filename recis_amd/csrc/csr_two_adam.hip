@@ -15,16 +15,16 @@ int recis_csr_gather_reduce2_adamw(const recis_csr_input* a, const recis_csr_inp
                                    const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, int64_t U,
                                    int64_t D, const int64_t* row_index, void* const* emb_blocks_dev,
                                    void* const* exp_avg_blocks_dev, void* const* exp_avg_sq_blocks_dev,
-                                   int64_t n_blocks, int64_t block_size, int row_dtype, void* beta1_t, void* beta2_t,
-                                   int beta_is_f64, double lr, double beta1, double beta2, double weight_decay,
-                                   double eps, void* stream_) {
+                                   int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes, int row_dtype,
+                                   void* beta1_t, void* beta2_t, int beta_is_f64, double lr, double beta1, double beta2,
+                                   double weight_decay, double eps, void* stream_) {
   RECIS_REQUIRE(a && b, "both inputs must be given");
   RECIS_REQUIRE(a->n_parts == 0, "only the second input may come in parts");
   RECIS_REQUIRE(beta1_t != nullptr && beta2_t != nullptr, "beta1_t / beta2_t must not be NULL");
   FuseArgs f{};
   if (U > 0) {
     if (int rc = fill_fuse_args(f, row_index, emb_blocks_dev, exp_avg_blocks_dev, exp_avg_sq_blocks_dev, true, n_blocks,
-                                block_size, D, row_dtype))
+                                block_size, row_pitch_bytes, D, row_dtype))
       return rc;
   }
   CsrInput second;

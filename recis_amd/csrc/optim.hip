@@ -27,13 +27,14 @@ struct OptArgs {
   int64_t n;
   int64_t n_blocks;
   int64_t block_size;
+  int64_t pitch;
   int D;
   int lpr_log2;
   int* err;
 };
 
 __device__ __forceinline__ bool row_offset(const OptArgs& a, int64_t idx, int64_t& b, int64_t& off) {
-  const RowBlocks r{a.n_blocks, a.block_size, a.D};
+  const RowBlocks r{a.n_blocks, a.block_size, a.D, a.pitch};
   return block_row(r, idx, b, off);
 }
 
@@ -65,9 +66,9 @@ adamw_rows_kernel(OptArgs a, const TG* __restrict__ grad, T* const* __restrict__
   }
   const double alpha = alpha_ptr[0];
   const AdamCoef coef{alpha_ptr, beta1, beta2, decay, eps};
-  T* w_row = emb_blocks[b] + off * a.D;
-  T* m_row = m_blocks[b] + off * a.D;
-  T* v_row = v_blocks[b] + off * a.D;
+  T* w_row = emb_blocks[b] + off * a.pitch;
+  T* m_row = m_blocks[b] + off * a.pitch;
+  T* v_row = v_blocks[b] + off * a.pitch;
   const TG* g_row = grad + i * a.D;
   for (int c0 = cl * VEC; c0 < a.D; c0 += VEC << a.lpr_log2) {
     float g[VEC];
@@ -89,8 +90,8 @@ adagrad_rows_kernel(OptArgs a, const TG* __restrict__ grad, T* const* __restrict
     raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
     return;
   }
-  T* w_row = emb_blocks[b] + off * a.D;
-  T* s_row = acc_blocks[b] + off * a.D;
+  T* w_row = emb_blocks[b] + off * a.pitch;
+  T* s_row = acc_blocks[b] + off * a.pitch;
   const TG* g_row = grad + i * a.D;
   for (int c0 = cl * VEC; c0 < a.D; c0 += VEC << a.lpr_log2) {
     float g[VEC];
@@ -121,7 +122,7 @@ int dispatch_vec4(int vec, F&& f) {
 }
 
 int fill_opt_args(OptArgs& a, const int64_t* index, const void* grad, int64_t n, int64_t n_blocks,
-                  int64_t block_size, int64_t D, int row_dtype, int grad_dtype, int& vec) {
+                  int64_t block_size, int64_t row_pitch_bytes, int64_t D, int row_dtype, int grad_dtype, int& vec) {
   RECIS_REQUIRE(n >= 0 && n_blocks >= 1 && block_size >= 1, "bad sizes (n=%lld n_blocks=%lld block_size=%lld)",
                 (long long)n, (long long)n_blocks, (long long)block_size);
   RECIS_REQUIRE(D >= 1 && D <= (1 << 20), "embedding dim %lld out of range", (long long)D);
@@ -136,6 +137,9 @@ int fill_opt_args(OptArgs& a, const int64_t* index, const void* grad, int64_t n,
   a.n = n;
   a.n_blocks = n_blocks;
   a.block_size = block_size;
+  a.pitch = pitch_elements(row_pitch_bytes, D, rsz, vb_row);
+  RECIS_REQUIRE(a.pitch >= D, "row pitch of %lld bytes does not fit rows of %lld elements", (long long)row_pitch_bytes,
+                (long long)D);
   a.D = static_cast<int>(D);
   a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
   a.err = device_error_word(current_device());
@@ -166,7 +170,7 @@ extern "C" {
 int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dtype,
                             void* const* emb_blocks_dev, void* const* exp_avg_blocks_dev,
                             void* const* exp_avg_sq_blocks_dev, int64_t n_blocks, int64_t block_size,
-                            int row_dtype, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
+                            int64_t row_pitch_bytes, int row_dtype, void* beta1_t, void* beta2_t, int beta_is_f64, double lr,
                             double beta1, double beta2, double weight_decay, double eps, int64_t n,
                             int64_t D, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -180,7 +184,7 @@ int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dty
   RECIS_REQUIRE(emb_blocks_dev && exp_avg_blocks_dev && exp_avg_sq_blocks_dev, "block tables must not be NULL");
   OptArgs a;
   int vec = 1;
-  if (int rc = fill_opt_args(a, index, grad, n, n_blocks, block_size, D, row_dtype, grad_dtype, vec)) return rc;
+  if (int rc = fill_opt_args(a, index, grad, n, n_blocks, block_size, row_pitch_bytes, D, row_dtype, grad_dtype, vec)) return rc;
   const int rows_per_block = kBlock >> a.lpr_log2;
   const int64_t grid = (n + rows_per_block - 1) / rows_per_block;
   return dispatch_row_types(row_dtype, grad_dtype, [&](auto t, auto tg) {
@@ -205,14 +209,15 @@ int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dty
 
 int recis_block_apply_adagrad(const int64_t* index, const void* grad, int grad_dtype,
                               void* const* emb_blocks_dev, void* const* accum_blocks_dev,
-                              int64_t n_blocks, int64_t block_size, int row_dtype, double lr, double eps,
+                              int64_t n_blocks, int64_t block_size, int64_t row_pitch_bytes, int row_dtype, double lr,
+                              double eps,
                               int64_t n, int64_t D, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (n == 0) return RECIS_OK;
   RECIS_REQUIRE(emb_blocks_dev && accum_blocks_dev, "block tables must not be NULL");
   OptArgs a;
   int vec = 1;
-  if (int rc = fill_opt_args(a, index, grad, n, n_blocks, block_size, D, row_dtype, grad_dtype, vec)) return rc;
+  if (int rc = fill_opt_args(a, index, grad, n, n_blocks, block_size, row_pitch_bytes, D, row_dtype, grad_dtype, vec)) return rc;
   const int rows_per_block = kBlock >> a.lpr_log2;
   const int64_t grid = (n + rows_per_block - 1) / rows_per_block;
   return dispatch_row_types(row_dtype, grad_dtype, [&](auto t, auto tg) {

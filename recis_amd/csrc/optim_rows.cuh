@@ -10,6 +10,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "common.cuh"
 
 namespace recis_hip {
@@ -19,7 +21,16 @@ struct RowBlocks {
   int64_t n_blocks;
   int64_t block_size;
   int D;
+  int64_t pitch;  // elements from one row of a block to the next (D when rows lie back to back)
 };
+
+// The row pitch in elements of a row_pitch_bytes argument (0 = rows lie back to back); negative
+// when the pitch does not fit rows of D elements of elem_size bytes moved vec_bytes at a time.
+inline int64_t pitch_elements(int64_t row_pitch_bytes, int64_t D, int elem_size, int vec_bytes) {
+  if (row_pitch_bytes == 0) return D;
+  if (row_pitch_bytes < D * elem_size || row_pitch_bytes % elem_size || row_pitch_bytes % vec_bytes) return -1;
+  return row_pitch_bytes / elem_size;
+}
 
 // Block and row-in-block of table row idx; false when idx is negative or beyond the blocks.
 __device__ __forceinline__ bool block_row(const RowBlocks& r, int64_t idx, int64_t& b, int64_t& off) {
@@ -39,6 +50,19 @@ __device__ __forceinline__ bool block_row(const RowBlocks& r, int64_t idx, int64
     off = static_cast<uint32_t>(idx) - q * bs;
   }
   return b < r.n_blocks;
+}
+
+// Whether a row update should touch the table rows with the streaming (non-temporal) hint: yes
+// when the `slots` arrays it works on (parameter and state) are together larger than what the
+// caches keep from one step to the next (the 256 MB of memory-side cache; RECIS_STREAM_ROWS_MIN_MB
+// in the environment moves the line, 0 = always stream), no for a small table, whose rows the
+// next step would otherwise have to fetch from memory again.
+inline bool stream_table_rows(const RowBlocks& rb, size_t elem_size, int slots) {
+  static const int64_t min_bytes = [] {
+    const char* s = std::getenv("RECIS_STREAM_ROWS_MIN_MB");
+    return (s != nullptr && *s ? std::atoll(s) : 256) << 20;
+  }();
+  return rb.n_blocks * rb.block_size * rb.pitch * static_cast<int64_t>(elem_size) * (rb.pitch > rb.D ? 1 : slots) >= min_bytes;
 }
 
 struct AdamCoef {

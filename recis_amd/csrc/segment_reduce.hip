@@ -46,6 +46,7 @@ struct SegArgs {
   const int64_t* row_index;
   const void* const* blocks;
   int64_t block_rows, n_blocks;
+  int64_t pitch;  // elements from one row of a block to the next
 };
 
 // Address of unique row idx (idx < U checked by the caller) in the block list, nullptr = zero row.
@@ -62,7 +63,7 @@ __device__ __forceinline__ const TIn* block_row(const SegArgs& a, int64_t idx) {
     raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
     return nullptr;
   }
-  return static_cast<const TIn*>(a.blocks[b]) + r * a.D;
+  return static_cast<const TIn*>(a.blocks[b]) + r * a.pitch;
 }
 
 // Stage offsets[s0 .. s0 + teams_per_block] into LDS and return this team's
@@ -974,6 +975,7 @@ struct BlockSource {
   const int64_t* row_index;
   const void* const* blocks;
   int64_t block_rows, n_blocks;
+  int64_t row_pitch_bytes;  // 0: rows lie back to back
 };
 
 static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_dtype, const void* weight,
@@ -1028,6 +1030,14 @@ static int forward_impl(const void* unique_emb, const BlockSource* blk, int emb_
   a.blocks = blk ? blk->blocks : nullptr;
   a.block_rows = blk ? blk->block_rows : 1;
   a.n_blocks = blk ? blk->n_blocks : 0;
+  a.pitch = D;
+  if (blk && blk->row_pitch_bytes) {
+    RECIS_REQUIRE(blk->row_pitch_bytes >= D * in_sz && blk->row_pitch_bytes % in_sz == 0 &&
+                      blk->row_pitch_bytes % vb_in == 0,
+                  "row pitch of %lld bytes does not fit rows of %lld elements", (long long)blk->row_pitch_bytes,
+                  (long long)D);
+    a.pitch = blk->row_pitch_bytes / in_sz;
+  }
 
   return dispatch_types(emb_dtype, out_dtype, [&](auto tin, auto tout) {
     using TIn = decltype(tin);
@@ -1127,14 +1137,14 @@ extern "C" int recis_segment_reduce_forward(
 }
 
 extern "C" int recis_segment_reduce_forward_blocks(
-    const void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows, const int64_t* row_index,
-    int emb_dtype, const void* weight, int weight_dtype, const void* reverse_indices, int rev_is64,
+    const void* const* emb_blocks_dev, int64_t n_blocks, int64_t block_rows, int64_t row_pitch_bytes,
+    const int64_t* row_index, int emb_dtype, const void* weight, int weight_dtype, const void* reverse_indices, int rev_is64,
     const void* offsets, int off_is64, void* out, int out_dtype, int64_t B, int64_t U, int64_t S,
     int64_t D, int mode, void* stream_) {
   RECIS_REQUIRE(mode != RECIS_MAX, "the MAX combiner takes dense rows (recis_segment_reduce_forward)");
   RECIS_REQUIRE(n_blocks >= 0 && block_rows > 0, "bad block list");
   RECIS_REQUIRE(U == 0 || (emb_blocks_dev != nullptr && row_index != nullptr), "NULL block list / row_index");
-  BlockSource blk{row_index, emb_blocks_dev, block_rows, n_blocks};
+  BlockSource blk{row_index, emb_blocks_dev, block_rows, n_blocks, row_pitch_bytes};
   return forward_impl(nullptr, &blk, emb_dtype, weight, weight_dtype, reverse_indices, rev_is64, offsets, off_is64,
                       out, out_dtype, nullptr, B, U, S, D, mode, stream_);
 }

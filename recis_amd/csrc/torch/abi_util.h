@@ -64,9 +64,27 @@ inline int64_t row_bytes(const at::Tensor& block) {
   return n;
 }
 
-// Checks a block list (one dtype, one row shape, contiguous, at least block_size rows each) and
-// returns its first block.
+// Every row of the block is contiguous and rows do not overlap; rows may lie a pitch apart (a slot
+// that shares its allocation with the optimizer state of the same keys).
+inline bool rows_dense(const at::Tensor& block) {
+  if (block.is_contiguous()) return true;
+  if (block.dim() < 1) return false;
+  int64_t row = 1;
+  for (int64_t d = block.dim() - 1; d >= 1; --d) {
+    if (block.size(d) != 1 && block.stride(d) != row) return false;
+    row *= block.size(d);
+  }
+  return block.stride(0) >= row;
+}
+
+// Checks a block list (one dtype, one row shape, contiguous rows at one pitch, at least block_size
+// rows each) and returns its first block.
 const at::Tensor& check_blocks(const std::vector<at::Tensor>& blocks, int64_t block_size);
+
+// The row_pitch_bytes argument of the C header for a block: 0 when its rows lie back to back.
+int64_t row_pitch_bytes(const at::Tensor& block);
+// The same for slots that go into one call (their first blocks): they must agree.
+int64_t shared_row_pitch_bytes(std::initializer_list<const at::Tensor*> first_blocks);
 
 // Device array holding the base pointer of every block, as the row kernels take it. Cached on the
 // pointer values, so a slot that does not grow pays the host-to-device copy once, not per launch

@@ -21,12 +21,24 @@ const at::Tensor& check_blocks(const std::vector<at::Tensor>& blocks, int64_t bl
   for (const auto& b : blocks) {
     require_gpu(b, "blocks");
     TORCH_CHECK(b.scalar_type() == b0.scalar_type() && b.sizes().slice(1) == b0.sizes().slice(1) &&
-                    b.is_contiguous() && b.device() == b0.device(),
-                "blocks must be contiguous and share dtype, device and row shape");
+                    rows_dense(b) && b.stride(0) == b0.stride(0) && b.device() == b0.device(),
+                "blocks must hold contiguous rows at one pitch and share dtype, device and row shape");
     TORCH_CHECK(b.size(0) >= block_size, "block with ", b.size(0), " rows is smaller than block_size ",
                 block_size);
   }
   return b0;
+}
+
+int64_t row_pitch_bytes(const at::Tensor& block) {
+  return block.is_contiguous() ? 0 : block.stride(0) * static_cast<int64_t>(block.element_size());
+}
+
+int64_t shared_row_pitch_bytes(std::initializer_list<const at::Tensor*> first_blocks) {
+  const at::Tensor& b0 = **first_blocks.begin();
+  for (const at::Tensor* b : first_blocks)
+    TORCH_CHECK(b->stride(0) == b0.stride(0) && b->scalar_type() == b0.scalar_type(),
+                "slots that are updated together must share dtype and row pitch");
+  return row_pitch_bytes(b0);
 }
 
 at::Tensor block_ptr_table(const std::vector<at::Tensor>& blocks) {
@@ -247,7 +259,8 @@ Tensor block_gather(const Tensor ids, TensorList emb_blocks, int64_t block_size,
   Tensor out = at::empty(shape, b0.options());
   Tensor tab = block_ptr_table(emb_blocks);
   check(recis_block_gather(i.data_ptr<int64_t>(), static_cast<void* const*>(tab.data_ptr()),
-                           static_cast<int64_t>(emb_blocks.size()), block_size, default_key, readonly ? 1 : 0,
+                           static_cast<int64_t>(emb_blocks.size()), block_size, row_pitch_bytes(b0), default_key,
+                           readonly ? 1 : 0,
                            out.data_ptr(), i.numel(), row_bytes(b0), stream_of(b0.device())));
   return out;
 }
@@ -275,7 +288,7 @@ void block_insert_impl(const Tensor& ids, const Tensor& embedding, const Tensor*
   check(recis_block_insert(i.data_ptr<int64_t>(), e.data_ptr(), broadcast,
                            m.defined() ? static_cast<const uint8_t*>(m.data_ptr()) : nullptr,
                            static_cast<void* const*>(tab.data_ptr()), static_cast<int64_t>(emb_blocks.size()),
-                           block_size, i.numel(), row_bytes(b0), stream_of(b0.device())));
+                           block_size, row_pitch_bytes(b0), i.numel(), row_bytes(b0), stream_of(b0.device())));
 }
 }  // namespace
 
@@ -329,7 +342,8 @@ void block_apply_adamw(const Tensor index, const Tensor grad, TensorList emb_blo
   check(recis_block_apply_adamw(i.data_ptr<int64_t>(), g.data_ptr(), dtype_code(g.scalar_type()),
                                 static_cast<void* const*>(t0.data_ptr()), static_cast<void* const*>(t1.data_ptr()),
                                 static_cast<void* const*>(t2.data_ptr()), static_cast<int64_t>(emb_blocks.size()),
-                                block_size, dtype_code(b0.scalar_type()), beta1_t.data_ptr(), beta2_t.data_ptr(),
+                                block_size, shared_row_pitch_bytes({&b0, &exp_avg[0], &exp_avg_sq[0]}),
+                                dtype_code(b0.scalar_type()), beta1_t.data_ptr(), beta2_t.data_ptr(),
                                 beta1_t.scalar_type() == at::kDouble ? 1 : 0, lr, beta1, beta2, weight_decay, eps,
                                 i.numel(), D, stream_of(b0.device())));
 }
@@ -348,8 +362,9 @@ void block_apply_adagrad(const Tensor index, const Tensor grad, TensorList emb_b
   Tensor t0 = block_ptr_table(emb_blocks), t1 = block_ptr_table(accum);
   check(recis_block_apply_adagrad(i.data_ptr<int64_t>(), g.data_ptr(), dtype_code(g.scalar_type()),
                                   static_cast<void* const*>(t0.data_ptr()), static_cast<void* const*>(t1.data_ptr()),
-                                  static_cast<int64_t>(emb_blocks.size()), block_size, dtype_code(b0.scalar_type()),
-                                  lr, eps, i.numel(), D, stream_of(b0.device())));
+                                  static_cast<int64_t>(emb_blocks.size()), block_size,
+                                  shared_row_pitch_bytes({&b0, &accum[0]}), dtype_code(b0.scalar_type()), lr, eps,
+                                  i.numel(), D, stream_of(b0.device())));
 }
 
 // ------------------------------------------------------------------------------------ allocator ops

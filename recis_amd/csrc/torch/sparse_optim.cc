@@ -139,15 +139,6 @@ template <AdamDecay kDecay>
 void SparseAdamFamily<kDecay>::InitParamState(const std::string& name, const HashTablePtr& table) {
   (void)name;
   auto sg = table->RawSlotGroup();
-  auto emb = sg->EmbSlot();
-  auto blocks = emb->Chunks();
-  std::vector<int64_t> partial{1};
-  if (!blocks.empty()) {
-    auto s = blocks[0].sizes();
-    partial.insert(partial.end(), s.begin() + 1, s.end());
-  } else {
-    partial.push_back(emb->FlatSize());
-  }
   AdamState st;
   // SparseAdam keeps its running beta powers in float64 (csrc/embedding/adam.h:37), the other two in
   // float32 scalars
@@ -157,8 +148,10 @@ void SparseAdamFamily<kDecay>::InitParamState(const std::string& name, const Has
   st.beta1 = at::ones(beta_shape, beta_opt);
   st.beta2 = at::ones(beta_shape, beta_opt);
   st.step = at::zeros({1}, at::TensorOptions().device(table->device()).dtype(at::kLong));
-  st.exp_avg = sg->AppendSlot(std::string(Prefix()) + "exp_avg", emb->Dtype(), partial, 0.0);
-  st.exp_avg_sq = sg->AppendSlot(std::string(Prefix()) + "exp_avg_sq", emb->Dtype(), partial, 0.0);
+  // the two moments live next to the parameter row they belong to
+  auto moments = sg->AppendPackedSlots({std::string(Prefix()) + "exp_avg", std::string(Prefix()) + "exp_avg_sq"}, 0.0);
+  st.exp_avg = moments[0];
+  st.exp_avg_sq = moments[1];
   state_[table.get()] = st;
 }
 
@@ -198,6 +191,7 @@ void SparseAdamFamily<kDecay>::UpdatePlanned(const HashTablePtr& table, const st
   auto tab = [](const at::Tensor& t) { return reinterpret_cast<void* const*>(t.data_ptr()); };
   const int64_t n_blocks = static_cast<int64_t>(chunks.size());
   const int beta_f64 = st.beta1.scalar_type() == at::kDouble ? 1 : 0;
+  const int64_t pitch = shared_row_pitch_bytes({&chunks[0], &st.exp_avg->Chunks()[0], &st.exp_avg_sq->Chunks()[0]});
   const BatchPlan& plan = *planned[0].plan;
   void* stream = stream_of(table->device());
   if (planned.size() == 1) {
@@ -209,7 +203,7 @@ void SparseAdamFamily<kDecay>::UpdatePlanned(const HashTablePtr& table, const st
         plan.row_start().data_ptr<int32_t>(), plan.hot_items().data_ptr<int32_t>(), plan.hot_cap(),
         plan.counts().data_ptr<int64_t>(), h.U, h.D, g.cover.defined() ? g.cover.data_ptr() : nullptr,
         g.cover.defined() ? index_kind(g.cover, "offsets") : 0, g.cover.defined() ? g.cover.numel() - 1 : 0,
-        h.index.data_ptr<int64_t>(), tab(t_emb), tab(t_m), tab(t_v), n_blocks, emb->ChunkRows(),
+        h.index.data_ptr<int64_t>(), tab(t_emb), tab(t_m), tab(t_v), n_blocks, emb->ChunkRows(), pitch,
         dtype_code(emb->Dtype()), st.beta1.data_ptr(), st.beta2.data_ptr(), beta_f64, lr_, beta1_, beta2_, Decay(), eps_,
         stream));
     return;
@@ -223,8 +217,8 @@ void SparseAdamFamily<kDecay>::UpdatePlanned(const HashTablePtr& table, const st
   check(recis_csr_gather_reduce2_adamw(
       &a.in, &b.in, plan.row_start().data_ptr<int32_t>(), plan.hot_items().data_ptr<int32_t>(), plan.hot_cap(),
       plan.counts().data_ptr<int64_t>(), U, D, planned[0].index.data_ptr<int64_t>(), tab(t_emb), tab(t_m), tab(t_v),
-      n_blocks, emb->ChunkRows(), dtype_code(emb->Dtype()), st.beta1.data_ptr(), st.beta2.data_ptr(), beta_f64, lr_,
-      beta1_, beta2_, Decay(), eps_, stream));
+      n_blocks, emb->ChunkRows(), pitch, dtype_code(emb->Dtype()), st.beta1.data_ptr(), st.beta2.data_ptr(), beta_f64,
+      lr_, beta1_, beta2_, Decay(), eps_, stream));
 }
 
 template <AdamDecay kDecay>
@@ -257,16 +251,7 @@ c10::intrusive_ptr<SparseAdagrad> SparseAdagrad::Make(const c10::Dict<std::strin
 void SparseAdagrad::InitParamState(const std::string& name, const HashTablePtr& table) {
   (void)name;
   auto sg = table->RawSlotGroup();
-  auto emb = sg->EmbSlot();
-  std::vector<int64_t> partial{1};
-  auto blocks = emb->Chunks();
-  if (!blocks.empty()) {
-    auto s = blocks[0].sizes();
-    partial.insert(partial.end(), s.begin() + 1, s.end());
-  } else {
-    partial.push_back(emb->FlatSize());
-  }
-  accum_[table.get()] = sg->AppendSlot("sparse_adagrad_accum", emb->Dtype(), partial, 0.0);
+  accum_[table.get()] = sg->AppendPackedSlots({"sparse_adagrad_accum"}, 0.0)[0];
 }
 
 void SparseAdagrad::Update(const HashTablePtr& table, const at::Tensor& index, const at::Tensor& grad) {
@@ -285,6 +270,7 @@ void SparseAdagrad::UpdatePlanned(const HashTablePtr& table, const std::vector<P
   at::Tensor t_emb = block_ptr_table(chunks), t_acc = block_ptr_table(accum->Chunks());
   auto tab = [](const at::Tensor& t) { return reinterpret_cast<void* const*>(t.data_ptr()); };
   const int64_t n_blocks = static_cast<int64_t>(chunks.size());
+  const int64_t pitch = shared_row_pitch_bytes({&chunks[0], &accum->Chunks()[0]});
   const BatchPlan& plan = *planned[0].plan;
   void* stream = stream_of(table->device());
   if (planned.size() == 1) {
@@ -296,8 +282,8 @@ void SparseAdagrad::UpdatePlanned(const HashTablePtr& table, const std::vector<P
         plan.row_start().data_ptr<int32_t>(), plan.hot_items().data_ptr<int32_t>(), plan.hot_cap(),
         plan.counts().data_ptr<int64_t>(), h.U, h.D, g.cover.defined() ? g.cover.data_ptr() : nullptr,
         g.cover.defined() ? index_kind(g.cover, "offsets") : 0, g.cover.defined() ? g.cover.numel() - 1 : 0,
-        h.index.data_ptr<int64_t>(), tab(t_emb), tab(t_acc), n_blocks, emb->ChunkRows(), dtype_code(emb->Dtype()), lr_,
-        eps_, stream));
+        h.index.data_ptr<int64_t>(), tab(t_emb), tab(t_acc), n_blocks, emb->ChunkRows(), pitch, dtype_code(emb->Dtype()),
+        lr_, eps_, stream));
     return;
   }
   CsrInputHolder a, b;
@@ -309,8 +295,8 @@ void SparseAdagrad::UpdatePlanned(const HashTablePtr& table, const std::vector<P
   check(recis_csr_gather_reduce2_adagrad(&a.in, &b.in, plan.row_start().data_ptr<int32_t>(),
                                          plan.hot_items().data_ptr<int32_t>(), plan.hot_cap(),
                                          plan.counts().data_ptr<int64_t>(), U, D, planned[0].index.data_ptr<int64_t>(),
-                                         tab(t_emb), tab(t_acc), n_blocks, emb->ChunkRows(), dtype_code(emb->Dtype()),
-                                         lr_, eps_, stream));
+                                         tab(t_emb), tab(t_acc), n_blocks, emb->ChunkRows(), pitch,
+                                         dtype_code(emb->Dtype()), lr_, eps_, stream));
 }
 
 std::tuple<c10::Dict<std::string, HashTablePtr>, c10::Dict<std::string, at::Tensor>> SparseAdagrad::state_dict() {

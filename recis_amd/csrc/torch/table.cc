@@ -3,6 +3,7 @@
 #include <ATen/record_function.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <set>
 
 #include "abi_util.h"
@@ -318,12 +319,25 @@ void Slot::SetChunkRows(int64_t chunk_rows) {
   chunk_rows_ = chunk_rows;
 }
 
-void Slot::EnsureChunks(int64_t n_chunks) {
+at::Tensor Slot::NewChunkValues() {
   std::vector<int64_t> shape{chunk_rows_}, fan{block_size_};
   shape.insert(shape.end(), row_shape_.begin(), row_shape_.end());
   fan.insert(fan.end(), row_shape_.begin(), row_shape_.end());
   // one tensor for several blocks; fan-dependent initialisers still see one [block_size, D] block
-  while (static_cast<int64_t>(chunks_.size()) < n_chunks) chunks_.push_back(generator_->Generate(shape, fan));
+  return generator_->Generate(shape, fan);
+}
+
+void Slot::EnsureChunks(int64_t n_chunks) {
+  TORCH_CHECK(!packed_, "slot ", name_, " does not own its storage");
+  while (static_cast<int64_t>(chunks_.size()) < n_chunks) chunks_.push_back(NewChunkValues());
+}
+
+void Slot::SetChunk(int64_t c, at::Tensor view) {
+  TORCH_CHECK(c >= 0 && c <= static_cast<int64_t>(chunks_.size()), "chunk ", c, " out of order");
+  if (c == static_cast<int64_t>(chunks_.size()))
+    chunks_.push_back(std::move(view));
+  else
+    chunks_[c] = std::move(view);
 }
 
 void Slot::Clear() { chunks_.clear(); }
@@ -354,6 +368,82 @@ void SlotGroup::AppendEmbSlot(at::ScalarType dtype, const std::vector<int64_t>& 
                               GeneratorPtr generator) {
   AppendSlot(EmbSlotName(), dtype, partial_shape, std::move(generator));
   emb_slot_index_ = static_cast<int64_t>(slots_.size()) - 1;
+}
+
+at::Tensor SlotGroup::PackedView(const at::Tensor& store, int64_t member, int64_t members,
+                                 const SlotPtr& slot) const {
+  (void)members;
+  std::vector<int64_t> shape{chunk_rows_};
+  const auto row = slot->RowShape();
+  shape.insert(shape.end(), row.begin(), row.end());
+  return store.narrow(1, member * slot->FlatSize(), slot->FlatSize()).view(shape);
+}
+
+void SlotGroup::AddPackedChunk() {
+  const int64_t members = static_cast<int64_t>(packed_.size());
+  const SlotPtr& emb = slots_[packed_[0]];
+  at::Tensor store = at::empty({chunk_rows_, members * emb->FlatSize()},
+                               at::TensorOptions().dtype(emb->Dtype()).device(device_));
+  const int64_t c = static_cast<int64_t>(packed_chunks_.size());
+  for (int64_t g = 0; g < members; ++g) {
+    const SlotPtr& slot = slots_[packed_[g]];
+    at::Tensor view = PackedView(store, g, members, slot);
+    view.copy_(slot->NewChunkValues());
+    slot->SetChunk(c, view);
+  }
+  packed_chunks_.push_back(store);
+}
+
+std::vector<SlotPtr> SlotGroup::AppendPackedSlots(const std::vector<std::string>& names, double init_val) {
+  TORCH_CHECK(emb_slot_index_ >= 0, "the table has no embedding slot yet");
+  SlotPtr emb = slots_[emb_slot_index_];
+  std::vector<int64_t> partial{1};
+  const auto row = emb->RowShape();
+  partial.insert(partial.end(), row.begin(), row.end());
+  const char* knob = std::getenv("RECIS_PACKED_STATE");
+  std::vector<SlotPtr> added;
+  if (knob == nullptr || std::string(knob) != "1") {
+    for (const auto& name : names) added.push_back(AppendSlot(name, emb->Dtype(), partial, init_val));
+    return added;
+  }
+  for (const auto& name : names)
+    TORCH_CHECK(name_to_index_.find(name) == name_to_index_.end(), "slot ", name, " already exists");
+  const size_t had = packed_.size();
+  if (packed_.empty()) {
+    packed_.push_back(emb_slot_index_);
+    emb->SetPacked();
+  }
+  std::vector<int64_t> shape{block_size_};
+  shape.insert(shape.end(), row.begin(), row.end());
+  for (const auto& name : names) {
+    auto slot = c10::make_intrusive<Slot>(name, block_size_, emb->Dtype(), partial,
+                                          MakeConstantGenerator(shape, emb->Dtype(), init_val), device_, chunk_rows_,
+                                          map_);
+    slot->SetPacked();
+    name_to_index_[name] = static_cast<int64_t>(slots_.size());
+    packed_.push_back(static_cast<int64_t>(slots_.size()));
+    slots_.push_back(slot);
+    added.push_back(slot);
+  }
+  // storage that exists moves into the wider layout, one chunk at a time (the old chunk is let go
+  // as soon as its rows are copied)
+  const int64_t members = static_cast<int64_t>(packed_.size());
+  std::vector<at::Tensor> stores;
+  for (int64_t c = 0; c < n_chunks_; ++c) {
+    at::Tensor store = at::empty({chunk_rows_, members * emb->FlatSize()},
+                                 at::TensorOptions().dtype(emb->Dtype()).device(device_));
+    for (int64_t g = 0; g < members; ++g) {
+      const SlotPtr& slot = slots_[packed_[g]];
+      at::Tensor view = PackedView(store, g, members, slot);
+      const bool old = g < static_cast<int64_t>(std::max<size_t>(had, 1));
+      view.copy_(old ? slot->Chunks()[c] : slot->NewChunkValues());
+      slot->SetChunk(c, view);
+    }
+    if (c < static_cast<int64_t>(packed_chunks_.size())) packed_chunks_[c] = at::Tensor();
+    stores.push_back(store);
+  }
+  packed_chunks_ = std::move(stores);
+  return added;
 }
 
 void SlotGroup::AppendStepFilterSlot(const std::string& name, int64_t init_step) {
@@ -392,12 +482,15 @@ void SlotGroup::EnsureRows(int64_t rows) {
   const int64_t need = (rows + chunk_rows_ - 1) / chunk_rows_;
   if (need > n_chunks_) {
     n_chunks_ = need;
-    for (auto& s : slots_) s->EnsureChunks(need);
+    while (!packed_.empty() && static_cast<int64_t>(packed_chunks_.size()) < need) AddPackedChunk();
+    for (auto& s : slots_)
+      if (!s->Packed()) s->EnsureChunks(need);
   }
 }
 
 void SlotGroup::Clear() {
   for (auto& s : slots_) s->Clear();
+  packed_chunks_.clear();
   n_chunks_ = 0;
 }
 
@@ -716,7 +809,7 @@ at::Tensor Hashtable::ExpandRows(const BatchPlanPtr& plan, const at::Tensor& row
   const int code = dtype_code(dtype_);
   check(recis_csr_expand_rows_stamped(
       nullptr, reinterpret_cast<void* const*>(table.data_ptr()), static_cast<int64_t>(chunks.size()), emb->ChunkRows(),
-      row_index.data_ptr<int64_t>(), code, w.defined() ? w.data_ptr() : nullptr,
+      recis::hipabi::row_pitch_bytes(chunks[0]), row_index.data_ptr<int64_t>(), code, w.defined() ? w.data_ptr() : nullptr,
       w.defined() ? dtype_code(w.scalar_type()) : 0, plan->row_start().data_ptr<int32_t>(),
       plan->occ().data_ptr<int32_t>(), plan->hot_items().data_ptr<int32_t>(), plan->hot_cap(),
       plan->counts().data_ptr<int64_t>(), out.data_ptr(), code, plan->U_bound(), n, D,

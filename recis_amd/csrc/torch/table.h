@@ -128,8 +128,14 @@ class Slot : public torch::CustomClassHolder {
   const std::vector<at::Tensor>& Chunks() const { return chunks_; }
   int64_t ChunkRows() const { return chunk_rows_; }
   void SetChunkRows(int64_t chunk_rows);  // only while no storage exists
-  void EnsureChunks(int64_t n_chunks);
+  void EnsureChunks(int64_t n_chunks);    // (a slot that owns its storage)
   void Clear();
+  // A slot whose rows live in an allocation it shares with other slots of the table (see
+  // SlotGroup::AppendPackedSlots): the group hands it one strided [chunk_rows, D] view per chunk.
+  bool Packed() const { return packed_; }
+  void SetPacked() { packed_ = true; }
+  at::Tensor NewChunkValues();  // initial values of one chunk, from the slot's generator
+  void SetChunk(int64_t c, at::Tensor view);  // replaces chunk c, or appends it when c == Chunks().size()
 
  private:
   // block_num = (id_num + block_size) / block_size (csrc/embedding/hashtable.cc:255-261), read from
@@ -147,6 +153,7 @@ class Slot : public torch::CustomClassHolder {
   int64_t flat_size_;
   std::shared_ptr<IdMapHolder> map_;
   std::vector<at::Tensor> chunks_;
+  bool packed_ = false;
 };
 
 using SlotPtr = c10::intrusive_ptr<Slot>;
@@ -161,6 +168,19 @@ class SlotGroup : public torch::CustomClassHolder {
   SlotPtr AppendSlot(const std::string& name, at::ScalarType dtype, const std::vector<int64_t>& partial_shape,
                      double init_val = 0.0);
   void AppendEmbSlot(at::ScalarType dtype, const std::vector<int64_t>& partial_shape, GeneratorPtr generator);
+  // Appends constant-initialised slots of the embedding's dtype and row shape (an optimizer's
+  // state). With RECIS_PACKED_STATE=1 in the environment they share one allocation with the
+  // embedding slot: row r of a chunk holds emb | state 0 | state 1 ... back to back, so the rows one
+  // key's update touches lie in the same cache lines and DRAM page. Every slot still answers
+  // values() / index_select / index_insert as before; its blocks are strided views. Storage that
+  // exists is moved into the new layout chunk by chunk: views handed out earlier keep the old memory
+  // and no longer alias the table.
+  // The default is the reference's layout, one array per slot (csrc/embedding/slot_group.cc:40-75),
+  // because that measured no slower: the fused update is bound by the loads each wave keeps in
+  // flight, not by the lines it touches (D = 16 fp32, 2e8-row table: update 106 vs 112 us, but the
+  // forward expansion 91 vs 85 us, its 64-byte rows no longer sharing 128-byte lines with their
+  // neighbours; densely touched tables fetch 6 % more).
+  std::vector<SlotPtr> AppendPackedSlots(const std::vector<std::string>& names, double init_val);
   void AppendStepFilterSlot(const std::string& name, int64_t init_step);
   SlotPtr GetSlotByName(const std::string& name);
   SlotPtr GetSlotByIndex(int64_t index);
@@ -185,6 +205,12 @@ class SlotGroup : public torch::CustomClassHolder {
   int64_t n_chunks_ = 0;
   std::unordered_map<std::string, int64_t> name_to_index_;
   std::vector<SlotPtr> slots_;
+  // the slots that share an allocation (the embedding slot first) and that allocation's chunks,
+  // [chunk_rows, packed_.size() * D] each
+  at::Tensor PackedView(const at::Tensor& store, int64_t member, int64_t members, const SlotPtr& slot) const;
+  void AddPackedChunk();
+  std::vector<int64_t> packed_;
+  std::vector<at::Tensor> packed_chunks_;
 };
 
 }  // namespace embedding

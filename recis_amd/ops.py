@@ -90,8 +90,8 @@ def segment_reduce_forward_blocks(emb_blocks, block_size, row_index, weight, rev
     out = torch.empty((B if mode == "tile" else S, D), dtype=out_dtype, device=b0.device)
     tab = block_ptr_table(emb_blocks)
     check(lib().recis_segment_reduce_forward_blocks(
-        ptr(tab), i64(len(emb_blocks)), i64(block_size), ptr(row_index), dtype_code(b0.dtype),
-        ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
+        ptr(tab), i64(len(emb_blocks)), i64(block_size), i64(_pitch_bytes(emb_blocks)), ptr(row_index),
+        dtype_code(b0.dtype), ptr(weight), dtype_code(weight.dtype) if weight is not None else 0,
         _rev_ptr(reverse_indices, offsets),
         _index_kind(reverse_indices, "reverse_indices") if reverse_indices is not None else 1,
         ptr(offsets), _index_kind(offsets, "offsets"), ptr(out), dtype_code(out_dtype),
@@ -165,11 +165,29 @@ def _check_blocks(blocks, block_size):
     b0 = blocks[0]
     for b in blocks:
         require_cuda(b)
-        if b.dtype != b0.dtype or b.shape[1:] != b0.shape[1:] or not b.is_contiguous():
-            raise ValueError("blocks must be contiguous and share dtype and row shape")
+        if b.dtype != b0.dtype or b.shape[1:] != b0.shape[1:] or not _rows_dense(b) or b.stride(0) != b0.stride(0):
+            raise ValueError("blocks must hold contiguous rows at one pitch and share dtype and row shape")
         if b.shape[0] < block_size:
             raise ValueError("block with %d rows is smaller than block_size %d" % (b.shape[0], block_size))
     return b0
+
+
+def _rows_dense(block):
+    """Every row of ``block`` is contiguous and rows do not overlap (rows may lie a pitch apart: a slot
+    that shares its allocation with the optimizer state of the same keys)."""
+    if block.is_contiguous():
+        return True
+    return block.dim() >= 1 and block[0].is_contiguous() and block.stride(0) >= block[0].numel()
+
+
+def _pitch_bytes(*block_lists):
+    """``row_pitch_bytes`` of the C header for block lists that go into one call: 0 when rows lie back to
+    back, else the distance between rows, which all the lists must share."""
+    b0 = block_lists[0][0]
+    for blocks in block_lists:
+        if blocks[0].stride(0) != b0.stride(0) or blocks[0].dtype != b0.dtype:
+            raise ValueError("slots that are updated together must share dtype and row pitch")
+    return 0 if b0.is_contiguous() else b0.stride(0) * b0.element_size()
 
 
 def _row_bytes(block):
@@ -207,7 +225,7 @@ def block_gather(ids, emb_blocks, block_size, default_key=-1, readonly=False):
     out = torch.empty((ids.numel(),) + tuple(b0.shape[1:]), dtype=b0.dtype, device=b0.device)
     tab = block_ptr_table(emb_blocks)
     check(lib().recis_block_gather(ptr(ids), ptr(tab), i64(len(emb_blocks)), i64(block_size),
-                                   i64(default_key), int(bool(readonly)), ptr(out), i64(ids.numel()),
+                                   i64(_pitch_bytes(emb_blocks)), i64(default_key), int(bool(readonly)), ptr(out), i64(ids.numel()),
                                    i64(_row_bytes(b0)), stream_ptr(b0.device)))
     return out
 
@@ -230,8 +248,8 @@ def block_insert(ids, embedding, emb_blocks, block_size):
     broadcast = int(embedding.shape[0] == 1 and ids.numel() != 1)
     tab = block_ptr_table(emb_blocks)
     check(lib().recis_block_insert(ptr(ids), ptr(embedding), broadcast, ptr(None), ptr(tab),
-                                   i64(len(emb_blocks)), i64(block_size), i64(ids.numel()),
-                                   i64(_row_bytes(b0)), stream_ptr(b0.device)))
+                                   i64(len(emb_blocks)), i64(block_size), i64(_pitch_bytes(emb_blocks)),
+                                   i64(ids.numel()), i64(_row_bytes(b0)), stream_ptr(b0.device)))
 
 
 def block_insert_with_mask(ids, embedding, mask, emb_blocks, block_size):
@@ -247,8 +265,8 @@ def block_insert_with_mask(ids, embedding, mask, emb_blocks, block_size):
     mask = _contig(mask)
     tab = block_ptr_table(emb_blocks)
     check(lib().recis_block_insert(ptr(ids), ptr(embedding), 0, ptr(mask), ptr(tab),
-                                   i64(len(emb_blocks)), i64(block_size), i64(ids.numel()),
-                                   i64(_row_bytes(b0)), stream_ptr(b0.device)))
+                                   i64(len(emb_blocks)), i64(block_size), i64(_pitch_bytes(emb_blocks)),
+                                   i64(ids.numel()), i64(_row_bytes(b0)), stream_ptr(b0.device)))
 
 
 def block_filter(ids, emb_blocks, block_size, threshold):
@@ -290,8 +308,8 @@ def block_apply_adamw(index, grad, emb_blocks, beta1_t, beta2_t, step, exp_avg, 
     check(lib().recis_block_apply_adamw(
         ptr(index), ptr(grad), dtype_code(grad.dtype), ptr(block_ptr_table(emb_blocks)),
         ptr(block_ptr_table(exp_avg)), ptr(block_ptr_table(exp_avg_sq)), i64(len(emb_blocks)),
-        i64(block_size), dtype_code(b0.dtype), ptr(beta1_t), ptr(beta2_t),
-        int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1),
+        i64(block_size), i64(_pitch_bytes(emb_blocks, exp_avg, exp_avg_sq)), dtype_code(b0.dtype), ptr(beta1_t),
+        ptr(beta2_t), int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1),
         ctypes.c_double(beta2), ctypes.c_double(weight_decay), ctypes.c_double(eps),
         i64(index.numel()), i64(D), stream_ptr(b0.device)))
 
@@ -310,7 +328,8 @@ def block_apply_adagrad(index, grad, emb_blocks, accum_blocks, lr, eps, block_si
         raise ValueError("grad has %d elements, expected %d x %d" % (grad.numel(), index.numel(), D))
     check(lib().recis_block_apply_adagrad(
         ptr(index), ptr(grad), dtype_code(grad.dtype), ptr(block_ptr_table(emb_blocks)),
-        ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)), i64(block_size), dtype_code(b0.dtype),
+        ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)), i64(block_size),
+        i64(_pitch_bytes(emb_blocks, accum_blocks)), dtype_code(b0.dtype),
         ctypes.c_double(lr), ctypes.c_double(eps), i64(index.numel()), i64(D), stream_ptr(b0.device)))
 
 
@@ -863,7 +882,8 @@ def csr_gather_reduce_adamw(rows, plan, src, coef, row_index, emb_blocks, beta1_
         raise TypeError("beta1_t / beta2_t must both be float32 or float64")
     check(lib().recis_csr_gather_reduce_adamw(
         *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(exp_avg)), ptr(block_ptr_table(exp_avg_sq)),
-        i64(len(emb_blocks)), i64(block_size), dtype_code(b0.dtype), ptr(beta1_t), ptr(beta2_t),
+        i64(len(emb_blocks)), i64(block_size), i64(_pitch_bytes(emb_blocks, exp_avg, exp_avg_sq)), dtype_code(b0.dtype),
+        ptr(beta1_t), ptr(beta2_t),
         int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1), ctypes.c_double(beta2),
         ctypes.c_double(weight_decay), ctypes.c_double(eps), stream_ptr(rows.device)))
 
@@ -877,7 +897,8 @@ def csr_gather_reduce_adagrad(rows, plan, src, coef, row_index, emb_blocks, accu
         raise ValueError("state slot must have as many blocks as the embedding slot")
     check(lib().recis_csr_gather_reduce_adagrad(
         *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)),
-        i64(block_size), dtype_code(b0.dtype), ctypes.c_double(lr), ctypes.c_double(eps), stream_ptr(rows.device)))
+        i64(block_size), i64(_pitch_bytes(emb_blocks, accum_blocks)), dtype_code(b0.dtype), ctypes.c_double(lr),
+        ctypes.c_double(eps), stream_ptr(rows.device)))
 
 
 class _CsrInput(ctypes.Structure):
@@ -970,7 +991,8 @@ def csr_gather_reduce2_adamw(plan, first, second, row_index, emb_blocks, beta1_t
         raise TypeError("beta1_t / beta2_t must both be float32 or float64")
     check(lib().recis_csr_gather_reduce2_adamw(
         *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(exp_avg)), ptr(block_ptr_table(exp_avg_sq)),
-        i64(len(emb_blocks)), i64(block_size), dtype_code(b0.dtype), ptr(beta1_t), ptr(beta2_t),
+        i64(len(emb_blocks)), i64(block_size), i64(_pitch_bytes(emb_blocks, exp_avg, exp_avg_sq)), dtype_code(b0.dtype),
+        ptr(beta1_t), ptr(beta2_t),
         int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1), ctypes.c_double(beta2),
         ctypes.c_double(weight_decay), ctypes.c_double(eps), stream_ptr(dev)))
 
@@ -983,7 +1005,8 @@ def csr_gather_reduce2_adagrad(plan, first, second, row_index, emb_blocks, accum
         raise ValueError("state slot must have as many blocks as the embedding slot")
     check(lib().recis_csr_gather_reduce2_adagrad(
         *head, ptr(block_ptr_table(emb_blocks)), ptr(block_ptr_table(accum_blocks)), i64(len(emb_blocks)),
-        i64(block_size), dtype_code(b0.dtype), ctypes.c_double(lr), ctypes.c_double(eps), stream_ptr(dev)))
+        i64(block_size), i64(_pitch_bytes(emb_blocks, accum_blocks)), dtype_code(b0.dtype), ctypes.c_double(lr),
+        ctypes.c_double(eps), stream_ptr(dev)))
 
 
 def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_index=None, weight=None, out_dtype=None,
@@ -1015,7 +1038,8 @@ def plan_expand_rows(plan, n_out, rows=None, blocks=None, block_size=0, row_inde
         stamp_table = block_ptr_table(stamp_blocks)
     out = torch.empty((n_out, D), dtype=out_dtype or dt, device=dev)
     weight = _contig(weight)
-    check(lib().recis_csr_expand_rows_stamped(ptr(rows_arg), ptr(table), i64(n_blocks), i64(block_size), ptr(row_index),
+    check(lib().recis_csr_expand_rows_stamped(ptr(rows_arg), ptr(table), i64(n_blocks), i64(block_size),
+                                              i64(_pitch_bytes(blocks) if blocks is not None else 0), ptr(row_index),
                                               dtype_code(dt), ptr(weight),
                                               dtype_code(weight.dtype) if weight is not None else 0,
                                               ptr(plan.row_start), ptr(plan.occ), ptr(plan.hot_items), i64(plan.hot_cap),

@@ -55,8 +55,12 @@ def _trained_table(name, n, dim=8, slice_=None, seed=0):
     return ht, opt, ids
 
 
+@pytest.mark.parametrize("packed", ["0", "1"])
 @pytest.mark.parametrize("parallel", [1, 8])
-def test_save_then_read_load_and_save_again(tmp_path, parallel, monkeypatch):
+def test_save_then_read_load_and_save_again(tmp_path, parallel, packed, monkeypatch):
+    """``packed``: the saved table keeps its optimizer state next to the embedding rows
+    (RECIS_PACKED_STATE=1) or in arrays of its own; the table that loads it does the opposite."""
+    monkeypatch.setenv("RECIS_PACKED_STATE", packed)
     monkeypatch.setenv("RECIS_BLOCK_WRITE_SIZE", "3000")   # several pieces per slot
     monkeypatch.setenv("RECIS_BLOCK_READ_SIZE", "1700")
     n, dim = 10000, 8
@@ -80,11 +84,14 @@ def test_save_then_read_load_and_save_again(tmp_path, parallel, monkeypatch):
 
     # (2) a fresh table with the same slots loads it; every slot agrees key by key
     HashtableRegister().clear()   # as in a new process that restores the checkpoint
+    monkeypatch.setenv("RECIS_PACKED_STATE", "1" if packed == "0" else "0")
     ht2 = HashTable([dim], block_size=1024, device="cuda", name=name + "_copy", children=[name])
     SparseAdamW(filter_out_sparse_param(ht2), lr=1e-2)
     dense2 = {"tower.weight": torch.zeros(5, 3, device="cuda"), "step": torch.tensor(0)}
     Loader(path, hashtables={"t": ht2}, tensors=dense2, parallel=parallel).load()
     impl2 = ht2._hashtable_impl
+    assert impl.emb_blocks()[0][0].is_contiguous() == (packed == "0")
+    assert impl2.emb_blocks()[0][0].is_contiguous() == (packed == "1")
     assert impl2.ids_num() == n
     rows2 = impl2.lookup_index_readonly(ids)
     rows1 = impl.lookup_index_readonly(ids)
