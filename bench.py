@@ -813,20 +813,101 @@ class ModulePath5:
 # counter is scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC = {
-    "c4": {"csr_rows_adam_kernel": 733113958, "csr_expand_kernel": 258937651, "plan_bucket_kernel": 192621772,
-           "plan_scatter_kernel": 60780339, "plan_hist_kernel": 23678156, "bucketize_kernel": 10267033,
-           "plan_colscan_kernel": 3316121, "csr_hot_finish_kernel": 1168384, "plan_assign_new_kernel": 60825},
-    "c3": {"csr_rows_adam_kernel": 762296729, "csr_expand_kernel": 369877094, "plan_bucket_kernel": 201006899,
-           "plan_scatter_kernel": 49638809, "plan_hist_kernel": 19164467},
-    "c5": {"tile_fwd_kernel": 549494886, "csr_rows_adagrad_kernel": 769086668, "seg_pool_fwd_kernel": 93490380,
-           "block_gather_kernel": 109106995, "plan_bucket_kernel": 95353446, "plan_scatter_kernel": 46209536},
-    "c2": {"seg_pool_fwd_kernel(sum)": 4319621529, "seg_pool_bwd_kernel(sum)": 4321926758,
-           "seg_max_fwd_kernel": 4453851545, "seg_max_bwd_kernel": 4453888307},
+    "c4": {"csr_rows_adam_kernel": 733137612, "csr_expand_kernel": 279684505, "plan_bucket_kernel": 192615833,
+           "plan_scatter_kernel": 60778086, "plan_hist_kernel": 23677952, "bucketize_kernel": 10267238,
+           "plan_colscan_kernel": 3305881, "csr_hot_finish_kernel": 1179648, "plan_assign_new_kernel": 60825},
+    "c3": {"csr_rows_adam_kernel": 767397478, "csr_expand_kernel": 389580390, "plan_bucket_kernel": 200619008,
+           "plan_scatter_kernel": 49669427, "plan_assign_new_kernel": 23479500, "plan_hist_kernel": 19194368},
+    "c5": {"tile_fwd_kernel": 549505638, "csr_rows_adagrad_kernel": 769052876, "seg_pool_fwd_kernel": 93497753,
+           "block_gather_kernel": 109106995, "plan_bucket_kernel": 95373721, "plan_scatter_kernel": 46198784},
+    "c2": {"seg_pool_fwd_kernel(sum)": 4319621529, "seg_pool_bwd_kernel(sum)": 4321946419,
+           "seg_max_fwd_kernel": 4453851545, "seg_max_bwd_kernel": 4453874585},
 }
 
 
 def _measured_traffic(wl):
+    if "_variant_" in wl.name:   # the counters were read on the named configurations only
+        return {}
     return MEASURED_TRAFFIC.get(type(wl).__name__.lower().replace("config", "c"), {})
+
+
+# Requests per launch that leave the compute units' first-level caches for the L2, reads + writes
+# (rocprofv3 --pmc TCP_TCC_READ_REQ_sum TCP_TCC_WRITE_REQ_sum of this file with --workload W; a read
+# request carries up to 128 bytes, a write request up to 64). The kernels of these steps touch rows
+# of 64-256 bytes at random places, so what they wait for is the number of requests, not the bytes:
+# see _random_request_ceiling.
+MEASURED_REQUESTS = {
+    "c4": {"csr_rows_adam_kernel": 7273000, "csr_expand_kernel": 3625000, "plan_bucket_kernel": 3371000,
+           "plan_scatter_kernel": 1006000, "plan_hist_kernel": 692000, "plan_assign_new_kernel": 198000,
+           "bucketize_kernel": 134000, "plan_colscan_kernel": 47000, "csr_hot_finish_kernel": 11000},
+    "c3": {"csr_rows_adam_kernel": 8436000, "csr_expand_kernel": 5576000, "plan_bucket_kernel": 3292000,
+           "plan_scatter_kernel": 934000, "plan_hist_kernel": 647000, "plan_assign_new_kernel": 400000,
+           "plan_colscan_kernel": 46000, "csr_hot_finish_kernel": 11000},
+    "c5": {"csr_rows_adagrad_kernel": 9528000, "plan_bucket_kernel": 1780000, "seg_pool_fwd_kernel": 1710000,
+           "block_gather_kernel": 1272000, "plan_scatter_kernel": 1090000, "plan_hist_kernel": 574000},
+}
+
+
+def _random_request_ceiling(slot_mb=4096, n=1 << 24):
+    """Requests per second this device serves when every lane asks for another random line: the
+    step filter's own kernel (recis_block_filter: one 8-byte read at a random row of an int64 slot
+    per thread, one byte written per thread in order). Measured live; it reads 5.0-5.3e10/s over a
+    64 MB - 1 GB slot and 4.2-4.4e10/s over 4 - 8 GB, whatever is fetched per request (8 bytes here,
+    64-byte rows in the steps), while requests that follow one another in memory are served at
+    1.1e11/s (config 5's padded gather): every random request opens another page of the memory, and
+    that rate, not the bytes, is what a step of 64- or 128-byte rows at random places runs into."""
+    from recis_amd import ops
+    rows = slot_mb * 2**20 // 8
+    slot = torch.zeros(rows, 1, dtype=torch.int64, device="cuda")
+    idx = torch.randint(0, rows, (n,), device="cuda")
+    ms = _event_ms(lambda: ops.block_filter(idx, [slot], rows, 1), 10)
+    return n / ms * 1e3
+
+
+def request_ceiling_probe():
+    """What this device does with random accesses, by the product's own row movers (--workload probe):
+    requests per second of recis_block_filter (8 bytes per request) over slots of several sizes, and
+    rows per second of recis_gather (random rows in, one output row each) for 64- and 128-byte rows,
+    next to the same calls with the rows in order."""
+    from recis_amd import ops
+    out = {"metric": "random requests per second", "block_filter_8B_reads": {}, "gather_rows": {}}
+    n = 1 << 24
+    for mb in (64, 1024, 4096, 8192):
+        out["block_filter_8B_reads"]["%d_MB_slot" % mb] = round(_random_request_ceiling(mb, n) / 1e9, 2)
+    n = 1 << 22
+    for D in (16, 32):
+        rows = (4 << 30) // (4 * D)
+        table = torch.zeros(rows, D, device="cuda")
+        idx = torch.randint(0, rows, (n,), device="cuda")
+        seq = torch.arange(n, device="cuda")
+        t_rand = _event_ms(lambda: ops.gather(idx, table), 10)
+        t_seq = _event_ms(lambda: ops.gather(seq, table), 10)
+        out["gather_rows"]["%d_byte_rows_4096_MB" % (4 * D)] = {
+            "random_G_rows_per_s": round(n / t_rand / 1e6, 2), "in_order_G_rows_per_s": round(n / t_seq / 1e6, 2),
+            "random_GBps_read": round(n * 4 * D / t_rand / 1e6, 1), "in_order_GBps_read": round(n * 4 * D / t_seq / 1e6, 1)}
+        del table, idx, seq
+        torch.cuda.empty_cache()
+    out["unit"] = "G requests/s (block_filter), G rows/s (gather)"
+    return out
+
+
+def _request_roofline(wl, kernels_us, ms_per_step, ceiling):
+    """The step against the random-request ceiling: requests per launch (MEASURED_REQUESTS) over
+    the launch times measured in this run, per kernel and for the whole step."""
+    req = MEASURED_REQUESTS.get(type(wl).__name__.lower().replace("config", "c"))
+    if not req or "_variant_" in wl.name:
+        return None
+    per_kernel = {k: round(req[k] / kernels_us[k] / 1e3, 1) for k in req if kernels_us.get(k)}
+    dom = max((k for k in per_kernel), key=lambda k: kernels_us[k])
+    out = {"bound": "random requests to memory", "unit": "G requests/s", "peak": round(ceiling / 1e9, 1),
+           "peak_source": "recis_block_filter at random rows of a 64 MB slot (4.3e10/s over 4 GB), this run",
+           "kernel": dom, "achieved": per_kernel[dom], "frac": round(per_kernel[dom] * 1e9 / ceiling, 3),
+           "requests_per_launch": req[dom], "kernels_g_requests_per_s": per_kernel}
+    if type(wl).__name__ in ("Config3", "Config4"):   # steps whose every kernel of weight works at random places
+        total = sum(req.values())
+        out.update({"step_requests": total, "step_floor_ms": round(total / ceiling * 1e3, 4),
+                    "step_frac": round(total / ceiling * 1e3 / ms_per_step, 3)})
+    return out
 
 
 def checkpoint_round_trip(rows=8 << 20, dim=16, parallel=8):
@@ -943,8 +1024,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "ckpt"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "ckpt", "probe"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--batch", type=int, default=0,
+                    help="config 4 with another number of samples per step (default 65536): a smaller table")
+    ap.add_argument("--rotate", type=int, default=0,
+                    help="config 4 rotating over this many batches (default 8): the table holds that many batches' keys")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-stages", action="store_true",
                     help="skip the stage-by-stage timings, so that every kernel launch of the run belongs to a "
@@ -964,8 +1049,16 @@ def main():
     if args.workload == "ckpt":
         print(json.dumps(checkpoint_round_trip()))
         return
+    if args.workload == "probe":
+        print(json.dumps(request_ceiling_probe()))
+        return
     classes = {"c4": Config4, "c2": Config2, "c3": Config3, "c5": Config5}
-    main_wl = classes[args.workload]()
+    if args.workload == "c4" and (args.batch or args.rotate):   # a variant for experiments, named as such
+        main_wl = Config4(batch=args.batch or 65536, n_batches=args.rotate or 8)
+        main_wl.name += "_variant_batch%d_rotate%d" % (args.batch or 65536, args.rotate or 8)
+        args.no_extra = args.no_cpu_baseline = True
+    else:
+        main_wl = classes[args.workload]()
     # part of set-up, before the W warm-up steps: the first steps of a process pay for the device
     # allocations of the step's outputs (config 5: 2 GB blocks, tens of ms)
     if hasattr(main_wl, "prepare"):
@@ -1006,9 +1099,12 @@ def main():
         roof, kernels_us, _ = _kernel_roofline(wl, iters)
         nbytes = wl.algorithmic_bytes()
         nbytes = sum(nbytes.values()) if isinstance(nbytes, dict) else nbytes
-        return {"ms_per_step": round(ms, 4), "ids_per_s": wl.ids_per_step / ms * 1e3,
-                "unique_ids_per_step": wl.U, "step_roofline": _step_roofline(wl, ms), "roofline": roof,
-                "kernels_us": kernels_us}
+        res = {"ms_per_step": round(ms, 4), "ids_per_s": wl.ids_per_step / ms * 1e3,
+               "unique_ids_per_step": wl.U, "step_roofline": _step_roofline(wl, ms), "roofline": roof,
+               "kernels_us": kernels_us}
+        if out.get("request_roofline"):
+            res["request_roofline"] = _request_roofline(wl, kernels_us, ms, out["request_roofline"]["peak"] * 1e9)
+        return res
 
     if args.calib_copy:
         src = torch.zeros(1 << 28, device="cuda")
@@ -1037,6 +1133,8 @@ def main():
         out["kernels_us"] = kernels_us
         out["kernels_gbs"] = kernels_gbs
         out["step_roofline"] = _step_roofline(main_wl, ms_per_step)
+        ceiling = _random_request_ceiling(64)
+        out["request_roofline"] = _request_roofline(main_wl, kernels_us, ms_per_step, ceiling)
         if stages is not None:
             ab = main_wl.algorithmic_bytes()
             out["stages_ms"] = {k: round(v, 4) for k, v in stages.items()}
