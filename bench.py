@@ -887,7 +887,32 @@ def request_ceiling_probe():
             "random_GBps_read": round(n * 4 * D / t_rand / 1e6, 1), "in_order_GBps_read": round(n * 4 * D / t_seq / 1e6, 1)}
         del table, idx, seq
         torch.cuda.empty_cache()
-    out["unit"] = "G requests/s (block_filter), G rows/s (gather)"
+    # the bare probe: rows at random places and nothing else (recis_hip_probe_random_rows)
+    from recis_amd import _lib
+    lib, i64, ptr = _lib.lib(), _lib.i64, _lib.ptr
+    sink = torch.zeros(4096, dtype=torch.int32, device="cuda")
+    n = 1 << 23
+    out["bare_rows"] = {}
+    for mb in (256, 4096, 16384):
+        table = torch.zeros(mb << 18, dtype=torch.int32, device="cuda")
+        for row_bytes in (64, 128, 256):
+            rows = (mb << 20) // row_bytes
+            rand = torch.randint(0, rows, (n,), device="cuda", dtype=torch.int32)
+            seq = (torch.arange(n, device="cuda", dtype=torch.int32) % rows).contiguous()
+            res = {}
+            for name, idx, in_flight, write in (("random_read", rand, 1, 0), ("random_read_4_in_flight", rand, 4, 0),
+                                                ("random_write", rand, 1, 1), ("in_order_read", seq, 1, 0),
+                                                ("in_order_write", seq, 1, 1)):
+                def call():
+                    _lib.check(lib.recis_hip_probe_random_rows(ptr(table), i64(rows), i64(row_bytes), ptr(idx), i64(n),
+                                                               in_flight, write, ptr(sink), _lib.stream_ptr(table.device)))
+                ms = _event_ms(call, 10)
+                res[name] = {"G_rows_per_s": round(n / ms / 1e6, 1), "GBps": round(n * row_bytes / ms / 1e6)}
+            out["bare_rows"]["%d_MB_table_%d_byte_rows" % (mb, row_bytes)] = res
+            del rand, seq
+        del table
+        torch.cuda.empty_cache()
+    out["unit"] = "G requests/s (block_filter), G rows/s (gather, bare_rows)"
     return out
 
 

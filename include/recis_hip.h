@@ -70,6 +70,18 @@ int recis_hip_abi_version(void);
 int recis_hip_profile_enable(int on);
 int recis_hip_profile_report(char* buf, int64_t cap);
 
+/*
+ * Measurement support, no reference counterpart: n rows of row_bytes (a power of two, 16..1024;
+ * 16 bytes per lane) of `table` (rows of that width back to back, `rows` of them) at the places
+ * idx[0..n), read (write == 0: nothing is written; `sink`, 16 KB of device memory, only keeps the
+ * loads alive) or overwritten with a pattern (write != 0), rows_in_flight (1, 2 or 4) rows per
+ * lane group at a time. With random idx it shows how many rows per second the device serves when
+ * every row is somewhere else, which is what the row kernels of the training step are held
+ * against (bench.py --workload probe).
+ */
+int recis_hip_probe_random_rows(void* table, int64_t rows, int64_t row_bytes, const int32_t* idx,
+                                int64_t n, int rows_in_flight, int write, void* sink, void* stream);
+
 /* Synchronises the current device, returns the soft-error bits raised by
  * kernels since the last poll in *bits and clears them. */
 int recis_hip_poll_device_errors(int* bits);

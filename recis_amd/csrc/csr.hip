@@ -55,7 +55,7 @@ constexpr int kExpandRows = 2;  // unique rows a lane group works at a time: the
 // dense array of rows: each row is read once here); without it for a small table, whose rows the
 // update at the end of the step and the next step's lookups find in the caches again.
 template <typename TIn, typename TOut, int VEC, bool BLK, bool STREAM = true>
-__global__ void __launch_bounds__(kBlock)
+__global__ void __launch_bounds__(kBlock, 8)
 csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs a) {
   const int D = a.D;
   const int cl = threadIdx.x & ((1 << a.lpr_log2) - 1);
@@ -141,37 +141,50 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
   // ---- cold rows: kExpandRows of them per lane group. The kernel is a chain of dependent accesses
   // per row (list bounds -> row index -> row -> destinations -> stores) with 16 bytes per lane in
   // flight; with every resident wave busy that is still too little to fill the memory system, so a
-  // group walks the chain for two rows at once.
+  // group walks the chain for two rows at once, and the cold workgroups stride over the batches of
+  // rows with the NEXT batch's list bounds and table rows asked for before this batch is worked
+  // (their round trip runs under this batch's row reads and stores).
   const int groups_per_block = kBlock >> a.lpr_log2;
-  const int64_t first = (static_cast<int64_t>(blockIdx.x) - hot_blocks) * (kExpandRows * groups_per_block) +
-                        (threadIdx.x >> a.lpr_log2);
-  // Everything that depends on the row number alone is asked for at once: the plan's count, the
-  // list bounds, the table row (and, for a table in one block, the block's address): one round
-  // trip instead of three in a row. U may be the caller's upper bound (the plan's own count
-  // decides which rows exist): the arrays hold U entries, so a row below U is safe to read.
-  int64_t u[kExpandRows];
-  int32_t start[kExpandRows], end[kExpandRows];
-  int64_t ri_read[kExpandRows];
-  bool is_long[kExpandRows], is_short[kExpandRows];
+  const int32_t per_batch = kExpandRows * groups_per_block;
   const void* base0 = nullptr;
   void* stamp_base0 = nullptr;
   if constexpr (BLK) {
     base0 = a.blocks[0];
     if (a.stamp_blocks) stamp_base0 = a.stamp_blocks[0];
   }
+  // U may be the caller's upper bound (the plan's own count decides which rows exist): the arrays
+  // hold U entries, so a row below U is safe to read.
+  const int32_t n_unique = static_cast<int32_t>(min(a.U, a.counts[0]));
+  const int32_t n_batches = (n_unique + per_batch - 1) / per_batch;
+  const int32_t stride = static_cast<int32_t>(a.cold_blocks);
+  int32_t start_n[kExpandRows], end_n[kExpandRows];
+  int64_t ri_n[kExpandRows];
+  auto ask = [&](int32_t bt) {
+#pragma unroll
+    for (int r = 0; r < kExpandRows; ++r) {
+      const int32_t un = bt * per_batch + (threadIdx.x >> a.lpr_log2) + r * groups_per_block;
+      const int32_t at = un < n_unique ? un : 0;
+      start_n[r] = a.row_start[at];
+      end_n[r] = a.row_start[at + 1];
+      ri_n[r] = BLK ? a.row_index[at] : 0;
+    }
+  };
+  int32_t batch = static_cast<int32_t>(static_cast<int64_t>(blockIdx.x) - hot_blocks);
+  if (batch < n_batches) ask(batch);
+  for (; batch < n_batches; batch += stride) {
+  int64_t u[kExpandRows];
+  int32_t start[kExpandRows], end[kExpandRows];
+  int64_t ri_read[kExpandRows];
+  bool is_long[kExpandRows], is_short[kExpandRows];
 #pragma unroll
   for (int r = 0; r < kExpandRows; ++r) {
-    u[r] = first + r * groups_per_block;
-    const int64_t at = u[r] < a.U ? u[r] : 0;
-    start[r] = a.row_start[at];
-    end[r] = a.row_start[at + 1];
-    ri_read[r] = BLK ? a.row_index[at] : 0;
-  }
-  const int64_t n_unique = min(a.U, a.counts[0]);
-#pragma unroll
-  for (int r = 0; r < kExpandRows; ++r) {
+    u[r] = static_cast<int64_t>(batch) * per_batch + (threadIdx.x >> a.lpr_log2) + r * groups_per_block;
+    start[r] = start_n[r];
+    end[r] = end_n[r];
+    ri_read[r] = ri_n[r];
     if (u[r] >= n_unique) start[r] = end[r] = 0;
   }
+  if (batch + stride < n_batches) ask(batch + stride);
 #pragma unroll
   for (int r = 0; r < kExpandRows; ++r) {
     if (end[r] - start[r] > a.hot_len) end[r] = start[r];  // written by the work items
@@ -262,6 +275,7 @@ csr_expand_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, ExpArgs 
       }
     }
   }
+  }  // batches
 }
 
 // src / coef of every list entry, for the backward of pooled segments and of the padded gather over
@@ -587,7 +601,9 @@ int recis_csr_expand_rows_stamped(const void* rows, void* const* emb_blocks_dev,
   a.stamp_blocks = stamp_blocks_dev;
   a.stamp_value = stamp_value_dev;
   const int rows_per_block = kExpandRows * (kBlock >> a.lpr_log2);
-  a.cold_blocks = (U + rows_per_block - 1) / rows_per_block;
+  RECIS_REQUIRE(U <= INT32_MAX, "more unique rows than 32-bit list entries name");
+  // the cold workgroups stride over the batches of rows: as many as the device holds at once
+  a.cold_blocks = std::min<int64_t>((U + rows_per_block - 1) / rows_per_block, cold_grid_blocks());
   const int64_t hot_blocks = hot_cap > 0 ? std::min<int64_t>(hot_cap, 4096) : 0;
   const dim3 grid(static_cast<unsigned>(a.cold_blocks + hot_blocks));
   auto with_types = [&](auto tin, auto tout) {

@@ -284,6 +284,20 @@ __device__ __forceinline__ void wave_gather_range(const SrcView<TIn>& s, const C
   }
 }
 
+// Workgroups of kBlock threads that a row kernel which strides over its rows launches on the current
+// device: 32 per compute unit (four times what a unit holds at once, so that the workgroups that finish
+// early leave their place to others; 4 - 96 were measured), RECIS_COLD_GRID_PER_CU to try another number.
+inline int64_t cold_grid_blocks() {
+  static const int64_t n = [] {
+    int cus = 256;
+    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, current_device());
+    const char* s = std::getenv("RECIS_COLD_GRID_PER_CU");
+    const int per = s != nullptr && *s ? std::atoi(s) : 32;
+    return static_cast<int64_t>(cus) * std::max(1, per);
+  }();
+  return n;
+}
+
 constexpr int kCoopLen = 8;  // longer lists are shared among the lane groups of a wave
 
 // One launch for all rows. The last cold_blocks workgroups: one group of LPR lanes per unique row
