@@ -4,6 +4,7 @@
 // csrc/ops/ids_partition_kernel.cu:86-131 followed by atomic scatters over duplicated ids; the
 // plan is what lets every gradient scatter over duplicates run as a gather-reduce per unique row.
 #pragma once
+#include <cstdlib>
 
 #include <ATen/ATen.h>
 #include <torch/custom_class.h>
