@@ -813,10 +813,10 @@ class ModulePath5:
 # counter is scaled by what it reads for the calibration kernel that moves 1 GiB each way
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 MEASURED_TRAFFIC = {
-    "c4": {"csr_rows_adam_kernel": 733137612, "csr_expand_kernel": 279684505, "plan_bucket_kernel": 192615833,
+    "c4": {"csr_rows_adam_kernel": 733263974, "csr_expand_kernel": 267866214, "plan_bucket_kernel": 192615833,
            "plan_scatter_kernel": 60778086, "plan_hist_kernel": 23677952, "bucketize_kernel": 10267238,
            "plan_colscan_kernel": 3305881, "csr_hot_finish_kernel": 1179648, "plan_assign_new_kernel": 60825},
-    "c3": {"csr_rows_adam_kernel": 767397478, "csr_expand_kernel": 389580390, "plan_bucket_kernel": 200619008,
+    "c3": {"csr_rows_adam_kernel": 768038502, "csr_expand_kernel": 386756403, "plan_bucket_kernel": 200619008,
            "plan_scatter_kernel": 49669427, "plan_assign_new_kernel": 23479500, "plan_hist_kernel": 19194368},
     "c5": {"tile_fwd_kernel": 549505638, "csr_rows_adagrad_kernel": 769052876, "seg_pool_fwd_kernel": 93497753,
            "block_gather_kernel": 109106995, "plan_bucket_kernel": 95373721, "plan_scatter_kernel": 46198784},
@@ -837,10 +837,10 @@ def _measured_traffic(wl):
 # of 64-256 bytes at random places, so what they wait for is the number of requests, not the bytes:
 # see _random_request_ceiling.
 MEASURED_REQUESTS = {
-    "c4": {"csr_rows_adam_kernel": 7273000, "csr_expand_kernel": 3625000, "plan_bucket_kernel": 3371000,
+    "c4": {"csr_rows_adam_kernel": 7283000, "csr_expand_kernel": 3640000, "plan_bucket_kernel": 3408000,
            "plan_scatter_kernel": 1006000, "plan_hist_kernel": 692000, "plan_assign_new_kernel": 198000,
            "bucketize_kernel": 134000, "plan_colscan_kernel": 47000, "csr_hot_finish_kernel": 11000},
-    "c3": {"csr_rows_adam_kernel": 8436000, "csr_expand_kernel": 5576000, "plan_bucket_kernel": 3292000,
+    "c3": {"csr_rows_adam_kernel": 8435000, "csr_expand_kernel": 5635000, "plan_bucket_kernel": 3292000,
            "plan_scatter_kernel": 934000, "plan_hist_kernel": 647000, "plan_assign_new_kernel": 400000,
            "plan_colscan_kernel": 46000, "csr_hot_finish_kernel": 11000},
     "c5": {"csr_rows_adagrad_kernel": 9528000, "plan_bucket_kernel": 1780000, "seg_pool_fwd_kernel": 1710000,
