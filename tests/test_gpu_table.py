@@ -423,3 +423,29 @@ def test_look_back_gives_up_instead_of_hanging():
     p = ops.ids_unique_plan(ids)
     assert torch.equal(torch.sort(p.unique).values, torch.unique(ids))
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("row_bytes", [64, 256])
+def test_random_row_probe_reads_nothing_away_and_writes_whole_rows(rng, row_bytes):
+    """recis_hip_probe_random_rows (measurement support): the read mode leaves table and sink alone,
+    the write mode overwrites exactly the rows it was given, whole; arguments it cannot serve are refused."""
+    lib, i64, ptr = _lib.lib(), _lib.i64, _lib.ptr
+    rows, n = 5000, 3000
+    table = torch.full((rows, row_bytes // 4), 7, dtype=torch.int32, device="cuda")
+    sink = torch.zeros(4096, dtype=torch.int32, device="cuda")
+    idx = torch.from_numpy(rng.permutation(rows)[:n].astype(np.int32)).cuda()
+    stream = _lib.stream_ptr(table.device)
+    for in_flight in (1, 2, 4):
+        _lib.check(lib.recis_hip_probe_random_rows(ptr(table), i64(rows), i64(row_bytes), ptr(idx), i64(n), in_flight, 0,
+                                                   ptr(sink), stream))
+    assert int((table != 7).sum()) == 0 and int(sink.abs().sum()) == 0
+    _lib.check(lib.recis_hip_probe_random_rows(ptr(table), i64(rows), i64(row_bytes), ptr(idx), i64(n), 2, 1, ptr(sink), stream))
+    touched = torch.zeros(rows, dtype=torch.bool, device="cuda")
+    touched[idx.long()] = True
+    changed = (table != 7).any(dim=1)
+    assert torch.equal(changed, touched)
+    assert bool((table[touched][:, 1::4] == 1).all()) and bool((table[touched][:, 3::4] == 3).all())
+    assert bool((table[~touched] == 7).all())
+    assert lib.recis_hip_probe_random_rows(ptr(table), i64(rows), i64(48), ptr(idx), i64(n), 1, 0, ptr(sink), stream) == 1
+    assert lib.recis_hip_probe_random_rows(ptr(table), i64(rows), i64(row_bytes), ptr(idx), i64(n), 3, 0, ptr(sink), stream) == 1
+    assert _lib.poll_device_errors() == 0
