@@ -356,7 +356,9 @@ int recis_block_filter(const int64_t* ids, void* const* blocks_dev, int64_t n_bl
  *   w *= weight_decay; m = m*beta1 + g*(1-beta1); v = v*beta2 + (1-beta2)*g*g;
  *   w += alpha * (m / (sqrtf(v) + eps))
  * computed as the reference CPU functor does (double products, float sqrt, one
- * rounding per assignment). index must not contain duplicates.
+ * rounding per assignment; on 16-bit rows every assignment rounds double -> float ->
+ * row type and the last line rounds the step to the row type before it is added, as
+ * `Half += double` does in block_apply_adamw_op.cc:55-56). index must not contain duplicates.
  */
 int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dtype,
                             void* const* emb_blocks_dev, void* const* exp_avg_blocks_dev,

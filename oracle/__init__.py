@@ -333,6 +333,33 @@ def block_apply_adamw(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, 
     return alpha
 
 
+def block_apply_adamw_f16(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, lr, beta1, beta2,
+                          weight_decay, eps, block_size):
+    """block_apply_adamw on float16 rows and gradients, as the reference's CPU functor computes it
+    when TEmb = at::Half (block_apply_adamw_op.cc:32-58): every product and sum in double (a Half
+    operand meets a double), every assignment rounds double -> float -> half, sqrtf of the Half in
+    float, and `emb_elem += <double>` converts the step to Half first and adds the two Halves in
+    float (c10::Half defines += for Half operands only). numpy, vectorised over the rows of a call;
+    ``index`` holds no duplicates. Pinned bit for bit against the compiled reference
+    (tests/test_oracle_ref_ops.py)."""
+    index = _i64(index)
+    alpha = cal_alpha(b1_t, b2_t, lr, beta1, beta2)
+    r16 = lambda x: x.astype(np.float32).astype(np.float16)
+    g = np.asarray(grad, dtype=np.float16).astype(np.float64)
+    blk, row = index // block_size, index % block_size
+    for b in np.unique(blk):
+        sel = blk == b
+        r = row[sel]
+        w = r16(emb_blocks[b][r].astype(np.float64) * weight_decay)
+        m = r16(exp_avg[b][r].astype(np.float64) * beta1 + g[sel] * (1 - beta1))
+        v = r16(exp_avg_sq[b][r].astype(np.float64) * beta2 + (1 - beta2) * g[sel] * g[sel])
+        step = r16(alpha * (m.astype(np.float64) / (np.sqrt(v.astype(np.float32)).astype(np.float64) + eps)))
+        emb_blocks[b][r] = (w.astype(np.float32) + step.astype(np.float32)).astype(np.float16)
+        exp_avg[b][r] = m
+        exp_avg_sq[b][r] = v
+    return alpha
+
+
 def block_apply_adagrad(index, grad, emb_blocks, accum, lr, eps, block_size):
     index, grad = _i64(index), _f32(grad)
     D = emb_blocks[0].shape[1]

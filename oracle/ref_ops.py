@@ -10,7 +10,7 @@ import numpy as np
 
 BINARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_ref", "ref_ops")
 _CODES = {np.dtype(np.float32): 0, np.dtype(np.float64): 1, np.dtype(np.int64): 2, np.dtype(np.int32): 3,
-          np.dtype(np.bool_): 4, np.dtype(np.int8): 5}
+          np.dtype(np.bool_): 4, np.dtype(np.int8): 5, np.dtype(np.float16): 6}
 _TYPES = {v: k for k, v in _CODES.items()}
 
 

@@ -23,7 +23,7 @@
 // left unresolved at link time (lazy binding) and are never reached: every tensor here is on the CPU.
 //
 // File format (little endian): int64 count, then per tensor: int32 dtype code, int32 ndim,
-// int64 dims[ndim], raw bytes. dtype codes: 0 f32, 1 f64, 2 i64, 3 i32, 4 bool, 5 i8.
+// int64 dims[ndim], raw bytes. dtype codes: 0 f32, 1 f64, 2 i64, 3 i32, 4 bool, 5 i8, 6 f16.
 #include <torch/extension.h>
 
 #include <chrono>
@@ -63,6 +63,7 @@ static at::ScalarType code_to_type(int c) {
     case 3: return at::kInt;
     case 4: return at::kBool;
     case 5: return at::kChar;
+    case 6: return at::kHalf;
   }
   TORCH_CHECK(false, "bad dtype code ", c);
 }
@@ -74,6 +75,7 @@ static int type_to_code(at::ScalarType t) {
     case at::kInt: return 3;
     case at::kBool: return 4;
     case at::kChar: return 5;
+    case at::kHalf: return 6;
     default: TORCH_CHECK(false, "unsupported output dtype");
   }
 }

@@ -98,7 +98,14 @@ __device__ __forceinline__ void adam_compute_pack(Pack<T, VEC>& w, Pack<T, VEC>&
     we = to_float(from_float<T>(static_cast<float>(we * c.decay)));
     me = to_float(from_float<T>(static_cast<float>(me * c.beta1 + ge * omb1)));
     ve = to_float(from_float<T>(static_cast<float>(ve * c.beta2 + omb2 * ge * ge)));
-    we = to_float(from_float<T>(static_cast<float>(we + alpha * (me / (sqrtf(ve) + c.eps)))));
+    if constexpr (sizeof(T) == 2) {
+      // 16-bit rows: `emb_elem += <double>` (block_apply_adamw_op.cc:55-56) converts the step to the row
+      // type first and adds the two in float (c10::Half has no += for a double): two roundings
+      const float upd = to_float(from_float<T>(static_cast<float>(alpha * (me / (sqrtf(ve) + c.eps)))));
+      we = to_float(from_float<T>(we + upd));
+    } else {
+      we = to_float(from_float<T>(static_cast<float>(we + alpha * (me / (sqrtf(ve) + c.eps)))));
+    }
     w.v[j] = from_float<T>(we);
     m.v[j] = from_float<T>(me);
     v.v[j] = from_float<T>(ve);

@@ -449,3 +449,34 @@ def test_random_row_probe_reads_nothing_away_and_writes_whole_rows(rng, row_byte
     assert lib.recis_hip_probe_random_rows(ptr(table), i64(rows), i64(48), ptr(idx), i64(n), 1, 0, ptr(sink), stream) == 1
     assert lib.recis_hip_probe_random_rows(ptr(table), i64(rows), i64(row_bytes), ptr(idx), i64(n), 3, 0, ptr(sink), stream) == 1
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("D,bs", [(16, 64), (24, 33)])
+def test_adamw_half_rows_bit_exact_vs_oracle(rng, D, bs):
+    """float16 rows and gradients: the roundings of the reference's CPU functor with TEmb = at::Half
+    (oracle.block_apply_adamw_f16, itself pinned against the compiled reference): every assignment
+    rounds double -> float -> half and the step is rounded to half before it is added. The stand-alone
+    row kernel and the fused gather-reduce ending, which share the arithmetic."""
+    U, steps = 300, 8
+    lr, b1, b2, eps, decay = 1e-2, 0.9, 0.999, 1e-8, 0.99
+    rows0 = (0.5 * rng.standard_normal((U, D))).astype(np.float16)
+    c_emb, c_m, c_v = _np_blocks(rows0, bs), _np_blocks(np.zeros_like(rows0), bs), _np_blocks(np.zeros_like(rows0), bs)
+    g_emb, g_m, g_v = [_dev(b) for b in c_emb], [_dev(b) for b in c_m], [_dev(b) for b in c_v]
+    f_emb, f_m, f_v = [b.clone() for b in g_emb], [b.clone() for b in g_m], [b.clone() for b in g_v]
+    cb1, cb2 = np.ones(1, np.float32), np.ones(1, np.float32)
+    gb1, gb2, fb1, fb2 = _dev(cb1), _dev(cb2), _dev(cb1), _dev(cb2)
+    for _ in range(steps):
+        idx = np.sort(rng.permutation(U)[:rng.integers(1, U)])
+        g = rng.standard_normal((len(idx), D)).astype(np.float16)
+        oracle.block_apply_adamw_f16(idx, g, c_emb, cb1, cb2, c_m, c_v, lr, b1, b2, decay, eps, bs)
+        ops.block_apply_adamw(_dev(idx), _dev(g), g_emb, gb1, gb2, None, g_m, g_v, lr, b1, b2, decay, eps, bs)
+        # the same step through the fused ending: one occurrence per row, so the sum is the gradient itself
+        plan = ops.ids_unique_plan(_dev(np.arange(len(idx), dtype=np.int64) * 7919))
+        order = plan.unique.cpu().numpy() // 7919          # unique id u is occurrence order[u]
+        ops.csr_gather_reduce_adamw(_dev(g), plan, plan.occ, None, _dev(idx[order]), f_emb, fb1, fb2, f_m, f_v, lr, b1, b2,
+                                    decay, eps, bs)
+    for gl, fl, cl in ((g_emb, f_emb, c_emb), (g_m, f_m, c_m), (g_v, f_v, c_v)):
+        np.testing.assert_array_equal(torch.cat(gl).cpu().numpy(), np.concatenate(cl))
+        np.testing.assert_array_equal(torch.cat(fl).cpu().numpy(), np.concatenate(cl))
+    np.testing.assert_array_equal(gb1.cpu().numpy(), cb1)
+    assert _lib.poll_device_errors() == 0

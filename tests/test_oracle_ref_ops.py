@@ -184,6 +184,34 @@ def test_block_apply_adamw_bit_exact(beta_dtype):
     np.testing.assert_array_equal(emb, r_emb)
 
 
+@pytest.mark.parametrize("beta_dtype", [np.float32, np.float64])
+def test_block_apply_adamw_half_rows_bit_exact(beta_dtype):
+    # the same functor with TEmb = at::Half (rows AND gradients float16): where the roundings fall,
+    # and that `emb_elem += <double>` rounds the step to Half before it is added
+    rng = np.random.default_rng(17)
+    bs, nb, D, T, n = 32, 3, 12, 6, 50
+    R = bs * nb
+    emb = (0.5 * rng.standard_normal((R, D))).astype(np.float16)
+    m = np.zeros((R, D), np.float16)
+    v = np.zeros((R, D), np.float16)
+    index = np.stack([rng.permutation(R)[:n] for _ in range(T)]).astype(np.int64)
+    grad = rng.standard_normal((T, n, D)).astype(np.float16)
+    lr, b1, b2, wd, eps = 0.013, 0.9, 0.999, 0.99, 1e-8
+    b1t, b2t = np.ones(1, beta_dtype), np.ones(1, beta_dtype)
+    r_emb, r_m, r_v, r_b1t, r_b2t = ref_ops.run(
+        "adamw", [index, grad, emb.copy(), m.copy(), v.copy(), b1t.copy(), b2t.copy(),
+                  np.asarray([lr, b1, b2, wd, eps, bs], np.float64)])
+    assert r_emb.dtype == np.float16
+    blocks = lambda t: [t[i * bs:(i + 1) * bs] for i in range(nb)]
+    for t in range(T):
+        oracle.block_apply_adamw_f16(index[t], grad[t], blocks(emb), b1t, b2t, blocks(m), blocks(v), lr, b1, b2, wd,
+                                     eps, bs)
+    np.testing.assert_array_equal(b1t, r_b1t)
+    np.testing.assert_array_equal(m, r_m)
+    np.testing.assert_array_equal(v, r_v)
+    np.testing.assert_array_equal(emb, r_emb)
+
+
 # ------------------------------------------------------------------ dedup / tagging / feature ops
 def test_ids_partition_matches_cpu_op():
     # csrc/ops/ids_partition.cc:6-37. Non-negative ids: for a negative id the CPU op takes the shard
