@@ -34,6 +34,7 @@ extern "C" {
 #define RECIS_F32 0
 #define RECIS_BF16 1
 #define RECIS_F16 2
+#define RECIS_F64 3 /* rows and gradients of recis_block_apply_adamw only */
 
 /* combiners (csrc/ops/embedding_segment_reduce.h:8 has SUM, MEAN, TILE; MAX is
  * an addition with no reference counterpart) */
@@ -359,6 +360,8 @@ int recis_block_filter(const int64_t* ids, void* const* blocks_dev, int64_t n_bl
  * rounding per assignment; on 16-bit rows every assignment rounds double -> float ->
  * row type and the last line rounds the step to the row type before it is added, as
  * `Half += double` does in block_apply_adamw_op.cc:55-56). index must not contain duplicates.
+ * Rows of RECIS_F64 take RECIS_F64 gradients (the functor's TEmb = double: nothing is rounded but
+ * the argument of sqrtf); the other entry points know the three narrower types only.
  */
 int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dtype,
                             void* const* emb_blocks_dev, void* const* exp_avg_blocks_dev,

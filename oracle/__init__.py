@@ -360,6 +360,28 @@ def block_apply_adamw_f16(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_
     return alpha
 
 
+def block_apply_adamw_f64(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, lr, beta1, beta2,
+                          weight_decay, eps, block_size):
+    """block_apply_adamw on float64 rows and gradients (the functor with TEmb = double,
+    block_apply_adamw_op.cc:32-58): everything in double, nothing rounded but the argument of
+    sqrtf, which is converted to float first. numpy; ``index`` holds no duplicates. Pinned bit for
+    bit against the compiled reference (tests/test_oracle_ref_ops.py)."""
+    index = _i64(index)
+    alpha = cal_alpha(b1_t, b2_t, lr, beta1, beta2)
+    g = np.asarray(grad, dtype=np.float64)
+    blk, row = index // block_size, index % block_size
+    for b in np.unique(blk):
+        sel = blk == b
+        r = row[sel]
+        w = emb_blocks[b][r] * weight_decay
+        m = exp_avg[b][r] * beta1 + g[sel] * (1 - beta1)
+        v = exp_avg_sq[b][r] * beta2 + (1 - beta2) * g[sel] * g[sel]
+        emb_blocks[b][r] = w + alpha * (m / (np.sqrt(v.astype(np.float32)).astype(np.float64) + eps))
+        exp_avg[b][r] = m
+        exp_avg_sq[b][r] = v
+    return alpha
+
+
 def block_apply_adagrad(index, grad, emb_blocks, accum, lr, eps, block_size):
     index, grad = _i64(index), _f32(grad)
     D = emb_blocks[0].shape[1]

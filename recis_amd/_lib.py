@@ -16,6 +16,7 @@ HEADER_PATH = os.path.join(_HERE, "..", "include", "recis_hip.h")
 _lib = None
 
 F32, BF16, F16 = 0, 1, 2
+F64 = 3   # rows and gradients of block_apply_adamw only
 SUM, MEAN, TILE, MAX = 0, 1, 2, 3
 FLAG_REV_UNIQUE = 1
 

@@ -77,6 +77,34 @@ adamw_rows_kernel(OptArgs a, const TG* __restrict__ grad, T* const* __restrict__
   }
 }
 
+// Rows of doubles (the functor with TEmb = double, block_apply_adamw_op.cc:32-58): an element per
+// thread, everything in double but the square root (sqrtf of the value converted to float).
+__global__ void __launch_bounds__(kBlock)
+adamw_rows_f64_kernel(OptArgs a, const double* __restrict__ grad, double* const* __restrict__ emb_blocks,
+                      double* const* __restrict__ m_blocks, double* const* __restrict__ v_blocks,
+                      const double* __restrict__ alpha_ptr, double beta1, double beta2, double decay, double eps) {
+#pragma clang fp contract(off)
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (e >= a.n * a.D) return;
+  const int64_t i = e / a.D;
+  const int d = static_cast<int>(e - i * a.D);
+  int64_t b, off;
+  if (!row_offset(a, a.index[i], b, off)) {
+    if (d == 0) raise_device_error(a.err, RECIS_DEVERR_INDEX_RANGE);
+    return;
+  }
+  const int64_t at = off * a.pitch + d;
+  const double g = grad[e], alpha = alpha_ptr[0];
+  double w = emb_blocks[b][at], m = m_blocks[b][at], v = v_blocks[b][at];
+  w = w * decay;
+  m = m * beta1 + g * (1 - beta1);
+  v = v * beta2 + (1 - beta2) * g * g;
+  w += alpha * (m / (sqrtf(static_cast<float>(v)) + eps));
+  emb_blocks[b][at] = w;
+  m_blocks[b][at] = m;
+  v_blocks[b][at] = v;
+}
+
 template <typename T, typename TG, int VEC>
 __global__ void __launch_bounds__(kBlock)
 adagrad_rows_kernel(OptArgs a, const TG* __restrict__ grad, T* const* __restrict__ emb_blocks,
@@ -182,6 +210,29 @@ int recis_block_apply_adamw(const int64_t* index, const void* grad, int grad_dty
   if (int rc = launch_cal_alpha(beta1_t, beta2_t, beta_is_f64, alpha, lr, beta1, beta2, stream)) return rc;
   if (n == 0) return RECIS_OK;
   RECIS_REQUIRE(emb_blocks_dev && exp_avg_blocks_dev && exp_avg_sq_blocks_dev, "block tables must not be NULL");
+  if (row_dtype == RECIS_F64) {
+    RECIS_REQUIRE(grad_dtype == RECIS_F64, "rows of doubles take gradients of doubles");
+    RECIS_REQUIRE(n >= 0 && n_blocks >= 1 && block_size >= 1 && D >= 1 && D <= (1 << 20) && index && grad, "bad arguments");
+    RECIS_REQUIRE(row_pitch_bytes == 0 || (row_pitch_bytes >= D * 8 && row_pitch_bytes % 8 == 0),
+                  "row pitch of %lld bytes does not fit rows of %lld doubles", (long long)row_pitch_bytes, (long long)D);
+    OptArgs a{};
+    a.index = index;
+    a.n = n;
+    a.n_blocks = n_blocks;
+    a.block_size = block_size;
+    a.pitch = row_pitch_bytes ? row_pitch_bytes / 8 : D;
+    a.D = static_cast<int>(D);
+    a.err = device_error_word(current_device());
+    RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");
+    const int64_t grid = (n * D + kBlock - 1) / kBlock;
+    RECIS_TIME_KERNEL("adamw_rows_kernel", stream)
+    adamw_rows_f64_kernel<<<dim3(grid), dim3(kBlock), 0, stream>>>(
+        a, static_cast<const double*>(grad), reinterpret_cast<double* const*>(emb_blocks_dev),
+        reinterpret_cast<double* const*>(exp_avg_blocks_dev), reinterpret_cast<double* const*>(exp_avg_sq_blocks_dev),
+        alpha, beta1, beta2, weight_decay, eps);
+    RECIS_LAUNCH_CHECK();
+    return RECIS_OK;
+  }
   OptArgs a;
   int vec = 1;
   if (int rc = fill_opt_args(a, index, grad, n, n_blocks, block_size, row_pitch_bytes, D, row_dtype, grad_dtype, vec)) return rc;

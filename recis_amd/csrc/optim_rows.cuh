@@ -76,6 +76,9 @@ struct AdamCoef {
 template <typename beta_t>
 __device__ __forceinline__ double cal_alpha_step(beta_t b1_old, beta_t b2_old, double lr, double beta1, double beta2,
                                                  beta_t& b1_new, beta_t& b2_new) {
+  // no fused multiply-add: with double powers `1 - b1_old * beta1` would otherwise skip the rounding of
+  // the product that the reference's `beta1_t[0] *= beta1` makes
+#pragma clang fp contract(off)
   b1_new = static_cast<beta_t>(b1_old * beta1);
   b2_new = static_cast<beta_t>(b2_old * beta2);
   const beta_t bc1 = 1 - b1_new;

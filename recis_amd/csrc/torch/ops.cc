@@ -339,11 +339,15 @@ void block_apply_adamw(const Tensor index, const Tensor grad, TensorList emb_blo
   const int64_t D = row_bytes(b0) / static_cast<int64_t>(b0.element_size());
   TORCH_CHECK(g.numel() == i.numel() * D, "grad has ", g.numel(), " elements, expected ", i.numel(), " x ", D);
   Tensor t0 = block_ptr_table(emb_blocks), t1 = block_ptr_table(exp_avg), t2 = block_ptr_table(exp_avg_sq);
-  check(recis_block_apply_adamw(i.data_ptr<int64_t>(), g.data_ptr(), dtype_code(g.scalar_type()),
+  // rows of doubles (the reference's functor is dispatched for them too) go with gradients of doubles
+  auto code = [&](at::ScalarType t) {
+    return t == at::kDouble && b0.scalar_type() == at::kDouble ? RECIS_F64 : dtype_code(t);
+  };
+  check(recis_block_apply_adamw(i.data_ptr<int64_t>(), g.data_ptr(), code(g.scalar_type()),
                                 static_cast<void* const*>(t0.data_ptr()), static_cast<void* const*>(t1.data_ptr()),
                                 static_cast<void* const*>(t2.data_ptr()), static_cast<int64_t>(emb_blocks.size()),
                                 block_size, shared_row_pitch_bytes({&b0, &exp_avg[0], &exp_avg_sq[0]}),
-                                dtype_code(b0.scalar_type()), beta1_t.data_ptr(), beta2_t.data_ptr(),
+                                code(b0.scalar_type()), beta1_t.data_ptr(), beta2_t.data_ptr(),
                                 beta1_t.scalar_type() == at::kDouble ? 1 : 0, lr, beta1, beta2, weight_decay, eps,
                                 i.numel(), D, stream_of(b0.device())));
 }

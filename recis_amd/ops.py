@@ -305,10 +305,12 @@ def block_apply_adamw(index, grad, emb_blocks, beta1_t, beta2_t, step, exp_avg, 
     D = _row_bytes(b0) // b0.element_size()
     if grad.numel() != index.numel() * D:
         raise ValueError("grad has %d elements, expected %d x %d" % (grad.numel(), index.numel(), D))
+    # rows of doubles (the reference's functor is dispatched for them too) go with gradients of doubles
+    code = lambda dt: _lib.F64 if dt == torch.float64 and b0.dtype == torch.float64 else dtype_code(dt)
     check(lib().recis_block_apply_adamw(
-        ptr(index), ptr(grad), dtype_code(grad.dtype), ptr(block_ptr_table(emb_blocks)),
+        ptr(index), ptr(grad), code(grad.dtype), ptr(block_ptr_table(emb_blocks)),
         ptr(block_ptr_table(exp_avg)), ptr(block_ptr_table(exp_avg_sq)), i64(len(emb_blocks)),
-        i64(block_size), i64(_pitch_bytes(emb_blocks, exp_avg, exp_avg_sq)), dtype_code(b0.dtype), ptr(beta1_t),
+        i64(block_size), i64(_pitch_bytes(emb_blocks, exp_avg, exp_avg_sq)), code(b0.dtype), ptr(beta1_t),
         ptr(beta2_t), int(beta1_t.dtype == torch.float64), ctypes.c_double(lr), ctypes.c_double(beta1),
         ctypes.c_double(beta2), ctypes.c_double(weight_decay), ctypes.c_double(eps),
         i64(index.numel()), i64(D), stream_ptr(b0.device)))

@@ -480,3 +480,27 @@ def test_adamw_half_rows_bit_exact_vs_oracle(rng, D, bs):
         np.testing.assert_array_equal(torch.cat(fl).cpu().numpy(), np.concatenate(cl))
     np.testing.assert_array_equal(gb1.cpu().numpy(), cb1)
     assert _lib.poll_device_errors() == 0
+
+
+@pytest.mark.parametrize("beta_dtype", [np.float32, np.float64])
+def test_adamw_double_rows_bit_exact_vs_oracle(rng, beta_dtype):
+    """float64 rows and gradients (the reference's functor is dispatched for them): bit for bit the
+    oracle's restatement, which the compiled reference pins; other gradient types are refused."""
+    U, D, bs, steps = 200, 5, 64, 6
+    lr, b1, b2, eps, decay = 1e-2, 0.9, 0.999, 1e-8, 0.99
+    rows0 = rng.standard_normal((U, D))
+    c_emb, c_m, c_v = _np_blocks(rows0, bs), _np_blocks(np.zeros_like(rows0), bs), _np_blocks(np.zeros_like(rows0), bs)
+    g_emb, g_m, g_v = [_dev(b) for b in c_emb], [_dev(b) for b in c_m], [_dev(b) for b in c_v]
+    cb1, cb2 = np.ones(1, beta_dtype), np.ones(1, beta_dtype)
+    gb1, gb2 = _dev(cb1), _dev(cb2)
+    for _ in range(steps):
+        idx = np.sort(rng.permutation(U)[:rng.integers(1, U)])
+        g = rng.standard_normal((len(idx), D))
+        oracle.block_apply_adamw_f64(idx, g, c_emb, cb1, cb2, c_m, c_v, lr, b1, b2, decay, eps, bs)
+        ops.block_apply_adamw(_dev(idx), _dev(g), g_emb, gb1, gb2, None, g_m, g_v, lr, b1, b2, decay, eps, bs)
+    for gl, cl in ((g_emb, c_emb), (g_m, c_m), (g_v, c_v)):
+        np.testing.assert_array_equal(torch.cat(gl).cpu().numpy(), np.concatenate(cl))
+    np.testing.assert_array_equal(gb1.cpu().numpy(), cb1)
+    with pytest.raises((TypeError, _lib.RecisHipError)):
+        ops.block_apply_adamw(_dev(idx), _dev(g.astype(np.float32)), g_emb, gb1, gb2, None, g_m, g_v, lr, b1, b2, decay, eps, bs)
+    assert _lib.poll_device_errors() == 0

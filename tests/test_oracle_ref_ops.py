@@ -212,6 +212,31 @@ def test_block_apply_adamw_half_rows_bit_exact(beta_dtype):
     np.testing.assert_array_equal(emb, r_emb)
 
 
+@pytest.mark.parametrize("beta_dtype", [np.float32, np.float64])
+def test_block_apply_adamw_double_rows_bit_exact(beta_dtype):
+    # the functor with TEmb = double: no rounding but sqrtf's float argument
+    rng = np.random.default_rng(27)
+    bs, nb, D, T, n = 32, 3, 5, 5, 50
+    R = bs * nb
+    emb = rng.standard_normal((R, D))
+    m, v = np.zeros((R, D)), np.zeros((R, D))
+    index = np.stack([rng.permutation(R)[:n] for _ in range(T)]).astype(np.int64)
+    grad = rng.standard_normal((T, n, D))
+    lr, b1, b2, wd, eps = 0.013, 0.9, 0.999, 0.99, 1e-8
+    b1t, b2t = np.ones(1, beta_dtype), np.ones(1, beta_dtype)
+    r_emb, r_m, r_v, r_b1t, r_b2t = ref_ops.run(
+        "adamw", [index, grad, emb.copy(), m.copy(), v.copy(), b1t.copy(), b2t.copy(),
+                  np.asarray([lr, b1, b2, wd, eps, bs], np.float64)])
+    assert r_emb.dtype == np.float64
+    blocks = lambda t: [t[i * bs:(i + 1) * bs] for i in range(nb)]
+    for t in range(T):
+        oracle.block_apply_adamw_f64(index[t], grad[t], blocks(emb), b1t, b2t, blocks(m), blocks(v), lr, b1, b2, wd,
+                                     eps, bs)
+    np.testing.assert_array_equal(m, r_m)
+    np.testing.assert_array_equal(v, r_v)
+    np.testing.assert_array_equal(emb, r_emb)
+
+
 # ------------------------------------------------------------------ dedup / tagging / feature ops
 def test_ids_partition_matches_cpu_op():
     # csrc/ops/ids_partition.cc:6-37. Non-negative ids: for a negative id the CPU op takes the shard
