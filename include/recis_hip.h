@@ -412,6 +412,18 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
                  int inverse_is64, int64_t* count_out_dev, void* stream);
 
 /*
+ * The ordering half of ids_partition_cuda (csrc/ops/ids_partition_kernel.cu:36-55, the sort by
+ * PartitionKey): n ids without duplicates are put in ascending order of rotr64(id, 16) taken as
+ * unsigned, which is by shard slot (id & 0xFFFF) first. One radix sort of (key, position) pairs.
+ *   sorted_ids [n]   the ids in that order
+ *   order      [n]   order[k] = input position of sorted_ids[k]
+ *   rank       [n]   rank[order[k]] = k (the sorted position of every input position)
+ * n must fit 32 bits. Scratch comes from the stream's workspace.
+ */
+int recis_partition_order(const int64_t* ids, int64_t n, int64_t* sorted_ids, int32_t* order,
+                          int32_t* rank, void* stream);
+
+/*
  * Batch plan: dedup plus the transposed index. Unique ids (no duplicates, every id of the
  * batch present), an int32 inverse with unique_out[inverse[i]] == ids[i], the count, and the
  * occurrences grouped by unique id:

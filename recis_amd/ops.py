@@ -433,23 +433,33 @@ def ids_partition(ids, num_parts):
     """``torch.ops.recis.ids_partition`` (ids_partition.h:14), device ordering
     (ids_partition_kernel.cu:36-55): unique ids ascending by ``rotr64(id, 16)`` as
     unsigned, per-shard counts, int32 inverse. The dedup is the hash kernel; the
-    ordering of the (much smaller) unique set uses torch.sort."""
+    (much smaller) unique set is ordered by a radix sort of (rotated id, position)
+    pairs, and the inverse is a gather of 4-byte rows out of the rank table."""
     if ids.dim() != 1:
         raise ValueError("ids must be 1-dim")
     uniq, inv, count = ids_unique(ids)
     u = uniq[: int(count.item())]
-    rot = torch.bitwise_or(torch.bitwise_left_shift(u, 48),
-                           torch.bitwise_and(torch.bitwise_right_shift(u, 16), (1 << 48) - 1))
-    order = torch.argsort(torch.bitwise_xor(rot, -(1 << 63)))  # signed sort of the flipped key = unsigned sort
-    rank = torch.empty_like(order)
-    rank[order] = torch.arange(order.numel(), device=ids.device)
-    sorted_u = u[order]
+    sorted_u, _, rank = partition_order(u)
     m, r = divmod(_SLICE_SIZE, num_parts)
     slot = torch.bitwise_and(sorted_u, _SLICE_SIZE - 1)
     part = torch.maximum(torch.div(slot, m + 1, rounding_mode="floor"),
                          torch.div(slot - r, m, rounding_mode="trunc"))
     counts = torch.bincount(part, minlength=num_parts).to(torch.int64)
-    return sorted_u, counts, rank[inv.long()].to(torch.int32)
+    return sorted_u, counts, gather(inv, rank)
+
+
+def partition_order(unique_ids):
+    """The sort by PartitionKey of ids_partition_kernel.cu:36-55 on ids without duplicates:
+    ``(sorted_ids, order, rank)`` with ``sorted_ids == unique_ids[order]`` ascending by
+    ``rotr64(id, 16)`` as unsigned and ``rank[order[k]] == k`` (both int32)."""
+    require_cuda(unique_ids)
+    u = _ids64(unique_ids)
+    n = u.numel()
+    sorted_u = torch.empty_like(u)
+    order = torch.empty(n, dtype=torch.int32, device=u.device)
+    rank = torch.empty(n, dtype=torch.int32, device=u.device)
+    check(lib().recis_partition_order(ptr(u), i64(n), ptr(sorted_u), ptr(order), ptr(rank), stream_ptr(u.device)))
+    return sorted_u, order, rank
 
 
 # --------------------------------------------------------- sparse-mode pooling

@@ -147,6 +147,25 @@ def test_ids_partition_matches_oracle(rng, n, world):
     assert inv.dtype == torch.int32
 
 
+@pytest.mark.parametrize("n", [0, 1, 255, 70000, 3000000])
+def test_partition_order_is_the_unsigned_sort_of_the_rotated_ids(rng, n):
+    # ids_partition_kernel.cu:36-43: ascending by rotr64(id, 16) compared as unsigned
+    ids = rng.integers(-(1 << 62), 1 << 62, size=n)
+    if n > 100:  # the extremes of the key, and neighbours that differ in the rotated-out bits only
+        ids = np.concatenate([ids, [-(1 << 63), (1 << 63) - 1, -1, 0, 65535, 65536], ids[:50] ^ 1, ids[:50] ^ (1 << 15)])
+    ids = np.unique(ids)
+    rng.shuffle(ids)
+    s, order, rank = ops.partition_order(_dev(ids))
+    key = (ids.view(np.uint64) >> np.uint64(16)) | (ids.view(np.uint64) << np.uint64(48))
+    eorder = np.argsort(key, kind="stable")
+    np.testing.assert_array_equal(order.cpu().numpy(), eorder)
+    np.testing.assert_array_equal(s.cpu().numpy(), ids[eorder])
+    erank = np.empty(ids.size, np.int32)
+    erank[eorder] = np.arange(ids.size, dtype=np.int32)
+    np.testing.assert_array_equal(rank.cpu().numpy(), erank)
+    assert order.dtype == torch.int32 and rank.dtype == torch.int32
+
+
 def test_sparse_mode_ops(rng):
     # tests/nn/segment_ops_test.py:62-113
     data = torch.tensor([[1.0, 1.0], [2.0, 2.0], [3.0, 3.0]]).cuda()
