@@ -15,6 +15,7 @@ HEADER_PATH = os.path.join(_HERE, "..", "include", "recis_hip.h")
 
 _lib = None
 
+ABI_VERSION = 2  # RECIS_HIP_ABI_VERSION of include/recis_hip.h
 F32, BF16, F16 = 0, 1, 2
 F64 = 3   # rows and gradients of block_apply_adamw only
 SUM, MEAN, TILE, MAX = 0, 1, 2, 3
@@ -55,9 +56,9 @@ def lib():
         _lib = ctypes.CDLL(LIB_PATH)
         _lib.recis_hip_last_error.restype = ctypes.c_char_p
         abi = _lib.recis_hip_abi_version()
-        if abi != 2:
-            raise RecisHipError("librecis_hip.so ABI %d, expected 2: rebuild with "
-                                "python -m recis_amd.build" % abi)
+        if abi != ABI_VERSION:
+            raise RecisHipError("librecis_hip.so ABI %d, expected %d: rebuild with "
+                                "python -m recis_amd.build" % (abi, ABI_VERSION))
     return _lib
 
 
