@@ -405,8 +405,8 @@ int recis_merge_offsets(const void* const* offsets_ptrs, const int64_t* sizes,
  * device word count_out_dev. unique_out must have room for n entries.
  * Replaces the unique half of ids_partition_cuda (csrc/ops/ids_partition_kernel.cu:86-131)
  * and the torch.unique of recis/nn/modules/hashtable.py:278; the reference orders
- * the unique ids by sort key instead (sorted variants are built on top of this by
- * the host layer).
+ * the unique ids by sort key instead (recis_partition_order below puts them in that
+ * order).
  */
 int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inverse_out,
                  int inverse_is64, int64_t* count_out_dev, void* stream);
