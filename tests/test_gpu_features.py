@@ -166,6 +166,24 @@ def test_partition_order_is_the_unsigned_sort_of_the_rotated_ids(rng, n):
     assert order.dtype == torch.int32 and rank.dtype == torch.int32
 
 
+def test_partition_order_refuses_bad_arguments():
+    import ctypes
+
+    lib = _lib.lib()
+    u = _dev(np.arange(8, dtype=np.int64))
+    out = torch.empty(8, dtype=torch.int64, device="cuda")
+    o32 = torch.empty(8, dtype=torch.int32, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    n = ctypes.c_int64
+    st = _lib.stream_ptr(u.device)
+    assert lib.recis_partition_order(p(u), n(8), None, p(o32), p(o32), st) != 0       # a NULL output
+    assert lib.recis_partition_order(p(u), n(-1), p(out), p(o32), p(o32), st) != 0    # a negative count
+    assert lib.recis_partition_order(p(u), n(1 << 31), p(out), p(o32), p(o32), st) != 0  # positions are 32-bit
+    assert lib.recis_partition_order(None, n(0), None, None, None, st) == 0            # nothing to do
+    with pytest.raises(TypeError):
+        ops.partition_order(o32)
+
+
 def test_sparse_mode_ops(rng):
     # tests/nn/segment_ops_test.py:62-113
     data = torch.tensor([[1.0, 1.0], [2.0, 2.0], [3.0, 3.0]]).cuda()
