@@ -301,9 +301,9 @@ class Config4:
             "pool_bwd+adam": S * D * 4 + N * 4 + (U + 1) * 4 + U * 8 + U * D * 4 * 6,
         }
 
-    def survey_bytes(self):
-        """The step's compulsory bytes by the formula the survey of the reference prices config 4 with
-        (the [U, D] gradient between pooling backward and Adam counted as kept on chip)."""
+    def fused_minimum_bytes(self):
+        """The step's compulsory bytes with every intermediate counted as kept on chip (the [U, D]
+        gradient between pooling backward and Adam among them): the lowest price of this config."""
         N, U, S = self.N, self.U, self.N
         return N * (8 + 4 + 4) + U * (16 + 8 + 384 + 8) + S * (64 + 64) + 13 * self.c["batch"] * (4 + 8 + 8 + 8)
 
@@ -485,7 +485,7 @@ class Config3:
             self.step()
         return self.sweeps[-1]
 
-    def survey_bytes(self):
+    def fused_minimum_bytes(self):
         N, U, D = self.N, self.U, self.D
         return U * (16 + 8 + 768 + 8) + int(0.1 * N) * 16 + N * (8 + 4 + 128 + 128)
 
@@ -590,7 +590,7 @@ class Config5:
         self.opt.step()       # both gradients of the plan summed and the rows updated in one launch
         self.opt.zero_grad()
 
-    def survey_bytes(self):
+    def fused_minimum_bytes(self):
         N, U, S, D = self.N, self.U, self.S, self.D
         return 12 * N + U * (24 + 1024) + S * (256 + 256) + self.pad_rows * 256
 
@@ -1008,16 +1008,16 @@ def _kernel_roofline(wl, iters):
 
 
 def _step_roofline(wl, ms):
-    """Whole-step fractions of the HBM peak, by this build's count of compulsory bytes and by the
-    survey's formula for the same config."""
+    """Whole-step fractions of the HBM peak, by the bytes the kernels as built must move and by the
+    lowest price of the same config (every intermediate kept on chip)."""
     nbytes = wl.algorithmic_bytes()
     nbytes = sum(nbytes.values()) if isinstance(nbytes, dict) else nbytes
     out = {"algorithmic_bytes": nbytes, "achieved": nbytes / ms / 1e6, "frac": nbytes / ms / 1e6 / HBM_PEAK_GBS,
            "unit": "GB/s"}
-    if hasattr(wl, "survey_bytes"):
-        sb = wl.survey_bytes()
-        out["survey_bytes"] = sb
-        out["survey_frac"] = sb / ms / 1e6 / HBM_PEAK_GBS
+    if hasattr(wl, "fused_minimum_bytes"):
+        sb = wl.fused_minimum_bytes()
+        out["fused_minimum_bytes"] = sb
+        out["fused_minimum_frac"] = sb / ms / 1e6 / HBM_PEAK_GBS
     return out
 
 
