@@ -414,11 +414,15 @@ int recis_unique(const int64_t* ids, int64_t n, int64_t* unique_out, void* inver
 /*
  * The ordering half of ids_partition_cuda (csrc/ops/ids_partition_kernel.cu:36-55, the sort by
  * PartitionKey): n ids without duplicates are put in ascending order of rotr64(id, 16) taken as
- * unsigned, which is by shard slot (id & 0xFFFF) first. One radix sort of (key, position) pairs.
+ * unsigned, which is by shard slot (id & 0xFFFF) first: the stable order of (key, position).
+ * From 32768 ids up to some 8 million the keys are split into bins by their top bits and every bin is
+ * put in order in LDS; the host waits once, early, for a word that says whether every bin fits (ids
+ * whose shard slots are very unevenly spread do not). Those, and smaller and larger inputs, take a
+ * library sort of (key, position) pairs. Both ways give the same result.
  *   sorted_ids [n]   the ids in that order
  *   order      [n]   order[k] = input position of sorted_ids[k]
  *   rank       [n]   rank[order[k]] = k (the sorted position of every input position)
- * n must fit 32 bits. Scratch comes from the stream's workspace.
+ * n must fit 32 bits. Scratch comes from the stream's workspace. Waits for the stream (see above).
  */
 int recis_partition_order(const int64_t* ids, int64_t n, int64_t* sorted_ids, int32_t* order,
                           int32_t* rank, void* stream);

@@ -166,6 +166,44 @@ def test_partition_order_is_the_unsigned_sort_of_the_rotated_ids(rng, n):
     assert order.dtype == torch.int32 and rank.dtype == torch.int32
 
 
+def _check_partition_order(ids):
+    s, order, rank = ops.partition_order(_dev(ids))
+    key = (ids.view(np.uint64) >> np.uint64(16)) | (ids.view(np.uint64) << np.uint64(48))
+    eorder = np.argsort(key, kind="stable")
+    np.testing.assert_array_equal(order.cpu().numpy(), eorder)
+    np.testing.assert_array_equal(s.cpu().numpy(), ids[eorder])
+    erank = np.empty(ids.size, np.int32)
+    erank[eorder] = np.arange(ids.size, dtype=np.int32)
+    np.testing.assert_array_equal(rank.cpu().numpy(), erank)
+
+
+@pytest.mark.parametrize("case", ["one_slot", "two_slots", "few_top_bits", "sequential", "duplicates", "odd_bins",
+                                  "half_empty", "nine_million"])
+def test_partition_order_whatever_the_spread_of_the_shard_slots(rng, case):
+    # the bins of the fast way are cut by the top bits of the shard slot: inputs that fill them unevenly (down to
+    # every id in one slot) must come out the same, by the library sort
+    if case == "one_slot":
+        ids = np.unique(rng.integers(0, 1 << 40, size=200000)) * 65536 + 77
+    elif case == "two_slots":
+        ids = np.unique(rng.integers(0, 1 << 40, size=150000)) * 65536 + rng.integers(0, 2, size=1)[0] * 65535
+        ids = np.unique(np.concatenate([ids, ids[:70000] ^ 65535]))
+    elif case == "few_top_bits":  # slots 0..63 only: the low bits of the slot do not choose the bin
+        ids = np.unique(rng.integers(0, 1 << 30, size=300000) * 65536 + rng.integers(0, 64, size=300000))
+    elif case == "sequential":
+        ids = np.arange(1_000_003, dtype=np.int64) - 500_000
+    elif case == "duplicates":  # outside the contract (ids without duplicates), still the stable order
+        ids = rng.integers(0, 50000, size=400000)
+    elif case == "half_empty":  # every second bin empty, the others fit
+        ids = np.unique(rng.integers(0, 1 << 30, size=300000) * 65536 + (rng.integers(0, 32768, size=300000) & ~16))
+    elif case == "odd_bins":
+        ids = np.unique(rng.integers(-(1 << 62), 1 << 62, size=32769 + 4096))[:32769 + 2048]
+    else:  # past the most ids the bins take
+        ids = np.unique(rng.integers(-(1 << 62), 1 << 62, size=9_000_000))
+    ids = ids.astype(np.int64)
+    rng.shuffle(ids)
+    _check_partition_order(ids)
+
+
 def test_partition_order_refuses_bad_arguments():
     import ctypes
 
