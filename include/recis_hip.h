@@ -585,6 +585,22 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
                             void* stream);
 
 /*
+ * recis_csr_gather_reduce with the sum of unique id u stored at out[out_rows[u], :] instead of
+ * out[u, :] (no reference counterpart). out_rows [U] must name every row of out at most once and
+ * stay below the rows out holds: a permutation of 0 .. U-1 when U is the exact count. For a caller
+ * that wants the rows in another order than the plan's (ids_partition hands the unique ids out in
+ * the order of their shard slots: the backward of the pooling writes the gradient rows in that
+ * order at once, where it would otherwise write them in the plan's order and copy them).
+ */
+int recis_csr_gather_reduce_mapped(const void* rows, int rows_dtype, int64_t n_rows,
+                                   const int32_t* src, const void* coef, int coef_dtype,
+                                   const int32_t* row_start, const int32_t* hot_items,
+                                   int64_t hot_cap, const int64_t* counts_dev, void* out,
+                                   int out_dtype, int64_t U, int64_t D, int accumulate,
+                                   const void* cover_offsets, int cover_is64, int64_t cover_S,
+                                   const int32_t* out_rows, void* stream);
+
+/*
  * recis_csr_gather_reduce over input rows that live in n_parts (1 to 8) separate arrays instead
  * of one (no reference counterpart): src numbers the rows of part 0, then those of part 1, and so
  * on (part f holds part_counts[f] rows of D elements of rows_dtype). No coefficients, fp32 output

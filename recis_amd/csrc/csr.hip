@@ -473,6 +473,21 @@ int recis_csr_gather_reduce(const void* rows, int rows_dtype, int64_t n_rows, co
   return csr_gather_reduce_run<false>(r);
 }
 
+int recis_csr_gather_reduce_mapped(const void* rows, int rows_dtype, int64_t n_rows, const int32_t* src,
+                                   const void* coef, int coef_dtype, const int32_t* row_start,
+                                   const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, void* out,
+                                   int out_dtype, int64_t U, int64_t D, int accumulate, const void* cover_offsets,
+                                   int cover_is64, int64_t cover_S, const int32_t* out_rows, void* stream_) {
+  RECIS_REQUIRE(out_rows != nullptr || U == 0, "out_rows must not be NULL");
+  CsrRequest r = one_input_request(rows, rows_dtype, n_rows, src, coef, coef_dtype, row_start, hot_items, hot_cap,
+                                   counts_dev, U, D, cover_offsets, cover_is64, cover_S, stream_);
+  r.out = out;
+  r.out_dtype = out_dtype;
+  r.accumulate = accumulate;
+  r.out_rows = out_rows;
+  return csr_gather_reduce_run<false>(r);
+}
+
 int recis_csr_gather_reduce_parts(const void* const* part_rows, const int64_t* part_counts, int n_parts,
                                   int rows_dtype, const int32_t* src, const int32_t* row_start,
                                   const int32_t* hot_items, int64_t hot_cap, const int64_t* counts_dev, void* out,

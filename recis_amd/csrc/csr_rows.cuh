@@ -35,6 +35,7 @@ struct CsrArgs {
   int D;
   int lpr_log2;
   int accumulate;
+  const int32_t* out_rows;  // kEpiStore only: the sum of row u goes to out[out_rows[u]] (NULL: to out[u])
   int nt_in;  // the gathered rows are too many to stay cached: non-temporal loads
   // a second input over the same lists (kernels with TIn2 != void): entry k also adds
   // coef2[k] * rows2[src2[k]]; the cover range does not apply to it
@@ -491,7 +492,7 @@ csr_rows_kernel(const TIn* __restrict__ rows, TOut* __restrict__ out, CsrArgs a,
       else
         fused_row_update<TOut, VEC, EPI>(f, a.err, idx_mine, c0, acc, epi_is_adam(EPI) ? s_alpha : 0.0);
     } else {
-      TOut* dst = out + row * D + c0;
+      TOut* dst = out + (a.out_rows ? static_cast<int64_t>(a.out_rows[row]) : row) * D + c0;
       if (a.accumulate) {
         float old[VEC];
         load_pack<TOut, VEC>(dst, old);
@@ -600,7 +601,7 @@ csr_hot_finish_kernel(TOut* __restrict__ out, CsrArgs a, FuseArgs f) {
       if constexpr (EPI != kEpiStore) {
         fused_row_update<TOut, VEC, EPI>(f, a.err, f.row_index[u], c0, acc, alpha);
       } else {
-        TOut* dst = out + static_cast<int64_t>(u) * D + c0;
+        TOut* dst = out + static_cast<int64_t>(a.out_rows ? a.out_rows[u] : u) * D + c0;
         if (a.accumulate) {
           float old[VEC];
           load_pack<TOut, VEC>(dst, old);
@@ -658,6 +659,7 @@ struct CsrRequest {
   int out_dtype = RECIS_F32;                    // the table's row type when epi != kEpiStore
   int64_t U = 0, D = 0;
   int accumulate = 0;
+  const int32_t* out_rows = nullptr;            // kEpiStore only: where the sum of row u goes (see CsrArgs)
   const void* cover = nullptr;
   int cover64 = 0;
   int64_t cover_S = 0;
@@ -741,6 +743,7 @@ int csr_gather_reduce_run(const CsrRequest& r) {
   a.D = static_cast<int>(D);
   a.lpr_log2 = std::min(6, ilog2_ceil((D + vec - 1) / vec));
   a.accumulate = r.accumulate;
+  a.out_rows = r.out_rows;
   a.nt_in = r.in1.n_rows * D * in_sz >= (int64_t(1) << 30);
   a.err = device_error_word(current_device());
   RECIS_REQUIRE(a.err != nullptr, "could not reach the device error word");

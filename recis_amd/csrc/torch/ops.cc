@@ -138,14 +138,14 @@ Tensor segment_reduce_backward(Tensor grad_output, c10::optional<Tensor> weight,
   {
     // reverse_indices as ids_partition handed them out, untouched since: the occurrence lists of that
     // dedup are still there, so the gradient of every unique id is a gather-reduce over its list (no
-    // atomics), computed in the plan's order and brought into the sorted order of the unique ids
+    // atomics), each row stored at its place in the sorted order of the unique ids
     BatchPlanPtr plan;
-    Tensor order;
-    if ((m == RECIS_SUM || m == RECIS_MEAN) && known_partition(reverse_indices, &plan, &order) &&
-        plan->U() == unique_size) {
+    Tensor rank;
+    if ((m == RECIS_SUM || m == RECIS_MEAN) && known_partition(reverse_indices, &plan, &rank) &&
+        plan->U() == unique_size && rank.numel() == unique_size) {
       auto sc = plan->SrcCoefForPool(offsets, w.defined() ? c10::optional<Tensor>(w) : c10::nullopt, m == RECIS_MEAN);
       Tensor coef = std::get<1>(sc).has_value() ? *std::get<1>(sc) : Tensor();
-      Tensor out = gather(order, csr_gather_reduce(grad_output, plan, std::get<0>(sc), coef, Tensor()));
+      Tensor out = csr_gather_reduce(grad_output, plan, std::get<0>(sc), coef, Tensor(), rank);
       return grad_output.scalar_type() == at::kFloat ? out : out.to(grad_output.scalar_type());
     }
   }
@@ -475,7 +475,7 @@ std::tuple<Tensor, Tensor, Tensor> ids_partition(const Tensor& ids, int64_t num_
     check(recis_gather(inv.data_ptr(), index_kind(inv, "inverse"), rank.data_ptr(), U, inverse.data_ptr(), i.numel(),
                        sizeof(int32_t), stream_of(i.device())));
   note_unique(sorted_u);
-  note_partition(inverse, plan, order);
+  note_partition(inverse, plan, rank);
   return std::make_tuple(sorted_u, counts, inverse);
 }
 
@@ -484,18 +484,18 @@ struct NotedPartition {
   Tensor inverse;
   uint32_t version;
   BatchPlanPtr plan;
-  Tensor order;  // sorted position -> the plan's unique id
+  Tensor rank;  // the plan's unique id -> its position in the sorted order
 };
 std::vector<NotedPartition> g_noted_partitions;  // the last few, newest last
 }  // namespace
 
-void note_partition(const Tensor& inverse, const BatchPlanPtr& plan, const Tensor& order) {
+void note_partition(const Tensor& inverse, const BatchPlanPtr& plan, const Tensor& rank) {
   std::lock_guard<std::mutex> lock(g_unique_mu);
   if (g_noted_partitions.size() >= 2) g_noted_partitions.erase(g_noted_partitions.begin());
-  g_noted_partitions.push_back({inverse, inverse._version(), plan, order});
+  g_noted_partitions.push_back({inverse, inverse._version(), plan, rank});
 }
 
-bool known_partition(const Tensor& inverse, BatchPlanPtr* plan, Tensor* order) {
+bool known_partition(const Tensor& inverse, BatchPlanPtr* plan, Tensor* rank) {
   if (!inverse.defined() || inverse.numel() == 0) return false;
   std::lock_guard<std::mutex> lock(g_unique_mu);
   for (const auto& e : g_noted_partitions) {
@@ -503,7 +503,7 @@ bool known_partition(const Tensor& inverse, BatchPlanPtr* plan, Tensor* order) {
         e.inverse.scalar_type() == inverse.scalar_type() && inverse.is_contiguous() &&
         e.version == inverse._version() && e.inverse._version() == e.version) {
       *plan = e.plan;
-      *order = e.order;
+      *rank = e.rank;
       return true;
     }
   }
@@ -538,7 +538,7 @@ bool known_unique(const Tensor& t) {
 
 // ------------------------------------------------------------------------------------ over a batch plan
 Tensor csr_gather_reduce(const Tensor& rows_in, const BatchPlanPtr& plan, const Tensor& src, const Tensor& coef,
-                         const Tensor& cover) {
+                         const Tensor& cover, const Tensor& out_rows) {
   require_gpu(rows_in, "rows");
   require_gpu(src, "src");
   TORCH_CHECK(rows_in.dim() == 2, "gradient rows must be [rows, D]");
@@ -546,13 +546,27 @@ Tensor csr_gather_reduce(const Tensor& rows_in, const BatchPlanPtr& plan, const 
   Tensor rows = rows_in.contiguous();
   const int64_t D = rows.size(1), U = plan->U();
   Tensor out = at::empty({U, D}, rows.options().dtype(at::kFloat));
-  check(recis_csr_gather_reduce(
-      rows.data_ptr(), dtype_code(rows.scalar_type()), rows.size(0), src.data_ptr<int32_t>(),
-      coef.defined() ? coef.data_ptr() : nullptr, coef.defined() ? dtype_code(coef.scalar_type()) : 0,
-      plan->row_start().data_ptr<int32_t>(), plan->hot_items().data_ptr<int32_t>(), plan->hot_cap(),
-      plan->counts().data_ptr<int64_t>(), out.data_ptr(), RECIS_F32, U, D, 0, cover.defined() ? cover.data_ptr() : nullptr,
-      cover.defined() ? index_kind(cover, "offsets") : 0, cover.defined() ? cover.numel() - 1 : 0,
-      stream_of(rows.device())));
+  const void* coef_p = coef.defined() ? coef.data_ptr() : nullptr;
+  const int coef_dt = coef.defined() ? dtype_code(coef.scalar_type()) : 0;
+  const void* cover_p = cover.defined() ? cover.data_ptr() : nullptr;
+  const int cover64 = cover.defined() ? index_kind(cover, "offsets") : 0;
+  const int64_t cover_S = cover.defined() ? cover.numel() - 1 : 0;
+  if (out_rows.defined()) {
+    require_gpu(out_rows, "out_rows");
+    TORCH_CHECK(out_rows.scalar_type() == at::kInt && out_rows.is_contiguous() && out_rows.numel() >= U,
+                "out_rows must be a contiguous int32 tensor with an entry per unique id");
+    check(recis_csr_gather_reduce_mapped(
+        rows.data_ptr(), dtype_code(rows.scalar_type()), rows.size(0), src.data_ptr<int32_t>(), coef_p, coef_dt,
+        plan->row_start().data_ptr<int32_t>(), plan->hot_items().data_ptr<int32_t>(), plan->hot_cap(),
+        plan->counts().data_ptr<int64_t>(), out.data_ptr(), RECIS_F32, U, D, 0, cover_p, cover64, cover_S,
+        out_rows.data_ptr<int32_t>(), stream_of(rows.device())));
+  } else {
+    check(recis_csr_gather_reduce(
+        rows.data_ptr(), dtype_code(rows.scalar_type()), rows.size(0), src.data_ptr<int32_t>(), coef_p, coef_dt,
+        plan->row_start().data_ptr<int32_t>(), plan->hot_items().data_ptr<int32_t>(), plan->hot_cap(),
+        plan->counts().data_ptr<int64_t>(), out.data_ptr(), RECIS_F32, U, D, 0, cover_p, cover64, cover_S,
+        stream_of(rows.device())));
+  }
   return out;
 }
 

@@ -89,9 +89,10 @@ std::tuple<Tensor, Tensor> calc_ragged_index(Tensor drop_num, Tensor pad_num, Te
 
 // ---- over a batch plan (additions: the reference scatters with atomics instead)
 // out[u] = sum over the occurrence list of unique id u of coef[k] * rows[src[k]]: fp32 [U, D]. coef
-// and cover may be undefined (see recis_csr_gather_reduce).
+// and cover may be undefined (see recis_csr_gather_reduce). out_rows (int32 [U], a permutation) or
+// undefined: the sum of unique id u goes to row out_rows[u] of the result.
 Tensor csr_gather_reduce(const Tensor& rows, const BatchPlanPtr& plan, const Tensor& src, const Tensor& coef,
-                         const Tensor& cover);
+                         const Tensor& cover, const Tensor& out_rows = Tensor());
 // the same over rows that live in up to 8 arrays laid end to end in src's numbering
 Tensor csr_gather_reduce_parts(const TensorList& parts, const BatchPlanPtr& plan, const Tensor& src);
 // ids_partition notes the unique ids it hands out; known_unique(t) says whether t is one of those
@@ -99,10 +100,11 @@ Tensor csr_gather_reduce_parts(const TensorList& parts, const BatchPlanPtr& plan
 // kept alive, so their addresses cannot be handed out to another tensor meanwhile.
 void note_unique(const Tensor& t);
 bool known_unique(const Tensor& t);
-// The same for the inverse ids_partition hands out: the plan of that dedup and the order its unique
-// ids were sorted into stay available to the backward over that inverse (the last two calls).
-void note_partition(const Tensor& inverse, const BatchPlanPtr& plan, const Tensor& order);
-bool known_partition(const Tensor& inverse, BatchPlanPtr* plan, Tensor* order);
+// The same for the inverse ids_partition hands out: the plan of that dedup and the place of each of
+// its unique ids in the sorted order (rank, int32 [U]) stay available to the backward over that
+// inverse (the last two calls).
+void note_partition(const Tensor& inverse, const BatchPlanPtr& plan, const Tensor& rank);
+bool known_partition(const Tensor& inverse, BatchPlanPtr* plan, Tensor* rank);
 
 }  // namespace functional
 }  // namespace recis

@@ -823,22 +823,29 @@ def ids_unique_plan(ids, wait=True, need_inverse=True, need_pos=True, idmap=None
                                     bool(need_inverse), bool(need_pos))
 
 
-def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False, cover=None):
+def csr_gather_reduce(rows, plan, src, coef=None, out=None, accumulate=False, cover=None, out_rows=None):
     """``out[u] (+)= sum_k coef[k] * rows[src[k]]`` over the list of every unique id of
-    ``plan``; returns the fp32 ``[U, D]`` result."""
+    ``plan``; returns the fp32 ``[U, D]`` result. With ``out_rows`` (int32 ``[U]``, each row of
+    ``out`` named at most once) the sum of unique id ``u`` goes to ``out[out_rows[u]]``."""
     require_cuda(rows, src, coef)
     rows = _contig(rows)
     D = rows.shape[1]
     if out is None:
         out = torch.empty((plan.U, D), dtype=torch.float32, device=rows.device)
         accumulate = False
-    check(lib().recis_csr_gather_reduce(ptr(rows), dtype_code(rows.dtype), i64(rows.shape[0]), ptr(src), ptr(coef),
-                                        dtype_code(coef.dtype) if coef is not None else 0, ptr(plan.row_start),
-                                        ptr(plan.hot_items), i64(plan.hot_cap), ptr(plan.counts), ptr(out),
-                                        dtype_code(out.dtype), i64(plan.U), i64(D), int(bool(accumulate)),
-                                        ptr(cover), _index_kind(cover, "offsets") if cover is not None else 0,
-                                        i64(cover.numel() - 1 if cover is not None else 0),
-                                        stream_ptr(rows.device)))
+    head = (ptr(rows), dtype_code(rows.dtype), i64(rows.shape[0]), ptr(src), ptr(coef),
+            dtype_code(coef.dtype) if coef is not None else 0, ptr(plan.row_start),
+            ptr(plan.hot_items), i64(plan.hot_cap), ptr(plan.counts), ptr(out),
+            dtype_code(out.dtype), i64(plan.U), i64(D), int(bool(accumulate)),
+            ptr(cover), _index_kind(cover, "offsets") if cover is not None else 0,
+            i64(cover.numel() - 1 if cover is not None else 0))
+    if out_rows is None:
+        check(lib().recis_csr_gather_reduce(*head, stream_ptr(rows.device)))
+    else:
+        require_cuda(out_rows)
+        if out_rows.dtype != torch.int32 or out_rows.numel() < plan.U:
+            raise TypeError("out_rows must be int32 with an entry per unique id")
+        check(lib().recis_csr_gather_reduce_mapped(*head, ptr(_contig(out_rows)), stream_ptr(rows.device)))
     return out
 
 

@@ -445,6 +445,29 @@ def test_gather_reduce_over_separate_arrays_equals_the_concatenation(rng, dtype,
     assert _lib.poll_device_errors() == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [16, 40, 128])
+def test_gather_reduce_to_mapped_rows_equals_gather_reduce_then_permutation(rng, dtype, D):
+    """recis_csr_gather_reduce_mapped: the sum of unique id u stored at out[out_rows[u]]; the same sums as the
+    plain call (hot and cold rows), so bit for bit its result permuted."""
+    n = 50000
+    ids = np.concatenate([rng.integers(0, 30, n // 2), rng.integers(0, 15000, n - n // 2)])  # hot and cold rows
+    plan = ops.ids_unique_plan(_dev(ids))
+    rows = torch.randn((n, D), device="cuda").to(dtype)
+    src = torch.from_numpy(rng.permutation(n).astype(np.int32)).cuda()
+    src[::13] = -1
+    coef = torch.rand(n, device="cuda")
+    perm = torch.from_numpy(rng.permutation(plan.U).astype(np.int32)).cuda()
+    plain = ops.csr_gather_reduce(rows, plan, src, coef)
+    mapped = ops.csr_gather_reduce(rows, plan, src, coef, out_rows=perm)
+    assert torch.equal(mapped[perm.long()], plain)
+    again = ops.csr_gather_reduce(rows, plan, src, coef, out=mapped.clone(), accumulate=True, out_rows=perm)
+    torch.testing.assert_close(again[perm.long()], 2 * plain, rtol=1e-6, atol=1e-6)
+    with pytest.raises(TypeError):
+        ops.csr_gather_reduce(rows, plan, src, coef, out_rows=perm.long())
+    assert _lib.poll_device_errors() == 0
+
+
 @pytest.mark.parametrize("kind", ["adamw", "adagrad"])
 @pytest.mark.parametrize("D,row_dtype,grad_dtype", [(16, torch.float32, torch.float32), (128, torch.bfloat16, torch.bfloat16),
                                                     (40, torch.float32, torch.float32), (32, torch.bfloat16, torch.float32)])
