@@ -1049,7 +1049,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "ckpt", "probe"])
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "ckpt", "probe", "c4_unfused"],
+                    help="c4_unfused: config 4 through the reference's own operator sequence alone (the torch_library_path_ms "
+                         "leg of the default run), for a kernel trace of that sequence")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--batch", type=int, default=0,
                     help="config 4 with another number of samples per step (default 65536): a smaller table")
@@ -1076,6 +1078,14 @@ def main():
         return
     if args.workload == "probe":
         print(json.dumps(request_ceiling_probe()))
+        return
+    if args.workload == "c4_unfused":
+        wl = TorchLibraryPath4()
+        ms = _timed_steps(wl, args.steps, args.warmup)
+        print(json.dumps({"workload": "config 4 through ids_encode -> ids_partition -> embedding_lookup -> "
+                                      "segment_reduce_forward -> segment_reduce_backward -> accept_grad -> SparseAdam.step",
+                          "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+                          "ids_per_s": wl.N / ms * 1e3}))
         return
     classes = {"c4": Config4, "c2": Config2, "c3": Config3, "c5": Config5}
     if args.workload == "c4" and (args.batch or args.rotate):   # a variant for experiments, named as such
