@@ -342,10 +342,18 @@ def block_apply_adamw_f16(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_
     float (c10::Half defines += for Half operands only). numpy, vectorised over the rows of a call;
     ``index`` holds no duplicates. Pinned bit for bit against the compiled reference
     (tests/test_oracle_ref_ops.py)."""
+    g = np.asarray(grad, dtype=np.float16).astype(np.float64)
+    return _block_apply_adamw_16(index, g, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, lr, beta1, beta2, weight_decay,
+                                 eps, block_size, lambda x: x.astype(np.float32).astype(np.float16))
+
+
+def _block_apply_adamw_16(index, g, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, lr, beta1, beta2, weight_decay, eps,
+                          block_size, r16):
+    """The functor of block_apply_adamw_op.cc:32-58 with a 16-bit TEmb; ``r16`` is the rounding of a
+    float to that type (the result in an array type that holds its values exactly), ``g`` the
+    gradient in float64."""
     index = _i64(index)
     alpha = cal_alpha(b1_t, b2_t, lr, beta1, beta2)
-    r16 = lambda x: x.astype(np.float32).astype(np.float16)
-    g = np.asarray(grad, dtype=np.float16).astype(np.float64)
     blk, row = index // block_size, index % block_size
     for b in np.unique(blk):
         sel = blk == b
@@ -354,10 +362,35 @@ def block_apply_adamw_f16(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_
         m = r16(exp_avg[b][r].astype(np.float64) * beta1 + g[sel] * (1 - beta1))
         v = r16(exp_avg_sq[b][r].astype(np.float64) * beta2 + (1 - beta2) * g[sel] * g[sel])
         step = r16(alpha * (m.astype(np.float64) / (np.sqrt(v.astype(np.float32)).astype(np.float64) + eps)))
-        emb_blocks[b][r] = (w.astype(np.float32) + step.astype(np.float32)).astype(np.float16)
+        emb_blocks[b][r] = r16(w.astype(np.float32) + step.astype(np.float32))
         exp_avg[b][r] = m
         exp_avg_sq[b][r] = v
     return alpha
+
+
+def round_bf16(x):
+    """float -> bfloat16 as c10::BFloat16(float) rounds (round to nearest even on the upper 16 bits
+    of the float32 pattern, NaN stays NaN), returned as float32 (which holds every bfloat16 value).
+    Pinned against torch's own conversion on the CPU (tests/test_oracle_ref_ops.py)."""
+    f = np.ascontiguousarray(np.asarray(x).astype(np.float32))
+    u = f.view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    out = (r & 0xFFFFFFFF).astype(np.uint32).view(np.float32).copy()
+    out[np.isnan(f)] = np.nan
+    return out
+
+
+def block_apply_adamw_bf16(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, lr, beta1, beta2,
+                           weight_decay, eps, block_size):
+    """block_apply_adamw on bfloat16 rows (held as float32 arrays of bfloat16 values). The reference
+    dispatches its functor for float, double and Half only (block_apply_adamw_op.cc:96-102), so this
+    is that functor with TEmb = c10::BFloat16, which has the operators of c10::Half: the same
+    statements as block_apply_adamw_f16 (pinned by the compiled reference) with the rounding of
+    round_bf16 (pinned by torch's conversion). ``grad``: bfloat16 values, or float32 (the library
+    also takes full-precision gradients for 16-bit rows: the functor with a float gradient)."""
+    g = np.asarray(grad, dtype=np.float32).astype(np.float64)
+    return _block_apply_adamw_16(index, g, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, lr, beta1, beta2, weight_decay,
+                                 eps, block_size, lambda x: round_bf16(x.astype(np.float32)))
 
 
 def block_apply_adamw_f64(index, grad, emb_blocks, b1_t, b2_t, exp_avg, exp_avg_sq, lr, beta1, beta2,

@@ -482,6 +482,39 @@ def test_adamw_half_rows_bit_exact_vs_oracle(rng, D, bs):
     assert _lib.poll_device_errors() == 0
 
 
+@pytest.mark.parametrize("grad_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("D,bs", [(128, 64), (16, 1024), (7, 5)])
+def test_adamw_bfloat16_rows_bit_exact_vs_oracle(rng, D, bs, grad_dtype):
+    """bfloat16 rows (what config 5 trains on), gradients in bfloat16 or float32: bit for bit
+    oracle.block_apply_adamw_bf16, the Half restatement the compiled reference pins with bfloat16's
+    rounding in its place (the reference itself dispatches no bfloat16). The stand-alone row kernel and
+    the fused gather-reduce ending."""
+    U, steps = 300, 8
+    lr, b1, b2, eps, decay = 1e-2, 0.9, 0.999, 1e-8, 0.99
+    rows0 = oracle.round_bf16(0.5 * rng.standard_normal((U, D)))
+    c_emb, c_m, c_v = _np_blocks(rows0, bs), _np_blocks(np.zeros_like(rows0), bs), _np_blocks(np.zeros_like(rows0), bs)
+    g_emb, g_m, g_v = ([_dev(b, torch.bfloat16) for b in c] for c in (c_emb, c_m, c_v))
+    f_emb, f_m, f_v = [b.clone() for b in g_emb], [b.clone() for b in g_m], [b.clone() for b in g_v]
+    cb1, cb2 = np.ones(1, np.float32), np.ones(1, np.float32)
+    gb1, gb2, fb1, fb2 = _dev(cb1), _dev(cb2), _dev(cb1), _dev(cb2)
+    for _ in range(steps):
+        idx = np.sort(rng.permutation(U)[:rng.integers(1, U)])
+        g = rng.standard_normal((len(idx), D)).astype(np.float32)
+        if grad_dtype == torch.bfloat16:
+            g = oracle.round_bf16(g)
+        oracle.block_apply_adamw_bf16(idx, g, c_emb, cb1, cb2, c_m, c_v, lr, b1, b2, decay, eps, bs)
+        ops.block_apply_adamw(_dev(idx), _dev(g, grad_dtype), g_emb, gb1, gb2, None, g_m, g_v, lr, b1, b2, decay, eps, bs)
+        plan = ops.ids_unique_plan(_dev(np.arange(len(idx), dtype=np.int64) * 7919))
+        order = plan.unique.cpu().numpy() // 7919          # unique id u is occurrence order[u]
+        ops.csr_gather_reduce_adamw(_dev(g, grad_dtype), plan, plan.occ, None, _dev(idx[order]), f_emb, fb1, fb2, f_m, f_v,
+                                    lr, b1, b2, decay, eps, bs)
+    for gl, fl, cl in ((g_emb, f_emb, c_emb), (g_m, f_m, c_m), (g_v, f_v, c_v)):
+        np.testing.assert_array_equal(torch.cat(gl).float().cpu().numpy(), np.concatenate(cl))
+        np.testing.assert_array_equal(torch.cat(fl).float().cpu().numpy(), np.concatenate(cl))
+    np.testing.assert_array_equal(gb1.cpu().numpy(), cb1)
+    assert _lib.poll_device_errors() == 0
+
+
 @pytest.mark.parametrize("beta_dtype", [np.float32, np.float64])
 def test_adamw_double_rows_bit_exact_vs_oracle(rng, beta_dtype):
     """float64 rows and gradients (the reference's functor is dispatched for them): bit for bit the

@@ -377,3 +377,24 @@ def test_dense_to_ragged_matches_cpu_op():
             np.testing.assert_array_equal(v, rv)
             np.testing.assert_array_equal(o, ro)
             assert ro.dtype == np.int32
+
+
+def test_round_bf16_is_torchs_conversion():
+    """oracle.round_bf16 (what block_apply_adamw_bf16 adds to the Half restatement the compiled reference
+    pins) against torch's float32 -> bfloat16 on the CPU: random magnitudes, exact ties between two
+    neighbours (both parities), subnormals, the largest floats, infinities, NaN."""
+    import torch
+
+    rng = np.random.default_rng(11)
+    with np.errstate(over="ignore", invalid="ignore"):
+        x = (rng.standard_normal(200000) * 10.0 ** rng.integers(-44, 39, 200000)).astype(np.float32)
+    ties = ((rng.integers(0, 1 << 16, 100000).astype(np.uint32) << 16) | np.uint32(0x8000)).view(np.float32)
+    edge = np.array([0.0, -0.0, np.inf, -np.inf, 1e-45, -1e-45, 3.4e38, -3.4e38, 3.3895e38, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -9,
+                     1.00390625, 65504.0], np.float32)
+    x = np.concatenate([x, ties, edge])
+    x = x[~np.isnan(x)]
+    got = oracle.round_bf16(x)
+    exp = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    np.testing.assert_array_equal(got.view(np.uint32), exp.view(np.uint32))
+    assert np.isnan(oracle.round_bf16(np.array([np.nan, 1.0], np.float32))[0])
+    assert got.dtype == np.float32
