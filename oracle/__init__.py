@@ -424,6 +424,29 @@ def block_apply_adagrad(index, grad, emb_blocks, accum, lr, eps, block_size):
                                      c_i64(D))
 
 
+def block_apply_adagrad_exact(index, grad, emb_blocks, accum, lr, eps, block_size, bf16=False):
+    """The Adagrad row update operation by operation, every one rounded once in float32 and the two
+    results rounded to the rows' storage type (float32, or bfloat16 with ``bf16``: float32 arrays of
+    bfloat16 values) when they are assigned:  s = r(s + g * g);  w = r(w - lr * (g / (sqrt(s) + eps))).
+    The reference has no sparse Adagrad; the formula is torch.optim.Adagrad's (lr_decay 0, initial
+    accumulator 0) on the rows that received a gradient, and this function is held to
+    block_apply_adagrad above (which tests/test_oracle_table.py holds to torch.optim.Adagrad) within
+    float32 rounding (tests/test_oracle_table.py). What it adds is the order and place of the
+    roundings, so that the kernels can be compared bit for bit, bfloat16 rows included."""
+    index = _i64(index)
+    g = np.asarray(grad, dtype=np.float32)
+    lr, eps = np.float32(lr), np.float32(eps)
+    r = round_bf16 if bf16 else (lambda x: x)
+    blk, row = index // block_size, index % block_size
+    for b in np.unique(blk):
+        sel = blk == b
+        rr, gg = row[sel], g[sel]
+        s = r(accum[b][rr].astype(np.float32) + gg * gg)
+        w = r(emb_blocks[b][rr].astype(np.float32) - lr * (gg / (np.sqrt(s) + eps)))
+        accum[b][rr] = s
+        emb_blocks[b][rr] = w
+
+
 # ----------------------------------------------------------- dedup / tagging
 
 

@@ -329,6 +329,37 @@ def test_adagrad_vs_oracle(rng, D, bs):
     np.testing.assert_allclose(torch.cat(g_acc).cpu().numpy(), np.concatenate(c_acc), rtol=1e-6, atol=1e-8)
 
 
+@pytest.mark.parametrize("row_dtype,grad_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                                  (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("D,bs", [(128, 64), (16, 1024), (7, 5)])
+def test_adagrad_rows_bit_exact_vs_the_update_with_its_roundings_spelled_out(rng, D, bs, row_dtype, grad_dtype):
+    """oracle.block_apply_adagrad_exact (every operation rounded once in float32, the rows rounded to their
+    storage type when assigned) against the stand-alone row kernel and the fused gather-reduce ending,
+    float32 and bfloat16 rows (what config 5 trains on), bit for bit."""
+    U, steps, lr, eps = 300, 8, 0.05, 1e-8
+    bf = row_dtype == torch.bfloat16
+    rows0 = (0.5 * rng.standard_normal((U, D))).astype(np.float32)
+    if bf:
+        rows0 = oracle.round_bf16(rows0)
+    c_emb, c_acc = _np_blocks(rows0, bs), _np_blocks(np.zeros_like(rows0), bs)
+    g_emb, g_acc = [_dev(b, row_dtype) for b in c_emb], [_dev(b, row_dtype) for b in c_acc]
+    f_emb, f_acc = [b.clone() for b in g_emb], [b.clone() for b in g_acc]
+    for _ in range(steps):
+        idx = np.sort(rng.permutation(U)[:rng.integers(1, U)])
+        g = rng.standard_normal((len(idx), D)).astype(np.float32)
+        if grad_dtype == torch.bfloat16:
+            g = oracle.round_bf16(g)
+        oracle.block_apply_adagrad_exact(idx, g, c_emb, c_acc, lr, eps, bs, bf16=bf)
+        ops.block_apply_adagrad(_dev(idx), _dev(g, grad_dtype), g_emb, g_acc, lr, eps, bs)
+        plan = ops.ids_unique_plan(_dev(np.arange(len(idx), dtype=np.int64) * 7919))
+        order = plan.unique.cpu().numpy() // 7919          # unique id u is occurrence order[u]
+        ops.csr_gather_reduce_adagrad(_dev(g, grad_dtype), plan, plan.occ, None, _dev(idx[order]), f_emb, f_acc, lr, eps, bs)
+    for gl, fl, cl in ((g_emb, f_emb, c_emb), (g_acc, f_acc, c_acc)):
+        np.testing.assert_array_equal(torch.cat(gl).float().cpu().numpy(), np.concatenate(cl))
+        np.testing.assert_array_equal(torch.cat(fl).float().cpu().numpy(), np.concatenate(cl))
+    assert _lib.poll_device_errors() == 0
+
+
 def test_bf16_rows_fp32_grads_track_fp32_path(rng):
     """bf16 row storage: compared with the fp32 oracle within rtol 1e-2 (there is no
     bf16 CPU path in the reference)."""

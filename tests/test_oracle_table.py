@@ -245,3 +245,37 @@ def test_adagrad_vs_torch_adagrad(rng):
         opt.step()
     np.testing.assert_allclose(np.concatenate(emb)[:U], p.detach().numpy(), rtol=1e-6, atol=1e-7)
     np.testing.assert_allclose(np.concatenate(acc)[:U], opt.state[p]["sum"].numpy(), rtol=1e-6, atol=1e-7)
+
+
+def test_adagrad_exact_restatement_vs_torch_adagrad_and_the_c_oracle(rng):
+    """block_apply_adagrad_exact (the update with its roundings spelled out, what the kernels are held to
+    bit for bit): float32 rows against torch.optim.Adagrad and against the C restatement; bfloat16
+    rows hold bfloat16 values and stay within a bfloat16 step per update of the float32 rows."""
+    U, D, steps, lr, eps, bs = 40, 6, 25, 0.01, 1e-8, 16
+    rows0 = (0.01 * rng.standard_normal((U, D))).astype(np.float32)
+    blocks = lambda w: [np.ascontiguousarray(np.concatenate([w, np.zeros((48 - U, D), np.float32)])[i * bs:(i + 1) * bs])
+                        for i in range(3)]
+    emb, acc = blocks(rows0), blocks(np.zeros_like(rows0))
+    emb_c, acc_c = blocks(rows0), blocks(np.zeros_like(rows0))
+    emb_b, acc_b = blocks(oracle.round_bf16(rows0)), blocks(np.zeros_like(rows0))
+    p = torch.nn.Parameter(torch.tensor(rows0))
+    opt = torch.optim.Adagrad([p], lr=lr, eps=eps, lr_decay=0, initial_accumulator_value=0)
+    for _ in range(steps):
+        idx = np.sort(rng.permutation(U)[:rng.integers(1, U)])
+        g = rng.standard_normal((len(idx), D)).astype(np.float32)
+        oracle.block_apply_adagrad_exact(idx, g, emb, acc, lr, eps, bs)
+        oracle.block_apply_adagrad(idx, g, emb_c, acc_c, lr, eps, bs)
+        oracle.block_apply_adagrad_exact(idx, g, emb_b, acc_b, lr, eps, bs, bf16=True)
+        dense = np.zeros((U, D), np.float32)
+        dense[idx] = g
+        p.grad = torch.tensor(dense)
+        opt.step()
+    np.testing.assert_allclose(np.concatenate(emb)[:U], p.detach().numpy(), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(np.concatenate(acc)[:U], opt.state[p]["sum"].numpy(), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(np.concatenate(emb), np.concatenate(emb_c), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(np.concatenate(acc), np.concatenate(acc_c), rtol=1e-6, atol=1e-7)
+    for arr in (np.concatenate(emb_b), np.concatenate(acc_b)):
+        np.testing.assert_array_equal(arr, oracle.round_bf16(arr))        # bfloat16 values
+    # bfloat16 storage: 8 bits of mantissa, 25 updates
+    np.testing.assert_allclose(np.concatenate(emb_b), np.concatenate(emb), rtol=0, atol=25 * 2.0 ** -8 * 0.05)
+    np.testing.assert_allclose(np.concatenate(acc_b), np.concatenate(acc), rtol=25 * 2.0 ** -8, atol=1e-6)
